@@ -1,0 +1,199 @@
+// Shared host/device helpers for the gfx950 backend.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "axhip.h"
+
+namespace axhip {
+
+// ---------------------------------------------------------------- host side
+void set_last_error(const char *fmt, ...);
+hipStream_t resolve_stream(void *stream);
+int ensure_init();
+
+#define AXHIP_CHECK_HIP(expr)                                                          \
+    do {                                                                               \
+        hipError_t _e = (expr);                                                        \
+        if (_e != hipSuccess) {                                                        \
+            ::axhip::set_last_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                                    __FILE__, __LINE__);                               \
+            return static_cast<int>(_e);                                               \
+        }                                                                              \
+    } while (0)
+
+#define AXHIP_REQUIRE(cond, code, ...)                \
+    do {                                              \
+        if (!(cond)) {                                \
+            ::axhip::set_last_error(__VA_ARGS__);     \
+            return (code);                            \
+        }                                             \
+    } while (0)
+
+inline bool valid_dtype(int dt) { return dt >= AXHIP_DTYPE_F32 && dt <= AXHIP_DTYPE_BF16; }
+inline size_t dtype_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
+
+// -------------------------------------------------------------- device side
+constexpr int WAVE = 64;
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+// bf16 <-> f32 with the same rounding as Axiom's bfloat16_t: round to nearest
+// even, NaN canonicalised to 0x7FC0.
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? 0x7FC0u : r;
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); // v_cvt_f16_f32: RNE
+}
+
+template <int DT> struct Elem;
+template <> struct Elem<AXHIP_DTYPE_F32> {
+    using type = float;
+    __device__ static float load(const void *p, int64_t i) { return static_cast<const float *>(p)[i]; }
+    __device__ static void store(void *p, int64_t i, float v) { static_cast<float *>(p)[i] = v; }
+};
+template <> struct Elem<AXHIP_DTYPE_F16> {
+    using type = uint16_t;
+    __device__ static float load(const void *p, int64_t i) { return f16_bits_to_f32(static_cast<const uint16_t *>(p)[i]); }
+    __device__ static void store(void *p, int64_t i, float v) { static_cast<uint16_t *>(p)[i] = static_cast<uint16_t>(f32_to_f16_bits(v)); }
+};
+template <> struct Elem<AXHIP_DTYPE_BF16> {
+    using type = uint16_t;
+    __device__ static float load(const void *p, int64_t i) { return bf16_bits_to_f32(static_cast<const uint16_t *>(p)[i]); }
+    __device__ static void store(void *p, int64_t i, float v) { static_cast<uint16_t *>(p)[i] = static_cast<uint16_t>(f32_to_bf16_bits(v)); }
+};
+
+__device__ __forceinline__ float load_any(const void *p, int dt, int64_t i) {
+    if (dt == AXHIP_DTYPE_F32) return static_cast<const float *>(p)[i];
+    uint32_t h = static_cast<const uint16_t *>(p)[i];
+    return dt == AXHIP_DTYPE_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+}
+__device__ __forceinline__ void store_any(void *p, int dt, int64_t i, float v) {
+    if (dt == AXHIP_DTYPE_F32) {
+        static_cast<float *>(p)[i] = v;
+    } else {
+        static_cast<uint16_t *>(p)[i] =
+            static_cast<uint16_t>(dt == AXHIP_DTYPE_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v));
+    }
+}
+
+// Load / store N consecutive elements (N*sizeof(elem) is 16 or 32 bytes and the
+// address is aligned to min(16, that)) as fp32 values.
+template <int N>
+__device__ __forceinline__ void load_vec(const void *p, int dt, int64_t i, float (&v)[N]) {
+    if (dt == AXHIP_DTYPE_F32) {
+        const float4_t *q = reinterpret_cast<const float4_t *>(static_cast<const float *>(p) + i);
+#pragma unroll
+        for (int j = 0; j < N / 4; ++j) {
+            float4_t t = q[j];
+            v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w;
+        }
+    } else {
+        static_assert(N % 4 == 0, "vector width");
+        if constexpr (N % 8 == 0) {
+            const uint4_t *q = reinterpret_cast<const uint4_t *>(static_cast<const uint16_t *>(p) + i);
+#pragma unroll
+            for (int j = 0; j < N / 8; ++j) {
+                uint4_t t = q[j];
+                uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (dt == AXHIP_DTYPE_BF16) {
+                        v[8 * j + 2 * k] = __uint_as_float(w[k] << 16);
+                        v[8 * j + 2 * k + 1] = __uint_as_float(w[k] & 0xFFFF0000u);
+                    } else {
+                        v[8 * j + 2 * k] = f16_bits_to_f32(w[k] & 0xFFFFu);
+                        v[8 * j + 2 * k + 1] = f16_bits_to_f32(w[k] >> 16);
+                    }
+                }
+            }
+        } else {
+            const uint2_t *q = reinterpret_cast<const uint2_t *>(static_cast<const uint16_t *>(p) + i);
+            uint2_t t = q[0];
+            uint32_t w[2] = {t.x, t.y};
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                if (dt == AXHIP_DTYPE_BF16) {
+                    v[2 * k] = __uint_as_float(w[k] << 16);
+                    v[2 * k + 1] = __uint_as_float(w[k] & 0xFFFF0000u);
+                } else {
+                    v[2 * k] = f16_bits_to_f32(w[k] & 0xFFFFu);
+                    v[2 * k + 1] = f16_bits_to_f32(w[k] >> 16);
+                }
+            }
+        }
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const float (&v)[N]) {
+    if (dt == AXHIP_DTYPE_F32) {
+        float4_t *q = reinterpret_cast<float4_t *>(static_cast<float *>(p) + i);
+#pragma unroll
+        for (int j = 0; j < N / 4; ++j) {
+            float4_t t = {v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
+            q[j] = t;
+        }
+    } else {
+        uint32_t w[N / 2];
+#pragma unroll
+        for (int k = 0; k < N / 2; ++k) {
+            uint32_t lo, hi;
+            if (dt == AXHIP_DTYPE_BF16) {
+                lo = f32_to_bf16_bits(v[2 * k]);
+                hi = f32_to_bf16_bits(v[2 * k + 1]);
+            } else {
+                lo = f32_to_f16_bits(v[2 * k]);
+                hi = f32_to_f16_bits(v[2 * k + 1]);
+            }
+            w[k] = lo | (hi << 16);
+        }
+        if constexpr (N % 8 == 0) {
+            uint4_t *q = reinterpret_cast<uint4_t *>(static_cast<uint16_t *>(p) + i);
+#pragma unroll
+            for (int j = 0; j < N / 8; ++j) {
+                uint4_t t = {w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
+                q[j] = t;
+            }
+        } else {
+            uint2_t *q = reinterpret_cast<uint2_t *>(static_cast<uint16_t *>(p) + i);
+            uint2_t t = {w[0], w[1]};
+            q[0] = t;
+        }
+    }
+}
+
+// wavefront (64 lanes) all-reduce through cross-lane shuffles
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+} // namespace axhip

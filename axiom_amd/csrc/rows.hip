@@ -1,0 +1,692 @@
+// Fused row programs: elementwise chain -> row op (softmax / layer norm / RMS
+// norm) -> elementwise chain -> optional row reduction, one launch, every input
+// element read from HBM once, nothing intermediate written.
+//
+// Layout: a [rows, cols] row-major view.  A row is held in registers as fp32:
+// each thread owns IT chunks of E consecutive elements (E*elem = 16 or 32 bytes,
+// so every global access is a full-width vector), chunk c = it*GROUP + lane_in_group,
+// which makes consecutive lanes touch consecutive 16/32-byte segments.
+// Reductions are wave64 shuffles plus one LDS hop when a row spans several waves.
+#include "common.hpp"
+
+#include <algorithm>
+
+namespace axhip {
+
+constexpr float NEG_INF = -__builtin_huge_valf();
+constexpr float POS_INF = __builtin_huge_valf();
+
+__device__ __forceinline__ float apply_unary(int op, float a) {
+    switch (op) {
+    case AXHIP_OP_RELU: return a > 0.0f ? a : 0.0f;
+    case AXHIP_OP_GELU: return 0.5f * a * (1.0f + erff(a * 0.70710678118654752f));
+    case AXHIP_OP_SQRT: return sqrtf(a);
+    case AXHIP_OP_EXP: return expf(a);
+    case AXHIP_OP_NEG: return -a;
+    case AXHIP_OP_ABS: return fabsf(a);
+    case AXHIP_OP_SIGMOID: {
+        float e = expf(-fabsf(a)), d = 1.0f + e;
+        return a >= 0.0f ? 1.0f / d : e / d;
+    }
+    case AXHIP_OP_TANH: return tanhf(a);
+    case AXHIP_OP_SILU: return a / (1.0f + expf(-a));
+    case AXHIP_OP_LOG: return logf(a);
+    case AXHIP_OP_SQUARE: return a * a;
+    case AXHIP_OP_RSQRT: return 1.0f / sqrtf(a);
+    case AXHIP_OP_RECIP: return 1.0f / a;
+    default: return a;
+    }
+}
+
+__device__ __forceinline__ float apply_binary(int op, float a, float b) {
+    switch (op) {
+    case AXHIP_OP_ADD: return a + b;
+    case AXHIP_OP_SUB: return a - b;
+    case AXHIP_OP_MUL: return a * b;
+    case AXHIP_OP_DIV: return a / b;
+    case AXHIP_OP_MAX: return fmaxf(a, b);
+    case AXHIP_OP_MIN: return fminf(a, b);
+    case AXHIP_OP_RSUB: return b - a;
+    case AXHIP_OP_RDIV: return b / a;
+    default: return a;
+    }
+}
+
+__host__ __device__ inline bool is_binary_op(int op) { return op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV; }
+
+// Apply one chain op to a thread's register tile.  The op code is a kernel
+// argument, so the switch is a scalar (wave-uniform) branch taken once per op;
+// each arm is straight-line vector code over the whole tile.
+template <int IT, int E, typename F>
+__device__ __forceinline__ void for_each_value(float (&v)[IT][E], F f) {
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[it][e] = f(v[it][e], it, e);
+}
+
+template <int IT, int E>
+__device__ __forceinline__ void apply_unary_tile(int op, float (&v)[IT][E]) {
+#define AXHIP_UNARY_CASE(code) \
+    case code: for_each_value<IT, E>(v, [](float a, int, int) { return apply_unary(code, a); }); break
+    switch (op) {
+        AXHIP_UNARY_CASE(AXHIP_OP_RELU);
+        AXHIP_UNARY_CASE(AXHIP_OP_GELU);
+        AXHIP_UNARY_CASE(AXHIP_OP_SQRT);
+        AXHIP_UNARY_CASE(AXHIP_OP_EXP);
+        AXHIP_UNARY_CASE(AXHIP_OP_NEG);
+        AXHIP_UNARY_CASE(AXHIP_OP_ABS);
+        AXHIP_UNARY_CASE(AXHIP_OP_SIGMOID);
+        AXHIP_UNARY_CASE(AXHIP_OP_TANH);
+        AXHIP_UNARY_CASE(AXHIP_OP_SILU);
+        AXHIP_UNARY_CASE(AXHIP_OP_LOG);
+        AXHIP_UNARY_CASE(AXHIP_OP_SQUARE);
+        AXHIP_UNARY_CASE(AXHIP_OP_RSQRT);
+        AXHIP_UNARY_CASE(AXHIP_OP_RECIP);
+    default: break;
+    }
+#undef AXHIP_UNARY_CASE
+}
+
+// w(it, e) yields the second operand of element (it, e)
+template <int IT, int E, typename W>
+__device__ __forceinline__ void apply_binary_tile(int op, float (&v)[IT][E], W w) {
+#define AXHIP_BINARY_CASE(code) \
+    case code: for_each_value<IT, E>(v, [&](float a, int it, int e) { return apply_binary(code, a, w(it, e)); }); break
+    switch (op) {
+        AXHIP_BINARY_CASE(AXHIP_OP_ADD);
+        AXHIP_BINARY_CASE(AXHIP_OP_SUB);
+        AXHIP_BINARY_CASE(AXHIP_OP_MUL);
+        AXHIP_BINARY_CASE(AXHIP_OP_DIV);
+        AXHIP_BINARY_CASE(AXHIP_OP_MAX);
+        AXHIP_BINARY_CASE(AXHIP_OP_MIN);
+        AXHIP_BINARY_CASE(AXHIP_OP_RSUB);
+        AXHIP_BINARY_CASE(AXHIP_OP_RDIV);
+    default: break;
+    }
+#undef AXHIP_BINARY_CASE
+}
+
+// Loads the [IT][E] tile of a FULL or ROWVEC operand.
+template <int IT, int E>
+__device__ __forceinline__ void load_operand_tile(const AxhipOperand &o, const AxhipRowsProgram &P, int64_t row,
+                                                  const int64_t (&col0)[IT], const bool (&ok)[IT], float (&w)[IT][E]) {
+    const int64_t base = o.kind == AXHIP_BK_FULL ? row * P.cols : 0;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        if (ok[it]) {
+            if constexpr (E == 1) w[it][0] = load_any(o.ptr, o.dtype, base + col0[it]);
+            else load_vec<E>(o.ptr, o.dtype, base + col0[it], w[it]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) w[it][e] = 1.0f;
+        }
+    }
+}
+
+template <int IT, int E>
+__device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsProgram &P, float (&v)[IT][E],
+                                         int64_t row, const int64_t (&col0)[IT], const bool (&ok)[IT]) {
+    if (!is_binary_op(c.op)) {
+        apply_unary_tile<IT, E>(c.op, v);
+        return;
+    }
+    if (c.imm_kind == AXHIP_BK_IMM) {
+        const float s = c.imm;
+        apply_binary_tile<IT, E>(c.op, v, [&](int, int) { return s; });
+        return;
+    }
+    const AxhipOperand &o = P.operands[c.operand];
+    if (o.kind == AXHIP_BK_SCALAR || o.kind == AXHIP_BK_COLVEC) {
+        const float s = load_any(o.ptr, o.dtype, o.kind == AXHIP_BK_SCALAR ? 0 : row);
+        apply_binary_tile<IT, E>(c.op, v, [&](int, int) { return s; });
+        return;
+    }
+    float w[IT][E];
+    load_operand_tile<IT, E>(o, P, row, col0, ok, w);
+    apply_binary_tile<IT, E>(c.op, v, [&](int it, int e) { return w[it][e]; });
+}
+
+// norm weight / bias: v = v * w  or  v = v + b with a ROWVEC operand
+template <int IT, int E, bool MUL>
+__device__ __forceinline__ void apply_affine(int operand, const AxhipRowsProgram &P, float (&v)[IT][E], int64_t row,
+                                             const int64_t (&col0)[IT], const bool (&ok)[IT]) {
+    float w[IT][E];
+    load_operand_tile<IT, E>(P.operands[operand], P, row, col0, ok, w);
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[it][e] = MUL ? v[it][e] * w[it][e] : v[it][e] + w[it][e];
+}
+
+// Reduce across the GROUP threads that share a row.  GROUP == 64: shuffles
+// only.  GROUP == blockDim: shuffles, then one LDS exchange between waves.
+template <int GROUP, int THREADS, int KIND /*0 sum, 1 max, 2 min*/>
+__device__ __forceinline__ float group_reduce(float x, float *lds) {
+    x = KIND == 0 ? wave_sum(x) : KIND == 1 ? wave_max(x) : wave_min(x);
+    if constexpr (GROUP > WAVE) {
+        constexpr int NW = THREADS / WAVE;
+        const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+        __syncthreads(); // lds may still be read by a previous reduction
+        if (lane == 0) lds[wave] = x;
+        __syncthreads();
+        float y = lds[lane % NW];
+#pragma unroll
+        for (int o = NW / 2; o > 0; o >>= 1) {
+            float z = __shfl_xor(y, o, WAVE);
+            y = KIND == 0 ? y + z : KIND == 1 ? fmaxf(y, z) : fminf(y, z);
+        }
+        x = y;
+    }
+    return x;
+}
+
+// One row per GROUP threads, the whole row resident in registers.
+template <int THREADS, int GROUP, int IT, int E>
+__global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsProgram P) {
+    __shared__ float lds[THREADS / WAVE];
+    constexpr int ROWS_PER_BLOCK = THREADS / GROUP;
+    const int lane_in_group = threadIdx.x % GROUP;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / GROUP;
+    const bool row_ok = row < P.rows;
+    const int64_t cols = P.cols;
+    const int64_t r = row_ok ? row : 0; // idle groups mirror row 0 so barriers stay uniform; they never store
+
+    float v[IT][E];
+    int64_t col0[IT];
+    bool ok[IT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        col0[it] = (static_cast<int64_t>(it) * GROUP + lane_in_group) * E;
+        ok[it] = col0[it] < cols;
+        if (ok[it]) {
+            if constexpr (E == 1) v[it][0] = load_any(P.input, P.input_dtype, r * cols + col0[it]);
+            else load_vec<E>(P.input, P.input_dtype, r * cols + col0[it], v[it]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[it][e] = 0.0f;
+        }
+    }
+
+    const float inv_n = 1.0f / static_cast<float>(cols);
+    // stage 0: pre chain then the row op; stage 1: post chain.  One loop so the
+    // chain interpreter is instantiated once per kernel.
+#pragma nounroll
+    for (int stage = 0; stage < 2; ++stage) {
+    const int n_ops = stage == 0 ? P.n_pre : P.n_post;
+    for (int i = 0; i < n_ops; ++i) apply_op<IT, E>(stage == 0 ? P.pre[i] : P.post[i], P, v, r, col0, ok);
+    if (stage == 1) break;
+    if (P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX) {
+        float m = NEG_INF;
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+            if (ok[it])
+#pragma unroll
+                for (int e = 0; e < E; ++e) m = fmaxf(m, v[it][e]);
+        m = group_reduce<GROUP, THREADS, 1>(m, lds);
+        const float mm = m == NEG_INF ? 0.0f : m;
+        float s = 0.0f;
+        if (P.row_op == AXHIP_ROWOP_SOFTMAX) {
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    v[it][e] = ok[it] ? __expf(v[it][e] - mm) : 0.0f;
+                    s += v[it][e];
+                }
+            s = group_reduce<GROUP, THREADS, 0>(s, lds);
+            const float inv = 1.0f / s;
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[it][e] *= inv;
+        } else {
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+#pragma unroll
+                for (int e = 0; e < E; ++e) s += ok[it] ? __expf(v[it][e] - mm) : 0.0f;
+            s = group_reduce<GROUP, THREADS, 0>(s, lds);
+            const float ls = __logf(s) + mm;
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[it][e] -= ls;
+        }
+    } else if (P.row_op == AXHIP_ROWOP_LAYERNORM || P.row_op == AXHIP_ROWOP_RMSNORM) {
+        float mean = 0.0f;
+        if (P.row_op == AXHIP_ROWOP_LAYERNORM) {
+            float s = 0.0f;
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+                if (ok[it])
+#pragma unroll
+                    for (int e = 0; e < E; ++e) s += v[it][e];
+            mean = group_reduce<GROUP, THREADS, 0>(s, lds) * inv_n;
+        }
+        float q = 0.0f;
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+            if (ok[it])
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    v[it][e] -= mean;
+                    q += v[it][e] * v[it][e];
+                }
+        const float var = group_reduce<GROUP, THREADS, 0>(q, lds) * inv_n;
+        const float rstd = 1.0f / sqrtf(var + P.eps);
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[it][e] *= rstd;
+        if (P.norm_weight >= 0) apply_affine<IT, E, true>(P.norm_weight, P, v, r, col0, ok);
+        if (P.norm_bias >= 0) apply_affine<IT, E, false>(P.norm_bias, P, v, r, col0, ok);
+    }
+
+    } // stage loop
+
+    if (P.reduce == AXHIP_RED_NONE) {
+        if (row_ok) {
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+                if (ok[it]) {
+                    if constexpr (E == 1) store_any(P.output, P.output_dtype, r * cols + col0[it], v[it][0]);
+                    else store_vec<E>(P.output, P.output_dtype, r * cols + col0[it], v[it]);
+                }
+        }
+        return;
+    }
+    float acc;
+    if (P.reduce == AXHIP_RED_SUM || P.reduce == AXHIP_RED_MEAN) {
+        acc = 0.0f;
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+            if (ok[it])
+#pragma unroll
+                for (int e = 0; e < E; ++e) acc += v[it][e];
+        acc = group_reduce<GROUP, THREADS, 0>(acc, lds);
+        if (P.reduce == AXHIP_RED_MEAN) acc *= inv_n;
+    } else if (P.reduce == AXHIP_RED_MAX) {
+        acc = NEG_INF;
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+            if (ok[it])
+#pragma unroll
+                for (int e = 0; e < E; ++e) acc = fmaxf(acc, v[it][e]);
+        acc = group_reduce<GROUP, THREADS, 1>(acc, lds);
+    } else {
+        acc = POS_INF;
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+            if (ok[it])
+#pragma unroll
+                for (int e = 0; e < E; ++e) acc = fminf(acc, v[it][e]);
+        acc = group_reduce<GROUP, THREADS, 2>(acc, lds);
+    }
+    if (row_ok && lane_in_group == 0) store_any(P.output, P.output_dtype, r, acc);
+}
+
+// Rows too long for registers: one row per block, streamed in up to three
+// passes (two for statistics, one to produce the output).  The pre-chain is
+// recomputed in every pass instead of spilling the row.
+template <int THREADS, int E>
+__global__ __launch_bounds__(THREADS) void rows_streamed_kernel(const AxhipRowsProgram P) {
+    __shared__ float lds[THREADS / WAVE];
+    const int64_t row = blockIdx.x;
+    const int64_t cols = P.cols;
+    const int64_t nchunk = cols / E;
+    const float inv_n = 1.0f / static_cast<float>(cols);
+    const bool is_sm = P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
+    const bool is_norm = P.row_op == AXHIP_ROWOP_LAYERNORM || P.row_op == AXHIP_ROWOP_RMSNORM;
+    // pass 0: softmax max / layer-norm mean; pass 1: softmax sum / variance; pass 2: output
+    const int first_pass = is_sm || P.row_op == AXHIP_ROWOP_LAYERNORM ? 0 : is_norm ? 1 : 2;
+
+    float stat_a = 0.0f, stat_b = 1.0f; // softmax: (max, 1/sum or log-sum); norms: (mean, rstd)
+    float out_acc = P.reduce == AXHIP_RED_MAX ? NEG_INF : P.reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+#pragma nounroll
+    for (int pass = first_pass; pass < 3; ++pass) {
+        float acc = (pass == 0 && is_sm) ? NEG_INF : 0.0f;
+        for (int64_t c = threadIdx.x; c < nchunk; c += THREADS) {
+            float v[1][E];
+            const int64_t col0[1] = {c * E};
+            const bool ok[1] = {true};
+            if constexpr (E == 1) v[0][0] = load_any(P.input, P.input_dtype, row * cols + col0[0]);
+            else load_vec<E>(P.input, P.input_dtype, row * cols + col0[0], v[0]);
+            for (int i = 0; i < P.n_pre; ++i) apply_op<1, E>(P.pre[i], P, v, row, col0, ok);
+            if (pass == 0) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) acc = is_sm ? fmaxf(acc, v[0][e]) : acc + v[0][e];
+            } else if (pass == 1) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const float d = v[0][e] - stat_a;
+                    acc += is_sm ? __expf(d) : d * d;
+                }
+            } else {
+                if (P.row_op == AXHIP_ROWOP_SOFTMAX) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[0][e] = __expf(v[0][e] - stat_a) * stat_b;
+                } else if (P.row_op == AXHIP_ROWOP_LOGSOFTMAX) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[0][e] = v[0][e] - stat_a - stat_b;
+                } else if (is_norm) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[0][e] = (v[0][e] - stat_a) * stat_b;
+                    if (P.norm_weight >= 0) apply_affine<1, E, true>(P.norm_weight, P, v, row, col0, ok);
+                    if (P.norm_bias >= 0) apply_affine<1, E, false>(P.norm_bias, P, v, row, col0, ok);
+                }
+                for (int i = 0; i < P.n_post; ++i) apply_op<1, E>(P.post[i], P, v, row, col0, ok);
+                if (P.reduce == AXHIP_RED_NONE) {
+                    if constexpr (E == 1) store_any(P.output, P.output_dtype, row * cols + col0[0], v[0][0]);
+                    else store_vec<E>(P.output, P.output_dtype, row * cols + col0[0], v[0]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        out_acc = P.reduce == AXHIP_RED_MAX ? fmaxf(out_acc, v[0][e])
+                                  : P.reduce == AXHIP_RED_MIN ? fminf(out_acc, v[0][e]) : out_acc + v[0][e];
+                }
+            }
+        }
+        if (pass == 0) {
+            if (is_sm) {
+                const float m = group_reduce<THREADS, THREADS, 1>(acc, lds);
+                stat_a = m == NEG_INF ? 0.0f : m;
+            } else {
+                stat_a = group_reduce<THREADS, THREADS, 0>(acc, lds) * inv_n;
+            }
+        } else if (pass == 1) {
+            const float t = group_reduce<THREADS, THREADS, 0>(acc, lds);
+            if (is_sm) stat_b = P.row_op == AXHIP_ROWOP_SOFTMAX ? 1.0f / t : __logf(t);
+            else stat_b = 1.0f / sqrtf(t * inv_n + P.eps);
+        }
+    }
+    if (P.reduce != AXHIP_RED_NONE) {
+        if (P.reduce == AXHIP_RED_MAX) out_acc = group_reduce<THREADS, THREADS, 1>(out_acc, lds);
+        else if (P.reduce == AXHIP_RED_MIN) out_acc = group_reduce<THREADS, THREADS, 2>(out_acc, lds);
+        else out_acc = group_reduce<THREADS, THREADS, 0>(out_acc, lds);
+        if (P.reduce == AXHIP_RED_MEAN) out_acc *= inv_n;
+        if (threadIdx.x == 0) store_any(P.output, P.output_dtype, row, out_acc);
+    }
+}
+
+// Flat elementwise chain (no row op, no reduction): grid-stride over chunks of
+// E elements of the flattened [rows*cols] range.  Requires cols % E == 0 so a
+// chunk never straddles two rows.
+template <int THREADS, int E>
+__global__ __launch_bounds__(THREADS) void elementwise_kernel(const AxhipRowsProgram P) {
+    const int64_t cols = P.cols;
+    const int64_t nchunk = P.rows * cols / E;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * THREADS;
+    for (int64_t c = static_cast<int64_t>(blockIdx.x) * THREADS + threadIdx.x; c < nchunk; c += stride) {
+        const int64_t flat = c * E;
+        const int64_t row = flat / cols;
+        const int64_t col0[1] = {flat - row * cols};
+        const bool ok[1] = {true};
+        float v[1][E];
+        if constexpr (E == 1) v[0][0] = load_any(P.input, P.input_dtype, flat);
+        else load_vec<E>(P.input, P.input_dtype, flat, v[0]);
+        for (int i = 0; i < P.n_pre + P.n_post; ++i) apply_op<1, E>(i < P.n_pre ? P.pre[i] : P.post[i - P.n_pre], P, v, row, col0, ok);
+        if constexpr (E == 1) store_any(P.output, P.output_dtype, flat, v[0][0]);
+        else store_vec<E>(P.output, P.output_dtype, flat, v[0]);
+    }
+}
+
+// Chain + reduction over every element: stage 1 leaves one partial per block in
+// the workspace, stage 2 (one block) folds the partials.
+constexpr int FULL_RED_BLOCKS = 2048;
+
+template <int THREADS, int E>
+__global__ __launch_bounds__(THREADS) void full_reduce_stage1(const AxhipRowsProgram P, float *partials) {
+    __shared__ float lds[THREADS / WAVE];
+    const int64_t cols = P.cols;
+    const int64_t nchunk = P.rows * cols / E;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * THREADS;
+    float acc = P.reduce == AXHIP_RED_MAX ? NEG_INF : P.reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+    for (int64_t c = static_cast<int64_t>(blockIdx.x) * THREADS + threadIdx.x; c < nchunk; c += stride) {
+        const int64_t flat = c * E;
+        const int64_t row = flat / cols;
+        const int64_t col0[1] = {flat - row * cols};
+        const bool ok[1] = {true};
+        float v[1][E];
+        if constexpr (E == 1) v[0][0] = load_any(P.input, P.input_dtype, flat);
+        else load_vec<E>(P.input, P.input_dtype, flat, v[0]);
+        for (int i = 0; i < P.n_pre; ++i) apply_op<1, E>(P.pre[i], P, v, row, col0, ok);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            acc = P.reduce == AXHIP_RED_MAX ? fmaxf(acc, v[0][e]) : P.reduce == AXHIP_RED_MIN ? fminf(acc, v[0][e]) : acc + v[0][e];
+    }
+    if (P.reduce == AXHIP_RED_MAX) acc = group_reduce<THREADS, THREADS, 1>(acc, lds);
+    else if (P.reduce == AXHIP_RED_MIN) acc = group_reduce<THREADS, THREADS, 2>(acc, lds);
+    else acc = group_reduce<THREADS, THREADS, 0>(acc, lds);
+    if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+}
+
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void full_reduce_stage2(const float *partials, int n, int reduce, float inv_count,
+                                                              void *out, int out_dtype) {
+    __shared__ float lds[THREADS / WAVE];
+    float acc = reduce == AXHIP_RED_MAX ? NEG_INF : reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+    for (int i = threadIdx.x; i < n; i += THREADS) {
+        float x = partials[i];
+        acc = reduce == AXHIP_RED_MAX ? fmaxf(acc, x) : reduce == AXHIP_RED_MIN ? fminf(acc, x) : acc + x;
+    }
+    if (reduce == AXHIP_RED_MAX) acc = group_reduce<THREADS, THREADS, 1>(acc, lds);
+    else if (reduce == AXHIP_RED_MIN) acc = group_reduce<THREADS, THREADS, 2>(acc, lds);
+    else acc = group_reduce<THREADS, THREADS, 0>(acc, lds);
+    if (reduce == AXHIP_RED_MEAN) acc *= inv_count;
+    if (threadIdx.x == 0) store_any(out, out_dtype, 0, acc);
+}
+
+// ------------------------------------------------------------------ host side
+
+namespace {
+
+bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+int validate_chain(const AxhipChainOp *ops, int n, const AxhipRowsProgram &P, const char *which) {
+    AXHIP_REQUIRE(n >= 0 && n <= AXHIP_MAX_CHAIN, AXHIP_ERR_INVALID_ARG, "fused rows: %s chain length %d out of range", which, n);
+    for (int i = 0; i < n; ++i) {
+        const int op = ops[i].op;
+        const bool bin = is_binary_op(op);
+        const bool un = op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP;
+        AXHIP_REQUIRE(bin || un, AXHIP_ERR_INVALID_ARG, "fused rows: %s[%d] has unknown op code %d", which, i, op);
+        if (bin && ops[i].imm_kind != AXHIP_BK_IMM)
+            AXHIP_REQUIRE(ops[i].operand >= 0 && ops[i].operand < P.n_operands, AXHIP_ERR_INVALID_ARG,
+                          "fused rows: %s[%d] operand index %d out of range", which, i, ops[i].operand);
+    }
+    return AXHIP_OK;
+}
+
+// Picks the vector width E (elements per access): the widest for which every
+// row start and every vector operand stays naturally aligned.
+int pick_vector_width(const AxhipRowsProgram &P) {
+    auto fits = [&](int e) {
+        if (P.cols % e != 0) return false;
+        auto ok = [&](const void *p, int dt) { return aligned_to(p, std::min<size_t>(16, e * dtype_size(dt))); };
+        if (!ok(P.input, P.input_dtype)) return false;
+        if (P.reduce == AXHIP_RED_NONE && !ok(P.output, P.output_dtype)) return false;
+        for (int i = 0; i < P.n_operands; ++i)
+            if ((P.operands[i].kind == AXHIP_BK_FULL || P.operands[i].kind == AXHIP_BK_ROWVEC) &&
+                !ok(P.operands[i].ptr, P.operands[i].dtype))
+                return false;
+        return true;
+    };
+    bool any16 = P.input_dtype != AXHIP_DTYPE_F32;
+    if (any16 && fits(8)) return 8;
+    if (fits(4)) return 4;
+    return 1;
+}
+
+int validate_program(const AxhipRowsProgram &P, const char *who) {
+    AXHIP_REQUIRE(P.rows >= 0 && P.cols >= 0, AXHIP_ERR_INVALID_ARG, "%s: negative extent", who);
+    AXHIP_REQUIRE(valid_dtype(P.input_dtype) && valid_dtype(P.output_dtype), AXHIP_ERR_INVALID_ARG, "%s: bad dtype", who);
+    AXHIP_REQUIRE(P.n_operands >= 0 && P.n_operands <= AXHIP_MAX_OPERANDS, AXHIP_ERR_INVALID_ARG, "%s: bad operand count %d", who, P.n_operands);
+    for (int i = 0; i < P.n_operands; ++i) {
+        AXHIP_REQUIRE(P.operands[i].ptr != nullptr, AXHIP_ERR_INVALID_ARG, "%s: operand %d is NULL", who, i);
+        AXHIP_REQUIRE(valid_dtype(P.operands[i].dtype), AXHIP_ERR_INVALID_ARG, "%s: operand %d has bad dtype", who, i);
+        AXHIP_REQUIRE(P.operands[i].kind >= AXHIP_BK_FULL && P.operands[i].kind <= AXHIP_BK_SCALAR, AXHIP_ERR_INVALID_ARG, "%s: operand %d has bad kind", who, i);
+    }
+    int rc = validate_chain(P.pre, P.n_pre, P, "pre");
+    if (rc) return rc;
+    rc = validate_chain(P.post, P.n_post, P, "post");
+    if (rc) return rc;
+    AXHIP_REQUIRE(P.row_op >= AXHIP_ROWOP_NONE && P.row_op <= AXHIP_ROWOP_RMSNORM, AXHIP_ERR_INVALID_ARG, "%s: bad row_op %d", who, P.row_op);
+    AXHIP_REQUIRE(P.reduce >= AXHIP_RED_NONE && P.reduce <= AXHIP_RED_MIN, AXHIP_ERR_INVALID_ARG, "%s: bad reduce %d", who, P.reduce);
+    for (int idx : {P.norm_weight, P.norm_bias})
+        if (idx >= 0) {
+            AXHIP_REQUIRE(idx < P.n_operands && P.operands[idx].kind == AXHIP_BK_ROWVEC, AXHIP_ERR_INVALID_ARG, "%s: norm weight/bias must be a ROWVEC operand", who);
+        }
+    if (P.rows > 0 && P.cols > 0) AXHIP_REQUIRE(P.input && P.output, AXHIP_ERR_INVALID_ARG, "%s: NULL input/output", who);
+    return AXHIP_OK;
+}
+
+struct RowsPlan {
+    enum Kind { EMPTY, ELEMENTWISE, RESIDENT, STREAMED } kind;
+    int e, it, group, threads;
+    char name[64];
+};
+
+RowsPlan plan_rows(const AxhipRowsProgram &P) {
+    RowsPlan pl{};
+    if (P.rows == 0 || P.cols == 0) {
+        pl.kind = RowsPlan::EMPTY;
+        snprintf(pl.name, sizeof(pl.name), "empty");
+        return pl;
+    }
+    pl.e = pick_vector_width(P);
+    if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) {
+        pl.kind = RowsPlan::ELEMENTWISE;
+        pl.threads = 256;
+        snprintf(pl.name, sizeof(pl.name), "elementwise_e%d", pl.e);
+        return pl;
+    }
+    const int64_t chunks = (P.cols + pl.e - 1) / pl.e;
+    pl.threads = 256;
+    if (chunks <= 64 * 4) { // a row fits one wave with <= 4 chunks per lane
+        pl.group = 64;
+        pl.it = chunks <= 64 ? 1 : chunks <= 128 ? 2 : 4;
+        pl.kind = RowsPlan::RESIDENT;
+    } else if (chunks <= 256 * 8) {
+        pl.group = 256;
+        pl.it = chunks <= 256 ? 1 : chunks <= 512 ? 2 : chunks <= 1024 ? 4 : 8;
+        pl.kind = RowsPlan::RESIDENT;
+    } else {
+        pl.kind = RowsPlan::STREAMED;
+        pl.threads = 1024;
+        pl.group = 1024;
+        pl.it = 0;
+    }
+    if (pl.kind == RowsPlan::RESIDENT) snprintf(pl.name, sizeof(pl.name), "rows_resident_g%d_it%d_e%d", pl.group, pl.it, pl.e);
+    else snprintf(pl.name, sizeof(pl.name), "rows_streamed_e%d", pl.e);
+    return pl;
+}
+
+template <int GROUP, int IT, int E>
+void launch_resident(const AxhipRowsProgram &P, hipStream_t s) {
+    constexpr int THREADS = 256;
+    const int64_t rows_per_block = THREADS / GROUP;
+    const unsigned grid = static_cast<unsigned>((P.rows + rows_per_block - 1) / rows_per_block);
+    hipLaunchKernelGGL((rows_resident_kernel<THREADS, GROUP, IT, E>), dim3(grid), dim3(THREADS), 0, s, P);
+}
+
+template <int GROUP, int E>
+int launch_resident_it(const AxhipRowsProgram &P, int it, hipStream_t s) {
+    switch (it) {
+    case 1: launch_resident<GROUP, 1, E>(P, s); return AXHIP_OK;
+    case 2: launch_resident<GROUP, 2, E>(P, s); return AXHIP_OK;
+    case 4: launch_resident<GROUP, 4, E>(P, s); return AXHIP_OK;
+    case 8:
+        if constexpr (GROUP == 256) {
+            launch_resident<GROUP, 8, E>(P, s);
+            return AXHIP_OK;
+        }
+        [[fallthrough]];
+    default:
+        set_last_error("fused rows: no resident variant for it=%d", it);
+        return AXHIP_ERR_UNSUPPORTED;
+    }
+}
+
+template <int E>
+int launch_plan_e(const AxhipRowsProgram &P, const RowsPlan &pl, hipStream_t s) {
+    switch (pl.kind) {
+    case RowsPlan::ELEMENTWISE: {
+        const int64_t nchunk = P.rows * P.cols / E;
+        const int64_t blocks = std::min<int64_t>((nchunk + 255) / 256, 256 * 32);
+        hipLaunchKernelGGL((elementwise_kernel<256, E>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, P);
+        return AXHIP_OK;
+    }
+    case RowsPlan::RESIDENT:
+        return pl.group == 64 ? launch_resident_it<64, E>(P, pl.it, s) : launch_resident_it<256, E>(P, pl.it, s);
+    case RowsPlan::STREAMED:
+        hipLaunchKernelGGL((rows_streamed_kernel<1024, E>), dim3(static_cast<unsigned>(P.rows)), dim3(1024), 0, s, P);
+        return AXHIP_OK;
+    default:
+        return AXHIP_OK;
+    }
+}
+
+} // namespace
+} // namespace axhip
+
+using namespace axhip;
+
+extern "C" {
+
+const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *P) {
+    static thread_local char name[64];
+    if (!P) return "invalid";
+    RowsPlan pl = plan_rows(*P);
+    snprintf(name, sizeof(name), "%s", pl.name);
+    return name;
+}
+
+int axhip_fused_rows(const AxhipRowsProgram *program, void *stream) {
+    AXHIP_REQUIRE(program != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_fused_rows: program is NULL");
+    const AxhipRowsProgram &P = *program;
+    int rc = validate_program(P, "axhip_fused_rows");
+    if (rc) return rc;
+    AXHIP_REQUIRE(P.rows < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_fused_rows: more than 2^31 rows");
+    rc = ensure_init();
+    if (rc) return rc;
+    RowsPlan pl = plan_rows(P);
+    if (pl.kind == RowsPlan::EMPTY) return AXHIP_OK;
+    hipStream_t s = resolve_stream(stream);
+    rc = pl.e == 8 ? launch_plan_e<8>(P, pl, s) : pl.e == 4 ? launch_plan_e<4>(P, pl, s) : launch_plan_e<1>(P, pl, s);
+    if (rc) return rc;
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+size_t axhip_full_reduce_workspace_bytes(void) { return FULL_RED_BLOCKS * sizeof(float); }
+
+int axhip_fused_full_reduce(const AxhipRowsProgram *program, void *workspace, size_t workspace_bytes, void *stream) {
+    AXHIP_REQUIRE(program != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: program is NULL");
+    const AxhipRowsProgram &P = *program;
+    int rc = validate_program(P, "axhip_fused_full_reduce");
+    if (rc) return rc;
+    AXHIP_REQUIRE(P.row_op == AXHIP_ROWOP_NONE && P.n_post == 0, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: row_op/post must be empty");
+    AXHIP_REQUIRE(P.reduce != AXHIP_RED_NONE, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: reduce is NONE");
+    AXHIP_REQUIRE(P.rows > 0 && P.cols > 0, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: empty input");
+    AXHIP_REQUIRE(workspace && workspace_bytes >= axhip_full_reduce_workspace_bytes() && aligned_to(workspace, 4), AXHIP_ERR_WORKSPACE,
+                  "axhip_fused_full_reduce: workspace too small (%zu < %zu)", workspace_bytes, axhip_full_reduce_workspace_bytes());
+    rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = resolve_stream(stream);
+    AxhipRowsProgram Q = P;
+    Q.reduce = AXHIP_RED_SUM; // only used by pick_vector_width to skip the output alignment test
+    const int e = pick_vector_width(Q);
+    const int64_t n = P.rows * P.cols;
+    const int64_t nchunk = n / e;
+    const int blocks = static_cast<int>(std::min<int64_t>((nchunk + 255) / 256, FULL_RED_BLOCKS));
+    float *partials = static_cast<float *>(workspace);
+    if (e == 8) hipLaunchKernelGGL((full_reduce_stage1<256, 8>), dim3(blocks), dim3(256), 0, s, P, partials);
+    else if (e == 4) hipLaunchKernelGGL((full_reduce_stage1<256, 4>), dim3(blocks), dim3(256), 0, s, P, partials);
+    else hipLaunchKernelGGL((full_reduce_stage1<256, 1>), dim3(blocks), dim3(256), 0, s, P, partials);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    hipLaunchKernelGGL((full_reduce_stage2<256>), dim3(1), dim3(256), 0, s, partials, blocks, P.reduce,
+                       1.0f / static_cast<float>(n), P.output, P.output_dtype);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+} // extern "C"

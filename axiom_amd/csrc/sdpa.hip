@@ -1,0 +1,500 @@
+// Scaled-dot-product attention, forward, for gfx950.
+//
+// Two kernels:
+//   sdpa_mfma_kernel    bf16 / f16, head_dim 32 / 64 / 128.  FlashAttention-2
+//                       schedule on v_mfma_f32_32x32x16_{bf16,f16}: one
+//                       workgroup = 4 wave64 = 128 query rows, each wave owns 32
+//                       query rows whose fragments stay in registers; K and V
+//                       tiles of 64 keys are staged through LDS; fp32 online
+//                       softmax in the exp2 domain; fp32 accumulators.
+//   sdpa_generic_kernel any dtype, head_dim <= 256, fp32 FMA arithmetic; used
+//                       for fp32 inputs and for head sizes the MFMA kernel does
+//                       not cover.
+//
+// The MFMA kernel computes the TRANSPOSED score tile S^T = K * Q^T, so that in
+// the 32x32 accumulator layout every lane owns ONE query column (lane % 32) and
+// 16 key rows.  Row statistics of the softmax are then in-lane reductions plus a
+// single exchange with lane ^ 32, and the exponentiated tile is already laid out
+// as the B operand of the second product O^T += V^T * P^T: no trip through LDS
+// for P.
+#include "common.hpp"
+
+#include <algorithm>
+#include <cmath>
+
+namespace axhip {
+
+struct SdpaArgs {
+    const void *q, *k, *v;
+    void *o;
+    const uint8_t *mask;
+    int B, H, Sq, Skv, D;
+    float scale;       // softmax scale
+    float scale_log2e; // scale * log2(e)
+    int causal;
+    int nqb; // query blocks per (batch, head)
+    int dtype;
+    int64_t qs[3], ks[3], vs[3], os[3], ms[2];
+};
+
+constexpr float NEG_INF_F = -__builtin_huge_valf();
+
+// ---------------------------------------------------------------- MFMA kernel
+
+constexpr int BM = 128; // query rows per workgroup (4 waves x 32)
+constexpr int BN = 64;  // keys per LDS tile
+constexpr int VT_STRIDE = BN + 4; // V^T row stride in elements: 136 B = 34 banks
+
+template <bool BF16>
+__device__ __forceinline__ float16_t mfma_32x32x16(uint4_t a, uint4_t b, float16_t c) {
+    if constexpr (BF16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+}
+
+template <bool BF16> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    if constexpr (BF16) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        float2_t f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t)); // v_cvt_pk_bf16_f32, RNE
+    } else {
+        return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+    }
+}
+
+// Position of key `kv` (0..63) inside a V^T row.  The second MFMA contracts over
+// keys in the order the score accumulator hands them out: slot j of k-step ks in
+// lane group g holds key ks*16 + (j/4)*8 + g*4 + j%4, so V^T stores key
+// ks*16 + h*8 + g*4 + jj at position ks*16 + g*8 + h*4 + jj.
+__device__ __forceinline__ int vt_pos_of_group(int r /* kv / 4 */) {
+    const int ks = r >> 2, h = (r >> 1) & 1, g = r & 1;
+    return (ks * 4 + g * 2 + h) * 4;
+}
+
+template <bool BF16, int D>
+__global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
+    constexpr int KS_STRIDE = D + 8;  // K row stride in elements (272 B at D=128: rows shift by 4 banks)
+    constexpr int KT = D / 16;        // k-steps of the first product
+    constexpr int DT = D / 32;        // 32-row tiles of O^T
+    constexpr int KCH = D / 8;        // 16-byte chunks per K/V row
+    constexpr int KV_CHUNKS = BN * KCH / 256; // 16-byte K chunks per thread per tile (4 at D=128)
+    constexpr int KLD = KV_CHUNKS > 0 ? KV_CHUNKS : 1;
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KS_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[D * VT_STRIDE];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int ql = lane % 32, g = lane / 32;
+
+    // Work-group -> (batch*head, query block).  Work-groups are dealt to the 8
+    // XCDs round-robin by id; keeping one (batch, head) on one XCD lets its K/V
+    // live in that XCD's L2.  Causal blocks are issued heaviest first.
+    const int L = blockIdx.x;
+    const int BH = a.B * a.H;
+    int bh, qb;
+    if (BH % 8 == 0) {
+        const int xcd = L % 8, j = L / 8;
+        bh = (j / a.nqb) * 8 + xcd;
+        qb = j % a.nqb;
+    } else {
+        bh = L / a.nqb;
+        qb = L % a.nqb;
+    }
+    if (a.causal) qb = a.nqb - 1 - qb;
+    const int b = bh / a.H, h = bh % a.H;
+
+    const uint16_t *Q = static_cast<const uint16_t *>(a.q) + b * a.qs[0] + h * a.qs[1];
+    const uint16_t *K = static_cast<const uint16_t *>(a.k) + b * a.ks[0] + h * a.ks[1];
+    const uint16_t *V = static_cast<const uint16_t *>(a.v) + b * a.vs[0] + h * a.vs[1];
+    uint16_t *O = static_cast<uint16_t *>(a.o) + b * a.os[0] + h * a.os[1];
+    const uint8_t *M = a.mask ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
+
+    const int q0 = qb * BM;
+    const int qw0 = q0 + wave * 32; // first query row of this wave
+    const int q = qw0 + ql;
+    const bool q_ok = q < a.Sq;
+
+    // Q^T fragments (B operand): lane holds Q[q][16t + 8g .. +8]
+    uint4_t qf[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+        qf[t] = uint4_t{0, 0, 0, 0};
+        if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
+    }
+
+    float16_t oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
+    float m_run = NEG_INF_F; // running max, scaled log2 domain
+    float l_run = 0.0f;      // this lane's share of the running denominator
+
+    int kv_end = a.Skv;
+    if (a.causal) kv_end = min(a.Skv, q0 + BM);
+    const int ntiles = (kv_end + BN - 1) / BN;
+
+    // staging registers for the next K / V tile
+    uint4_t kreg[KLD], vreg[4];
+    // K: chunk id = tid + 256*n -> row id / KCH, chunk id % KCH
+    // V: thread owns keys 4r..4r+3 x dims 8c..8c+7
+    // (lane bits 0-1 pick the dim chunk, bits 2-4 the key group: 32 consecutive
+    // lanes then hit 32 distinct 8-byte bank pairs when writing V^T)
+    constexpr int CHB = D == 128 ? 2 : D == 64 ? 1 : 0; // bits of the high part of the dim-chunk index
+    const int v_c = ((tid >> 5) & ((1 << CHB) - 1)) * 4 + (tid & 3);
+    const int v_r = ((tid >> (5 + CHB)) & 1) * 8 + ((tid >> 2) & 7);
+    const bool v_active = tid < 2 * D;
+
+    auto load_tile = [&](int tile) {
+        const int kv0 = tile * BN;
+#pragma unroll
+        for (int n = 0; n < KLD; ++n) {
+            const int id = tid + 256 * n;
+            const int row = id / KCH, cc = id % KCH;
+            kreg[n] = uint4_t{0, 0, 0, 0};
+            if (id < BN * KCH && kv0 + row < a.Skv)
+                kreg[n] = *reinterpret_cast<const uint4_t *>(K + static_cast<int64_t>(kv0 + row) * a.ks[2] + 8 * cc);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            vreg[j] = uint4_t{0, 0, 0, 0};
+            const int row = kv0 + 4 * v_r + j;
+            if (v_active && row < a.Skv)
+                vreg[j] = *reinterpret_cast<const uint4_t *>(V + static_cast<int64_t>(row) * a.vs[2] + 8 * v_c);
+        }
+    };
+
+    auto stage_tile = [&]() {
+#pragma unroll
+        for (int n = 0; n < KLD; ++n) {
+            const int id = tid + 256 * n;
+            const int row = id / KCH, cc = id % KCH;
+            if (id < BN * KCH) *reinterpret_cast<uint4_t *>(&Ks[row * KS_STRIDE + 8 * cc]) = kreg[n];
+        }
+        if (v_active) {
+            const int pos = vt_pos_of_group(v_r);
+            const uint32_t r0[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
+            const uint32_t r1[4] = {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w};
+            const uint32_t r2[4] = {vreg[2].x, vreg[2].y, vreg[2].z, vreg[2].w};
+            const uint32_t r3[4] = {vreg[3].x, vreg[3].y, vreg[3].z, vreg[3].w};
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                // even dim 8c+2m: low halves; odd dim 8c+2m+1: high halves
+                uint2_t ev = {__builtin_amdgcn_perm(r1[m], r0[m], 0x05040100u), __builtin_amdgcn_perm(r3[m], r2[m], 0x05040100u)};
+                uint2_t od = {__builtin_amdgcn_perm(r1[m], r0[m], 0x07060302u), __builtin_amdgcn_perm(r3[m], r2[m], 0x07060302u)};
+                *reinterpret_cast<uint2_t *>(&Vt[(8 * v_c + 2 * m) * VT_STRIDE + pos]) = ev;
+                *reinterpret_cast<uint2_t *>(&Vt[(8 * v_c + 2 * m + 1) * VT_STRIDE + pos]) = od;
+            }
+        }
+    };
+
+    if (ntiles > 0) load_tile(0);
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int kv0 = tile * BN;
+        __syncthreads(); // all waves are done reading the previous tile
+        stage_tile();
+        __syncthreads();
+        if (tile + 1 < ntiles) load_tile(tile + 1);
+
+        // a wave whose last query row precedes this tile has nothing to add
+        if (a.causal && kv0 > qw0 + 31) continue;
+
+        // ---- S^T = K Q^T : two 32-key sub-tiles
+        float16_t s[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < KT; ++t) {
+                const uint4_t kf = *reinterpret_cast<const uint4_t *>(&Ks[(kt * 32 + ql) * KS_STRIDE + 16 * t + 8 * g]);
+                s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+            }
+        }
+
+        // ---- masking: only tiles that touch the diagonal, the key tail or an explicit mask
+        const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || M != nullptr;
+        if (need_mask) {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                    bool dead = kv >= a.Skv || (a.causal && kv > q);
+                    if (M != nullptr && q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                    if (dead) s[kt][i] = NEG_INF_F;
+                }
+        }
+
+        // ---- online softmax (per lane: one query column, 32 of the 64 keys)
+        float mloc = NEG_INF_F;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+        const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
+        const float m_use = m_new == NEG_INF_F ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        m_run = m_new;
+        float lsum = 0.0f;
+        uint4_t pf[4]; // P^T fragments (B operand), one per 16-key k-step
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], a.scale_log2e, -m_use));
+                lsum += p[i];
+            }
+            pf[2 * kt] = uint4_t{pack2<BF16>(p[0], p[1]), pack2<BF16>(p[2], p[3]), pack2<BF16>(p[4], p[5]), pack2<BF16>(p[6], p[7])};
+            pf[2 * kt + 1] = uint4_t{pack2<BF16>(p[8], p[9]), pack2<BF16>(p[10], p[11]), pack2<BF16>(p[12], p[13]), pack2<BF16>(p[14], p[15])};
+        }
+        l_run = l_run * alpha + lsum;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const uint16_t *p = &Vt[(dt * 32 + ql) * VT_STRIDE + ks * 16 + g * 8];
+                const uint2_t lo = *reinterpret_cast<const uint2_t *>(p);
+                const uint2_t hi = *reinterpret_cast<const uint2_t *>(p + 4);
+                const uint4_t vf = {lo.x, lo.y, hi.x, hi.y};
+                oacc[dt] = mfma_32x32x16<BF16>(vf, pf[ks], oacc[dt]);
+            }
+    }
+
+    // ---- epilogue: O = O^T / l, written as 4 consecutive dims (8 bytes) per store
+    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (q_ok) {
+        uint16_t *orow = O + static_cast<int64_t>(q) * a.os[2];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int d = dt * 32 + i4 * 8 + g * 4;
+                uint2_t w = {pack2<BF16>(oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv),
+                             pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
+                *reinterpret_cast<uint2_t *>(orow + d) = w;
+            }
+    }
+}
+
+// ------------------------------------------------------------- generic kernel
+// 256 threads = 16 query rows x 16 lanes.  K/V tiles of 32 keys are widened to
+// fp32 in LDS.  Lane c of a row computes scores for keys c, c+16 and output dims
+// c, c+16, ...
+
+constexpr int GM = 16, GN = 32, GMAXD = 256;
+
+__global__ __launch_bounds__(256) void sdpa_generic_kernel(const SdpaArgs a) {
+    extern __shared__ float smem[];
+    const int D = a.D;
+    const int ksd = D + 1;
+    float *Qs = smem;                 // [GM][D]
+    float *Ksm = Qs + GM * D;         // [GN][D+1]
+    float *Vs = Ksm + GN * ksd;       // [GN][D]
+    float *Ps = Vs + GN * D;          // [GM][GN]
+
+    const int tid = threadIdx.x;
+    const int r = tid / 16, c = tid % 16;
+    const int bh = blockIdx.y;
+    const int b = bh / a.H, h = bh % a.H;
+    const int q0 = blockIdx.x * GM;
+    const int q = q0 + r;
+    const bool q_ok = q < a.Sq;
+    const int64_t qoff = b * a.qs[0] + h * a.qs[1], koff = b * a.ks[0] + h * a.ks[1];
+    const int64_t voff = b * a.vs[0] + h * a.vs[1], ooff = b * a.os[0] + h * a.os[1];
+    const uint8_t *M = a.mask ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
+
+    for (int i = tid; i < GM * D; i += 256) {
+        const int rr = i / D, d = i % D;
+        Qs[i] = (q0 + rr < a.Sq) ? load_any(a.q, a.dtype, qoff + static_cast<int64_t>(q0 + rr) * a.qs[2] + d) : 0.0f;
+    }
+
+    float acc[GMAXD / 16];
+#pragma unroll
+    for (int i = 0; i < GMAXD / 16; ++i) acc[i] = 0.0f;
+    float m_run = NEG_INF_F, l_run = 0.0f;
+
+    int kv_end = a.Skv;
+    if (a.causal) kv_end = min(a.Skv, q0 + GM);
+    for (int kv0 = 0; kv0 < kv_end; kv0 += GN) {
+        __syncthreads();
+        for (int i = tid; i < GN * D; i += 256) {
+            const int rr = i / D, d = i % D;
+            const bool ok = kv0 + rr < a.Skv;
+            Ksm[rr * ksd + d] = ok ? load_any(a.k, a.dtype, koff + static_cast<int64_t>(kv0 + rr) * a.ks[2] + d) : 0.0f;
+            Vs[rr * D + d] = ok ? load_any(a.v, a.dtype, voff + static_cast<int64_t>(kv0 + rr) * a.vs[2] + d) : 0.0f;
+        }
+        __syncthreads();
+        float s[GN / 16];
+#pragma unroll
+        for (int jj = 0; jj < GN / 16; ++jj) {
+            const int j = c + 16 * jj;
+            float dot = 0.0f;
+            for (int d = 0; d < D; ++d) dot = __builtin_fmaf(Qs[r * D + d], Ksm[j * ksd + d], dot);
+            dot *= a.scale;
+            const int kv = kv0 + j;
+            bool dead = kv >= a.Skv || (a.causal && kv > q);
+            if (M != nullptr && q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+            s[jj] = dead ? NEG_INF_F : dot;
+        }
+        float mloc = NEG_INF_F;
+#pragma unroll
+        for (int jj = 0; jj < GN / 16; ++jj) mloc = fmaxf(mloc, s[jj]);
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, o, WAVE));
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_use = m_new == NEG_INF_F ? 0.0f : m_new;
+        const float alpha = __expf(m_run - m_use);
+        m_run = m_new;
+        float lsum = 0.0f;
+#pragma unroll
+        for (int jj = 0; jj < GN / 16; ++jj) {
+            const float p = __expf(s[jj] - m_use);
+            Ps[r * GN + c + 16 * jj] = p;
+            lsum += p;
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) lsum += __shfl_xor(lsum, o, WAVE);
+        l_run = l_run * alpha + lsum;
+        __syncthreads();
+#pragma unroll
+        for (int dd = 0; dd < GMAXD / 16; ++dd) {
+            const int d = c + 16 * dd;
+            if (d < D) {
+                float t = acc[dd] * alpha;
+                for (int j = 0; j < GN; ++j) t = __builtin_fmaf(Ps[r * GN + j], Vs[j * D + d], t);
+                acc[dd] = t;
+            }
+        }
+    }
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    if (q_ok) {
+#pragma unroll
+        for (int dd = 0; dd < GMAXD / 16; ++dd) {
+            const int d = c + 16 * dd;
+            if (d < D) store_any(a.o, a.dtype, ooff + static_cast<int64_t>(q) * a.os[2] + d, acc[dd] * inv);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host side
+namespace {
+
+enum class SdpaKind { EMPTY, MFMA, GENERIC, INVALID };
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, const void *v, const void *o) {
+    if (p.batch == 0 || p.heads == 0 || p.seq_q == 0 || p.head_dim == 0) return SdpaKind::EMPTY;
+    const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
+    const bool d_ok = p.head_dim == 32 || p.head_dim == 64 || p.head_dim == 128;
+    if (half && d_ok) {
+        bool ok = true;
+        // 16-byte vector access to every row of q/k/v, 8-byte to o
+        for (int i = 0; i < 3; ++i)
+            ok = ok && p.q_strides[i] % 8 == 0 && p.k_strides[i] % 8 == 0 && p.v_strides[i] % 8 == 0 && p.o_strides[i] % 4 == 0;
+        ok = ok && (!q || aligned16(q)) && (!k || aligned16(k)) && (!v || aligned16(v)) && (!o || aligned16(o));
+        if (ok) return SdpaKind::MFMA;
+    }
+    if (p.head_dim <= GMAXD) return SdpaKind::GENERIC;
+    return SdpaKind::INVALID;
+}
+
+int validate(const AxhipSdpaParams &p) {
+    AXHIP_REQUIRE(valid_dtype(p.dtype), AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: bad dtype %d", p.dtype);
+    AXHIP_REQUIRE(p.batch >= 0 && p.heads >= 0 && p.seq_q >= 0 && p.seq_kv >= 0 && p.head_dim >= 0, AXHIP_ERR_INVALID_ARG,
+                  "axhip_sdpa_fwd: negative extent");
+    for (int i = 0; i < 3; ++i)
+        AXHIP_REQUIRE(p.q_strides[i] >= 0 && p.k_strides[i] >= 0 && p.v_strides[i] >= 0 && p.o_strides[i] >= 0, AXHIP_ERR_INVALID_ARG,
+                      "axhip_sdpa_fwd: negative stride");
+    AXHIP_REQUIRE(p.mask_strides[0] >= 0 && p.mask_strides[1] >= 0, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: negative mask stride");
+    return AXHIP_OK;
+}
+
+template <bool BF16, int D> void launch_mfma(const SdpaArgs &a, hipStream_t s) {
+    const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
+    hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D>), dim3(grid), dim3(256), 0, s, a);
+}
+
+} // namespace
+} // namespace axhip
+
+using namespace axhip;
+
+extern "C" {
+
+const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *p) {
+    static thread_local char name[48];
+    if (!p) return "invalid";
+    switch (pick_kernel(*p, nullptr, nullptr, nullptr, nullptr)) {
+    case SdpaKind::EMPTY: return "empty";
+    case SdpaKind::MFMA:
+        snprintf(name, sizeof(name), "mfma_%s_d%d", p->dtype == AXHIP_DTYPE_BF16 ? "bf16" : "f16", p->head_dim);
+        return name;
+    case SdpaKind::GENERIC: return "generic";
+    default: return "invalid";
+    }
+}
+
+int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const uint8_t *mask,
+                   const AxhipSdpaParams *params, void *stream) {
+    AXHIP_REQUIRE(params != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: params is NULL");
+    const AxhipSdpaParams &p = *params;
+    int rc = validate(p);
+    if (rc) return rc;
+    const SdpaKind kind = pick_kernel(p, q, k, v, o);
+    if (kind == SdpaKind::EMPTY) return AXHIP_OK;
+    AXHIP_REQUIRE(kind != SdpaKind::INVALID, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: head_dim %d > %d is not supported", p.head_dim, GMAXD);
+    AXHIP_REQUIRE(q && k && v && o, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: NULL tensor");
+    AXHIP_REQUIRE(static_cast<int64_t>(p.batch) * p.heads < 65536 || kind == SdpaKind::MFMA, AXHIP_ERR_UNSUPPORTED,
+                  "axhip_sdpa_fwd: batch*heads too large for the generic kernel");
+    rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = resolve_stream(stream);
+
+    SdpaArgs a{};
+    a.q = q; a.k = k; a.v = v; a.o = o; a.mask = mask;
+    a.B = p.batch; a.H = p.heads; a.Sq = p.seq_q; a.Skv = p.seq_kv; a.D = p.head_dim;
+    a.scale = p.scale > 0.0f ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
+    a.scale_log2e = a.scale * 1.44269504088896340736f;
+    a.causal = p.is_causal ? 1 : 0;
+    a.dtype = p.dtype;
+    for (int i = 0; i < 3; ++i) { a.qs[i] = p.q_strides[i]; a.ks[i] = p.k_strides[i]; a.vs[i] = p.v_strides[i]; a.os[i] = p.o_strides[i]; }
+    a.ms[0] = p.mask_strides[0]; a.ms[1] = p.mask_strides[1];
+
+    if (kind == SdpaKind::MFMA) {
+        a.nqb = (p.seq_q + BM - 1) / BM;
+        AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
+        const bool bf = p.dtype == AXHIP_DTYPE_BF16;
+        switch (p.head_dim) {
+        case 32: bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
+        case 64: bf ? launch_mfma<true, 64>(a, s) : launch_mfma<false, 64>(a, s); break;
+        default: bf ? launch_mfma<true, 128>(a, s) : launch_mfma<false, 128>(a, s); break;
+        }
+    } else {
+        a.nqb = (p.seq_q + GM - 1) / GM;
+        const size_t lds = sizeof(float) * (static_cast<size_t>(GM) * a.D + static_cast<size_t>(GN) * (a.D + 1) + static_cast<size_t>(GN) * a.D + GM * GN);
+        static bool attr_set = false;
+        if (!attr_set) {
+            AXHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_generic_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(sdpa_generic_kernel, dim3(a.nqb, a.B * a.H), dim3(256), lds, s, a);
+    }
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,254 @@
+/*
+ * axhip.h -- C ABI of the gfx950 (MI355X) GPU backend for Axiom's two GPU hot
+ * paths: scaled-dot-product attention and the fused elementwise / softmax /
+ * norm chains that the lazy graph emits.
+ *
+ * Conventions
+ *   - every function returns int: 0 on success, a positive value is a
+ *     hipError_t, a negative value is one of AXHIP_ERR_*.  A human-readable
+ *     message for the calling thread's last failure is at axhip_last_error().
+ *   - the caller owns every buffer; kernels never allocate.  Pointers are
+ *     device pointers unless a parameter says "host".
+ *   - `stream` is a hipStream_t passed as void* (NULL = the backend's own
+ *     stream, created by axhip_init and shared process-wide).
+ *   - no exception crosses this boundary.
+ *
+ * Each entry point names the Axiom interface it stands behind (paths relative
+ * to the Axiom source tree).
+ */
+#ifndef AXHIP_H
+#define AXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AXHIP_OK 0
+#define AXHIP_ERR_INVALID_ARG (-1)
+#define AXHIP_ERR_UNSUPPORTED (-2)
+#define AXHIP_ERR_NO_DEVICE (-3)
+#define AXHIP_ERR_WORKSPACE (-4)
+
+/* element types (DType subset of include/axiom/dtype.hpp:171-191) */
+#define AXHIP_DTYPE_F32 0
+#define AXHIP_DTYPE_F16 1
+#define AXHIP_DTYPE_BF16 2
+
+/* ------------------------------------------------------------------ runtime
+ * Stands behind system::is_metal_available (src/tensor/system.cpp:11-29),
+ * make_storage(bytes, Device::GPU) (src/tensor/storage.cpp:26-48),
+ * MetalStorage::copy_to/copy_from (src/backends/metal/metal_storage.mm:66-142)
+ * and MetalExecutionStream::synchronize (src/backends/metal/metal_common.mm:
+ * 285-335).  The Apple unified-memory retag (src/tensor/tensor.cpp:1600-1623)
+ * has no counterpart: transfers are explicit hipMemcpyAsync. */
+int axhip_device_count(int *count);
+int axhip_init(int device);
+const char *axhip_last_error(void);
+const char *axhip_version(void);
+void *axhip_default_stream(void);
+int axhip_malloc(void **ptr, size_t bytes);
+int axhip_free(void *ptr);
+int axhip_memcpy_h2d_async(void *dst_device, const void *src_host, size_t bytes, void *stream);
+int axhip_memcpy_d2h_async(void *dst_host, const void *src_device, size_t bytes, void *stream);
+int axhip_memcpy_d2d_async(void *dst_device, const void *src_device, size_t bytes, void *stream);
+int axhip_stream_sync(void *stream);
+
+/* --------------------------------------------------------------------- SDPA
+ * Stands behind backends::metal::gpu_scaled_dot_product_attention
+ * (src/backends/metal/metal_operations.hpp:47-50, dispatch in
+ * src/backends/metal/flash_attention_dispatch.mm:168-304, kernel
+ * src/backends/metal/flash_attention.metal:50-224), called from
+ * ops::scaled_dot_product_attention (src/tensor/operations.cpp:3979-4044).
+ *
+ * q (B,H,Sq,D), k/v (B,H,Skv,D), o (B,H,Sq,D).  The last dimension is
+ * contiguous; the other three carry explicit element strides so the
+ * (B,S,H,D)->(B,H,S,D) head-split view of nn::MultiHeadAttention
+ * (src/nn/attention.cpp:44-52) needs no copy.  mask is NULL or uint8,
+ * nonzero = masked out (include/axiom/operations.hpp:650), laid out
+ * (Sq,Skv) row-major per (batch, head) with element strides mask_strides
+ * (0 = broadcast).  is_causal masks kv_pos > q_pos (top-left aligned,
+ * src/backends/cpu/flash_attention_cpu.cpp:78-89).  scale <= 0 means
+ * 1/sqrt(D) (src/tensor/operations.cpp:4013-4015).  A row whose keys are all
+ * masked yields zeros.  fp32 accumulation; output in `dtype`.
+ * bf16/f16 with D in {32,64,128} run on MFMA; everything else (fp32, other
+ * head sizes up to 256) runs on the generic fp32-FMA kernel, which takes the
+ * place of the reference's decomposed_attention fallback
+ * (flash_attention_dispatch.mm:125-162). */
+typedef struct {
+    int32_t dtype;
+    int32_t batch, heads, seq_q, seq_kv, head_dim;
+    float scale;
+    int32_t is_causal;
+    int64_t q_strides[3]; /* batch, head, seq (elements) */
+    int64_t k_strides[3];
+    int64_t v_strides[3];
+    int64_t o_strides[3];
+    int64_t mask_strides[2]; /* batch, head (elements; 0 = shared) */
+} AxhipSdpaParams;
+
+int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o,
+                   const uint8_t *mask, const AxhipSdpaParams *params_host, void *stream);
+/* name of the kernel axhip_sdpa_fwd would launch for these parameters
+ * ("mfma_bf16_d128", "generic", ...); the pointer stays valid for the life of
+ * the process. */
+const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *params_host);
+
+/* ------------------------------------------------------------ fused chains
+ * Stands behind graph::materialize_gpu_graph (called from
+ * src/graph/graph_registry.cpp:834-850, Metal implementation
+ * src/backends/metal/mpsgraph_graph_compiler.mm:706-944), the CPU-planned
+ * hooks execute_gpu_fused_chain / execute_gpu_fused_reduction
+ * (include/axiom/graph/gpu_fusion.hpp:14-22), the norm fast paths
+ * gpu_layer_norm / gpu_rms_norm (src/backends/metal/metal_operations.hpp:
+ * 20-24; kernels src/backends/metal/kernels.metal:167-381,
+ * src/backends/metal/mpsgraph_operations.mm:2139-2210) and the per-op GPU
+ * registry entries (src/backends/metal/mpsgraph_operations.mm:2925-3150).
+ *
+ * A program describes ONE pass over a [rows, cols] row-major view:
+ *     v = input
+ *     v = pre[0..n_pre)(v)            elementwise chain
+ *     v = row_op(v)                   softmax / log-softmax / layer norm / RMS norm over cols
+ *     v = post[0..n_post)(v)          elementwise chain
+ *     out = reduce(v) over cols       -> [rows], or out = v -> [rows, cols]
+ * Every value is computed in fp32 and rounded once on store.  One kernel
+ * launch, each input element read once, no intermediate ever written.
+ *
+ * Chain op codes follow ops::OpType (include/axiom/operations.hpp:55-208) for
+ * the hot-path subset. */
+#define AXHIP_OP_ADD 1
+#define AXHIP_OP_SUB 2
+#define AXHIP_OP_MUL 3
+#define AXHIP_OP_DIV 4
+#define AXHIP_OP_MAX 5
+#define AXHIP_OP_MIN 6
+#define AXHIP_OP_RSUB 7 /* operand - v  (chain value is the right-hand side) */
+#define AXHIP_OP_RDIV 8 /* operand / v */
+#define AXHIP_OP_RELU 16
+#define AXHIP_OP_GELU 17
+#define AXHIP_OP_SQRT 18
+#define AXHIP_OP_EXP 19
+#define AXHIP_OP_NEG 20
+#define AXHIP_OP_ABS 21
+#define AXHIP_OP_SIGMOID 22
+#define AXHIP_OP_TANH 23
+#define AXHIP_OP_SILU 24
+#define AXHIP_OP_LOG 25
+#define AXHIP_OP_SQUARE 26
+#define AXHIP_OP_RSQRT 27
+#define AXHIP_OP_RECIP 28
+
+#define AXHIP_ROWOP_NONE 0
+#define AXHIP_ROWOP_SOFTMAX 1
+#define AXHIP_ROWOP_LOGSOFTMAX 2
+#define AXHIP_ROWOP_LAYERNORM 3 /* (x-mean)/sqrt(var+eps) [*w] [+b], population variance */
+#define AXHIP_ROWOP_RMSNORM 4   /* x/sqrt(mean(x^2)+eps) [*w] */
+
+#define AXHIP_RED_NONE 0
+#define AXHIP_RED_SUM 1
+#define AXHIP_RED_MEAN 2
+#define AXHIP_RED_MAX 3
+#define AXHIP_RED_MIN 4
+
+/* how a binary op's second operand maps onto the [rows, cols] view */
+#define AXHIP_BK_FULL 0   /* [rows, cols] */
+#define AXHIP_BK_ROWVEC 1 /* [cols]  broadcast down the rows (weights, biases) */
+#define AXHIP_BK_COLVEC 2 /* [rows]  one value per row (keep_dims reductions) */
+#define AXHIP_BK_SCALAR 3 /* [1]     Axiom's make_scalar operand, device resident */
+#define AXHIP_BK_IMM 4    /* immediate in AxhipChainOp.imm, no memory operand */
+
+#define AXHIP_MAX_CHAIN 16
+#define AXHIP_MAX_OPERANDS 8
+
+typedef struct {
+    const void *ptr;
+    int32_t dtype;
+    int32_t kind; /* AXHIP_BK_* */
+} AxhipOperand;
+
+typedef struct {
+    int32_t op;      /* AXHIP_OP_* */
+    int32_t operand; /* index into operands[] for binary ops, -1 otherwise */
+    float imm;       /* value for AXHIP_BK_IMM */
+    int32_t imm_kind; /* AXHIP_BK_IMM when imm is the operand, else 0 */
+} AxhipChainOp;
+
+typedef struct {
+    int64_t rows, cols;
+    const void *input;
+    int32_t input_dtype;
+    int32_t n_operands;
+    AxhipOperand operands[AXHIP_MAX_OPERANDS];
+    int32_t n_pre;
+    AxhipChainOp pre[AXHIP_MAX_CHAIN];
+    int32_t row_op; /* AXHIP_ROWOP_* */
+    float eps;
+    int32_t norm_weight; /* operand index (ROWVEC) or -1 */
+    int32_t norm_bias;   /* operand index (ROWVEC) or -1 */
+    int32_t n_post;
+    AxhipChainOp post[AXHIP_MAX_CHAIN];
+    int32_t reduce; /* AXHIP_RED_* over cols */
+    void *output;   /* [rows] if reduce != NONE else [rows, cols] */
+    int32_t output_dtype;
+} AxhipRowsProgram;
+
+int axhip_fused_rows(const AxhipRowsProgram *program_host, void *stream);
+/* name of the kernel variant axhip_fused_rows would launch */
+const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *program_host);
+
+/* Elementwise chain followed by a reduction over ALL elements -> one value
+ * (the FusedReductionStep of include/axiom/graph/compiled_graph.hpp:41-70,
+ * GPU hook execute_gpu_fused_reduction).  Uses program->pre only; row_op and
+ * post must be empty; program->reduce selects the reduction; output is one
+ * element.  workspace: device scratch of at least
+ * axhip_full_reduce_workspace_bytes() bytes. */
+size_t axhip_full_reduce_workspace_bytes(void);
+int axhip_fused_full_reduce(const AxhipRowsProgram *program_host, void *workspace,
+                            size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------- data movers
+ * Stands behind gpu_make_contiguous (src/backends/metal/metal_operations.hpp:
+ * 60-63, kernel gather_strided src/backends/metal/kernels.metal:33-149) and
+ * the GPU Cast op (src/tensor/tensor.cpp:1665-1670).  Copies a strided view
+ * (<= 8 dims, non-negative element strides) into a contiguous row-major
+ * buffer, converting dtype on the way. */
+#define AXHIP_MAX_DIMS 8
+int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t dst_dtype,
+                       int32_t ndim, const int64_t *shape_host, const int64_t *src_strides_host,
+                       void *stream);
+int axhip_fill(void *dst, int32_t dtype, double value, int64_t count, void *stream);
+
+/* -------------------------------------------------------------------- GEMM
+ * Stands behind the GPU MatMul registry entry and gpu_linear
+ * (src/backends/metal/mpsgraph_operations.mm:2409-2532; lazy builder
+ * src/backends/metal/mpsgraph_graph_compiler.mm:271-284), used by nn::Linear
+ * as matmul(x, W, false, true) + bias (src/nn/linear.cpp:15-27).
+ * C[b] = op(A[b]) * op(B[b]) (+ bias[N]) (+ residual[b]) for b < batch;
+ * row-major, lda/ldb/ldc and batch strides in elements (stride 0 shares an
+ * operand across the batch).  fp32 accumulation; bf16/f16 on MFMA. */
+typedef struct {
+    int32_t dtype;
+    int32_t trans_a, trans_b;
+    int64_t m, n, k;
+    int64_t lda, ldb, ldc;
+    int64_t batch;
+    int64_t stride_a, stride_b, stride_c;
+    const void *bias;     /* [n] or NULL */
+    const void *residual; /* same layout as C or NULL */
+    int32_t epilogue_op;  /* 0 or AXHIP_OP_RELU / GELU / SILU / SIGMOID / TANH (MatMul+activation fusion) */
+} AxhipGemmParams;
+
+int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemmParams *params_host, void *stream);
+
+/* sizeof() of the parameter structs as this library was compiled, so that a
+ * foreign-language binding can verify its own struct layout at load time:
+ * which = 0 AxhipSdpaParams, 1 AxhipRowsProgram, 2 AxhipGemmParams,
+ * 3 AxhipOperand, 4 AxhipChainOp; anything else returns 0. */
+size_t axhip_sizeof(int which);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,54 @@
+"""GPU parity of axhip_gemm (the nn::Linear / ops::matmul path) against float64
+and against the CPU oracle's matmul."""
+import numpy as np
+import pytest
+
+from oracle import axo
+from tests import gpu_harness as gh
+
+pytestmark = pytest.mark.gpu
+F32, F16, BF16 = axo.F32, axo.F16, axo.BF16
+
+
+def test_linear_known_answers():
+    # tests/test_nn_layers.cpp:12-73
+    x, W = np.ones((1, 3), np.float32), np.ones((2, 3), np.float32)
+    assert np.all(gh.gemm(x, W, F32, trans_b=True) == 3.0)
+    assert np.all(gh.gemm(x, W, F32, trans_b=True, bias=np.ones(2, np.float32)) == 4.0)
+    assert np.all(gh.gemm(np.ones((2, 4), np.float32), np.full((3, 4), 0.5, np.float32), F32, trans_b=True) == 2.0)
+    assert np.all(gh.gemm(np.ones((5, 8), np.float32), np.ones((8, 8), np.float32), F32) == 8.0)
+
+
+@pytest.mark.parametrize("M,N,K,ta,tb", [(7, 5, 9, False, False), (64, 64, 64, False, True), (70, 130, 300, True, False),
+                                          (33, 129, 65, True, True), (1500, 1280, 1280, False, True)])
+def test_f32_matches_oracle(M, N, K, ta, tb):
+    g = axo.PCG64(M + N)
+    A = g.normal((K, M) if ta else (M, K))
+    B = g.normal((N, K) if tb else (K, N)) * (0.02 if K > 1000 else 1.0)
+    got = gh.gemm(A, B, F32, ta, tb)[0]
+    want = axo.matmul(A, B, F32, ta, tb)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K", [(1, 3, 8), (128, 128, 64), (130, 70, 200), (1500, 1280, 1280)])
+def test_half_linear_matches_fp32_reference(dt, M, N, K):
+    g = axo.PCG64(K)
+    x, W = axo.to_bits(g.normal((M, K)), dt), axo.to_bits(g.normal((N, K)) * 0.02, dt)
+    bias = axo.to_bits(g.normal((N,)) * 0.1, dt)
+    res = axo.to_bits(g.normal((M, N)), dt)
+    got = axo.to_f32(gh.gemm(x, W, dt, trans_b=True, bias=bias, residual=res)[0], dt)
+    xf, Wf = axo.to_f32(x, dt).astype(np.float64), axo.to_f32(W, dt).astype(np.float64)
+    want = xf @ Wf.T + axo.to_f32(bias, dt) + axo.to_f32(res, dt)
+    assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
+
+
+def test_batched_shared_weight_and_gelu_epilogue():
+    g = axo.PCG64(5)
+    x, W = axo.to_bits(g.normal((3, 40, 64)), BF16), axo.to_bits(g.normal((48, 64)) * 0.1, BF16)
+    got = axo.to_f32(gh.gemm(x, W, BF16, trans_b=True, epilogue="gelu"), BF16)
+    y = axo.to_f32(x, BF16).astype(np.float64) @ axo.to_f32(W, BF16).astype(np.float64).T
+    import math
+
+    want = 0.5 * y * (1 + np.vectorize(math.erf)(y / math.sqrt(2)))
+    assert np.max(np.abs(got - want)) < 2e-2

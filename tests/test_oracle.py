@@ -1,0 +1,384 @@
+"""Pins the CPU oracle (oracle/axiom_oracle.c) before anything is compared
+against it: reference golden values, the buildable slice of the reference
+(oracle/_ref), closed forms and float64 brute force.  CPU only."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import axo
+
+F32, F16, BF16 = axo.F32, axo.F16, axo.BF16
+
+
+def rng(seed=0):
+    return np.random.default_rng(seed)
+
+
+# ---------------------------------------------------------------- conversions
+
+def test_bf16_golden_bits():
+    # tests/test_bfloat16.cpp:27-57 of the reference
+    L = axo.lib()
+    assert L.axo_f32_to_bf16(0.0) == 0x0000
+    assert L.axo_f32_to_bf16(-0.0) == 0x8000
+    assert L.axo_f32_to_bf16(float("inf")) == 0x7F80
+    assert L.axo_f32_to_bf16(float("-inf")) == 0xFF80
+    assert L.axo_f32_to_bf16(float("nan")) == 0x7FC0
+    assert L.axo_bf16_to_f32(0x3F80) == 1.0
+    assert L.axo_bf16_to_f32(0x4000) == 2.0
+    for v in (0.0, 1.0, -1.0, 3.14, -2.5, 100.0):  # :14-25
+        back = L.axo_bf16_to_f32(L.axo_f32_to_bf16(v))
+        assert abs(back - v) <= abs(v) * 0.01 + 1e-3
+
+
+def test_bf16_is_round_to_nearest_even():
+    x = rng(1).standard_normal(200000).astype(np.float32) * 37.0
+    bits = axo.to_bits(x, BF16)
+    u = x.view(np.uint32).astype(np.uint64)
+    lo, hi = (u >> 16) << 16, ((u >> 16) + 1) << 16
+    flo = lo.astype(np.uint32).view(np.float32).astype(np.float64)
+    fhi = hi.astype(np.uint32).view(np.float32).astype(np.float64)
+    xd = x.astype(np.float64)
+    pick_hi = (np.abs(fhi - xd) < np.abs(flo - xd)) | ((np.abs(fhi - xd) == np.abs(flo - xd)) & (((u >> 16) & 1) == 1))
+    want = np.where(pick_hi, hi >> 16, lo >> 16).astype(np.uint16)
+    assert np.array_equal(bits, want)
+    # exact ties go to even
+    assert axo.lib().axo_f32_to_bf16(np.uint32(0x3F808000).view(np.float32).item()) == 0x3F80
+    assert axo.lib().axo_f32_to_bf16(np.uint32(0x3F818000).view(np.float32).item()) == 0x3F82
+
+
+def test_f16_matches_ieee_exhaustively():
+    allbits = np.arange(65536, dtype=np.uint16)
+    f = axo.to_f32(allbits, F16)
+    want = allbits.view(np.float16).astype(np.float32)
+    assert np.array_equal(f.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.all(np.isnan(f[np.isnan(want)]))
+    x = np.concatenate([rng(2).standard_normal(200000).astype(np.float32) * s for s in (1e-7, 1e-4, 1.0, 300.0, 7e4)])
+    x = np.concatenate([x, np.array([65504.0, 65519.9, 65520.0, 2.0**-24, 2.0**-25, 2.0**-25 * 1.0001, 0.0, -0.0], np.float32)])
+    got = axo.to_bits(x, F16)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+# --------------------------------------------------------------------- PCG64
+
+def test_pcg64_matches_reference_build():
+    r = axo.ref()
+    if r is None:
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    import ctypes as C
+
+    for seed, stream in ((42, 1), (0, 1), (123456789, 7)):
+        want = np.empty(64, np.uint64)
+        r.axref_pcg64(seed, stream, want.ctypes.data_as(C.c_void_p), want.size)
+        g = axo.PCG64(seed, stream)
+        got = np.array([g.next() for _ in range(64)], np.uint64)
+        assert np.array_equal(got, want)
+
+
+def test_pcg64_known_structure():
+    # seed(): state=0, inc=(stream<<1)|1, step, state+=seed, step (include/axiom/random.hpp:24-30)
+    mult, mask = 6364136223846793005, (1 << 64) - 1
+    inc = (1 << 1) | 1
+    st = 0
+
+    def step32(s):
+        xs = (((s >> 18) ^ s) >> 27) & 0xFFFFFFFF
+        rot = s >> 59
+        return ((xs >> rot) | (xs << ((32 - rot) & 31))) & 0xFFFFFFFF, (s * mult + inc) & mask
+
+    def next64(s):
+        hi, s = step32(s)
+        lo, s = step32(s)
+        return (hi << 32) | lo, s
+
+    _, st = next64(st)
+    st = (st + 42) & mask
+    _, st = next64(st)
+    g = axo.PCG64(42, 1)
+    for _ in range(8):
+        want, st = next64(st)
+        assert g.next() == want
+
+
+def test_normal_fill_moments():
+    x = axo.PCG64(7).normal((400000,))
+    assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 1.0) < 0.01
+    u = axo.PCG64(7).uniform((100000,), 0.5, 1.5)
+    assert u.min() >= 0.5 and u.max() < 1.5 and abs(float(u.mean()) - 1.0) < 0.01
+
+
+# --------------------------------------------------------------------- sgemm
+
+@pytest.mark.parametrize("M,N,K,tA,tB,alpha,beta", [
+    (7, 5, 9, False, False, 1.0, 0.0), (64, 64, 64, False, True, 0.125, 0.0), (37, 64, 37, False, False, 1.0, 1.0),
+    (70, 130, 300, True, False, 0.5, 0.75), (3, 129, 513, True, True, 2.0, 0.0), (5, 4, 3, False, False, 0.0, 0.5)])
+def test_sgemm_vs_reference_build_and_float64(M, N, K, tA, tB, alpha, beta):
+    import ctypes as C
+
+    r0 = rng(M * 131 + N)
+    A = r0.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = r0.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    C0 = r0.standard_normal((M, N)).astype(np.float32)
+    got = axo.sgemm(A, B, tA, tB, alpha, beta, C0)
+    opA = A.T if tA else A
+    opB = B.T if tB else B
+    want64 = alpha * (opA.astype(np.float64) @ opB.astype(np.float64)) + beta * C0
+    assert np.allclose(got, want64, rtol=1e-4, atol=1e-4)
+    r = axo.ref()
+    if r is not None:
+        ref_out = C0.copy()
+        p = lambda a: a.ctypes.data_as(C.c_void_p)
+        r.axref_sgemm(int(tA), int(tB), M, N, K, alpha, p(A), A.shape[1], p(B), B.shape[1], beta, p(ref_out), N)
+        # same loop order; the only freedom left is fused vs unfused multiply-add
+        assert np.allclose(got, ref_out, rtol=2e-6, atol=2e-6)
+
+
+# ---------------------------------------------------------------------- SDPA
+
+def naive_attention64(q, k, v, scale, causal=False, mask=None):
+    """softmax(scale*QK^T + mask) V in float64 (tests/test_flash_attention.cpp:14-45)."""
+    q, k, v = (t.astype(np.float64) for t in (q, k, v))
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) * scale
+    Sq, Skv = s.shape[-2:]
+    if causal:
+        s = np.where(np.triu(np.ones((Sq, Skv), bool), 1), -np.inf, s)
+    if mask is not None:
+        s = np.where(np.broadcast_to(mask.astype(bool), s.shape), -np.inf, s)
+    m = s.max(-1, keepdims=True)
+    m = np.where(np.isinf(m), 0.0, m)
+    p = np.exp(s - m)
+    den = p.sum(-1, keepdims=True)
+    p = np.divide(p, den, out=np.zeros_like(p), where=den > 0)
+    return np.einsum("bhqk,bhkd->bhqd", p, v)
+
+
+SDPA_CASES = [  # (B,H,Sq,Skv,D, scale, causal, mask) -- tests/test_flash_attention.cpp:76-213,334-355
+    (1, 2, 8, 8, 32, None, False, None), (1, 2, 16, 32, 32, None, False, None), (1, 2, 16, 16, 32, None, True, None),
+    (1, 1, 8, 8, 32, None, False, "mod3"), (1, 1, 37, 37, 32, None, False, None), (1, 1, 256, 256, 64, None, False, None),
+    (1, 2, 8, 8, 64, None, False, None), (1, 2, 8, 8, 128, None, False, None), (1, 1, 8, 8, 32, 0.5, False, None),
+    (1, 1, 8, 8, 64, -1.0, False, None), (4, 8, 16, 16, 32, None, False, None), (1, 1, 1, 1, 32, None, False, None),
+    (1, 1, 8, 8, 48, None, False, None), (2, 3, 130, 70, 64, None, True, None), (1, 8, 512, 512, 64, 0.125, False, None)]
+
+
+def make_mask(kind, Sq, Skv):
+    if kind is None:
+        return None
+    i, j = np.meshgrid(np.arange(Sq), np.arange(Skv), indexing="ij")
+    return ((i + j) % 3 == 0).astype(np.uint8)  # tests/test_flash_attention.cpp:113-121
+
+
+@pytest.mark.parametrize("case", SDPA_CASES, ids=lambda c: "x".join(str(x) for x in c))
+def test_sdpa_f32_vs_float64_naive(case):
+    B, H, Sq, Skv, D, scale, causal, mk = case
+    g = axo.PCG64(42)
+    q, k, v = g.normal((B, H, Sq, D)), g.normal((B, H, Skv, D)), g.normal((B, H, Skv, D))
+    mask = make_mask(mk, Sq, Skv)
+    eff = 1.0 / math.sqrt(D) if (scale is None or scale <= 0) else scale
+    got = axo.sdpa(q, k, v, F32, scale if scale is not None else eff, causal, mask)
+    want = naive_attention64(q, k, v, eff, causal, mask)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_sdpa_special_cases():
+    g = axo.PCG64(3)
+    q, k, v = g.normal((1, 1, 1, 32)), g.normal((1, 1, 1, 32)), g.normal((1, 1, 1, 32))
+    assert np.allclose(axo.sdpa(q, k, v), v, atol=1e-6)  # S=1 -> O=V
+    # uniform input -> output 1 with or without causal mask (tests/test_flash_attention.cpp:283-328)
+    ones = np.ones((1, 1, 4, 2), np.float32)
+    assert np.allclose(axo.sdpa(ones, ones, ones, causal=True), 1.0, atol=1e-6)
+    # causal == explicit strictly-upper-triangular mask
+    q, k, v = g.normal((2, 2, 70, 32)), g.normal((2, 2, 70, 32)), g.normal((2, 2, 70, 32))
+    tri = np.triu(np.ones((70, 70), np.uint8), 1)
+    assert np.array_equal(axo.sdpa(q, k, v, causal=True), axo.sdpa(q, k, v, mask=tri))
+    # A row whose keys are all masked: the reference's update computes
+    # alpha = exp(m_old - m_new) with both -inf (flash_attention_cpu.cpp:122-125), i.e. NaN,
+    # and the l>0 guard at :166 then yields 0 * NaN.  The restatement reproduces that faithfully;
+    # the GPU kernels deliberately return zeros for such a row instead (tested on the GPU side).
+    m = np.zeros((70, 70), np.uint8)
+    m[5, :] = 1
+    o = axo.sdpa(q, k, v, mask=m)
+    assert np.isnan(o[:, :, 5, :]).all()
+    assert np.isfinite(np.delete(o, 5, axis=2)).all()
+    # 4-D per-(batch, head) mask
+    m4 = (rng(5).random((2, 2, 70, 70)) < 0.3).astype(np.uint8)
+    m4[..., 0] = 0
+    assert np.allclose(axo.sdpa(q, k, v, mask=m4), naive_attention64(q, k, v, 1 / math.sqrt(32), mask=m4), atol=1e-4)
+
+
+@pytest.mark.parametrize("dt,tol", [(BF16, 2e-2), (F16, 2e-3)])
+def test_sdpa_half_inputs_fp32_compute(dt, tol):
+    g = axo.PCG64(11)
+    q, k, v = (axo.to_bits(g.normal((1, 2, 96, 64)), dt) for _ in range(3))
+    o = axo.to_f32(axo.sdpa(q, k, v, dt, causal=True), dt)
+    want = naive_attention64(axo.to_f32(q, dt), axo.to_f32(k, dt), axo.to_f32(v, dt), 0.125, causal=True)
+    assert np.max(np.abs(o - want)) < tol
+
+
+# ------------------------------------------------- softmax / elementwise / reduce
+
+def test_softmax_properties_and_closed_form():
+    x = rng(3).standard_normal((6, 5, 33)).astype(np.float32) * 3
+    for axis in (-1, 0, 1):
+        y = axo.softmax(x, axis=axis)
+        assert np.allclose(y.sum(axis), 1.0, atol=1e-5)  # tests/test_tensor_activations.cpp:11-30
+        e = np.exp(x.astype(np.float64) - x.max(axis, keepdims=True))
+        assert np.allclose(y, e / e.sum(axis, keepdims=True), atol=1e-6)
+        ly = axo.softmax(x, axis=axis, log=True)
+        assert np.allclose(ly, np.log(e / e.sum(axis, keepdims=True)), atol=1e-5)
+    same = axo.softmax(np.full((2, 4), 3.0, np.float32))
+    assert np.allclose(same, 0.25)  # equal inputs -> equal outputs (:32-52)
+    xb = axo.to_bits(x, BF16)
+    yb = axo.to_f32(axo.softmax(xb, BF16), BF16)
+    xf = axo.to_f32(xb, BF16).astype(np.float64)
+    e = np.exp(xf - xf.max(-1, keepdims=True))
+    assert np.max(np.abs(yb - e / e.sum(-1, keepdims=True))) < 4e-3  # one bf16 rounding of values <= 1
+
+
+def test_unary_known_answers():
+    x = np.array([-2.0, -0.5, 0.0, 0.5, 1.0, 2.0], np.float32)
+    assert np.array_equal(axo.unary("relu", x), np.maximum(x, 0))
+    gel = axo.unary("gelu", x)
+    assert gel[2] == 0.0 and 1.9 < gel[5] < 2.1  # tests/test_tensor_activations.cpp:310-334
+    want = np.array([0.5 * t * (1 + math.erf(t / math.sqrt(2))) for t in x.astype(np.float64)])
+    assert np.allclose(gel, want, atol=1e-6)
+    assert abs(math.erf(1.0) - 0.8427) < 1e-4  # the erf the gelu is built on (:356-375)
+    assert np.allclose(axo.unary("sqrt", np.array([4.0, 9.0], np.float32)), [2.0, 3.0])
+    assert np.allclose(axo.unary("sigmoid", x), 1 / (1 + np.exp(-x.astype(np.float64))), atol=1e-6)
+    assert np.allclose(axo.unary("silu", x), x / (1 + np.exp(-x.astype(np.float64))), atol=1e-6)
+    # half types: computed in float, rounded once
+    xb = axo.to_bits(x, BF16)
+    assert np.array_equal(axo.unary("gelu", xb, BF16), axo.to_bits(want.astype(np.float32), BF16))
+
+
+def test_binary_exact_and_broadcast():
+    r0 = rng(4)
+    a, b = r0.standard_normal((5, 8)).astype(np.float32), r0.standard_normal((5, 8)).astype(np.float32)
+    assert np.array_equal(axo.binary("add", a, b), a + b)
+    assert np.array_equal(axo.binary("mul", a, b), a * b)
+    assert np.array_equal(axo.binary("sub", a, b), a - b)
+    assert np.array_equal(axo.binary("div", a, b), a / b)
+    assert np.array_equal(axo.binary("add", a, np.array([1.0], np.float32), kind="scalar"), a + np.float32(1))
+    assert np.array_equal(axo.binary("mul", a, b[0], kind="rowvec"), a * b[0])
+    assert np.array_equal(axo.binary("sub", a, b[:, 0].copy(), kind="colvec"), a - b[:, :1])
+    ab, bb = axo.to_bits(a, BF16), axo.to_bits(b, BF16)
+    want = axo.to_bits(axo.to_f32(ab, BF16) * axo.to_f32(bb, BF16), BF16)
+    assert np.array_equal(axo.binary("mul", ab, bb, BF16), want)
+
+
+def test_fused_pattern_known_answers():
+    # tests/test_fusion_extended.cpp:114-220: a=3,b=2,c=4 and the fused patterns' values
+    a, b, c = (np.full((4, 4), x, np.float32) for x in (3.0, 2.0, 4.0))
+    add, sub, mul = (lambda x, y: axo.binary("add", x, y)), (lambda x, y: axo.binary("sub", x, y)), (lambda x, y: axo.binary("mul", x, y))
+    assert np.all(axo.unary("relu", add(a, b)) == 5.0)
+    assert np.all(axo.unary("relu", sub(b, a)) == 0.0)
+    assert np.all(axo.unary("relu", mul(a, b)) == 6.0)
+    assert np.all(axo.unary("square", add(a, b)) == 25.0)
+    assert np.all(axo.unary("abs", sub(b, a)) == 1.0)
+    assert np.all(axo.unary("sqrt", add(a, np.full((4, 4), 6.0, np.float32))) == 3.0)
+    assert np.all(add(mul(a, b), c) == 10.0)
+    assert np.all(mul(add(a, b), c) == 20.0)
+    assert np.all(mul(sub(a, b), c) == 4.0)
+    assert np.allclose(axo.unary("sigmoid", add(a, b)), 1 / (1 + math.exp(-5)), atol=1e-6)
+    assert np.allclose(axo.unary("exp", sub(b, a)), math.exp(-1), atol=1e-6)
+    # long chain (tests/test_fusion_extended.cpp:561-572): ((((1+1)*2)+3)*... ends at 11
+    x = np.ones((8,), np.float32)
+    for _ in range(10):
+        x = axo.binary("add", x, np.array([1.0], np.float32), kind="scalar")
+    assert np.all(x == 11.0)
+
+
+def test_reduce_known_answers():
+    a, b = np.full((4, 4), 3.0, np.float32), np.full((4, 4), 2.0, np.float32)
+    s = axo.reduce_last("sum", axo.binary("add", a, b).reshape(1, 16))
+    assert s[0] == 80.0  # tests/test_fusion_extended.cpp:346-352
+    big = axo.binary("mul", np.ones((1, 1 << 20), np.float32), np.array([2.0], np.float32), kind="scalar")
+    assert axo.reduce_last("sum", big)[0] == 2097152.0  # :436-443
+    x = rng(6).standard_normal((33, 257)).astype(np.float32)
+    assert np.allclose(axo.reduce_last("sum", x), x.astype(np.float64).sum(-1), atol=1e-4)
+    assert np.allclose(axo.reduce_last("mean", x), x.astype(np.float64).mean(-1), atol=1e-5)
+    assert np.array_equal(axo.reduce_last("max", x), x.max(-1))
+    assert np.array_equal(axo.reduce_last("min", x), x.min(-1))
+    xb = axo.to_bits(x, BF16)
+    m = axo.reduce_last("mean", xb, BF16)  # float accumulate, rounded to bf16 (cpu_operations.cpp:1613-1614)
+    assert np.array_equal(m, axo.to_bits(axo.to_f32(xb, BF16).astype(np.float64).mean(-1).astype(np.float32), BF16))
+
+
+# ----------------------------------------------------------------------- norms
+
+def test_layer_norm_closed_form():
+    x = rng(7).standard_normal((16, 96)).astype(np.float32) * 2 + 0.7
+    y = axo.layer_norm(x)
+    assert np.allclose(y.mean(-1), 0, atol=1e-5) and np.allclose(y.var(-1), 1, atol=1e-3)  # test_tensor_normalization.cpp:9-74
+    w, b = rng(8).uniform(0.5, 1.5, 96).astype(np.float32), rng(9).uniform(-0.1, 0.1, 96).astype(np.float32)
+    xd = x.astype(np.float64)
+    want = (xd - xd.mean(-1, keepdims=True)) / np.sqrt(xd.var(-1, keepdims=True) + 1e-5) * w + b
+    assert np.allclose(axo.layer_norm(x, w, b), want, atol=1e-5)
+
+
+def test_layer_norm_bf16_dtype_flow():
+    # bf16 input: float32 output, first mean rounded to bf16, the rest float32
+    x = axo.PCG64(5).normal((8, 256))
+    xb = axo.to_bits(x, BF16)
+    xf = axo.to_f32(xb, BF16)
+    y = axo.layer_norm(xb, dt=BF16)
+    assert y.dtype == np.float32
+    mean_b = axo.to_f32(axo.to_bits(xf.astype(np.float64).mean(-1).astype(np.float32), BF16), BF16)
+    xc = xf - mean_b[:, None]
+    want = xc / np.sqrt((xc.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-5)
+    assert np.allclose(y, want, atol=1e-5)
+    exact = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5)
+    assert np.max(np.abs(y - exact)) < 2e-2  # the rounded mean costs at most a bf16 ulp of the mean
+
+
+def test_rms_norm_known_answers():
+    x = np.array([[3.0, 4.0]], np.float32)
+    y = axo.rms_norm(x, np.ones(2, np.float32), eps=0.0)
+    assert np.allclose(y, x / math.sqrt(12.5), atol=1e-6)  # tests/test_tensor_normalization.cpp:80-141
+    x4 = np.array([[1.0, 2.0, 3.0, 4.0]], np.float32)
+    assert abs(axo.rms_norm(x4, np.ones(4, np.float32))[0, 0] - 1 / math.sqrt(7.5)) < 1e-4  # tests/test_nn_layers.cpp:191-207
+    x = rng(10).standard_normal((9, 200)).astype(np.float32)
+    w = rng(11).uniform(0.5, 1.5, 200).astype(np.float32)
+    xd = x.astype(np.float64)
+    assert np.allclose(axo.rms_norm(x, w), xd / np.sqrt((xd**2).mean(-1, keepdims=True) + 1e-5) * w, atol=1e-5)
+
+
+# ---------------------------------------------------------------------- matmul
+
+def test_matmul_linear_known_answers():
+    # tests/test_nn_layers.cpp:12-73: ones(1,3) @ ones(2,3)^T -> 3 ; + bias 1 -> 4
+    x, W = np.ones((1, 3), np.float32), np.ones((2, 3), np.float32)
+    assert np.all(axo.matmul(x, W, transB=True) == 3.0)
+    x2, W2 = np.ones((2, 4), np.float32), np.full((3, 4), 0.5, np.float32)
+    assert np.all(axo.matmul(x2, W2, transB=True) == 2.0)
+    assert np.all(axo.matmul(np.ones((5, 8), np.float32), np.ones((8, 8), np.float32)) == 8.0)
+    A, B = rng(12).standard_normal((70, 300)).astype(np.float32), rng(13).standard_normal((300, 65)).astype(np.float32)
+    assert np.allclose(axo.matmul(A, B), A.astype(np.float64) @ B.astype(np.float64), atol=1e-3)
+
+
+def test_matmul_bf16_accumulates_in_bf16():
+    A = axo.to_bits(rng(14).standard_normal((3, 40)).astype(np.float32), BF16)
+    B = axo.to_bits(rng(15).standard_normal((4, 40)).astype(np.float32), BF16)
+    got = axo.matmul(A, B, BF16, transB=True)
+    Af, Bf = axo.to_f32(A, BF16), axo.to_f32(B, BF16)
+    r = lambda t: axo.to_f32(axo.to_bits(np.float32(t).reshape(1), BF16), BF16)[0]
+    want = np.zeros((3, 4), np.float32)
+    for i in range(3):
+        for j in range(4):
+            c = np.float32(0)
+            for k in range(40):
+                c = r(c + r(Af[i, k] * Bf[j, k]))
+            want[i, j] = c
+    assert np.array_equal(got, axo.to_bits(want, BF16))
+
+
+def test_chain_c2_small():
+    g = axo.PCG64(42)
+    a, b = g.normal((16, 64)), g.normal((16, 64))
+    out, sm = axo.chain_relu_add_mul_softmax_sum(a, b, want_softmax=True)
+    x = (np.maximum(a, 0).astype(np.float64) + 1) * b
+    e = np.exp(x - x.max(-1, keepdims=True))
+    assert np.allclose(sm, e / e.sum(-1, keepdims=True), atol=1e-6)
+    assert np.allclose(out, 1.0, atol=1e-5)

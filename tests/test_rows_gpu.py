@@ -1,0 +1,216 @@
+"""GPU parity of axhip_fused_rows / axhip_fused_full_reduce against the CPU
+oracle (Axiom's op-by-op CPU path restated) and float64 closed forms.
+
+Tolerances: fp32 1e-4 abs + 1e-4 rel (relu/add/mul chains bit-exact); bf16 / f16
+2e-2 abs against an fp32-or-better evaluation of the same half inputs."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import axo
+from tests import gpu_harness as gh
+
+pytestmark = pytest.mark.gpu
+F32, F16, BF16 = axo.F32, axo.F16, axo.BF16
+ONE = np.array([1.0], np.float32)
+
+
+def close32(a, b):
+    return np.allclose(a, b, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape", [(4, 5), (1, 1), (3, 37), (64, 256), (7, 1000), (33, 4096), (5, 8200), (2, 70000), (1024, 64)])
+def test_relu_add_mul_chain_is_bit_exact(shape):
+    g = axo.PCG64(1)
+    a, b = g.normal(shape), g.normal(shape)
+    prog = gh.Rows(a, F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b)
+    got = prog.run()
+    want = axo.binary("mul", axo.binary("add", axo.unary("relu", a), ONE, kind="scalar"), b)
+    assert np.array_equal(got, want), prog.kernel_name()
+
+
+def test_fused_pattern_known_answers_on_gpu():
+    # tests/test_fusion_extended.cpp:114-220
+    a, b, c = (np.full((4, 4), x, np.float32) for x in (3.0, 2.0, 4.0))
+    assert np.all(gh.Rows(a, F32).binary("add", b).unary("relu").run() == 5.0)
+    assert np.all(gh.Rows(b, F32).binary("sub", a).unary("relu").run() == 0.0)
+    assert np.all(gh.Rows(a, F32).binary("add", b).unary("square").run() == 25.0)
+    assert np.all(gh.Rows(b, F32).binary("sub", a).unary("abs").run() == 1.0)
+    assert np.all(gh.Rows(a, F32).binary("mul", b).binary("add", c).run() == 10.0)
+    assert np.all(gh.Rows(a, F32).binary("add", b).binary("mul", c).run() == 20.0)
+    assert np.all(gh.Rows(a, F32).binary("rsub", b).run() == -1.0)  # b - a
+    assert np.allclose(gh.Rows(a, F32).binary("add", b).unary("sigmoid").run(), 1 / (1 + math.exp(-5)), atol=1e-6)
+    x = np.ones((8,), np.float32)
+    p = gh.Rows(x.reshape(1, 8), F32)
+    for _ in range(10):
+        p.imm("add", 1.0)
+    assert np.all(p.run() == 11.0)  # long chain, tests/test_fusion_extended.cpp:561-572
+
+
+@pytest.mark.parametrize("op", ["relu", "gelu", "sqrt", "exp", "neg", "abs", "sigmoid", "tanh", "silu", "log", "square", "rsqrt", "recip"])
+def test_unary_ops_match_oracle(op):
+    x = axo.PCG64(2).normal((17, 96))
+    if op in ("sqrt", "log", "rsqrt"):
+        x = np.abs(x) + 0.1
+    got = gh.Rows(x, F32).unary(op).run()
+    assert close32(got, axo.unary(op, x)), op
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "max", "min"])
+@pytest.mark.parametrize("kind", ["full", "rowvec", "colvec", "scalar"])
+def test_binary_ops_and_broadcast_kinds(op, kind):
+    g = axo.PCG64(3)
+    a = g.normal((9, 40))
+    b = {"full": g.normal((9, 40)), "rowvec": g.normal((40,)), "colvec": g.normal((9,)), "scalar": g.normal((1,))}[kind] + 3.0
+    got = gh.Rows(a, F32).binary(op, b, kind).run()
+    assert np.array_equal(got, axo.binary(op, a, b, kind=kind))
+
+
+@pytest.mark.parametrize("shape", [(4, 5), (2, 3, 33), (16, 256), (8, 1024), (3, 8192), (2, 20000), (1, 70001)])
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_matches_oracle(shape, log):
+    x = axo.PCG64(4).normal(shape) * 3
+    p = gh.Rows(x, F32).row_op("logsoftmax" if log else "softmax")
+    got = p.run()
+    want = axo.softmax(x, log=log)
+    assert close32(got, want), p.kernel_name()
+    if not log:
+        assert np.allclose(got.sum(-1), 1.0, atol=1e-4)
+
+
+@pytest.mark.parametrize("dt,tol", [(BF16, 4e-3), (F16, 5e-4)])
+def test_softmax_half(dt, tol):
+    x = axo.to_bits(axo.PCG64(5).normal((33, 1000)) * 2, dt)
+    got = axo.to_f32(gh.Rows(x, dt).row_op("softmax").run(), dt)
+    assert np.max(np.abs(got - axo.to_f32(axo.softmax(x, dt), dt))) <= tol
+
+
+@pytest.mark.parametrize("red", ["sum", "mean", "max", "min"])
+@pytest.mark.parametrize("shape", [(4, 5), (64, 64), (5, 4096), (3, 50000)])
+def test_row_reductions(red, shape):
+    x = axo.PCG64(6).normal(shape)
+    got = gh.Rows(x, F32).run(reduce=red)
+    want = axo.reduce_last(red, x)
+    assert close32(got, want)
+    if red in ("max", "min"):
+        assert np.array_equal(got, want)
+
+
+def test_reduce_known_answers_on_gpu():
+    a, b = np.full((1, 16), 3.0, np.float32), np.full((1, 16), 2.0, np.float32)
+    assert gh.Rows(a, F32).binary("add", b).run(reduce="sum")[0] == 80.0  # tests/test_fusion_extended.cpp:346-352
+    big = np.ones((1, 1 << 20), np.float32)
+    assert gh.Rows(big, F32).imm("mul", 2.0).run(reduce="sum")[0] == 2097152.0  # :436-443
+    assert gh.Rows(big.reshape(1024, 1024), F32).imm("mul", 2.0).run_full_reduce("sum")[0] == 2097152.0
+    x = axo.PCG64(8).normal((300, 777))
+    got = gh.Rows(x, F32).unary("square").run_full_reduce("mean")[0]
+    assert abs(got - float((x.astype(np.float64) ** 2).mean())) < 1e-4
+    assert gh.Rows(x, F32).run_full_reduce("max")[0] == x.max()
+    assert gh.Rows(x, F32).run_full_reduce("min")[0] == x.min()
+
+
+@pytest.mark.parametrize("rows,cols", [(256, 512), (16, 8192), (3, 100)])
+def test_c2_chain_softmax_then_row_sum(rows, cols):
+    """softmax((relu(a)+1)*b, -1).sum(1) in ONE launch; plus the intermediate softmax."""
+    g = axo.PCG64(42)
+    a, b = g.normal((rows, cols)), g.normal((rows, cols))
+    want_sum, want_sm = axo.chain_relu_add_mul_softmax_sum(a, b, want_softmax=True)
+    got_sm = gh.Rows(a, F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b).row_op("softmax").run()
+    assert close32(got_sm, want_sm)
+    got_sum = gh.Rows(a, F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b).row_op("softmax").run(reduce="sum")
+    assert close32(got_sum, want_sum) and np.allclose(got_sum, 1.0, atol=1e-4)
+
+
+def ln64(xf, w=None, b=None, eps=1e-5, gelu=False, rms=False):
+    x = xf.astype(np.float64)
+    if rms:
+        y = x / np.sqrt((x**2).mean(-1, keepdims=True) + eps)
+    else:
+        y = (x - x.mean(-1, keepdims=True)) / np.sqrt(x.var(-1, keepdims=True) + eps)
+    if w is not None:
+        y = y * w
+    if b is not None:
+        y = y + b
+    if gelu:
+        y = 0.5 * y * (1 + np.vectorize(math.erf)(y / math.sqrt(2)))
+    return y
+
+
+@pytest.mark.parametrize("shape", [(4, 5), (16, 96), (32, 4096), (4, 20000), (2, 3, 1280)])
+def test_layer_norm_f32(shape):
+    g = axo.PCG64(10)
+    x = g.normal(shape) * 2 + 0.5
+    w, b = g.uniform((shape[-1],), 0.5, 1.5), g.uniform((shape[-1],), -0.1, 0.1)
+    got = gh.Rows(x, F32).row_op("layernorm", 1e-5, w, b).run()
+    assert close32(got, axo.layer_norm(x, w, b))
+    plain = gh.Rows(x, F32).row_op("layernorm", 1e-5).run()
+    assert np.allclose(plain.mean(-1), 0, atol=1e-4) and np.allclose(plain.var(-1), 1, atol=1e-2)
+
+
+def test_rms_norm_f32_known_answers():
+    x = np.array([[3.0, 4.0]], np.float32)
+    got = gh.Rows(x, F32).row_op("rmsnorm", 0.0, np.ones(2, np.float32)).run()
+    assert np.allclose(got, x / math.sqrt(12.5), atol=1e-6)  # tests/test_tensor_normalization.cpp:80-141
+    x4 = np.array([[1.0, 2.0, 3.0, 4.0]], np.float32)
+    assert abs(gh.Rows(x4, F32).row_op("rmsnorm", 1e-5, np.ones(4, np.float32)).run()[0, 0] - 1 / math.sqrt(7.5)) < 1e-4
+    g = axo.PCG64(11)
+    x, w = g.normal((9, 200)), g.uniform((200,), 0.5, 1.5)
+    assert close32(gh.Rows(x, F32).row_op("rmsnorm", 1e-5, w).run(), axo.rms_norm(x, w))
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("rms", [False, True], ids=["layernorm", "rmsnorm"])
+@pytest.mark.parametrize("shape", [(64, 4096), (7, 1280), (3, 100)])
+def test_c3_norm_gelu_chain_half(dt, rms, shape):
+    """gelu(layer_norm(x)*gamma+beta) and the RMSNorm variant, half in / half out, one launch."""
+    g = axo.PCG64(42)
+    x = axo.to_bits(g.normal(shape), dt)
+    w = axo.to_bits(g.uniform((shape[-1],), 0.5, 1.5), dt)
+    b = axo.to_bits(g.uniform((shape[-1],), -0.1, 0.1), dt)
+    p = gh.Rows(x, dt).row_op("rmsnorm" if rms else "layernorm", 1e-5, w, None if rms else b).unary("gelu")
+    got = axo.to_f32(p.run(), dt)
+    xf, wf, bf = (axo.to_f32(t, dt) for t in (x, w, b))
+    want = ln64(xf, wf, None if rms else bf, gelu=True, rms=rms)
+    err = np.abs(got - want)
+    # one rounding of the result to the half type: half an ulp of |y| (bf16: 2^-8 relative)
+    ulp = np.maximum(np.abs(want), 1e-3) * (2.0**-8 if dt == BF16 else 2.0**-11)
+    assert np.all(err <= np.maximum(2e-2, ulp * 1.01)) and np.max(err[np.abs(want) < 4]) < 2e-2
+    # distance to the literal CPU path (float32 output, half-rounded first mean): reported bound
+    lit = axo.rms_norm(x, w, dt) if rms else axo.layer_norm(x, w, b, dt)
+    lit = axo.unary("gelu", lit)
+    assert np.max(np.abs(got - lit)) < 6e-2
+
+
+def test_mixed_dtype_operands_and_output_dtype():
+    g = axo.PCG64(12)
+    x = axo.to_bits(g.normal((8, 256)), BF16)
+    w = g.uniform((256,), 0.5, 1.5)  # fp32 weights on a bf16 activation
+    got = gh.Rows(x, BF16, out_dt=F32).row_op("layernorm", 1e-5, w, None, wdt=F32).run()
+    assert got.dtype == np.float32
+    assert np.allclose(got, ln64(axo.to_f32(x, BF16), w), atol=1e-4)
+
+
+def test_full_size_c2_and_c3_properties():
+    """BASELINE shapes: C2 fp32 [8192,8192] chain -> every row sums to 1; C3 bf16 [16384,4096]
+    layer norm: per-row mean ~ 0 and variance ~ 1; a 256-row slice of each against the oracle."""
+    g = axo.PCG64(42)
+    a, b = g.normal((8192, 8192)), g.normal((8192, 8192))
+    p = gh.Rows(a, F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b).row_op("softmax")
+    assert p.kernel_name() == "rows_resident_g256_it8_e4"
+    s = p.run(reduce="sum")
+    assert np.allclose(s, 1.0, atol=1e-4)
+    sm = gh.Rows(a[:256], F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b[:256]).row_op("softmax").run()
+    _, want_sm = axo.chain_relu_add_mul_softmax_sum(a[:256], b[:256], want_softmax=True)
+    assert close32(sm, want_sm)
+    del a, b
+    x = axo.to_bits(g.normal((16384, 4096)), BF16)
+    y = axo.to_f32(gh.Rows(x, BF16).row_op("layernorm", 1e-5).run(), BF16)
+    assert np.allclose(y.mean(-1), 0, atol=2e-3) and np.allclose(y.var(-1), 1, atol=2e-2)
+    want = ln64(axo.to_f32(x[:256], BF16))
+    assert np.max(np.abs(y[:256] - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
+
+
+def test_empty_inputs_are_no_ops():
+    x = np.zeros((0, 16), np.float32)
+    assert gh.Rows(x, F32).unary("relu").run().shape == (0, 16)

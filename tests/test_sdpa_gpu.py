@@ -1,0 +1,146 @@
+"""GPU parity of axhip_sdpa_fwd against the CPU oracle (Axiom's tiled flash
+attention restated) and the float64 textbook formula.  Shape cases follow the
+reference's tests/test_flash_attention.cpp and tests/test_nn_attention.cpp.
+
+Tolerances: fp32 1e-4 abs + 1e-4 rel; bf16 / f16 2e-2 abs against an fp32-or-better
+evaluation of the SAME half-precision inputs."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import axo
+from tests import gpu_harness as gh
+from tests.test_oracle import SDPA_CASES, make_mask, naive_attention64
+
+pytestmark = pytest.mark.gpu
+F32, F16, BF16 = axo.F32, axo.F16, axo.BF16
+
+
+def inputs(B, H, Sq, Skv, D, dt, seed=42):
+    g = axo.PCG64(seed)
+    return tuple(axo.to_bits(g.normal(s), dt) for s in ((B, H, Sq, D), (B, H, Skv, D), (B, H, Skv, D)))
+
+
+@pytest.mark.parametrize("case", SDPA_CASES, ids=lambda c: "x".join(str(x) for x in c))
+def test_f32_matches_cpu_oracle(case):
+    B, H, Sq, Skv, D, scale, causal, mk = case
+    q, k, v = inputs(B, H, Sq, Skv, D, F32)
+    mask = make_mask(mk, Sq, Skv)
+    sc = -1.0 if scale is None else scale
+    got, kern = gh.sdpa(q, k, v, F32, sc, causal, mask)
+    assert kern == "generic"
+    want = axo.sdpa(q, k, v, F32, sc, causal, mask)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4), np.max(np.abs(got - want))
+
+
+HALF_CASES = [  # (B,H,Sq,Skv,D, causal, mask)
+    (1, 2, 16, 16, 64, False, None),       # tests/test_flash_attention.cpp:233-249 (Float16 GPU case)
+    (1, 2, 8, 8, 32, False, None), (1, 2, 8, 8, 128, False, None), (1, 2, 16, 32, 32, False, None),
+    (1, 2, 16, 16, 32, True, None), (1, 1, 8, 8, 32, False, "mod3"), (1, 1, 37, 37, 32, False, None),
+    (1, 1, 256, 256, 64, False, None), (4, 8, 16, 16, 32, False, None), (1, 1, 1, 1, 32, False, None),
+    (2, 3, 130, 70, 64, True, None), (2, 3, 70, 130, 64, True, None), (1, 2, 300, 300, 128, True, None),
+    (1, 3, 257, 511, 128, False, "mod3"), (1, 20, 1500, 1500, 64, False, None),  # Whisper encoder shape
+    (2, 8, 1024, 1024, 128, True, None), (1, 1, 8, 8, 48, False, None), (1, 1, 64, 64, 96, True, None)]
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", HALF_CASES, ids=lambda c: "x".join(str(x) for x in c))
+def test_half_matches_fp32_reference_of_same_inputs(case, dt):
+    B, H, Sq, Skv, D, causal, mk = case
+    q, k, v = inputs(B, H, Sq, Skv, D, dt, seed=7)
+    mask = make_mask(mk, Sq, Skv)
+    got, kern = gh.sdpa(q, k, v, dt, -1.0, causal, mask)
+    assert kern == ("generic" if D in (48, 96) else f"mfma_{'bf16' if dt == BF16 else 'f16'}_d{D}")
+    qf, kf, vf = (axo.to_f32(t, dt) for t in (q, k, v))
+    if B * H * Sq * Skv <= 1 << 24:
+        want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), causal, mask)
+    else:  # large cases: the CPU oracle's fp32 tiled algorithm on the widened inputs
+        want = axo.sdpa(qf, kf, vf, F32, -1.0, causal, mask)
+    gotf = axo.to_f32(got, dt)
+    assert np.isfinite(gotf).all()
+    err = np.max(np.abs(gotf - want))
+    assert err < 2e-2, err
+    # and the distance to the literal CPU path (half output of the tiled algorithm)
+    lit = axo.to_f32(axo.sdpa(q, k, v, dt, -1.0, causal, mask), dt)
+    assert np.max(np.abs(gotf - lit)) < 4e-2
+
+
+def test_fully_masked_rows_give_zeros_everywhere_else_matches():
+    q, k, v = inputs(1, 2, 70, 70, 64, BF16, seed=3)
+    m = np.zeros((70, 70), np.uint8)
+    m[5, :] = 1
+    m[9, :64] = 1  # first 64-key tile fully masked, the tail visible
+    for dt, (qq, kk, vv) in ((BF16, (q, k, v)), (F32, tuple(axo.to_f32(t, BF16) for t in (q, k, v)))):
+        got, _ = gh.sdpa(qq, kk, vv, dt, -1.0, False, m)
+        gf = axo.to_f32(got, dt)
+        assert np.all(gf[:, :, 5, :] == 0.0)
+        want = naive_attention64(*(axo.to_f32(t, dt) for t in (qq, kk, vv)), 0.125, False, m)
+        assert np.max(np.abs(gf - want)) < (2e-2 if dt == BF16 else 1e-4)
+
+
+def test_per_batch_head_mask_and_broadcast_masks():
+    B, H, S, D = 2, 3, 96, 64
+    q, k, v = inputs(B, H, S, S, D, BF16, seed=5)
+    r = np.random.default_rng(0)
+    for shape in ((B, H, S, S), (1, 1, S, S), (B, 1, S, S), (1, H, S, S)):
+        m = (r.random(shape) < 0.3).astype(np.uint8)
+        m[..., 0] = 0
+        got, _ = gh.sdpa(q, k, v, BF16, -1.0, False, m)
+        want = naive_attention64(*(axo.to_f32(t, BF16) for t in (q, k, v)), 0.125, False, m)
+        assert np.max(np.abs(axo.to_f32(got, BF16) - want)) < 2e-2
+
+
+def test_head_split_view_strides_need_no_copy():
+    # nn::MultiHeadAttention hands (B,S,H*D) projections viewed as (B,H,S,D): strides (S*H*D, D, H*D)
+    B, S, H, D = 2, 200, 4, 64
+    g = axo.PCG64(9)
+    packed = [axo.to_bits(g.normal((B, S, H, D)), BF16) for _ in range(3)]
+    st = (S * H * D, D, H * D)
+    got, kern = gh.sdpa(*packed, BF16, -1.0, True, None, q_strides=st, k_strides=st, v_strides=st, shape=(B, H, S, S, D))
+    assert kern == "mfma_bf16_d64"
+    qf, kf, vf = (axo.to_f32(t, BF16).transpose(0, 2, 1, 3) for t in packed)
+    want = naive_attention64(qf, kf, vf, 0.125, True)
+    assert np.max(np.abs(axo.to_f32(got, BF16) - want)) < 2e-2
+
+
+def test_scale_parameter_and_auto_scale():
+    q, k, v = inputs(1, 1, 64, 64, 64, BF16, seed=1)
+    f = [axo.to_f32(t, BF16) for t in (q, k, v)]
+    a, _ = gh.sdpa(q, k, v, BF16, 0.5)
+    assert np.max(np.abs(axo.to_f32(a, BF16) - naive_attention64(*f, 0.5))) < 2e-2
+    b, _ = gh.sdpa(q, k, v, BF16, -1.0)
+    c, _ = gh.sdpa(q, k, v, BF16, 0.125)
+    assert np.array_equal(b, c)  # scale <= 0 -> 1/sqrt(D)
+
+
+def test_uniform_input_gives_ones():
+    ones = axo.to_bits(np.ones((1, 1, 4, 32), np.float32), BF16)
+    got, _ = gh.sdpa(ones, ones, ones, BF16, -1.0, True)
+    assert np.allclose(axo.to_f32(got, BF16), 1.0, atol=1e-2)
+
+
+def test_full_size_causal_bf16_properties():
+    """B4 H32 S4096 D128 causal bf16: size-independent checks on the whole tensor plus the
+    oracle on a deterministic subset of (batch, head) slices."""
+    B, H, S, D = 4, 32, 4096, 128
+    g = axo.PCG64(42)
+    q, k, v = (axo.to_bits(g.normal((B, H, S, D)), BF16) for _ in range(3))
+    got, kern = gh.sdpa(q, k, v, BF16, -1.0, True)
+    assert kern == "mfma_bf16_d128"
+    gf = axo.to_f32(got, BF16)
+    assert np.isfinite(gf).all()
+    vf = axo.to_f32(v, BF16)
+    # causal row 0 attends to key 0 only: O[...,0,:] == V[...,0,:] exactly
+    assert np.array_equal(gf[:, :, 0, :], vf[:, :, 0, :])
+    # every output is a convex combination of the visible values
+    run_max = np.maximum.accumulate(vf, axis=2)
+    run_min = np.minimum.accumulate(vf, axis=2)
+    assert np.all(gf <= run_max + 2e-2) and np.all(gf >= run_min - 2e-2)
+    # oracle on slices 0, 37, 127 (fp32 tiled algorithm on the widened bf16 inputs)
+    for sl in (0, 37, 127):
+        b, h = divmod(sl, H)
+        qs, ks, vs = (axo.to_f32(t[b:b + 1, h:h + 1], BF16) for t in (q, k, v))
+        want = axo.sdpa(qs, ks, vs, F32, -1.0, True)
+        err = np.max(np.abs(gf[b:b + 1, h:h + 1] - want))
+        assert err < 2e-2, (sl, err)
