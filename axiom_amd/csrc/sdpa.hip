@@ -43,7 +43,9 @@ constexpr float NEG_INF_F = -__builtin_huge_valf();
 
 constexpr int BM = 128; // query rows per workgroup (4 waves x 32)
 constexpr int BN = 64;  // keys per LDS tile
-constexpr int VT_STRIDE = BN + 4; // V^T row stride in elements: 136 B = 34 banks
+// Growth of the running row maximum (log2 domain) that is tolerated before the
+// accumulators are rescaled: exponentials stay below 2^8, far inside fp32/bf16/f16 range.
+constexpr float RESCALE_THRESHOLD = 8.0f;
 
 template <bool BF16>
 __device__ __forceinline__ float16_t mfma_32x32x16(uint4_t a, uint4_t b, float16_t c) {
@@ -64,25 +66,39 @@ template <bool BF16> __device__ __forceinline__ uint32_t pack2(float lo, float h
     }
 }
 
-// Position of key `kv` (0..63) inside a V^T row.  The second MFMA contracts over
-// keys in the order the score accumulator hands them out: slot j of k-step ks in
-// lane group g holds key ks*16 + (j/4)*8 + g*4 + j%4, so V^T stores key
-// ks*16 + h*8 + g*4 + jj at position ks*16 + g*8 + h*4 + jj.
-__device__ __forceinline__ int vt_pos_of_group(int r /* kv / 4 */) {
-    const int ks = r >> 2, h = (r >> 1) & 1, g = r & 1;
-    return (ks * 4 + g * 2 + h) * 4;
+// acc + lo + hi of a packed pair, one v_dot2c instruction
+template <bool BF16> __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+    if constexpr (BF16) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, packed), __builtin_bit_cast(bf16x2_t, 0x3F803F80u), acc, false);
+    } else {
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, packed), __builtin_bit_cast(half2_t, 0x3C003C00u), acc, false);
+    }
 }
 
-template <bool BF16, int D>
+// LDS transpose read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane i
+// receives element (i & 3) of the 8-byte rows addressed by lanes (i >> 2) + 4*j,
+// j = 0..3.  Addressed as below, lane i of a group ends up with 4 consecutive keys
+// of ONE head dimension although V sits in LDS in its natural [key][dim] layout.
+__device__ __forceinline__ uint2_t lds_read_tr16(const uint16_t *p) {
+    typedef short short4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+    short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)(p));
+    return __builtin_bit_cast(uint2_t, v);
+}
+
+template <bool BF16, int D, bool HAS_MASK>
 __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
-    constexpr int KS_STRIDE = D + 8;  // K row stride in elements (272 B at D=128: rows shift by 4 banks)
-    constexpr int KT = D / 16;        // k-steps of the first product
-    constexpr int DT = D / 32;        // 32-row tiles of O^T
-    constexpr int KCH = D / 8;        // 16-byte chunks per K/V row
-    constexpr int KV_CHUNKS = BN * KCH / 256; // 16-byte K chunks per thread per tile (4 at D=128)
-    constexpr int KLD = KV_CHUNKS > 0 ? KV_CHUNKS : 1;
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KS_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[D * VT_STRIDE];
+    constexpr int KS_STRIDE = D + 8;   // K row stride (elements): +16 B shifts consecutive rows by 4 banks
+    constexpr int VS_STRIDE = D + 32;  // V row stride: +64 B shifts rows by 16 banks, what the 4-row transpose reads need
+    constexpr int KT = D / 16;         // k-steps of the first product
+    constexpr int DT = D / 32;         // 32-row tiles of O^T
+    constexpr int KCH = D / 8;         // 16-byte chunks per K/V row
+    constexpr int NLD = BN * KCH / 256 > 0 ? BN * KCH / 256 : 1; // 16-byte chunks per thread per tile
+    constexpr int ROWS_PER_PASS = 256 / KCH; // rows covered by one chunk pass of the whole workgroup
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][BN * KS_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[2][BN * VS_STRIDE];
 
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
@@ -109,12 +125,23 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
     const uint16_t *K = static_cast<const uint16_t *>(a.k) + b * a.ks[0] + h * a.ks[1];
     const uint16_t *V = static_cast<const uint16_t *>(a.v) + b * a.vs[0] + h * a.vs[1];
     uint16_t *O = static_cast<uint16_t *>(a.o) + b * a.os[0] + h * a.os[1];
-    const uint8_t *M = a.mask ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
+    const uint8_t *M = HAS_MASK ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
 
     const int q0 = qb * BM;
     const int qw0 = q0 + wave * 32; // first query row of this wave
     const int q = qw0 + ql;
     const bool q_ok = q < a.Sq;
+
+    // K / V are fetched through buffer descriptors: rows past the end of the
+    // sequence read as zero instead of touching memory.
+    const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(K), 0, a.Skv > 0 ? (a.Skv - 1) * krow_bytes + D * 2 : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(V), 0, a.Skv > 0 ? (a.Skv - 1) * vrow_bytes + D * 2 : 0, 0x00020000);
+    const int ld_row = tid / KCH, ld_cc = tid % KCH; // this thread's chunk in pass 0
+    const bool ld_active = KCH * BN >= 256 || tid < KCH * BN;
+    const int k_voff = ld_row * krow_bytes + ld_cc * 16, v_voff = ld_row * vrow_bytes + ld_cc * 16;
 
     // Q^T fragments (B operand): lane holds Q[q][16t + 8g .. +8]
     uint4_t qf[KT];
@@ -129,147 +156,142 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
-    float m_run = NEG_INF_F; // running max, scaled log2 domain
+    float m_run = NEG_INF_F; // reference maximum of the exponentials (scaled log2 domain); may lag the true maximum
     float l_run = 0.0f;      // this lane's share of the running denominator
 
     int kv_end = a.Skv;
     if (a.causal) kv_end = min(a.Skv, q0 + BM);
     const int ntiles = (kv_end + BN - 1) / BN;
 
-    // staging registers for the next K / V tile
-    uint4_t kreg[KLD], vreg[4];
-    // K: chunk id = tid + 256*n -> row id / KCH, chunk id % KCH
-    // V: thread owns keys 4r..4r+3 x dims 8c..8c+7
-    // (lane bits 0-1 pick the dim chunk, bits 2-4 the key group: 32 consecutive
-    // lanes then hit 32 distinct 8-byte bank pairs when writing V^T)
-    constexpr int CHB = D == 128 ? 2 : D == 64 ? 1 : 0; // bits of the high part of the dim-chunk index
-    const int v_c = ((tid >> 5) & ((1 << CHB) - 1)) * 4 + (tid & 3);
-    const int v_r = ((tid >> (5 + CHB)) & 1) * 8 + ((tid >> 2) & 7);
-    const bool v_active = tid < 2 * D;
-
+    uint4_t kreg[NLD], vreg[NLD];
     auto load_tile = [&](int tile) {
-        const int kv0 = tile * BN;
 #pragma unroll
-        for (int n = 0; n < KLD; ++n) {
-            const int id = tid + 256 * n;
-            const int row = id / KCH, cc = id % KCH;
+        for (int n = 0; n < NLD; ++n) {
+            // the whole offset rides in the vector operand: only that one is bounds-checked
+            const int row0 = tile * BN + n * ROWS_PER_PASS;
             kreg[n] = uint4_t{0, 0, 0, 0};
-            if (id < BN * KCH && kv0 + row < a.Skv)
-                kreg[n] = *reinterpret_cast<const uint4_t *>(K + static_cast<int64_t>(kv0 + row) * a.ks[2] + 8 * cc);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            vreg[j] = uint4_t{0, 0, 0, 0};
-            const int row = kv0 + 4 * v_r + j;
-            if (v_active && row < a.Skv)
-                vreg[j] = *reinterpret_cast<const uint4_t *>(V + static_cast<int64_t>(row) * a.vs[2] + 8 * v_c);
+            vreg[n] = uint4_t{0, 0, 0, 0};
+            if (ld_active) {
+                kreg[n] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, k_voff + row0 * krow_bytes, 0, 0);
+                vreg[n] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, v_voff + row0 * vrow_bytes, 0, 0);
+            }
         }
     };
-
-    auto stage_tile = [&]() {
+    auto stage_tile = [&](int buf) {
+        if (ld_active) {
 #pragma unroll
-        for (int n = 0; n < KLD; ++n) {
-            const int id = tid + 256 * n;
-            const int row = id / KCH, cc = id % KCH;
-            if (id < BN * KCH) *reinterpret_cast<uint4_t *>(&Ks[row * KS_STRIDE + 8 * cc]) = kreg[n];
-        }
-        if (v_active) {
-            const int pos = vt_pos_of_group(v_r);
-            const uint32_t r0[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
-            const uint32_t r1[4] = {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w};
-            const uint32_t r2[4] = {vreg[2].x, vreg[2].y, vreg[2].z, vreg[2].w};
-            const uint32_t r3[4] = {vreg[3].x, vreg[3].y, vreg[3].z, vreg[3].w};
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                // even dim 8c+2m: low halves; odd dim 8c+2m+1: high halves
-                uint2_t ev = {__builtin_amdgcn_perm(r1[m], r0[m], 0x05040100u), __builtin_amdgcn_perm(r3[m], r2[m], 0x05040100u)};
-                uint2_t od = {__builtin_amdgcn_perm(r1[m], r0[m], 0x07060302u), __builtin_amdgcn_perm(r3[m], r2[m], 0x07060302u)};
-                *reinterpret_cast<uint2_t *>(&Vt[(8 * v_c + 2 * m) * VT_STRIDE + pos]) = ev;
-                *reinterpret_cast<uint2_t *>(&Vt[(8 * v_c + 2 * m + 1) * VT_STRIDE + pos]) = od;
+            for (int n = 0; n < NLD; ++n) {
+                const int row = ld_row + n * ROWS_PER_PASS;
+                *reinterpret_cast<uint4_t *>(&Ks[buf][row * KS_STRIDE + 8 * ld_cc]) = kreg[n];
+                *reinterpret_cast<uint4_t *>(&Vs[buf][row * VS_STRIDE + 8 * ld_cc]) = vreg[n];
             }
         }
     };
 
-    if (ntiles > 0) load_tile(0);
+    // per-lane element offsets of the LDS fragment reads
+    const int k_frag = ql * KS_STRIDE + 8 * g;                                         // + kt*32*KS_STRIDE + 16*t
+    const int v_frag = (g * 4 + ((lane & 15) >> 2)) * VS_STRIDE + ((lane >> 4) & 1) * 16 + 4 * (lane & 3); // + ks*16*VS_STRIDE + dt*32
+
+    // ntiles >= 1: the host never launches this kernel with an empty key sequence.
+    // The prologue is deliberately unconditional and ends in an explicit vmcnt(0)
+    // (Q and tile 0 have landed by then anyway): with that the compiler's in-loop
+    // waits cover only the tile they need, not the prefetch issued just before.
+    load_tile(0);
+    stage_tile(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    if (ntiles > 1) load_tile(1);
+    __syncthreads();
 
     for (int tile = 0; tile < ntiles; ++tile) {
         const int kv0 = tile * BN;
-        __syncthreads(); // all waves are done reading the previous tile
-        stage_tile();
-        __syncthreads();
-        if (tile + 1 < ntiles) load_tile(tile + 1);
+        const int buf = tile & 1;
+        // registers hold tile+1: park it in the other buffer (every wave left that
+        // buffer at the barrier that closed the previous iteration), then start on tile+2
+        if (tile + 1 < ntiles) stage_tile(buf ^ 1);
+        if (tile + 2 < ntiles) load_tile(tile + 2);
 
         // a wave whose last query row precedes this tile has nothing to add
-        if (a.causal && kv0 > qw0 + 31) continue;
+        if (!(a.causal && kv0 > qw0 + 31)) {
+            const uint16_t *Kb = Ks[buf], *Vb = Vs[buf];
 
-        // ---- S^T = K Q^T : two 32-key sub-tiles
-        float16_t s[2];
+            // ---- S^T = K Q^T : two 32-key sub-tiles
+            float16_t s[2];
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
+            for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+                for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
 #pragma unroll
-            for (int t = 0; t < KT; ++t) {
-                const uint4_t kf = *reinterpret_cast<const uint4_t *>(&Ks[(kt * 32 + ql) * KS_STRIDE + 16 * t + 8 * g]);
-                s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+                for (int t = 0; t < KT; ++t) {
+                    const uint4_t kf = *reinterpret_cast<const uint4_t *>(&Kb[k_frag + kt * 32 * KS_STRIDE + 16 * t]);
+                    s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+                }
             }
-        }
 
-        // ---- masking: only tiles that touch the diagonal, the key tail or an explicit mask
-        const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || M != nullptr;
-        if (need_mask) {
+            // ---- masking: only tiles that touch the diagonal, the key tail or an explicit mask
+            const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
+            if (need_mask) {
+                const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1; // last visible key of this row
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                        bool dead = kv > kv_limit;
+                        if constexpr (HAS_MASK) {
+                            if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                        }
+                        if (dead) s[kt][i] = NEG_INF_F;
+                    }
+            }
+
+            // ---- online softmax (per lane: one query column, 32 of the 64 keys)
+            float mloc = NEG_INF_F;
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
-                    bool dead = kv >= a.Skv || (a.causal && kv > q);
-                    if (M != nullptr && q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
-                    if (dead) s[kt][i] = NEG_INF_F;
+                for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+            const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
+            // rescale only when some row's maximum outgrew its reference by the threshold
+            // (-inf - -inf = NaN compares false: a row with no visible key yet keeps -inf)
+            if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
+                const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+            }
+            const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
+            uint4_t pf[4]; // P^T fragments (B operand), one per 16-key k-step
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                uint32_t w[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * i], a.scale_log2e, -m_use));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * i + 1], a.scale_log2e, -m_use));
+                    w[i] = pack2<BF16>(p0, p1);
+                    l_run = add_pair<BF16>(w[i], l_run); // the denominator sums exactly what the MFMA multiplies
+                }
+                pf[2 * kt] = uint4_t{w[0], w[1], w[2], w[3]};
+                pf[2 * kt + 1] = uint4_t{w[4], w[5], w[6], w[7]};
+            }
+
+            // ---- O^T += V^T P^T, V^T fragments through the LDS transpose read
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const uint16_t *p = &Vb[v_frag + ks * 16 * VS_STRIDE + dt * 32];
+                    const uint2_t lo = lds_read_tr16(p);
+                    const uint2_t hi = lds_read_tr16(p + 8 * VS_STRIDE);
+                    const uint4_t vf = {lo.x, lo.y, hi.x, hi.y};
+                    oacc[dt] = mfma_32x32x16<BF16>(vf, pf[ks], oacc[dt]);
                 }
         }
-
-        // ---- online softmax (per lane: one query column, 32 of the 64 keys)
-        float mloc = NEG_INF_F;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-        const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
-        const float m_use = m_new == NEG_INF_F ? 0.0f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        m_run = m_new;
-        float lsum = 0.0f;
-        uint4_t pf[4]; // P^T fragments (B operand), one per 16-key k-step
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            float p[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], a.scale_log2e, -m_use));
-                lsum += p[i];
-            }
-            pf[2 * kt] = uint4_t{pack2<BF16>(p[0], p[1]), pack2<BF16>(p[2], p[3]), pack2<BF16>(p[4], p[5]), pack2<BF16>(p[6], p[7])};
-            pf[2 * kt + 1] = uint4_t{pack2<BF16>(p[8], p[9]), pack2<BF16>(p[10], p[11]), pack2<BF16>(p[12], p[13]), pack2<BF16>(p[14], p[15])};
-        }
-        l_run = l_run * alpha + lsum;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const uint16_t *p = &Vt[(dt * 32 + ql) * VT_STRIDE + ks * 16 + g * 8];
-                const uint2_t lo = *reinterpret_cast<const uint2_t *>(p);
-                const uint2_t hi = *reinterpret_cast<const uint2_t *>(p + 4);
-                const uint4_t vf = {lo.x, lo.y, hi.x, hi.y};
-                oacc[dt] = mfma_32x32x16<BF16>(vf, pf[ks], oacc[dt]);
-            }
+        __syncthreads();
     }
 
     // ---- epilogue: O = O^T / l, written as 4 consecutive dims (8 bytes) per store
@@ -405,6 +427,9 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
         // 16-byte vector access to every row of q/k/v, 8-byte to o
         for (int i = 0; i < 3; ++i)
             ok = ok && p.q_strides[i] % 8 == 0 && p.k_strides[i] % 8 == 0 && p.v_strides[i] % 8 == 0 && p.o_strides[i] % 4 == 0;
+        // K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice
+        const int64_t span = (static_cast<int64_t>(p.seq_kv) + 64) * std::max(p.k_strides[2], p.v_strides[2]) * 2;
+        ok = ok && span < (int64_t(1) << 31);
         ok = ok && (!q || aligned16(q)) && (!k || aligned16(k)) && (!v || aligned16(v)) && (!o || aligned16(o));
         if (ok) return SdpaKind::MFMA;
     }
@@ -425,7 +450,8 @@ int validate(const AxhipSdpaParams &p) {
 
 template <bool BF16, int D> void launch_mfma(const SdpaArgs &a, hipStream_t s) {
     const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
-    hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D>), dim3(grid), dim3(256), 0, s, a);
+    if (a.mask) hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, true>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, false>), dim3(grid), dim3(256), 0, s, a);
 }
 
 } // namespace
@@ -456,6 +482,17 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
     if (rc) return rc;
     const SdpaKind kind = pick_kernel(p, q, k, v, o);
     if (kind == SdpaKind::EMPTY) return AXHIP_OK;
+    if (p.seq_kv == 0) { // no key at all: every row is "fully masked" -> zeros
+        AXHIP_REQUIRE(o != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: NULL tensor");
+        for (int b = 0; b < p.batch; ++b)
+            for (int h = 0; h < p.heads; ++h)
+                for (int sq = 0; sq < p.seq_q; ++sq) {
+                    char *row = static_cast<char *>(o) + (b * p.o_strides[0] + h * p.o_strides[1] + sq * p.o_strides[2]) * dtype_size(p.dtype);
+                    int rc0 = axhip_fill(row, p.dtype, 0.0, p.head_dim, stream);
+                    if (rc0) return rc0;
+                }
+        return AXHIP_OK;
+    }
     AXHIP_REQUIRE(kind != SdpaKind::INVALID, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: head_dim %d > %d is not supported", p.head_dim, GMAXD);
     AXHIP_REQUIRE(q && k && v && o, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: NULL tensor");
     AXHIP_REQUIRE(static_cast<int64_t>(p.batch) * p.heads < 65536 || kind == SdpaKind::MFMA, AXHIP_ERR_UNSUPPORTED,
