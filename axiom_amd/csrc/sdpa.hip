@@ -311,6 +311,252 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
     }
 }
 
+// ------------------------------------------------- MFMA kernel, head_dim 128
+// Same tiling as sdpa_mfma_kernel, restructured for throughput:
+//  * K and V tiles go HBM -> LDS directly (buffer_load ... lds), no staging
+//    registers and no ds_write; rows sit unpadded (256 B) in LDS with the 16-byte
+//    chunk index XOR-swizzled by the row, which keeps both the K fragment reads
+//    (16 consecutive rows, one chunk) and the V transpose reads (4 rows x 64 B)
+//    free of bank conflicts.
+//  * software pipeline: while the softmax of tile j runs on the VALU, the score
+//    MFMAs of tile j+1 are already in flight, so one wave keeps both pipes busy.
+//    K therefore runs one tile ahead of V in LDS.
+
+typedef int int4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int swizzle_d128(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+// One 16-byte element per lane from a buffer straight into LDS: lane i's data lands at
+// lds_base + 16*i.  Out-of-range lanes (voffset beyond the descriptor) write zeros.
+__device__ __forceinline__ void load_to_lds_16(const int4_t &rsrc, uint32_t lds_base_uniform, int voffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(lds_base_uniform), "v"(voffset), "s"(rsrc) : "memory");
+}
+
+__device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
+    const uint64_t pa = reinterpret_cast<uint64_t>(base);
+    return int4_t{static_cast<int>(static_cast<uint32_t>(pa)), static_cast<int>(static_cast<uint32_t>(pa >> 32) & 0xFFFFu), bytes, 0x00020000};
+}
+
+template <bool BF16, bool HAS_MASK>
+__global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a) {
+    constexpr int D = 128, KT = 8, DT = 4;
+    constexpr int ROWB = 256;            // bytes per LDS row
+    constexpr int TILEB = BN * ROWB;     // 16 KiB per K or V tile
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILEB]; // K0 K1 V0 V1
+
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int ql = lane % 32, g = lane / 32;
+
+    const int L = blockIdx.x;
+    const int BH = a.B * a.H;
+    int bh, qb;
+    if (BH % 8 == 0) { // one (batch, head) per XCD at a time: its K/V stay in that XCD's L2
+        const int xcd = L % 8, j = L / 8;
+        bh = (j / a.nqb) * 8 + xcd;
+        qb = j % a.nqb;
+    } else {
+        bh = L / a.nqb;
+        qb = L % a.nqb;
+    }
+    if (a.causal) qb = a.nqb - 1 - qb; // heaviest blocks first
+    const int b = bh / a.H, h = bh % a.H;
+
+    const uint16_t *Q = static_cast<const uint16_t *>(a.q) + b * a.qs[0] + h * a.qs[1];
+    const uint16_t *K = static_cast<const uint16_t *>(a.k) + b * a.ks[0] + h * a.ks[1];
+    const uint16_t *V = static_cast<const uint16_t *>(a.v) + b * a.vs[0] + h * a.vs[1];
+    uint16_t *O = static_cast<uint16_t *>(a.o) + b * a.os[0] + h * a.os[1];
+    const uint8_t *M = HAS_MASK ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
+
+    const int q0 = qb * BM;
+    const int qw0 = q0 + wave * 32;
+    const int q = qw0 + ql;
+    const bool q_ok = q < a.Sq;
+
+    const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
+    const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + D * 2);
+    const int4_t vrsrc = make_rsrc(V, (a.Skv - 1) * vrow_bytes + D * 2);
+
+    // ---- HBM -> LDS mapping.  A wave-wide load moves 4 rows; load n of wave w covers
+    // tile rows 16n + 4w + (lane >> 4); the lane fetches the chunk that belongs at
+    // position (lane & 15) of the swizzled row.
+    const int ld_r = 4 * wave + (lane >> 4);
+    const int ld_c = (lane & 15) ^ swizzle_d128(ld_r);
+    const int k_voff = ld_r * krow_bytes + ld_c * 16, v_voff = ld_r * vrow_bytes + ld_c * 16;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)); // LDS addresses fit 32 bits
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 4 * wave * ROWB);
+    auto load_k = [&](int tile, int buf) {
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+            load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * 16 * ROWB, k_voff + (tile * BN + 16 * n) * krow_bytes);
+    };
+    auto load_v = [&](int tile, int buf) {
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+            load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * 16 * ROWB, v_voff + (tile * BN + 16 * n) * vrow_bytes);
+    };
+
+    // ---- LDS fragment offsets (bytes)
+    int k_off[KT]; // K fragment of k-step t: row ql (+32 per sub-tile), chunk 2t+g
+#pragma unroll
+    for (int t = 0; t < KT; ++t) k_off[t] = ql * ROWB + (((2 * t + g) ^ swizzle_d128(ql)) * 16);
+    int v_off[2][DT]; // V transpose read: rows g*4 + s2 (+8), dims dt*32 + (lane & 31)
+    {
+        const int s2 = (lane & 15) >> 2, cl = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1), half = lane & 1;
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                v_off[hi][dt] = (g * 4 + s2 + 8 * hi) * ROWB + ((((dt ^ s2) << 2) | (cl ^ (g + 2 * hi))) * 16) + half * 8;
+    }
+
+    uint4_t qf[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+        qf[t] = uint4_t{0, 0, 0, 0};
+        if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
+    }
+
+    float16_t oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
+    float m_run = NEG_INF_F, l_run = 0.0f;
+
+    int kv_end = a.Skv;
+    if (a.causal) kv_end = min(a.Skv, q0 + BM);
+    const int ntiles = (kv_end + BN - 1) / BN; // >= 1
+
+    // S^T = K Q^T for one tile (two 32-key sub-tiles)
+    auto scores = [&](const unsigned char *Kb, float16_t (&s)[2]) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < KT; ++t) {
+                const uint4_t kf = *reinterpret_cast<const uint4_t *>(Kb + kt * 32 * ROWB + k_off[t]);
+                s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+            }
+        }
+    };
+
+    // masking + running maximum + (rare) rescale for tile j
+    auto prepare = [&](int kv0, float16_t (&s)[2]) {
+        const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
+        if (need_mask) {
+            const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                    bool dead = kv > kv_limit;
+                    if constexpr (HAS_MASK) {
+                        if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                    }
+                    if (dead) s[kt][i] = NEG_INF_F;
+                }
+        }
+        float mloc = NEG_INF_F;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+        const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
+        if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
+            const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+        }
+    };
+
+    // P = exp2(S*c - m), packed; O^T += V^T P^T
+    auto softmax_pv = [&](const unsigned char *Vb, const float16_t (&s)[2]) {
+        const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
+        uint4_t pf[4];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            uint32_t w[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * i], a.scale_log2e, -m_use));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * i + 1], a.scale_log2e, -m_use));
+                w[i] = pack2<BF16>(p0, p1);
+                l_run = add_pair<BF16>(w[i], l_run);
+            }
+            pf[2 * kt] = uint4_t{w[0], w[1], w[2], w[3]};
+            pf[2 * kt + 1] = uint4_t{w[4], w[5], w[6], w[7]};
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint2_t lo = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[0][dt]));
+                const uint2_t hi = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[1][dt]));
+                const uint4_t vf = {lo.x, lo.y, hi.x, hi.y};
+                oacc[dt] = mfma_32x32x16<BF16>(vf, pf[ks], oacc[dt]);
+            }
+    };
+
+    // ---- prologue: K(0), V(0), K(1) in flight; first score tile
+    load_k(0, 0);
+    load_v(0, 0);
+    if (ntiles > 1) load_k(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): Q fragments and this wave's share of the tiles
+    __syncthreads();
+    float16_t sA[2], sB[2];
+    scores(lds, sA);
+    __syncthreads(); // every wave is done with K buffer 0 before K(2) lands in it
+
+    // One pipeline step: tile j is in `cur` (scores already computed), tile j+1's scores go to `nxt`.
+    auto step = [&](int j, float16_t (&cur)[2], float16_t (&nxt)[2]) {
+        const int kv0 = j * BN;
+        if (j + 2 < ntiles) load_k(j + 2, j & 1);
+        if (j + 1 < ntiles) load_v(j + 1, (j + 1) & 1);
+        const bool active = !(a.causal && kv0 > qw0 + 31);
+        const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
+        const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
+        if (active) {
+            prepare(kv0, cur);
+            // The next tile's scores are issued unconditionally so that they share a
+            // basic block with this tile's softmax and the scheduler can interleave
+            // the two; after the last tile (or the last tile this wave needs) they are
+            // computed from a stale K buffer and never used: ~1.5 % extra MFMA work.
+            scores(Kn, nxt);
+            softmax_pv(Vb, cur);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's async loads have landed
+        __syncthreads();
+    };
+    for (int j = 0; j < ntiles; j += 2) {
+        step(j, sA, sB);
+        if (j + 1 < ntiles) step(j + 1, sB, sA);
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (q_ok) {
+        uint16_t *orow = O + static_cast<int64_t>(q) * a.os[2];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int d = dt * 32 + i4 * 8 + g * 4;
+                uint2_t w = {pack2<BF16>(oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv),
+                             pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
+                *reinterpret_cast<uint2_t *>(orow + d) = w;
+            }
+    }
+}
+
 // ------------------------------------------------------------- generic kernel
 // 256 threads = 16 query rows x 16 lanes.  K/V tiles of 32 keys are widened to
 // fp32 in LDS.  Lane c of a row computes scores for keys c, c+16 and output dims
@@ -515,10 +761,16 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         a.nqb = (p.seq_q + BM - 1) / BM;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
+        const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
         switch (p.head_dim) {
         case 32: bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
         case 64: bf ? launch_mfma<true, 64>(a, s) : launch_mfma<false, 64>(a, s); break;
-        default: bf ? launch_mfma<true, 128>(a, s) : launch_mfma<false, 128>(a, s); break;
+        default:
+            if (bf && mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, true>), dim3(grid), dim3(256), 0, s, a);
+            else if (bf) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, false>), dim3(grid), dim3(256), 0, s, a);
+            else if (mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, true>), dim3(grid), dim3(256), 0, s, a);
+            else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, false>), dim3(grid), dim3(256), 0, s, a);
+            break;
         }
     } else {
         a.nqb = (p.seq_q + GM - 1) / GM;
