@@ -429,7 +429,26 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
     if (a.causal) kv_end = min(a.Skv, q0 + BM);
     const int ntiles = (kv_end + BN - 1) / BN; // >= 1
 
-    // S^T = K Q^T for one tile (two 32-key sub-tiles)
+    // v_maximum3_f32: NaN-propagating maximum, which (unlike maxnum) needs no input canonicalisation
+    auto max3 = [](float x, float y, float z) { return __builtin_elementwise_maximum(__builtin_elementwise_maximum(x, y), z); };
+    // exchange between the two half-waves that share a query column
+    auto max_across_halves = [&](float x) {
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        return __builtin_elementwise_maximum(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    };
+    // row maximum of a score tile, as four short chains instead of one long one
+    auto row_max = [&](const float16_t (&s)[2]) {
+        float m0 = max3(s[0][0], s[0][1], s[0][2]), m1 = max3(s[0][8], s[0][9], s[0][10]);
+        float m2 = max3(s[1][0], s[1][1], s[1][2]), m3 = max3(s[1][8], s[1][9], s[1][10]);
+        m0 = max3(m0, s[0][3], s[0][4]); m1 = max3(m1, s[0][11], s[0][12]);
+        m2 = max3(m2, s[1][3], s[1][4]); m3 = max3(m3, s[1][11], s[1][12]);
+        m0 = max3(m0, s[0][5], s[0][6]); m1 = max3(m1, s[0][13], s[0][14]);
+        m2 = max3(m2, s[1][5], s[1][6]); m3 = max3(m3, s[1][13], s[1][14]);
+        m0 = max3(m0, s[0][7], m1); m2 = max3(m2, s[1][7], m3);
+        return max_across_halves(max3(m0, s[0][15], __builtin_elementwise_maximum(m2, s[1][15])));
+    };
+
+    // S^T = K Q^T for one tile (two 32-key sub-tiles); prologue only
     auto scores = [&](const unsigned char *Kb, float16_t (&s)[2]) {
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
@@ -443,30 +462,26 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         }
     };
 
-    // masking + running maximum + (rare) rescale for tile j
-    auto prepare = [&](int kv0, float16_t (&s)[2]) {
-        const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
-        if (need_mask) {
-            const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
-                    bool dead = kv > kv_limit;
-                    if constexpr (HAS_MASK) {
-                        if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
-                    }
-                    if (dead) s[kt][i] = NEG_INF_F;
-                }
-        }
-        float mloc = NEG_INF_F;
+    // Key masking of tile j (diagonal, key tail, explicit mask), then the row maximum.
+    auto mask_and_max = [&](int kv0, float16_t (&s)[2]) {
+        const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-        const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
+            for (int i = 0; i < 16; ++i) {
+                const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                bool dead = kv > kv_limit;
+                if constexpr (HAS_MASK) {
+                    if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                }
+                if (dead) s[kt][i] = NEG_INF_F;
+            }
+        return row_max(s);
+    };
+
+    // Running maximum and the (rare) rescale of the accumulators.
+    auto update_max = [&](float mloc) {
+        const float m_new = __builtin_elementwise_maximum(m_run, mloc * a.scale_log2e);
         if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
             const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
             m_run = m_new;
@@ -478,32 +493,66 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         }
     };
 
-    // P = exp2(S*c - m), packed; O^T += V^T P^T
-    auto softmax_pv = [&](const unsigned char *Vb, const float16_t (&s)[2]) {
+    // The fused step body, hand-scheduled in 32 slots, one MFMA each:
+    //   slots  0..15  score MFMAs of the NEXT tile (K fragments from Kn)
+    //   slots 16..31  O^T += V^T P^T of the CURRENT tile (V fragments from Vb)
+    // LDS fragment reads run PF slots ahead of their MFMA.  The VALU work of the current
+    // tile's softmax (fma, exp2, pack, row sum) is dealt out 2 exponentials per slot over
+    // 12 of the first 16 slots and slots 16..19, always ahead of the P fragment that the
+    // PV MFMAs need; the row maximum of the next tile fills slots 20..28.  A scheduling
+    // barrier closes every slot so the compiler keeps this order.
+    auto fused = [&](const unsigned char *Kn, const unsigned char *Vb, const float16_t (&cur)[2], float16_t (&nxt)[2], float &mx_next) {
+        constexpr int PF = 3, RING = 4;
         const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
-        uint4_t pf[4];
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            uint32_t w[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * i], a.scale_log2e, -m_use));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * i + 1], a.scale_log2e, -m_use));
-                w[i] = pack2<BF16>(p0, p1);
-                l_run = add_pair<BF16>(w[i], l_run);
-            }
-            pf[2 * kt] = uint4_t{w[0], w[1], w[2], w[3]};
-            pf[2 * kt + 1] = uint4_t{w[4], w[5], w[6], w[7]};
-        }
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
+        uint4_t fr[RING];
+        uint32_t w[16];
+        float pm[4];
+        auto read_frag = [&](int m) {
+            if (m < 16) {
+                fr[m % RING] = *reinterpret_cast<const uint4_t *>(Kn + (m / 8) * 32 * ROWB + k_off[m % 8]);
+            } else {
+                const int ks = (m - 16) / 4, dt = (m - 16) % 4;
                 const uint2_t lo = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[0][dt]));
                 const uint2_t hi = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[1][dt]));
-                const uint4_t vf = {lo.x, lo.y, hi.x, hi.y};
-                oacc[dt] = mfma_32x32x16<BF16>(vf, pf[ks], oacc[dt]);
+                fr[m % RING] = uint4_t{lo.x, lo.y, hi.x, hi.y};
             }
+        };
+        auto exp_pair = [&](int pr) { // elements 2*pr, 2*pr+1 of the current tile
+            const int kt = pr / 8, i = (pr % 8) * 2;
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i], a.scale_log2e, -m_use));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i + 1], a.scale_log2e, -m_use));
+            w[pr] = pack2<BF16>(p0, p1);
+            l_run = add_pair<BF16>(w[pr], l_run);
+        };
+#pragma unroll
+        for (int m = 0; m < PF; ++m) read_frag(m);
+#pragma unroll
+        for (int m = 0; m < 32; ++m) {
+            if (m + PF < 32) read_frag(m + PF);
+            if (m < 16) {
+                if (m % 8 == 0) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) nxt[m / 8][i] = 0.0f;
+                }
+                nxt[m / 8] = mfma_32x32x16<BF16>(fr[m % RING], qf[m % 8], nxt[m / 8]);
+                if (m % 4 != 3) exp_pair((m / 4) * 3 + m % 4);
+            } else {
+                const int ks = (m - 16) / 4, dt = (m - 16) % 4;
+                const uint4_t pf = {w[4 * ks], w[4 * ks + 1], w[4 * ks + 2], w[4 * ks + 3]};
+                oacc[dt] = mfma_32x32x16<BF16>(fr[m % RING], pf, oacc[dt]);
+                if (m < 20) exp_pair(12 + (m - 16));
+                if (m >= 20 && m < 28) { // two partial maxima per slot over the next tile's 32 scores
+                    const int c = m - 20, kt = c / 4, i0 = (c % 4) * 4;
+                    if (c % 4 < 2) {
+                        pm[kt * 2 + c % 4] = max3(max3(nxt[kt][i0], nxt[kt][i0 + 1], nxt[kt][i0 + 2]), nxt[kt][i0 + 3], NEG_INF_F);
+                    } else {
+                        pm[kt * 2 + c % 4 - 2] = max3(max3(pm[kt * 2 + c % 4 - 2], nxt[kt][i0], nxt[kt][i0 + 1]), nxt[kt][i0 + 2], nxt[kt][i0 + 3]);
+                    }
+                }
+                if (m == 28) mx_next = max_across_halves(max3(max3(pm[0], pm[1], pm[2]), pm[3], NEG_INF_F));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
     // ---- prologue: K(0), V(0), K(1) in flight; first score tile
@@ -514,10 +563,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
     __syncthreads();
     float16_t sA[2], sB[2];
     scores(lds, sA);
+    float mxA = row_max(sA), mxB = NEG_INF_F; // unmasked row maxima, valid when the tile needs no masking
     __syncthreads(); // every wave is done with K buffer 0 before K(2) lands in it
 
     // One pipeline step: tile j is in `cur` (scores already computed), tile j+1's scores go to `nxt`.
-    auto step = [&](int j, float16_t (&cur)[2], float16_t (&nxt)[2]) {
+    auto step = [&](int j, float16_t (&cur)[2], float mx_cur, float16_t (&nxt)[2], float &mx_nxt) {
         const int kv0 = j * BN;
         if (j + 2 < ntiles) load_k(j + 2, j & 1);
         if (j + 1 < ntiles) load_v(j + 1, (j + 1) & 1);
@@ -525,20 +575,21 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
         const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
         if (active) {
-            prepare(kv0, cur);
-            // The next tile's scores are issued unconditionally so that they share a
-            // basic block with this tile's softmax and the scheduler can interleave
-            // the two; after the last tile (or the last tile this wave needs) they are
-            // computed from a stale K buffer and never used: ~1.5 % extra MFMA work.
-            scores(Kn, nxt);
-            softmax_pv(Vb, cur);
+            const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
+            float mloc = mx_cur;
+            if (need_mask) mloc = mask_and_max(kv0, cur);
+            update_max(mloc);
+            // The next tile's scores are issued unconditionally so that they share a basic
+            // block with this tile's softmax; after the last tile (or the last one this wave
+            // needs) they come from a stale K buffer and are never used: ~1.5 % extra MFMAs.
+            fused(Kn, Vb, cur, nxt, mx_nxt);
         }
         __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's async loads have landed
         __syncthreads();
     };
     for (int j = 0; j < ntiles; j += 2) {
-        step(j, sA, sB);
-        if (j + 1 < ntiles) step(j + 1, sB, sA);
+        step(j, sA, mxA, sB, mxB);
+        if (j + 1 < ntiles) step(j + 1, sB, mxB, sA, mxA);
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
