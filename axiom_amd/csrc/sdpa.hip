@@ -349,30 +349,31 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int ql = lane % 32, g = lane / 32;
 
+    // Work-group -> (batch*head, query block(s)).  Under a causal mask query block i needs
+    // i+1 key blocks, so a work-group takes the pair (i, nqb-1-i): every work-group then
+    // carries the same load and the launch has no ragged tail.  Work-groups are dealt to
+    // the 8 XCDs round-robin by id; one (batch, head) stays on one XCD so that its K/V
+    // live in that XCD's L2.
     const int L = blockIdx.x;
     const int BH = a.B * a.H;
-    int bh, qb;
-    if (BH % 8 == 0) { // one (batch, head) per XCD at a time: its K/V stay in that XCD's L2
+    const int per_bh = a.causal ? (a.nqb + 1) / 2 : a.nqb; // work-groups per (batch, head)
+    int bh, slot;
+    if (BH % 8 == 0) {
         const int xcd = L % 8, j = L / 8;
-        bh = (j / a.nqb) * 8 + xcd;
-        qb = j % a.nqb;
+        bh = (j / per_bh) * 8 + xcd;
+        slot = j % per_bh;
     } else {
-        bh = L / a.nqb;
-        qb = L % a.nqb;
+        bh = L / per_bh;
+        slot = L % per_bh;
     }
-    if (a.causal) qb = a.nqb - 1 - qb; // heaviest blocks first
     const int b = bh / a.H, h = bh % a.H;
+    const int npass = (a.causal && slot != a.nqb - 1 - slot) ? 2 : 1;
 
     const uint16_t *Q = static_cast<const uint16_t *>(a.q) + b * a.qs[0] + h * a.qs[1];
     const uint16_t *K = static_cast<const uint16_t *>(a.k) + b * a.ks[0] + h * a.ks[1];
     const uint16_t *V = static_cast<const uint16_t *>(a.v) + b * a.vs[0] + h * a.vs[1];
     uint16_t *O = static_cast<uint16_t *>(a.o) + b * a.os[0] + h * a.os[1];
     const uint8_t *M = HAS_MASK ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
-
-    const int q0 = qb * BM;
-    const int qw0 = q0 + wave * 32;
-    const int q = qw0 + ql;
-    const bool q_ok = q < a.Sq;
 
     const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
     const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + D * 2);
@@ -411,200 +412,209 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
                 v_off[hi][dt] = (g * 4 + s2 + 8 * hi) * ROWB + ((((dt ^ s2) << 2) | (cl ^ (g + 2 * hi))) * 16) + half * 8;
     }
 
-    uint4_t qf[KT];
-#pragma unroll
-    for (int t = 0; t < KT; ++t) {
-        qf[t] = uint4_t{0, 0, 0, 0};
-        if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
-    }
+    for (int pass = 0; pass < npass; ++pass) {
+        // heavier block of the pair first
+        const int qb = a.causal ? (pass == 0 ? a.nqb - 1 - slot : slot) : slot;
+        const int q0 = qb * BM;
+        const int qw0 = q0 + wave * 32; // first query row of this wave
+        const int q = qw0 + ql;
+        const bool q_ok = q < a.Sq;
 
-    float16_t oacc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
-    float m_run = NEG_INF_F, l_run = 0.0f;
-
-    int kv_end = a.Skv;
-    if (a.causal) kv_end = min(a.Skv, q0 + BM);
-    const int ntiles = (kv_end + BN - 1) / BN; // >= 1
-
-    // v_maximum3_f32: NaN-propagating maximum, which (unlike maxnum) needs no input canonicalisation
-    auto max3 = [](float x, float y, float z) { return __builtin_elementwise_maximum(__builtin_elementwise_maximum(x, y), z); };
-    // exchange between the two half-waves that share a query column
-    auto max_across_halves = [&](float x) {
-        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-        return __builtin_elementwise_maximum(__uint_as_float(r[0]), __uint_as_float(r[1]));
-    };
-    // row maximum of a score tile, as four short chains instead of one long one
-    auto row_max = [&](const float16_t (&s)[2]) {
-        float m0 = max3(s[0][0], s[0][1], s[0][2]), m1 = max3(s[0][8], s[0][9], s[0][10]);
-        float m2 = max3(s[1][0], s[1][1], s[1][2]), m3 = max3(s[1][8], s[1][9], s[1][10]);
-        m0 = max3(m0, s[0][3], s[0][4]); m1 = max3(m1, s[0][11], s[0][12]);
-        m2 = max3(m2, s[1][3], s[1][4]); m3 = max3(m3, s[1][11], s[1][12]);
-        m0 = max3(m0, s[0][5], s[0][6]); m1 = max3(m1, s[0][13], s[0][14]);
-        m2 = max3(m2, s[1][5], s[1][6]); m3 = max3(m3, s[1][13], s[1][14]);
-        m0 = max3(m0, s[0][7], m1); m2 = max3(m2, s[1][7], m3);
-        return max_across_halves(max3(m0, s[0][15], __builtin_elementwise_maximum(m2, s[1][15])));
-    };
-
-    // S^T = K Q^T for one tile (two 32-key sub-tiles); prologue only
-    auto scores = [&](const unsigned char *Kb, float16_t (&s)[2]) {
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
-#pragma unroll
-            for (int t = 0; t < KT; ++t) {
-                const uint4_t kf = *reinterpret_cast<const uint4_t *>(Kb + kt * 32 * ROWB + k_off[t]);
-                s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
-            }
+        uint4_t qf[KT];
+    #pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            qf[t] = uint4_t{0, 0, 0, 0};
+            if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
         }
-    };
 
-    // Key masking of tile j (diagonal, key tail, explicit mask), then the row maximum.
-    auto mask_and_max = [&](int kv0, float16_t (&s)[2]) {
-        const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
-                bool dead = kv > kv_limit;
-                if constexpr (HAS_MASK) {
-                    if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
-                }
-                if (dead) s[kt][i] = NEG_INF_F;
-            }
-        return row_max(s);
-    };
-
-    // Running maximum and the (rare) rescale of the accumulators.
-    auto update_max = [&](float mloc) {
-        const float m_new = __builtin_elementwise_maximum(m_run, mloc * a.scale_log2e);
-        if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
-            const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-            l_run *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-        }
-    };
-
-    // The fused step body, hand-scheduled in 32 slots, one MFMA each:
-    //   slots  0..15  score MFMAs of the NEXT tile (K fragments from Kn)
-    //   slots 16..31  O^T += V^T P^T of the CURRENT tile (V fragments from Vb)
-    // LDS fragment reads run PF slots ahead of their MFMA.  The VALU work of the current
-    // tile's softmax (fma, exp2, pack, row sum) is dealt out 2 exponentials per slot over
-    // 12 of the first 16 slots and slots 16..19, always ahead of the P fragment that the
-    // PV MFMAs need; the row maximum of the next tile fills slots 20..28.  A scheduling
-    // barrier closes every slot so the compiler keeps this order.
-    auto fused = [&](const unsigned char *Kn, const unsigned char *Vb, const float16_t (&cur)[2], float16_t (&nxt)[2], float &mx_next) {
-        constexpr int PF = 3, RING = 4;
-        const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
-        uint4_t fr[RING];
-        uint32_t w[16];
-        float pm[4];
-        auto read_frag = [&](int m) {
-            if (m < 16) {
-                fr[m % RING] = *reinterpret_cast<const uint4_t *>(Kn + (m / 8) * 32 * ROWB + k_off[m % 8]);
-            } else {
-                const int ks = (m - 16) / 4, dt = (m - 16) % 4;
-                const uint2_t lo = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[0][dt]));
-                const uint2_t hi = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[1][dt]));
-                fr[m % RING] = uint4_t{lo.x, lo.y, hi.x, hi.y};
-            }
-        };
-        auto exp_pair = [&](int pr) { // elements 2*pr, 2*pr+1 of the current tile
-            const int kt = pr / 8, i = (pr % 8) * 2;
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i], a.scale_log2e, -m_use));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i + 1], a.scale_log2e, -m_use));
-            w[pr] = pack2<BF16>(p0, p1);
-            l_run = add_pair<BF16>(w[pr], l_run);
-        };
-#pragma unroll
-        for (int m = 0; m < PF; ++m) read_frag(m);
-#pragma unroll
-        for (int m = 0; m < 32; ++m) {
-            if (m + PF < 32) read_frag(m + PF);
-            if (m < 16) {
-                if (m % 8 == 0) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) nxt[m / 8][i] = 0.0f;
-                }
-                nxt[m / 8] = mfma_32x32x16<BF16>(fr[m % RING], qf[m % 8], nxt[m / 8]);
-                if (m % 4 != 3) exp_pair((m / 4) * 3 + m % 4);
-            } else {
-                const int ks = (m - 16) / 4, dt = (m - 16) % 4;
-                const uint4_t pf = {w[4 * ks], w[4 * ks + 1], w[4 * ks + 2], w[4 * ks + 3]};
-                oacc[dt] = mfma_32x32x16<BF16>(fr[m % RING], pf, oacc[dt]);
-                if (m < 20) exp_pair(12 + (m - 16));
-                if (m >= 20 && m < 28) { // two partial maxima per slot over the next tile's 32 scores
-                    const int c = m - 20, kt = c / 4, i0 = (c % 4) * 4;
-                    if (c % 4 < 2) {
-                        pm[kt * 2 + c % 4] = max3(max3(nxt[kt][i0], nxt[kt][i0 + 1], nxt[kt][i0 + 2]), nxt[kt][i0 + 3], NEG_INF_F);
-                    } else {
-                        pm[kt * 2 + c % 4 - 2] = max3(max3(pm[kt * 2 + c % 4 - 2], nxt[kt][i0], nxt[kt][i0 + 1]), nxt[kt][i0 + 2], nxt[kt][i0 + 3]);
-                    }
-                }
-                if (m == 28) mx_next = max_across_halves(max3(max3(pm[0], pm[1], pm[2]), pm[3], NEG_INF_F));
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // ---- prologue: K(0), V(0), K(1) in flight; first score tile
-    load_k(0, 0);
-    load_v(0, 0);
-    if (ntiles > 1) load_k(1, 1);
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): Q fragments and this wave's share of the tiles
-    __syncthreads();
-    float16_t sA[2], sB[2];
-    scores(lds, sA);
-    float mxA = row_max(sA), mxB = NEG_INF_F; // unmasked row maxima, valid when the tile needs no masking
-    __syncthreads(); // every wave is done with K buffer 0 before K(2) lands in it
-
-    // One pipeline step: tile j is in `cur` (scores already computed), tile j+1's scores go to `nxt`.
-    auto step = [&](int j, float16_t (&cur)[2], float mx_cur, float16_t (&nxt)[2], float &mx_nxt) {
-        const int kv0 = j * BN;
-        if (j + 2 < ntiles) load_k(j + 2, j & 1);
-        if (j + 1 < ntiles) load_v(j + 1, (j + 1) & 1);
-        const bool active = !(a.causal && kv0 > qw0 + 31);
-        const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
-        const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
-        if (active) {
-            const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
-            float mloc = mx_cur;
-            if (need_mask) mloc = mask_and_max(kv0, cur);
-            update_max(mloc);
-            // The next tile's scores are issued unconditionally so that they share a basic
-            // block with this tile's softmax; after the last tile (or the last one this wave
-            // needs) they come from a stale K buffer and are never used: ~1.5 % extra MFMAs.
-            fused(Kn, Vb, cur, nxt, mx_nxt);
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's async loads have landed
-        __syncthreads();
-    };
-    for (int j = 0; j < ntiles; j += 2) {
-        step(j, sA, mxA, sB, mxB);
-        if (j + 1 < ntiles) step(j + 1, sB, mxB, sA, mxA);
-    }
-
-    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
-    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    if (q_ok) {
-        uint16_t *orow = O + static_cast<int64_t>(q) * a.os[2];
-#pragma unroll
+        float16_t oacc[DT];
+    #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                const int d = dt * 32 + i4 * 8 + g * 4;
-                uint2_t w = {pack2<BF16>(oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv),
-                             pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
-                *reinterpret_cast<uint2_t *>(orow + d) = w;
+    #pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
+        float m_run = NEG_INF_F, l_run = 0.0f;
+
+        int kv_end = a.Skv;
+        if (a.causal) kv_end = min(a.Skv, q0 + BM);
+        const int ntiles = (kv_end + BN - 1) / BN; // >= 1
+
+        // v_maximum3_f32: NaN-propagating maximum, which (unlike maxnum) needs no input canonicalisation
+        auto max3 = [](float x, float y, float z) { return __builtin_elementwise_maximum(__builtin_elementwise_maximum(x, y), z); };
+        // exchange between the two half-waves that share a query column
+        auto max_across_halves = [&](float x) {
+            const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+            return __builtin_elementwise_maximum(__uint_as_float(r[0]), __uint_as_float(r[1]));
+        };
+        // row maximum of a score tile, as four short chains instead of one long one
+        auto row_max = [&](const float16_t (&s)[2]) {
+            float m0 = max3(s[0][0], s[0][1], s[0][2]), m1 = max3(s[0][8], s[0][9], s[0][10]);
+            float m2 = max3(s[1][0], s[1][1], s[1][2]), m3 = max3(s[1][8], s[1][9], s[1][10]);
+            m0 = max3(m0, s[0][3], s[0][4]); m1 = max3(m1, s[0][11], s[0][12]);
+            m2 = max3(m2, s[1][3], s[1][4]); m3 = max3(m3, s[1][11], s[1][12]);
+            m0 = max3(m0, s[0][5], s[0][6]); m1 = max3(m1, s[0][13], s[0][14]);
+            m2 = max3(m2, s[1][5], s[1][6]); m3 = max3(m3, s[1][13], s[1][14]);
+            m0 = max3(m0, s[0][7], m1); m2 = max3(m2, s[1][7], m3);
+            return max_across_halves(max3(m0, s[0][15], __builtin_elementwise_maximum(m2, s[1][15])));
+        };
+
+        // S^T = K Q^T for one tile (two 32-key sub-tiles); prologue only
+        auto scores = [&](const unsigned char *Kb, float16_t (&s)[2]) {
+    #pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+    #pragma unroll
+                for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+    #pragma unroll
+                for (int t = 0; t < KT; ++t) {
+                    const uint4_t kf = *reinterpret_cast<const uint4_t *>(Kb + kt * 32 * ROWB + k_off[t]);
+                    s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+                }
             }
+        };
+
+        // Key masking of tile j (diagonal, key tail, explicit mask), then the row maximum.
+        auto mask_and_max = [&](int kv0, float16_t (&s)[2]) {
+            const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
+    #pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+    #pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                    bool dead = kv > kv_limit;
+                    if constexpr (HAS_MASK) {
+                        if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                    }
+                    if (dead) s[kt][i] = NEG_INF_F;
+                }
+            return row_max(s);
+        };
+
+        // Running maximum and the (rare) rescale of the accumulators.
+        auto update_max = [&](float mloc) {
+            const float m_new = __builtin_elementwise_maximum(m_run, mloc * a.scale_log2e);
+            if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
+                const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
+    #pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+    #pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+            }
+        };
+
+        // The fused step body, hand-scheduled in 32 slots, one MFMA each:
+        //   slots  0..15  score MFMAs of the NEXT tile (K fragments from Kn)
+        //   slots 16..31  O^T += V^T P^T of the CURRENT tile (V fragments from Vb)
+        // LDS fragment reads run PF slots ahead of their MFMA.  The VALU work of the current
+        // tile's softmax (fma, exp2, pack, row sum) is dealt out 2 exponentials per slot over
+        // 12 of the first 16 slots and slots 16..19, always ahead of the P fragment that the
+        // PV MFMAs need; the row maximum of the next tile fills slots 20..28.  A scheduling
+        // barrier closes every slot so the compiler keeps this order.
+        auto fused = [&](const unsigned char *Kn, const unsigned char *Vb, const float16_t (&cur)[2], float16_t (&nxt)[2], float &mx_next) {
+            constexpr int PF = 3, RING = 4;
+            const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
+            uint4_t fr[RING];
+            uint32_t w[16];
+            float pm[4];
+            auto read_frag = [&](int m) {
+                if (m < 16) {
+                    fr[m % RING] = *reinterpret_cast<const uint4_t *>(Kn + (m / 8) * 32 * ROWB + k_off[m % 8]);
+                } else {
+                    const int ks = (m - 16) / 4, dt = (m - 16) % 4;
+                    const uint2_t lo = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[0][dt]));
+                    const uint2_t hi = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[1][dt]));
+                    fr[m % RING] = uint4_t{lo.x, lo.y, hi.x, hi.y};
+                }
+            };
+            auto exp_pair = [&](int pr) { // elements 2*pr, 2*pr+1 of the current tile
+                const int kt = pr / 8, i = (pr % 8) * 2;
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i], a.scale_log2e, -m_use));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i + 1], a.scale_log2e, -m_use));
+                w[pr] = pack2<BF16>(p0, p1);
+                l_run = add_pair<BF16>(w[pr], l_run);
+            };
+    #pragma unroll
+            for (int m = 0; m < PF; ++m) read_frag(m);
+    #pragma unroll
+            for (int m = 0; m < 32; ++m) {
+                if (m + PF < 32) read_frag(m + PF);
+                if (m < 16) {
+                    if (m % 8 == 0) {
+    #pragma unroll
+                        for (int i = 0; i < 16; ++i) nxt[m / 8][i] = 0.0f;
+                    }
+                    nxt[m / 8] = mfma_32x32x16<BF16>(fr[m % RING], qf[m % 8], nxt[m / 8]);
+                    if (m % 4 != 3) exp_pair((m / 4) * 3 + m % 4);
+                } else {
+                    const int ks = (m - 16) / 4, dt = (m - 16) % 4;
+                    const uint4_t pf = {w[4 * ks], w[4 * ks + 1], w[4 * ks + 2], w[4 * ks + 3]};
+                    oacc[dt] = mfma_32x32x16<BF16>(fr[m % RING], pf, oacc[dt]);
+                    if (m < 20) exp_pair(12 + (m - 16));
+                    if (m >= 20 && m < 28) { // two partial maxima per slot over the next tile's 32 scores
+                        const int c = m - 20, kt = c / 4, i0 = (c % 4) * 4;
+                        if (c % 4 < 2) {
+                            pm[kt * 2 + c % 4] = max3(max3(nxt[kt][i0], nxt[kt][i0 + 1], nxt[kt][i0 + 2]), nxt[kt][i0 + 3], NEG_INF_F);
+                        } else {
+                            pm[kt * 2 + c % 4 - 2] = max3(max3(pm[kt * 2 + c % 4 - 2], nxt[kt][i0], nxt[kt][i0 + 1]), nxt[kt][i0 + 2], nxt[kt][i0 + 3]);
+                        }
+                    }
+                    if (m == 28) mx_next = max_across_halves(max3(max3(pm[0], pm[1], pm[2]), pm[3], NEG_INF_F));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        // ---- prologue: K(0), V(0), K(1) in flight; first score tile
+        load_k(0, 0);
+        load_v(0, 0);
+        if (ntiles > 1) load_k(1, 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): Q fragments and this wave's share of the tiles
+        __syncthreads();
+        float16_t sA[2], sB[2];
+        scores(lds, sA);
+        float mxA = row_max(sA), mxB = NEG_INF_F; // unmasked row maxima, valid when the tile needs no masking
+        __syncthreads(); // every wave is done with K buffer 0 before K(2) lands in it
+
+        // One pipeline step: tile j is in `cur` (scores already computed), tile j+1's scores go to `nxt`.
+        auto step = [&](int j, float16_t (&cur)[2], float mx_cur, float16_t (&nxt)[2], float &mx_nxt) {
+            const int kv0 = j * BN;
+            if (j + 2 < ntiles) load_k(j + 2, j & 1);
+            if (j + 1 < ntiles) load_v(j + 1, (j + 1) & 1);
+            const bool active = !(a.causal && kv0 > qw0 + 31);
+            const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
+            const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
+            if (active) {
+                const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
+                float mloc = mx_cur;
+                if (need_mask) mloc = mask_and_max(kv0, cur);
+                update_max(mloc);
+                // The next tile's scores are issued unconditionally so that they share a basic
+                // block with this tile's softmax; after the last tile (or the last one this wave
+                // needs) they come from a stale K buffer and are never used: ~1.5 % extra MFMAs.
+                fused(Kn, Vb, cur, nxt, mx_nxt);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's async loads have landed
+            __syncthreads();
+        };
+        for (int j = 0; j < ntiles; j += 2) {
+            step(j, sA, mxA, sB, mxB);
+            if (j + 1 < ntiles) step(j + 1, sB, mxB, sA, mxA);
+        }
+
+        const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        if (q_ok) {
+            uint16_t *orow = O + static_cast<int64_t>(q) * a.os[2];
+    #pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+    #pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const int d = dt * 32 + i4 * 8 + g * 4;
+                    uint2_t w = {pack2<BF16>(oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv),
+                                 pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
+                    *reinterpret_cast<uint2_t *>(orow + d) = w;
+                }
+        }
     }
 }
 
@@ -812,15 +822,15 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         a.nqb = (p.seq_q + BM - 1) / BM;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
-        const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
+        const unsigned grid128 = static_cast<unsigned>(a.causal ? (a.nqb + 1) / 2 : a.nqb) * static_cast<unsigned>(a.B * a.H);
         switch (p.head_dim) {
         case 32: bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
         case 64: bf ? launch_mfma<true, 64>(a, s) : launch_mfma<false, 64>(a, s); break;
         default:
-            if (bf && mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, true>), dim3(grid), dim3(256), 0, s, a);
-            else if (bf) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, false>), dim3(grid), dim3(256), 0, s, a);
-            else if (mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, true>), dim3(grid), dim3(256), 0, s, a);
-            else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, false>), dim3(grid), dim3(256), 0, s, a);
+            if (bf && mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, true>), dim3(grid128), dim3(256), 0, s, a);
+            else if (bf) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, false>), dim3(grid128), dim3(256), 0, s, a);
+            else if (mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, true>), dim3(grid128), dim3(256), 0, s, a);
+            else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, false>), dim3(grid128), dim3(256), 0, s, a);
             break;
         }
     } else {
