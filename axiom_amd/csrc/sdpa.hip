@@ -21,6 +21,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 
 namespace axhip {
 
@@ -338,9 +339,13 @@ __device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
     return int4_t{static_cast<int>(static_cast<uint32_t>(pa)), static_cast<int>(static_cast<uint32_t>(pa >> 32) & 0xFFFFu), bytes, 0x00020000};
 }
 
-template <bool BF16, bool HAS_MASK>
-__global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a) {
+// NW waves per work-group (4: two work-groups share a CU; 8: one work-group per CU, each
+// K/V tile fetched once for 256 query rows instead of 128).
+template <bool BF16, bool HAS_MASK, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kernel(const SdpaArgs a) {
     constexpr int D = 128, KT = 8, DT = 4;
+    constexpr int BMW = 32 * NW;          // query rows per work-group
+    constexpr int NLOAD = 16 / NW;        // wave-wide loads per wave per tile (a tile is 16 of them)
     constexpr int ROWB = 256;            // bytes per LDS row
     constexpr int TILEB = BN * ROWB;     // 16 KiB per K or V tile
     __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILEB]; // K0 K1 V0 V1
@@ -356,7 +361,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
     // live in that XCD's L2.
     const int L = blockIdx.x;
     const int BH = a.B * a.H;
-    const int per_bh = a.causal ? (a.nqb + 1) / 2 : a.nqb; // work-groups per (batch, head)
+    const int nqb = (a.Sq + BMW - 1) / BMW;
+    const int per_bh = a.causal ? (nqb + 1) / 2 : nqb; // work-groups per (batch, head)
     int bh, slot;
     if (BH % 8 == 0) {
         const int xcd = L % 8, j = L / 8;
@@ -367,7 +373,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         slot = L % per_bh;
     }
     const int b = bh / a.H, h = bh % a.H;
-    const int npass = (a.causal && slot != a.nqb - 1 - slot) ? 2 : 1;
+    const int npass = (a.causal && slot != nqb - 1 - slot) ? 2 : 1;
 
     const uint16_t *Q = static_cast<const uint16_t *>(a.q) + b * a.qs[0] + h * a.qs[1];
     const uint16_t *K = static_cast<const uint16_t *>(a.k) + b * a.ks[0] + h * a.ks[1];
@@ -380,22 +386,27 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
     const int4_t vrsrc = make_rsrc(V, (a.Skv - 1) * vrow_bytes + D * 2);
 
     // ---- HBM -> LDS mapping.  A wave-wide load moves 4 rows; load n of wave w covers
-    // tile rows 16n + 4w + (lane >> 4); the lane fetches the chunk that belongs at
-    // position (lane & 15) of the swizzled row.
+    // tile rows 4*NW*n + 4w + (lane >> 4); the lane fetches the chunk that belongs at
+    // position (lane & 15) of the swizzled row (the swizzle only sees row & 15).
     const int ld_r = 4 * wave + (lane >> 4);
     const int ld_c = (lane & 15) ^ swizzle_d128(ld_r);
     const int k_voff = ld_r * krow_bytes + ld_c * 16, v_voff = ld_r * vrow_bytes + ld_c * 16;
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)); // LDS addresses fit 32 bits
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 4 * wave * ROWB);
+    // load n (0 .. NLOAD-1) of this wave's share of a K / V tile
+    auto load_k1 = [&](int tile, int buf, int n) {
+        load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * 4 * NW * ROWB, k_voff + (tile * BN + 4 * NW * n) * krow_bytes);
+    };
+    auto load_v1 = [&](int tile, int buf, int n) {
+        load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * 4 * NW * ROWB, v_voff + (tile * BN + 4 * NW * n) * vrow_bytes);
+    };
     auto load_k = [&](int tile, int buf) {
 #pragma unroll
-        for (int n = 0; n < 4; ++n)
-            load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * 16 * ROWB, k_voff + (tile * BN + 16 * n) * krow_bytes);
+        for (int n = 0; n < NLOAD; ++n) load_k1(tile, buf, n);
     };
     auto load_v = [&](int tile, int buf) {
 #pragma unroll
-        for (int n = 0; n < 4; ++n)
-            load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * 16 * ROWB, v_voff + (tile * BN + 16 * n) * vrow_bytes);
+        for (int n = 0; n < NLOAD; ++n) load_v1(tile, buf, n);
     };
 
     // ---- LDS fragment offsets (bytes)
@@ -414,8 +425,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
 
     for (int pass = 0; pass < npass; ++pass) {
         // heavier block of the pair first
-        const int qb = a.causal ? (pass == 0 ? a.nqb - 1 - slot : slot) : slot;
-        const int q0 = qb * BM;
+        const int qb = a.causal ? (pass == 0 ? nqb - 1 - slot : slot) : slot;
+        const int q0 = qb * BMW;
         const int qw0 = q0 + wave * 32; // first query row of this wave
         const int q = qw0 + ql;
         const bool q_ok = q < a.Sq;
@@ -435,7 +446,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         float m_run = NEG_INF_F, l_run = 0.0f;
 
         int kv_end = a.Skv;
-        if (a.causal) kv_end = min(a.Skv, q0 + BM);
+        if (a.causal) kv_end = min(a.Skv, q0 + BMW);
         const int ntiles = (kv_end + BN - 1) / BN; // >= 1
 
         // v_maximum3_f32: NaN-propagating maximum, which (unlike maxnum) needs no input canonicalisation
@@ -510,7 +521,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         // 12 of the first 16 slots and slots 16..19, always ahead of the P fragment that the
         // PV MFMAs need; the row maximum of the next tile fills slots 20..28.  A scheduling
         // barrier closes every slot so the compiler keeps this order.
-        auto fused = [&](const unsigned char *Kn, const unsigned char *Vb, const float16_t (&cur)[2], float16_t (&nxt)[2], float &mx_next) {
+        auto fused = [&](int j, const unsigned char *Kn, const unsigned char *Vb, const float16_t (&cur)[2], float16_t (&nxt)[2], float &mx_next) {
+            const bool want_k = j + 2 < ntiles, want_v = j + 1 < ntiles;
             constexpr int PF = 3, RING = 4;
             const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
             uint4_t fr[RING];
@@ -560,6 +572,13 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
                     }
                     if (m == 28) mx_next = max_across_halves(max3(max3(pm[0], pm[1], pm[2]), pm[3], NEG_INF_F));
                 }
+                // the tile prefetch is spread over the slots instead of bursting at the step start:
+                // K(j+2) in slots 1, 3, .., V(j+1) in slots 2, 4, ..
+                if (m % 2 == 1 && m / 2 < NLOAD) {
+                    if (want_k) load_k1(j + 2, j & 1, m / 2);
+                } else if (m % 2 == 0 && m >= 2 && m / 2 - 1 < NLOAD) {
+                    if (want_v) load_v1(j + 1, (j + 1) & 1, m / 2 - 1);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -578,8 +597,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
         // One pipeline step: tile j is in `cur` (scores already computed), tile j+1's scores go to `nxt`.
         auto step = [&](int j, float16_t (&cur)[2], float mx_cur, float16_t (&nxt)[2], float &mx_nxt) {
             const int kv0 = j * BN;
-            if (j + 2 < ntiles) load_k(j + 2, j & 1);
-            if (j + 1 < ntiles) load_v(j + 1, (j + 1) & 1);
             const bool active = !(a.causal && kv0 > qw0 + 31);
             const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
             const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
@@ -591,7 +608,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_d128_kernel(const SdpaArgs a
                 // The next tile's scores are issued unconditionally so that they share a basic
                 // block with this tile's softmax; after the last tile (or the last one this wave
                 // needs) they come from a stale K buffer and are never used: ~1.5 % extra MFMAs.
-                fused(Kn, Vb, cur, nxt, mx_nxt);
+                fused(j, Kn, Vb, cur, nxt, mx_nxt);
+            } else { // a wave with nothing to compute still fetches its share of the tiles
+                if (j + 2 < ntiles) load_k(j + 2, j & 1);
+                if (j + 1 < ntiles) load_v(j + 1, (j + 1) & 1);
             }
             __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's async loads have landed
             __syncthreads();
@@ -723,6 +743,12 @@ namespace {
 
 enum class SdpaKind { EMPTY, MFMA, GENERIC, INVALID };
 
+// 0 = automatic; 4 / 8 forces the work-group width of the head_dim-128 kernel (AXHIP_SDPA_D128_WAVES)
+int sdpa_d128_waves = [] {
+    const char *e = getenv("AXHIP_SDPA_D128_WAVES");
+    return e ? atoi(e) : 0;
+}();
+
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, const void *v, const void *o) {
@@ -767,6 +793,15 @@ template <bool BF16, int D> void launch_mfma(const SdpaArgs &a, hipStream_t s) {
 using namespace axhip;
 
 extern "C" {
+
+// diagnostic: resident work-groups per CU of the head_dim-128 bf16 kernel (waves = 4 or 8)
+int axhip_sdpa_d128_occupancy(int waves) {
+    int n = -1;
+    hipError_t e = waves == 8
+        ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 8>, 512, 0)
+        : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 4>, 256, 0);
+    return e == hipSuccess ? n : -static_cast<int>(e);
+}
 
 const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *p) {
     static thread_local char name[48];
@@ -822,15 +857,26 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         a.nqb = (p.seq_q + BM - 1) / BM;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
-        const unsigned grid128 = static_cast<unsigned>(a.causal ? (a.nqb + 1) / 2 : a.nqb) * static_cast<unsigned>(a.B * a.H);
         switch (p.head_dim) {
         case 32: bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
         case 64: bf ? launch_mfma<true, 64>(a, s) : launch_mfma<false, 64>(a, s); break;
-        default:
-            if (bf && mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, true>), dim3(grid128), dim3(256), 0, s, a);
-            else if (bf) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<true, false>), dim3(grid128), dim3(256), 0, s, a);
-            else if (mask) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, true>), dim3(grid128), dim3(256), 0, s, a);
-            else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<false, false>), dim3(grid128), dim3(256), 0, s, a);
+        default: {
+            // 8-wave work-groups (256 query rows) once there are enough rows to fill them
+            const bool wide = p.seq_q > 128 && sdpa_d128_waves != 4;
+            const int bmw = wide ? 256 : 128;
+            const int nqbw = (p.seq_q + bmw - 1) / bmw;
+            const unsigned g = static_cast<unsigned>(a.causal ? (nqbw + 1) / 2 : nqbw) * static_cast<unsigned>(a.B * a.H);
+#define AXHIP_LAUNCH_D128(BF, MK)                                                                                         \
+    do {                                                                                                                  \
+        if (wide) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 8>), dim3(g), dim3(512), 0, s, a);                    \
+        else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 4>), dim3(g), dim3(256), 0, s, a);                         \
+    } while (0)
+            if (bf && mask) AXHIP_LAUNCH_D128(true, true);
+            else if (bf) AXHIP_LAUNCH_D128(true, false);
+            else if (mask) AXHIP_LAUNCH_D128(false, true);
+            else AXHIP_LAUNCH_D128(false, false);
+#undef AXHIP_LAUNCH_D128
+        }
             break;
         }
     } else {
