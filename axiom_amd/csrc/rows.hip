@@ -8,104 +8,13 @@
 // which makes consecutive lanes touch consecutive 16/32-byte segments.
 // Reductions are wave64 shuffles plus one LDS hop when a row spans several waves.
 #include "common.hpp"
+#include "rows_ops.hpp"
+#include "rows_static.hpp"
 
 #include <algorithm>
 
 namespace axhip {
 
-constexpr float NEG_INF = -__builtin_huge_valf();
-constexpr float POS_INF = __builtin_huge_valf();
-
-__device__ __forceinline__ float apply_unary(int op, float a) {
-    switch (op) {
-    case AXHIP_OP_RELU: return a > 0.0f ? a : 0.0f;
-    case AXHIP_OP_GELU: return 0.5f * a * (1.0f + erff(a * 0.70710678118654752f));
-    case AXHIP_OP_SQRT: return sqrtf(a);
-    case AXHIP_OP_EXP: return expf(a);
-    case AXHIP_OP_NEG: return -a;
-    case AXHIP_OP_ABS: return fabsf(a);
-    case AXHIP_OP_SIGMOID: {
-        float e = expf(-fabsf(a)), d = 1.0f + e;
-        return a >= 0.0f ? 1.0f / d : e / d;
-    }
-    case AXHIP_OP_TANH: return tanhf(a);
-    case AXHIP_OP_SILU: return a / (1.0f + expf(-a));
-    case AXHIP_OP_LOG: return logf(a);
-    case AXHIP_OP_SQUARE: return a * a;
-    case AXHIP_OP_RSQRT: return 1.0f / sqrtf(a);
-    case AXHIP_OP_RECIP: return 1.0f / a;
-    default: return a;
-    }
-}
-
-__device__ __forceinline__ float apply_binary(int op, float a, float b) {
-    switch (op) {
-    case AXHIP_OP_ADD: return a + b;
-    case AXHIP_OP_SUB: return a - b;
-    case AXHIP_OP_MUL: return a * b;
-    case AXHIP_OP_DIV: return a / b;
-    case AXHIP_OP_MAX: return fmaxf(a, b);
-    case AXHIP_OP_MIN: return fminf(a, b);
-    case AXHIP_OP_RSUB: return b - a;
-    case AXHIP_OP_RDIV: return b / a;
-    default: return a;
-    }
-}
-
-__host__ __device__ inline bool is_binary_op(int op) { return op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV; }
-
-// Apply one chain op to a thread's register tile.  The op code is a kernel
-// argument, so the switch is a scalar (wave-uniform) branch taken once per op;
-// each arm is straight-line vector code over the whole tile.
-template <int IT, int E, typename F>
-__device__ __forceinline__ void for_each_value(float (&v)[IT][E], F f) {
-#pragma unroll
-    for (int it = 0; it < IT; ++it)
-#pragma unroll
-        for (int e = 0; e < E; ++e) v[it][e] = f(v[it][e], it, e);
-}
-
-template <int IT, int E>
-__device__ __forceinline__ void apply_unary_tile(int op, float (&v)[IT][E]) {
-#define AXHIP_UNARY_CASE(code) \
-    case code: for_each_value<IT, E>(v, [](float a, int, int) { return apply_unary(code, a); }); break
-    switch (op) {
-        AXHIP_UNARY_CASE(AXHIP_OP_RELU);
-        AXHIP_UNARY_CASE(AXHIP_OP_GELU);
-        AXHIP_UNARY_CASE(AXHIP_OP_SQRT);
-        AXHIP_UNARY_CASE(AXHIP_OP_EXP);
-        AXHIP_UNARY_CASE(AXHIP_OP_NEG);
-        AXHIP_UNARY_CASE(AXHIP_OP_ABS);
-        AXHIP_UNARY_CASE(AXHIP_OP_SIGMOID);
-        AXHIP_UNARY_CASE(AXHIP_OP_TANH);
-        AXHIP_UNARY_CASE(AXHIP_OP_SILU);
-        AXHIP_UNARY_CASE(AXHIP_OP_LOG);
-        AXHIP_UNARY_CASE(AXHIP_OP_SQUARE);
-        AXHIP_UNARY_CASE(AXHIP_OP_RSQRT);
-        AXHIP_UNARY_CASE(AXHIP_OP_RECIP);
-    default: break;
-    }
-#undef AXHIP_UNARY_CASE
-}
-
-// w(it, e) yields the second operand of element (it, e)
-template <int IT, int E, typename W>
-__device__ __forceinline__ void apply_binary_tile(int op, float (&v)[IT][E], W w) {
-#define AXHIP_BINARY_CASE(code) \
-    case code: for_each_value<IT, E>(v, [&](float a, int it, int e) { return apply_binary(code, a, w(it, e)); }); break
-    switch (op) {
-        AXHIP_BINARY_CASE(AXHIP_OP_ADD);
-        AXHIP_BINARY_CASE(AXHIP_OP_SUB);
-        AXHIP_BINARY_CASE(AXHIP_OP_MUL);
-        AXHIP_BINARY_CASE(AXHIP_OP_DIV);
-        AXHIP_BINARY_CASE(AXHIP_OP_MAX);
-        AXHIP_BINARY_CASE(AXHIP_OP_MIN);
-        AXHIP_BINARY_CASE(AXHIP_OP_RSUB);
-        AXHIP_BINARY_CASE(AXHIP_OP_RDIV);
-    default: break;
-    }
-#undef AXHIP_BINARY_CASE
-}
 
 // Loads the [IT][E] tile of a FULL or ROWVEC operand.
 template <int IT, int E>
@@ -635,6 +544,8 @@ extern "C" {
 const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *P) {
     static thread_local char name[64];
     if (!P) return "invalid";
+    if (validate_program(*P, "axhip_fused_rows_kernel_name") == AXHIP_OK && rows_static_dispatch(*P, nullptr, false, name, sizeof(name)))
+        return name;
     RowsPlan pl = plan_rows(*P);
     snprintf(name, sizeof(name), "%s", pl.name);
     return name;
@@ -651,6 +562,10 @@ int axhip_fused_rows(const AxhipRowsProgram *program, void *stream) {
     RowsPlan pl = plan_rows(P);
     if (pl.kind == RowsPlan::EMPTY) return AXHIP_OK;
     hipStream_t s = resolve_stream(stream);
+    if (rows_static_dispatch(P, s, true, nullptr, 0)) {
+        AXHIP_CHECK_HIP(hipGetLastError());
+        return AXHIP_OK;
+    }
     rc = pl.e == 8 ? launch_plan_e<8>(P, pl, s) : pl.e == 4 ? launch_plan_e<4>(P, pl, s) : launch_plan_e<1>(P, pl, s);
     if (rc) return rc;
     AXHIP_CHECK_HIP(hipGetLastError());
