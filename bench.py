@@ -29,6 +29,14 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch of the SDPA kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script, each scaled by the reading of the plain-copy leg below
+# (FETCH_SIZE 0.50013, WRITE_SIZE 1.0): 598.7 MB read + 134.2 MB written.
+SDPA_TRAFFIC_BYTES = 732.9e6
+# same measurement for the fused chains: they move the algorithmic bytes (ratio 1.001 - 1.003)
+CHAIN_TRAFFIC_BYTES = {"chain_relu_add_mul_softmax_sum_f32_8192x8192": 537.2e6,
+                       "chain_gelu_layernorm_bf16_16384x4096": 269.3e6,
+                       "chain_gelu_rmsnorm_bf16_16384x4096": 269.2e6}
 
 
 def time_launches(torch, stream, launch, steps: int, warmup: int):
@@ -115,7 +123,19 @@ def bench_chains(torch, capi, stream, steps, warmup):
         "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
         "rows_sum_to_one": bool(torch.allclose(out, torch.ones_like(out), atol=1e-4)),
     }
-    del a, b
+    # plain copy of the same matrix through the elementwise kernel (empty chain): the kernel of
+    # known traffic that the rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by
+    cp = torch.empty_like(a)
+    pc = _rows_program(capi, a, cp, capi.DTYPE_F32, capi.DTYPE_F32)
+    torch.cuda.synchronize()
+    avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(pc), sp)), steps, warmup)
+    nbytes = 2 * R * Cc * 4
+    res["copy_f32_8192x8192"] = {
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(pc)).decode(), "avg_ms": avg_ms, "min_ms": min_ms,
+        "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "bit_exact": bool(torch.equal(cp, a)),
+    }
+    del a, b, cp
 
     # configs[2]: gelu(layernorm(x)*gamma+beta) and the RMSNorm variant, bf16 [16384, 4096]
     R, Cc = 16384, 4096
@@ -220,11 +240,14 @@ def main() -> int:
     if sd:
         line["roofline"] = {
             "bound": "mfma", "kernel": "sdpa_" + sd["kernel"], "achieved": sd["tflops"], "peak": PEAK_BF16_TFLOPS,
-            "unit": "TFLOP/s", "frac": sd["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+            "unit": "TFLOP/s", "frac": sd["tflops"] / PEAK_BF16_TFLOPS, "traffic": SDPA_TRAFFIC_BYTES,
             "algorithmic_flops_per_launch": sd["flops"], "avg_launch_ms": sd["avg_ms"], "min_launch_ms": sd["min_ms"],
         }
         line["output_finite"] = sd["finite"]
     if ch:
+        for name, rec in ch.items():
+            if name in CHAIN_TRAFFIC_BYTES:
+                rec["traffic"] = CHAIN_TRAFFIC_BYTES[name]
         line["fused_chains"] = ch
     if cpu:
         line["cpu_baseline"] = cpu
