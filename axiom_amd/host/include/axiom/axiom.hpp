@@ -1,0 +1,16 @@
+// Umbrella header of the gfx950 host layer.
+#pragma once
+
+#include "axiom/dtype.hpp"
+#include "axiom/error.hpp"
+#include "axiom/graph/graph_cache.hpp"
+#include "axiom/graph/graph_node.hpp"
+#include "axiom/graph/graph_registry.hpp"
+#include "axiom/graph/graph_signature.hpp"
+#include "axiom/nn.hpp"
+#include "axiom/operations.hpp"
+#include "axiom/random.hpp"
+#include "axiom/shape.hpp"
+#include "axiom/storage.hpp"
+#include "axiom/system.hpp"
+#include "axiom/tensor.hpp"

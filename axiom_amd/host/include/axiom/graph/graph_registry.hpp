@@ -1,0 +1,73 @@
+// Lazy tensor creation and materialisation
+// (include/axiom/graph/graph_registry.hpp:23-154).
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "axiom/graph/graph_node.hpp"
+
+namespace axiom {
+class Tensor;
+
+namespace graph {
+
+bool is_eager_mode_enabled(); // AXIOM_EAGER_MODE=1 or an active EagerModeScope
+size_t get_max_pending_nodes();
+void set_max_pending_nodes(size_t max_nodes);
+
+Shape infer_binary_shape(const Shape &lhs, const Shape &rhs);
+Shape infer_reduction_shape(const Shape &input, const std::vector<int> &axes, bool keep_dims);
+Shape infer_matmul_shape(const Shape &a, const Shape &b, bool transpose_a, bool transpose_b);
+DType infer_binary_dtype(DType lhs, DType rhs);
+DType infer_unary_dtype(ops::OpType op, DType input);
+DType infer_reduction_dtype(ops::OpType op, DType input); // Mean of a non-f64 dtype is Float32
+
+class GraphRegistry {
+  public:
+    static Tensor create_lazy_unary(ops::OpType op, const Tensor &input, const OpParams &params = NoParams{});
+    static Tensor create_lazy_binary(ops::OpType op, const Tensor &lhs, const Tensor &rhs, const OpParams &params = NoParams{});
+    static Tensor create_lazy_reduction(ops::OpType op, const Tensor &input, const std::vector<int> &axes, bool keep_dims);
+    static Tensor create_lazy_matmul(const Tensor &a, const Tensor &b, bool transpose_a, bool transpose_b);
+    static Tensor create_lazy_softmax(ops::OpType op, const Tensor &input, int axis);
+    static Tensor create_lazy_layernorm(const Tensor &input, const Tensor &weight, const Tensor &bias, int axis, float eps);
+    // RMS norm is captured lazily too, so that rms_norm + activation is one kernel
+    static Tensor create_lazy_rmsnorm(const Tensor &input, const Tensor &weight, int axis, float eps);
+    static Tensor create_lazy_reshape(const Tensor &input, const Shape &new_shape);
+    static Tensor create_lazy_transpose(const Tensor &input, const std::vector<int> &axes);
+
+    // signature -> plan cache -> compile -> execute; GPU graphs go to materialize_gpu_graph
+    static void materialize(GraphNode *node);
+    static size_t pending_node_count();
+    static void materialize_all();
+    static Tensor finalize_lazy_node(std::shared_ptr<GraphNode> node);
+
+  private:
+    static thread_local std::vector<std::weak_ptr<GraphNode>> pending_nodes_;
+};
+
+class EagerModeScope {
+  public:
+    EagerModeScope();
+    ~EagerModeScope();
+    EagerModeScope(const EagerModeScope &) = delete;
+    EagerModeScope &operator=(const EagerModeScope &) = delete;
+
+  private:
+    bool previous_mode_;
+};
+
+// The GPU hook of GraphRegistry::materialize (src/graph/graph_registry.cpp:834-850;
+// Metal counterpart src/backends/metal/mpsgraph_graph_compiler.mm:706-944): turns the DAG
+// under `root` into fused row programs, GEMMs and copies of libaxhip, runs them on the
+// backend stream and leaves the result in root->cached_result_ / cached_shape_ /
+// cached_strides_ with is_materialized_ set.
+void materialize_gpu_graph(GraphNode *root);
+
+// kernels launched by the last materialize_gpu_graph on this thread, in order
+// (e.g. "rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"); for tests and AXIOM_DEBUG_FUSION
+const std::vector<std::string> &last_gpu_plan_kernels();
+
+} // namespace graph
+} // namespace axiom

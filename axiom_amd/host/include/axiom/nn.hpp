@@ -1,0 +1,93 @@
+// nn modules on the attention / norm path (include/axiom/nn/{module,linear,
+// normalization,attention,activation}.hpp; src/nn/*.cpp).  Inference only.
+#pragma once
+
+#include <map>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "axiom/tensor.hpp"
+
+namespace axiom::nn {
+
+class Module {
+  public:
+    Module() = default;
+    virtual ~Module() = default;
+    Module(const Module &) = delete;
+    Module &operator=(const Module &) = delete;
+
+    virtual Tensor forward(const Tensor &input) const;
+    virtual Module &to(Device device);
+    virtual Module &to(DType dtype);
+    // parameters are looked up as prefix + name; submodules add "name." (src/nn/module.cpp:36-50)
+    virtual void load_state_dict(const std::map<std::string, Tensor> &state_dict, const std::string &prefix = "", bool strict = true);
+    std::map<std::string, Tensor> state_dict(const std::string &prefix = "") const;
+    std::vector<std::pair<std::string, Tensor *>> named_parameters(const std::string &prefix = "") const; // insertion order
+    std::vector<Tensor *> parameters() const;
+
+  protected:
+    void register_parameter(const std::string &name, Tensor &param);
+    void register_module(const std::string &name, Module &submodule);
+
+  private:
+    std::vector<std::pair<std::string, Tensor *>> params_;
+    std::vector<std::pair<std::string, Module *>> submodules_;
+};
+
+// y = x W^T + b, weight (out_features, in_features) (src/nn/linear.cpp:15-27)
+class Linear : public Module {
+  public:
+    explicit Linear(bool bias = true);
+    Tensor forward(const Tensor &input) const override;
+    bool has_bias() const { return has_bias_; }
+
+  private:
+    Tensor weight_, bias_;
+    bool has_bias_;
+};
+
+class LayerNorm : public Module {
+  public:
+    explicit LayerNorm(float eps = 1e-5f);
+    Tensor forward(const Tensor &input) const override;
+
+  private:
+    Tensor weight_, bias_;
+    float eps_;
+};
+
+class RMSNorm : public Module {
+  public:
+    explicit RMSNorm(float eps = 1e-5f);
+    Tensor forward(const Tensor &input) const override;
+
+  private:
+    Tensor weight_;
+    float eps_;
+};
+
+class ReLU : public Module {
+  public:
+    Tensor forward(const Tensor &input) const override;
+};
+class GELU : public Module {
+  public:
+    Tensor forward(const Tensor &input) const override;
+};
+
+// q/k/v/out projections + scaled_dot_product_attention over num_heads heads
+// (src/nn/attention.cpp:17-65).  Inputs (batch, seq, d_model).
+class MultiHeadAttention : public Module {
+  public:
+    explicit MultiHeadAttention(int num_heads, bool bias = true);
+    Tensor forward(const Tensor &query, const Tensor &key, const Tensor &value, const Tensor &mask = Tensor(), bool is_causal = false) const;
+    int num_heads() const { return num_heads_; }
+
+  private:
+    int num_heads_;
+    Linear q_proj_, k_proj_, v_proj_, out_proj_;
+};
+
+} // namespace axiom::nn

@@ -1,0 +1,100 @@
+// ops:: free functions for the GPU hot paths, same names and argument meaning
+// as Axiom's include/axiom/operations.hpp.  Every function needs its tensors
+// on Device::GPU: elementwise / softmax / norm / reduction / matmul calls build
+// lazy graph nodes (src/tensor/operations.cpp:660-669, 857-869, 930-959,
+// 1420-1435, 1775-1795); scaled_dot_product_attention runs eagerly
+// (operations.cpp:3979-4044).  CPU tensors throw RuntimeError: this library
+// carries no CPU compute path.
+#pragma once
+
+#include <vector>
+
+#include "axiom/dtype.hpp"
+
+namespace axiom {
+class Tensor;
+
+namespace ops {
+
+// Axiom's OpType (include/axiom/operations.hpp:55-208), same order and names.
+enum class OpType {
+    Add, Subtract, Multiply, Divide, Power, Modulo,
+    Equal, NotEqual, Less, LessEqual, Greater, GreaterEqual,
+    LogicalAnd, LogicalOr, LogicalXor, LogicalNot,
+    BitwiseAnd, BitwiseOr, BitwiseXor, LeftShift, RightShift,
+    Maximum, Minimum, Atan2, Hypot,
+    Negate, Abs, Sqrt, Exp, Log, Sin, Cos, Tan, Erf,
+    Sign, Floor, Ceil, Trunc, Round, Reciprocal, Square, Cbrt,
+    IsNaN, IsInf, IsFinite,
+    Conj, Real, Imag,
+    ReLU, LeakyReLU, SiLU, Sigmoid, Tanh, GELU, Softmax, LogSoftmax,
+    Sum, Mean, Max, Min, ArgMax, ArgMin, Any, All, Prod,
+    MatMul, BatchMatMul,
+    Where,
+    MaskedFill, MaskedSelect,
+    Gather, Scatter, IndexSelect, Take, TakeAlongAxis,
+    LayerNorm, RMSNorm,
+    Dropout,
+    Cast,
+    MaxPool1D, MaxPool2D, MaxPool3D, AvgPool1D, AvgPool2D, AvgPool3D, AdaptiveMaxPool2D, AdaptiveAvgPool2D,
+    Conv1D, Conv2D, ConvTranspose1D, ConvTranspose2D,
+    ScaledDotProductAttention,
+    Reshape, Transpose, Pad, Slice, Unsqueeze, Concat,
+    GLU, BatchNorm1D,
+    Sort, Argsort, TopK,
+    _Count
+};
+
+const char *op_name(OpType op);
+DType promote_types(DType lhs, DType rhs); // src/tensor/operations.cpp:346-397
+
+Tensor add(const Tensor &a, const Tensor &b);
+Tensor subtract(const Tensor &a, const Tensor &b);
+Tensor multiply(const Tensor &a, const Tensor &b);
+Tensor divide(const Tensor &a, const Tensor &b);
+Tensor maximum(const Tensor &a, const Tensor &b);
+Tensor minimum(const Tensor &a, const Tensor &b);
+
+Tensor negate(const Tensor &x);
+Tensor abs(const Tensor &x);
+Tensor sqrt(const Tensor &x);
+Tensor exp(const Tensor &x);
+Tensor log(const Tensor &x);
+Tensor reciprocal(const Tensor &x);
+Tensor square(const Tensor &x);
+Tensor relu(const Tensor &x);
+Tensor silu(const Tensor &x);
+Tensor sigmoid(const Tensor &x);
+Tensor tanh(const Tensor &x);
+Tensor gelu(const Tensor &x);
+
+Tensor softmax(const Tensor &x, int axis = -1);
+Tensor log_softmax(const Tensor &x, int axis = -1);
+
+Tensor sum(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+Tensor mean(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+Tensor max(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+Tensor min(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+
+// population variance, eps inside the square root; weight / bias may be empty tensors
+Tensor layer_norm(const Tensor &x, const Tensor &weight, const Tensor &bias, int axis = -1, float eps = 1e-5f);
+Tensor rms_norm(const Tensor &x, const Tensor &weight, int axis = -1, float eps = 1e-5f);
+
+Tensor matmul(const Tensor &a, const Tensor &b, bool transpose_a = false, bool transpose_b = false);
+
+// q (B,H,Sq,D), k/v (B,H,Skv,D); mask Bool (Sq,Skv) or (B,H,Sq,Skv), true = masked out;
+// scale <= 0 means 1/sqrt(D).  ShapeError on bad ranks / mismatched batch, heads, Skv or D.
+Tensor scaled_dot_product_attention(const Tensor &query, const Tensor &key, const Tensor &value, const Tensor &mask,
+                                    float scale = -1.0f, bool is_causal = false);
+
+namespace detail {
+// as above; with out_bshd the output is written head-merged, (B, Sq, H, D) in memory, and
+// returned as the (B, H, Sq, D) view of it, so MultiHeadAttention's merge needs no copy
+Tensor sdpa(const Tensor &query, const Tensor &key, const Tensor &value, const Tensor &mask, float scale, bool is_causal, bool out_bshd);
+} // namespace detail
+
+// name of the gfx950 kernel the last scaled_dot_product_attention call on this thread launched
+const char *last_sdpa_kernel();
+
+} // namespace ops
+} // namespace axiom

@@ -1,0 +1,648 @@
+// materialize_gpu_graph: the GPU hook of the lazy graph.  Cuts the DAG under a root
+// into launches of libaxhip -- fused row programs, full reductions, GEMMs with epilogue,
+// strided gathers -- and caches the resulting plan by graph signature.
+//
+// Contract (src/graph/graph_registry.cpp:834-850 and the Metal implementation
+// src/backends/metal/mpsgraph_graph_compiler.mm:706-944): on return the root holds its
+// result (cached_result_, cached_shape_, cached_strides_, is_materialized_), nodes that
+// other consumers share were materialised on the way, and the inputs of every
+// materialised node lost one reference.
+//
+// Fusion rule: walking down from a node through inputs that nobody else consumes,
+//     [row reduction] <- [elementwise chain] <- [softmax | log-softmax | layer norm | rms norm]
+//                     <- [elementwise chain] <- input
+// becomes ONE axhip_fused_rows launch; [full reduction] <- [elementwise chain] one
+// axhip_fused_full_reduce; [activation] <- [+ residual] <- [+ bias] <- matmul one
+// axhip_gemm.  Reshape and transpose are views; a view that a kernel cannot address
+// directly is gathered with axhip_strided_copy first.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+
+#include "axiom/error.hpp"
+#include "axiom/graph/graph_cache.hpp"
+#include "axiom/graph/graph_registry.hpp"
+#include "axiom/graph/graph_signature.hpp"
+#include "hip_call.hpp"
+
+namespace axiom::graph {
+
+namespace {
+
+using ops::OpType;
+
+// ---------------------------------------------------------------- plan types
+struct ValueSpec {
+    bool is_leaf = false;
+    int index = 0; // leaf index or temp index
+    Shape shape;
+    Strides strides; // bytes
+    DType dtype = DType::Float32;
+};
+
+struct RowsStep {
+    AxhipRowsProgram prog{}; // pointers filled at run time
+    int input = -1, output = -1;
+    int operand_value[AXHIP_MAX_OPERANDS] = {};
+    bool full_reduce = false;
+    int workspace = -1; // temp index of the full-reduce scratch
+};
+
+struct GemmStep {
+    AxhipGemmParams p{};
+    int a = -1, b = -1, c = -1, bias = -1, residual = -1;
+};
+
+struct CopyStep {
+    int src = -1, dst = -1;
+    Shape shape;         // iteration space
+    Strides src_strides; // bytes; 0 on broadcast dims
+};
+
+struct Step {
+    enum Kind { ROWS, GEMM, COPY } kind;
+    RowsStep rows;
+    GemmStep gemm;
+    CopyStep copy;
+};
+
+struct Plan {
+    std::vector<ValueSpec> values;
+    std::vector<size_t> temp_bytes;
+    std::vector<Step> steps;
+    std::vector<std::pair<int, int>> node_results; // (topological index of a node, value holding its result)
+    size_t n_leaves = 0;
+};
+
+bool is_leaf(const GraphNode *n, const GraphNode *root) { return n->is_constant || (n->is_materialized_ && n != root); }
+
+bool is_unary_ew(OpType op) {
+    switch (op) {
+    case OpType::Negate: case OpType::Abs: case OpType::Sqrt: case OpType::Exp: case OpType::Log: case OpType::Reciprocal:
+    case OpType::Square: case OpType::ReLU: case OpType::SiLU: case OpType::Sigmoid: case OpType::Tanh: case OpType::GELU:
+        return true;
+    default: return false;
+    }
+}
+bool is_binary_ew(OpType op) {
+    return op == OpType::Add || op == OpType::Subtract || op == OpType::Multiply || op == OpType::Divide || op == OpType::Maximum ||
+           op == OpType::Minimum;
+}
+bool is_elementwise(OpType op) { return is_unary_ew(op) || is_binary_ew(op); }
+bool is_row_op(OpType op) { return op == OpType::Softmax || op == OpType::LogSoftmax || op == OpType::LayerNorm || op == OpType::RMSNorm; }
+bool is_reduction(OpType op) { return op == OpType::Sum || op == OpType::Mean || op == OpType::Max || op == OpType::Min; }
+
+int unary_code(OpType op) {
+    switch (op) {
+    case OpType::Negate: return AXHIP_OP_NEG;
+    case OpType::Abs: return AXHIP_OP_ABS;
+    case OpType::Sqrt: return AXHIP_OP_SQRT;
+    case OpType::Exp: return AXHIP_OP_EXP;
+    case OpType::Log: return AXHIP_OP_LOG;
+    case OpType::Reciprocal: return AXHIP_OP_RECIP;
+    case OpType::Square: return AXHIP_OP_SQUARE;
+    case OpType::ReLU: return AXHIP_OP_RELU;
+    case OpType::SiLU: return AXHIP_OP_SILU;
+    case OpType::Sigmoid: return AXHIP_OP_SIGMOID;
+    case OpType::Tanh: return AXHIP_OP_TANH;
+    case OpType::GELU: return AXHIP_OP_GELU;
+    default: return 0;
+    }
+}
+// chain_is_rhs: the running value is the op's second operand
+int binary_code(OpType op, bool chain_is_rhs) {
+    switch (op) {
+    case OpType::Add: return AXHIP_OP_ADD;
+    case OpType::Multiply: return AXHIP_OP_MUL;
+    case OpType::Maximum: return AXHIP_OP_MAX;
+    case OpType::Minimum: return AXHIP_OP_MIN;
+    case OpType::Subtract: return chain_is_rhs ? AXHIP_OP_RSUB : AXHIP_OP_SUB;
+    case OpType::Divide: return chain_is_rhs ? AXHIP_OP_RDIV : AXHIP_OP_DIV;
+    default: return 0;
+    }
+}
+
+// ------------------------------------------------------------------ builder
+class PlanBuilder {
+  public:
+    PlanBuilder(const GraphNode *root, const std::vector<const GraphNode *> &topo) : root_(root) {
+        for (size_t i = 0; i < topo.size(); ++i) {
+            topo_index_[topo[i]] = static_cast<int>(i);
+            if (is_leaf(topo[i], root)) {
+                ValueSpec v;
+                v.is_leaf = true;
+                v.index = static_cast<int>(plan_.n_leaves++);
+                const GraphNode *n = topo[i];
+                v.shape = n->is_constant ? n->output_shape : n->cached_shape_;
+                v.strides = n->is_constant ? n->constant_strides : n->cached_strides_;
+                v.dtype = n->output_dtype;
+                memo_[n] = add_value(v);
+            }
+        }
+    }
+
+    Plan build() {
+        eval(root_);
+        return std::move(plan_);
+    }
+
+  private:
+    int add_value(const ValueSpec &v) {
+        plan_.values.push_back(v);
+        return static_cast<int>(plan_.values.size()) - 1;
+    }
+    int new_temp(const Shape &shape, DType dt) {
+        ValueSpec v;
+        v.index = static_cast<int>(plan_.temp_bytes.size());
+        v.shape = shape;
+        v.dtype = dt;
+        v.strides = ShapeUtils::contiguous_strides(shape, dtype_size(dt));
+        plan_.temp_bytes.push_back(std::max<size_t>(ShapeUtils::size(shape) * dtype_size(dt), 16));
+        return add_value(v);
+    }
+    const ValueSpec &val(int v) const { return plan_.values[v]; }
+    bool contiguous(int v) const { return ShapeUtils::is_contiguous(val(v).shape, val(v).strides, dtype_size(val(v).dtype)); }
+
+    // a contiguous value with the same contents (gathered if necessary), optionally broadcast to `to`
+    int make_contiguous(int v, const Shape *to = nullptr) {
+        const Shape target = to ? *to : val(v).shape;
+        if (target == val(v).shape && contiguous(v)) return v;
+        detail::to_axhip_dtype(val(v).dtype); // only kernel dtypes can be gathered on the device
+        const ValueSpec src = val(v);
+        const int out = new_temp(target, src.dtype);
+        Step s{};
+        s.kind = Step::COPY;
+        s.copy.src = v;
+        s.copy.dst = out;
+        s.copy.shape = target;
+        s.copy.src_strides.assign(target.size(), 0);
+        const size_t lead = target.size() - src.shape.size();
+        for (size_t i = 0; i < src.shape.size(); ++i) s.copy.src_strides[lead + i] = src.shape[i] == 1 ? 0 : src.strides[i];
+        if (target.size() > AXHIP_MAX_DIMS) throw RuntimeError::not_implemented("GPU gather of more than 8 dimensions");
+        for (int64_t st : s.copy.src_strides)
+            if (st < 0) throw RuntimeError::not_implemented("negative strides (flipped views)");
+        plan_.steps.push_back(s);
+        return out;
+    }
+
+    bool consumable(const GraphNode *c, const GraphNode *entry) const {
+        return !is_leaf(c, root_) && (c == entry || c->ref_count.load() <= 1) && !memo_.count(c);
+    }
+
+    int eval(const GraphNode *n) {
+        auto it = memo_.find(n);
+        if (it != memo_.end()) return it->second;
+        int v;
+        const OpType op = n->op_type;
+        if (op == OpType::Reshape) {
+            const int in = make_contiguous(eval(n->inputs[0].get()));
+            ValueSpec s = val(in);
+            s.shape = n->output_shape;
+            s.strides = ShapeUtils::contiguous_strides(s.shape, dtype_size(s.dtype));
+            v = add_value(s);
+        } else if (op == OpType::Transpose) {
+            const int in = eval(n->inputs[0].get());
+            const auto &axes = get_params<TransposeParams>(n->params).axes;
+            ValueSpec s = val(in);
+            for (size_t i = 0; i < axes.size(); ++i) {
+                s.shape[i] = val(in).shape[axes[i]];
+                s.strides[i] = val(in).strides[axes[i]];
+            }
+            v = add_value(s);
+        } else if (op == OpType::MatMul) {
+            v = emit_gemm(n, {}, -1, -1, 0);
+        } else if (is_elementwise(op) || is_row_op(op) || is_reduction(op)) {
+            v = emit_rows(n);
+        } else {
+            throw RuntimeError::not_implemented(std::string("GPU lazy graph node '") + ops::op_name(op) + "'");
+        }
+        memo_[n] = v;
+        if (n == root_ || n->ref_count.load() > 1) plan_.node_results.emplace_back(topo_index_.at(n), v);
+        return v;
+    }
+
+    struct ChainItem {
+        const GraphNode *node;
+        int primary; // input index the chain continues through
+    };
+
+    // Collects elementwise nodes downwards from `c` while each is consumable and keeps the full shape F.
+    void collect(const GraphNode *&c, const GraphNode *entry, const Shape &F, std::vector<ChainItem> &list, size_t limit, size_t &operands) {
+        while (consumable(c, entry) && is_elementwise(c->op_type) && c->output_shape == F && list.size() < limit) {
+            int primary = 0;
+            if (is_binary_ew(c->op_type)) {
+                const GraphNode *l = c->inputs[0].get(), *r = c->inputs[1].get();
+                const bool lf = l->output_shape == F, rf = r->output_shape == F;
+                if (!lf && !rf) break; // both operands broadcast: evaluated on its own (see emit_rows)
+                // continue through the operand that can still be fused; a leaf is the better memory operand
+                if (lf && rf) primary = (is_leaf(l, root_) && !is_leaf(r, root_)) ? 1 : 0;
+                else primary = lf ? 0 : 1;
+                if (operands + 1 > AXHIP_MAX_OPERANDS - 2) break; // keep room for norm weight / bias
+                ++operands;
+            }
+            list.push_back({c, primary});
+            c = c->inputs[primary].get();
+        }
+    }
+
+    // classifies / prepares the memory operand of a binary op against the full shape F = [rows..., cols]
+    void add_operand(RowsStep &rs, AxhipChainOp &cop, const GraphNode *operand, const Shape &F, bool chain_is_rhs, OpType op) {
+        int v = eval(operand);
+        const Shape S = val(v).shape;
+        const size_t numel = ShapeUtils::size(S), cols = F.empty() ? 1 : F.back();
+        int kind;
+        Shape stripped = S;
+        while (stripped.size() > 1 && stripped.front() == 1) stripped.erase(stripped.begin());
+        bool colvec = S.size() == F.size() && !S.empty() && S.back() == 1 && F.back() != 1;
+        for (size_t i = 0; colvec && i + 1 < S.size(); ++i) colvec = S[i] == F[i];
+        if (numel == 1) kind = AXHIP_BK_SCALAR;
+        else if (S == F) kind = AXHIP_BK_FULL;
+        else if (stripped.size() == 1 && stripped[0] == cols) kind = AXHIP_BK_ROWVEC;
+        else if (colvec) kind = AXHIP_BK_COLVEC;
+        else {
+            v = make_contiguous(v, &F); // general broadcast: expand once
+            kind = AXHIP_BK_FULL;
+        }
+        v = make_contiguous(v);
+        const int slot = rs.prog.n_operands++;
+        rs.prog.operands[slot].dtype = detail::to_axhip_dtype(val(v).dtype);
+        rs.prog.operands[slot].kind = kind;
+        rs.operand_value[slot] = v;
+        cop.op = binary_code(op, chain_is_rhs);
+        cop.operand = slot;
+        cop.imm = 0.0f;
+        cop.imm_kind = 0;
+    }
+
+    void fill_chain(RowsStep &rs, const std::vector<ChainItem> &bottom_up, AxhipChainOp *dst, int32_t &count, const Shape &F) {
+        for (const ChainItem &it : bottom_up) {
+            AxhipChainOp &cop = dst[count++];
+            if (is_unary_ew(it.node->op_type)) {
+                cop.op = unary_code(it.node->op_type);
+                cop.operand = -1;
+                cop.imm = 0.0f;
+                cop.imm_kind = 0;
+            } else {
+                add_operand(rs, cop, it.node->inputs[1 - it.primary].get(), F, it.primary == 1, it.node->op_type);
+            }
+        }
+    }
+
+    int emit_rows(const GraphNode *n) {
+        RowsStep rs;
+        rs.prog.norm_weight = rs.prog.norm_bias = -1;
+        const GraphNode *cur = n;
+        const GraphNode *entry = n;
+        Shape F = n->output_shape;
+
+        if (is_reduction(n->op_type)) {
+            const auto &rp = get_params<ReductionParams>(n->params);
+            const GraphNode *in = n->inputs[0].get();
+            F = in->output_shape;
+            const int nd = static_cast<int>(F.size());
+            std::vector<bool> red(nd, rp.axes.empty());
+            for (int a : rp.axes) red[ShapeUtils::normalize_axis(a, nd)] = true;
+            size_t n_red = 0, kept_elems = 1;
+            for (int i = 0; i < nd; ++i) {
+                n_red += red[i];
+                if (!red[i]) kept_elems *= F[i];
+            }
+            const bool all = n_red == static_cast<size_t>(nd) || kept_elems == 1;
+            const bool last_only = !all && n_red == 1 && red[nd - 1];
+            if (!all && !last_only) throw RuntimeError::not_implemented("GPU reduction over axes other than the last one (or all)");
+            rs.full_reduce = all;
+            rs.prog.reduce = n->op_type == OpType::Sum ? AXHIP_RED_SUM : n->op_type == OpType::Mean ? AXHIP_RED_MEAN
+                             : n->op_type == OpType::Max ? AXHIP_RED_MAX : AXHIP_RED_MIN;
+            cur = in;
+            entry = nullptr; // below the reduction only unshared nodes fuse
+        }
+
+        size_t operands = 0;
+        std::vector<ChainItem> upper, lower;
+        collect(cur, entry, F, upper, AXHIP_MAX_CHAIN, operands);
+        const GraphNode *rowop = nullptr;
+        if (!rs.full_reduce && consumable(cur, entry) && is_row_op(cur->op_type) && cur->output_shape == F) {
+            const int axis = cur->op_type == OpType::Softmax || cur->op_type == OpType::LogSoftmax ? get_params<ActivationParams>(cur->params).axis
+                                                                                                  : get_params<NormParams>(cur->params).axis;
+            if (ShapeUtils::normalize_axis(axis, static_cast<int>(F.size())) != static_cast<int>(F.size()) - 1)
+                throw RuntimeError::not_implemented("GPU softmax / norm over an axis other than the last one");
+            rowop = cur;
+            cur = cur->inputs[0].get();
+            collect(cur, nullptr, F, lower, AXHIP_MAX_CHAIN, operands);
+        } else if (upper.empty() && !is_reduction(n->op_type)) {
+            // an elementwise node whose two operands are both broadcast: expand the left one and chain through it
+            if (!is_binary_ew(n->op_type)) throw RuntimeError::not_implemented(std::string("GPU lazy graph node '") + ops::op_name(n->op_type) + "'");
+            upper.push_back({n, 0});
+            cur = n->inputs[0].get();
+        }
+
+        // MatMul feeding a short epilogue chain: one GEMM launch
+        if (!rowop && rs.prog.reduce == AXHIP_RED_NONE && consumable(cur, entry) && cur->op_type == OpType::MatMul && !upper.empty()) {
+            const int g = try_gemm_epilogue(n, cur, upper, F);
+            if (g >= 0) return g;
+        }
+
+        // the pre chain runs bottom-up: reverse the collected (top-down) lists
+        std::reverse(upper.begin(), upper.end());
+        std::reverse(lower.begin(), lower.end());
+        int in_v = eval(cur);
+        if (val(in_v).shape != F) in_v = make_contiguous(in_v, &F);
+        in_v = make_contiguous(in_v);
+        rs.input = in_v;
+        rs.prog.input_dtype = detail::to_axhip_dtype(val(in_v).dtype);
+        rs.prog.cols = F.empty() ? 1 : static_cast<int64_t>(F.back());
+        rs.prog.rows = static_cast<int64_t>(ShapeUtils::size(F)) / std::max<int64_t>(rs.prog.cols, 1);
+        if (ShapeUtils::size(F) == 0) rs.prog.rows = 0;
+
+        if (rowop) {
+            fill_chain(rs, lower, rs.prog.pre, rs.prog.n_pre, F);
+            switch (rowop->op_type) {
+            case OpType::Softmax: rs.prog.row_op = AXHIP_ROWOP_SOFTMAX; break;
+            case OpType::LogSoftmax: rs.prog.row_op = AXHIP_ROWOP_LOGSOFTMAX; break;
+            case OpType::LayerNorm: rs.prog.row_op = AXHIP_ROWOP_LAYERNORM; break;
+            default: rs.prog.row_op = AXHIP_ROWOP_RMSNORM; break;
+            }
+            if (rowop->op_type == OpType::LayerNorm || rowop->op_type == OpType::RMSNorm) {
+                rs.prog.eps = get_params<NormParams>(rowop->params).eps;
+                for (size_t i = 1; i < rowop->inputs.size(); ++i) {
+                    const int wv = make_contiguous(eval(rowop->inputs[i].get()));
+                    const int slot = rs.prog.n_operands++;
+                    rs.prog.operands[slot].dtype = detail::to_axhip_dtype(val(wv).dtype);
+                    rs.prog.operands[slot].kind = AXHIP_BK_ROWVEC;
+                    rs.operand_value[slot] = wv;
+                    (i == 1 ? rs.prog.norm_weight : rs.prog.norm_bias) = slot;
+                }
+            }
+            fill_chain(rs, upper, rs.prog.post, rs.prog.n_post, F);
+        } else {
+            fill_chain(rs, upper, rs.prog.pre, rs.prog.n_pre, F);
+        }
+
+        rs.output = new_temp(n->output_shape, n->output_dtype);
+        rs.prog.output_dtype = detail::to_axhip_dtype(n->output_dtype);
+        if (rs.full_reduce) {
+            rs.workspace = static_cast<int>(plan_.temp_bytes.size());
+            plan_.temp_bytes.push_back(axhip_full_reduce_workspace_bytes());
+        }
+        Step s{};
+        s.kind = Step::ROWS;
+        s.rows = rs;
+        plan_.steps.push_back(s);
+        return rs.output;
+    }
+
+    // [activation] <- [+ residual FULL] <- [+ bias ROWVEC] <- matmul, all in the GEMM's dtype
+    int try_gemm_epilogue(const GraphNode *n, const GraphNode *mm, const std::vector<ChainItem> &top_down, const Shape &F) {
+        std::vector<ChainItem> ops(top_down.rbegin(), top_down.rend()); // bottom-up
+        size_t i = 0;
+        const GraphNode *bias = nullptr, *residual = nullptr;
+        int act = 0;
+        const size_t N = F.back();
+        auto other = [](const ChainItem &c) { return c.node->inputs[1 - c.primary].get(); };
+        if (i < ops.size() && ops[i].node->op_type == OpType::Add) {
+            const Shape &s = other(ops[i])->output_shape;
+            Shape stripped = s;
+            while (stripped.size() > 1 && stripped.front() == 1) stripped.erase(stripped.begin());
+            if (stripped.size() == 1 && stripped[0] == N && other(ops[i])->output_dtype == mm->output_dtype) bias = other(ops[i++]);
+        }
+        if (i < ops.size() && ops[i].node->op_type == OpType::Add && other(ops[i])->output_shape == F && other(ops[i])->output_dtype == mm->output_dtype)
+            residual = other(ops[i++]);
+        if (i < ops.size() && is_unary_ew(ops[i].node->op_type)) {
+            const OpType a = ops[i].node->op_type;
+            if (a == OpType::ReLU || a == OpType::GELU || a == OpType::SiLU || a == OpType::Sigmoid || a == OpType::Tanh) act = unary_code(ops[i++].node->op_type);
+        }
+        if (i != ops.size() || n->output_dtype != mm->output_dtype) return -1;
+        const int bias_v = bias ? make_contiguous(eval(bias)) : -1;
+        const int res_v = residual ? make_contiguous(eval(residual)) : -1;
+        return emit_gemm(mm, n->output_shape, bias_v, res_v, act);
+    }
+
+    int emit_gemm(const GraphNode *n, const Shape &out_shape_override, int bias_v, int res_v, int act) {
+        const auto &mp = get_params<MatMulParams>(n->params);
+        int a = make_contiguous(eval(n->inputs[0].get())), b = make_contiguous(eval(n->inputs[1].get()));
+        const Shape &as = val(a).shape, &bs = val(b).shape;
+        if (val(a).dtype != val(b).dtype) throw TypeError("GPU matmul needs operands of one dtype");
+        GemmStep g;
+        g.p.dtype = detail::to_axhip_dtype(val(a).dtype);
+        g.p.trans_a = mp.transpose_a;
+        g.p.trans_b = mp.transpose_b;
+        const size_t ar = as[as.size() - 2], ac = as.back(), br = bs[bs.size() - 2], bc = bs.back();
+        g.p.m = static_cast<int64_t>(mp.transpose_a ? ac : ar);
+        g.p.k = static_cast<int64_t>(mp.transpose_a ? ar : ac);
+        g.p.n = static_cast<int64_t>(mp.transpose_b ? br : bc);
+        g.p.lda = static_cast<int64_t>(ac);
+        g.p.ldb = static_cast<int64_t>(bc);
+        g.p.ldc = g.p.n;
+        const size_t batch_a = ShapeUtils::size(as) / (ar * ac), batch_b = ShapeUtils::size(bs) / (br * bc);
+        if (batch_b == 1 && !mp.transpose_a) { // shared right operand (a Linear weight): fold the batch into M
+            g.p.m *= static_cast<int64_t>(batch_a);
+            g.p.batch = 1;
+        } else if (batch_a == batch_b || batch_b == 1 || batch_a == 1) {
+            if (batch_a == batch_b && batch_a > 1 && Shape(as.begin(), as.end() - 2) != Shape(bs.begin(), bs.end() - 2))
+                throw RuntimeError::not_implemented("GPU matmul with differently shaped batch dimensions");
+            g.p.batch = static_cast<int64_t>(std::max(batch_a, batch_b));
+            g.p.stride_a = batch_a == 1 ? 0 : static_cast<int64_t>(ar * ac);
+            g.p.stride_b = batch_b == 1 ? 0 : static_cast<int64_t>(br * bc);
+            g.p.stride_c = g.p.m * g.p.n;
+        } else {
+            throw RuntimeError::not_implemented("GPU matmul with broadcast batch dimensions");
+        }
+        g.p.epilogue_op = act;
+        g.a = a;
+        g.b = b;
+        g.bias = bias_v;
+        g.residual = res_v;
+        g.c = new_temp(out_shape_override.empty() ? n->output_shape : out_shape_override, n->output_dtype);
+        Step s{};
+        s.kind = Step::GEMM;
+        s.gemm = g;
+        plan_.steps.push_back(s);
+        if (!out_shape_override.empty()) memo_[n] = g.c; // the bare product never exists
+        return g.c;
+    }
+
+    const GraphNode *root_;
+    Plan plan_;
+    std::unordered_map<const GraphNode *, int> memo_;
+    std::unordered_map<const GraphNode *, int> topo_index_;
+};
+
+// ------------------------------------------------------------------- cache
+struct CacheState {
+    std::mutex mu;
+    std::unordered_map<uint64_t, std::shared_ptr<const Plan>> plans;
+    size_t hits = 0, misses = 0;
+};
+CacheState &cache() {
+    static CacheState c;
+    return c;
+}
+
+thread_local std::vector<std::string> tl_last_kernels;
+
+uint64_t mix_u64(uint64_t h, uint64_t v) {
+    for (int i = 0; i < 8; ++i) h = (h ^ ((v >> (8 * i)) & 0xFF)) * 1099511628211ULL;
+    return h;
+}
+
+// The structural signature plus what else decides the plan: which interior nodes are
+// shared (they are materialised on their own) and the layout of materialised leaves.
+uint64_t plan_key(const GraphNode *root, const std::vector<const GraphNode *> &topo) {
+    uint64_t h = compute_signature(root).hash;
+    for (const GraphNode *n : topo) {
+        if (is_leaf(n, root)) {
+            if (!n->is_constant) {
+                h = mix_u64(h, 0x6C656166); // materialised leaf: shape and strides
+                for (size_t d : n->cached_shape_) h = mix_u64(h, d);
+                for (int64_t s : n->cached_strides_) h = mix_u64(h, static_cast<uint64_t>(s));
+            }
+        } else {
+            h = mix_u64(h, n->ref_count.load() > 1 ? 2 : 1);
+        }
+    }
+    return h;
+}
+
+bool debug_fusion() {
+    static const bool v = std::getenv("AXIOM_DEBUG_FUSION") != nullptr;
+    return v;
+}
+
+} // namespace
+
+GraphCache &GraphCache::instance() {
+    static GraphCache g;
+    return g;
+}
+void GraphCache::clear() {
+    auto &c = cache();
+    std::lock_guard<std::mutex> lk(c.mu);
+    c.plans.clear();
+    c.hits = c.misses = 0;
+}
+size_t GraphCache::size() const {
+    auto &c = cache();
+    std::lock_guard<std::mutex> lk(c.mu);
+    return c.plans.size();
+}
+size_t GraphCache::hits() const { return cache().hits; }
+size_t GraphCache::misses() const { return cache().misses; }
+
+const std::vector<std::string> &last_gpu_plan_kernels() { return tl_last_kernels; }
+
+void materialize_gpu_graph(GraphNode *root) {
+    if (!root || root->is_materialized_) return;
+    const auto topo = topo_sort(root);
+
+    // ---- plan: cached by signature
+    const uint64_t key = plan_key(root, topo);
+    std::shared_ptr<const Plan> plan;
+    {
+        auto &c = cache();
+        std::lock_guard<std::mutex> lk(c.mu);
+        auto it = c.plans.find(key);
+        if (it != c.plans.end()) {
+            plan = it->second;
+            ++c.hits;
+        } else {
+            ++c.misses;
+        }
+    }
+    if (!plan) {
+        plan = std::make_shared<const Plan>(PlanBuilder(root, topo).build());
+        auto &c = cache();
+        std::lock_guard<std::mutex> lk(c.mu);
+        if (c.plans.size() >= GraphCache::max_entries) c.plans.clear(); // src/backends/metal/mpsgraph_graph_compiler.mm:899-900
+        c.plans.emplace(key, plan);
+    }
+
+    // ---- bind leaves (same order as the builder: topological order) and allocate temporaries
+    struct Bound {
+        std::shared_ptr<Storage> storage;
+        size_t offset = 0;
+    };
+    std::vector<Bound> leaves;
+    for (const GraphNode *n : topo)
+        if (is_leaf(n, root)) {
+            Bound b;
+            b.storage = n->is_constant ? n->constant_storage : n->cached_result_;
+            b.offset = n->is_constant ? n->constant_offset : n->cached_offset_;
+            if (!b.storage || b.storage->device() != Device::GPU) throw DeviceError("GPU graph input is not resident on the GPU");
+            leaves.push_back(std::move(b));
+        }
+    if (leaves.size() != plan->n_leaves) throw RuntimeError("GPU plan cache: leaf count mismatch");
+    std::vector<std::shared_ptr<Storage>> temps(plan->temp_bytes.size());
+    for (size_t i = 0; i < temps.size(); ++i) temps[i] = make_storage(plan->temp_bytes[i], Device::GPU);
+
+    auto storage_of = [&](int v) -> std::shared_ptr<Storage> {
+        const ValueSpec &s = plan->values[v];
+        return s.is_leaf ? leaves[s.index].storage : temps[s.index];
+    };
+    auto ptr_of = [&](int v) -> void * {
+        const ValueSpec &s = plan->values[v];
+        char *base = static_cast<char *>(s.is_leaf ? leaves[s.index].storage->raw() : temps[s.index]->raw());
+        return base + (s.is_leaf ? leaves[s.index].offset : 0);
+    };
+
+    // ---- run
+    tl_last_kernels.clear();
+    for (const Step &st : plan->steps) {
+        if (st.kind == Step::ROWS) {
+            AxhipRowsProgram p = st.rows.prog;
+            p.input = ptr_of(st.rows.input);
+            p.output = ptr_of(st.rows.output);
+            for (int i = 0; i < p.n_operands; ++i) p.operands[i].ptr = ptr_of(st.rows.operand_value[i]);
+            if (st.rows.full_reduce) {
+                tl_last_kernels.emplace_back("full_reduce");
+                if (p.rows > 0 && p.cols > 0)
+                    AXHIP_CALL(axhip_fused_full_reduce(&p, temps[st.rows.workspace]->raw(), temps[st.rows.workspace]->size_bytes(), nullptr));
+            } else {
+                tl_last_kernels.emplace_back(axhip_fused_rows_kernel_name(&p));
+                AXHIP_CALL(axhip_fused_rows(&p, nullptr));
+            }
+        } else if (st.kind == Step::GEMM) {
+            AxhipGemmParams p = st.gemm.p;
+            p.bias = st.gemm.bias >= 0 ? ptr_of(st.gemm.bias) : nullptr;
+            p.residual = st.gemm.residual >= 0 ? ptr_of(st.gemm.residual) : nullptr;
+            tl_last_kernels.emplace_back("gemm");
+            AXHIP_CALL(axhip_gemm(ptr_of(st.gemm.a), ptr_of(st.gemm.b), ptr_of(st.gemm.c), &p, nullptr));
+        } else {
+            const ValueSpec &src = plan->values[st.copy.src];
+            const int dt = detail::to_axhip_dtype(src.dtype);
+            std::vector<int64_t> shp(st.copy.shape.begin(), st.copy.shape.end()), est(st.copy.src_strides.size());
+            for (size_t i = 0; i < est.size(); ++i) est[i] = st.copy.src_strides[i] / static_cast<int64_t>(dtype_size(src.dtype));
+            tl_last_kernels.emplace_back("strided_copy");
+            AXHIP_CALL(axhip_strided_copy(ptr_of(st.copy.src), dt, ptr_of(st.copy.dst), dt, static_cast<int32_t>(shp.size()), shp.data(),
+                                          est.data(), nullptr));
+        }
+    }
+    if (debug_fusion()) {
+        std::string line = "[axiom gpu graph] " + std::to_string(topo.size()) + " nodes ->";
+        for (const auto &k : tl_last_kernels) line += " " + k;
+        fprintf(stderr, "%s\n", line.c_str());
+    }
+
+    // ---- publish results: the root and every shared node the plan materialised
+    for (const auto &[idx, v] : plan->node_results) {
+        GraphNode *n = const_cast<GraphNode *>(topo[idx]);
+        const ValueSpec &s = plan->values[v];
+        n->cached_result_ = storage_of(v);
+        n->cached_shape_ = s.shape;
+        n->cached_strides_ = s.strides;
+        n->cached_offset_ = s.is_leaf ? leaves[s.index].offset : 0;
+        n->is_materialized_ = true;
+    }
+    // a materialised node no longer needs its inputs: drop the edges (src/backends/metal/
+    // mpsgraph_graph_compiler.mm:931-942 decrements the same counts)
+    for (const auto &[idx, v] : plan->node_results) {
+        (void)v;
+        GraphNode *n = const_cast<GraphNode *>(topo[idx]);
+        for (auto &in : n->inputs)
+            if (!in->is_constant && in->ref_count.load() > 0) in->ref_count.fetch_sub(1);
+        n->inputs.clear();
+    }
+}
+
+} // namespace axiom::graph

@@ -1,0 +1,374 @@
+// Lazy graph: node construction with shape / dtype inference, eager-mode switches,
+// the pending list, the structural signature and GraphRegistry::materialize
+// (behaviour of src/graph/graph_registry.cpp and graph_signature.cpp for the hot-path ops).
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "axiom/error.hpp"
+#include "axiom/graph/graph_registry.hpp"
+#include "axiom/graph/graph_signature.hpp"
+#include "axiom/tensor.hpp"
+
+namespace axiom::graph {
+
+// ------------------------------------------------------------ eager switches
+namespace {
+thread_local bool tl_eager_scope = false;
+size_t g_max_pending = 10000; // src/graph/graph_registry.cpp:30-35
+
+bool env_eager() {
+    static const bool v = [] {
+        const char *e = std::getenv("AXIOM_EAGER_MODE");
+        return e && std::string(e) == "1";
+    }();
+    return v;
+}
+} // namespace
+
+bool is_eager_mode_enabled() { return tl_eager_scope || env_eager(); }
+size_t get_max_pending_nodes() { return g_max_pending; }
+void set_max_pending_nodes(size_t n) { g_max_pending = n; }
+
+EagerModeScope::EagerModeScope() : previous_mode_(tl_eager_scope) { tl_eager_scope = true; }
+EagerModeScope::~EagerModeScope() { tl_eager_scope = previous_mode_; }
+
+// ----------------------------------------------------------------- inference
+Shape infer_binary_shape(const Shape &lhs, const Shape &rhs) { return ShapeUtils::broadcast(lhs, rhs); }
+
+// a full reduction without keep_dims yields shape {1} (src/graph/graph_registry.cpp:102-111)
+Shape infer_reduction_shape(const Shape &input, const std::vector<int> &axes, bool keep_dims) {
+    const int nd = static_cast<int>(input.size());
+    std::vector<bool> red(nd, axes.empty());
+    for (int a : axes) red[ShapeUtils::normalize_axis(a, nd)] = true;
+    Shape out;
+    for (int i = 0; i < nd; ++i) {
+        if (!red[i]) out.push_back(input[i]);
+        else if (keep_dims) out.push_back(1);
+    }
+    if (out.empty()) out.push_back(1);
+    return out;
+}
+
+Shape infer_matmul_shape(const Shape &a, const Shape &b, bool ta, bool tb) {
+    if (a.size() < 2 || b.size() < 2) throw ShapeError("matmul needs operands with at least 2 dimensions");
+    const size_t m = ta ? a[a.size() - 1] : a[a.size() - 2], ka = ta ? a[a.size() - 2] : a[a.size() - 1];
+    const size_t kb = tb ? b[b.size() - 1] : b[b.size() - 2], n = tb ? b[b.size() - 2] : b[b.size() - 1];
+    if (ka != kb) throw ShapeError("matmul: inner dimensions differ (" + std::to_string(ka) + " vs " + std::to_string(kb) + ")");
+    Shape out = ShapeUtils::broadcast(Shape(a.begin(), a.end() - 2), Shape(b.begin(), b.end() - 2));
+    out.push_back(m);
+    out.push_back(n);
+    return out;
+}
+
+DType infer_binary_dtype(DType lhs, DType rhs) { return ops::promote_types(lhs, rhs); }
+DType infer_unary_dtype(ops::OpType, DType input) { return input; }
+DType infer_reduction_dtype(ops::OpType op, DType input) {
+    if (op == ops::OpType::Mean) return input == DType::Float64 ? input : DType::Float32; // src/graph/graph_registry.cpp:278-287
+    return input;
+}
+
+// ------------------------------------------------------------------ registry
+thread_local std::vector<std::weak_ptr<GraphNode>> GraphRegistry::pending_nodes_;
+
+namespace {
+
+// Wraps an input tensor as a graph node: a lazy tensor contributes its node (ref_count++),
+// an eager one a constant node over its storage, strides and offset
+// (src/graph/graph_registry.cpp:297-311).
+std::shared_ptr<GraphNode> input_node(const Tensor &t) {
+    if (t.is_lazy() && !t.lazy_node()->is_materialized_) {
+        auto n = t.lazy_node();
+        n->ref_count.fetch_add(1);
+        return n;
+    }
+    auto n = std::make_shared<GraphNode>();
+    n->is_constant = true;
+    n->output_shape = t.shape();
+    n->output_dtype = t.dtype();
+    n->target_device = t.device();
+    n->constant_storage = t.storage();
+    n->constant_strides = t.strides();
+    n->constant_offset = t.offset();
+    return n;
+}
+
+Device pick_device(std::initializer_list<const Tensor *> ts) {
+    for (const Tensor *t : ts)
+        if (!t->empty() && t->device() == Device::GPU) return Device::GPU;
+    return Device::CPU;
+}
+
+void require_gpu(Device d, ops::OpType op) {
+    if (d != Device::GPU)
+        throw RuntimeError(std::string("ops::") + ops::op_name(op) + " on CPU tensors: this library is the gfx950 GPU backend only; move the operands with .gpu()");
+}
+
+// operands of a GPU op living on the host are moved over (src/tensor/operations.cpp:4018-4029)
+Tensor on_gpu(const Tensor &t) { return t.empty() || t.device() == Device::GPU ? t : t.to(Device::GPU); }
+
+} // namespace
+
+Tensor GraphRegistry::finalize_lazy_node(std::shared_ptr<GraphNode> node) {
+    if (is_eager_mode_enabled()) { // every op is its own graph
+        Tensor t(node);
+        t.sync();
+        return t;
+    }
+    auto &pend = pending_nodes_;
+    pend.push_back(node);
+    if (pend.size() >= g_max_pending) { // src/graph/graph_registry.cpp:379-382
+        Tensor t(node);
+        materialize_all();
+        return t;
+    }
+    return Tensor(std::move(node));
+}
+
+Tensor GraphRegistry::create_lazy_unary(ops::OpType op, const Tensor &input, const OpParams &params) {
+    require_gpu(pick_device({&input}), op);
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = op;
+    n->inputs = {input_node(input)};
+    n->output_shape = input.shape();
+    n->output_dtype = infer_unary_dtype(op, input.dtype());
+    n->target_device = Device::GPU;
+    n->params = params;
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_binary(ops::OpType op, const Tensor &lhs, const Tensor &rhs, const OpParams &params) {
+    require_gpu(pick_device({&lhs, &rhs}), op);
+    const Shape out = infer_binary_shape(lhs.shape(), rhs.shape());
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = op;
+    n->inputs = {input_node(on_gpu(lhs)), input_node(on_gpu(rhs))};
+    n->output_shape = out;
+    n->output_dtype = infer_binary_dtype(lhs.dtype(), rhs.dtype());
+    n->target_device = Device::GPU;
+    n->params = params;
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_reduction(ops::OpType op, const Tensor &input, const std::vector<int> &axes, bool keep_dims) {
+    require_gpu(pick_device({&input}), op);
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = op;
+    n->output_shape = infer_reduction_shape(input.shape(), axes, keep_dims); // validates the axes
+    n->inputs = {input_node(input)};
+    n->output_dtype = infer_reduction_dtype(op, input.dtype());
+    n->target_device = Device::GPU;
+    n->params = ReductionParams{axes, keep_dims};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_matmul(const Tensor &a, const Tensor &b, bool ta, bool tb) {
+    require_gpu(pick_device({&a, &b}), ops::OpType::MatMul);
+    const Shape out = infer_matmul_shape(a.shape(), b.shape(), ta, tb);
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::MatMul;
+    n->inputs = {input_node(on_gpu(a)), input_node(on_gpu(b))};
+    n->output_shape = out;
+    n->output_dtype = infer_binary_dtype(a.dtype(), b.dtype());
+    n->target_device = Device::GPU;
+    n->params = MatMulParams{ta, tb};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_softmax(ops::OpType op, const Tensor &input, int axis) {
+    require_gpu(pick_device({&input}), op);
+    const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = op;
+    n->inputs = {input_node(input)};
+    n->output_shape = input.shape();
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    ActivationParams p;
+    p.axis = a;
+    n->params = p;
+    return finalize_lazy_node(std::move(n));
+}
+
+// the norm output keeps the input dtype on GPU (src/graph/graph_registry.cpp:622-627)
+Tensor GraphRegistry::create_lazy_layernorm(const Tensor &input, const Tensor &weight, const Tensor &bias, int axis, float eps) {
+    require_gpu(pick_device({&input}), ops::OpType::LayerNorm);
+    const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::LayerNorm;
+    n->inputs = {input_node(input)};
+    if (!weight.empty()) n->inputs.push_back(input_node(on_gpu(weight)));
+    if (!bias.empty()) {
+        if (weight.empty()) throw ValueError("layer_norm: bias without weight");
+        n->inputs.push_back(input_node(on_gpu(bias)));
+    }
+    n->output_shape = input.shape();
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = NormParams{a, eps};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_rmsnorm(const Tensor &input, const Tensor &weight, int axis, float eps) {
+    require_gpu(pick_device({&input}), ops::OpType::RMSNorm);
+    const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::RMSNorm;
+    n->inputs = {input_node(input)};
+    if (!weight.empty()) n->inputs.push_back(input_node(on_gpu(weight)));
+    n->output_shape = input.shape();
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = NormParams{a, eps};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_reshape(const Tensor &input, const Shape &new_shape) {
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Reshape;
+    n->inputs = {input_node(input)};
+    n->output_shape = new_shape;
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = ReshapeParams{new_shape};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_transpose(const Tensor &input, const std::vector<int> &axes) {
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Transpose;
+    n->inputs = {input_node(input)};
+    const Shape &in = input.shape();
+    Shape out(in.size());
+    for (size_t i = 0; i < axes.size(); ++i) out[i] = in[axes[i]];
+    n->output_shape = out;
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = TransposeParams{axes};
+    return finalize_lazy_node(std::move(n));
+}
+
+// src/graph/graph_registry.cpp:830-927; GPU graphs bypass the CPU compiler (:834-850)
+void GraphRegistry::materialize(GraphNode *node) {
+    if (!node || node->is_materialized_) return;
+    if (node->target_device != Device::GPU)
+        throw RuntimeError("lazy CPU graphs cannot be materialised: this library is the gfx950 GPU backend only");
+    materialize_gpu_graph(node);
+}
+
+size_t GraphRegistry::pending_node_count() {
+    auto &p = pending_nodes_;
+    p.erase(std::remove_if(p.begin(), p.end(), [](const std::weak_ptr<GraphNode> &w) {
+                auto s = w.lock();
+                return !s || s->is_materialized_;
+            }),
+            p.end());
+    return p.size();
+}
+
+void GraphRegistry::materialize_all() {
+    auto pending = std::move(pending_nodes_);
+    pending_nodes_.clear();
+    // newest first: a root materialises its whole subgraph, older entries are then done
+    for (auto it = pending.rbegin(); it != pending.rend(); ++it)
+        if (auto n = it->lock())
+            if (!n->is_materialized_) materialize(n.get());
+}
+
+// ----------------------------------------------------------------- signature
+std::vector<const GraphNode *> topo_sort(const GraphNode *root) {
+    std::vector<const GraphNode *> order;
+    std::unordered_set<const GraphNode *> seen;
+    struct Frame {
+        const GraphNode *n;
+        size_t next;
+    };
+    std::vector<Frame> stack{{root, 0}};
+    seen.insert(root);
+    while (!stack.empty()) {
+        Frame &f = stack.back();
+        const bool leaf = f.n->is_constant || (f.n->is_materialized_ && f.n != root);
+        if (!leaf && f.next < f.n->inputs.size()) {
+            const GraphNode *c = f.n->inputs[f.next++].get();
+            if (seen.insert(c).second) stack.push_back({c, 0});
+        } else {
+            order.push_back(f.n);
+            stack.pop_back();
+        }
+    }
+    return order;
+}
+
+namespace {
+constexpr uint64_t FNV_OFFSET = 14695981039346656037ULL, FNV_PRIME = 1099511628211ULL;
+inline uint64_t mix_bytes(uint64_t h, const void *p, size_t n) {
+    const unsigned char *b = static_cast<const unsigned char *>(p);
+    for (size_t i = 0; i < n; ++i) h = (h ^ b[i]) * FNV_PRIME;
+    return h;
+}
+inline uint64_t mix(uint64_t h, uint64_t v) { return mix_bytes(h, &v, 8); }
+inline uint64_t mix_i32(uint64_t h, int32_t v) { return mix_bytes(h, &v, 4); }
+inline uint64_t mix_f32(uint64_t h, float v) { return mix_bytes(h, &v, 4); }
+inline uint64_t mix_bool(uint64_t h, bool v) {
+    const unsigned char b = v ? 1 : 0;
+    return mix_bytes(h, &b, 1);
+}
+} // namespace
+
+GraphSignature compute_signature(const GraphNode *root) {
+    const auto sorted = topo_sort(root);
+    std::unordered_map<const GraphNode *, uint32_t> index;
+    for (uint32_t i = 0; i < sorted.size(); ++i) index[sorted[i]] = i;
+    uint64_t h = mix(FNV_OFFSET, sorted.size());
+    for (const GraphNode *n : sorted) {
+        h = mix(h, static_cast<uint64_t>(n->op_type));
+        h = mix(h, n->output_shape.size());
+        for (size_t d : n->output_shape) h = mix(h, d);
+        h = mix(h, static_cast<uint64_t>(n->output_dtype));
+        h = mix(h, static_cast<uint64_t>(n->target_device));
+        h = mix_bool(h, n->is_constant);
+        if (n->is_constant) {
+            h = mix(h, n->constant_strides.size());
+            for (int64_t s : n->constant_strides) h = mix(h, static_cast<uint64_t>(s));
+        }
+        const bool leaf = n->is_constant || (n->is_materialized_ && n != root);
+        h = mix(h, leaf ? 0 : n->inputs.size());
+        if (!leaf)
+            for (const auto &in : n->inputs) {
+                auto it = index.find(in.get());
+                h = mix(h, it != index.end() ? it->second : UINT64_MAX);
+            }
+        h = mix(h, n->params.index());
+        std::visit(
+            [&](const auto &p) {
+                using T = std::decay_t<decltype(p)>;
+                if constexpr (std::is_same_v<T, ReductionParams>) {
+                    h = mix(h, p.axes.size());
+                    for (int a : p.axes) h = mix_i32(h, a);
+                    h = mix_bool(h, p.keep_dims);
+                } else if constexpr (std::is_same_v<T, MatMulParams>) {
+                    h = mix_bool(h, p.transpose_a);
+                    h = mix_bool(h, p.transpose_b);
+                } else if constexpr (std::is_same_v<T, ActivationParams>) {
+                    h = mix_f32(h, p.alpha);
+                    h = mix_i32(h, p.axis);
+                } else if constexpr (std::is_same_v<T, ReshapeParams>) {
+                    h = mix(h, p.new_shape.size());
+                    for (size_t d : p.new_shape) h = mix(h, d);
+                } else if constexpr (std::is_same_v<T, NormParams>) {
+                    h = mix_i32(h, p.axis);
+                    h = mix_f32(h, p.eps);
+                } else if constexpr (std::is_same_v<T, TransposeParams>) {
+                    h = mix(h, p.axes.size());
+                    for (int a : p.axes) h = mix_i32(h, a);
+                }
+            },
+            n->params);
+    }
+    return GraphSignature{h};
+}
+
+} // namespace axiom::graph

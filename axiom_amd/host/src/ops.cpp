@@ -1,0 +1,198 @@
+// ops:: entry points: validation, device unification and routing into the lazy graph
+// or the eager attention call (behaviour of src/tensor/operations.cpp for the hot-path ops).
+#include "axiom/operations.hpp"
+
+#include <cmath>
+#include <map>
+
+#include "axiom/error.hpp"
+#include "axiom/graph/graph_registry.hpp"
+#include "axiom/tensor.hpp"
+#include "hip_call.hpp"
+
+namespace axiom::ops {
+
+const char *op_name(OpType op) {
+    switch (op) {
+    case OpType::Add: return "add";
+    case OpType::Subtract: return "subtract";
+    case OpType::Multiply: return "multiply";
+    case OpType::Divide: return "divide";
+    case OpType::Maximum: return "maximum";
+    case OpType::Minimum: return "minimum";
+    case OpType::Negate: return "negate";
+    case OpType::Abs: return "abs";
+    case OpType::Sqrt: return "sqrt";
+    case OpType::Exp: return "exp";
+    case OpType::Log: return "log";
+    case OpType::Reciprocal: return "reciprocal";
+    case OpType::Square: return "square";
+    case OpType::ReLU: return "relu";
+    case OpType::SiLU: return "silu";
+    case OpType::Sigmoid: return "sigmoid";
+    case OpType::Tanh: return "tanh";
+    case OpType::GELU: return "gelu";
+    case OpType::Softmax: return "softmax";
+    case OpType::LogSoftmax: return "log_softmax";
+    case OpType::Sum: return "sum";
+    case OpType::Mean: return "mean";
+    case OpType::Max: return "max";
+    case OpType::Min: return "min";
+    case OpType::MatMul: return "matmul";
+    case OpType::LayerNorm: return "layer_norm";
+    case OpType::RMSNorm: return "rms_norm";
+    case OpType::Reshape: return "reshape";
+    case OpType::Transpose: return "transpose";
+    case OpType::ScaledDotProductAttention: return "scaled_dot_product_attention";
+    default: return "op";
+    }
+}
+
+// src/tensor/operations.cpp:346-397: the higher rank wins among floats; mixed-sign
+// integers of equal width widen
+DType promote_types(DType lhs, DType rhs) {
+    if (lhs == rhs) return lhs;
+    static const std::map<DType, int> rank = {
+        {DType::Bool, 0}, {DType::Int8, 1}, {DType::UInt8, 2}, {DType::Int16, 3}, {DType::UInt16, 4},
+        {DType::Int32, 5}, {DType::UInt32, 6}, {DType::Int64, 7}, {DType::UInt64, 8}, {DType::Float16, 9},
+        {DType::BFloat16, 10}, {DType::Float32, 11}, {DType::Float64, 12}, {DType::Complex64, 13}, {DType::Complex128, 14}};
+    const bool l_hi = rank.at(lhs) > rank.at(rhs);
+    const DType t1 = l_hi ? lhs : rhs, t2 = l_hi ? rhs : lhs;
+    if (is_complex_dtype(t1) || is_floating_dtype(t1)) return t1;
+    auto is_signed = [](DType d) { return d == DType::Int8 || d == DType::Int16 || d == DType::Int32 || d == DType::Int64; };
+    const bool s1 = is_signed(t1), s2 = is_signed(t2);
+    const size_t z1 = dtype_size(t1), z2 = dtype_size(t2);
+    if (s1 == s2 || z1 > z2) return t1;
+    switch (std::max(z1, z2)) {
+    case 1: return DType::Int16;
+    case 2: return DType::Int32;
+    case 4: return DType::Int64;
+    default: return DType::Float64;
+    }
+}
+
+using graph::GraphRegistry;
+
+Tensor add(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Add, a, b); }
+Tensor subtract(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Subtract, a, b); }
+Tensor multiply(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Multiply, a, b); }
+Tensor divide(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Divide, a, b); }
+Tensor maximum(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Maximum, a, b); }
+Tensor minimum(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Minimum, a, b); }
+
+Tensor negate(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Negate, x); }
+Tensor abs(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Abs, x); }
+Tensor sqrt(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Sqrt, x); }
+Tensor exp(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Exp, x); }
+Tensor log(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Log, x); }
+Tensor reciprocal(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Reciprocal, x); }
+Tensor square(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Square, x); }
+Tensor relu(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::ReLU, x); }
+Tensor silu(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::SiLU, x); }
+Tensor sigmoid(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Sigmoid, x); }
+Tensor tanh(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Tanh, x); }
+Tensor gelu(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::GELU, x); }
+
+// on GPU softmax and the norms are captured lazily (src/tensor/operations.cpp:1420-1425, 1791-1795)
+Tensor softmax(const Tensor &x, int axis) { return GraphRegistry::create_lazy_softmax(OpType::Softmax, x, axis); }
+Tensor log_softmax(const Tensor &x, int axis) { return GraphRegistry::create_lazy_softmax(OpType::LogSoftmax, x, axis); }
+
+Tensor sum(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Sum, x, axes, keep); }
+Tensor mean(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Mean, x, axes, keep); }
+Tensor max(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Max, x, axes, keep); }
+Tensor min(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Min, x, axes, keep); }
+
+Tensor layer_norm(const Tensor &x, const Tensor &weight, const Tensor &bias, int axis, float eps) {
+    const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(x.ndim()));
+    for (const Tensor *p : {&weight, &bias})
+        if (!p->empty() && (p->ndim() != 1 || p->shape()[0] != x.shape()[a]))
+            throw ShapeError("layer_norm: weight / bias must have shape [" + std::to_string(x.shape()[a]) + "]");
+    return GraphRegistry::create_lazy_layernorm(x, weight, bias, axis, eps);
+}
+
+Tensor rms_norm(const Tensor &x, const Tensor &weight, int axis, float eps) {
+    const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(x.ndim()));
+    if (!weight.empty() && (weight.ndim() != 1 || weight.shape()[0] != x.shape()[a]))
+        throw ShapeError("rms_norm: weight must have shape [" + std::to_string(x.shape()[a]) + "]");
+    return GraphRegistry::create_lazy_rmsnorm(x, weight, axis, eps);
+}
+
+Tensor matmul(const Tensor &a, const Tensor &b, bool ta, bool tb) { return GraphRegistry::create_lazy_matmul(a, b, ta, tb); }
+
+// ---------------------------------------------------------------- attention
+namespace {
+thread_local std::string tl_sdpa_kernel = "";
+
+// last dimension contiguous, non-negative strides: what axhip_sdpa_fwd addresses directly
+Tensor sdpa_operand(const Tensor &t) {
+    Tensor g = t.device() == Device::GPU ? t : t.to(Device::GPU);
+    const Strides &st = g.strides(); // materialises a lazy operand
+    bool ok = st.back() == static_cast<int64_t>(g.itemsize()) || g.shape().back() == 1;
+    for (int64_t s : st) ok = ok && s >= 0 && s % static_cast<int64_t>(g.itemsize()) == 0;
+    return ok ? g : g.ascontiguousarray();
+}
+} // namespace
+
+const char *last_sdpa_kernel() { return tl_sdpa_kernel.c_str(); }
+
+Tensor scaled_dot_product_attention(const Tensor &query, const Tensor &key, const Tensor &value, const Tensor &mask, float scale, bool is_causal) {
+    return detail::sdpa(query, key, value, mask, scale, is_causal, false);
+}
+
+// src/tensor/operations.cpp:3979-4044
+Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value, const Tensor &mask, float scale, bool is_causal, bool out_bshd) {
+    if (query.ndim() != 4 || key.ndim() != 4 || value.ndim() != 4)
+        throw ShapeError("scaled_dot_product_attention expects 4-D (batch, heads, seq, head_dim) tensors");
+    const Shape &qs = query.shape(), &ks = key.shape(), &vs = value.shape();
+    if (qs[0] != ks[0] || qs[0] != vs[0]) throw ShapeError("scaled_dot_product_attention: batch sizes differ");
+    if (qs[1] != ks[1] || qs[1] != vs[1]) throw ShapeError("scaled_dot_product_attention: head counts differ");
+    if (ks[2] != vs[2]) throw ShapeError("scaled_dot_product_attention: key and value sequence lengths differ");
+    if (qs[3] != ks[3] || qs[3] != vs[3]) throw ShapeError("scaled_dot_product_attention: head dimensions differ");
+    if (query.dtype() != key.dtype() || query.dtype() != value.dtype()) throw TypeError("scaled_dot_product_attention: q, k, v dtypes differ");
+    const size_t B = qs[0], H = qs[1], Sq = qs[2], Skv = ks[2], D = qs[3];
+
+    if (query.device() != Device::GPU && key.device() != Device::GPU && value.device() != Device::GPU)
+        throw RuntimeError("ops::scaled_dot_product_attention on CPU tensors: this library is the gfx950 GPU backend only; move the operands with .gpu()");
+    const Tensor q = sdpa_operand(query), k = sdpa_operand(key), v = sdpa_operand(value);
+
+    AxhipSdpaParams p{};
+    p.dtype = ::axiom::detail::to_axhip_dtype(q.dtype());
+    p.batch = static_cast<int32_t>(B);
+    p.heads = static_cast<int32_t>(H);
+    p.seq_q = static_cast<int32_t>(Sq);
+    p.seq_kv = static_cast<int32_t>(Skv);
+    p.head_dim = static_cast<int32_t>(D);
+    p.scale = scale; // <= 0: the library uses 1/sqrt(D) (operations.cpp:4013-4015)
+    p.is_causal = is_causal ? 1 : 0;
+    const int64_t isz = static_cast<int64_t>(q.itemsize());
+    for (int i = 0; i < 3; ++i) {
+        p.q_strides[i] = q.strides()[i] / isz;
+        p.k_strides[i] = k.strides()[i] / isz;
+        p.v_strides[i] = v.strides()[i] / isz;
+    }
+    // out_bshd: the result is laid out (B, Sq, H, D) in memory and returned as its (B, H, Sq, D) view
+    Tensor out = out_bshd ? Tensor(Shape{B, Sq, H, D}, q.dtype(), Device::GPU).transpose({0, 2, 1, 3}) : Tensor(Shape{B, H, Sq, D}, q.dtype(), Device::GPU);
+    for (int i = 0; i < 3; ++i) p.o_strides[i] = out.strides()[i] / isz;
+
+    Tensor m;
+    const uint8_t *mask_ptr = nullptr;
+    if (!mask.empty()) {
+        if (mask.dtype() != DType::Bool && mask.dtype() != DType::UInt8) throw TypeError("scaled_dot_product_attention: mask must be Bool");
+        const Shape &ms = mask.shape();
+        const bool two_d = ms.size() == 2 && ms[0] == Sq && ms[1] == Skv;
+        const bool four_d = ms.size() == 4 && ms[2] == Sq && ms[3] == Skv && (ms[0] == B || ms[0] == 1) && (ms[1] == H || ms[1] == 1);
+        if (!two_d && !four_d) throw ShapeError("scaled_dot_product_attention: mask must be (Sq, Skv) or (B|1, H|1, Sq, Skv)");
+        m = (mask.device() == Device::GPU ? mask : mask.to(Device::GPU)).ascontiguousarray();
+        mask_ptr = static_cast<const uint8_t *>(m.storage()->raw()) + m.offset();
+        if (four_d) { // size-1 dims broadcast with stride 0
+            p.mask_strides[0] = ms[0] == 1 ? 0 : static_cast<int64_t>(ms[1] * Sq * Skv);
+            p.mask_strides[1] = ms[1] == 1 ? 0 : static_cast<int64_t>(Sq * Skv);
+        }
+    }
+    auto ptr = [](const Tensor &t) { return static_cast<const char *>(t.storage()->raw()) + t.offset(); };
+    tl_sdpa_kernel = axhip_sdpa_kernel_name(&p);
+    AXHIP_CALL(axhip_sdpa_fwd(ptr(q), ptr(k), ptr(v), out.storage()->raw(), mask_ptr, &p, nullptr));
+    return out; // asynchronous; .cpu() / item() synchronise
+}
+
+} // namespace axiom::ops

@@ -1,0 +1,440 @@
+// GPU cases through the host layer: device semantics, lazy fusion, attention, nn modules.
+// They follow the reference's tests/test_unified_memory.cpp (device-tag / round-trip /
+// auto-sync cases), test_fusion_extended.cpp:456-523, test_cpu_gpu_parity.cpp,
+// test_flash_attention.cpp, test_nn_attention.cpp, test_nn_layers.cpp and
+// test_tensor_normalization.cpp, with the CPU side of each comparison supplied by the oracle.
+#include <map>
+
+#include "oracle_util.hpp"
+#include "test_framework.hpp"
+
+using namespace axiom;
+using axtest::max_abs_diff;
+
+static std::vector<float> host_floats(const Tensor &t) {
+    Tensor c = t.cpu().astype(DType::Float32).ascontiguousarray();
+    return std::vector<float>(c.typed_data<float>(), c.typed_data<float>() + c.size());
+}
+
+// ------------------------------------------------------------ device semantics
+GPU_TEST(DeviceTransfer, GpuTagRoundTripAndAutoSync) { // tests/test_unified_memory.cpp:102-122, 160-191
+    auto a = axtest::randn({37, 53}, 1);
+    auto g = a.gpu();
+    EXPECT_TRUE(g.device() == Device::GPU);
+    EXPECT_TRUE(a.device() == Device::CPU);
+    EXPECT_NE(g.storage().get(), a.storage().get()); // explicit copy, no shared memory
+    EXPECT_TRUE(g.cpu().allclose(a, 0, 0));
+    EXPECT_THROW(g.typed_data<float>(), DeviceError);
+    EXPECT_THROW(g.item<float>({0, 0}), DeviceError);
+    auto r = ops::add(g, g); // compute, then .cpu() waits for it
+    EXPECT_TRUE(r.is_lazy());
+    EXPECT_NEAR(r.cpu().item<float>({3, 4}), 2 * a.item<float>({3, 4}), 0);
+    auto h = a.astype(DType::BFloat16).gpu();
+    EXPECT_EQ(h.dtype(), DType::BFloat16);
+    EXPECT_TRUE(h.astype(DType::Float32).cpu().allclose(a.astype(DType::BFloat16).astype(DType::Float32), 0, 0)); // GPU cast
+    auto t = g.transpose({1, 0});
+    EXPECT_FALSE(t.is_contiguous());
+    EXPECT_TRUE(t.ascontiguousarray().cpu().allclose(a.transpose({1, 0}).ascontiguousarray(), 0, 0)); // GPU gather
+    EXPECT_NEAR(Tensor::full<float>({1}, 7.0f, Device::GPU).item<float>(), 7.0f, 0);
+}
+
+// ------------------------------------------------------------------ fusion
+GPU_TEST(FusionGpu, BasicAdd) {
+    auto a = Tensor::full<float>({64, 64}, 2.0f, Device::GPU);
+    auto b = Tensor::full<float>({64, 64}, 3.0f, Device::GPU);
+    ASSERT_NEAR(ops::add(a, b).cpu().item<float>({0, 0}), 5.0f, 1e-5f);
+}
+GPU_TEST(FusionGpu, UnaryChain) {
+    auto x = Tensor::full<float>({64, 64}, 4.0f, Device::GPU);
+    ASSERT_NEAR(ops::exp(ops::sqrt(x)).cpu().item<float>({0, 0}), std::exp(2.0f), 1e-4f);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u); // one launch
+}
+GPU_TEST(FusionGpu, BinaryUnaryFusion) {
+    auto a = Tensor::full<float>({64, 64}, -1.0f, Device::GPU);
+    auto b = Tensor::full<float>({64, 64}, 0.5f, Device::GPU);
+    ASSERT_NEAR(ops::relu(ops::add(a, b)).cpu().item<float>({0, 0}), 0.0f, 1e-6f);
+}
+GPU_TEST(FusionGpu, LongerChain) {
+    auto a = Tensor::full<float>({64, 64}, 0.5f, Device::GPU);
+    auto b = Tensor::full<float>({64, 64}, 2.0f, Device::GPU);
+    auto c = Tensor::full<float>({64, 64}, -0.5f, Device::GPU);
+    auto result = ops::tanh(ops::sigmoid(ops::add(ops::multiply(a, b), c)));
+    ASSERT_NEAR(result.cpu().item<float>({0, 0}), std::tanh(1.0f / (1.0f + std::exp(-0.5f))), 1e-4f);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+}
+GPU_TEST(FusionGpu, ReductionAndFusedReduction) {
+    auto a = Tensor::full<float>({4, 4}, 2.0f, Device::GPU);
+    auto b = Tensor::full<float>({4, 4}, 3.0f, Device::GPU);
+    ASSERT_NEAR(ops::sum(a).cpu().item<float>(), 32.0f, 1e-4f);
+    auto r = ops::sum(ops::add(a, b));
+    EXPECT_EQ(r.shape(), Shape({1}));
+    ASSERT_NEAR(r.cpu().item<float>(), 80.0f, 1e-4f); // tests/test_fusion_extended.cpp:346-352
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    auto big = Tensor::full<float>({1024, 1024}, 2.0f, Device::GPU);
+    ASSERT_NEAR(ops::sum(big).cpu().item<float>(), 2097152.0f, 1.0f); // :436-443
+    ASSERT_NEAR(ops::mean(big).cpu().item<float>(), 2.0f, 1e-5f);
+}
+GPU_TEST(FusionGpu, EagerParity) {
+    auto a = Tensor::full<float>({32, 32}, 1.5f, Device::GPU);
+    auto b = Tensor::full<float>({32, 32}, 0.5f, Device::GPU);
+    const float lazy_val = ops::sigmoid(ops::add(a, b)).cpu().item<float>({0, 0});
+    {
+        graph::EagerModeScope eager;
+        auto s = ops::add(a, b);
+        EXPECT_FALSE(s.is_lazy() && !s.lazy_node()->is_materialized_); // every op ran at once
+        ASSERT_NEAR(lazy_val, ops::sigmoid(s).cpu().item<float>({0, 0}), 1e-6f);
+    }
+}
+GPU_TEST(FusionGpu, LongChainOfScalars) { // tests/test_fusion_extended.cpp:561-572
+    auto x = Tensor::ones({8}, DType::Float32, Device::GPU);
+    for (int i = 0; i < 10; ++i) x = x + 1.0f;
+    EXPECT_NEAR(x.cpu().item<float>({3}), 11.0f, 0);
+    auto y = Tensor::ones({8}, DType::Float32, Device::GPU);
+    for (int i = 0; i < 40; ++i) y = y * 1.0f + 1.0f; // longer than one kernel's chain: split, still right
+    EXPECT_NEAR(y.cpu().item<float>({0}), 41.0f, 0);
+}
+GPU_TEST(FusionGpu, SharedNodesAndRecompute) { // tests/test_fusion_extended.cpp:252-299
+    auto a = axtest::randn({16, 32}, 3).gpu();
+    auto s = ops::exp(a);             // consumed twice below: materialised once
+    auto y = ops::add(ops::relu(s), ops::sqrt(s));
+    auto want = host_floats(a);
+    auto got = host_floats(y);
+    for (size_t i = 0; i < want.size(); ++i) {
+        const float e = std::exp(want[i]);
+        EXPECT_NEAR(got[i], std::max(e, 0.0f) + std::sqrt(e), 1e-4 * (1 + std::fabs(e)));
+    }
+    EXPECT_TRUE(s.lazy_node() == nullptr || s.lazy_node()->is_materialized_); // the shared node kept its result
+    EXPECT_NEAR(s.cpu().item<float>({0, 0}), std::exp(want[0]), 1e-5 * std::exp(want[0]) + 1e-6);
+    auto x = ops::relu(a);            // fused through by z; reading x later recomputes it
+    auto z = x + 1.0f;
+    EXPECT_NEAR(z.cpu().item<float>({1, 1}), std::max(want[33], 0.0f) + 1.0f, 1e-6);
+    EXPECT_NEAR(x.cpu().item<float>({1, 1}), std::max(want[33], 0.0f), 0);
+}
+GPU_TEST(FusionGpu, PlanCacheHitsAndMisses) { // tests/test_graph_compiler.cpp:79-125
+    auto &cache = graph::GraphCache::instance();
+    cache.clear();
+    auto run = [](size_t n, float v) {
+        auto a = Tensor::full<float>({n, 8}, v, Device::GPU);
+        return ops::relu(a * 2.0f).cpu().item<float>({0, 0});
+    };
+    EXPECT_NEAR(run(4, 1.0f), 2.0f, 0);
+    EXPECT_EQ(cache.misses(), 1u);
+    EXPECT_EQ(cache.hits(), 0u);
+    EXPECT_NEAR(run(4, -3.0f), 0.0f, 0); // same structure, other data
+    EXPECT_EQ(cache.hits(), 1u);
+    EXPECT_NEAR(run(5, 1.5f), 3.0f, 0);  // other shape: new plan
+    EXPECT_EQ(cache.misses(), 2u);
+    EXPECT_EQ(cache.size(), 2u);
+}
+GPU_TEST(FusionGpu, BroadcastKinds) { // tests/test_cpu_gpu_parity.cpp broadcast cases
+    auto a = axtest::randn({4, 5}, 5), row = axtest::randn({5}, 6), col = axtest::randn({4, 1}, 7);
+    auto ga = a.gpu();
+    auto r = host_floats(ops::multiply(ops::add(ga, row.gpu()), col.gpu()));
+    auto d = host_floats(ops::subtract(col.gpu(), ga)); // chain on the right-hand side
+    auto o = host_floats(ops::add(col.gpu(), row.gpu())); // both operands broadcast
+    for (size_t i = 0; i < 4; ++i)
+        for (size_t j = 0; j < 5; ++j) {
+            const float av = a.item<float>({i, j}), rv = row.item<float>({j}), cv = col.item<float>({i, 0});
+            EXPECT_NEAR(r[i * 5 + j], (av + rv) * cv, 0);
+            EXPECT_NEAR(d[i * 5 + j], cv - av, 0);
+            EXPECT_NEAR(o[i * 5 + j], cv + rv, 0);
+        }
+    EXPECT_NEAR((2.0f / Tensor::full<float>({3}, 4.0f, Device::GPU)).cpu().item<float>({1}), 0.5f, 0);
+}
+
+// ------------------------------------------------- BASELINE configs[1]: C2 chain
+GPU_TEST(FusedChain, ReluAddMulSoftmaxRowSumIsOneKernel) {
+    const size_t R = 256, C = 8192;
+    auto a = axtest::randn({R, C}, 11), b = axtest::randn({R, C}, 12);
+    auto ga = a.gpu(), gb = b.gpu();
+    auto sm = ops::softmax((ops::relu(ga) + 1) * gb, -1);
+    auto out = sm.sum(1);
+    auto got = host_floats(out);
+    ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"));
+    std::vector<float> want(R), want_sm(R * C);
+    axo_chain_relu_add_mul_softmax_sum(a.typed_data<float>(), b.typed_data<float>(), want.data(), want_sm.data(), R, C);
+    for (size_t i = 0; i < R; ++i) EXPECT_NEAR(got[i], want[i], 1e-4 + 1e-4 * std::fabs(want[i]));
+    // the intermediate softmax, evaluated on its own
+    auto got_sm = host_floats(ops::softmax((ops::relu(ga) + 1) * gb, -1));
+    double worst = 0;
+    for (size_t i = 0; i < R * C; ++i) worst = std::max(worst, std::fabs(double(got_sm[i]) - want_sm[i]) - 1e-4 * std::fabs(want_sm[i]));
+    EXPECT_LE(worst, 1e-4);
+}
+
+// ---------------------------------------------- BASELINE configs[2]: norm chains
+static void norm_chain_case(DType dt, bool rms, size_t R, size_t C) {
+    auto x = axtest::randn({R, C}, 21, dt), gamma = axtest::uniform({C}, 22, 0.5f, 1.5f, dt), beta = axtest::uniform({C}, 23, -0.1f, 0.1f, dt);
+    auto gx = x.gpu(), gg = gamma.gpu(), gb = beta.gpu();
+    auto y = rms ? ops::gelu(ops::rms_norm(gx, gg, -1, 1e-5f)) : ops::gelu(ops::layer_norm(gx, gg, gb, -1, 1e-5f));
+    EXPECT_EQ(y.dtype(), dt); // the GPU keeps the input dtype (src/graph/graph_registry.cpp:622-627)
+    auto got = host_floats(y);
+    ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u); // norm + gelu in one launch
+    // fp32 evaluation of the same (rounded) inputs through the oracle: norm then gelu.  This is the
+    // reference's own yardstick for half types (tests/test_flash_attention.cpp:233-249).
+    std::vector<float> n(R * C), want(R * C);
+    auto xf = x.astype(DType::Float32), gf = gamma.astype(DType::Float32), bf = beta.astype(DType::Float32);
+    if (rms) axo_rms_norm(AXO_F32, xf.data(), gf.data(), n.data(), R, C, 1e-5f);
+    else axo_layer_norm(AXO_F32, xf.data(), gf.data(), bf.data(), n.data(), R, C, 1e-5f);
+    axo_unary(AXO_OP_GELU, AXO_F32, n.data(), want.data(), R * C);
+    const double tol = dt == DType::Float32 ? 1e-4 : 2e-2;
+    double worst = 0;
+    for (size_t i = 0; i < R * C; ++i) worst = std::max(worst, std::fabs(double(got[i]) - want[i]) - (dt == DType::Float32 ? 1e-4 * std::fabs(want[i]) : 0.0));
+    EXPECT_LE(worst, tol);
+    if (dt != DType::Float32) {
+        // distance to the literal CPU path, which rounds the row mean (and for RMS every x*x) to the
+        // half type before continuing in fp32 and returns float32: one half-precision ulp of the
+        // statistic on top of the output rounding
+        const int odt = axtest::oracle_dtype(dt);
+        if (rms) axo_rms_norm(odt, x.data(), gamma.data(), n.data(), R, C, 1e-5f);
+        else axo_layer_norm(odt, x.data(), gamma.data(), beta.data(), n.data(), R, C, 1e-5f);
+        axo_unary(AXO_OP_GELU, AXO_F32, n.data(), want.data(), R * C);
+        double lit = 0;
+        for (size_t i = 0; i < R * C; ++i) lit = std::max(lit, std::fabs(double(got[i]) - want[i]));
+        std::printf("    distance to the literal CPU path (%s, %s): %.4f\n", dtype_name(dt).c_str(), rms ? "rms" : "layer", lit);
+        EXPECT_LE(lit, 6e-2);
+    }
+}
+GPU_TEST(FusedChain, GeluLayerNormBf16) { norm_chain_case(DType::BFloat16, false, 64, 4096); }
+GPU_TEST(FusedChain, GeluRmsNormBf16) { norm_chain_case(DType::BFloat16, true, 64, 4096); }
+GPU_TEST(FusedChain, GeluLayerNormF16OddWidth) { norm_chain_case(DType::Float16, false, 33, 1000); }
+GPU_TEST(FusedChain, GeluLayerNormF32) { norm_chain_case(DType::Float32, false, 17, 768); }
+GPU_TEST(FusedChain, GeluRmsNormF32Unaligned) { norm_chain_case(DType::Float32, true, 5, 37); }
+
+GPU_TEST(Normalization, KnownAnswers) {
+    // tests/test_tensor_normalization.cpp:80-141: [3,4] -> [3,4]/sqrt(12.5)
+    float v[2] = {3.0f, 4.0f};
+    auto x = Tensor::from_data(v, {1, 2}, Device::GPU);
+    auto r = ops::rms_norm(x, Tensor::ones({2}, DType::Float32, Device::GPU), -1, 0.0f).cpu();
+    EXPECT_NEAR(r.item<float>({0, 0}), 3.0f / std::sqrt(12.5f), 1e-5);
+    EXPECT_NEAR(r.item<float>({0, 1}), 4.0f / std::sqrt(12.5f), 1e-5);
+    // layer norm: mean ~ 0, var ~ 1 (tests/test_tensor_normalization.cpp:9-74)
+    auto a = axtest::randn({8, 64}, 31);
+    auto ln = host_floats(ops::layer_norm(a.gpu(), Tensor(), Tensor(), -1, 1e-5f));
+    for (size_t i = 0; i < 8; ++i) {
+        double m = 0, q = 0;
+        for (size_t j = 0; j < 64; ++j) m += ln[i * 64 + j];
+        m /= 64;
+        for (size_t j = 0; j < 64; ++j) q += (ln[i * 64 + j] - m) * (ln[i * 64 + j] - m);
+        EXPECT_NEAR(m, 0.0, 1e-5);
+        EXPECT_NEAR(q / 64, 1.0, 1e-3);
+    }
+    // softmax rows sum to 1 (tests/test_tensor_activations.cpp:11-52); log_softmax = log(softmax)
+    auto sm = host_floats(ops::softmax(a.gpu(), -1)), lsm = host_floats(ops::log_softmax(a.gpu(), -1));
+    for (size_t i = 0; i < 8; ++i) {
+        double s = 0;
+        for (size_t j = 0; j < 64; ++j) s += sm[i * 64 + j];
+        EXPECT_NEAR(s, 1.0, 1e-5);
+    }
+    for (size_t i = 0; i < sm.size(); ++i) EXPECT_NEAR(lsm[i], std::log(sm[i]), 1e-4);
+    EXPECT_NEAR(ops::gelu(Tensor::zeros({4}, DType::Float32, Device::GPU)).cpu().item<float>({0}), 0.0f, 0); // :310-334
+    EXPECT_THROW(ops::softmax(a.gpu(), 0).cpu(), RuntimeError); // only the last axis is on the GPU path
+}
+
+// ---------------------------------------------------------------- parity ops
+GPU_TEST(CpuGpuParity, ElementwiseReductionsMatmul) { // tests/test_cpu_gpu_parity.cpp:12-492 (hot-path ops)
+    auto a = axtest::randn({4, 5}, 41), b = axtest::randn({4, 5}, 42);
+    auto ga = a.gpu(), gb = b.gpu();
+    std::vector<float> want(20);
+    auto check_bin = [&](int op, const Tensor &got) {
+        axo_binary(op, AXO_F32, a.data(), b.data(), want.data(), 4, 5, AXO_BK_FULL);
+        auto g = host_floats(got);
+        for (size_t i = 0; i < 20; ++i) EXPECT_NEAR(g[i], want[i], 1e-5 + 1e-5 * std::fabs(want[i]));
+    };
+    check_bin(AXO_OP_ADD, ga + gb);
+    check_bin(AXO_OP_SUB, ga - gb);
+    check_bin(AXO_OP_MUL, ga * gb);
+    check_bin(AXO_OP_DIV, ga / gb);
+    check_bin(AXO_OP_MAX, ops::maximum(ga, gb));
+    auto check_un = [&](int op, const Tensor &got, const Tensor &src) {
+        axo_unary(op, AXO_F32, src.data(), want.data(), 20);
+        auto g = host_floats(got);
+        for (size_t i = 0; i < 20; ++i) EXPECT_NEAR(g[i], want[i], 1e-5 + 1e-5 * std::fabs(want[i]));
+    };
+    check_un(AXO_OP_EXP, ops::exp(ga), a);
+    check_un(AXO_OP_TANH, ops::tanh(ga), a);
+    check_un(AXO_OP_SIGMOID, ops::sigmoid(ga), a);
+    check_un(AXO_OP_SILU, ops::silu(ga), a);
+    check_un(AXO_OP_GELU, ops::gelu(ga), a);
+    check_un(AXO_OP_NEG, ops::negate(ga), a);
+    std::vector<float> rs(4);
+    axo_reduce_last(AXO_RED_SUM, AXO_F32, a.data(), rs.data(), 4, 5);
+    auto gs = host_floats(ga.sum(-1));
+    auto gm = host_floats(ga.mean(-1, true));
+    EXPECT_EQ(ga.mean(-1, true).shape(), Shape({4, 1}));
+    for (size_t i = 0; i < 4; ++i) {
+        EXPECT_NEAR(gs[i], rs[i], 1e-5);
+        EXPECT_NEAR(gm[i], rs[i] / 5, 1e-5);
+    }
+    axo_reduce_last(AXO_RED_MAX, AXO_F32, a.data(), rs.data(), 4, 5);
+    auto gx = host_floats(ga.max(-1));
+    for (size_t i = 0; i < 4; ++i) EXPECT_NEAR(gx[i], rs[i], 0);
+    // matmul against the oracle's sgemm
+    auto m1 = axtest::randn({7, 12}, 43), m2 = axtest::randn({12, 9}, 44);
+    std::vector<float> mm(63);
+    axo_matmul(AXO_F32, m1.data(), m2.data(), mm.data(), 7, 9, 12, 0, 0);
+    auto gmm = host_floats(ops::matmul(m1.gpu(), m2.gpu()));
+    for (size_t i = 0; i < 63; ++i) EXPECT_NEAR(gmm[i], mm[i], 1e-4 + 1e-4 * std::fabs(mm[i]));
+    auto gmt = host_floats(ops::matmul(m1.gpu(), m2.transpose({1, 0}).ascontiguousarray().gpu(), false, true));
+    for (size_t i = 0; i < 63; ++i) EXPECT_NEAR(gmt[i], mm[i], 1e-4 + 1e-4 * std::fabs(mm[i]));
+    EXPECT_THROW(ops::sum(axtest::randn({3, 4, 5}, 1).gpu(), {1}).cpu(), RuntimeError); // middle-axis reduction: not on the path
+}
+
+// ----------------------------------------------------------------- attention
+static std::tuple<Tensor, Tensor, Tensor> make_inputs(size_t B, size_t H, size_t Sq, size_t Skv, size_t D, DType dt = DType::Float32, uint64_t seed = 42) {
+    return {axtest::randn({B, H, Sq, D}, seed, dt), axtest::randn({B, H, Skv, D}, seed + 1, dt), axtest::randn({B, H, Skv, D}, seed + 2, dt)};
+}
+
+GPU_TEST(FlashAttentionGPU, ShapeCasesFloat32MatchCpuPath) { // tests/test_flash_attention.cpp:76-213, 219-277, 334-355
+    struct Case { size_t B, H, Sq, Skv, D; bool causal; float scale; };
+    const Case cases[] = {{1, 2, 8, 8, 32, false, -1}, {1, 2, 16, 32, 32, false, -1}, {1, 2, 16, 16, 32, true, -1}, {1, 1, 37, 37, 32, false, -1},
+                          {1, 2, 256, 256, 64, false, -1}, {1, 1, 16, 16, 128, false, -1}, {1, 2, 16, 16, 32, false, 0.5f}, {4, 8, 16, 16, 32, false, -1},
+                          {1, 1, 1, 1, 32, false, -1}, {1, 2, 16, 16, 48, false, -1}, {2, 4, 32, 32, 64, false, 0.125f}};
+    for (const Case &c : cases) {
+        auto [q, k, v] = make_inputs(c.B, c.H, c.Sq, c.Skv, c.D);
+        auto cpu_result = axtest::oracle_sdpa(q, k, v, Tensor(), c.scale, c.causal);
+        auto gpu_result = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), c.scale, c.causal);
+        EXPECT_EQ(gpu_result.shape(), q.shape());
+        ASSERT_TENSORS_CLOSE(gpu_result.cpu(), cpu_result, 1e-4, 1e-4);
+    }
+}
+GPU_TEST(FlashAttentionGPU, BoolMasks) { // tests/test_flash_attention.cpp (mask (i+j)%3==0), tests/test_nn_attention.cpp:131-165
+    auto [q, k, v] = make_inputs(2, 2, 16, 16, 32);
+    Tensor m2({16, 16}, DType::Bool), m4({2, 1, 16, 16}, DType::Bool);
+    for (size_t i = 0; i < 16; ++i)
+        for (size_t j = 0; j < 16; ++j) {
+            m2.set_item<int>({i, j}, (i + j) % 3 == 0);
+            m4.set_item<int>({0, 0, i, j}, (i + j) % 3 == 0);
+            m4.set_item<int>({1, 0, i, j}, j > i + 2);
+        }
+    ASSERT_TENSORS_CLOSE(ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), m2.gpu(), -1, false).cpu(), axtest::oracle_sdpa(q, k, v, m2, -1, false), 1e-4, 1e-4);
+    ASSERT_TENSORS_CLOSE(ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), m4, -1, false).cpu(), axtest::oracle_sdpa(q, k, v, m4, -1, false), 1e-4, 1e-4); // host mask is moved over
+    EXPECT_THROW(ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor::zeros({8, 8}, DType::Bool), -1, false), ShapeError);
+}
+GPU_TEST(FlashAttentionGPU, HalfTypesRunOnMfma) { // tests/test_flash_attention.cpp:233-249 (vs f32 computation of the same inputs)
+    for (DType dt : {DType::Float16, DType::BFloat16})
+        for (size_t D : {size_t(32), size_t(64), size_t(128)})
+            for (bool causal : {false, true}) {
+                auto [q, k, v] = make_inputs(1, 2, 200, 200, D, dt);
+                auto ref = axtest::oracle_sdpa(q.astype(DType::Float32), k.astype(DType::Float32), v.astype(DType::Float32), Tensor(), -1, causal);
+                auto got = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), -1, causal);
+                EXPECT_EQ(got.dtype(), dt);
+                EXPECT_EQ(std::string(ops::last_sdpa_kernel()).substr(0, 5), std::string("mfma_"));
+                EXPECT_LE(max_abs_diff(got, ref), 2e-2);
+            }
+}
+GPU_TEST(FlashAttentionGPU, Config1Float32) { // BASELINE configs[0]: B1 H8 S512 D64, no mask, scale 0.125
+    auto [q, k, v] = make_inputs(1, 8, 512, 512, 64);
+    auto got = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), 0.125f, false);
+    ASSERT_TENSORS_CLOSE(got.cpu(), axtest::oracle_sdpa(q, k, v, Tensor(), 0.125f, false), 1e-4, 1e-4);
+}
+
+// ------------------------------------------------------------------------ nn
+GPU_TEST(NNLayers, LinearKnownAnswers) { // tests/test_nn_layers.cpp:12-73
+    nn::Linear lin;
+    lin.load_state_dict({{"weight", Tensor::ones({2, 3})}, {"bias", Tensor::zeros({2})}});
+    lin.to(Device::GPU);
+    auto y = lin.forward(Tensor::ones({1, 3}, DType::Float32, Device::GPU)).cpu();
+    EXPECT_EQ(y.shape(), Shape({1, 2}));
+    EXPECT_NEAR(y.item<float>({0, 0}), 3.0f, 1e-5);
+    lin.load_state_dict({{"weight", Tensor::ones({2, 3}, DType::Float32, Device::GPU)}, {"bias", Tensor::ones({2}, DType::Float32, Device::GPU)}});
+    EXPECT_NEAR(lin.forward(Tensor::ones({1, 3}, DType::Float32, Device::GPU)).cpu().item<float>({0, 1}), 4.0f, 1e-5);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u); // bias rides in the GEMM epilogue
+    nn::Linear nob(false);
+    nob.load_state_dict({{"weight", Tensor::ones({4, 2}, DType::Float32, Device::GPU)}});
+    auto yb = nob.forward(Tensor::ones({5, 3, 2}, DType::Float32, Device::GPU)).cpu(); // batched input
+    EXPECT_EQ(yb.shape(), Shape({5, 3, 4}));
+    EXPECT_NEAR(yb.item<float>({4, 2, 3}), 2.0f, 1e-5);
+}
+GPU_TEST(NNLayers, NormModules) { // tests/test_nn_layers.cpp:191-207
+    nn::RMSNorm rms;
+    rms.load_state_dict({{"weight", Tensor::ones({4})}});
+    rms.to(Device::GPU);
+    float v[4] = {1, 2, 3, 4};
+    auto y = rms.forward(Tensor::from_data(v, {1, 4}, Device::GPU)).cpu();
+    EXPECT_NEAR(y.item<float>({0, 0}), 1.0f / std::sqrt(7.5f), 1e-4);
+    nn::LayerNorm ln;
+    ln.load_state_dict({{"weight", Tensor::ones({4})}, {"bias", Tensor::zeros({4})}});
+    ln.to(Device::GPU).to(DType::Float32);
+    auto z = host_floats(ln.forward(Tensor::from_data(v, {1, 4}, Device::GPU)));
+    EXPECT_NEAR(z[0] + z[1] + z[2] + z[3], 0.0, 1e-5);
+    EXPECT_NEAR(z[3], 1.5 / std::sqrt(1.25 + 1e-5), 1e-4);
+}
+GPU_TEST(FlashAttentionMHA, UniformInputIdentityProjections) { // tests/test_flash_attention.cpp:283-328, test_nn_attention.cpp:68-92
+    nn::MultiHeadAttention mha(1);
+    const size_t d = 2;
+    std::map<std::string, Tensor> state;
+    for (const char *p : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+        state[std::string(p) + ".weight"] = Tensor::eye(d);
+        state[std::string(p) + ".bias"] = Tensor::zeros({d});
+    }
+    mha.load_state_dict(state);
+    mha.to(Device::GPU);
+    auto input = Tensor::ones({1, 3, 2}, DType::Float32, Device::GPU);
+    auto out = mha.forward(input, input, input).cpu();
+    EXPECT_EQ(out.shape(), Shape({1, 3, 2}));
+    for (size_t i = 0; i < 3; ++i)
+        for (size_t j = 0; j < 2; ++j) EXPECT_NEAR(out.item<float>({0, i, j}), 1.0f, 1e-5);
+    auto causal = mha.forward(input, input, input, Tensor(), true).cpu();
+    EXPECT_NEAR(causal.item<float>({0, 2, 1}), 1.0f, 1e-5);
+}
+
+// BASELINE configs[4]: Whisper-style encoder self-attention block, here at S=150 for the exact
+// comparison (the full S=1500 size is covered by properties below)
+static Tensor whisper_block(const Tensor &x, nn::MultiHeadAttention &mha, nn::LayerNorm &ln) { return ln.forward(x + mha.forward(x, x, x)); }
+
+static void whisper_case(size_t S, bool compare) {
+    const size_t Dm = 1280, H = 20, Dh = 64;
+    const DType dt = DType::BFloat16;
+    auto x = axtest::randn({1, S, Dm}, 51, dt);
+    std::map<std::string, Tensor> w;
+    uint64_t seed = 60;
+    for (const char *p : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+        w[std::string(p) + ".weight"] = axtest::randn({Dm, Dm}, seed++, dt, 0.02f);
+        w[std::string(p) + ".bias"] = Tensor::zeros({Dm}, dt);
+    }
+    nn::MultiHeadAttention mha(static_cast<int>(H));
+    mha.load_state_dict(w);
+    mha.to(Device::GPU);
+    nn::LayerNorm ln;
+    ln.load_state_dict({{"weight", Tensor::ones({Dm}, dt)}, {"bias", Tensor::zeros({Dm}, dt)}});
+    ln.to(Device::GPU);
+    auto y = whisper_block(x.gpu(), mha, ln);
+    EXPECT_EQ(y.dtype(), dt);
+    EXPECT_EQ(y.shape(), Shape({1, S, Dm}));
+    auto got = host_floats(y);
+    EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("mfma_bf16_d64"));
+    // layer-norm output: every row has mean ~ 0 and variance ~ 1
+    for (size_t r : {size_t(0), S / 2, S - 1}) {
+        double m = 0, q = 0;
+        for (size_t j = 0; j < Dm; ++j) m += got[r * Dm + j];
+        m /= Dm;
+        for (size_t j = 0; j < Dm; ++j) q += (got[r * Dm + j] - m) * (got[r * Dm + j] - m);
+        EXPECT_NEAR(m, 0.0, 2e-2);
+        EXPECT_NEAR(q / Dm, 1.0, 5e-2);
+    }
+    if (!compare) return;
+    // fp32 evaluation of the same bf16 inputs with the oracle's pieces
+    auto xf = x.astype(DType::Float32);
+    auto proj = [&](const Tensor &in, const char *name) {
+        Tensor wf = w[std::string(name) + ".weight"].astype(DType::Float32), out({S, Dm}, DType::Float32);
+        axo_matmul(AXO_F32, in.data(), wf.data(), out.data(), S, Dm, Dm, 0, 1);
+        return out;
+    };
+    auto split = [&](const Tensor &t) { return t.reshape({1, S, H, Dh}).transpose({0, 2, 1, 3}).ascontiguousarray(); };
+    Tensor x2 = xf.reshape({S, Dm});
+    auto att = axtest::oracle_sdpa(split(proj(x2, "q_proj")), split(proj(x2, "k_proj")), split(proj(x2, "v_proj")), Tensor(), -1, false);
+    Tensor merged = att.transpose({0, 2, 1, 3}).ascontiguousarray().reshape({S, Dm});
+    Tensor o = proj(merged, "out_proj");
+    std::vector<float> res(S * Dm), want(S * Dm);
+    for (size_t i = 0; i < S * Dm; ++i) res[i] = o.typed_data<float>()[i] + x2.typed_data<float>()[i];
+    axo_layer_norm(AXO_F32, res.data(), nullptr, nullptr, want.data(), S, Dm, 1e-5f);
+    double worst = 0;
+    for (size_t i = 0; i < S * Dm; ++i) worst = std::max(worst, std::fabs(double(got[i]) - want[i]));
+    EXPECT_LE(worst, 6e-2); // bf16 ulp at |y| ~ 4 is 3e-2: two roundings (residual, output) stay inside 6e-2
+    size_t beyond = 0;
+    for (size_t i = 0; i < S * Dm; ++i) beyond += std::fabs(double(got[i]) - want[i]) > 2e-2;
+    EXPECT_LE(double(beyond) / (S * Dm), 0.01); // 2e-2 holds for all but the largest-magnitude outputs
+}
+GPU_TEST(WhisperBlock, ReducedSequenceMatchesFp32Reference) { whisper_case(150, true); }
+GPU_TEST(WhisperBlock, FullSizeProperties) { whisper_case(1500, false); }

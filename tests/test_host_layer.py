@@ -1,0 +1,51 @@
+"""Runs the C++ test program of the host layer (axiom_amd/host/tests): the cases that
+mirror the reference's GoogleTest files.  Device-free cases run everywhere; GPU cases
+go through libaxiom_hip.so -> libaxhip.so on the card and take their expected values
+from the oracle linked into the test program only."""
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+LIB = ROOT / "axiom_amd" / "lib"
+BIN = LIB / "host_tests"
+
+
+def _ensure_built():
+    if not BIN.exists():  # normally built beforehand by __graft_entry__.build()
+        from axiom_amd import build_host
+        from oracle import axo
+
+        axo.build()
+        build_host.build_all()
+
+
+def _run(*args, timeout=600):
+    _ensure_built()
+    p = subprocess.run([str(BIN), *args], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
+    print(p.stdout[-6000:])
+    return p
+
+
+def test_host_cases_without_device():
+    p = _run("--cpu")
+    assert p.returncode == 0, p.stdout[-3000:]
+    assert " 0 failed" in p.stdout
+
+
+def test_product_libraries_do_not_link_the_oracle():
+    _ensure_built()
+    for lib in ("libaxhip.so", "libaxiom_hip.so"):
+        out = subprocess.run(["readelf", "-d", str(LIB / lib)], stdout=subprocess.PIPE, text=True, check=True).stdout
+        needed = [l for l in out.splitlines() if "NEEDED" in l]
+        assert not any("oracle" in l for l in needed), needed
+    out = subprocess.run(["readelf", "-d", str(LIB / "libaxiom_hip.so")], stdout=subprocess.PIPE, text=True, check=True).stdout
+    assert "libaxhip.so" in out  # the host layer sits on the C ABI
+
+
+@pytest.mark.gpu
+def test_host_cases_on_gpu():
+    p = _run("--gpu")
+    assert p.returncode == 0, p.stdout[-6000:]
+    assert " 0 failed" in p.stdout and " 0 skipped" in p.stdout
