@@ -12,6 +12,11 @@ fused-chain kernels' achieved HBM bandwidth (configs[1] and configs[2]) and a
 CPU baseline (the oracle's restatement of Axiom's CPU algorithm, timed on this
 host on a bounded sample).
 
+The defaults (50 warm-up, 200 timed launches per kernel) are sized for the device's clock
+governor: coming from idle the first ~20 ms of MFMA work run at reduced clocks (the same SDPA
+launch measures ~650 us in a 5+20 run and ~550 us from the 50th launch on), so a short run
+reports the ramp, not the kernel.
+
 Everything runs on ONE GPU; --gpus above 1 is refused.
 """
 from __future__ import annotations
@@ -39,12 +44,23 @@ CHAIN_TRAFFIC_BYTES = {"chain_relu_add_mul_softmax_sum_f32_8192x8192": 537.2e6,
                        "chain_gelu_rmsnorm_bf16_16384x4096": 269.2e6}
 
 
+MIN_WARMUP_MS = 30.0  # the clock governor needs about this much work of one kind to settle
+
+
 def time_launches(torch, stream, launch, steps: int, warmup: int):
-    """Average launch duration in ms over `steps` launches, HIP events on `stream`."""
+    """Average launch duration in ms over `steps` launches, HIP events on `stream`.
+    Warm-up: `warmup` launches, continued until MIN_WARMUP_MS of work has run (short kernels
+    would otherwise be timed while the device is still changing clocks)."""
     with torch.cuda.stream(stream):
+        t0 = time.time()
         for _ in range(warmup):
             launch()
         stream.synchronize()
+        spent_ms = (time.time() - t0) * 1e3
+        if warmup > 0 and spent_ms < MIN_WARMUP_MS:
+            for _ in range(int((MIN_WARMUP_MS - spent_ms) / (spent_ms / warmup)) + 1):
+                launch()
+            stream.synchronize()
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         evs[0].record(stream)
         for i in range(steps):
@@ -201,8 +217,8 @@ def cpu_baseline(seconds_budget: float = 20.0):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["sdpa", "chains"], default=None)
     args = ap.parse_args()
