@@ -2,6 +2,7 @@
 
     libaxiom_hip.so     Axiom's Tensor / ops / lazy graph / nn interface for the hot path,
                         over the C ABI of libaxhip.so (no CPU compute, no fallback)
+    host_bench          times BASELINE's configurations along the whole host-layer path
     host_tests          test program; links the host layer and, as the checker only, the
                         CPU oracle (oracle/libaxiom_oracle.so)
 """
@@ -21,6 +22,7 @@ LIB_DIR = PKG / "lib"
 OBJ_DIR = PKG / "build" / "host"
 HOST_LIB = LIB_DIR / "libaxiom_hip.so"
 TEST_BIN = LIB_DIR / "host_tests"
+BENCH_BIN = LIB_DIR / "host_bench"
 
 CXXFLAGS = ["-O2", "-g", "-std=c++20", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
             f"-I{HOST / 'include'}", f"-I{HOST / 'src'}", f"-I{ROOT / 'include'}"]
@@ -63,6 +65,9 @@ def build_all(verbose: bool = True) -> None:
         oracle_dir = ROOT / "oracle"
         _run([cxx, "-o", str(TEST_BIN), *map(str, tobjs), f"-L{LIB_DIR}", "-laxiom_hip", "-laxhip", f"-L{oracle_dir}", "-laxiom_oracle",
               "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,$ORIGIN/../../oracle", "-lpthread"], "link host_tests")
+    bench = HOST / "bench" / "host_bench.cpp"
+    if bench.exists():
+        _run([cxx, *CXXFLAGS, str(bench), "-o", str(BENCH_BIN), f"-L{LIB_DIR}", "-laxiom_hip", "-laxhip", "-Wl,-rpath,$ORIGIN"], "build host_bench")
     if verbose:
         print(f"[axiom_amd.build_host] built {HOST_LIB.name}" + (f" and {TEST_BIN.name}" if tests else "") + f" ({time.time() - t0:.1f}s)", flush=True)
 

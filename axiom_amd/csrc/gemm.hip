@@ -2,8 +2,9 @@
 //
 //   gemm_mfma_nt_kernel   bf16 / f16, A [M,K] and B [N,K] both K-contiguous (the
 //                         nn::Linear case x W^T): v_mfma_f32_32x32x16, workgroup
-//                         tile 128x128x64, 4 waves each owning a 64x64 quadrant,
-//                         A/B tiles staged through LDS, fp32 accumulation.
+//                         tile 128x128x64 or 64x128x64, 4 waves, A/B tiles staged
+//                         through LDS with up to three k-tiles in flight, fp32
+//                         accumulation.
 //   gemm_generic_kernel   any dtype / any transpose combination, 16x16 LDS tiles,
 //                         fp32 FMA.
 #include "common.hpp"
@@ -58,69 +59,71 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const GemmArgs g) {
 }
 
 // ------------------------------------------------------------------- MFMA NT
-constexpr int TM = 128, TN = 128, TK = 64;
+// Work-group tile BM x 128 x 64 (BM = 128 or 64), 4 waves in a 2 x 2 layout, each
+// owning a (BM/2) x 64 block of C as 32x32 MFMA tiles.  A and B k-tiles travel
+// HBM/L2 -> registers -> LDS; NPRE k-tiles are in flight in registers at any
+// time, which is what hides the load latency when a small problem leaves one
+// work-group per CU (the nn::Linear shapes of a single sequence).  The k loop is
+// unrolled NPRE times so that each in-flight tile has its own registers.
+constexpr int TN = 128, TK = 64;
 constexpr int LDS_STRIDE = TK + 8; // 144 B rows: consecutive rows shift by 4 banks (+32)
 
-template <bool BF16>
-__global__ __launch_bounds__(256, 2) void gemm_mfma_nt_kernel(const GemmArgs g) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[TM * LDS_STRIDE];
+template <bool BF16, int BM, int NPRE>
+__global__ __launch_bounds__(256, BM == 128 ? 2 : 1) void gemm_mfma_nt_kernel(const GemmArgs g) {
+    constexpr int MI = BM / 64;  // 32-row MFMA tiles per wave in M
+    constexpr int NA = BM / 32;  // 16-byte chunks of A per thread per k-tile (BM rows x 8 chunks / 256 threads)
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[TN * LDS_STRIDE];
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int l32 = lane % 32, g2 = lane / 32;
-    const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
-    const int64_t m0 = static_cast<int64_t>(blockIdx.y) * TM, n0 = static_cast<int64_t>(blockIdx.x) * TN;
+    const int wm = (wave / 2) * (BM / 2), wn = (wave % 2) * 64;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM, n0 = static_cast<int64_t>(blockIdx.x) * TN;
     const int64_t bz = blockIdx.z;
     const uint16_t *A = static_cast<const uint16_t *>(g.a) + bz * g.sa;
     const uint16_t *B = static_cast<const uint16_t *>(g.b) + bz * g.sb;
 
-    float16_t acc[2][2];
+    float16_t acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    // each thread moves 4 16-byte chunks of A and of B per k-tile: 128 rows x 8 chunks
-    uint4_t ra[4], rb[4];
-    auto load_tiles = [&](int64_t k0) {
+    uint4_t ra[NPRE][NA], rb[NPRE][4];
+    auto load_tiles = [&](int s, int64_t k0) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int id = tid + 256 * i;
             const int row = id / 8, cc = id % 8;
             const int64_t k = k0 + 8 * cc;
-            ra[i] = uint4_t{0, 0, 0, 0};
-            rb[i] = uint4_t{0, 0, 0, 0};
-            if (m0 + row < g.M && k < g.K) ra[i] = *reinterpret_cast<const uint4_t *>(A + (m0 + row) * g.a_rs + k);
-            if (n0 + row < g.N && k < g.K) rb[i] = *reinterpret_cast<const uint4_t *>(B + (n0 + row) * g.b_cs + k);
+            if (i < NA) {
+                ra[s][i < NA ? i : 0] = uint4_t{0, 0, 0, 0};
+                if (m0 + row < g.M && k < g.K) ra[s][i < NA ? i : 0] = *reinterpret_cast<const uint4_t *>(A + (m0 + row) * g.a_rs + k);
+            }
+            rb[s][i] = uint4_t{0, 0, 0, 0};
+            if (n0 + row < g.N && k < g.K) rb[s][i] = *reinterpret_cast<const uint4_t *>(B + (n0 + row) * g.b_cs + k);
         }
     };
-    auto stage_tiles = [&]() {
+    auto stage_tiles = [&](int s) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int id = tid + 256 * i;
             const int row = id / 8, cc = id % 8;
-            *reinterpret_cast<uint4_t *>(&As[row * LDS_STRIDE + 8 * cc]) = ra[i];
-            *reinterpret_cast<uint4_t *>(&Bs[row * LDS_STRIDE + 8 * cc]) = rb[i];
+            if (i < NA) *reinterpret_cast<uint4_t *>(&As[row * LDS_STRIDE + 8 * cc]) = ra[s][i < NA ? i : 0];
+            *reinterpret_cast<uint4_t *>(&Bs[row * LDS_STRIDE + 8 * cc]) = rb[s][i];
         }
     };
-
-    load_tiles(0);
-    for (int64_t k0 = 0; k0 < g.K; k0 += TK) {
-        __syncthreads();
-        stage_tiles();
-        __syncthreads();
-        if (k0 + TK < g.K) load_tiles(k0 + TK);
+    auto multiply_tile = [&]() {
 #pragma unroll
         for (int ks = 0; ks < TK / 16; ++ks) {
-            uint4_t af[2], bf[2];
+            uint4_t af[MI], bf[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                af[i] = *reinterpret_cast<const uint4_t *>(&As[(wm + 32 * i + l32) * LDS_STRIDE + 16 * ks + 8 * g2]);
-                bf[i] = *reinterpret_cast<const uint4_t *>(&Bs[(wn + 32 * i + l32) * LDS_STRIDE + 16 * ks + 8 * g2]);
-            }
+            for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const uint4_t *>(&As[(wm + 32 * i + l32) * LDS_STRIDE + 16 * ks + 8 * g2]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const uint4_t *>(&Bs[(wn + 32 * j + l32) * LDS_STRIDE + 16 * ks + 8 * g2]);
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     if constexpr (BF16)
@@ -129,12 +132,29 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_nt_kernel(const GemmArgs g) 
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[i]), __builtin_bit_cast(half8_t, bf[j]), acc[i][j], 0, 0, 0);
                 }
         }
+    };
+
+#pragma unroll
+    for (int s = 0; s < NPRE; ++s)
+        if (static_cast<int64_t>(s) * TK < g.K) load_tiles(s, static_cast<int64_t>(s) * TK);
+    for (int64_t k0 = 0; k0 < g.K; k0 += NPRE * TK) {
+#pragma unroll
+        for (int s = 0; s < NPRE; ++s) {
+            const int64_t k = k0 + static_cast<int64_t>(s) * TK;
+            if (k < g.K) {
+                __syncthreads(); // every wave is done reading the previous tile
+                stage_tiles(s);
+                __syncthreads();
+                if (k + NPRE * TK < g.K) load_tiles(s, k + NPRE * TK);
+                multiply_tile();
+            }
+        }
     }
 
     // accumulator element e of tile (i, j): row = 8*(e/4) + 4*g2 + e%4, col = l32
     const int64_t coff = bz * g.sc;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int64_t n = n0 + wn + 32 * j + l32;
@@ -184,9 +204,19 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     const bool nt = !p.trans_a && p.trans_b && p.k % 8 == 0 && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.stride_a % 8 == 0 &&
                     p.stride_b % 8 == 0 && al16(a) && al16(b);
     if (half && nt && p.k > 0) {
-        dim3 grid(static_cast<unsigned>((p.n + TN - 1) / TN), static_cast<unsigned>((p.m + TM - 1) / TM), static_cast<unsigned>(p.batch));
-        if (p.dtype == AXHIP_DTYPE_BF16) hipLaunchKernelGGL(gemm_mfma_nt_kernel<true>, grid, dim3(256), 0, s, g);
-        else hipLaunchKernelGGL(gemm_mfma_nt_kernel<false>, grid, dim3(256), 0, s, g);
+        // Tall tiles (two work-groups per CU, one k-tile in flight) once they fill the chip;
+        // otherwise 64-row tiles, one work-group per CU with three k-tiles in flight.
+        const int64_t tiles128 = ((p.n + TN - 1) / TN) * ((p.m + 127) / 128) * p.batch;
+        const bool bf = p.dtype == AXHIP_DTYPE_BF16;
+        if (tiles128 >= 512) {
+            dim3 grid(static_cast<unsigned>((p.n + TN - 1) / TN), static_cast<unsigned>((p.m + 127) / 128), static_cast<unsigned>(p.batch));
+            if (bf) hipLaunchKernelGGL((gemm_mfma_nt_kernel<true, 128, 1>), grid, dim3(256), 0, s, g);
+            else hipLaunchKernelGGL((gemm_mfma_nt_kernel<false, 128, 1>), grid, dim3(256), 0, s, g);
+        } else {
+            dim3 grid(static_cast<unsigned>((p.n + TN - 1) / TN), static_cast<unsigned>((p.m + 63) / 64), static_cast<unsigned>(p.batch));
+            if (bf) hipLaunchKernelGGL((gemm_mfma_nt_kernel<true, 64, 3>), grid, dim3(256), 0, s, g);
+            else hipLaunchKernelGGL((gemm_mfma_nt_kernel<false, 64, 3>), grid, dim3(256), 0, s, g);
+        }
     } else {
         dim3 grid(static_cast<unsigned>((p.n + 15) / 16), static_cast<unsigned>((p.m + 15) / 16), static_cast<unsigned>(p.batch));
         AXHIP_REQUIRE(grid.y < 65536, AXHIP_ERR_UNSUPPORTED, "axhip_gemm: m too large for the generic kernel");

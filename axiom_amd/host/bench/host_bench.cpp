@@ -1,0 +1,78 @@
+// Times BASELINE's configurations through the host layer, i.e. along the whole drop-in path:
+// lazy graph construction, signature, plan cache, kernel launches, with a device
+// synchronisation closing every materialisation (the reference's fusion benchmark
+// materialises through item(): benchmarks/core/fusion/fusion_benchmark.cpp:38-49, 62-72).
+// Prints one JSON object.  Inputs are synthetic and resident on the GPU before timing.
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "axiom/axiom.hpp"
+
+using namespace axiom;
+using Clock = std::chrono::steady_clock;
+
+template <typename F> static void measure(const char *name, F f, int warmup, int iters, double work, const char *unit, bool last) {
+    for (int i = 0; i < warmup; ++i) f();
+    backends::hip::synchronize();
+    std::vector<double> us;
+    for (int i = 0; i < iters; ++i) {
+        const auto t0 = Clock::now();
+        f();
+        backends::hip::synchronize();
+        us.push_back(std::chrono::duration<double, std::micro>(Clock::now() - t0).count());
+    }
+    std::sort(us.begin(), us.end());
+    const double med = us[us.size() / 2];
+    std::string kernels;
+    for (const auto &k : graph::last_gpu_plan_kernels()) kernels += (kernels.empty() ? "" : " ") + k;
+    std::printf("  \"%s\": {\"median_us\": %.1f, \"min_us\": %.1f, \"%s\": %.1f, \"last_graph_kernels\": \"%s\"}%s\n", name, med, us.front(), unit,
+                work / (med * 1e-6) / 1e9, kernels.c_str(), last ? "" : ",");
+}
+
+int main(int argc, char **argv) {
+    const int iters = argc > 1 ? std::atoi(argv[1]) : 50, warmup = argc > 2 ? std::atoi(argv[2]) : 10;
+    if (!system::is_gpu_available()) {
+        std::fprintf(stderr, "host_bench: no GPU visible; the gfx950 backend has no CPU fallback\n");
+        return 3;
+    }
+    Tensor::manual_seed(42);
+    std::printf("{\n");
+    { // configs[1]
+        auto a = Tensor::randn({8192, 8192}, DType::Float32, Device::GPU), b = Tensor::randn({8192, 8192}, DType::Float32, Device::GPU);
+        measure("c2_chain_f32_8192x8192", [&] { ops::softmax((ops::relu(a) + 1) * b, -1).sum(1).sync(); }, warmup, iters, 536903680.0, "GB_per_s", false);
+    }
+    { // configs[2]
+        auto x = Tensor::randn({16384, 4096}, DType::BFloat16, Device::GPU);
+        auto gamma = Tensor::uniform(0.5, 1.5, {4096}, DType::BFloat16, Device::GPU), beta = Tensor::uniform(-0.1, 0.1, {4096}, DType::BFloat16, Device::GPU);
+        measure("c3_gelu_layernorm_bf16_16384x4096", [&] { ops::gelu(ops::layer_norm(x, gamma, beta, -1, 1e-5f)).sync(); }, warmup, iters, 268451840.0, "GB_per_s", false);
+        measure("c3_gelu_rmsnorm_bf16_16384x4096", [&] { ops::gelu(ops::rms_norm(x, gamma, -1, 1e-5f)).sync(); }, warmup, iters, 268443648.0, "GB_per_s", false);
+    }
+    { // configs[3]
+        auto q = Tensor::randn({4, 32, 4096, 128}, DType::BFloat16, Device::GPU), k = Tensor::randn({4, 32, 4096, 128}, DType::BFloat16, Device::GPU),
+             v = Tensor::randn({4, 32, 4096, 128}, DType::BFloat16, Device::GPU);
+        measure("c4_sdpa_bf16_causal_b4h32s4096d128", [&] { ops::scaled_dot_product_attention(q, k, v, Tensor(), -1.0f, true).sync(); }, warmup, iters, 549755813888.0,
+                "GFLOP_per_s", false);
+    }
+    { // configs[4]: y = LN(x + out_proj(SDPA(split(q, k, v))))
+        const size_t S = 1500, Dm = 1280;
+        auto x = Tensor::randn({1, S, Dm}, DType::BFloat16, Device::GPU);
+        std::map<std::string, Tensor> w;
+        for (const char *p : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+            w[std::string(p) + ".weight"] = (Tensor::randn({Dm, Dm}, DType::Float32, Device::GPU) * 0.02f).astype(DType::BFloat16);
+            w[std::string(p) + ".bias"] = Tensor::zeros({Dm}, DType::BFloat16);
+        }
+        nn::MultiHeadAttention mha(20);
+        mha.load_state_dict(w);
+        mha.to(Device::GPU);
+        nn::LayerNorm ln;
+        ln.load_state_dict({{"weight", Tensor::ones({Dm}, DType::BFloat16)}, {"bias", Tensor::zeros({Dm}, DType::BFloat16)}});
+        ln.to(Device::GPU);
+        measure("c5_whisper_block_bf16_s1500_d1280_h20", [&] { ln.forward(x + mha.forward(x, x, x)).sync(); }, warmup, iters, 31180800000.0, "GFLOP_per_s", true);
+    }
+    std::printf("}\n");
+    return 0;
+}

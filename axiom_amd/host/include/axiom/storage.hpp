@@ -31,6 +31,9 @@ namespace backends::hip {
 // waits for every kernel and copy queued on the backend stream
 void synchronize();
 bool is_available();
+// device blocks freed by tensors are kept for reuse; this returns them to the driver
+void empty_cache();
+size_t cached_bytes();
 } // namespace backends::hip
 
 } // namespace axiom

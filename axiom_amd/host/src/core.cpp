@@ -3,7 +3,9 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <sstream>
+#include <unordered_map>
 
 #include "axhip.h"
 #include "axiom/dtype.hpp"
@@ -204,6 +206,65 @@ class CpuStorage final : public Storage {
     size_t bytes_;
 };
 
+// Device allocations are recycled: a freed block goes to a size-keyed free list and serves the
+// next request of the same (256-byte rounded) size.  Every kernel and copy of the host layer
+// runs on the backend's one stream, so a block handed out again is only ever touched by work
+// queued AFTER the work of its previous owner: no synchronisation on free, no hipMalloc /
+// hipFree in steady state (each costs far more than a fused row kernel).
+class HipPool {
+  public:
+    static HipPool &instance() {
+        static HipPool *p = new HipPool; // never destroyed: the HIP runtime may be gone at static teardown
+        return *p;
+    }
+    void *allocate(size_t bytes) {
+        const size_t key = round_up(bytes);
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            auto it = free_.find(key);
+            if (it != free_.end()) {
+                void *p = it->second;
+                free_.erase(it);
+                cached_ -= key;
+                return p;
+            }
+        }
+        void *p = nullptr;
+        if (axhip_malloc(&p, key) != 0) { // out of memory: give the cached blocks back and retry
+            release_all();
+            AXHIP_CALL(axhip_malloc(&p, key));
+        }
+        return p;
+    }
+    void deallocate(void *p, size_t bytes) {
+        const size_t key = round_up(bytes);
+        std::lock_guard<std::mutex> lk(mu_);
+        free_.emplace(key, p);
+        cached_ += key;
+    }
+    void release_all() {
+        std::unordered_multimap<size_t, void *> blocks;
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            blocks.swap(free_);
+            cached_ = 0;
+        }
+        if (blocks.empty()) return;
+        axhip_stream_sync(nullptr); // work that still uses a cached block has been queued before this point
+        for (auto &kv : blocks) axhip_free(kv.second);
+    }
+    size_t cached_bytes() {
+        std::lock_guard<std::mutex> lk(mu_);
+        return cached_;
+    }
+
+  private:
+    static size_t round_up(size_t b) { return std::max<size_t>((b + 255) / 256 * 256, 256); }
+    std::mutex mu_;
+    std::unordered_multimap<size_t, void *> free_;
+    size_t cached_ = 0;
+};
+
 // Device memory of the gfx950 backend; the role of MetalStorage
 // (src/backends/metal/metal_storage.mm:54-142) with explicit copies in place of
 // shared memory.
@@ -211,14 +272,10 @@ class HipStorage final : public Storage {
   public:
     explicit HipStorage(size_t bytes) : bytes_(bytes) {
         AXHIP_CALL(axhip_init(0));
-        if (bytes) AXHIP_CALL(axhip_malloc(&ptr_, bytes));
+        if (bytes) ptr_ = HipPool::instance().allocate(bytes);
     }
     ~HipStorage() override {
-        if (ptr_) {
-            // kernels still reading this buffer run on the backend stream: drain it first
-            axhip_stream_sync(nullptr);
-            axhip_free(ptr_);
-        }
+        if (ptr_) HipPool::instance().deallocate(ptr_, bytes_);
     }
     void *data() override { throw DeviceError("GPU storage has no host pointer; call .cpu() first"); }
     const void *data() const override { throw DeviceError("GPU storage has no host pointer; call .cpu() first"); }
@@ -261,6 +318,8 @@ bool is_available() {
     return axhip_device_count(&n) == 0 && n > 0;
 }
 void synchronize() { AXHIP_CALL(axhip_stream_sync(nullptr)); }
+void empty_cache() { HipPool::instance().release_all(); }
+size_t cached_bytes() { return HipPool::instance().cached_bytes(); }
 } // namespace backends::hip
 
 namespace system {

@@ -320,6 +320,7 @@ class PlanBuilder {
         }
 
         size_t operands = 0;
+        int gemm_input = -1; // value of a GEMM that absorbed the pre chain
         std::vector<ChainItem> upper, lower;
         collect(cur, entry, F, upper, AXHIP_MAX_CHAIN, operands);
         const GraphNode *rowop = nullptr;
@@ -331,6 +332,15 @@ class PlanBuilder {
             rowop = cur;
             cur = cur->inputs[0].get();
             collect(cur, nullptr, F, lower, AXHIP_MAX_CHAIN, operands);
+            // bias / residual / activation directly above a matmul ride in the GEMM epilogue, and the
+            // row kernel reads the finished product (Linear -> + x -> LayerNorm is GEMM + one row kernel)
+            if (!lower.empty() && consumable(cur, nullptr) && cur->op_type == OpType::MatMul) {
+                const int g = try_gemm_epilogue(lower.front().node->output_dtype, F, cur, lower, F);
+                if (g >= 0) {
+                    lower.clear();
+                    gemm_input = g;
+                }
+            }
         } else if (upper.empty() && !is_reduction(n->op_type)) {
             // an elementwise node whose two operands are both broadcast: expand the left one and chain through it
             if (!is_binary_ew(n->op_type)) throw RuntimeError::not_implemented(std::string("GPU lazy graph node '") + ops::op_name(n->op_type) + "'");
@@ -340,14 +350,14 @@ class PlanBuilder {
 
         // MatMul feeding a short epilogue chain: one GEMM launch
         if (!rowop && rs.prog.reduce == AXHIP_RED_NONE && consumable(cur, entry) && cur->op_type == OpType::MatMul && !upper.empty()) {
-            const int g = try_gemm_epilogue(n, cur, upper, F);
+            const int g = try_gemm_epilogue(n->output_dtype, n->output_shape, cur, upper, F);
             if (g >= 0) return g;
         }
 
         // the pre chain runs bottom-up: reverse the collected (top-down) lists
         std::reverse(upper.begin(), upper.end());
         std::reverse(lower.begin(), lower.end());
-        int in_v = eval(cur);
+        int in_v = gemm_input >= 0 ? gemm_input : eval(cur);
         if (val(in_v).shape != F) in_v = make_contiguous(in_v, &F);
         in_v = make_contiguous(in_v);
         rs.input = in_v;
@@ -394,7 +404,7 @@ class PlanBuilder {
     }
 
     // [activation] <- [+ residual FULL] <- [+ bias ROWVEC] <- matmul, all in the GEMM's dtype
-    int try_gemm_epilogue(const GraphNode *n, const GraphNode *mm, const std::vector<ChainItem> &top_down, const Shape &F) {
+    int try_gemm_epilogue(DType out_dtype, const Shape &out_shape, const GraphNode *mm, const std::vector<ChainItem> &top_down, const Shape &F) {
         std::vector<ChainItem> ops(top_down.rbegin(), top_down.rend()); // bottom-up
         size_t i = 0;
         const GraphNode *bias = nullptr, *residual = nullptr;
@@ -413,10 +423,10 @@ class PlanBuilder {
             const OpType a = ops[i].node->op_type;
             if (a == OpType::ReLU || a == OpType::GELU || a == OpType::SiLU || a == OpType::Sigmoid || a == OpType::Tanh) act = unary_code(ops[i++].node->op_type);
         }
-        if (i != ops.size() || n->output_dtype != mm->output_dtype) return -1;
+        if (i != ops.size() || out_dtype != mm->output_dtype) return -1;
         const int bias_v = bias ? make_contiguous(eval(bias)) : -1;
         const int res_v = residual ? make_contiguous(eval(residual)) : -1;
-        return emit_gemm(mm, n->output_shape, bias_v, res_v, act);
+        return emit_gemm(mm, out_shape, bias_v, res_v, act);
     }
 
     int emit_gemm(const GraphNode *n, const Shape &out_shape_override, int bias_v, int res_v, int act) {

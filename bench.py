@@ -214,6 +214,21 @@ def cpu_baseline(seconds_budget: float = 20.0):
     }
 
 
+def host_layer_bench():
+    """The same configurations along the whole drop-in path (C++ host layer: lazy graph, plan cache,
+    caching allocator, launches, one device synchronisation per materialisation): wall-clock
+    microseconds per materialisation from axiom_amd/lib/host_bench."""
+    import subprocess
+
+    exe = ROOT / "axiom_amd" / "lib" / "host_bench"
+    if not exe.exists():
+        return {"error": "axiom_amd/lib/host_bench is not built (python -m axiom_amd.build_host)"}
+    p = subprocess.run([str(exe), "100", "20"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    if p.returncode != 0:
+        return {"error": f"host_bench exited with {p.returncode}: {p.stderr[-300:]}"}
+    return json.loads(p.stdout)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -265,6 +280,8 @@ def main() -> int:
             if name in CHAIN_TRAFFIC_BYTES:
                 rec["traffic"] = CHAIN_TRAFFIC_BYTES[name]
         line["fused_chains"] = ch
+    if args.only is None:
+        line["host_layer"] = host_layer_bench()
     if cpu:
         line["cpu_baseline"] = cpu
     line["bench_wall_s"] = time.time() - t_wall0
