@@ -431,11 +431,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
         const int q = qw0 + ql;
         const bool q_ok = q < a.Sq;
 
+        // Q fragments, pre-multiplied by scale * log2(e) (rounded back to the 16-bit type): the
+        // score MFMAs then deliver base-2 logits directly
         uint4_t qf[KT];
     #pragma unroll
         for (int t = 0; t < KT; ++t) {
             qf[t] = uint4_t{0, 0, 0, 0};
             if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
+    #pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t w = qf[t][c];
+                const float lo = BF16 ? bf16_bits_to_f32(w & 0xFFFFu) : f16_bits_to_f32(w & 0xFFFFu);
+                const float hi = BF16 ? bf16_bits_to_f32(w >> 16) : f16_bits_to_f32(w >> 16);
+                qf[t][c] = pack2<BF16>(lo * a.scale_log2e, hi * a.scale_log2e);
+            }
         }
 
         float16_t oacc[DT];
@@ -499,17 +508,27 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
             return row_max(s);
         };
 
-        // Running maximum and the (rare) rescale of the accumulators.
-        auto update_max = [&](float mloc) {
-            const float m_new = __builtin_elementwise_maximum(m_run, mloc * a.scale_log2e);
+        // Running maximum and the (rare) rescale of the accumulators.  The score accumulators of a
+        // tile start at MINUS the reference maximum that was current when its MFMAs were issued, so
+        // `cur` already holds logit - reference and the exponentials need no subtraction; mloc is
+        // the tile's row maximum in that relative form.  When the reference moves, the accumulators
+        // are rescaled and the tile re-referenced.
+        auto update_max = [&](float mloc, float16_t (&cur)[2]) {
+            const float ref = m_run == NEG_INF_F ? 0.0f : m_run;
+            const float m_new = __builtin_elementwise_maximum(m_run, mloc + ref);
             if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
                 const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                const float delta = (m_new == NEG_INF_F ? 0.0f : m_new) - ref;
                 m_run = m_new;
                 l_run *= alpha;
     #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
     #pragma unroll
                     for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+    #pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+    #pragma unroll
+                    for (int i = 0; i < 16; ++i) cur[kt][i] -= delta;
             }
         };
 
@@ -540,8 +559,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
             };
             auto exp_pair = [&](int pr) { // elements 2*pr, 2*pr+1 of the current tile
                 const int kt = pr / 8, i = (pr % 8) * 2;
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i], a.scale_log2e, -m_use));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kt][i + 1], a.scale_log2e, -m_use));
+                const float p0 = __builtin_amdgcn_exp2f(cur[kt][i]);
+                const float p1 = __builtin_amdgcn_exp2f(cur[kt][i + 1]);
                 w[pr] = pack2<BF16>(p0, p1);
                 l_run = add_pair<BF16>(w[pr], l_run);
             };
@@ -553,7 +572,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
                 if (m < 16) {
                     if (m % 8 == 0) {
     #pragma unroll
-                        for (int i = 0; i < 16; ++i) nxt[m / 8][i] = 0.0f;
+                        for (int i = 0; i < 16; ++i) nxt[m / 8][i] = -m_use; // logits come out relative to the reference
                     }
                     nxt[m / 8] = mfma_32x32x16<BF16>(fr[m % RING], qf[m % 8], nxt[m / 8]);
                     if (m % 4 != 3) exp_pair((m / 4) * 3 + m % 4);
@@ -604,7 +623,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
                 const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
                 float mloc = mx_cur;
                 if (need_mask) mloc = mask_and_max(kv0, cur);
-                update_max(mloc);
+                update_max(mloc, cur);
                 // The next tile's scores are issued unconditionally so that they share a basic
                 // block with this tile's softmax; after the last tile (or the last one this wave
                 // needs) they come from a stale K buffer and are never used: ~1.5 % extra MFMAs.
