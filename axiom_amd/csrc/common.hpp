@@ -62,6 +62,15 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); // v_cvt_f16_f32: RNE
 }
 
+// two fp32 values to one packed bf16 pair with the hardware conversion (v_cvt_pk_bf16_f32:
+// round to nearest even; a NaN stays a quiet NaN)
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const float2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
 template <int DT> struct Elem;
 template <> struct Elem<AXHIP_DTYPE_F32> {
     using type = float;
@@ -154,15 +163,11 @@ __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const floa
         uint32_t w[N / 2];
 #pragma unroll
         for (int k = 0; k < N / 2; ++k) {
-            uint32_t lo, hi;
             if (dt == AXHIP_DTYPE_BF16) {
-                lo = f32_to_bf16_bits(v[2 * k]);
-                hi = f32_to_bf16_bits(v[2 * k + 1]);
+                w[k] = pack_bf16x2(v[2 * k], v[2 * k + 1]);
             } else {
-                lo = f32_to_f16_bits(v[2 * k]);
-                hi = f32_to_f16_bits(v[2 * k + 1]);
+                w[k] = f32_to_f16_bits(v[2 * k]) | (f32_to_f16_bits(v[2 * k + 1]) << 16);
             }
-            w[k] = lo | (hi << 16);
         }
         if constexpr (N % 8 == 0) {
             uint4_t *q = reinterpret_cast<uint4_t *>(static_cast<uint16_t *>(p) + i);

@@ -197,8 +197,8 @@ def test_full_size_c2_and_c3_properties():
     g = axo.PCG64(42)
     a, b = g.normal((8192, 8192)), g.normal((8192, 8192))
     p = gh.Rows(a, F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b).row_op("softmax")
-    assert p.kernel_name() == "rows_resident_g256_it8_e4"
     s = p.run(reduce="sum")
+    assert p.kernel_name() == "rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"  # one specialised launch
     assert np.allclose(s, 1.0, atol=1e-4)
     sm = gh.Rows(a[:256], F32).unary("relu").binary("add", ONE, "scalar").binary("mul", b[:256]).row_op("softmax").run()
     _, want_sm = axo.chain_relu_add_mul_softmax_sum(a[:256], b[:256], want_softmax=True)
@@ -214,3 +214,36 @@ def test_full_size_c2_and_c3_properties():
 def test_empty_inputs_are_no_ops():
     x = np.zeros((0, 16), np.float32)
     assert gh.Rows(x, F32).unary("relu").run().shape == (0, 16)
+
+
+def test_mixed_chains_around_row_ops_match_oracle():
+    """Chains that the specialised kernels do not cover (scalar and unary ops before the row op,
+    a reversed subtraction, two full-size operands, a row dot product) run on the interpreter;
+    results match the oracle composed op by op."""
+    g = axo.PCG64(77)
+    x, f = g.normal((48, 2048)), g.normal((48, 2048))
+    half = np.array([0.5], np.float32)
+    # softmax(exp(x * 0.5) - f) * 3 -> row sum
+    p = gh.Rows(x, F32).binary("mul", half, "scalar").unary("exp").binary("sub", f).row_op("softmax").imm("mul", 3.0)
+    got = p.run(reduce="sum")
+    t = axo.binary("sub", axo.unary("exp", axo.binary("mul", x, half, kind="scalar")), f)
+    want = (axo.softmax(t) * np.float32(3.0)).sum(-1)
+    assert close32(got, want)
+    # f - x (chain on the right-hand side), then rms norm, then sigmoid; bf16
+    xb, fb = axo.to_bits(x, BF16), axo.to_bits(f, BF16)
+    w = axo.to_bits(g.uniform((2048,), 0.5, 1.5), BF16)
+    p = gh.Rows(xb, BF16).binary("rsub", fb).row_op("rmsnorm", 1e-5, w=w).unary("sigmoid")
+    got = axo.to_f32(p.run(), BF16)
+    d = (axo.to_f32(fb, BF16) - axo.to_f32(xb, BF16)).astype(np.float64)
+    r = d / np.sqrt((d * d).mean(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16)
+    assert np.max(np.abs(got - 1 / (1 + np.exp(-r)))) < 2e-2
+    # two different full-size operands do not fit the specialised kernels: the interpreter takes over
+    f2 = g.normal((48, 2048))
+    p = gh.Rows(x, F32).binary("add", f).binary("mul", f2).row_op("softmax")
+    got = p.run()
+    assert p.kernel_name().startswith("rows_resident_"), p.kernel_name()
+    assert close32(got, axo.softmax((x + f) * f2))
+    # row dot product: sum(x * f) per row
+    p = gh.Rows(x, F32).binary("mul", f)
+    got = p.run(reduce="sum")
+    assert np.allclose(got, (x.astype(np.float64) * f).sum(-1), rtol=1e-4, atol=1e-3)
