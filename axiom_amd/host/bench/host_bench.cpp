@@ -71,7 +71,22 @@ int main(int argc, char **argv) {
         nn::LayerNorm ln;
         ln.load_state_dict({{"weight", Tensor::ones({Dm}, DType::BFloat16)}, {"bias", Tensor::zeros({Dm}, DType::BFloat16)}});
         ln.to(Device::GPU);
-        measure("c5_whisper_block_bf16_s1500_d1280_h20", [&] { ln.forward(x + mha.forward(x, x, x)).sync(); }, warmup, iters, 31180800000.0, "GFLOP_per_s", true);
+        measure("c5_whisper_block_bf16_s1500_d1280_h20", [&] { ln.forward(x + mha.forward(x, x, x)).sync(); }, warmup, iters, 31180800000.0, "GFLOP_per_s", false);
+        // the whole pre-norm encoder layer of the reference's examples/whisper_poc.cpp:57-86:
+        // LN -> MHA -> +x -> LN -> fc1 -> gelu -> fc2 -> +h   (24*S*D^2 + 4*S^2*D flop)
+        nn::LayerNorm ln2;
+        ln2.load_state_dict({{"weight", Tensor::ones({Dm}, DType::BFloat16)}, {"bias", Tensor::zeros({Dm}, DType::BFloat16)}});
+        ln2.to(Device::GPU);
+        nn::Linear fc1, fc2;
+        fc1.load_state_dict({{"weight", (Tensor::randn({4 * Dm, Dm}, DType::Float32, Device::GPU) * 0.02f).astype(DType::BFloat16)}, {"bias", Tensor::zeros({4 * Dm}, DType::BFloat16, Device::GPU)}});
+        fc2.load_state_dict({{"weight", (Tensor::randn({Dm, 4 * Dm}, DType::Float32, Device::GPU) * 0.02f).astype(DType::BFloat16)}, {"bias", Tensor::zeros({Dm}, DType::BFloat16, Device::GPU)}});
+        auto layer = [&] {
+            auto h = ln(x);
+            h = x + mha.forward(h, h, h);
+            auto y = h + fc2(fc1(ln2(h)).gelu());
+            y.sync();
+        };
+        measure("whisper_encoder_layer_bf16_s1500_d1280_h20", layer, warmup, iters, 24.0 * S * Dm * Dm + 4.0 * S * S * Dm, "GFLOP_per_s", true);
     }
     std::printf("}\n");
     return 0;

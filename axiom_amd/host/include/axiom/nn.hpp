@@ -19,6 +19,7 @@ class Module {
     Module &operator=(const Module &) = delete;
 
     virtual Tensor forward(const Tensor &input) const;
+    Tensor operator()(const Tensor &input) const { return forward(input); }
     virtual Module &to(Device device);
     virtual Module &to(DType dtype);
     // parameters are looked up as prefix + name; submodules add "name." (src/nn/module.cpp:36-50)

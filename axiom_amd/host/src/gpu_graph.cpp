@@ -236,8 +236,9 @@ class PlanBuilder {
                 const GraphNode *l = c->inputs[0].get(), *r = c->inputs[1].get();
                 const bool lf = l->output_shape == F, rf = r->output_shape == F;
                 if (!lf && !rf) break; // both operands broadcast: evaluated on its own (see emit_rows)
-                // continue through the operand that can still be fused; a leaf is the better memory operand
-                if (lf && rf) primary = (is_leaf(l, root_) && !is_leaf(r, root_)) ? 1 : 0;
+                // continue through the operand that can still be fused; a leaf, a shared node or one that
+                // already has a value is the better memory operand
+                if (lf && rf) primary = (!consumable(l, nullptr) && consumable(r, nullptr)) ? 1 : 0;
                 else primary = lf ? 0 : 1;
                 if (operands + 1 > AXHIP_MAX_OPERANDS - 2) break; // keep room for norm weight / bias
                 ++operands;

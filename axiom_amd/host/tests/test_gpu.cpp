@@ -438,3 +438,121 @@ static void whisper_case(size_t S, bool compare) {
 }
 GPU_TEST(WhisperBlock, ReducedSequenceMatchesFp32Reference) { whisper_case(150, true); }
 GPU_TEST(WhisperBlock, FullSizeProperties) { whisper_case(1500, false); }
+
+// ---------------------------------------------------------------------------
+// A whole pre-norm transformer encoder layer as in the reference's examples/whisper_poc.cpp:57-86
+// (the module is written the way that file writes it), bf16 on the GPU against an fp32
+// evaluation of the same bf16 parameters built from the oracle's pieces.
+namespace {
+struct WhisperEncoderLayer : nn::Module {
+    nn::MultiHeadAttention self_attn_;
+    nn::LayerNorm self_attn_layer_norm_;
+    nn::Linear fc1_{true};
+    nn::Linear fc2_{true};
+    nn::LayerNorm final_layer_norm_;
+
+    explicit WhisperEncoderLayer(int num_heads) : self_attn_(num_heads) {
+        register_module("self_attn", self_attn_);
+        register_module("self_attn_layer_norm", self_attn_layer_norm_);
+        register_module("fc1", fc1_);
+        register_module("fc2", fc2_);
+        register_module("final_layer_norm", final_layer_norm_);
+    }
+    Tensor forward(const Tensor &x) const override {
+        auto residual = x;
+        auto h = self_attn_layer_norm_(x);
+        h = self_attn_.forward(h, h, h);
+        h = ops::add(residual, h);
+        residual = h;
+        h = final_layer_norm_(h);
+        h = fc1_(h).gelu();
+        h = fc2_(h);
+        return ops::add(residual, h);
+    }
+};
+
+// fp32 helpers over the oracle
+Tensor ref_linear(const Tensor &x2d, const Tensor &w, const Tensor &b) { // x [S, in] f32, w [out, in], b [out]
+    const size_t S = x2d.shape()[0], in = x2d.shape()[1], out = w.shape()[0];
+    Tensor wf = w.astype(DType::Float32), bf = b.astype(DType::Float32), y({S, out}, DType::Float32);
+    axo_matmul(AXO_F32, x2d.data(), wf.data(), y.data(), S, out, in, 0, 1);
+    for (size_t i = 0; i < S; ++i)
+        for (size_t j = 0; j < out; ++j) y.typed_data<float>()[i * out + j] += bf.typed_data<float>()[j];
+    return y;
+}
+Tensor ref_layer_norm(const Tensor &x2d, const Tensor &w, const Tensor &b) {
+    Tensor wf = w.astype(DType::Float32), bf = b.astype(DType::Float32), y(x2d.shape(), DType::Float32);
+    axo_layer_norm(AXO_F32, x2d.data(), wf.data(), bf.data(), y.typed_data<float>(), x2d.shape()[0], x2d.shape()[1], 1e-5f);
+    return y;
+}
+} // namespace
+
+GPU_TEST(WhisperEncoderLayer, MatchesFp32ReferenceAndStaysFused) {
+    const size_t S = 96, Dm = 1280, H = 20, Dh = 64, F = 5120;
+    const DType dt = DType::BFloat16;
+    std::map<std::string, Tensor> w;
+    uint64_t seed = 100;
+    auto mat = [&](size_t o, size_t i) { return axtest::randn({o, i}, seed++, dt, 0.02f); };
+    auto vec = [&](size_t n, float lo, float hi) { return axtest::uniform({n}, seed++, lo, hi, dt); };
+    for (const char *p : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+        w[std::string("self_attn.") + p + ".weight"] = mat(Dm, Dm);
+        w[std::string("self_attn.") + p + ".bias"] = vec(Dm, -0.05f, 0.05f);
+    }
+    w["self_attn_layer_norm.weight"] = vec(Dm, 0.8f, 1.2f);
+    w["self_attn_layer_norm.bias"] = vec(Dm, -0.1f, 0.1f);
+    w["final_layer_norm.weight"] = vec(Dm, 0.8f, 1.2f);
+    w["final_layer_norm.bias"] = vec(Dm, -0.1f, 0.1f);
+    w["fc1.weight"] = mat(F, Dm);
+    w["fc1.bias"] = vec(F, -0.05f, 0.05f);
+    w["fc2.weight"] = mat(Dm, F);
+    w["fc2.bias"] = vec(Dm, -0.05f, 0.05f);
+    WhisperEncoderLayer layer(static_cast<int>(H));
+    layer.load_state_dict(w);
+    layer.to(Device::GPU);
+    EXPECT_EQ(layer.named_parameters().size(), 16u);
+
+    auto x = axtest::randn({1, S, Dm}, 99, dt);
+    auto y = layer.forward(x.gpu());
+    EXPECT_EQ(y.dtype(), dt);
+    auto got = host_floats(y);
+    // the tail of the layer is one graph of four launches: out_proj+bias+residual (GEMM; its result is
+    // shared by the norm and the last residual), LN, fc1+bias+gelu (GEMM), fc2+bias+residual (GEMM)
+    const auto &ks = graph::last_gpu_plan_kernels();
+    {
+        std::string all;
+        for (const auto &k : ks) all += " " + k;
+        std::printf("    kernels of the last materialisation:%s\n", all.c_str());
+    }
+    ASSERT_EQ(ks.size(), 4u);
+    EXPECT_EQ(ks[0], std::string("gemm"));
+    EXPECT_EQ(ks[1].substr(0, 21), std::string("rows_static_layernorm"));
+    EXPECT_EQ(ks[2], std::string("gemm"));
+    EXPECT_EQ(ks[3], std::string("gemm"));
+
+    // fp32 reference
+    Tensor x2 = x.astype(DType::Float32).reshape({S, Dm});
+    Tensor h = ref_layer_norm(x2, w["self_attn_layer_norm.weight"], w["self_attn_layer_norm.bias"]);
+    auto split = [&](const Tensor &t) { return t.reshape({1, S, H, Dh}).transpose({0, 2, 1, 3}).ascontiguousarray(); };
+    auto proj = [&](const Tensor &in, const char *n) { return ref_linear(in, w[std::string("self_attn.") + n + ".weight"], w[std::string("self_attn.") + n + ".bias"]); };
+    Tensor att = axtest::oracle_sdpa(split(proj(h, "q_proj")), split(proj(h, "k_proj")), split(proj(h, "v_proj")), Tensor(), -1, false);
+    Tensor merged = att.transpose({0, 2, 1, 3}).ascontiguousarray().reshape({S, Dm});
+    Tensor o = proj(merged, "out_proj");
+    Tensor r1({S, Dm}, DType::Float32);
+    for (size_t i = 0; i < S * Dm; ++i) r1.typed_data<float>()[i] = x2.typed_data<float>()[i] + o.typed_data<float>()[i];
+    Tensor h2 = ref_layer_norm(r1, w["final_layer_norm.weight"], w["final_layer_norm.bias"]);
+    Tensor f1 = ref_linear(h2, w["fc1.weight"], w["fc1.bias"]);
+    Tensor g1(f1.shape(), DType::Float32);
+    axo_unary(AXO_OP_GELU, AXO_F32, f1.data(), g1.data(), f1.size());
+    Tensor f2 = ref_linear(g1, w["fc2.weight"], w["fc2.bias"]);
+    double worst = 0;
+    size_t beyond = 0;
+    for (size_t i = 0; i < S * Dm; ++i) {
+        const double want = double(r1.typed_data<float>()[i]) + f2.typed_data<float>()[i];
+        const double d = std::fabs(got[i] - want);
+        worst = std::max(worst, d);
+        beyond += d > 2e-2;
+    }
+    std::printf("    encoder layer: max |err| %.4f, %.3f %% of outputs beyond 2e-2\n", worst, 100.0 * beyond / (S * Dm));
+    EXPECT_LE(worst, 8e-2);                         // several bf16 roundings of values up to |4|
+    EXPECT_LE(double(beyond) / (S * Dm), 0.03);
+}
