@@ -15,7 +15,7 @@ host on a bounded sample).
 The defaults (50 warm-up, 200 timed launches per kernel) are sized for the device's clock
 governor: coming from idle the first ~20 ms of MFMA work run at reduced clocks (the same SDPA
 launch measures ~650 us in a 5+20 run and ~550 us from the 50th launch on), so a short run
-reports the ramp, not the kernel.
+reports the ramp, not the kernel.  Every kernel is therefore warmed up for at least 100 ms.
 
 Everything runs on ONE GPU; --gpus above 1 is refused.
 """
@@ -44,7 +44,7 @@ CHAIN_TRAFFIC_BYTES = {"chain_relu_add_mul_softmax_sum_f32_8192x8192": 537.2e6,
                        "chain_gelu_rmsnorm_bf16_16384x4096": 269.2e6}
 
 
-MIN_WARMUP_MS = 30.0  # the clock governor needs about this much work of one kind to settle
+MIN_WARMUP_MS = 100.0  # clocks and power settle within about this much work of one kind
 
 
 def time_launches(torch, stream, launch, steps: int, warmup: int):
