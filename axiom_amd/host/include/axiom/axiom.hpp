@@ -1,8 +1,11 @@
 // Umbrella header of the gfx950 host layer.
 #pragma once
 
+#include "axiom/backends/hip/hip_operations.hpp"
 #include "axiom/dtype.hpp"
 #include "axiom/error.hpp"
+#include "axiom/graph/compiled_graph.hpp"
+#include "axiom/graph/gpu_fusion.hpp"
 #include "axiom/graph/graph_cache.hpp"
 #include "axiom/graph/graph_node.hpp"
 #include "axiom/graph/graph_registry.hpp"

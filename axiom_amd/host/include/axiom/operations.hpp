@@ -7,9 +7,13 @@
 // carries no CPU compute path.
 #pragma once
 
+#include <map>
+#include <memory>
+#include <string>
 #include <vector>
 
 #include "axiom/dtype.hpp"
+#include "axiom/storage.hpp"
 
 namespace axiom {
 class Tensor;
@@ -46,6 +50,33 @@ enum class OpType {
 };
 
 const char *op_name(OpType op);
+
+// Per-device implementation of one OpType (include/axiom/operations.hpp:210-279).  The base
+// implementations throw RuntimeError::not_implemented (src/tensor/operations.cpp:466-549).
+class Operation {
+  public:
+    virtual ~Operation() = default;
+    virtual OpType type() const = 0;
+    virtual std::string name() const = 0;
+    virtual Device device() const = 0;
+    virtual bool supports_binary(const Tensor &lhs, const Tensor &rhs) const;
+    virtual Tensor execute_binary(const Tensor &lhs, const Tensor &rhs) const;
+    virtual Tensor execute_unary(const Tensor &input) const;
+    virtual Tensor execute_reduction(const Tensor &input, const std::vector<int> &axis, bool keep_dims) const;
+    virtual Tensor execute_matmul(const Tensor &a, const Tensor &b, bool transpose_a, bool transpose_b) const;
+    virtual Tensor execute_cast(const Tensor &input, DType target_dtype) const;
+};
+
+// (OpType, Device) -> Operation (include/axiom/operations.hpp:285-302).  This library registers
+// Device::GPU entries only; get_operation(op, Device::CPU) is null.
+class OperationRegistry {
+  public:
+    static void register_operation(OpType op_type, Device device, std::unique_ptr<Operation> operation);
+    static const Operation *get_operation(OpType op_type, Device device);
+    static std::vector<Device> available_devices_for_operation(OpType op_type);
+    static bool is_operation_available(OpType op_type, Device device);
+    static void initialize_builtin_operations();
+};
 DType promote_types(DType lhs, DType rhs); // src/tensor/operations.cpp:346-397
 
 Tensor add(const Tensor &a, const Tensor &b);

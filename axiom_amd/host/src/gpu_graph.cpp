@@ -194,6 +194,8 @@ class PlanBuilder {
     int eval(const GraphNode *n) {
         auto it = memo_.find(n);
         if (it != memo_.end()) return it->second;
+        const size_t arity = is_binary_ew(n->op_type) || n->op_type == OpType::MatMul ? 2 : 1;
+        if (n->inputs.size() < arity) throw RuntimeError(std::string("malformed graph node '") + ops::op_name(n->op_type) + "': missing inputs");
         int v;
         const OpType op = n->op_type;
         if (op == OpType::Reshape) {
@@ -233,6 +235,7 @@ class PlanBuilder {
         while (consumable(c, entry) && is_elementwise(c->op_type) && c->output_shape == F && list.size() < limit) {
             int primary = 0;
             if (is_binary_ew(c->op_type)) {
+                if (c->inputs.size() < 2) throw RuntimeError(std::string("malformed graph node '") + ops::op_name(c->op_type) + "': missing inputs");
                 const GraphNode *l = c->inputs[0].get(), *r = c->inputs[1].get();
                 const bool lf = l->output_shape == F, rf = r->output_shape == F;
                 if (!lf && !rf) break; // both operands broadcast: evaluated on its own (see emit_rows)

@@ -556,3 +556,93 @@ GPU_TEST(WhisperEncoderLayer, MatchesFp32ReferenceAndStaysFused) {
     EXPECT_LE(worst, 8e-2);                         // several bf16 roundings of values up to |4|
     EXPECT_LE(double(beyond) / (S * Dm), 0.03);
 }
+
+// ---------------------------------------------------------------------------
+// The remaining backend hooks: per-op registry, gpu_* free functions, CPU-planned fused steps
+GPU_TEST(BackendHooks, OperationRegistryServesGpuOps) {
+    using ops::OpType;
+    ops::OperationRegistry::initialize_builtin_operations(); // tests/axiom_test_utils.hpp:17-22
+    EXPECT_TRUE(ops::OperationRegistry::is_operation_available(OpType::Add, Device::GPU));
+    EXPECT_TRUE(ops::OperationRegistry::get_operation(OpType::Add, Device::CPU) == nullptr); // no CPU backend in this library
+    EXPECT_TRUE(ops::OperationRegistry::get_operation(OpType::Conv2D, Device::GPU) == nullptr);
+    auto a = axtest::randn({4, 5}, 201), b = axtest::randn({5}, 202);
+    const auto *add = ops::OperationRegistry::get_operation(OpType::Add, Device::GPU);
+    ASSERT_TRUE(add != nullptr);
+    EXPECT_EQ(add->name(), std::string("hip::add"));
+    EXPECT_TRUE(add->supports_binary(a, b));
+    EXPECT_FALSE(add->supports_binary(a, axtest::randn({4}, 1)));
+    auto r = add->execute_binary(a.gpu(), b.gpu());
+    EXPECT_FALSE(r.is_lazy() && !r.lazy_node()->is_materialized_); // registry ops run at once
+    EXPECT_NEAR(r.cpu().item<float>({2, 3}), a.item<float>({2, 3}) + b.item<float>({3}), 0);
+    auto sm = ops::OperationRegistry::get_operation(OpType::Softmax, Device::GPU)->execute_reduction(a.gpu(), {-1}, false).cpu();
+    double s = 0;
+    for (size_t j = 0; j < 5; ++j) s += sm.item<float>({1, j});
+    EXPECT_NEAR(s, 1.0, 1e-5);
+    auto mm = ops::OperationRegistry::get_operation(OpType::MatMul, Device::GPU)->execute_matmul(a.gpu(), a.gpu(), false, true).cpu();
+    EXPECT_EQ(mm.shape(), Shape({4, 4}));
+    EXPECT_THROW(add->execute_unary(a.gpu()).cpu(), AxiomError);
+    auto devs = ops::OperationRegistry::available_devices_for_operation(OpType::ReLU);
+    ASSERT_EQ(devs.size(), 1u);
+    EXPECT_TRUE(devs[0] == Device::GPU);
+}
+
+GPU_TEST(BackendHooks, GpuFreeFunctions) {
+    using namespace backends::hip;
+    EXPECT_TRUE(is_hip_available());
+    float v[4] = {1, 2, 3, 4};
+    auto x = Tensor::from_data(v, {1, 4}, Device::GPU);
+    auto r = gpu_rms_norm(x, Tensor::ones({4}, DType::Float32, Device::GPU), -1, 1e-5f);
+    EXPECT_FALSE(r.is_lazy() && !r.lazy_node()->is_materialized_);
+    EXPECT_NEAR(r.cpu().item<float>({0, 0}), 1.0f / std::sqrt(7.5f), 1e-4);
+    auto ln = gpu_layer_norm(x, Tensor(), Tensor(), -1, 1e-5f).cpu();
+    EXPECT_NEAR(ln.item<float>({0, 0}) + ln.item<float>({0, 3}), 0.0, 1e-5);
+    EXPECT_NEAR(gpu_fill_constant({3, 3}, DType::BFloat16, 1.5).cpu().item<float>({2, 2}), 1.5f, 0);
+    auto t = axtest::randn({6, 7}, 203).gpu().transpose({1, 0});
+    auto c = gpu_make_contiguous(t);
+    EXPECT_TRUE(c.is_contiguous());
+    EXPECT_TRUE(c.cpu().allclose(t.cpu().ascontiguousarray(), 0, 0));
+    auto y = gpu_linear(Tensor::ones({2, 3}, DType::Float32, Device::GPU), Tensor::ones({4, 3}, DType::Float32, Device::GPU), Tensor::ones({4}, DType::Float32, Device::GPU), true);
+    EXPECT_NEAR(y.cpu().item<float>({1, 2}), 4.0f, 1e-5);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    auto [q, k, vv] = make_inputs(1, 2, 8, 8, 32);
+    ASSERT_TENSORS_CLOSE(gpu_scaled_dot_product_attention(q.gpu(), k.gpu(), vv.gpu(), Tensor(), -1, true).cpu(), axtest::oracle_sdpa(q, k, vv, Tensor(), -1, true), 1e-4, 1e-4);
+}
+
+GPU_TEST(BackendHooks, CpuPlannedFusedSteps) { // include/axiom/graph/gpu_fusion.hpp:14-22
+    using ops::OpType;
+    // buffers: slot 0 = a, slot 1 = b, slot 2 = c (host-resident: moved over), slot 3 = output
+    auto a = axtest::randn({8, 16}, 211), b = axtest::randn({8, 16}, 212), c = axtest::randn({16}, 213);
+    std::vector<Tensor> buffers = {a.gpu(), b.gpu(), c, Tensor()};
+    graph::FusedGenericStep step;
+    step.output_slot = 3;
+    step.output_shape = {8, 16};
+    step.output_dtype = DType::Float32;
+    step.device = Device::GPU;
+    step.op_chain = {OpType::Multiply, OpType::Add, OpType::ReLU}; // relu(a * b + c)
+    step.input_slot_indices = {{0, 1}, {-1, 2}, {-1}};
+    ASSERT_TRUE(graph::execute_gpu_fused_chain(step, step.op_chain, buffers));
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u); // the whole step is one launch
+    auto got = buffers[3].cpu();
+    for (size_t i = 0; i < 8; ++i)
+        for (size_t j = 0; j < 16; ++j)
+            EXPECT_NEAR(got.item<float>({i, j}), std::max(a.item<float>({i, j}) * b.item<float>({i, j}) + c.item<float>({j}), 0.0f), 1e-6);
+    // an op without a GPU kernel: the hook declines, the caller falls back
+    graph::FusedGenericStep bad = step;
+    bad.op_chain = {OpType::Multiply, OpType::Atan2};
+    bad.input_slot_indices = {{0, 1}, {-1, 2}};
+    EXPECT_FALSE(graph::execute_gpu_fused_chain(bad, bad.op_chain, buffers));
+    // chain + full reduction: sum(a + b) (tests/test_fusion_extended.cpp:346-352)
+    graph::FusedReductionStep red;
+    red.output_slot = 3;
+    red.output_shape = {1};
+    red.output_dtype = DType::Float32;
+    red.reduction_op = OpType::Sum;
+    red.params = graph::ReductionParams{{}, false};
+    red.op_chain = {OpType::Add};
+    red.input_slot_indices = {{0, 1}};
+    ASSERT_TRUE(graph::execute_gpu_fused_reduction(red, buffers));
+    double want = 0;
+    for (size_t i = 0; i < 8; ++i)
+        for (size_t j = 0; j < 16; ++j) want += double(a.item<float>({i, j})) + b.item<float>({i, j});
+    EXPECT_NEAR(buffers[3].cpu().item<float>(), want, 1e-3);
+}
