@@ -58,6 +58,57 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const GemmArgs g) {
     }
 }
 
+// Epilogue of the MFMA kernels: accumulator element e of 32x32 tile (i, j) is
+// C[m_base + 32 i + 8 (e/4) + 4 g2 + e%4][n_base + 32 j + l32].  bias, residual and
+// the activation are applied in fp32 before the one rounding to the output type.
+// The activation is resolved outside the element loops.
+template <bool BF16>
+__device__ __forceinline__ float load16(const void *p, int64_t i) {
+    const uint16_t b = static_cast<const uint16_t *>(p)[i];
+    return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b);
+}
+template <bool BF16>
+__device__ __forceinline__ void store16(void *p, int64_t i, float x) {
+    static_cast<uint16_t *>(p)[i] = BF16 ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
+}
+
+template <bool BF16, bool RESIDUAL, int OP, int MI, int NJ>
+__device__ __forceinline__ void gemm_store_tiles_as(const GemmArgs &g, const float16_t (&acc)[MI][NJ], int64_t m_base, int64_t n_base, int64_t coff, int l32, int g2) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int64_t n = n_base + 32 * j + l32;
+        if (n >= g.N) continue;
+        const float bias = g.bias ? load16<BF16>(g.bias, n) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int64_t m = m_base + 32 * i + 8 * (e / 4) + 4 * g2 + (e % 4);
+                if (m >= g.M) continue;
+                float x = acc[i][j][e] + bias;
+                if (RESIDUAL) x += load16<BF16>(g.residual, coff + m * g.ldc + n);
+                store16<BF16>(g.c, coff + m * g.ldc + n, gemm_epilogue(OP, x));
+            }
+    }
+}
+
+template <bool BF16, int MI, int NJ>
+__device__ __forceinline__ void gemm_store_tiles(const GemmArgs &g, const float16_t (&acc)[MI][NJ], int64_t m_base, int64_t n_base, int64_t coff, int l32, int g2) {
+#define AXHIP_GEMM_EPI(OP)                                                                                              \
+    if (g.residual) gemm_store_tiles_as<BF16, true, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);                 \
+    else gemm_store_tiles_as<BF16, false, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);
+    switch (g.epilogue) {
+    case AXHIP_OP_RELU: AXHIP_GEMM_EPI(AXHIP_OP_RELU) break;
+    case AXHIP_OP_GELU: AXHIP_GEMM_EPI(AXHIP_OP_GELU) break;
+    case AXHIP_OP_SILU: AXHIP_GEMM_EPI(AXHIP_OP_SILU) break;
+    case AXHIP_OP_SIGMOID: AXHIP_GEMM_EPI(AXHIP_OP_SIGMOID) break;
+    case AXHIP_OP_TANH: AXHIP_GEMM_EPI(AXHIP_OP_TANH) break;
+    default: AXHIP_GEMM_EPI(0) break;
+    }
+#undef AXHIP_GEMM_EPI
+}
+
+
 // ------------------------------------------------------------------- MFMA NT
 // Work-group tile BM x 128 x 64 (BM = 128 or 64), 4 waves in a 2 x 2 layout, each
 // owning a (BM/2) x 64 block of C as 32x32 MFMA tiles.  A and B k-tiles travel
@@ -151,24 +202,127 @@ __global__ __launch_bounds__(256, BM == 128 ? 2 : 1) void gemm_mfma_nt_kernel(co
         }
     }
 
-    // accumulator element e of tile (i, j): row = 8*(e/4) + 4*g2 + e%4, col = l32
-    const int64_t coff = bz * g.sc;
+    gemm_store_tiles<BF16, MI, 2>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
+}
+
+// ----------------------------------------------------------- MFMA NT, 256x256
+// Large products: work-group tile 256 x 256 x 64, 8 waves in a 2 x 4 layout, each
+// owning 128 x 64 of C (4 x 2 MFMA tiles, 128 accumulator registers).  A and B
+// k-tiles go L2 -> LDS directly (buffer_load ... lds: no staging registers, no
+// ds_write) into two 64 KiB buffers; tile j+1 streams in while tile j is multiplied,
+// one barrier per k-tile.  LDS rows are the 128 bytes of one k-tile row with the
+// 16-byte chunk index XOR-ed by (row >> 1) & 7, which spreads the 16 rows of a
+// fragment read over all banks.  Work-groups are dealt to the 8 XCDs so that each
+// XCD owns a compact block of C tiles and its L2 sees every A / B panel few times.
+typedef int int4_t __attribute__((ext_vector_type(4)));
+constexpr int BIG = 256;              // tile rows (M) and columns (N)
+constexpr int BIG_ROWB = TK * 2;      // bytes per LDS row
+constexpr int BIG_TILEB = BIG * BIG_ROWB; // 32 KiB per A or B k-tile
+
+// 16 bytes per lane from a buffer straight into LDS: lane i's data lands at lds_base + 16 i.
+// Lanes whose voffset lies beyond the descriptor's extent write zeros.
+__device__ __forceinline__ void gemm_load_to_lds(const int4_t &rsrc, uint32_t lds_base_uniform, int voffset, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_base_uniform), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+
+__device__ __forceinline__ int4_t gemm_rsrc(const void *base, int bytes) {
+    const uint64_t pa = reinterpret_cast<uint64_t>(base);
+    return int4_t{static_cast<int>(static_cast<uint32_t>(pa)), static_cast<int>(static_cast<uint32_t>(pa >> 32) & 0xFFFFu), bytes, 0x00020000};
+}
+
+// Requires K % 64 == 0 and 256 * max(lda, ldb) * 2 < 2^31 (checked by the launcher).
+template <bool BF16>
+__global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs g, const int tiles_m, const int tiles_n) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char big_lds[]; // A0 B0 A1 B1
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int l32 = lane % 32, g2 = lane / 32;
+
+    // work-group -> C tile: XCD x (work-groups x, x+8, ...) owns a contiguous range of the
+    // tile order; within it tiles run down groups of 4 tile rows
+    const int per_xcd = gridDim.x / 8;
+    const int t = (static_cast<int>(blockIdx.x) % 8) * per_xcd + static_cast<int>(blockIdx.x) / 8;
+    if (t >= tiles_m * tiles_n) return;
+    constexpr int GR = 4;
+    const int group = t / (GR * tiles_n), first_m = group * GR;
+    const int gsz = min(GR, tiles_m - first_m);
+    const int rem = t - group * GR * tiles_n;
+    const int tm = first_m + rem % gsz, tn = rem / gsz;
+    const int64_t m0 = static_cast<int64_t>(tm) * BIG, n0 = static_cast<int64_t>(tn) * BIG;
+    const int64_t bz = blockIdx.y;
+    const uint16_t *A = static_cast<const uint16_t *>(g.a) + bz * g.sa + m0 * g.a_rs;
+    const uint16_t *B = static_cast<const uint16_t *>(g.b) + bz * g.sb + n0 * g.b_cs;
+    const int arow_bytes = static_cast<int>(g.a_rs) * 2, brow_bytes = static_cast<int>(g.b_cs) * 2;
+    const int rows_a = static_cast<int>(min<int64_t>(BIG, g.M - m0)), rows_b = static_cast<int>(min<int64_t>(BIG, g.N - n0));
+    const int4_t arsrc = gemm_rsrc(A, (rows_a - 1) * arow_bytes + static_cast<int>(g.K) * 2);
+    const int4_t brsrc = gemm_rsrc(B, (rows_b - 1) * brow_bytes + static_cast<int>(g.K) * 2);
+
+    // ---- L2 -> LDS mapping: one wave-wide load moves 8 rows of 128 bytes; load n of wave w
+    // covers tile rows 64 n + 8 w + (lane >> 3); the lane fetches the chunk that belongs at
+    // position lane & 7 of the swizzled row
+    const int ld_r = 8 * wave + (lane >> 3);
+    const int ld_c = (lane & 7) ^ ((ld_r >> 1) & 7);
+    int a_voff[4], b_voff[4];
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int n = 0; n < 4; ++n) {
+        a_voff[n] = (64 * n + ld_r) * arow_bytes + ld_c * 16;
+        b_voff[n] = (64 * n + ld_r) * brow_bytes + ld_c * 16;
+    }
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(big_lds));
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 8 * wave * BIG_ROWB);
+    auto load_tile = [&](int kt, int buf) {
+        const int soff = kt * BIG_ROWB;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t n = n0 + wn + 32 * j + l32;
-            if (n >= g.N) continue;
-            const float bias = g.bias ? load_any(g.bias, g.dtype, n) : 0.0f;
+        for (int n = 0; n < 4; ++n) gemm_load_to_lds(arsrc, lds_wave + buf * 2 * BIG_TILEB + n * 64 * BIG_ROWB, a_voff[n], soff);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int64_t m = m0 + wm + 32 * i + 8 * (e / 4) + 4 * g2 + (e % 4);
-                if (m >= g.M) continue;
-                float x = acc[i][j][e] + bias;
-                if (g.residual) x += load_any(g.residual, g.dtype, coff + m * g.ldc + n);
-                store_any(g.c, g.dtype, coff + m * g.ldc + n, gemm_epilogue(g.epilogue, x));
-            }
+        for (int n = 0; n < 4; ++n) gemm_load_to_lds(brsrc, lds_wave + buf * 2 * BIG_TILEB + BIG_TILEB + n * 64 * BIG_ROWB, b_voff[n], soff);
+    };
+
+    // ---- fragment reads: row l32 (+ tile origin, a multiple of 32), k chunk 2 ks + g2
+    const int wm = (wave / 4) * 128, wn = (wave % 4) * 64;
+    int f_off[TK / 16];
+#pragma unroll
+    for (int ks = 0; ks < TK / 16; ++ks) f_off[ks] = l32 * BIG_ROWB + (((2 * ks + g2) ^ ((l32 >> 1) & 7)) * 16);
+
+    float16_t acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const int nk = static_cast<int>(g.K / TK);
+    load_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load_tile(kt + 1, buf ^ 1);
+        const unsigned char *As = big_lds + buf * 2 * BIG_TILEB + wm * BIG_ROWB;
+        const unsigned char *Bs = big_lds + buf * 2 * BIG_TILEB + BIG_TILEB + wn * BIG_ROWB;
+#pragma unroll
+        for (int ks = 0; ks < TK / 16; ++ks) {
+            uint4_t af[4], bf[2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const uint4_t *>(As + 32 * i * BIG_ROWB + f_off[ks]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const uint4_t *>(Bs + 32 * j * BIG_ROWB + f_off[ks]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if constexpr (BF16)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]), __builtin_bit_cast(bf16x8_t, bf[j]), acc[i][j], 0, 0, 0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[i]), __builtin_bit_cast(half8_t, bf[j]), acc[i][j], 0, 0, 0);
+                }
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's share of tile kt+1 has landed
+        __syncthreads();                    // ... everyone's has, and tile kt is no longer read
+    }
+
+    gemm_store_tiles<BF16, 4, 2>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
 }
 
 } // namespace axhip
@@ -203,7 +357,22 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool nt = !p.trans_a && p.trans_b && p.k % 8 == 0 && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.stride_a % 8 == 0 &&
                     p.stride_b % 8 == 0 && al16(a) && al16(b);
-    if (half && nt && p.k > 0) {
+    if (half && nt && p.k > 0 && p.k % TK == 0 && p.m >= BIG && p.n >= BIG && p.lda < (1 << 21) && p.ldb < (1 << 21) && p.batch < 65536 &&
+        ((p.m + BIG - 1) / BIG) * ((p.n + BIG - 1) / BIG) * p.batch >= 128) {
+        // 256 x 256 tiles once they give at least half the CUs a work-group
+        const int tiles_m = static_cast<int>((p.m + BIG - 1) / BIG), tiles_n = static_cast<int>((p.n + BIG - 1) / BIG);
+        const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+        const dim3 grid(static_cast<unsigned>(8 * per_xcd), static_cast<unsigned>(p.batch));
+        constexpr size_t lds_bytes = 4 * BIG_TILEB;
+        static const bool configured = [] {
+            bool ok = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_nt_256_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) == hipSuccess;
+            ok = ok && hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_nt_256_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) == hipSuccess;
+            return ok;
+        }();
+        AXHIP_REQUIRE(configured, AXHIP_ERR_UNSUPPORTED, "axhip_gemm: cannot reserve %zu bytes of LDS", lds_bytes);
+        if (p.dtype == AXHIP_DTYPE_BF16) hipLaunchKernelGGL((gemm_mfma_nt_256_kernel<true>), grid, dim3(512), lds_bytes, s, g, tiles_m, tiles_n);
+        else hipLaunchKernelGGL((gemm_mfma_nt_256_kernel<false>), grid, dim3(512), lds_bytes, s, g, tiles_m, tiles_n);
+    } else if (half && nt && p.k > 0) {
         // Tall tiles (two work-groups per CU, one k-tile in flight) once they fill the chip;
         // otherwise 64-row tiles, one work-group per CU with three k-tiles in flight.
         const int64_t tiles128 = ((p.n + TN - 1) / TN) * ((p.m + 127) / 128) * p.batch;

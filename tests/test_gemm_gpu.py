@@ -52,3 +52,24 @@ def test_batched_shared_weight_and_gelu_epilogue():
 
     want = 0.5 * y * (1 + np.vectorize(math.erf)(y / math.sqrt(2)))
     assert np.max(np.abs(got - want)) < 2e-2
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,extras", [(2300, 3800, 192, True), (2304, 3840, 64, False), (4096, 2048, 320, False)])
+def test_half_large_tile_path_matches_fp64(dt, M, N, K, extras):
+    """Shapes that take the 256 x 256 work-group tiles, with ragged last tiles in both
+    directions, a k extent of one and of several tiles, and the full epilogue."""
+    g = axo.PCG64(M + K)
+    x, W = axo.to_bits(g.normal((M, K)), dt), axo.to_bits(g.normal((N, K)) * 0.05, dt)
+    bias = axo.to_bits(g.normal((N,)) * 0.1, dt) if extras else None
+    res = axo.to_bits(g.normal((M, N)), dt) if extras else None
+    got = axo.to_f32(gh.gemm(x, W, dt, trans_b=True, bias=bias, residual=res, epilogue="relu" if extras else None)[0], dt)
+    want = axo.to_f32(x, dt).astype(np.float64) @ axo.to_f32(W, dt).astype(np.float64).T
+    if extras:
+        want = np.maximum(want + axo.to_f32(bias, dt) + axo.to_f32(res, dt), 0.0)
+    assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
+    # and the CPU oracle's matmul (accumulates in the 16-bit type as the reference's CPU path
+    # does, cpu_operations.cpp:1840-1872) stays within its own, wider, band on a corner block
+    if not extras and K <= 64:
+        o = axo.to_f32(axo.matmul(x[:64], W[:64], dt, False, True), dt)
+        assert np.max(np.abs(o - got[:64, :64])) < 0.25
