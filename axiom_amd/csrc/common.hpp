@@ -102,6 +102,27 @@ __device__ __forceinline__ void store_any(void *p, int dt, int64_t i, float v) {
     }
 }
 
+// x * Phi(x) for 16-bit outputs: Phi(x) = 0.5 + u*P(u^2) with u = clamp(x, -C, C),
+// P a degree-8 minimax fit; the result is clamped to [0, 1] so both tails are
+// exact.  |error| <= 5e-5 absolute over the whole line, under half a bf16 ulp
+// for |gelu| > 0.02, at 12 VALU operations and no transcendental (erff costs ~3x).
+__device__ __forceinline__ float gelu_fast(float x) {
+    constexpr float C = 4.45f;
+    const float u = __builtin_amdgcn_fmed3f(x, -C, C);
+    const float t = u * u;
+    float p = 3.455728e-11f;
+    p = __builtin_fmaf(p, t, -3.6776806e-09f);
+    p = __builtin_fmaf(p, t, 1.7219786e-07f);
+    p = __builtin_fmaf(p, t, -4.7068065e-06f);
+    p = __builtin_fmaf(p, t, 8.4325635e-05f);
+    p = __builtin_fmaf(p, t, -0.0010570257f);
+    p = __builtin_fmaf(p, t, 0.009658655f);
+    p = __builtin_fmaf(p, t, -0.06612378f);
+    p = __builtin_fmaf(p, t, 0.39880943f);
+    const float phi = __builtin_amdgcn_fmed3f(__builtin_fmaf(u, p, 0.5f), 0.0f, 1.0f);
+    return x * phi;
+}
+
 // Load / store N consecutive elements (N*sizeof(elem) is 16 or 32 bytes and the
 // address is aligned to min(16, that)) as fp32 values.
 template <int N>

@@ -34,6 +34,17 @@ __device__ __forceinline__ float gemm_epilogue(int op, float x) {
     }
 }
 
+// The same for results that are rounded to a 16-bit type: GELU through the polynomial
+// form (|error| <= 5e-5) and tanh through one exponential, both far below the output
+// resolution and a fraction of the code of erff / tanhf.
+__device__ __forceinline__ float gemm_epilogue16(int op, float x) {
+    switch (op) {
+    case AXHIP_OP_GELU: return gelu_fast(x);
+    case AXHIP_OP_TANH: return 1.0f - 2.0f / (1.0f + __expf(2.0f * x));
+    default: return gemm_epilogue(op, x);
+    }
+}
+
 // ------------------------------------------------------------------- generic
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const GemmArgs g) {
     __shared__ float As[16][17], Bs[16][17];
@@ -72,40 +83,78 @@ __device__ __forceinline__ void store16(void *p, int64_t i, float x) {
     static_cast<uint16_t *>(p)[i] = BF16 ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
 }
 
-template <bool BF16, bool RESIDUAL, int OP, int MI, int NJ>
+// C and the residual are addressed through buffer descriptors that cover exactly the valid
+// rows of the block, so a row past the end of C is dropped by the hardware bounds check;
+// columns past the end are masked per lane.  When all MI*32 rows are valid (FULL_ROWS)
+// the row offset travels in the scalar offset of the instruction, otherwise it is added
+// to the lane's offset, which is what the bounds check looks at.
+// Requires MI*32 * ldc * 2 < 2^31.
+template <bool BF16, int RESIDUAL_T, bool FULL_ROWS, int OP, int MI, int NJ> // RESIDUAL_T: 0 no, 1 yes, 2 decided at run time
 __device__ __forceinline__ void gemm_store_tiles_as(const GemmArgs &g, const float16_t (&acc)[MI][NJ], int64_t m_base, int64_t n_base, int64_t coff, int l32, int g2) {
+    const bool RESIDUAL = RESIDUAL_T == 1 || (RESIDUAL_T == 2 && g.residual != nullptr);
+    const int ldc2 = static_cast<int>(g.ldc) * 2;
+    const int cols_valid = static_cast<int>(min<int64_t>(32 * NJ, g.N - n_base));
+    const int rows_valid = static_cast<int>(min<int64_t>(32 * MI, g.M - m_base));
+    const int extent = (rows_valid - 1) * ldc2 + cols_valid * 2;
+    const int64_t origin = coff + m_base * g.ldc + n_base;
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(static_cast<uint16_t *>(g.c) + origin, 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(static_cast<const uint16_t *>(RESIDUAL ? g.residual : g.c)) + origin, 0, extent, 0x00020000);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        const int64_t n = n_base + 32 * j + l32;
-        if (n >= g.N) continue;
-        const float bias = g.bias ? load16<BF16>(g.bias, n) : 0.0f;
+        const int col = 32 * j + l32;
+        if (col >= cols_valid) continue;
+        const float bias = g.bias ? load16<BF16>(g.bias, n_base + col) : 0.0f;
+        const int voff = 4 * g2 * ldc2 + col * 2;
 #pragma unroll
-        for (int i = 0; i < MI; ++i)
+        for (int i = 0; i < MI; ++i) {
+            float x[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int64_t m = m_base + 32 * i + 8 * (e / 4) + 4 * g2 + (e % 4);
-                if (m >= g.M) continue;
-                float x = acc[i][j][e] + bias;
-                if (RESIDUAL) x += load16<BF16>(g.residual, coff + m * g.ldc + n);
-                store16<BF16>(g.c, coff + m * g.ldc + n, gemm_epilogue(OP, x));
+                x[e] = acc[i][j][e] + bias;
+                if (RESIDUAL) {
+                    const int roff = (32 * i + 8 * (e / 4) + e % 4) * ldc2;
+                    const uint16_t r = __builtin_amdgcn_raw_buffer_load_b16(rrsrc, FULL_ROWS ? voff : voff + roff, FULL_ROWS ? roff : 0, 0);
+                    x[e] += BF16 ? bf16_bits_to_f32(r) : f16_bits_to_f32(r);
+                }
             }
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+                const float y0 = gemm_epilogue16(OP, x[e]), y1 = gemm_epilogue16(OP, x[e + 1]);
+                const uint32_t w = BF16 ? pack_bf16x2(y0, y1) : (f32_to_f16_bits(y0) | (f32_to_f16_bits(y1) << 16));
+                const int roff = (32 * i + 8 * (e / 4) + e % 4) * ldc2;
+                __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(w & 0xFFFFu), crsrc, FULL_ROWS ? voff : voff + roff, FULL_ROWS ? roff : 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(w >> 16), crsrc, FULL_ROWS ? voff : voff + roff + ldc2, FULL_ROWS ? roff + ldc2 : 0, 0);
+            }
+        }
     }
 }
 
 template <bool BF16, int MI, int NJ>
 __device__ __forceinline__ void gemm_store_tiles(const GemmArgs &g, const float16_t (&acc)[MI][NJ], int64_t m_base, int64_t n_base, int64_t coff, int l32, int g2) {
-#define AXHIP_GEMM_EPI(OP)                                                                                              \
-    if (g.residual) gemm_store_tiles_as<BF16, true, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);                 \
-    else gemm_store_tiles_as<BF16, false, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);
-    switch (g.epilogue) {
-    case AXHIP_OP_RELU: AXHIP_GEMM_EPI(AXHIP_OP_RELU) break;
-    case AXHIP_OP_GELU: AXHIP_GEMM_EPI(AXHIP_OP_GELU) break;
-    case AXHIP_OP_SILU: AXHIP_GEMM_EPI(AXHIP_OP_SILU) break;
-    case AXHIP_OP_SIGMOID: AXHIP_GEMM_EPI(AXHIP_OP_SIGMOID) break;
-    case AXHIP_OP_TANH: AXHIP_GEMM_EPI(AXHIP_OP_TANH) break;
-    default: AXHIP_GEMM_EPI(0) break;
+    if (m_base >= g.M || n_base >= g.N) return;
+    const bool full_rows = m_base + MI * 32 <= g.M;
+    // the cheap epilogues get a specialisation per (residual, full rows); the transcendental
+    // ones are large when unrolled 128 times, and one general instance each is enough
+#define AXHIP_GEMM_EPI_FAST(OP)                                                                                         \
+    if (full_rows) {                                                                                                    \
+        if (g.residual) gemm_store_tiles_as<BF16, 1, true, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);          \
+        else gemm_store_tiles_as<BF16, 0, true, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);                     \
+    } else {                                                                                                            \
+        if (g.residual) gemm_store_tiles_as<BF16, 1, false, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);         \
+        else gemm_store_tiles_as<BF16, 0, false, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);                    \
     }
-#undef AXHIP_GEMM_EPI
+#define AXHIP_GEMM_EPI_GENERAL(OP) gemm_store_tiles_as<BF16, 2, false, OP, MI, NJ>(g, acc, m_base, n_base, coff, l32, g2);
+    switch (g.epilogue) {
+    case AXHIP_OP_RELU: AXHIP_GEMM_EPI_FAST(AXHIP_OP_RELU) break;
+    case AXHIP_OP_GELU: AXHIP_GEMM_EPI_GENERAL(AXHIP_OP_GELU) break;
+    case AXHIP_OP_SILU: AXHIP_GEMM_EPI_GENERAL(AXHIP_OP_SILU) break;
+    case AXHIP_OP_SIGMOID: AXHIP_GEMM_EPI_GENERAL(AXHIP_OP_SIGMOID) break;
+    case AXHIP_OP_TANH: AXHIP_GEMM_EPI_GENERAL(AXHIP_OP_TANH) break;
+    default: AXHIP_GEMM_EPI_FAST(0) break;
+    }
+#undef AXHIP_GEMM_EPI_FAST
+#undef AXHIP_GEMM_EPI_GENERAL
 }
 
 
@@ -125,7 +174,7 @@ __global__ __launch_bounds__(256, BM == 128 ? 2 : 1) void gemm_mfma_nt_kernel(co
     constexpr int NA = BM / 32;  // 16-byte chunks of A per thread per k-tile (BM rows x 8 chunks / 256 threads)
     __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[TN * LDS_STRIDE];
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
     const int l32 = lane % 32, g2 = lane / 32;
     const int wm = (wave / 2) * (BM / 2), wn = (wave % 2) * 64;
     const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM, n0 = static_cast<int64_t>(blockIdx.x) * TN;
@@ -235,7 +284,7 @@ __device__ __forceinline__ int4_t gemm_rsrc(const void *base, int bytes) {
 template <bool BF16>
 __global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs g, const int tiles_m, const int tiles_n) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char big_lds[]; // A0 B0 A1 B1
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
     const int l32 = lane % 32, g2 = lane / 32;
 
     // work-group -> C tile: XCD x (work-groups x, x+8, ...) owns a contiguous range of the
@@ -356,7 +405,7 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     const bool half = p.dtype != AXHIP_DTYPE_F32;
     auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool nt = !p.trans_a && p.trans_b && p.k % 8 == 0 && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.stride_a % 8 == 0 &&
-                    p.stride_b % 8 == 0 && al16(a) && al16(b);
+                    p.stride_b % 8 == 0 && al16(a) && al16(b) && p.ldc < (1 << 21);
     if (half && nt && p.k > 0 && p.k % TK == 0 && p.m >= BIG && p.n >= BIG && p.lda < (1 << 21) && p.ldb < (1 << 21) && p.batch < 65536 &&
         ((p.m + BIG - 1) / BIG) * ((p.n + BIG - 1) / BIG) * p.batch >= 128) {
         // 256 x 256 tiles once they give at least half the CUs a work-group
