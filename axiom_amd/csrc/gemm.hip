@@ -341,34 +341,58 @@ __global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+    // Fragments are double-buffered in registers and the loop is rotated: the reads of
+    // k-step 0 of the next tile are issued right after the barrier, under the MFMAs of
+    // k-step 3 of the current one, so no LDS latency is exposed at the tile boundary.
+    uint4_t fa[2][4], fb[2][2];
+    auto read_frags = [&](int slot, int buf, int ks) {
+        const unsigned char *As = big_lds + buf * 2 * BIG_TILEB + wm * BIG_ROWB;
+        const unsigned char *Bs = big_lds + buf * 2 * BIG_TILEB + BIG_TILEB + wn * BIG_ROWB;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[slot][j] = *reinterpret_cast<const uint4_t *>(Bs + 32 * j * BIG_ROWB + f_off[ks]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[slot][i] = *reinterpret_cast<const uint4_t *>(As + 32 * i * BIG_ROWB + f_off[ks]);
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if constexpr (BF16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[slot][i]), __builtin_bit_cast(bf16x8_t, fb[slot][j]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fa[slot][i]), __builtin_bit_cast(half8_t, fb[slot][j]), acc[i][j], 0, 0, 0);
+            }
+    };
+
     const int nk = static_cast<int>(g.K / TK);
     load_tile(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     __syncthreads();
+    read_frags(0, 0, 0);
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
         if (kt + 1 < nk) load_tile(kt + 1, buf ^ 1);
-        const unsigned char *As = big_lds + buf * 2 * BIG_TILEB + wm * BIG_ROWB;
-        const unsigned char *Bs = big_lds + buf * 2 * BIG_TILEB + BIG_TILEB + wn * BIG_ROWB;
-#pragma unroll
-        for (int ks = 0; ks < TK / 16; ++ks) {
-            uint4_t af[4], bf[2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const uint4_t *>(As + 32 * i * BIG_ROWB + f_off[ks]);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const uint4_t *>(Bs + 32 * j * BIG_ROWB + f_off[ks]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if constexpr (BF16)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i]), __builtin_bit_cast(bf16x8_t, bf[j]), acc[i][j], 0, 0, 0);
-                    else
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[i]), __builtin_bit_cast(half8_t, bf[j]), acc[i][j], 0, 0, 0);
-                }
-        }
+        // the scheduling fences keep each batch of reads ahead of the MFMAs it overlaps with
+        // (left alone, the scheduler sinks every read to just before its first use)
+        read_frags(1, buf, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(0, buf, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(1, buf, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(0);
+        __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's share of tile kt+1 has landed
         __syncthreads();                    // ... everyone's has, and tile kt is no longer read
+        read_frags(0, buf ^ 1, 0);          // (after the last tile: a harmless read of stale LDS)
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     gemm_store_tiles<BF16, 4, 2>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
