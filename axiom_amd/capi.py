@@ -20,6 +20,7 @@ RED = dict(none=0, sum=1, mean=2, max=3, min=4)
 BK = dict(full=0, rowvec=1, colvec=2, scalar=3, imm=4)
 
 MAX_CHAIN, MAX_OPERANDS = 16, 8
+ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_WORKSPACE = -1, -2, -3, -4
 
 
 class AxhipError(RuntimeError):
@@ -105,6 +106,10 @@ def lib() -> C.CDLL:
                                          C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p]
         l.axhip_fill.argtypes = [C.c_void_p, C.c_int32, C.c_double, C.c_int64, C.c_void_p]
         l.axhip_gemm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(GemmParams), C.c_void_p]
+        i64p = C.POINTER(C.c_int64)
+        l.axhip_pad.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, i64p, i64p, i64p, i64p, C.c_double, C.c_void_p]
+        l.axhip_masked_fill.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, i64p, i64p, i64p, C.c_double, C.c_void_p]
+        l.axhip_gather_rows.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]
         _lib = l
     return _lib
 

@@ -1,5 +1,6 @@
-// Strided gather into a contiguous buffer (with dtype conversion) and constant
-// fill.  One thread per output element; the output side is fully coalesced.
+// Strided gather into a contiguous buffer (with dtype conversion), constant fill,
+// constant padding, masked fill and embedding-row gather.  One thread per output
+// element (16 bytes per thread for the row gather); the output side is fully coalesced.
 #include "common.hpp"
 
 #include <algorithm>
@@ -31,6 +32,69 @@ __global__ __launch_bounds__(256) void strided_copy_kernel(const CopyArgs a) {
 __global__ __launch_bounds__(256) void fill_kernel(void *dst, int dtype, float value, int64_t n) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) store_any(dst, dtype, i, value);
+}
+
+struct PadArgs {
+    const void *src;
+    void *dst;
+    int dtype, ndim;
+    int64_t total;
+    float value;
+    int64_t out_shape[AXHIP_MAX_DIMS], src_shape[AXHIP_MAX_DIMS], src_strides[AXHIP_MAX_DIMS], before[AXHIP_MAX_DIMS];
+};
+
+__global__ __launch_bounds__(256) void pad_kernel(const PadArgs a) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < a.total; i += stride) {
+        int64_t rem = i, off = 0;
+        bool inside = true;
+        for (int d = a.ndim - 1; d >= 0; --d) {
+            const int64_t c = rem % a.out_shape[d] - a.before[d];
+            rem /= a.out_shape[d];
+            inside = inside && c >= 0 && c < a.src_shape[d];
+            off += c * a.src_strides[d];
+        }
+        store_any(a.dst, a.dtype, i, inside ? load_any(a.src, a.dtype, off) : a.value);
+    }
+}
+
+struct MaskedFillArgs {
+    const void *src;
+    const uint8_t *mask;
+    void *dst;
+    int dtype, ndim;
+    int64_t total;
+    float value;
+    int64_t shape[AXHIP_MAX_DIMS], src_strides[AXHIP_MAX_DIMS], mask_strides[AXHIP_MAX_DIMS];
+};
+
+__global__ __launch_bounds__(256) void masked_fill_kernel(const MaskedFillArgs a) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < a.total; i += stride) {
+        int64_t rem = i, soff = 0, moff = 0;
+        for (int d = a.ndim - 1; d >= 0; --d) {
+            const int64_t c = rem % a.shape[d];
+            rem /= a.shape[d];
+            soff += c * a.src_strides[d];
+            moff += c * a.mask_strides[d];
+        }
+        store_any(a.dst, a.dtype, i, a.mask[moff] ? a.value : load_any(a.src, a.dtype, soff));
+    }
+}
+
+// One thread moves `chunk` bytes (16, or the element size when rows are not 16-byte
+// multiples) of one output row.
+template <typename V>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const V *table, int64_t table_rows, int64_t row_chunks, const void *indices,
+                                                           int index_bytes, int64_t n_indices, V *dst) {
+    const int64_t total = n_indices * row_chunks, stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / row_chunks, c = i - r * row_chunks;
+        const int64_t idx = index_bytes == 8 ? static_cast<const int64_t *>(indices)[r] : static_cast<const int32_t *>(indices)[r];
+        V v{};
+        if (idx >= 0 && idx < table_rows) v = table[idx * row_chunks + c];
+        dst[i] = v;
+    }
 }
 
 } // namespace axhip
@@ -74,6 +138,88 @@ int axhip_fill(void *dst, int32_t dtype, double value, int64_t count, void *stre
     const int64_t blocks = std::min<int64_t>((count + 255) / 256, 256 * 64);
     hipLaunchKernelGGL(fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), dst, dtype,
                        static_cast<float>(value), count);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+int axhip_pad(const void *src, void *dst, int32_t dtype, int32_t ndim, const int64_t *src_shape, const int64_t *src_strides,
+              const int64_t *pad_before, const int64_t *pad_after, double value, void *stream) {
+    AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_pad: bad dtype");
+    AXHIP_REQUIRE(ndim >= 1 && ndim <= AXHIP_MAX_DIMS, AXHIP_ERR_INVALID_ARG, "axhip_pad: ndim %d out of range", ndim);
+    AXHIP_REQUIRE(src_shape && src_strides && pad_before && pad_after, AXHIP_ERR_INVALID_ARG, "axhip_pad: NULL shape/strides/pads");
+    PadArgs a{};
+    a.src = src; a.dst = dst; a.dtype = dtype; a.ndim = ndim; a.value = static_cast<float>(value);
+    a.total = 1;
+    int64_t src_total = 1;
+    for (int d = 0; d < ndim; ++d) {
+        AXHIP_REQUIRE(src_shape[d] >= 0 && pad_before[d] >= 0 && pad_after[d] >= 0, AXHIP_ERR_INVALID_ARG, "axhip_pad: negative extent or pad");
+        AXHIP_REQUIRE(src_strides[d] >= 0, AXHIP_ERR_UNSUPPORTED, "axhip_pad: negative strides (flipped views) are not supported");
+        a.src_shape[d] = src_shape[d];
+        a.src_strides[d] = src_strides[d];
+        a.before[d] = pad_before[d];
+        a.out_shape[d] = src_shape[d] + pad_before[d] + pad_after[d];
+        a.total *= a.out_shape[d];
+        src_total *= src_shape[d];
+    }
+    if (a.total == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(dst && (src || src_total == 0), AXHIP_ERR_INVALID_ARG, "axhip_pad: NULL buffer");
+    int rc = ensure_init();
+    if (rc) return rc;
+    const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
+    hipLaunchKernelGGL(pad_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), a);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+int axhip_masked_fill(const void *src, int32_t dtype, const uint8_t *mask, void *dst, int32_t ndim, const int64_t *shape,
+                      const int64_t *src_strides, const int64_t *mask_strides, double value, void *stream) {
+    AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_masked_fill: bad dtype");
+    AXHIP_REQUIRE(ndim >= 0 && ndim <= AXHIP_MAX_DIMS, AXHIP_ERR_INVALID_ARG, "axhip_masked_fill: ndim %d out of range", ndim);
+    AXHIP_REQUIRE(ndim == 0 || (shape && src_strides && mask_strides), AXHIP_ERR_INVALID_ARG, "axhip_masked_fill: NULL shape/strides");
+    MaskedFillArgs a{};
+    a.src = src; a.mask = mask; a.dst = dst; a.dtype = dtype; a.ndim = ndim; a.value = static_cast<float>(value);
+    a.total = 1;
+    for (int d = 0; d < ndim; ++d) {
+        AXHIP_REQUIRE(shape[d] >= 0, AXHIP_ERR_INVALID_ARG, "axhip_masked_fill: negative extent");
+        AXHIP_REQUIRE(src_strides[d] >= 0 && mask_strides[d] >= 0, AXHIP_ERR_UNSUPPORTED, "axhip_masked_fill: negative strides are not supported");
+        a.shape[d] = shape[d];
+        a.src_strides[d] = src_strides[d];
+        a.mask_strides[d] = mask_strides[d];
+        a.total *= shape[d];
+    }
+    if (a.total == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(src && mask && dst, AXHIP_ERR_INVALID_ARG, "axhip_masked_fill: NULL buffer");
+    int rc = ensure_init();
+    if (rc) return rc;
+    const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
+    hipLaunchKernelGGL(masked_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), a);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int64_t row_elems, const void *indices, int32_t index_bytes,
+                      int64_t n_indices, void *dst, void *stream) {
+    AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_gather_rows: bad dtype");
+    AXHIP_REQUIRE(index_bytes == 4 || index_bytes == 8, AXHIP_ERR_INVALID_ARG, "axhip_gather_rows: index_bytes must be 4 or 8");
+    AXHIP_REQUIRE(table_rows >= 0 && row_elems >= 0 && n_indices >= 0, AXHIP_ERR_INVALID_ARG, "axhip_gather_rows: negative extent");
+    if (n_indices == 0 || row_elems == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(indices && dst && (table || table_rows == 0), AXHIP_ERR_INVALID_ARG, "axhip_gather_rows: NULL buffer");
+    int rc = ensure_init();
+    if (rc) return rc;
+    const int64_t esz = dtype == AXHIP_DTYPE_F32 ? 4 : 2, row_bytes = row_elems * esz;
+    const bool wide = row_bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(table) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0;
+    const int64_t chunks = wide ? row_bytes / 16 : row_elems;
+    const int64_t blocks = std::min<int64_t>((n_indices * chunks + 255) / 256, 256 * 64);
+    hipStream_t s = resolve_stream(stream);
+    if (wide)
+        hipLaunchKernelGGL(gather_rows_kernel<uint4_t>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, static_cast<const uint4_t *>(table),
+                           table_rows, chunks, indices, index_bytes, n_indices, static_cast<uint4_t *>(dst));
+    else if (esz == 4)
+        hipLaunchKernelGGL(gather_rows_kernel<uint32_t>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, static_cast<const uint32_t *>(table),
+                           table_rows, chunks, indices, index_bytes, n_indices, static_cast<uint32_t *>(dst));
+    else
+        hipLaunchKernelGGL(gather_rows_kernel<uint16_t>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, static_cast<const uint16_t *>(table),
+                           table_rows, chunks, indices, index_bytes, n_indices, static_cast<uint16_t *>(dst));
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;
 }

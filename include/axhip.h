@@ -220,6 +220,31 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
                        void *stream);
 int axhip_fill(void *dst, int32_t dtype, double value, int64_t count, void *stream);
 
+/* Constant padding (ops::pad, mode "constant": src/tensor/operations.cpp pad();
+ * lazy Pad node, src/backends/metal/mpsgraph_graph_compiler.mm:335-573).  dst is
+ * contiguous row-major with extents src_shape[d] + pad_before[d] + pad_after[d];
+ * src may be a strided view (non-negative element strides).  One pass: each
+ * output element is either copied or set to `value`. */
+int axhip_pad(const void *src, void *dst, int32_t dtype, int32_t ndim, const int64_t *src_shape_host,
+              const int64_t *src_strides_host, const int64_t *pad_before_host,
+              const int64_t *pad_after_host, double value, void *stream);
+
+/* masked_fill (include/axiom/operations.hpp:437-440): dst[i] = mask[i] ? value :
+ * src[i] over an iteration space of <= 8 dims; src and the byte mask (Bool:
+ * nonzero = fill) are strided views with element strides, 0 on broadcast dims;
+ * dst is contiguous and has src's dtype. */
+int axhip_masked_fill(const void *src, int32_t dtype, const uint8_t *mask, void *dst, int32_t ndim,
+                      const int64_t *shape_host, const int64_t *src_strides_host,
+                      const int64_t *mask_strides_host, double value, void *stream);
+
+/* Embedding lookup (ops::embedding, include/axiom/operations.hpp:483-486):
+ * dst[i, :] = table[indices[i], :] for n_indices rows of row_elems elements.
+ * index_bytes is 4 (int32) or 8 (int64).  An index outside [0, table_rows)
+ * yields a row of zeros (the device cannot throw IndexError). */
+int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int64_t row_elems,
+                      const void *indices, int32_t index_bytes, int64_t n_indices, void *dst,
+                      void *stream);
+
 /* -------------------------------------------------------------------- GEMM
  * Stands behind the GPU MatMul registry entry and gpu_linear
  * (src/backends/metal/mpsgraph_operations.mm:2409-2532; lazy builder

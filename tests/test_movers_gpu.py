@@ -1,0 +1,130 @@
+"""GPU parity of the data movers behind gpu_make_contiguous / Cast / Pad / MaskedFill /
+Embedding: pure data movement, so every comparison is bit-exact against numpy."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from axiom_amd import capi
+from oracle import axo
+from tests import gpu_harness as gh
+
+pytestmark = pytest.mark.gpu
+F32, F16, BF16 = axo.F32, axo.F16, axo.BF16
+
+
+def i64(values):
+    return (C.c_int64 * len(values))(*[int(v) for v in values])
+
+
+def sample(shape, dt, seed):
+    x = axo.PCG64(seed).normal(shape)
+    return x if dt == F32 else axo.to_bits(x, dt)
+
+
+def elem_strides(a):
+    return [s // a.itemsize for s in a.strides]
+
+
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+def test_strided_copy_of_transposed_and_broadcast_views(dt):
+    base = sample((6, 5, 7), dt, 3)
+    d = gh.to_dev(base)
+    for view in (base.transpose(2, 0, 1), base[:, ::2, 1:6], np.broadcast_to(base[:, :1, :], (6, 4, 7))):
+        out = gh.empty_dev(view.shape, dt)
+        off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0])
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr() + off, dt, out.data_ptr(), dt, view.ndim, i64(view.shape), i64(elem_strides(view)), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view))
+
+
+def test_strided_copy_casts_like_the_oracle():
+    x = axo.PCG64(9).normal((33, 17))
+    d = gh.to_dev(x)
+    for dt in (F16, BF16):
+        out = gh.empty_dev(x.shape, dt)
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr(), F32, out.data_ptr(), dt, 2, i64(x.shape), i64([17, 1]), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, np.uint16), axo.to_bits(x, dt))
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_fill(dt):
+    out = gh.empty_dev((1000,), dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_fill(out.data_ptr(), dt, 1.5, 1000, None))
+    gh.sync()
+    got = gh.to_host(out, gh.np_store_dtype(dt))
+    want = np.full(1000, 1.5, np.float32)
+    assert np.array_equal(got, want if dt == F32 else axo.to_bits(want, dt))
+
+
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape,before,after", [((5,), (2,), (3,)), ((3, 4), (0, 1), (2, 0)), ((2, 3, 50), (0, 0, 1), (0, 0, 1)),
+                                                ((2, 1, 3, 4), (1, 0, 2, 0), (0, 3, 0, 5))])
+def test_pad_matches_numpy(dt, shape, before, after):
+    x = sample(shape, dt, 11)
+    value = -2.5
+    fill = np.float32(value) if dt == F32 else axo.to_bits(np.array([value], np.float32), dt)[0]
+    want = np.pad(x, list(zip(before, after)), constant_values=fill)
+    d = gh.to_dev(x)
+    out = gh.empty_dev(want.shape, dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_pad(d.data_ptr(), out.data_ptr(), dt, x.ndim, i64(shape), i64(elem_strides(x)), i64(before), i64(after), value, None))
+    gh.sync()
+    assert np.array_equal(gh.to_host(out, x.dtype), want)
+
+
+def test_pad_of_a_transposed_view():
+    base = sample((4, 6), F32, 12)
+    view = base.T
+    want = np.pad(view, [(1, 1), (0, 2)])
+    d = gh.to_dev(base)
+    out = gh.empty_dev(want.shape, F32)
+    gh.sync()
+    capi.check(capi.lib().axhip_pad(d.data_ptr(), out.data_ptr(), F32, 2, i64(view.shape), i64(elem_strides(view)), i64([1, 0]), i64([1, 2]), 0.0, None))
+    gh.sync()
+    assert np.array_equal(gh.to_host(out, np.float32), want)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_masked_fill_with_broadcast_masks(dt):
+    x = sample((2, 3, 8, 8), dt, 13)
+    d = gh.to_dev(x)
+    i, j = np.meshgrid(np.arange(8), np.arange(8), indexing="ij")
+    causal = (j > i).astype(np.uint8)  # the attention use: mask (Sq, Skv) over (B, H, Sq, Skv)
+    full = (axo.PCG64(14).normal(x.shape) > 0.5).astype(np.uint8)
+    fill = np.float32(-1e9) if dt == F32 else axo.to_bits(np.array([-1e9], np.float32), dt)[0]
+    for mask, mstr in ((causal, [0, 0, 8, 1]), (full, [192, 64, 8, 1]), (full[:, :1, :, :1].copy(), [8, 0, 1, 0])):
+        m = torch.from_numpy(mask).cuda()
+        out = gh.empty_dev(x.shape, dt)
+        gh.sync()
+        capi.check(capi.lib().axhip_masked_fill(d.data_ptr(), dt, m.data_ptr(), out.data_ptr(), 4, i64(x.shape), i64(elem_strides(x)), i64(mstr), -1e9, None))
+        gh.sync()
+        bm = np.broadcast_to(mask.reshape([x.shape[k] if mstr[k] else 1 for k in range(4)]) if mask.ndim == 4 else mask, x.shape)
+        assert np.array_equal(gh.to_host(out, x.dtype), np.where(bm != 0, fill, x))
+
+
+@pytest.mark.parametrize("dt,cols", [(F32, 8), (BF16, 64), (F16, 7), (F32, 3)], ids=["f32x8", "bf16x64", "f16x7", "f32x3"])
+@pytest.mark.parametrize("itype", [np.int64, np.int32], ids=["i64", "i32"])
+def test_gather_rows_is_an_embedding_lookup(dt, cols, itype):
+    table = sample((50, cols), dt, 15)
+    idx = np.array([0, 49, 7, 7, 23, -1, 50, 3], itype)  # two out-of-range entries -> zero rows
+    d, di = gh.to_dev(table), torch.from_numpy(idx).cuda()
+    out = gh.empty_dev((idx.size, cols), dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_gather_rows(d.data_ptr(), dt, 50, cols, di.data_ptr(), idx.itemsize, idx.size, out.data_ptr(), None))
+    gh.sync()
+    want = np.where(((idx >= 0) & (idx < 50))[:, None], table[np.clip(idx, 0, 49)], np.zeros((), table.dtype))
+    assert np.array_equal(gh.to_host(out, table.dtype), want)
+
+
+def test_mover_argument_errors():
+    L = capi.lib()
+    assert L.axhip_pad(None, None, 7, 1, i64([1]), i64([1]), i64([0]), i64([0]), 0.0, None) == capi.ERR_INVALID_ARG
+    assert L.axhip_pad(None, None, F32, 9, i64([1]), i64([1]), i64([0]), i64([0]), 0.0, None) == capi.ERR_INVALID_ARG
+    assert L.axhip_gather_rows(None, F32, 4, 4, None, 2, 1, None, None) == capi.ERR_INVALID_ARG
+    assert L.axhip_masked_fill(None, F32, None, None, 1, i64([4]), i64([-1]), i64([1]), 0.0, None) == capi.ERR_UNSUPPORTED
