@@ -4,6 +4,7 @@
 
 #include <atomic>
 #include <memory>
+#include <utility>
 #include <variant>
 #include <vector>
 
@@ -38,7 +39,22 @@ struct TransposeParams {
     std::vector<int> axes;
 };
 
-using OpParams = std::variant<NoParams, ReductionParams, MatMulParams, ActivationParams, ReshapeParams, NormParams, TransposeParams>;
+struct SliceParams { // per dimension; steps are positive
+    std::vector<int64_t> starts, ends, steps;
+};
+struct PadParams {
+    std::vector<std::pair<size_t, size_t>> pad_widths;
+    double value = 0.0;
+};
+struct MaskedFillParams {
+    float value = 0.0f;
+};
+struct UnfoldParams { // windows of `kernel` taps along the last dimension
+    int kernel = 1, stride = 1, dilation = 1;
+};
+
+using OpParams = std::variant<NoParams, ReductionParams, MatMulParams, ActivationParams, ReshapeParams, NormParams, TransposeParams, SliceParams,
+                              PadParams, MaskedFillParams, UnfoldParams>;
 
 template <typename T> const T &get_params(const OpParams &p) { return std::get<T>(p); }
 

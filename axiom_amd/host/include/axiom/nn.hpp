@@ -1,8 +1,9 @@
-// nn modules on the attention / norm path (include/axiom/nn/{module,linear,
-// normalization,attention,activation}.hpp; src/nn/*.cpp).  Inference only.
+// nn modules on the attention / norm path and around it (include/axiom/nn/{module,linear,
+// normalization,attention,activation,conv,embedding,container}.hpp; src/nn/*.cpp).  Inference only.
 #pragma once
 
 #include <map>
+#include <memory>
 #include <string>
 #include <utility>
 #include <vector>
@@ -76,6 +77,59 @@ class ReLU : public Module {
 class GELU : public Module {
   public:
     Tensor forward(const Tensor &input) const override;
+};
+
+// 1-D convolution, weight (C_out, C_in, K) (include/axiom/nn/conv.hpp:25-48)
+class Conv1d : public Module {
+  public:
+    explicit Conv1d(int stride = 1, int padding = 0, int dilation = 1, int groups = 1, bool bias = true);
+    Tensor forward(const Tensor &input) const override;
+    const Tensor &weight() const { return weight_; }
+    const Tensor &bias() const { return bias_; }
+
+  private:
+    Tensor weight_, bias_;
+    int stride_, padding_, dilation_, groups_;
+    bool has_bias_;
+};
+
+// rows of weight (vocab, dim) by integer index (include/axiom/nn/embedding.hpp:7-16)
+class Embedding : public Module {
+  public:
+    Embedding();
+    Tensor forward(const Tensor &indices) const override;
+
+  private:
+    Tensor weight_;
+};
+
+// inference batch norm with running statistics (include/axiom/nn/normalization.hpp:37-58)
+class BatchNorm1d : public Module {
+  public:
+    explicit BatchNorm1d(float eps = 1e-5f);
+    Tensor forward(const Tensor &input) const override;
+
+  private:
+    Tensor weight_, bias_, running_mean_, running_var_;
+    float eps_;
+};
+
+// owning list of submodules named "0", "1", ... (include/axiom/nn/container.hpp:11-35)
+class ModuleList : public Module {
+  public:
+    template <typename T, typename... Args> T &emplace_back(Args &&...args) {
+        auto ptr = std::make_unique<T>(std::forward<Args>(args)...);
+        T &ref = *ptr;
+        register_module(std::to_string(modules_.size()), ref);
+        modules_.push_back(std::move(ptr));
+        return ref;
+    }
+    Module &operator[](size_t index) { return *modules_.at(index); }
+    const Module &operator[](size_t index) const { return *modules_.at(index); }
+    size_t size() const { return modules_.size(); }
+
+  private:
+    std::vector<std::unique_ptr<Module>> modules_;
 };
 
 // q/k/v/out projections + scaled_dot_product_attention over num_heads heads

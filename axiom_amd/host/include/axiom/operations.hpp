@@ -9,6 +9,7 @@
 
 #include <map>
 #include <memory>
+#include <utility>
 #include <string>
 #include <vector>
 
@@ -46,7 +47,10 @@ enum class OpType {
     Reshape, Transpose, Pad, Slice, Unsqueeze, Concat,
     GLU, BatchNorm1D,
     Sort, Argsort, TopK,
-    _Count
+    _Count,
+    // internal to this backend's planner, after Axiom's own values: the (N, L_out, C_in, K) window view a
+    // convolution is lowered through
+    Unfold1D
 };
 
 const char *op_name(OpType op);
@@ -112,6 +116,26 @@ Tensor layer_norm(const Tensor &x, const Tensor &weight, const Tensor &bias, int
 Tensor rms_norm(const Tensor &x, const Tensor &weight, int axis = -1, float eps = 1e-5f);
 
 Tensor matmul(const Tensor &a, const Tensor &b, bool transpose_a = false, bool transpose_b = false);
+
+// a * sigmoid(b) over the two halves of `dim` (src/tensor/operations.cpp:1451-1476); ValueError on an odd extent
+Tensor glu(const Tensor &x, int dim = -1);
+// where the Bool (or nonzero) mask, broadcast against x, is set the result holds `value`
+// (include/axiom/operations.hpp:437-440)
+Tensor masked_fill(const Tensor &x, const Tensor &mask, float value);
+Tensor masked_fill(const Tensor &x, const Tensor &mask, double value);
+// constant padding; pad_width holds (before, after) per dimension (include/axiom/operations.hpp:519-526)
+Tensor pad(const Tensor &x, const std::vector<std::pair<size_t, size_t>> &pad_width, const std::string &mode = "constant", double value = 0.0);
+// rows of weight (vocab, dim) selected by integer indices of any shape -> (*indices.shape, dim)
+// (include/axiom/operations.hpp:483-486).  On the GPU an index out of range gives a row of zeros.
+Tensor embedding(const Tensor &weight, const Tensor &indices);
+// PyTorch-compatible 1-D convolution: input (N, C_in, L) or (C_in, L), weight (C_out, C_in, K),
+// output (N, C_out, L_out), L_out = (L + 2 padding - dilation (K-1) - 1) / stride + 1
+// (include/axiom/operations.hpp:594-601).  groups must be 1.
+Tensor conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride = 1, int padding = 0, int dilation = 1, int groups = 1);
+Tensor conv1d(const Tensor &input, const Tensor &weight); // no bias, stride 1, no padding
+// inference batch norm over the channel dimension (dim 1) of (N, C) or (N, C, L):
+// (x - running_mean) / sqrt(running_var + eps) * weight + bias
+Tensor batch_norm1d(const Tensor &x, const Tensor &weight, const Tensor &bias, const Tensor &running_mean, const Tensor &running_var, float eps = 1e-5f);
 
 // q (B,H,Sq,D), k/v (B,H,Skv,D); mask Bool (Sq,Skv) or (B,H,Sq,Skv), true = masked out;
 // scale <= 0 means 1/sqrt(D).  ShapeError on bad ranks / mismatched batch, heads, Skv or D.

@@ -6,6 +6,7 @@
 
 #include <initializer_list>
 #include <memory>
+#include <optional>
 #include <string>
 #include <vector>
 
@@ -19,6 +20,15 @@ namespace axiom {
 namespace graph {
 struct GraphNode;
 }
+
+// start:stop:step along one dimension, Python semantics for negative and absent bounds
+// (include/axiom/indexing.hpp:13-22); the step must be positive here
+struct Slice {
+    std::optional<int64_t> start, stop, step;
+    Slice(std::optional<int64_t> start_val = std::nullopt, std::optional<int64_t> stop_val = std::nullopt,
+          std::optional<int64_t> step_val = std::nullopt)
+        : start(start_val), stop(stop_val), step(step_val) {}
+};
 
 class Tensor {
   public:
@@ -75,6 +85,9 @@ class Tensor {
     Tensor permute(const std::vector<int> &axes) const { return transpose(axes); }
     Tensor squeeze(int axis = -1) const;
     Tensor unsqueeze(int axis) const;
+    // one Slice per leading dimension; a view of materialised storage, a lazy Slice node on a lazy GPU tensor
+    Tensor slice(const std::vector<Slice> &slice_args) const;
+    std::vector<Tensor> chunk(size_t n_chunks, int axis = 0) const;
 
     // ---- device and dtype
     Tensor to(Device device) const;
@@ -99,6 +112,12 @@ class Tensor {
     Tensor log_softmax(int axis = -1) const;
     Tensor relu() const;
     Tensor gelu() const;
+    Tensor sigmoid() const;
+    Tensor silu() const;
+    Tensor tanh() const;
+    Tensor glu(int dim = -1) const;
+    Tensor masked_fill(const Tensor &mask, float value) const;
+    Tensor masked_fill(const Tensor &mask, double value) const;
     Tensor matmul(const Tensor &other, bool transpose_self = false, bool transpose_other = false) const;
 
     // ---- factories: built on the host, then moved (src/tensor/tensor.cpp:1785-1935)
@@ -106,6 +125,7 @@ class Tensor {
     static Tensor ones(const Shape &shape, DType dtype = DType::Float32, Device device = Device::CPU);
     static Tensor empty(const Shape &shape, DType dtype = DType::Float32, Device device = Device::CPU);
     static Tensor eye(size_t n, DType dtype = DType::Float32, Device device = Device::CPU);
+    static Tensor arange(int64_t start, int64_t end, int64_t step = 1, DType dtype = DType::Int64, Device device = Device::CPU);
     template <typename T> static Tensor full(const Shape &shape, const T &value, Device device = Device::CPU) {
         Tensor t(shape, dtype_of<T>::value, Device::CPU);
         t.fill_double(static_cast<double>(value));

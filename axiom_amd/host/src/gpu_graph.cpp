@@ -40,6 +40,7 @@ struct ValueSpec {
     Shape shape;
     Strides strides; // bytes
     DType dtype = DType::Float32;
+    size_t offset = 0; // bytes past the start of the leaf's data / the temporary (views cut by Slice)
 };
 
 struct RowsStep {
@@ -61,11 +62,30 @@ struct CopyStep {
     Strides src_strides; // bytes; 0 on broadcast dims
 };
 
+struct PadStep {
+    int src = -1, dst = -1;
+    std::vector<int64_t> before, after;
+    double value = 0.0;
+};
+
+struct MaskedFillStep {
+    int src = -1, mask = -1, dst = -1;
+    Strides mask_strides; // bytes == elements for the one-byte mask; 0 on broadcast dims
+    float value = 0.0f;
+};
+
+struct GatherStep {
+    int table = -1, indices = -1, dst = -1;
+};
+
 struct Step {
-    enum Kind { ROWS, GEMM, COPY } kind;
+    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER } kind;
     RowsStep rows;
     GemmStep gemm;
     CopyStep copy;
+    PadStep pad;
+    MaskedFillStep mfill;
+    GatherStep gather;
 };
 
 struct Plan {
@@ -213,6 +233,67 @@ class PlanBuilder {
                 s.strides[i] = val(in).strides[axes[i]];
             }
             v = add_value(s);
+        } else if (op == OpType::Slice) {
+            const int in = eval(n->inputs[0].get());
+            const auto &sp = get_params<SliceParams>(n->params);
+            ValueSpec s = val(in);
+            for (size_t d = 0; d < s.shape.size(); ++d) {
+                s.offset += static_cast<size_t>(sp.starts[d] * val(in).strides[d]);
+                s.strides[d] = val(in).strides[d] * sp.steps[d];
+            }
+            s.shape = n->output_shape;
+            v = add_value(s);
+        } else if (op == OpType::Unfold1D) {
+            // (N, C, L) -> windows (N, L_out, C, K): element (n, l, c, k) is input (n, c, l * stride + k * dilation)
+            const int in = eval(n->inputs[0].get());
+            const auto &up = get_params<UnfoldParams>(n->params);
+            ValueSpec s = val(in);
+            const Strides is = val(in).strides;
+            s.shape = n->output_shape;
+            s.strides = {is[0], is[2] * up.stride, is[1], is[2] * up.dilation};
+            v = add_value(s);
+        } else if (op == OpType::Pad) {
+            const int in = eval(n->inputs[0].get());
+            detail::to_axhip_dtype(val(in).dtype);
+            const auto &pp = get_params<PadParams>(n->params);
+            if (val(in).shape.size() > AXHIP_MAX_DIMS) throw RuntimeError::not_implemented("GPU pad of more than 8 dimensions");
+            Step st{};
+            st.kind = Step::PAD;
+            st.pad.src = in;
+            st.pad.dst = v = new_temp(n->output_shape, n->output_dtype);
+            for (const auto &w : pp.pad_widths) {
+                st.pad.before.push_back(static_cast<int64_t>(w.first));
+                st.pad.after.push_back(static_cast<int64_t>(w.second));
+            }
+            st.pad.value = pp.value;
+            plan_.steps.push_back(st);
+        } else if (op == OpType::MaskedFill) {
+            if (n->inputs.size() < 2) throw RuntimeError("malformed graph node 'masked_fill': missing inputs");
+            const int in = eval(n->inputs[0].get()), mk = eval(n->inputs[1].get());
+            detail::to_axhip_dtype(val(in).dtype);
+            const Shape F = val(in).shape, M = val(mk).shape; // copies: new_temp() below grows the value table
+            const Strides mask_strides = val(mk).strides;
+            if (F.size() > AXHIP_MAX_DIMS) throw RuntimeError::not_implemented("GPU masked_fill of more than 8 dimensions");
+            Step st{};
+            st.kind = Step::MASKED_FILL;
+            st.mfill.src = in;
+            st.mfill.mask = mk;
+            st.mfill.dst = v = new_temp(F, n->output_dtype);
+            st.mfill.value = get_params<MaskedFillParams>(n->params).value;
+            st.mfill.mask_strides.assign(F.size(), 0);
+            const size_t lead = F.size() - M.size();
+            for (size_t i = 0; i < M.size(); ++i) st.mfill.mask_strides[lead + i] = M[i] == 1 ? 0 : mask_strides[i];
+            plan_.steps.push_back(st);
+        } else if (op == OpType::Gather) { // embedding rows
+            if (n->inputs.size() < 2) throw RuntimeError("malformed graph node 'embedding': missing inputs");
+            const int table = make_contiguous(eval(n->inputs[0].get())), idx = eval(n->inputs[1].get());
+            if (!contiguous(idx)) throw RuntimeError::not_implemented("embedding with non-contiguous indices on the GPU");
+            Step st{};
+            st.kind = Step::GATHER;
+            st.gather.table = table;
+            st.gather.indices = idx;
+            st.gather.dst = v = new_temp(n->output_shape, n->output_dtype);
+            plan_.steps.push_back(st);
         } else if (op == OpType::MatMul) {
             v = emit_gemm(n, {}, -1, -1, 0);
         } else if (is_elementwise(op) || is_row_op(op) || is_reduction(op)) {
@@ -597,7 +678,7 @@ void materialize_gpu_graph(GraphNode *root) {
     auto ptr_of = [&](int v) -> void * {
         const ValueSpec &s = plan->values[v];
         char *base = static_cast<char *>(s.is_leaf ? leaves[s.index].storage->raw() : temps[s.index]->raw());
-        return base + (s.is_leaf ? leaves[s.index].offset : 0);
+        return base + (s.is_leaf ? leaves[s.index].offset : 0) + s.offset;
     };
 
     // ---- run
@@ -622,6 +703,28 @@ void materialize_gpu_graph(GraphNode *root) {
             p.residual = st.gemm.residual >= 0 ? ptr_of(st.gemm.residual) : nullptr;
             tl_last_kernels.emplace_back("gemm");
             AXHIP_CALL(axhip_gemm(ptr_of(st.gemm.a), ptr_of(st.gemm.b), ptr_of(st.gemm.c), &p, nullptr));
+        } else if (st.kind == Step::PAD) {
+            const ValueSpec &src = plan->values[st.pad.src];
+            const int64_t isz = static_cast<int64_t>(dtype_size(src.dtype));
+            std::vector<int64_t> shp(src.shape.begin(), src.shape.end()), est(src.strides.size());
+            for (size_t i = 0; i < est.size(); ++i) est[i] = src.strides[i] / isz;
+            tl_last_kernels.emplace_back("pad");
+            AXHIP_CALL(axhip_pad(ptr_of(st.pad.src), ptr_of(st.pad.dst), detail::to_axhip_dtype(src.dtype), static_cast<int32_t>(shp.size()), shp.data(),
+                                 est.data(), st.pad.before.data(), st.pad.after.data(), st.pad.value, nullptr));
+        } else if (st.kind == Step::MASKED_FILL) {
+            const ValueSpec &src = plan->values[st.mfill.src];
+            const int64_t isz = static_cast<int64_t>(dtype_size(src.dtype));
+            std::vector<int64_t> shp(src.shape.begin(), src.shape.end()), est(src.strides.size()), mst(st.mfill.mask_strides.begin(), st.mfill.mask_strides.end());
+            for (size_t i = 0; i < est.size(); ++i) est[i] = src.strides[i] / isz;
+            tl_last_kernels.emplace_back("masked_fill");
+            AXHIP_CALL(axhip_masked_fill(ptr_of(st.mfill.src), detail::to_axhip_dtype(src.dtype), static_cast<const uint8_t *>(ptr_of(st.mfill.mask)),
+                                         ptr_of(st.mfill.dst), static_cast<int32_t>(shp.size()), shp.data(), est.data(), mst.data(), st.mfill.value, nullptr));
+        } else if (st.kind == Step::GATHER) {
+            const ValueSpec &tab = plan->values[st.gather.table], &idx = plan->values[st.gather.indices];
+            tl_last_kernels.emplace_back("gather_rows");
+            AXHIP_CALL(axhip_gather_rows(ptr_of(st.gather.table), detail::to_axhip_dtype(tab.dtype), static_cast<int64_t>(tab.shape[0]),
+                                         static_cast<int64_t>(tab.shape[1]), ptr_of(st.gather.indices), static_cast<int32_t>(dtype_size(idx.dtype)),
+                                         static_cast<int64_t>(ShapeUtils::size(idx.shape)), ptr_of(st.gather.dst), nullptr));
         } else {
             const ValueSpec &src = plan->values[st.copy.src];
             const int dt = detail::to_axhip_dtype(src.dtype);
@@ -645,7 +748,7 @@ void materialize_gpu_graph(GraphNode *root) {
         n->cached_result_ = storage_of(v);
         n->cached_shape_ = s.shape;
         n->cached_strides_ = s.strides;
-        n->cached_offset_ = s.is_leaf ? leaves[s.index].offset : 0;
+        n->cached_offset_ = (s.is_leaf ? leaves[s.index].offset : 0) + s.offset;
         n->is_materialized_ = true;
     }
     // a materialised node no longer needs its inputs: drop the edges (src/backends/metal/

@@ -130,6 +130,17 @@ Tensor GraphRegistry::finalize_lazy_node(std::shared_ptr<GraphNode> node) {
 
 Tensor GraphRegistry::create_lazy_unary(ops::OpType op, const Tensor &input, const OpParams &params) {
     require_gpu(pick_device({&input}), op);
+    // f(transpose(x)) == transpose(f(x)) for an elementwise f: apply it below a pending transpose, where it
+    // can still fuse into whatever produces x (a GEMM epilogue, a row kernel) instead of forcing a gather
+    if (input.is_lazy() && !input.lazy_node()->is_materialized_ && input.lazy_node()->op_type == ops::OpType::Transpose &&
+        input.lazy_node()->ref_count.load() == 0 && !is_eager_mode_enabled()) {
+        const auto tn = input.lazy_node();
+        const Tensor inner = tn->inputs[0]->is_constant
+                                 ? Tensor(tn->inputs[0]->constant_storage, tn->inputs[0]->output_shape, tn->inputs[0]->constant_strides,
+                                          tn->inputs[0]->output_dtype, tn->inputs[0]->constant_offset)
+                                 : Tensor(tn->inputs[0]);
+        return create_lazy_transpose(create_lazy_unary(op, inner, params), get_params<TransposeParams>(tn->params).axes);
+    }
     auto n = std::make_shared<GraphNode>();
     n->op_type = op;
     n->inputs = {input_node(input)};
@@ -238,6 +249,20 @@ Tensor GraphRegistry::create_lazy_reshape(const Tensor &input, const Shape &new_
 }
 
 Tensor GraphRegistry::create_lazy_transpose(const Tensor &input, const std::vector<int> &axes) {
+    // transpose(transpose(x, p), q) == transpose(x, p o q); the identity gives x back
+    if (input.is_lazy() && !input.lazy_node()->is_materialized_ && input.lazy_node()->op_type == ops::OpType::Transpose &&
+        !input.lazy_node()->inputs[0]->is_constant) {
+        const auto tn = input.lazy_node();
+        const auto &inner_axes = get_params<TransposeParams>(tn->params).axes;
+        std::vector<int> composed(axes.size());
+        bool identity = true;
+        for (size_t i = 0; i < axes.size(); ++i) {
+            composed[i] = inner_axes[axes[i]];
+            identity = identity && composed[i] == static_cast<int>(i);
+        }
+        const Tensor inner(tn->inputs[0]);
+        return identity ? inner : create_lazy_transpose(inner, composed);
+    }
     auto n = std::make_shared<GraphNode>();
     n->op_type = ops::OpType::Transpose;
     n->inputs = {input_node(input)};
@@ -248,6 +273,119 @@ Tensor GraphRegistry::create_lazy_transpose(const Tensor &input, const std::vect
     n->output_dtype = input.dtype();
     n->target_device = Device::GPU;
     n->params = TransposeParams{axes};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_slice(const Tensor &input, const std::vector<int64_t> &starts, const std::vector<int64_t> &ends,
+                                        const std::vector<int64_t> &steps, const Shape &output_shape) {
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Slice;
+    n->inputs = {input_node(input)};
+    n->output_shape = output_shape;
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = SliceParams{starts, ends, steps};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_pad(const Tensor &input, const std::vector<std::pair<size_t, size_t>> &pad_widths, double value,
+                                      const Shape &output_shape) {
+    require_gpu(pick_device({&input}), ops::OpType::Pad);
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Pad;
+    n->inputs = {input_node(input)};
+    n->output_shape = output_shape;
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = PadParams{pad_widths, value};
+    return finalize_lazy_node(std::move(n));
+}
+
+Tensor GraphRegistry::create_lazy_masked_fill(const Tensor &input, const Tensor &mask, float value) {
+    require_gpu(pick_device({&input, &mask}), ops::OpType::MaskedFill);
+    if (dtype_size(mask.dtype()) != 1) throw TypeError("masked_fill: the mask must be Bool (or a one-byte integer type)");
+    const Shape out = infer_binary_shape(input.shape(), mask.shape());
+    if (out != input.shape()) throw ShapeError("masked_fill: the mask must broadcast to the input's shape");
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::MaskedFill;
+    n->inputs = {input_node(on_gpu(input)), input_node(on_gpu(mask))};
+    n->output_shape = input.shape();
+    n->output_dtype = input.dtype();
+    n->target_device = Device::GPU;
+    n->params = MaskedFillParams{value};
+    return finalize_lazy_node(std::move(n));
+}
+
+// a * sigmoid(b) over the halves of `dim`: two Slice views (gathered when the cut leaves them strided),
+// then Sigmoid and Multiply in one row kernel
+Tensor GraphRegistry::create_lazy_glu(const Tensor &input, int dim, const Shape &output_shape) {
+    require_gpu(pick_device({&input}), ops::OpType::GLU);
+    const size_t nd = input.ndim(), half = output_shape[dim];
+    std::vector<int64_t> lo(nd, 0), hi(input.shape().begin(), input.shape().end()), st(nd, 1);
+    auto a_hi = hi, b_lo = lo;
+    a_hi[dim] = static_cast<int64_t>(half);
+    b_lo[dim] = static_cast<int64_t>(half);
+    const Tensor a = create_lazy_slice(input, lo, a_hi, st, output_shape), b = create_lazy_slice(input, b_lo, hi, st, output_shape);
+    return create_lazy_binary(ops::OpType::Multiply, a, create_lazy_unary(ops::OpType::Sigmoid, b));
+}
+
+// (x - mean) / sqrt(var + eps) * w + b per channel (dim 1), lowered to x * scale + shift with the two
+// per-channel vectors computed by tiny elementwise graphs of their own
+Tensor GraphRegistry::create_lazy_batchnorm(const Tensor &input, const Tensor &weight, const Tensor &bias, const Tensor &running_mean,
+                                            const Tensor &running_var, float eps) {
+    require_gpu(pick_device({&input}), ops::OpType::BatchNorm1D);
+    if (input.ndim() != 2 && input.ndim() != 3) throw ShapeError("batch_norm1d expects (N, C) or (N, C, L), got " + std::to_string(input.ndim()) + " dimensions");
+    const size_t C = input.shape()[1];
+    for (const Tensor *t : {&running_mean, &running_var})
+        if (t->ndim() != 1 || t->shape()[0] != C) throw ShapeError("batch_norm1d: running statistics must have shape (C)");
+    const Tensor var = on_gpu(running_var), mean = on_gpu(running_mean);
+    Tensor scale = create_lazy_unary(ops::OpType::Reciprocal, create_lazy_unary(ops::OpType::Sqrt, var + eps));
+    if (!weight.empty()) scale = create_lazy_binary(ops::OpType::Multiply, scale, on_gpu(weight));
+    Tensor shift = create_lazy_unary(ops::OpType::Negate, create_lazy_binary(ops::OpType::Multiply, mean, scale));
+    if (!bias.empty()) shift = create_lazy_binary(ops::OpType::Add, shift, on_gpu(bias));
+    if (input.ndim() == 3) {
+        scale = scale.reshape({C, 1});
+        shift = shift.reshape({C, 1});
+    }
+    return create_lazy_binary(ops::OpType::Add, create_lazy_binary(ops::OpType::Multiply, input, scale), shift);
+}
+
+// Convolution as a GEMM: constant padding, the (N, L_out, C_in, K) window view of the padded signal, its
+// gather to (N, L_out, C_in K), a product with the (C_out, C_in K) filter matrix (bias and a following
+// activation ride in the GEMM epilogue), and the (N, C_out, L_out) view of the result.
+Tensor GraphRegistry::create_lazy_conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation) {
+    require_gpu(pick_device({&input}), ops::OpType::Conv1D);
+    const size_t N = input.shape()[0], Cin = input.shape()[1], L = input.shape()[2];
+    const size_t Cout = weight.shape()[0], K = weight.shape()[2];
+    const size_t Lp = L + 2 * static_cast<size_t>(padding), span = static_cast<size_t>(dilation) * (K - 1) + 1;
+    if (Lp < span) throw ShapeError("conv1d: the kernel does not fit the padded input");
+    const size_t Lout = (Lp - span) / static_cast<size_t>(stride) + 1;
+    Tensor x = on_gpu(input);
+    if (padding > 0) x = create_lazy_pad(x, {{0, 0}, {0, 0}, {static_cast<size_t>(padding), static_cast<size_t>(padding)}}, 0.0, Shape{N, Cin, Lp});
+    auto un = std::make_shared<GraphNode>();
+    un->op_type = ops::OpType::Unfold1D;
+    un->inputs = {input_node(x)};
+    un->output_shape = Shape{N, Lout, Cin, K};
+    un->output_dtype = x.dtype();
+    un->target_device = Device::GPU;
+    un->params = UnfoldParams{static_cast<int>(K), stride, dilation};
+    const Tensor cols = create_lazy_reshape(finalize_lazy_node(std::move(un)), Shape{N, Lout, Cin * K});
+    const Tensor w2 = on_gpu(weight).reshape({Cout, Cin * K});
+    Tensor y = create_lazy_matmul(cols, w2, false, true);
+    if (!bias.empty()) y = create_lazy_binary(ops::OpType::Add, y, on_gpu(bias));
+    return create_lazy_transpose(y, {0, 2, 1});
+}
+
+Tensor GraphRegistry::create_lazy_embedding(const Tensor &weight, const Tensor &indices) {
+    require_gpu(pick_device({&weight, &indices}), ops::OpType::Gather);
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Gather;
+    n->inputs = {input_node(on_gpu(weight)), input_node(on_gpu(indices))};
+    Shape out = indices.shape();
+    out.push_back(weight.shape()[1]);
+    n->output_shape = out;
+    n->output_dtype = weight.dtype();
+    n->target_device = Device::GPU;
     return finalize_lazy_node(std::move(n));
 }
 
@@ -364,6 +502,26 @@ GraphSignature compute_signature(const GraphNode *root) {
                 } else if constexpr (std::is_same_v<T, TransposeParams>) {
                     h = mix(h, p.axes.size());
                     for (int a : p.axes) h = mix_i32(h, a);
+                } else if constexpr (std::is_same_v<T, SliceParams>) {
+                    h = mix(h, p.starts.size());
+                    for (size_t i = 0; i < p.starts.size(); ++i) {
+                        h = mix(h, static_cast<uint64_t>(p.starts[i]));
+                        h = mix(h, static_cast<uint64_t>(p.ends[i]));
+                        h = mix(h, static_cast<uint64_t>(p.steps[i]));
+                    }
+                } else if constexpr (std::is_same_v<T, PadParams>) {
+                    h = mix(h, p.pad_widths.size());
+                    for (const auto &w : p.pad_widths) {
+                        h = mix(h, w.first);
+                        h = mix(h, w.second);
+                    }
+                    h = mix_bytes(h, &p.value, sizeof(p.value));
+                } else if constexpr (std::is_same_v<T, MaskedFillParams>) {
+                    h = mix_f32(h, p.value);
+                } else if constexpr (std::is_same_v<T, UnfoldParams>) {
+                    h = mix_i32(h, p.kernel);
+                    h = mix_i32(h, p.stride);
+                    h = mix_i32(h, p.dilation);
                 }
             },
             n->params);

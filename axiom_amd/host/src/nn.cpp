@@ -88,6 +88,34 @@ Tensor RMSNorm::forward(const Tensor &input) const {
 Tensor ReLU::forward(const Tensor &input) const { return ops::relu(input); }
 Tensor GELU::forward(const Tensor &input) const { return ops::gelu(input); }
 
+// ------------------------------------------- conv, embedding, batch norm
+Conv1d::Conv1d(int stride, int padding, int dilation, int groups, bool bias)
+    : stride_(stride), padding_(padding), dilation_(dilation), groups_(groups), has_bias_(bias) {
+    register_parameter("weight", weight_);
+    if (has_bias_) register_parameter("bias", bias_);
+}
+Tensor Conv1d::forward(const Tensor &input) const {
+    if (weight_.empty()) throw RuntimeError("Conv1d: weight not initialized (load_state_dict first)");
+    return ops::conv1d(input, weight_, has_bias_ ? bias_ : Tensor(), stride_, padding_, dilation_, groups_);
+}
+
+Embedding::Embedding() { register_parameter("weight", weight_); }
+Tensor Embedding::forward(const Tensor &indices) const {
+    if (weight_.empty()) throw RuntimeError("Embedding: weight not initialized (load_state_dict first)");
+    return ops::embedding(weight_, indices);
+}
+
+BatchNorm1d::BatchNorm1d(float eps) : eps_(eps) {
+    register_parameter("weight", weight_);
+    register_parameter("bias", bias_);
+    register_parameter("running_mean", running_mean_);
+    register_parameter("running_var", running_var_);
+}
+Tensor BatchNorm1d::forward(const Tensor &input) const {
+    if (running_mean_.empty() || running_var_.empty()) throw RuntimeError("BatchNorm1d: running statistics not initialized (load_state_dict first)");
+    return ops::batch_norm1d(input, weight_, bias_, running_mean_, running_var_, eps_);
+}
+
 // ------------------------------------------------------- MultiHeadAttention
 MultiHeadAttention::MultiHeadAttention(int num_heads, bool bias) : num_heads_(num_heads), q_proj_(bias), k_proj_(bias), v_proj_(bias), out_proj_(bias) {
     register_module("q_proj", q_proj_);

@@ -43,6 +43,14 @@ const char *op_name(OpType op) {
     case OpType::RMSNorm: return "rms_norm";
     case OpType::Reshape: return "reshape";
     case OpType::Transpose: return "transpose";
+    case OpType::Slice: return "slice";
+    case OpType::Pad: return "pad";
+    case OpType::MaskedFill: return "masked_fill";
+    case OpType::GLU: return "glu";
+    case OpType::Gather: return "embedding";
+    case OpType::Conv1D: return "conv1d";
+    case OpType::BatchNorm1D: return "batch_norm1d";
+    case OpType::Unfold1D: return "unfold1d";
     case OpType::ScaledDotProductAttention: return "scaled_dot_product_attention";
     default: return "op";
     }
@@ -118,6 +126,55 @@ Tensor rms_norm(const Tensor &x, const Tensor &weight, int axis, float eps) {
 }
 
 Tensor matmul(const Tensor &a, const Tensor &b, bool ta, bool tb) { return GraphRegistry::create_lazy_matmul(a, b, ta, tb); }
+
+// src/tensor/operations.cpp:1451-1476
+Tensor glu(const Tensor &x, int dim) {
+    const int nd = static_cast<int>(x.ndim());
+    const int d = dim < 0 ? dim + nd : dim;
+    if (d < 0 || d >= nd) throw ValueError("glu: dim " + std::to_string(dim) + " out of range for tensor with " + std::to_string(nd) + " dimensions");
+    if (x.shape()[d] % 2 != 0)
+        throw ValueError("glu: dimension " + std::to_string(d) + " size (" + std::to_string(x.shape()[d]) + ") must be divisible by 2");
+    Shape out = x.shape();
+    out[d] /= 2;
+    return GraphRegistry::create_lazy_glu(x, d, out);
+}
+
+Tensor masked_fill(const Tensor &x, const Tensor &mask, float value) { return GraphRegistry::create_lazy_masked_fill(x, mask, value); }
+Tensor masked_fill(const Tensor &x, const Tensor &mask, double value) { return masked_fill(x, mask, static_cast<float>(value)); }
+
+Tensor pad(const Tensor &x, const std::vector<std::pair<size_t, size_t>> &pad_width, const std::string &mode, double value) {
+    if (mode != "constant") throw RuntimeError::not_implemented("pad mode '" + mode + "' on the GPU (constant only)");
+    if (pad_width.size() != x.ndim()) throw ShapeError("pad: pad_width must have one (before, after) pair per dimension");
+    Shape out = x.shape();
+    for (size_t d = 0; d < out.size(); ++d) out[d] += pad_width[d].first + pad_width[d].second;
+    return GraphRegistry::create_lazy_pad(x, pad_width, value, out);
+}
+
+Tensor embedding(const Tensor &weight, const Tensor &indices) {
+    if (weight.ndim() != 2) throw ShapeError("embedding: weight must be (vocab_size, embed_dim)");
+    if (indices.dtype() != DType::Int64 && indices.dtype() != DType::Int32) throw TypeError("embedding: indices must be Int32 or Int64");
+    return GraphRegistry::create_lazy_embedding(weight, indices);
+}
+
+Tensor conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation, int groups) {
+    if (groups != 1) throw RuntimeError::not_implemented("grouped conv1d on the GPU");
+    if (stride < 1 || dilation < 1 || padding < 0) throw ValueError("conv1d: stride and dilation must be positive, padding non-negative");
+    if (input.ndim() == 2) { // unbatched (C_in, L)
+        const Tensor y = conv1d(input.unsqueeze(0), weight, bias, stride, padding, dilation, groups);
+        return y.squeeze(0);
+    }
+    if (input.ndim() != 3 || weight.ndim() != 3) throw ShapeError("conv1d expects input (N, C_in, L) and weight (C_out, C_in, K)");
+    if (input.shape()[1] != weight.shape()[1])
+        throw ShapeError("conv1d: input has " + std::to_string(input.shape()[1]) + " channels, weight expects " + std::to_string(weight.shape()[1]));
+    if (!bias.empty() && (bias.ndim() != 1 || bias.shape()[0] != weight.shape()[0])) throw ShapeError("conv1d: bias must have shape (C_out)");
+    return GraphRegistry::create_lazy_conv1d(input, weight, bias, stride, padding, dilation);
+}
+
+Tensor conv1d(const Tensor &input, const Tensor &weight) { return conv1d(input, weight, Tensor(), 1, 0, 1, 1); }
+
+Tensor batch_norm1d(const Tensor &x, const Tensor &weight, const Tensor &bias, const Tensor &running_mean, const Tensor &running_var, float eps) {
+    return GraphRegistry::create_lazy_batchnorm(x, weight, bias, running_mean, running_var, eps);
+}
 
 // ---------------------------------------------------------------- attention
 namespace {

@@ -218,6 +218,51 @@ Tensor Tensor::transpose(const std::vector<int> &axes) const {
     return Tensor(storage_, s, st, dtype_, offset_);
 }
 
+// Python slice semantics per dimension (src/tensor/tensor.cpp slice(); include/axiom/indexing.hpp:13-22)
+Tensor Tensor::slice(const std::vector<Slice> &args) const {
+    const Shape &in = shape();
+    if (args.size() > in.size()) throw IndexError("slice: " + std::to_string(args.size()) + " slices for a tensor with " + std::to_string(in.size()) + " dimensions");
+    const size_t nd = in.size();
+    std::vector<int64_t> starts(nd, 0), ends(in.begin(), in.end()), steps(nd, 1);
+    Shape out = in;
+    for (size_t d = 0; d < args.size(); ++d) {
+        const int64_t n = static_cast<int64_t>(in[d]), step = args[d].step.value_or(1);
+        if (step <= 0) throw ValueError("slice: only positive steps are supported");
+        int64_t b = args[d].start.value_or(0), e = args[d].stop.value_or(n);
+        if (b < 0) b += n;
+        if (e < 0) e += n;
+        b = std::min(std::max<int64_t>(b, 0), n);
+        e = std::min(std::max<int64_t>(e, b), n);
+        starts[d] = b;
+        ends[d] = e;
+        steps[d] = step;
+        out[d] = static_cast<size_t>((e - b + step - 1) / step);
+    }
+    if (lazy_node_ && lazy_node_->target_device == Device::GPU && !lazy_node_->is_materialized_)
+        return graph::GraphRegistry::create_lazy_slice(*this, starts, ends, steps, out);
+    materialize_if_needed();
+    Strides st = strides_;
+    size_t off = offset_;
+    for (size_t d = 0; d < nd; ++d) {
+        off += static_cast<size_t>(starts[d] * strides_[d]);
+        st[d] = strides_[d] * steps[d];
+    }
+    return Tensor(storage_, out, st, dtype_, off);
+}
+
+std::vector<Tensor> Tensor::chunk(size_t n_chunks, int axis) const {
+    if (n_chunks == 0) throw ValueError("chunk: the number of chunks must be positive");
+    const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(ndim()));
+    const size_t n = shape()[a], each = (n + n_chunks - 1) / n_chunks;
+    std::vector<Tensor> out;
+    for (size_t b = 0; b < n; b += each) {
+        std::vector<Slice> args(a + 1);
+        args[a] = Slice(static_cast<int64_t>(b), static_cast<int64_t>(std::min(n, b + each)));
+        out.push_back(slice(args));
+    }
+    return out;
+}
+
 Tensor Tensor::squeeze(int axis) const {
     const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(ndim()));
     if (shape()[a] != 1) throw ShapeError("squeeze: dimension " + std::to_string(a) + " has extent " + std::to_string(shape()[a]));
@@ -313,6 +358,12 @@ Tensor Tensor::softmax(int axis) const { return ops::softmax(*this, axis); }
 Tensor Tensor::log_softmax(int axis) const { return ops::log_softmax(*this, axis); }
 Tensor Tensor::relu() const { return ops::relu(*this); }
 Tensor Tensor::gelu() const { return ops::gelu(*this); }
+Tensor Tensor::sigmoid() const { return ops::sigmoid(*this); }
+Tensor Tensor::silu() const { return ops::silu(*this); }
+Tensor Tensor::tanh() const { return ops::tanh(*this); }
+Tensor Tensor::glu(int dim) const { return ops::glu(*this, dim); }
+Tensor Tensor::masked_fill(const Tensor &mask, float value) const { return ops::masked_fill(*this, mask, value); }
+Tensor Tensor::masked_fill(const Tensor &mask, double value) const { return ops::masked_fill(*this, mask, value); }
 Tensor Tensor::matmul(const Tensor &o, bool ta, bool tb) const { return ops::matmul(*this, o, ta, tb); }
 
 // --------------------------------------------------------------- factories
@@ -330,6 +381,14 @@ Tensor Tensor::empty(const Shape &shape, DType dtype, Device device) { return Te
 Tensor Tensor::eye(size_t n, DType dtype, Device device) {
     Tensor t = zeros({n, n}, dtype, Device::CPU);
     for (size_t i = 0; i < n; ++i) t.set_item_double({i, i}, 1.0);
+    return device == Device::GPU ? t.to(device) : t;
+}
+
+Tensor Tensor::arange(int64_t start, int64_t end, int64_t step, DType dtype, Device device) {
+    if (step == 0) throw ValueError("arange: step must not be zero");
+    const int64_t n = step > 0 ? std::max<int64_t>(0, (end - start + step - 1) / step) : std::max<int64_t>(0, (start - end - step - 1) / -step);
+    Tensor t(Shape{static_cast<size_t>(n)}, dtype, Device::CPU);
+    for (int64_t i = 0; i < n; ++i) t.set_item_double({static_cast<size_t>(i)}, static_cast<double>(start + i * step));
     return device == Device::GPU ? t.to(device) : t;
 }
 

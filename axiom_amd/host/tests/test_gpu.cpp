@@ -646,3 +646,199 @@ GPU_TEST(BackendHooks, CpuPlannedFusedSteps) { // include/axiom/graph/gpu_fusion
         for (size_t j = 0; j < 16; ++j) want += double(a.item<float>({i, j})) + b.item<float>({i, j});
     EXPECT_NEAR(buffers[3].cpu().item<float>(), want, 1e-3);
 }
+
+// ------------------------------------------------- remaining lazy node kinds
+// Known answers of the reference's tests/test_conv1d.cpp, test_embedding.cpp,
+// test_nn_ergonomics.cpp:41-90 (glu), test_shape_ops_extended.cpp:42-77 (pad) and
+// test_tensor_where.cpp:212-218 (masked_fill), plus float64 loops on random inputs.
+static Tensor gpu_f32(std::initializer_list<float> v, const Shape &shape) {
+    std::vector<float> d(v);
+    return Tensor::from_data(d.data(), shape, Device::GPU);
+}
+
+GPU_TEST(LazyNodes, Conv1dKnownAnswers) {
+    auto x5 = gpu_f32({1, 2, 3, 4, 5}, {1, 1, 5});
+    auto w3 = gpu_f32({1, 1, 1}, {1, 1, 3});
+    auto r = ops::conv1d(x5, w3); // :3-16
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 3}));
+    auto h = host_floats(r);
+    EXPECT_NEAR(h[0], 6.0f, 0); EXPECT_NEAR(h[1], 9.0f, 0); EXPECT_NEAR(h[2], 12.0f, 0);
+    h = host_floats(ops::conv1d(x5, w3, Tensor(), 1, 1)); // :18-33, pad 1
+    ASSERT_EQ(h.size(), 5u);
+    const float want_pad[5] = {3, 6, 9, 12, 9};
+    for (int i = 0; i < 5; ++i) EXPECT_NEAR(h[i], want_pad[i], 0);
+    r = ops::conv1d(gpu_f32({1, 2, 3, 4, 5, 6}, {1, 1, 6}), w3, Tensor(), 2); // :35-46, stride 2
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 2}));
+    h = host_floats(r);
+    EXPECT_NEAR(h[0], 6.0f, 0); EXPECT_NEAR(h[1], 12.0f, 0);
+    r = ops::conv1d(x5, w3, Tensor(), 1, 0, 2); // :48-61, dilation 2
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 1}));
+    EXPECT_NEAR(r.item<float>(), 9.0f, 0);
+    EXPECT_NEAR(ops::conv1d(gpu_f32({1, 2, 3}, {1, 1, 3}), w3, gpu_f32({10}, {1})).item<float>(), 16.0f, 0); // :63-75, bias
+    r = ops::conv1d(gpu_f32({1, 2, 3, 4, 5, 6, 7, 8}, {1, 2, 4}), gpu_f32({1, 0, 0, 1, 1, 0, 0, 1, 1, 1, 1, 1}, {3, 2, 2})); // :77-90
+    EXPECT_TRUE(r.shape() == Shape({1, 3, 3}));
+    h = host_floats(r); // out[co][l] = sum_ci,k w[co][ci][k] x[ci][l+k]
+    const float want_mc[9] = {7, 9, 11, 7, 9, 11, 14, 18, 22};
+    for (int i = 0; i < 9; ++i) EXPECT_NEAR(h[i], want_mc[i], 0);
+    r = ops::conv1d(gpu_f32({1, 2, 3, 4, 5}, {1, 5}), w3); // :92-102, unbatched
+    EXPECT_TRUE(r.shape() == Shape({1, 3}));
+    EXPECT_NEAR(host_floats(r)[0], 6.0f, 0);
+    EXPECT_THROW(ops::conv1d(x5, w3, Tensor(), 1, 0, 1, 2), RuntimeError);               // groups
+    EXPECT_THROW(ops::conv1d(x5, gpu_f32({1, 1, 1, 1, 1, 1}, {1, 2, 3})), ShapeError); // channel mismatch
+}
+
+static void conv1d_case(DType dt, size_t N, size_t Cin, size_t L, size_t Cout, size_t K, int stride, int padding, int dilation, bool gelu, double tol) {
+    auto x = axtest::randn({N, Cin, L}, 70, dt), w = axtest::randn({Cout, Cin, K}, 71, dt, 0.2f), b = axtest::randn({Cout}, 72, dt, 0.5f);
+    Tensor y = ops::conv1d(x.gpu(), w.gpu(), b.gpu(), stride, padding, dilation);
+    if (gelu) y = y.gelu();
+    const size_t Lout = (L + 2 * padding - dilation * (K - 1) - 1) / stride + 1;
+    ASSERT_TRUE(y.shape() == Shape({N, Cout, Lout}));
+    auto got = host_floats(y);
+    if (gelu) { // pad (if any), window gather, one GEMM carrying bias and GELU: no separate elementwise pass, no transposing copy
+        const auto &k = graph::last_gpu_plan_kernels();
+        EXPECT_EQ(k.size(), padding > 0 ? 3u : 2u);
+        EXPECT_EQ(k.back(), std::string("gemm"));
+    }
+    auto xf = host_floats(x), wf = host_floats(w), bf = host_floats(b);
+    double worst = 0;
+    for (size_t n = 0; n < N; ++n)
+        for (size_t co = 0; co < Cout; ++co)
+            for (size_t l = 0; l < Lout; ++l) {
+                double acc = bf[co];
+                for (size_t ci = 0; ci < Cin; ++ci)
+                    for (size_t k = 0; k < K; ++k) {
+                        const long pos = static_cast<long>(l * stride + k * dilation) - padding;
+                        if (pos >= 0 && pos < static_cast<long>(L)) acc += double(wf[(co * Cin + ci) * K + k]) * xf[(n * Cin + ci) * L + pos];
+                    }
+                if (gelu) acc = 0.5 * acc * (1.0 + std::erf(acc / std::sqrt(2.0)));
+                worst = std::max(worst, std::fabs(acc - got[(n * Cout + co) * Lout + l]));
+            }
+    EXPECT_LT(worst, tol);
+}
+GPU_TEST(LazyNodes, Conv1dMatchesFloat64Loops) {
+    conv1d_case(DType::Float32, 2, 5, 37, 7, 3, 1, 1, 1, false, 1e-4);
+    conv1d_case(DType::Float32, 1, 4, 50, 6, 4, 3, 2, 2, true, 1e-4);
+    conv1d_case(DType::BFloat16, 2, 16, 64, 24, 3, 2, 1, 1, true, 2e-2);  // the Whisper stem pattern: conv, GELU
+    conv1d_case(DType::Float16, 1, 8, 40, 8, 3, 1, 0, 1, false, 2e-2);
+}
+
+GPU_TEST(LazyNodes, EmbeddingLookup) { // tests/test_embedding.cpp:3-39
+    std::vector<float> wd(12);
+    for (int i = 0; i < 12; ++i) wd[i] = float(i);
+    auto w = Tensor::from_data(wd.data(), {4, 3}, Device::GPU);
+    std::vector<int64_t> id{0, 2};
+    auto r = ops::embedding(w, Tensor::from_data(id.data(), {2}, Device::GPU));
+    EXPECT_TRUE(r.shape() == Shape({2, 3}));
+    auto h = host_floats(r);
+    const float want[6] = {0, 1, 2, 6, 7, 8};
+    for (int i = 0; i < 6; ++i) EXPECT_NEAR(h[i], want[i], 0);
+    std::vector<int64_t> id2{0, 1, 2, 3, 4, 0};
+    auto w2 = Tensor::from_data(wd.data(), {5, 2}, Device::GPU);
+    r = ops::embedding(w2, Tensor::from_data(id2.data(), {2, 3})); // host indices are moved over
+    EXPECT_TRUE(r.shape() == Shape({2, 3, 2}));
+    h = host_floats(r);
+    EXPECT_NEAR(h[0], 0.0f, 0); EXPECT_NEAR(h[1], 1.0f, 0); EXPECT_NEAR(h[10], 0.0f, 0); EXPECT_NEAR(h[11], 1.0f, 0);
+    // positions = arange: the embedding table's leading rows, added to a sequence (the Whisper encoder's use)
+    auto pos = Tensor::arange(0, 3).gpu();
+    auto x = Tensor::full<float>({1, 3, 2}, 1.0f, Device::GPU);
+    h = host_floats(ops::add(x, ops::embedding(w2, pos)));
+    for (int i = 0; i < 6; ++i) EXPECT_NEAR(h[i], 1.0f + float(i), 0);
+    std::vector<float> fidx{0.0f};
+    EXPECT_THROW(ops::embedding(w, Tensor::from_data(fidx.data(), {1}, Device::GPU)), TypeError);
+}
+
+GPU_TEST(LazyNodes, GluSliceChunk) { // tests/test_nn_ergonomics.cpp:44-76
+    auto in = gpu_f32({1, 2, 3, 0, 0, 0, 4, 5, 6, 0, 0, 0}, {2, 6});
+    auto r = ops::glu(in, -1);
+    EXPECT_TRUE(r.shape() == Shape({2, 3}));
+    auto h = host_floats(r);
+    const float want[6] = {0.5f, 1.0f, 1.5f, 2.0f, 2.5f, 3.0f}; // sigmoid(0) = 0.5
+    for (int i = 0; i < 6; ++i) EXPECT_NEAR(h[i], want[i], 1e-5);
+    auto x = axtest::randn({6, 4}, 80);
+    auto g = x.gpu();
+    EXPECT_TRUE(g.glu(0).shape() == Shape({3, 4}));
+    auto xf = host_floats(x), g0 = host_floats(g.glu(0)), g1 = host_floats(ops::glu(ops::add(g, g), 1)); // the second on a lazy input
+    for (size_t i = 0; i < 12; ++i) EXPECT_NEAR(g0[i], xf[i] / (1.0 + std::exp(-double(xf[12 + i]))), 1e-5);
+    for (size_t r2 = 0; r2 < 6; ++r2)
+        for (size_t c = 0; c < 2; ++c) EXPECT_NEAR(g1[r2 * 2 + c], 2 * xf[r2 * 4 + c] / (1.0 + std::exp(-2.0 * xf[r2 * 4 + 2 + c])), 1e-5);
+    EXPECT_THROW(ops::glu(Tensor::zeros({2, 5}, DType::Float32, Device::GPU), -1), ValueError);
+    // slices and chunks of device tensors are views; of lazy tensors, lazy Slice nodes
+    auto parts = g.chunk(2, 1);
+    ASSERT_EQ(parts.size(), 2u);
+    EXPECT_EQ(parts[1].storage().get(), g.storage().get());
+    auto ph = host_floats(parts[1]);
+    for (size_t r2 = 0; r2 < 6; ++r2) EXPECT_NEAR(ph[r2 * 2], xf[r2 * 4 + 2], 0);
+    auto lz = ops::relu(g).slice({Slice(1, 5, 2), Slice(-3)}); // rows 1 and 3, last three columns
+    EXPECT_TRUE(lz.is_lazy());
+    EXPECT_TRUE(lz.shape() == Shape({2, 3}));
+    auto lh = host_floats(lz);
+    for (size_t i = 0; i < 2; ++i)
+        for (size_t c = 0; c < 3; ++c) EXPECT_NEAR(lh[i * 3 + c], std::max(0.0f, xf[(1 + 2 * i) * 4 + 1 + c]), 0);
+}
+
+GPU_TEST(LazyNodes, PadAndMaskedFill) { // tests/test_shape_ops_extended.cpp:42-67, tests/test_tensor_where.cpp:212-218
+    auto p = ops::pad(Tensor::ones({3, 3}, DType::Float32, Device::GPU), {{1, 1}, {1, 1}}, "constant", 0.0);
+    EXPECT_TRUE(p.shape() == Shape({5, 5}));
+    auto h = host_floats(p);
+    EXPECT_NEAR(h[0], 0.0f, 0); EXPECT_NEAR(h[2 * 5 + 2], 1.0f, 0);
+    p = ops::pad(Tensor::ones({2, 2}, DType::Float32, Device::GPU), {{1, 2}, {0, 3}}, "constant", 5.0);
+    EXPECT_TRUE(p.shape() == Shape({5, 5}));
+    h = host_floats(p);
+    EXPECT_NEAR(h[0], 5.0f, 0); EXPECT_NEAR(h[24], 5.0f, 0); EXPECT_NEAR(h[5], 1.0f, 0);
+    EXPECT_THROW(ops::pad(p, {{1, 1}, {1, 1}}, "reflect"), RuntimeError);
+    EXPECT_THROW(ops::pad(p, {{1, 1}}), ShapeError);
+    // ReLU through masked_fill, and the attention use: a (Sq, Skv) causal mask over (B, H, Sq, Skv) scores
+    auto x = axtest::randn({2, 3, 4, 4}, 81);
+    auto xf = host_floats(x);
+    Tensor neg(x.shape(), DType::Bool), causal(Shape{4, 4}, DType::Bool);
+    for (size_t i = 0; i < x.size(); ++i) static_cast<uint8_t *>(neg.data())[i] = xf[i] < 0;
+    for (size_t i = 0; i < 4; ++i)
+        for (size_t j = 0; j < 4; ++j) static_cast<uint8_t *>(causal.data())[i * 4 + j] = j > i;
+    auto r1 = host_floats(x.gpu().masked_fill(neg.gpu(), 0.0f)), r2 = host_floats(ops::masked_fill(x.gpu() * 2.0f, causal, -1e9));
+    for (size_t i = 0; i < x.size(); ++i) {
+        EXPECT_NEAR(r1[i], std::max(0.0f, xf[i]), 0);
+        EXPECT_NEAR(r2[i], (i % 4) > ((i / 4) % 4) ? -1e9f : 2 * xf[i], 0);
+    }
+    auto sm = host_floats(ops::softmax(ops::masked_fill(x.gpu(), causal.gpu(), -1e9f), -1)); // masked scores then softmax: row 0 keeps key 0 only
+    EXPECT_NEAR(sm[0], 1.0f, 1e-6); EXPECT_NEAR(sm[1], 0.0f, 1e-6);
+    std::vector<float> fm(16, 0.0f);
+    EXPECT_THROW(ops::masked_fill(x.gpu(), Tensor::from_data(fm.data(), {4, 4}, Device::GPU), 0.0f), TypeError);
+}
+
+GPU_TEST(LazyNodes, BatchNorm1dInference) {
+    const size_t N = 3, C = 5, L = 7;
+    auto w = axtest::uniform({C}, 90, 0.5f, 1.5f), b = axtest::randn({C}, 91), rm = axtest::randn({C}, 92), rv = axtest::uniform({C}, 93, 0.2f, 2.0f);
+    std::map<std::string, Tensor> sd{{"weight", w.gpu()}, {"bias", b.gpu()}, {"running_mean", rm.gpu()}, {"running_var", rv.gpu()}};
+    nn::BatchNorm1d bn;
+    EXPECT_THROW(bn(Tensor::zeros({N, C}, DType::Float32, Device::GPU)), RuntimeError);
+    bn.load_state_dict(sd);
+    auto wf = host_floats(w), bf = host_floats(b), mf = host_floats(rm), vf = host_floats(rv);
+    for (int nd = 2; nd <= 3; ++nd) {
+        auto x = nd == 2 ? axtest::randn({N, C}, 94) : axtest::randn({N, C, L}, 95);
+        auto xf = host_floats(x), got = host_floats(bn(x.gpu()));
+        const size_t inner = nd == 2 ? 1 : L;
+        for (size_t i = 0; i < xf.size(); ++i) {
+            const size_t c = (i / inner) % C;
+            EXPECT_NEAR(got[i], (double(xf[i]) - mf[c]) / std::sqrt(double(vf[c]) + 1e-5) * wf[c] + bf[c], 1e-4);
+        }
+    }
+    EXPECT_THROW(bn(Tensor::zeros({N, C, L, 2}, DType::Float32, Device::GPU)), ShapeError);
+}
+
+GPU_TEST(LazyNodes, TransposeRewritesKeepFusion) {
+    // unary over a pending transpose sinks below it; transposes compose, the identity disappears
+    auto x = axtest::randn({8, 16, 32}, 96);
+    auto g = x.gpu();
+    auto y = (g + 1.0f).transpose({0, 2, 1}).gelu().transpose({0, 2, 1}); // == gelu(x + 1), no gather
+    EXPECT_TRUE(y.shape() == x.shape());
+    auto got = host_floats(y), xf = host_floats(x);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    for (size_t i = 0; i < xf.size(); ++i) {
+        const double v = double(xf[i]) + 1.0;
+        EXPECT_NEAR(got[i], 0.5 * v * (1.0 + std::erf(v / std::sqrt(2.0))), 1e-4);
+    }
+    auto z = host_floats(ops::relu(g.transpose({2, 0, 1})).transpose({1, 0, 2})); // composed permutation (0, 2, 1) of x
+    for (size_t a = 0; a < 8; ++a)
+        for (size_t c = 0; c < 32; ++c)
+            for (size_t b2 = 0; b2 < 16; ++b2) EXPECT_NEAR(z[(a * 32 + c) * 16 + b2], std::max(0.0f, xf[(a * 16 + b2) * 32 + c]), 0);
+}
