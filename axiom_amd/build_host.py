@@ -68,6 +68,9 @@ def build_all(verbose: bool = True) -> None:
     bench = HOST / "bench" / "host_bench.cpp"
     if bench.exists():
         _run([cxx, *CXXFLAGS, str(bench), "-o", str(BENCH_BIN), f"-L{LIB_DIR}", "-laxiom_hip", "-laxhip", "-Wl,-rpath,$ORIGIN"], "build host_bench")
+    for example in sorted((HOST / "examples").glob("*.cpp")):
+        _run([cxx, *CXXFLAGS, str(example), "-o", str(LIB_DIR / example.stem), f"-L{LIB_DIR}", "-laxiom_hip", "-laxhip", "-Wl,-rpath,$ORIGIN"],
+             f"build {example.stem}")
     if verbose:
         print(f"[axiom_amd.build_host] built {HOST_LIB.name}" + (f" and {TEST_BIN.name}" if tests else "") + f" ({time.time() - t0:.1f}s)", flush=True)
 

@@ -245,3 +245,135 @@ TEST(Random, Pcg64StreamIsFixed) {
     PCG64 other(43, 54);
     EXPECT_NE(other(), PCG64(42, 54)());
 }
+
+// ------------------------------------------------------------- safetensors
+// tests/test_io_safetensors.cpp:31-141 of the reference, plus malformed files.
+#include <cstdio>
+#include <fstream>
+
+namespace {
+std::string st_path(const std::string &name) {
+    const char *tmp = std::getenv("TMPDIR");
+    return std::string(tmp && *tmp ? tmp : "/tmp") + "/axiom_hip_test_" + name + ".safetensors";
+}
+void write_st(const std::string &path, const std::string &header, const std::vector<uint8_t> &data, int64_t header_len_override = -1) {
+    std::ofstream f(path, std::ios::binary);
+    const uint64_t n = header_len_override >= 0 ? static_cast<uint64_t>(header_len_override) : header.size();
+    f.write(reinterpret_cast<const char *>(&n), 8);
+    f.write(header.data(), static_cast<std::streamsize>(header.size()));
+    f.write(reinterpret_cast<const char *>(data.data()), static_cast<std::streamsize>(data.size()));
+}
+template <typename T> std::vector<uint8_t> bytes_of(const std::vector<T> &v) {
+    std::vector<uint8_t> b(v.size() * sizeof(T));
+    std::memcpy(b.data(), v.data(), b.size());
+    return b;
+}
+} // namespace
+
+TEST(SafeTensors, DetectionAndSingleTensor) { // :31-63
+    namespace st = io::safetensors;
+    EXPECT_TRUE(st::is_safetensors_file("model.safetensors"));
+    EXPECT_TRUE(st::is_safetensors_file("/path/to/weights.safetensors"));
+    EXPECT_FALSE(st::is_safetensors_file("model.bin"));
+    EXPECT_FALSE(st::is_safetensors_file("model.npy"));
+    const std::string path = st_path("single");
+    write_st(path, R"({"weight":{"dtype":"F32","shape":[2,3],"data_offsets":[0,24]}})", bytes_of<float>({1, 2, 3, 4, 5, 6}));
+    auto tensors = st::load(path);
+    ASSERT_EQ(tensors.size(), 1u);
+    ASSERT_TRUE(tensors.count("weight") > 0);
+    auto &t = tensors["weight"];
+    EXPECT_TRUE(t.shape() == Shape({2, 3}));
+    EXPECT_EQ(t.dtype(), DType::Float32);
+    EXPECT_TRUE(t.device() == Device::CPU);
+    EXPECT_NEAR(t.item<float>({0, 0}), 1.0f, 0);
+    EXPECT_NEAR(t.item<float>({1, 2}), 6.0f, 0);
+    std::remove(path.c_str());
+}
+
+TEST(SafeTensors, SeveralTensorsListingMetadataAndDtypes) { // :65-141
+    namespace st = io::safetensors;
+    const std::string path = st_path("multi");
+    std::vector<uint8_t> data = bytes_of<float>({1, 2, 3, 4});
+    const auto i64 = bytes_of<int64_t>({10, 20, 30});
+    data.insert(data.end(), i64.begin(), i64.end());
+    const auto bf = bytes_of<uint16_t>({0x3F80, 0x4000}); // bf16 1.0, 2.0
+    data.insert(data.end(), bf.begin(), bf.end());
+    data.push_back(1); // BOOL
+    data.push_back(0);
+    write_st(path,
+             "{ \"__metadata__\": {\"format\": \"pt\", \"note\": \"a \\\"quoted\\\" value\", \"nested\": {\"k\": [1, 2.5, true, null]}},\n"
+             "  \"a\": {\"dtype\": \"F32\", \"shape\": [2, 2], \"data_offsets\": [0, 16]},\n"
+             "  \"b\": {\"dtype\":\"I64\",\"shape\":[3],\"data_offsets\":[16,40]},\n"
+             "  \"c.weight\": {\"shape\":[2],\"data_offsets\":[40,44],\"dtype\":\"BF16\"},\n"
+             "  \"flag\": {\"dtype\":\"BOOL\",\"shape\":[2],\"data_offsets\":[44,46]},\n"
+             "  \"empty\": {\"dtype\":\"F16\",\"shape\":[0,4],\"data_offsets\":[46,46]} }",
+             data);
+    auto names = st::list_tensors(path);
+    ASSERT_EQ(names.size(), 5u); // __metadata__ is not a tensor
+    std::set<std::string> ns(names.begin(), names.end());
+    EXPECT_TRUE(ns.count("a") && ns.count("b") && ns.count("c.weight") && ns.count("flag") && ns.count("empty"));
+    auto all = st::load(path);
+    ASSERT_EQ(all.size(), 5u);
+    EXPECT_NEAR(all["a"].item<float>({1, 1}), 4.0f, 0);
+    EXPECT_EQ(all["b"].dtype(), DType::Int64);
+    EXPECT_EQ(all["b"].item<int64_t>({2}), 30);
+    EXPECT_EQ(all["c.weight"].dtype(), DType::BFloat16);
+    EXPECT_NEAR(all["c.weight"].item<float>({1}), 2.0f, 0);
+    EXPECT_EQ(all["flag"].dtype(), DType::Bool);
+    EXPECT_EQ(all["flag"].item<int>({0}), 1);
+    EXPECT_EQ(all["empty"].size(), 0u);
+    auto one = st::load_tensor(path, "b");
+    EXPECT_TRUE(one.shape() == Shape({3}));
+    EXPECT_EQ(one.item<int64_t>({0}), 10);
+    EXPECT_THROW(st::load_tensor(path, "missing"), io::SerializationError);
+    std::remove(path.c_str());
+}
+
+TEST(SafeTensors, MalformedFilesAreRejected) {
+    namespace st = io::safetensors;
+    EXPECT_THROW(st::load(st_path("does_not_exist")), io::SerializationError);
+    const std::string path = st_path("bad");
+    const auto four = bytes_of<float>({1, 2, 3, 4});
+    auto expect_format_error = [&](const std::string &header, const std::vector<uint8_t> &data, int64_t len = -1) {
+        write_st(path, header, data, len);
+        EXPECT_THROW(st::load(path), io::FileFormatError);
+    };
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2],"data_offsets":[0,16]}})", four, 1 << 30);           // header length beyond the file
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2],"data_offsets":[0,32]}})", four);                    // byte range does not match the shape
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[4,2],"data_offsets":[0,32]}})", four);                    // range outside the file
+    expect_format_error(R"({"w":{"dtype":"Q4","shape":[2,2],"data_offsets":[0,16]}})", four);                     // unknown dtype
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2]}})", four);                                          // no offsets
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[2,-2],"data_offsets":[0,16]}})", four);                   // negative extent
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2],"data_offsets":[16,0]}})", four);                    // reversed range
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2],"data_offsets":[0,16]})", four);                     // unterminated object
+    {
+        std::ofstream f(path, std::ios::binary); // shorter than the length field
+        f.write("abc", 3);
+    }
+    EXPECT_THROW(st::load(path), io::FileFormatError);
+    std::remove(path.c_str());
+}
+
+// A file written by the safetensors Python package itself (tests/test_host_layer.py names it in
+// AXIOM_TEST_SAFETENSORS): "ramp_<dtype>" tensors hold 0, 1, 2, ... in shape (3, 5); skipped when unset.
+TEST(SafeTensors, ReadsFilesWrittenByTheReferenceImplementation) {
+    const char *path = std::getenv("AXIOM_TEST_SAFETENSORS");
+    if (!path || !*path) throw axtest::Skip("AXIOM_TEST_SAFETENSORS not set");
+    auto all = io::safetensors::load(path);
+    const std::pair<const char *, DType> want[] = {{"ramp_f32", DType::Float32}, {"ramp_f16", DType::Float16}, {"ramp_bf16", DType::BFloat16},
+                                                   {"ramp_i64", DType::Int64},   {"ramp_i32", DType::Int32},   {"ramp_u8", DType::UInt8}};
+    for (const auto &[name, dt] : want) {
+        ASSERT_TRUE(all.count(name) > 0);
+        const Tensor &t = all.at(name);
+        EXPECT_EQ(t.dtype(), dt);
+        EXPECT_TRUE(t.shape() == Shape({3, 5}));
+        for (size_t i = 0; i < 3; ++i)
+            for (size_t j = 0; j < 5; ++j) EXPECT_NEAR(t.item<double>({i, j}), double(i * 5 + j), 0);
+    }
+    ASSERT_TRUE(all.count("mask") > 0);
+    EXPECT_EQ(all.at("mask").dtype(), DType::Bool);
+    EXPECT_EQ(all.at("mask").item<int>({1}), 1);
+    EXPECT_EQ(all.at("mask").item<int>({2}), 0);
+    EXPECT_EQ(all.at("scalar").ndim(), 0u);
+    EXPECT_NEAR(all.at("scalar").item<float>({}), 2.5f, 0);
+}

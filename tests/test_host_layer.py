@@ -21,9 +21,9 @@ def _ensure_built():
         build_host.build_all()
 
 
-def _run(*args, timeout=600):
+def _run(*args, timeout=600, env=None):
     _ensure_built()
-    p = subprocess.run([str(BIN), *args], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
+    p = subprocess.run([str(BIN), *args], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout, env=env)
     print(p.stdout[-6000:])
     return p
 
@@ -32,6 +32,26 @@ def test_host_cases_without_device():
     p = _run("--cpu")
     assert p.returncode == 0, p.stdout[-3000:]
     assert " 0 failed" in p.stdout
+
+
+def test_safetensors_reader_on_a_file_from_the_python_package(tmp_path):
+    """The C++ reader against the format's own implementation: every dtype the weights of a
+    model can have, a 0-d tensor, and the package's metadata block."""
+    import os
+
+    import numpy as np
+    import torch
+    from safetensors.torch import save_file
+
+    ramp = torch.arange(15, dtype=torch.float32).reshape(3, 5)
+    tensors = {"ramp_f32": ramp, "ramp_f16": ramp.half(), "ramp_bf16": ramp.bfloat16(), "ramp_i64": ramp.long(), "ramp_i32": ramp.int(),
+               "ramp_u8": ramp.to(torch.uint8), "mask": torch.tensor([False, True, False]), "scalar": torch.tensor(2.5)}
+    path = tmp_path / "from_python.safetensors"
+    save_file(tensors, str(path), metadata={"format": "pt", "note": "written by safetensors"})
+    assert np.frombuffer(path.read_bytes()[:8], np.uint64)[0] > 0
+    p = _run("--cpu", "SafeTensors", env={**os.environ, "AXIOM_TEST_SAFETENSORS": str(path)})
+    assert p.returncode == 0, p.stdout[-3000:]
+    assert " 0 failed" in p.stdout and " 0 skipped" in p.stdout
 
 
 def test_product_libraries_do_not_link_the_oracle():
