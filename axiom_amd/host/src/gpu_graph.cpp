@@ -20,6 +20,7 @@
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
+#include <unordered_set>
 
 #include "axiom/error.hpp"
 #include "axiom/graph/graph_cache.hpp"
@@ -144,10 +145,38 @@ int binary_code(OpType op, bool chain_is_rhs) {
     }
 }
 
+// Interior nodes whose result must exist on its own after the graph has run: those with more than one
+// consumer in the graph, and those a live Tensor handle still refers to (the handle may feed a later graph,
+// e.g. the residual stream kept across an attention call) when recomputing them would repeat a GEMM.  Cheap
+// elementwise / row work held by a handle stays fused and is recomputed if it is ever asked for, which is
+// what keeps softmax(...).sum() one kernel when the softmax has a name in user code.
+using SharedSet = std::unordered_set<const GraphNode *>;
+SharedSet shared_nodes(const GraphNode *root, const std::vector<const GraphNode *> &topo) {
+    std::unordered_map<const GraphNode *, long> holders; // shared_ptr owners: graph edges + Tensor handles
+    std::unordered_map<const GraphNode *, bool> heavy;   // a MatMul at or below the node, above the leaves
+    SharedSet out;
+    for (const GraphNode *n : topo) { // inputs precede their consumers
+        if (is_leaf(n, root)) continue;
+        bool h = n->op_type == OpType::MatMul;
+        for (const auto &in : n->inputs) {
+            holders[in.get()] = in.use_count();
+            auto it = heavy.find(in.get());
+            h = h || (it != heavy.end() && it->second);
+        }
+        heavy[n] = h;
+    }
+    for (const GraphNode *n : topo) {
+        if (is_leaf(n, root) || n == root) continue;
+        const long refs = static_cast<long>(n->ref_count.load());
+        if (refs > 1 || (heavy[n] && holders[n] > refs)) out.insert(n);
+    }
+    return out;
+}
+
 // ------------------------------------------------------------------ builder
 class PlanBuilder {
   public:
-    PlanBuilder(const GraphNode *root, const std::vector<const GraphNode *> &topo) : root_(root) {
+    PlanBuilder(const GraphNode *root, const std::vector<const GraphNode *> &topo, const SharedSet &shared) : root_(root), shared_(shared) {
         for (size_t i = 0; i < topo.size(); ++i) {
             topo_index_[topo[i]] = static_cast<int>(i);
             if (is_leaf(topo[i], root)) {
@@ -208,7 +237,7 @@ class PlanBuilder {
     }
 
     bool consumable(const GraphNode *c, const GraphNode *entry) const {
-        return !is_leaf(c, root_) && (c == entry || c->ref_count.load() <= 1) && !memo_.count(c);
+        return !is_leaf(c, root_) && (c == entry || !shared_.count(c)) && !memo_.count(c);
     }
 
     int eval(const GraphNode *n) {
@@ -302,7 +331,7 @@ class PlanBuilder {
             throw RuntimeError::not_implemented(std::string("GPU lazy graph node '") + ops::op_name(op) + "'");
         }
         memo_[n] = v;
-        if (n == root_ || n->ref_count.load() > 1) plan_.node_results.emplace_back(topo_index_.at(n), v);
+        if (n == root_ || shared_.count(n)) plan_.node_results.emplace_back(topo_index_.at(n), v);
         return v;
     }
 
@@ -342,8 +371,10 @@ class PlanBuilder {
         while (stripped.size() > 1 && stripped.front() == 1) stripped.erase(stripped.begin());
         bool colvec = S.size() == F.size() && !S.empty() && S.back() == 1 && F.back() != 1;
         for (size_t i = 0; colvec && i + 1 < S.size(); ++i) colvec = S[i] == F[i];
+        Shape f_stripped = F;
+        while (f_stripped.size() > 1 && f_stripped.front() == 1) f_stripped.erase(f_stripped.begin());
         if (numel == 1) kind = AXHIP_BK_SCALAR;
-        else if (S == F) kind = AXHIP_BK_FULL;
+        else if (S == F || stripped == f_stripped) kind = AXHIP_BK_FULL; // leading unit dimensions change nothing in memory
         else if (stripped.size() == 1 && stripped[0] == cols) kind = AXHIP_BK_ROWVEC;
         else if (colvec) kind = AXHIP_BK_COLVEC;
         else {
@@ -559,6 +590,7 @@ class PlanBuilder {
     }
 
     const GraphNode *root_;
+    const SharedSet &shared_;
     Plan plan_;
     std::unordered_map<const GraphNode *, int> memo_;
     std::unordered_map<const GraphNode *, int> topo_index_;
@@ -584,7 +616,7 @@ uint64_t mix_u64(uint64_t h, uint64_t v) {
 
 // The structural signature plus what else decides the plan: which interior nodes are
 // shared (they are materialised on their own) and the layout of materialised leaves.
-uint64_t plan_key(const GraphNode *root, const std::vector<const GraphNode *> &topo) {
+uint64_t plan_key(const GraphNode *root, const std::vector<const GraphNode *> &topo, const SharedSet &shared) {
     uint64_t h = compute_signature(root).hash;
     for (const GraphNode *n : topo) {
         if (is_leaf(n, root)) {
@@ -594,7 +626,7 @@ uint64_t plan_key(const GraphNode *root, const std::vector<const GraphNode *> &t
                 for (int64_t s : n->cached_strides_) h = mix_u64(h, static_cast<uint64_t>(s));
             }
         } else {
-            h = mix_u64(h, n->ref_count.load() > 1 ? 2 : 1);
+            h = mix_u64(h, shared.count(n) ? 2 : 1);
         }
     }
     return h;
@@ -632,7 +664,8 @@ void materialize_gpu_graph(GraphNode *root) {
     const auto topo = topo_sort(root);
 
     // ---- plan: cached by signature
-    const uint64_t key = plan_key(root, topo);
+    const SharedSet shared = shared_nodes(root, topo);
+    const uint64_t key = plan_key(root, topo, shared);
     std::shared_ptr<const Plan> plan;
     {
         auto &c = cache();
@@ -646,7 +679,7 @@ void materialize_gpu_graph(GraphNode *root) {
         }
     }
     if (!plan) {
-        plan = std::make_shared<const Plan>(PlanBuilder(root, topo).build());
+        plan = std::make_shared<const Plan>(PlanBuilder(root, topo, shared).build());
         auto &c = cache();
         std::lock_guard<std::mutex> lk(c.mu);
         if (c.plans.size() >= GraphCache::max_entries) c.plans.clear(); // src/backends/metal/mpsgraph_graph_compiler.mm:899-900
