@@ -1,14 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the gfx950 backend on BASELINE.json's headline workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sdpa|chains]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sdpa|chains|gemm]
 
 A step is one pass of the hot path over one batch of synthetic input already
 resident in HBM: causal bf16 scaled-dot-product attention, B=4 H=32 S=4096
 D=128 (BASELINE.json configs[3], the configuration the metric is quoted on).
 Prints ONE JSON line.  `value` is TFLOP/s over the algorithmic FLOP count
 4*B*H*S^2*D/2.  The same line carries the roofline of the SDPA kernel, the
-fused-chain kernels' achieved HBM bandwidth (configs[1] and configs[2]) and a
+fused-chain kernels' achieved HBM bandwidth (configs[1] and configs[2]), the
+MFMA GEMM behind nn::Linear, the timings of the C++ host layer and a
 CPU baseline (the oracle's restatement of Axiom's CPU algorithm, timed on this
 host on a bounded sample).
 
@@ -180,6 +181,32 @@ def bench_chains(torch, capi, stream, steps, warmup):
     return res
 
 
+def bench_gemm(torch, capi, stream, steps, warmup):
+    """x W^T through axhip_gemm (the nn::Linear product): a large square, the tall product of a
+    long batch, and the Whisper-block projection of BASELINE.json configs[4]."""
+    lib = capi.lib()
+    sp = C.c_void_p(stream.cuda_stream)
+    res = {}
+    g = torch.Generator(device="cuda").manual_seed(42)
+    for M, N, K in ((4096, 4096, 4096), (8192, 4096, 4096), (1500, 1280, 1280)):
+        a = torch.randn((M, K), generator=g, device="cuda").to(torch.bfloat16)
+        w = (torch.randn((N, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+        c = torch.empty((M, N), device="cuda", dtype=torch.bfloat16)
+        p = capi.GemmParams()
+        p.dtype, p.trans_a, p.trans_b = capi.DTYPE_BF16, 0, 1
+        p.m, p.n, p.k = M, N, K
+        p.lda, p.ldb, p.ldc, p.batch = K, K, N, 1
+        args = (a.data_ptr(), w.data_ptr(), c.data_ptr(), C.byref(p), sp)
+        torch.cuda.synchronize()
+        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps, warmup)
+        flops = 2.0 * M * N * K
+        res[f"gemm_nt_bf16_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
+                                             "frac_of_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                             "finite": bool(torch.isfinite(c.float()).all().item())}
+        del a, w, c
+    return res
+
+
 def cpu_baseline(seconds_budget: float = 20.0):
     """Axiom's CPU flash attention (oracle restatement, native BLAS tier) on a bounded
     sample of the same workload: `n` (batch, head) slices of the bf16 S=4096 D=128 causal
@@ -235,7 +262,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["sdpa", "chains"], default=None)
+    ap.add_argument("--only", choices=["sdpa", "chains", "gemm"], default=None)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (both hot paths shard without communication; "
@@ -253,8 +280,9 @@ def main() -> int:
     stream = torch.cuda.Stream()
 
     t_wall0 = time.time()
-    sd = bench_sdpa(torch, capi, stream, args.steps, args.warmup) if args.only != "chains" else None
-    ch = bench_chains(torch, capi, stream, args.steps, args.warmup) if args.only != "sdpa" else None
+    sd = bench_sdpa(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "sdpa") else None
+    ch = bench_chains(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "chains") else None
+    gm = bench_gemm(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "gemm") else None
     cpu = None if (args.no_cpu or sd is None) else cpu_baseline()
 
     line = {
@@ -280,6 +308,8 @@ def main() -> int:
             if name in CHAIN_TRAFFIC_BYTES:
                 rec["traffic"] = CHAIN_TRAFFIC_BYTES[name]
         line["fused_chains"] = ch
+    if gm:
+        line["gemm"] = gm
     if args.only is None:
         line["host_layer"] = host_layer_bench()
     if cpu:
