@@ -200,9 +200,14 @@ def bench_gemm(torch, capi, stream, steps, warmup):
         torch.cuda.synchronize()
         avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps, warmup)
         flops = 2.0 * M * N * K
+        # the vendor library on the same operands (torch.matmul -> hipBLASLt), for context only
+        with torch.cuda.stream(stream):
+            wt = w.t()
+            lib_ms, _, _ = time_launches(torch, stream, lambda: torch.matmul(a, wt), steps, warmup)
         res[f"gemm_nt_bf16_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
                                              "frac_of_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-                                             "finite": bool(torch.isfinite(c.float()).all().item())}
+                                             "finite": bool(torch.isfinite(c.float()).all().item()),
+                                             "hipblaslt_avg_ms": lib_ms}
         del a, w, c
     return res
 
