@@ -37,6 +37,18 @@ template <int IT, int E>
 __device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsProgram &P, float (&v)[IT][E],
                                          int64_t row, const int64_t (&col0)[IT], const bool (&ok)[IT]) {
     if (!is_binary_op(c.op)) {
+        // results that are rounded to a 16-bit type do not need erff / expf / IEEE division: the polynomial
+        // GELU (|error| <= 5e-5) and fast-exponential forms are far below the output resolution and keep
+        // these chains on the memory roofline
+        if (P.output_dtype != AXHIP_DTYPE_F32) {
+            switch (c.op) {
+            case AXHIP_OP_GELU: for_each_value<IT, E>(v, [](float a, int, int) { return gelu_fast(a); }); return;
+            case AXHIP_OP_SILU: for_each_value<IT, E>(v, [](float a, int, int) { return a * __frcp_rn(1.0f + __expf(-a)); }); return;
+            case AXHIP_OP_SIGMOID: for_each_value<IT, E>(v, [](float a, int, int) { return __frcp_rn(1.0f + __expf(-a)); }); return;
+            case AXHIP_OP_TANH: for_each_value<IT, E>(v, [](float a, int, int) { return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * a)); }); return;
+            default: break;
+            }
+        }
         apply_unary_tile<IT, E>(c.op, v);
         return;
     }
