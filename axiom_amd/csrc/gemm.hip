@@ -10,6 +10,10 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <cstdlib>
+#include <mutex>
+#include <set>
+#include <type_traits>
 
 namespace axhip {
 
@@ -398,9 +402,142 @@ __global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs
     gemm_store_tiles<BF16, 4, 2>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
 }
 
+// --------------------------------------------------- MFMA NT, multi-stage ring
+// Mid-size products (too few 256 x 256 tiles to fill the chip): work-group tile TM x TN x 64,
+// 4 waves in a 2 x 2 layout, and an S-stage ring of k-tiles in LDS filled by buffer_load ... lds.
+// One work-group per CU cannot hide the L2 latency (about 1 us under load) behind a k-tile's
+// 0.15 - 0.3 us of MFMA work by occupancy, so S - 1 k-tiles are kept in flight instead and the
+// wait before a k-tile is a counted vmcnt that only covers the oldest one.  The k loop is unrolled
+// by S so that every stage address is an immediate.  Same LDS row layout and XOR swizzle, same
+// tile order over the XCDs and same epilogue as the 256 x 256 kernel.
+// Requires K % 64 == 0 and max(TM, TN) * max(lda, ldb) * 2 < 2^31 (checked by the launcher).
+template <bool BF16, int TM, int TNR, int S>
+__global__ __launch_bounds__(256, 1) void gemm_mfma_nt_ring_kernel(const GemmArgs g, const int tiles_m, const int tiles_n) {
+    constexpr int MI = TM / 64, NJ = TNR / 64;       // 32x32 MFMA tiles per wave
+    constexpr int NLA = TM / 32, NLB = TNR / 32;      // wave-wide loads (8 rows each) per wave per k-tile
+    constexpr int STAGEB = (TM + TNR) * BIG_ROWB;     // bytes per ring stage: A rows, then B rows
+    extern __shared__ __attribute__((aligned(1024))) unsigned char big_lds[];
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+    const int l32 = lane % 32, g2 = lane / 32;
+
+    const int per_xcd = gridDim.x / 8;
+    const int t = (static_cast<int>(blockIdx.x) % 8) * per_xcd + static_cast<int>(blockIdx.x) / 8;
+    if (t >= tiles_m * tiles_n) return;
+    constexpr int GR = 4;
+    const int group = t / (GR * tiles_n), first_m = group * GR;
+    const int gsz = min(GR, tiles_m - first_m);
+    const int rem = t - group * GR * tiles_n;
+    const int tm = first_m + rem % gsz, tn = rem / gsz;
+    const int64_t m0 = static_cast<int64_t>(tm) * TM, n0 = static_cast<int64_t>(tn) * TNR;
+    const int64_t bz = blockIdx.y;
+    const uint16_t *A = static_cast<const uint16_t *>(g.a) + bz * g.sa + m0 * g.a_rs;
+    const uint16_t *B = static_cast<const uint16_t *>(g.b) + bz * g.sb + n0 * g.b_cs;
+    const int arow_bytes = static_cast<int>(g.a_rs) * 2, brow_bytes = static_cast<int>(g.b_cs) * 2;
+    const int rows_a = static_cast<int>(min<int64_t>(TM, g.M - m0)), rows_b = static_cast<int>(min<int64_t>(TNR, g.N - n0));
+    const int4_t arsrc = gemm_rsrc(A, (rows_a - 1) * arow_bytes + static_cast<int>(g.K) * 2);
+    const int4_t brsrc = gemm_rsrc(B, (rows_b - 1) * brow_bytes + static_cast<int>(g.K) * 2);
+
+    // load n of wave w covers tile rows 32 n + 8 w + (lane >> 3)
+    const int ld_r = 8 * wave + (lane >> 3);
+    const int ld_c = (lane & 7) ^ ((ld_r >> 1) & 7);
+    int a_voff[NLA], b_voff[NLB];
+#pragma unroll
+    for (int n = 0; n < NLA; ++n) a_voff[n] = (32 * n + ld_r) * arow_bytes + ld_c * 16;
+#pragma unroll
+    for (int n = 0; n < NLB; ++n) b_voff[n] = (32 * n + ld_r) * brow_bytes + ld_c * 16;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(big_lds));
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 8 * wave * BIG_ROWB);
+    auto load_tile = [&](int kt, int stage) {
+        const int soff = kt * BIG_ROWB;
+#pragma unroll
+        for (int n = 0; n < NLA; ++n) gemm_load_to_lds(arsrc, lds_wave + stage * STAGEB + n * 32 * BIG_ROWB, a_voff[n], soff);
+#pragma unroll
+        for (int n = 0; n < NLB; ++n) gemm_load_to_lds(brsrc, lds_wave + stage * STAGEB + TM * BIG_ROWB + n * 32 * BIG_ROWB, b_voff[n], soff);
+    };
+
+    const int wm = (wave / 2) * (TM / 2), wn = (wave % 2) * (TNR / 2);
+    int f_off[TK / 16];
+#pragma unroll
+    for (int ks = 0; ks < TK / 16; ++ks) f_off[ks] = l32 * BIG_ROWB + (((2 * ks + g2) ^ ((l32 >> 1) & 7)) * 16);
+
+    float16_t acc[MI][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    uint4_t fa[2][MI], fb[2][NJ];
+    auto read_frags = [&](int slot, int stage, int ks) {
+        const unsigned char *As = big_lds + stage * STAGEB + wm * BIG_ROWB;
+        const unsigned char *Bs = big_lds + stage * STAGEB + (TM + wn) * BIG_ROWB;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) fb[slot][j] = *reinterpret_cast<const uint4_t *>(Bs + 32 * j * BIG_ROWB + f_off[ks]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[slot][i] = *reinterpret_cast<const uint4_t *>(As + 32 * i * BIG_ROWB + f_off[ks]);
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                if constexpr (BF16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[slot][i]), __builtin_bit_cast(bf16x8_t, fb[slot][j]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fa[slot][i]), __builtin_bit_cast(half8_t, fb[slot][j]), acc[i][j], 0, 0, 0);
+            }
+    };
+
+    const int nk = static_cast<int>(g.K / TK);
+    // s_waitcnt vmcnt(N) with the other counters left alone: N = loads of the S - 2 k-tiles that may still be in flight
+    constexpr int INFLIGHT = (NLA + NLB) * (S - 2);
+    static_assert(INFLIGHT < 64, "vmcnt is a 6-bit counter");
+    constexpr int WAIT_OLDEST = (INFLIGHT & 0xF) | 0x0F70 | ((INFLIGHT >> 4) << 14);
+#pragma unroll
+    for (int st = 0; st < S - 1; ++st)
+        if (st < nk) load_tile(st, st);
+
+    // k-tile kt lives in ring stage ST (= kt % S, a compile-time value in the unrolled loop)
+    auto step = [&](auto stage_tag, int kt) {
+        constexpr int ST = decltype(stage_tag)::value;
+        if (kt + S - 2 < nk) __builtin_amdgcn_s_waitcnt(WAIT_OLDEST); // everything older than the S - 2 newest k-tiles has landed
+        else __builtin_amdgcn_s_waitcnt(0x0F70);                      // tail: fewer loads behind this one, wait for all
+        __syncthreads(); // k-tile kt is complete for every wave, and k-tile kt - 1 (whose stage is refilled next) is no longer read
+        if (kt + S - 1 < nk) load_tile(kt + S - 1, (ST + S - 1) % S);
+        read_frags(0, ST, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < TK / 16; ++ks) {
+            if (ks + 1 < TK / 16) read_frags((ks + 1) & 1, ST, ks + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(ks & 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto steps = [&](auto self, auto stage_tag, int kt0) -> void { // step<0>(kt0), step<1>(kt0 + 1), ... step<S-1>
+        constexpr int ST = decltype(stage_tag)::value;
+        if constexpr (ST < S) {
+            if (kt0 + ST < nk) {
+                step(stage_tag, kt0 + ST);
+                self(self, std::integral_constant<int, ST + 1>{}, kt0);
+            }
+        }
+    };
+    for (int kt0 = 0; kt0 < nk; kt0 += S) steps(steps, std::integral_constant<int, 0>{}, kt0);
+
+    gemm_store_tiles<BF16, MI, NJ>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
+}
+
 } // namespace axhip
 
 using namespace axhip;
+
+// AXHIP_GEMM_RING=0 routes mid-size products to the register-staged kernels (for A/B timing)
+static bool ring_enabled() {
+    static const bool on = [] { const char *e = std::getenv("AXHIP_GEMM_RING"); return !(e && e[0] == '0'); }();
+    return on;
+}
 
 extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemmParams *params, void *stream) {
     AXHIP_REQUIRE(params != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_gemm: params is NULL");
@@ -445,6 +582,33 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
         AXHIP_REQUIRE(configured, AXHIP_ERR_UNSUPPORTED, "axhip_gemm: cannot reserve %zu bytes of LDS", lds_bytes);
         if (p.dtype == AXHIP_DTYPE_BF16) hipLaunchKernelGGL((gemm_mfma_nt_256_kernel<true>), grid, dim3(512), lds_bytes, s, g, tiles_m, tiles_n);
         else hipLaunchKernelGGL((gemm_mfma_nt_256_kernel<false>), grid, dim3(512), lds_bytes, s, g, tiles_m, tiles_n);
+    } else if (half && nt && p.k > 0 && p.k % TK == 0 && p.k >= 4 * TK && p.lda < (1 << 22) && p.ldb < (1 << 22) && p.batch < 65536 &&
+               ring_enabled()) {
+        // mid-size: the ring kernels
+        const bool bf = p.dtype == AXHIP_DTYPE_BF16;
+        auto launch = [&](auto kernel, int tm_rows, int tn_cols, size_t lds_bytes) -> int {
+            static std::mutex mu;
+            static std::set<const void *> configured;
+            {
+                std::lock_guard<std::mutex> lk(mu);
+                if (!configured.count(reinterpret_cast<const void *>(kernel))) {
+                    AXHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+                    configured.insert(reinterpret_cast<const void *>(kernel));
+                }
+            }
+            const int tiles_m = static_cast<int>((p.m + tm_rows - 1) / tm_rows), tiles_n = static_cast<int>((p.n + tn_cols - 1) / tn_cols);
+            const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+            hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(8 * per_xcd), static_cast<unsigned>(p.batch)), dim3(256), lds_bytes, s, g, tiles_m, tiles_n);
+            return AXHIP_OK;
+        };
+        // 128 x 128 tiles (4 stages) once they give most CUs a work-group, else 64 x 128 tiles (6 stages).  (256 x 128
+        // tiles with 3 stages measured the same as 128 x 128: what bounds these shapes is the bytes in flight per
+        // CU, i.e. the LDS ring itself, against the latency of the first touch of every k-tile.)
+        const int64_t t128 = ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch;
+        int rc2;
+        if (t128 >= 192) rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 128, 128, 4>, 128, 128, 4 * 256 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 128, 128, 4>, 128, 128, 4 * 256 * BIG_ROWB);
+        else rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 64, 128, 6>, 64, 128, 6 * 192 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 64, 128, 6>, 64, 128, 6 * 192 * BIG_ROWB);
+        if (rc2) return rc2;
     } else if (half && nt && p.k > 0) {
         // Tall tiles (two work-groups per CU, one k-tile in flight) once they fill the chip;
         // otherwise 64-row tiles, one work-group per CU with three k-tiles in flight.

@@ -73,3 +73,23 @@ def test_half_large_tile_path_matches_fp64(dt, M, N, K, extras):
     if not extras and K <= 64:
         o = axo.to_f32(axo.matmul(x[:64], W[:64], dt, False, True), dt)
         assert np.max(np.abs(o - got[:64, :64])) < 0.25
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,extras", [(1500, 5120, 1280, False), (1500, 1280, 5120, True), (200, 330, 256, True), (129, 257, 320, False),
+                                          (1000, 2000, 448, True), (64, 128, 4096, False)])
+def test_half_ring_path_matches_fp64(dt, M, N, K, extras):
+    """Mid-size products: the multi-stage LDS ring kernels (128 x 128 and 64 x 128 tiles), with k extents of
+    exactly, fewer and more k-tiles than the ring has stages, ragged tiles, and the full epilogue."""
+    g = axo.PCG64(M * 7 + K)
+    x, W = axo.to_bits(g.normal((M, K)), dt), axo.to_bits(g.normal((N, K)) * (2.0 / np.sqrt(K)), dt)
+    bias = axo.to_bits(g.normal((N,)) * 0.1, dt) if extras else None
+    res = axo.to_bits(g.normal((M, N)), dt) if extras else None
+    got = axo.to_f32(gh.gemm(x, W, dt, trans_b=True, bias=bias, residual=res, epilogue="gelu" if extras else None)[0], dt)
+    want = axo.to_f32(x, dt).astype(np.float64) @ axo.to_f32(W, dt).astype(np.float64).T
+    if extras:
+        import math
+
+        y = want + axo.to_f32(bias, dt) + axo.to_f32(res, dt)
+        want = 0.5 * y * (1 + np.vectorize(math.erf)(y / math.sqrt(2)))
+    assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
