@@ -44,6 +44,8 @@ class Linear : public Module {
     explicit Linear(bool bias = true);
     Tensor forward(const Tensor &input) const override;
     bool has_bias() const { return has_bias_; }
+    const Tensor &weight() const { return weight_; }
+    const Tensor &bias() const { return bias_; }
 
   private:
     Tensor weight_, bias_;
@@ -139,10 +141,20 @@ class MultiHeadAttention : public Module {
     explicit MultiHeadAttention(int num_heads, bool bias = true);
     Tensor forward(const Tensor &query, const Tensor &key, const Tensor &value, const Tensor &mask = Tensor(), bool is_causal = false) const;
     int num_heads() const { return num_heads_; }
+    // anything that replaces the parameters drops the stacked projection weight
+    void load_state_dict(const std::map<std::string, Tensor> &state_dict, const std::string &prefix = "", bool strict = true) override;
+    Module &to(Device device) override;
+    Module &to(DType dtype) override;
 
   private:
+    // self-attention on the GPU runs the three input projections as ONE product against the stacked
+    // (3 d_model, d_model) weight; the stack is built on first use and rebuilt when a projection's weight changes
+    bool fused_qkv(const Tensor &x, Tensor &q, Tensor &k, Tensor &v) const;
+
     int num_heads_;
     Linear q_proj_, k_proj_, v_proj_, out_proj_;
+    mutable Tensor qkv_weight_, qkv_bias_;
+    mutable const void *qkv_sources_[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 };
 
 } // namespace axiom::nn

@@ -1,8 +1,11 @@
 // nn modules on the attention / norm path (behaviour of src/nn/{module,linear,
 // normalization,attention,activation}.cpp).
+#include <cstring>
+
 #include "axiom/nn.hpp"
 
 #include "axiom/operations.hpp"
+#include "hip_call.hpp"
 
 namespace axiom::nn {
 
@@ -133,12 +136,74 @@ Tensor MultiHeadAttention::forward(const Tensor &query, const Tensor &key, const
     const size_t H = static_cast<size_t>(num_heads_);
     if (Dm % H != 0) throw ShapeError("MultiHeadAttention: d_model " + std::to_string(Dm) + " is not divisible by " + std::to_string(H) + " heads");
     const size_t Dh = Dm / H;
-    Tensor q = q_proj_.forward(query).reshape({B, Sq, H, Dh}).transpose({0, 2, 1, 3});
-    Tensor k = k_proj_.forward(key).reshape({B, Skv, H, Dh}).transpose({0, 2, 1, 3});
-    Tensor v = v_proj_.forward(value).reshape({B, Skv, H, Dh}).transpose({0, 2, 1, 3});
+    Tensor q, k, v;
+    if (!(&query == &key && &key == &value && fused_qkv(query, q, k, v))) {
+        q = q_proj_.forward(query).reshape({B, Sq, H, Dh}).transpose({0, 2, 1, 3});
+        k = k_proj_.forward(key).reshape({B, Skv, H, Dh}).transpose({0, 2, 1, 3});
+        v = v_proj_.forward(value).reshape({B, Skv, H, Dh}).transpose({0, 2, 1, 3});
+    }
     Tensor attn = ops::detail::sdpa(q, k, v, mask, -1.0f, is_causal, /*out_bshd=*/true);
     Tensor merged = attn.transpose({0, 2, 1, 3}).reshape({B, Sq, Dm});
     return out_proj_.forward(merged);
+}
+
+void MultiHeadAttention::load_state_dict(const std::map<std::string, Tensor> &sd, const std::string &prefix, bool strict) {
+    qkv_weight_ = qkv_bias_ = Tensor();
+    Module::load_state_dict(sd, prefix, strict);
+}
+Module &MultiHeadAttention::to(Device device) {
+    qkv_weight_ = qkv_bias_ = Tensor();
+    return Module::to(device);
+}
+Module &MultiHeadAttention::to(DType dtype) {
+    qkv_weight_ = qkv_bias_ = Tensor();
+    return Module::to(dtype);
+}
+
+// q, k, v of self-attention as (B, H, S, Dh) views of one (B, S, 3 d_model) product.  False when the
+// projections are not three same-typed contiguous GPU matrices (the caller then projects one by one).
+bool MultiHeadAttention::fused_qkv(const Tensor &x, Tensor &q, Tensor &k, Tensor &v) const {
+    const Linear *proj[3] = {&q_proj_, &k_proj_, &v_proj_};
+    if (x.device() != Device::GPU) return false;
+    const DType dt = x.dtype();
+    const size_t B = x.shape()[0], S = x.shape()[1], Dm = x.shape()[2], H = static_cast<size_t>(num_heads_), Dh = Dm / H;
+    bool any_bias = false;
+    const void *sources[6];
+    for (int i = 0; i < 3; ++i) {
+        const Tensor &w = proj[i]->weight(), &b = proj[i]->bias();
+        if (w.empty() || w.is_lazy() || w.device() != Device::GPU || w.dtype() != dt || !w.is_contiguous() || w.ndim() != 2 || w.shape()[0] != Dm || w.shape()[1] != Dm)
+            return false;
+        const bool has_b = proj[i]->has_bias() && !b.empty();
+        if (has_b && (b.is_lazy() || b.device() != Device::GPU || b.dtype() != dt || !b.is_contiguous() || b.size() != Dm)) return false;
+        any_bias = any_bias || has_b;
+        sources[2 * i] = static_cast<const char *>(w.storage()->raw()) + w.offset();
+        sources[2 * i + 1] = has_b ? static_cast<const char *>(b.storage()->raw()) + b.offset() : nullptr;
+    }
+    if (qkv_weight_.empty() || qkv_weight_.dtype() != dt || std::memcmp(sources, qkv_sources_, sizeof(sources)) != 0) {
+        const size_t isz = dtype_size(dt);
+        Tensor w3(Shape{3 * Dm, Dm}, dt, Device::GPU), b3;
+        if (any_bias) b3 = Tensor(Shape{3 * Dm}, dt, Device::GPU);
+        for (int i = 0; i < 3; ++i) {
+            AXHIP_CALL(axhip_memcpy_d2d_async(static_cast<char *>(w3.storage()->raw()) + i * Dm * Dm * isz, sources[2 * i], Dm * Dm * isz, nullptr));
+            if (!any_bias) continue;
+            char *dst = static_cast<char *>(b3.storage()->raw()) + i * Dm * isz;
+            if (sources[2 * i + 1]) AXHIP_CALL(axhip_memcpy_d2d_async(dst, sources[2 * i + 1], Dm * isz, nullptr));
+            else AXHIP_CALL(axhip_fill(dst, detail::to_axhip_dtype(dt), 0.0, static_cast<int64_t>(Dm), nullptr));
+        }
+        qkv_weight_ = w3;
+        qkv_bias_ = b3;
+        std::memcpy(qkv_sources_, sources, sizeof(sources));
+    }
+    Tensor qkv = ops::matmul(x, qkv_weight_, false, true);
+    if (!qkv_bias_.empty()) qkv = ops::add(qkv, qkv_bias_);
+    const auto st = qkv.storage(); // materialises: the attention kernel needs the memory anyway
+    const int64_t e = static_cast<int64_t>(dtype_size(dt));
+    const Strides strides{static_cast<int64_t>(S * 3 * Dm) * e, static_cast<int64_t>(Dh) * e, static_cast<int64_t>(3 * Dm) * e, e};
+    const Shape shape{B, H, S, Dh};
+    q = Tensor(st, shape, strides, dt, qkv.offset());
+    k = Tensor(st, shape, strides, dt, qkv.offset() + Dm * static_cast<size_t>(e));
+    v = Tensor(st, shape, strides, dt, qkv.offset() + 2 * Dm * static_cast<size_t>(e));
+    return true;
 }
 
 } // namespace axiom::nn

@@ -842,3 +842,28 @@ GPU_TEST(LazyNodes, TransposeRewritesKeepFusion) {
         for (size_t c = 0; c < 32; ++c)
             for (size_t b2 = 0; b2 < 16; ++b2) EXPECT_NEAR(z[(a * 32 + c) * 16 + b2], std::max(0.0f, xf[(a * 16 + b2) * 32 + c]), 0);
 }
+
+// Self-attention stacks the three input projections into one product; passing the same values as
+// three distinct tensor objects takes the projection-by-projection path.  Both must agree, before
+// and after the parameters are replaced (the stacked weight is rebuilt), with and without biases.
+GPU_TEST(FlashAttentionMHA, FusedQkvProjectionMatchesSeparateProjections) {
+    const size_t B = 2, S = 70, Dm = 64;
+    auto x = axtest::randn({B, S, Dm}, 300).gpu();
+    for (bool with_bias : {true, false}) {
+        nn::MultiHeadAttention mha(4, with_bias);
+        for (uint64_t round = 0; round < 2; ++round) {
+            std::map<std::string, Tensor> sd;
+            uint64_t seed = 310 + 20 * round;
+            for (const char *name : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+                sd[std::string(name) + ".weight"] = axtest::randn({Dm, Dm}, seed++, DType::Float32, 0.125f).gpu();
+                if (with_bias && std::string(name) != "k_proj") sd[std::string(name) + ".bias"] = axtest::randn({Dm}, seed++, DType::Float32, 0.1f).gpu(); // no key bias, as in Whisper
+            }
+            mha.load_state_dict(sd, "", /*strict=*/false);
+            const Tensor x2 = x, x3 = x; // same storage, different objects
+            auto fused = host_floats(mha.forward(x, x, x)), separate = host_floats(mha.forward(x, x2, x3));
+            double worst = 0;
+            for (size_t i = 0; i < fused.size(); ++i) worst = std::max(worst, std::fabs(double(fused[i]) - separate[i]));
+            EXPECT_LT(worst, 1e-4);
+        }
+    }
+}
