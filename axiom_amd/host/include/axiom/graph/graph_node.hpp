@@ -49,8 +49,9 @@ struct PadParams {
 struct MaskedFillParams {
     float value = 0.0f;
 };
-struct UnfoldParams { // windows of `kernel` taps along the last dimension
+struct UnfoldParams { // windows of `kernel` taps along the last dimension (and `kernel_h` along the one before it, for 2-D)
     int kernel = 1, stride = 1, dilation = 1;
+    int kernel_h = 1, stride_h = 1, dilation_h = 1;
 };
 
 using OpParams = std::variant<NoParams, ReductionParams, MatMulParams, ActivationParams, ReshapeParams, NormParams, TransposeParams, SliceParams,

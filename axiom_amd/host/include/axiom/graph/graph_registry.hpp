@@ -2,6 +2,8 @@
 // (include/axiom/graph/graph_registry.hpp:23-154).
 #pragma once
 
+#include <array>
+
 #include <memory>
 #include <string>
 #include <vector>
@@ -45,6 +47,8 @@ class GraphRegistry {
     static Tensor create_lazy_batchnorm(const Tensor &input, const Tensor &weight, const Tensor &bias, const Tensor &running_mean,
                                         const Tensor &running_var, float eps);
     static Tensor create_lazy_conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation);
+    static Tensor create_lazy_conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride,
+                                     std::array<int, 2> padding, std::array<int, 2> dilation);
     static Tensor create_lazy_embedding(const Tensor &weight, const Tensor &indices);
 
     // signature -> plan cache -> compile -> execute; GPU graphs go to materialize_gpu_graph

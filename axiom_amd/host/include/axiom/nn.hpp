@@ -2,6 +2,7 @@
 // normalization,attention,activation,conv,embedding,container}.hpp; src/nn/*.cpp).  Inference only.
 #pragma once
 
+#include <array>
 #include <map>
 #include <memory>
 #include <string>
@@ -92,6 +93,20 @@ class Conv1d : public Module {
   private:
     Tensor weight_, bias_;
     int stride_, padding_, dilation_, groups_;
+    bool has_bias_;
+};
+
+// 2-D convolution, weight (C_out, C_in, KH, KW) (include/axiom/nn/conv.hpp:50-75)
+class Conv2d : public Module {
+  public:
+    explicit Conv2d(std::array<int, 2> stride = {1, 1}, std::array<int, 2> padding = {0, 0}, std::array<int, 2> dilation = {1, 1}, int groups = 1,
+                    bool bias = true);
+    Tensor forward(const Tensor &input) const override;
+
+  private:
+    Tensor weight_, bias_;
+    std::array<int, 2> stride_, padding_, dilation_;
+    int groups_;
     bool has_bias_;
 };
 

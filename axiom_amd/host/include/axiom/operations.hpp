@@ -7,6 +7,7 @@
 // carries no CPU compute path.
 #pragma once
 
+#include <array>
 #include <map>
 #include <memory>
 #include <utility>
@@ -50,7 +51,8 @@ enum class OpType {
     _Count,
     // internal to this backend's planner, after Axiom's own values: the (N, L_out, C_in, K) window view a
     // convolution is lowered through
-    Unfold1D
+    Unfold1D,
+    Unfold2D // (N, H_out, W_out, C_in, KH, KW)
 };
 
 const char *op_name(OpType op);
@@ -133,6 +135,11 @@ Tensor embedding(const Tensor &weight, const Tensor &indices);
 // (include/axiom/operations.hpp:594-601).  groups must be 1.
 Tensor conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride = 1, int padding = 0, int dilation = 1, int groups = 1);
 Tensor conv1d(const Tensor &input, const Tensor &weight); // no bias, stride 1, no padding
+// 2-D convolution: input (N, C_in, H, W) or (C_in, H, W), weight (C_out, C_in, KH, KW), output (N, C_out, H_out, W_out)
+// (include/axiom/operations.hpp:603-611).  groups must be 1.
+Tensor conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride = {1, 1}, std::array<int, 2> padding = {0, 0},
+              std::array<int, 2> dilation = {1, 1}, int groups = 1);
+Tensor conv2d(const Tensor &input, const Tensor &weight);
 // inference batch norm over the channel dimension (dim 1) of (N, C) or (N, C, L):
 // (x - running_mean) / sqrt(running_var + eps) * weight + bias
 Tensor batch_norm1d(const Tensor &x, const Tensor &weight, const Tensor &bias, const Tensor &running_mean, const Tensor &running_var, float eps = 1e-5f);

@@ -281,6 +281,15 @@ class PlanBuilder {
             s.shape = n->output_shape;
             s.strides = {is[0], is[2] * up.stride, is[1], is[2] * up.dilation};
             v = add_value(s);
+        } else if (op == OpType::Unfold2D) {
+            // (N, C, H, W) -> windows (N, H_out, W_out, C, KH, KW): element (n, i, j, c, a, b) is input (n, c, i sh + a dh, j sw + b dw)
+            const int in = eval(n->inputs[0].get());
+            const auto &up = get_params<UnfoldParams>(n->params);
+            ValueSpec s = val(in);
+            const Strides is = val(in).strides;
+            s.shape = n->output_shape;
+            s.strides = {is[0], is[2] * up.stride_h, is[3] * up.stride, is[1], is[2] * up.dilation_h, is[3] * up.dilation};
+            v = add_value(s);
         } else if (op == OpType::Pad) {
             const int in = eval(n->inputs[0].get());
             detail::to_axhip_dtype(val(in).dtype);

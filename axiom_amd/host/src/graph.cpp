@@ -132,14 +132,28 @@ Tensor GraphRegistry::create_lazy_unary(ops::OpType op, const Tensor &input, con
     require_gpu(pick_device({&input}), op);
     // f(transpose(x)) == transpose(f(x)) for an elementwise f: apply it below a pending transpose, where it
     // can still fuse into whatever produces x (a GEMM epilogue, a row kernel) instead of forcing a gather
-    if (input.is_lazy() && !input.lazy_node()->is_materialized_ && input.lazy_node()->op_type == ops::OpType::Transpose &&
-        input.lazy_node()->ref_count.load() == 0 && !is_eager_mode_enabled()) {
+    // (the same holds for a pending reshape, which a convolution's result passes through)
+    // `sinking` > 0: this call comes from the rewrite one level up, whose view node is the one consumer allowed
+    static thread_local int sinking = 0;
+    if (input.is_lazy() && !input.lazy_node()->is_materialized_ &&
+        (input.lazy_node()->op_type == ops::OpType::Transpose || input.lazy_node()->op_type == ops::OpType::Reshape) &&
+        input.lazy_node()->ref_count.load() == (sinking > 0 ? 1u : 0u) && !is_eager_mode_enabled()) {
         const auto tn = input.lazy_node();
         const Tensor inner = tn->inputs[0]->is_constant
                                  ? Tensor(tn->inputs[0]->constant_storage, tn->inputs[0]->output_shape, tn->inputs[0]->constant_strides,
                                           tn->inputs[0]->output_dtype, tn->inputs[0]->constant_offset)
                                  : Tensor(tn->inputs[0]);
-        return create_lazy_transpose(create_lazy_unary(op, inner, params), get_params<TransposeParams>(tn->params).axes);
+        ++sinking;
+        Tensor below;
+        try {
+            below = create_lazy_unary(op, inner, params);
+        } catch (...) {
+            --sinking;
+            throw;
+        }
+        --sinking;
+        if (tn->op_type == ops::OpType::Transpose) return create_lazy_transpose(below, get_params<TransposeParams>(tn->params).axes);
+        return create_lazy_reshape(below, get_params<ReshapeParams>(tn->params).new_shape);
     }
     auto n = std::make_shared<GraphNode>();
     n->op_type = op;
@@ -376,6 +390,42 @@ Tensor GraphRegistry::create_lazy_conv1d(const Tensor &input, const Tensor &weig
     return create_lazy_transpose(y, {0, 2, 1});
 }
 
+// The same lowering in two dimensions: windows (N, H_out, W_out, C_in, KH, KW), product with the (C_out, C_in KH KW)
+// filter matrix, result laid out (N, H_out, W_out, C_out) and returned as its (N, C_out, H_out, W_out) view.
+Tensor GraphRegistry::create_lazy_conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride,
+                                         std::array<int, 2> padding, std::array<int, 2> dilation) {
+    require_gpu(pick_device({&input}), ops::OpType::Conv2D);
+    const size_t N = input.shape()[0], Cin = input.shape()[1], Hin = input.shape()[2], Win = input.shape()[3];
+    const size_t Cout = weight.shape()[0], KH = weight.shape()[2], KW = weight.shape()[3];
+    const size_t Hp = Hin + 2 * static_cast<size_t>(padding[0]), Wp = Win + 2 * static_cast<size_t>(padding[1]);
+    const size_t span_h = static_cast<size_t>(dilation[0]) * (KH - 1) + 1, span_w = static_cast<size_t>(dilation[1]) * (KW - 1) + 1;
+    if (Hp < span_h || Wp < span_w) throw ShapeError("conv2d: the kernel does not fit the padded input");
+    const size_t Hout = (Hp - span_h) / static_cast<size_t>(stride[0]) + 1, Wout = (Wp - span_w) / static_cast<size_t>(stride[1]) + 1;
+    Tensor x = on_gpu(input);
+    if (padding[0] > 0 || padding[1] > 0)
+        x = create_lazy_pad(x, {{0, 0}, {0, 0}, {static_cast<size_t>(padding[0]), static_cast<size_t>(padding[0])}, {static_cast<size_t>(padding[1]), static_cast<size_t>(padding[1])}},
+                            0.0, Shape{N, Cin, Hp, Wp});
+    auto un = std::make_shared<GraphNode>();
+    un->op_type = ops::OpType::Unfold2D;
+    un->inputs = {input_node(x)};
+    un->output_shape = Shape{N, Hout, Wout, Cin, KH, KW};
+    un->output_dtype = x.dtype();
+    un->target_device = Device::GPU;
+    UnfoldParams up;
+    up.kernel = static_cast<int>(KW);
+    up.stride = stride[1];
+    up.dilation = dilation[1];
+    up.kernel_h = static_cast<int>(KH);
+    up.stride_h = stride[0];
+    up.dilation_h = dilation[0];
+    un->params = up;
+    const Tensor cols = create_lazy_reshape(finalize_lazy_node(std::move(un)), Shape{N, Hout * Wout, Cin * KH * KW});
+    const Tensor w2 = on_gpu(weight).reshape({Cout, Cin * KH * KW});
+    Tensor y = create_lazy_matmul(cols, w2, false, true);
+    if (!bias.empty()) y = create_lazy_binary(ops::OpType::Add, y, on_gpu(bias));
+    return create_lazy_transpose(create_lazy_reshape(y, Shape{N, Hout, Wout, Cout}), {0, 3, 1, 2});
+}
+
 Tensor GraphRegistry::create_lazy_embedding(const Tensor &weight, const Tensor &indices) {
     require_gpu(pick_device({&weight, &indices}), ops::OpType::Gather);
     auto n = std::make_shared<GraphNode>();
@@ -522,6 +572,9 @@ GraphSignature compute_signature(const GraphNode *root) {
                     h = mix_i32(h, p.kernel);
                     h = mix_i32(h, p.stride);
                     h = mix_i32(h, p.dilation);
+                    h = mix_i32(h, p.kernel_h);
+                    h = mix_i32(h, p.stride_h);
+                    h = mix_i32(h, p.dilation_h);
                 }
             },
             n->params);

@@ -102,6 +102,16 @@ Tensor Conv1d::forward(const Tensor &input) const {
     return ops::conv1d(input, weight_, has_bias_ ? bias_ : Tensor(), stride_, padding_, dilation_, groups_);
 }
 
+Conv2d::Conv2d(std::array<int, 2> stride, std::array<int, 2> padding, std::array<int, 2> dilation, int groups, bool bias)
+    : stride_(stride), padding_(padding), dilation_(dilation), groups_(groups), has_bias_(bias) {
+    register_parameter("weight", weight_);
+    if (has_bias_) register_parameter("bias", bias_);
+}
+Tensor Conv2d::forward(const Tensor &input) const {
+    if (weight_.empty()) throw RuntimeError("Conv2d: weight not initialized (load_state_dict first)");
+    return ops::conv2d(input, weight_, has_bias_ ? bias_ : Tensor(), stride_, padding_, dilation_, groups_);
+}
+
 Embedding::Embedding() { register_parameter("weight", weight_); }
 Tensor Embedding::forward(const Tensor &indices) const {
     if (weight_.empty()) throw RuntimeError("Embedding: weight not initialized (load_state_dict first)");

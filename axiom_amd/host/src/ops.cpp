@@ -51,6 +51,8 @@ const char *op_name(OpType op) {
     case OpType::Conv1D: return "conv1d";
     case OpType::BatchNorm1D: return "batch_norm1d";
     case OpType::Unfold1D: return "unfold1d";
+    case OpType::Unfold2D: return "unfold2d";
+    case OpType::Conv2D: return "conv2d";
     case OpType::ScaledDotProductAttention: return "scaled_dot_product_attention";
     default: return "op";
     }
@@ -171,6 +173,20 @@ Tensor conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int
 }
 
 Tensor conv1d(const Tensor &input, const Tensor &weight) { return conv1d(input, weight, Tensor(), 1, 0, 1, 1); }
+
+Tensor conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride, std::array<int, 2> padding,
+              std::array<int, 2> dilation, int groups) {
+    if (groups != 1) throw RuntimeError::not_implemented("grouped conv2d on the GPU");
+    for (int i = 0; i < 2; ++i)
+        if (stride[i] < 1 || dilation[i] < 1 || padding[i] < 0) throw ValueError("conv2d: stride and dilation must be positive, padding non-negative");
+    if (input.ndim() == 3) return conv2d(input.unsqueeze(0), weight, bias, stride, padding, dilation, groups).squeeze(0); // unbatched (C_in, H, W)
+    if (input.ndim() != 4 || weight.ndim() != 4) throw ShapeError("conv2d expects input (N, C_in, H, W) and weight (C_out, C_in, KH, KW)");
+    if (input.shape()[1] != weight.shape()[1])
+        throw ShapeError("conv2d: input has " + std::to_string(input.shape()[1]) + " channels, weight expects " + std::to_string(weight.shape()[1]));
+    if (!bias.empty() && (bias.ndim() != 1 || bias.shape()[0] != weight.shape()[0])) throw ShapeError("conv2d: bias must have shape (C_out)");
+    return GraphRegistry::create_lazy_conv2d(input, weight, bias, stride, padding, dilation);
+}
+Tensor conv2d(const Tensor &input, const Tensor &weight) { return conv2d(input, weight, Tensor(), {1, 1}, {0, 0}, {1, 1}, 1); }
 
 Tensor batch_norm1d(const Tensor &x, const Tensor &weight, const Tensor &bias, const Tensor &running_mean, const Tensor &running_var, float eps) {
     return GraphRegistry::create_lazy_batchnorm(x, weight, bias, running_mean, running_var, eps);

@@ -867,3 +867,66 @@ GPU_TEST(FlashAttentionMHA, FusedQkvProjectionMatchesSeparateProjections) {
         }
     }
 }
+
+GPU_TEST(LazyNodes, Conv2dKnownAnswers) { // tests/test_conv2d.cpp:3-111 of the reference
+    auto x9 = gpu_f32({1, 2, 3, 4, 5, 6, 7, 8, 9}, {1, 1, 3, 3});
+    auto w4 = gpu_f32({1, 1, 1, 1}, {1, 1, 2, 2});
+    auto r = ops::conv2d(x9, w4);
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 2, 2}));
+    auto h = host_floats(r);
+    const float want[4] = {12, 16, 24, 28};
+    for (int i = 0; i < 4; ++i) EXPECT_NEAR(h[i], want[i], 0);
+    r = ops::conv2d(x9, Tensor::ones({1, 1, 3, 3}, DType::Float32, Device::GPU), Tensor(), {1, 1}, {1, 1}); // padding 1
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 3, 3}));
+    EXPECT_NEAR(host_floats(r)[4], 45.0f, 0);
+    std::vector<float> d16(16), d25(25);
+    for (int i = 0; i < 16; ++i) d16[i] = float(i + 1);
+    for (int i = 0; i < 25; ++i) d25[i] = float(i + 1);
+    r = ops::conv2d(Tensor::from_data(d16.data(), {1, 1, 4, 4}, Device::GPU), w4, Tensor(), {2, 2}); // stride 2
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 2, 2}));
+    h = host_floats(r);
+    const float want_s[4] = {14, 22, 46, 54};
+    for (int i = 0; i < 4; ++i) EXPECT_NEAR(h[i], want_s[i], 0);
+    r = ops::conv2d(Tensor::from_data(d25.data(), {1, 1, 5, 5}, Device::GPU), w4, Tensor(), {1, 1}, {0, 0}, {2, 2}); // dilation 2
+    EXPECT_TRUE(r.shape() == Shape({1, 1, 3, 3}));
+    EXPECT_NEAR(host_floats(r)[0], 28.0f, 0);
+    EXPECT_NEAR(ops::conv2d(gpu_f32({1, 2, 3, 4}, {1, 1, 2, 2}), w4, gpu_f32({10}, {1})).item<float>(), 20.0f, 0); // bias
+    r = ops::conv2d(gpu_f32({1, 2, 3, 4, 5, 6, 7, 8, 9}, {1, 3, 3}), w4); // unbatched
+    EXPECT_TRUE(r.shape() == Shape({1, 2, 2}));
+    EXPECT_NEAR(host_floats(r)[0], 12.0f, 0);
+    EXPECT_THROW(ops::conv2d(x9, w4, Tensor(), {1, 1}, {0, 0}, {1, 1}, 2), RuntimeError); // groups
+}
+
+GPU_TEST(LazyNodes, Conv2dMatchesFloat64Loops) {
+    struct Case { DType dt; size_t N, C, H, W, Co, KH, KW; int sh, sw, ph, pw, dh, dw; bool relu; double tol; };
+    const Case cases[] = {{DType::Float32, 2, 3, 9, 11, 5, 3, 3, 1, 1, 1, 1, 1, 1, false, 1e-4},
+                          {DType::Float32, 1, 4, 12, 10, 6, 2, 3, 2, 1, 0, 2, 1, 2, true, 1e-4},
+                          {DType::BFloat16, 2, 8, 16, 16, 16, 3, 3, 2, 2, 1, 1, 1, 1, true, 2e-2}};
+    for (const Case &c : cases) {
+        auto x = axtest::randn({c.N, c.C, c.H, c.W}, 400, c.dt), w = axtest::randn({c.Co, c.C, c.KH, c.KW}, 401, c.dt, 0.2f), b = axtest::randn({c.Co}, 402, c.dt, 0.5f);
+        Tensor y = ops::conv2d(x.gpu(), w.gpu(), b.gpu(), {c.sh, c.sw}, {c.ph, c.pw}, {c.dh, c.dw});
+        if (c.relu) y = y.relu();
+        const size_t Ho = (c.H + 2 * c.ph - c.dh * (c.KH - 1) - 1) / c.sh + 1, Wo = (c.W + 2 * c.pw - c.dw * (c.KW - 1) - 1) / c.sw + 1;
+        ASSERT_TRUE(y.shape() == Shape({c.N, c.Co, Ho, Wo}));
+        auto got = host_floats(y);
+        if (c.relu) EXPECT_EQ(graph::last_gpu_plan_kernels().back(), std::string("gemm")); // relu rode in the GEMM epilogue, through the reshape and the transpose
+        auto xf = host_floats(x), wf = host_floats(w), bf = host_floats(b);
+        double worst = 0;
+        for (size_t n = 0; n < c.N; ++n)
+            for (size_t co = 0; co < c.Co; ++co)
+                for (size_t i = 0; i < Ho; ++i)
+                    for (size_t j = 0; j < Wo; ++j) {
+                        double acc = bf[co];
+                        for (size_t ci = 0; ci < c.C; ++ci)
+                            for (size_t a = 0; a < c.KH; ++a)
+                                for (size_t bb = 0; bb < c.KW; ++bb) {
+                                    const long hi = long(i * c.sh + a * c.dh) - c.ph, wi = long(j * c.sw + bb * c.dw) - c.pw;
+                                    if (hi >= 0 && hi < long(c.H) && wi >= 0 && wi < long(c.W))
+                                        acc += double(wf[((co * c.C + ci) * c.KH + a) * c.KW + bb]) * xf[((n * c.C + ci) * c.H + hi) * c.W + wi];
+                                }
+                        if (c.relu) acc = std::max(acc, 0.0);
+                        worst = std::max(worst, std::fabs(acc - got[((n * c.Co + co) * Ho + i) * Wo + j]));
+                    }
+        EXPECT_LT(worst, c.tol);
+    }
+}
