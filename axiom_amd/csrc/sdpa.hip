@@ -325,7 +325,12 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
 
 typedef int int4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ int swizzle_d128(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// XOR applied to the 16-byte chunk index of an LDS row, per buffer and head size.  256-byte rows (D = 128) span all
+// banks, so one function of row & 15 with 16 distinct values serves the K fragment reads (16 consecutive rows, one
+// chunk) and the V transpose reads (4 rows x 64 bytes).  128-byte rows (D = 64) put two rows in one bank sweep: K rows
+// are spread by (row >> 1) & 7, V rows of a 4-row transpose read alternate between the two halves of the row.
+template <int D> __device__ __forceinline__ int swizzle_k(int row) { return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((row >> 1) & 7); }
+template <int D> __device__ __forceinline__ int swizzle_v(int row) { return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : (((row >> 1) & 1) << 2); }
 
 // One 16-byte element per lane from a buffer straight into LDS: lane i's data lands at
 // lds_base + 16*i.  Out-of-range lanes (voffset beyond the descriptor) write zeros.
@@ -341,13 +346,17 @@ __device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
 
 // NW waves per work-group (4: two work-groups share a CU; 8: one work-group per CU, each
 // K/V tile fetched once for 256 query rows instead of 128).
-template <bool BF16, bool HAS_MASK, int NW>
+template <bool BF16, bool HAS_MASK, int NW, int D>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kernel(const SdpaArgs a) {
-    constexpr int D = 128, KT = 8, DT = 4;
+    static_assert(D == 128 || D == 64, "head sizes with a direct-to-LDS pipeline");
+    constexpr int KT = D / 16;            // k-steps of the score product
+    constexpr int DT = D / 32;            // 32-row tiles of O^T
     constexpr int BMW = 32 * NW;          // query rows per work-group
-    constexpr int NLOAD = 16 / NW;        // wave-wide loads per wave per tile (a tile is 16 of them)
-    constexpr int ROWB = 256;            // bytes per LDS row
-    constexpr int TILEB = BN * ROWB;     // 16 KiB per K or V tile
+    constexpr int ROWB = 2 * D;           // bytes per LDS row
+    constexpr int CHUNKS = ROWB / 16;     // 16-byte chunks per row
+    constexpr int RPL = 64 / CHUNKS;      // rows moved by one wave-wide load
+    constexpr int NLOAD = BN / (RPL * NW); // wave-wide loads per wave per tile
+    constexpr int TILEB = BN * ROWB;      // 16 / 8 KiB per K or V tile
     __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILEB]; // K0 K1 V0 V1
 
     const int tid = threadIdx.x;
@@ -385,20 +394,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
     const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + D * 2);
     const int4_t vrsrc = make_rsrc(V, (a.Skv - 1) * vrow_bytes + D * 2);
 
-    // ---- HBM -> LDS mapping.  A wave-wide load moves 4 rows; load n of wave w covers
-    // tile rows 4*NW*n + 4w + (lane >> 4); the lane fetches the chunk that belongs at
-    // position (lane & 15) of the swizzled row (the swizzle only sees row & 15).
-    const int ld_r = 4 * wave + (lane >> 4);
-    const int ld_c = (lane & 15) ^ swizzle_d128(ld_r);
-    const int k_voff = ld_r * krow_bytes + ld_c * 16, v_voff = ld_r * vrow_bytes + ld_c * 16;
+    // ---- HBM -> LDS mapping.  A wave-wide load moves RPL rows; load n of wave w covers
+    // tile rows RPL*NW*n + RPL*w + lane / CHUNKS; the lane fetches the chunk that belongs at
+    // position lane % CHUNKS of the swizzled row (the swizzles only see row & 15).
+    const int ld_r = RPL * wave + lane / CHUNKS;
+    const int k_voff = ld_r * krow_bytes + ((lane % CHUNKS) ^ swizzle_k<D>(ld_r)) * 16;
+    const int v_voff = ld_r * vrow_bytes + ((lane % CHUNKS) ^ swizzle_v<D>(ld_r)) * 16;
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)); // LDS addresses fit 32 bits
-    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 4 * wave * ROWB);
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + RPL * wave * ROWB);
     // load n (0 .. NLOAD-1) of this wave's share of a K / V tile
     auto load_k1 = [&](int tile, int buf, int n) {
-        load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * 4 * NW * ROWB, k_voff + (tile * BN + 4 * NW * n) * krow_bytes);
+        load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * RPL * NW * ROWB, k_voff + (tile * BN + RPL * NW * n) * krow_bytes);
     };
     auto load_v1 = [&](int tile, int buf, int n) {
-        load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * 4 * NW * ROWB, v_voff + (tile * BN + 4 * NW * n) * vrow_bytes);
+        load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * RPL * NW * ROWB, v_voff + (tile * BN + RPL * NW * n) * vrow_bytes);
     };
     auto load_k = [&](int tile, int buf) {
 #pragma unroll
@@ -412,15 +421,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
     // ---- LDS fragment offsets (bytes)
     int k_off[KT]; // K fragment of k-step t: row ql (+32 per sub-tile), chunk 2t+g
 #pragma unroll
-    for (int t = 0; t < KT; ++t) k_off[t] = ql * ROWB + (((2 * t + g) ^ swizzle_d128(ql)) * 16);
+    for (int t = 0; t < KT; ++t) k_off[t] = ql * ROWB + (((2 * t + g) ^ swizzle_k<D>(ql)) * 16);
     int v_off[2][DT]; // V transpose read: rows g*4 + s2 (+8), dims dt*32 + (lane & 31)
     {
         const int s2 = (lane & 15) >> 2, cl = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1), half = lane & 1;
 #pragma unroll
         for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                v_off[hi][dt] = (g * 4 + s2 + 8 * hi) * ROWB + ((((dt ^ s2) << 2) | (cl ^ (g + 2 * hi))) * 16) + half * 8;
+            for (int dt = 0; dt < DT; ++dt) {
+                const int row = g * 4 + s2 + 8 * hi;
+                v_off[hi][dt] = row * ROWB + (((dt * 4 + cl) ^ swizzle_v<D>(row)) * 16) + half * 8;
+            }
     }
 
     for (int pass = 0; pass < npass; ++pass) {
@@ -532,13 +543,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
             }
         };
 
-        // The fused step body, hand-scheduled in 32 slots, one MFMA each:
-        //   slots  0..15  score MFMAs of the NEXT tile (K fragments from Kn)
-        //   slots 16..31  O^T += V^T P^T of the CURRENT tile (V fragments from Vb)
+        // The fused step body, hand-scheduled in NS + NP slots, one MFMA each (D = 128: 16 + 16, D = 64: 8 + 8):
+        //   slots  0..NS-1      score MFMAs of the NEXT tile (K fragments from Kn)
+        //   slots NS..NS+NP-1   O^T += V^T P^T of the CURRENT tile (V fragments from Vb)
         // LDS fragment reads run PF slots ahead of their MFMA.  The VALU work of the current
-        // tile's softmax (fma, exp2, pack, row sum) is dealt out 2 exponentials per slot over
-        // 12 of the first 16 slots and slots 16..19, always ahead of the P fragment that the
-        // PV MFMAs need; the row maximum of the next tile fills slots 20..28.  A scheduling
+        // tile's softmax (exp2, pack, row sum: 16 pairs) is dealt out over the score slots (D = 128: one pair in
+        // 12 of them and in the first four PV slots; D = 64: two pairs in each), always ahead of the P fragment
+        // that the PV MFMAs need; the row maximum of the next tile is spread over PV slots.  A scheduling
         // barrier closes every slot so the compiler keeps this order.
         auto fused = [&](int j, const unsigned char *Kn, const unsigned char *Vb, const float16_t (&cur)[2], float16_t (&nxt)[2], float &mx_next) {
             const bool want_k = j + 2 < ntiles, want_v = j + 1 < ntiles;
@@ -547,11 +558,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
             uint4_t fr[RING];
             uint32_t w[16];
             float pm[4];
+            constexpr int NS = 2 * KT, NP = 4 * DT;
             auto read_frag = [&](int m) {
-                if (m < 16) {
-                    fr[m % RING] = *reinterpret_cast<const uint4_t *>(Kn + (m / 8) * 32 * ROWB + k_off[m % 8]);
+                if (m < NS) {
+                    fr[m % RING] = *reinterpret_cast<const uint4_t *>(Kn + (m / KT) * 32 * ROWB + k_off[m % KT]);
                 } else {
-                    const int ks = (m - 16) / 4, dt = (m - 16) % 4;
+                    const int ks = (m - NS) / DT, dt = (m - NS) % DT;
                     const uint2_t lo = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[0][dt]));
                     const uint2_t hi = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[1][dt]));
                     fr[m % RING] = uint4_t{lo.x, lo.y, hi.x, hi.y};
@@ -567,29 +579,35 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kerne
     #pragma unroll
             for (int m = 0; m < PF; ++m) read_frag(m);
     #pragma unroll
-            for (int m = 0; m < 32; ++m) {
-                if (m + PF < 32) read_frag(m + PF);
-                if (m < 16) {
-                    if (m % 8 == 0) {
+            for (int m = 0; m < NS + NP; ++m) {
+                if (m + PF < NS + NP) read_frag(m + PF);
+                if (m < NS) {
+                    if (m % KT == 0) {
     #pragma unroll
-                        for (int i = 0; i < 16; ++i) nxt[m / 8][i] = -m_use; // logits come out relative to the reference
+                        for (int i = 0; i < 16; ++i) nxt[m / KT][i] = -m_use; // logits come out relative to the reference
                     }
-                    nxt[m / 8] = mfma_32x32x16<BF16>(fr[m % RING], qf[m % 8], nxt[m / 8]);
-                    if (m % 4 != 3) exp_pair((m / 4) * 3 + m % 4);
+                    nxt[m / KT] = mfma_32x32x16<BF16>(fr[m % RING], qf[m % KT], nxt[m / KT]);
+                    if constexpr (D == 128) {
+                        if (m % 4 != 3) exp_pair((m / 4) * 3 + m % 4);
+                    } else {
+                        exp_pair(2 * m);
+                        exp_pair(2 * m + 1);
+                    }
                 } else {
-                    const int ks = (m - 16) / 4, dt = (m - 16) % 4;
+                    const int idx = m - NS, ks = idx / DT, dt = idx % DT;
                     const uint4_t pf = {w[4 * ks], w[4 * ks + 1], w[4 * ks + 2], w[4 * ks + 3]};
                     oacc[dt] = mfma_32x32x16<BF16>(fr[m % RING], pf, oacc[dt]);
-                    if (m < 20) exp_pair(12 + (m - 16));
-                    if (m >= 20 && m < 28) { // two partial maxima per slot over the next tile's 32 scores
-                        const int c = m - 20, kt = c / 4, i0 = (c % 4) * 4;
+                    constexpr int MAX0 = D == 128 ? 4 : 0; // first PV slot that works on the next tile's maximum
+                    if (D == 128 && idx < 4) exp_pair(12 + idx);
+                    if (idx >= MAX0 && idx < MAX0 + 8) { // two partial maxima per slot over the next tile's 32 scores
+                        const int c = idx - MAX0, kt = c / 4, i0 = (c % 4) * 4;
                         if (c % 4 < 2) {
                             pm[kt * 2 + c % 4] = max3(max3(nxt[kt][i0], nxt[kt][i0 + 1], nxt[kt][i0 + 2]), nxt[kt][i0 + 3], NEG_INF_F);
                         } else {
                             pm[kt * 2 + c % 4 - 2] = max3(max3(pm[kt * 2 + c % 4 - 2], nxt[kt][i0], nxt[kt][i0 + 1]), nxt[kt][i0 + 2], nxt[kt][i0 + 3]);
                         }
                     }
-                    if (m == 28) mx_next = max_across_halves(max3(max3(pm[0], pm[1], pm[2]), pm[3], NEG_INF_F));
+                    if (idx == (D == 128 ? MAX0 + 8 : MAX0 + 7)) mx_next = max_across_halves(max3(max3(pm[0], pm[1], pm[2]), pm[3], NEG_INF_F));
                 }
                 // the tile prefetch is spread over the slots instead of bursting at the step start:
                 // K(j+2) in slots 1, 3, .., V(j+1) in slots 2, 4, ..
@@ -817,8 +835,8 @@ extern "C" {
 int axhip_sdpa_d128_occupancy(int waves) {
     int n = -1;
     hipError_t e = waves == 8
-        ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 8>, 512, 0)
-        : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 4>, 256, 0);
+        ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 8, 128>, 512, 0)
+        : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 4, 128>, 256, 0);
     return e == hipSuccess ? n : -static_cast<int>(e);
 }
 
@@ -878,23 +896,32 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
         switch (p.head_dim) {
         case 32: bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
-        case 64: bf ? launch_mfma<true, 64>(a, s) : launch_mfma<false, 64>(a, s); break;
+        case 64:
         default: {
-            // 8-wave work-groups (256 query rows) once there are enough rows to fill them
-            const bool wide = p.seq_q > 128 && sdpa_d128_waves != 4;
+            // 8-wave work-groups (256 query rows, each K/V tile fetched once for all of them) when that still gives
+            // every CU a work-group; 4-wave work-groups (128 rows, two per CU) for shorter or narrower problems
+            const int nqb8 = (p.seq_q + 255) / 256;
+            const int64_t g8 = static_cast<int64_t>(a.causal ? (nqb8 + 1) / 2 : nqb8) * a.B * a.H;
+            const bool wide = p.seq_q > 128 && sdpa_d128_waves != 4 && (g8 >= 256 || sdpa_d128_waves == 8);
             const int bmw = wide ? 256 : 128;
             const int nqbw = (p.seq_q + bmw - 1) / bmw;
             const unsigned g = static_cast<unsigned>(a.causal ? (nqbw + 1) / 2 : nqbw) * static_cast<unsigned>(a.B * a.H);
-#define AXHIP_LAUNCH_D128(BF, MK)                                                                                         \
+#define AXHIP_LAUNCH_DX(BF, MK, DD)                                                                                       \
     do {                                                                                                                  \
-        if (wide) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 8>), dim3(g), dim3(512), 0, s, a);                    \
-        else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 4>), dim3(g), dim3(256), 0, s, a);                         \
+        if (wide) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 8, DD>), dim3(g), dim3(512), 0, s, a);                \
+        else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 4, DD>), dim3(g), dim3(256), 0, s, a);                     \
     } while (0)
-            if (bf && mask) AXHIP_LAUNCH_D128(true, true);
-            else if (bf) AXHIP_LAUNCH_D128(true, false);
-            else if (mask) AXHIP_LAUNCH_D128(false, true);
-            else AXHIP_LAUNCH_D128(false, false);
-#undef AXHIP_LAUNCH_D128
+#define AXHIP_LAUNCH_D(DD)                                                                                                \
+    do {                                                                                                                  \
+        if (bf && mask) AXHIP_LAUNCH_DX(true, true, DD);                                                                  \
+        else if (bf) AXHIP_LAUNCH_DX(true, false, DD);                                                                    \
+        else if (mask) AXHIP_LAUNCH_DX(false, true, DD);                                                                  \
+        else AXHIP_LAUNCH_DX(false, false, DD);                                                                           \
+    } while (0)
+            if (p.head_dim == 64) AXHIP_LAUNCH_D(64);
+            else AXHIP_LAUNCH_D(128);
+#undef AXHIP_LAUNCH_D
+#undef AXHIP_LAUNCH_DX
         }
             break;
         }
