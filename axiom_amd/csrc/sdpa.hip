@@ -312,10 +312,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
     }
 }
 
-// ------------------------------------------------- MFMA kernel, head_dim 128
+// --------------------------------- pipelined MFMA kernel, head_dim 128 and 64
 // Same tiling as sdpa_mfma_kernel, restructured for throughput:
 //  * K and V tiles go HBM -> LDS directly (buffer_load ... lds), no staging
-//    registers and no ds_write; rows sit unpadded (256 B) in LDS with the 16-byte
+//    registers and no ds_write; rows sit unpadded (2 D bytes) in LDS with the 16-byte
 //    chunk index XOR-swizzled by the row, which keeps both the K fragment reads
 //    (16 consecutive rows, one chunk) and the V transpose reads (4 rows x 64 B)
 //    free of bank conflicts.
@@ -347,7 +347,7 @@ __device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
 // NW waves per work-group (4: two work-groups share a CU; 8: one work-group per CU, each
 // K/V tile fetched once for 256 query rows instead of 128).
 template <bool BF16, bool HAS_MASK, int NW, int D>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_d128_kernel(const SdpaArgs a) {
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_kernel(const SdpaArgs a) {
     static_assert(D == 128 || D == 64, "head sizes with a direct-to-LDS pipeline");
     constexpr int KT = D / 16;            // k-steps of the score product
     constexpr int DT = D / 32;            // 32-row tiles of O^T
@@ -835,8 +835,8 @@ extern "C" {
 int axhip_sdpa_d128_occupancy(int waves) {
     int n = -1;
     hipError_t e = waves == 8
-        ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 8, 128>, 512, 0)
-        : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_d128_kernel<true, false, 4, 128>, 256, 0);
+        ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_pipelined_kernel<true, false, 8, 128>, 512, 0)
+        : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, sdpa_mfma_pipelined_kernel<true, false, 4, 128>, 256, 0);
     return e == hipSuccess ? n : -static_cast<int>(e);
 }
 
@@ -908,8 +908,8 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             const unsigned g = static_cast<unsigned>(a.causal ? (nqbw + 1) / 2 : nqbw) * static_cast<unsigned>(a.B * a.H);
 #define AXHIP_LAUNCH_DX(BF, MK, DD)                                                                                       \
     do {                                                                                                                  \
-        if (wide) hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 8, DD>), dim3(g), dim3(512), 0, s, a);                \
-        else hipLaunchKernelGGL((sdpa_mfma_d128_kernel<BF, MK, 4, DD>), dim3(g), dim3(256), 0, s, a);                     \
+        if (wide) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 8, DD>), dim3(g), dim3(512), 0, s, a);                \
+        else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 4, DD>), dim3(g), dim3(256), 0, s, a);                     \
     } while (0)
 #define AXHIP_LAUNCH_D(DD)                                                                                                \
     do {                                                                                                                  \
