@@ -62,6 +62,14 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); // v_cvt_f16_f32: RNE
 }
 
+// two fp32 values to one packed f16 pair (v_cvt_pk_f16_f32: round to nearest even)
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    float2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, half2_t));
+}
+
 // two fp32 values to one packed bf16 pair with the hardware conversion (v_cvt_pk_bf16_f32:
 // round to nearest even; a NaN stays a quiet NaN)
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
@@ -187,7 +195,7 @@ __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const floa
             if (dt == AXHIP_DTYPE_BF16) {
                 w[k] = pack_bf16x2(v[2 * k], v[2 * k + 1]);
             } else {
-                w[k] = f32_to_f16_bits(v[2 * k]) | (f32_to_f16_bits(v[2 * k + 1]) << 16);
+                w[k] = pack_f16x2(v[2 * k], v[2 * k + 1]);
             }
         }
         if constexpr (N % 8 == 0) {

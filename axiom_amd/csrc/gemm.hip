@@ -125,7 +125,7 @@ __device__ __forceinline__ void gemm_store_tiles_as(const GemmArgs &g, const flo
 #pragma unroll
             for (int e = 0; e < 16; e += 2) {
                 const float y0 = gemm_epilogue16(OP, x[e]), y1 = gemm_epilogue16(OP, x[e + 1]);
-                const uint32_t w = BF16 ? pack_bf16x2(y0, y1) : (f32_to_f16_bits(y0) | (f32_to_f16_bits(y1) << 16));
+                const uint32_t w = BF16 ? pack_bf16x2(y0, y1) : pack_f16x2(y0, y1);
                 const int roff = (32 * i + 8 * (e / 4) + e % 4) * ldc2;
                 __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(w & 0xFFFFu), crsrc, FULL_ROWS ? voff : voff + roff, FULL_ROWS ? roff : 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(w >> 16), crsrc, FULL_ROWS ? voff : voff + roff + ldc2, FULL_ROWS ? roff + ldc2 : 0, 0);

@@ -1,17 +1,22 @@
 // Scaled-dot-product attention, forward, for gfx950.
 //
-// Two kernels:
-//   sdpa_mfma_kernel    bf16 / f16, head_dim 32 / 64 / 128.  FlashAttention-2
+// Three kernels:
+//   sdpa_mfma_pipelined_kernel  bf16 / f16, head_dim 64 / 128.  FlashAttention-2
 //                       schedule on v_mfma_f32_32x32x16_{bf16,f16}: one
-//                       workgroup = 4 wave64 = 128 query rows, each wave owns 32
-//                       query rows whose fragments stay in registers; K and V
-//                       tiles of 64 keys are staged through LDS; fp32 online
+//                       workgroup = 4 or 8 wave64, each wave owns 32 query
+//                       rows whose fragments stay in registers; K and V tiles
+//                       of 64 keys go from HBM straight into swizzled LDS
+//                       (buffer_load ... lds) two tiles ahead of their use;
+//                       the softmax of tile j is interleaved with the two
+//                       matrix products of tiles j+1 and j-1; fp32 online
 //                       softmax in the exp2 domain; fp32 accumulators.
+//   sdpa_mfma_kernel    bf16 / f16, head_dim 32: same arithmetic, K and V tiles
+//                       staged through registers into LDS.
 //   sdpa_generic_kernel any dtype, head_dim <= 256, fp32 FMA arithmetic; used
-//                       for fp32 inputs and for head sizes the MFMA kernel does
+//                       for fp32 inputs and for head sizes the MFMA kernels do
 //                       not cover.
 //
-// The MFMA kernel computes the TRANSPOSED score tile S^T = K * Q^T, so that in
+// The MFMA kernels compute the TRANSPOSED score tile S^T = K * Q^T, so that in
 // the 32x32 accumulator layout every lane owns ONE query column (lane % 32) and
 // 16 key rows.  Row statistics of the softmax are then in-lane reductions plus a
 // single exchange with lane ^ 32, and the exponentiated tile is already laid out
@@ -63,7 +68,7 @@ template <bool BF16> __device__ __forceinline__ uint32_t pack2(float lo, float h
         float2_t f = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t)); // v_cvt_pk_bf16_f32, RNE
     } else {
-        return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+        return pack_f16x2(lo, hi); // v_cvt_pk_f16_f32, RNE
     }
 }
 

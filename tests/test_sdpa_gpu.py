@@ -41,7 +41,9 @@ HALF_CASES = [  # (B,H,Sq,Skv,D, causal, mask)
     (1, 1, 256, 256, 64, False, None), (4, 8, 16, 16, 32, False, None), (1, 1, 1, 1, 32, False, None),
     (2, 3, 130, 70, 64, True, None), (2, 3, 70, 130, 64, True, None), (1, 2, 300, 300, 128, True, None),
     (1, 3, 257, 511, 128, False, "mod3"), (1, 20, 1500, 1500, 64, False, None),  # Whisper encoder shape
-    (2, 8, 1024, 1024, 128, True, None), (1, 1, 8, 8, 48, False, None), (1, 1, 64, 64, 96, True, None)]
+    (2, 8, 1024, 1024, 128, True, None), (1, 1, 8, 8, 48, False, None), (1, 1, 64, 64, 96, True, None),
+    # head_dim 64 with enough (batch, head, block) units for the 8-wave work-groups: causal pairs, ragged blocks, a mask
+    (2, 64, 600, 600, 64, True, None), (1, 128, 300, 520, 64, False, "mod3")]
 
 
 @pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
