@@ -36,6 +36,10 @@ int ensure_init();
 
 inline bool valid_dtype(int dt) { return dt >= AXHIP_DTYPE_F32 && dt <= AXHIP_DTYPE_BF16; }
 inline size_t dtype_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
+// Outputs of at least this size are written with non-temporal stores: they cannot stay in the
+// 256 MiB last-level cache next to the launch's inputs anyway, and a consumer that follows
+// immediately could not find them there either.
+constexpr int64_t STREAMING_OUTPUT_BYTES = 64ll << 20;
 
 // -------------------------------------------------------------- device side
 constexpr int WAVE = 64;
@@ -179,14 +183,23 @@ __device__ __forceinline__ void load_vec(const void *p, int dt, int64_t i, float
     }
 }
 
+// 16-byte non-temporal store.  Written as an instruction because a builtin non-temporal store in
+// one arm of a run-time branch is merged with the ordinary store of the other arm, losing the hint.
+__device__ __forceinline__ void store16_streaming(void *p, uint4_t v) {
+    asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(v) : "memory");
+}
+
+// `streaming`: non-temporal stores, for outputs far larger than the caches (they then do not
+// push the inputs of the same launch out of the last-level cache)
 template <int N>
-__device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const float (&v)[N]) {
+__device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const float (&v)[N], bool streaming = false) {
     if (dt == AXHIP_DTYPE_F32) {
         float4_t *q = reinterpret_cast<float4_t *>(static_cast<float *>(p) + i);
 #pragma unroll
         for (int j = 0; j < N / 4; ++j) {
             float4_t t = {v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
-            q[j] = t;
+            if (streaming) store16_streaming(&q[j], __builtin_bit_cast(uint4_t, t));
+            else q[j] = t;
         }
     } else {
         uint32_t w[N / 2];
@@ -203,7 +216,8 @@ __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const floa
 #pragma unroll
             for (int j = 0; j < N / 8; ++j) {
                 uint4_t t = {w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
-                q[j] = t;
+                if (streaming) store16_streaming(&q[j], t);
+                else q[j] = t;
             }
         } else {
             uint2_t *q = reinterpret_cast<uint2_t *>(static_cast<uint16_t *>(p) + i);

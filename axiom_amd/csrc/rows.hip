@@ -333,7 +333,7 @@ __global__ __launch_bounds__(THREADS) void rows_streamed_kernel(const AxhipRowsP
 // E elements of the flattened [rows*cols] range.  Requires cols % E == 0 so a
 // chunk never straddles two rows.
 template <int THREADS, int E>
-__global__ __launch_bounds__(THREADS) void elementwise_kernel(const AxhipRowsProgram P) {
+__global__ __launch_bounds__(THREADS) void elementwise_kernel(const AxhipRowsProgram P, const bool streaming) {
     const int64_t cols = P.cols;
     const int64_t nchunk = P.rows * cols / E;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * THREADS;
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(THREADS) void elementwise_kernel(const AxhipRowsPro
         else load_vec<E>(P.input, P.input_dtype, flat, v[0]);
         for (int i = 0; i < P.n_pre + P.n_post; ++i) apply_op<1, E>(i < P.n_pre ? P.pre[i] : P.post[i - P.n_pre], P, v, row, col0, ok);
         if constexpr (E == 1) store_any(P.output, P.output_dtype, flat, v[0][0]);
-        else store_vec<E>(P.output, P.output_dtype, flat, v[0]);
+        else store_vec<E>(P.output, P.output_dtype, flat, v[0], streaming);
     }
 }
 
@@ -533,7 +533,8 @@ int launch_plan_e(const AxhipRowsProgram &P, const RowsPlan &pl, hipStream_t s) 
     case RowsPlan::ELEMENTWISE: {
         const int64_t nchunk = P.rows * P.cols / E;
         const int64_t blocks = std::min<int64_t>((nchunk + 255) / 256, 256 * 32);
-        hipLaunchKernelGGL((elementwise_kernel<256, E>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, P);
+        const bool streaming = P.rows * P.cols * static_cast<int64_t>(dtype_size(P.output_dtype)) >= STREAMING_OUTPUT_BYTES;
+        hipLaunchKernelGGL((elementwise_kernel<256, E>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, P, streaming);
         return AXHIP_OK;
     }
     case RowsPlan::RESIDENT:

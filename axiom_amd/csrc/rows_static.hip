@@ -48,6 +48,7 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     a.cols = P.cols;
     a.eps = P.eps;
     a.out_dtype = P.output_dtype;
+    a.stream_out = P.reduce == AXHIP_RED_NONE && P.rows * P.cols * static_cast<int64_t>(dtype_size(P.output_dtype)) >= STREAMING_OUTPUT_BYTES;
 
     auto vector_operand = [&](int idx, int kind) -> const void * {
         if (idx < 0 || idx >= P.n_operands) return nullptr;

@@ -34,6 +34,7 @@ struct RowsStaticArgs {
     int32_t post_op;    // 0 or a unary AXHIP_OP_*
     int32_t red_mean;   // reduce == MEAN: scale the sum by 1/cols
     int32_t out_dtype;  // dtype of a reduced [rows] output
+    int32_t stream_out; // full-size output written with non-temporal stores
 };
 
 struct RowsStaticKey {
