@@ -539,6 +539,12 @@ static bool ring_enabled() {
     return on;
 }
 
+// AXHIP_GEMM_RING_TILE=0..2 forces one ring tile shape (128x128, 64x128, 128x192) for A/B timing
+static int ring_tile_override() {
+    static const int v = [] { const char *e = std::getenv("AXHIP_GEMM_RING_TILE"); return (e && e[0] >= '0' && e[0] <= '2') ? e[0] - '0' : -1; }();
+    return v;
+}
+
 extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemmParams *params, void *stream) {
     AXHIP_REQUIRE(params != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_gemm: params is NULL");
     const AxhipGemmParams &p = *params;
@@ -601,13 +607,30 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
             hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(8 * per_xcd), static_cast<unsigned>(p.batch)), dim3(256), lds_bytes, s, g, tiles_m, tiles_n);
             return AXHIP_OK;
         };
-        // 128 x 128 tiles (4 stages) once they give most CUs a work-group, else 64 x 128 tiles (6 stages).  (256 x 128
-        // tiles with 3 stages measured the same as 128 x 128: what bounds these shapes is the bytes in flight per
-        // CU, i.e. the LDS ring itself, against the latency of the first touch of every k-tile.)
-        const int64_t t128 = ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch;
+        // Tile shape by modelled time: rounds of work-groups over the 256 CUs x (ring fill and epilogue + the tile's
+        // k loop).  The k-loop cost per tile element is calibrated on the Whisper projections (64 x 128 tiles pay 1.4x
+        // per element for their lower reuse of the LDS fragments, 128 x 192 tiles 1.13x for their shorter ring).  The
+        // wide tile exists because a product such as 1500 x 3840 x 1280 makes 360 tiles of 128 x 128 (two rounds, the
+        // second 40 % full) but 240 of 128 x 192.
+        struct RingTile { int tm, tn; double per_elem; };
+        static const RingTile candidates[] = {{128, 128, 1.0}, {64, 128, 1.42}, {128, 192, 1.13}};
+        int best = 0;
+        double best_cost = 0.0;
+        for (int c = 0; c < 3; ++c) {
+            const RingTile &rt = candidates[c];
+            if (ring_tile_override() >= 0 && c != ring_tile_override()) continue;
+            const int64_t tiles = ((p.m + rt.tm - 1) / rt.tm) * ((p.n + rt.tn - 1) / rt.tn) * p.batch;
+            const double rounds = static_cast<double>((tiles + 255) / 256);
+            // fixed part: 3 us, in units where a 128 x 128 x 1280 k loop costs 12.25 us
+            const double cost = rounds * (3.0 + 12.25 * rt.per_elem * (rt.tm * rt.tn / 16384.0) * (static_cast<double>(p.k) / 1280.0));
+            if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best = c; }
+        }
         int rc2;
-        if (t128 >= 192) rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 128, 128, 4>, 128, 128, 4 * 256 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 128, 128, 4>, 128, 128, 4 * 256 * BIG_ROWB);
-        else rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 64, 128, 6>, 64, 128, 6 * 192 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 64, 128, 6>, 64, 128, 6 * 192 * BIG_ROWB);
+        switch (best) {
+        case 0: rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 128, 128, 4>, 128, 128, 4 * 256 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 128, 128, 4>, 128, 128, 4 * 256 * BIG_ROWB); break;
+        case 1: rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 64, 128, 6>, 64, 128, 6 * 192 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 64, 128, 6>, 64, 128, 6 * 192 * BIG_ROWB); break;
+        default: rc2 = bf ? launch(gemm_mfma_nt_ring_kernel<true, 128, 192, 4>, 128, 192, 4 * 320 * BIG_ROWB) : launch(gemm_mfma_nt_ring_kernel<false, 128, 192, 4>, 128, 192, 4 * 320 * BIG_ROWB); break; // all 160 KiB of LDS
+        }
         if (rc2) return rc2;
     } else if (half && nt && p.k > 0) {
         // Tall tiles (two work-groups per CU, one k-tile in flight) once they fill the chip;

@@ -77,10 +77,12 @@ def test_half_large_tile_path_matches_fp64(dt, M, N, K, extras):
 
 @pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("M,N,K,extras", [(1500, 5120, 1280, False), (1500, 1280, 5120, True), (200, 330, 256, True), (129, 257, 320, False),
-                                          (1000, 2000, 448, True), (64, 128, 4096, False)])
+                                          (1000, 2000, 448, True), (64, 128, 4096, False),
+                                          (1500, 3840, 1280, False), (1500, 3700, 320, True)])
 def test_half_ring_path_matches_fp64(dt, M, N, K, extras):
-    """Mid-size products: the multi-stage LDS ring kernels (128 x 128 and 64 x 128 tiles), with k extents of
-    exactly, fewer and more k-tiles than the ring has stages, ragged tiles, and the full epilogue."""
+    """Mid-size products: the multi-stage LDS ring kernels (128 x 128, 64 x 128 and, for the last two shapes,
+    128 x 192 tiles), with k extents of exactly, fewer and more k-tiles than the ring has stages, ragged tiles,
+    and the full epilogue."""
     g = axo.PCG64(M * 7 + K)
     x, W = axo.to_bits(g.normal((M, K)), dt), axo.to_bits(g.normal((N, K)) * (2.0 / np.sqrt(K)), dt)
     bias = axo.to_bits(g.normal((N,)) * 0.1, dt) if extras else None
