@@ -529,6 +529,145 @@ __global__ __launch_bounds__(256, 1) void gemm_mfma_nt_ring_kernel(const GemmArg
     gemm_store_tiles<BF16, MI, NJ>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
 }
 
+// ------------------------------------------------------------------ fp32, MFMA
+// C = A B^T in fp32 on v_mfma_f32_32x32x2_f32 (fp32 products, fp32 accumulation: no precision is given up against
+// the FMA kernel), A [M,K] and B [N,K] both K-contiguous.  Same skeleton as the 16-bit ring kernel: a k-tile is 32
+// floats, i.e. the same 128-byte LDS rows, XOR swizzle and direct-to-LDS loads; a lane's 16-byte fragment read holds
+// four k values that feed four successive MFMAs (which k a lane contributes to which MFMA is free as long as A and B
+// agree).  K only has to be a multiple of 4: the chunks of the last k-tile that lie past K are sent out of the
+// descriptor's range and arrive as zeros.  At 1/16 of the 16-bit MFMA rate the kernel is bound by the matrix pipe,
+// not by the ring.
+template <int TM, int TNR, int S>
+__global__ __launch_bounds__(256, 1) void gemm_mfma_f32_ring_kernel(const GemmArgs g, const int tiles_m, const int tiles_n) {
+    constexpr int MI = TM / 64, NJ = TNR / 64;
+    constexpr int NLA = TM / 32, NLB = TNR / 32;
+    constexpr int KF = 32;                            // floats per k-tile
+    constexpr int STAGEB = (TM + TNR) * BIG_ROWB;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char big_lds[];
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+    const int l32 = lane % 32, g2 = lane / 32;
+
+    const int per_xcd = gridDim.x / 8;
+    const int t = (static_cast<int>(blockIdx.x) % 8) * per_xcd + static_cast<int>(blockIdx.x) / 8;
+    if (t >= tiles_m * tiles_n) return;
+    constexpr int GR = 4;
+    const int group = t / (GR * tiles_n), first_m = group * GR;
+    const int gsz = min(GR, tiles_m - first_m);
+    const int rem = t - group * GR * tiles_n;
+    const int tm = first_m + rem % gsz, tn = rem / gsz;
+    const int64_t m0 = static_cast<int64_t>(tm) * TM, n0 = static_cast<int64_t>(tn) * TNR;
+    const int64_t bz = blockIdx.y;
+    const float *A = static_cast<const float *>(g.a) + bz * g.sa + m0 * g.a_rs;
+    const float *B = static_cast<const float *>(g.b) + bz * g.sb + n0 * g.b_cs;
+    const int arow_bytes = static_cast<int>(g.a_rs) * 4, brow_bytes = static_cast<int>(g.b_cs) * 4;
+    const int rows_a = static_cast<int>(min<int64_t>(TM, g.M - m0)), rows_b = static_cast<int>(min<int64_t>(TNR, g.N - n0));
+    const int K = static_cast<int>(g.K);
+    const int4_t arsrc = gemm_rsrc(A, (rows_a - 1) * arow_bytes + K * 4);
+    const int4_t brsrc = gemm_rsrc(B, (rows_b - 1) * brow_bytes + K * 4);
+
+    const int ld_r = 8 * wave + (lane >> 3);
+    const int ld_c = (lane & 7) ^ ((ld_r >> 1) & 7); // source chunk of this lane: floats 4 ld_c .. 4 ld_c + 3 of the k-tile
+    int a_voff[NLA], b_voff[NLB];
+#pragma unroll
+    for (int n = 0; n < NLA; ++n) a_voff[n] = (32 * n + ld_r) * arow_bytes + ld_c * 16;
+#pragma unroll
+    for (int n = 0; n < NLB; ++n) b_voff[n] = (32 * n + ld_r) * brow_bytes + ld_c * 16;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(big_lds));
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 8 * wave * BIG_ROWB);
+    constexpr int OUT_OF_RANGE = 0x7FFFFFF0;
+    auto load_tile = [&](int kt, int stage) {
+        const int soff = kt * BIG_ROWB;
+        const bool k_ok = kt * KF + ld_c * 4 < K; // false only for the trailing chunks of a ragged last k-tile
+#pragma unroll
+        for (int n = 0; n < NLA; ++n) gemm_load_to_lds(arsrc, lds_wave + stage * STAGEB + n * 32 * BIG_ROWB, k_ok ? a_voff[n] : OUT_OF_RANGE, soff);
+#pragma unroll
+        for (int n = 0; n < NLB; ++n) gemm_load_to_lds(brsrc, lds_wave + stage * STAGEB + TM * BIG_ROWB + n * 32 * BIG_ROWB, k_ok ? b_voff[n] : OUT_OF_RANGE, soff);
+    };
+
+    const int wm = (wave / 2) * (TM / 2), wn = (wave % 2) * (TNR / 2);
+    int f_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) f_off[ks] = l32 * BIG_ROWB + (((2 * ks + g2) ^ ((l32 >> 1) & 7)) * 16);
+
+    float16_t acc[MI][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    float4_t fa[2][MI], fb[2][NJ];
+    auto read_frags = [&](int slot, int stage, int ks) {
+        const unsigned char *As = big_lds + stage * STAGEB + wm * BIG_ROWB;
+        const unsigned char *Bs = big_lds + stage * STAGEB + (TM + wn) * BIG_ROWB;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) fb[slot][j] = *reinterpret_cast<const float4_t *>(Bs + 32 * j * BIG_ROWB + f_off[ks]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[slot][i] = *reinterpret_cast<const float4_t *>(As + 32 * i * BIG_ROWB + f_off[ks]);
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][i][c], fb[slot][j][c], acc[i][j], 0, 0, 0);
+    };
+
+    const int nk = (K + KF - 1) / KF;
+    constexpr int INFLIGHT = (NLA + NLB) * (S - 2);
+    static_assert(INFLIGHT < 64, "vmcnt is a 6-bit counter");
+    constexpr int WAIT_OLDEST = (INFLIGHT & 0xF) | 0x0F70 | ((INFLIGHT >> 4) << 14);
+#pragma unroll
+    for (int st = 0; st < S - 1; ++st)
+        if (st < nk) load_tile(st, st);
+
+    auto step = [&](auto stage_tag, int kt) {
+        constexpr int ST = decltype(stage_tag)::value;
+        if (kt + S - 2 < nk) __builtin_amdgcn_s_waitcnt(WAIT_OLDEST);
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        if (kt + S - 1 < nk) load_tile(kt + S - 1, (ST + S - 1) % S);
+        read_frags(0, ST, 0);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            if (ks + 1 < 4) read_frags((ks + 1) & 1, ST, ks + 1);
+            multiply(ks & 1);
+        }
+    };
+    auto steps = [&](auto self, auto stage_tag, int kt0) -> void {
+        constexpr int ST = decltype(stage_tag)::value;
+        if constexpr (ST < S) {
+            if (kt0 + ST < nk) {
+                step(stage_tag, kt0 + ST);
+                self(self, std::integral_constant<int, ST + 1>{}, kt0);
+            }
+        }
+    };
+    for (int kt0 = 0; kt0 < nk; kt0 += S) steps(steps, std::integral_constant<int, 0>{}, kt0);
+
+    // epilogue: accumulator element e of tile (i, j) is C[m + 32 i + 8 (e / 4) + 4 g2 + e % 4][n + 32 j + l32]
+    float *Cb = static_cast<float *>(g.c) + bz * g.sc;
+    const float *Rb = g.residual ? static_cast<const float *>(g.residual) + bz * g.sc : nullptr;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int64_t col = n0 + wn + 32 * j + l32;
+        if (col >= g.N) continue;
+        const float bias = g.bias ? static_cast<const float *>(g.bias)[col] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int64_t row = m0 + wm + 32 * i + 8 * (e / 4) + 4 * g2 + e % 4;
+                if (row >= g.M) continue;
+                float x = acc[i][j][e] + bias;
+                if (Rb) x += Rb[row * g.ldc + col];
+                Cb[row * g.ldc + col] = gemm_epilogue(g.epilogue, x);
+            }
+    }
+}
+
 } // namespace axhip
 
 using namespace axhip;
@@ -536,6 +675,12 @@ using namespace axhip;
 // AXHIP_GEMM_RING=0 routes mid-size products to the register-staged kernels (for A/B timing)
 static bool ring_enabled() {
     static const bool on = [] { const char *e = std::getenv("AXHIP_GEMM_RING"); return !(e && e[0] == '0'); }();
+    return on;
+}
+
+// AXHIP_GEMM_F32_MFMA=0 routes fp32 products to the FMA kernel (for A/B timing)
+static bool f32_mfma_enabled() {
+    static const bool on = [] { const char *e = std::getenv("AXHIP_GEMM_F32_MFMA"); return !(e && e[0] == '0'); }();
     return on;
 }
 
@@ -646,6 +791,41 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
             if (bf) hipLaunchKernelGGL((gemm_mfma_nt_kernel<true, 64, 3>), grid, dim3(256), 0, s, g);
             else hipLaunchKernelGGL((gemm_mfma_nt_kernel<false, 64, 3>), grid, dim3(256), 0, s, g);
         }
+    } else if (p.dtype == AXHIP_DTYPE_F32 && !p.trans_a && p.trans_b && p.k >= 32 && p.k % 4 == 0 && p.lda % 4 == 0 && p.ldb % 4 == 0 &&
+               p.stride_a % 4 == 0 && p.stride_b % 4 == 0 && al16(a) && al16(b) && p.lda < (1 << 21) && p.ldb < (1 << 21) && p.k < (1 << 24) &&
+               p.batch < 65536 && p.m * p.n * p.batch >= 64 * 64 * 16 && f32_mfma_enabled()) {
+        // fp32 x W^T on the fp32 MFMA; tile shape by rounds of work-groups x tile area (the kernel is bound by the matrix pipe)
+        auto launch = [&](auto kernel, int tm_rows, int tn_cols, size_t lds_bytes) -> int {
+            static std::mutex mu;
+            static std::set<const void *> configured;
+            {
+                std::lock_guard<std::mutex> lk(mu);
+                if (!configured.count(reinterpret_cast<const void *>(kernel))) {
+                    AXHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+                    configured.insert(reinterpret_cast<const void *>(kernel));
+                }
+            }
+            const int tiles_m = static_cast<int>((p.m + tm_rows - 1) / tm_rows), tiles_n = static_cast<int>((p.n + tn_cols - 1) / tn_cols);
+            const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+            hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(8 * per_xcd), static_cast<unsigned>(p.batch)), dim3(256), lds_bytes, s, g, tiles_m, tiles_n);
+            return AXHIP_OK;
+        };
+        static const int shapes[4][2] = {{128, 128}, {64, 128}, {128, 192}, {64, 64}};
+        int best = 0;
+        double best_cost = 0.0;
+        for (int c = 0; c < 4; ++c) {
+            const int64_t tiles = ((p.m + shapes[c][0] - 1) / shapes[c][0]) * ((p.n + shapes[c][1] - 1) / shapes[c][1]) * p.batch;
+            const double cost = static_cast<double>((tiles + 255) / 256) * (0.05 + shapes[c][0] * shapes[c][1] / 16384.0);
+            if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best = c; }
+        }
+        int rc2;
+        switch (best) {
+        case 0: rc2 = launch(gemm_mfma_f32_ring_kernel<128, 128, 3>, 128, 128, 3 * 256 * BIG_ROWB); break;
+        case 1: rc2 = launch(gemm_mfma_f32_ring_kernel<64, 128, 3>, 64, 128, 3 * 192 * BIG_ROWB); break;
+        case 3: rc2 = launch(gemm_mfma_f32_ring_kernel<64, 64, 3>, 64, 64, 3 * 128 * BIG_ROWB); break;
+        default: rc2 = launch(gemm_mfma_f32_ring_kernel<128, 192, 3>, 128, 192, 3 * 320 * BIG_ROWB); break;
+        }
+        if (rc2) return rc2;
     } else {
         dim3 grid(static_cast<unsigned>((p.n + 15) / 16), static_cast<unsigned>((p.m + 15) / 16), static_cast<unsigned>(p.batch));
         AXHIP_REQUIRE(grid.y < 65536, AXHIP_ERR_UNSUPPORTED, "axhip_gemm: m too large for the generic kernel");

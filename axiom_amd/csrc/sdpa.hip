@@ -27,6 +27,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 
 namespace axhip {
 
@@ -680,6 +681,206 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     }
 }
 
+// ------------------------------------------------------------- fp32 MFMA kernel
+// fp32 inputs, head_dim 32 / 64 / 128, on v_mfma_f32_32x32x2_f32: fp32 products and fp32 accumulation, so nothing
+// is given up against the FMA kernel below, at about ten times its rate.  Same transposed formulation as the 16-bit
+// kernels: S^T = K Q^T leaves every lane with one query column and 16 of a sub-tile's 32 keys, and the
+// exponentiated scores are, as they sit in the accumulator registers, the B operand (P^T, two keys per MFMA) of
+// O^T += V^T P^T -- no conversion and no trip through LDS.  One work-group = 4 waves = 128 query rows; K and V tiles
+// of 64 keys are staged through registers into padded LDS rows (K: +4 floats, conflict-free 16-byte fragment reads;
+// V: +8 floats, so the two half-waves of a 4-byte read hit disjoint banks), double-buffered.  At 64 cycles per MFMA
+// the kernel is bound by the matrix pipe; the softmax in between is a few percent.
+template <int D> constexpr int sdpa_f32_lds_bytes() { return 2 * BN * ((D + 4) + (D + 8)) * 4; }
+
+template <bool HAS_MASK, int D>
+__global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
+    constexpr int KSTR = D + 4, VSTR = D + 8; // LDS row strides in floats
+    constexpr int DT = D / 32;                // 32-row tiles of O^T
+    constexpr int QJ = D / 8;                 // 16-byte Q / K fragments per lane
+    constexpr int KCH = D / 4;                // 16-byte chunks per K / V row
+    constexpr int NLD = BN * KCH / 256;       // chunks per thread per tile (2, 4, 8)
+    constexpr int ROWS_PER_PASS = 256 / KCH;
+    extern __shared__ __attribute__((aligned(16))) float f32_lds[];
+    auto Ks = [&](int buf) { return f32_lds + buf * BN * KSTR; };              // K tile `buf`
+    auto Vs = [&](int buf) { return f32_lds + 2 * BN * KSTR + buf * BN * VSTR; }; // V tile `buf`
+
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int ql = lane % 32, g = lane / 32;
+
+    const int L = blockIdx.x;
+    const int BH = a.B * a.H;
+    int bh, qb;
+    if (BH % 8 == 0) { // one (batch, head) stays on one XCD, whose L2 then holds its K / V
+        const int xcd = L % 8, j = L / 8;
+        bh = (j / a.nqb) * 8 + xcd;
+        qb = j % a.nqb;
+    } else {
+        bh = L / a.nqb;
+        qb = L % a.nqb;
+    }
+    if (a.causal) qb = a.nqb - 1 - qb; // heaviest blocks first
+    const int b = bh / a.H, h = bh % a.H;
+
+    const float *Q = static_cast<const float *>(a.q) + b * a.qs[0] + h * a.qs[1];
+    const float *K = static_cast<const float *>(a.k) + b * a.ks[0] + h * a.ks[1];
+    const float *V = static_cast<const float *>(a.v) + b * a.vs[0] + h * a.vs[1];
+    float *O = static_cast<float *>(a.o) + b * a.os[0] + h * a.os[1];
+    const uint8_t *M = HAS_MASK ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
+
+    const int q0 = qb * BM;
+    const int qw0 = q0 + wave * 32;
+    const int q = qw0 + ql;
+    const bool q_ok = q < a.Sq;
+
+    // K / V through buffer descriptors: rows past the end of the sequence read as zero
+    const int krow_bytes = static_cast<int>(a.ks[2]) * 4, vrow_bytes = static_cast<int>(a.vs[2]) * 4;
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(K), 0, (a.Skv - 1) * krow_bytes + D * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(V), 0, (a.Skv - 1) * vrow_bytes + D * 4, 0x00020000);
+    const int ld_row = tid / KCH, ld_cc = tid % KCH;
+    const int k_voff = ld_row * krow_bytes + ld_cc * 16, v_voff = ld_row * vrow_bytes + ld_cc * 16;
+
+    // Q^T fragments (B operand): lane holds Q[q][8 j + 4 g .. + 3]; component c of fragment j meets K's component c
+    float4_t qf[QJ];
+#pragma unroll
+    for (int j = 0; j < QJ; ++j) {
+        qf[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (q_ok) qf[j] = *reinterpret_cast<const float4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 8 * j + 4 * g);
+    }
+
+    float16_t oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
+    float m_run = NEG_INF_F, l_run = 0.0f;
+
+    int kv_end = a.Skv;
+    if (a.causal) kv_end = min(a.Skv, q0 + BM);
+    const int ntiles = (kv_end + BN - 1) / BN; // >= 1
+
+    uint4_t kreg[NLD], vreg[NLD];
+    auto load_tile = [&](int tile) {
+#pragma unroll
+        for (int n = 0; n < NLD; ++n) {
+            const int row0 = tile * BN + n * ROWS_PER_PASS;
+            kreg[n] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, k_voff + row0 * krow_bytes, 0, 0);
+            vreg[n] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, v_voff + row0 * vrow_bytes, 0, 0);
+        }
+    };
+    auto stage_tile = [&](int buf) {
+#pragma unroll
+        for (int n = 0; n < NLD; ++n) {
+            const int row = ld_row + n * ROWS_PER_PASS;
+            *reinterpret_cast<uint4_t *>(Ks(buf) + row * KSTR + 4 * ld_cc) = kreg[n];
+            *reinterpret_cast<uint4_t *>(Vs(buf) + row * VSTR + 4 * ld_cc) = vreg[n];
+        }
+    };
+
+    const int k_frag = ql * KSTR + 4 * g; // + kt * 32 * KSTR + 8 j
+    const int v_frag = 4 * g * VSTR + ql; // + (kt * 32 + 8 (e / 4) + e % 4) * VSTR + 32 dt
+
+    load_tile(0);
+    stage_tile(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    if (ntiles > 1) load_tile(1);
+    __syncthreads();
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int kv0 = tile * BN;
+        const int buf = tile & 1;
+        if (tile + 1 < ntiles) stage_tile(buf ^ 1);
+        if (tile + 2 < ntiles) load_tile(tile + 2);
+
+        if (!(a.causal && kv0 > qw0 + 31)) { // a wave whose last query row precedes this tile has nothing to add
+            const float *Kb = Ks(buf), *Vb = Vs(buf);
+
+            // ---- S^T = K Q^T: two 32-key sub-tiles, D / 2 MFMAs of two dims each
+            float16_t s[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < QJ; ++j) {
+                    const float4_t kf = *reinterpret_cast<const float4_t *>(&Kb[k_frag + kt * 32 * KSTR + 8 * j]);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[c], qf[j][c], s[kt], 0, 0, 0);
+                }
+            }
+
+            const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
+            if (need_mask) {
+                const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                        bool dead = kv > kv_limit;
+                        if constexpr (HAS_MASK) {
+                            if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                        }
+                        if (dead) s[kt][i] = NEG_INF_F;
+                    }
+            }
+
+            // ---- online softmax (per lane: one query column, 32 of the 64 keys), base-2 domain
+            float mloc = NEG_INF_F;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+            const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
+            if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
+                const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+            }
+            const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float pexp = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], a.scale_log2e, -m_use));
+                    s[kt][i] = pexp;
+                    l_run += pexp;
+                }
+
+            // ---- O^T += V^T P^T: MFMA e of a sub-tile multiplies keys 8 (e / 4) + e % 4 (lower half-wave) and + 4 (upper)
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const float vf = Vb[v_frag + (kt * 32 + 8 * (e / 4) + e % 4) * VSTR + 32 * dt];
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, s[kt][e], oacc[dt], 0, 0, 0);
+                    }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: O = O^T / l, four consecutive dims per store
+    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (q_ok) {
+        float *orow = O + static_cast<int64_t>(q) * a.os[2];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const float4_t w = {oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv, oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv};
+                *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
+            }
+    }
+}
+
 // ------------------------------------------------------------- generic kernel
 // 256 threads = 16 query rows x 16 lanes.  K/V tiles of 32 keys are widened to
 // fp32 in LDS.  Lane c of a row computes scores for keys c, c+16 and output dims
@@ -783,12 +984,18 @@ __global__ __launch_bounds__(256) void sdpa_generic_kernel(const SdpaArgs a) {
 // ------------------------------------------------------------------ host side
 namespace {
 
-enum class SdpaKind { EMPTY, MFMA, GENERIC, INVALID };
+enum class SdpaKind { EMPTY, MFMA, MFMA_F32, GENERIC, INVALID };
 
 // 0 = automatic; 4 / 8 forces the work-group width of the head_dim-128 kernel (AXHIP_SDPA_D128_WAVES)
 int sdpa_d128_waves = [] {
     const char *e = getenv("AXHIP_SDPA_D128_WAVES");
     return e ? atoi(e) : 0;
+}();
+
+// AXHIP_SDPA_F32_MFMA=0 sends fp32 attention to the FMA kernel (for A/B timing)
+bool sdpa_f32_mfma = [] {
+    const char *e = getenv("AXHIP_SDPA_F32_MFMA");
+    return !(e && e[0] == '0');
 }();
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -807,6 +1014,15 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
         ok = ok && span < (int64_t(1) << 31);
         ok = ok && (!q || aligned16(q)) && (!k || aligned16(k)) && (!v || aligned16(v)) && (!o || aligned16(o));
         if (ok) return SdpaKind::MFMA;
+    }
+    if (p.dtype == AXHIP_DTYPE_F32 && d_ok && sdpa_f32_mfma) {
+        bool ok = true;
+        for (int i = 0; i < 3; ++i) // 16-byte vector access to every row
+            ok = ok && p.q_strides[i] % 4 == 0 && p.k_strides[i] % 4 == 0 && p.v_strides[i] % 4 == 0 && p.o_strides[i] % 4 == 0;
+        const int64_t span = (static_cast<int64_t>(p.seq_kv) + 64) * std::max(p.k_strides[2], p.v_strides[2]) * 4;
+        ok = ok && span < (int64_t(1) << 31);
+        ok = ok && (!q || aligned16(q)) && (!k || aligned16(k)) && (!v || aligned16(v)) && (!o || aligned16(o));
+        if (ok) return SdpaKind::MFMA_F32;
     }
     if (p.head_dim <= GMAXD) return SdpaKind::GENERIC;
     return SdpaKind::INVALID;
@@ -827,6 +1043,22 @@ template <bool BF16, int D> void launch_mfma(const SdpaArgs &a, hipStream_t s) {
     const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
     if (a.mask) hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, true>), dim3(grid), dim3(256), 0, s, a);
     else hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, false>), dim3(grid), dim3(256), 0, s, a);
+}
+
+template <int D> int launch_mfma_f32(const SdpaArgs &a, hipStream_t s) {
+    constexpr int lds = sdpa_f32_lds_bytes<D>();
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel<false, D>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (attr == hipSuccess)
+            attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel<true, D>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    });
+    AXHIP_CHECK_HIP(attr);
+    const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
+    if (a.mask) hipLaunchKernelGGL((sdpa_mfma_f32_kernel<true, D>), dim3(grid), dim3(256), lds, s, a);
+    else hipLaunchKernelGGL((sdpa_mfma_f32_kernel<false, D>), dim3(grid), dim3(256), lds, s, a);
+    return AXHIP_OK;
 }
 
 } // namespace
@@ -852,6 +1084,9 @@ const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *p) {
     case SdpaKind::EMPTY: return "empty";
     case SdpaKind::MFMA:
         snprintf(name, sizeof(name), "mfma_%s_d%d", p->dtype == AXHIP_DTYPE_BF16 ? "bf16" : "f16", p->head_dim);
+        return name;
+    case SdpaKind::MFMA_F32:
+        snprintf(name, sizeof(name), "mfma_f32_d%d", p->head_dim);
         return name;
     case SdpaKind::GENERIC: return "generic";
     default: return "invalid";
@@ -879,7 +1114,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
     }
     AXHIP_REQUIRE(kind != SdpaKind::INVALID, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: head_dim %d > %d is not supported", p.head_dim, GMAXD);
     AXHIP_REQUIRE(q && k && v && o, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: NULL tensor");
-    AXHIP_REQUIRE(static_cast<int64_t>(p.batch) * p.heads < 65536 || kind == SdpaKind::MFMA, AXHIP_ERR_UNSUPPORTED,
+    AXHIP_REQUIRE(static_cast<int64_t>(p.batch) * p.heads < 65536 || kind != SdpaKind::GENERIC, AXHIP_ERR_UNSUPPORTED,
                   "axhip_sdpa_fwd: batch*heads too large for the generic kernel");
     rc = ensure_init();
     if (rc) return rc;
@@ -930,6 +1165,11 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         }
             break;
         }
+    } else if (kind == SdpaKind::MFMA_F32) {
+        a.nqb = (p.seq_q + BM - 1) / BM;
+        AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
+        rc = p.head_dim == 32 ? launch_mfma_f32<32>(a, s) : p.head_dim == 64 ? launch_mfma_f32<64>(a, s) : launch_mfma_f32<128>(a, s);
+        if (rc) return rc;
     } else {
         a.nqb = (p.seq_q + GM - 1) / GM;
         const size_t lds = sizeof(float) * (static_cast<size_t>(GM) * a.D + static_cast<size_t>(GN) * (a.D + 1) + static_cast<size_t>(GN) * a.D + GM * GN);

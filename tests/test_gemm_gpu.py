@@ -30,6 +30,29 @@ def test_f32_matches_oracle(M, N, K, ta, tb):
     assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("M,N,K,extras,batch", [(1500, 1280, 1280, False, 1), (300, 250, 36, True, 1), (260, 257, 100, True, 1),
+                                                (1500, 3840, 384, False, 1), (2000, 330, 240, True, 1), (256, 256, 32, False, 1),
+                                                (200, 136, 520, True, 3)])
+def test_f32_mfma_path_matches_fp64(M, N, K, extras, batch):
+    """fp32 x W^T on the fp32 matrix instruction: ragged tiles, k extents that are not a multiple of the 32-float
+    k-tile (36, 100, 240, 520), fewer k-tiles than ring stages, every tile shape, batches against a shared weight,
+    and the bias / residual / GELU epilogue.  fp32 products and sums: held to the fp32 bar against float64."""
+    import math
+
+    g = axo.PCG64(M * 3 + K)
+    x = g.normal((batch, M, K)).astype(np.float32)
+    W = (g.normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    bias = (g.normal((N,)) * 0.1).astype(np.float32) if extras else None
+    res = g.normal((batch, M, N)).astype(np.float32) if extras else None
+    got = gh.gemm(x, W, F32, trans_b=True, bias=bias, residual=res, epilogue="gelu" if extras else None)
+    want = x.astype(np.float64) @ W.astype(np.float64).T
+    if extras:
+        y = want + bias + res
+        want = 0.5 * y * (1 + np.vectorize(math.erf)(y / math.sqrt(2)))
+    assert got.shape == (batch, M, N)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4), np.max(np.abs(got - want))
+
+
 @pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("M,N,K", [(1, 3, 8), (128, 128, 64), (130, 70, 200), (1500, 1280, 1280)])
 def test_half_linear_matches_fp32_reference(dt, M, N, K):

@@ -29,7 +29,7 @@ def test_f32_matches_cpu_oracle(case):
     mask = make_mask(mk, Sq, Skv)
     sc = -1.0 if scale is None else scale
     got, kern = gh.sdpa(q, k, v, F32, sc, causal, mask)
-    assert kern == "generic"
+    assert kern == (f"mfma_f32_d{D}" if D in (32, 64, 128) else "generic")
     want = axo.sdpa(q, k, v, F32, sc, causal, mask)
     assert np.allclose(got, want, rtol=1e-4, atol=1e-4), np.max(np.abs(got - want))
 
@@ -44,6 +44,22 @@ HALF_CASES = [  # (B,H,Sq,Skv,D, causal, mask)
     (2, 8, 1024, 1024, 128, True, None), (1, 1, 8, 8, 48, False, None), (1, 1, 64, 64, 96, True, None),
     # head_dim 64 with enough (batch, head, block) units for the 8-wave work-groups: causal pairs, ragged blocks, a mask
     (2, 64, 600, 600, 64, True, None), (1, 128, 300, 520, 64, False, "mod3")]
+
+
+@pytest.mark.parametrize("case", HALF_CASES, ids=lambda c: "x".join(str(x) for x in c))
+def test_f32_on_the_larger_shapes(case):
+    """fp32 through the fp32-MFMA kernel (head_dim 32 / 64 / 128; 48 and 96 take the FMA kernel) on the multi-tile,
+    ragged, causal, cross-attention and masked shapes, held to the fp32 bar."""
+    B, H, Sq, Skv, D, causal, mk = case
+    q, k, v = inputs(B, H, Sq, Skv, D, F32, seed=11)
+    mask = make_mask(mk, Sq, Skv)
+    got, kern = gh.sdpa(q, k, v, F32, -1.0, causal, mask)
+    assert kern == (f"mfma_f32_d{D}" if D in (32, 64, 128) else "generic")
+    if B * H * Sq * Skv <= 1 << 24:
+        want = naive_attention64(q, k, v, 1 / math.sqrt(D), causal, mask)
+    else:
+        want = axo.sdpa(q, k, v, F32, -1.0, causal, mask)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4), np.max(np.abs(got - want))
 
 
 @pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])

@@ -57,14 +57,11 @@ def reference_forward(w, mel, n_layers, heads):
     return F.layer_norm(x, (Dm,), w["layer_norm.weight"], w["layer_norm.bias"])
 
 
-# whisper-tiny's encoder geometry (d_model 384, 4 layers, 6 heads, 80 mel bins), at a short
-# and at the full 30 s (3000-frame) input
-@pytest.mark.parametrize("dtype,frames,tol", [("f32", 200, 2e-3), ("f32", 3000, 2e-3), ("bf16", 3000, None), ("f16", 600, None)])
-def test_encoder_matches_fp32_reference(tmp_path, dtype, frames, tol):
+def run_case(tmp_path, geometry, dtype, frames, tol):
     from safetensors.torch import save_file
 
     assert BIN.exists(), f"{BIN} is missing: run python -m axiom_amd.build --host"
-    d_model, n_layers, heads, ffn, n_mels = 384, 4, 6, 1536, 80
+    d_model, n_layers, heads, ffn, n_mels = geometry
     w = make_weights(d_model, n_layers, ffn, n_mels, 1500, seed=7)
     mel = torch.randn(1, n_mels, frames, generator=torch.Generator().manual_seed(8))
     if dtype != "f32":  # the reference sees the same rounded parameters and input
@@ -85,8 +82,22 @@ def test_encoder_matches_fp32_reference(tmp_path, dtype, frames, tol):
     with torch.no_grad():
         want = reference_forward(w, mel, n_layers, heads).numpy()
     err = np.abs(got - want)
-    if tol is not None:  # fp32: the library's own 1e-4 per op, accumulated over 4 layers of O(1)-scaled activations
+    if tol is not None:  # fp32: the library's own 1e-4 per op, accumulated over the layers of O(1)-scaled activations
         assert err.max() < tol, err.max()
     else:  # 16-bit: every intermediate is rounded to the type; outputs are layer-normed, O(1)
         eps = 2.0**-8 if dtype == "bf16" else 2.0**-11
         assert err.max() < 40 * eps and err.mean() < 4 * eps, (err.max(), err.mean())
+
+
+# whisper-tiny's encoder geometry (d_model 384, 4 layers, 6 heads, 80 mel bins), at a short
+# and at the full 30 s (3000-frame) input
+@pytest.mark.parametrize("dtype,frames,tol", [("f32", 200, 2e-3), ("f32", 3000, 2e-3), ("bf16", 3000, None), ("f16", 600, None)])
+def test_encoder_matches_fp32_reference(tmp_path, dtype, frames, tol):
+    run_case(tmp_path, (384, 4, 6, 1536, 80), dtype, frames, tol)
+
+
+# one layer at whisper-large's width (d_model 1280, 20 heads of 64, ffn 5120, 128 mel bins) over the full
+# 3000 frames: the shapes of the Whisper-style block the benchmarks time ([1, 1500, 1280], 20 x 64)
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_large_width_layer_matches_fp32_reference(tmp_path, dtype):
+    run_case(tmp_path, (1280, 1, 20, 5120, 128), dtype, 3000, None)
