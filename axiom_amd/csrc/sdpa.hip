@@ -692,21 +692,30 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
 // the kernel is bound by the matrix pipe; the softmax in between is a few percent.
 template <int D> constexpr int sdpa_f32_lds_bytes() { return 2 * BN * ((D + 4) + (D + 8)) * 4; }
 
-template <bool HAS_MASK, int D>
+// SPLIT = 1, 2 or 4 waves share one 32-row query block and divide its keys among themselves (32-key sub-tiles in
+// turn); their (reference maximum, denominator, O^T) states are merged through LDS at the end.  A wave's MFMAs form
+// one dependent chain over its keys, so short problems (few work-groups, e.g. one batch of 8 heads x 512 rows) are
+// bound by that chain's length rather than by the chip: splitting the keys shortens it SPLIT-fold.
+template <bool HAS_MASK, int D, int SPLIT>
 __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
+    static_assert(SPLIT == 1 || SPLIT == 2 || SPLIT == 4, "waves per query block");
     constexpr int KSTR = D + 4, VSTR = D + 8; // LDS row strides in floats
     constexpr int DT = D / 32;                // 32-row tiles of O^T
     constexpr int QJ = D / 8;                 // 16-byte Q / K fragments per lane
     constexpr int KCH = D / 4;                // 16-byte chunks per K / V row
-    constexpr int NLD = BN * KCH / 256;       // chunks per thread per tile (2, 4, 8)
+    constexpr int NLD = BN * KCH / 256;       // chunks per thread per 64-key tile (2, 4, 8)
     constexpr int ROWS_PER_PASS = 256 / KCH;
+    constexpr int BMW = 32 * (4 / SPLIT);     // query rows per work-group
+    constexpr int TPI = SPLIT == 4 ? 2 : 1;   // 64-key tiles per iteration (one 32-key sub-tile per wave when split)
+    constexpr int NSUB = SPLIT == 1 ? 2 : 1;  // sub-tiles a wave multiplies per iteration
     extern __shared__ __attribute__((aligned(16))) float f32_lds[];
-    auto Ks = [&](int buf) { return f32_lds + buf * BN * KSTR; };              // K tile `buf`
+    auto Ks = [&](int buf) { return f32_lds + buf * BN * KSTR; };                 // K tile `buf`
     auto Vs = [&](int buf) { return f32_lds + 2 * BN * KSTR + buf * BN * VSTR; }; // V tile `buf`
 
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
     const int ql = lane % 32, g = lane / 32;
+    const int rb = wave / SPLIT, part = wave % SPLIT; // query block within the work-group, share of its keys
 
     const int L = blockIdx.x;
     const int BH = a.B * a.H;
@@ -728,8 +737,8 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
     float *O = static_cast<float *>(a.o) + b * a.os[0] + h * a.os[1];
     const uint8_t *M = HAS_MASK ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
 
-    const int q0 = qb * BM;
-    const int qw0 = q0 + wave * 32;
+    const int q0 = qb * BMW;
+    const int qw0 = q0 + rb * 32;
     const int q = qw0 + ql;
     const bool q_ok = q < a.Sq;
 
@@ -756,128 +765,199 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
     float m_run = NEG_INF_F, l_run = 0.0f;
 
     int kv_end = a.Skv;
-    if (a.causal) kv_end = min(a.Skv, q0 + BM);
-    const int ntiles = (kv_end + BN - 1) / BN; // >= 1
+    if (a.causal) kv_end = min(a.Skv, q0 + BMW);
+    const int nit = (kv_end + TPI * BN - 1) / (TPI * BN); // >= 1
 
-    uint4_t kreg[NLD], vreg[NLD];
-    auto load_tile = [&](int tile) {
+    uint4_t kreg[TPI * NLD], vreg[TPI * NLD];
+    auto load_it = [&](int it) {
 #pragma unroll
-        for (int n = 0; n < NLD; ++n) {
-            const int row0 = tile * BN + n * ROWS_PER_PASS;
-            kreg[n] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, k_voff + row0 * krow_bytes, 0, 0);
-            vreg[n] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, v_voff + row0 * vrow_bytes, 0, 0);
-        }
+        for (int tt = 0; tt < TPI; ++tt)
+#pragma unroll
+            for (int n = 0; n < NLD; ++n) {
+                const int row0 = (it * TPI + tt) * BN + n * ROWS_PER_PASS;
+                kreg[tt * NLD + n] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, k_voff + row0 * krow_bytes, 0, 0);
+                vreg[tt * NLD + n] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, v_voff + row0 * vrow_bytes, 0, 0);
+            }
     };
-    auto stage_tile = [&](int buf) {
+    auto stage_tile = [&](int tt, int buf) { // tile tt of the iteration held in registers -> LDS buffer buf
 #pragma unroll
         for (int n = 0; n < NLD; ++n) {
             const int row = ld_row + n * ROWS_PER_PASS;
-            *reinterpret_cast<uint4_t *>(Ks(buf) + row * KSTR + 4 * ld_cc) = kreg[n];
-            *reinterpret_cast<uint4_t *>(Vs(buf) + row * VSTR + 4 * ld_cc) = vreg[n];
+            *reinterpret_cast<uint4_t *>(Ks(buf) + row * KSTR + 4 * ld_cc) = kreg[tt * NLD + n];
+            *reinterpret_cast<uint4_t *>(Vs(buf) + row * VSTR + 4 * ld_cc) = vreg[tt * NLD + n];
         }
     };
 
     const int k_frag = ql * KSTR + 4 * g; // + kt * 32 * KSTR + 8 j
     const int v_frag = 4 * g * VSTR + ql; // + (kt * 32 + 8 (e / 4) + e % 4) * VSTR + 32 dt
 
-    load_tile(0);
-    stage_tile(0);
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-    if (ntiles > 1) load_tile(1);
-    __syncthreads();
+    // One iteration's share of this wave: NSUB sub-tiles of 32 keys.  Sub-tile u sits in LDS buffer sub_buf(u, buf)
+    // at key offset 32 * sub_kt(u) and starts at key sub_kv(u, it) of the sequence.
+    auto sub_kt = [&](int u) { return SPLIT == 1 ? u : part % 2; };
+    auto sub_buf = [&](int buf) { return SPLIT == 4 ? part / 2 : buf; };
+    auto sub_kv = [&](int u, int it) { return it * TPI * BN + (SPLIT == 4 ? (part / 2) * BN : 0) + 32 * sub_kt(u); };
 
-    for (int tile = 0; tile < ntiles; ++tile) {
-        const int kv0 = tile * BN;
-        const int buf = tile & 1;
-        if (tile + 1 < ntiles) stage_tile(buf ^ 1);
-        if (tile + 2 < ntiles) load_tile(tile + 2);
+    auto compute = [&](int it, int buf) {
+        const int kv_first = sub_kv(0, it);
+        if (a.causal && kv_first > qw0 + 31) return; // every key of this wave's share lies past its last query row
+        const float *Kb = Ks(sub_buf(buf)), *Vb = Vs(sub_buf(buf));
 
-        if (!(a.causal && kv0 > qw0 + 31)) { // a wave whose last query row precedes this tile has nothing to add
-            const float *Kb = Ks(buf), *Vb = Vs(buf);
-
-            // ---- S^T = K Q^T: two 32-key sub-tiles, D / 2 MFMAs of two dims each
-            float16_t s[2];
+        // ---- S^T = K Q^T: D / 2 MFMAs of two dims per 32-key sub-tile
+        float16_t s[NSUB];
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
+        for (int u = 0; u < NSUB; ++u) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+            for (int i = 0; i < 16; ++i) s[u][i] = 0.0f;
 #pragma unroll
-                for (int j = 0; j < QJ; ++j) {
-                    const float4_t kf = *reinterpret_cast<const float4_t *>(&Kb[k_frag + kt * 32 * KSTR + 8 * j]);
+            for (int j = 0; j < QJ; ++j) {
+                const float4_t kf = *reinterpret_cast<const float4_t *>(&Kb[k_frag + sub_kt(u) * 32 * KSTR + 8 * j]);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[c], qf[j][c], s[kt], 0, 0, 0);
-                }
+                for (int c = 0; c < 4; ++c) s[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[c], qf[j][c], s[u], 0, 0, 0);
             }
+        }
 
-            const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
-            if (need_mask) {
-                const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
+        const int kv_last = sub_kv(NSUB - 1, it) + 31;
+        const bool need_mask = (a.causal && kv_last > qw0) || (kv_last >= a.Skv) || HAS_MASK;
+        if (need_mask) {
+            const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
 #pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
-                        bool dead = kv > kv_limit;
-                        if constexpr (HAS_MASK) {
-                            if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
-                        }
-                        if (dead) s[kt][i] = NEG_INF_F;
-                    }
-            }
-
-            // ---- online softmax (per lane: one query column, 32 of the 64 keys), base-2 domain
-            float mloc = NEG_INF_F;
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-            const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
-            if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
-                const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-                m_run = m_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-            }
-            const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
+            for (int u = 0; u < NSUB; ++u)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float pexp = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], a.scale_log2e, -m_use));
-                    s[kt][i] = pexp;
-                    l_run += pexp;
-                }
-
-            // ---- O^T += V^T P^T: MFMA e of a sub-tile multiplies keys 8 (e / 4) + e % 4 (lower half-wave) and + 4 (upper)
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        const float vf = Vb[v_frag + (kt * 32 + 8 * (e / 4) + e % 4) * VSTR + 32 * dt];
-                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, s[kt][e], oacc[dt], 0, 0, 0);
+                    const int kv = sub_kv(u, it) + (i / 4) * 8 + g * 4 + (i % 4);
+                    bool dead = kv > kv_limit;
+                    if constexpr (HAS_MASK) {
+                        if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
                     }
+                    if (dead) s[u][i] = NEG_INF_F;
+                }
         }
+
+        // ---- online softmax (per lane: one query column, half of each sub-tile's keys), base-2 domain
+        float mloc = NEG_INF_F;
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[u][i]);
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+        const float m_new = fmaxf(m_run, mloc * a.scale_log2e);
+        if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
+            const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+        }
+        const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float pexp = __builtin_amdgcn_exp2f(__builtin_fmaf(s[u][i], a.scale_log2e, -m_use));
+                s[u][i] = pexp;
+                l_run += pexp;
+            }
+
+        // ---- O^T += V^T P^T: MFMA e of a sub-tile multiplies keys 8 (e / 4) + e % 4 (lower half-wave) and + 4 (upper)
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const float vf = Vb[v_frag + (sub_kt(u) * 32 + 8 * (e / 4) + e % 4) * VSTR + 32 * dt];
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, s[u][e], oacc[dt], 0, 0, 0);
+                }
+    };
+
+    if constexpr (SPLIT < 4) {
+        // one tile per iteration, double-buffered: tile it + 1 is parked in the other buffer while tile it is multiplied
+        load_it(0);
+        stage_tile(0, 0);
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        if (nit > 1) load_it(1);
         __syncthreads();
+        for (int it = 0; it < nit; ++it) {
+            const int buf = it & 1;
+            if (it + 1 < nit) stage_tile(0, buf ^ 1);
+            if (it + 2 < nit) load_it(it + 2);
+            compute(it, buf);
+            __syncthreads();
+        }
+    } else {
+        // two tiles per iteration fill both buffers; the next pair waits in registers meanwhile
+        load_it(0);
+        for (int it = 0; it < nit; ++it) {
+            stage_tile(0, 0);
+            stage_tile(1, 1);
+            if (it + 1 < nit) load_it(it + 1);
+            __syncthreads();
+            compute(it, 0);
+            __syncthreads();
+        }
     }
 
-    // ---- epilogue: O = O^T / l, four consecutive dims per store
     const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
-    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    if (q_ok) {
-        float *orow = O + static_cast<int64_t>(q) * a.os[2];
+    if constexpr (SPLIT == 1) {
+        // ---- epilogue: O = O^T / l, four consecutive dims per store
+        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        if (q_ok) {
+            float *orow = O + static_cast<int64_t>(q) * a.os[2];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const float4_t w = {oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv, oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv};
+                    *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
+                }
+        }
+    } else {
+        // ---- merge the SPLIT partial states of each query block through LDS (the K / V buffers are free: every wave
+        // has passed the barrier that closed the last iteration).  Wave `part` then finishes 4 / SPLIT of the 4
+        // four-dim groups of every O^T tile.
+        float4_t *part_o = reinterpret_cast<float4_t *>(f32_lds);   // [wave][dt][i4][lane]
+        float *part_m = f32_lds + 4 * DT * 4 * 64 * 4;              // [wave][32]
+        float *part_l = part_m + 4 * 32;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                const float4_t w = {oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv, oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv};
-                *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
-            }
+            for (int i4 = 0; i4 < 4; ++i4)
+                part_o[((wave * DT + dt) * 4 + i4) * 64 + lane] = float4_t{oacc[dt][4 * i4], oacc[dt][4 * i4 + 1], oacc[dt][4 * i4 + 2], oacc[dt][4 * i4 + 3]};
+        if (g == 0) {
+            part_m[wave * 32 + ql] = m_run;
+            part_l[wave * 32 + ql] = l_tot;
+        }
+        __syncthreads();
+        float m_star = NEG_INF_F;
+#pragma unroll
+        for (int p = 0; p < SPLIT; ++p) m_star = fmaxf(m_star, part_m[(rb * SPLIT + p) * 32 + ql]);
+        float sc[SPLIT], l_star = 0.0f;
+#pragma unroll
+        for (int p = 0; p < SPLIT; ++p) {
+            const float m_p = part_m[(rb * SPLIT + p) * 32 + ql];
+            sc[p] = m_p == NEG_INF_F ? 0.0f : __builtin_amdgcn_exp2f(m_p - m_star);
+            l_star += sc[p] * part_l[(rb * SPLIT + p) * 32 + ql];
+        }
+        const float inv = l_star > 0.0f ? 1.0f / l_star : 0.0f;
+        if (q_ok) {
+            float *orow = O + static_cast<int64_t>(q) * a.os[2];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int k4 = 0; k4 < 4 / SPLIT; ++k4) {
+                    const int i4 = part * (4 / SPLIT) + k4;
+                    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int p = 0; p < SPLIT; ++p) {
+                        const float4_t t = part_o[(((rb * SPLIT + p) * DT + dt) * 4 + i4) * 64 + lane];
+                        acc[0] += sc[p] * t[0]; acc[1] += sc[p] * t[1]; acc[2] += sc[p] * t[2]; acc[3] += sc[p] * t[3];
+                    }
+                    const float4_t w = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+                    *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
+                }
+        }
     }
 }
 
@@ -998,6 +1078,12 @@ bool sdpa_f32_mfma = [] {
     return !(e && e[0] == '0');
 }();
 
+// AXHIP_SDPA_F32_SPLIT=1|2|4 forces the number of waves that share a query block in the fp32 kernel
+int sdpa_f32_split = [] {
+    const char *e = getenv("AXHIP_SDPA_F32_SPLIT");
+    return e ? atoi(e) : 0;
+}();
+
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, const void *v, const void *o) {
@@ -1045,20 +1131,24 @@ template <bool BF16, int D> void launch_mfma(const SdpaArgs &a, hipStream_t s) {
     else hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, false>), dim3(grid), dim3(256), 0, s, a);
 }
 
-template <int D> int launch_mfma_f32(const SdpaArgs &a, hipStream_t s) {
+template <int D, int SPLIT> int launch_mfma_f32(const SdpaArgs &a, hipStream_t s) {
     constexpr int lds = sdpa_f32_lds_bytes<D>();
     static std::once_flag once;
     static hipError_t attr = hipSuccess;
     std::call_once(once, [] {
-        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel<false, D>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel<false, D, SPLIT>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (attr == hipSuccess)
-            attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel<true, D>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+            attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel<true, D, SPLIT>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     });
     AXHIP_CHECK_HIP(attr);
     const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
-    if (a.mask) hipLaunchKernelGGL((sdpa_mfma_f32_kernel<true, D>), dim3(grid), dim3(256), lds, s, a);
-    else hipLaunchKernelGGL((sdpa_mfma_f32_kernel<false, D>), dim3(grid), dim3(256), lds, s, a);
+    if (a.mask) hipLaunchKernelGGL((sdpa_mfma_f32_kernel<true, D, SPLIT>), dim3(grid), dim3(256), lds, s, a);
+    else hipLaunchKernelGGL((sdpa_mfma_f32_kernel<false, D, SPLIT>), dim3(grid), dim3(256), lds, s, a);
     return AXHIP_OK;
+}
+
+template <int D> int launch_mfma_f32_d(const SdpaArgs &a, int split, hipStream_t s) {
+    return split == 1 ? launch_mfma_f32<D, 1>(a, s) : split == 2 ? launch_mfma_f32<D, 2>(a, s) : launch_mfma_f32<D, 4>(a, s);
 }
 
 } // namespace
@@ -1166,9 +1256,15 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             break;
         }
     } else if (kind == SdpaKind::MFMA_F32) {
-        a.nqb = (p.seq_q + BM - 1) / BM;
+        // waves per 32-row query block, by how many such blocks there are for the 1024 SIMDs (thresholds from timings
+        // of 128 .. 1024 blocks: below 0.75 blocks per SIMD the four-way split wins by up to 2.7x, above 1.5 none is needed)
+        const int64_t blocks32 = static_cast<int64_t>((p.seq_q + 31) / 32) * p.batch * p.heads;
+        int split = blocks32 >= 1536 ? 1 : blocks32 >= 768 ? 2 : 4;
+        if (sdpa_f32_split == 1 || sdpa_f32_split == 2 || sdpa_f32_split == 4) split = sdpa_f32_split;
+        const int bmw = 128 / split;
+        a.nqb = (p.seq_q + bmw - 1) / bmw;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
-        rc = p.head_dim == 32 ? launch_mfma_f32<32>(a, s) : p.head_dim == 64 ? launch_mfma_f32<64>(a, s) : launch_mfma_f32<128>(a, s);
+        rc = p.head_dim == 32 ? launch_mfma_f32_d<32>(a, split, s) : p.head_dim == 64 ? launch_mfma_f32_d<64>(a, split, s) : launch_mfma_f32_d<128>(a, split, s);
         if (rc) return rc;
     } else {
         a.nqb = (p.seq_q + GM - 1) / GM;

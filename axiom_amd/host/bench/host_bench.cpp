@@ -41,6 +41,12 @@ int main(int argc, char **argv) {
     }
     Tensor::manual_seed(42);
     std::printf("{\n");
+    { // configs[0]: the reference's CPU-runnable case, fp32, on the fp32 matrix instruction here
+        auto q = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU), k = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU),
+             v = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU);
+        measure("c1_sdpa_f32_b1h8s512d64", [&] { ops::scaled_dot_product_attention(q, k, v, Tensor(), 0.125f, false).sync(); }, warmup, iters, 536870912.0,
+                "GFLOP_per_s", false);
+    }
     { // configs[1]
         auto a = Tensor::randn({8192, 8192}, DType::Float32, Device::GPU), b = Tensor::randn({8192, 8192}, DType::Float32, Device::GPU);
         measure("c2_chain_f32_8192x8192", [&] { ops::softmax((ops::relu(a) + 1) * b, -1).sum(1).sync(); }, warmup, iters, 536903680.0, "GB_per_s", false);

@@ -62,6 +62,24 @@ def test_f32_on_the_larger_shapes(case):
     assert np.allclose(got, want, rtol=1e-4, atol=1e-4), np.max(np.abs(got - want))
 
 
+@pytest.mark.parametrize("split", ["1", "2", "4"])
+def test_f32_with_each_key_split_forced(split):
+    """The fp32 kernel lets 1, 2 or 4 waves share a query block and merges their partial softmax states; the library
+    picks by problem size.  Here every mode runs every fp32 shape: the choice is an environment setting read when
+    the library loads, so each mode gets a process of its own."""
+    import os
+    import subprocess
+    import sys
+
+    if os.environ.get("AXHIP_SDPA_F32_SPLIT"):
+        pytest.skip("already inside a forced-split run")
+    env = dict(os.environ, AXHIP_SDPA_F32_SPLIT=split)
+    r = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-p", "no:cacheprovider", __file__, "-k",
+                        "test_f32_on_the_larger_shapes or test_f32_matches_cpu_oracle or test_fully_masked"],
+                       env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:]
+
+
 @pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", HALF_CASES, ids=lambda c: "x".join(str(x) for x in c))
 def test_half_matches_fp32_reference_of_same_inputs(case, dt):
