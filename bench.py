@@ -37,11 +37,11 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the SDPA kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, each scaled by the reading of the plain-copy leg below
-# (FETCH_SIZE 0.50011, WRITE_SIZE 1.0): 585.2 MB read + 134.3 MB written.
-SDPA_TRAFFIC_BYTES = 719.4e6
+# (FETCH_SIZE 0.50009, WRITE_SIZE 1.0): 561.7 MB read + 134.2 MB written.
+SDPA_TRAFFIC_BYTES = 695.9e6
 # same measurement for the fused chains: they move the algorithmic bytes (ratio 1.001 - 1.003)
 CHAIN_TRAFFIC_BYTES = {"chain_relu_add_mul_softmax_sum_f32_8192x8192": 537.2e6,
-                       "chain_gelu_layernorm_bf16_16384x4096": 269.3e6,
+                       "chain_gelu_layernorm_bf16_16384x4096": 269.4e6,
                        "chain_gelu_rmsnorm_bf16_16384x4096": 269.2e6}
 
 
