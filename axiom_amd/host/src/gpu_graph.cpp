@@ -556,22 +556,58 @@ class PlanBuilder {
 
     int emit_gemm(const GraphNode *n, const Shape &out_shape_override, int bias_v, int res_v, int act) {
         const auto &mp = get_params<MatMulParams>(n->params);
-        int a = make_contiguous(eval(n->inputs[0].get())), b = make_contiguous(eval(n->inputs[1].get()));
-        const Shape &as = val(a).shape, &bs = val(b).shape;
+        bool ta = mp.transpose_a, tb = mp.transpose_b;
+        int a = eval(n->inputs[0].get()), b = eval(n->inputs[1].get());
         if (val(a).dtype != val(b).dtype) throw TypeError("GPU matmul needs operands of one dtype");
+        // The matrix-core kernels want both operands contiguous along k: A stored [M, K], B stored [N, K].
+        //  * an operand that is a transposed view of contiguous memory is taken as that memory with its flag flipped
+        //    (matmul(x, w.transpose()) costs no copy);
+        //  * an operand stored the other way round is transposed once by the gather kernel when the product is large
+        //    enough for that pass to be small change against the FMA kernel it avoids.
+        auto swapped = [&](int v) {
+            ValueSpec t = val(v);
+            const size_t r = t.shape.size();
+            std::swap(t.shape[r - 1], t.shape[r - 2]);
+            std::swap(t.strides[r - 1], t.strides[r - 2]);
+            return add_value(t);
+        };
+        auto k_contiguous = [&](int v, bool &flag, bool wanted_flag, bool worth_a_copy) {
+            if (val(v).shape.size() >= 2 && !contiguous(v)) {
+                const int sw = swapped(v);
+                if (contiguous(sw)) {
+                    v = sw;
+                    flag = !flag;
+                }
+            }
+            v = make_contiguous(v);
+            if (flag != wanted_flag && worth_a_copy && val(v).shape.size() >= 2) {
+                v = make_contiguous(swapped(v));
+                flag = wanted_flag;
+            }
+            return v;
+        };
+        {
+            const Shape &as0 = val(a).shape, &bs0 = val(b).shape;
+            const double m0 = static_cast<double>(ta ? as0.back() : as0[as0.size() - 2]), k0 = static_cast<double>(ta ? as0[as0.size() - 2] : as0.back());
+            const double n0 = static_cast<double>(tb ? bs0[bs0.size() - 2] : bs0.back());
+            const bool big = m0 * n0 * k0 >= double(1 << 22) && m0 >= 64 && n0 >= 64 && k0 >= 32;
+            a = k_contiguous(a, ta, false, big);
+            b = k_contiguous(b, tb, true, big);
+        }
+        const Shape &as = val(a).shape, &bs = val(b).shape;
         GemmStep g;
         g.p.dtype = detail::to_axhip_dtype(val(a).dtype);
-        g.p.trans_a = mp.transpose_a;
-        g.p.trans_b = mp.transpose_b;
+        g.p.trans_a = ta;
+        g.p.trans_b = tb;
         const size_t ar = as[as.size() - 2], ac = as.back(), br = bs[bs.size() - 2], bc = bs.back();
-        g.p.m = static_cast<int64_t>(mp.transpose_a ? ac : ar);
-        g.p.k = static_cast<int64_t>(mp.transpose_a ? ar : ac);
-        g.p.n = static_cast<int64_t>(mp.transpose_b ? br : bc);
+        g.p.m = static_cast<int64_t>(ta ? ac : ar);
+        g.p.k = static_cast<int64_t>(ta ? ar : ac);
+        g.p.n = static_cast<int64_t>(tb ? br : bc);
         g.p.lda = static_cast<int64_t>(ac);
         g.p.ldb = static_cast<int64_t>(bc);
         g.p.ldc = g.p.n;
         const size_t batch_a = ShapeUtils::size(as) / (ar * ac), batch_b = ShapeUtils::size(bs) / (br * bc);
-        if (batch_b == 1 && !mp.transpose_a) { // shared right operand (a Linear weight): fold the batch into M
+        if (batch_b == 1 && !ta) { // shared right operand (a Linear weight): fold the batch into M
             g.p.m *= static_cast<int64_t>(batch_a);
             g.p.batch = 1;
         } else if (batch_a == batch_b || batch_b == 1 || batch_a == 1) {

@@ -722,6 +722,57 @@ GPU_TEST(LazyNodes, Conv1dMatchesFloat64Loops) {
     conv1d_case(DType::Float16, 1, 8, 40, 8, 3, 1, 0, 1, false, 2e-2);
 }
 
+static std::string plan_kernels() {
+    std::string s;
+    for (const auto &k : graph::last_gpu_plan_kernels()) s += (s.empty() ? "" : " ") + k;
+    return s;
+}
+// Every transpose combination of a product large enough for the matrix cores: operands stored the "wrong" way
+// round are transposed once by a gather, a transposed view of contiguous memory is consumed as it lies.
+static void matmul_layout_case(DType dt, double tol) {
+    const size_t M = 300, K = 200, N = 260;
+    auto a = axtest::randn({M, K}, 91).astype(dt), b = axtest::randn({K, N}, 92).astype(dt);
+    const auto af = host_floats(a.astype(DType::Float32)), bf = host_floats(b.astype(DType::Float32));
+    std::vector<double> want(M * N, 0.0);
+    for (size_t i = 0; i < M; ++i)
+        for (size_t k = 0; k < K; ++k)
+            for (size_t j = 0; j < N; ++j) want[i * N + j] += double(af[i * K + k]) * double(bf[k * N + j]);
+    auto check = [&](const Tensor &r, const char *what) {
+        EXPECT_TRUE(r.shape() == Shape({M, N}));
+        const auto h = host_floats(r.astype(DType::Float32));
+        double worst = 0.0;
+        for (size_t i = 0; i < M * N; ++i) worst = std::max(worst, std::abs(double(h[i]) - want[i]) / (1.0 + std::abs(want[i])));
+        if (!(worst < tol)) std::fprintf(stderr, "    matmul layout case: %s\n", what);
+        EXPECT_LT(worst, tol);
+    };
+    auto ag = a.gpu(), bg = b.gpu();
+    auto at = ag.transpose({1, 0}).ascontiguousarray(), bt = bg.transpose({1, 0}).ascontiguousarray(); // stored [K, M] and [N, K]
+    at.sync(); bt.sync();
+    check(ops::matmul(ag, bg), "a b");
+    EXPECT_EQ(plan_kernels(), std::string("strided_copy gemm")); // b transposed once
+    check(ops::matmul(ag, bt, false, true), "a bT'");
+    EXPECT_EQ(plan_kernels(), std::string("gemm"));
+    check(ops::matmul(at, bg, true, false), "aT' b");
+    EXPECT_EQ(plan_kernels(), std::string("strided_copy strided_copy gemm"));
+    check(ops::matmul(at, bt, true, true), "aT' bT'");
+    EXPECT_EQ(plan_kernels(), std::string("strided_copy gemm"));
+    // views: the transposes below are strides over memory that already has the wanted layout
+    check(ops::matmul(ag, bt.transpose({1, 0})), "a view(bT')");
+    EXPECT_EQ(plan_kernels(), std::string("gemm"));
+    check(ops::matmul(at.transpose({1, 0}), bt.transpose({1, 0})), "view(aT') view(bT')"); // a is stored [K, M]: one pass
+    EXPECT_EQ(plan_kernels(), std::string("strided_copy gemm"));
+    check(ops::matmul(ag, bg.transpose({1, 0}), false, true), "a view(b)T'");
+    EXPECT_EQ(plan_kernels(), std::string("strided_copy gemm"));
+}
+GPU_TEST(LazyNodes, MatMulOperandLayouts) {
+    matmul_layout_case(DType::Float32, 1e-4);
+    matmul_layout_case(DType::BFloat16, 2e-2);
+    // a small product stays as it is stored (FMA kernel, no transposing pass)
+    auto x = axtest::randn({8, 16}, 93).gpu(), w = axtest::randn({16, 8}, 94).gpu();
+    ops::matmul(x, w).sync();
+    EXPECT_EQ(plan_kernels(), std::string("gemm"));
+}
+
 GPU_TEST(LazyNodes, EmbeddingLookup) { // tests/test_embedding.cpp:3-39
     std::vector<float> wd(12);
     for (int i = 0; i < 12; ++i) wd[i] = float(i);
