@@ -16,16 +16,86 @@ struct CopyArgs {
     int64_t strides[AXHIP_MAX_DIMS];
 };
 
+// IDX: int32_t when every index and offset fits (32-bit divisions cost a fraction of the 64-bit ones)
+template <typename IDX>
 __global__ __launch_bounds__(256) void strided_copy_kernel(const CopyArgs a) {
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < a.total; i += stride) {
-        int64_t rem = i, off = 0;
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, total = static_cast<IDX>(a.total);
+    for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        IDX rem = i, off = 0;
         for (int d = a.ndim - 1; d >= 0; --d) {
-            const int64_t c = rem % a.shape[d];
-            rem /= a.shape[d];
-            off += c * a.strides[d];
+            const IDX n = static_cast<IDX>(a.shape[d]);
+            const IDX q = rem / n;
+            off += (rem - q * n) * static_cast<IDX>(a.strides[d]);
+            rem = q;
         }
         store_any(a.dst, a.dst_dtype, i, load_any(a.src, a.src_dtype, off));
+    }
+}
+
+// Views whose innermost dimension is contiguous (head splits, slices, broadcasts of rows, plain casts): one thread
+// moves V consecutive elements with 16-byte accesses; a.shape[ndim-1] counts such groups and a.strides[ndim-1] is V.
+// RAW: same dtype on both sides, the bytes are moved as they are.
+template <typename IDX, int V, bool RAW>
+__global__ __launch_bounds__(256) void strided_copy_vec_kernel(const CopyArgs a) {
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, total = static_cast<IDX>(a.total);
+    for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        IDX rem = i, off = 0;
+        for (int d = a.ndim - 1; d >= 0; --d) {
+            const IDX n = static_cast<IDX>(a.shape[d]);
+            const IDX q = rem / n;
+            off += (rem - q * n) * static_cast<IDX>(a.strides[d]);
+            rem = q;
+        }
+        if constexpr (RAW) { // V elements = 16 bytes
+            const int es = a.src_dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+            const uint4_t t = *reinterpret_cast<const uint4_t *>(static_cast<const char *>(a.src) + static_cast<int64_t>(off) * es);
+            reinterpret_cast<uint4_t *>(a.dst)[i] = t;
+        } else {
+            float v[V];
+            load_vec<V>(a.src, a.src_dtype, off, v);
+            store_vec<V>(a.dst, a.dst_dtype, static_cast<int64_t>(i) * V, v);
+        }
+    }
+}
+
+// Views whose innermost (destination) dimension is strided in the source while another dimension J is contiguous
+// there: transposes.  A work-group moves a 64 x 64 tile of (J, innermost) through LDS, so the reads run along J and
+// the writes along the innermost dimension, both in full lines; the remaining dimensions select the tile's origin.
+struct TransposeArgs {
+    const void *src;
+    void *dst;
+    int src_dtype, dst_dtype, n_other;
+    int64_t nJ, nL, src_stride_l, dst_stride_j; // the source stride of J and the destination stride of L are 1
+    int64_t tiles_j, tiles_l;
+    int64_t oshape[AXHIP_MAX_DIMS], osrc[AXHIP_MAX_DIMS], odst[AXHIP_MAX_DIMS];
+};
+
+__global__ __launch_bounds__(256) void transpose_copy_kernel(const TransposeArgs a) {
+    __shared__ float tile[64][65];
+    int64_t b = blockIdx.x;
+    const int64_t tl = b % a.tiles_l;
+    b /= a.tiles_l;
+    const int64_t tj = b % a.tiles_j;
+    int64_t o = b / a.tiles_j;
+    int64_t src_base = 0, dst_base = 0;
+    for (int d = a.n_other - 1; d >= 0; --d) {
+        const int64_t c = o % a.oshape[d];
+        o /= a.oshape[d];
+        src_base += c * a.osrc[d];
+        dst_base += c * a.odst[d];
+    }
+    const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+    const int64_t j0 = tj * 64, l0 = tl * 64;
+#pragma unroll 4
+    for (int r = ty; r < 64; r += 4) {
+        const int64_t l = l0 + r, j = j0 + tx;
+        if (l < a.nL && j < a.nJ) tile[r][tx] = load_any(a.src, a.src_dtype, src_base + l * a.src_stride_l + j);
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int r = ty; r < 64; r += 4) {
+        const int64_t j = j0 + r, l = l0 + tx;
+        if (l < a.nL && j < a.nJ) store_any(a.dst, a.dst_dtype, dst_base + j * a.dst_stride_j + l, tile[tx][r]);
     }
 }
 
@@ -122,8 +192,87 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
     AXHIP_REQUIRE(src && dst, AXHIP_ERR_INVALID_ARG, "axhip_strided_copy: NULL buffer");
     int rc = ensure_init();
     if (rc) return rc;
-    const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
-    hipLaunchKernelGGL(strided_copy_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), a);
+    hipStream_t s = resolve_stream(stream);
+
+    // drop unit dimensions and merge neighbours that are contiguous in the source: fewer divisions per element
+    int nd = 0;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] == 1) continue;
+        if (nd > 0 && a.strides[nd - 1] == strides[d] * shape[d]) {
+            a.shape[nd - 1] *= shape[d];
+            a.strides[nd - 1] = strides[d];
+        } else {
+            a.shape[nd] = shape[d];
+            a.strides[nd] = strides[d];
+            ++nd;
+        }
+    }
+    a.ndim = nd;
+    int64_t max_off = 0;
+    for (int d = 0; d < nd; ++d) max_off += (a.shape[d] - 1) * a.strides[d];
+    const bool idx32 = a.total < (int64_t(1) << 31) - (1 << 23) && max_off < (int64_t(1) << 31) - (1 << 23); // room for the grid stride
+
+    // vector path: innermost dimension contiguous and every row start aligned to the vector
+    const bool raw = src_dtype == dst_dtype;
+    const int v = raw ? (src_dtype == AXHIP_DTYPE_F32 ? 4 : 8) : (dst_dtype == AXHIP_DTYPE_F32 ? 4 : 8);
+    const int src_es = src_dtype == AXHIP_DTYPE_F32 ? 4 : 2, dst_es = dst_dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    const int src_align = src_es == 4 ? 16 : v * 2; // bytes a vector load needs
+    bool vec = nd >= 1 && a.strides[nd - 1] == 1 && a.shape[nd - 1] % v == 0 && reinterpret_cast<uintptr_t>(src) % src_align == 0 &&
+               reinterpret_cast<uintptr_t>(dst) % (v * dst_es >= 16 ? 16 : 8) == 0;
+    for (int d = 0; vec && d + 1 < nd; ++d) vec = (a.strides[d] * src_es) % src_align == 0;
+    // transposes: the innermost dimension is strided, some other dimension is contiguous in the source
+    int transpose_j = -1;
+    if (!vec && nd >= 2 && a.strides[nd - 1] > 1 && a.shape[nd - 1] >= 16) {
+        for (int d = 0; d + 1 < nd; ++d)
+            if (a.strides[d] == 1 && a.shape[d] >= 16) transpose_j = d;
+    }
+    if (vec) {
+        a.shape[nd - 1] /= v;
+        a.strides[nd - 1] = v;
+        a.total /= v;
+        const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        auto launch = [&](auto idx_tag) {
+            using IDX = decltype(idx_tag);
+            if (raw && v == 4) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 4, true>), grid, dim3(256), 0, s, a);
+            else if (raw) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 8, true>), grid, dim3(256), 0, s, a);
+            else if (v == 4) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 4, false>), grid, dim3(256), 0, s, a);
+            else hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 8, false>), grid, dim3(256), 0, s, a);
+        };
+        if (idx32) launch(int32_t{});
+        else launch(int64_t{});
+    } else if (transpose_j >= 0) {
+        TransposeArgs t{};
+        t.src = src; t.dst = dst; t.src_dtype = src_dtype; t.dst_dtype = dst_dtype;
+        const int L = nd - 1, J = transpose_j;
+        t.nJ = a.shape[J]; t.nL = a.shape[L];
+        t.src_stride_l = a.strides[L];
+        t.tiles_j = (t.nJ + 63) / 64; t.tiles_l = (t.nL + 63) / 64;
+        int64_t dst_stride = 1, blocks = t.tiles_j * t.tiles_l;
+        int no = 0;
+        int64_t dst_strides[AXHIP_MAX_DIMS]; // of the contiguous output
+        for (int d = nd - 1; d >= 0; --d) {
+            dst_strides[d] = dst_stride;
+            dst_stride *= a.shape[d];
+        }
+        t.dst_stride_j = dst_strides[J];
+        for (int d = 0; d < nd; ++d) {
+            if (d == J || d == L) continue;
+            t.oshape[no] = a.shape[d];
+            t.osrc[no] = a.strides[d];
+            t.odst[no] = dst_strides[d];
+            blocks *= a.shape[d];
+            ++no;
+        }
+        t.n_other = no;
+        AXHIP_REQUIRE(blocks < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_strided_copy: view too large");
+        hipLaunchKernelGGL(transpose_copy_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, t);
+    } else {
+        const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        if (idx32) hipLaunchKernelGGL((strided_copy_kernel<int32_t>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((strided_copy_kernel<int64_t>), grid, dim3(256), 0, s, a);
+    }
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;
 }

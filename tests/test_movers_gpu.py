@@ -40,6 +40,45 @@ def test_strided_copy_of_transposed_and_broadcast_views(dt):
         assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view))
 
 
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_strided_copy_fast_paths_are_bit_exact(dt):
+    """Views big enough for the 16-byte path (innermost dimension contiguous: head splits, row and column slices,
+    broadcast rows) and for the tiled transpose (innermost dimension strided, another one contiguous), ragged
+    against the 64 x 64 tile and with further dimensions around the transposed pair."""
+    base = sample((3, 40, 70, 48), dt, 5)
+    d = gh.to_dev(base)
+    views = [base.transpose(0, 2, 1, 3), base[:, 3:35, ::2, 8:40], np.broadcast_to(base[:, :1], base.shape),  # vector path
+             base.transpose(0, 1, 3, 2), base.transpose(3, 2, 1, 0), base.transpose(1, 3, 0, 2), base.transpose(2, 0, 3, 1),
+             base[1].transpose(2, 1, 0), base[0, 5].T, base[:, :, 1:66, 3:41].transpose(0, 3, 2, 1)]
+    for view in views:
+        out = gh.empty_dev(view.shape, dt)
+        off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0])
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr() + off, dt, out.data_ptr(), dt, view.ndim, i64(view.shape), i64(elem_strides(view)), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view)), view.shape
+
+
+def test_strided_copy_casts_on_the_fast_paths():
+    x = axo.PCG64(10).normal((96, 200))
+    d = gh.to_dev(x)
+    for dt in (F16, BF16):
+        for view, strides in ((x, [200, 1]), (x.T, [1, 200])):
+            out = gh.empty_dev(view.shape, dt)
+            gh.sync()
+            capi.check(capi.lib().axhip_strided_copy(d.data_ptr(), F32, out.data_ptr(), dt, 2, i64(view.shape), i64(strides), None))
+            gh.sync()
+            assert np.array_equal(gh.to_host(out, np.uint16), axo.to_bits(np.ascontiguousarray(view), dt))
+        # and back: 16-bit source, fp32 destination
+        bits = axo.to_bits(x, dt)
+        db = gh.to_dev(bits)
+        out = gh.empty_dev(x.shape, F32)
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(db.data_ptr(), dt, out.data_ptr(), F32, 2, i64(x.shape), i64([200, 1]), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, np.float32), axo.to_f32(bits, dt))
+
+
 def test_strided_copy_casts_like_the_oracle():
     x = axo.PCG64(9).normal((33, 17))
     d = gh.to_dev(x)
