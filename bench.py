@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gfx950 backend on BASELINE.json's headline workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sdpa|chains|gemm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sdpa|chains|gemm|f32]
 
 A step is one pass of the hot path over one batch of synthetic input already
 resident in HBM: causal bf16 scaled-dot-product attention, B=4 H=32 S=4096
@@ -212,6 +212,53 @@ def bench_gemm(torch, capi, stream, steps, warmup):
     return res
 
 
+PEAK_F32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+
+
+def bench_f32(torch, capi, stream, steps, warmup):
+    """The fp32 matrix-instruction kernels (the dtype the reference's GPU path and its Whisper example run in):
+    attention on BASELINE.json configs[0] and on a chip-filling shape, x W^T on the Whisper projection and a
+    large square.  fp32 products and sums; priced against the 157.3 TFLOP/s fp32 matrix peak."""
+    lib = capi.lib()
+    sp = C.c_void_p(stream.cuda_stream)
+    res = {}
+    g = torch.Generator(device="cuda").manual_seed(42)
+    steps_f32, warmup_f32 = max(10, steps // 4), max(5, warmup // 4)  # these launches are 10-1000x longer than the 16-bit ones
+    for B, H, S, D in ((1, 8, 512, 64), (4, 32, 2048, 64)):
+        q, k, v = (torch.randn((B, H, S, D), generator=g, device="cuda") for _ in range(3))
+        o = torch.empty_like(q)
+        p = capi.SdpaParams()
+        p.dtype, p.batch, p.heads, p.seq_q, p.seq_kv, p.head_dim = capi.DTYPE_F32, B, H, S, S, D
+        p.scale, p.is_causal = -1.0, 0
+        for arr in (p.q_strides, p.k_strides, p.v_strides, p.o_strides):
+            arr[0], arr[1], arr[2] = H * S * D, S * D, D
+        args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, C.byref(p), sp)
+        torch.cuda.synchronize()
+        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_sdpa_fwd(*args)), steps_f32, warmup_f32)
+        flops = 4.0 * B * H * S * S * D
+        res[f"sdpa_f32_b{B}h{H}s{S}d{D}"] = {"kernel": lib.axhip_sdpa_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "flops": flops,
+                                             "tflops": flops / (avg_ms * 1e-3) / 1e12, "frac_of_f32_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_F32_MFMA_TFLOPS,
+                                             "finite": bool(torch.isfinite(o).all().item())}
+        del q, k, v, o
+    for M, N, K in ((1500, 1280, 1280), (4096, 4096, 4096)):
+        a = torch.randn((M, K), generator=g, device="cuda")
+        w = torch.randn((N, K), generator=g, device="cuda") * 0.02
+        c = torch.empty((M, N), device="cuda")
+        p = capi.GemmParams()
+        p.dtype, p.trans_a, p.trans_b = capi.DTYPE_F32, 0, 1
+        p.m, p.n, p.k = M, N, K
+        p.lda, p.ldb, p.ldc, p.batch = K, K, N, 1
+        args = (a.data_ptr(), w.data_ptr(), c.data_ptr(), C.byref(p), sp)
+        torch.cuda.synchronize()
+        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps_f32, warmup_f32)
+        flops = 2.0 * M * N * K
+        res[f"gemm_nt_f32_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
+                                            "frac_of_f32_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_F32_MFMA_TFLOPS,
+                                            "finite": bool(torch.isfinite(c).all().item())}
+        del a, w, c
+    return res
+
+
 def cpu_baseline(seconds_budget: float = 20.0):
     """Axiom's CPU flash attention (oracle restatement, native BLAS tier) on a bounded
     sample of the same workload: `n` (batch, head) slices of the bf16 S=4096 D=128 causal
@@ -267,7 +314,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["sdpa", "chains", "gemm"], default=None)
+    ap.add_argument("--only", choices=["sdpa", "chains", "gemm", "f32"], default=None)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (both hot paths shard without communication; "
@@ -288,6 +335,7 @@ def main() -> int:
     sd = bench_sdpa(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "sdpa") else None
     ch = bench_chains(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "chains") else None
     gm = bench_gemm(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "gemm") else None
+    f32 = bench_f32(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "f32") else None
     cpu = None if (args.no_cpu or sd is None) else cpu_baseline()
 
     line = {
@@ -315,6 +363,8 @@ def main() -> int:
         line["fused_chains"] = ch
     if gm:
         line["gemm"] = gm
+    if f32:
+        line["f32_matrix_kernels"] = f32
     if args.only is None:
         line["host_layer"] = host_layer_bench()
     if cpu:
