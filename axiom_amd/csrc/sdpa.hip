@@ -395,6 +395,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     const uint16_t *V = static_cast<const uint16_t *>(a.v) + b * a.vs[0] + h * a.vs[1];
     uint16_t *O = static_cast<uint16_t *>(a.o) + b * a.os[0] + h * a.os[1];
     const uint8_t *M = HAS_MASK ? a.mask + b * a.ms[0] + h * a.ms[1] : nullptr;
+    // Explicit masks are read as the eight 4-byte words that cover this lane's keys of a tile (the lane's 32 keys are
+    // 8 runs of 4 consecutive ones), a step before the tile's score MFMAs are issued, and applied by starting the
+    // masked elements' accumulators at -inf: the mask costs two VALU operations per score and no pass of its own.
+    // Needs 4-byte aligned rows (else, and for the ragged last tile, single bytes are read after the MFMAs).
+    const bool mask_words = HAS_MASK && a.Skv % 4 == 0 && (reinterpret_cast<uintptr_t>(M) & 3u) == 0;
+    uint32_t mk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 
     const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
     const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + D * 2);
@@ -494,16 +500,41 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
             return max_across_halves(max3(m0, s[0][15], __builtin_elementwise_maximum(m2, s[1][15])));
         };
 
+        // initial value of the score accumulators of tile `tile`: `base`, or -inf where the mask words (already in
+        // mk) say so
+        auto init_scores = [&](int tile, float base, float16_t (&s)[2]) {
+            const bool use_words = HAS_MASK && mask_words && tile * BN + BN <= a.Skv;
+    #pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+    #pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    bool dead = false;
+                    if constexpr (HAS_MASK) dead = use_words && ((mk[kt * 4 + i / 4] >> (8 * (i % 4))) & 0xFFu) != 0;
+                    s[kt][i] = dead ? NEG_INF_F : base;
+                }
+        };
+
         // S^T = K Q^T for one tile (two 32-key sub-tiles); prologue only
         auto scores = [&](const unsigned char *Kb, float16_t (&s)[2]) {
+            init_scores(0, 0.0f, s);
     #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
-    #pragma unroll
-                for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
     #pragma unroll
                 for (int t = 0; t < KT; ++t) {
                     const uint4_t kf = *reinterpret_cast<const uint4_t *>(Kb + kt * 32 * ROWB + k_off[t]);
                     s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+                }
+            }
+        };
+
+        // the mask words of this lane's keys of one tile: bytes 32 kt + 8 i4 + 4 g .. + 3 of the tile's 64, kt < 2, i4 < 4
+        auto load_mask_words = [&](int tile) {
+            if constexpr (HAS_MASK) {
+                const int kvb = tile * BN;
+                if (mask_words && q_ok && kvb + BN <= a.Skv) {
+                    const uint32_t *row = reinterpret_cast<const uint32_t *>(M + static_cast<int64_t>(q) * a.Skv + kvb + 4 * g);
+    #pragma unroll
+                    for (int w8 = 0; w8 < 8; ++w8) mk[w8] = row[(w8 / 4) * 8 + (w8 % 4) * 2];
                 }
             }
         };
@@ -518,7 +549,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
                     const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
                     bool dead = kv > kv_limit;
                     if constexpr (HAS_MASK) {
-                        if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                        if (!(mask_words && kv0 + BN <= a.Skv) && q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
                     }
                     if (dead) s[kt][i] = NEG_INF_F;
                 }
@@ -588,7 +619,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
             for (int m = 0; m < NS + NP; ++m) {
                 if (m + PF < NS + NP) read_frag(m + PF);
                 if (m < NS) {
-                    if (m % KT == 0) {
+                    if constexpr (HAS_MASK) {
+                        if (m == 0) { // both sub-tiles at once: the mask words are then free for the tile after
+                            init_scores(j + 1, -m_use, nxt);
+                            if (j + 2 < ntiles) load_mask_words(j + 2);
+                        }
+                    } else if (m % KT == 0) {
     #pragma unroll
                         for (int i = 0; i < 16; ++i) nxt[m / KT][i] = -m_use; // logits come out relative to the reference
                     }
@@ -627,6 +663,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
         };
 
         // ---- prologue: K(0), V(0), K(1) in flight; first score tile
+        load_mask_words(0);
         load_k(0, 0);
         load_v(0, 0);
         if (ntiles > 1) load_k(1, 1);
@@ -634,6 +671,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
         __syncthreads();
         float16_t sA[2], sB[2];
         scores(lds, sA);
+        if (ntiles > 1) load_mask_words(1); // for the scores of tile 1, issued in step 0
         float mxA = row_max(sA), mxB = NEG_INF_F; // unmasked row maxima, valid when the tile needs no masking
         __syncthreads(); // every wave is done with K buffer 0 before K(2) lands in it
 
@@ -644,7 +682,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
             const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
             const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
             if (active) {
-                const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
+                const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || (HAS_MASK && !mask_words);
                 float mloc = mx_cur;
                 if (need_mask) mloc = mask_and_max(kv0, cur);
                 update_max(mloc, cur);
@@ -797,6 +835,28 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
     auto sub_buf = [&](int buf) { return SPLIT == 4 ? part / 2 : buf; };
     auto sub_kv = [&](int u, int it) { return it * TPI * BN + (SPLIT == 4 ? (part / 2) * BN : 0) + 32 * sub_kt(u); };
 
+    // explicit mask: the four 4-byte words per sub-tile that cover this lane's keys (4 runs of 4 consecutive ones).
+    // They are requested before the iteration's K / V prefetch is issued and consumed after the score MFMAs.  Loads
+    // return in order, so the wait for the words must not cover the prefetch behind them: every vector load of the
+    // loop is issued unconditionally (lanes or iterations with nothing to fetch aim past the descriptor's end and
+    // read zeros), which lets the wait be an exact count.  Rows must be 4-byte aligned and the sub-tile complete,
+    // otherwise single bytes are read after the MFMAs.
+    uint32_t mw[NSUB * 4];
+    bool words_ok[NSUB];
+    const __amdgpu_buffer_rsrc_t mrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(HAS_MASK ? M : nullptr), 0, HAS_MASK ? a.Sq * a.Skv : 0, 0x00020000);
+    auto load_mask_words = [&](int it) {
+        if constexpr (HAS_MASK) {
+#pragma unroll
+            for (int u = 0; u < NSUB; ++u) {
+                const int kvs = sub_kv(u, it);
+                words_ok[u] = a.Skv % 4 == 0 && (reinterpret_cast<uintptr_t>(M) & 3u) == 0 && kvs + 32 <= a.Skv;
+                const int row_off = (words_ok[u] && q_ok) ? q * a.Skv + kvs + 4 * g : 0x7FFFFF00;
+#pragma unroll
+                for (int w4 = 0; w4 < 4; ++w4) mw[u * 4 + w4] = __builtin_amdgcn_raw_buffer_load_b32(mrsrc, row_off + 8 * w4, 0, 0);
+            }
+        }
+    };
+
     auto compute = [&](int it, int buf) {
         const int kv_first = sub_kv(0, it);
         if (a.causal && kv_first > qw0 + 31) return; // every key of this wave's share lies past its last query row
@@ -820,17 +880,36 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
         const bool need_mask = (a.causal && kv_last > qw0) || (kv_last >= a.Skv) || HAS_MASK;
         if (need_mask) {
             const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
+            bool all_words = HAS_MASK;
+            if constexpr (HAS_MASK) {
 #pragma unroll
-            for (int u = 0; u < NSUB; ++u)
+                for (int u = 0; u < NSUB; ++u) all_words = all_words && words_ok[u];
+            }
+            if (!HAS_MASK || all_words) {
+                // the usual case, free of branches and loads: selects on values that are already in registers
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int kv = sub_kv(u, it) + (i / 4) * 8 + g * 4 + (i % 4);
-                    bool dead = kv > kv_limit;
-                    if constexpr (HAS_MASK) {
-                        if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int kv = sub_kv(u, it) + (i / 4) * 8 + g * 4 + (i % 4);
+                        bool dead = kv > kv_limit;
+                        if constexpr (HAS_MASK) dead = dead || ((mw[u * 4 + i / 4] >> (8 * (i % 4))) & 0xFFu) != 0;
+                        s[u][i] = dead ? NEG_INF_F : s[u][i];
                     }
-                    if (dead) s[u][i] = NEG_INF_F;
-                }
+            } else {
+                // ragged last sub-tile or unaligned mask rows: byte by byte
+#pragma unroll
+                for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int kv = sub_kv(u, it) + (i / 4) * 8 + g * 4 + (i % 4);
+                        bool dead = kv > kv_limit;
+                        if constexpr (HAS_MASK) {
+                            if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                        }
+                        s[u][i] = dead ? NEG_INF_F : s[u][i];
+                    }
+            }
         }
 
         // ---- online softmax (per lane: one query column, half of each sub-tile's keys), base-2 domain
@@ -882,7 +961,8 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
         for (int it = 0; it < nit; ++it) {
             const int buf = it & 1;
             if (it + 1 < nit) stage_tile(0, buf ^ 1);
-            if (it + 2 < nit) load_it(it + 2);
+            load_mask_words(it);
+            load_it(it + 2); // past the last tile: zeros, nothing is fetched
             compute(it, buf);
             __syncthreads();
         }
@@ -892,7 +972,8 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
         for (int it = 0; it < nit; ++it) {
             stage_tile(0, 0);
             stage_tile(1, 1);
-            if (it + 1 < nit) load_it(it + 1);
+            load_mask_words(it);
+            load_it(it + 1); // past the last tile: zeros, nothing is fetched
             __syncthreads();
             compute(it, 0);
             __syncthreads();
@@ -1107,6 +1188,7 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
             ok = ok && p.q_strides[i] % 4 == 0 && p.k_strides[i] % 4 == 0 && p.v_strides[i] % 4 == 0 && p.o_strides[i] % 4 == 0;
         const int64_t span = (static_cast<int64_t>(p.seq_kv) + 64) * std::max(p.k_strides[2], p.v_strides[2]) * 4;
         ok = ok && span < (int64_t(1) << 31);
+        ok = ok && static_cast<int64_t>(p.seq_q) * p.seq_kv < (int64_t(1) << 31) - (1 << 20); // mask offsets are 32-bit
         ok = ok && (!q || aligned16(q)) && (!k || aligned16(k)) && (!v || aligned16(v)) && (!o || aligned16(o));
         if (ok) return SdpaKind::MFMA_F32;
     }

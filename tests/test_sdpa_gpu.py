@@ -115,16 +115,19 @@ def test_fully_masked_rows_give_zeros_everywhere_else_matches():
         assert np.max(np.abs(gf - want)) < (2e-2 if dt == BF16 else 1e-4)
 
 
-def test_per_batch_head_mask_and_broadcast_masks():
-    B, H, S, D = 2, 3, 96, 64
-    q, k, v = inputs(B, H, S, S, D, BF16, seed=5)
+@pytest.mark.parametrize("dt,S", [(BF16, 96), (BF16, 256), (F32, 96), (F32, 256), (F16, 192)], ids=["bf16-96", "bf16-256", "f32-96", "f32-256", "f16-192"])
+def test_per_batch_head_mask_and_broadcast_masks(dt, S):
+    """Random masks of every supported shape; S = 96 ends in a ragged tile (mask bytes read one by one), the other
+    lengths are whole tiles with 4-byte aligned rows (mask words applied through the accumulators' initial value)."""
+    B, H, D = 2, 3, 64
+    q, k, v = inputs(B, H, S, S, D, dt, seed=5)
     r = np.random.default_rng(0)
     for shape in ((B, H, S, S), (1, 1, S, S), (B, 1, S, S), (1, H, S, S)):
-        m = (r.random(shape) < 0.3).astype(np.uint8)
+        m = (r.random(shape) < 0.3).astype(np.uint8) * r.choice(np.array([1, 2, 128, 255], np.uint8), shape)  # any nonzero byte masks
         m[..., 0] = 0
-        got, _ = gh.sdpa(q, k, v, BF16, -1.0, False, m)
-        want = naive_attention64(*(axo.to_f32(t, BF16) for t in (q, k, v)), 0.125, False, m)
-        assert np.max(np.abs(axo.to_f32(got, BF16) - want)) < 2e-2
+        got, _ = gh.sdpa(q, k, v, dt, -1.0, False, m)
+        want = naive_attention64(*(axo.to_f32(t, dt) for t in (q, k, v)), 0.125, False, m)
+        assert np.max(np.abs(axo.to_f32(got, dt) - want)) < (1e-4 if dt == F32 else 2e-2)
 
 
 def test_head_split_view_strides_need_no_copy():
