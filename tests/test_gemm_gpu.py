@@ -118,3 +118,49 @@ def test_half_ring_path_matches_fp64(dt, M, N, K, extras):
         y = want + axo.to_f32(bias, dt) + axo.to_f32(res, dt)
         want = 0.5 * y * (1 + np.vectorize(math.erf)(y / math.sqrt(2)))
     assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_seeded_random_shapes_match_fp64(dt):
+    """Forty seeded random products per dtype, shaped to land on every kernel and tile shape (matrix-core ring tiles,
+    the 256 x 256 kernel, the register-staged and FMA fallbacks): ragged m and n, k with and without the alignment the
+    matrix-core paths need, batches against a shared or a per-batch right operand, random epilogues."""
+    import math
+
+    r = np.random.default_rng(1234 + dt)
+    erf = np.vectorize(math.erf)
+    for case in range(40):
+        big = case % 8 == 0
+        M = int(r.integers(1, 2200 if big else 700))
+        N = int(r.integers(1, 2200 if big else 700))
+        K = int(r.choice([r.integers(1, 600), 8 * r.integers(1, 80), 64 * r.integers(1, 12)]))
+        batch = int(r.choice([1, 1, 2, 3])) if not big else 1
+        shared_w = bool(r.integers(0, 2))
+        extras = bool(r.integers(0, 2))
+        epi = [None, "relu", "gelu"][int(r.integers(0, 3))] if extras else None
+        g = axo.PCG64(case * 7 + 1)
+        x = g.normal((batch, M, K))
+        W = g.normal((N, K) if shared_w else (batch, N, K)) / np.sqrt(K)
+        bias = g.normal((N,)) * 0.1 if extras else None
+        res = g.normal((batch, M, N)) if extras else None
+        if dt == F32:
+            xs, Ws = x.astype(np.float32), W.astype(np.float32)
+            bs, rs = (bias.astype(np.float32), res.astype(np.float32)) if extras else (None, None)
+            xf, Wf, bf, rf = xs, Ws, bs, rs
+        else:
+            xs, Ws = axo.to_bits(x, dt), axo.to_bits(W, dt)
+            bs, rs = (axo.to_bits(bias, dt), axo.to_bits(res, dt)) if extras else (None, None)
+            xf, Wf = axo.to_f32(xs, dt), axo.to_f32(Ws, dt)
+            bf, rf = (axo.to_f32(bs, dt), axo.to_f32(rs, dt)) if extras else (None, None)
+        got = gh.gemm(xs, Ws, dt, trans_b=True, bias=bs, residual=rs, epilogue=epi)
+        got = got.astype(np.float64) if dt == F32 else axo.to_f32(got, dt).astype(np.float64)
+        want = xf.astype(np.float64) @ np.swapaxes(Wf.astype(np.float64), -1, -2)
+        if extras:
+            want = want + bf + rf
+            if epi == "relu":
+                want = np.maximum(want, 0.0)
+            elif epi == "gelu":
+                want = 0.5 * want * (1 + erf(want / math.sqrt(2)))
+        tol = 1e-4 * (1 + np.abs(want)) if dt == F32 else 2e-2 + 2.0**-8 * np.abs(want)
+        assert got.shape == (batch, M, N)
+        assert np.all(np.abs(got - want) <= tol), (case, M, N, K, batch, shared_w, epi, float(np.max(np.abs(got - want))))
