@@ -314,8 +314,12 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--min-warmup-ms", type=float, default=None, help="warm every kernel for at least this long (default 100)")
     ap.add_argument("--only", choices=["sdpa", "chains", "gemm", "f32"], default=None)
     args = ap.parse_args()
+    if args.min_warmup_ms is not None:
+        global MIN_WARMUP_MS
+        MIN_WARMUP_MS = args.min_warmup_ms
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (both hot paths shard without communication; "
               "no multi-GPU figure is produced). Re-run with --gpus 1.", file=sys.stderr)
