@@ -221,6 +221,19 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
         if (!(a.causal && kv0 > qw0 + 31)) {
             const uint16_t *Kb = Ks[buf], *Vb = Vs[buf];
 
+            // explicit mask: the eight 4-byte words that cover this lane's keys of the tile (8 runs of 4 consecutive
+            // keys), requested ahead of the score MFMAs; needs whole tiles and 4-byte aligned mask rows
+            uint32_t mw[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            bool mask_words_tile = false;
+            if constexpr (HAS_MASK) {
+                mask_words_tile = a.Skv % 4 == 0 && (reinterpret_cast<uintptr_t>(M) & 3u) == 0 && kv0 + BN <= a.Skv;
+                if (mask_words_tile && q_ok) {
+                    const uint32_t *row = reinterpret_cast<const uint32_t *>(M + static_cast<int64_t>(q) * a.Skv + kv0 + 4 * g);
+#pragma unroll
+                    for (int w8 = 0; w8 < 8; ++w8) mw[w8] = row[(w8 / 4) * 8 + (w8 % 4) * 2];
+                }
+            }
+
             // ---- S^T = K Q^T : two 32-key sub-tiles
             float16_t s[2];
 #pragma unroll
@@ -238,17 +251,31 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
             const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv) || HAS_MASK;
             if (need_mask) {
                 const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1; // last visible key of this row
+                if (!HAS_MASK || mask_words_tile) {
+                    // selects on values already in registers (for an explicit mask: the words fetched above)
 #pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
+                    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
-                        bool dead = kv > kv_limit;
-                        if constexpr (HAS_MASK) {
-                            if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                        for (int i = 0; i < 16; ++i) {
+                            const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                            bool dead = kv > kv_limit;
+                            if constexpr (HAS_MASK) dead = dead || ((mw[kt * 4 + i / 4] >> (8 * (i % 4))) & 0xFFu) != 0;
+                            s[kt][i] = dead ? NEG_INF_F : s[kt][i];
                         }
-                        if (dead) s[kt][i] = NEG_INF_F;
-                    }
+                } else {
+                    // ragged last tile, unaligned mask rows: byte by byte
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                            bool dead = kv > kv_limit;
+                            if constexpr (HAS_MASK) {
+                                if (q_ok && kv < a.Skv) dead = dead || M[static_cast<int64_t>(q) * a.Skv + kv] != 0;
+                            }
+                            s[kt][i] = dead ? NEG_INF_F : s[kt][i];
+                        }
+                }
             }
 
             // ---- online softmax (per lane: one query column, 32 of the 64 keys)
