@@ -226,6 +226,19 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
 
     if (query.device() != Device::GPU && key.device() != Device::GPU && value.device() != Device::GPU)
         throw RuntimeError("ops::scaled_dot_product_attention on CPU tensors: this library is the gfx950 GPU backend only; move the operands with .gpu()");
+    // Head sizes between the matrix-core kernels' 32 / 64 / 128 are padded with zero dims up to the next one (zeros
+    // change neither Q K^T nor the wanted part of P V) once the problem is large enough for three pad passes and an
+    // output slice to be small change against the FMA kernel they avoid (two orders of magnitude slower); this is
+    // where the reference's decomposed fallback for such sizes (flash_attention_dispatch.mm:180-196) ends up.
+    if (D != 32 && D != 64 && D > 0 && D < 128 && static_cast<double>(B) * H * Sq * Skv * D >= double(1 << 24) &&
+        (query.dtype() == DType::Float32 || query.dtype() == DType::Float16 || query.dtype() == DType::BFloat16)) {
+        const size_t Dp = D < 32 ? 32 : D < 64 ? 64 : 128;
+        const std::vector<std::pair<size_t, size_t>> widen{{0, 0}, {0, 0}, {0, 0}, {0, Dp - D}};
+        auto on_gpu = [](const Tensor &t) { return t.device() == Device::GPU ? t : t.to(Device::GPU); };
+        const float sc = scale > 0.0f ? scale : 1.0f / std::sqrt(static_cast<float>(D));
+        Tensor wide = detail::sdpa(ops::pad(on_gpu(query), widen), ops::pad(on_gpu(key), widen), ops::pad(on_gpu(value), widen), mask, sc, is_causal, out_bshd);
+        return wide.slice({Slice(), Slice(), Slice(), Slice(0, static_cast<int64_t>(D))});
+    }
     const Tensor q = sdpa_operand(query), k = sdpa_operand(key), v = sdpa_operand(value);
 
     AxhipSdpaParams p{};

@@ -323,6 +323,25 @@ GPU_TEST(FlashAttentionGPU, HalfTypesRunOnMfma) { // tests/test_flash_attention.
                 EXPECT_LE(max_abs_diff(got, ref), 2e-2);
             }
 }
+GPU_TEST(FlashAttentionGPU, OddHeadSizesArePaddedOntoTheMatrixCores) {
+    // large enough problems with head_dim 48 / 80 / 96 / 20 run as the next of 32 / 64 / 128; the result is the same
+    struct Case { DType dt; size_t B, H, Sq, Skv, D; bool causal; const char *kernel; double tol; };
+    const Case cases[] = {{DType::Float32, 1, 4, 300, 300, 48, false, "mfma_f32_d64", 1e-4}, {DType::Float32, 2, 2, 256, 200, 96, true, "mfma_f32_d128", 1e-4},
+                          {DType::BFloat16, 1, 4, 300, 300, 80, true, "mfma_bf16_d128", 2e-2}, {DType::Float16, 2, 4, 400, 400, 20, false, "mfma_f16_d32", 2e-2}};
+    for (const Case &c : cases) {
+        auto [q, k, v] = make_inputs(c.B, c.H, c.Sq, c.Skv, c.D, c.dt);
+        auto ref = axtest::oracle_sdpa(q.astype(DType::Float32), k.astype(DType::Float32), v.astype(DType::Float32), Tensor(), -1, c.causal);
+        auto got = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), -1, c.causal);
+        EXPECT_EQ(got.shape(), q.shape());
+        EXPECT_EQ(got.dtype(), c.dt);
+        EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string(c.kernel));
+        EXPECT_LE(max_abs_diff(got, ref), c.tol);
+    }
+    // a small one stays on the kernel for arbitrary head sizes
+    auto [q, k, v] = make_inputs(1, 2, 16, 16, 48);
+    ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), -1, false).sync();
+    EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("generic"));
+}
 GPU_TEST(FlashAttentionGPU, Config1Float32) { // BASELINE configs[0]: B1 H8 S512 D64, no mask, scale 0.125
     auto [q, k, v] = make_inputs(1, 8, 512, 512, 64);
     auto got = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), 0.125f, false);
