@@ -17,7 +17,9 @@ bool has_pattern(int pre, int row_op, int reduce) {
     return false;
 }
 
-const char *pre_name(int pre) { return pre == RP_NONE ? "" : pre == RP_ADDF ? "addf_" : "relu_adds_mulf_"; }
+const char *pre_name(int pre) {
+    return pre == RP_NONE ? "" : pre == RP_ADDF ? "addf_" : pre == RP_MULS ? "muls_" : pre == RP_MULS_ADDF ? "muls_addf_" : "relu_adds_mulf_";
+}
 const char *rowop_name(int r) {
     switch (r) {
     case AXHIP_ROWOP_SOFTMAX: return "softmax";
@@ -56,13 +58,35 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
         return (o.kind == kind && o.dtype == dt && aligned16(o.ptr)) ? o.ptr : nullptr;
     };
 
+    // a scalar of the pre chain: an immediate, or a one-element device operand
+    auto scalar_of = [&](const AxhipChainOp &c) -> bool {
+        if (c.imm_kind == AXHIP_BK_IMM) {
+            a.s_imm = c.imm;
+            return true;
+        }
+        const int idx = c.operand;
+        if (idx < 0 || idx >= P.n_operands || P.operands[idx].kind != AXHIP_BK_SCALAR) return false;
+        a.s_ptr = P.operands[idx].ptr;
+        a.s_dtype = P.operands[idx].dtype;
+        return true;
+    };
+
     // pre chain
     if (P.n_pre == 0) {
         k.pre = RP_NONE;
-    } else if (P.n_pre == 1 && P.pre[0].op == AXHIP_OP_ADD && P.pre[0].imm_kind != AXHIP_BK_IMM) {
+    } else if (P.n_pre == 1 && P.pre[0].op == AXHIP_OP_ADD && P.pre[0].imm_kind != AXHIP_BK_IMM &&
+               P.pre[0].operand >= 0 && P.pre[0].operand < P.n_operands && P.operands[P.pre[0].operand].kind == AXHIP_BK_FULL) {
         a.f = vector_operand(P.pre[0].operand, AXHIP_BK_FULL);
         if (!a.f) return false;
         k.pre = RP_ADDF;
+    } else if (P.n_pre == 1 && P.pre[0].op == AXHIP_OP_MUL) { // x * s: the scaled softmax
+        if (!scalar_of(P.pre[0])) return false;
+        k.pre = RP_MULS;
+    } else if (P.n_pre == 2 && P.pre[0].op == AXHIP_OP_MUL && P.pre[1].op == AXHIP_OP_ADD && P.pre[1].imm_kind != AXHIP_BK_IMM) { // x * s + bias tensor
+        if (!scalar_of(P.pre[0])) return false;
+        a.f = vector_operand(P.pre[1].operand, AXHIP_BK_FULL);
+        if (!a.f) return false;
+        k.pre = RP_MULS_ADDF;
     } else if (P.n_pre == 3 && P.pre[0].op == AXHIP_OP_RELU && P.pre[1].op == AXHIP_OP_ADD && P.pre[2].op == AXHIP_OP_MUL &&
                P.pre[2].imm_kind != AXHIP_BK_IMM) {
         if (P.pre[1].imm_kind == AXHIP_BK_IMM) {

@@ -247,3 +247,45 @@ def test_mixed_chains_around_row_ops_match_oracle():
     p = gh.Rows(x, F32).binary("mul", f)
     got = p.run(reduce="sum")
     assert np.allclose(got, (x.astype(np.float64) * f).sum(-1), rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_scaled_and_biased_softmax_on_the_specialised_kernels(dt):
+    """softmax(x * s), softmax(x + y) and softmax(x * s + y) -- the forms a decomposed attention or a masked
+    classifier head produces -- are specialised kernels; s as an immediate and as a one-element device operand."""
+    g = axo.PCG64(91)
+    tol = 1e-4 if dt == F32 else 2e-2
+    for rows, cols in ((33, 512), (7, 4096), (5, 8200 if dt != F32 else 8192)):
+        x, y = g.normal((rows, cols)) * 3, g.normal((rows, cols))
+        xs, ys = (x.astype(np.float32), y.astype(np.float32)) if dt == F32 else (axo.to_bits(x, dt), axo.to_bits(y, dt))
+        xf, yf = (xs, ys) if dt == F32 else (axo.to_f32(xs, dt), axo.to_f32(ys, dt))
+        sc = np.array([0.125], np.float32) if dt == F32 else axo.to_bits(np.array([0.125]), dt)
+        cases = [(gh.Rows(xs, dt).imm("mul", 0.125).row_op("softmax"), "muls_softmax", xf.astype(np.float64) * 0.125),
+                 (gh.Rows(xs, dt).binary("mul", sc, "scalar").row_op("softmax"), "muls_softmax", xf.astype(np.float64) * 0.125),
+                 (gh.Rows(xs, dt).binary("add", ys).row_op("softmax"), "addf_softmax", xf.astype(np.float64) + yf),
+                 (gh.Rows(xs, dt).imm("mul", 0.125).binary("add", ys).row_op("softmax"), "muls_addf_softmax", xf.astype(np.float64) * 0.125 + yf)]
+        for prog, tag, logits in cases:
+            got = prog.run()
+            assert prog.kernel_name().startswith("rows_static_" + tag), prog.kernel_name()
+            got = got.astype(np.float64) if dt == F32 else axo.to_f32(got, dt).astype(np.float64)
+            e = np.exp(logits - logits.max(-1, keepdims=True))
+            want = e / e.sum(-1, keepdims=True)
+            assert np.max(np.abs(got - want)) < tol, (tag, rows, cols)
+    # fp32: the same roundings as the chain evaluated op by op (product, then sum)
+    x, y = g.normal((9, 1024)).astype(np.float32), g.normal((9, 1024)).astype(np.float32)
+    got = gh.Rows(x, F32).imm("mul", 0.3).binary("add", y).row_op("softmax").run()
+    assert close32(got, axo.softmax(axo.binary("add", axo.binary("mul", x, np.array([0.3], np.float32), kind="scalar"), y)))
+
+
+@pytest.mark.parametrize("post", ["silu", "sigmoid", "tanh"])
+def test_fast_activations_after_a_norm_in_16_bit(post):
+    g = axo.PCG64(17)
+    x = axo.to_bits(g.normal((19, 1024)) * 2, BF16)
+    w, b = axo.to_bits(g.uniform((1024,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((1024,), -0.5, 0.5), BF16)
+    prog = gh.Rows(x, BF16).row_op("layernorm", 1e-5, w=w, b=b).unary(post)
+    got = axo.to_f32(prog.run(), BF16).astype(np.float64)
+    assert prog.kernel_name().startswith("rows_static_layernorm_bf16"), prog.kernel_name()
+    xf = axo.to_f32(x, BF16).astype(np.float64)
+    n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
+    want = {"silu": n / (1 + np.exp(-n)), "sigmoid": 1 / (1 + np.exp(-n)), "tanh": np.tanh(n)}[post]
+    assert np.max(np.abs(got - want)) < 2e-2
