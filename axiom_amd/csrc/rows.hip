@@ -120,14 +120,18 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
     for (int it = 0; it < IT; ++it) {
         col0[it] = (static_cast<int64_t>(it) * GROUP + lane_in_group) * E;
         ok[it] = col0[it] < cols;
-        if (ok[it]) {
-            if constexpr (E == 1) v[it][0] = load_any(P.input, P.input_dtype, r * cols + col0[it]);
-            else load_vec<E>(P.input, P.input_dtype, r * cols + col0[it], v[it]);
-        } else {
+        // idle lanes re-read the row's first chunk, so that no load sits behind a branch and all of them are in
+        // flight together; what they read is replaced by zeros below
+        const int64_t at = r * cols + (ok[it] ? col0[it] : 0);
+        if constexpr (E == 1) v[it][0] = load_any(P.input, P.input_dtype, at);
+        else load_vec<E>(P.input, P.input_dtype, at, v[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+        if (!ok[it]) {
 #pragma unroll
             for (int e = 0; e < E; ++e) v[it][e] = 0.0f;
         }
-    }
 
     const float inv_n = 1.0f / static_cast<float>(cols);
     // stage 0: pre chain then the row op; stage 1: post chain.  One loop so the
