@@ -494,6 +494,11 @@ RowsPlan plan_rows(const AxhipRowsProgram &P) {
         pl.group = 256;
         pl.it = chunks <= 256 ? 1 : chunks <= 512 ? 2 : chunks <= 1024 ? 4 : 8;
         pl.kind = RowsPlan::RESIDENT;
+    } else if (chunks <= 1024 * 4) { // up to 64 KiB of 16-bit or 64 KiB of fp32 columns: still one read, in the registers of 1024 threads
+        pl.group = 1024;
+        pl.threads = 1024;
+        pl.it = 4;
+        pl.kind = RowsPlan::RESIDENT;
     } else {
         pl.kind = RowsPlan::STREAMED;
         pl.threads = 1024;
@@ -507,7 +512,7 @@ RowsPlan plan_rows(const AxhipRowsProgram &P) {
 
 template <int GROUP, int IT, int E>
 void launch_resident(const AxhipRowsProgram &P, hipStream_t s) {
-    constexpr int THREADS = 256;
+    constexpr int THREADS = GROUP > 256 ? GROUP : 256;
     const int64_t rows_per_block = THREADS / GROUP;
     const unsigned grid = static_cast<unsigned>((P.rows + rows_per_block - 1) / rows_per_block);
     hipLaunchKernelGGL((rows_resident_kernel<THREADS, GROUP, IT, E>), dim3(grid), dim3(THREADS), 0, s, P);
@@ -542,6 +547,10 @@ int launch_plan_e(const AxhipRowsProgram &P, const RowsPlan &pl, hipStream_t s) 
         return AXHIP_OK;
     }
     case RowsPlan::RESIDENT:
+        if (pl.group == 1024) {
+            launch_resident<1024, 4, E>(P, s);
+            return AXHIP_OK;
+        }
         return pl.group == 64 ? launch_resident_it<64, E>(P, pl.it, s) : launch_resident_it<256, E>(P, pl.it, s);
     case RowsPlan::STREAMED:
         hipLaunchKernelGGL((rows_streamed_kernel<1024, E>), dim3(static_cast<unsigned>(P.rows)), dim3(1024), 0, s, P);

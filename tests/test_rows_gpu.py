@@ -289,3 +289,27 @@ def test_fast_activations_after_a_norm_in_16_bit(post):
     n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
     want = {"silu": n / (1 + np.exp(-n)), "sigmoid": 1 / (1 + np.exp(-n)), "tanh": np.tanh(n)}[post]
     assert np.max(np.abs(got - want)) < 2e-2
+
+
+def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
+    """Rows beyond the 32 KiB the specialised kernels hold: up to 4096 16-byte chunks stay in the registers of a
+    1024-thread block (one read), longer ones are streamed in passes."""
+    g = axo.PCG64(123)
+    for cols, plan in ((12000, "rows_resident_g1024_it4_e4"), (16384, "rows_resident_g1024_it4_e4"), (20000, "rows_streamed_e4")):
+        x = (g.normal((3, cols)) * 2).astype(np.float32)
+        p = gh.Rows(x, F32).row_op("softmax")
+        got = p.run()
+        assert p.kernel_name() == plan, p.kernel_name()
+        assert close32(got, axo.softmax(x))
+    xb = axo.to_bits(g.normal((2, 30000)), BF16)
+    w, b = axo.to_bits(g.uniform((30000,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((30000,), -0.5, 0.5), BF16)
+    p = gh.Rows(xb, BF16).row_op("layernorm", 1e-5, w=w, b=b).unary("gelu")
+    got = axo.to_f32(p.run(), BF16).astype(np.float64)
+    assert p.kernel_name() == "rows_resident_g1024_it4_e8", p.kernel_name()
+    xf = axo.to_f32(xb, BF16).astype(np.float64)
+    n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
+    import math
+    want = 0.5 * n * (1 + np.vectorize(math.erf)(n / math.sqrt(2)))
+    assert np.max(np.abs(got - want)) < 2e-2
+    got = gh.Rows(x, F32).unary("square").run(reduce="mean")
+    assert np.allclose(got, (x.astype(np.float64) ** 2).mean(-1), rtol=1e-4, atol=1e-5)
