@@ -72,8 +72,15 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     };
 
     // pre chain
+    bool pre_is_post = false;
     if (P.n_pre == 0) {
         k.pre = RP_NONE;
+    } else if (P.n_pre == 1 && P.row_op == AXHIP_ROWOP_NONE && P.reduce != AXHIP_RED_NONE && P.n_post == 0 &&
+               P.pre[0].op >= AXHIP_OP_RELU && P.pre[0].op <= AXHIP_OP_RECIP) {
+        // one unary op, then a row reduction (sum(relu(x)), mean(x^2), max(abs(x))): with no row op in between the
+        // op can run where the post op does, right before the accumulation
+        k.pre = RP_NONE;
+        pre_is_post = true;
     } else if (P.n_pre == 1 && P.pre[0].op == AXHIP_OP_ADD && P.pre[0].imm_kind != AXHIP_BK_IMM &&
                P.pre[0].operand >= 0 && P.pre[0].operand < P.n_operands && P.operands[P.pre[0].operand].kind == AXHIP_BK_FULL) {
         a.f = vector_operand(P.pre[0].operand, AXHIP_BK_FULL);
@@ -119,7 +126,8 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     }
 
     // post chain: nothing or one unary op
-    if (P.n_post == 1 && P.post[0].op >= AXHIP_OP_RELU && P.post[0].op <= AXHIP_OP_RECIP) a.post_op = P.post[0].op;
+    if (pre_is_post) a.post_op = P.pre[0].op;
+    else if (P.n_post == 1 && P.post[0].op >= AXHIP_OP_RELU && P.post[0].op <= AXHIP_OP_RECIP) a.post_op = P.post[0].op;
     else if (P.n_post != 0) return false;
 
     k.reduce = P.reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : P.reduce;

@@ -313,3 +313,28 @@ def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
     assert np.max(np.abs(got - want)) < 2e-2
     got = gh.Rows(x, F32).unary("square").run(reduce="mean")
     assert np.allclose(got, (x.astype(np.float64) ** 2).mean(-1), rtol=1e-4, atol=1e-5)
+
+
+def test_unary_then_row_reduction_runs_on_the_specialised_reduce_kernels():
+    g = axo.PCG64(321)
+    x = (g.normal((37, 4096)) * 2).astype(np.float32)
+    xb = axo.to_bits(x, BF16)
+    xbf = axo.to_f32(xb, BF16).astype(np.float64)
+    p = gh.Rows(x, F32).unary("relu")
+    got = p.run(reduce="sum")
+    assert p.kernel_name().startswith("rows_static_reduce_sum_f32"), p.kernel_name()
+    assert np.allclose(got, np.maximum(x.astype(np.float64), 0).sum(-1), rtol=1e-4, atol=1e-3)
+    p = gh.Rows(xb, BF16, F32).unary("square")
+    got = p.run(reduce="mean")
+    assert p.kernel_name().startswith("rows_static_reduce_sum_bf16"), p.kernel_name()
+    assert np.allclose(got, (xbf * xbf).mean(-1), rtol=1e-4, atol=1e-5)
+    p = gh.Rows(xb, BF16).unary("abs")
+    got = axo.to_f32(p.run(reduce="max"), BF16)
+    assert p.kernel_name().startswith("rows_static_reduce_max_bf16"), p.kernel_name()
+    assert np.array_equal(got.reshape(-1), np.abs(xbf).max(-1).astype(np.float32))
+    # an fp32 result keeps the exact activation (no polynomial GELU under a sum)
+    import math
+    p = gh.Rows(xb, BF16, F32).unary("gelu")
+    got = p.run(reduce="sum")
+    want = (0.5 * xbf * (1 + np.vectorize(math.erf)(xbf / math.sqrt(2)))).sum(-1)
+    assert np.allclose(got.reshape(-1), want, rtol=1e-4, atol=2e-3)
