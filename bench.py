@@ -37,21 +37,24 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the SDPA kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, each scaled by the reading of the plain-copy leg below
-# (FETCH_SIZE 0.50009, WRITE_SIZE 1.0): 561.7 MB read + 134.2 MB written.
-SDPA_TRAFFIC_BYTES = 695.9e6
+# (FETCH_SIZE 0.50012, WRITE_SIZE 1.0): 585.2 MB read + 134.2 MB written.
+SDPA_TRAFFIC_BYTES = 719.5e6
 # same measurement for the fused chains: they move the algorithmic bytes (ratio 1.001 - 1.003)
 CHAIN_TRAFFIC_BYTES = {"chain_relu_add_mul_softmax_sum_f32_8192x8192": 537.2e6,
-                       "chain_gelu_layernorm_bf16_16384x4096": 269.4e6,
+                       "chain_gelu_layernorm_bf16_16384x4096": 269.1e6,
                        "chain_gelu_rmsnorm_bf16_16384x4096": 269.2e6}
 
 
-MIN_WARMUP_MS = 100.0  # clocks and power settle within about this much work of one kind
+MIN_WARMUP_MS = 100.0  # clocks and power settle within about this much work of one kind ...
+MAX_SETTLE_MS = 1500.0  # ... but a leg that follows a very different one can take longer: see time_launches
 
 
 def time_launches(torch, stream, launch, steps: int, warmup: int):
     """Average launch duration in ms over `steps` launches, HIP events on `stream`.
     Warm-up: `warmup` launches, continued until MIN_WARMUP_MS of work has run (short kernels
-    would otherwise be timed while the device is still changing clocks)."""
+    would otherwise be timed while the device is still changing clocks), then batches of launches
+    until two consecutive batches agree within 1 % (at most MAX_SETTLE_MS): the figure is the steady
+    state of this kernel, not the tail of the previous leg's power state."""
     with torch.cuda.stream(stream):
         t0 = time.time()
         for _ in range(warmup):
@@ -62,6 +65,21 @@ def time_launches(torch, stream, launch, steps: int, warmup: int):
             for _ in range(int((MIN_WARMUP_MS - spent_ms) / (spent_ms / warmup)) + 1):
                 launch()
             stream.synchronize()
+        if warmup > 0:
+            batch = max(10, warmup)
+            prev, agree, settle_t0 = None, 0, time.time()
+            while (time.time() - settle_t0) * 1e3 < MAX_SETTLE_MS:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(batch):
+                    launch()
+                e1.record(stream)
+                stream.synchronize()
+                t = e0.elapsed_time(e1)
+                agree = agree + 1 if prev is not None and abs(t - prev) <= 0.01 * prev else 0
+                prev = t
+                if agree >= 2:
+                    break
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         evs[0].record(stream)
         for i in range(steps):
