@@ -18,7 +18,7 @@ bool has_pattern(int pre, int row_op, int reduce) {
 }
 
 const char *pre_name(int pre) {
-    return pre == RP_NONE ? "" : pre == RP_ADDF ? "addf_" : pre == RP_MULS ? "muls_" : pre == RP_MULS_ADDF ? "muls_addf_" : "relu_adds_mulf_";
+    return pre == RP_NONE ? "" : pre == RP_ADDF ? "addf_" : pre == RP_MULS ? "muls_" : pre == RP_MULS_ADDF ? "muls_addf_" : pre == RP_MULF ? "mulf_" : "relu_adds_mulf_";
 }
 const char *rowop_name(int r) {
     switch (r) {
@@ -86,6 +86,11 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
         a.f = vector_operand(P.pre[0].operand, AXHIP_BK_FULL);
         if (!a.f) return false;
         k.pre = RP_ADDF;
+    } else if (P.n_pre == 1 && P.pre[0].op == AXHIP_OP_MUL && P.pre[0].imm_kind != AXHIP_BK_IMM && P.pre[0].operand >= 0 &&
+               P.pre[0].operand < P.n_operands && P.operands[P.pre[0].operand].kind == AXHIP_BK_FULL) { // x * y: the row dot product
+        a.f = vector_operand(P.pre[0].operand, AXHIP_BK_FULL);
+        if (!a.f) return false;
+        k.pre = RP_MULF;
     } else if (P.n_pre == 1 && P.pre[0].op == AXHIP_OP_MUL) { // x * s: the scaled softmax
         if (!scalar_of(P.pre[0])) return false;
         k.pre = RP_MULS;

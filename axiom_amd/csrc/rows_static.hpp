@@ -18,7 +18,7 @@
 
 namespace axhip {
 
-enum RowsPre { RP_NONE = 0, RP_ADDF = 1, RP_RELU_ADDS_MULF = 2, RP_MULS = 3, RP_MULS_ADDF = 4 }; // F: full-size operand, S: scalar
+enum RowsPre { RP_NONE = 0, RP_ADDF = 1, RP_RELU_ADDS_MULF = 2, RP_MULS = 3, RP_MULS_ADDF = 4, RP_MULF = 5 }; // F: full-size operand, S: scalar
 
 struct RowsStaticArgs {
     const void *x;      // [rows, cols]
@@ -58,6 +58,8 @@ struct RowsStaticKey {
     X(RP_NONE, AXHIP_ROWOP_RMSNORM, AXHIP_RED_NONE)            \
     X(RP_ADDF, AXHIP_ROWOP_RMSNORM, AXHIP_RED_NONE)            \
     X(RP_NONE, AXHIP_ROWOP_NONE, AXHIP_RED_SUM)                \
+    X(RP_ADDF, AXHIP_ROWOP_NONE, AXHIP_RED_SUM)                \
+    X(RP_MULF, AXHIP_ROWOP_NONE, AXHIP_RED_SUM)                \
     X(RP_NONE, AXHIP_ROWOP_NONE, AXHIP_RED_MAX)                \
     X(RP_NONE, AXHIP_ROWOP_NONE, AXHIP_RED_MIN)
 

@@ -338,3 +338,23 @@ def test_unary_then_row_reduction_runs_on_the_specialised_reduce_kernels():
     got = p.run(reduce="sum")
     want = (0.5 * xbf * (1 + np.vectorize(math.erf)(xbf / math.sqrt(2)))).sum(-1)
     assert np.allclose(got.reshape(-1), want, rtol=1e-4, atol=2e-3)
+
+
+def test_sum_of_a_sum_and_row_dot_product_on_the_specialised_kernels():
+    # tests/test_fusion_extended.cpp:346-352: sum(a + b) over 1s and 3s
+    a, b = np.full((4, 2048), 1.0, np.float32), np.full((4, 2048), 3.0, np.float32)
+    p = gh.Rows(a, F32).binary("add", b)
+    got = p.run(reduce="sum")
+    assert p.kernel_name().startswith("rows_static_addf_reduce_sum_f32"), p.kernel_name()
+    assert np.all(got == 4.0 * 2048)
+    g = axo.PCG64(55)
+    x, y = g.normal((21, 4096)).astype(np.float32), g.normal((21, 4096)).astype(np.float32)
+    p = gh.Rows(x, F32).binary("mul", y)
+    got = p.run(reduce="sum")
+    assert p.kernel_name().startswith("rows_static_mulf_reduce_sum_f32"), p.kernel_name()
+    assert np.allclose(got.reshape(-1), (x.astype(np.float64) * y).sum(-1), rtol=1e-4, atol=1e-3)
+    xb, yb = axo.to_bits(x, BF16), axo.to_bits(y, BF16)
+    p = gh.Rows(xb, BF16, F32).binary("mul", yb)
+    got = p.run(reduce="mean")
+    assert p.kernel_name().startswith("rows_static_mulf_reduce_sum_bf16"), p.kernel_name()
+    assert np.allclose(got.reshape(-1), (axo.to_f32(xb, BF16).astype(np.float64) * axo.to_f32(yb, BF16)).mean(-1), rtol=1e-4, atol=1e-5)
