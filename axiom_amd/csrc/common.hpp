@@ -135,15 +135,45 @@ __device__ __forceinline__ float gelu_fast(float x) {
     return x * phi;
 }
 
-// Load / store N consecutive elements (N*sizeof(elem) is 16 or 32 bytes and the
+// Vector accesses at element alignment only (rows of odd length): the same 16-byte instructions, which the
+// hardware executes at any alignment; the packed types tell the compiler not to assume more.
+struct __attribute__((packed, aligned(4))) float4_unaligned_t { float4_t v; };
+struct __attribute__((packed, aligned(2))) uint4_unaligned_t { uint4_t v; };
+struct __attribute__((packed, aligned(2))) uint2_unaligned_t { uint2_t v; };
+template <bool UNALIGNED> __device__ __forceinline__ float4_t vec_load(const float4_t *p) {
+    if constexpr (UNALIGNED) return reinterpret_cast<const float4_unaligned_t *>(p)->v;
+    else return *p;
+}
+template <bool UNALIGNED> __device__ __forceinline__ uint4_t vec_load(const uint4_t *p) {
+    if constexpr (UNALIGNED) return reinterpret_cast<const uint4_unaligned_t *>(p)->v;
+    else return *p;
+}
+template <bool UNALIGNED> __device__ __forceinline__ uint2_t vec_load(const uint2_t *p) {
+    if constexpr (UNALIGNED) return reinterpret_cast<const uint2_unaligned_t *>(p)->v;
+    else return *p;
+}
+template <bool UNALIGNED> __device__ __forceinline__ void vec_store(float4_t *p, float4_t t) {
+    if constexpr (UNALIGNED) reinterpret_cast<float4_unaligned_t *>(p)->v = t;
+    else *p = t;
+}
+template <bool UNALIGNED> __device__ __forceinline__ void vec_store(uint4_t *p, uint4_t t) {
+    if constexpr (UNALIGNED) reinterpret_cast<uint4_unaligned_t *>(p)->v = t;
+    else *p = t;
+}
+template <bool UNALIGNED> __device__ __forceinline__ void vec_store(uint2_t *p, uint2_t t) {
+    if constexpr (UNALIGNED) reinterpret_cast<uint2_unaligned_t *>(p)->v = t;
+    else *p = t;
+}
+
+// Load / store N consecutive elements (N*sizeof(elem) is 16 or 32 bytes and, unless UNALIGNED, the
 // address is aligned to min(16, that)) as fp32 values.
-template <int N>
+template <int N, bool UNALIGNED = false>
 __device__ __forceinline__ void load_vec(const void *p, int dt, int64_t i, float (&v)[N]) {
     if (dt == AXHIP_DTYPE_F32) {
         const float4_t *q = reinterpret_cast<const float4_t *>(static_cast<const float *>(p) + i);
 #pragma unroll
         for (int j = 0; j < N / 4; ++j) {
-            float4_t t = q[j];
+            float4_t t = vec_load<UNALIGNED>(q + j);
             v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w;
         }
     } else {
@@ -152,7 +182,7 @@ __device__ __forceinline__ void load_vec(const void *p, int dt, int64_t i, float
             const uint4_t *q = reinterpret_cast<const uint4_t *>(static_cast<const uint16_t *>(p) + i);
 #pragma unroll
             for (int j = 0; j < N / 8; ++j) {
-                uint4_t t = q[j];
+                uint4_t t = vec_load<UNALIGNED>(q + j);
                 uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -167,7 +197,7 @@ __device__ __forceinline__ void load_vec(const void *p, int dt, int64_t i, float
             }
         } else {
             const uint2_t *q = reinterpret_cast<const uint2_t *>(static_cast<const uint16_t *>(p) + i);
-            uint2_t t = q[0];
+            uint2_t t = vec_load<UNALIGNED>(q);
             uint32_t w[2] = {t.x, t.y};
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
@@ -191,7 +221,7 @@ __device__ __forceinline__ void store16_streaming(void *p, uint4_t v) {
 
 // `streaming`: non-temporal stores, for outputs far larger than the caches (they then do not
 // push the inputs of the same launch out of the last-level cache)
-template <int N>
+template <int N, bool UNALIGNED = false>
 __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const float (&v)[N], bool streaming = false) {
     if (dt == AXHIP_DTYPE_F32) {
         float4_t *q = reinterpret_cast<float4_t *>(static_cast<float *>(p) + i);
@@ -199,7 +229,7 @@ __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const floa
         for (int j = 0; j < N / 4; ++j) {
             float4_t t = {v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
             if (streaming) store16_streaming(&q[j], __builtin_bit_cast(uint4_t, t));
-            else q[j] = t;
+            else vec_store<UNALIGNED>(q + j, t);
         }
     } else {
         uint32_t w[N / 2];
@@ -217,12 +247,12 @@ __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const floa
             for (int j = 0; j < N / 8; ++j) {
                 uint4_t t = {w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
                 if (streaming) store16_streaming(&q[j], t);
-                else q[j] = t;
+                else vec_store<UNALIGNED>(q + j, t);
             }
         } else {
             uint2_t *q = reinterpret_cast<uint2_t *>(static_cast<uint16_t *>(p) + i);
             uint2_t t = {w[0], w[1]};
-            q[0] = t;
+            vec_store<UNALIGNED>(q, t);
         }
     }
 }

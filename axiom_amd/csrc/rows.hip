@@ -16,14 +16,23 @@
 namespace axhip {
 
 
-// Loads the [IT][E] tile of a FULL or ROWVEC operand.
-template <int IT, int E>
+// Loads the [IT][E] tile of a FULL or ROWVEC operand.  RAGGED (rows whose length is not a multiple of E, or whose
+// start is not vector-aligned): nv[it] counts the chunk's valid elements; whole chunks use unaligned vector loads,
+// the row's last, partial chunk is read element by element.
+template <int IT, int E, bool RAGGED = false>
 __device__ __forceinline__ void load_operand_tile(const AxhipOperand &o, const AxhipRowsProgram &P, int64_t row,
-                                                  const int64_t (&col0)[IT], const bool (&ok)[IT], float (&w)[IT][E]) {
+                                                  const int64_t (&col0)[IT], const bool (&ok)[IT], float (&w)[IT][E], const int *nv = nullptr) {
     const int64_t base = o.kind == AXHIP_BK_FULL ? row * P.cols : 0;
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
-        if (ok[it]) {
+        if constexpr (RAGGED) {
+            if (nv[it] == E) {
+                load_vec<E, true>(o.ptr, o.dtype, base + col0[it], w[it]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) w[it][e] = e < nv[it] ? load_any(o.ptr, o.dtype, base + col0[it] + e) : 1.0f;
+            }
+        } else if (ok[it]) {
             if constexpr (E == 1) w[it][0] = load_any(o.ptr, o.dtype, base + col0[it]);
             else load_vec<E>(o.ptr, o.dtype, base + col0[it], w[it]);
         } else {
@@ -33,9 +42,9 @@ __device__ __forceinline__ void load_operand_tile(const AxhipOperand &o, const A
     }
 }
 
-template <int IT, int E>
+template <int IT, int E, bool RAGGED = false>
 __device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsProgram &P, float (&v)[IT][E],
-                                         int64_t row, const int64_t (&col0)[IT], const bool (&ok)[IT]) {
+                                         int64_t row, const int64_t (&col0)[IT], const bool (&ok)[IT], const int *nv = nullptr) {
     if (!is_binary_op(c.op)) {
         // results that are rounded to a 16-bit type do not need erff / expf / IEEE division: the polynomial
         // GELU (|error| <= 5e-5) and fast-exponential forms are far below the output resolution and keep
@@ -64,16 +73,16 @@ __device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsP
         return;
     }
     float w[IT][E];
-    load_operand_tile<IT, E>(o, P, row, col0, ok, w);
+    load_operand_tile<IT, E, RAGGED>(o, P, row, col0, ok, w, nv);
     apply_binary_tile<IT, E>(c.op, v, [&](int it, int e) { return w[it][e]; });
 }
 
 // norm weight / bias: v = v * w  or  v = v + b with a ROWVEC operand
-template <int IT, int E, bool MUL>
+template <int IT, int E, bool MUL, bool RAGGED = false>
 __device__ __forceinline__ void apply_affine(int operand, const AxhipRowsProgram &P, float (&v)[IT][E], int64_t row,
-                                             const int64_t (&col0)[IT], const bool (&ok)[IT]) {
+                                             const int64_t (&col0)[IT], const bool (&ok)[IT], const int *nv = nullptr) {
     float w[IT][E];
-    load_operand_tile<IT, E>(P.operands[operand], P, row, col0, ok, w);
+    load_operand_tile<IT, E, RAGGED>(P.operands[operand], P, row, col0, ok, w, nv);
 #pragma unroll
     for (int it = 0; it < IT; ++it)
 #pragma unroll
@@ -103,7 +112,7 @@ __device__ __forceinline__ float group_reduce(float x, float *lds) {
 }
 
 // One row per GROUP threads, the whole row resident in registers.
-template <int THREADS, int GROUP, int IT, int E>
+template <int THREADS, int GROUP, int IT, int E, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsProgram P) {
     __shared__ float lds[THREADS / WAVE];
     constexpr int ROWS_PER_BLOCK = THREADS / GROUP;
@@ -116,15 +125,28 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
     float v[IT][E];
     int64_t col0[IT];
     bool ok[IT];
+    int nv[IT]; // valid elements of the chunk: E, 0 past the end of the row, in between only for a RAGGED row's last chunk
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
         col0[it] = (static_cast<int64_t>(it) * GROUP + lane_in_group) * E;
         ok[it] = col0[it] < cols;
+        const int64_t left = cols - col0[it];
+        nv[it] = left >= E ? E : left > 0 ? static_cast<int>(left) : 0;
         // idle lanes re-read the row's first chunk, so that no load sits behind a branch and all of them are in
         // flight together; what they read is replaced by zeros below
         const int64_t at = r * cols + (ok[it] ? col0[it] : 0);
-        if constexpr (E == 1) v[it][0] = load_any(P.input, P.input_dtype, at);
-        else load_vec<E>(P.input, P.input_dtype, at, v[it]);
+        if constexpr (E == 1) {
+            v[it][0] = load_any(P.input, P.input_dtype, at);
+        } else if constexpr (RAGGED) {
+            if (nv[it] == E || nv[it] == 0) {
+                load_vec<E, true>(P.input, P.input_dtype, at, v[it]); // cols >= E: the first chunk is whole
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[it][e] = e < nv[it] ? load_any(P.input, P.input_dtype, at + e) : 0.0f;
+            }
+        } else {
+            load_vec<E>(P.input, P.input_dtype, at, v[it]);
+        }
     }
 #pragma unroll
     for (int it = 0; it < IT; ++it)
@@ -132,6 +154,8 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
 #pragma unroll
             for (int e = 0; e < E; ++e) v[it][e] = 0.0f;
         }
+    // is element e of chunk it part of the row
+    auto valid = [&](int it, int e) { return RAGGED ? e < nv[it] : ok[it]; };
 
     const float inv_n = 1.0f / static_cast<float>(cols);
     // stage 0: pre chain then the row op; stage 1: post chain.  One loop so the
@@ -139,15 +163,15 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
 #pragma nounroll
     for (int stage = 0; stage < 2; ++stage) {
     const int n_ops = stage == 0 ? P.n_pre : P.n_post;
-    for (int i = 0; i < n_ops; ++i) apply_op<IT, E>(stage == 0 ? P.pre[i] : P.post[i], P, v, r, col0, ok);
+    for (int i = 0; i < n_ops; ++i) apply_op<IT, E, RAGGED>(stage == 0 ? P.pre[i] : P.post[i], P, v, r, col0, ok, nv);
     if (stage == 1) break;
     if (P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX) {
         float m = NEG_INF;
 #pragma unroll
         for (int it = 0; it < IT; ++it)
-            if (ok[it])
 #pragma unroll
-                for (int e = 0; e < E; ++e) m = fmaxf(m, v[it][e]);
+            for (int e = 0; e < E; ++e)
+                if (valid(it, e)) m = fmaxf(m, v[it][e]);
         m = group_reduce<GROUP, THREADS, 1>(m, lds);
         const float mm = m == NEG_INF ? 0.0f : m;
         float s = 0.0f;
@@ -156,7 +180,7 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
             for (int it = 0; it < IT; ++it)
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
-                    v[it][e] = ok[it] ? __expf(v[it][e] - mm) : 0.0f;
+                    v[it][e] = valid(it, e) ? __expf(v[it][e] - mm) : 0.0f;
                     s += v[it][e];
                 }
             s = group_reduce<GROUP, THREADS, 0>(s, lds);
@@ -169,7 +193,7 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
 #pragma unroll
             for (int it = 0; it < IT; ++it)
 #pragma unroll
-                for (int e = 0; e < E; ++e) s += ok[it] ? __expf(v[it][e] - mm) : 0.0f;
+                for (int e = 0; e < E; ++e) s += valid(it, e) ? __expf(v[it][e] - mm) : 0.0f;
             s = group_reduce<GROUP, THREADS, 0>(s, lds);
             const float ls = __logf(s) + mm;
 #pragma unroll
@@ -183,17 +207,17 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
             float s = 0.0f;
 #pragma unroll
             for (int it = 0; it < IT; ++it)
-                if (ok[it])
 #pragma unroll
-                    for (int e = 0; e < E; ++e) s += v[it][e];
+                for (int e = 0; e < E; ++e)
+                    if (valid(it, e)) s += v[it][e];
             mean = group_reduce<GROUP, THREADS, 0>(s, lds) * inv_n;
         }
         float q = 0.0f;
 #pragma unroll
         for (int it = 0; it < IT; ++it)
-            if (ok[it])
 #pragma unroll
-                for (int e = 0; e < E; ++e) {
+            for (int e = 0; e < E; ++e)
+                if (valid(it, e)) {
                     v[it][e] -= mean;
                     q += v[it][e] * v[it][e];
                 }
@@ -203,8 +227,8 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
         for (int it = 0; it < IT; ++it)
 #pragma unroll
             for (int e = 0; e < E; ++e) v[it][e] *= rstd;
-        if (P.norm_weight >= 0) apply_affine<IT, E, true>(P.norm_weight, P, v, r, col0, ok);
-        if (P.norm_bias >= 0) apply_affine<IT, E, false>(P.norm_bias, P, v, r, col0, ok);
+        if (P.norm_weight >= 0) apply_affine<IT, E, true, RAGGED>(P.norm_weight, P, v, r, col0, ok, nv);
+        if (P.norm_bias >= 0) apply_affine<IT, E, false, RAGGED>(P.norm_bias, P, v, r, col0, ok, nv);
     }
 
     } // stage loop
@@ -214,8 +238,19 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
 #pragma unroll
             for (int it = 0; it < IT; ++it)
                 if (ok[it]) {
-                    if constexpr (E == 1) store_any(P.output, P.output_dtype, r * cols + col0[it], v[it][0]);
-                    else store_vec<E>(P.output, P.output_dtype, r * cols + col0[it], v[it]);
+                    if constexpr (E == 1) {
+                        store_any(P.output, P.output_dtype, r * cols + col0[it], v[it][0]);
+                    } else if constexpr (RAGGED) {
+                        if (nv[it] == E) {
+                            store_vec<E, true>(P.output, P.output_dtype, r * cols + col0[it], v[it]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < E; ++e)
+                                if (e < nv[it]) store_any(P.output, P.output_dtype, r * cols + col0[it] + e, v[it][e]);
+                        }
+                    } else {
+                        store_vec<E>(P.output, P.output_dtype, r * cols + col0[it], v[it]);
+                    }
                 }
         }
         return;
@@ -225,26 +260,26 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
         acc = 0.0f;
 #pragma unroll
         for (int it = 0; it < IT; ++it)
-            if (ok[it])
 #pragma unroll
-                for (int e = 0; e < E; ++e) acc += v[it][e];
+            for (int e = 0; e < E; ++e)
+                if (valid(it, e)) acc += v[it][e];
         acc = group_reduce<GROUP, THREADS, 0>(acc, lds);
         if (P.reduce == AXHIP_RED_MEAN) acc *= inv_n;
     } else if (P.reduce == AXHIP_RED_MAX) {
         acc = NEG_INF;
 #pragma unroll
         for (int it = 0; it < IT; ++it)
-            if (ok[it])
 #pragma unroll
-                for (int e = 0; e < E; ++e) acc = fmaxf(acc, v[it][e]);
+            for (int e = 0; e < E; ++e)
+                if (valid(it, e)) acc = fmaxf(acc, v[it][e]);
         acc = group_reduce<GROUP, THREADS, 1>(acc, lds);
     } else {
         acc = POS_INF;
 #pragma unroll
         for (int it = 0; it < IT; ++it)
-            if (ok[it])
 #pragma unroll
-                for (int e = 0; e < E; ++e) acc = fminf(acc, v[it][e]);
+            for (int e = 0; e < E; ++e)
+                if (valid(it, e)) acc = fminf(acc, v[it][e]);
         acc = group_reduce<GROUP, THREADS, 2>(acc, lds);
     }
     if (row_ok && lane_in_group == 0) store_any(P.output, P.output_dtype, r, acc);
@@ -467,6 +502,7 @@ int validate_program(const AxhipRowsProgram &P, const char *who) {
 struct RowsPlan {
     enum Kind { EMPTY, ELEMENTWISE, RESIDENT, STREAMED } kind;
     int e, it, group, threads;
+    bool ragged; // resident plan on rows that are not whole, aligned vectors: unaligned accesses, element-wise last chunk
     char name[64];
 };
 
@@ -483,6 +519,13 @@ RowsPlan plan_rows(const AxhipRowsProgram &P) {
         pl.threads = 256;
         snprintf(pl.name, sizeof(pl.name), "elementwise_e%d", pl.e);
         return pl;
+    }
+    // rows of odd length or alignment: keep the full vector width (the hardware takes 16-byte accesses at element
+    // alignment) and treat the row's last, partial chunk element by element, as long as the row fits a resident plan
+    const int natural = P.input_dtype != AXHIP_DTYPE_F32 ? 8 : 4;
+    if (pl.e == 1 && P.cols >= natural && (P.cols + natural - 1) / natural <= 1024 * 4) { // (a narrower aligned vector, when one fits, measured faster)
+        pl.e = natural;
+        pl.ragged = true;
     }
     const int64_t chunks = (P.cols + pl.e - 1) / pl.e;
     pl.threads = 256;
@@ -505,28 +548,34 @@ RowsPlan plan_rows(const AxhipRowsProgram &P) {
         pl.group = 1024;
         pl.it = 0;
     }
-    if (pl.kind == RowsPlan::RESIDENT) snprintf(pl.name, sizeof(pl.name), "rows_resident_g%d_it%d_e%d", pl.group, pl.it, pl.e);
+    if (pl.kind == RowsPlan::RESIDENT) snprintf(pl.name, sizeof(pl.name), "rows_resident_g%d_it%d_e%d%s", pl.group, pl.it, pl.e, pl.ragged ? "_ragged" : "");
     else snprintf(pl.name, sizeof(pl.name), "rows_streamed_e%d", pl.e);
     return pl;
 }
 
 template <int GROUP, int IT, int E>
-void launch_resident(const AxhipRowsProgram &P, hipStream_t s) {
+void launch_resident(const AxhipRowsProgram &P, bool ragged, hipStream_t s) {
     constexpr int THREADS = GROUP > 256 ? GROUP : 256;
     const int64_t rows_per_block = THREADS / GROUP;
     const unsigned grid = static_cast<unsigned>((P.rows + rows_per_block - 1) / rows_per_block);
-    hipLaunchKernelGGL((rows_resident_kernel<THREADS, GROUP, IT, E>), dim3(grid), dim3(THREADS), 0, s, P);
+    if constexpr (E > 1) {
+        if (ragged) {
+            hipLaunchKernelGGL((rows_resident_kernel<THREADS, GROUP, IT, E, true>), dim3(grid), dim3(THREADS), 0, s, P);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((rows_resident_kernel<THREADS, GROUP, IT, E, false>), dim3(grid), dim3(THREADS), 0, s, P);
 }
 
 template <int GROUP, int E>
-int launch_resident_it(const AxhipRowsProgram &P, int it, hipStream_t s) {
+int launch_resident_it(const AxhipRowsProgram &P, int it, bool ragged, hipStream_t s) {
     switch (it) {
-    case 1: launch_resident<GROUP, 1, E>(P, s); return AXHIP_OK;
-    case 2: launch_resident<GROUP, 2, E>(P, s); return AXHIP_OK;
-    case 4: launch_resident<GROUP, 4, E>(P, s); return AXHIP_OK;
+    case 1: launch_resident<GROUP, 1, E>(P, ragged, s); return AXHIP_OK;
+    case 2: launch_resident<GROUP, 2, E>(P, ragged, s); return AXHIP_OK;
+    case 4: launch_resident<GROUP, 4, E>(P, ragged, s); return AXHIP_OK;
     case 8:
         if constexpr (GROUP == 256) {
-            launch_resident<GROUP, 8, E>(P, s);
+            launch_resident<GROUP, 8, E>(P, ragged, s);
             return AXHIP_OK;
         }
         [[fallthrough]];
@@ -548,10 +597,10 @@ int launch_plan_e(const AxhipRowsProgram &P, const RowsPlan &pl, hipStream_t s) 
     }
     case RowsPlan::RESIDENT:
         if (pl.group == 1024) {
-            launch_resident<1024, 4, E>(P, s);
+            launch_resident<1024, 4, E>(P, pl.ragged, s);
             return AXHIP_OK;
         }
-        return pl.group == 64 ? launch_resident_it<64, E>(P, pl.it, s) : launch_resident_it<256, E>(P, pl.it, s);
+        return pl.group == 64 ? launch_resident_it<64, E>(P, pl.it, pl.ragged, s) : launch_resident_it<256, E>(P, pl.it, pl.ragged, s);
     case RowsPlan::STREAMED:
         hipLaunchKernelGGL((rows_streamed_kernel<1024, E>), dim3(static_cast<unsigned>(P.rows)), dim3(1024), 0, s, P);
         return AXHIP_OK;

@@ -358,3 +358,37 @@ def test_sum_of_a_sum_and_row_dot_product_on_the_specialised_kernels():
     got = p.run(reduce="mean")
     assert p.kernel_name().startswith("rows_static_mulf_reduce_sum_bf16"), p.kernel_name()
     assert np.allclose(got.reshape(-1), (axo.to_f32(xb, BF16).astype(np.float64) * axo.to_f32(yb, BF16)).mean(-1), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_rows_of_odd_length_on_the_ragged_resident_plan(dt):
+    """Column counts that no aligned vector divides (4097, 1001, 77): full-width unaligned accesses plus an
+    element-wise last chunk; softmax, layer norm with weight and bias, a full-size operand, a row reduction."""
+    g = axo.PCG64(808)
+    for cols in (77, 1001, 4097):
+        x, y = g.normal((11, cols)) * 2, g.normal((11, cols))
+        w, b = g.uniform((cols,), 0.5, 1.5), g.uniform((cols,), -0.5, 0.5)
+        if dt == F32:
+            xs, ys, ws, bs = (t.astype(np.float32) for t in (x, y, w, b))
+            f = lambda t: t.astype(np.float64)
+            out = lambda t: t.astype(np.float64)
+        else:
+            xs, ys, ws, bs = (axo.to_bits(t, dt) for t in (x, y, w, b))
+            f = lambda t: axo.to_f32(t, dt).astype(np.float64)
+            out = lambda t: axo.to_f32(t, dt).astype(np.float64)
+        tol = 1e-4 if dt == F32 else 2e-2
+        p = gh.Rows(xs, dt).binary("add", ys).row_op("softmax")
+        got = out(p.run())
+        assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+        lg = f(xs) + f(ys)
+        e = np.exp(lg - lg.max(-1, keepdims=True))
+        assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
+        p = gh.Rows(xs, dt).row_op("layernorm", 1e-5, w=ws, b=bs).unary("relu")
+        got = out(p.run())
+        assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+        xf = f(xs)
+        n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * f(ws) + f(bs)
+        assert np.max(np.abs(got - np.maximum(n, 0))) < tol * (1 if dt == F32 else 2)
+        p = gh.Rows(xs, dt, F32).unary("square")
+        got = p.run(reduce="sum")
+        assert np.allclose(got.reshape(-1), (xf * xf).sum(-1), rtol=1e-4, atol=1e-3)
