@@ -42,7 +42,7 @@ __device__ __forceinline__ void load_operand_tile(const AxhipOperand &o, const A
     }
 }
 
-template <int IT, int E, bool RAGGED = false>
+template <int IT, int E, bool RAGGED = false, bool GROUPS = true>
 __device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsProgram &P, float (&v)[IT][E],
                                          int64_t row, const int64_t (&col0)[IT], const bool (&ok)[IT], const int *nv = nullptr) {
     if (!is_binary_op(c.op)) {
@@ -58,23 +58,23 @@ __device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsP
             default: break;
             }
         }
-        apply_unary_tile<IT, E>(c.op, v);
+        apply_unary_tile<IT, E, GROUPS>(c.op, v);
         return;
     }
     if (c.imm_kind == AXHIP_BK_IMM) {
         const float s = c.imm;
-        apply_binary_tile<IT, E>(c.op, v, [&](int, int) { return s; });
+        apply_binary_tile<IT, E, GROUPS>(c.op, v, [&](int, int) { return s; });
         return;
     }
     const AxhipOperand &o = P.operands[c.operand];
     if (o.kind == AXHIP_BK_SCALAR || o.kind == AXHIP_BK_COLVEC) {
         const float s = load_any(o.ptr, o.dtype, o.kind == AXHIP_BK_SCALAR ? 0 : row);
-        apply_binary_tile<IT, E>(c.op, v, [&](int, int) { return s; });
+        apply_binary_tile<IT, E, GROUPS>(c.op, v, [&](int, int) { return s; });
         return;
     }
     float w[IT][E];
     load_operand_tile<IT, E, RAGGED>(o, P, row, col0, ok, w, nv);
-    apply_binary_tile<IT, E>(c.op, v, [&](int it, int e) { return w[it][e]; });
+    apply_binary_tile<IT, E, GROUPS>(c.op, v, [&](int it, int e) { return w[it][e]; });
 }
 
 // norm weight / bias: v = v * w  or  v = v + b with a ROWVEC operand
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
 #pragma nounroll
     for (int stage = 0; stage < 2; ++stage) {
     const int n_ops = stage == 0 ? P.n_pre : P.n_post;
-    for (int i = 0; i < n_ops; ++i) apply_op<IT, E, RAGGED>(stage == 0 ? P.pre[i] : P.post[i], P, v, r, col0, ok, nv);
+    for (int i = 0; i < n_ops; ++i) apply_op<IT, E, RAGGED, (THREADS < 1024)>(stage == 0 ? P.pre[i] : P.post[i], P, v, r, col0, ok, nv);
     if (stage == 1) break;
     if (P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX) {
         float m = NEG_INF;

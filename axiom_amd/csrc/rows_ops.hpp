@@ -59,46 +59,67 @@ __device__ __forceinline__ void for_each_value(float (&v)[IT][E], F f) {
         for (int e = 0; e < E; ++e) v[it][e] = f(v[it][e], it, e);
 }
 
-template <int IT, int E>
+// The same for the long-running functions (erff, expf, IEEE division ...): four values at a time, with a scheduling
+// barrier between the groups.  Left to itself the scheduler interleaves all IT * E evaluations, and the
+// temporaries of that one arm then set the register count of the whole kernel.  GROUPS = false (the 1024-thread
+// kernels, whose register file share is fixed at 128 by the block size) keeps the free schedule.
+template <int IT, int E, bool GROUPS, typename F>
+__device__ __forceinline__ void for_each_value_in_groups(float (&v)[IT][E], F f) {
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            v[it][e] = f(v[it][e], it, e);
+            if (GROUPS && (it * E + e) % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+}
+
+template <int IT, int E, bool GROUPS = true>
 __device__ __forceinline__ void apply_unary_tile(int op, float (&v)[IT][E]) {
 #define AXHIP_UNARY_CASE(code) \
     case code: for_each_value<IT, E>(v, [](float a, int, int) { return apply_unary(code, a); }); break
+#define AXHIP_UNARY_LONG(code) \
+    case code: for_each_value_in_groups<IT, E, GROUPS>(v, [](float a, int, int) { return apply_unary(code, a); }); break
     switch (op) {
         AXHIP_UNARY_CASE(AXHIP_OP_RELU);
-        AXHIP_UNARY_CASE(AXHIP_OP_GELU);
-        AXHIP_UNARY_CASE(AXHIP_OP_SQRT);
-        AXHIP_UNARY_CASE(AXHIP_OP_EXP);
+        AXHIP_UNARY_LONG(AXHIP_OP_GELU);
+        AXHIP_UNARY_LONG(AXHIP_OP_SQRT);
+        AXHIP_UNARY_LONG(AXHIP_OP_EXP);
         AXHIP_UNARY_CASE(AXHIP_OP_NEG);
         AXHIP_UNARY_CASE(AXHIP_OP_ABS);
-        AXHIP_UNARY_CASE(AXHIP_OP_SIGMOID);
-        AXHIP_UNARY_CASE(AXHIP_OP_TANH);
-        AXHIP_UNARY_CASE(AXHIP_OP_SILU);
-        AXHIP_UNARY_CASE(AXHIP_OP_LOG);
+        AXHIP_UNARY_LONG(AXHIP_OP_SIGMOID);
+        AXHIP_UNARY_LONG(AXHIP_OP_TANH);
+        AXHIP_UNARY_LONG(AXHIP_OP_SILU);
+        AXHIP_UNARY_LONG(AXHIP_OP_LOG);
         AXHIP_UNARY_CASE(AXHIP_OP_SQUARE);
-        AXHIP_UNARY_CASE(AXHIP_OP_RSQRT);
-        AXHIP_UNARY_CASE(AXHIP_OP_RECIP);
+        AXHIP_UNARY_LONG(AXHIP_OP_RSQRT);
+        AXHIP_UNARY_LONG(AXHIP_OP_RECIP);
     default: break;
     }
 #undef AXHIP_UNARY_CASE
+#undef AXHIP_UNARY_LONG
 }
 
 // w(it, e) yields the second operand of element (it, e)
-template <int IT, int E, typename W>
+template <int IT, int E, bool GROUPS = true, typename W>
 __device__ __forceinline__ void apply_binary_tile(int op, float (&v)[IT][E], W w) {
 #define AXHIP_BINARY_CASE(code) \
     case code: for_each_value<IT, E>(v, [&](float a, int it, int e) { return apply_binary(code, a, w(it, e)); }); break
+#define AXHIP_BINARY_LONG(code) \
+    case code: for_each_value_in_groups<IT, E, GROUPS>(v, [&](float a, int it, int e) { return apply_binary(code, a, w(it, e)); }); break
     switch (op) {
         AXHIP_BINARY_CASE(AXHIP_OP_ADD);
         AXHIP_BINARY_CASE(AXHIP_OP_SUB);
         AXHIP_BINARY_CASE(AXHIP_OP_MUL);
-        AXHIP_BINARY_CASE(AXHIP_OP_DIV);
+        AXHIP_BINARY_LONG(AXHIP_OP_DIV);
         AXHIP_BINARY_CASE(AXHIP_OP_MAX);
         AXHIP_BINARY_CASE(AXHIP_OP_MIN);
         AXHIP_BINARY_CASE(AXHIP_OP_RSUB);
-        AXHIP_BINARY_CASE(AXHIP_OP_RDIV);
+        AXHIP_BINARY_LONG(AXHIP_OP_RDIV);
     default: break;
     }
 #undef AXHIP_BINARY_CASE
+#undef AXHIP_BINARY_LONG
 }
 
 } // namespace axhip
