@@ -38,8 +38,10 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     if (P.rows <= 0 || P.cols <= 0) return false;
     const int dt = P.input_dtype;
     const int e = dt == AXHIP_DTYPE_F32 ? 4 : 8;
-    if (P.cols % e != 0 || !aligned16(P.input)) return false;
-    if (P.reduce == AXHIP_RED_NONE && (P.output_dtype != dt || !aligned16(P.output))) return false;
+    if (P.cols < e) return false;
+    if (P.reduce == AXHIP_RED_NONE && P.output_dtype != dt) return false;
+    // anything that keeps a 16-byte access from being aligned selects the ragged variant of the kernel
+    bool ragged = P.cols % e != 0 || !aligned16(P.input) || (P.reduce == AXHIP_RED_NONE && !aligned16(P.output));
 
     RowsStaticArgs a{};
     RowsStaticKey k{};
@@ -55,7 +57,9 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     auto vector_operand = [&](int idx, int kind) -> const void * {
         if (idx < 0 || idx >= P.n_operands) return nullptr;
         const AxhipOperand &o = P.operands[idx];
-        return (o.kind == kind && o.dtype == dt && aligned16(o.ptr)) ? o.ptr : nullptr;
+        if (o.kind != kind || o.dtype != dt) return nullptr;
+        if (!aligned16(o.ptr)) ragged = true;
+        return o.ptr;
     };
 
     // a scalar of the pre chain: an immediate, or a one-element device operand
@@ -140,7 +144,9 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     if (!has_pattern(k.pre, k.row_op, k.reduce)) return false;
 
     // register plan
-    const int64_t chunks = P.cols / e;
+    const int64_t chunks = (P.cols + e - 1) / e;
+    a.ragged = ragged;
+    if (ragged) a.stream_out = 0;
     if (chunks <= 512) {
         k.group = 64;
         k.it = chunks <= 64 ? 1 : chunks <= 128 ? 2 : chunks <= 256 ? 4 : 8;
@@ -154,8 +160,8 @@ bool rows_static_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch,
     if ((P.rows + rows_per_block - 1) / rows_per_block >= (int64_t(1) << 31)) return false;
 
     if (name) {
-        snprintf(name, name_len, "rows_static_%s%s%s_%s_g%d_it%d", pre_name(k.pre), rowop_name(k.row_op), red_name(k.reduce),
-                 dtype_name(dt), k.group, k.it);
+        snprintf(name, name_len, "rows_static_%s%s%s_%s_g%d_it%d%s", pre_name(k.pre), rowop_name(k.row_op), red_name(k.reduce),
+                 dtype_name(dt), k.group, k.it, ragged ? "_ragged" : "");
     }
     if (!launch) return true;
     return dt == AXHIP_DTYPE_F32 ? rows_static_launch_f32(k, a, s)

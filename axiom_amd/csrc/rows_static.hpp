@@ -5,8 +5,9 @@
 //
 // A program qualifies when
 //   - input, full-size output and every vector operand share one dtype,
-//   - cols is a multiple of the 16-byte vector width and all pointers are
-//     16-byte aligned,
+//   - cols holds at least one 16-byte vector (any other length, and pointers
+//     that are only element-aligned, run the kernels' ragged variant: unaligned
+//     16-byte accesses and an element-wise last chunk),
 //   - a row fits in registers (cols <= 8192 fp32 / 16384 half elements),
 //   - the pre chain is empty, [add FULL] (residual) or
 //     [relu, add scalar, mul FULL]; the post chain is empty or one unary op,
@@ -35,6 +36,7 @@ struct RowsStaticArgs {
     int32_t red_mean;   // reduce == MEAN: scale the sum by 1/cols
     int32_t out_dtype;  // dtype of a reduced [rows] output
     int32_t stream_out; // full-size output written with non-temporal stores
+    int32_t ragged;     // cols is not a multiple of the 16-byte vector, or a pointer is not 16-byte aligned
 };
 
 struct RowsStaticKey {

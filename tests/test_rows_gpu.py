@@ -361,9 +361,10 @@ def test_sum_of_a_sum_and_row_dot_product_on_the_specialised_kernels():
 
 
 @pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
-def test_rows_of_odd_length_on_the_ragged_resident_plan(dt):
-    """Column counts that no aligned vector divides (4097, 1001, 77): full-width unaligned accesses plus an
-    element-wise last chunk; softmax, layer norm with weight and bias, a full-size operand, a row reduction."""
+def test_rows_of_odd_length_on_the_ragged_plans(dt):
+    """Column counts that no aligned vector divides (4097, 1001, 77): full-width unaligned accesses plus a partial
+    last chunk, on the specialised kernels (softmax of a sum, layer norm with weight and bias, a row reduction) and
+    on the interpreter (a chain the specialised set does not hold)."""
     g = axo.PCG64(808)
     for cols in (77, 1001, 4097):
         x, y = g.normal((11, cols)) * 2, g.normal((11, cols))
@@ -392,3 +393,47 @@ def test_rows_of_odd_length_on_the_ragged_resident_plan(dt):
         p = gh.Rows(xs, dt, F32).unary("square")
         got = p.run(reduce="sum")
         assert np.allclose(got.reshape(-1), (xf * xf).sum(-1), rtol=1e-4, atol=1e-3)
+        if cols >= 8:
+            assert p.kernel_name().startswith("rows_static_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+        p = gh.Rows(xs, dt).unary("abs").binary("mul", ys).row_op("softmax")
+        got = out(p.run())
+        assert p.kernel_name().startswith("rows_resident_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+        lg = np.abs(f(xs)) * f(ys)
+        e = np.exp(lg - lg.max(-1, keepdims=True))
+        assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_bases_that_are_only_element_aligned(dt):
+    """Input, residual, weight and bias start a few elements into their buffers (views into larger tensors): the
+    specialised kernels take them on their ragged variant, with a column count the vector does divide."""
+    g = axo.PCG64(909)
+    rows, cols = 9, 1024
+    es = 4 if dt == F32 else 2
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    f = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    x, y = store(g.normal((rows, cols)) * 2), store(g.normal((rows, cols)))
+    w, b = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((cols,), -0.5, 0.5))
+
+    def shifted(p, arr, off):
+        pad = gh.to_dev(np.concatenate([np.zeros(off, arr.dtype), arr.ravel()]))
+        p.keep.append(pad)
+        return pad.data_ptr() + off * es
+
+    p = gh.Rows(x, dt).binary("add", y).row_op("layernorm", 1e-5, w=w, b=b)
+    p.p.input = shifted(p, x, 3)
+    p.p.operands[0].ptr = shifted(p, y, 1)
+    p.p.operands[1].ptr = shifted(p, w, 5)
+    p.p.operands[2].ptr = shifted(p, b, 2)
+    got = f(p.run())
+    assert p.kernel_name().startswith("rows_static_addf_layernorm") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+    t = f(x) + f(y)
+    ref = (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * f(w) + f(b)
+    assert np.max(np.abs(got - ref)) < (1e-4 if dt == F32 else 4e-2)
+
+    p = gh.Rows(x, dt).row_op("softmax")
+    p.p.input = shifted(p, x, 1)
+    got = f(p.run())
+    assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+    e = np.exp(f(x) - f(x).max(-1, keepdims=True))
+    assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < (1e-4 if dt == F32 else 2e-2)
