@@ -196,6 +196,21 @@ def bench_chains(torch, capi, stream, steps, warmup):
             "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
             "finite": bool(torch.isfinite(y.float()).all().item()),
         }
+    # a row length that the 16-byte vector does not divide (Whisper's 1500 frames): the kernels' ragged variant
+    Rr, Cr = 30000, 1500
+    xr = torch.randn((Rr, Cr), generator=g, device="cuda").to(torch.bfloat16)
+    yr = torch.empty_like(xr)
+    p = _rows_program(capi, xr, yr, capi.DTYPE_BF16, capi.DTYPE_BF16)
+    p.row_op, p.reduce = capi.ROWOP["softmax"], capi.RED["none"]
+    torch.cuda.synchronize()
+    avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+    nbytes = 2 * Rr * Cr * 2
+    sums = yr.float().sum(1)
+    res["softmax_bf16_30000x1500_odd_row_length"] = {
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms,
+        "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "rows_sum_to_one": bool(((sums - 1.0).abs() < 2e-2).all().item()),
+    }
     return res
 
 
