@@ -52,9 +52,9 @@ __device__ __forceinline__ void apply_op(const AxhipChainOp &c, const AxhipRowsP
         if (P.output_dtype != AXHIP_DTYPE_F32) {
             switch (c.op) {
             case AXHIP_OP_GELU: for_each_value<IT, E>(v, [](float a, int, int) { return gelu_fast(a); }); return;
-            case AXHIP_OP_SILU: for_each_value<IT, E>(v, [](float a, int, int) { return a * __frcp_rn(1.0f + __expf(-a)); }); return;
-            case AXHIP_OP_SIGMOID: for_each_value<IT, E>(v, [](float a, int, int) { return __frcp_rn(1.0f + __expf(-a)); }); return;
-            case AXHIP_OP_TANH: for_each_value<IT, E>(v, [](float a, int, int) { return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * a)); }); return;
+            case AXHIP_OP_SILU: for_each_value<IT, E>(v, [](float a, int, int) { return a * __builtin_amdgcn_rcpf(1.0f + __expf(-a)); }); return;
+            case AXHIP_OP_SIGMOID: for_each_value<IT, E>(v, [](float a, int, int) { return __builtin_amdgcn_rcpf(1.0f + __expf(-a)); }); return;
+            case AXHIP_OP_TANH: for_each_value<IT, E>(v, [](float a, int, int) { return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * a)); }); return;
             default: break;
             }
         }
