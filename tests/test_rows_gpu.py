@@ -360,7 +360,7 @@ def test_sum_of_a_sum_and_row_dot_product_on_the_specialised_kernels():
     assert np.allclose(got.reshape(-1), (axo.to_f32(xb, BF16).astype(np.float64) * axo.to_f32(yb, BF16)).mean(-1), rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_rows_of_odd_length_on_the_ragged_plans(dt):
     """Column counts that no aligned vector divides (4097, 1001, 77): full-width unaligned accesses plus a partial
     last chunk, on the specialised kernels (softmax of a sum, layer norm with weight and bias, a row reduction) and
@@ -403,7 +403,7 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
         assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
 
 
-@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_bases_that_are_only_element_aligned(dt):
     """Input, residual, weight and bias start a few elements into their buffers (views into larger tensors): the
     specialised kernels take them on their ragged variant, with a column count the vector does divide."""
