@@ -395,6 +395,16 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
         assert np.allclose(got.reshape(-1), (xf * xf).sum(-1), rtol=1e-4, atol=1e-3)
         if cols >= 8:
             assert p.kernel_name().startswith("rows_static_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+        p = gh.Rows(xs, dt).row_op("logsoftmax")
+        got = out(p.run())
+        assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+        ref = xf - xf.max(-1, keepdims=True)
+        ref = ref - np.log(np.exp(ref).sum(-1, keepdims=True))
+        assert np.max(np.abs(got - ref)) < (1e-4 if dt == F32 else 8e-2)  # |log p| reaches 16: half an ulp of a 16-bit result
+        for red, fn in (("max", np.max), ("min", np.min)):
+            p = gh.Rows(xs, dt, F32)
+            got = p.run(reduce=red)
+            assert np.array_equal(got.reshape(-1).astype(np.float64), fn(xf, axis=-1)), red  # exact: a selection
         p = gh.Rows(xs, dt).unary("abs").binary("mul", ys).row_op("softmax")
         got = out(p.run())
         assert p.kernel_name().startswith("rows_resident_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
