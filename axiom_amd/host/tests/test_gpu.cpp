@@ -231,6 +231,31 @@ GPU_TEST(Normalization, KnownAnswers) {
     EXPECT_THROW(ops::softmax(a.gpu(), 0).cpu(), RuntimeError); // only the last axis is on the GPU path
 }
 
+// Rows whose length no 16-byte vector divides (Whisper's 1500 frames, an odd vocabulary) take the specialised
+// kernels' ragged variant; the results are checked against a double-precision evaluation on the host.
+GPU_TEST(FusedRows, OddRowLengthsRunOnTheRaggedKernels) {
+    const size_t R = 37, C = 1501;
+    auto a = axtest::randn({R, C}, 77);
+    const float *x = a.typed_data<float>();
+    auto sm = host_floats(ops::softmax(a.gpu() * 0.5f, -1));
+    ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_static_muls_softmax_f32_g64_it8_ragged"));
+    auto ln = host_floats(ops::layer_norm(a.gpu(), Tensor(), Tensor(), -1, 1e-5f));
+    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_static_layernorm_f32_g64_it8_ragged"));
+    for (size_t i = 0; i < R; ++i) {
+        double mx = -1e300, s = 0, mean = 0, var = 0;
+        for (size_t j = 0; j < C; ++j) mx = std::max(mx, 0.5 * x[i * C + j]);
+        for (size_t j = 0; j < C; ++j) s += std::exp(0.5 * x[i * C + j] - mx), mean += x[i * C + j];
+        mean /= C;
+        for (size_t j = 0; j < C; ++j) var += (x[i * C + j] - mean) * (x[i * C + j] - mean);
+        var /= C;
+        for (size_t j = 0; j < C; ++j) {
+            EXPECT_NEAR(sm[i * C + j], std::exp(0.5 * x[i * C + j] - mx) / s, 1e-6);
+            EXPECT_NEAR(ln[i * C + j], (x[i * C + j] - mean) / std::sqrt(var + 1e-5), 1e-4);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- parity ops
 GPU_TEST(CpuGpuParity, ElementwiseReductionsMatmul) { // tests/test_cpu_gpu_parity.cpp:12-492 (hot-path ops)
     auto a = axtest::randn({4, 5}, 41), b = axtest::randn({4, 5}, 42);
