@@ -102,6 +102,8 @@ def lib() -> C.CDLL:
         l.axhip_sdpa_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(SdpaParams), C.c_void_p]
         l.axhip_fused_rows.argtypes = [C.POINTER(RowsProgram), C.c_void_p]
         l.axhip_fused_full_reduce.argtypes = [C.POINTER(RowsProgram), C.c_void_p, C.c_size_t, C.c_void_p]
+        l.axhip_fused_full_reduce_noalloc.argtypes = [C.POINTER(RowsProgram), C.c_void_p]
+        l.axhip_full_reduce_noalloc_max_elements.restype = C.c_int64
         l.axhip_strided_copy.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32,
                                          C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p]
         l.axhip_fill.argtypes = [C.c_void_p, C.c_int32, C.c_double, C.c_int64, C.c_void_p]

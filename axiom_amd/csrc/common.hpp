@@ -15,6 +15,7 @@ namespace axhip {
 void set_last_error(const char *fmt, ...);
 hipStream_t resolve_stream(void *stream);
 int ensure_init();
+int rows_setup_device(); // per-device set-up of the fused-row kernels (rows.hip), run by axhip_init
 
 #define AXHIP_CHECK_HIP(expr)                                                          \
     do {                                                                               \

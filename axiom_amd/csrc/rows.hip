@@ -12,6 +12,12 @@
 #include "rows_static.hpp"
 
 #include <algorithm>
+#include <mutex>
+
+// Partial sums of axhip_fused_full_reduce_noalloc: one float per stage-1 block (2048 blocks at most, 8 KiB).  Every
+// device the library runs on holds its own copy until the process ends.  In host code this name is only a handle
+// for hipGetSymbolAddress; kernels and copies take the per-device address kept in g_scratch_ptr.
+static __device__ __align__(256) float scratch[2048];
 
 namespace axhip {
 
@@ -609,7 +615,69 @@ int launch_plan_e(const AxhipRowsProgram &P, const RowsPlan &pl, hipStream_t s) 
     }
 }
 
+
+int check_full_reduce_program(const AxhipRowsProgram *program, const char *who) {
+    AXHIP_REQUIRE(program != nullptr, AXHIP_ERR_INVALID_ARG, "%s: program is NULL", who);
+    const AxhipRowsProgram &P = *program;
+    int rc = validate_program(P, who);
+    if (rc) return rc;
+    AXHIP_REQUIRE(P.row_op == AXHIP_ROWOP_NONE && P.n_post == 0, AXHIP_ERR_INVALID_ARG, "%s: row_op/post must be empty", who);
+    AXHIP_REQUIRE(P.reduce != AXHIP_RED_NONE, AXHIP_ERR_INVALID_ARG, "%s: reduce is NONE", who);
+    AXHIP_REQUIRE(P.rows > 0 && P.cols > 0, AXHIP_ERR_INVALID_ARG, "%s: empty input", who);
+    return AXHIP_OK;
+}
+
+// stage 1 leaves `blocks` partials in `partials` (FULL_RED_BLOCKS floats), stage 2 reads exactly those
+int launch_full_reduce(const AxhipRowsProgram &P, float *partials, hipStream_t s) {
+    AxhipRowsProgram Q = P;
+    Q.reduce = AXHIP_RED_SUM; // only used by pick_vector_width to skip the output alignment test
+    const int e = pick_vector_width(Q);
+    const int64_t n = P.rows * P.cols;
+    const int64_t nchunk = n / e;
+    const int blocks = static_cast<int>(std::min<int64_t>((nchunk + 255) / 256, FULL_RED_BLOCKS));
+    if (e == 8) hipLaunchKernelGGL((full_reduce_stage1<256, 8>), dim3(blocks), dim3(256), 0, s, P, partials);
+    else if (e == 4) hipLaunchKernelGGL((full_reduce_stage1<256, 4>), dim3(blocks), dim3(256), 0, s, P, partials);
+    else hipLaunchKernelGGL((full_reduce_stage1<256, 1>), dim3(blocks), dim3(256), 0, s, P, partials);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    hipLaunchKernelGGL((full_reduce_stage2<256>), dim3(1), dim3(256), 0, s, partials, blocks, P.reduce,
+                       1.0f / static_cast<float>(n), P.output, P.output_dtype);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+// Largest input axhip_fused_full_reduce_noalloc accepts (2^40 elements): the partials fit the fixed array whatever
+// the size, the bound keeps rows * cols and the blocks' strided loops far inside 64-bit range.
+constexpr int64_t FULL_REDUCE_NOALLOC_MAX_ELEMENTS = int64_t(1) << 40;
+
+// Device address of `scratch` on the calling thread's current device, resolved once per device.
+constexpr int MAX_SCRATCH_DEVICES = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[MAX_SCRATCH_DEVICES] = {};
+
+int scratch_of_current_device(float **out) {
+    int dev = -1;
+    AXHIP_CHECK_HIP(hipGetDevice(&dev));
+    AXHIP_REQUIRE(dev >= 0 && dev < MAX_SCRATCH_DEVICES, AXHIP_ERR_UNSUPPORTED, "device ordinal %d beyond the %d this library keeps scratch for", dev,
+                  MAX_SCRATCH_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        AXHIP_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        AXHIP_REQUIRE(p != nullptr, AXHIP_ERR_WORKSPACE, "hipGetSymbolAddress returned no address for the reduction scratch");
+        g_scratch_ptr[dev] = static_cast<float *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return AXHIP_OK;
+}
+
 } // namespace
+
+// Called by axhip_init with the device current, so that the first no-allocation call on it finds the address resolved.
+int rows_setup_device() {
+    float *unused = nullptr;
+    return scratch_of_current_device(&unused);
+}
+
 } // namespace axhip
 
 using namespace axhip;
@@ -650,33 +718,31 @@ int axhip_fused_rows(const AxhipRowsProgram *program, void *stream) {
 size_t axhip_full_reduce_workspace_bytes(void) { return FULL_RED_BLOCKS * sizeof(float); }
 
 int axhip_fused_full_reduce(const AxhipRowsProgram *program, void *workspace, size_t workspace_bytes, void *stream) {
-    AXHIP_REQUIRE(program != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: program is NULL");
-    const AxhipRowsProgram &P = *program;
-    int rc = validate_program(P, "axhip_fused_full_reduce");
+    int rc = check_full_reduce_program(program, "axhip_fused_full_reduce");
     if (rc) return rc;
-    AXHIP_REQUIRE(P.row_op == AXHIP_ROWOP_NONE && P.n_post == 0, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: row_op/post must be empty");
-    AXHIP_REQUIRE(P.reduce != AXHIP_RED_NONE, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: reduce is NONE");
-    AXHIP_REQUIRE(P.rows > 0 && P.cols > 0, AXHIP_ERR_INVALID_ARG, "axhip_fused_full_reduce: empty input");
     AXHIP_REQUIRE(workspace && workspace_bytes >= axhip_full_reduce_workspace_bytes() && aligned_to(workspace, 4), AXHIP_ERR_WORKSPACE,
                   "axhip_fused_full_reduce: workspace too small (%zu < %zu)", workspace_bytes, axhip_full_reduce_workspace_bytes());
     rc = ensure_init();
     if (rc) return rc;
-    hipStream_t s = resolve_stream(stream);
-    AxhipRowsProgram Q = P;
-    Q.reduce = AXHIP_RED_SUM; // only used by pick_vector_width to skip the output alignment test
-    const int e = pick_vector_width(Q);
-    const int64_t n = P.rows * P.cols;
-    const int64_t nchunk = n / e;
-    const int blocks = static_cast<int>(std::min<int64_t>((nchunk + 255) / 256, FULL_RED_BLOCKS));
-    float *partials = static_cast<float *>(workspace);
-    if (e == 8) hipLaunchKernelGGL((full_reduce_stage1<256, 8>), dim3(blocks), dim3(256), 0, s, P, partials);
-    else if (e == 4) hipLaunchKernelGGL((full_reduce_stage1<256, 4>), dim3(blocks), dim3(256), 0, s, P, partials);
-    else hipLaunchKernelGGL((full_reduce_stage1<256, 1>), dim3(blocks), dim3(256), 0, s, P, partials);
-    AXHIP_CHECK_HIP(hipGetLastError());
-    hipLaunchKernelGGL((full_reduce_stage2<256>), dim3(1), dim3(256), 0, s, partials, blocks, P.reduce,
-                       1.0f / static_cast<float>(n), P.output, P.output_dtype);
-    AXHIP_CHECK_HIP(hipGetLastError());
-    return AXHIP_OK;
+    return launch_full_reduce(*program, static_cast<float *>(workspace), resolve_stream(stream));
+}
+
+int64_t axhip_full_reduce_noalloc_max_elements(void) { return FULL_REDUCE_NOALLOC_MAX_ELEMENTS; }
+
+int axhip_fused_full_reduce_noalloc(const AxhipRowsProgram *program, void *stream) {
+    int rc = check_full_reduce_program(program, "axhip_fused_full_reduce_noalloc");
+    if (rc) return rc;
+    // rows and cols are positive here; the division keeps the product from overflowing
+    AXHIP_REQUIRE(program->rows <= FULL_REDUCE_NOALLOC_MAX_ELEMENTS / program->cols, AXHIP_ERR_UNSUPPORTED,
+                  "axhip_fused_full_reduce_noalloc: %lld x %lld elements exceed the maximum of %lld", static_cast<long long>(program->rows),
+                  static_cast<long long>(program->cols), static_cast<long long>(FULL_REDUCE_NOALLOC_MAX_ELEMENTS));
+    rc = ensure_init();
+    if (rc) return rc;
+    float *partials = nullptr;
+    rc = scratch_of_current_device(&partials);
+    if (rc) return rc;
+    // Nothing in the array has to start at zero: stage 1 writes every partial stage 2 reads.
+    return launch_full_reduce(*program, partials, resolve_stream(stream));
 }
 
 } // extern "C"

@@ -87,6 +87,8 @@ int axhip_init(int device) {
         return AXHIP_ERR_UNSUPPORTED;
     }
     if (!g_stream) AXHIP_CHECK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    int rc = rows_setup_device();
+    if (rc) return rc;
     g_device = device;
     g_initialised = true;
     return AXHIP_OK;

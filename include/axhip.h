@@ -208,6 +208,23 @@ size_t axhip_full_reduce_workspace_bytes(void);
 int axhip_fused_full_reduce(const AxhipRowsProgram *program_host, void *workspace,
                             size_t workspace_bytes, void *stream);
 
+/* axhip_fused_full_reduce for callers that cannot allocate device memory or
+ * bring a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * Same program, same kernels and the same result, bit for bit; the partial
+ * sums live in an 8 KiB array inside the library's device image (one copy on
+ * every device the library runs on, held until the process ends), whose
+ * address is resolved when axhip_init runs on the device.  The call itself
+ * performs no hipMalloc / hipFree and calls no allocating routine.
+ * Limits: rows * cols <= axhip_full_reduce_noalloc_max_elements() (2^40),
+ * larger inputs return AXHIP_ERR_UNSUPPORTED.  All calls on one device share
+ * that one array: two calls that overlap in time on the same device (different
+ * streams, or different threads on different streams) race; calls on one
+ * stream are ordered and safe.  Nothing in the array has to be cleared
+ * between calls. */
+int64_t axhip_full_reduce_noalloc_max_elements(void);
+int axhip_fused_full_reduce_noalloc(const AxhipRowsProgram *program_host, void *stream);
+
 /* ------------------------------------------------------------- data movers
  * Stands behind gpu_make_contiguous (src/backends/metal/metal_operations.hpp:
  * 60-63, kernel gather_strided src/backends/metal/kernels.metal:33-149) and
