@@ -101,6 +101,7 @@ def lib() -> C.CDLL:
         l.axhip_stream_sync.argtypes = [C.c_void_p]
         l.axhip_sdpa_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(SdpaParams), C.c_void_p]
         l.axhip_fused_rows.argtypes = [C.POINTER(RowsProgram), C.c_void_p]
+        l.axhip_fused_rows_prepare.argtypes = [C.POINTER(RowsProgram)]
         l.axhip_fused_full_reduce.argtypes = [C.POINTER(RowsProgram), C.c_void_p, C.c_size_t, C.c_void_p]
         l.axhip_fused_full_reduce_noalloc.argtypes = [C.POINTER(RowsProgram), C.c_void_p]
         l.axhip_full_reduce_noalloc_max_elements.restype = C.c_int64

@@ -9,10 +9,12 @@
 // Reductions are wave64 shuffles plus one LDS hop when a row spans several waves.
 #include "common.hpp"
 #include "rows_ops.hpp"
-#include "rows_static.hpp"
+#include "rows_prog.hpp"
 
 #include <algorithm>
+#include <cstring>
 #include <mutex>
+#include <string>
 
 // Partial sums of axhip_fused_full_reduce_noalloc: one float per stage-1 block (2048 blocks at most, 8 KiB).  Every
 // device the library runs on holds its own copy until the process ends.  In host code this name is only a handle
@@ -685,9 +687,9 @@ using namespace axhip;
 extern "C" {
 
 const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *P) {
-    static thread_local char name[64];
+    static thread_local char name[192];
     if (!P) return "invalid";
-    if (validate_program(*P, "axhip_fused_rows_kernel_name") == AXHIP_OK && rows_static_dispatch(*P, nullptr, false, name, sizeof(name)))
+    if (validate_program(*P, "axhip_fused_rows_kernel_name") == AXHIP_OK && rows_prog_dispatch(*P, nullptr, false, name, sizeof(name), nullptr))
         return name;
     RowsPlan pl = plan_rows(*P);
     snprintf(name, sizeof(name), "%s", pl.name);
@@ -705,13 +707,32 @@ int axhip_fused_rows(const AxhipRowsProgram *program, void *stream) {
     RowsPlan pl = plan_rows(P);
     if (pl.kind == RowsPlan::EMPTY) return AXHIP_OK;
     hipStream_t s = resolve_stream(stream);
-    if (rows_static_dispatch(P, s, true, nullptr, 0)) {
+    // a kernel compiled for this program's shape (built in, or compiled now if this is its first launch) ...
+    int launch_rc = AXHIP_OK;
+    if (rows_prog_dispatch(P, s, true, nullptr, 0, &launch_rc)) {
+        if (launch_rc) return launch_rc;
         AXHIP_CHECK_HIP(hipGetLastError());
         return AXHIP_OK;
     }
+    // ... or the interpreter
     rc = pl.e == 8 ? launch_plan_e<8>(P, pl, s) : pl.e == 4 ? launch_plan_e<4>(P, pl, s) : launch_plan_e<1>(P, pl, s);
     if (rc) return rc;
     AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+int axhip_fused_rows_prepare(const AxhipRowsProgram *program) {
+    AXHIP_REQUIRE(program != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_fused_rows_prepare: program is NULL");
+    int rc = validate_program(*program, "axhip_fused_rows_prepare");
+    if (rc) return rc;
+    char name[192];
+    if (!rows_prog_dispatch(*program, nullptr, false, name, sizeof(name), nullptr)) return AXHIP_OK; // the interpreter's: nothing to prepare
+    if (strncmp(name, "rows_static_", 12) == 0) return AXHIP_OK;                                    // built into the library
+    std::string label, error;
+    if (!rows_prog_compile_only(*program, &label, &error)) {
+        set_last_error("axhip_fused_rows_prepare: %s: %.400s", label.c_str(), error.c_str());
+        return AXHIP_ERR_UNSUPPORTED;
+    }
     return AXHIP_OK;
 }
 

@@ -1,0 +1,186 @@
+// Build-time tool: writes the source files of the fused-row kernels that are compiled into the library.
+//
+//     rows_aot_gen <output directory> <number of files>
+//
+// The program shapes listed here are the counterpart of Axiom's known fused patterns
+// (src/graph/fused_patterns.cpp:12-71): softmax / log-softmax / layer norm / RMS norm / row reductions, optionally
+// behind x+y, x*s, x*s+y or (relu(x)+s)*y and, for the norms, followed by one activation -- for the three element
+// types, every register plan and both the aligned and the ragged row form.  Any other shape is compiled by the
+// library at run time, from the same generator.
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "rows_codegen.hpp"
+
+using namespace axhip;
+
+namespace {
+
+struct Shape {
+    AxhipRowsProgram p;
+};
+
+void *fake(int i) { return reinterpret_cast<void *>(static_cast<uintptr_t>(0x1000 * (i + 1))); }
+
+AxhipRowsProgram base(int dt) {
+    AxhipRowsProgram p;
+    memset(&p, 0, sizeof(p));
+    p.rows = 1;
+    p.cols = 8;
+    p.input = fake(0);
+    p.output = fake(1);
+    p.input_dtype = p.output_dtype = dt;
+    p.norm_weight = p.norm_bias = -1;
+    return p;
+}
+int add_operand(AxhipRowsProgram &p, int dt, int kind) {
+    p.operands[p.n_operands] = {fake(2 + p.n_operands), dt, kind};
+    return p.n_operands++;
+}
+void push(AxhipChainOp *chain, int32_t &n, int op, int operand, bool imm) {
+    chain[n].op = op;
+    chain[n].operand = imm ? -1 : operand;
+    chain[n].imm = 0.0f;
+    chain[n].imm_kind = imm ? AXHIP_BK_IMM : 0;
+    ++n;
+}
+// `s`: the chain's scalar as an immediate (true) or as a one-element device operand (false)
+enum Pre { PRE_NONE, PRE_ADDF, PRE_MULF, PRE_MULS, PRE_MULS_ADDF, PRE_RELU_ADDS_MULF };
+void add_pre(AxhipRowsProgram &p, int dt, Pre pre, bool imm) {
+    const int s = (pre == PRE_MULS || pre == PRE_MULS_ADDF || pre == PRE_RELU_ADDS_MULF) && !imm ? add_operand(p, dt, AXHIP_BK_SCALAR) : -1;
+    switch (pre) {
+    case PRE_NONE: break;
+    case PRE_ADDF: push(p.pre, p.n_pre, AXHIP_OP_ADD, add_operand(p, dt, AXHIP_BK_FULL), false); break;
+    case PRE_MULF: push(p.pre, p.n_pre, AXHIP_OP_MUL, add_operand(p, dt, AXHIP_BK_FULL), false); break;
+    case PRE_MULS: push(p.pre, p.n_pre, AXHIP_OP_MUL, s, imm); break;
+    case PRE_MULS_ADDF:
+        push(p.pre, p.n_pre, AXHIP_OP_MUL, s, imm);
+        push(p.pre, p.n_pre, AXHIP_OP_ADD, add_operand(p, dt, AXHIP_BK_FULL), false);
+        break;
+    case PRE_RELU_ADDS_MULF:
+        push(p.pre, p.n_pre, AXHIP_OP_RELU, -1, false);
+        push(p.pre, p.n_pre, AXHIP_OP_ADD, s, imm);
+        push(p.pre, p.n_pre, AXHIP_OP_MUL, add_operand(p, dt, AXHIP_BK_FULL), false);
+        break;
+    }
+}
+
+std::vector<AxhipRowsProgram> shapes_of(int dt) {
+    std::vector<AxhipRowsProgram> out;
+    // softmax family
+    for (int red : {AXHIP_RED_NONE, AXHIP_RED_SUM}) {
+        AxhipRowsProgram p = base(dt);
+        p.row_op = AXHIP_ROWOP_SOFTMAX;
+        p.reduce = red;
+        out.push_back(p);
+        for (bool imm : {true, false}) {
+            AxhipRowsProgram q = base(dt);
+            add_pre(q, dt, PRE_RELU_ADDS_MULF, imm);
+            q.row_op = AXHIP_ROWOP_SOFTMAX;
+            q.reduce = red;
+            out.push_back(q);
+        }
+    }
+    {
+        AxhipRowsProgram p = base(dt);
+        p.row_op = AXHIP_ROWOP_LOGSOFTMAX;
+        out.push_back(p);
+    }
+    for (Pre pre : {PRE_MULS, PRE_ADDF, PRE_MULS_ADDF})
+        for (bool imm : {true, false}) {
+            if (pre == PRE_ADDF && !imm) continue;
+            AxhipRowsProgram p = base(dt);
+            add_pre(p, dt, pre, imm);
+            p.row_op = AXHIP_ROWOP_SOFTMAX;
+            out.push_back(p);
+        }
+    // norms: plain or behind a residual sum, with and without the affine part, followed by nothing or one activation
+    for (int rowop : {AXHIP_ROWOP_LAYERNORM, AXHIP_ROWOP_RMSNORM})
+        for (Pre pre : {PRE_NONE, PRE_ADDF})
+            for (bool affine : {false, true})
+                for (int post : {0, AXHIP_OP_GELU, AXHIP_OP_SILU, AXHIP_OP_RELU}) {
+                    AxhipRowsProgram p = base(dt);
+                    if (affine) {
+                        p.norm_weight = add_operand(p, dt, AXHIP_BK_ROWVEC);
+                        if (rowop == AXHIP_ROWOP_LAYERNORM) p.norm_bias = add_operand(p, dt, AXHIP_BK_ROWVEC);
+                    }
+                    add_pre(p, dt, pre, true);
+                    p.row_op = rowop;
+                    if (post) push(p.post, p.n_post, post, -1, false);
+                    out.push_back(p);
+                }
+    // row reductions of x, f(x), x + y, x * y
+    for (Pre pre : {PRE_NONE, PRE_ADDF, PRE_MULF}) {
+        AxhipRowsProgram p = base(dt);
+        add_pre(p, dt, pre, true);
+        p.reduce = AXHIP_RED_SUM;
+        out.push_back(p);
+    }
+    for (int unary : {AXHIP_OP_RELU, AXHIP_OP_SQUARE, AXHIP_OP_ABS}) {
+        AxhipRowsProgram p = base(dt);
+        push(p.pre, p.n_pre, unary, -1, false);
+        p.reduce = AXHIP_RED_SUM;
+        out.push_back(p);
+    }
+    for (int red : {AXHIP_RED_MAX, AXHIP_RED_MIN}) {
+        AxhipRowsProgram p = base(dt);
+        p.reduce = red;
+        out.push_back(p);
+    }
+    {
+        AxhipRowsProgram p = base(dt);
+        push(p.pre, p.n_pre, AXHIP_OP_ABS, -1, false);
+        p.reduce = AXHIP_RED_MAX;
+        out.push_back(p);
+    }
+    return out;
+}
+
+} // namespace
+
+int main(int argc, char **argv) {
+    if (argc < 3) {
+        fprintf(stderr, "usage: %s <output directory> <number of files>\n", argv[0]);
+        return 2;
+    }
+    const std::string dir = argv[1];
+    const int n_files = atoi(argv[2]);
+    if (n_files <= 0) return 2;
+    static const int plans[][2] = {{64, 1}, {64, 2}, {64, 4}, {64, 8}, {256, 4}, {256, 8}};
+    std::vector<RowsProgSpec> specs;
+    std::set<std::string> seen;
+    for (int dt : {AXHIP_DTYPE_F32, AXHIP_DTYPE_F16, AXHIP_DTYPE_BF16})
+        for (const AxhipRowsProgram &p : shapes_of(dt))
+            for (const auto &pl : plans)
+                for (bool ragged : {false, true}) {
+                    RowsProgPlan plan;
+                    rows_prog_plan_for(p, pl[0], pl[1], ragged, &plan);
+                    RowsProgSpec s;
+                    if (!rows_prog_spec(p, plan, &s)) {
+                        fprintf(stderr, "rows_aot_gen: a listed shape was refused by the generator\n");
+                        return 1;
+                    }
+                    if (seen.insert(s.symbol).second) specs.push_back(s);
+                }
+    std::vector<std::ofstream> files;
+    for (int i = 0; i < n_files; ++i) {
+        char name[64];
+        snprintf(name, sizeof(name), "/rows_aot_%02d.hip", i);
+        files.emplace_back(dir + name);
+        files.back() << "// generated by rows_aot_gen: fused-row kernels built into the library\n"
+                        "#include <hip/hip_runtime.h>\n#include \"rows_codegen.hpp\"\n";
+    }
+    for (size_t i = 0; i < specs.size(); ++i) {
+        std::ofstream &f = files[i % n_files];
+        const RowsProgSpec &s = specs[i];
+        f << "\n// " << s.label << "\n" << rows_prog_source(s, "#include \"rows_prog.inc\"\n");
+        f << "static const axhip::RowsProgRegistrar reg_" << s.symbol << "(R\"AXPKEY(" << s.config << s.chains << ")AXPKEY\", reinterpret_cast<const void *>(&"
+          << s.symbol << "));\n";
+    }
+    printf("%zu kernels in %d files\n", specs.size(), n_files);
+    return 0;
+}

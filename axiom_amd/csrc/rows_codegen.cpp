@@ -1,0 +1,418 @@
+// Generator of the compiled fused-row programs (see rows_codegen.hpp).
+#include "rows_codegen.hpp"
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <sstream>
+
+namespace axhip {
+
+namespace {
+
+int elem_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+const char *dt_name(int dt) { return dt == AXHIP_DTYPE_F32 ? "f32" : dt == AXHIP_DTYPE_F16 ? "f16" : "bf16"; }
+bool is_unary(int op) { return op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP; }
+bool is_binary(int op) { return op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV; }
+
+const char *op_token(int op) {
+    switch (op) {
+    case AXHIP_OP_ADD: return "add";
+    case AXHIP_OP_SUB: return "sub";
+    case AXHIP_OP_MUL: return "mul";
+    case AXHIP_OP_DIV: return "div";
+    case AXHIP_OP_MAX: return "max";
+    case AXHIP_OP_MIN: return "min";
+    case AXHIP_OP_RSUB: return "rsub";
+    case AXHIP_OP_RDIV: return "rdiv";
+    case AXHIP_OP_RELU: return "relu";
+    case AXHIP_OP_GELU: return "gelu";
+    case AXHIP_OP_SQRT: return "sqrt";
+    case AXHIP_OP_EXP: return "exp";
+    case AXHIP_OP_NEG: return "neg";
+    case AXHIP_OP_ABS: return "abs";
+    case AXHIP_OP_SIGMOID: return "sigmoid";
+    case AXHIP_OP_TANH: return "tanh";
+    case AXHIP_OP_SILU: return "silu";
+    case AXHIP_OP_LOG: return "log";
+    case AXHIP_OP_SQUARE: return "square";
+    case AXHIP_OP_RSQRT: return "rsqrt";
+    case AXHIP_OP_RECIP: return "recip";
+    default: return nullptr;
+    }
+}
+const char *rowop_token(int r) {
+    switch (r) {
+    case AXHIP_ROWOP_SOFTMAX: return "softmax";
+    case AXHIP_ROWOP_LOGSOFTMAX: return "logsoftmax";
+    case AXHIP_ROWOP_LAYERNORM: return "layernorm";
+    case AXHIP_ROWOP_RMSNORM: return "rmsnorm";
+    default: return "reduce";
+    }
+}
+
+uint64_t fnv1a(const std::string &s, uint64_t h = 14695981039346656037ull) {
+    for (unsigned char c : s) {
+        h ^= c;
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+// operands of the chains, by kind, in the order the chains first name them
+struct OperandTables {
+    int n[4] = {0, 0, 0, 0};      // per AXHIP_BK_FULL / ROWVEC / COLVEC / SCALAR
+    int dt[4][8] = {};
+    int slot[4][8] = {};
+    int of_operand[AXHIP_MAX_OPERANDS]; // operand index -> position in its kind's table, or -1
+    OperandTables() { for (int &v : of_operand) v = -1; }
+};
+
+struct Builder {
+    const AxhipRowsProgram &P;
+    RowsProgSpec &S;
+    OperandTables T;
+    int slot_of_operand[AXHIP_MAX_OPERANDS];
+    bool post_full = false;
+    bool ok = true;
+
+    Builder(const AxhipRowsProgram &p, RowsProgSpec &s) : P(p), S(s) {
+        for (int &v : slot_of_operand) v = -1;
+    }
+
+    int pointer_slot(int operand) {
+        if (slot_of_operand[operand] < 0) {
+            if (S.n_slots >= 8) {
+                ok = false;
+                return 0;
+            }
+            slot_of_operand[operand] = S.n_slots;
+            S.slot_operand[S.n_slots++] = operand;
+        }
+        return slot_of_operand[operand];
+    }
+
+    // expression text of a binary op's second operand
+    std::string operand_expr(const AxhipChainOp &c, bool post, int position, std::string *token) {
+        char buf[64];
+        if (c.imm_kind == AXHIP_BK_IMM) {
+            if (S.n_imm >= 32) {
+                ok = false;
+                return "0.0f";
+            }
+            S.imm_ref[S.n_imm] = {post, position};
+            snprintf(buf, sizeof(buf), "q.imm[%d]", S.n_imm++);
+            *token += "s";
+            return buf;
+        }
+        const int idx = c.operand;
+        if (idx < 0 || idx >= P.n_operands) {
+            ok = false;
+            return "0.0f";
+        }
+        const AxhipOperand &o = P.operands[idx];
+        if (o.kind < AXHIP_BK_FULL || o.kind > AXHIP_BK_SCALAR) {
+            ok = false;
+            return "0.0f";
+        }
+        if (T.of_operand[idx] < 0) {
+            const int k = o.kind;
+            if (T.n[k] >= 8) {
+                ok = false;
+                return "0.0f";
+            }
+            T.of_operand[idx] = T.n[k];
+            T.dt[k][T.n[k]] = o.dtype;
+            T.slot[k][T.n[k]] = pointer_slot(idx);
+            ++T.n[k];
+        }
+        const int at = T.of_operand[idx];
+        switch (o.kind) {
+        case AXHIP_BK_FULL:
+            if (post) post_full = true;
+            snprintf(buf, sizeof(buf), "q.full[%d][e]", at);
+            *token += "f";
+            break;
+        case AXHIP_BK_ROWVEC:
+            snprintf(buf, sizeof(buf), "q.rowv[%d][e]", at);
+            *token += "r";
+            break;
+        case AXHIP_BK_COLVEC:
+            snprintf(buf, sizeof(buf), "q.colv[%d]", at);
+            *token += "c";
+            break;
+        default:
+            snprintf(buf, sizeof(buf), "q.scal[%d]", at);
+            *token += "s";
+            break;
+        }
+        return buf;
+    }
+
+    // one chain as statements on `t`; appends the chain's tokens to the label
+    std::string chain_text(const AxhipChainOp *ops, int n, bool post, bool fast, std::string *label) {
+        std::ostringstream o;
+        for (int i = 0; i < n; ++i) {
+            const int op = ops[i].op;
+            const char *tok = op_token(op);
+            if (!tok) {
+                ok = false;
+                return "";
+            }
+            std::string token = tok;
+            if (is_binary(op)) {
+                const std::string b = operand_expr(ops[i], post, i, &token);
+                switch (op) {
+                case AXHIP_OP_ADD: o << "    t = t + " << b << ";\n"; break;
+                case AXHIP_OP_SUB: o << "    t = t - " << b << ";\n"; break;
+                case AXHIP_OP_MUL: o << "    t = t * " << b << ";\n"; break;
+                case AXHIP_OP_DIV: o << "    t = t / " << b << ";\n"; break;
+                case AXHIP_OP_MAX: o << "    t = fmaxf(t, " << b << ");\n"; break;
+                case AXHIP_OP_MIN: o << "    t = fminf(t, " << b << ");\n"; break;
+                case AXHIP_OP_RSUB: o << "    t = " << b << " - t;\n"; break;
+                default: o << "    t = " << b << " / t;\n"; break;
+                }
+            } else if (is_unary(op)) {
+                switch (op) {
+                case AXHIP_OP_RELU: o << "    t = t > 0.0f ? t : 0.0f;\n"; break;
+                case AXHIP_OP_GELU: o << (fast ? "    t = gelu_fast(t);\n" : "    t = gelu_exact(t);\n"); break;
+                case AXHIP_OP_SQRT: o << "    t = sqrtf(t);\n"; break;
+                case AXHIP_OP_EXP: o << "    t = expf(t);\n"; break;
+                case AXHIP_OP_NEG: o << "    t = -t;\n"; break;
+                case AXHIP_OP_ABS: o << "    t = fabsf(t);\n"; break;
+                case AXHIP_OP_SIGMOID: o << (fast ? "    t = sigmoid_fast(t);\n" : "    t = sigmoid_exact(t);\n"); break;
+                case AXHIP_OP_TANH: o << (fast ? "    t = tanh_fast(t);\n" : "    t = tanhf(t);\n"); break;
+                case AXHIP_OP_SILU: o << (fast ? "    t = silu_fast(t);\n" : "    t = t / (1.0f + expf(-t));\n"); break;
+                case AXHIP_OP_LOG: o << "    t = logf(t);\n"; break;
+                case AXHIP_OP_SQUARE: o << "    t = t * t;\n"; break;
+                case AXHIP_OP_RSQRT: o << "    t = 1.0f / sqrtf(t);\n"; break;
+                default: o << "    t = 1.0f / t;\n"; break;
+                }
+            } else {
+                ok = false;
+                return "";
+            }
+            *label += token + "_";
+        }
+        return o.str();
+    }
+};
+
+std::string int_table(const char *name, const int *v, int n) {
+    std::ostringstream o;
+    o << "constexpr int " << name << "[" << (n > 0 ? n : 1) << "] = {";
+    for (int i = 0; i < (n > 0 ? n : 1); ++i) o << (i ? ", " : "") << (i < n ? v[i] : 0);
+    o << "};\n";
+    return o.str();
+}
+
+} // namespace
+
+namespace {
+// 32-bit words of raw input a thread holds per chunk: the input and every full-size operand the chains name
+int raw_words_per_chunk(const AxhipRowsProgram &P) {
+    const int e = P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8;
+    int words = 4;
+    bool used[AXHIP_MAX_OPERANDS] = {};
+    auto mark = [&](const AxhipChainOp *ops, int n) {
+        for (int i = 0; i < n; ++i)
+            if (is_binary(ops[i].op) && ops[i].imm_kind != AXHIP_BK_IMM && ops[i].operand >= 0 && ops[i].operand < P.n_operands) used[ops[i].operand] = true;
+    };
+    mark(P.pre, P.n_pre);
+    mark(P.post, P.n_post);
+    for (int i = 0; i < P.n_operands; ++i)
+        if (used[i] && P.operands[i].kind == AXHIP_BK_FULL) words += e * elem_size(P.operands[i].dtype) / 4;
+    return words;
+}
+// the same for the norm weight and bias of a row that spans several waves (a wavefront row reads them from LDS)
+int affine_words_per_chunk(const AxhipRowsProgram &P, int group) {
+    if (group == 64) return 0;
+    const int e = P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8;
+    int words = 0;
+    for (int idx : {P.norm_weight, P.norm_bias})
+        if (idx >= 0 && idx < P.n_operands) words += e * elem_size(P.operands[idx].dtype) / 4;
+    return words;
+}
+} // namespace
+
+void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan) {
+    plan->group = group;
+    plan->it = it;
+    plan->ragged = ragged;
+    // Pipelining keeps a second set of raw words alive: worth it while that set is at most 32 registers (a 16-bit
+    // row of 4096 columns per wavefront, or a row with one operand at half that).  The 1024-thread plan has 128
+    // registers per thread and none to spare.
+    // Ragged rows carry their chunk bookkeeping in registers too and pipeline at half that.
+    const int raw = raw_words_per_chunk(P), all = raw + affine_words_per_chunk(P, group);
+    plan->pipe = group < 1024 && all * it <= (ragged ? 16 : 32);
+    // Register allocation aims at 4 waves per SIMD (128 registers per thread).  The widest plans hold more than
+    // that with their operands: they get the registers of 2 waves per SIMD instead of spilling.
+    const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
+    const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? (P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8) * it : 0);
+    plan->min_waves = group >= 1024 ? 4 : held + (ragged ? 3 * it + 16 : 0) > 72 ? 2 : 4;
+}
+
+bool rows_prog_plan(const AxhipRowsProgram &P, RowsProgPlan *plan) {
+    if (P.cols <= 0) return false;
+    if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) return false; // flat elementwise chains have a kernel of their own
+    const int dt = P.input_dtype;
+    const int e = dt == AXHIP_DTYPE_F32 ? 4 : 8;
+    if (P.cols < e) return false;
+    bool ragged = P.cols % e != 0 || !aligned16(P.input) || (P.reduce == AXHIP_RED_NONE && !aligned16(P.output));
+    bool same_size = P.reduce != AXHIP_RED_NONE || elem_size(P.output_dtype) == elem_size(dt);
+    bool used[AXHIP_MAX_OPERANDS] = {};
+    auto mark = [&](const AxhipChainOp *ops, int n) {
+        for (int i = 0; i < n; ++i)
+            if (is_binary(ops[i].op) && ops[i].imm_kind != AXHIP_BK_IMM && ops[i].operand >= 0 && ops[i].operand < P.n_operands) used[ops[i].operand] = true;
+    };
+    mark(P.pre, P.n_pre);
+    mark(P.post, P.n_post);
+    if (P.norm_weight >= 0 && P.norm_weight < P.n_operands) used[P.norm_weight] = true;
+    if (P.norm_bias >= 0 && P.norm_bias < P.n_operands) used[P.norm_bias] = true;
+    for (int i = 0; i < P.n_operands; ++i) {
+        if (!used[i]) continue;
+        const AxhipOperand &o = P.operands[i];
+        if (o.kind == AXHIP_BK_FULL || o.kind == AXHIP_BK_ROWVEC) {
+            if (!aligned16(o.ptr)) ragged = true;
+            if (elem_size(o.dtype) != elem_size(dt)) same_size = false;
+        }
+    }
+    // a ragged row is addressed in 16-byte chunks of every vector it touches: all of them must share the element size
+    if (ragged && !same_size) return false;
+    const int64_t chunks = (P.cols + e - 1) / e;
+    int group, it;
+    if (chunks <= 512) {
+        group = 64;
+        it = chunks <= 64 ? 1 : chunks <= 128 ? 2 : chunks <= 256 ? 4 : 8;
+    } else if (chunks <= 2048) {
+        group = 256;
+        it = chunks <= 1024 ? 4 : 8;
+    } else if (chunks <= 4096 && raw_words_per_chunk(P) <= 8) {
+        group = 1024;
+        it = 4;
+    } else {
+        return false;
+    }
+    rows_prog_plan_for(P, group, it, ragged, plan);
+    return true;
+}
+
+bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsProgSpec *spec) {
+    RowsProgSpec &S = *spec;
+    S = RowsProgSpec{};
+    Builder B(P, S);
+    const int dt = P.input_dtype;
+    const bool fast = P.output_dtype != AXHIP_DTYPE_F32; // the result is rounded to 16 bits: fast activation forms
+    const bool is_norm = P.row_op == AXHIP_ROWOP_LAYERNORM || P.row_op == AXHIP_ROWOP_RMSNORM;
+
+    int w_dt = -1, b_dt = -1, w_slot = -1, b_slot = -1;
+    if (P.norm_weight >= 0) {
+        if (!is_norm || P.norm_weight >= P.n_operands || P.operands[P.norm_weight].kind != AXHIP_BK_ROWVEC) return false;
+        w_dt = P.operands[P.norm_weight].dtype;
+        w_slot = B.pointer_slot(P.norm_weight);
+    }
+    if (P.norm_bias >= 0) {
+        if (P.row_op != AXHIP_ROWOP_LAYERNORM || P.norm_bias >= P.n_operands || P.operands[P.norm_bias].kind != AXHIP_BK_ROWVEC) return false;
+        b_dt = P.operands[P.norm_bias].dtype;
+        b_slot = B.pointer_slot(P.norm_bias);
+    }
+    std::string pre_label, post_label;
+    const std::string pre = B.chain_text(P.pre, P.n_pre, false, fast, &pre_label);
+    const std::string post = B.chain_text(P.post, P.n_post, true, fast, &post_label);
+    if (!B.ok) return false;
+    bool pipe = plan.pipe;
+    const bool resident = P.row_op != AXHIP_ROWOP_NONE && !(is_norm && dt != AXHIP_DTYPE_F32 && P.n_pre == 0);
+    if (resident && B.post_full) pipe = false;
+
+    const int red = P.reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : P.reduce;
+    std::ostringstream c;
+    c << "constexpr int DT_IN = " << dt << ", DT_OUT = " << (P.reduce == AXHIP_RED_NONE ? P.output_dtype : dt) << ";\n";
+    c << "constexpr int GROUP = " << plan.group << ", IT = " << plan.it << ";\n";
+    c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ";\n";
+    c << "constexpr int MIN_WAVES = " << plan.min_waves << ";\n";
+    c << "constexpr int ROWOP = " << P.row_op << ", RED = " << red << ";\n";
+    c << "constexpr int W_DT = " << w_dt << ", B_DT = " << b_dt << ", W_SLOT = " << w_slot << ", B_SLOT = " << b_slot << ";\n";
+    static const char *kind_name[4] = {"FULL", "ROWV", "COLV", "SCAL"};
+    for (int k = 0; k < 4; ++k) {
+        c << "constexpr int N" << kind_name[k] << " = " << B.T.n[k] << ";\n";
+        c << int_table((std::string(kind_name[k]) + "_DT").c_str(), B.T.dt[k], B.T.n[k]);
+        c << int_table((std::string(kind_name[k]) + "_SLOT").c_str(), B.T.slot[k], B.T.n[k]);
+    }
+    c << "constexpr bool HAS_PRE = " << (P.n_pre > 0 ? "true" : "false") << ", POST_FULL = " << (B.post_full ? "true" : "false") << ";\n";
+    S.config = c.str();
+
+    std::ostringstream f;
+    f << "__device__ __forceinline__ float pre_chain(float t, const Env &q, int e) {\n" << pre << "    return t;\n}\n";
+    f << "__device__ __forceinline__ float post_chain(float t, const Env &q, int e) {\n" << post << "    return t;\n}\n";
+    S.chains = f.str();
+
+    char sym[40];
+    snprintf(sym, sizeof(sym), "axp_%016llx", static_cast<unsigned long long>(fnv1a(S.chains, fnv1a(S.config))));
+    S.symbol = sym;
+    S.threads = plan.group > 256 ? plan.group : 256;
+    S.rows_per_block = S.threads / plan.group;
+
+    std::string label = pre_label + rowop_token(P.row_op) + "_" + post_label;
+    if (w_dt >= 0) label += b_dt >= 0 ? "wb_" : "w_";
+    else if (b_dt >= 0) label += "b_";
+    if (red != AXHIP_RED_NONE) label += red == AXHIP_RED_SUM ? "sum_" : red == AXHIP_RED_MAX ? "max_" : "min_";
+    char tail[48];
+    snprintf(tail, sizeof(tail), "%s_g%d_it%d%s", dt_name(dt), plan.group, plan.it, plan.ragged ? "_ragged" : "");
+    S.label = label + tail;
+    return true;
+}
+
+void rows_prog_bind(const AxhipRowsProgram &P, const RowsProgSpec &S, RowsProgArgs *a) {
+    *a = RowsProgArgs{};
+    a->x = P.input;
+    a->y = P.output;
+    a->rows = P.rows;
+    a->cols = P.cols;
+    for (int i = 0; i < S.n_slots; ++i) a->ptr[i] = P.operands[S.slot_operand[i]].ptr;
+    for (int i = 0; i < S.n_imm; ++i) a->imm[i] = S.imm_ref[i].post ? P.post[S.imm_ref[i].index].imm : P.pre[S.imm_ref[i].index].imm;
+    a->eps = P.eps;
+    // a full-size output far larger than the caches is written around them, so that it does not push the launch's own
+    // inputs out of the last-level cache
+    const int64_t out_bytes = P.rows * P.cols * static_cast<int64_t>(elem_size(P.output_dtype));
+    a->stream_out = P.reduce == AXHIP_RED_NONE && out_bytes >= (64ll << 20);
+    a->red_scale = P.reduce == AXHIP_RED_MEAN ? 1.0f / static_cast<float>(P.cols) : 1.0f;
+    a->red_dt = P.output_dtype;
+}
+
+std::string rows_prog_source(const RowsProgSpec &S, const std::string &body) {
+    std::string ns = "ns_" + S.symbol;
+    std::string src;
+    src.reserve(body.size() + S.config.size() + S.chains.size() + 256);
+    src += "#define AXP_NS " + ns + "\n#define AXP_KERNEL_NAME " + S.symbol + "\n";
+    src += "namespace " + ns + " { namespace cfg {\n" + S.config + "} }\n";
+    src += body;
+    src += "\nnamespace " + ns + " {\n" + S.chains + "}\n";
+    return src;
+}
+
+// ------------------------------------------------------------------ kernels built into the library
+namespace {
+std::map<std::string, const void *> &builtin_table() {
+    static std::map<std::string, const void *> t;
+    return t;
+}
+std::mutex &builtin_mutex() {
+    static std::mutex m;
+    return m;
+}
+} // namespace
+
+RowsProgRegistrar::RowsProgRegistrar(const char *key, const void *kernel) {
+    std::lock_guard<std::mutex> lock(builtin_mutex());
+    builtin_table()[key] = kernel;
+}
+
+const void *rows_prog_find_builtin(const std::string &key) {
+    std::lock_guard<std::mutex> lock(builtin_mutex());
+    auto it = builtin_table().find(key);
+    return it == builtin_table().end() ? nullptr : it->second;
+}
+
+} // namespace axhip

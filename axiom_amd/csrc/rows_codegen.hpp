@@ -1,0 +1,77 @@
+// Compiled fused-row programs: from an AxhipRowsProgram to the source text of its kernel.
+//
+// Every row program (pre chain -> row op -> post chain -> optional row reduction) whose rows fit a register plan has
+// one kernel of its own: rows_prog.inc compiled with a small configuration text in front (element types, plan, the
+// two chains as straight-line code).  The same generator serves two users:
+//   - the build, which writes the kernels of the common program shapes to source files that hipcc compiles into the
+//     library (the counterpart of Axiom's known fused patterns, src/graph/fused_patterns.cpp:12-71), and
+//   - the library at run time, which compiles any other shape through hipRTC the first time it is seen (the
+//     counterpart of the reference's any-DAG-to-one-program graph compiler,
+//     src/backends/metal/mpsgraph_graph_compiler.mm:706-944).
+// Plain host C++: no HIP types, so that the build's generator tool compiles with g++.
+#pragma once
+
+#include <cstdint>
+#include <string>
+
+#include "axhip.h"
+
+namespace axhip {
+
+// kernel arguments; rows_prog.inc declares the same layout as axp::Args
+struct RowsProgArgs {
+    const void *x;
+    void *y;
+    int64_t rows, cols;
+    const void *ptr[8];
+    float imm[32];
+    float eps;
+    int32_t stream_out;
+    float red_scale;  // 1, or 1/cols for a mean
+    int32_t red_dt;   // element type of a reduced [rows] output
+};
+
+struct RowsProgPlan {
+    int group = 0, it = 0; // threads per row, 16-byte input chunks per thread
+    bool ragged = false;   // rows are not whole aligned vectors
+    bool pipe = false;     // the next row is requested before the current one is computed
+    int min_waves = 4;     // waves per SIMD the kernel's register allocation aims for
+};
+
+// everything that is compiled into one kernel
+struct RowsProgSpec {
+    std::string config;     // configuration text; doubles as the cache key
+    std::string chains;     // definitions of the two chain functions (appended after the body)
+    std::string label;      // human-readable kernel label, e.g. layernorm_gelu_bf16_g64_it8
+    std::string symbol;     // extern "C" name of the kernel: axp_<hash of config and chains>
+    int threads = 256;
+    int rows_per_block = 4;
+    int n_slots = 0;
+    int slot_operand[8] = {}; // pointer slot -> index into AxhipRowsProgram::operands
+    int n_imm = 0;
+    struct ImmRef { bool post; int index; } imm_ref[32] = {}; // immediate slot -> chain position
+};
+
+// Picks the register plan; false when the program does not qualify (no row op and no reduction, rows too long or
+// too short, a vector operand whose element size keeps a ragged row from its 16-byte chunks): the interpreter takes it.
+bool rows_prog_plan(const AxhipRowsProgram &P, RowsProgPlan *plan);
+// The plan with its shape given (the build's generator enumerates the shapes itself).
+void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan);
+
+// Builds the kernel's configuration for a program under a plan; false when the program names an operand kind or
+// op code the generator does not know.
+bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsProgSpec *spec);
+
+// Fills the kernel arguments of one launch.
+void rows_prog_bind(const AxhipRowsProgram &P, const RowsProgSpec &spec, RowsProgArgs *args);
+
+// Full source text of the kernel: configuration, `body` (the text of rows_prog.inc), chain functions.
+std::string rows_prog_source(const RowsProgSpec &spec, const std::string &body);
+
+// ---- kernels compiled into the library register themselves here (static initialisers of the generated files)
+struct RowsProgRegistrar {
+    RowsProgRegistrar(const char *key, const void *kernel);
+};
+const void *rows_prog_find_builtin(const std::string &key);
+
+} // namespace axhip

@@ -1,0 +1,242 @@
+// Run-time side of the compiled fused-row programs: finds the kernel of a program among those built into the
+// library, compiles it through hipRTC when it is not there, and launches it as a persistent grid.
+#include "rows_prog.hpp"
+
+#include <hip/hiprtc.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "rows_prog_body.h" // kRowsProgBody: the text of rows_prog.inc, written by the build
+
+namespace axhip {
+namespace {
+
+// A program with everything a kernel does not depend on taken out (addresses, extents along rows, immediate
+// values): two programs with equal keys run the same kernel under the same plan.
+struct StructKey {
+    AxhipRowsProgram p;
+};
+
+void make_struct_key(const AxhipRowsProgram &P, StructKey *k) {
+    memset(k, 0, sizeof(*k));
+    AxhipRowsProgram &q = k->p;
+    auto align_tag = [](const void *p) { return reinterpret_cast<const void *>(static_cast<uintptr_t>((reinterpret_cast<uintptr_t>(p) & 15u) == 0)); };
+    q.cols = P.cols;
+    q.input = align_tag(P.input);
+    q.input_dtype = P.input_dtype;
+    q.n_operands = P.n_operands;
+    for (int i = 0; i < P.n_operands && i < AXHIP_MAX_OPERANDS; ++i) {
+        q.operands[i].ptr = align_tag(P.operands[i].ptr);
+        q.operands[i].dtype = P.operands[i].dtype;
+        q.operands[i].kind = P.operands[i].kind;
+    }
+    auto copy_chain = [](const AxhipChainOp *src, int n, AxhipChainOp *dst) {
+        for (int i = 0; i < n && i < AXHIP_MAX_CHAIN; ++i) {
+            dst[i].op = src[i].op;
+            dst[i].imm_kind = src[i].imm_kind;
+            dst[i].operand = src[i].imm_kind == AXHIP_BK_IMM ? -1 : src[i].operand;
+        }
+    };
+    q.n_pre = P.n_pre;
+    copy_chain(P.pre, P.n_pre, q.pre);
+    q.row_op = P.row_op;
+    q.norm_weight = P.norm_weight;
+    q.norm_bias = P.norm_bias;
+    q.n_post = P.n_post;
+    copy_chain(P.post, P.n_post, q.post);
+    q.reduce = P.reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : P.reduce;
+    q.output = const_cast<void *>(align_tag(P.output));
+    q.output_dtype = P.output_dtype;
+}
+
+uint64_t hash_bytes(const void *p, size_t n) {
+    const unsigned char *b = static_cast<const unsigned char *>(p);
+    uint64_t h = 14695981039346656037ull;
+    for (size_t i = 0; i < n; ++i) {
+        h ^= b[i];
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+struct Kernel {
+    const void *builtin = nullptr; // address of a kernel compiled into the library, or
+    hipModule_t module = nullptr;  // a module compiled at run time
+    hipFunction_t function = nullptr;
+    int blocks_per_cu = 0;         // resident blocks per compute unit (0: not yet asked)
+};
+
+struct Entry {
+    StructKey key;
+    bool eligible = false;
+    RowsProgSpec spec;
+    std::shared_ptr<Kernel> kernel; // null until the program is first launched (a name query compiles nothing)
+    bool is_builtin = false;
+    bool jit_failed = false;
+};
+
+std::mutex g_mutex;
+std::unordered_multimap<uint64_t, std::unique_ptr<Entry>> g_entries;      // by structure
+std::unordered_map<std::string, std::shared_ptr<Kernel>> g_kernels;      // by configuration text
+int g_num_cus = 0;
+
+// read at every dispatch (a getenv is cheap against a launch), so that a test can switch within one process
+bool jit_enabled() {
+    const char *e = getenv("AXHIP_JIT");
+    return !(e && e[0] == '0');
+}
+
+Entry *find_or_make_entry(const AxhipRowsProgram &P) {
+    StructKey k;
+    make_struct_key(P, &k);
+    const uint64_t h = hash_bytes(&k, sizeof(k));
+    auto range = g_entries.equal_range(h);
+    for (auto it = range.first; it != range.second; ++it)
+        if (memcmp(&it->second->key, &k, sizeof(k)) == 0) return it->second.get();
+    auto e = std::make_unique<Entry>();
+    e->key = k;
+    RowsProgPlan plan;
+    e->eligible = rows_prog_plan(P, &plan) && rows_prog_spec(P, plan, &e->spec);
+    if (e->eligible) e->is_builtin = rows_prog_find_builtin(e->spec.config + e->spec.chains) != nullptr;
+    Entry *raw = e.get();
+    g_entries.emplace(h, std::move(e));
+    return raw;
+}
+
+// compiles the program's kernel through hipRTC; on failure the reason goes to the library's error text
+std::shared_ptr<Kernel> compile(const RowsProgSpec &spec) {
+    const std::string src = rows_prog_source(spec, kRowsProgBody);
+    hiprtcProgram prog = nullptr;
+    if (hiprtcCreateProgram(&prog, src.c_str(), (spec.symbol + ".hip").c_str(), 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+        set_last_error("fused rows: hiprtcCreateProgram failed for %s", spec.label.c_str());
+        return nullptr;
+    }
+    const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    const hiprtcResult r = hiprtcCompileProgram(prog, static_cast<int>(sizeof(opts) / sizeof(opts[0])), opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0;
+        hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, '\0');
+        if (n) hiprtcGetProgramLog(prog, log.data());
+        set_last_error("fused rows: run-time compilation of %s failed: %s: %.300s", spec.label.c_str(), hiprtcGetErrorString(r), log.c_str());
+        hiprtcDestroyProgram(&prog);
+        return nullptr;
+    }
+    size_t size = 0;
+    hiprtcGetCodeSize(prog, &size);
+    std::vector<char> code(size);
+    hiprtcGetCode(prog, code.data());
+    hiprtcDestroyProgram(&prog);
+    auto k = std::make_shared<Kernel>();
+    hipError_t e = hipModuleLoadData(&k->module, code.data());
+    if (e == hipSuccess) e = hipModuleGetFunction(&k->function, k->module, spec.symbol.c_str());
+    if (e != hipSuccess) {
+        set_last_error("fused rows: loading the compiled %s failed: %s", spec.label.c_str(), hipGetErrorString(e));
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return k;
+}
+
+} // namespace
+
+bool rows_prog_compile_only(const AxhipRowsProgram &P, std::string *label, std::string *error) {
+    RowsProgPlan plan;
+    RowsProgSpec spec;
+    if (!rows_prog_plan(P, &plan) || !rows_prog_spec(P, plan, &spec)) {
+        if (error) *error = "the program does not qualify for a compiled kernel";
+        return false;
+    }
+    if (label) *label = spec.label;
+    const std::string src = rows_prog_source(spec, kRowsProgBody);
+    hiprtcProgram prog = nullptr;
+    if (hiprtcCreateProgram(&prog, src.c_str(), "probe.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+        if (error) *error = "hiprtcCreateProgram failed";
+        return false;
+    }
+    const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    const hiprtcResult r = hiprtcCompileProgram(prog, static_cast<int>(sizeof(opts) / sizeof(opts[0])), opts);
+    if (r != HIPRTC_SUCCESS && error) {
+        size_t n = 0;
+        hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, '\0');
+        if (n) hiprtcGetProgramLog(prog, log.data());
+        *error = std::string(hiprtcGetErrorString(r)) + ": " + log;
+    }
+    hiprtcDestroyProgram(&prog);
+    return r == HIPRTC_SUCCESS;
+}
+
+bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, char *name, size_t name_len, int *rc) {
+    if (rc) *rc = AXHIP_OK;
+    if (P.rows <= 0 || P.cols <= 0 || P.rows >= (int64_t(1) << 31)) return false;
+    std::shared_ptr<Kernel> kernel;
+    RowsProgArgs args;
+    int threads = 0, rows_per_block = 1;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        Entry *e = find_or_make_entry(P);
+        if (!e->eligible) return false;
+        if (!e->is_builtin && (!jit_enabled() || e->jit_failed)) return false;
+        if (name) snprintf(name, name_len, "%s%s", e->is_builtin ? "rows_static_" : "rows_jit_", e->spec.label.c_str());
+        if (!launch) return true;
+        if (!e->kernel) {
+            const std::string key = e->spec.config + e->spec.chains;
+            auto it = g_kernels.find(key);
+            if (it != g_kernels.end()) {
+                e->kernel = it->second;
+            } else {
+                std::shared_ptr<Kernel> k;
+                if (e->is_builtin) {
+                    k = std::make_shared<Kernel>();
+                    k->builtin = rows_prog_find_builtin(key);
+                } else {
+                    k = compile(e->spec);
+                    if (!k) {
+                        e->jit_failed = true; // the interpreter serves this program from now on
+                        return false;
+                    }
+                }
+                g_kernels.emplace(key, k);
+                e->kernel = k;
+            }
+        }
+        kernel = e->kernel;
+        if (kernel->blocks_per_cu == 0) {
+            int n = 0;
+            hipError_t err = kernel->builtin ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->builtin, e->spec.threads, 0)
+                                             : hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->function, e->spec.threads, 0);
+            if (err != hipSuccess) (void)hipGetLastError();
+            kernel->blocks_per_cu = err == hipSuccess && n > 0 ? n : 2;
+        }
+        if (g_num_cus == 0) {
+            int dev = 0, n = 0;
+            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+                (void)hipGetLastError();
+                n = 256;
+            }
+            g_num_cus = n;
+        }
+        rows_prog_bind(P, e->spec, &args);
+        threads = e->spec.threads;
+        rows_per_block = e->spec.rows_per_block;
+    }
+    const int64_t row_groups = (P.rows + rows_per_block - 1) / rows_per_block;
+    const int64_t resident = static_cast<int64_t>(kernel->blocks_per_cu) * g_num_cus;
+    const unsigned grid = static_cast<unsigned>(row_groups < resident ? row_groups : resident);
+    void *params[] = {&args};
+    hipError_t err = kernel->builtin ? hipLaunchKernel(kernel->builtin, dim3(grid), dim3(threads), params, 0, s)
+                                     : hipModuleLaunchKernel(kernel->function, grid, 1, 1, threads, 1, 1, 0, s, params, nullptr);
+    if (err != hipSuccess) {
+        set_last_error("fused rows: launch failed: %s", hipGetErrorString(err));
+        if (rc) *rc = static_cast<int>(err);
+    }
+    return true;
+}
+
+} // namespace axhip

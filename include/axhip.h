@@ -195,8 +195,16 @@ typedef struct {
 } AxhipRowsProgram;
 
 int axhip_fused_rows(const AxhipRowsProgram *program_host, void *stream);
-/* name of the kernel variant axhip_fused_rows would launch */
+/* name of the kernel variant axhip_fused_rows would launch: "rows_static_..." a kernel of
+ * this program shape built into the library, "rows_jit_..." one the library compiles (hipRTC)
+ * when the shape is first launched -- the counterpart of the reference compiling a graph on
+ * first use (mpsgraph_graph_compiler.mm:706-944) -- anything else the generic interpreter.
+ * AXHIP_JIT=0 in the environment turns run-time compilation off. */
 const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *program_host);
+/* Compiles the kernel of a "rows_jit_" program now (for gfx950; needs no device) and reports
+ * a compile error instead of leaving it to the first launch, which would fall back to the
+ * interpreter.  Pointers in the program are only looked at for their alignment. */
+int axhip_fused_rows_prepare(const AxhipRowsProgram *program_host);
 
 /* Elementwise chain followed by a reduction over ALL elements -> one value
  * (the FusedReductionStep of include/axiom/graph/compiled_graph.hpp:41-70,

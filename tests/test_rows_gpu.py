@@ -211,6 +211,12 @@ def test_full_size_c2_and_c3_properties():
     assert np.max(np.abs(y[:256] - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
 
 
+@pytest.fixture
+def no_jit(monkeypatch):
+    """Run-time compilation off: programs without a built-in kernel run on the interpreter."""
+    monkeypatch.setenv("AXHIP_JIT", "0")
+
+
 def test_empty_inputs_are_no_ops():
     x = np.zeros((0, 16), np.float32)
     assert gh.Rows(x, F32).unary("relu").run().shape == (0, 16)
@@ -237,11 +243,11 @@ def test_mixed_chains_around_row_ops_match_oracle():
     d = (axo.to_f32(fb, BF16) - axo.to_f32(xb, BF16)).astype(np.float64)
     r = d / np.sqrt((d * d).mean(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16)
     assert np.max(np.abs(got - 1 / (1 + np.exp(-r)))) < 2e-2
-    # two different full-size operands do not fit the specialised kernels: the interpreter takes over
+    # two different full-size operands: no built-in kernel has that shape, the library compiles one when it is first launched
     f2 = g.normal((48, 2048))
     p = gh.Rows(x, F32).binary("add", f).binary("mul", f2).row_op("softmax")
     got = p.run()
-    assert p.kernel_name().startswith("rows_resident_"), p.kernel_name()
+    assert p.kernel_name() == "rows_jit_addf_mulf_softmax_f32_g64_it8", p.kernel_name()
     assert close32(got, axo.softmax((x + f) * f2))
     # row dot product: sum(x * f) per row
     p = gh.Rows(x, F32).binary("mul", f)
@@ -284,7 +290,7 @@ def test_fast_activations_after_a_norm_in_16_bit(post):
     w, b = axo.to_bits(g.uniform((1024,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((1024,), -0.5, 0.5), BF16)
     prog = gh.Rows(x, BF16).row_op("layernorm", 1e-5, w=w, b=b).unary(post)
     got = axo.to_f32(prog.run(), BF16).astype(np.float64)
-    assert prog.kernel_name().startswith("rows_static_layernorm_bf16"), prog.kernel_name()
+    assert prog.kernel_name() == ("rows_static_" if post == "silu" else "rows_jit_") + f"layernorm_{post}_wb_bf16_g64_it2", prog.kernel_name()
     xf = axo.to_f32(x, BF16).astype(np.float64)
     n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
     want = {"silu": n / (1 + np.exp(-n)), "sigmoid": 1 / (1 + np.exp(-n)), "tanh": np.tanh(n)}[post]
@@ -295,7 +301,7 @@ def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
     """Rows beyond the 32 KiB the specialised kernels hold: up to 4096 16-byte chunks stay in the registers of a
     1024-thread block (one read), longer ones are streamed in passes."""
     g = axo.PCG64(123)
-    for cols, plan in ((12000, "rows_resident_g1024_it4_e4"), (16384, "rows_resident_g1024_it4_e4"), (20000, "rows_streamed_e4")):
+    for cols, plan in ((12000, "rows_jit_softmax_f32_g1024_it4"), (16384, "rows_jit_softmax_f32_g1024_it4"), (20000, "rows_streamed_e4")):
         x = (g.normal((3, cols)) * 2).astype(np.float32)
         p = gh.Rows(x, F32).row_op("softmax")
         got = p.run()
@@ -305,7 +311,7 @@ def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
     w, b = axo.to_bits(g.uniform((30000,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((30000,), -0.5, 0.5), BF16)
     p = gh.Rows(xb, BF16).row_op("layernorm", 1e-5, w=w, b=b).unary("gelu")
     got = axo.to_f32(p.run(), BF16).astype(np.float64)
-    assert p.kernel_name() == "rows_resident_g1024_it4_e8", p.kernel_name()
+    assert p.kernel_name() == "rows_jit_layernorm_gelu_wb_bf16_g1024_it4", p.kernel_name()
     xf = axo.to_f32(xb, BF16).astype(np.float64)
     n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
     import math
@@ -322,15 +328,15 @@ def test_unary_then_row_reduction_runs_on_the_specialised_reduce_kernels():
     xbf = axo.to_f32(xb, BF16).astype(np.float64)
     p = gh.Rows(x, F32).unary("relu")
     got = p.run(reduce="sum")
-    assert p.kernel_name().startswith("rows_static_reduce_sum_f32"), p.kernel_name()
+    assert p.kernel_name().startswith("rows_static_relu_reduce_sum_f32"), p.kernel_name()
     assert np.allclose(got, np.maximum(x.astype(np.float64), 0).sum(-1), rtol=1e-4, atol=1e-3)
     p = gh.Rows(xb, BF16, F32).unary("square")
     got = p.run(reduce="mean")
-    assert p.kernel_name().startswith("rows_static_reduce_sum_bf16"), p.kernel_name()
+    assert p.kernel_name().startswith("rows_static_square_reduce_sum_bf16"), p.kernel_name()
     assert np.allclose(got, (xbf * xbf).mean(-1), rtol=1e-4, atol=1e-5)
     p = gh.Rows(xb, BF16).unary("abs")
     got = axo.to_f32(p.run(reduce="max"), BF16)
-    assert p.kernel_name().startswith("rows_static_reduce_max_bf16"), p.kernel_name()
+    assert p.kernel_name().startswith("rows_static_abs_reduce_max_bf16"), p.kernel_name()
     assert np.array_equal(got.reshape(-1), np.abs(xbf).max(-1).astype(np.float32))
     # an fp32 result keeps the exact activation (no polynomial GELU under a sum)
     import math
@@ -407,7 +413,7 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
             assert np.array_equal(got.reshape(-1).astype(np.float64), fn(xf, axis=-1)), red  # exact: a selection
         p = gh.Rows(xs, dt).unary("abs").binary("mul", ys).row_op("softmax")
         got = out(p.run())
-        assert p.kernel_name().startswith("rows_resident_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+        assert p.kernel_name().startswith("rows_jit_abs_mulf_softmax_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
         lg = np.abs(f(xs)) * f(ys)
         e = np.exp(lg - lg.max(-1, keepdims=True))
         assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
@@ -447,3 +453,30 @@ def test_bases_that_are_only_element_aligned(dt):
     assert p.kernel_name().endswith("_ragged"), p.kernel_name()
     e = np.exp(f(x) - f(x).max(-1, keepdims=True))
     assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < (1e-4 if dt == F32 else 2e-2)
+
+
+def test_interpreter_serves_programs_without_a_built_in_kernel_when_run_time_compilation_is_off(no_jit):
+    """AXHIP_JIT=0: the shapes the library would compile on first use run on the generic interpreter instead
+    (resident plans, their ragged variant, the 1024-thread plan), with the same results."""
+    g = axo.PCG64(4242)
+    x, f, f2 = g.normal((48, 2048)), g.normal((48, 2048)), g.normal((48, 2048))
+    p = gh.Rows(x, F32).binary("add", f).binary("mul", f2).row_op("softmax")
+    got = p.run()
+    assert p.kernel_name() == "rows_resident_g256_it2_e4", p.kernel_name()
+    assert close32(got, axo.softmax((x + f) * f2))
+    xs, ys = axo.to_bits(g.normal((11, 1001)) * 2, BF16), axo.to_bits(g.normal((11, 1001)), BF16)
+    p = gh.Rows(xs, BF16).unary("abs").binary("mul", ys).row_op("softmax")
+    got = axo.to_f32(p.run(), BF16).astype(np.float64)
+    assert p.kernel_name().startswith("rows_resident_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+    lg = np.abs(axo.to_f32(xs, BF16).astype(np.float64)) * axo.to_f32(ys, BF16)
+    e = np.exp(lg - lg.max(-1, keepdims=True))
+    assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < 2e-2
+    xl = (g.normal((3, 12000)) * 2).astype(np.float32)
+    p = gh.Rows(xl, F32).row_op("softmax")
+    got = p.run()
+    assert p.kernel_name() == "rows_resident_g1024_it4_e4", p.kernel_name()
+    assert close32(got, axo.softmax(xl))
+    # a built-in shape is not affected by the switch
+    p = gh.Rows(x, F32).row_op("softmax")
+    p.run()
+    assert p.kernel_name() == "rows_static_softmax_f32_g64_it8", p.kernel_name()
