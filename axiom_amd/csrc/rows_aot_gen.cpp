@@ -150,7 +150,9 @@ int main(int argc, char **argv) {
     const std::string dir = argv[1];
     const int n_files = atoi(argv[2]);
     if (n_files <= 0) return 2;
-    static const int plans[][2] = {{64, 1}, {64, 2}, {64, 4}, {64, 8}, {256, 4}, {256, 8}};
+    // a wavefront per row up to 512 chunks (1, 2, 4, 8 chunks per lane, and 3 / 5 / 6 for the row lengths between the
+    // powers of two: 1280, 1536, 2560, 3072 ... columns of 16-bit data), a 256-thread block per row beyond
+    static const int plans[][2] = {{64, 1}, {64, 2}, {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}, {256, 3}, {256, 4}, {256, 8}};
     std::vector<RowsProgSpec> specs;
     std::set<std::string> seen;
     for (int dt : {AXHIP_DTYPE_F32, AXHIP_DTYPE_F16, AXHIP_DTYPE_BF16})

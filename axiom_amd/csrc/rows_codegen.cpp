@@ -242,19 +242,18 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     plan->it = it;
     plan->ragged = ragged;
     // Pipelining keeps a second set of raw words alive: worth it while that set is at most 32 registers (a 16-bit
-    // row of 4096 columns per wavefront, or a row with one operand at half that).  The 1024-thread plan has 128
-    // registers per thread and none to spare.
-    // Ragged rows carry their chunk bookkeeping in registers too and pipeline at half that.
+    // row of 4096 columns per wavefront, or a row with one operand at half that).  Ragged rows carry their chunk
+    // bookkeeping in registers too and pipeline at half that.
     const int raw = raw_words_per_chunk(P), all = raw + affine_words_per_chunk(P, group);
-    plan->pipe = group < 1024 && all * it <= (ragged ? 16 : 32);
+    plan->pipe = all * it <= (ragged ? 16 : 32);
     // Register allocation aims at 4 waves per SIMD (128 registers per thread).  The widest plans hold more than
     // that with their operands: they get the registers of 2 waves per SIMD instead of spilling.
     const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
     const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? (P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8) * it : 0);
-    plan->min_waves = group >= 1024 ? 4 : held + (ragged ? 3 * it + 16 : 0) > 72 ? 2 : 4;
+    plan->min_waves = held + (ragged ? 3 * it + 16 : 0) > 72 ? 2 : 4;
 }
 
-bool rows_prog_plan(const AxhipRowsProgram &P, RowsProgPlan *plan) {
+bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     if (P.cols <= 0) return false;
     if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) return false; // flat elementwise chains have a kernel of their own
     const int dt = P.input_dtype;
@@ -282,18 +281,35 @@ bool rows_prog_plan(const AxhipRowsProgram &P, RowsProgPlan *plan) {
     // a ragged row is addressed in 16-byte chunks of every vector it touches: all of them must share the element size
     if (ragged && !same_size) return false;
     const int64_t chunks = (P.cols + e - 1) / e;
-    int group, it;
-    if (chunks <= 512) {
-        group = 64;
-        it = chunks <= 64 ? 1 : chunks <= 128 ? 2 : chunks <= 256 ? 4 : 8;
-    } else if (chunks <= 2048) {
-        group = 256;
-        it = chunks <= 1024 ? 4 : 8;
-    } else if (chunks <= 4096 && raw_words_per_chunk(P) <= 8) {
-        group = 1024;
-        it = 4;
+    int group = 0, it = 0;
+    if (!tight) {
+        // the shapes the build compiles (rows_aot_gen.cpp): a wavefront per row with 1, 2, 3, 4, 5, 6 or 8 chunks per
+        // lane, a 256-thread block per row with 3, 4 or 8 chunks per thread
+        if (chunks <= 512) {
+            group = 64;
+            it = static_cast<int>((chunks + 63) / 64);
+            if (it == 7) it = 8;
+        } else if (chunks <= 2048) {
+            group = 256;
+            it = chunks <= 768 ? 3 : chunks <= 1024 ? 4 : 8;
+        } else {
+            return false;
+        }
     } else {
-        return false;
+        // the tightest fit among 64, 256 and 512 threads per row with up to 8 chunks each: fewest chunk slots (idle lanes
+        // still issue their loads and arithmetic), then the smaller group
+        static const int groups[3] = {64, 256, 512};
+        int64_t best = 0;
+        for (int i = 0; i < 3; ++i) {
+            const int64_t n = (chunks + groups[i] - 1) / groups[i];
+            if (n > 8) continue;
+            if (group == 0 || n * groups[i] < best) {
+                group = groups[i];
+                it = static_cast<int>(n);
+                best = n * groups[i];
+            }
+        }
+        if (group == 0) return false;
     }
     rows_prog_plan_for(P, group, it, ragged, plan);
     return true;

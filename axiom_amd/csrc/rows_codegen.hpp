@@ -36,6 +36,7 @@ struct RowsProgPlan {
     bool ragged = false;   // rows are not whole aligned vectors
     bool pipe = false;     // the next row is requested before the current one is computed
     int min_waves = 4;     // waves per SIMD the kernel's register allocation aims for
+    int slots() const { return group * it; }
 };
 
 // everything that is compiled into one kernel
@@ -54,7 +55,9 @@ struct RowsProgSpec {
 
 // Picks the register plan; false when the program does not qualify (no row op and no reduction, rows too long or
 // too short, a vector operand whose element size keeps a ragged row from its 16-byte chunks): the interpreter takes it.
-bool rows_prog_plan(const AxhipRowsProgram &P, RowsProgPlan *plan);
+// tight = false: among the plan shapes the build compiles (64 or 256 threads per row, a few chunk counts per thread);
+// tight = true: the plan with the fewest idle chunk slots for this row length (64, 256 or 512 threads per row, any chunk count up to 8).
+bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan);
 // The plan with its shape given (the build's generator enumerates the shapes itself).
 void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan);
 

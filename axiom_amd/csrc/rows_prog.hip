@@ -78,6 +78,9 @@ struct Entry {
     std::shared_ptr<Kernel> kernel; // null until the program is first launched (a name query compiles nothing)
     bool is_builtin = false;
     bool jit_failed = false;
+    bool has_builtin_alternative = false; // a built-in kernel under a looser plan exists next to the tight plan's spec
+    RowsProgSpec builtin_spec;
+    std::shared_ptr<Kernel> alt_kernel;
 };
 
 std::mutex g_mutex;
@@ -100,9 +103,26 @@ Entry *find_or_make_entry(const AxhipRowsProgram &P) {
         if (memcmp(&it->second->key, &k, sizeof(k)) == 0) return it->second.get();
     auto e = std::make_unique<Entry>();
     e->key = k;
-    RowsProgPlan plan;
-    e->eligible = rows_prog_plan(P, &plan) && rows_prog_spec(P, plan, &e->spec);
-    if (e->eligible) e->is_builtin = rows_prog_find_builtin(e->spec.config + e->spec.chains) != nullptr;
+    // Two candidate plans: the tightest fit for this row length, and the nearest of the shapes the build compiles.
+    // The built-in kernel wins when it exists and its idle lanes cost at most 15 % more chunk slots; otherwise the
+    // tight plan's kernel is compiled at first launch.
+    RowsProgPlan tight, stock;
+    RowsProgSpec stock_spec;
+    const bool has_tight = rows_prog_plan(P, true, &tight) && rows_prog_spec(P, tight, &e->spec);
+    const bool has_stock = rows_prog_plan(P, false, &stock) && rows_prog_spec(P, stock, &stock_spec) &&
+                           rows_prog_find_builtin(stock_spec.config + stock_spec.chains) != nullptr;
+    e->eligible = has_tight || has_stock;
+    e->has_builtin_alternative = false;
+    if (has_stock && (!has_tight || stock.slots() * 100 <= tight.slots() * 115)) {
+        e->spec = stock_spec;
+        e->is_builtin = true;
+    } else if (has_tight) {
+        e->is_builtin = rows_prog_find_builtin(e->spec.config + e->spec.chains) != nullptr;
+        if (!e->is_builtin && has_stock) { // kept for when run-time compilation is off or fails
+            e->has_builtin_alternative = true;
+            e->builtin_spec = stock_spec;
+        }
+    }
     Entry *raw = e.get();
     g_entries.emplace(h, std::move(e));
     return raw;
@@ -148,7 +168,7 @@ std::shared_ptr<Kernel> compile(const RowsProgSpec &spec) {
 bool rows_prog_compile_only(const AxhipRowsProgram &P, std::string *label, std::string *error) {
     RowsProgPlan plan;
     RowsProgSpec spec;
-    if (!rows_prog_plan(P, &plan) || !rows_prog_spec(P, plan, &spec)) {
+    if (!rows_prog_plan(P, true, &plan) || !rows_prog_spec(P, plan, &spec)) {
         if (error) *error = "the program does not qualify for a compiled kernel";
         return false;
     }
@@ -182,10 +202,14 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
         std::lock_guard<std::mutex> lock(g_mutex);
         Entry *e = find_or_make_entry(P);
         if (!e->eligible) return false;
-        if (!e->is_builtin && (!jit_enabled() || e->jit_failed)) return false;
-        if (name) snprintf(name, name_len, "%s%s", e->is_builtin ? "rows_static_" : "rows_jit_", e->spec.label.c_str());
-        if (!launch) return true;
-        if (!e->kernel) {
+        // the tight plan's kernel, compiled on first launch -- or, with run-time compilation off or failed, the
+        // looser built-in plan when there is one, else the interpreter
+        bool use_alt = false;
+        if (!e->is_builtin && (!jit_enabled() || e->jit_failed)) {
+            if (!e->has_builtin_alternative) return false;
+            use_alt = true;
+        }
+        if (!use_alt && !e->kernel && launch) {
             const std::string key = e->spec.config + e->spec.chains;
             auto it = g_kernels.find(key);
             if (it != g_kernels.end()) {
@@ -198,19 +222,29 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
                 } else {
                     k = compile(e->spec);
                     if (!k) {
-                        e->jit_failed = true; // the interpreter serves this program from now on
-                        return false;
+                        e->jit_failed = true;
+                        if (!e->has_builtin_alternative) return false;
+                        use_alt = true;
                     }
                 }
-                g_kernels.emplace(key, k);
-                e->kernel = k;
+                if (k) {
+                    g_kernels.emplace(key, k);
+                    e->kernel = k;
+                }
             }
         }
-        kernel = e->kernel;
+        if (use_alt && !e->alt_kernel) {
+            e->alt_kernel = std::make_shared<Kernel>();
+            e->alt_kernel->builtin = rows_prog_find_builtin(e->builtin_spec.config + e->builtin_spec.chains);
+        }
+        const RowsProgSpec &spec = use_alt ? e->builtin_spec : e->spec;
+        if (name) snprintf(name, name_len, "%s%s", (use_alt || e->is_builtin) ? "rows_static_" : "rows_jit_", spec.label.c_str());
+        if (!launch) return true;
+        kernel = use_alt ? e->alt_kernel : e->kernel;
         if (kernel->blocks_per_cu == 0) {
             int n = 0;
-            hipError_t err = kernel->builtin ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->builtin, e->spec.threads, 0)
-                                             : hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->function, e->spec.threads, 0);
+            hipError_t err = kernel->builtin ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->builtin, spec.threads, 0)
+                                             : hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->function, spec.threads, 0);
             if (err != hipSuccess) (void)hipGetLastError();
             kernel->blocks_per_cu = err == hipSuccess && n > 0 ? n : 2;
         }
@@ -222,13 +256,16 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
             }
             g_num_cus = n;
         }
-        rows_prog_bind(P, e->spec, &args);
-        threads = e->spec.threads;
-        rows_per_block = e->spec.rows_per_block;
+        rows_prog_bind(P, spec, &args);
+        threads = spec.threads;
+        rows_per_block = spec.rows_per_block;
     }
     const int64_t row_groups = (P.rows + rows_per_block - 1) / rows_per_block;
+    // As many blocks as fit on the device at once, then fewer, so that every block walks the same number of rows
+    // (4096 row groups on 1280 resident blocks would leave most blocks idle during a fourth pass: 1024 blocks of 4).
     const int64_t resident = static_cast<int64_t>(kernel->blocks_per_cu) * g_num_cus;
-    const unsigned grid = static_cast<unsigned>(row_groups < resident ? row_groups : resident);
+    const int64_t passes = (row_groups + resident - 1) / resident;
+    const unsigned grid = static_cast<unsigned>((row_groups + passes - 1) / passes);
     void *params[] = {&args};
     hipError_t err = kernel->builtin ? hipLaunchKernel(kernel->builtin, dim3(grid), dim3(threads), params, 0, s)
                                      : hipModuleLaunchKernel(kernel->function, grid, 1, 1, threads, 1, 1, 0, s, params, nullptr);

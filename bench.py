@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gfx950 backend on BASELINE.json's headline workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sdpa|chains|gemm|f32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sdpa|chains|gemm|f32|survey]
 
 A step is one pass of the hot path over one batch of synthetic input already
 resident in HBM: causal bf16 scaled-dot-product attention, B=4 H=32 S=4096
@@ -214,6 +214,139 @@ def bench_chains(torch, capi, stream, steps, warmup):
     return res
 
 
+
+class _Prog:
+    """A row program over torch device tensors (bench-side builder for the survey)."""
+
+    def __init__(self, capi, x, out_dtype=None):
+        import torch
+
+        self.capi, self.x, self.keep = capi, x, []
+        self.dt = {torch.float32: capi.DTYPE_F32, torch.float16: capi.DTYPE_F16, torch.bfloat16: capi.DTYPE_BF16}[x.dtype]
+        self.p = capi.RowsProgram()
+        self.p.rows, self.p.cols = x.shape
+        self.p.input, self.p.input_dtype = x.data_ptr(), self.dt
+        self.p.norm_weight = self.p.norm_bias = -1
+        self.post_stage = False
+        self.read_bytes = x.numel() * x.element_size()
+        self.out_dtype = out_dtype
+
+    def _operand(self, t, kind):
+        i = self.p.n_operands
+        self.keep.append(t)
+        self.p.operands[i].ptr, self.p.operands[i].kind = t.data_ptr(), self.capi.BK[kind]
+        self.p.operands[i].dtype = self.dt if t.dtype == self.x.dtype else self.capi.DTYPE_F32
+        self.p.n_operands = i + 1
+        self.read_bytes += t.numel() * t.element_size()
+        return i
+
+    def op(self, name, operand=None, kind="full", imm=None):
+        chain, n = (self.p.post, self.p.n_post) if self.post_stage else (self.p.pre, self.p.n_pre)
+        chain[n].op = self.capi.OP[name]
+        chain[n].operand = -1 if operand is None else self._operand(operand, kind)
+        if imm is not None:
+            chain[n].imm, chain[n].imm_kind = imm, self.capi.BK["imm"]
+        if self.post_stage:
+            self.p.n_post = n + 1
+        else:
+            self.p.n_pre = n + 1
+        return self
+
+    def row(self, name, w=None, b=None):
+        self.p.row_op, self.p.eps = self.capi.ROWOP[name], 1e-5
+        if w is not None:
+            self.p.norm_weight = self._operand(w, "rowvec")
+        if b is not None:
+            self.p.norm_bias = self._operand(b, "rowvec")
+        self.post_stage = True
+        return self
+
+    def finish(self, torch, reduce="none"):
+        self.p.reduce = self.capi.RED[reduce]
+        odt = self.out_dtype or self.x.dtype
+        shape = self.x.shape if reduce == "none" else (self.x.shape[0],)
+        self.out = torch.empty(shape, device="cuda", dtype=odt)
+        self.p.output = self.out.data_ptr()
+        self.p.output_dtype = {torch.float32: self.capi.DTYPE_F32, torch.float16: self.capi.DTYPE_F16, torch.bfloat16: self.capi.DTYPE_BF16}[odt]
+        self.bytes = self.read_bytes + self.out.numel() * self.out.element_size()
+        return self
+
+
+def bench_survey(torch, capi, stream, steps, warmup):
+    """Achieved HBM bandwidth of a spread of row programs: the built-in kernel shapes, shapes the library compiles
+    at run time (rows_jit_*), and rows of odd length.  Bytes are the algorithmic ones: every operand read once, the
+    result written once."""
+    lib = capi.lib()
+    sp = C.c_void_p(stream.cuda_stream)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    res = {}
+
+    def rnd(shape, dtype, scale=1.0, shift=0.0):
+        return (torch.randn(shape, generator=g, device="cuda") * scale + shift).to(dtype)
+
+    def run(name, prog):
+        lib.axhip_fused_rows_prepare(C.byref(prog.p))
+        torch.cuda.synchronize()
+        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(prog.p), sp)), steps, warmup)
+        res[name] = {"kernel": lib.axhip_fused_rows_kernel_name(C.byref(prog.p)).decode(), "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3,
+                     "bytes": prog.bytes, "frac_of_hbm_peak": prog.bytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                     "finite": bool(torch.isfinite(prog.out.float()).all().item())}
+
+    bf, f32 = torch.bfloat16, torch.float32
+    R, Cc = 16384, 4096
+    x, y = rnd((R, Cc), bf), rnd((R, Cc), bf)
+    w, b = rnd((Cc,), bf, 0.3, 1.0), rnd((Cc,), bf, 0.1)
+    cvec, half = rnd((R,), bf), torch.full((1,), 0.5, device="cuda", dtype=bf)
+    P = lambda t=x, od=None: _Prog(capi, t, od)
+    tag = "bf16_16384x4096"
+    run(f"softmax_{tag}", P().row("softmax").finish(torch))
+    run(f"softmax(x*s)_{tag}", P().op("mul", imm=0.125).row("softmax").finish(torch))
+    run(f"softmax(x+y)_{tag}", P().op("add", y).row("softmax").finish(torch))
+    run(f"softmax(x*s+y)_{tag}", P().op("mul", half, "scalar").op("add", y).row("softmax").finish(torch))
+    run(f"logsoftmax_{tag}", P().row("logsoftmax").finish(torch))
+    run(f"layernorm_{tag}", P().row("layernorm", w, b).finish(torch))
+    run(f"layernorm(x+y)_{tag}", P().op("add", y).row("layernorm", w, b).finish(torch))
+    run(f"gelu(layernorm)_{tag}", P().row("layernorm", w, b).op("gelu").finish(torch))
+    run(f"silu(layernorm)_{tag}", P().row("layernorm", w, b).op("silu").finish(torch))
+    run(f"rmsnorm_{tag}", P().row("rmsnorm", w).finish(torch))
+    run(f"gelu(rmsnorm)_{tag}", P().row("rmsnorm", w).op("gelu").finish(torch))
+    run(f"rmsnorm(x+y)_{tag}", P().op("add", y).row("rmsnorm", w).finish(torch))
+    run(f"sum(x)_{tag}", P().finish(torch, "sum"))
+    run(f"mean(x^2)_{tag}", P(od=f32).op("square").finish(torch, "mean"))
+    run(f"sum(x*y)_{tag}", P().op("mul", y).finish(torch, "sum"))
+    run(f"max(|x|)_{tag}", P().op("abs").finish(torch, "max"))
+    # shapes without a built-in kernel: compiled when first seen
+    run(f"sigmoid(layernorm)_{tag}", P().row("layernorm", w, b).op("sigmoid").finish(torch))
+    run(f"softmax(exp(x))_{tag}", P().op("exp").row("softmax").finish(torch))
+    run(f"softmax(tanh(x*s)+y)_{tag}", P().op("mul", imm=0.5).op("tanh").op("add", y).row("softmax").finish(torch))
+    run(f"layernorm(relu(x)*y+r)_{tag}", P().op("relu").op("mul", y).op("add", w, "rowvec").row("layernorm", w, b).finish(torch))
+    run(f"softmax(x*c)*y_{tag}", P().op("mul", cvec, "colvec").row("softmax").op("mul", y).finish(torch))
+    run(f"rmsnorm(x)*sigmoid(y)_fp32out_{tag}", P(od=f32).row("rmsnorm", w).op("mul", y).finish(torch))
+    del x, y
+    a, c = rnd((8192, 8192), f32), rnd((8192, 8192), f32)
+    w32, b32 = rnd((8192,), f32, 0.3, 1.0), rnd((8192,), f32, 0.1)
+    one = torch.ones(1, device="cuda")
+    tag = "f32_8192x8192"
+    run(f"softmax((relu(a)+1)*b).sum_{tag}", P(a).op("relu").op("add", one, "scalar").op("mul", c).row("softmax").finish(torch, "sum"))
+    run(f"softmax_{tag}", P(a).row("softmax").finish(torch))
+    run(f"layernorm_{tag}", P(a).row("layernorm", w32, b32).finish(torch))
+    run(f"gelu(layernorm(a+b))_{tag}", P(a).op("add", c).row("layernorm", w32, b32).op("gelu").finish(torch))
+    run(f"sum(a)_{tag}", P(a).finish(torch, "sum"))
+    del a, c
+    # rows of odd length
+    for rows, cols, dt, name in ((30000, 1500, bf, "bf16"), (16384, 4100, bf, "bf16"), (16384, 4097, bf, "bf16"), (16384, 1501, f32, "f32")):
+        t = rnd((rows, cols), dt)
+        run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
+    t, u = rnd((30000, 1001), bf), rnd((30000, 1001), bf)
+    wr, br = rnd((1001,), bf, 0.3, 1.0), rnd((1001,), bf, 0.1)
+    run("layernorm_bf16_30000x1001", P(t).row("layernorm", wr, br).finish(torch))
+    run("softmax(|x|*y)_bf16_30000x1001", P(t).op("abs").op("mul", u).row("softmax").finish(torch))
+    t, u = rnd((16384, 4099), bf), rnd((16384, 4099), bf)
+    wr, br = rnd((4099,), bf, 0.3, 1.0), rnd((4099,), bf, 0.1)
+    run("layernorm(x+y)_bf16_16384x4099", P(t).op("add", u).row("layernorm", wr, br).finish(torch))
+    run("mean(x^2)_bf16_16384x4099", P(t, f32).op("square").finish(torch, "mean"))
+    return res
+
 def bench_gemm(torch, capi, stream, steps, warmup):
     """x W^T through axhip_gemm (the nn::Linear product): a large square, the tall product of a
     long batch, and the Whisper-block projection of BASELINE.json configs[4]."""
@@ -348,7 +481,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--min-warmup-ms", type=float, default=None, help="warm every kernel for at least this long (default 100)")
-    ap.add_argument("--only", choices=["sdpa", "chains", "gemm", "f32"], default=None)
+    ap.add_argument("--only", choices=["sdpa", "chains", "gemm", "f32", "survey"], default=None)
     args = ap.parse_args()
     if args.min_warmup_ms is not None:
         global MIN_WARMUP_MS
@@ -373,6 +506,7 @@ def main() -> int:
     ch = bench_chains(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "chains") else None
     gm = bench_gemm(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "gemm") else None
     f32 = bench_f32(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "f32") else None
+    survey = bench_survey(torch, capi, stream, args.steps, args.warmup) if args.only == "survey" else None
     cpu = None if (args.no_cpu or sd is None) else cpu_baseline()
 
     line = {
@@ -402,6 +536,8 @@ def main() -> int:
         line["gemm"] = gm
     if f32:
         line["f32_matrix_kernels"] = f32
+    if survey:
+        line["row_program_survey"] = survey
     if args.only is None:
         line["host_layer"] = host_layer_bench()
     if cpu:

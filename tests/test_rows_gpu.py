@@ -272,7 +272,9 @@ def test_scaled_and_biased_softmax_on_the_specialised_kernels(dt):
                  (gh.Rows(xs, dt).imm("mul", 0.125).binary("add", ys).row_op("softmax"), "muls_addf_softmax", xf.astype(np.float64) * 0.125 + yf)]
         for prog, tag, logits in cases:
             got = prog.run()
-            assert prog.kernel_name().startswith("rows_static_" + tag), prog.kernel_name()
+            # a built-in kernel, or for a row length between the built-in plans (8200 columns) one compiled for it
+            assert prog.kernel_name().startswith(("rows_static_" + tag, "rows_jit_" + tag)), prog.kernel_name()
+            assert cols % 1024 != 0 or prog.kernel_name().startswith("rows_static_"), prog.kernel_name()
             got = got.astype(np.float64) if dt == F32 else axo.to_f32(got, dt).astype(np.float64)
             e = np.exp(logits - logits.max(-1, keepdims=True))
             want = e / e.sum(-1, keepdims=True)
@@ -298,10 +300,10 @@ def test_fast_activations_after_a_norm_in_16_bit(post):
 
 
 def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
-    """Rows beyond the 32 KiB the specialised kernels hold: up to 4096 16-byte chunks stay in the registers of a
-    1024-thread block (one read), longer ones are streamed in passes."""
+    """Rows beyond the 32 KiB the built-in kernels hold: up to 4096 16-byte chunks stay in the registers of a
+    512-thread block (one read; kernels compiled at first launch), longer ones are streamed in passes."""
     g = axo.PCG64(123)
-    for cols, plan in ((12000, "rows_jit_softmax_f32_g1024_it4"), (16384, "rows_jit_softmax_f32_g1024_it4"), (20000, "rows_streamed_e4")):
+    for cols, plan in ((12000, "rows_jit_softmax_f32_g512_it6"), (16384, "rows_jit_softmax_f32_g512_it8"), (20000, "rows_streamed_e4")):
         x = (g.normal((3, cols)) * 2).astype(np.float32)
         p = gh.Rows(x, F32).row_op("softmax")
         got = p.run()
@@ -311,7 +313,7 @@ def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
     w, b = axo.to_bits(g.uniform((30000,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((30000,), -0.5, 0.5), BF16)
     p = gh.Rows(xb, BF16).row_op("layernorm", 1e-5, w=w, b=b).unary("gelu")
     got = axo.to_f32(p.run(), BF16).astype(np.float64)
-    assert p.kernel_name() == "rows_jit_layernorm_gelu_wb_bf16_g1024_it4", p.kernel_name()
+    assert p.kernel_name() == "rows_jit_layernorm_gelu_wb_bf16_g512_it8", p.kernel_name()
     xf = axo.to_f32(xb, BF16).astype(np.float64)
     n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
     import math
@@ -400,7 +402,7 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
         got = p.run(reduce="sum")
         assert np.allclose(got.reshape(-1), (xf * xf).sum(-1), rtol=1e-4, atol=1e-3)
         if cols >= 8:
-            assert p.kernel_name().startswith("rows_static_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+            assert p.kernel_name().startswith(("rows_static_square_reduce_sum", "rows_jit_square_reduce_sum")) and p.kernel_name().endswith("_ragged"), p.kernel_name()
         p = gh.Rows(xs, dt).row_op("logsoftmax")
         got = out(p.run())
         assert p.kernel_name().endswith("_ragged"), p.kernel_name()
