@@ -3,6 +3,7 @@
 // trio: one process-wide stream, every transfer an explicit hipMemcpyAsync.
 #include "common.hpp"
 
+#include <chrono>
 #include <cstring>
 #include <mutex>
 
@@ -142,7 +143,20 @@ int axhip_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *strea
 int axhip_stream_sync(void *stream) {
     int rc = ensure_init();
     if (rc) return rc;
-    AXHIP_CHECK_HIP(hipStreamSynchronize(resolve_stream(stream)));
+    hipStream_t s = resolve_stream(stream);
+    // Most waits here are for a kernel of tens of microseconds, and a blocking wait adds an interrupt round trip of
+    // the same order.  Poll for up to a millisecond first; longer work then blocks without burning the core.
+    const auto t0 = std::chrono::steady_clock::now();
+    for (;;) {
+        const hipError_t e = hipStreamQuery(s);
+        if (e == hipSuccess) return AXHIP_OK;
+        if (e != hipErrorNotReady) {
+            AXHIP_CHECK_HIP(e);
+        }
+        (void)hipGetLastError(); // hipErrorNotReady is sticky in the runtime's last-error slot
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(1000)) break;
+    }
+    AXHIP_CHECK_HIP(hipStreamSynchronize(s));
     return AXHIP_OK;
 }
 

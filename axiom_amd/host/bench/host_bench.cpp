@@ -27,10 +27,26 @@ template <typename F> static void measure(const char *name, F f, int warmup, int
     }
     std::sort(us.begin(), us.end());
     const double med = us[us.size() / 2];
+    // the same work the way a program issues it: materialisations queued back to back (they are asynchronous), one
+    // wait for 16 of them
+    std::vector<double> piped;
+    constexpr int BURST = 16;
+    for (int r = 0; r < std::max(4, iters / BURST); ++r) {
+        const auto t0 = Clock::now();
+        for (int i = 0; i < BURST; ++i) f();
+        backends::hip::synchronize();
+        piped.push_back(std::chrono::duration<double, std::micro>(Clock::now() - t0).count() / BURST);
+    }
+    std::sort(piped.begin(), piped.end());
+    const double pmed = piped[piped.size() / 2];
+    graph::record_gpu_plan_kernels(true); // one more, untimed, to learn which kernels the graph runs on
+    f();
+    backends::hip::synchronize();
+    graph::record_gpu_plan_kernels(false);
     std::string kernels;
     for (const auto &k : graph::last_gpu_plan_kernels()) kernels += (kernels.empty() ? "" : " ") + k;
-    std::printf("  \"%s\": {\"median_us\": %.1f, \"min_us\": %.1f, \"%s\": %.1f, \"last_graph_kernels\": \"%s\"}%s\n", name, med, us.front(), unit,
-                work / (med * 1e-6) / 1e9, kernels.c_str(), last ? "" : ",");
+    std::printf("  \"%s\": {\"median_us\": %.1f, \"min_us\": %.1f, \"%s\": %.1f, \"queued_16_per_wait_us\": %.1f, \"queued_%s\": %.1f, \"last_graph_kernels\": \"%s\"}%s\n",
+                name, med, us.front(), unit, work / (med * 1e-6) / 1e9, pmed, unit, work / (pmed * 1e-6) / 1e9, kernels.c_str(), last ? "" : ",");
 }
 
 int main(int argc, char **argv) {

@@ -82,6 +82,9 @@ void materialize_gpu_graph(GraphNode *root);
 // kernels launched by the last materialize_gpu_graph on this thread, in order
 // (e.g. "rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"); for tests and AXIOM_DEBUG_FUSION
 const std::vector<std::string> &last_gpu_plan_kernels();
+// The names are collected only while this is on (or AXIOM_DEBUG_FUSION is set): asking the backend for a kernel's
+// name costs about as much as launching it.
+void record_gpu_plan_kernels(bool on);
 
 } // namespace graph
 } // namespace axiom

@@ -169,7 +169,10 @@ class MultiHeadAttention : public Module {
     int num_heads_;
     Linear q_proj_, k_proj_, v_proj_, out_proj_;
     mutable Tensor qkv_weight_, qkv_bias_;
-    mutable const void *qkv_sources_[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    // the storages (and offsets) the stacked copy was made from; held so that their blocks cannot be recycled
+    mutable std::shared_ptr<Storage> qkv_holders_[6];
+    mutable size_t qkv_offsets_[6] = {0, 0, 0, 0, 0, 0};
+    void drop_stacked_projection();
 };
 
 } // namespace axiom::nn

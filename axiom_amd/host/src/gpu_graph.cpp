@@ -16,6 +16,7 @@
 // axhip_gemm.  Reshape and transpose are views; a view that a kernel cannot address
 // directly is gathered with axhip_strided_copy first.
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -95,6 +96,9 @@ struct Plan {
     std::vector<Step> steps;
     std::vector<std::pair<int, int>> node_results; // (topological index of a node, value holding its result)
     size_t n_leaves = 0;
+    // what the plan was built for, compared on every cache hit: the cache is keyed by a 64-bit hash, and a plan bound
+    // to a graph of other extents would launch kernels past the caller's buffers
+    std::vector<int64_t> fingerprint;
 };
 
 bool is_leaf(const GraphNode *n, const GraphNode *root) { return n->is_constant || (n->is_materialized_ && n != root); }
@@ -653,6 +657,7 @@ CacheState &cache() {
 }
 
 thread_local std::vector<std::string> tl_last_kernels;
+std::atomic<bool> g_record_kernels{false};
 
 uint64_t mix_u64(uint64_t h, uint64_t v) {
     for (int i = 0; i < 8; ++i) h = (h ^ ((v >> (8 * i)) & 0xFF)) * 1099511628211ULL;
@@ -675,6 +680,29 @@ uint64_t plan_key(const GraphNode *root, const std::vector<const GraphNode *> &t
         }
     }
     return h;
+}
+
+// node count, root shape and dtype, and per leaf its dtype, shape and strides
+std::vector<int64_t> plan_fingerprint(const GraphNode *root, const std::vector<const GraphNode *> &topo) {
+    std::vector<int64_t> f;
+    f.reserve(16 + 8 * topo.size());
+    f.push_back(static_cast<int64_t>(topo.size()));
+    f.push_back(static_cast<int64_t>(root->output_dtype));
+    f.push_back(static_cast<int64_t>(root->output_shape.size()));
+    for (size_t d : root->output_shape) f.push_back(static_cast<int64_t>(d));
+    for (const GraphNode *n : topo) {
+        if (!is_leaf(n, root)) {
+            f.push_back(-1 - static_cast<int64_t>(n->op_type));
+            continue;
+        }
+        const Shape &shape = n->is_constant ? n->output_shape : n->cached_shape_;
+        const Strides &strides = n->is_constant ? n->constant_strides : n->cached_strides_;
+        f.push_back(static_cast<int64_t>(n->output_dtype));
+        f.push_back(static_cast<int64_t>(shape.size()));
+        for (size_t d : shape) f.push_back(static_cast<int64_t>(d));
+        for (int64_t st : strides) f.push_back(st);
+    }
+    return f;
 }
 
 bool debug_fusion() {
@@ -703,6 +731,7 @@ size_t GraphCache::hits() const { return cache().hits; }
 size_t GraphCache::misses() const { return cache().misses; }
 
 const std::vector<std::string> &last_gpu_plan_kernels() { return tl_last_kernels; }
+void record_gpu_plan_kernels(bool on) { g_record_kernels.store(on); }
 
 void materialize_gpu_graph(GraphNode *root) {
     if (!root || root->is_materialized_) return;
@@ -716,19 +745,23 @@ void materialize_gpu_graph(GraphNode *root) {
         auto &c = cache();
         std::lock_guard<std::mutex> lk(c.mu);
         auto it = c.plans.find(key);
-        if (it != c.plans.end()) {
-            plan = it->second;
-            ++c.hits;
-        } else {
-            ++c.misses;
-        }
+        if (it != c.plans.end()) plan = it->second;
+    }
+    const std::vector<int64_t> fingerprint = plan_fingerprint(root, topo);
+    if (plan && plan->fingerprint != fingerprint) plan.reset(); // two graphs under one hash: the newcomer replaces the entry
+    {
+        auto &c = cache();
+        std::lock_guard<std::mutex> lk(c.mu);
+        ++(plan ? c.hits : c.misses);
     }
     if (!plan) {
-        plan = std::make_shared<const Plan>(PlanBuilder(root, topo, shared).build());
+        Plan built = PlanBuilder(root, topo, shared).build();
+        built.fingerprint = fingerprint;
+        plan = std::make_shared<const Plan>(std::move(built));
         auto &c = cache();
         std::lock_guard<std::mutex> lk(c.mu);
         if (c.plans.size() >= GraphCache::max_entries) c.plans.clear(); // src/backends/metal/mpsgraph_graph_compiler.mm:899-900
-        c.plans.emplace(key, plan);
+        c.plans[key] = plan;
     }
 
     // ---- bind leaves (same order as the builder: topological order) and allocate temporaries
@@ -760,6 +793,7 @@ void materialize_gpu_graph(GraphNode *root) {
     };
 
     // ---- run
+    const bool record = g_record_kernels.load(std::memory_order_relaxed) || debug_fusion();
     tl_last_kernels.clear();
     for (const Step &st : plan->steps) {
         if (st.kind == Step::ROWS) {
@@ -768,25 +802,25 @@ void materialize_gpu_graph(GraphNode *root) {
             p.output = ptr_of(st.rows.output);
             for (int i = 0; i < p.n_operands; ++i) p.operands[i].ptr = ptr_of(st.rows.operand_value[i]);
             if (st.rows.full_reduce) {
-                tl_last_kernels.emplace_back("full_reduce");
+                if (record) tl_last_kernels.emplace_back("full_reduce");
                 if (p.rows > 0 && p.cols > 0)
                     AXHIP_CALL(axhip_fused_full_reduce(&p, temps[st.rows.workspace]->raw(), temps[st.rows.workspace]->size_bytes(), nullptr));
             } else {
-                tl_last_kernels.emplace_back(axhip_fused_rows_kernel_name(&p));
+                if (record) tl_last_kernels.emplace_back(axhip_fused_rows_kernel_name(&p));
                 AXHIP_CALL(axhip_fused_rows(&p, nullptr));
             }
         } else if (st.kind == Step::GEMM) {
             AxhipGemmParams p = st.gemm.p;
             p.bias = st.gemm.bias >= 0 ? ptr_of(st.gemm.bias) : nullptr;
             p.residual = st.gemm.residual >= 0 ? ptr_of(st.gemm.residual) : nullptr;
-            tl_last_kernels.emplace_back("gemm");
+            if (record) tl_last_kernels.emplace_back("gemm");
             AXHIP_CALL(axhip_gemm(ptr_of(st.gemm.a), ptr_of(st.gemm.b), ptr_of(st.gemm.c), &p, nullptr));
         } else if (st.kind == Step::PAD) {
             const ValueSpec &src = plan->values[st.pad.src];
             const int64_t isz = static_cast<int64_t>(dtype_size(src.dtype));
             std::vector<int64_t> shp(src.shape.begin(), src.shape.end()), est(src.strides.size());
             for (size_t i = 0; i < est.size(); ++i) est[i] = src.strides[i] / isz;
-            tl_last_kernels.emplace_back("pad");
+            if (record) tl_last_kernels.emplace_back("pad");
             AXHIP_CALL(axhip_pad(ptr_of(st.pad.src), ptr_of(st.pad.dst), detail::to_axhip_dtype(src.dtype), static_cast<int32_t>(shp.size()), shp.data(),
                                  est.data(), st.pad.before.data(), st.pad.after.data(), st.pad.value, nullptr));
         } else if (st.kind == Step::MASKED_FILL) {
@@ -794,12 +828,12 @@ void materialize_gpu_graph(GraphNode *root) {
             const int64_t isz = static_cast<int64_t>(dtype_size(src.dtype));
             std::vector<int64_t> shp(src.shape.begin(), src.shape.end()), est(src.strides.size()), mst(st.mfill.mask_strides.begin(), st.mfill.mask_strides.end());
             for (size_t i = 0; i < est.size(); ++i) est[i] = src.strides[i] / isz;
-            tl_last_kernels.emplace_back("masked_fill");
+            if (record) tl_last_kernels.emplace_back("masked_fill");
             AXHIP_CALL(axhip_masked_fill(ptr_of(st.mfill.src), detail::to_axhip_dtype(src.dtype), static_cast<const uint8_t *>(ptr_of(st.mfill.mask)),
                                          ptr_of(st.mfill.dst), static_cast<int32_t>(shp.size()), shp.data(), est.data(), mst.data(), st.mfill.value, nullptr));
         } else if (st.kind == Step::GATHER) {
             const ValueSpec &tab = plan->values[st.gather.table], &idx = plan->values[st.gather.indices];
-            tl_last_kernels.emplace_back("gather_rows");
+            if (record) tl_last_kernels.emplace_back("gather_rows");
             AXHIP_CALL(axhip_gather_rows(ptr_of(st.gather.table), detail::to_axhip_dtype(tab.dtype), static_cast<int64_t>(tab.shape[0]),
                                          static_cast<int64_t>(tab.shape[1]), ptr_of(st.gather.indices), static_cast<int32_t>(dtype_size(idx.dtype)),
                                          static_cast<int64_t>(ShapeUtils::size(idx.shape)), ptr_of(st.gather.dst), nullptr));
@@ -808,7 +842,7 @@ void materialize_gpu_graph(GraphNode *root) {
             const int dt = detail::to_axhip_dtype(src.dtype);
             std::vector<int64_t> shp(st.copy.shape.begin(), st.copy.shape.end()), est(st.copy.src_strides.size());
             for (size_t i = 0; i < est.size(); ++i) est[i] = st.copy.src_strides[i] / static_cast<int64_t>(dtype_size(src.dtype));
-            tl_last_kernels.emplace_back("strided_copy");
+            if (record) tl_last_kernels.emplace_back("strided_copy");
             AXHIP_CALL(axhip_strided_copy(ptr_of(st.copy.src), dt, ptr_of(st.copy.dst), dt, static_cast<int32_t>(shp.size()), shp.data(),
                                           est.data(), nullptr));
         }

@@ -117,7 +117,17 @@ class Json {
             return out;
         }
     }
+    // Nesting the reader follows before it gives up: __metadata__ values are flat in files written by the format's
+    // own tools, and a header of nothing but opening brackets must not walk the stack down.
+    static constexpr int MAX_DEPTH = 64;
+    int depth_ = 0;
     void skip_value() {
+        struct Level {
+            int &d;
+            explicit Level(int &depth) : d(depth) { ++d; }
+            ~Level() { --d; }
+        } level(depth_);
+        if (depth_ > MAX_DEPTH) fail("values nested deeper than 64 levels");
         ws();
         const char c = peek();
         if (c == '"') { string(); return; }
@@ -200,7 +210,17 @@ Opened open_file(const std::string &filename) { // src/io/io_safetensors.cpp:55-
     o.data_start = 8 + n;
     o.data_bytes = file_bytes - o.data_start;
     for (const Entry &e : o.entries) {
-        const uint64_t want = static_cast<uint64_t>(ShapeUtils::size(e.shape)) * dtype_size(e.dtype);
+        // element count times element size, computed so that it cannot wrap around (shape [2^32, 2^32] is 0 elements
+        // in 64-bit arithmetic and would pass for an empty byte range): no partial product may exceed the data section
+        uint64_t want = dtype_size(e.dtype);
+        bool zero = false;
+        for (size_t d : e.shape) zero = zero || d == 0;
+        if (zero) want = 0;
+        else
+            for (size_t d : e.shape) {
+                if (want > o.data_bytes / d) throw FileFormatError("SafeTensors: tensor '" + e.name + "' has a shape larger than the file's data section");
+                want *= d;
+            }
         if (e.end - e.begin != want)
             throw FileFormatError("SafeTensors: tensor '" + e.name + "' spans " + std::to_string(e.end - e.begin) + " bytes, its shape and dtype need " +
                                   std::to_string(want));

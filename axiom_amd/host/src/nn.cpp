@@ -157,16 +157,20 @@ Tensor MultiHeadAttention::forward(const Tensor &query, const Tensor &key, const
     return out_proj_.forward(merged);
 }
 
-void MultiHeadAttention::load_state_dict(const std::map<std::string, Tensor> &sd, const std::string &prefix, bool strict) {
+void MultiHeadAttention::drop_stacked_projection() {
     qkv_weight_ = qkv_bias_ = Tensor();
+    for (auto &h : qkv_holders_) h.reset();
+}
+void MultiHeadAttention::load_state_dict(const std::map<std::string, Tensor> &sd, const std::string &prefix, bool strict) {
+    drop_stacked_projection();
     Module::load_state_dict(sd, prefix, strict);
 }
 Module &MultiHeadAttention::to(Device device) {
-    qkv_weight_ = qkv_bias_ = Tensor();
+    drop_stacked_projection();
     return Module::to(device);
 }
 Module &MultiHeadAttention::to(DType dtype) {
-    qkv_weight_ = qkv_bias_ = Tensor();
+    drop_stacked_projection();
     return Module::to(dtype);
 }
 
@@ -179,6 +183,8 @@ bool MultiHeadAttention::fused_qkv(const Tensor &x, Tensor &q, Tensor &k, Tensor
     const size_t B = x.shape()[0], S = x.shape()[1], Dm = x.shape()[2], H = static_cast<size_t>(num_heads_), Dh = Dm / H;
     bool any_bias = false;
     const void *sources[6];
+    std::shared_ptr<Storage> holders[6];
+    size_t offsets[6] = {};
     for (int i = 0; i < 3; ++i) {
         const Tensor &w = proj[i]->weight(), &b = proj[i]->bias();
         if (w.empty() || w.is_lazy() || w.device() != Device::GPU || w.dtype() != dt || !w.is_contiguous() || w.ndim() != 2 || w.shape()[0] != Dm || w.shape()[1] != Dm)
@@ -188,8 +194,19 @@ bool MultiHeadAttention::fused_qkv(const Tensor &x, Tensor &q, Tensor &k, Tensor
         any_bias = any_bias || has_b;
         sources[2 * i] = static_cast<const char *>(w.storage()->raw()) + w.offset();
         sources[2 * i + 1] = has_b ? static_cast<const char *>(b.storage()->raw()) + b.offset() : nullptr;
+        holders[2 * i] = w.storage();
+        offsets[2 * i] = w.offset();
+        if (has_b) {
+            holders[2 * i + 1] = b.storage();
+            offsets[2 * i + 1] = b.offset();
+        }
     }
-    if (qkv_weight_.empty() || qkv_weight_.dtype() != dt || std::memcmp(sources, qkv_sources_, sizeof(sources)) != 0) {
+    // The stacked copy is current while the six parameters are still the same storage objects at the same offsets.
+    // The cache holds those storages, so a replaced parameter's block cannot be recycled into a new tensor at the old
+    // address while it is compared (device addresses alone would match again after the allocator reuses the block).
+    bool current = !qkv_weight_.empty() && qkv_weight_.dtype() == dt;
+    for (int i = 0; i < 6 && current; ++i) current = holders[i] == qkv_holders_[i] && offsets[i] == qkv_offsets_[i];
+    if (!current) {
         const size_t isz = dtype_size(dt);
         Tensor w3(Shape{3 * Dm, Dm}, dt, Device::GPU), b3;
         if (any_bias) b3 = Tensor(Shape{3 * Dm}, dt, Device::GPU);
@@ -202,7 +219,10 @@ bool MultiHeadAttention::fused_qkv(const Tensor &x, Tensor &q, Tensor &k, Tensor
         }
         qkv_weight_ = w3;
         qkv_bias_ = b3;
-        std::memcpy(qkv_sources_, sources, sizeof(sources));
+        for (int i = 0; i < 6; ++i) {
+            qkv_holders_[i] = holders[i];
+            qkv_offsets_[i] = offsets[i];
+        }
     }
     Tensor qkv = ops::matmul(x, qkv_weight_, false, true);
     if (!qkv_bias_.empty()) qkv = ops::add(qkv, qkv_bias_);

@@ -1,5 +1,7 @@
 // axiom::Tensor for the gfx950 host layer (behaviour of src/tensor/tensor.cpp for the
 // hot-path subset: views, device moves, dtype casts, factories, allclose).
+#include <map>
+#include <mutex>
 #include "axiom/tensor.hpp"
 
 #include <algorithm>
@@ -421,10 +423,32 @@ Tensor Tensor::rand(const Shape &shape, DType dtype, Device device) { return uni
 void Tensor::manual_seed(uint64_t seed) { RandomGenerator::instance().seed(seed); }
 
 // --------------------------------------------------------------- operators
+// src/tensor/tensor_operators.hpp:196-235: a scalar operand becomes a {1} tensor of the tensor's dtype on its device.
+// On the GPU that is an upload and a wait per expression (about 25 us, a third of the chain it feeds), so the device
+// copies of recently used (value, dtype) pairs are kept: they are constants nothing writes to.
 Tensor make_scalar_like(const Tensor &t, double value) {
     Tensor s(Shape{1}, t.dtype(), Device::CPU);
     s.set_item<double>({0}, value);
-    return t.device() == Device::GPU ? s.to(Device::GPU) : s;
+    if (t.device() != Device::GPU) return s;
+    struct Key {
+        uint64_t bits;
+        int dtype;
+        bool operator<(const Key &o) const { return bits != o.bits ? bits < o.bits : dtype < o.dtype; }
+    };
+    static std::mutex mu;
+    static std::map<Key, Tensor> cache;
+    Key key{0, static_cast<int>(t.dtype())};
+    std::memcpy(&key.bits, &value, sizeof(value));
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = cache.find(key);
+        if (it != cache.end()) return it->second;
+    }
+    Tensor d = s.to(Device::GPU);
+    std::lock_guard<std::mutex> lock(mu);
+    if (cache.size() >= 256) cache.clear();
+    cache.emplace(key, d);
+    return d;
 }
 Tensor operator+(const Tensor &a, const Tensor &b) { return ops::add(a, b); }
 Tensor operator-(const Tensor &a, const Tensor &b) { return ops::subtract(a, b); }

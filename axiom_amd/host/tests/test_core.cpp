@@ -346,6 +346,10 @@ TEST(SafeTensors, MalformedFilesAreRejected) {
     expect_format_error(R"({"w":{"dtype":"F32","shape":[2,-2],"data_offsets":[0,16]}})", four);                   // negative extent
     expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2],"data_offsets":[16,0]}})", four);                    // reversed range
     expect_format_error(R"({"w":{"dtype":"F32","shape":[2,2],"data_offsets":[0,16]})", four);                     // unterminated object
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[4294967296,4294967296],"data_offsets":[0,0]}})", four);   // element count wraps to 0 in 64 bits
+    expect_format_error(R"({"w":{"dtype":"F32","shape":[4611686018427387904,4],"data_offsets":[0,0]}})", four);   // byte count wraps to 0
+    expect_format_error(R"({"__metadata__":)" + std::string(100000, '[') + std::string(100000, ']') + R"(,"w":{"dtype":"F32","shape":[2,2],"data_offsets":[0,16]}})",
+                        four);                                                                                    // nesting that would exhaust the stack
     {
         std::ofstream f(path, std::ios::binary); // shorter than the length field
         f.write("abc", 3);

@@ -423,11 +423,11 @@ GPU_TEST(FlashAttentionMHA, UniformInputIdentityProjections) { // tests/test_fla
     EXPECT_NEAR(causal.item<float>({0, 2, 1}), 1.0f, 1e-5);
 }
 
-// BASELINE configs[4]: Whisper-style encoder self-attention block, here at S=150 for the exact
-// comparison (the full S=1500 size is covered by properties below)
+// BASELINE configs[4]: Whisper-style encoder self-attention block, at S=150 compared in full and at the full
+// S=1500 on 48 sequence positions from the start, the middle and the end
 static Tensor whisper_block(const Tensor &x, nn::MultiHeadAttention &mha, nn::LayerNorm &ln) { return ln.forward(x + mha.forward(x, x, x)); }
 
-static void whisper_case(size_t S, bool compare) {
+static void whisper_case(size_t S, bool /*compare*/) {
     const size_t Dm = 1280, H = 20, Dh = 64;
     const DType dt = DType::BFloat16;
     auto x = axtest::randn({1, S, Dm}, 51, dt);
@@ -457,31 +457,51 @@ static void whisper_case(size_t S, bool compare) {
         EXPECT_NEAR(m, 0.0, 2e-2);
         EXPECT_NEAR(q / Dm, 1.0, 5e-2);
     }
-    if (!compare) return;
-    // fp32 evaluation of the same bf16 inputs with the oracle's pieces
+    // fp32 evaluation of the same bf16 inputs with the oracle's pieces, on a subset of the sequence positions: the
+    // projections and the norm are row-wise, and a query row's attention needs every key and value but no other query
+    std::vector<size_t> rows;
+    if (S <= 256) {
+        for (size_t r = 0; r < S; ++r) rows.push_back(r);
+    } else {
+        for (size_t r = 0; r < 16; ++r) rows.push_back(r);
+        for (size_t r = S / 2 - 8; r < S / 2 + 8; ++r) rows.push_back(r);
+        for (size_t r = S - 16; r < S; ++r) rows.push_back(r);
+    }
+    const size_t Q = rows.size();
     auto xf = x.astype(DType::Float32);
-    auto proj = [&](const Tensor &in, const char *name) {
-        Tensor wf = w[std::string(name) + ".weight"].astype(DType::Float32), out({S, Dm}, DType::Float32);
-        axo_matmul(AXO_F32, in.data(), wf.data(), out.data(), S, Dm, Dm, 0, 1);
+    Tensor x2 = xf.reshape({S, Dm});
+    Tensor xq({Q, Dm}, DType::Float32);
+    for (size_t i = 0; i < Q; ++i) std::memcpy(xq.typed_data<float>() + i * Dm, x2.typed_data<float>() + rows[i] * Dm, Dm * sizeof(float));
+    auto proj = [&](const Tensor &in, size_t n, const char *name) {
+        Tensor wf = w[std::string(name) + ".weight"].astype(DType::Float32), out({n, Dm}, DType::Float32);
+        axo_matmul(AXO_F32, in.data(), wf.data(), out.data(), n, Dm, Dm, 0, 1);
         return out;
     };
-    auto split = [&](const Tensor &t) { return t.reshape({1, S, H, Dh}).transpose({0, 2, 1, 3}).ascontiguousarray(); };
-    Tensor x2 = xf.reshape({S, Dm});
-    auto att = axtest::oracle_sdpa(split(proj(x2, "q_proj")), split(proj(x2, "k_proj")), split(proj(x2, "v_proj")), Tensor(), -1, false);
-    Tensor merged = att.transpose({0, 2, 1, 3}).ascontiguousarray().reshape({S, Dm});
-    Tensor o = proj(merged, "out_proj");
-    std::vector<float> res(S * Dm), want(S * Dm);
-    for (size_t i = 0; i < S * Dm; ++i) res[i] = o.typed_data<float>()[i] + x2.typed_data<float>()[i];
-    axo_layer_norm(AXO_F32, res.data(), nullptr, nullptr, want.data(), S, Dm, 1e-5f);
-    double worst = 0;
-    for (size_t i = 0; i < S * Dm; ++i) worst = std::max(worst, std::fabs(double(got[i]) - want[i]));
-    EXPECT_LE(worst, 6e-2); // bf16 ulp at |y| ~ 4 is 3e-2: two roundings (residual, output) stay inside 6e-2
+    auto split = [&](const Tensor &t, size_t n) { return t.reshape({1, n, H, Dh}).transpose({0, 2, 1, 3}).ascontiguousarray(); };
+    auto att = axtest::oracle_sdpa(split(proj(xq, Q, "q_proj"), Q), split(proj(x2, S, "k_proj"), S), split(proj(x2, S, "v_proj"), S), Tensor(), -1, false);
+    Tensor merged = att.transpose({0, 2, 1, 3}).ascontiguousarray().reshape({Q, Dm});
+    Tensor o = proj(merged, Q, "out_proj");
+    std::vector<float> res(Q * Dm), want(Q * Dm);
+    for (size_t i = 0; i < Q * Dm; ++i) res[i] = o.typed_data<float>()[i] + xq.typed_data<float>()[i];
+    axo_layer_norm(AXO_F32, res.data(), nullptr, nullptr, want.data(), Q, Dm, 1e-5f);
+    // The bar: 2e-2 absolute plus half a bf16 ulp of the expected value.  The block rounds to bf16 six times (q, k, v,
+    // attention output, residual sum, norm output) where the fp32 evaluation rounds never; the last rounding alone
+    // is up to 2^-8 |y|, i.e. 1.6e-2 at |y| = 4, so a flat 2e-2 cannot hold for the largest outputs of any bf16 pipeline.
+    double worst = 0, worst_excess = 0;
     size_t beyond = 0;
-    for (size_t i = 0; i < S * Dm; ++i) beyond += std::fabs(double(got[i]) - want[i]) > 2e-2;
-    EXPECT_LE(double(beyond) / (S * Dm), 0.01); // 2e-2 holds for all but the largest-magnitude outputs
+    for (size_t i = 0; i < Q; ++i)
+        for (size_t j = 0; j < Dm; ++j) {
+            const double g0 = got[rows[i] * Dm + j], w0 = want[i * Dm + j], d = std::fabs(g0 - w0);
+            worst = std::max(worst, d);
+            worst_excess = std::max(worst_excess, d - (2e-2 + std::fabs(w0) * 0.00390625));
+            beyond += d > 2e-2;
+        }
+    std::printf("    S=%zu: %zu rows compared, max |err| %.4f, %zu of %zu beyond 2e-2\n", S, Q, worst, beyond, Q * Dm);
+    EXPECT_LE(worst_excess, 0.0);
+    EXPECT_LE(double(beyond) / (Q * Dm), 0.002);
 }
 GPU_TEST(WhisperBlock, ReducedSequenceMatchesFp32Reference) { whisper_case(150, true); }
-GPU_TEST(WhisperBlock, FullSizeProperties) { whisper_case(1500, false); }
+GPU_TEST(WhisperBlock, FullSizeMatchesFp32ReferenceOnSampledRows) { whisper_case(1500, true); }
 
 // ---------------------------------------------------------------------------
 // A whole pre-norm transformer encoder layer as in the reference's examples/whisper_poc.cpp:57-86
@@ -961,6 +981,41 @@ GPU_TEST(FlashAttentionMHA, FusedQkvProjectionMatchesSeparateProjections) {
             EXPECT_LT(worst, 1e-4);
         }
     }
+}
+
+// A projection weight replaced through the module's mutable parameter list (no load_state_dict, no to()): the old
+// weight's device block is freed and the same-sized new one is likely to land at the same address, which an
+// address comparison would take for "unchanged".  The stacked q/k/v weight must follow the new parameter.
+GPU_TEST(FlashAttentionMHA, StackedProjectionFollowsAParameterSwappedInPlace) {
+    const size_t B = 1, S = 40, Dm = 64;
+    auto x = axtest::randn({B, S, Dm}, 400).gpu();
+    nn::MultiHeadAttention mha(4);
+    std::map<std::string, Tensor> sd;
+    uint64_t seed = 410;
+    for (const char *name : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+        sd[std::string(name) + ".weight"] = axtest::randn({Dm, Dm}, seed++, DType::Float32, 0.125f).gpu();
+        sd[std::string(name) + ".bias"] = axtest::randn({Dm}, seed++, DType::Float32, 0.1f).gpu();
+    }
+    mha.load_state_dict(sd);
+    const Tensor x2 = x, x3 = x;
+    auto before = host_floats(mha.forward(x, x, x));
+    auto params = mha.named_parameters();
+    bool swapped = false;
+    for (auto &np : params)
+        if (np.first == "q_proj.weight") {
+            *np.second = Tensor(); // frees the old block first, so that the new weight can take its place
+            *np.second = axtest::randn({Dm, Dm}, 999, DType::Float32, 0.125f).gpu();
+            swapped = true;
+        }
+    ASSERT_TRUE(swapped);
+    auto fused = host_floats(mha.forward(x, x, x)), separate = host_floats(mha.forward(x, x2, x3));
+    double moved = 0, apart = 0;
+    for (size_t i = 0; i < fused.size(); ++i) {
+        moved = std::max(moved, std::fabs(double(fused[i]) - before[i]));
+        apart = std::max(apart, std::fabs(double(fused[i]) - separate[i]));
+    }
+    EXPECT_GT(moved, 1e-3); // the output changed with the weight ...
+    EXPECT_LT(apart, 1e-4); // ... to what the three separate projections give
 }
 
 GPU_TEST(LazyNodes, Conv2dKnownAnswers) { // tests/test_conv2d.cpp:3-111 of the reference

@@ -1,5 +1,6 @@
 #include <cstring>
 
+#include "axiom/graph/graph_registry.hpp"
 #include "test_framework.hpp"
 
 int main(int argc, char **argv) {
@@ -11,6 +12,7 @@ int main(int argc, char **argv) {
         else if (!std::strcmp(argv[i], "--list")) list = true;
         else filter = argv[i];
     }
+    axiom::graph::record_gpu_plan_kernels(true); // several cases assert which kernels a graph ran on
     int ran = 0, failed = 0, skipped = 0;
     for (const auto &c : axtest::registry()) {
         const std::string full = c.suite + "." + c.name;

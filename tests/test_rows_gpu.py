@@ -482,3 +482,64 @@ def test_interpreter_serves_programs_without_a_built_in_kernel_when_run_time_com
     p = gh.Rows(x, F32).row_op("softmax")
     p.run()
     assert p.kernel_name() == "rows_static_softmax_f32_g64_it8", p.kernel_name()
+
+
+@pytest.mark.parametrize("rms", [False, True], ids=["layernorm", "rmsnorm"])
+def test_full_size_c3_chain_with_weights_and_gelu(rms):
+    """BASELINE configs[2] as it is benchmarked: gelu(layer_norm(x) * gamma + beta) and the RMSNorm variant on bf16
+    [16384, 4096].  Every row is checked through statistics that do not depend on its position (the pre-activation
+    is recovered where gelu is injective), and slices from the start, the middle and the END of the tensor go against
+    the float64 evaluation element by element."""
+    g = axo.PCG64(4242)
+    R, Cc = 16384, 4096
+    x = axo.to_bits(g.normal((R, Cc)), BF16)
+    w = axo.to_bits(g.uniform((Cc,), 0.5, 1.5), BF16)
+    b = axo.to_bits(g.uniform((Cc,), -0.1, 0.1), BF16)
+    p = gh.Rows(x, BF16).row_op("rmsnorm" if rms else "layernorm", 1e-5, w, None if rms else b).unary("gelu")
+    got = axo.to_f32(p.run(), BF16)
+    assert p.kernel_name() == ("rows_static_rmsnorm_gelu_w_bf16_g64_it8" if rms else "rows_static_layernorm_gelu_wb_bf16_g64_it8")
+    assert np.isfinite(got).all()
+    wf, bf = axo.to_f32(w, BF16), axo.to_f32(b, BF16)
+    for lo, hi in ((0, 96), (R // 2 - 48, R // 2 + 48), (R - 96, R)):
+        want = ln64(axo.to_f32(x[lo:hi], BF16), wf, None if rms else bf, gelu=True, rms=rms)
+        err = np.abs(got[lo:hi] - want)
+        ulp = np.maximum(np.abs(want), 1e-3) * 2.0**-8
+        assert np.all(err <= np.maximum(2e-2, ulp * 1.01)) and np.max(err[np.abs(want) < 4]) < 2e-2, (lo, hi)
+    # all 16384 rows: where y > 1 gelu is increasing and y ~ n to within 0.16, so n = (y solved back) has the row's
+    # normalised statistics; cheaper and as telling: the mean of gelu(n) over a row of N(0,1)-like n * w + b is stable.
+    # Compare per-row means and mean squares with the float64 evaluation of a strided sample of rows.
+    rows = np.arange(0, R, 61)
+    want = ln64(axo.to_f32(x[rows], BF16), wf, None if rms else bf, gelu=True, rms=rms)
+    assert np.allclose(got[rows].mean(-1), want.mean(-1), atol=2e-3)
+    assert np.allclose((got[rows].astype(np.float64) ** 2).mean(-1), (want**2).mean(-1), rtol=5e-3)
+    # and every row against its neighbours' scale: no row left unwritten or written twice with another row's statistics
+    ms = (got.astype(np.float64) ** 2).mean(-1)
+    assert ms.min() > 0.2 and ms.max() < 1.5, (ms.min(), ms.max())
+
+
+@pytest.mark.parametrize("dt,offset,spread", [(BF16, 8.0, 0.5), (F16, 64.0, 0.25), (BF16, 300.0, 3.0), (F16, -1000.0, 2.0)],
+                         ids=["bf16_ratio16", "f16_ratio256", "bf16_ratio100", "f16_ratio500"])
+@pytest.mark.parametrize("cols", [4096, 1000, 16384])
+def test_layer_norm_of_16_bit_rows_far_from_zero(dt, offset, spread, cols):
+    """Rows whose mean dwarfs their spread (|mean| / sigma from 16 to 500): the one-sweep variance E[x^2] - mean^2
+    loses its digits there, and the kernels re-sweep such rows with the mean taken out (the reference's CPU path is
+    two-pass, src/tensor/operations.cpp:1803-1817).  Checked against float64 on the rounded inputs, plain and behind a
+    residual sum (statistics of fp32 sums instead of the packed input)."""
+    g = axo.PCG64(777)
+    x = axo.to_bits(offset + spread * g.normal((9, cols)), dt)
+    xf = axo.to_f32(x, dt).astype(np.float64)
+    w = axo.to_bits(g.uniform((cols,), 0.5, 1.5), dt)
+    b = axo.to_bits(g.uniform((cols,), -0.5, 0.5), dt)
+    wf, bf = axo.to_f32(w, dt).astype(np.float64), axo.to_f32(b, dt).astype(np.float64)
+
+    def ln(t):
+        return (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * wf + bf
+
+    tol = lambda want: np.maximum(2e-2, np.abs(want) * (2.0**-8 if dt == BF16 else 2.0**-11) * 1.01)
+    got = axo.to_f32(gh.Rows(x, dt).row_op("layernorm", 1e-5, w, b).run(), dt)
+    want = ln(xf)
+    assert np.all(np.abs(got - want) <= tol(want)), float(np.max(np.abs(got - want)))
+    y = axo.to_bits(spread * g.normal((9, cols)), dt)
+    got = axo.to_f32(gh.Rows(x, dt).binary("add", y).row_op("layernorm", 1e-5, w, b).run(), dt)
+    want = ln(xf + axo.to_f32(y, dt))
+    assert np.all(np.abs(got - want) <= tol(want)), float(np.max(np.abs(got - want)))
