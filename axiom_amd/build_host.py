@@ -5,6 +5,12 @@
     host_bench          times BASELINE's configurations along the whole host-layer path
     host_tests          test program; links the host layer and, as the checker only, the
                         CPU oracle (oracle/libaxiom_oracle.so)
+
+    python -m axiom_amd.build_host              the above, into axiom_amd/lib/
+    python -m axiom_amd.build_host --sanitize   the host layer and host_tests once more with AddressSanitizer and
+                                                UndefinedBehaviorSanitizer (host code only: the HIP library underneath
+                                                is the ordinary one), into axiom_amd/lib/sanitize/; run its CPU cases
+                                                with run_sanitized_cpu_tests()
 """
 from __future__ import annotations
 
@@ -38,14 +44,14 @@ def _run(cmd, what):
     return time.time() - t0
 
 
-def _compile_all(sources, tag, extra=()):
+def _compile_all(sources, tag, extra=(), flags=None):
     cxx = shutil.which("g++") or "g++"
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     objs = []
 
     def one(src: Path):
         obj = OBJ_DIR / f"{tag}_{src.stem}.o"
-        _run([cxx, *CXXFLAGS, *extra, "-c", str(src), "-o", str(obj)], f"compile {src.name}")
+        _run([cxx, *(CXXFLAGS if flags is None else flags), *extra, "-c", str(src), "-o", str(obj)], f"compile {src.name}")
         return obj
 
     with cf.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 4)) as pool:
@@ -75,5 +81,45 @@ def build_all(verbose: bool = True) -> None:
         print(f"[axiom_amd.build_host] built {HOST_LIB.name}" + (f" and {TEST_BIN.name}" if tests else "") + f" ({time.time() - t0:.1f}s)", flush=True)
 
 
+SANITIZE_DIR = LIB_DIR / "sanitize"
+SANITIZE_FLAGS = ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"]
+
+
+def build_sanitized(verbose: bool = True) -> Path:
+    """The host layer and its test program with -fsanitize=address,undefined (g++, host code), beside the ordinary
+    build.  Returns the test program's path."""
+    cxx = shutil.which("g++") or "g++"
+    SANITIZE_DIR.mkdir(parents=True, exist_ok=True)
+    t0 = time.time()
+    flags = ["-O1" if f == "-O2" else f for f in CXXFLAGS] + SANITIZE_FLAGS
+    objs = _compile_all(sorted((HOST / "src").glob("*.cpp")), "san_lib", flags=flags)
+    lib = SANITIZE_DIR / "libaxiom_hip.so"
+    _run([cxx, "-shared", *SANITIZE_FLAGS, "-o", str(lib), *map(str, objs), f"-L{LIB_DIR}", "-laxhip", "-Wl,-rpath,$ORIGIN/.."], "link sanitized libaxiom_hip.so")
+    tobjs = _compile_all(sorted((HOST / "tests").glob("*.cpp")), "san_test", extra=(f"-I{ROOT / 'oracle'}",), flags=flags)
+    exe = SANITIZE_DIR / "host_tests"
+    _run([cxx, *SANITIZE_FLAGS, "-o", str(exe), *map(str, tobjs), f"-L{SANITIZE_DIR}", "-laxiom_hip", f"-L{LIB_DIR}", "-laxhip", f"-L{ROOT / 'oracle'}",
+          "-laxiom_oracle", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath,$ORIGIN/../../../oracle", "-lpthread"], "link sanitized host_tests")
+    if verbose:
+        print(f"[axiom_amd.build_host] built {exe.relative_to(ROOT)} ({time.time() - t0:.1f}s)", flush=True)
+    return exe
+
+
+def run_sanitized_cpu_tests(timeout: float = 600.0) -> subprocess.CompletedProcess:
+    """Runs the sanitized test program's CPU cases (`host_tests --cpu`), building it first when it is missing.
+    Leak detection is off: the HIP runtime the library links keeps its own allocations until exit."""
+    exe = SANITIZE_DIR / "host_tests"
+    if not exe.exists():
+        build_sanitized(verbose=False)
+    env = dict(os.environ)
+    env["ASAN_OPTIONS"] = "detect_leaks=0:verify_asan_link_order=0:abort_on_error=0"
+    env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
+    return subprocess.run([str(exe), "--cpu"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout, env=env)
+
+
 if __name__ == "__main__":
-    build_all()
+    import sys
+
+    if "--sanitize" in sys.argv[1:]:
+        build_sanitized()
+    else:
+        build_all()

@@ -701,7 +701,19 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
                   AXHIP_ERR_INVALID_ARG, "axhip_gemm: unsupported epilogue op %d", p.epilogue_op);
     if (p.m == 0 || p.n == 0 || p.batch == 0) return AXHIP_OK;
     AXHIP_REQUIRE(a && b && c, AXHIP_ERR_INVALID_ARG, "axhip_gemm: NULL matrix");
-    AXHIP_REQUIRE(p.batch < 65536, AXHIP_ERR_UNSUPPORTED, "axhip_gemm: batch too large");
+    if (p.batch >= 65536) {
+        // the batch index is a grid dimension (at most 65 535): a larger batch runs as consecutive launches
+        const int64_t es = p.dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+        for (int64_t b0 = 0; b0 < p.batch; b0 += 65535) {
+            AxhipGemmParams part = p;
+            part.batch = std::min<int64_t>(65535, p.batch - b0);
+            if (p.residual) part.residual = static_cast<const char *>(p.residual) + b0 * p.stride_c * es;
+            const int rc_part = axhip_gemm(static_cast<const char *>(a) + b0 * p.stride_a * es, static_cast<const char *>(b) + b0 * p.stride_b * es,
+                                           static_cast<char *>(c) + b0 * p.stride_c * es, &part, stream);
+            if (rc_part) return rc_part;
+        }
+        return AXHIP_OK;
+    }
     int rc = ensure_init();
     if (rc) return rc;
     hipStream_t s = resolve_stream(stream);

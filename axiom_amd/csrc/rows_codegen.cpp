@@ -152,7 +152,7 @@ struct Builder {
     }
 
     // one chain as statements on `t`; appends the chain's tokens to the label
-    std::string chain_text(const AxhipChainOp *ops, int n, bool post, bool fast, std::string *label) {
+    std::string chain_text(const AxhipChainOp *ops, int n, bool post, int fast, std::string *label) {
         std::ostringstream o;
         for (int i = 0; i < n; ++i) {
             const int op = ops[i].op;
@@ -177,7 +177,7 @@ struct Builder {
             } else if (is_unary(op)) {
                 switch (op) {
                 case AXHIP_OP_RELU: o << "    t = t > 0.0f ? t : 0.0f;\n"; break;
-                case AXHIP_OP_GELU: o << (fast ? "    t = gelu_fast(t);\n" : "    t = gelu_exact(t);\n"); break;
+                case AXHIP_OP_GELU: o << (fast == 2 ? "    t = gelu_fast_bf16(t);\n" : fast ? "    t = gelu_fast(t);\n" : "    t = gelu_exact(t);\n"); break;
                 case AXHIP_OP_SQRT: o << "    t = sqrtf(t);\n"; break;
                 case AXHIP_OP_EXP: o << "    t = expf(t);\n"; break;
                 case AXHIP_OP_NEG: o << "    t = -t;\n"; break;
@@ -320,7 +320,8 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     S = RowsProgSpec{};
     Builder B(P, S);
     const int dt = P.input_dtype;
-    const bool fast = P.output_dtype != AXHIP_DTYPE_F32; // the result is rounded to 16 bits: fast activation forms
+    // the result is rounded to 16 bits: fast activation forms, sized to the result's precision (8 bits for bf16, 11 for f16)
+    const int fast = P.output_dtype == AXHIP_DTYPE_BF16 ? 2 : P.output_dtype == AXHIP_DTYPE_F16 ? 1 : 0;
     const bool is_norm = P.row_op == AXHIP_ROWOP_LAYERNORM || P.row_op == AXHIP_ROWOP_RMSNORM;
 
     int w_dt = -1, b_dt = -1, w_slot = -1, b_slot = -1;
@@ -364,9 +365,8 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     f << "__device__ __forceinline__ float post_chain(float t, const Env &q, int e) {\n" << post << "    return t;\n}\n";
     S.chains = f.str();
 
-    char sym[40];
-    snprintf(sym, sizeof(sym), "axp_%016llx", static_cast<unsigned long long>(fnv1a(S.chains, fnv1a(S.config))));
-    S.symbol = sym;
+    char hash[24];
+    snprintf(hash, sizeof(hash), "%016llx", static_cast<unsigned long long>(fnv1a(S.chains, fnv1a(S.config))));
     S.threads = plan.group > 256 ? plan.group : 256;
     S.rows_per_block = S.threads / plan.group;
 
@@ -377,6 +377,8 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     char tail[48];
     snprintf(tail, sizeof(tail), "%s_g%d_it%d%s", dt_name(dt), plan.group, plan.it, plan.ragged ? "_ragged" : "");
     S.label = label + tail;
+    // the kernel's symbol: the readable label (what a profiler lists) plus a hash of everything that shapes the code
+    S.symbol = "axp_" + S.label + "_" + hash;
     return true;
 }
 

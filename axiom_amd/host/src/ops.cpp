@@ -204,6 +204,22 @@ Tensor sdpa_operand(const Tensor &t) {
     for (int64_t s : st) ok = ok && s >= 0 && s % static_cast<int64_t>(g.itemsize()) == 0;
     return ok ? g : g.ascontiguousarray();
 }
+
+// src/backends/metal/flash_attention_dispatch.mm:125-162: S = Q K^T * scale, masked entries set to -1e9, softmax, P V
+Tensor decomposed_sdpa(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor &mask, float scale, bool is_causal) {
+    Tensor scores = ops::matmul(q, k, false, true);
+    scores = ops::multiply(scores, Tensor::full({1}, scale, Device::GPU).astype(scores.dtype()));
+    if (is_causal) {
+        const size_t sq = q.shape()[2], skv = k.shape()[2];
+        Tensor above = Tensor::zeros({sq, skv}, DType::Bool, Device::CPU);
+        uint8_t *a = above.typed_data<uint8_t>();
+        for (size_t i = 0; i < sq; ++i)
+            for (size_t j = i + 1; j < skv; ++j) a[i * skv + j] = 1;
+        scores = ops::masked_fill(scores, above.to(Device::GPU), -1e9f);
+    }
+    if (!mask.empty()) scores = ops::masked_fill(scores, mask, -1e9f);
+    return ops::matmul(ops::softmax(scores, -1), v);
+}
 } // namespace
 
 const char *last_sdpa_kernel() { return tl_sdpa_kernel.c_str(); }
@@ -277,6 +293,15 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
     }
     auto ptr = [](const Tensor &t) { return static_cast<const char *>(t.storage()->raw()) + t.offset(); };
     tl_sdpa_kernel = axhip_sdpa_kernel_name(&p);
+    // Shapes no attention kernel takes (head sizes above 256; 65 536 or more (batch, head) slices on the FMA kernel)
+    // are composed from the matrix product, masking and softmax kernels, as the reference composes what its own
+    // kernels do not take (src/backends/metal/flash_attention_dispatch.mm:125-162, 180-196).
+    if (tl_sdpa_kernel == "invalid" || (tl_sdpa_kernel == "generic" && B * H >= 65536)) {
+        tl_sdpa_kernel = "decomposed";
+        Tensor o = decomposed_sdpa(q, k, v, m, scale > 0.0f ? scale : 1.0f / std::sqrt(static_cast<float>(D)), is_causal);
+        if (!out_bshd) return o;
+        return o.transpose({0, 2, 1, 3}).ascontiguousarray().transpose({0, 2, 1, 3});
+    }
     AXHIP_CALL(axhip_sdpa_fwd(ptr(q), ptr(k), ptr(v), out.storage()->raw(), mask_ptr, &p, nullptr));
     return out; // asynchronous; .cpu() / item() synchronise
 }

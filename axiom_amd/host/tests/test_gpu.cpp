@@ -5,6 +5,9 @@
 // test_tensor_normalization.cpp, with the CPU side of each comparison supplied by the oracle.
 #include <map>
 
+#include <atomic>
+#include <thread>
+
 #include "oracle_util.hpp"
 #include "test_framework.hpp"
 
@@ -125,6 +128,47 @@ GPU_TEST(FusionGpu, PlanCacheHitsAndMisses) { // tests/test_graph_compiler.cpp:7
     EXPECT_NEAR(run(5, 1.5f), 3.0f, 0);  // other shape: new plan
     EXPECT_EQ(cache.misses(), 2u);
     EXPECT_EQ(cache.size(), 2u);
+}
+GPU_TEST(FusionGpu, TwoHostThreadsMaterialiseAtOnce) {
+    // Two host threads build and materialise graphs at the same time: one plan that both share (the plan cache is hit
+    // from both sides) and one per thread; every result is checked.  What the threads share is the plan cache, the
+    // caching allocator, the device scalar cache and the library's stream.
+    auto a = axtest::randn({64, 96}, 5), b = axtest::randn({64, 96}, 6);
+    const Tensor ag = a.gpu(), bg = b.gpu();
+    const std::vector<float> av = host_floats(a), bv = host_floats(b);
+    std::atomic<int> bad{0}, done{0};
+    auto worker = [&](int id) {
+        try {
+            for (int it = 0; it < 200; ++it) {
+                Tensor shared = ops::relu(ag + bg) * 2.0f;                                   // same signature in both threads
+                Tensor own = id == 0 ? ops::softmax(ag * 0.5f, -1) : ops::sum(ops::square(bg - 1.0f), {1}, false); // one per thread
+                const std::vector<float> s = host_floats(shared.cpu()), o = host_floats(own.cpu());
+                for (size_t i = 0; i < s.size(); i += 97)
+                    if (std::fabs(s[i] - std::max(av[i] + bv[i], 0.0f) * 2.0f) > 1e-5f) ++bad;
+                if (id == 0) {
+                    for (size_t r = 0; r < 64; r += 9) {
+                        double sum = 0;
+                        for (size_t c = 0; c < 96; ++c) sum += o[r * 96 + c];
+                        if (std::fabs(sum - 1.0) > 1e-4) ++bad;
+                    }
+                } else {
+                    for (size_t r = 0; r < 64; r += 9) {
+                        double want = 0;
+                        for (size_t c = 0; c < 96; ++c) want += (bv[r * 96 + c] - 1.0) * (bv[r * 96 + c] - 1.0);
+                        if (std::fabs(o[r] - want) > 1e-3 * (1.0 + want)) ++bad;
+                    }
+                }
+            }
+            ++done;
+        } catch (const std::exception &) {
+            ++bad;
+        }
+    };
+    std::thread t0(worker, 0), t1(worker, 1);
+    t0.join();
+    t1.join();
+    EXPECT_EQ(done.load(), 2);
+    EXPECT_EQ(bad.load(), 0);
 }
 GPU_TEST(FusionGpu, BroadcastKinds) { // tests/test_cpu_gpu_parity.cpp broadcast cases
     auto a = axtest::randn({4, 5}, 5), row = axtest::randn({5}, 6), col = axtest::randn({4, 1}, 7);
@@ -371,6 +415,38 @@ GPU_TEST(FlashAttentionGPU, Config1Float32) { // BASELINE configs[0]: B1 H8 S512
     auto [q, k, v] = make_inputs(1, 8, 512, 512, 64);
     auto got = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), 0.125f, false);
     ASSERT_TENSORS_CLOSE(got.cpu(), axtest::oracle_sdpa(q, k, v, Tensor(), 0.125f, false), 1e-4, 1e-4);
+}
+
+GPU_TEST(FlashAttentionGPU, ShapesNoKernelTakesAreComposedFromMatmulMaskAndSoftmax) { // flash_attention_dispatch.mm:125-162
+    // head sizes above 256: plain, causal (query and key counts differ), and with a Bool mask shared by all heads
+    auto [q, k, v] = make_inputs(1, 2, 40, 56, 320);
+    for (bool causal : {false, true}) {
+        auto got = ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), Tensor(), -1, causal);
+        EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("decomposed"));
+        EXPECT_EQ(got.shape(), q.shape());
+        ASSERT_TENSORS_CLOSE(got.cpu(), axtest::oracle_sdpa(q, k, v, Tensor(), -1, causal), 1e-4, 1e-4);
+    }
+    Tensor m2({40, 56}, DType::Bool);
+    for (size_t i = 0; i < 40; ++i)
+        for (size_t j = 0; j < 56; ++j) m2.set_item<int>({i, j}, (i + j) % 3 == 0);
+    ASSERT_TENSORS_CLOSE(ops::scaled_dot_product_attention(q.gpu(), k.gpu(), v.gpu(), m2.gpu(), 0.05f, false).cpu(), axtest::oracle_sdpa(q, k, v, m2, 0.05f, false), 1e-4, 1e-4);
+    EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("decomposed"));
+    // bf16 at head size 512
+    {
+        auto [qh, kh, vh] = make_inputs(2, 3, 33, 33, 512, DType::BFloat16);
+        auto ref = axtest::oracle_sdpa(qh.astype(DType::Float32), kh.astype(DType::Float32), vh.astype(DType::Float32), Tensor(), -1, true);
+        auto got = ops::scaled_dot_product_attention(qh.gpu(), kh.gpu(), vh.gpu(), Tensor(), -1, true);
+        EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("decomposed"));
+        EXPECT_EQ(got.dtype(), DType::BFloat16);
+        EXPECT_LE(max_abs_diff(got, ref), 3e-2); // the scores and the weights each pass through bf16 on the composed path
+    }
+    // 65 536 (batch, head) slices of a head size that only the FMA kernel takes
+    {
+        auto [qs, ks, vs] = make_inputs(256, 256, 4, 4, 8);
+        auto got = ops::scaled_dot_product_attention(qs.gpu(), ks.gpu(), vs.gpu(), Tensor(), -1, false);
+        EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("decomposed"));
+        ASSERT_TENSORS_CLOSE(got.cpu(), axtest::oracle_sdpa(qs, ks, vs, Tensor(), -1, false), 1e-4, 1e-4);
+    }
 }
 
 // ------------------------------------------------------------------------ nn

@@ -35,14 +35,24 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-# HBM bytes per launch of the SDPA kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script, each scaled by the reading of the plain-copy leg below
-# (FETCH_SIZE 0.50012, WRITE_SIZE 1.0): 585.2 MB read + 134.2 MB written.
-SDPA_TRAFFIC_BYTES = 719.5e6
-# same measurement for the fused chains: they move the algorithmic bytes (ratio 1.001 - 1.003)
-CHAIN_TRAFFIC_BYTES = {"chain_relu_add_mul_softmax_sum_f32_8192x8192": 537.2e6,
-                       "chain_gelu_layernorm_bf16_16384x4096": 269.1e6,
-                       "chain_gelu_rmsnorm_bf16_16384x4096": 269.2e6}
+# HBM bytes per launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a copy kernel of known size:
+# read from the committed summary of those runs (a table whose rows start with the workload's key in backticks and end
+# with the bytes per launch); a workload the summary does not hold reports null
+TRAFFIC_PROFILE = ROOT / "profiles" / "bench_kernels_hbm_traffic.md"
+
+
+def traffic_from_profile() -> dict:
+    out = {}
+    if not TRAFFIC_PROFILE.exists():
+        return out
+    for ln in TRAFFIC_PROFILE.read_text().splitlines():
+        cells = [c.strip() for c in ln.strip().strip("|").split("|")]
+        if len(cells) >= 3 and cells[0].startswith("`") and cells[0].endswith("`"):
+            try:
+                out[cells[0].strip("`")] = float(cells[-1].replace(" ", ""))
+            except ValueError:
+                pass
+    return out
 
 
 MIN_WARMUP_MS = 100.0  # clocks and power settle within about this much work of one kind ...
@@ -50,20 +60,26 @@ MAX_SETTLE_MS = 1500.0  # ... but a leg that follows a very different one can ta
 
 
 def time_launches(torch, stream, launch, steps: int, warmup: int):
-    """Average launch duration in ms over `steps` launches, HIP events on `stream`.
-    Warm-up: `warmup` launches, continued until MIN_WARMUP_MS of work has run (short kernels
-    would otherwise be timed while the device is still changing clocks), then batches of launches
-    until two consecutive batches agree within 1 % (at most MAX_SETTLE_MS): the figure is the steady
-    state of this kernel, not the tail of the previous leg's power state."""
+    """(average launch duration in ms over exactly `steps` launches, shortest single launch in ms, number of
+    warm-up launches that ran before the timed region).  The average is the time between two HIP events on `stream`
+    that bracket the `steps` launches; the shortest launch comes from a second, untimed round with an event after
+    every launch.  Warm-up: `warmup` launches, continued until MIN_WARMUP_MS of work has run (short kernels would
+    otherwise be timed while the device is still changing clocks), then batches of launches until two consecutive
+    batches agree within 1 % (at most MAX_SETTLE_MS): the figure is the steady state of this kernel, not the tail of
+    the previous leg's power state."""
+    ran = 0
     with torch.cuda.stream(stream):
         t0 = time.time()
         for _ in range(warmup):
             launch()
+        ran += warmup
         stream.synchronize()
         spent_ms = (time.time() - t0) * 1e3
         if warmup > 0 and spent_ms < MIN_WARMUP_MS:
-            for _ in range(int((MIN_WARMUP_MS - spent_ms) / (spent_ms / warmup)) + 1):
+            more = int((MIN_WARMUP_MS - spent_ms) / (spent_ms / warmup)) + 1
+            for _ in range(more):
                 launch()
+            ran += more
             stream.synchronize()
         if warmup > 0:
             batch = max(10, warmup)
@@ -75,11 +91,19 @@ def time_launches(torch, stream, launch, steps: int, warmup: int):
                     launch()
                 e1.record(stream)
                 stream.synchronize()
+                ran += batch
                 t = e0.elapsed_time(e1)
                 agree = agree + 1 if prev is not None and abs(t - prev) <= 0.01 * prev else 0
                 prev = t
                 if agree >= 2:
                     break
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            launch()
+        e1.record(stream)
+        stream.synchronize()
+        total = e0.elapsed_time(e1)
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         evs[0].record(stream)
         for i in range(steps):
@@ -87,8 +111,7 @@ def time_launches(torch, stream, launch, steps: int, warmup: int):
             evs[i + 1].record(stream)
         stream.synchronize()
     per = [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)]
-    total = evs[0].elapsed_time(evs[steps])
-    return total / steps, min(per), sorted(per)[len(per) // 2]
+    return total / steps, min(per), ran
 
 
 def bench_sdpa(torch, capi, stream, steps, warmup):
@@ -109,11 +132,11 @@ def bench_sdpa(torch, capi, stream, steps, warmup):
         capi.check(lib.axhip_sdpa_fwd(*args))
 
     torch.cuda.synchronize()
-    avg_ms, min_ms, med_ms = time_launches(torch, stream, launch, steps, warmup)
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
     flops = 4.0 * B * H * S * S * D / 2.0
     return {
         "kernel": lib.axhip_sdpa_kernel_name(C.byref(p)).decode(),
-        "avg_ms": avg_ms, "min_ms": min_ms, "median_ms": med_ms,
+        "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
         "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
         "finite": bool(torch.isfinite(o.float()).all().item()),
     }
@@ -151,10 +174,10 @@ def bench_chains(torch, capi, stream, steps, warmup):
     p.row_op = capi.ROWOP["softmax"]
     p.reduce = capi.RED["sum"]
     torch.cuda.synchronize()
-    avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
     nbytes = 2 * R * Cc * 4 + R * 4
     res["chain_relu_add_mul_softmax_sum_f32_8192x8192"] = {
-        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms,
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
         "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
         "rows_sum_to_one": bool(torch.allclose(out, torch.ones_like(out), atol=1e-4)),
     }
@@ -163,10 +186,10 @@ def bench_chains(torch, capi, stream, steps, warmup):
     cp = torch.empty_like(a)
     pc = _rows_program(capi, a, cp, capi.DTYPE_F32, capi.DTYPE_F32)
     torch.cuda.synchronize()
-    avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(pc), sp)), steps, warmup)
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(pc), sp)), steps, warmup)
     nbytes = 2 * R * Cc * 4
     res["copy_f32_8192x8192"] = {
-        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(pc)).decode(), "avg_ms": avg_ms, "min_ms": min_ms,
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(pc)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
         "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
         "bit_exact": bool(torch.equal(cp, a)),
     }
@@ -189,10 +212,10 @@ def bench_chains(torch, capi, stream, steps, warmup):
         p.post[0].op, p.post[0].operand = capi.OP["gelu"], -1
         p.reduce = capi.RED["none"]
         torch.cuda.synchronize()
-        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
         nbytes = 2 * R * Cc * 2 + Cc * 2 * (2 if has_bias else 1)
         res[f"chain_gelu_{name}_bf16_16384x4096"] = {
-            "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms,
+            "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
             "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
             "finite": bool(torch.isfinite(y.float()).all().item()),
         }
@@ -203,11 +226,11 @@ def bench_chains(torch, capi, stream, steps, warmup):
     p = _rows_program(capi, xr, yr, capi.DTYPE_BF16, capi.DTYPE_BF16)
     p.row_op, p.reduce = capi.ROWOP["softmax"], capi.RED["none"]
     torch.cuda.synchronize()
-    avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
     nbytes = 2 * Rr * Cr * 2
     sums = yr.float().sum(1)
     res["softmax_bf16_30000x1500_odd_row_length"] = {
-        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms,
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
         "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
         "rows_sum_to_one": bool(((sums - 1.0).abs() < 2e-2).all().item()),
     }
@@ -287,7 +310,7 @@ def bench_survey(torch, capi, stream, steps, warmup):
     def run(name, prog):
         lib.axhip_fused_rows_prepare(C.byref(prog.p))
         torch.cuda.synchronize()
-        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(prog.p), sp)), steps, warmup)
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(prog.p), sp)), steps, warmup)
         res[name] = {"kernel": lib.axhip_fused_rows_kernel_name(C.byref(prog.p)).decode(), "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3,
                      "bytes": prog.bytes, "frac_of_hbm_peak": prog.bytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                      "finite": bool(torch.isfinite(prog.out.float()).all().item())}
@@ -364,13 +387,13 @@ def bench_gemm(torch, capi, stream, steps, warmup):
         p.lda, p.ldb, p.ldc, p.batch = K, K, N, 1
         args = (a.data_ptr(), w.data_ptr(), c.data_ptr(), C.byref(p), sp)
         torch.cuda.synchronize()
-        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps, warmup)
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps, warmup)
         flops = 2.0 * M * N * K
         # the vendor library on the same operands (torch.matmul -> hipBLASLt), for context only
         with torch.cuda.stream(stream):
             wt = w.t()
             lib_ms, _, _ = time_launches(torch, stream, lambda: torch.matmul(a, wt), steps, warmup)
-        res[f"gemm_nt_bf16_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
+        res[f"gemm_nt_bf16_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
                                              "frac_of_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                                              "finite": bool(torch.isfinite(c.float()).all().item()),
                                              "hipblaslt_avg_ms": lib_ms}
@@ -400,9 +423,9 @@ def bench_f32(torch, capi, stream, steps, warmup):
             arr[0], arr[1], arr[2] = H * S * D, S * D, D
         args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, C.byref(p), sp)
         torch.cuda.synchronize()
-        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_sdpa_fwd(*args)), steps_f32, warmup_f32)
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_sdpa_fwd(*args)), steps_f32, warmup_f32)
         flops = 4.0 * B * H * S * S * D
-        res[f"sdpa_f32_b{B}h{H}s{S}d{D}"] = {"kernel": lib.axhip_sdpa_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "flops": flops,
+        res[f"sdpa_f32_b{B}h{H}s{S}d{D}"] = {"kernel": lib.axhip_sdpa_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n, "flops": flops,
                                              "tflops": flops / (avg_ms * 1e-3) / 1e12, "frac_of_f32_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_F32_MFMA_TFLOPS,
                                              "finite": bool(torch.isfinite(o).all().item())}
         del q, k, v, o
@@ -416,13 +439,24 @@ def bench_f32(torch, capi, stream, steps, warmup):
         p.lda, p.ldb, p.ldc, p.batch = K, K, N, 1
         args = (a.data_ptr(), w.data_ptr(), c.data_ptr(), C.byref(p), sp)
         torch.cuda.synchronize()
-        avg_ms, min_ms, _ = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps_f32, warmup_f32)
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_gemm(*args)), steps_f32, warmup_f32)
         flops = 2.0 * M * N * K
-        res[f"gemm_nt_f32_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
+        res[f"gemm_nt_f32_{M}x{N}x{K}"] = {"avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n, "flops": flops, "tflops": flops / (avg_ms * 1e-3) / 1e12,
                                             "frac_of_f32_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_F32_MFMA_TFLOPS,
                                             "finite": bool(torch.isfinite(c).all().item())}
         del a, w, c
     return res
+
+
+def _oracle_build_flags() -> str:
+    """The compiler line the oracle library was built with (oracle/Makefile), for the baseline's description."""
+    cc, flags = "gcc", "?"
+    for ln in (ROOT / "oracle" / "Makefile").read_text().splitlines():
+        if ln.startswith("CFLAGS ?="):
+            flags = ln.split("=", 1)[1].strip()
+        if ln.startswith("CC ?="):
+            cc = ln.split("=", 1)[1].strip()
+    return f"{cc} {flags}"
 
 
 def cpu_baseline(seconds_budget: float = 20.0):
@@ -455,8 +489,78 @@ def cpu_baseline(seconds_budget: float = 20.0):
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
         "sample": f"{n} of 128 (batch, head) slices of the bf16 B4 H32 S4096 D128 causal problem, {dt:.2f} s wall, "
                   f"tiled CPU flash attention (64x64 blocks, native sgemm tier, masked blocks not skipped), "
-                  f"{threads} OpenMP threads; FLOPs counted as 4*S^2*D/2 per slice",
+                  f"{threads} OpenMP threads; FLOPs counted as 4*S^2*D/2 per slice; built with `{_oracle_build_flags()}` "
+                  f"(x86-64-v3 = AVX2+FMA, not -march=native: the library is compiled on another host than the one it is timed on)",
     }
+
+
+def cpu_baselines_other_configs():
+    """The oracle's restatement of Axiom's CPU path on the other configurations (BASELINE.json configs[0], [1], [2]
+    and [4]) in full size, each in the unit of its GPU figure: one untimed pass, then the median of three."""
+    import numpy as np
+
+    from oracle import axo
+
+    threads = axo.num_threads()
+    g = axo.PCG64(42)
+    how = f"{threads} OpenMP threads, 1 warm-up + median of 3 passes, built with `{_oracle_build_flags()}`"
+
+    def median3(fn):
+        fn()
+        ts = []
+        for _ in range(3):
+            t0 = time.time()
+            fn()
+            ts.append(time.time() - t0)
+        return sorted(ts)[1]
+
+    res = {}
+    # configs[0]: fp32 attention B1 H8 S512 D64
+    q, k, v = (g.normal((1, 8, 512, 64)).astype(np.float32) for _ in range(3))
+    t = median3(lambda: axo.sdpa(q, k, v, axo.F32, -1.0, False))
+    res["c1_sdpa_f32_b1h8s512d64"] = {"value": 4.0 * 8 * 512 * 512 * 64 / t / 1e9, "unit": "GFLOP/s", "seconds": t, "cores": threads, "kind": "port",
+                                      "sample": "the whole configuration; tiled CPU flash attention, native sgemm tier; " + how}
+    # configs[1]: softmax((relu(a)+1)*b).sum(1), fp32 [8192, 8192], op by op as the CPU path runs it
+    R = Cc = 8192
+    a, b = g.normal((R, Cc)).astype(np.float32), g.normal((R, Cc)).astype(np.float32)
+    t = median3(lambda: axo.chain_relu_add_mul_softmax_sum(a, b))
+    res["c2_chain_f32_8192x8192"] = {"value": (2 * R * Cc * 4 + R * 4) / t / 1e9, "unit": "GB/s", "seconds": t, "cores": threads, "kind": "port",
+                                     "sample": "the whole configuration; one pass per operation (relu, +1, *b, 3-pass softmax, row sum), "
+                                               "rate over the fused kernel's algorithmic bytes; " + how}
+    del a, b
+    # configs[2]: gelu(layernorm(x)*gamma+beta) and the RMSNorm variant, bf16 [16384, 4096]
+    R, Cc = 16384, 4096
+    x = axo.to_bits(g.normal((R, Cc)), axo.BF16)
+    gamma, beta = axo.to_bits(g.uniform((Cc,), 0.5, 1.5), axo.BF16), axo.to_bits(g.uniform((Cc,), -0.1, 0.1), axo.BF16)
+    t = median3(lambda: axo.unary("gelu", axo.to_bits(axo.layer_norm(x, gamma, beta, axo.BF16, 1e-5), axo.BF16), axo.BF16))
+    res["c3_gelu_layernorm_bf16_16384x4096"] = {"value": (2 * R * Cc * 2 + 2 * Cc * 2) / t / 1e9, "unit": "GB/s", "seconds": t, "cores": threads, "kind": "port",
+                                                "sample": "the whole configuration; decomposed layer norm, conversion to bf16, gelu pass; rate over the fused "
+                                                          "kernel's algorithmic bytes; " + how}
+    t = median3(lambda: axo.unary("gelu", axo.to_bits(axo.rms_norm(x, gamma, axo.BF16, 1e-5), axo.BF16), axo.BF16))
+    res["c3_gelu_rmsnorm_bf16_16384x4096"] = {"value": (2 * R * Cc * 2 + Cc * 2) / t / 1e9, "unit": "GB/s", "seconds": t, "cores": threads, "kind": "port",
+                                              "sample": "as the layer-norm variant, with the decomposed RMS norm"}
+    del x
+    # configs[4]: x + out_proj(attention(q_proj x, k_proj x, v_proj x)), then layer norm; x [1500, 1280] bf16, 20 heads of 64
+    S, Dm, Hh = 1500, 1280, 20
+    xb = axo.to_bits(g.normal((S, Dm)), axo.BF16)
+    w = [axo.to_bits(g.normal((Dm, Dm)) * 0.02, axo.BF16) for _ in range(4)]
+    ones, zeros = axo.to_bits(np.ones(Dm), axo.BF16), axo.to_bits(np.zeros(Dm), axo.BF16)
+
+    def block():
+        heads = [np.ascontiguousarray(axo.matmul(xb, w[i], axo.BF16, False, True).reshape(1, S, Hh, Dm // Hh).transpose(0, 2, 1, 3)) for i in range(3)]
+        o = axo.sdpa(heads[0], heads[1], heads[2], axo.BF16, -1.0, False)
+        o = np.ascontiguousarray(o.transpose(0, 2, 1, 3)).reshape(S, Dm)
+        y = axo.binary("add", xb, axo.matmul(o, w[3], axo.BF16, False, True), axo.BF16)
+        return axo.layer_norm(y, ones, zeros, axo.BF16, 1e-5)
+
+    t0 = time.time()  # its 16-bit x W^T is a plain triple loop on the CPU path: ~15 s a pass, so one pass only
+    block()
+    t = time.time() - t0
+    res["c5_whisper_block_bf16_s1500_d1280_h20"] = {"value": (8.0 * S * Dm * Dm + 4.0 * S * S * Dm) / t / 1e9, "unit": "GFLOP/s", "seconds": t, "cores": threads,
+                                                    "kind": "port", "sample": "the whole configuration; four x W^T on the native sgemm tier, tiled attention, "
+                                                                              "residual add, decomposed layer norm; "
+                                                                              f"ONE pass, no warm-up, {threads} OpenMP threads, built with `{_oracle_build_flags()}`"}
+    return res
 
 
 def host_layer_bench():
@@ -508,12 +612,15 @@ def main() -> int:
     f32 = bench_f32(torch, capi, stream, args.steps, args.warmup) if args.only in (None, "f32") else None
     survey = bench_survey(torch, capi, stream, args.steps, args.warmup) if args.only == "survey" else None
     cpu = None if (args.no_cpu or sd is None) else cpu_baseline()
+    cpu_other = None if (args.no_cpu or args.only is not None) else cpu_baselines_other_configs()
+    traffic = traffic_from_profile()
 
     line = {
         "metric": "SDPA TFLOP/s (bf16 B4 H32 S4096 D128) + fused-chain HBM GB/s, % of peak",
         "value": sd["tflops"] if sd else None,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "warmup_launches_run": sd["warmup_launches"] if sd else None,
         "ms_per_step": sd["avg_ms"] if sd else None,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
@@ -523,14 +630,14 @@ def main() -> int:
     if sd:
         line["roofline"] = {
             "bound": "mfma", "kernel": "sdpa_" + sd["kernel"], "achieved": sd["tflops"], "peak": PEAK_BF16_TFLOPS,
-            "unit": "TFLOP/s", "frac": sd["tflops"] / PEAK_BF16_TFLOPS, "traffic": SDPA_TRAFFIC_BYTES,
+            "unit": "TFLOP/s", "frac": sd["tflops"] / PEAK_BF16_TFLOPS, "traffic": traffic.get("sdpa_bf16_causal_b4h32s4096d128"),
+            "traffic_source": str(TRAFFIC_PROFILE.relative_to(ROOT)),
             "algorithmic_flops_per_launch": sd["flops"], "avg_launch_ms": sd["avg_ms"], "min_launch_ms": sd["min_ms"],
         }
         line["output_finite"] = sd["finite"]
     if ch:
         for name, rec in ch.items():
-            if name in CHAIN_TRAFFIC_BYTES:
-                rec["traffic"] = CHAIN_TRAFFIC_BYTES[name]
+            rec["traffic"] = traffic.get(name)
         line["fused_chains"] = ch
     if gm:
         line["gemm"] = gm
@@ -539,9 +646,30 @@ def main() -> int:
     if survey:
         line["row_program_survey"] = survey
     if args.only is None:
-        line["host_layer"] = host_layer_bench()
+        hl = host_layer_bench()
+        # fractions of peak along the whole drop-in path: one materialisation with its own wait, and 16 queued per wait
+        for rec in hl.values():
+            if not isinstance(rec, dict):
+                continue
+            for key, peak, tag in (("GB_per_s", PEAK_HBM_GBS, "frac_of_hbm_peak"), ("GFLOP_per_s", PEAK_BF16_TFLOPS * 1e3, "frac_of_bf16_mfma_peak")):
+                if key in rec:
+                    rec[tag] = rec[key] / peak
+                    if "queued_" + key in rec:
+                        rec["queued_" + tag] = rec["queued_" + key] / peak
+        line["host_layer"] = hl
     if cpu:
         line["cpu_baseline"] = cpu
+    if cpu_other:
+        # the GPU figure of the same configuration beside each CPU figure, in the same unit
+        hl = line.get("host_layer", {})
+        gpu = {"c1_sdpa_f32_b1h8s512d64": (f32 or {}).get("sdpa_f32_b1h8s512d64", {}).get("tflops", 0.0) * 1e3 or None,
+               "c2_chain_f32_8192x8192": (ch or {}).get("chain_relu_add_mul_softmax_sum_f32_8192x8192", {}).get("gbs"),
+               "c3_gelu_layernorm_bf16_16384x4096": (ch or {}).get("chain_gelu_layernorm_bf16_16384x4096", {}).get("gbs"),
+               "c3_gelu_rmsnorm_bf16_16384x4096": (ch or {}).get("chain_gelu_rmsnorm_bf16_16384x4096", {}).get("gbs"),
+               "c5_whisper_block_bf16_s1500_d1280_h20": hl.get("c5_whisper_block_bf16_s1500_d1280_h20", {}).get("GFLOP_per_s")}
+        for name, rec in cpu_other.items():
+            rec["gpu_value"] = gpu.get(name)
+        line["cpu_baselines_other_configs"] = cpu_other
     line["bench_wall_s"] = time.time() - t_wall0
     print(json.dumps(line))
     return 0

@@ -54,6 +54,21 @@ def test_safetensors_reader_on_a_file_from_the_python_package(tmp_path):
     assert " 0 failed" in p.stdout and " 0 skipped" in p.stdout
 
 
+def test_host_cases_without_device_under_address_and_undefined_behaviour_sanitizers():
+    """The host layer built once more with -fsanitize=address,undefined (python -m axiom_amd.build_host --sanitize;
+    built here when it is missing) passes its device-free cases with no report from either sanitizer."""
+    from axiom_amd import build_host
+    from oracle import axo
+
+    _ensure_built()
+    axo.build()
+    p = build_host.run_sanitized_cpu_tests()
+    print(p.stdout[-6000:])
+    assert p.returncode == 0, p.stdout[-3000:]
+    assert " 0 failed" in p.stdout
+    assert "AddressSanitizer" not in p.stdout and "runtime error:" not in p.stdout
+
+
 def test_product_libraries_do_not_link_the_oracle():
     _ensure_built()
     for lib in ("libaxhip.so", "libaxiom_hip.so"):
