@@ -478,8 +478,13 @@ int pick_vector_width(const AxhipRowsProgram &P) {
                 return false;
         return true;
     };
-    bool any16 = P.input_dtype != AXHIP_DTYPE_F32;
-    if (any16 && fits(8)) return 8;
+    // 8 elements per access only when every full-size stream is 16-bit: with an fp32 stream among them that stream's
+    // 32 bytes per lane would go out as two accesses that each fill half of every 32-byte run (bf16 -> fp32 casts
+    // ran at 42 % of the HBM peak that way)
+    bool wide = P.input_dtype == AXHIP_DTYPE_F32 || (P.reduce == AXHIP_RED_NONE && P.output_dtype == AXHIP_DTYPE_F32);
+    for (int i = 0; i < P.n_operands; ++i)
+        if (P.operands[i].kind == AXHIP_BK_FULL && P.operands[i].dtype == AXHIP_DTYPE_F32) wide = true;
+    if (!wide && fits(8)) return 8;
     if (fits(4)) return 4;
     return 1;
 }

@@ -177,14 +177,14 @@ struct Builder {
             } else if (is_unary(op)) {
                 switch (op) {
                 case AXHIP_OP_RELU: o << "    t = t > 0.0f ? t : 0.0f;\n"; break;
-                case AXHIP_OP_GELU: o << (fast == 2 ? "    t = gelu_fast_bf16(t);\n" : fast ? "    t = gelu_fast(t);\n" : "    t = gelu_exact(t);\n"); break;
+                case AXHIP_OP_GELU: o << (fast == 2 ? "    t = gelu_fast_bf16(t);\n" : fast ? "    t = gelu_fast(t);\n" : "    t = gelu_erfc(t);\n"); break;
                 case AXHIP_OP_SQRT: o << "    t = sqrtf(t);\n"; break;
                 case AXHIP_OP_EXP: o << "    t = expf(t);\n"; break;
                 case AXHIP_OP_NEG: o << "    t = -t;\n"; break;
                 case AXHIP_OP_ABS: o << "    t = fabsf(t);\n"; break;
-                case AXHIP_OP_SIGMOID: o << (fast ? "    t = sigmoid_fast(t);\n" : "    t = sigmoid_exact(t);\n"); break;
+                case AXHIP_OP_SIGMOID: o << "    t = sigmoid_fast(t);\n"; break;
                 case AXHIP_OP_TANH: o << (fast ? "    t = tanh_fast(t);\n" : "    t = tanhf(t);\n"); break;
-                case AXHIP_OP_SILU: o << (fast ? "    t = silu_fast(t);\n" : "    t = t / (1.0f + expf(-t));\n"); break;
+                case AXHIP_OP_SILU: o << "    t = silu_fast(t);\n"; break;
                 case AXHIP_OP_LOG: o << "    t = logf(t);\n"; break;
                 case AXHIP_OP_SQUARE: o << "    t = t * t;\n"; break;
                 case AXHIP_OP_RSQRT: o << "    t = 1.0f / sqrtf(t);\n"; break;
@@ -211,10 +211,31 @@ std::string int_table(const char *name, const int *v, int n) {
 } // namespace
 
 namespace {
+bool names_operand(const AxhipRowsProgram &P, int idx) {
+    auto in = [&](const AxhipChainOp *ops, int n) {
+        for (int i = 0; i < n; ++i)
+            if (is_binary(ops[i].op) && ops[i].imm_kind != AXHIP_BK_IMM && ops[i].operand == idx) return true;
+        return false;
+    };
+    return in(P.pre, P.n_pre) || in(P.post, P.n_post);
+}
+} // namespace
+
+// Elements per chunk: 16 bytes of the widest full-size stream (the input, a full-size output, the full-size operands
+// the chains name), so that every access of every stream is a contiguous run across the lanes of a wave: 4 as soon as
+// one of them is fp32 (a 16-bit stream then moves 8 bytes per lane), else 8.
+int rows_prog_chunk_elems(const AxhipRowsProgram &P) {
+    bool wide = P.input_dtype == AXHIP_DTYPE_F32 || (P.reduce == AXHIP_RED_NONE && P.output_dtype == AXHIP_DTYPE_F32);
+    for (int i = 0; i < P.n_operands; ++i)
+        if (P.operands[i].kind == AXHIP_BK_FULL && P.operands[i].dtype == AXHIP_DTYPE_F32 && names_operand(P, i)) wide = true;
+    return wide ? 4 : 8;
+}
+
+namespace {
 // 32-bit words of raw input a thread holds per chunk: the input and every full-size operand the chains name
 int raw_words_per_chunk(const AxhipRowsProgram &P) {
-    const int e = P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8;
-    int words = 4;
+    const int e = rows_prog_chunk_elems(P);
+    int words = e * elem_size(P.input_dtype) / 4;
     bool used[AXHIP_MAX_OPERANDS] = {};
     auto mark = [&](const AxhipChainOp *ops, int n) {
         for (int i = 0; i < n; ++i)
@@ -229,7 +250,7 @@ int raw_words_per_chunk(const AxhipRowsProgram &P) {
 // the same for the norm weight and bias of a row that spans several waves (a wavefront row reads them from LDS)
 int affine_words_per_chunk(const AxhipRowsProgram &P, int group) {
     if (group == 64) return 0;
-    const int e = P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8;
+    const int e = rows_prog_chunk_elems(P);
     int words = 0;
     for (int idx : {P.norm_weight, P.norm_bias})
         if (idx >= 0 && idx < P.n_operands) words += e * elem_size(P.operands[idx].dtype) / 4;
@@ -249,7 +270,7 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     // Register allocation aims at 4 waves per SIMD (128 registers per thread).  The widest plans hold more than
     // that with their operands: they get the registers of 2 waves per SIMD instead of spilling.
     const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
-    const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? (P.input_dtype == AXHIP_DTYPE_F32 ? 4 : 8) * it : 0);
+    const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? rows_prog_chunk_elems(P) * it : 0);
     plan->min_waves = held + (ragged ? 3 * it + 16 : 0) > 72 ? 2 : 4;
 }
 
@@ -257,7 +278,7 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     if (P.cols <= 0) return false;
     if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) return false; // flat elementwise chains have a kernel of their own
     const int dt = P.input_dtype;
-    const int e = dt == AXHIP_DTYPE_F32 ? 4 : 8;
+    const int e = rows_prog_chunk_elems(P);
     if (P.cols < e) return false;
     bool ragged = P.cols % e != 0 || !aligned16(P.input) || (P.reduce == AXHIP_RED_NONE && !aligned16(P.output));
     bool same_size = P.reduce != AXHIP_RED_NONE || elem_size(P.output_dtype) == elem_size(dt);
@@ -346,7 +367,7 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     const int red = P.reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : P.reduce;
     std::ostringstream c;
     c << "constexpr int DT_IN = " << dt << ", DT_OUT = " << (P.reduce == AXHIP_RED_NONE ? P.output_dtype : dt) << ";\n";
-    c << "constexpr int GROUP = " << plan.group << ", IT = " << plan.it << ";\n";
+    c << "constexpr int GROUP = " << plan.group << ", IT = " << plan.it << ", E = " << rows_prog_chunk_elems(P) << ";\n";
     c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ";\n";
     c << "constexpr int MIN_WAVES = " << plan.min_waves << ";\n";
     c << "constexpr int ROWOP = " << P.row_op << ", RED = " << red << ";\n";
@@ -374,8 +395,10 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     if (w_dt >= 0) label += b_dt >= 0 ? "wb_" : "w_";
     else if (b_dt >= 0) label += "b_";
     if (red != AXHIP_RED_NONE) label += red == AXHIP_RED_SUM ? "sum_" : red == AXHIP_RED_MAX ? "max_" : "min_";
-    char tail[48];
-    snprintf(tail, sizeof(tail), "%s_g%d_it%d%s", dt_name(dt), plan.group, plan.it, plan.ragged ? "_ragged" : "");
+    char tail[64];
+    const bool other_out = P.reduce == AXHIP_RED_NONE && P.output_dtype != dt;
+    snprintf(tail, sizeof(tail), "%s%s%s_g%d_it%d%s", dt_name(dt), other_out ? "_to_" : "", other_out ? dt_name(P.output_dtype) : "", plan.group, plan.it,
+             plan.ragged ? "_ragged" : "");
     S.label = label + tail;
     // the kernel's symbol: the readable label (what a profiler lists) plus a hash of everything that shapes the code
     S.symbol = "axp_" + S.label + "_" + hash;

@@ -57,6 +57,7 @@ struct RowsProgSpec {
 // too short, a vector operand whose element size keeps a ragged row from its 16-byte chunks): the interpreter takes it.
 // tight = false: among the plan shapes the build compiles (64 or 256 threads per row, a few chunk counts per thread);
 // tight = true: the plan with the fewest idle chunk slots for this row length (64, 256 or 512 threads per row, any chunk count up to 8).
+int rows_prog_chunk_elems(const AxhipRowsProgram &P); // elements per chunk: 4 when a full-size stream is fp32, else 8
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan);
 // The plan with its shape given (the build's generator enumerates the shapes itself).
 void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan);

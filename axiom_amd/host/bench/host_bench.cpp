@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "axhip.h"
 #include "axiom/axiom.hpp"
 
 using namespace axiom;
@@ -57,6 +58,19 @@ int main(int argc, char **argv) {
     }
     Tensor::manual_seed(42);
     std::printf("{\n");
+    { // the floor under every figure below: one launch of a kernel that writes four bytes, then the wait for it
+        auto one = Tensor::zeros({1}, DType::Float32).gpu();
+        void *dst = one.storage()->raw();
+        std::vector<double> us;
+        for (int i = 0; i < warmup + iters; ++i) {
+            const auto t0 = Clock::now();
+            axhip_fill(dst, AXHIP_DTYPE_F32, 1.0, 1, nullptr);
+            backends::hip::synchronize();
+            if (i >= warmup) us.push_back(std::chrono::duration<double, std::micro>(Clock::now() - t0).count());
+        }
+        std::sort(us.begin(), us.end());
+        std::printf("  \"launch_and_wait_floor\": {\"median_us\": %.1f, \"min_us\": %.1f},\n", us[us.size() / 2], us.front());
+    }
     { // configs[0]: the reference's CPU-runnable case, fp32, on the fp32 matrix instruction here
         auto q = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU), k = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU),
              v = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU);

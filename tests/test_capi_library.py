@@ -52,6 +52,9 @@ def test_version_and_kernel_selection_without_device():
     r.row_op = capi.ROWOP["softmax"]
     assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"rows_resident_g256_it8_e4"
     r.cols, r.input_dtype = 4096, capi.DTYPE_BF16
+    # a 16-bit input with an fp32 output moves in chunks of 4 elements (16 bytes of the wider stream) ...
+    assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"rows_resident_g256_it4_e4"
+    r.output_dtype = capi.DTYPE_BF16  # ... and of 8 when every full-size stream is 16-bit
     assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"rows_resident_g256_it2_e8"
     r.cols = 1 << 20
     assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"rows_streamed_e8"
