@@ -323,7 +323,13 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
         int64_t best = 0;
         for (int i = 0; i < 3; ++i) {
             const int64_t n = (chunks + groups[i] - 1) / groups[i];
-            if (n > 8) continue;
+            // up to 8 chunks per thread; a wavefront row may take 9 or 10 (a row just past 512 chunks would otherwise
+            // leave a third of a 256-thread block idle) while its registers still allow 4 waves per SIMD
+            if (n > 8) {
+                const bool resident_f32 = P.row_op != AXHIP_ROWOP_NONE && (dt == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX);
+                const int64_t held = (raw_words_per_chunk(P) + (resident_f32 ? rows_prog_chunk_elems(P) : 0)) * n;
+                if (!(groups[i] == 64 && n <= 10 && held <= 112)) continue;
+            }
             if (group == 0 || n * groups[i] < best) {
                 group = groups[i];
                 it = static_cast<int>(n);

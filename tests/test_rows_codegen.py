@@ -1,0 +1,129 @@
+"""The row-program generator without a device: which kernel a program maps to (built in, compiled at run time, or the
+interpreter's), the plan it gets, and that the text the generator writes for shapes outside the built-in set compiles
+(hipRTC compiles for gfx950 without a GPU).  The addresses are made up: nothing here launches."""
+import ctypes as C
+import os
+
+import pytest
+
+from axiom_amd import capi
+
+F32, F16, BF16 = capi.DTYPE_F32, capi.DTYPE_F16, capi.DTYPE_BF16
+
+
+class Prog:
+    """A row program over made-up, 256-byte aligned addresses."""
+
+    def __init__(self, rows, cols, dt, out_dt=None, misalign=0):
+        self.p = capi.RowsProgram()
+        self.p.rows, self.p.cols = rows, cols
+        self.p.input, self.p.input_dtype = 0x7F0000000000 + misalign, dt
+        self.p.output, self.p.output_dtype = 0x7F1000000000 + misalign, dt if out_dt is None else out_dt
+        self.p.norm_weight = self.p.norm_bias = -1
+        self.dt, self.post_stage = dt, False
+
+    def _operand(self, kind, dt=None):
+        i = self.p.n_operands
+        self.p.operands[i].ptr, self.p.operands[i].dtype, self.p.operands[i].kind = 0x7F2000000000 + (i << 32), self.dt if dt is None else dt, capi.BK[kind]
+        self.p.n_operands = i + 1
+        return i
+
+    def op(self, name, kind=None, imm=None, dt=None):
+        chain, n = (self.p.post, self.p.n_post) if self.post_stage else (self.p.pre, self.p.n_pre)
+        chain[n].op = capi.OP[name]
+        chain[n].operand = -1 if kind is None else self._operand(kind, dt)
+        if imm is not None:
+            chain[n].imm, chain[n].imm_kind = imm, capi.BK["imm"]
+        if self.post_stage:
+            self.p.n_post = n + 1
+        else:
+            self.p.n_pre = n + 1
+        return self
+
+    def row(self, name, affine=0):
+        self.p.row_op, self.p.eps, self.post_stage = capi.ROWOP[name], 1e-5, True
+        if affine >= 1:
+            self.p.norm_weight = self._operand("rowvec")
+        if affine >= 2:
+            self.p.norm_bias = self._operand("rowvec")
+        return self
+
+    def reduce(self, name):
+        self.p.reduce = capi.RED[name]
+        return self
+
+    def name(self):
+        return capi.lib().axhip_fused_rows_kernel_name(C.byref(self.p)).decode()
+
+    def prepare(self):
+        lib = capi.lib()
+        rc = lib.axhip_fused_rows_prepare(C.byref(self.p))
+        return rc, (lib.axhip_last_error() or b"").decode()
+
+
+def test_known_patterns_map_to_built_in_kernels():
+    assert Prog(16384, 4096, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it8"
+    assert Prog(16384, 4096, BF16).row("layernorm", 2).op("gelu").name() == "rows_static_layernorm_gelu_wb_bf16_g64_it8"
+    assert Prog(16384, 4096, BF16).row("rmsnorm", 1).op("gelu").name() == "rows_static_rmsnorm_gelu_w_bf16_g64_it8"
+    assert Prog(8192, 8192, F32).op("relu").op("add", imm=1.0).op("mul", "full").row("softmax").reduce("sum").name() == \
+        "rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"
+    assert Prog(30000, 1500, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it3_ragged"  # 1500 * 2 bytes: rows not 16-byte aligned
+    assert Prog(64, 1024, F16).op("add", "full").row("layernorm", 2).name() == "rows_static_addf_layernorm_wb_f16_g64_it2"
+
+
+def test_other_shapes_are_compiled_at_run_time_and_named_after_their_chain():
+    assert Prog(4096, 4096, BF16).row("layernorm", 2).op("sigmoid").name() == "rows_jit_layernorm_sigmoid_wb_bf16_g64_it8"
+    assert Prog(4096, 4096, BF16).op("mul", imm=0.5).op("tanh").op("add", "full").row("softmax").name() == "rows_jit_muls_tanh_addf_softmax_bf16_g64_it8"
+    # a built-in kernel whose plan has at most 1.15 times the chunk slots of the tightest one serves (8 chunks per lane for 7) ...
+    assert Prog(128, 3584, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it8"
+    # ... beyond that the tight plan is compiled: a wavefront row of 9 or 10 chunks per lane instead of a 256-thread
+    # block with a third of it idle
+    assert Prog(128, 4104, BF16).row("layernorm", 2).name() == "rows_jit_layernorm_wb_bf16_g64_it9"
+    assert Prog(128, 5000, BF16).row("rmsnorm", 1).name() == "rows_jit_rmsnorm_w_bf16_g64_it10"
+    # softmax holds the row as fp32 as well: 9 chunks per lane would not leave registers for 3 waves per SIMD
+    assert Prog(128, 5000, BF16).row("softmax").name() in ("rows_static_softmax_bf16_g256_it3", "rows_jit_softmax_bf16_g256_it3")
+
+
+def test_chunks_are_16_bytes_of_the_widest_full_size_stream():
+    # 16-bit in, 16-bit out: 8 elements per chunk -> 4096 columns are 512 chunks, 8 per lane of a wavefront
+    assert Prog(1024, 4096, BF16).row("rmsnorm", 1).name().endswith("_bf16_g64_it8")
+    # fp32 output: 4 elements per chunk -> 1024 chunks, 4 per thread of a 256-thread block; the label names the result type
+    assert Prog(1024, 4096, BF16, out_dt=F32).row("rmsnorm", 1).name() == "rows_jit_rmsnorm_w_bf16_to_f32_g256_it4"
+    # an fp32 full-size operand: the same
+    assert Prog(1024, 4096, BF16).op("add", "full", dt=F32).row("softmax").name().endswith("_g256_it4")
+    # an fp32 per-column operand does not change the chunk: it is read from cache, not streamed
+    assert Prog(1024, 4096, BF16).op("mul", "rowvec", dt=F32).row("softmax").name().endswith("_g64_it8")
+    # a reduced output ([rows] values) has no chunks
+    assert Prog(1024, 4096, BF16, out_dt=F32).op("square").reduce("mean").name().endswith("_bf16_g64_it8")
+
+
+def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
+    assert Prog(1024, 4096, F32).op("relu").op("mul", "full").name() == "elementwise_e4"  # no row op, no reduction
+    assert Prog(4, 1 << 20, BF16).row("softmax").name() == "rows_streamed_e8"  # beyond 5120 chunks
+    # ragged rows whose streams differ in element size
+    assert Prog(64, 1001, BF16, out_dt=F32).row("softmax").name().startswith("rows_resident_")
+
+
+@pytest.mark.parametrize("build", [
+    lambda: Prog(4096, 4096, BF16).row("layernorm", 2).op("sigmoid"),
+    lambda: Prog(4096, 4096, BF16, out_dt=F32).row("rmsnorm", 1).op("mul", "full"),
+    lambda: Prog(4096, 4099, F16).op("abs").op("mul", "full").row("softmax"),
+    lambda: Prog(4096, 12000, F32).op("mul", "colvec").op("add", "scalar").row("logsoftmax").op("exp"),
+    lambda: Prog(4096, 5000, BF16).op("relu").op("max", imm=0.25).reduce("max"),
+], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10"])
+def test_generated_kernels_compile(build):
+    prog = build()
+    assert prog.name().startswith("rows_jit_"), prog.name()
+    rc, err = prog.prepare()
+    assert rc == 0, err
+
+
+def test_run_time_compilation_can_be_switched_off():
+    prog = Prog(128, 4104, BF16).row("layernorm", 2)
+    assert prog.name() == "rows_jit_layernorm_wb_bf16_g64_it9"
+    os.environ["AXHIP_JIT"] = "0"  # read at every dispatch
+    try:
+        assert prog.name() == "rows_static_layernorm_wb_bf16_g256_it3"  # the built-in kernel of the next looser plan
+        assert Prog(128, 4096, BF16).row("layernorm", 2).op("sigmoid").name().startswith("rows_resident_")  # no built-in kernel: the interpreter
+    finally:
+        del os.environ["AXHIP_JIT"]
