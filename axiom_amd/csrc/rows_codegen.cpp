@@ -247,9 +247,10 @@ int raw_words_per_chunk(const AxhipRowsProgram &P) {
         if (used[i] && P.operands[i].kind == AXHIP_BK_FULL) words += e * elem_size(P.operands[i].dtype) / 4;
     return words;
 }
-// the same for the norm weight and bias of a row that spans several waves (a wavefront row reads them from LDS)
+// the same for the norm weight and bias of a row that spans several waves (a wavefront row reads them from LDS, a
+// 1024-thread block requests them one chunk at a time)
 int affine_words_per_chunk(const AxhipRowsProgram &P, int group) {
-    if (group == 64) return 0;
+    if (group == 64 || group == 1024) return 0;
     const int e = rows_prog_chunk_elems(P);
     int words = 0;
     for (int idx : {P.norm_weight, P.norm_bias})
@@ -272,6 +273,8 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
     const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? rows_prog_chunk_elems(P) * it : 0);
     plan->min_waves = held + (ragged ? 3 * it + 16 : 0) > 72 ? 2 : 4;
+    // a 1024-thread block has 128 registers per thread whatever is asked for: no second set of raw words beyond that
+    if (group == 1024 && held + (plan->pipe ? raw * it : 0) > 115) plan->pipe = false;
 }
 
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
@@ -317,11 +320,11 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
             return false;
         }
     } else {
-        // the tightest fit among 64, 256 and 512 threads per row with up to 8 chunks each: fewest chunk slots (idle lanes
+        // the tightest fit among 64, 256, 512 and 1024 threads per row with up to 8 chunks each: fewest chunk slots (idle lanes
         // still issue their loads and arithmetic), then the smaller group
-        static const int groups[3] = {64, 256, 512};
+        static const int groups[4] = {64, 256, 512, 1024};
         int64_t best = 0;
-        for (int i = 0; i < 3; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const int64_t n = (chunks + groups[i] - 1) / groups[i];
             // up to 8 chunks per thread; a wavefront row may take 9 or 10 (a row just past 512 chunks would otherwise
             // leave a third of a 256-thread block idle) while its registers still allow 4 waves per SIMD
@@ -336,7 +339,23 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
                 best = n * groups[i];
             }
         }
-        if (group == 0) return false;
+        bool rerun = false;
+        if (group == 0) {
+            // Longer rows: up to 16 chunks per thread of a 1024-thread block, held as the raw words they were loaded as
+            // (at most 64 registers) instead of as fp32 -- still one read of the row, at the price of unpacking it and
+            // running the pre chain once per pass.
+            const int64_t n = (chunks + 1023) / 1024;
+            if (n > 16 || raw_words_per_chunk(P) * n > 72) return false;
+            group = 1024;
+            it = static_cast<int>(n);
+            rerun = true;
+        }
+        rows_prog_plan_for(P, group, it, ragged, plan);
+        if (rerun) {
+            plan->rerun = true;
+            plan->pipe = false;
+        }
+        return true;
     }
     rows_prog_plan_for(P, group, it, ragged, plan);
     return true;
@@ -374,7 +393,9 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     std::ostringstream c;
     c << "constexpr int DT_IN = " << dt << ", DT_OUT = " << (P.reduce == AXHIP_RED_NONE ? P.output_dtype : dt) << ";\n";
     c << "constexpr int GROUP = " << plan.group << ", IT = " << plan.it << ", E = " << rows_prog_chunk_elems(P) << ";\n";
-    c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ";\n";
+    const bool rerun = plan.rerun && resident; // (a 16-bit norm without a pre chain never holds its row as fp32 anyway)
+    if (rerun) pipe = false;
+    c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ", RERUN = " << (rerun ? "true" : "false") << ";\n";
     c << "constexpr int MIN_WAVES = " << plan.min_waves << ";\n";
     c << "constexpr int ROWOP = " << P.row_op << ", RED = " << red << ";\n";
     c << "constexpr int W_DT = " << w_dt << ", B_DT = " << b_dt << ", W_SLOT = " << w_slot << ", B_SLOT = " << b_slot << ";\n";

@@ -35,6 +35,7 @@ struct RowsProgPlan {
     int group = 0, it = 0; // threads per row, 16-byte input chunks per thread
     bool ragged = false;   // rows are not whole aligned vectors
     bool pipe = false;     // the next row is requested before the current one is computed
+    bool rerun = false;    // the row stays in registers as raw words; every pass unpacks it and applies the pre chain again
     int min_waves = 4;     // waves per SIMD the kernel's register allocation aims for
     int slots() const { return group * it; }
 };

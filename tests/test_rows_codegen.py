@@ -97,9 +97,22 @@ def test_chunks_are_16_bytes_of_the_widest_full_size_stream():
     assert Prog(1024, 4096, BF16, out_dt=F32).op("square").reduce("mean").name().endswith("_bf16_g64_it8")
 
 
+def test_long_rows_get_a_1024_thread_block_and_beyond_8_chunks_per_thread_stay_as_raw_words():
+    # up to 8192 chunks: held as fp32 like the shorter rows
+    assert Prog(64, 50304, BF16).row("softmax").name() == "rows_jit_softmax_bf16_g1024_it7"
+    assert Prog(64, 32768, F32).row("logsoftmax").name() == "rows_jit_logsoftmax_f32_g1024_it8"
+    # 8193 to 16384 chunks: the raw words stay, every pass unpacks them again (a vocabulary of 128 256 16-bit logits)
+    assert Prog(64, 128256, BF16).row("softmax").name() == "rows_jit_softmax_bf16_g1024_it16"
+    assert Prog(64, 50304, F32).row("layernorm", 2).name() == "rows_jit_layernorm_wb_f32_g1024_it13"
+    assert Prog(64, 50257, F32).op("mul", imm=0.5).row("softmax").name() == "rows_jit_muls_softmax_f32_g1024_it13_ragged"
+    # two 16-bit streams fit up to 9 chunks each per thread, not 16
+    assert Prog(64, 70000, BF16).op("add", "full").row("softmax").name() == "rows_jit_addf_softmax_bf16_g1024_it9"
+    assert Prog(64, 128256, BF16).op("add", "full").row("softmax").name() == "rows_streamed_e8"
+
+
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     assert Prog(1024, 4096, F32).op("relu").op("mul", "full").name() == "elementwise_e4"  # no row op, no reduction
-    assert Prog(4, 1 << 20, BF16).row("softmax").name() == "rows_streamed_e8"  # beyond 5120 chunks
+    assert Prog(4, 1 << 20, BF16).row("softmax").name() == "rows_streamed_e8"  # beyond 16384 chunks
     # ragged rows whose streams differ in element size
     assert Prog(64, 1001, BF16, out_dt=F32).row("softmax").name().startswith("rows_resident_")
 
@@ -110,7 +123,8 @@ def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     lambda: Prog(4096, 4099, F16).op("abs").op("mul", "full").row("softmax"),
     lambda: Prog(4096, 12000, F32).op("mul", "colvec").op("add", "scalar").row("logsoftmax").op("exp"),
     lambda: Prog(4096, 5000, BF16).op("relu").op("max", imm=0.25).reduce("max"),
-], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10"])
+    lambda: Prog(64, 128256, F16).op("mul", imm=0.5).row("logsoftmax"),
+], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10", "raw_resident_it16"])
 def test_generated_kernels_compile(build):
     prog = build()
     assert prog.name().startswith("rows_jit_"), prog.name()

@@ -299,11 +299,71 @@ def test_fast_activations_after_a_norm_in_16_bit(post):
     assert np.max(np.abs(got - want)) < 2e-2
 
 
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_vocabulary_sized_rows_stay_in_registers_as_raw_words(dt):
+    """Rows of 8193 to 16384 chunks (a language model's vocabulary: 50 304 fp32 or 128 256 16-bit logits) are read once:
+    the 1024 threads of a block keep the raw words and every pass -- maximum, sum of exponentials, output -- unpacks
+    them and applies the pre chain again.  Aligned and odd lengths, softmax / log-softmax behind a pre chain, both
+    norms, a row reduction."""
+    g = axo.PCG64(2024)
+    tol = 1e-4 if dt == F32 else 2e-2
+    to_dev = (lambda a: a.astype(np.float32)) if dt == F32 else (lambda a: axo.to_bits(a, dt))
+    to_f64 = (lambda a: a.astype(np.float64)) if dt == F32 else (lambda a: axo.to_f32(a, dt).astype(np.float64))
+    tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
+    for cols in ((50304, 50257) if dt == F32 else (128256, 100001)):
+        ragged = "_ragged" if cols % 2 else ""
+        it = (cols + (4 if dt == F32 else 8) * 1024 - 1) // ((4 if dt == F32 else 8) * 1024)
+        x = to_dev(g.normal((3, cols)) * 3)
+        xf = to_f64(x)
+        # softmax(x * 0.5): scaled logits
+        p = gh.Rows(x, dt).imm("mul", 0.5).row_op("softmax")
+        got = to_f64(p.run())
+        assert p.kernel_name() == f"rows_jit_muls_softmax_{tag}_g1024_it{it}{ragged}", p.kernel_name()
+        e = np.exp(xf * 0.5 - (xf * 0.5).max(-1, keepdims=True))
+        assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
+        assert np.max(np.abs(got.sum(-1) - 1.0)) < (1e-4 if dt == F32 else 2e-2)
+        # log-softmax
+        p = gh.Rows(x, dt).row_op("logsoftmax")
+        got = to_f64(p.run())
+        assert p.kernel_name() == f"rows_jit_logsoftmax_{tag}_g1024_it{it}{ragged}", p.kernel_name()
+        want = xf - xf.max(-1, keepdims=True) - np.log(np.exp(xf - xf.max(-1, keepdims=True)).sum(-1, keepdims=True))
+        assert np.max(np.abs(got - want)) < (1e-4 if dt == F32 else 2e-2 * 8)  # |log-softmax| reaches 20 here: 16-bit steps of 2^-3
+        # layer norm with weight and bias (off-centre rows: mean 3), RMS norm
+        w, b = to_dev(g.uniform((cols,), 0.5, 1.5)), to_dev(g.uniform((cols,), -0.5, 0.5))
+        x3 = to_dev(g.normal((2, cols)) + 3.0)
+        x3f = to_f64(x3)
+        p = gh.Rows(x3, dt).row_op("layernorm", 1e-5, w=w, b=b)
+        got = to_f64(p.run())
+        assert p.kernel_name() == f"rows_jit_layernorm_wb_{tag}_g1024_it{it}{ragged}", p.kernel_name()
+        want = (x3f - x3f.mean(-1, keepdims=True)) / np.sqrt(x3f.var(-1, keepdims=True) + 1e-5) * to_f64(w) + to_f64(b)
+        assert np.max(np.abs(got - want)) < tol * (1 if dt == F32 else 2)
+        p = gh.Rows(x3, dt).row_op("rmsnorm", 1e-5, w=w)
+        got = to_f64(p.run())
+        want = x3f / np.sqrt((x3f * x3f).mean(-1, keepdims=True) + 1e-5) * to_f64(w)
+        assert np.max(np.abs(got - want)) < tol * (1 if dt == F32 else 2)
+        # max |x| per row
+        p = gh.Rows(x, dt, F32).unary("abs")
+        got = p.run(reduce="max")
+        assert p.kernel_name() == f"rows_jit_abs_reduce_max_{tag}_g1024_it{it}{ragged}", p.kernel_name()
+        assert np.allclose(got.reshape(-1), np.abs(xf).max(-1), rtol=1e-6)
+    # two streams: softmax(x + y) over 70 000 16-bit columns is 9 chunks of each per thread
+    if dt != F32:
+        x, y = to_dev(g.normal((2, 70000)) * 2), to_dev(g.normal((2, 70000)))
+        p = gh.Rows(x, dt).binary("add", y).row_op("softmax")
+        got = to_f64(p.run())
+        assert p.kernel_name() == f"rows_jit_addf_softmax_{tag}_g1024_it9", p.kernel_name()
+        lg = to_f64(x) + to_f64(y)
+        e = np.exp(lg - lg.max(-1, keepdims=True))
+        assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
+
+
 def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
-    """Rows beyond the 32 KiB the built-in kernels hold: up to 4096 16-byte chunks stay in the registers of a
-    512-thread block (one read; kernels compiled at first launch), longer ones are streamed in passes."""
+    """Rows beyond the 32 KiB the built-in kernels hold: up to 8192 16-byte chunks stay in the registers of a
+    512- or 1024-thread block as fp32, up to 16384 as the raw words they were loaded as (one read either way; kernels
+    compiled at first launch); longer ones are streamed in passes by the interpreter."""
     g = axo.PCG64(123)
-    for cols, plan in ((12000, "rows_jit_softmax_f32_g512_it6"), (16384, "rows_jit_softmax_f32_g512_it8"), (20000, "rows_streamed_e4")):
+    for cols, plan in ((12000, "rows_jit_softmax_f32_g512_it6"), (16384, "rows_jit_softmax_f32_g512_it8"), (20000, "rows_jit_softmax_f32_g1024_it5"),
+                       (40000, "rows_jit_softmax_f32_g1024_it10"), (70000, "rows_streamed_e4")):
         x = (g.normal((3, cols)) * 2).astype(np.float32)
         p = gh.Rows(x, F32).row_op("softmax")
         got = p.run()
