@@ -259,20 +259,38 @@ int affine_words_per_chunk(const AxhipRowsProgram &P, int group) {
 }
 } // namespace
 
-void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan) {
+bool rows_prog_grid_pays(const AxhipRowsProgram &P, int64_t chunk_slots) {
+    // Measured on rows of 1001 to 4100 columns: chunks on memory's grid gain 2 to 25 % where every stream is full-size;
+    // a per-column operand ([cols] weights: their position in the row no longer matches their address) costs more than
+    // that in unaligned gathers, and at two chunks per lane the extra chunk does.
+    if (chunk_slots <= 128) return false;
+    auto rowvec = [&](int idx) { return idx >= 0 && idx < P.n_operands && P.operands[idx].kind == AXHIP_BK_ROWVEC; };
+    if (rowvec(P.norm_weight) || rowvec(P.norm_bias)) return false;
+    for (int stage = 0; stage < 2; ++stage) {
+        const AxhipChainOp *ops = stage ? P.post : P.pre;
+        const int n = stage ? P.n_post : P.n_pre;
+        for (int i = 0; i < n; ++i)
+            if (is_binary(ops[i].op) && ops[i].imm_kind != AXHIP_BK_IMM && rowvec(ops[i].operand)) return false;
+    }
+    return true;
+}
+
+void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan, bool grid) {
     plan->group = group;
     plan->it = it;
     plan->ragged = ragged;
+    plan->grid = ragged && grid;
+    const bool heavy = ragged && !grid; // unaligned chunks carry an address and an element count each in registers
     // Pipelining keeps a second set of raw words alive: worth it while that set is at most 32 registers (a 16-bit
     // row of 4096 columns per wavefront, or a row with one operand at half that).  Ragged rows carry their chunk
     // bookkeeping in registers too and pipeline at half that.
     const int raw = raw_words_per_chunk(P), all = raw + affine_words_per_chunk(P, group);
-    plan->pipe = all * it <= (ragged ? 16 : 32);
+    plan->pipe = all * it <= (heavy ? 16 : ragged ? 24 : 32); // (rows on the moving grid keep their end-of-row masks too)
     // Register allocation aims at 4 waves per SIMD (128 registers per thread).  The widest plans hold more than
     // that with their operands: they get the registers of 2 waves per SIMD instead of spilling.
     const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
     const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? rows_prog_chunk_elems(P) * it : 0);
-    plan->min_waves = held + (ragged ? 3 * it + 16 : 0) > 72 ? 2 : 4;
+    plan->min_waves = (held + (heavy ? 3 * it + 16 : 0) > 72 || it > 8) ? 2 : 4;
     // a 1024-thread block has 128 registers per thread whatever is asked for: no second set of raw words beyond that
     if (group == 1024 && held + (plan->pipe ? raw * it : 0) > 115) plan->pipe = false;
 }
@@ -304,7 +322,17 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     }
     // a ragged row is addressed in 16-byte chunks of every vector it touches: all of them must share the element size
     if (ragged && !same_size) return false;
-    const int64_t chunks = (P.cols + e - 1) / e;
+    // When the input, the full-size operands and a full-size output sit at the same address modulo 16 (the usual case:
+    // aligned allocations, a row length that is not a multiple of the chunk), the chunks follow memory's 16-byte grid:
+    // every access aligned, a partial chunk at either end of a row, hence one chunk more than the row's own count.
+    bool grid = ragged && rows_prog_grid_pays(P, P.cols / e);
+    if (grid) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(P.input) & 15u;
+        if (P.reduce == AXHIP_RED_NONE && (reinterpret_cast<uintptr_t>(P.output) & 15u) != a) grid = false;
+        for (int i = 0; i < P.n_operands; ++i)
+            if (used[i] && P.operands[i].kind == AXHIP_BK_FULL && (reinterpret_cast<uintptr_t>(P.operands[i].ptr) & 15u) != a) grid = false;
+    }
+    const int64_t chunks = grid ? (P.cols + 2 * e - 2) / e : (P.cols + e - 1) / e;
     int group = 0, it = 0;
     if (!tight) {
         // the shapes the build compiles (rows_aot_gen.cpp): a wavefront per row with 1, 2, 3, 4, 5, 6 or 8 chunks per
@@ -350,14 +378,17 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
             it = static_cast<int>(n);
             rerun = true;
         }
-        rows_prog_plan_for(P, group, it, ragged, plan);
+        rows_prog_plan_for(P, group, it, ragged, plan, grid);
+        // chunk c of a row on the grid lies inside the row for every shift when (c + 1) * e <= cols (and c > 0): true of
+        // all chunks of a thread's first cols / e / group -- the last one or two per thread in a tight plan are in doubt
+        if (plan->grid) plan->tail_from = static_cast<int>(std::min<int64_t>(std::max(it - 2, 0), P.cols / e / group));
         if (rerun) {
             plan->rerun = true;
             plan->pipe = false;
         }
         return true;
     }
-    rows_prog_plan_for(P, group, it, ragged, plan);
+    rows_prog_plan_for(P, group, it, ragged, plan, grid);
     return true;
 }
 
@@ -395,7 +426,9 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     c << "constexpr int GROUP = " << plan.group << ", IT = " << plan.it << ", E = " << rows_prog_chunk_elems(P) << ";\n";
     const bool rerun = plan.rerun && resident; // (a 16-bit norm without a pre chain never holds its row as fp32 anyway)
     if (rerun) pipe = false;
-    c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ", RERUN = " << (rerun ? "true" : "false") << ";\n";
+    c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ", RERUN = " << (rerun ? "true" : "false")
+      << ", GRID = " << (plan.ragged && plan.grid ? "true" : "false") << ";\n";
+    c << "constexpr int TAIL_FROM = " << (plan.ragged && plan.grid ? plan.tail_from : 0) << ";\n";
     c << "constexpr int MIN_WAVES = " << plan.min_waves << ";\n";
     c << "constexpr int ROWOP = " << P.row_op << ", RED = " << red << ";\n";
     c << "constexpr int W_DT = " << w_dt << ", B_DT = " << b_dt << ", W_SLOT = " << w_slot << ", B_SLOT = " << b_slot << ";\n";

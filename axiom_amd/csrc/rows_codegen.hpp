@@ -34,6 +34,8 @@ struct RowsProgArgs {
 struct RowsProgPlan {
     int group = 0, it = 0; // threads per row, 16-byte input chunks per thread
     bool ragged = false;   // rows are not whole aligned vectors
+    bool grid = false;     // ragged rows whose full-size streams share their address modulo 16: chunks on memory's 16-byte grid
+    int tail_from = 0;     // grid rows: a thread's chunks before this one are known to lie inside the row (0: nothing known)
     bool pipe = false;     // the next row is requested before the current one is computed
     bool rerun = false;    // the row stays in registers as raw words; every pass unpacks it and applies the pre chain again
     int min_waves = 4;     // waves per SIMD the kernel's register allocation aims for
@@ -61,7 +63,9 @@ struct RowsProgSpec {
 int rows_prog_chunk_elems(const AxhipRowsProgram &P); // elements per chunk: 4 when a full-size stream is fp32, else 8
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan);
 // The plan with its shape given (the build's generator enumerates the shapes itself).
-void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan);
+// whether ragged rows of this program are better served with chunks on memory's 16-byte grid (given equally aligned streams)
+bool rows_prog_grid_pays(const AxhipRowsProgram &P, int64_t chunk_slots);
+void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan, bool grid = false);
 
 // Builds the kernel's configuration for a program under a plan; false when the program names an operand kind or
 // op code the generator does not know.

@@ -25,7 +25,8 @@ struct StructKey {
 void make_struct_key(const AxhipRowsProgram &P, StructKey *k) {
     memset(k, 0, sizeof(*k));
     AxhipRowsProgram &q = k->p;
-    auto align_tag = [](const void *p) { return reinterpret_cast<const void *>(static_cast<uintptr_t>((reinterpret_cast<uintptr_t>(p) & 15u) == 0)); };
+    // (the address modulo 16 decides between the aligned, the grid and the unaligned form of a kernel)
+    auto align_tag = [](const void *p) { return reinterpret_cast<const void *>(static_cast<uintptr_t>(reinterpret_cast<uintptr_t>(p) & 15u) + 16u); };
     q.cols = P.cols;
     q.input = align_tag(P.input);
     q.input_dtype = P.input_dtype;

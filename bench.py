@@ -368,7 +368,17 @@ def bench_survey(torch, capi, stream, steps, warmup):
     wr, br = rnd((4099,), bf, 0.3, 1.0), rnd((4099,), bf, 0.1)
     run("layernorm(x+y)_bf16_16384x4099", P(t).op("add", u).row("layernorm", wr, br).finish(torch))
     run("mean(x^2)_bf16_16384x4099", P(t, f32).op("square").finish(torch, "mean"))
+    del t, u
+    # vocabulary-sized rows (language-model logits): 1024-thread blocks; beyond 8 chunks per thread the row stays in
+    # registers as raw words
+    for rows, cols, dt, name in ((4096, 50304, bf, "bf16"), (2048, 128256, bf, "bf16"), (2048, 50304, f32, "f32"), (4096, 50257, bf, "bf16")):
+        t = rnd((rows, cols), dt, 3.0)
+        run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
+        run(f"logsoftmax(x*s)_{name}_{rows}x{cols}", P(t).op("mul", imm=0.5).row("logsoftmax").finish(torch))
+        run(f"max(x)_{name}_{rows}x{cols}", P(t).finish(torch, "max"))
+        del t
     return res
+
 
 def bench_gemm(torch, capi, stream, steps, warmup):
     """x W^T through axhip_gemm (the nn::Linear product): a large square, the tall product of a
