@@ -458,7 +458,7 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     char tail[64];
     const bool other_out = P.reduce == AXHIP_RED_NONE && P.output_dtype != dt;
     snprintf(tail, sizeof(tail), "%s%s%s_g%d_it%d%s", dt_name(dt), other_out ? "_to_" : "", other_out ? dt_name(P.output_dtype) : "", plan.group, plan.it,
-             plan.ragged ? "_ragged" : "");
+             !plan.ragged ? "" : plan.grid ? "_grid" : "_ragged"); // (grid: ragged rows addressed on memory's 16-byte grid)
     S.label = label + tail;
     // the kernel's symbol: the readable label (what a profiler lists) plus a hash of everything that shapes the code
     S.symbol = "axp_" + S.label + "_" + hash;

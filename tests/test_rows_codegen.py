@@ -67,7 +67,7 @@ def test_known_patterns_map_to_built_in_kernels():
     assert Prog(16384, 4096, BF16).row("rmsnorm", 1).op("gelu").name() == "rows_static_rmsnorm_gelu_w_bf16_g64_it8"
     assert Prog(8192, 8192, F32).op("relu").op("add", imm=1.0).op("mul", "full").row("softmax").reduce("sum").name() == \
         "rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"
-    assert Prog(30000, 1500, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it3_ragged"  # 1500 * 2 bytes: rows not 16-byte aligned
+    assert Prog(30000, 1500, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it3_grid"  # 1500 * 2 bytes: rows not 16-byte aligned
     assert Prog(64, 1024, F16).op("add", "full").row("layernorm", 2).name() == "rows_static_addf_layernorm_wb_f16_g64_it2"
 
 
@@ -104,10 +104,36 @@ def test_long_rows_get_a_1024_thread_block_and_beyond_8_chunks_per_thread_stay_a
     # 8193 to 16384 chunks: the raw words stay, every pass unpacks them again (a vocabulary of 128 256 16-bit logits)
     assert Prog(64, 128256, BF16).row("softmax").name() == "rows_jit_softmax_bf16_g1024_it16"
     assert Prog(64, 50304, F32).row("layernorm", 2).name() == "rows_jit_layernorm_wb_f32_g1024_it13"
-    assert Prog(64, 50257, F32).op("mul", imm=0.5).row("softmax").name() == "rows_jit_muls_softmax_f32_g1024_it13_ragged"
+    assert Prog(64, 50257, F32).op("mul", imm=0.5).row("softmax").name() == "rows_jit_muls_softmax_f32_g1024_it13_grid"
     # two 16-bit streams fit up to 9 chunks each per thread, not 16
     assert Prog(64, 70000, BF16).op("add", "full").row("softmax").name() == "rows_jit_addf_softmax_bf16_g1024_it9"
     assert Prog(64, 128256, BF16).op("add", "full").row("softmax").name() == "rows_streamed_e8"
+
+
+def test_ragged_rows_take_the_grid_form_when_every_stream_is_full_size_and_equally_aligned():
+    """Rows whose length the 16-byte chunk does not divide.  Chunks on memory's 16-byte grid ("_grid": aligned accesses,
+    a masked partial chunk at either end of the row) need the input, the full-size operands and the output at one
+    address modulo 16, no per-column operand, and more than two chunks per lane; everything else is addressed from
+    the row's start ("_ragged": every access unaligned)."""
+    assert Prog(4096, 4099, BF16).row("softmax").name() == "rows_jit_softmax_bf16_g64_it9_grid"
+    assert Prog(4096, 4099, BF16, misalign=6).row("softmax").name() == "rows_jit_softmax_bf16_g64_it9_grid"  # input and output shifted alike
+    assert Prog(4096, 1500, F16).op("add", "full").row("softmax").name() == "rows_static_addf_softmax_f16_g64_it3_grid"
+    assert Prog(4096, 4099, BF16, out_dt=F32).op("square").reduce("sum").name() == "rows_jit_square_reduce_sum_bf16_g64_it9_grid"  # [rows] results: any alignment
+    # a per-column operand: its position in the row does not follow the grid
+    assert Prog(4096, 1500, BF16).row("layernorm", 2).name() == "rows_static_layernorm_wb_bf16_g64_it3_ragged"
+    assert Prog(4096, 1500, BF16).op("mul", "rowvec").row("softmax").name().endswith("_it3_ragged")
+    assert Prog(4096, 1500, BF16).row("layernorm").name() == "rows_static_layernorm_bf16_g64_it3_grid"  # no weight, no bias
+    # at most two chunks per lane: the extra chunk of the grid form costs more than its aligned accesses gain
+    assert Prog(4096, 1001, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it2_ragged"
+    # streams at different addresses modulo 16
+    p = Prog(4096, 1500, BF16).op("add", "full").row("softmax")
+    p.p.operands[0].ptr += 2
+    assert p.name().endswith("_it3_ragged")
+    p = Prog(4096, 1500, BF16).row("softmax")
+    p.p.output += 4
+    assert p.name().endswith("_it3_ragged")
+    # rows of 16-byte multiples from a base that is not: one shift for every row, still the grid
+    assert Prog(4096, 4096, BF16, misalign=2).row("softmax").name() == "rows_jit_softmax_bf16_g64_it9_grid"
 
 
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():

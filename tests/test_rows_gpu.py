@@ -311,7 +311,8 @@ def test_vocabulary_sized_rows_stay_in_registers_as_raw_words(dt):
     to_f64 = (lambda a: a.astype(np.float64)) if dt == F32 else (lambda a: axo.to_f32(a, dt).astype(np.float64))
     tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
     for cols in ((50304, 50257) if dt == F32 else (128256, 100001)):
-        ragged = "_ragged" if cols % 2 else ""
+        ragged = "_grid" if cols % 2 else ""  # odd lengths: chunks on memory's 16-byte grid, but for the norms ...
+        ragged_wb = "_ragged" if cols % 2 else ""  # ... whose weights do not follow it
         it = (cols + (4 if dt == F32 else 8) * 1024 - 1) // ((4 if dt == F32 else 8) * 1024)
         x = to_dev(g.normal((3, cols)) * 3)
         xf = to_f64(x)
@@ -334,7 +335,7 @@ def test_vocabulary_sized_rows_stay_in_registers_as_raw_words(dt):
         x3f = to_f64(x3)
         p = gh.Rows(x3, dt).row_op("layernorm", 1e-5, w=w, b=b)
         got = to_f64(p.run())
-        assert p.kernel_name() == f"rows_jit_layernorm_wb_{tag}_g1024_it{it}{ragged}", p.kernel_name()
+        assert p.kernel_name() == f"rows_jit_layernorm_wb_{tag}_g1024_it{it}{ragged_wb}", p.kernel_name()
         want = (x3f - x3f.mean(-1, keepdims=True)) / np.sqrt(x3f.var(-1, keepdims=True) + 1e-5) * to_f64(w) + to_f64(b)
         assert np.max(np.abs(got - want)) < tol * (1 if dt == F32 else 2)
         p = gh.Rows(x3, dt).row_op("rmsnorm", 1e-5, w=w)
@@ -448,7 +449,7 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
         tol = 1e-4 if dt == F32 else 2e-2
         p = gh.Rows(xs, dt).binary("add", ys).row_op("softmax")
         got = out(p.run())
-        assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+        assert p.kernel_name().endswith("_grid" if cols // (4 if dt == F32 else 8) > 128 else "_ragged"), p.kernel_name()  # (the grid form from 3 chunks per lane on)
         lg = f(xs) + f(ys)
         e = np.exp(lg - lg.max(-1, keepdims=True))
         assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
@@ -462,10 +463,10 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
         got = p.run(reduce="sum")
         assert np.allclose(got.reshape(-1), (xf * xf).sum(-1), rtol=1e-4, atol=1e-3)
         if cols >= 8:
-            assert p.kernel_name().startswith(("rows_static_square_reduce_sum", "rows_jit_square_reduce_sum")) and p.kernel_name().endswith("_ragged"), p.kernel_name()
+            assert p.kernel_name().startswith(("rows_static_square_reduce_sum", "rows_jit_square_reduce_sum")) and p.kernel_name().endswith(("_ragged", "_grid")), p.kernel_name()
         p = gh.Rows(xs, dt).row_op("logsoftmax")
         got = out(p.run())
-        assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+        assert p.kernel_name().endswith(("_ragged", "_grid")), p.kernel_name()
         ref = xf - xf.max(-1, keepdims=True)
         ref = ref - np.log(np.exp(ref).sum(-1, keepdims=True))
         assert np.max(np.abs(got - ref)) < (1e-4 if dt == F32 else 8e-2)  # |log p| reaches 16: half an ulp of a 16-bit result
@@ -475,7 +476,7 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
             assert np.array_equal(got.reshape(-1).astype(np.float64), fn(xf, axis=-1)), red  # exact: a selection
         p = gh.Rows(xs, dt).unary("abs").binary("mul", ys).row_op("softmax")
         got = out(p.run())
-        assert p.kernel_name().startswith("rows_jit_abs_mulf_softmax_") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+        assert p.kernel_name().startswith("rows_jit_abs_mulf_softmax_") and p.kernel_name().endswith(("_ragged", "_grid")), p.kernel_name()
         lg = np.abs(f(xs)) * f(ys)
         e = np.exp(lg - lg.max(-1, keepdims=True))
         assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
@@ -512,9 +513,58 @@ def test_bases_that_are_only_element_aligned(dt):
     p = gh.Rows(x, dt).row_op("softmax")
     p.p.input = shifted(p, x, 1)
     got = f(p.run())
-    assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+    assert p.kernel_name().endswith("_ragged"), p.kernel_name()  # the output is aligned, the input is not
     e = np.exp(f(x) - f(x).max(-1, keepdims=True))
     assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < (1e-4 if dt == F32 else 2e-2)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_ragged_rows_on_the_16_byte_grid_at_the_ends_of_a_plan(dt):
+    """Rows addressed on memory's 16-byte grid: the shortest and the longest row each plan takes (the row's last chunk
+    in a thread's second-to-last slot for some shifts and in its last slot for others; every slot of the plan used),
+    from a base 3 elements past a boundary and with odd lengths, so that consecutive rows meet every shift.  A masked
+    store that went wrong would write outside the row: the words around the output keep their pattern, and every
+    row is checked against the oracle.  Wavefront, 256- and 1024-thread plans, built in and compiled here, rows held
+    as fp32 and as raw words."""
+    e, es = (4, 4) if dt == F32 else (8, 2)
+    tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    f = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    g = axo.PCG64(1616)
+    rows, off, pad = 19, 3, 64
+    sentinel = np.float32(-77.0) if dt == F32 else np.uint16(0x7FC1)
+    for group, it in ((64, 4), (64, 9), (256, 5), (1024, 9)):
+        shortest = e * ((it - 1) * group + 1) - (2 * e - 2)
+        longest = e * it * group - e + 1
+        for cols in (shortest, shortest + 1, longest - 1, longest):
+            x = store(g.normal((rows, cols)) * 2)
+            xf = f(x)
+            src = gh.to_dev(np.concatenate([np.full(off, sentinel, x.dtype), x.ravel()]))
+            dst = gh.to_dev(np.full(pad + off + rows * cols + pad, sentinel, x.dtype))
+            p = gh.Rows(x[:1], dt).row_op("softmax")
+            p.keep += [src, dst]
+            p.p.rows, p.p.input = rows, src.data_ptr() + off * es
+            p.p.output, p.p.output_dtype = dst.data_ptr() + (pad + off) * es, dt  # pad * es is a multiple of 16: input and output shifted alike
+            assert p.kernel_name().endswith(f"softmax_{tag}_g{group}_it{it}_grid"), (cols, p.kernel_name())
+            gh.sync()
+            gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
+            gh.sync()
+            out = gh.to_host(dst, x.dtype)
+            assert np.all(out[:pad + off] == sentinel) and np.all(out[pad + off + rows * cols:] == sentinel), cols
+            got = f(out[pad + off:pad + off + rows * cols].reshape(rows, cols))
+            ex = np.exp(xf - xf.max(-1, keepdims=True))
+            assert np.max(np.abs(got - ex / ex.sum(-1, keepdims=True))) < (1e-5 if dt == F32 else 2e-3), cols
+            # a reduction to [rows] values: exact (a selection), whatever the alignment of its output
+            p = gh.Rows(x[:1], dt, F32).unary("abs")
+            p.keep.append(src)
+            p.p.rows, p.p.input = rows, src.data_ptr() + off * es
+            res = gh.empty_dev((rows,), F32)
+            p.keep.append(res)
+            p.p.output, p.p.output_dtype, p.p.reduce = res.data_ptr(), F32, gh.capi.RED["max"]
+            assert p.kernel_name().endswith(f"abs_reduce_max_{tag}_g{group}_it{it}_grid"), (cols, p.kernel_name())
+            gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
+            gh.sync()
+            assert np.array_equal(gh.to_host(res, np.float32).astype(np.float64), np.abs(xf).max(-1)), cols
 
 
 def test_interpreter_serves_programs_without_a_built_in_kernel_when_run_time_compilation_is_off(no_jit):
