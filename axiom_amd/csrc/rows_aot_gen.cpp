@@ -160,7 +160,7 @@ int main(int argc, char **argv) {
             for (const auto &pl : plans)
                 for (bool ragged : {false, true}) {
                     RowsProgPlan plan;
-                    rows_prog_plan_for(p, pl[0], pl[1], ragged, &plan, /*the built-in ragged kernels are those for equally aligned streams*/ ragged && rows_prog_grid_pays(p, pl[0] * pl[1]));
+                    rows_prog_plan_for(p, pl[0], pl[1], ragged, &plan, /*the built-in ragged kernels are those for equally aligned streams*/ ragged && rows_prog_grid_pays(p, pl[0], pl[1]));
                     RowsProgSpec s;
                     if (!rows_prog_spec(p, plan, &s)) {
                         fprintf(stderr, "rows_aot_gen: a listed shape was refused by the generator\n");

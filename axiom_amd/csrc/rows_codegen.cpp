@@ -259,11 +259,14 @@ int affine_words_per_chunk(const AxhipRowsProgram &P, int group) {
 }
 } // namespace
 
-bool rows_prog_grid_pays(const AxhipRowsProgram &P, int64_t chunk_slots) {
-    // Measured on rows of 1001 to 4100 columns: chunks on memory's grid gain 2 to 25 % where every stream is full-size;
-    // a per-column operand ([cols] weights: their position in the row no longer matches their address) costs more than
-    // that in unaligned gathers, and at two chunks per lane the extra chunk does.
-    if (chunk_slots <= 128) return false;
+bool rows_prog_grid_pays(const AxhipRowsProgram &P, int group, int it) {
+    // Measured on rows of 1001 to 100 003 columns: chunks on memory's grid gain 2 to 25 % where every stream is
+    // full-size; at two chunks per lane the extra chunk costs more than that.  A per-column operand ([cols] weights:
+    // their position in the row no longer matches their address) costs 5 to 20 % on the grid in rows of up to 512
+    // threads (wavefront rows stage it in LDS once per block when the chunks start at the row's first element) --
+    // 1024-thread rows gain even so: their unaligned form spills (layer norm over 50 257 fp32 columns: 404 -> 172 us).
+    if (group * it <= 128) return false;
+    if (group > 512) return true;
     auto rowvec = [&](int idx) { return idx >= 0 && idx < P.n_operands && P.operands[idx].kind == AXHIP_BK_ROWVEC; };
     if (rowvec(P.norm_weight) || rowvec(P.norm_bias)) return false;
     for (int stage = 0; stage < 2; ++stage) {
@@ -293,6 +296,10 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     plan->min_waves = (held + (heavy ? 3 * it + 16 : 0) > 72 || it > 8) ? 2 : 4;
     // a 1024-thread block has 128 registers per thread whatever is asked for: no second set of raw words beyond that
     if (group == 1024 && held + (plan->pipe ? raw * it : 0) > 115) plan->pipe = false;
+}
+
+namespace {
+bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, RowsProgPlan *plan);
 }
 
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
@@ -325,13 +332,22 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     // When the input, the full-size operands and a full-size output sit at the same address modulo 16 (the usual case:
     // aligned allocations, a row length that is not a multiple of the chunk), the chunks follow memory's 16-byte grid:
     // every access aligned, a partial chunk at either end of a row, hence one chunk more than the row's own count.
-    bool grid = ragged && rows_prog_grid_pays(P, P.cols / e);
+    bool grid = ragged && P.cols >= 2 * e;
     if (grid) {
         const uintptr_t a = reinterpret_cast<uintptr_t>(P.input) & 15u;
         if (P.reduce == AXHIP_RED_NONE && (reinterpret_cast<uintptr_t>(P.output) & 15u) != a) grid = false;
         for (int i = 0; i < P.n_operands; ++i)
             if (used[i] && P.operands[i].kind == AXHIP_BK_FULL && (reinterpret_cast<uintptr_t>(P.operands[i].ptr) & 15u) != a) grid = false;
     }
+    if (grid && plan_rows(P, tight, ragged, true, plan) && rows_prog_grid_pays(P, plan->group, plan->it)) return true;
+    return plan_rows(P, tight, ragged, false, plan);
+}
+
+namespace {
+bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, RowsProgPlan *plan) {
+    *plan = RowsProgPlan{};
+    const int dt = P.input_dtype;
+    const int e = rows_prog_chunk_elems(P);
     const int64_t chunks = grid ? (P.cols + 2 * e - 2) / e : (P.cols + e - 1) / e;
     int group = 0, it = 0;
     if (!tight) {
@@ -391,6 +407,7 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     rows_prog_plan_for(P, group, it, ragged, plan, grid);
     return true;
 }
+} // namespace
 
 bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsProgSpec *spec) {
     RowsProgSpec &S = *spec;

@@ -64,7 +64,7 @@ int rows_prog_chunk_elems(const AxhipRowsProgram &P); // elements per chunk: 4 w
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan);
 // The plan with its shape given (the build's generator enumerates the shapes itself).
 // whether ragged rows of this program are better served with chunks on memory's 16-byte grid (given equally aligned streams)
-bool rows_prog_grid_pays(const AxhipRowsProgram &P, int64_t chunk_slots);
+bool rows_prog_grid_pays(const AxhipRowsProgram &P, int group, int it);
 void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragged, RowsProgPlan *plan, bool grid = false);
 
 // Builds the kernel's configuration for a program under a plan; false when the program names an operand kind or

@@ -123,6 +123,9 @@ def test_ragged_rows_take_the_grid_form_when_every_stream_is_full_size_and_equal
     assert Prog(4096, 1500, BF16).row("layernorm", 2).name() == "rows_static_layernorm_wb_bf16_g64_it3_ragged"
     assert Prog(4096, 1500, BF16).op("mul", "rowvec").row("softmax").name().endswith("_it3_ragged")
     assert Prog(4096, 1500, BF16).row("layernorm").name() == "rows_static_layernorm_bf16_g64_it3_grid"  # no weight, no bias
+    assert Prog(4096, 4099, F32).row("layernorm", 2).name() == "rows_jit_layernorm_wb_f32_g256_it5_ragged"
+    # ... but for 1024-thread rows, whose unaligned form would spill
+    assert Prog(64, 50257, F32).row("layernorm", 2).name() == "rows_jit_layernorm_wb_f32_g1024_it13_grid"
     # at most two chunks per lane: the extra chunk of the grid form costs more than its aligned accesses gain
     assert Prog(4096, 1001, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it2_ragged"
     # streams at different addresses modulo 16

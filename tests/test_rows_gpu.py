@@ -311,8 +311,7 @@ def test_vocabulary_sized_rows_stay_in_registers_as_raw_words(dt):
     to_f64 = (lambda a: a.astype(np.float64)) if dt == F32 else (lambda a: axo.to_f32(a, dt).astype(np.float64))
     tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
     for cols in ((50304, 50257) if dt == F32 else (128256, 100001)):
-        ragged = "_grid" if cols % 2 else ""  # odd lengths: chunks on memory's 16-byte grid, but for the norms ...
-        ragged_wb = "_ragged" if cols % 2 else ""  # ... whose weights do not follow it
+        ragged = "_grid" if cols % 2 else ""  # odd lengths: chunks on memory's 16-byte grid
         it = (cols + (4 if dt == F32 else 8) * 1024 - 1) // ((4 if dt == F32 else 8) * 1024)
         x = to_dev(g.normal((3, cols)) * 3)
         xf = to_f64(x)
@@ -335,7 +334,7 @@ def test_vocabulary_sized_rows_stay_in_registers_as_raw_words(dt):
         x3f = to_f64(x3)
         p = gh.Rows(x3, dt).row_op("layernorm", 1e-5, w=w, b=b)
         got = to_f64(p.run())
-        assert p.kernel_name() == f"rows_jit_layernorm_wb_{tag}_g1024_it{it}{ragged_wb}", p.kernel_name()
+        assert p.kernel_name() == f"rows_jit_layernorm_wb_{tag}_g1024_it{it}{ragged}", p.kernel_name()
         want = (x3f - x3f.mean(-1, keepdims=True)) / np.sqrt(x3f.var(-1, keepdims=True) + 1e-5) * to_f64(w) + to_f64(b)
         assert np.max(np.abs(got - want)) < tol * (1 if dt == F32 else 2)
         p = gh.Rows(x3, dt).row_op("rmsnorm", 1e-5, w=w)
