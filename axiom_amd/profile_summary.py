@@ -5,6 +5,7 @@
                                                                        (this library's kernels only)
     python -m axiom_amd.profile_summary traffic <FETCH_SIZE dir> <WRITE_SIZE dir>
                                                                        HBM bytes per launch of bench.py's workloads
+    python -m axiom_amd.profile_summary survey  <bench.py output>      the `row_program_survey` of a bench line as a table
 
 `<dir>` is what `rocprofv3 ... -f csv -d <dir> -o <name>` wrote: `<name>_kernel_trace.csv` and, for a counter run,
 `<name>_counter_collection.csv` (searched recursively).  `traffic` scales FETCH_SIZE / WRITE_SIZE (KiB per dispatch) by
@@ -103,6 +104,19 @@ def traffic(fetch_dir: str, write_dir: str) -> None:
         print(f"| `{key}` | `{kn}` | {f:.0f} | {w:.0f} | {rd / 1e6:.1f} | {wr / 1e6:.1f} | {algo / 1e6:.1f} | {(rd + wr) / algo:.3f} | {rd + wr:.0f} |")
 
 
+def survey(path: str) -> None:
+    import json
+
+    line = json.loads(Path(path).read_text().strip().splitlines()[-1])
+    rows = line["row_program_survey"]
+    print("| program | kernel | MB | us | of HBM peak |\n|---|---|---:|---:|---:|")
+    for name, r in rows.items():
+        print(f"| `{name}` | `{r['kernel']}` | {r['bytes'] / 1e6:.0f} | {r['avg_us']:.1f} | {100 * r['frac_of_hbm_peak']:.1f} % |")
+    fr = [r["frac_of_hbm_peak"] for r in rows.values()]
+    print(f"\n{sum(f >= 0.7 for f in fr)} of {len(fr)} programs are at or above 70 % of the peak (lowest {100 * min(fr):.1f} %, highest {100 * max(fr):.1f} %); "
+          f"every result finite: {all(r['finite'] for r in rows.values())}.")
+
+
 def main() -> int:
     if len(sys.argv) >= 3 and sys.argv[1] == "trace":
         trace(sys.argv[2])
@@ -110,6 +124,8 @@ def main() -> int:
         counters(sys.argv[2:])
     elif len(sys.argv) == 4 and sys.argv[1] == "traffic":
         traffic(sys.argv[2], sys.argv[3])
+    elif len(sys.argv) == 3 and sys.argv[1] == "survey":
+        survey(sys.argv[2])
     else:
         print(__doc__, file=sys.stderr)
         return 2
