@@ -379,21 +379,32 @@ __device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
 
 // NW waves per work-group (4: two work-groups share a CU; 8: one work-group per CU, each
 // K/V tile fetched once for 256 query rows instead of 128).
-template <bool BF16, bool HAS_MASK, int NW, int D>
+// SPLIT = 2 (problems too small to give every SIMD two waves otherwise): the work-group's waves form two halves that
+// take the same 32 * NW / 2 query rows and one half of the keys each, through K/V tile buffers of their own; the second
+// half hands its accumulators, reference maximum and row sums to the first through LDS at the end.  No causal mask, no
+// explicit mask, at least two key tiles.
+// (Four K and four V tile buffers with counted waits, so that a tile is requested three steps before its use, made the
+// 4-wave head_dim-64 kernel 5 % slower on small problems: its step is not waiting for tiles.)
+template <bool BF16, bool HAS_MASK, int NW, int D, int SPLIT = 1>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_kernel(const SdpaArgs a) {
     static_assert(D == 128 || D == 64, "head sizes with a direct-to-LDS pipeline");
+    static_assert(SPLIT == 1 || (SPLIT == 2 && !HAS_MASK && NW == 4 && D == 64), "key split: the 64 KiB of static LDS hold two sets of head_dim-64 tiles");
+    constexpr int NWH = NW / SPLIT;       // waves that share a key range
     constexpr int KT = D / 16;            // k-steps of the score product
     constexpr int DT = D / 32;            // 32-row tiles of O^T
-    constexpr int BMW = 32 * NW;          // query rows per work-group
+    constexpr int BMW = 32 * NWH;         // query rows per work-group
     constexpr int ROWB = 2 * D;           // bytes per LDS row
     constexpr int CHUNKS = ROWB / 16;     // 16-byte chunks per row
     constexpr int RPL = 64 / CHUNKS;      // rows moved by one wave-wide load
-    constexpr int NLOAD = BN / (RPL * NW); // wave-wide loads per wave per tile
+    constexpr int NLOAD = BN / (RPL * NWH); // wave-wide loads per wave per tile
     constexpr int TILEB = BN * ROWB;      // 16 / 8 KiB per K or V tile
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILEB]; // K0 K1 V0 V1
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_all[SPLIT * 4 * TILEB]; // per half: K0 K1 V0 V1
 
     const int tid = threadIdx.x;
-    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int lane = tid % WAVE;
+    const int part = SPLIT == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid / WAVE / NWH); // which half of the keys
+    const int wave = SPLIT == 1 ? tid / WAVE : __builtin_amdgcn_readfirstlane(tid / WAVE % NWH); // position among the waves of its half
+    unsigned char *const lds = lds_all + part * 4 * TILEB;
     const int ql = lane % 32, g = lane / 32;
 
     // Work-group -> (batch*head, query block(s)).  Under a causal mask query block i needs
@@ -442,11 +453,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)); // LDS addresses fit 32 bits
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + RPL * wave * ROWB);
     // load n (0 .. NLOAD-1) of this wave's share of a K / V tile
+    // (tile: counted from the first tile of this half's key range, tile0 -- set per pass below)
+    int tile0 = 0;
     auto load_k1 = [&](int tile, int buf, int n) {
-        load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * RPL * NW * ROWB, k_voff + (tile * BN + RPL * NW * n) * krow_bytes);
+        load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * RPL * NWH * ROWB, k_voff + ((tile0 + tile) * BN + RPL * NWH * n) * krow_bytes);
     };
     auto load_v1 = [&](int tile, int buf, int n) {
-        load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * RPL * NW * ROWB, v_voff + (tile * BN + RPL * NW * n) * vrow_bytes);
+        load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * RPL * NWH * ROWB, v_voff + ((tile0 + tile) * BN + RPL * NWH * n) * vrow_bytes);
     };
     auto load_k = [&](int tile, int buf) {
 #pragma unroll
@@ -506,7 +519,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
 
         int kv_end = a.Skv;
         if (a.causal) kv_end = min(a.Skv, q0 + BMW);
-        const int ntiles = (kv_end + BN - 1) / BN; // >= 1
+        const int ntiles_all = (kv_end + BN - 1) / BN; // >= 1
+        // key split: the first half takes the larger share; `nsteps` is what the work-group's barriers are counted by
+        const int nsteps = SPLIT == 1 ? ntiles_all : (ntiles_all + 1) / 2;
+        const int ntiles = SPLIT == 1 ? ntiles_all : part == 0 ? nsteps : ntiles_all - nsteps; // >= 1 (the launcher sees to two tiles)
+        tile0 = SPLIT == 1 ? 0 : part * nsteps;
 
         // v_maximum3_f32: NaN-propagating maximum, which (unlike maxnum) needs no input canonicalisation
         auto max3 = [](float x, float y, float z) { return __builtin_elementwise_maximum(__builtin_elementwise_maximum(x, y), z); };
@@ -530,7 +547,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
         // initial value of the score accumulators of tile `tile`: `base`, or -inf where the mask words (already in
         // mk) say so
         auto init_scores = [&](int tile, float base, float16_t (&s)[2]) {
-            const bool use_words = HAS_MASK && mask_words && tile * BN + BN <= a.Skv;
+            const bool use_words = HAS_MASK && mask_words && (tile0 + tile) * BN + BN <= a.Skv;
     #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
     #pragma unroll
@@ -557,7 +574,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
         // the mask words of this lane's keys of one tile: bytes 32 kt + 8 i4 + 4 g .. + 3 of the tile's 64, kt < 2, i4 < 4
         auto load_mask_words = [&](int tile) {
             if constexpr (HAS_MASK) {
-                const int kvb = tile * BN;
+                const int kvb = (tile0 + tile) * BN;
                 if (mask_words && q_ok && kvb + BN <= a.Skv) {
                     const uint32_t *row = reinterpret_cast<const uint32_t *>(M + static_cast<int64_t>(q) * a.Skv + kvb + 4 * g);
     #pragma unroll
@@ -704,8 +721,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
 
         // One pipeline step: tile j is in `cur` (scores already computed), tile j+1's scores go to `nxt`.
         auto step = [&](int j, float16_t (&cur)[2], float mx_cur, float16_t (&nxt)[2], float &mx_nxt) {
-            const int kv0 = j * BN;
-            const bool active = !(a.causal && kv0 > qw0 + 31);
+            const int kv0 = (tile0 + j) * BN;
+            const bool active = !(a.causal && kv0 > qw0 + 31) && (SPLIT == 1 || j < ntiles);
             const unsigned char *Vb = lds + (2 + (j & 1)) * TILEB;
             const unsigned char *Kn = lds + ((j + 1) & 1) * TILEB;
             if (active) {
@@ -724,9 +741,35 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
             __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's async loads have landed
             __syncthreads();
         };
-        for (int j = 0; j < ntiles; j += 2) {
+        for (int j = 0; j < nsteps; j += 2) {
             step(j, sA, mxA, sB, mxB);
-            if (j + 1 < ntiles) step(j + 1, sB, mxB, sA, mxA);
+            if (j + 1 < nsteps) step(j + 1, sB, mxB, sA, mxA);
+        }
+
+        if constexpr (SPLIT == 2) {
+            // The second half's state goes to the first through LDS (the tile buffers are free: every step ends in a
+            // barrier), value-major so that the 64 lanes of a wave touch consecutive words.  Both halves hold sums of
+            // 2^(logit - reference) with a reference of their own: brought to the larger one and added.
+            float *xch = reinterpret_cast<float *>(lds_all) + wave * (DT * 16 + 2) * WAVE + lane;
+            if (part == 1) {
+    #pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+    #pragma unroll
+                    for (int i = 0; i < 16; ++i) xch[(dt * 16 + i) * WAVE] = oacc[dt][i];
+                xch[DT * 16 * WAVE] = m_run;
+                xch[(DT * 16 + 1) * WAVE] = l_run;
+            }
+            __syncthreads();
+            if (part == 1) return; // (one pass: no causal mask)
+            const float m_other = xch[DT * 16 * WAVE], l_other = xch[(DT * 16 + 1) * WAVE];
+            const float m_new = __builtin_elementwise_maximum(m_run, m_other);
+            const float a_mine = m_run == NEG_INF_F ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            const float a_other = m_other == NEG_INF_F ? 0.0f : __builtin_amdgcn_exp2f(m_other - m_new);
+            l_run = l_run * a_mine + l_other * a_other;
+    #pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+    #pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[dt][i] = oacc[dt][i] * a_mine + xch[(dt * 16 + i) * WAVE] * a_other;
         }
 
         const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
@@ -1180,6 +1223,12 @@ int sdpa_d128_waves = [] {
     return e ? atoi(e) : 0;
 }();
 
+// AXHIP_SDPA_KEY_SPLIT=0 keeps small head_dim-64 problems on the unsplit kernel (for A/B timing)
+bool sdpa_key_split = [] {
+    const char *e = getenv("AXHIP_SDPA_KEY_SPLIT");
+    return !(e && e[0] == '0');
+}();
+
 // AXHIP_SDPA_F32_MFMA=0 sends fp32 attention to the FMA kernel (for A/B timing)
 bool sdpa_f32_mfma = [] {
     const char *e = getenv("AXHIP_SDPA_F32_MFMA");
@@ -1342,6 +1391,17 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             const int nqb8 = (p.seq_q + 255) / 256;
             const int64_t g8 = static_cast<int64_t>(a.causal ? (nqb8 + 1) / 2 : nqb8) * a.B * a.H;
             const bool wide = p.seq_q > 128 && sdpa_d128_waves != 4 && (g8 >= 256 || sdpa_d128_waves == 8);
+            // Problems with 4-wave work-groups for at most half of the CUs split the keys between the two halves of a
+            // work-group of 64 query rows instead: twice the work-groups, half the steps each (12 heads of 1024 rows:
+            // 14.8 -> 10.6 us).  With a work-group for nearly every CU (Whisper's 20 heads of 1500 frames: 240) the
+            // split changes nothing -- a SIMD issues the same instructions as one wave or as two.
+            const int64_t g4 = static_cast<int64_t>((p.seq_q + 127) / 128) * a.B * a.H;
+            if (p.head_dim == 64 && !mask && !a.causal && p.seq_kv > BN && g4 <= 128 && sdpa_key_split) {
+                const unsigned gs = static_cast<unsigned>((p.seq_q + 63) / 64) * static_cast<unsigned>(a.B * a.H);
+                if (bf) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<true, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
+                else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<false, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
+                break;
+            }
             const int bmw = wide ? 256 : 128;
             const int nqbw = (p.seq_q + bmw - 1) / bmw;
             const unsigned g = static_cast<unsigned>(a.causal ? (nqbw + 1) / 2 : nqbw) * static_cast<unsigned>(a.B * a.H);

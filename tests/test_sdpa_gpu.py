@@ -102,6 +102,30 @@ def test_half_matches_fp32_reference_of_same_inputs(case, dt):
     assert np.max(np.abs(gotf - lit)) < 4e-2
 
 
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+def test_small_head_dim_64_problems_split_their_keys_between_the_halves_of_a_work_group(dt):
+    """Unmasked head_dim-64 problems with 128-row work-groups for at most half of the compute units run with
+    work-groups of 64 query rows whose two halves take half of the key tiles each and merge their softmax states at
+    the end.  Key counts around the tile size (two tiles with one key in the second, an odd number of tiles, a ragged
+    last tile), a single query row, cross attention, and the Whisper shape (which stays unsplit: 240 work-groups);
+    against float64, and with V = 1 (every output is then the merged normalisation itself: exactly 1)."""
+    for B, H, Sq, Skv in ((2, 3, 64, 65), (1, 2, 1, 1000), (1, 4, 200, 130), (1, 1, 70, 128), (2, 2, 130, 129), (1, 3, 300, 77),
+                          (1, 5, 33, 192), (1, 20, 1500, 1500)):
+        q, k, v = inputs(B, H, Sq, Skv, 64, dt, seed=100 + Skv)
+        got, kern = gh.sdpa(q, k, v, dt, -1.0, False, None)
+        assert kern == f"mfma_{'bf16' if dt == BF16 else 'f16'}_d64"
+        qf, kf, vf = (axo.to_f32(t, dt) for t in (q, k, v))
+        if B * H * Sq * Skv <= 1 << 24:
+            want = naive_attention64(qf, kf, vf, 0.125, False, None)
+        else:
+            want = axo.sdpa(qf, kf, vf, F32, -1.0, False, None)
+        err = np.max(np.abs(axo.to_f32(got, dt) - want))
+        assert err < 2e-2, (B, H, Sq, Skv, err)
+        ones = axo.to_bits(np.ones(v.shape, np.float32), dt)
+        got, _ = gh.sdpa(q, k, ones, dt, -1.0, False, None)
+        assert np.max(np.abs(axo.to_f32(got, dt) - 1.0)) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -10), (B, H, Sq, Skv)
+
+
 def test_fully_masked_rows_give_zeros_everywhere_else_matches():
     q, k, v = inputs(1, 2, 70, 70, 64, BF16, seed=3)
     m = np.zeros((70, 70), np.uint8)
