@@ -491,95 +491,107 @@ std::vector<const GraphNode *> topo_sort(const GraphNode *root) {
 }
 
 namespace {
-constexpr uint64_t FNV_OFFSET = 14695981039346656037ULL, FNV_PRIME = 1099511628211ULL;
-inline uint64_t mix_bytes(uint64_t h, const void *p, size_t n) {
-    const unsigned char *b = static_cast<const unsigned char *>(p);
-    for (size_t i = 0; i < n; ++i) h = (h ^ b[i]) * FNV_PRIME;
-    return h;
+// FNV-1a over the bytes of everything that decides what a graph computes.  A value is fed in the width named by the
+// call (sizes and indices as 64 bits, axes and window sizes as 32, floats by their bit pattern, flags as one byte).
+class Fnv1a {
+  public:
+    void bytes(const void *p, size_t n) {
+        const unsigned char *b = static_cast<const unsigned char *>(p);
+        for (size_t i = 0; i < n; ++i) state_ = (state_ ^ b[i]) * 1099511628211ULL;
+    }
+    void u64(uint64_t v) { bytes(&v, 8); }
+    void i32(int32_t v) { bytes(&v, 4); }
+    void f32(float v) { bytes(&v, 4); }
+    void flag(bool v) {
+        const unsigned char b = v ? 1 : 0;
+        bytes(&b, 1);
+    }
+    template <typename T, typename F> void list(const std::vector<T> &v, F &&each) {
+        u64(v.size());
+        for (const T &x : v) each(x);
+    }
+    uint64_t value() const { return state_; }
+
+  private:
+    uint64_t state_ = 14695981039346656037ULL;
+};
+
+// what each kind of node parameters contributes (nodes without parameters: nothing beyond the variant's index)
+void feed(Fnv1a &h, const NoParams &) { (void)h; }
+void feed(Fnv1a &h, const ReductionParams &p) {
+    h.list(p.axes, [&](int a) { h.i32(a); });
+    h.flag(p.keep_dims);
 }
-inline uint64_t mix(uint64_t h, uint64_t v) { return mix_bytes(h, &v, 8); }
-inline uint64_t mix_i32(uint64_t h, int32_t v) { return mix_bytes(h, &v, 4); }
-inline uint64_t mix_f32(uint64_t h, float v) { return mix_bytes(h, &v, 4); }
-inline uint64_t mix_bool(uint64_t h, bool v) {
-    const unsigned char b = v ? 1 : 0;
-    return mix_bytes(h, &b, 1);
+void feed(Fnv1a &h, const MatMulParams &p) {
+    h.flag(p.transpose_a);
+    h.flag(p.transpose_b);
+}
+void feed(Fnv1a &h, const ActivationParams &p) {
+    h.f32(p.alpha);
+    h.i32(p.axis);
+}
+void feed(Fnv1a &h, const ReshapeParams &p) {
+    h.list(p.new_shape, [&](size_t d) { h.u64(d); });
+}
+void feed(Fnv1a &h, const NormParams &p) {
+    h.i32(p.axis);
+    h.f32(p.eps);
+}
+void feed(Fnv1a &h, const TransposeParams &p) {
+    h.list(p.axes, [&](int a) { h.i32(a); });
+}
+void feed(Fnv1a &h, const SliceParams &p) {
+    h.u64(p.starts.size());
+    for (size_t i = 0; i < p.starts.size(); ++i) {
+        h.u64(static_cast<uint64_t>(p.starts[i]));
+        h.u64(static_cast<uint64_t>(p.ends[i]));
+        h.u64(static_cast<uint64_t>(p.steps[i]));
+    }
+}
+void feed(Fnv1a &h, const PadParams &p) {
+    h.list(p.pad_widths, [&](const auto &w) {
+        h.u64(w.first);
+        h.u64(w.second);
+    });
+    h.bytes(&p.value, sizeof(p.value));
+}
+void feed(Fnv1a &h, const MaskedFillParams &p) { h.f32(p.value); }
+void feed(Fnv1a &h, const UnfoldParams &p) {
+    for (int v : {p.kernel, p.stride, p.dilation, p.kernel_h, p.stride_h, p.dilation_h}) h.i32(v);
+}
+
+// one node: operation, result, where it sits in the order, what it reads
+void feed_node(Fnv1a &h, const GraphNode *n, const GraphNode *root, const std::unordered_map<const GraphNode *, uint32_t> &position) {
+    h.u64(static_cast<uint64_t>(n->op_type));
+    h.list(n->output_shape, [&](size_t d) { h.u64(d); });
+    h.u64(static_cast<uint64_t>(n->output_dtype));
+    h.u64(static_cast<uint64_t>(n->target_device));
+    h.flag(n->is_constant);
+    if (n->is_constant) h.list(n->constant_strides, [&](int64_t s) { h.u64(static_cast<uint64_t>(s)); });
+    // a constant, and a node that already holds its result, are inputs of the plan: what produced them is not part of it
+    const bool leaf = n->is_constant || (n->is_materialized_ && n != root);
+    if (leaf) {
+        h.u64(0);
+    } else {
+        h.list(n->inputs, [&](const std::shared_ptr<GraphNode> &in) {
+            const auto it = position.find(in.get());
+            h.u64(it != position.end() ? it->second : UINT64_MAX);
+        });
+    }
+    h.u64(n->params.index());
+    std::visit([&](const auto &p) { feed(h, p); }, n->params);
 }
 } // namespace
 
 GraphSignature compute_signature(const GraphNode *root) {
-    const auto sorted = topo_sort(root);
-    std::unordered_map<const GraphNode *, uint32_t> index;
-    for (uint32_t i = 0; i < sorted.size(); ++i) index[sorted[i]] = i;
-    uint64_t h = mix(FNV_OFFSET, sorted.size());
-    for (const GraphNode *n : sorted) {
-        h = mix(h, static_cast<uint64_t>(n->op_type));
-        h = mix(h, n->output_shape.size());
-        for (size_t d : n->output_shape) h = mix(h, d);
-        h = mix(h, static_cast<uint64_t>(n->output_dtype));
-        h = mix(h, static_cast<uint64_t>(n->target_device));
-        h = mix_bool(h, n->is_constant);
-        if (n->is_constant) {
-            h = mix(h, n->constant_strides.size());
-            for (int64_t s : n->constant_strides) h = mix(h, static_cast<uint64_t>(s));
-        }
-        const bool leaf = n->is_constant || (n->is_materialized_ && n != root);
-        h = mix(h, leaf ? 0 : n->inputs.size());
-        if (!leaf)
-            for (const auto &in : n->inputs) {
-                auto it = index.find(in.get());
-                h = mix(h, it != index.end() ? it->second : UINT64_MAX);
-            }
-        h = mix(h, n->params.index());
-        std::visit(
-            [&](const auto &p) {
-                using T = std::decay_t<decltype(p)>;
-                if constexpr (std::is_same_v<T, ReductionParams>) {
-                    h = mix(h, p.axes.size());
-                    for (int a : p.axes) h = mix_i32(h, a);
-                    h = mix_bool(h, p.keep_dims);
-                } else if constexpr (std::is_same_v<T, MatMulParams>) {
-                    h = mix_bool(h, p.transpose_a);
-                    h = mix_bool(h, p.transpose_b);
-                } else if constexpr (std::is_same_v<T, ActivationParams>) {
-                    h = mix_f32(h, p.alpha);
-                    h = mix_i32(h, p.axis);
-                } else if constexpr (std::is_same_v<T, ReshapeParams>) {
-                    h = mix(h, p.new_shape.size());
-                    for (size_t d : p.new_shape) h = mix(h, d);
-                } else if constexpr (std::is_same_v<T, NormParams>) {
-                    h = mix_i32(h, p.axis);
-                    h = mix_f32(h, p.eps);
-                } else if constexpr (std::is_same_v<T, TransposeParams>) {
-                    h = mix(h, p.axes.size());
-                    for (int a : p.axes) h = mix_i32(h, a);
-                } else if constexpr (std::is_same_v<T, SliceParams>) {
-                    h = mix(h, p.starts.size());
-                    for (size_t i = 0; i < p.starts.size(); ++i) {
-                        h = mix(h, static_cast<uint64_t>(p.starts[i]));
-                        h = mix(h, static_cast<uint64_t>(p.ends[i]));
-                        h = mix(h, static_cast<uint64_t>(p.steps[i]));
-                    }
-                } else if constexpr (std::is_same_v<T, PadParams>) {
-                    h = mix(h, p.pad_widths.size());
-                    for (const auto &w : p.pad_widths) {
-                        h = mix(h, w.first);
-                        h = mix(h, w.second);
-                    }
-                    h = mix_bytes(h, &p.value, sizeof(p.value));
-                } else if constexpr (std::is_same_v<T, MaskedFillParams>) {
-                    h = mix_f32(h, p.value);
-                } else if constexpr (std::is_same_v<T, UnfoldParams>) {
-                    h = mix_i32(h, p.kernel);
-                    h = mix_i32(h, p.stride);
-                    h = mix_i32(h, p.dilation);
-                    h = mix_i32(h, p.kernel_h);
-                    h = mix_i32(h, p.stride_h);
-                    h = mix_i32(h, p.dilation_h);
-                }
-            },
-            n->params);
-    }
-    return GraphSignature{h};
+    const auto order = topo_sort(root);
+    std::unordered_map<const GraphNode *, uint32_t> position;
+    position.reserve(order.size());
+    for (uint32_t i = 0; i < order.size(); ++i) position.emplace(order[i], i);
+    Fnv1a h;
+    h.u64(order.size());
+    for (const GraphNode *n : order) feed_node(h, n, root, position);
+    return GraphSignature{h.value()};
 }
 
 } // namespace axiom::graph
