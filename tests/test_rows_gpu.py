@@ -652,3 +652,97 @@ def test_layer_norm_of_16_bit_rows_far_from_zero(dt, offset, spread, cols):
     got = axo.to_f32(gh.Rows(x, dt).binary("add", y).row_op("layernorm", 1e-5, w, b).run(), dt)
     want = ln(xf + axo.to_f32(y, dt))
     assert np.all(np.abs(got - want) <= tol(want)), float(np.max(np.abs(got - want)))
+
+
+def _random_row_program(r, g, dt):
+    """A seeded random program and its float64 evaluation on the values the device reads (16-bit inputs widened)."""
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    rows = int(r.integers(1, 24))
+    cols = int(r.choice([5, 64, 100, 777, 1001, 1024, 1500, 2048, 3000, 4097, 5000, 9000, 12288, 20000, 40001]))
+    x = store(g.normal((rows, cols)) * 1.5)
+    row_op = str(r.choice(["none", "softmax", "logsoftmax", "layernorm", "rmsnorm", "softmax", "layernorm"]))
+    reduce = str(r.choice(["sum", "max", "mean"])) if row_op == "none" else str(r.choice(["none", "none", "none", "sum", "max"]))
+    out_dt = F32 if (reduce != "none" or r.integers(0, 5) == 0) else dt
+    p = gh.Rows(x, dt, out_dt)
+    ref = wide(x)
+    desc = []
+
+    def operand(kind):
+        shape = {"full": (rows, cols), "rowvec": (cols,), "colvec": (rows,), "scalar": (1,)}[kind]
+        v = store(g.uniform(shape, 0.5, 1.5) * (1 if r.integers(0, 2) else -1))
+        w = wide(v)
+        return v, (w[:, None] if kind == "colvec" else w)
+
+    def chain(n_ops, choices):
+        nonlocal ref
+        for _ in range(n_ops):
+            op = str(r.choice(choices))
+            desc.append(op)
+            if op in ("relu", "abs", "neg", "tanh", "sigmoid", "silu", "gelu", "square"):
+                p.unary(op)
+                ref = {"relu": lambda t: np.maximum(t, 0), "abs": np.abs, "neg": lambda t: -t, "tanh": np.tanh,
+                       "sigmoid": lambda t: 1 / (1 + np.exp(-t)), "silu": lambda t: t / (1 + np.exp(-t)),
+                       "gelu": lambda t: 0.5 * t * (1 + np.vectorize(__import__("math").erf)(t / np.sqrt(2.0))), "square": lambda t: t * t}[op](ref)
+            elif op in ("mul_imm", "add_imm"):
+                c = float(np.float32(r.uniform(0.25, 2.0)))
+                p.imm(op[:3], c)
+                ref = ref * c if op == "mul_imm" else ref + c
+            else:  # add / mul / sub / max with an operand of some broadcast kind
+                name, kind = op.split("_")
+                v, w = operand(kind)
+                p.binary(name, v, kind)
+                ref = {"add": ref + w, "mul": ref * w, "sub": ref - w, "max": np.maximum(ref, w)}[name]
+
+    binary = [f"{o}_{k}" for o in ("add", "mul", "sub", "max") for k in ("full", "rowvec", "colvec", "scalar")]
+    chain(int(r.integers(0, 4)), ["relu", "abs", "neg", "tanh", "mul_imm", "add_imm"] + binary)
+    if row_op != "none":
+        desc.append(row_op)
+        if row_op in ("softmax", "logsoftmax"):
+            p.row_op(row_op)
+            z = ref - ref.max(-1, keepdims=True)
+            lse = np.log(np.exp(z).sum(-1, keepdims=True))
+            ref = np.exp(z - lse) if row_op == "softmax" else z - lse
+        else:
+            affine = int(r.integers(0, 3)) if row_op == "layernorm" else int(r.integers(0, 2))
+            w = store(g.uniform((cols,), 0.5, 1.5)) if affine >= 1 else None
+            b = store(g.uniform((cols,), -0.5, 0.5)) if affine >= 2 else None
+            p.row_op(row_op, 1e-5, w=w, b=b)
+            if row_op == "layernorm":
+                ref = (ref - ref.mean(-1, keepdims=True)) / np.sqrt(ref.var(-1, keepdims=True) + 1e-5)
+            else:
+                ref = ref / np.sqrt((ref * ref).mean(-1, keepdims=True) + 1e-5)
+            if w is not None:
+                ref = ref * wide(w)
+            if b is not None:
+                ref = ref + wide(b)
+        chain(int(r.integers(0, 3)), ["relu", "gelu", "silu", "sigmoid", "tanh", "mul_imm", "add_imm", "mul_full", "add_rowvec", "mul_colvec"])
+    if reduce != "none":
+        desc.append("reduce_" + reduce)
+        ref = {"sum": ref.sum(-1), "max": ref.max(-1), "mean": ref.mean(-1)}[reduce]
+    return p, reduce, ref, out_dt, f"{rows}x{cols} " + " ".join(desc)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_seeded_random_row_programs_match_fp64(dt):
+    """Forty seeded random programs per element type: up to three pre operations (unary, immediate, operands of all four
+    broadcast kinds), a row operation with or without affine part, up to two post operations, an optional row
+    reduction, fp32 or same-type results, over row lengths from 5 to 40 001 (aligned, odd, one to 1024 threads per
+    row) -- whatever kernel the library picks (built in, compiled here, interpreter), against float64."""
+    r = np.random.default_rng(4242 + dt)
+    g = axo.PCG64(99 + dt)
+    kinds = set()
+    for case in range(40):
+        p, reduce, ref, out_dt, desc = _random_row_program(r, g, dt)
+        got = p.run(reduce=reduce)
+        name = p.kernel_name()
+        kinds.add(name.split("_")[1])
+        got = got.astype(np.float64) if out_dt == F32 else axo.to_f32(got, out_dt).astype(np.float64)
+        # the device computes in fp32 from the same inputs; a 16-bit result adds half an ulp of its own
+        ulp = {F32: 0.0, BF16: 2.0 ** -8, F16: 2.0 ** -11}[out_dt]
+        tol = 1e-5 * np.maximum(1.0, np.abs(ref)) * (40.0 if reduce in ("sum", "mean") else 4.0) + ulp * np.abs(ref) + (0.0 if out_dt == F32 else 1e-7)
+        if dt != F32 and out_dt != F32:
+            tol = tol + 2e-4  # the polynomial activations behind a 16-bit result
+        err = np.abs(got.reshape(ref.shape) - ref)
+        assert np.all(err <= tol), (case, desc, name, float(np.max(err / tol)))
+    assert {"static", "jit"} <= kinds, kinds
