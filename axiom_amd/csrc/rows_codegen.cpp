@@ -389,7 +389,16 @@ bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, Ro
             // (at most 64 registers) instead of as fp32 -- still one read of the row, at the price of unpacking it and
             // running the pre chain once per pass.
             const int64_t n = (chunks + 1023) / 1024;
-            if (n > 16 || raw_words_per_chunk(P) * n > 72) return false;
+            if (n > 16 || raw_words_per_chunk(P) * n > 72) {
+                // Longer still (aligned rows): a 1024-thread block walks the row in steps of 4 chunks per thread (2 when
+                // the operands of a step would not fit 64 registers), once for the statistics and once for the output.
+                if (ragged) return false;
+                rows_prog_plan_for(P, 1024, raw_words_per_chunk(P) * 4 <= 64 ? 4 : 2, false, plan, false);
+                plan->loop = true;
+                plan->pipe = false;
+                plan->min_waves = 4;
+                return true;
+            }
             group = 1024;
             it = static_cast<int>(n);
             rerun = true;
@@ -445,6 +454,9 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     if (rerun) pipe = false;
     c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ", RERUN = " << (rerun ? "true" : "false")
       << ", GRID = " << (plan.ragged && plan.grid ? "true" : "false") << ";\n";
+    c << "constexpr bool LOOP = " << (plan.loop ? "true" : "false") << ";\n";
+    // looped rows with a row operation keep the raw words of their first steps: up to 48 registers per thread
+    c << "constexpr int HOLD = " << (plan.loop && P.row_op != AXHIP_ROWOP_NONE ? 48 / (raw_words_per_chunk(P) * plan.it) : 0) << ";\n";
     c << "constexpr int TAIL_FROM = " << (plan.ragged && plan.grid ? plan.tail_from : 0) << ";\n";
     c << "constexpr int MIN_WAVES = " << plan.min_waves << ";\n";
     c << "constexpr int ROWOP = " << P.row_op << ", RED = " << red << ";\n";
@@ -475,7 +487,7 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     char tail[64];
     const bool other_out = P.reduce == AXHIP_RED_NONE && P.output_dtype != dt;
     snprintf(tail, sizeof(tail), "%s%s%s_g%d_it%d%s", dt_name(dt), other_out ? "_to_" : "", other_out ? dt_name(P.output_dtype) : "", plan.group, plan.it,
-             !plan.ragged ? "" : plan.grid ? "_grid" : "_ragged"); // (grid: ragged rows addressed on memory's 16-byte grid)
+             plan.loop ? "_loop" : !plan.ragged ? "" : plan.grid ? "_grid" : "_ragged"); // (grid: ragged rows addressed on memory's 16-byte grid)
     S.label = label + tail;
     // the kernel's symbol: the readable label (what a profiler lists) plus a hash of everything that shapes the code
     S.symbol = "axp_" + S.label + "_" + hash;

@@ -35,6 +35,7 @@ struct RowsProgPlan {
     int group = 0, it = 0; // threads per row, 16-byte input chunks per thread
     bool ragged = false;   // rows are not whole aligned vectors
     bool grid = false;     // ragged rows whose full-size streams share their address modulo 16: chunks on memory's 16-byte grid
+    bool loop = false;     // rows beyond the registers of a block: every pass walks the row in steps of `it` chunks per thread
     int tail_from = 0;     // grid rows: a thread's chunks before this one are known to lie inside the row (0: nothing known)
     bool pipe = false;     // the next row is requested before the current one is computed
     bool rerun = false;    // the row stays in registers as raw words; every pass unpacks it and applies the pre chain again

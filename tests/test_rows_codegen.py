@@ -107,7 +107,11 @@ def test_long_rows_get_a_1024_thread_block_and_beyond_8_chunks_per_thread_stay_a
     assert Prog(64, 50257, F32).op("mul", imm=0.5).row("softmax").name() == "rows_jit_muls_softmax_f32_g1024_it13_grid"
     # two 16-bit streams fit up to 9 chunks each per thread, not 16
     assert Prog(64, 70000, BF16).op("add", "full").row("softmax").name() == "rows_jit_addf_softmax_bf16_g1024_it9"
-    assert Prog(64, 128256, BF16).op("add", "full").row("softmax").name() == "rows_streamed_e8"
+    # beyond that (aligned rows): the block walks the row in steps of 4 chunks per thread, once per pass
+    assert Prog(64, 128256, BF16).op("add", "full").row("softmax").name() == "rows_jit_addf_softmax_bf16_g1024_it4_loop"
+    assert Prog(64, 128256, F32).row("softmax").name() == "rows_jit_softmax_f32_g1024_it4_loop"
+    assert Prog(4, 1 << 20, BF16).row("layernorm", 2).op("gelu").name() == "rows_jit_layernorm_gelu_wb_bf16_g1024_it4_loop"
+    assert Prog(4, 200000, F32).op("abs").reduce("max").name() == "rows_jit_abs_reduce_max_f32_g1024_it4_loop"
 
 
 def test_ragged_rows_take_the_grid_form_when_every_stream_is_full_size_and_equally_aligned():
@@ -141,7 +145,7 @@ def test_ragged_rows_take_the_grid_form_when_every_stream_is_full_size_and_equal
 
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     assert Prog(1024, 4096, F32).op("relu").op("mul", "full").name() == "elementwise_e4"  # no row op, no reduction
-    assert Prog(4, 1 << 20, BF16).row("softmax").name() == "rows_streamed_e8"  # beyond 16384 chunks
+    assert Prog(4, 1000001, BF16).row("softmax").name() == "rows_streamed_e1"  # beyond 16384 chunks and not whole vectors
     # ragged rows whose streams differ in element size
     assert Prog(64, 1001, BF16, out_dt=F32).row("softmax").name().startswith("rows_resident_")
 
@@ -153,7 +157,9 @@ def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     lambda: Prog(4096, 12000, F32).op("mul", "colvec").op("add", "scalar").row("logsoftmax").op("exp"),
     lambda: Prog(4096, 5000, BF16).op("relu").op("max", imm=0.25).reduce("max"),
     lambda: Prog(64, 128256, F16).op("mul", imm=0.5).row("logsoftmax"),
-], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10", "raw_resident_it16"])
+    lambda: Prog(64, 128256, F32).op("mul", "rowvec").op("add", "full").row("logsoftmax").op("exp").reduce("sum"),
+], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10", "raw_resident_it16",
+        "looped_row"])
 def test_generated_kernels_compile(build):
     prog = build()
     assert prog.name().startswith("rows_jit_"), prog.name()

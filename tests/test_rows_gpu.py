@@ -360,10 +360,11 @@ def test_vocabulary_sized_rows_stay_in_registers_as_raw_words(dt):
 def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
     """Rows beyond the 32 KiB the built-in kernels hold: up to 8192 16-byte chunks stay in the registers of a
     512- or 1024-thread block as fp32, up to 16384 as the raw words they were loaded as (one read either way; kernels
-    compiled at first launch); longer ones are streamed in passes by the interpreter."""
+    compiled at first launch); longer aligned ones are walked in passes by a compiled kernel, longer odd ones by the
+    interpreter."""
     g = axo.PCG64(123)
     for cols, plan in ((12000, "rows_jit_softmax_f32_g512_it6"), (16384, "rows_jit_softmax_f32_g512_it8"), (20000, "rows_jit_softmax_f32_g1024_it5"),
-                       (40000, "rows_jit_softmax_f32_g1024_it10"), (70000, "rows_streamed_e4")):
+                       (40000, "rows_jit_softmax_f32_g1024_it10"), (70000, "rows_jit_softmax_f32_g1024_it4_loop"), (70001, "rows_streamed_e1")):
         x = (g.normal((3, cols)) * 2).astype(np.float32)
         p = gh.Rows(x, F32).row_op("softmax")
         got = p.run()
@@ -381,6 +382,65 @@ def test_long_rows_on_the_1024_thread_resident_plan_and_the_streamed_one():
     assert np.max(np.abs(got - want)) < 2e-2
     got = gh.Rows(x, F32).unary("square").run(reduce="mean")
     assert np.allclose(got, (x.astype(np.float64) ** 2).mean(-1), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_rows_beyond_the_registers_of_a_block_are_walked_in_passes(dt):
+    """Aligned rows of more than 16384 chunks (fp32 logits over a vocabulary of 128 256; two 16-bit streams of that
+    length): a 1024-thread block walks the row in steps of four chunks per thread, once for the statistics (online
+    softmax reference and sum per thread, merged across the block; sum and sum of squares for the norms, with a centred
+    second pass for rows far from zero) and once for the output.  Row lengths that end inside a step and on one."""
+    g = axo.PCG64(31 + dt)
+    tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
+    e = 4 if dt == F32 else 8
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    tol = 1e-5 if dt == F32 else (2.0 ** -8 if dt == BF16 else 2.0 ** -10)
+    for cols in (16385 * e, 4096 * e * 5, 128256 * (1 if dt == F32 else 2)):
+        x = store(g.normal((3, cols)) * 2)
+        xf = wide(x)
+        p = gh.Rows(x, dt).row_op("softmax")
+        got = wide(p.run())
+        assert p.kernel_name() == f"rows_jit_softmax_{tag}_g1024_it4_loop", p.kernel_name()
+        ex = np.exp(xf - xf.max(-1, keepdims=True))
+        want = ex / ex.sum(-1, keepdims=True)
+        assert np.all(np.abs(got - want) <= tol * want + (2.0 ** -24 if dt == F16 else 1e-9)), cols  # (f16: subnormal results step by 2^-24)
+        assert np.max(np.abs(got.sum(-1) - 1.0)) < (1e-4 if dt == F32 else 5e-3)
+    cols = 20000 * e
+    x, y = store(g.normal((2, cols)) * 2), store(g.normal((2, cols)))
+    xf, yf = wide(x), wide(y)
+    # log-softmax of scaled logits plus a full-size bias, exponentiated again and summed per row: 1
+    p = gh.Rows(x, dt, F32).imm("mul", 0.5).binary("add", y).row_op("logsoftmax").unary("exp")
+    got = p.run(reduce="sum")
+    assert p.kernel_name() == f"rows_jit_muls_addf_logsoftmax_exp_sum_{tag}_g1024_it4_loop", p.kernel_name()
+    assert np.max(np.abs(got.astype(np.float64) - 1.0)) < 1e-4
+    p = gh.Rows(x, dt).imm("mul", 0.5).binary("add", y).row_op("logsoftmax")
+    got = wide(p.run())
+    z = xf * 0.5 + yf
+    want = z - z.max(-1, keepdims=True) - np.log(np.exp(z - z.max(-1, keepdims=True)).sum(-1, keepdims=True))
+    assert np.all(np.abs(got - want) <= tol * np.abs(want) + 1e-5), np.max(np.abs(got - want))
+    # layer norm with weight and bias, rows near zero and far from it (mean 40 at sigma 1: the centred second pass)
+    w, b = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((cols,), -0.5, 0.5))
+    for shift in (0.0, 40.0):
+        x3 = store(g.normal((2, cols)) + shift)
+        x3f = wide(x3)
+        p = gh.Rows(x3, dt).row_op("layernorm", 1e-5, w=w, b=b)
+        got = wide(p.run())
+        assert p.kernel_name() == f"rows_jit_layernorm_wb_{tag}_g1024_it4_loop", p.kernel_name()
+        want = (x3f - x3f.mean(-1, keepdims=True)) / np.sqrt(x3f.var(-1, keepdims=True) + 1e-5) * wide(w) + wide(b)
+        assert np.max(np.abs(got - want)) < (1e-4 if dt == F32 else 2e-2 * 2), (shift, np.max(np.abs(got - want)))
+    p = gh.Rows(x, dt).row_op("rmsnorm", 1e-5, w=w).unary("silu")
+    got = wide(p.run())
+    n = xf / np.sqrt((xf * xf).mean(-1, keepdims=True) + 1e-5) * wide(w)
+    assert np.max(np.abs(got - n / (1 + np.exp(-n)))) < (1e-4 if dt == F32 else 2e-2)
+    # reductions without a row operation: one pass
+    p = gh.Rows(x, dt, F32).unary("abs")
+    got = p.run(reduce="max")
+    assert p.kernel_name() == f"rows_jit_abs_reduce_max_{tag}_g1024_it4_loop", p.kernel_name()
+    assert np.array_equal(got.reshape(-1).astype(np.float64), np.abs(xf).max(-1))
+    p = gh.Rows(x, dt, F32).binary("mul", y)
+    got = p.run(reduce="mean")
+    assert np.allclose(got.reshape(-1), (xf * yf).mean(-1), rtol=1e-4, atol=1e-5)
 
 
 def test_unary_then_row_reduction_runs_on_the_specialised_reduce_kernels():
@@ -659,7 +719,7 @@ def _random_row_program(r, g, dt):
     store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
     wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
     rows = int(r.integers(1, 24))
-    cols = int(r.choice([5, 64, 100, 777, 1001, 1024, 1500, 2048, 3000, 4097, 5000, 9000, 12288, 20000, 40001]))
+    cols = int(r.choice([5, 64, 100, 777, 1001, 1024, 1500, 2048, 3000, 4097, 5000, 9000, 12288, 20000, 40001, 140000]))
     x = store(g.normal((rows, cols)) * 1.5)
     row_op = str(r.choice(["none", "softmax", "logsoftmax", "layernorm", "rmsnorm", "softmax", "layernorm"]))
     reduce = str(r.choice(["sum", "max", "mean"])) if row_op == "none" else str(r.choice(["none", "none", "none", "sum", "max"]))
@@ -717,30 +777,32 @@ def _random_row_program(r, g, dt):
             if b is not None:
                 ref = ref + wide(b)
         chain(int(r.integers(0, 3)), ["relu", "gelu", "silu", "sigmoid", "tanh", "mul_imm", "add_imm", "mul_full", "add_rowvec", "mul_colvec"])
+    mag = np.abs(ref)  # what the result's rounding errors scale with: for a sum, the sum of the magnitudes
     if reduce != "none":
         desc.append("reduce_" + reduce)
+        mag = {"sum": mag.sum(-1), "max": np.abs(ref.max(-1)), "mean": mag.mean(-1)}[reduce]
         ref = {"sum": ref.sum(-1), "max": ref.max(-1), "mean": ref.mean(-1)}[reduce]
-    return p, reduce, ref, out_dt, f"{rows}x{cols} " + " ".join(desc)
+    return p, reduce, ref, mag, out_dt, f"{rows}x{cols} " + " ".join(desc)
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_seeded_random_row_programs_match_fp64(dt):
     """Forty seeded random programs per element type: up to three pre operations (unary, immediate, operands of all four
     broadcast kinds), a row operation with or without affine part, up to two post operations, an optional row
-    reduction, fp32 or same-type results, over row lengths from 5 to 40 001 (aligned, odd, one to 1024 threads per
-    row) -- whatever kernel the library picks (built in, compiled here, interpreter), against float64."""
+    reduction, fp32 or same-type results, over row lengths from 5 to 140 000 (aligned, odd, one to 1024 threads per
+    row, rows walked in passes) -- whatever kernel the library picks (built in, compiled here, interpreter), against float64."""
     r = np.random.default_rng(4242 + dt)
     g = axo.PCG64(99 + dt)
     kinds = set()
     for case in range(40):
-        p, reduce, ref, out_dt, desc = _random_row_program(r, g, dt)
+        p, reduce, ref, mag, out_dt, desc = _random_row_program(r, g, dt)
         got = p.run(reduce=reduce)
         name = p.kernel_name()
         kinds.add(name.split("_")[1])
         got = got.astype(np.float64) if out_dt == F32 else axo.to_f32(got, out_dt).astype(np.float64)
         # the device computes in fp32 from the same inputs; a 16-bit result adds half an ulp of its own
         ulp = {F32: 0.0, BF16: 2.0 ** -8, F16: 2.0 ** -11}[out_dt]
-        tol = 1e-5 * np.maximum(1.0, np.abs(ref)) * (40.0 if reduce in ("sum", "mean") else 4.0) + ulp * np.abs(ref) + (0.0 if out_dt == F32 else 1e-7)
+        tol = 4e-5 * np.maximum(1.0, mag) + ulp * np.abs(ref) + (0.0 if out_dt == F32 else 1e-7)
         if dt != F32 and out_dt != F32:
             tol = tol + 2e-4  # the polynomial activations behind a 16-bit result
         err = np.abs(got.reshape(ref.shape) - ref)
