@@ -370,8 +370,9 @@ def bench_survey(torch, capi, stream, steps, warmup):
     run("mean(x^2)_bf16_16384x4099", P(t, f32).op("square").finish(torch, "mean"))
     del t, u
     # vocabulary-sized rows (language-model logits): 1024-thread blocks; beyond 8 chunks per thread the row stays in
-    # registers as raw words
-    for rows, cols, dt, name in ((4096, 50304, bf, "bf16"), (2048, 128256, bf, "bf16"), (2048, 50304, f32, "f32"), (4096, 50257, bf, "bf16")):
+    # registers as raw words, beyond 16 (fp32 logits over 128 256 entries) the block walks the row once per pass
+    for rows, cols, dt, name in ((4096, 50304, bf, "bf16"), (2048, 128256, bf, "bf16"), (2048, 50304, f32, "f32"), (4096, 50257, bf, "bf16"),
+                                 (1024, 128256, f32, "f32")):
         t = rnd((rows, cols), dt, 3.0)
         run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
         run(f"logsoftmax(x*s)_{name}_{rows}x{cols}", P(t).op("mul", imm=0.5).row("logsoftmax").finish(torch))
