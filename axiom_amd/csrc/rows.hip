@@ -16,10 +16,10 @@
 #include <mutex>
 #include <string>
 
-// Partial sums of axhip_fused_full_reduce_noalloc: one float per stage-1 block (2048 blocks at most, 8 KiB).  Every
+// Partial sums of axhip_fused_full_reduce_noalloc: one float per stage-1 block or row (16640 at most, 65 KiB).  Every
 // device the library runs on holds its own copy until the process ends.  In host code this name is only a handle
 // for hipGetSymbolAddress; kernels and copies take the per-device address kept in g_scratch_ptr.
-static __device__ __align__(256) float scratch[2048];
+static __device__ __align__(256) float scratch[16640];
 
 namespace axhip {
 
@@ -398,9 +398,11 @@ __global__ __launch_bounds__(THREADS) void elementwise_kernel(const AxhipRowsPro
     }
 }
 
-// Chain + reduction over every element: stage 1 leaves one partial per block in
+// Chain + reduction over every element: stage 1 leaves one partial per block (or, on the row kernels, per row) in
 // the workspace, stage 2 (one block) folds the partials.
-constexpr int FULL_RED_BLOCKS = 2048;
+constexpr int FULL_RED_BLOCKS = 2048;      // blocks of the generic stage 1
+constexpr int FULL_RED_ROWS = 16384;       // rows of a flat array handed to a row-reduction kernel
+constexpr int FULL_RED_PARTIALS = FULL_RED_ROWS + 256; // capacity of the workspace, in floats (the rows plus the blocks of a remainder)
 
 template <int THREADS, int E>
 __global__ __launch_bounds__(THREADS) void full_reduce_stage1(const AxhipRowsProgram P, float *partials) {
@@ -433,6 +435,7 @@ __global__ __launch_bounds__(THREADS) void full_reduce_stage2(const float *parti
                                                               void *out, int out_dtype) {
     __shared__ float lds[THREADS / WAVE];
     float acc = reduce == AXHIP_RED_MAX ? NEG_INF : reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+#pragma unroll 4
     for (int i = threadIdx.x; i < n; i += THREADS) {
         float x = partials[i];
         acc = reduce == AXHIP_RED_MAX ? fmaxf(acc, x) : reduce == AXHIP_RED_MIN ? fminf(acc, x) : acc + x;
@@ -634,8 +637,68 @@ int check_full_reduce_program(const AxhipRowsProgram *program, const char *who) 
     return AXHIP_OK;
 }
 
-// stage 1 leaves `blocks` partials in `partials` (FULL_RED_BLOCKS floats), stage 2 reads exactly those
+// Large aligned arrays under chains without per-column or per-row operands are one flat array: seen as rows of 512 or
+// 2048 16-byte chunks it goes through the built-in row-reduction kernel of that plan, one partial per row (81-87 % of
+// the HBM peak where the generic stage 1 -- one chunk in flight per thread, a division per chunk -- reaches 30-60 %).
+// What is left behind the last whole row (less than a row) takes the generic stage 1, one partial per block.
+// Only kernels that are built into the library: nothing is compiled here, so the no-allocation entry point can share
+// the route.  Returns the number of partials written, 0 when the route does not apply.
+int full_reduce_on_row_kernels(const AxhipRowsProgram &P, float *partials, hipStream_t s, int *rc) {
+    *rc = AXHIP_OK;
+    const int64_t count = P.rows * P.cols;
+    if (!aligned_to(P.input, 16)) return 0;
+    bool wide = P.input_dtype == AXHIP_DTYPE_F32;
+    for (int i = 0; i < P.n_pre; ++i) {
+        if (!is_binary_op(P.pre[i].op) || P.pre[i].imm_kind == AXHIP_BK_IMM) continue;
+        const AxhipOperand &o = P.operands[P.pre[i].operand];
+        if (o.kind == AXHIP_BK_ROWVEC || o.kind == AXHIP_BK_COLVEC) return 0;
+        if (o.kind == AXHIP_BK_FULL) {
+            if (!aligned_to(o.ptr, 16)) return 0;
+            if (o.dtype == AXHIP_DTYPE_F32) wide = true;
+        }
+    }
+    const int e = wide ? 4 : 8;
+    const int64_t nchunk = count / e;
+    if (nchunk < 512 * 256) return 0; // (2 MiB: below that the generic kernel's launch is what counts)
+    const int64_t row_chunks = nchunk >= int64_t(2048) * 512 ? 2048 : 512;
+    const int64_t rows = nchunk / row_chunks;
+    if (rows > FULL_RED_ROWS) return 0;
+    AxhipRowsProgram Q = P;
+    Q.rows = rows;
+    Q.cols = row_chunks * e;
+    Q.reduce = P.reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : P.reduce;
+    Q.output = partials;
+    Q.output_dtype = AXHIP_DTYPE_F32;
+    if (!rows_prog_dispatch(Q, s, true, nullptr, 0, rc, /*builtin_only=*/true)) return 0;
+    if (*rc) return 0;
+    int written = static_cast<int>(rows);
+    const int64_t done = rows * Q.cols, rest = count - done;
+    if (rest > 0) {
+        AxhipRowsProgram R = P;
+        R.rows = 1;
+        R.cols = rest;
+        R.input = static_cast<const char *>(P.input) + done * dtype_size(P.input_dtype);
+        for (int i = 0; i < R.n_operands; ++i)
+            if (R.operands[i].kind == AXHIP_BK_FULL) R.operands[i].ptr = static_cast<const char *>(P.operands[i].ptr) + done * dtype_size(P.operands[i].dtype);
+        const int blocks = static_cast<int>((rest + 255) / 256); // rest < 2048 * 8 elements: at most 64 blocks
+        hipLaunchKernelGGL((full_reduce_stage1<256, 1>), dim3(blocks), dim3(256), 0, s, R, partials + written);
+        written += blocks;
+    }
+    return written;
+}
+
+// stage 1 leaves its partials in `partials` (FULL_RED_PARTIALS floats), stage 2 reads exactly those
 int launch_full_reduce(const AxhipRowsProgram &P, float *partials, hipStream_t s) {
+    int rc = AXHIP_OK;
+    const int on_rows = full_reduce_on_row_kernels(P, partials, s, &rc);
+    if (rc) return rc;
+    if (on_rows > 0) {
+        AXHIP_CHECK_HIP(hipGetLastError());
+        hipLaunchKernelGGL((full_reduce_stage2<1024>), dim3(1), dim3(1024), 0, s, partials, on_rows, P.reduce,
+                           1.0f / static_cast<float>(P.rows * P.cols), P.output, P.output_dtype);
+        AXHIP_CHECK_HIP(hipGetLastError());
+        return AXHIP_OK;
+    }
     AxhipRowsProgram Q = P;
     Q.reduce = AXHIP_RED_SUM; // only used by pick_vector_width to skip the output alignment test
     const int e = pick_vector_width(Q);
@@ -741,7 +804,7 @@ int axhip_fused_rows_prepare(const AxhipRowsProgram *program) {
     return AXHIP_OK;
 }
 
-size_t axhip_full_reduce_workspace_bytes(void) { return FULL_RED_BLOCKS * sizeof(float); }
+size_t axhip_full_reduce_workspace_bytes(void) { return FULL_RED_PARTIALS * sizeof(float); }
 
 int axhip_fused_full_reduce(const AxhipRowsProgram *program, void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_full_reduce_program(program, "axhip_fused_full_reduce");

@@ -193,7 +193,7 @@ bool rows_prog_compile_only(const AxhipRowsProgram &P, std::string *label, std::
     return r == HIPRTC_SUCCESS;
 }
 
-bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, char *name, size_t name_len, int *rc) {
+bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, char *name, size_t name_len, int *rc, bool builtin_only) {
     if (rc) *rc = AXHIP_OK;
     if (P.rows <= 0 || P.cols <= 0 || P.rows >= (int64_t(1) << 31)) return false;
     std::shared_ptr<Kernel> kernel;
@@ -203,6 +203,7 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
         std::lock_guard<std::mutex> lock(g_mutex);
         Entry *e = find_or_make_entry(P);
         if (!e->eligible) return false;
+        if (builtin_only && !e->is_builtin) return false; // (a caller that must not compile: the no-allocation reduction)
         // the tight plan's kernel, compiled on first launch -- or, with run-time compilation off or failed, the
         // looser built-in plan when there is one, else the interpreter
         bool use_alt = false;

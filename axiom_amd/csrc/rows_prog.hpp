@@ -12,7 +12,7 @@ namespace axhip {
 // one compiled through hipRTC when the program is first launched.  Fills `name` (when non-NULL) and launches when
 // `launch` is set; *rc receives the launch's error code.  Returns false when the interpreter has to take the
 // program (it does not qualify, or run-time compilation is off or failed).
-bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, char *name, size_t name_len, int *rc);
+bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, char *name, size_t name_len, int *rc, bool builtin_only = false);
 
 // Compiles the program's kernel through hipRTC for gfx950 without loading it (needs no device): the check that the
 // generator's text is valid for a program shape.

@@ -220,10 +220,11 @@ int axhip_fused_full_reduce(const AxhipRowsProgram *program_host, void *workspac
  * bring a workspace: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.
  * Same program, same kernels and the same result, bit for bit; the partial
- * sums live in an 8 KiB array inside the library's device image (one copy on
+ * sums live in a 65 KiB array inside the library's device image (one copy on
  * every device the library runs on, held until the process ends), whose
  * address is resolved when axhip_init runs on the device.  The call itself
- * performs no hipMalloc / hipFree and calls no allocating routine.
+ * performs no hipMalloc / hipFree, calls no allocating routine and compiles
+ * nothing (only kernels that are built into the library serve it).
  * Limits: rows * cols <= axhip_full_reduce_noalloc_max_elements() (2^40),
  * larger inputs return AXHIP_ERR_UNSUPPORTED.  All calls on one device share
  * that one array: two calls that overlap in time on the same device (different

@@ -110,6 +110,47 @@ def test_reduce_known_answers_on_gpu():
     assert gh.Rows(x, F32).run_full_reduce("min")[0] == x.min()
 
 
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_full_reductions_over_flat_and_row_dependent_chains(dt):
+    """A reduction over every element.  Chains of full-size, one-element and immediate operands over aligned arrays
+    are reduced as one flat array (16-byte chunks whatever the row length, the elements behind the last whole chunk
+    one by one); a per-column or per-row operand, or an array that starts inside a 16-byte block, keeps the
+    row-and-column form.  Sum, mean, maximum and minimum against float64."""
+    g = axo.PCG64(500 + dt)
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    for rows, cols in ((1, 5), (7, 3), (1, 13), (9, 1001), (300, 4097), (64, 2048), (2048, 4096), (3, 1 << 20)):
+        x, y = store(g.normal((rows, cols))), store(g.uniform((rows, cols), 0.5, 1.5))
+        xf, yf = wide(x), wide(y)
+        yw = g.uniform((rows, cols), 0.5, 1.5).astype(np.float32)  # an fp32 operand beside 16-bit data: 4-element chunks
+        rv, cv, sc = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((rows,), 0.5, 1.5)), store(g.uniform((1,), 0.5, 1.5))
+        n = rows * cols
+        cases = [
+            (lambda p: p, "sum", xf.sum()), (lambda p: p, "mean", xf.mean()), (lambda p: p, "max", xf.max()), (lambda p: p, "min", xf.min()),
+            (lambda p: p.unary("abs"), "max", np.abs(xf).max()),
+            (lambda p: p.binary("mul", y), "sum", (xf * yf).sum()),
+            (lambda p: p.imm("mul", 0.5).binary("add", yw, "full", F32).unary("square"), "mean", ((xf * 0.5 + yw) ** 2).mean()),
+            (lambda p: p.binary("sub", sc, "scalar").unary("relu"), "sum", np.maximum(xf - wide(sc), 0).sum()),
+            (lambda p: p.binary("mul", rv, "rowvec"), "sum", (xf * wide(rv)).sum()),
+            (lambda p: p.binary("add", cv, "colvec").unary("abs"), "min", np.abs(xf + wide(cv)[:, None]).min()),
+        ]
+        for build, red, want in cases:
+            got = float(build(gh.Rows(x, dt, F32)).run_full_reduce(red)[0])
+            if red in ("max", "min"):
+                assert abs(got - want) <= 1e-6 * abs(want), (rows, cols, red, got, want)
+            else:
+                scale = np.abs(xf).sum() * 3 if red == "sum" else np.abs(xf).mean() * 3
+                assert abs(got - want) <= 2e-6 * max(scale, 1.0) * (1 if red == "sum" else 4), (rows, cols, red, got, want)
+        # the same array from one element into a larger buffer: not 16-byte aligned
+        if n >= 2:
+            p = gh.Rows(x.reshape(-1)[1:].reshape(1, n - 1), dt, F32)
+            pad = gh.to_dev(x.reshape(-1))
+            p.keep.append(pad)
+            p.p.input = pad.data_ptr() + (4 if dt == F32 else 2)
+            got = float(p.run_full_reduce("sum")[0])
+            assert abs(got - xf.reshape(-1)[1:].sum()) <= 2e-6 * max(np.abs(xf).sum() * 3, 1.0), (rows, cols)
+
+
 @pytest.mark.parametrize("rows,cols", [(256, 512), (16, 8192), (3, 100)])
 def test_c2_chain_softmax_then_row_sum(rows, cols):
     """softmax((relu(a)+1)*b, -1).sum(1) in ONE launch; plus the intermediate softmax."""

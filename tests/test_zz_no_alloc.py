@@ -30,8 +30,8 @@ def both_ways(rows: gh.Rows, reduce: str):
 
 def test_noalloc_full_reduce_matches_workspace_entry_point_on_two_calls_in_a_row():
     g = axo.PCG64(20240607)
-    big = g.normal((4096, 1024))     # 2048 stage-1 blocks: every partial slot is written
-    small = g.normal((3, 40))        # one block: 2047 slots keep the first call's partials
+    big = g.normal((4096, 1024))     # 16 MiB: 512 rows of 2048 chunks on the row-reduction kernel, a partial each
+    small = g.normal((3, 40))        # one block of the generic kernel: the other slots keep the first call's partials
     for x, reduce in ((big, "sum"), (small, "sum"), (big, "max"), (small, "min"), (small, "mean")):
         want, got = both_ways(gh.Rows(x, F32).unary("square") if reduce in ("sum", "mean") else gh.Rows(x, F32), reduce)
         assert got.view(np.uint32)[0] == want.view(np.uint32)[0], (x.shape, reduce, got, want)
