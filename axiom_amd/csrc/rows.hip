@@ -398,6 +398,59 @@ __global__ __launch_bounds__(THREADS) void elementwise_kernel(const AxhipRowsPro
     }
 }
 
+// The same for arrays whose row length no vector divides (cols >= E, every full-size stream 16-byte aligned): the
+// array is walked as one flat run of E-element chunks, which may straddle two rows -- a full-size operand does not
+// care, a per-column or per-row operand is picked element by element where the chunk crosses a row end (and with one
+// unaligned vector load where it does not).  The n % E elements behind the last whole chunk go one by one.
+template <int THREADS, int E>
+__global__ __launch_bounds__(THREADS) void elementwise_flat_kernel(const AxhipRowsProgram P, const bool streaming) {
+    const int64_t cols = P.cols;
+    const int64_t n = P.rows * cols;
+    const int64_t nchunk = n / E;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * THREADS;
+    const int n_ops = P.n_pre + P.n_post;
+    for (int64_t c = static_cast<int64_t>(blockIdx.x) * THREADS + threadIdx.x; c < nchunk; c += stride) {
+        const int64_t flat = c * E;
+        const int64_t row = flat / cols, col = flat - row * cols;
+        const int64_t at[1] = {flat};
+        const bool ok[1] = {true};
+        float v[1][E];
+        load_vec<E>(P.input, P.input_dtype, flat, v[0]);
+        for (int i = 0; i < n_ops; ++i) {
+            const AxhipChainOp &op = i < P.n_pre ? P.pre[i] : P.post[i - P.n_pre];
+            const bool by_position = is_binary_op(op.op) && op.imm_kind != AXHIP_BK_IMM &&
+                                     (P.operands[op.operand].kind == AXHIP_BK_ROWVEC || P.operands[op.operand].kind == AXHIP_BK_COLVEC);
+            if (!by_position) {
+                apply_op<1, E>(op, P, v, 0, at, ok); // row 0, "column" = flat index: what a full-size operand's address is computed from
+                continue;
+            }
+            const AxhipOperand &o = P.operands[op.operand];
+            float w[E];
+            if (o.kind == AXHIP_BK_ROWVEC && col + E <= cols) {
+                load_vec<E, true>(o.ptr, o.dtype, col, w);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const bool next = col + e >= cols; // (cols >= E: a chunk crosses at most one row end)
+                    w[e] = load_any(o.ptr, o.dtype, o.kind == AXHIP_BK_ROWVEC ? col + e - (next ? cols : 0) : row + (next ? 1 : 0));
+                }
+            }
+            apply_binary_tile<1, E, true>(op.op, v, [&](int, int e) { return w[e]; });
+        }
+        store_vec<E>(P.output, P.output_dtype, flat, v[0], streaming);
+    }
+    const int64_t flat = nchunk * E + threadIdx.x;
+    if (blockIdx.x == 0 && flat < n) {
+        const int64_t row = flat / cols;
+        const int64_t col0[1] = {flat - row * cols};
+        const bool ok[1] = {true};
+        float v[1][1];
+        v[0][0] = load_any(P.input, P.input_dtype, flat);
+        for (int i = 0; i < n_ops; ++i) apply_op<1, 1>(i < P.n_pre ? P.pre[i] : P.post[i - P.n_pre], P, v, row, col0, ok);
+        store_any(P.output, P.output_dtype, flat, v[0][0]);
+    }
+}
+
 // Chain + reduction over every element: stage 1 leaves one partial per block (or, on the row kernels, per row) in
 // the workspace, stage 2 (one block) folds the partials.
 constexpr int FULL_RED_BLOCKS = 2048;      // blocks of the generic stage 1
@@ -492,6 +545,20 @@ int pick_vector_width(const AxhipRowsProgram &P) {
     return 1;
 }
 
+// Vector width for walking an elementwise program's arrays as one flat run (0: not possible): every full-size stream
+// 16-byte aligned, rows of at least one chunk.
+int flat_vector_width(const AxhipRowsProgram &P) {
+    bool wide = P.input_dtype == AXHIP_DTYPE_F32 || P.output_dtype == AXHIP_DTYPE_F32;
+    if (!aligned_to(P.input, 16) || !aligned_to(P.output, 16)) return 0;
+    for (int i = 0; i < P.n_operands; ++i) {
+        if (P.operands[i].kind != AXHIP_BK_FULL) continue;
+        if (!aligned_to(P.operands[i].ptr, 16)) return 0;
+        if (P.operands[i].dtype == AXHIP_DTYPE_F32) wide = true;
+    }
+    const int e = wide ? 4 : 8;
+    return P.cols >= e ? e : 0;
+}
+
 int validate_program(const AxhipRowsProgram &P, const char *who) {
     AXHIP_REQUIRE(P.rows >= 0 && P.cols >= 0, AXHIP_ERR_INVALID_ARG, "%s: negative extent", who);
     AXHIP_REQUIRE(valid_dtype(P.input_dtype) && valid_dtype(P.output_dtype), AXHIP_ERR_INVALID_ARG, "%s: bad dtype", who);
@@ -516,7 +583,7 @@ int validate_program(const AxhipRowsProgram &P, const char *who) {
 }
 
 struct RowsPlan {
-    enum Kind { EMPTY, ELEMENTWISE, RESIDENT, STREAMED } kind;
+    enum Kind { EMPTY, ELEMENTWISE, ELEMENTWISE_FLAT, RESIDENT, STREAMED } kind;
     int e, it, group, threads;
     bool ragged; // resident plan on rows that are not whole, aligned vectors: unaligned accesses, element-wise last chunk
     char name[64];
@@ -533,6 +600,14 @@ RowsPlan plan_rows(const AxhipRowsProgram &P) {
     if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) {
         pl.kind = RowsPlan::ELEMENTWISE;
         pl.threads = 256;
+        // a row length no vector divides, aligned arrays: one flat run of chunks instead of element by element
+        const int flat_e = flat_vector_width(P);
+        if (pl.e == 1 && flat_e > 1) {
+            pl.kind = RowsPlan::ELEMENTWISE_FLAT;
+            pl.e = flat_e;
+            snprintf(pl.name, sizeof(pl.name), "elementwise_flat_e%d", pl.e);
+            return pl;
+        }
         snprintf(pl.name, sizeof(pl.name), "elementwise_e%d", pl.e);
         return pl;
     }
@@ -609,6 +684,15 @@ int launch_plan_e(const AxhipRowsProgram &P, const RowsPlan &pl, hipStream_t s) 
         const int64_t blocks = std::min<int64_t>((nchunk + 255) / 256, 256 * 32);
         const bool streaming = P.rows * P.cols * static_cast<int64_t>(dtype_size(P.output_dtype)) >= STREAMING_OUTPUT_BYTES;
         hipLaunchKernelGGL((elementwise_kernel<256, E>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, P, streaming);
+        return AXHIP_OK;
+    }
+    case RowsPlan::ELEMENTWISE_FLAT: {
+        if constexpr (E > 1) {
+            const int64_t nchunk = P.rows * P.cols / E;
+            const int64_t blocks = std::max<int64_t>(1, std::min<int64_t>((nchunk + 255) / 256, 256 * 32));
+            const bool streaming = P.rows * P.cols * static_cast<int64_t>(dtype_size(P.output_dtype)) >= STREAMING_OUTPUT_BYTES;
+            hipLaunchKernelGGL((elementwise_flat_kernel<256, E>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, P, streaming);
+        }
         return AXHIP_OK;
     }
     case RowsPlan::RESIDENT:

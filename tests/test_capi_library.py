@@ -58,7 +58,9 @@ def test_version_and_kernel_selection_without_device():
     assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"rows_resident_g256_it2_e8"
     r.cols = 1 << 20
     assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"rows_streamed_e8"
-    r.cols, r.row_op = 37, 0
+    r.cols, r.row_op = 37, 0  # no vector divides 37: the aligned array is walked as one flat run of 8-element chunks
+    assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"elementwise_flat_e8"
+    r.cols = 5  # rows shorter than a chunk: element by element
     assert lib.axhip_fused_rows_kernel_name(C.byref(r)) == b"elementwise_e1"
 
 

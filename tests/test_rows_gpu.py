@@ -111,6 +111,50 @@ def test_reduce_known_answers_on_gpu():
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_elementwise_chains_over_rows_no_vector_divides(dt):
+    """Flat chains (no row operation, no reduction) over row lengths that no 16-byte vector divides walk the arrays as
+    one run of chunks: a chunk may straddle two rows, so per-column and per-row operands are picked by position.
+    Exact where the arithmetic is (relu, add, mul in fp32 from the same inputs), to a 16-bit step otherwise; rows
+    shorter than a chunk and arrays that start inside a 16-byte block keep the element-wise kernel."""
+    g = axo.PCG64(700 + dt)
+    e = 4 if dt == F32 else 8
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_f32(t, dt))
+    rnd = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_f32(axo.to_bits(t, dt), dt))  # the result's rounding
+    for rows, cols in ((9, 1001), (300, 4097), (4, e + 1), (1, 2 * e + 3), (5, e - 1), (33, 50257)):
+        x, y = store(g.normal((rows, cols))), store(g.normal((rows, cols)))
+        rv, cv, sc = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((rows,), 0.5, 1.5)), store(g.uniform((1,), 0.5, 1.5))
+        xf, yf, rf, cf, sf = wide(x), wide(y), wide(rv), wide(cv)[:, None], wide(sc)
+        name = f"elementwise_flat_e{e}" if cols >= e else "elementwise_e1"
+        p = gh.Rows(x, dt).unary("relu").binary("mul", rv, "rowvec").binary("add", y)
+        got = wide(p.run())
+        assert p.kernel_name() == name, p.kernel_name()
+        assert np.array_equal(got, rnd(np.maximum(xf, 0) * rf + yf)), (rows, cols)
+        p = gh.Rows(x, dt).binary("add", cv, "colvec").binary("sub", sc, "scalar").imm("mul", 0.5)
+        got = wide(p.run())
+        assert np.array_equal(got, rnd(((xf + cf) - sf) * np.float32(0.5))), (rows, cols)
+        p = gh.Rows(x, dt).unary("silu").binary("mul", y)
+        got = wide(p.run()).astype(np.float64)
+        want = xf.astype(np.float64) / (1 + np.exp(-xf.astype(np.float64))) * yf
+        step = 1e-6 if dt == F32 else (2.0 ** -8 if dt == BF16 else 2.0 ** -11)  # half a unit in the last place of the result, relative
+        assert np.all(np.abs(got - want) <= step * np.maximum(np.abs(want), 1e-2) + 1e-6), (rows, cols)
+        if dt != F32:  # widening cast: fp32 result, 4-element chunks
+            p = gh.Rows(x, dt, F32).binary("mul", rv, "rowvec")
+            got = p.run()
+            assert p.kernel_name() == ("elementwise_flat_e4" if cols >= 4 else "elementwise_e1"), p.kernel_name()
+            assert np.array_equal(got, xf * rf), (rows, cols)
+    # an input that starts one element into its buffer: element by element as before
+    x = store(g.normal((6, 1001)))
+    p = gh.Rows(x, dt).unary("relu")
+    pad = gh.to_dev(np.concatenate([np.zeros(1, x.dtype), x.ravel()]))
+    p.keep.append(pad)
+    p.p.input = pad.data_ptr() + (4 if dt == F32 else 2)
+    got = wide(p.run())
+    assert p.kernel_name() == "elementwise_e1", p.kernel_name()
+    assert np.array_equal(got, np.maximum(wide(x), 0))
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_full_reductions_over_flat_and_row_dependent_chains(dt):
     """A reduction over every element.  Chains of full-size, one-element and immediate operands over aligned arrays
     are reduced as one flat array (16-byte chunks whatever the row length, the elements behind the last whole chunk
