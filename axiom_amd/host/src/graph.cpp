@@ -180,6 +180,32 @@ Tensor GraphRegistry::create_lazy_binary(ops::OpType op, const Tensor &lhs, cons
 
 Tensor GraphRegistry::create_lazy_reduction(ops::OpType op, const Tensor &input, const std::vector<int> &axes, bool keep_dims) {
     require_gpu(pick_device({&input}), op);
+    // The device reduces over the last axis or over everything.  Any other set of axes is brought there first: the
+    // kept axes in front, the reduced ones behind them and folded into one (a transposed view that the planner
+    // gathers into a contiguous array), then the result takes the shape the caller asked for.
+    {
+        const int nd = static_cast<int>(input.ndim());
+        const Shape wanted = infer_reduction_shape(input.shape(), axes, keep_dims); // validates the axes
+        std::vector<bool> red(static_cast<size_t>(nd), axes.empty());
+        for (int a : axes) red[static_cast<size_t>(ShapeUtils::normalize_axis(a, nd))] = true;
+        std::vector<int> kept_axes, red_axes;
+        size_t kept = 1, folded = 1;
+        for (int i = 0; i < nd; ++i) {
+            (red[static_cast<size_t>(i)] ? red_axes : kept_axes).push_back(i);
+            (red[static_cast<size_t>(i)] ? folded : kept) *= input.shape()[static_cast<size_t>(i)];
+        }
+        const bool all = kept_axes.empty() || kept == 1;
+        const bool last_only = red_axes.size() == 1 && red_axes[0] == nd - 1;
+        if (!all && !last_only && !red_axes.empty() && kept * folded > 0) {
+            std::vector<int> order = kept_axes;
+            order.insert(order.end(), red_axes.begin(), red_axes.end());
+            bool identity = true;
+            for (int i = 0; i < nd; ++i) identity = identity && order[static_cast<size_t>(i)] == i;
+            const Tensor moved = identity ? input : create_lazy_transpose(input, order);
+            const Tensor rows = create_lazy_reshape(moved, Shape{kept, folded});
+            return create_lazy_reshape(create_lazy_reduction(op, rows, {1}, false), wanted);
+        }
+    }
     auto n = std::make_shared<GraphNode>();
     n->op_type = op;
     n->output_shape = infer_reduction_shape(input.shape(), axes, keep_dims); // validates the axes
@@ -206,6 +232,13 @@ Tensor GraphRegistry::create_lazy_matmul(const Tensor &a, const Tensor &b, bool 
 Tensor GraphRegistry::create_lazy_softmax(ops::OpType op, const Tensor &input, int axis) {
     require_gpu(pick_device({&input}), op);
     const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
+    // over another axis than the last: that axis and the last one change places, before and after
+    if (a != static_cast<int>(input.ndim()) - 1) {
+        std::vector<int> swap(input.ndim());
+        for (size_t i = 0; i < swap.size(); ++i) swap[i] = static_cast<int>(i);
+        std::swap(swap[static_cast<size_t>(a)], swap.back());
+        return create_lazy_transpose(create_lazy_softmax(op, create_lazy_transpose(input, swap), -1), swap);
+    }
     auto n = std::make_shared<GraphNode>();
     n->op_type = op;
     n->inputs = {input_node(input)};

@@ -272,7 +272,15 @@ GPU_TEST(Normalization, KnownAnswers) {
     }
     for (size_t i = 0; i < sm.size(); ++i) EXPECT_NEAR(lsm[i], std::log(sm[i]), 1e-4);
     EXPECT_NEAR(ops::gelu(Tensor::zeros({4}, DType::Float32, Device::GPU)).cpu().item<float>({0}), 0.0f, 0); // :310-334
-    EXPECT_THROW(ops::softmax(a.gpu(), 0).cpu(), RuntimeError); // only the last axis is on the GPU path
+    { // over the first axis: columns sum to one (the axis and the last one change places around the row kernel)
+        auto s0 = host_floats(ops::softmax(a.gpu(), 0));
+        const size_t R = a.shape()[0], C = a.shape()[1];
+        for (size_t j = 0; j < C; ++j) {
+            double t = 0;
+            for (size_t i = 0; i < R; ++i) t += s0[i * C + j];
+            EXPECT_NEAR(t, 1.0, 1e-5);
+        }
+    }
 }
 
 // Rows whose length no 16-byte vector divides (Whisper's 1500 frames, an odd vocabulary) take the specialised
@@ -296,6 +304,76 @@ GPU_TEST(FusedRows, OddRowLengthsRunOnTheRaggedKernels) {
         for (size_t j = 0; j < C; ++j) {
             EXPECT_NEAR(sm[i * C + j], std::exp(0.5 * x[i * C + j] - mx) / s, 1e-6);
             EXPECT_NEAR(ln[i * C + j], (x[i * C + j] - mean) / std::sqrt(var + 1e-5), 1e-4);
+        }
+    }
+}
+
+// Reductions and softmax over axes other than the last (tests/test_tensor_reductions.cpp: sum / mean / max along
+// each axis and along pairs of axes, keep_dims): the kept axes move to the front, the reduced ones fold into the last,
+// a row kernel reduces it.  Against double-precision loops on the host.
+GPU_TEST(CpuGpuParity, ReductionsAndSoftmaxOverAnyAxis) {
+    const Shape sh{5, 7, 6, 9};
+    auto a = axtest::randn(sh, 4141);
+    const float *x = a.typed_data<float>();
+    auto ga = a.gpu();
+    const size_t nd = sh.size();
+    size_t strides[4] = {7 * 6 * 9, 6 * 9, 9, 1};
+    const std::vector<std::vector<int>> axis_sets = {{0}, {1}, {2}, {3}, {0, 1}, {1, 3}, {0, 2, 3}, {-3}, {2, 0}, {0, 1, 2, 3}};
+    for (const auto &axes : axis_sets) {
+        bool red[4] = {false, false, false, false};
+        for (int ax : axes) red[(ax + 4) % 4] = true;
+        Shape kept_shape;
+        for (size_t i = 0; i < nd; ++i)
+            if (!red[i]) kept_shape.push_back(sh[i]);
+        size_t kept = 1, count = 1;
+        for (size_t i = 0; i < nd; ++i) (red[i] ? count : kept) *= sh[i];
+        std::vector<double> sum(kept, 0.0), mx(kept, -1e300);
+        for (size_t flat = 0; flat < a.size(); ++flat) {
+            size_t out = 0, rest = flat;
+            for (size_t i = 0; i < nd; ++i) {
+                const size_t idx = rest / strides[i];
+                rest %= strides[i];
+                if (!red[i]) out = out * sh[i] + idx;
+            }
+            sum[out] += x[flat];
+            mx[out] = std::max(mx[out], static_cast<double>(x[flat]));
+        }
+        auto gs = ops::sum(ga, axes, false), gm = ops::mean(ga, axes, true), gx = ops::max(ga, axes, false);
+        if (!kept_shape.empty()) EXPECT_EQ(gs.shape(), kept_shape); // (over every axis: one element, shaped as the all-axes reduction always was)
+        EXPECT_EQ(gm.ndim(), nd);
+        auto hs = host_floats(gs), hm = host_floats(gm), hx = host_floats(gx);
+        ASSERT_EQ(hs.size(), kept);
+        ASSERT_EQ(hm.size(), kept);
+        for (size_t i = 0; i < kept; ++i) {
+            EXPECT_NEAR(hs[i], sum[i], 1e-4);
+            EXPECT_NEAR(hm[i], sum[i] / static_cast<double>(count), 1e-5);
+            EXPECT_NEAR(hx[i], mx[i], 0);
+        }
+    }
+    // a chain below the reduction still fuses behind the gather: sum(relu(x) * 2, axis 1)
+    {
+        auto got = host_floats(ops::sum(ops::relu(ga) * 2.0f, {1}, false));
+        for (size_t i = 0; i < 5; ++i)
+            for (size_t k = 0; k < 6 * 9; ++k) {
+                double t = 0;
+                for (size_t j = 0; j < 7; ++j) t += 2.0 * std::max(0.0f, x[i * strides[0] + j * strides[1] + k]);
+                EXPECT_NEAR(got[i * 54 + k], t, 1e-4);
+            }
+    }
+    // softmax and log-softmax over each axis
+    for (int axis = 0; axis < 4; ++axis) {
+        auto sm = host_floats(ops::softmax(ga, axis)), lsm = host_floats(ops::log_softmax(ga, axis - 4));
+        ASSERT_EQ(sm.size(), a.size());
+        const size_t len = sh[static_cast<size_t>(axis)], st = strides[axis];
+        for (size_t flat = 0; flat < a.size(); ++flat) {
+            if ((flat / st) % len != 0) continue; // first element of each line along the axis
+            double m = -1e300, z = 0;
+            for (size_t k = 0; k < len; ++k) m = std::max(m, static_cast<double>(x[flat + k * st]));
+            for (size_t k = 0; k < len; ++k) z += std::exp(x[flat + k * st] - m);
+            for (size_t k = 0; k < len; ++k) {
+                EXPECT_NEAR(sm[flat + k * st], std::exp(x[flat + k * st] - m) / z, 1e-5);
+                EXPECT_NEAR(lsm[flat + k * st], x[flat + k * st] - m - std::log(z), 1e-4);
+            }
         }
     }
 }
@@ -346,7 +424,7 @@ GPU_TEST(CpuGpuParity, ElementwiseReductionsMatmul) { // tests/test_cpu_gpu_pari
     for (size_t i = 0; i < 63; ++i) EXPECT_NEAR(gmm[i], mm[i], 1e-4 + 1e-4 * std::fabs(mm[i]));
     auto gmt = host_floats(ops::matmul(m1.gpu(), m2.transpose({1, 0}).ascontiguousarray().gpu(), false, true));
     for (size_t i = 0; i < 63; ++i) EXPECT_NEAR(gmt[i], mm[i], 1e-4 + 1e-4 * std::fabs(mm[i]));
-    EXPECT_THROW(ops::sum(axtest::randn({3, 4, 5}, 1).gpu(), {1}).cpu(), RuntimeError); // middle-axis reduction: not on the path
+    EXPECT_EQ(ops::sum(axtest::randn({3, 4, 5}, 1).gpu(), {1}).shape(), Shape({3, 5})); // (ReductionsAndSoftmaxOverAnyAxis checks the values)
 }
 
 // ----------------------------------------------------------------- attention
