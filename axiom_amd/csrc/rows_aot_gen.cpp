@@ -152,13 +152,15 @@ int main(int argc, char **argv) {
     if (n_files <= 0) return 2;
     // a wavefront per row up to 512 chunks (1, 2, 4, 8 chunks per lane, and 3 / 5 / 6 for the row lengths between the
     // powers of two: 1280, 1536, 2560, 3072 ... columns of 16-bit data), a 256-thread block per row beyond
-    static const int plans[][2] = {{64, 1}, {64, 2}, {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}, {256, 3}, {256, 4}, {256, 8}};
+    // (4 to 32 lanes per row: short aligned rows, several to a wavefront)
+    static const int plans[][2] = {{4, 1}, {8, 1}, {16, 1}, {32, 1}, {64, 1}, {64, 2}, {64, 3}, {64, 4}, {64, 5}, {64, 6}, {64, 8}, {256, 3}, {256, 4}, {256, 8}};
     std::vector<RowsProgSpec> specs;
     std::set<std::string> seen;
     for (int dt : {AXHIP_DTYPE_F32, AXHIP_DTYPE_F16, AXHIP_DTYPE_BF16})
         for (const AxhipRowsProgram &p : shapes_of(dt))
             for (const auto &pl : plans)
                 for (bool ragged : {false, true}) {
+                    if (ragged && pl[0] < 64) continue;
                     RowsProgPlan plan;
                     rows_prog_plan_for(p, pl[0], pl[1], ragged, &plan, /*the built-in ragged kernels are those for equally aligned streams*/ ragged && rows_prog_grid_pays(p, pl[0], pl[1]));
                     RowsProgSpec s;

@@ -143,6 +143,20 @@ def test_ragged_rows_take_the_grid_form_when_every_stream_is_full_size_and_equal
     assert Prog(4096, 4096, BF16, misalign=2).row("softmax").name() == "rows_jit_softmax_bf16_g64_it9_grid"
 
 
+def test_short_aligned_rows_share_a_wavefront():
+    """Up to 32 chunks (256 16-bit or 128 fp32 columns): 4, 8, 16 or 32 lanes per row, one chunk each, several rows to
+    a wavefront; built in like the longer plans.  Odd lengths keep a wavefront per row."""
+    assert Prog(1 << 20, 64, BF16).row("softmax").name() == "rows_static_softmax_bf16_g8_it1"
+    assert Prog(1 << 20, 16, BF16).row("rmsnorm", 1).name() == "rows_static_rmsnorm_w_bf16_g4_it1"
+    assert Prog(1 << 20, 128, F16).row("layernorm", 2).op("gelu").name() == "rows_static_layernorm_gelu_wb_f16_g16_it1"
+    assert Prog(1 << 20, 128, F32).row("softmax").name() == "rows_static_softmax_f32_g32_it1"
+    assert Prog(1 << 20, 100, F32).row("softmax").name() == "rows_static_softmax_f32_g32_it1"  # 25 chunks: seven idle lanes per row
+    assert Prog(1 << 20, 256, BF16).op("square").reduce("mean").name() == "rows_static_square_reduce_sum_bf16_g32_it1"
+    assert Prog(1 << 20, 264, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1"  # 33 chunks
+    assert Prog(1 << 20, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1_ragged"
+    assert Prog(1 << 20, 96, BF16).op("mul", "colvec").op("tanh").row("softmax").name() == "rows_jit_mulc_tanh_softmax_bf16_g16_it1"
+
+
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     assert Prog(1024, 4096, F32).op("relu").op("mul", "full").name() == "elementwise_e4"  # no row op, no reduction
     assert Prog(4, 1000001, BF16).row("softmax").name() == "rows_streamed_e1"  # beyond 16384 chunks and not whole vectors
@@ -158,8 +172,9 @@ def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     lambda: Prog(4096, 5000, BF16).op("relu").op("max", imm=0.25).reduce("max"),
     lambda: Prog(64, 128256, F16).op("mul", imm=0.5).row("logsoftmax"),
     lambda: Prog(64, 128256, F32).op("mul", "rowvec").op("add", "full").row("logsoftmax").op("exp").reduce("sum"),
+    lambda: Prog(1 << 16, 96, BF16).op("mul", "colvec").op("add", "rowvec").row("layernorm", 2).op("silu"),
 ], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10", "raw_resident_it16",
-        "looped_row"])
+        "looped_row", "short_rows_16_lanes"])
 def test_generated_kernels_compile(build):
     prog = build()
     assert prog.name().startswith("rows_jit_"), prog.name()

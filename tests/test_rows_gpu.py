@@ -111,6 +111,48 @@ def test_reduce_known_answers_on_gpu():
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_short_rows_that_share_a_wavefront(dt):
+    """Aligned rows of up to 32 chunks run 4, 8, 16 or 32 lanes per row, several rows to a wavefront: every group size,
+    rows that fill their group and rows that leave lanes idle, row counts that leave a wavefront's (and a block's)
+    last set of rows partial, per-row and per-column operands, a reduction; guard words behind the output."""
+    g = axo.PCG64(900 + dt)
+    e = 4 if dt == F32 else 8
+    tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    tol = 1e-5 if dt == F32 else (2.0 ** -8 if dt == BF16 else 2.0 ** -10)
+    sentinel = np.float32(-77.0) if dt == F32 else np.uint16(0x7FC1)
+    for chunks, group in ((1, 4), (3, 4), (4, 4), (5, 8), (8, 8), (11, 16), (16, 16), (25, 32), (32, 32)):
+        cols = chunks * e
+        for rows in (1, 5, 64 // group * 4 + 1, 1000):
+            x = store(g.normal((rows, cols)) * 2)
+            xf = wide(x)
+            cv, rv = store(g.uniform((rows,), 0.5, 1.5)), store(g.uniform((cols,), 0.5, 1.5))
+            dst = gh.to_dev(np.full(rows * cols + 64, sentinel, x.dtype))
+            p = gh.Rows(x, dt).row_op("softmax")
+            p.keep.append(dst)
+            p.p.output, p.p.output_dtype = dst.data_ptr(), dt
+            assert p.kernel_name() == f"rows_static_softmax_{tag}_g{group}_it1", (cols, p.kernel_name())
+            gh.sync()
+            gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
+            gh.sync()
+            out = gh.to_host(dst, x.dtype)
+            assert np.all(out[rows * cols:] == sentinel), (rows, cols)
+            got = wide(out[:rows * cols].reshape(rows, cols))
+            ex = np.exp(xf - xf.max(-1, keepdims=True))
+            want = ex / ex.sum(-1, keepdims=True)
+            assert np.all(np.abs(got - want) <= tol * want + (2.0 ** -24 if dt == F16 else 1e-9)), (rows, cols)
+            # a per-row scale, a per-column weight, layer norm, then the row maximum
+            w, b = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((cols,), -0.5, 0.5))
+            p = gh.Rows(x, dt, F32).binary("mul", cv, "colvec").binary("add", rv, "rowvec").row_op("layernorm", 1e-5, w=w, b=b)
+            got = p.run(reduce="max").astype(np.float64).reshape(-1)
+            assert p.kernel_name().endswith(f"_g{group}_it1"), p.kernel_name()
+            t = xf * wide(cv)[:, None] + wide(rv)
+            n = (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * wide(w) + wide(b)
+            assert np.max(np.abs(got - n.max(-1))) < (1e-4 if dt == F32 else 1e-3), (rows, cols)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_elementwise_chains_over_rows_no_vector_divides(dt):
     """Flat chains (no row operation, no reduction) over row lengths that no 16-byte vector divides walk the arrays as
     one run of chunks: a chunk may straddle two rows, so per-column and per-row operands are picked by position.
