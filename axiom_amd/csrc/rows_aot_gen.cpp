@@ -160,7 +160,6 @@ int main(int argc, char **argv) {
         for (const AxhipRowsProgram &p : shapes_of(dt))
             for (const auto &pl : plans)
                 for (bool ragged : {false, true}) {
-                    if (ragged && pl[0] < 64) continue;
                     RowsProgPlan plan;
                     rows_prog_plan_for(p, pl[0], pl[1], ragged, &plan, /*the built-in ragged kernels are those for equally aligned streams*/ ragged && rows_prog_grid_pays(p, pl[0], pl[1]));
                     RowsProgSpec s;

@@ -265,6 +265,7 @@ bool rows_prog_grid_pays(const AxhipRowsProgram &P, int group, int it) {
     // their position in the row no longer matches their address) costs 5 to 20 % on the grid in rows of up to 512
     // threads (wavefront rows stage it in LDS once per block when the chunks start at the row's first element) --
     // 1024-thread rows gain even so: their unaligned form spills (layer norm over 50 257 fp32 columns: 404 -> 172 us).
+    if (group < 64) return true; // short rows: on the grid they share a wavefront, from their first element each takes one
     if (group * it <= 128) return false;
     if (group > 512) return true;
     auto rowvec = [&](int idx) { return idx >= 0 && idx < P.n_operands && P.operands[idx].kind == AXHIP_BK_ROWVEC; };
@@ -294,6 +295,8 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
     const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? rows_prog_chunk_elems(P) * it : 0);
     plan->min_waves = (held + (heavy ? 3 * it + 16 : 0) > 72 || it > 8) ? 2 : 4;
+    // short rows on the grid: every row has a shift of its own, so the next row's chunk offsets are not this row's
+    if (group < 64 && plan->grid) plan->pipe = false;
     // a 1024-thread block has 128 registers per thread whatever is asked for: no second set of raw words beyond that
     if (group == 1024 && held + (plan->pipe ? raw * it : 0) > 115) plan->pipe = false;
 }
@@ -307,7 +310,6 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) return false; // flat elementwise chains have a kernel of their own
     const int dt = P.input_dtype;
     const int e = rows_prog_chunk_elems(P);
-    if (P.cols < e) return false;
     bool ragged = P.cols % e != 0 || !aligned16(P.input) || (P.reduce == AXHIP_RED_NONE && !aligned16(P.output));
     bool same_size = P.reduce != AXHIP_RED_NONE || elem_size(P.output_dtype) == elem_size(dt);
     bool used[AXHIP_MAX_OPERANDS] = {};
@@ -332,7 +334,7 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     // When the input, the full-size operands and a full-size output sit at the same address modulo 16 (the usual case:
     // aligned allocations, a row length that is not a multiple of the chunk), the chunks follow memory's 16-byte grid:
     // every access aligned, a partial chunk at either end of a row, hence one chunk more than the row's own count.
-    bool grid = ragged && P.cols >= 2 * e;
+    bool grid = ragged;
     if (grid) {
         const uintptr_t a = reinterpret_cast<uintptr_t>(P.input) & 15u;
         if (P.reduce == AXHIP_RED_NONE && (reinterpret_cast<uintptr_t>(P.output) & 15u) != a) grid = false;
@@ -340,6 +342,7 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
             if (used[i] && P.operands[i].kind == AXHIP_BK_FULL && (reinterpret_cast<uintptr_t>(P.operands[i].ptr) & 15u) != a) grid = false;
     }
     if (grid && plan_rows(P, tight, ragged, true, plan) && rows_prog_grid_pays(P, plan->group, plan->it)) return true;
+    if (P.cols < e) return false; // (rows shorter than a chunk: on the grid or not at all)
     return plan_rows(P, tight, ragged, false, plan);
 }
 
@@ -353,11 +356,12 @@ bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, Ro
     // Short aligned rows (up to 32 chunks: 256 16-bit or 128 fp32 columns) share a wavefront: 4, 8, 16 or 32 lanes per
     // row, one chunk each, instead of a wavefront with most of its lanes idle (softmax over 64 16-bit columns ran at
     // 17 % of the HBM peak that way).  The build compiles these plans too.
-    if (!ragged && chunks <= 32) {
+    if ((!ragged || grid) && chunks <= 32) {
         const int g = chunks <= 4 ? 4 : chunks <= 8 ? 8 : chunks <= 16 ? 16 : 32;
-        rows_prog_plan_for(P, g, 1, false, plan, false);
+        rows_prog_plan_for(P, g, 1, ragged, plan, grid);
         return true;
     }
+    if (grid && P.cols < 2 * e) return false; // (longer plans on the grid count on a row's two ends lying in different chunks)
     if (!tight) {
         // the shapes the build compiles (rows_aot_gen.cpp): a wavefront per row with 1, 2, 3, 4, 5, 6 or 8 chunks per
         // lane, a 256-thread block per row with 3, 4 or 8 chunks per thread

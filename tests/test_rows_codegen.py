@@ -153,7 +153,15 @@ def test_short_aligned_rows_share_a_wavefront():
     assert Prog(1 << 20, 100, F32).row("softmax").name() == "rows_static_softmax_f32_g32_it1"  # 25 chunks: seven idle lanes per row
     assert Prog(1 << 20, 256, BF16).op("square").reduce("mean").name() == "rows_static_square_reduce_sum_bf16_g32_it1"
     assert Prog(1 << 20, 264, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1"  # 33 chunks
-    assert Prog(1 << 20, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1_ragged"
+    # odd lengths: the same on memory's 16-byte grid, a masked partial chunk at either end of every row
+    assert Prog(1 << 20, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g16_it1_grid"
+    assert Prog(1 << 20, 10, F32).row("logsoftmax").name() == "rows_static_logsoftmax_f32_g4_it1_grid"
+    assert Prog(1 << 20, 5, BF16).row("softmax").name() == "rows_static_softmax_bf16_g4_it1_grid"  # shorter than a chunk
+    assert Prog(1 << 20, 197, F16).row("layernorm", 2).name() == "rows_static_layernorm_wb_f16_g32_it1_grid"
+    assert Prog(1 << 20, 250, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1_ragged"  # 33 chunks on the grid
+    p = Prog(1 << 20, 77, BF16).row("softmax")
+    p.p.output += 2  # input and output at different addresses modulo 16: a wavefront per row, from the row's first element
+    assert p.name() == "rows_static_softmax_bf16_g64_it1_ragged"
     assert Prog(1 << 20, 96, BF16).op("mul", "colvec").op("tanh").row("softmax").name() == "rows_jit_mulc_tanh_softmax_bf16_g16_it1"
 
 

@@ -153,6 +153,57 @@ def test_short_rows_that_share_a_wavefront(dt):
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_short_rows_of_odd_length_share_a_wavefront_on_the_16_byte_grid(dt):
+    """Short rows whose length no vector divides (10 class logits, 77 or 197 tokens): the rows of a wavefront are
+    consecutive in memory, each on the 16-byte grid with a shift of its own, a masked partial chunk at either end
+    (two rows may share a 16-byte word: each stores its own elements only).  Lengths from one element to 32 grid
+    chunks, row counts that leave the last wavefront partial, from a base 3 elements past a boundary, with guard words
+    on both sides of the output; softmax against float64, a norm with weight, bias and per-row operand, a reduction."""
+    g = axo.PCG64(1300 + dt)
+    e, es = (4, 4) if dt == F32 else (8, 2)
+    tag = {F32: "f32", BF16: "bf16", F16: "f16"}[dt]
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    tol = 1e-5 if dt == F32 else (2.0 ** -8 if dt == BF16 else 2.0 ** -10)
+    sentinel = np.float32(-77.0) if dt == F32 else np.uint16(0x7FC1)
+    off, pad = 3, 64
+    for cols in (1, 3, e - 1, e + 1, 10, 3 * e + 1, 77, 15 * e - 1, 197 if dt != F32 else 101, 31 * e - 6):
+        chunks = (cols + 2 * e - 2) // e
+        group = 4 if chunks <= 4 else 8 if chunks <= 8 else 16 if chunks <= 16 else 32
+        for rows in (1, 7, 64 // group * 4 + 3, 501):
+            x = store(g.normal((rows, cols)) * 2)
+            xf = wide(x)
+            src = gh.to_dev(np.concatenate([np.full(off, sentinel, x.dtype), x.ravel()]))
+            dst = gh.to_dev(np.full(pad + off + rows * cols + pad, sentinel, x.dtype))
+            p = gh.Rows(x[:1], dt).row_op("softmax")
+            p.keep += [src, dst]
+            p.p.rows, p.p.input = rows, src.data_ptr() + off * es
+            p.p.output, p.p.output_dtype = dst.data_ptr() + (pad + off) * es, dt
+            assert p.kernel_name() == f"rows_static_softmax_{tag}_g{group}_it1_grid", (cols, p.kernel_name())
+            gh.sync()
+            gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
+            gh.sync()
+            out = gh.to_host(dst, x.dtype)
+            assert np.all(out[:pad + off] == sentinel) and np.all(out[pad + off + rows * cols:] == sentinel), (rows, cols)
+            got = wide(out[pad + off:pad + off + rows * cols].reshape(rows, cols))
+            ex = np.exp(xf - xf.max(-1, keepdims=True))
+            want = ex / ex.sum(-1, keepdims=True)
+            assert np.all(np.abs(got - want) <= tol * want + (2.0 ** -24 if dt == F16 else 1e-9)), (rows, cols)
+            if cols < 2:
+                continue
+            w, b, cv = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((cols,), -0.5, 0.5)), store(g.uniform((rows,), 0.5, 1.5))
+            p = gh.Rows(x, dt).binary("mul", cv, "colvec").row_op("layernorm", 1e-5, w=w, b=b)
+            got = wide(p.run())
+            assert p.kernel_name().endswith(f"_g{group}_it1_grid"), p.kernel_name()
+            t = xf * wide(cv)[:, None]
+            n = (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * wide(w) + wide(b)
+            assert np.max(np.abs(got - n)) < (2e-4 if dt == F32 else 4e-2), (rows, cols, np.max(np.abs(got - n)))
+            p = gh.Rows(x, dt, F32).unary("abs")
+            got = p.run(reduce="max").astype(np.float64).reshape(-1)
+            assert np.array_equal(got, np.abs(xf).max(-1)), (rows, cols)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_elementwise_chains_over_rows_no_vector_divides(dt):
     """Flat chains (no row operation, no reduction) over row lengths that no 16-byte vector divides walk the arrays as
     one run of chunks: a chunk may straddle two rows, so per-column and per-row operands are picked by position.
@@ -635,13 +686,16 @@ def test_rows_of_odd_length_on_the_ragged_plans(dt):
         tol = 1e-4 if dt == F32 else 2e-2
         p = gh.Rows(xs, dt).binary("add", ys).row_op("softmax")
         got = out(p.run())
-        assert p.kernel_name().endswith("_grid" if cols // (4 if dt == F32 else 8) > 128 else "_ragged"), p.kernel_name()  # (the grid form from 3 chunks per lane on)
+        ce = 4 if dt == F32 else 8
+        short = (cols + 2 * ce - 2) // ce <= 32  # rows that share a wavefront
+        on_grid = short or cols // ce > 128     # ... or 3 chunks per lane and more
+        assert p.kernel_name().endswith("_grid" if on_grid else "_ragged"), p.kernel_name()
         lg = f(xs) + f(ys)
         e = np.exp(lg - lg.max(-1, keepdims=True))
         assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < tol
         p = gh.Rows(xs, dt).row_op("layernorm", 1e-5, w=ws, b=bs).unary("relu")
         got = out(p.run())
-        assert p.kernel_name().endswith("_ragged"), p.kernel_name()
+        assert p.kernel_name().endswith("_grid" if short else "_ragged"), p.kernel_name()  # (per-column weights: on the grid only where rows share a wavefront)
         xf = f(xs)
         n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * f(ws) + f(bs)
         assert np.max(np.abs(got - np.maximum(n, 0))) < tol * (1 if dt == F32 else 2)
