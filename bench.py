@@ -369,6 +369,18 @@ def bench_survey(torch, capi, stream, steps, warmup):
     run("layernorm(x+y)_bf16_16384x4099", P(t).op("add", u).row("layernorm", wr, br).finish(torch))
     run("mean(x^2)_bf16_16384x4099", P(t, f32).op("square").finish(torch, "mean"))
     del t, u
+    # short rows (attention scores over short sequences, per-head norms, class logits): 4 to 32 lanes per row, several
+    # rows to a wavefront; odd lengths on the 16-byte grid
+    for rows, cols, dt, name in ((1 << 20, 64, bf, "bf16"), (1 << 19, 128, bf, "bf16"), (1 << 20, 64, f32, "f32"), (1 << 22, 16, bf, "bf16")):
+        t = rnd((rows, cols), dt, 2.0)
+        wr = rnd((cols,), dt, 0.3, 1.0)
+        run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
+        run(f"rmsnorm_{name}_{rows}x{cols}", P(t).row("rmsnorm", wr).finish(torch))
+        del t
+    for rows, cols, dt, name in ((3000000, 10, f32, "f32"), (400000, 77, bf, "bf16"), (170000, 197, bf, "bf16")):
+        t = rnd((rows, cols), dt, 2.0)
+        run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
+        del t
     # vocabulary-sized rows (language-model logits): 1024-thread blocks; beyond 8 chunks per thread the row stays in
     # registers as raw words, beyond 16 (fp32 logits over 128 256 entries) the block walks the row once per pass
     for rows, cols, dt, name in ((4096, 50304, bf, "bf16"), (2048, 128256, bf, "bf16"), (2048, 50304, f32, "f32"), (4096, 50257, bf, "bf16"),
