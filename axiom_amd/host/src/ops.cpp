@@ -296,7 +296,12 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
     // Shapes no attention kernel takes (head sizes above 256; 65 536 or more (batch, head) slices on the FMA kernel)
     // are composed from the matrix product, masking and softmax kernels, as the reference composes what its own
     // kernels do not take (src/backends/metal/flash_attention_dispatch.mm:125-162, 180-196).
-    if (tl_sdpa_kernel == "invalid" || (tl_sdpa_kernel == "generic" && B * H >= 65536)) {
+    // Head sizes between 129 and 256 have the FMA kernel only (a few TFLOP/s): once the problem is large enough to
+    // notice, and its score matrix small enough to hold (32 GiB), the composed form on the matrix-core GEMM is two
+    // orders of magnitude faster.
+    const double work = static_cast<double>(B) * H * Sq * Skv * D, score_bytes = static_cast<double>(B) * H * Sq * Skv * static_cast<double>(q.itemsize());
+    const bool wide_head = D > 128 && work >= double(1 << 24) && score_bytes <= 32.0 * double(1 << 30);
+    if (tl_sdpa_kernel == "invalid" || (tl_sdpa_kernel == "generic" && (B * H >= 65536 || wide_head))) {
         tl_sdpa_kernel = "decomposed";
         Tensor o = decomposed_sdpa(q, k, v, m, scale > 0.0f ? scale : 1.0f / std::sqrt(static_cast<float>(D)), is_causal);
         if (!out_bshd) return o;

@@ -518,6 +518,24 @@ GPU_TEST(FlashAttentionGPU, ShapesNoKernelTakesAreComposedFromMatmulMaskAndSoftm
         EXPECT_EQ(got.dtype(), DType::BFloat16);
         EXPECT_LE(max_abs_diff(got, ref), 3e-2); // the scores and the weights each pass through bf16 on the composed path
     }
+    // head sizes 192 and 256 (only the FMA kernel takes them): composed once the problem is large enough to notice,
+    // bf16 and fp32, causal and not; a small problem of the same head size stays on the kernel
+    for (size_t D : {192, 256}) {
+        auto [qw, kw, vw] = make_inputs(1, 2, 256, 320, D);
+        for (bool causal : {false, true}) {
+            auto got = ops::scaled_dot_product_attention(qw.gpu(), kw.gpu(), vw.gpu(), Tensor(), -1, causal);
+            EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("decomposed"));
+            ASSERT_TENSORS_CLOSE(got.cpu(), axtest::oracle_sdpa(qw, kw, vw, Tensor(), -1, causal), 2e-4, 2e-4);
+        }
+        auto qb = qw.astype(DType::BFloat16), kb = kw.astype(DType::BFloat16), vb = vw.astype(DType::BFloat16);
+        auto ref = axtest::oracle_sdpa(qb.astype(DType::Float32), kb.astype(DType::Float32), vb.astype(DType::Float32), Tensor(), -1, false);
+        auto got = ops::scaled_dot_product_attention(qb.gpu(), kb.gpu(), vb.gpu(), Tensor(), -1, false);
+        EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("decomposed"));
+        EXPECT_LE(max_abs_diff(got, ref), 3e-2);
+        auto [q1, k1, v1] = make_inputs(1, 1, 8, 8, D);
+        ops::scaled_dot_product_attention(q1.gpu(), k1.gpu(), v1.gpu(), Tensor(), -1, false).cpu();
+        EXPECT_EQ(std::string(ops::last_sdpa_kernel()), std::string("generic"));
+    }
     // 65 536 (batch, head) slices of a head size that only the FMA kernel takes
     {
         auto [qs, ks, vs] = make_inputs(256, 256, 4, 4, 8);
