@@ -379,6 +379,9 @@ __device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
 
 // NW waves per work-group (4: two work-groups share a CU; 8: one work-group per CU, each
 // K/V tile fetched once for 256 query rows instead of 128).
+// Head sizes between the compiled ones (a.D = 40 .. 56 on D = 64, 72 .. 120 on D = 128, multiples of 8) run as the next
+// compiled size with zeros in the missing dims: the Q fragments beyond a.D stay zero, the lanes that would fetch a K/V
+// chunk beyond a.D are sent outside the tile's descriptor (the load writes zeros to LDS), the output keeps a.D columns.
 // SPLIT = 2 (problems too small to give every SIMD two waves otherwise): the work-group's waves form two halves that
 // take the same 32 * NW / 2 query rows and one half of the keys each, through K/V tile buffers of their own; the second
 // half hands its accumulators, reference maximum and row sums to the first through LDS at the end.  No causal mask, no
@@ -440,16 +443,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     const bool mask_words = HAS_MASK && a.Skv % 4 == 0 && (reinterpret_cast<uintptr_t>(M) & 3u) == 0;
     uint32_t mk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 
+    const int dv = a.D; // the head size in memory (<= D, a multiple of 8)
     const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
-    const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + D * 2);
-    const int4_t vrsrc = make_rsrc(V, (a.Skv - 1) * vrow_bytes + D * 2);
+    const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + dv * 2);
+    const int4_t vrsrc = make_rsrc(V, (a.Skv - 1) * vrow_bytes + dv * 2);
 
     // ---- HBM -> LDS mapping.  A wave-wide load moves RPL rows; load n of wave w covers
     // tile rows RPL*NW*n + RPL*w + lane / CHUNKS; the lane fetches the chunk that belongs at
     // position lane % CHUNKS of the swizzled row (the swizzles only see row & 15).
     const int ld_r = RPL * wave + lane / CHUNKS;
-    const int k_voff = ld_r * krow_bytes + ((lane % CHUNKS) ^ swizzle_k<D>(ld_r)) * 16;
-    const int v_voff = ld_r * vrow_bytes + ((lane % CHUNKS) ^ swizzle_v<D>(ld_r)) * 16;
+    // (a chunk beyond the head size in memory: an offset that stays outside the descriptor whatever tile offset is
+    // added to it -- a (batch, head) slice spans less than 2^31 bytes)
+    const int k_chunk = (lane % CHUNKS) ^ swizzle_k<D>(ld_r), v_chunk = (lane % CHUNKS) ^ swizzle_v<D>(ld_r);
+    const int k_voff = k_chunk * 8 < dv ? ld_r * krow_bytes + k_chunk * 16 : static_cast<int>(0x80000000u);
+    const int v_voff = v_chunk * 8 < dv ? ld_r * vrow_bytes + v_chunk * 16 : static_cast<int>(0x80000000u);
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)); // LDS addresses fit 32 bits
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + RPL * wave * ROWB);
     // load n (0 .. NLOAD-1) of this wave's share of a K / V tile
@@ -500,7 +507,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     #pragma unroll
         for (int t = 0; t < KT; ++t) {
             qf[t] = uint4_t{0, 0, 0, 0};
-            if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
+            if (q_ok && 16 * t + 8 * g < dv) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
     #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t w = qf[t][c];
@@ -783,7 +790,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
                     const int d = dt * 32 + i4 * 8 + g * 4;
                     uint2_t w = {pack2<BF16>(oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv),
                                  pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
-                    *reinterpret_cast<uint2_t *>(orow + d) = w;
+                    if (d < dv) *reinterpret_cast<uint2_t *>(orow + d) = w;
                 }
         }
     }
@@ -1247,7 +1254,8 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
     if (p.batch == 0 || p.heads == 0 || p.seq_q == 0 || p.head_dim == 0) return SdpaKind::EMPTY;
     const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
     const bool d_ok = p.head_dim == 32 || p.head_dim == 64 || p.head_dim == 128;
-    if (half && d_ok) {
+    // the 16-bit pipelined kernels also take the multiples of 8 between their compiled sizes (zeros in the missing dims)
+    if (half && (d_ok || (p.head_dim > 32 && p.head_dim < 128 && p.head_dim % 8 == 0))) {
         bool ok = true;
         // 16-byte vector access to every row of q/k/v, 8-byte to o
         for (int i = 0; i < 3; ++i)
@@ -1396,7 +1404,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             // 14.8 -> 10.6 us).  With a work-group for nearly every CU (Whisper's 20 heads of 1500 frames: 240) the
             // split changes nothing -- a SIMD issues the same instructions as one wave or as two.
             const int64_t g4 = static_cast<int64_t>((p.seq_q + 127) / 128) * a.B * a.H;
-            if (p.head_dim == 64 && !mask && !a.causal && p.seq_kv > BN && g4 <= 128 && sdpa_key_split) {
+            if (p.head_dim > 32 && p.head_dim <= 64 && !mask && !a.causal && p.seq_kv > BN && g4 <= 128 && sdpa_key_split) {
                 const unsigned gs = static_cast<unsigned>((p.seq_q + 63) / 64) * static_cast<unsigned>(a.B * a.H);
                 if (bf) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<true, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
                 else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<false, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
@@ -1417,7 +1425,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         else if (mask) AXHIP_LAUNCH_DX(false, true, DD);                                                                  \
         else AXHIP_LAUNCH_DX(false, false, DD);                                                                           \
     } while (0)
-            if (p.head_dim == 64) AXHIP_LAUNCH_D(64);
+            if (p.head_dim <= 64) AXHIP_LAUNCH_D(64);
             else AXHIP_LAUNCH_D(128);
 #undef AXHIP_LAUNCH_D
 #undef AXHIP_LAUNCH_DX

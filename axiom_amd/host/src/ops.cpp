@@ -246,7 +246,9 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
     // change neither Q K^T nor the wanted part of P V) once the problem is large enough for three pad passes and an
     // output slice to be small change against the FMA kernel they avoid (two orders of magnitude slower); this is
     // where the reference's decomposed fallback for such sizes (flash_attention_dispatch.mm:180-196) ends up.
-    if (D != 32 && D != 64 && D > 0 && D < 128 && static_cast<double>(B) * H * Sq * Skv * D >= double(1 << 24) &&
+    // (16-bit head sizes that are multiples of 8 above 32 need none of this: the kernels take them as they are)
+    const bool kernel_takes_it = query.dtype() != DType::Float32 && D > 32 && D % 8 == 0;
+    if (D != 32 && D != 64 && D > 0 && D < 128 && !kernel_takes_it && static_cast<double>(B) * H * Sq * Skv * D >= double(1 << 24) &&
         (query.dtype() == DType::Float32 || query.dtype() == DType::Float16 || query.dtype() == DType::BFloat16)) {
         const size_t Dp = D < 32 ? 32 : D < 64 ? 64 : 128;
         const std::vector<std::pair<size_t, size_t>> widen{{0, 0}, {0, 0}, {0, 0}, {0, Dp - D}};

@@ -43,25 +43,29 @@ def contiguous_strides(H, S, D):
 
 
 def sdpa(q, k, v, dt, scale=-1.0, causal=False, mask=None, q_strides=None, k_strides=None, v_strides=None,
-         shape=None, poison=True):
+         shape=None, poison=True, o_strides=None, out_init=None):
     """q/k/v: numpy storage arrays.  With `shape`=(B,H,Sq,Skv,D) and explicit strides the
-    arrays are raw buffers viewed through those strides; otherwise (B,H,S,D) contiguous."""
+    arrays are raw buffers viewed through those strides; otherwise (B,H,S,D) contiguous.
+    `out_init` (with `o_strides`): the raw output buffer's initial content; it is returned whole."""
     if shape is None:
         B, H, Sq, D = q.shape
         Skv = k.shape[2]
     else:
         B, H, Sq, Skv, D = shape
     dq, dk, dv = to_dev(q), to_dev(k), to_dev(v)
-    o = empty_dev((B, H, Sq, D), dt)
-    if poison:
-        o.fill_(float("nan") if dt == F32 else 0x7FC1)
+    if out_init is not None:
+        o = to_dev(out_init)
+    else:
+        o = empty_dev((B, H, Sq, D), dt)
+        if poison:
+            o.fill_(float("nan") if dt == F32 else 0x7FC1)
     p = capi.SdpaParams()
     p.dtype, p.batch, p.heads, p.seq_q, p.seq_kv, p.head_dim = dt, B, H, Sq, Skv, D
     p.scale, p.is_causal = scale, int(causal)
     p.q_strides[:] = q_strides or contiguous_strides(H, Sq, D)
     p.k_strides[:] = k_strides or contiguous_strides(H, Skv, D)
     p.v_strides[:] = v_strides or contiguous_strides(H, Skv, D)
-    p.o_strides[:] = contiguous_strides(H, Sq, D)
+    p.o_strides[:] = o_strides or contiguous_strides(H, Sq, D)
     dm = None
     if mask is not None:
         mask = np.ascontiguousarray(mask, np.uint8)

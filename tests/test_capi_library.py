@@ -41,7 +41,9 @@ def test_version_and_kernel_selection_without_device():
     for i, s in enumerate((32 * 4096 * 128, 4096 * 128, 128)):
         p.q_strides[i] = p.k_strides[i] = p.v_strides[i] = p.o_strides[i] = s
     assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"mfma_bf16_d128"
-    p.head_dim = 48
+    p.head_dim = 48  # multiples of 8 between the compiled head sizes run on the next one, zeros in the missing dims
+    assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"mfma_bf16_d48"
+    p.head_dim = 20
     assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"generic"  # the fallback of the reference's unsupported head sizes
     p.dtype, p.head_dim = capi.DTYPE_F32, 64
     assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"mfma_f32_d64"

@@ -87,7 +87,7 @@ def test_half_matches_fp32_reference_of_same_inputs(case, dt):
     q, k, v = inputs(B, H, Sq, Skv, D, dt, seed=7)
     mask = make_mask(mk, Sq, Skv)
     got, kern = gh.sdpa(q, k, v, dt, -1.0, causal, mask)
-    assert kern == ("generic" if D in (48, 96) else f"mfma_{'bf16' if dt == BF16 else 'f16'}_d{D}")
+    assert kern == f"mfma_{'bf16' if dt == BF16 else 'f16'}_d{D}"  # (48 and 96: on the 64 and 128 kernels, zeros in the missing dims)
     qf, kf, vf = (axo.to_f32(t, dt) for t in (q, k, v))
     if B * H * Sq * Skv <= 1 << 24:
         want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), causal, mask)
@@ -124,6 +124,43 @@ def test_small_head_dim_64_problems_split_their_keys_between_the_halves_of_a_wor
         ones = axo.to_bits(np.ones(v.shape, np.float32), dt)
         got, _ = gh.sdpa(q, k, ones, dt, -1.0, False, None)
         assert np.max(np.abs(axo.to_f32(got, dt) - 1.0)) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -10), (B, H, Sq, Skv)
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+def test_head_sizes_between_the_compiled_ones(dt):
+    """Multiples of 8 between 32 and 128 run on the next compiled head size: Q fragments beyond the head size stay
+    zero, the K/V chunks beyond it are loaded as zeros, the output keeps its own width (guard values behind every
+    output row: the rows sit in a wider buffer).  Self and cross attention, causal, a mask, the 8- and 4-wave and the
+    key-split work-groups, packed (batch, seq, heads*dim) strides."""
+    tag = "bf16" if dt == BF16 else "f16"
+    for D, (B, H, Sq, Skv), causal, mk in ((40, (1, 2, 70, 70), False, None), (48, (2, 3, 130, 70), True, None), (56, (1, 4, 64, 200), False, "mod3"),
+                                           (72, (1, 2, 100, 100), True, None), (80, (2, 2, 257, 300), False, None), (96, (1, 3, 300, 300), True, "mod3"),
+                                           (104, (1, 1, 33, 129), False, None), (120, (1, 2, 64, 64), False, None), (96, (2, 70, 520, 520), True, None),
+                                           (80, (1, 130, 600, 600), False, None)):
+        q, k, v = inputs(B, H, Sq, Skv, D, dt, seed=300 + D)
+        mask = make_mask(mk, Sq, Skv)
+        got, kern = gh.sdpa(q, k, v, dt, -1.0, causal, mask)
+        assert kern == f"mfma_{tag}_d{D}", kern
+        qf, kf, vf = (axo.to_f32(t, dt) for t in (q, k, v))
+        if B * H * Sq * Skv <= 1 << 24:
+            want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), causal, mask)
+        else:
+            want = axo.sdpa(qf, kf, vf, F32, -1.0, causal, mask)
+        err = np.max(np.abs(axo.to_f32(got, dt) - want))
+        assert err < 2e-2, (D, B, H, Sq, Skv, err)
+    # rows of 80 inside rows of 128: what lies behind a row's 80 values must survive
+    B, S, H, D, W = 1, 150, 3, 80, 128
+    g = axo.PCG64(17)
+    packed = [axo.to_bits(g.normal((B, S, H, W)), dt) for _ in range(3)]
+    st = (S * H * W, W, H * W)
+    out_init = axo.to_bits(np.full((B, S, H, W), 7.0, np.float32), dt)
+    got, kern = gh.sdpa(*packed, dt, -1.0, False, None, q_strides=st, k_strides=st, v_strides=st, o_strides=st, shape=(B, H, S, S, D), out_init=out_init)
+    assert kern == f"mfma_{tag}_d80"
+    gf = axo.to_f32(got, dt).reshape(B, S, H, W)
+    assert np.all(gf[..., D:] == 7.0)
+    qf, kf, vf = (axo.to_f32(t, dt)[..., :D].transpose(0, 2, 1, 3) for t in packed)
+    want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), False)
+    assert np.max(np.abs(gf[..., :D].transpose(0, 2, 1, 3) - want)) < 2e-2
 
 
 def test_fully_masked_rows_give_zeros_everywhere_else_matches():
