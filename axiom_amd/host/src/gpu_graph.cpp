@@ -597,6 +597,29 @@ class PlanBuilder {
             const bool big = m0 * n0 * k0 >= double(1 << 22) && m0 >= 64 && n0 >= 64 && k0 >= 32;
             a = k_contiguous(a, ta, false, big);
             b = k_contiguous(b, tb, true, big);
+            // A reduction length that leaves the rows off their 16-byte alignment (K = 1001) would send a large product
+            // to the FMA kernel (two orders of magnitude slower): both operands get zero columns up to the next
+            // aligned length instead -- two copy passes, and zeros add nothing to the products.
+            const size_t align = val(a).dtype == DType::Float32 ? 4 : 8, k_now = val(a).shape.back();
+            if (big && !ta && tb && k_now % align != 0 && val(a).shape.size() <= AXHIP_MAX_DIMS && val(b).shape.size() <= AXHIP_MAX_DIMS) {
+                auto widen = [&](int v) {
+                    Shape wide = val(v).shape;
+                    wide.back() = (k_now + align - 1) / align * align;
+                    Step st{};
+                    st.kind = Step::PAD;
+                    st.pad.src = v;
+                    st.pad.dst = new_temp(wide, val(v).dtype);
+                    st.pad.before.assign(wide.size(), 0);
+                    st.pad.after.assign(wide.size(), 0);
+                    st.pad.after.back() = static_cast<int64_t>(wide.back() - k_now);
+                    st.pad.value = 0.0;
+                    const int dst = st.pad.dst;
+                    plan_.steps.push_back(st);
+                    return dst;
+                };
+                a = widen(a);
+                b = widen(b);
+            }
         }
         const Shape &as = val(a).shape, &bs = val(b).shape;
         GemmStep g;

@@ -427,6 +427,35 @@ GPU_TEST(CpuGpuParity, ElementwiseReductionsMatmul) { // tests/test_cpu_gpu_pari
     EXPECT_EQ(ops::sum(axtest::randn({3, 4, 5}, 1).gpu(), {1}).shape(), Shape({3, 5})); // (ReductionsAndSoftmaxOverAnyAxis checks the values)
 }
 
+// Products whose reduction length leaves the operands' rows off their 16-byte alignment (K = 301 fp32, 203 bf16), in
+// both storage orders of the right operand: the planner pads both operands with zero columns and stays on the
+// matrix-core kernels.  Against the oracle's sgemm.
+GPU_TEST(CpuGpuParity, LargeMatmulWithUnalignedReductionLength) {
+    const size_t M = 200, N = 160, K = 301;
+    auto a = axtest::randn({M, K}, 51), b = axtest::randn({K, N}, 52);
+    std::vector<float> want(M * N);
+    axo_matmul(AXO_F32, a.data(), b.data(), want.data(), M, N, K, 0, 0);
+    auto nn = host_floats(ops::matmul(a.gpu(), b.gpu()));
+    auto nt = host_floats(ops::matmul(a.gpu(), b.transpose({1, 0}).ascontiguousarray().gpu(), false, true));
+    for (size_t i = 0; i < M * N; ++i) {
+        EXPECT_NEAR(nn[i], want[i], 2e-4 + 1e-4 * std::fabs(want[i]));
+        EXPECT_NEAR(nt[i], want[i], 2e-4 + 1e-4 * std::fabs(want[i]));
+    }
+    ASSERT_TRUE(!graph::last_gpu_plan_kernels().empty());
+    EXPECT_EQ(graph::last_gpu_plan_kernels().back(), std::string("gemm"));
+    // bf16, batched, K = 203
+    auto ab = axtest::randn({3, 128, 203}, 53).astype(DType::BFloat16), bb = axtest::randn({3, 96, 203}, 54).astype(DType::BFloat16);
+    auto got = ops::matmul(ab.gpu(), bb.gpu(), false, true);
+    EXPECT_EQ(got.shape(), Shape({3, 128, 96}));
+    auto gh = host_floats(got.astype(DType::Float32));
+    auto af = ab.astype(DType::Float32), bf = bb.astype(DType::Float32);
+    std::vector<float> w2(128 * 96);
+    for (size_t i = 0; i < 3; ++i) {
+        axo_matmul(AXO_F32, af.typed_data<float>() + i * 128 * 203, bf.typed_data<float>() + i * 96 * 203, w2.data(), 128, 96, 203, 0, 1);
+        for (size_t j = 0; j < w2.size(); ++j) EXPECT_NEAR(gh[i * w2.size() + j], w2[j], 0.15 + 0.01 * std::fabs(w2[j]));
+    }
+}
+
 // ----------------------------------------------------------------- attention
 static std::tuple<Tensor, Tensor, Tensor> make_inputs(size_t B, size_t H, size_t Sq, size_t Skv, size_t D, DType dt = DType::Float32, uint64_t seed = 42) {
     return {axtest::randn({B, H, Sq, D}, seed, dt), axtest::randn({B, H, Skv, D}, seed + 1, dt), axtest::randn({B, H, Skv, D}, seed + 2, dt)};
