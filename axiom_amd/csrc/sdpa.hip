@@ -388,7 +388,8 @@ __device__ __forceinline__ int4_t make_rsrc(const void *base, int bytes) {
 // explicit mask, at least two key tiles.
 // (Four K and four V tile buffers with counted waits, so that a tile is requested three steps before its use, made the
 // 4-wave head_dim-64 kernel 5 % slower on small problems: its step is not waiting for tiles.)
-template <bool BF16, bool HAS_MASK, int NW, int D, int SPLIT = 1>
+// (PAD: such a head size; the exact sizes keep a kernel without its tests.)
+template <bool BF16, bool HAS_MASK, int NW, int D, int SPLIT = 1, bool PAD = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_kernel(const SdpaArgs a) {
     static_assert(D == 128 || D == 64, "head sizes with a direct-to-LDS pipeline");
     static_assert(SPLIT == 1 || (SPLIT == 2 && !HAS_MASK && NW == 4 && D == 64), "key split: the 64 KiB of static LDS hold two sets of head_dim-64 tiles");
@@ -443,7 +444,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     const bool mask_words = HAS_MASK && a.Skv % 4 == 0 && (reinterpret_cast<uintptr_t>(M) & 3u) == 0;
     uint32_t mk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    const int dv = a.D; // the head size in memory (<= D, a multiple of 8)
+    const int dv = PAD ? a.D : D; // the head size in memory (<= D, a multiple of 8)
     const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
     const int4_t krsrc = make_rsrc(K, (a.Skv - 1) * krow_bytes + dv * 2);
     const int4_t vrsrc = make_rsrc(V, (a.Skv - 1) * vrow_bytes + dv * 2);
@@ -1406,8 +1407,13 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             const int64_t g4 = static_cast<int64_t>((p.seq_q + 127) / 128) * a.B * a.H;
             if (p.head_dim > 32 && p.head_dim <= 64 && !mask && !a.causal && p.seq_kv > BN && g4 <= 128 && sdpa_key_split) {
                 const unsigned gs = static_cast<unsigned>((p.seq_q + 63) / 64) * static_cast<unsigned>(a.B * a.H);
-                if (bf) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<true, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
-                else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<false, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
+                if (p.head_dim == 64) {
+                    if (bf) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<true, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
+                    else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<false, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
+                } else {
+                    if (bf) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<true, false, 4, 64, 2, true>), dim3(gs), dim3(256), 0, s, a);
+                    else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<false, false, 4, 64, 2, true>), dim3(gs), dim3(256), 0, s, a);
+                }
                 break;
             }
             const int bmw = wide ? 256 : 128;
@@ -1415,8 +1421,13 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             const unsigned g = static_cast<unsigned>(a.causal ? (nqbw + 1) / 2 : nqbw) * static_cast<unsigned>(a.B * a.H);
 #define AXHIP_LAUNCH_DX(BF, MK, DD)                                                                                       \
     do {                                                                                                                  \
-        if (wide) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 8, DD>), dim3(g), dim3(512), 0, s, a);                \
-        else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 4, DD>), dim3(g), dim3(256), 0, s, a);                     \
+        if (p.head_dim == DD) {                                                                                           \
+            if (wide) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 8, DD>), dim3(g), dim3(512), 0, s, a);            \
+            else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 4, DD>), dim3(g), dim3(256), 0, s, a);                 \
+        } else {                                                                                                          \
+            if (wide) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 8, DD, 1, true>), dim3(g), dim3(512), 0, s, a);   \
+            else hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<BF, MK, 4, DD, 1, true>), dim3(g), dim3(256), 0, s, a);        \
+        }                                                                                                                 \
     } while (0)
 #define AXHIP_LAUNCH_D(DD)                                                                                                \
     do {                                                                                                                  \
