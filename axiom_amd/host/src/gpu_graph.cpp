@@ -621,6 +621,31 @@ class PlanBuilder {
                 b = widen(b);
             }
         }
+        // Batch dimensions that broadcast against each other in part ([B,1,M,K] x [1,H,K,N], or equal counts in
+        // different shapes): both operands are expanded to the common batch shape once (a gather with zero strides);
+        // a shared operand without batch dimensions, or with all of them 1, needs no copy (stride 0 below).
+        {
+            const Shape a_batch(val(a).shape.begin(), val(a).shape.end() - 2), b_batch(val(b).shape.begin(), val(b).shape.end() - 2);
+            const size_t na = ShapeUtils::size(a_batch), nb = ShapeUtils::size(b_batch);
+            if (na > 1 && nb > 1 && a_batch != b_batch) {
+                const size_t nd = std::max(a_batch.size(), b_batch.size());
+                Shape common(nd, 1);
+                for (size_t i = 0; i < nd; ++i) {
+                    const size_t da = i + a_batch.size() >= nd ? a_batch[i + a_batch.size() - nd] : 1;
+                    const size_t db = i + b_batch.size() >= nd ? b_batch[i + b_batch.size() - nd] : 1;
+                    if (da != db && da != 1 && db != 1) throw ShapeError("matmul: batch dimensions do not broadcast");
+                    common[i] = std::max(da, db);
+                }
+                auto expanded = [&](int v) {
+                    Shape target = common;
+                    target.push_back(val(v).shape[val(v).shape.size() - 2]);
+                    target.push_back(val(v).shape.back());
+                    return make_contiguous(v, &target);
+                };
+                a = expanded(a);
+                b = expanded(b);
+            }
+        }
         const Shape &as = val(a).shape, &bs = val(b).shape;
         GemmStep g;
         g.p.dtype = detail::to_axhip_dtype(val(a).dtype);

@@ -456,6 +456,31 @@ GPU_TEST(CpuGpuParity, LargeMatmulWithUnalignedReductionLength) {
     }
 }
 
+// Batch dimensions that broadcast in part (tests/test_tensor_matmul.cpp: batched products follow numpy's rules)
+GPU_TEST(CpuGpuParity, MatmulBroadcastsBatchDimensions) {
+    auto a = axtest::randn({3, 1, 20, 12}, 61), b = axtest::randn({1, 4, 12, 9}, 62);
+    auto got = ops::matmul(a.gpu(), b.gpu());
+    EXPECT_EQ(got.shape(), Shape({3, 4, 20, 9}));
+    auto g = host_floats(got);
+    std::vector<float> want(20 * 9);
+    for (size_t i = 0; i < 3; ++i)
+        for (size_t j = 0; j < 4; ++j) {
+            axo_matmul(AXO_F32, a.typed_data<float>() + i * 20 * 12, b.typed_data<float>() + j * 12 * 9, want.data(), 20, 9, 12, 0, 0);
+            for (size_t e = 0; e < want.size(); ++e) EXPECT_NEAR(g[(i * 4 + j) * want.size() + e], want[e], 1e-4 + 1e-4 * std::fabs(want[e]));
+        }
+    // equal batch counts in different shapes: [2,3,...] x [3,...] -> [2,3,...]
+    auto c = axtest::randn({2, 3, 8, 5}, 63), d = axtest::randn({3, 5, 7}, 64);
+    auto got2 = ops::matmul(c.gpu(), d.gpu());
+    EXPECT_EQ(got2.shape(), Shape({2, 3, 8, 7}));
+    auto g2 = host_floats(got2);
+    std::vector<float> w2(8 * 7);
+    for (size_t i = 0; i < 2; ++i)
+        for (size_t j = 0; j < 3; ++j) {
+            axo_matmul(AXO_F32, c.typed_data<float>() + (i * 3 + j) * 40, d.typed_data<float>() + j * 35, w2.data(), 8, 7, 5, 0, 0);
+            for (size_t e = 0; e < w2.size(); ++e) EXPECT_NEAR(g2[(i * 3 + j) * w2.size() + e], w2[e], 1e-4 + 1e-4 * std::fabs(w2[e]));
+        }
+}
+
 // ----------------------------------------------------------------- attention
 static std::tuple<Tensor, Tensor, Tensor> make_inputs(size_t B, size_t H, size_t Sq, size_t Skv, size_t D, DType dt = DType::Float32, uint64_t seed = 42) {
     return {axtest::randn({B, H, Sq, D}, seed, dt), axtest::randn({B, H, Skv, D}, seed + 1, dt), axtest::randn({B, H, Skv, D}, seed + 2, dt)};
