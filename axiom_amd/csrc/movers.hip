@@ -4,6 +4,8 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <climits>
+#include <cstdint>
 
 namespace axhip {
 
@@ -164,6 +166,106 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const V *table, int64_
         V v{};
         if (idx >= 0 && idx < table_rows) v = table[idx * row_chunks + c];
         dst[i] = v;
+    }
+}
+
+// ------------------------------------------------------------- argmax / argmin
+// Index of the extreme along the middle extent of an (outer, axis, inner) view, with the scan's rule of the CPU path:
+// start at index 0 with the type's lowest() (argmin: max()) as the value to beat, move on a strict comparison -- the
+// first occurrence of the extreme wins, a NaN never does, a slice with nothing beyond the start value answers 0.
+// A candidate is (value, index); "no candidate yet" carries index INT32_MAX, so that among equal values the lower
+// index wins and the start value loses to a real element of the same value only by the strict comparison.
+struct ArgBest {
+    float v;
+    int32_t i;
+};
+template <bool MIN> __device__ __forceinline__ void arg_take(ArgBest &b, float v, int32_t i) { // i increases along a thread's scan
+    if (MIN ? v < b.v : v > b.v) {
+        b.v = v;
+        b.i = i;
+    }
+}
+template <bool MIN> __device__ __forceinline__ void arg_merge(ArgBest &b, float v, int32_t i) { // candidates in any order
+    if ((MIN ? v < b.v : v > b.v) || (v == b.v && i < b.i)) {
+        b.v = v;
+        b.i = i;
+    }
+}
+template <bool MIN> __device__ __forceinline__ void arg_merge_wave(ArgBest &b) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const float v = __shfl_xor(b.v, d, WAVE);
+        const int32_t i = __shfl_xor(b.i, d, WAVE);
+        arg_merge<MIN>(b, v, i);
+    }
+}
+
+// inner == 1: a row per wavefront (THREADS = 64, four rows per work-group) or per work-group of 1024 threads.  A row
+// starts wherever rows * cols puts it: elements up to the next 16-byte boundary and behind the last whole vector are
+// read one by one, the body as 16-byte vectors.
+template <bool MIN, int THREADS>
+__global__ __launch_bounds__(THREADS == 64 ? 256 : THREADS) void argreduce_rows_kernel(const void *src, int dt, int64_t rows, int64_t cols, float start, int64_t *dst) {
+    constexpr int RPB = THREADS == 64 ? 4 : 1;
+    __shared__ float sv[THREADS == 64 ? 1 : THREADS / 64];
+    __shared__ int32_t si[THREADS == 64 ? 1 : THREADS / 64];
+    const int t = THREADS == 64 ? threadIdx.x % 64 : threadIdx.x;
+    const int es = dt == AXHIP_DTYPE_F32 ? 4 : 2, E = 16 / es;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * RPB + (THREADS == 64 ? threadIdx.x / 64 : 0); row < rows; row += static_cast<int64_t>(gridDim.x) * RPB) {
+        const int64_t base = row * cols;
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(src) + static_cast<uintptr_t>(base) * es;
+        const int64_t head = min(cols, static_cast<int64_t>(((16 - (addr & 15u)) & 15u) / es));
+        const int64_t nvec = (cols - head) / E, tail0 = head + nvec * E;
+        ArgBest b{start, INT32_MAX};
+        if (t < head) arg_take<MIN>(b, load_any(src, dt, base + t), t);
+        for (int64_t c = t; c < nvec; c += THREADS) {
+            const int64_t at = head + c * E;
+            if (es == 4) {
+                float v[4];
+                load_vec<4>(src, dt, base + at, v);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) arg_take<MIN>(b, v[e], static_cast<int32_t>(at + e));
+            } else {
+                float v[8];
+                load_vec<8>(src, dt, base + at, v);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) arg_take<MIN>(b, v[e], static_cast<int32_t>(at + e));
+            }
+        }
+        if (tail0 + t < cols) arg_take<MIN>(b, load_any(src, dt, base + tail0 + t), static_cast<int32_t>(tail0 + t));
+        arg_merge_wave<MIN>(b);
+        if constexpr (THREADS > 64) {
+            const int w = threadIdx.x / 64;
+            __syncthreads(); // the previous row's partials have been read
+            if (threadIdx.x % 64 == 0) {
+                sv[w] = b.v;
+                si[w] = b.i;
+            }
+            __syncthreads();
+            if (threadIdx.x == 0)
+                for (int k = 1; k < THREADS / 64; ++k) arg_merge<MIN>(b, sv[k], si[k]);
+        }
+        if (t == 0) dst[row] = b.i == INT32_MAX ? 0 : b.i;
+    }
+}
+
+// inner > 1: a thread per (outer, inner) position walks the axis; neighbouring threads read neighbouring addresses.
+template <bool MIN>
+__global__ __launch_bounds__(256) void argreduce_strided_kernel(const void *src, int dt, int64_t outer, int64_t axis, int64_t inner, float start, int64_t *dst) {
+    const int64_t total = outer * inner;
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; p < total; p += static_cast<int64_t>(gridDim.x) * 256) {
+        const int64_t o = p / inner, i = p - o * inner;
+        const int64_t first = o * axis * inner + i;
+        ArgBest b{start, INT32_MAX};
+        int64_t k = 0;
+        for (; k + 4 <= axis; k += 4) { // four loads in flight per thread
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load_any(src, dt, first + (k + u) * inner);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) arg_take<MIN>(b, v[u], static_cast<int32_t>(k + u));
+        }
+        for (; k < axis; ++k) arg_take<MIN>(b, load_any(src, dt, first + k * inner), static_cast<int32_t>(k));
+        dst[p] = b.i == INT32_MAX ? 0 : b.i;
     }
 }
 
@@ -369,6 +471,39 @@ int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int6
     else
         hipLaunchKernelGGL(gather_rows_kernel<uint16_t>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, static_cast<const uint16_t *>(table),
                            table_rows, chunks, indices, index_bytes, n_indices, static_cast<uint16_t *>(dst));
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t want_min, int64_t *dst, void *stream) {
+    AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_argreduce: bad dtype");
+    AXHIP_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, AXHIP_ERR_INVALID_ARG, "axhip_argreduce: negative extent");
+    if (outer == 0 || inner == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(axis > 0, AXHIP_ERR_INVALID_ARG, "axhip_argreduce: an empty axis has no extreme");
+    AXHIP_REQUIRE(axis < (int64_t(1) << 31) - 1, AXHIP_ERR_UNSUPPORTED, "axhip_argreduce: axis of %lld elements (indices are held in 32 bits)", static_cast<long long>(axis));
+    AXHIP_REQUIRE(src && dst, AXHIP_ERR_INVALID_ARG, "axhip_argreduce: NULL buffer");
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = resolve_stream(stream);
+    // lowest() of the element type (argmin: max()): the value the first element has to beat
+    const float lowest = dtype == AXHIP_DTYPE_F32 ? -3.402823466e+38f : dtype == AXHIP_DTYPE_F16 ? -65504.0f : -3.3895313892515355e+38f;
+    const float start = want_min ? -lowest : lowest;
+    if (inner == 1) {
+        const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+        if (axis * es <= 16384) {
+            const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer + 3) / 4, 256 * 32));
+            if (want_min) hipLaunchKernelGGL((argreduce_rows_kernel<true, 64>), dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, start, dst);
+            else hipLaunchKernelGGL((argreduce_rows_kernel<false, 64>), dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, start, dst);
+        } else {
+            const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer, 256 * 8));
+            if (want_min) hipLaunchKernelGGL((argreduce_rows_kernel<true, 1024>), dim3(blocks), dim3(1024), 0, s, src, dtype, outer, axis, start, dst);
+            else hipLaunchKernelGGL((argreduce_rows_kernel<false, 1024>), dim3(blocks), dim3(1024), 0, s, src, dtype, outer, axis, start, dst);
+        }
+    } else {
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
+        if (want_min) hipLaunchKernelGGL(argreduce_strided_kernel<true>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, start, dst);
+        else hipLaunchKernelGGL(argreduce_strided_kernel<false>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, start, dst);
+    }
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;
 }

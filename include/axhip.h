@@ -271,6 +271,17 @@ int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int6
                       const void *indices, int32_t index_bytes, int64_t n_indices, void *dst,
                       void *stream);
 
+/* argmax (want_min = 0) / argmin along the middle extent of a contiguous
+ * (outer, axis, inner) view -> outer * inner int64 indices: the Reduction node
+ * kinds ArgMax / ArgMin of the GPU graph compiler
+ * (src/backends/metal/mpsgraph_graph_compiler.mm:628-658), with the CPU scan's
+ * rule (src/backends/cpu/cpu_operations.cpp:2157-2229): the first occurrence of
+ * the extreme wins, a NaN never does, and a slice with nothing above the type's
+ * lowest() (argmin: below max()) -- all -inf, all NaN -- answers 0.  inner == 1
+ * is the row form (greedy decoding over [batch, vocabulary] logits). */
+int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
+                    int32_t want_min, int64_t *dst, void *stream);
+
 /* -------------------------------------------------------------------- GEMM
  * Stands behind the GPU MatMul registry entry and gpu_linear
  * (src/backends/metal/mpsgraph_operations.mm:2409-2532; lazy builder

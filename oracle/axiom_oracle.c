@@ -480,6 +480,37 @@ int axo_reduce_last(int red, int dtype, const void *in, void *out, size_t rows, 
 }
 
 /* ------------------------------------------------------------------------ */
+/* argmax / argmin over an axis: src/backends/cpu/cpu_operations.cpp:2157-2229 */
+/* (argmin: the same loop with `<` and max(), :2258-2330).  The scan starts */
+/* at index 0 with the type's lowest() (argmin: max()) as the value to beat */
+/* and moves on a STRICT comparison in the input's own type: the first      */
+/* occurrence of the extreme wins, a NaN never does, and a slice with       */
+/* nothing above lowest() (all -inf, all NaN) answers 0.  Indices are int64 */
+/* (:2186).  Half values compare as their exact float images.               */
+/* ------------------------------------------------------------------------ */
+
+int axo_argreduce(int want_min, int dtype, const void *in, int64_t *out, size_t outer, size_t axis, size_t inner) {
+    if (dtype < 0 || dtype > 2) return -1;
+    /* lowest() of the type: -FLT_MAX, -65504 (float16.hpp:82-), 0xFF7F as bfloat16 (bfloat16.hpp:116-118) */
+    const float lowest = dtype == AXO_F32 ? -3.402823466e+38f : dtype == AXO_F16 ? -65504.0f : axo_bf16_to_f32(0xFF7F);
+#pragma omp parallel for schedule(static) if (outer * inner >= 64)
+    for (ptrdiff_t oi = 0; oi < (ptrdiff_t)(outer * inner); ++oi) {
+        const size_t o = (size_t)oi / inner, i = (size_t)oi % inner;
+        size_t best_idx = 0;
+        float best = want_min ? -lowest : lowest;
+        for (size_t k = 0; k < axis; ++k) {
+            const float v = ld(dtype, in, (o * axis + k) * inner + i);
+            if (want_min ? v < best : v > best) {
+                best = v;
+                best_idx = k;
+            }
+        }
+        out[oi] = (int64_t)best_idx;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
 /* layer_norm on CPU: src/tensor/operations.cpp:1803-1817, a chain of       */
 /*   mean -> subtract -> multiply -> mean -> add(eps) -> sqrt -> divide ->  */
 /*   multiply(w) -> add(b).                                                 */

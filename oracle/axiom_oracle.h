@@ -41,6 +41,10 @@
  *       (tests/test_nn_layers.cpp:191-207).
  *   axo_matmul       float64 reference; Linear known answers 3/4/2/8
  *       (tests/test_nn_layers.cpp:12-73).
+ *   axo_argreduce    the known answers of tests/test_tensor_argmax_argmin.cpp:4-112
+ *       (1-D, both axes of [[1,5],[3,2]], arange(24) as (2,3,4)); numpy's
+ *       argmax / argmin on data without NaN (same first-occurrence rule); the
+ *       NaN / -inf cases by the scan's own definition on 3-element rows.
  */
 #ifndef AXIOM_ORACLE_H
 #define AXIOM_ORACLE_H
@@ -108,6 +112,11 @@ int axo_binary(int op, int dtype, const void *a, const void *b, void *out,
  * result rounded to dtype for half types). */
 int axo_reduce_last(int red, int dtype, const void *in, void *out, size_t rows,
                     size_t cols);
+
+/* argmax (want_min = 0) / argmin over the middle extent of an (outer, axis,
+ * inner) view; out has outer * inner int64 indices. */
+int axo_argreduce(int want_min, int dtype, const void *in, int64_t *out, size_t outer,
+                  size_t axis, size_t inner);
 
 /* CPU layer_norm / rms_norm decompositions.  Output is ALWAYS float32, as on
  * the reference's CPU path (half inputs are promoted by the first op that

@@ -59,6 +59,7 @@ def lib() -> C.CDLL:
         l.axo_softmax.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int]
         l.axo_unary.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]
         l.axo_binary.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int]
+        l.axo_argreduce.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]
         l.axo_reduce_last.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t]
         l.axo_layer_norm.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_float]
         l.axo_rms_norm.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_float]
@@ -191,6 +192,17 @@ def reduce_last(red, x, dt=F32):
     rows = int(np.prod(x.shape[:-1], dtype=np.int64))
     out = np.empty(x.shape[:-1], x.dtype)
     assert lib().axo_reduce_last(RED[red], dt, _p(x), _p(out), rows, x.shape[-1]) == 0
+    return out
+
+
+def argreduce(x, axis=-1, want_min=False, dt=F32):
+    """argmax / argmin along one axis (int64 indices, first occurrence wins)."""
+    x = np.ascontiguousarray(x)
+    axis %= x.ndim
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    out = np.empty(x.shape[:axis] + x.shape[axis + 1:], np.int64)
+    assert lib().axo_argreduce(int(want_min), dt, _p(x), _p(out), outer, x.shape[axis], inner) == 0
     return out
 
 

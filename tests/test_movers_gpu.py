@@ -161,6 +161,74 @@ def test_gather_rows_is_an_embedding_lookup(dt, cols, itype):
     assert np.array_equal(gh.to_host(out, table.dtype), want)
 
 
+def _argreduce(dev, dt, outer, axis, inner, want_min):
+    out = torch.full((outer * inner,), -7, dtype=torch.int64, device="cuda")
+    gh.sync()
+    capi.check(capi.lib().axhip_argreduce(dev.data_ptr(), dt, outer, axis, inner, int(want_min), out.data_ptr(), None))
+    gh.sync()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("rows,cols", [(37, 1), (513, 10), (300, 77), (64, 1001), (33, 4096), (9, 8192), (5, 50257), (3, 128256), (2, 200003)],
+                         ids=lambda v: str(v))
+def test_argmax_argmin_over_rows_match_the_cpu_scan(dt, rows, cols):
+    """Row form (inner == 1) against the oracle's scan, bit-exact indices; values drawn from a small set so that every row
+    has ties (the first occurrence must win), with NaN and infinities sprinkled in; odd row lengths start rows at
+    every alignment."""
+    rng = np.random.default_rng(rows * 1000 + cols)
+    x = rng.integers(-6, 7, (rows, cols)).astype(np.float32) * 0.5
+    x[rng.random((rows, cols)) < 0.01] = np.nan
+    x[rng.random((rows, cols)) < 0.002] = np.inf
+    x[rng.random((rows, cols)) < 0.002] = -np.inf
+    if rows > 2:
+        x[1, :] = np.nan  # nothing beats the start value: index 0
+        x[2, :] = -np.inf
+    bits = x if dt == F32 else axo.to_bits(x, dt)
+    d = gh.to_dev(bits)
+    for want_min in (False, True):
+        got = _argreduce(d, dt, rows, cols, 1, want_min)
+        assert np.array_equal(got, axo.argreduce(bits, -1, want_min, dt)), (want_min, rows, cols)
+    if rows > 2:
+        assert _argreduce(d, dt, rows, cols, 1, False)[1] == 0 and _argreduce(d, dt, rows, cols, 1, False)[2] == 0
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_argmax_argmin_along_inner_axes_and_on_unaligned_bases(dt):
+    rng = np.random.default_rng(11)
+    x = rng.integers(-9, 10, (6, 130, 70)).astype(np.float32)
+    bits = x if dt == F32 else axo.to_bits(x, dt)
+    d = gh.to_dev(bits)
+    for axis, (outer, n, inner) in ((0, (1, 6, 130 * 70)), (1, (6, 130, 70)), (2, (6 * 130, 70, 1))):
+        for want_min in (False, True):
+            got = _argreduce(d, dt, outer, n, inner, want_min).reshape(axo.argreduce(bits, axis, want_min, dt).shape)
+            assert np.array_equal(got, axo.argreduce(bits, axis, want_min, dt)), (axis, want_min)
+    # a view that starts one element into the buffer: rows of 4099 elements at every alignment
+    flat = rng.normal(size=1 + 12 * 4099).astype(np.float32)
+    fb = flat if dt == F32 else axo.to_bits(flat, dt)
+    df = gh.to_dev(fb)
+    out = torch.empty(12, dtype=torch.int64, device="cuda")
+    gh.sync()
+    capi.check(capi.lib().axhip_argreduce(df.data_ptr() + fb.itemsize, dt, 12, 4099, 1, 0, out.data_ptr(), None))
+    gh.sync()
+    assert np.array_equal(out.cpu().numpy(), axo.argreduce(fb[1:].reshape(12, 4099), -1, False, dt))
+
+
+def test_argreduce_known_answers_and_errors():
+    """tests/test_tensor_argmax_argmin.cpp:4-58 on the device; argument checks."""
+    L = capi.lib()
+    d = gh.to_dev(np.array([1, 5, 3, 9, 2], np.float32))
+    assert _argreduce(d, F32, 1, 5, 1, False).tolist() == [3]
+    m = gh.to_dev(np.array([[1, 5], [3, 2]], np.float32))
+    assert _argreduce(m, F32, 1, 2, 2, False).tolist() == [1, 0] and _argreduce(m, F32, 2, 2, 1, False).tolist() == [1, 0]
+    assert _argreduce(m, F32, 1, 2, 2, True).tolist() == [0, 1]
+    assert L.axhip_argreduce(None, F32, 0, 5, 1, 0, None, None) == 0  # nothing to do
+    assert L.axhip_argreduce(d.data_ptr(), F32, 1, 0, 1, 0, d.data_ptr(), None) == capi.ERR_INVALID_ARG  # empty axis
+    assert L.axhip_argreduce(d.data_ptr(), 9, 1, 5, 1, 0, d.data_ptr(), None) == capi.ERR_INVALID_ARG
+    assert L.axhip_argreduce(None, F32, 1, 5, 1, 0, None, None) == capi.ERR_INVALID_ARG
+    assert L.axhip_argreduce(d.data_ptr(), F32, 1, 1 << 31, 1, 0, d.data_ptr(), None) == capi.ERR_UNSUPPORTED
+
+
 def test_mover_argument_errors():
     L = capi.lib()
     assert L.axhip_pad(None, None, 7, 1, i64([1]), i64([1]), i64([0]), i64([0]), 0.0, None) == capi.ERR_INVALID_ARG

@@ -422,3 +422,30 @@ def test_chain_c2_small():
     e = np.exp(x - x.max(-1, keepdims=True))
     assert np.allclose(sm, e / e.sum(-1, keepdims=True), atol=1e-6)
     assert np.allclose(out, 1.0, atol=1e-5)
+
+
+def test_argreduce_known_answers_and_first_occurrence():
+    """tests/test_tensor_argmax_argmin.cpp:4-112 known answers; numpy on NaN-free data; the scan's edge cases."""
+    f = lambda v: np.array(v, np.float32)
+    assert axo.argreduce(f([1, 5, 3, 9, 2])) == 3  # :4-13
+    assert axo.argreduce(f([1, 5, 3, -2, 2]), want_min=True) == 3  # :16-25
+    m = f([[1, 5], [3, 2]])
+    assert axo.argreduce(m, 0).tolist() == [1, 0]  # :28-36
+    assert axo.argreduce(m, 1).tolist() == [1, 0]  # :39-47
+    assert axo.argreduce(m, 0, want_min=True).tolist() == [0, 1]  # :50-58
+    assert axo.argreduce(f([1, 5, -3, 9, 2]), want_min=True) == 2  # :90-96
+    assert axo.argreduce(np.arange(24, dtype=np.float32).reshape(2, 3, 4), 2).tolist() == [[3] * 3] * 2  # :99-112
+    rng = np.random.default_rng(3)
+    x = rng.integers(-4, 5, (7, 9, 11)).astype(np.float32)  # many ties: the first occurrence must win
+    for axis in range(3):
+        assert np.array_equal(axo.argreduce(x, axis), x.argmax(axis))
+        assert np.array_equal(axo.argreduce(x, axis, want_min=True), x.argmin(axis))
+    xb = (x.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)  # small integers are exact in bf16
+    assert np.array_equal(axo.argreduce(xb, 2, dt=BF16), x.argmax(2))
+    assert np.array_equal(axo.argreduce(x.astype(np.float16), 1, want_min=True, dt=F16), x.argmin(1))
+    nan, inf = np.nan, np.inf
+    assert axo.argreduce(f([nan, 1, 2])) == 2 and axo.argreduce(f([3, nan, 2])) == 0  # a NaN never compares greater
+    assert axo.argreduce(f([nan, nan, nan])) == 0 and axo.argreduce(f([-inf, -inf, -inf])) == 0  # nothing beats lowest()
+    assert axo.argreduce(f([-inf, -3.402823466e38, -inf])) == 0  # lowest() itself does not beat lowest()
+    assert axo.argreduce(f([inf, inf, nan]), want_min=True) == 0 and axo.argreduce(f([nan, inf, 7]), want_min=True) == 2
+
