@@ -191,48 +191,70 @@ template <bool MIN> __device__ __forceinline__ void arg_merge(ArgBest &b, float 
         b.i = i;
     }
 }
-template <bool MIN> __device__ __forceinline__ void arg_merge_wave(ArgBest &b) {
+// the E = 16 / sizeof(element) values of one 16-byte vector, as fp32
+template <int DT> __device__ __forceinline__ void arg_unpack(const uint4_t raw, float (&v)[DT == AXHIP_DTYPE_F32 ? 4 : 8]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        const float v = __shfl_xor(b.v, d, WAVE);
-        const int32_t i = __shfl_xor(b.i, d, WAVE);
-        arg_merge<MIN>(b, v, i);
+    for (int k = 0; k < 4; ++k) {
+        if constexpr (DT == AXHIP_DTYPE_F32) {
+            v[k] = __uint_as_float(w[k]);
+        } else if constexpr (DT == AXHIP_DTYPE_BF16) {
+            v[2 * k] = __uint_as_float(w[k] << 16);
+            v[2 * k + 1] = __uint_as_float(w[k] & 0xFFFF0000u);
+        } else {
+            v[2 * k] = f16_bits_to_f32(w[k] & 0xFFFFu);
+            v[2 * k + 1] = f16_bits_to_f32(w[k] >> 16);
+        }
     }
 }
 
-// inner == 1: a row per wavefront (THREADS = 64, four rows per work-group) or per work-group of 1024 threads.  A row
-// starts wherever rows * cols puts it: elements up to the next 16-byte boundary and behind the last whole vector are
-// read one by one, the body as 16-byte vectors.
-template <bool MIN, int THREADS>
-__global__ __launch_bounds__(THREADS == 64 ? 256 : THREADS) void argreduce_rows_kernel(const void *src, int dt, int64_t rows, int64_t cols, float start, int64_t *dst) {
-    constexpr int RPB = THREADS == 64 ? 4 : 1;
+// inner == 1.  THREADS = 64: `lanes` (a power of two up to 64) lanes of a wavefront per row, 64 / lanes rows per
+// wavefront and four wavefronts per work-group; THREADS = 256 / 1024: a work-group per row.  A row starts wherever
+// rows * cols puts it: elements up to the next 16-byte boundary and behind the last whole vector are read one by
+// one, the body as 16-byte vectors, four of them requested before the first is looked at (a vector past the row's
+// last one is fetched again from the last and not looked at: no branch between the loads).
+template <bool MIN, int THREADS, int DT>
+__global__ __launch_bounds__(THREADS == 64 ? 256 : THREADS) void argreduce_rows_kernel(const void *src, int64_t rows, int64_t cols, int lanes, float start, int64_t *dst) {
+    constexpr int U = 4, E = DT == AXHIP_DTYPE_F32 ? 4 : 8, ES = 16 / E;
     __shared__ float sv[THREADS == 64 ? 1 : THREADS / 64];
     __shared__ int32_t si[THREADS == 64 ? 1 : THREADS / 64];
-    const int t = THREADS == 64 ? threadIdx.x % 64 : threadIdx.x;
-    const int es = dt == AXHIP_DTYPE_F32 ? 4 : 2, E = 16 / es;
-    for (int64_t row = static_cast<int64_t>(blockIdx.x) * RPB + (THREADS == 64 ? threadIdx.x / 64 : 0); row < rows; row += static_cast<int64_t>(gridDim.x) * RPB) {
-        const int64_t base = row * cols;
-        const uintptr_t addr = reinterpret_cast<uintptr_t>(src) + static_cast<uintptr_t>(base) * es;
-        const int64_t head = min(cols, static_cast<int64_t>(((16 - (addr & 15u)) & 15u) / es));
-        const int64_t nvec = (cols - head) / E, tail0 = head + nvec * E;
+    const int span = THREADS == 64 ? lanes : THREADS;                 // threads per row
+    const int t = THREADS == 64 ? threadIdx.x % lanes : threadIdx.x;  // position among them
+    const int rpb = THREADS == 64 ? 256 / lanes : 1;                  // rows per work-group and sweep
+    for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb; row0 < rows; row0 += static_cast<int64_t>(gridDim.x) * rpb) {
+        const int64_t row = row0 + (THREADS == 64 ? threadIdx.x / lanes : 0);
+        const bool there = row < rows; // (a wavefront's lanes stay together for the exchanges below)
+        const int64_t base = there ? row * cols : 0;
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(src) + static_cast<uintptr_t>(base) * ES;
+        const int head = static_cast<int>(min(cols, static_cast<int64_t>(((16 - (addr & 15u)) & 15u) / ES)));
+        const int nvec = there ? static_cast<int>((cols - head) / E) : 0, tail0 = head + nvec * E;
+        const uint4_t *vec = reinterpret_cast<const uint4_t *>(addr + static_cast<uintptr_t>(head) * ES);
         ArgBest b{start, INT32_MAX};
-        if (t < head) arg_take<MIN>(b, load_any(src, dt, base + t), t);
-        for (int64_t c = t; c < nvec; c += THREADS) {
-            const int64_t at = head + c * E;
-            if (es == 4) {
-                float v[4];
-                load_vec<4>(src, dt, base + at, v);
+        if (there)
+            for (int h = t; h < head; h += span) arg_take<MIN>(b, load_any(src, DT, base + h), h); // (up to E - 1 of them)
+        for (int c = t; c < nvec; c += span * U) {
+            uint4_t raw[U];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) arg_take<MIN>(b, v[e], static_cast<int32_t>(at + e));
-            } else {
-                float v[8];
-                load_vec<8>(src, dt, base + at, v);
+            for (int u = 0; u < U; ++u) raw[u] = vec[min(c + u * span, nvec - 1)];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) arg_take<MIN>(b, v[e], static_cast<int32_t>(at + e));
+            for (int u = 0; u < U; ++u) {
+                const int cc = c + u * span;
+                if (cc < nvec) {
+                    float v[E];
+                    arg_unpack<DT>(raw[u], v);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) arg_take<MIN>(b, v[e], head + cc * E + e);
+                }
             }
         }
-        if (tail0 + t < cols) arg_take<MIN>(b, load_any(src, dt, base + tail0 + t), static_cast<int32_t>(tail0 + t));
-        arg_merge_wave<MIN>(b);
+        if (there)
+            for (int64_t h = tail0 + t; h < cols; h += span) arg_take<MIN>(b, load_any(src, DT, base + h), static_cast<int32_t>(h));
+        // lanes of one row are neighbours: exchanges at distances below the row's span stay inside it
+        for (int d = min(span, 64) >> 1; d >= 1; d >>= 1) {
+            const float v = __shfl_xor(b.v, d, WAVE);
+            const int32_t i = __shfl_xor(b.i, d, WAVE);
+            arg_merge<MIN>(b, v, i);
+        }
         if constexpr (THREADS > 64) {
             const int w = threadIdx.x / 64;
             __syncthreads(); // the previous row's partials have been read
@@ -244,7 +266,7 @@ __global__ __launch_bounds__(THREADS == 64 ? 256 : THREADS) void argreduce_rows_
             if (threadIdx.x == 0)
                 for (int k = 1; k < THREADS / 64; ++k) arg_merge<MIN>(b, sv[k], si[k]);
         }
-        if (t == 0) dst[row] = b.i == INT32_MAX ? 0 : b.i;
+        if (there && t == 0) dst[row] = b.i == INT32_MAX ? 0 : b.i;
     }
 }
 
@@ -266,6 +288,56 @@ __global__ __launch_bounds__(256) void argreduce_strided_kernel(const void *src,
         }
         for (; k < axis; ++k) arg_take<MIN>(b, load_any(src, dt, first + k * inner), static_cast<int32_t>(k));
         dst[p] = b.i == INT32_MAX ? 0 : b.i;
+    }
+}
+
+// inner > 1 with inner a multiple of the 16-byte vector and an aligned base: a thread owns the E neighbouring inner
+// positions of one vector, TX such threads side by side read TX * 16 consecutive bytes, and the TY = 256 / TX thread
+// rows of a work-group share the axis (k = ty, ty + TY, ..), merging through LDS at the end.  TX = 32 when that
+// still gives the chip a thousand work-groups, else 8 (whole 128-byte lines still).
+template <bool MIN, int DT, int TX>
+__global__ __launch_bounds__(256) void argreduce_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, float start, int64_t *dst) {
+    constexpr int TY = 256 / TX, U = 4, V = DT == AXHIP_DTYPE_F32 ? 4 : 8;
+    __shared__ float sv[TY][TX][V + 1];
+    __shared__ int32_t si[TY][TX][V + 1];
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t ivecs = inner / V, groups = (ivecs + TX - 1) / TX, total = outer * groups;
+    const int n = static_cast<int>(axis);
+    for (int64_t g = blockIdx.x; g < total; g += gridDim.x) {
+        const int64_t o = g / groups, iv = (g - o * groups) * TX + tx;
+        const bool there = iv < ivecs;
+        const uint4_t *first = reinterpret_cast<const uint4_t *>(src) + o * axis * ivecs + iv;
+        ArgBest b[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e) b[e] = ArgBest{start, INT32_MAX};
+        if (there)
+            for (int k = ty; k < n; k += TY * U) {
+                uint4_t raw[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (k + u * TY < n) {
+                        float v[V];
+                        arg_unpack<DT>(raw[u], v);
+#pragma unroll
+                        for (int e = 0; e < V; ++e) arg_take<MIN>(b[e], v[e], k + u * TY);
+                    }
+            }
+        __syncthreads(); // the previous group's partials have been read
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            sv[ty][tx][e] = b[e].v;
+            si[ty][tx][e] = b[e].i;
+        }
+        __syncthreads();
+        // thread (ty, tx) finishes elements ty, ty + TY, .. of column group tx
+        if (there)
+            for (int e = ty; e < V; e += TY) {
+                ArgBest r{sv[0][tx][e], si[0][tx][e]};
+                for (int y = 1; y < TY; ++y) arg_merge<MIN>(r, sv[y][tx][e], si[y][tx][e]);
+                dst[o * inner + iv * V + e] = r.i == INT32_MAX ? 0 : r.i;
+            }
     }
 }
 
@@ -488,17 +560,53 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
     // lowest() of the element type (argmin: max()): the value the first element has to beat
     const float lowest = dtype == AXHIP_DTYPE_F32 ? -3.402823466e+38f : dtype == AXHIP_DTYPE_F16 ? -65504.0f : -3.3895313892515355e+38f;
     const float start = want_min ? -lowest : lowest;
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
     if (inner == 1) {
-        const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
-        if (axis * es <= 16384) {
-            const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer + 3) / 4, 256 * 32));
-            if (want_min) hipLaunchKernelGGL((argreduce_rows_kernel<true, 64>), dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, start, dst);
-            else hipLaunchKernelGGL((argreduce_rows_kernel<false, 64>), dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, start, dst);
+        const int64_t row_bytes = axis * es;
+#define AXHIP_ARG_ROWS_DT(T, DT, BLOCKS, LANES)                                                                                            \
+    do {                                                                                                                                   \
+        if (want_min) hipLaunchKernelGGL((argreduce_rows_kernel<true, T, DT>), dim3(BLOCKS), dim3(T == 64 ? 256 : T), 0, s, src, outer, axis, LANES, start, dst); \
+        else hipLaunchKernelGGL((argreduce_rows_kernel<false, T, DT>), dim3(BLOCKS), dim3(T == 64 ? 256 : T), 0, s, src, outer, axis, LANES, start, dst);         \
+    } while (0)
+#define AXHIP_ARG_ROWS(T, BLOCKS, LANES)                                                                                                   \
+    do {                                                                                                                                   \
+        if (dtype == AXHIP_DTYPE_F32) AXHIP_ARG_ROWS_DT(T, AXHIP_DTYPE_F32, BLOCKS, LANES);                                                \
+        else if (dtype == AXHIP_DTYPE_F16) AXHIP_ARG_ROWS_DT(T, AXHIP_DTYPE_F16, BLOCKS, LANES);                                           \
+        else AXHIP_ARG_ROWS_DT(T, AXHIP_DTYPE_BF16, BLOCKS, LANES);                                                                        \
+    } while (0)
+        if (row_bytes <= 16384) {
+            // lanes per row: one 16-byte vector each up to a whole wavefront, four vectors each beyond
+            int lanes = 1;
+            while (lanes < 64 && static_cast<int64_t>(lanes) * 16 < row_bytes) lanes *= 2;
+            const int rpb = 256 / lanes;
+            const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer + rpb - 1) / rpb, 256 * 32));
+            AXHIP_ARG_ROWS(64, blocks, lanes);
+        } else if (row_bytes <= 65536) {
+            AXHIP_ARG_ROWS(256, static_cast<unsigned>(std::min<int64_t>(outer, 256 * 32)), 64);
         } else {
-            const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer, 256 * 8));
-            if (want_min) hipLaunchKernelGGL((argreduce_rows_kernel<true, 1024>), dim3(blocks), dim3(1024), 0, s, src, dtype, outer, axis, start, dst);
-            else hipLaunchKernelGGL((argreduce_rows_kernel<false, 1024>), dim3(blocks), dim3(1024), 0, s, src, dtype, outer, axis, start, dst);
+            AXHIP_ARG_ROWS(1024, static_cast<unsigned>(std::min<int64_t>(outer, 256 * 8)), 64);
         }
+#undef AXHIP_ARG_ROWS
+#undef AXHIP_ARG_ROWS_DT
+    } else if (inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
+        const int64_t ivecs = inner / (16 / es);
+        const bool wide = outer * ((ivecs + 31) / 32) >= 1024;
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
+#define AXHIP_ARG_VEC_TX(DT, TX)                                                                                                           \
+    do {                                                                                                                                   \
+        if (want_min) hipLaunchKernelGGL((argreduce_strided_vec_kernel<true, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, start, dst); \
+        else hipLaunchKernelGGL((argreduce_strided_vec_kernel<false, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, start, dst);         \
+    } while (0)
+#define AXHIP_ARG_VEC(DT)                                                                                                                  \
+    do {                                                                                                                                   \
+        if (wide) AXHIP_ARG_VEC_TX(DT, 32);                                                                                                \
+        else AXHIP_ARG_VEC_TX(DT, 8);                                                                                                      \
+    } while (0)
+        if (dtype == AXHIP_DTYPE_F32) AXHIP_ARG_VEC(AXHIP_DTYPE_F32);
+        else if (dtype == AXHIP_DTYPE_F16) AXHIP_ARG_VEC(AXHIP_DTYPE_F16);
+        else AXHIP_ARG_VEC(AXHIP_DTYPE_BF16);
+#undef AXHIP_ARG_VEC
+#undef AXHIP_ARG_VEC_TX
     } else {
         const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
         if (want_min) hipLaunchKernelGGL(argreduce_strided_kernel<true>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, start, dst);

@@ -112,6 +112,10 @@ Tensor sum(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = 
 Tensor mean(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
 Tensor max(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
 Tensor min(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+// Int64 index of the first occurrence of the extreme along one axis (include/axiom/operations.hpp:400-401); runs when
+// called, like scaled_dot_product_attention, on the materialised input
+Tensor argmax(const Tensor &x, int axis = -1, bool keep_dims = false);
+Tensor argmin(const Tensor &x, int axis = -1, bool keep_dims = false);
 
 // population variance, eps inside the square root; weight / bias may be empty tensors
 Tensor layer_norm(const Tensor &x, const Tensor &weight, const Tensor &bias, int axis = -1, float eps = 1e-5f);

@@ -108,6 +108,8 @@ class Tensor {
     Tensor mean(const std::vector<int> &axes, bool keep_dims = false) const;
     Tensor max(int axis = -1, bool keep_dims = false) const;
     Tensor min(int axis = -1, bool keep_dims = false) const;
+    Tensor argmax(int axis = -1, bool keep_dims = false) const;
+    Tensor argmin(int axis = -1, bool keep_dims = false) const;
     Tensor softmax(int axis = -1) const;
     Tensor log_softmax(int axis = -1) const;
     Tensor relu() const;

@@ -112,6 +112,40 @@ Tensor mean(const Tensor &x, const std::vector<int> &axes, bool keep) { return G
 Tensor max(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Max, x, axes, keep); }
 Tensor min(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Min, x, axes, keep); }
 
+namespace {
+// src/backends/cpu/cpu_operations.cpp:2157-2229 (shape rules) on the device kernel; the input is made contiguous
+// first, as the CPU path does (:2161)
+Tensor arg_reduce(const Tensor &x, int axis, bool keep_dims, bool want_min) {
+    const int nd = static_cast<int>(x.ndim());
+    if (nd == 0) throw ShapeError("argmax / argmin of a rank-0 tensor");
+    if (axis < 0) axis += nd;
+    if (axis < 0 || axis >= nd) throw ShapeError("argmax / argmin: axis out of range");
+    if (x.device() != Device::GPU)
+        throw RuntimeError("ops::argmax / argmin on CPU tensors: this library is the gfx950 GPU backend only; move the operand with .gpu()");
+    if (x.dtype() != DType::Float32 && x.dtype() != DType::Float16 && x.dtype() != DType::BFloat16)
+        throw TypeError("argmax / argmin: Float32, Float16 or BFloat16 input");
+    const Tensor src = x.ascontiguousarray(); // materialises a lazy input
+    const Shape &sh = src.shape();
+    size_t outer = 1, inner = 1;
+    Shape out_shape;
+    for (int d = 0; d < nd; ++d) {
+        if (d < axis) outer *= sh[d];
+        if (d > axis) inner *= sh[d];
+        if (d != axis) out_shape.push_back(sh[d]);
+        else if (keep_dims) out_shape.push_back(1);
+    }
+    if (sh[axis] == 0) throw ShapeError("argmax / argmin along an empty axis");
+    Tensor out(out_shape, DType::Int64, Device::GPU);
+    AXHIP_CALL(axhip_argreduce(static_cast<const char *>(src.storage()->raw()) + src.offset(), ::axiom::detail::to_axhip_dtype(src.dtype()),
+                               static_cast<int64_t>(outer), static_cast<int64_t>(sh[axis]), static_cast<int64_t>(inner), want_min ? 1 : 0,
+                               static_cast<int64_t *>(out.storage()->raw()), nullptr));
+    return out; // asynchronous; .cpu() / item() synchronise
+}
+} // namespace
+
+Tensor argmax(const Tensor &x, int axis, bool keep_dims) { return arg_reduce(x, axis, keep_dims, false); }
+Tensor argmin(const Tensor &x, int axis, bool keep_dims) { return arg_reduce(x, axis, keep_dims, true); }
+
 Tensor layer_norm(const Tensor &x, const Tensor &weight, const Tensor &bias, int axis, float eps) {
     const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(x.ndim()));
     for (const Tensor *p : {&weight, &bias})

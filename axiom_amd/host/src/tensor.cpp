@@ -356,6 +356,8 @@ Tensor Tensor::mean(int axis, bool keep_dims) const { return ops::mean(*this, {a
 Tensor Tensor::mean(const std::vector<int> &axes, bool keep_dims) const { return ops::mean(*this, axes, keep_dims); }
 Tensor Tensor::max(int axis, bool keep_dims) const { return ops::max(*this, {axis}, keep_dims); }
 Tensor Tensor::min(int axis, bool keep_dims) const { return ops::min(*this, {axis}, keep_dims); }
+Tensor Tensor::argmax(int axis, bool keep_dims) const { return ops::argmax(*this, axis, keep_dims); }
+Tensor Tensor::argmin(int axis, bool keep_dims) const { return ops::argmin(*this, axis, keep_dims); }
 Tensor Tensor::softmax(int axis) const { return ops::softmax(*this, axis); }
 Tensor Tensor::log_softmax(int axis) const { return ops::log_softmax(*this, axis); }
 Tensor Tensor::relu() const { return ops::relu(*this); }

@@ -481,6 +481,46 @@ GPU_TEST(CpuGpuParity, MatmulBroadcastsBatchDimensions) {
         }
 }
 
+// tests/test_cpu_gpu_parity.cpp:348-370 (argmax / argmin along axis 1 against the CPU scan) and the known answers of
+// tests/test_tensor_argmax_argmin.cpp:4-112
+GPU_TEST(CpuGpuParity, ArgmaxArgminParity) {
+    auto a = axtest::randn({37, 501}, 71);
+    std::vector<int64_t> want(37);
+    for (bool want_min : {false, true}) {
+        auto got = want_min ? ops::argmin(a.gpu(), 1, false) : ops::argmax(a.gpu(), 1, false);
+        EXPECT_EQ(got.dtype(), DType::Int64);
+        EXPECT_EQ(got.shape(), Shape({37}));
+        axo_argreduce(want_min, AXO_F32, a.typed_data<float>(), want.data(), 37, 501, 1);
+        auto host = got.cpu();
+        for (size_t i = 0; i < 37; ++i) EXPECT_EQ(host.typed_data<int64_t>()[i], want[i]);
+    }
+    // along axis 0 of a lazy chain's result, keep_dims
+    auto lazy = ops::relu(a.gpu()) * 2.0f;
+    auto got0 = lazy.argmax(0, true);
+    EXPECT_EQ(got0.shape(), Shape({1, 501}));
+    std::vector<float> chain(37 * 501);
+    for (size_t i = 0; i < chain.size(); ++i) chain[i] = std::max(a.typed_data<float>()[i], 0.0f) * 2.0f;
+    std::vector<int64_t> want0(501);
+    axo_argreduce(0, AXO_F32, chain.data(), want0.data(), 1, 37, 501);
+    auto host0 = got0.cpu();
+    for (size_t i = 0; i < 501; ++i) EXPECT_EQ(host0.typed_data<int64_t>()[i], want0[i]);
+    // known answers
+    const float v5[5] = {1.0f, 5.0f, 3.0f, 9.0f, 2.0f};
+    auto r = ops::argmax(Tensor::from_data(v5, {5}).gpu());
+    EXPECT_EQ(r.ndim(), 0u);
+    EXPECT_EQ(r.item<int64_t>(), 3);
+    const float m4[4] = {1.0f, 5.0f, 3.0f, 2.0f};
+    auto m = Tensor::from_data(m4, {2, 2}).gpu();
+    auto c0 = ops::argmin(m, 0).cpu();
+    EXPECT_EQ(c0.typed_data<int64_t>()[0], 0);
+    EXPECT_EQ(c0.typed_data<int64_t>()[1], 1);
+    // a transposed (non-contiguous) view gives what its contiguous copy gives (:117-131)
+    auto t3 = axtest::randn({3, 4, 5}, 72).gpu().transpose({0, 2, 1});
+    auto x1 = ops::argmax(t3, -1).cpu(), x2 = ops::argmax(t3.ascontiguousarray(), -1).cpu();
+    for (size_t i = 0; i < 15; ++i) EXPECT_EQ(x1.typed_data<int64_t>()[i], x2.typed_data<int64_t>()[i]);
+    EXPECT_THROW(ops::argmax(m, 2), ShapeError);
+}
+
 // ----------------------------------------------------------------- attention
 static std::tuple<Tensor, Tensor, Tensor> make_inputs(size_t B, size_t H, size_t Sq, size_t Skv, size_t D, DType dt = DType::Float32, uint64_t seed = 42) {
     return {axtest::randn({B, H, Sq, D}, seed, dt), axtest::randn({B, H, Skv, D}, seed + 1, dt), axtest::randn({B, H, Skv, D}, seed + 2, dt)};
