@@ -390,6 +390,19 @@ def bench_survey(torch, capi, stream, steps, warmup):
         run(f"logsoftmax(x*s)_{name}_{rows}x{cols}", P(t).op("mul", imm=0.5).row("logsoftmax").finish(torch))
         run(f"max(x)_{name}_{rows}x{cols}", P(t).finish(torch, "max"))
         del t
+    # argmax along the last axis (greedy decoding over logits) and along other axes of a contiguous array
+    for (outer, axis, inner), dt, name in (((16384, 4096, 1), bf, "bf16"), ((4096, 50304, 1), bf, "bf16"), ((8192, 8192, 1), f32, "f32"),
+                                           ((1 << 20, 64, 1), bf, "bf16"), ((64, 4096, 1024), bf, "bf16"), ((1, 4096, 16384), f32, "f32")):
+        t = rnd((outer, axis, inner), dt, 3.0)
+        out = torch.empty((outer * inner,), device="cuda", dtype=torch.int64)
+        code = capi.DTYPE_BF16 if dt == bf else capi.DTYPE_F32
+        torch.cuda.synchronize()
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_argreduce(t.data_ptr(), code, outer, axis, inner, 0, out.data_ptr(), sp)), steps, warmup)
+        nbytes = t.numel() * t.element_size() + out.numel() * 8
+        res[f"argmax_axis1_{name}_{outer}x{axis}x{inner}"] = {"kernel": "argreduce_rows" if inner == 1 else "argreduce_strided", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3,
+                                                               "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                                               "finite": bool(torch.equal(out.view(outer, inner), t.float().argmax(1)))}
+        del t, out
     return res
 
 
