@@ -718,6 +718,43 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     if (rc) return rc;
     hipStream_t s = resolve_stream(stream);
 
+    // The matrix-core kernels read both operands along k, in 16-byte vectors.  An operand stored the other way (A as
+    // [k, m], B as [k, n]: matmul(a, b) with a plain [k, n] right-hand side), or a reduction length that is not a whole
+    // number of vectors, leaves only the FMA kernel below, a hundred times slower on a large product.  Such a product
+    // is repacked first, into stream-ordered temporary memory (freed in stream order behind the product): the operand
+    // that lies the other way is transposed; an unaligned k is zero-padded to the next multiple of 64 in both operands.
+    const int64_t kvec = p.dtype == AXHIP_DTYPE_F32 ? 4 : 8;
+    const bool pad_k = p.k % kvec != 0;
+    if ((p.trans_a || !p.trans_b || pad_k) && p.k >= 32 &&
+        2.0 * static_cast<double>(p.m) * static_cast<double>(p.n) * static_cast<double>(p.k) * static_cast<double>(p.batch) >= double(1 << 30)) { // (about 70 us on the FMA kernel)
+        const int64_t es = p.dtype == AXHIP_DTYPE_F32 ? 4 : 2, kp = pad_k ? (p.k + 63) / 64 * 64 : p.k;
+        AxhipGemmParams q = p;
+        q.k = kp;
+        void *ta = nullptr, *tb = nullptr;
+        // a contiguous [copies, rows, kp] image of an operand whose element (row, kk) lies at row * rs + kk * cs
+        auto repacked = [&](const void *src, int64_t rows, int64_t rs, int64_t cs, int64_t batch_stride, void **out) -> int {
+            const int64_t copies = batch_stride == 0 ? 1 : p.batch;
+            AXHIP_CHECK_HIP(hipMallocAsync(out, static_cast<size_t>(copies * rows * kp * es), s));
+            const int64_t shape[3] = {copies, rows, p.k}, strides[3] = {batch_stride, rs, cs}, before[3] = {0, 0, 0}, after[3] = {0, 0, kp - p.k};
+            if (pad_k) return axhip_pad(src, *out, p.dtype, 3, shape, strides, before, after, 0.0, stream);
+            return axhip_strided_copy(src, p.dtype, *out, p.dtype, 3, shape, strides, stream);
+        };
+        if (p.trans_a || pad_k) {
+            rc = repacked(a, p.m, p.trans_a ? 1 : p.lda, p.trans_a ? p.lda : 1, p.stride_a, &ta);
+            q.trans_a = 0; q.lda = kp; q.stride_a = p.stride_a == 0 ? 0 : p.m * kp;
+        }
+        if (!rc && (!p.trans_b || pad_k)) {
+            rc = repacked(b, p.n, p.trans_b ? p.ldb : 1, p.trans_b ? 1 : p.ldb, p.stride_b, &tb);
+            q.trans_b = 1; q.ldb = kp; q.stride_b = p.stride_b == 0 ? 0 : p.n * kp;
+        }
+        if (!rc) rc = axhip_gemm(ta ? ta : a, tb ? tb : b, c, &q, stream);
+        hipError_t freed = ta ? hipFreeAsync(ta, s) : hipSuccess;
+        if (tb && freed == hipSuccess) freed = hipFreeAsync(tb, s);
+        else if (tb) (void)hipFreeAsync(tb, s);
+        if (!rc) AXHIP_CHECK_HIP(freed);
+        return rc;
+    }
+
     GemmArgs g{};
     g.a = a; g.b = b; g.c = c; g.bias = p.bias; g.residual = p.residual;
     g.dtype = p.dtype; g.epilogue = p.epilogue_op;

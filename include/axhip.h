@@ -289,7 +289,12 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
  * as matmul(x, W, false, true) + bias (src/nn/linear.cpp:15-27).
  * C[b] = op(A[b]) * op(B[b]) (+ bias[N]) (+ residual[b]) for b < batch;
  * row-major, lda/ldb/ldc and batch strides in elements (stride 0 shares an
- * operand across the batch).  fp32 accumulation; bf16/f16 on MFMA. */
+ * operand across the batch).  fp32 accumulation; bf16/f16 on MFMA.
+ * The matrix-core kernels read both operands along k (trans_a = 0,
+ * trans_b = 1: x W^T) in 16-byte vectors.  On a large product an operand
+ * stored the other way is transposed first, and a k that is not a multiple of
+ * 8 (fp32: 4) zero-padded, into temporary memory that the library takes and
+ * returns in stream order (hipMallocAsync / hipFreeAsync on `stream`). */
 typedef struct {
     int32_t dtype;
     int32_t trans_a, trans_b;

@@ -120,6 +120,32 @@ def test_half_ring_path_matches_fp64(dt, M, N, K, extras):
     assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
 
 
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("ta,tb,K", [(False, False, 264), (True, False, 264), (True, True, 264), (False, True, 263), (True, False, 301)],
+                         ids=["nn", "tn", "tt", "nt_k263", "tn_k301"])
+def test_large_products_with_operands_not_along_k(dt, ta, tb, K):
+    """Large products whose A is stored [k, m] and / or whose B is stored [k, n], or whose k is not a whole number of
+    16-byte vectors: the library repacks such operands into temporary memory (transposed, k zero-padded) and runs the
+    k-contiguous kernels; same bar as those.  Batched, with a shared B."""
+    M, N, nb = 1040, 784, 3  # (above the size from which the library repacks)
+    g = axo.PCG64(M + N + int(ta) + 2 * int(tb))
+    A = axo.to_bits(g.normal((nb, K, M) if ta else (nb, M, K)), dt)
+    B = axo.to_bits(g.normal((N, K) if tb else (K, N)) * 0.05, dt)
+    bias = axo.to_bits(g.normal((N,)) * 0.1, dt)
+    got = axo.to_f32(gh.gemm(A, B, dt, trans_a=ta, trans_b=tb, bias=bias, epilogue="relu"), dt)
+    a64, b64 = axo.to_f32(A, dt).astype(np.float64), axo.to_f32(B, dt).astype(np.float64)
+    want = np.maximum((a64.transpose(0, 2, 1) if ta else a64) @ (b64.T if tb else b64) + axo.to_f32(bias, dt), 0.0)
+    tol = 1e-4 + 1e-4 * np.abs(want) if dt == F32 else 2e-2 + 2.0**-8 * np.abs(want)
+    assert np.all(np.abs(got - want) <= tol)
+    # per-batch B as well
+    Bb = axo.to_bits(g.normal((nb, N, K) if tb else (nb, K, N)) * 0.05, dt)
+    got = axo.to_f32(gh.gemm(A, Bb, dt, trans_a=ta, trans_b=tb), dt)
+    bb64 = axo.to_f32(Bb, dt).astype(np.float64)
+    want = (a64.transpose(0, 2, 1) if ta else a64) @ (bb64.transpose(0, 2, 1) if tb else bb64)
+    tol = 1e-4 + 1e-4 * np.abs(want) if dt == F32 else 2e-2 + 2.0**-8 * np.abs(want)
+    assert np.all(np.abs(got - want) <= tol)
+
+
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_seeded_random_shapes_match_fp64(dt):
     """Forty seeded random products per dtype, shaped to land on every kernel and tile shape (matrix-core ring tiles,
