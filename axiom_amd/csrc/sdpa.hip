@@ -95,8 +95,13 @@ __device__ __forceinline__ uint2_t lds_read_tr16(const uint16_t *p) {
     return __builtin_bit_cast(uint2_t, v);
 }
 
+// D = 256: the two K and two V tile buffers (138 KiB) are dynamic LDS, one work-group per CU, one wave per SIMD
+// with the registers that go with it (the output accumulators alone are 128).
+template <int D> constexpr size_t sdpa_mfma_lds_bytes() { return 2 * BN * ((D + 8) + (D + 32)) * 2; }
+extern __shared__ __attribute__((aligned(16))) unsigned char sdpa_dyn_lds[];
+
 template <bool BF16, int D, bool HAS_MASK>
-__global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const SdpaArgs a) {
     constexpr int KS_STRIDE = D + 8;   // K row stride (elements): +16 B shifts consecutive rows by 4 banks
     constexpr int VS_STRIDE = D + 32;  // V row stride: +64 B shifts rows by 16 banks, what the 4-row transpose reads need
     constexpr int KT = D / 16;         // k-steps of the first product
@@ -104,8 +109,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
     constexpr int KCH = D / 8;         // 16-byte chunks per K/V row
     constexpr int NLD = BN * KCH / 256 > 0 ? BN * KCH / 256 : 1; // 16-byte chunks per thread per tile
     constexpr int ROWS_PER_PASS = 256 / KCH; // rows covered by one chunk pass of the whole workgroup
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][BN * KS_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[2][BN * VS_STRIDE];
+    constexpr int KBUF = BN * KS_STRIDE, VBUF = BN * VS_STRIDE; // elements per tile buffer
+    __shared__ __attribute__((aligned(16))) uint16_t Ks_static[D > 128 ? 8 : 2 * KBUF];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs_static[D > 128 ? 8 : 2 * VBUF];
+    uint16_t *const Ks = D > 128 ? reinterpret_cast<uint16_t *>(sdpa_dyn_lds) : Ks_static;
+    uint16_t *const Vs = D > 128 ? reinterpret_cast<uint16_t *>(sdpa_dyn_lds) + 2 * KBUF : Vs_static;
 
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
@@ -189,8 +197,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
 #pragma unroll
             for (int n = 0; n < NLD; ++n) {
                 const int row = ld_row + n * ROWS_PER_PASS;
-                *reinterpret_cast<uint4_t *>(&Ks[buf][row * KS_STRIDE + 8 * ld_cc]) = kreg[n];
-                *reinterpret_cast<uint4_t *>(&Vs[buf][row * VS_STRIDE + 8 * ld_cc]) = vreg[n];
+                *reinterpret_cast<uint4_t *>(&Ks[buf * KBUF + row * KS_STRIDE + 8 * ld_cc]) = kreg[n];
+                *reinterpret_cast<uint4_t *>(&Vs[buf * VBUF + row * VS_STRIDE + 8 * ld_cc]) = vreg[n];
             }
         }
     };
@@ -219,7 +227,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs a) {
 
         // a wave whose last query row precedes this tile has nothing to add
         if (!(a.causal && kv0 > qw0 + 31)) {
-            const uint16_t *Kb = Ks[buf], *Vb = Vs[buf];
+            const uint16_t *Kb = Ks + buf * KBUF, *Vb = Vs + buf * VBUF;
 
             // explicit mask: the eight 4-byte words that cover this lane's keys of the tile (8 runs of 4 consecutive
             // keys), requested ahead of the score MFMAs; needs whole tiles and 4-byte aligned mask rows
@@ -1255,8 +1263,9 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
     if (p.batch == 0 || p.heads == 0 || p.seq_q == 0 || p.head_dim == 0) return SdpaKind::EMPTY;
     const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
     const bool d_ok = p.head_dim == 32 || p.head_dim == 64 || p.head_dim == 128;
-    // the 16-bit pipelined kernels also take the multiples of 8 between their compiled sizes (zeros in the missing dims)
-    if (half && (d_ok || (p.head_dim > 32 && p.head_dim < 128 && p.head_dim % 8 == 0))) {
+    // the 16-bit pipelined kernels also take the multiples of 8 between their compiled sizes (zeros in the missing dims);
+    // head_dim 256 has the register-staged 16-bit kernel
+    if (half && (d_ok || p.head_dim == 256 || (p.head_dim > 32 && p.head_dim < 128 && p.head_dim % 8 == 0))) {
         bool ok = true;
         // 16-byte vector access to every row of q/k/v, 8-byte to o
         for (int i = 0; i < 3; ++i)
@@ -1292,10 +1301,19 @@ int validate(const AxhipSdpaParams &p) {
     return AXHIP_OK;
 }
 
-template <bool BF16, int D> void launch_mfma(const SdpaArgs &a, hipStream_t s) {
+template <bool BF16, int D> int launch_mfma(const SdpaArgs &a, hipStream_t s) {
     const unsigned grid = static_cast<unsigned>(a.nqb) * static_cast<unsigned>(a.B * a.H);
-    if (a.mask) hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, true>), dim3(grid), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, false>), dim3(grid), dim3(256), 0, s, a);
+    constexpr size_t lds = D > 128 ? sdpa_mfma_lds_bytes<D>() : 0;
+    if constexpr (D > 128) {
+        static const bool configured = [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_mfma_kernel<BF16, D, true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
+                   hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_mfma_kernel<BF16, D, false>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
+        }();
+        AXHIP_REQUIRE(configured, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: cannot reserve %zu bytes of LDS", lds);
+    }
+    if (a.mask) hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, true>), dim3(grid), dim3(256), lds, s, a);
+    else hipLaunchKernelGGL((sdpa_mfma_kernel<BF16, D, false>), dim3(grid), dim3(256), lds, s, a);
+    return AXHIP_OK;
 }
 
 template <int D, int SPLIT> int launch_mfma_f32(const SdpaArgs &a, hipStream_t s) {
@@ -1392,7 +1410,8 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
         switch (p.head_dim) {
-        case 32: bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
+        case 32: rc = bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
+        case 256: rc = bf ? launch_mfma<true, 256>(a, s) : launch_mfma<false, 256>(a, s); break;
         case 64:
         default: {
             // 8-wave work-groups (256 query rows, each K/V tile fetched once for all of them) when that still gives

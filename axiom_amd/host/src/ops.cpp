@@ -281,10 +281,13 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
     // output slice to be small change against the FMA kernel they avoid (two orders of magnitude slower); this is
     // where the reference's decomposed fallback for such sizes (flash_attention_dispatch.mm:180-196) ends up.
     // (16-bit head sizes that are multiples of 8 above 32 need none of this: the kernels take them as they are)
-    const bool kernel_takes_it = query.dtype() != DType::Float32 && D > 32 && D % 8 == 0;
-    if (D != 32 && D != 64 && D > 0 && D < 128 && !kernel_takes_it && static_cast<double>(B) * H * Sq * Skv * D >= double(1 << 24) &&
-        (query.dtype() == DType::Float32 || query.dtype() == DType::Float16 || query.dtype() == DType::BFloat16)) {
-        const size_t Dp = D < 32 ? 32 : D < 64 ? 64 : 128;
+    // 16-bit head sizes between 128 and 256 go to the head_dim-256 kernel the same way.
+    const bool half = query.dtype() == DType::Float16 || query.dtype() == DType::BFloat16;
+    const bool kernel_takes_it = half && D > 32 && D < 128 && D % 8 == 0;
+    const bool below_a_kernel = (D > 0 && D < 128 && D != 32 && D != 64) || (half && D > 128 && D < 256);
+    if (below_a_kernel && !kernel_takes_it && static_cast<double>(B) * H * Sq * Skv * D >= double(1 << 24) &&
+        (query.dtype() == DType::Float32 || half)) {
+        const size_t Dp = D < 32 ? 32 : D < 64 ? 64 : D < 128 ? 128 : 256;
         const std::vector<std::pair<size_t, size_t>> widen{{0, 0}, {0, 0}, {0, 0}, {0, Dp - D}};
         auto on_gpu = [](const Tensor &t) { return t.device() == Device::GPU ? t : t.to(Device::GPU); };
         const float sc = scale > 0.0f ? scale : 1.0f / std::sqrt(static_cast<float>(D));
@@ -332,9 +335,9 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
     // Shapes no attention kernel takes (head sizes above 256; 65 536 or more (batch, head) slices on the FMA kernel)
     // are composed from the matrix product, masking and softmax kernels, as the reference composes what its own
     // kernels do not take (src/backends/metal/flash_attention_dispatch.mm:125-162, 180-196).
-    // Head sizes between 129 and 256 have the FMA kernel only (a few TFLOP/s): once the problem is large enough to
+    // fp32 head sizes between 129 and 256 have the FMA kernel only (a few TFLOP/s): once the problem is large enough to
     // notice, and its score matrix small enough to hold (32 GiB), the composed form on the matrix-core GEMM is two
-    // orders of magnitude faster.
+    // orders of magnitude faster.  (16-bit: 256 has a matrix-core kernel, the sizes below it were padded to it above.)
     const double work = static_cast<double>(B) * H * Sq * Skv * D, score_bytes = static_cast<double>(B) * H * Sq * Skv * static_cast<double>(q.itemsize());
     const bool wide_head = D > 128 && work >= double(1 << 24) && score_bytes <= 32.0 * double(1 << 30);
     if (tl_sdpa_kernel == "invalid" || (tl_sdpa_kernel == "generic" && (B * H >= 65536 || wide_head))) {

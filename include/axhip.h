@@ -73,10 +73,12 @@ int axhip_stream_sync(void *stream);
  * src/backends/cpu/flash_attention_cpu.cpp:78-89).  scale <= 0 means
  * 1/sqrt(D) (src/tensor/operations.cpp:4013-4015).  A row whose keys are all
  * masked yields zeros.  fp32 accumulation; output in `dtype`.
- * bf16/f16 with D in {32,64,128} run on MFMA; everything else (fp32, other
- * head sizes up to 256) runs on the generic fp32-FMA kernel, which takes the
+ * bf16/f16 with D in {32, 64, 128, 256} or a multiple of 8 between 32 and 128,
+ * and fp32 with D in {32, 64, 128}, run on MFMA (16-byte aligned base
+ * pointers, strides that are multiples of 8 elements; fp32: 4); everything
+ * else up to D = 256 runs on the generic fp32-FMA kernel, which takes the
  * place of the reference's decomposed_attention fallback
- * (flash_attention_dispatch.mm:125-162). */
+ * (flash_attention_dispatch.mm:125-162).  axhip_sdpa_kernel_name tells which. */
 typedef struct {
     int32_t dtype;
     int32_t batch, heads, seq_q, seq_kv, head_dim;

@@ -43,7 +43,9 @@ HALF_CASES = [  # (B,H,Sq,Skv,D, causal, mask)
     (1, 3, 257, 511, 128, False, "mod3"), (1, 20, 1500, 1500, 64, False, None),  # Whisper encoder shape
     (2, 8, 1024, 1024, 128, True, None), (1, 1, 8, 8, 48, False, None), (1, 1, 64, 64, 96, True, None),
     # head_dim 64 with enough (batch, head, block) units for the 8-wave work-groups: causal pairs, ragged blocks, a mask
-    (2, 64, 600, 600, 64, True, None), (1, 128, 300, 520, 64, False, "mod3")]
+    (2, 64, 600, 600, 64, True, None), (1, 128, 300, 520, 64, False, "mod3"),
+    # head_dim 256 (16-bit: the register-staged matrix-core kernel with its tiles in dynamic LDS)
+    (1, 2, 8, 8, 256, False, None), (2, 3, 130, 200, 256, True, None), (1, 2, 300, 300, 256, False, "mod3"), (1, 4, 257, 129, 256, False, "mod3"), (1, 2, 200, 333, 256, True, None)]
 
 
 @pytest.mark.parametrize("case", HALF_CASES, ids=lambda c: "x".join(str(x) for x in c))
@@ -244,6 +246,33 @@ def test_full_size_causal_bf16_properties():
         want = axo.sdpa(qs, ks, vs, F32, -1.0, True)
         err = np.max(np.abs(gf[b:b + 1, h:h + 1] - want))
         assert err < 2e-2, (sl, err)
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+def test_head_dim_256_seeded_random_problems_match_fp64(dt):
+    """Twelve seeded random head_dim-256 problems per 16-bit type (ragged lengths, causal, shared and per-(batch, head)
+    masks of either alignment, explicit scales) on the matrix-core kernel, against float64."""
+    r = np.random.default_rng(256 + dt)
+    for case in range(12):
+        B, H = int(r.integers(1, 3)), int(r.integers(1, 5))
+        Sq = int(r.integers(1, 400))
+        Skv = Sq if r.integers(0, 2) else int(r.integers(1, 400))
+        if r.integers(0, 3) == 0:
+            Skv = 4 * max(1, Skv // 4)
+        causal = bool(r.integers(0, 2))
+        mkind = int(r.integers(0, 3))
+        scale = float(r.choice([-1.0, 2.0 / math.sqrt(256), 0.03]))
+        q, k, v = inputs(B, H, Sq, Skv, 256, dt, seed=300 + case)
+        mask = None
+        if mkind:
+            shape = (Sq, Skv) if mkind == 1 else (B, H, Sq, Skv)
+            mask = (r.random(shape) < 0.25).astype(np.uint8) * r.choice(np.array([1, 7, 255], np.uint8), shape)
+        got, kern = gh.sdpa(q, k, v, dt, scale, causal, mask)
+        assert kern == f"mfma_{'bf16' if dt == BF16 else 'f16'}_d256"
+        sc = 1 / math.sqrt(256) if scale < 0 else scale
+        want = naive_attention64(*(axo.to_f32(t, dt) for t in (q, k, v)), sc, causal, mask)
+        err = np.max(np.abs(axo.to_f32(got, dt).astype(np.float64) - want))
+        assert err < 2e-2, (case, B, H, Sq, Skv, causal, mkind, scale, float(err))
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
