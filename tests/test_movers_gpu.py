@@ -103,7 +103,10 @@ def test_fill(dt):
 
 @pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape,before,after", [((5,), (2,), (3,)), ((3, 4), (0, 1), (2, 0)), ((2, 3, 50), (0, 0, 1), (0, 0, 1)),
-                                                ((2, 1, 3, 4), (1, 0, 2, 0), (0, 3, 0, 5))])
+                                                ((2, 1, 3, 4), (1, 0, 2, 0), (0, 3, 0, 5)),
+                                                # innermost output extents of whole 16-byte vectors: one store per vector
+                                                ((3, 5, 27), (1, 0, 2), (0, 2, 3)), ((2, 2, 30, 48), (0, 0, 0, 0), (0, 0, 0, 16)), ((7, 1001), (0, 0), (0, 23)),
+                                                ((64,), (0,), (0,))])
 def test_pad_matches_numpy(dt, shape, before, after):
     x = sample(shape, dt, 11)
     value = -2.5
@@ -127,6 +130,21 @@ def test_pad_of_a_transposed_view():
     capi.check(capi.lib().axhip_pad(d.data_ptr(), out.data_ptr(), F32, 2, i64(view.shape), i64(elem_strides(view)), i64([1, 0]), i64([1, 2]), 0.0, None))
     gh.sync()
     assert np.array_equal(gh.to_host(out, np.float32), want)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+def test_pad_of_a_transposed_operand_to_an_aligned_reduction_length(dt):
+    """What the matrix product's repacking asks for: a [k, n] operand read as its (batch, n, k) transpose, k padded
+    with zeros to the next multiple of 64."""
+    base = sample((2, 301, 40), dt, 21)
+    view = base.transpose(0, 2, 1)
+    want = np.pad(view, [(0, 0), (0, 0), (0, 19)])
+    d = gh.to_dev(base)
+    out = gh.empty_dev(want.shape, dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_pad(d.data_ptr(), out.data_ptr(), dt, 3, i64(view.shape), i64(elem_strides(view)), i64([0, 0, 0]), i64([0, 0, 19]), 0.0, None))
+    gh.sync()
+    assert np.array_equal(gh.to_host(out, base.dtype), want)
 
 
 @pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
