@@ -97,6 +97,8 @@ __device__ __forceinline__ uint2_t lds_read_tr16(const uint16_t *p) {
 
 // D = 256: the two K and two V tile buffers (138 KiB) are dynamic LDS, one work-group per CU, one wave per SIMD
 // with the registers that go with it (the output accumulators alone are 128).
+// A head size below D (a.D, a multiple of 8) runs with zeros in the missing dims: Q fragments and K/V chunks beyond
+// a.D are not fetched, the output keeps a.D columns.
 template <int D> constexpr size_t sdpa_mfma_lds_bytes() { return 2 * BN * ((D + 8) + (D + 32)) * 2; }
 extern __shared__ __attribute__((aligned(16))) unsigned char sdpa_dyn_lds[];
 
@@ -150,12 +152,14 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
     // K / V are fetched through buffer descriptors: rows past the end of the
     // sequence read as zero instead of touching memory.
     const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
+    const int dv = a.D; // the head size in memory (<= D, a multiple of 8)
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(K), 0, a.Skv > 0 ? (a.Skv - 1) * krow_bytes + D * 2 : 0, 0x00020000);
+        const_cast<uint16_t *>(K), 0, a.Skv > 0 ? (a.Skv - 1) * krow_bytes + dv * 2 : 0, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(V), 0, a.Skv > 0 ? (a.Skv - 1) * vrow_bytes + D * 2 : 0, 0x00020000);
+        const_cast<uint16_t *>(V), 0, a.Skv > 0 ? (a.Skv - 1) * vrow_bytes + dv * 2 : 0, 0x00020000);
     const int ld_row = tid / KCH, ld_cc = tid % KCH; // this thread's chunk in pass 0
     const bool ld_active = KCH * BN >= 256 || tid < KCH * BN;
+    const bool ld_fetch = ld_active && ld_cc * 8 < dv; // (a chunk beyond the head size is staged as zeros)
     const int k_voff = ld_row * krow_bytes + ld_cc * 16, v_voff = ld_row * vrow_bytes + ld_cc * 16;
 
     // Q^T fragments (B operand): lane holds Q[q][16t + 8g .. +8]
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
         qf[t] = uint4_t{0, 0, 0, 0};
-        if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
+        if (q_ok && 16 * t + 8 * g < dv) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
     }
 
     float16_t oacc[DT];
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
             const int row0 = tile * BN + n * ROWS_PER_PASS;
             kreg[n] = uint4_t{0, 0, 0, 0};
             vreg[n] = uint4_t{0, 0, 0, 0};
-            if (ld_active) {
+            if (ld_fetch) {
                 kreg[n] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, k_voff + row0 * krow_bytes, 0, 0);
                 vreg[n] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, v_voff + row0 * vrow_bytes, 0, 0);
             }
@@ -348,7 +352,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
                 const int d = dt * 32 + i4 * 8 + g * 4;
                 uint2_t w = {pack2<BF16>(oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv),
                              pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
-                *reinterpret_cast<uint2_t *>(orow + d) = w;
+                if (d < dv) *reinterpret_cast<uint2_t *>(orow + d) = w;
             }
     }
 }
@@ -1264,8 +1268,8 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
     const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
     const bool d_ok = p.head_dim == 32 || p.head_dim == 64 || p.head_dim == 128;
     // the 16-bit pipelined kernels also take the multiples of 8 between their compiled sizes (zeros in the missing dims);
-    // head_dim 256 has the register-staged 16-bit kernel
-    if (half && (d_ok || p.head_dim == 256 || (p.head_dim > 32 && p.head_dim < 128 && p.head_dim % 8 == 0))) {
+    // so does the register-staged head_dim-256 kernel (136 .. 256)
+    if (half && (d_ok || (p.head_dim > 32 && p.head_dim <= 256 && p.head_dim % 8 == 0))) {
         bool ok = true;
         // 16-byte vector access to every row of q/k/v, 8-byte to o
         for (int i = 0; i < 3; ++i)
@@ -1409,10 +1413,9 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         a.nqb = (p.seq_q + BM - 1) / BM;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
-        switch (p.head_dim) {
+        switch (p.head_dim <= 32 ? 32 : p.head_dim > 128 ? 256 : 64) {
         case 32: rc = bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
         case 256: rc = bf ? launch_mfma<true, 256>(a, s) : launch_mfma<false, 256>(a, s); break;
-        case 64:
         default: {
             // 8-wave work-groups (256 query rows, each K/V tile fetched once for all of them) when that still gives
             // every CU a work-group; 4-wave work-groups (128 rows, two per CU) for shorter or narrower problems

@@ -45,7 +45,9 @@ HALF_CASES = [  # (B,H,Sq,Skv,D, causal, mask)
     # head_dim 64 with enough (batch, head, block) units for the 8-wave work-groups: causal pairs, ragged blocks, a mask
     (2, 64, 600, 600, 64, True, None), (1, 128, 300, 520, 64, False, "mod3"),
     # head_dim 256 (16-bit: the register-staged matrix-core kernel with its tiles in dynamic LDS)
-    (1, 2, 8, 8, 256, False, None), (2, 3, 130, 200, 256, True, None), (1, 2, 300, 300, 256, False, "mod3"), (1, 4, 257, 129, 256, False, "mod3"), (1, 2, 200, 333, 256, True, None)]
+    (1, 2, 8, 8, 256, False, None), (2, 3, 130, 200, 256, True, None), (1, 2, 300, 300, 256, False, "mod3"), (1, 4, 257, 129, 256, False, "mod3"), (1, 2, 200, 333, 256, True, None),
+    # head sizes between 128 and 256 on the head_dim-256 kernel, zeros in the missing dims
+    (1, 2, 130, 130, 192, True, None), (2, 2, 100, 257, 136, False, "mod3"), (1, 3, 64, 64, 248, False, None)]
 
 
 @pytest.mark.parametrize("case", HALF_CASES, ids=lambda c: "x".join(str(x) for x in c))
@@ -162,6 +164,18 @@ def test_head_sizes_between_the_compiled_ones(dt):
     assert np.all(gf[..., D:] == 7.0)
     qf, kf, vf = (axo.to_f32(t, dt)[..., :D].transpose(0, 2, 1, 3) for t in packed)
     want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), False)
+    assert np.max(np.abs(gf[..., :D].transpose(0, 2, 1, 3) - want)) < 2e-2
+    # and rows of 192 inside rows of 256 (the head_dim-256 kernel)
+    B, S, H, D, W = 1, 90, 2, 192, 256
+    packed = [axo.to_bits(g.normal((B, S, H, W)), dt) for _ in range(3)]
+    st = (S * H * W, W, H * W)
+    out_init = axo.to_bits(np.full((B, S, H, W), 7.0, np.float32), dt)
+    got, kern = gh.sdpa(*packed, dt, -1.0, True, None, q_strides=st, k_strides=st, v_strides=st, o_strides=st, shape=(B, H, S, S, D), out_init=out_init)
+    assert kern == f"mfma_{tag}_d192"
+    gf = axo.to_f32(got, dt).reshape(B, S, H, W)
+    assert np.all(gf[..., D:] == 7.0)
+    qf, kf, vf = (axo.to_f32(t, dt)[..., :D].transpose(0, 2, 1, 3) for t in packed)
+    want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), True)
     assert np.max(np.abs(gf[..., :D].transpose(0, 2, 1, 3) - want)) < 2e-2
 
 
