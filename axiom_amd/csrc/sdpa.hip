@@ -872,17 +872,23 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
 
     // K / V through buffer descriptors: rows past the end of the sequence read as zero
     const int krow_bytes = static_cast<int>(a.ks[2]) * 4, vrow_bytes = static_cast<int>(a.vs[2]) * 4;
-    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(K), 0, (a.Skv - 1) * krow_bytes + D * 4, 0x00020000);
-    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(V), 0, (a.Skv - 1) * vrow_bytes + D * 4, 0x00020000);
+    // A head size below D (a.D, a multiple of 4) runs with zeros in the missing dims: the lanes that would fetch a
+    // chunk beyond it aim past the descriptors' ends (they stage zeros), Q fragments there stay zero, the output keeps
+    // a.D columns.
+    const int dv = a.D;
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(K), 0, (a.Skv - 1) * krow_bytes + dv * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(V), 0, (a.Skv - 1) * vrow_bytes + dv * 4, 0x00020000);
     const int ld_row = tid / KCH, ld_cc = tid % KCH;
-    const int k_voff = ld_row * krow_bytes + ld_cc * 16, v_voff = ld_row * vrow_bytes + ld_cc * 16;
+    const bool ld_inside = ld_cc * 4 < dv;
+    const int k_voff = ld_inside ? ld_row * krow_bytes + ld_cc * 16 : static_cast<int>(0x80000000u);
+    const int v_voff = ld_inside ? ld_row * vrow_bytes + ld_cc * 16 : static_cast<int>(0x80000000u);
 
     // Q^T fragments (B operand): lane holds Q[q][8 j + 4 g .. + 3]; component c of fragment j meets K's component c
     float4_t qf[QJ];
 #pragma unroll
     for (int j = 0; j < QJ; ++j) {
         qf[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        if (q_ok) qf[j] = *reinterpret_cast<const float4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 8 * j + 4 * g);
+        if (q_ok && 8 * j + 4 * g < dv) qf[j] = *reinterpret_cast<const float4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 8 * j + 4 * g);
     }
 
     float16_t oacc[DT];
@@ -1081,7 +1087,7 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
                     const float4_t w = {oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv, oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv};
-                    *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
+                    if (dt * 32 + i4 * 8 + g * 4 < dv) *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
                 }
         }
     } else {
@@ -1126,7 +1132,7 @@ __global__ __launch_bounds__(256) void sdpa_mfma_f32_kernel(const SdpaArgs a) {
                         acc[0] += sc[p] * t[0]; acc[1] += sc[p] * t[1]; acc[2] += sc[p] * t[2]; acc[3] += sc[p] * t[3];
                     }
                     const float4_t w = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
-                    *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
+                    if (dt * 32 + i4 * 8 + g * 4 < dv) *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
                 }
         }
     }
@@ -1266,10 +1272,9 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, const void *v, const void *o) {
     if (p.batch == 0 || p.heads == 0 || p.seq_q == 0 || p.head_dim == 0) return SdpaKind::EMPTY;
     const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
-    const bool d_ok = p.head_dim == 32 || p.head_dim == 64 || p.head_dim == 128;
     // the 16-bit pipelined kernels also take the multiples of 8 between their compiled sizes (zeros in the missing dims);
-    // so does the register-staged head_dim-256 kernel (136 .. 256)
-    if (half && (d_ok || (p.head_dim > 32 && p.head_dim <= 256 && p.head_dim % 8 == 0))) {
+    // so do the register-staged head_dim-32 and head_dim-256 kernels (8 .. 24, 136 .. 256)
+    if (half && p.head_dim <= 256 && p.head_dim % 8 == 0) {
         bool ok = true;
         // 16-byte vector access to every row of q/k/v, 8-byte to o
         for (int i = 0; i < 3; ++i)
@@ -1280,7 +1285,8 @@ SdpaKind pick_kernel(const AxhipSdpaParams &p, const void *q, const void *k, con
         ok = ok && (!q || aligned16(q)) && (!k || aligned16(k)) && (!v || aligned16(v)) && (!o || aligned16(o));
         if (ok) return SdpaKind::MFMA;
     }
-    if (p.dtype == AXHIP_DTYPE_F32 && d_ok && sdpa_f32_mfma) {
+    // fp32: every multiple of 4 up to 128, as the next of 32 / 64 / 128
+    if (p.dtype == AXHIP_DTYPE_F32 && p.head_dim <= 128 && p.head_dim % 4 == 0 && sdpa_f32_mfma) {
         bool ok = true;
         for (int i = 0; i < 3; ++i) // 16-byte vector access to every row
             ok = ok && p.q_strides[i] % 4 == 0 && p.k_strides[i] % 4 == 0 && p.v_strides[i] % 4 == 0 && p.o_strides[i] % 4 == 0;
@@ -1474,7 +1480,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         const int bmw = 128 / split;
         a.nqb = (p.seq_q + bmw - 1) / bmw;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
-        rc = p.head_dim == 32 ? launch_mfma_f32_d<32>(a, split, s) : p.head_dim == 64 ? launch_mfma_f32_d<64>(a, split, s) : launch_mfma_f32_d<128>(a, split, s);
+        rc = p.head_dim <= 32 ? launch_mfma_f32_d<32>(a, split, s) : p.head_dim <= 64 ? launch_mfma_f32_d<64>(a, split, s) : launch_mfma_f32_d<128>(a, split, s);
         if (rc) return rc;
     } else {
         a.nqb = (p.seq_q + GM - 1) / GM;

@@ -283,7 +283,7 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
     // (16-bit head sizes that are multiples of 8 above 32 need none of this: the kernels take them as they are)
     // 16-bit head sizes between 128 and 256 go to the head_dim-256 kernel the same way.
     const bool half = query.dtype() == DType::Float16 || query.dtype() == DType::BFloat16;
-    const bool kernel_takes_it = half && D > 32 && D <= 256 && D % 8 == 0;
+    const bool kernel_takes_it = (half && D <= 256 && D % 8 == 0) || (query.dtype() == DType::Float32 && D <= 128 && D % 4 == 0);
     const bool below_a_kernel = (D > 0 && D < 128 && D != 32 && D != 64) || (half && D > 128 && D < 256);
     if (below_a_kernel && !kernel_takes_it && static_cast<double>(B) * H * Sq * Skv * D >= double(1 << 24) &&
         (query.dtype() == DType::Float32 || half)) {

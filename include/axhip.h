@@ -73,8 +73,8 @@ int axhip_stream_sync(void *stream);
  * src/backends/cpu/flash_attention_cpu.cpp:78-89).  scale <= 0 means
  * 1/sqrt(D) (src/tensor/operations.cpp:4013-4015).  A row whose keys are all
  * masked yields zeros.  fp32 accumulation; output in `dtype`.
- * bf16/f16 with D = 32 or a multiple of 8 between 32 and 256,
- * and fp32 with D in {32, 64, 128}, run on MFMA (16-byte aligned base
+ * bf16/f16 with D a multiple of 8 up to 256, and fp32 with D a multiple of
+ * 4 up to 128, run on MFMA (16-byte aligned base
  * pointers, strides that are multiples of 8 elements; fp32: 4); everything
  * else up to D = 256 runs on the generic fp32-FMA kernel, which takes the
  * place of the reference's decomposed_attention fallback

@@ -47,7 +47,9 @@ def test_version_and_kernel_selection_without_device():
     assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"generic"  # the fallback of the reference's unsupported head sizes
     p.dtype, p.head_dim = capi.DTYPE_F32, 64
     assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"mfma_f32_d64"
-    p.head_dim = 96
+    p.head_dim = 96  # fp32: multiples of 4 up to 128 run as the next of 32 / 64 / 128
+    assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"mfma_f32_d96"
+    p.head_dim = 98
     assert lib.axhip_sdpa_kernel_name(C.byref(p)) == b"generic"
     r = capi.RowsProgram()
     r.rows, r.cols, r.input_dtype, r.output_dtype = 8192, 8192, capi.DTYPE_F32, capi.DTYPE_F32

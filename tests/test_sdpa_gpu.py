@@ -29,7 +29,7 @@ def test_f32_matches_cpu_oracle(case):
     mask = make_mask(mk, Sq, Skv)
     sc = -1.0 if scale is None else scale
     got, kern = gh.sdpa(q, k, v, F32, sc, causal, mask)
-    assert kern == (f"mfma_f32_d{D}" if D in (32, 64, 128) else "generic")
+    assert kern == (f"mfma_f32_d{D}" if D <= 128 and D % 4 == 0 else "generic")
     want = axo.sdpa(q, k, v, F32, sc, causal, mask)
     assert np.allclose(got, want, rtol=1e-4, atol=1e-4), np.max(np.abs(got - want))
 
@@ -58,7 +58,7 @@ def test_f32_on_the_larger_shapes(case):
     q, k, v = inputs(B, H, Sq, Skv, D, F32, seed=11)
     mask = make_mask(mk, Sq, Skv)
     got, kern = gh.sdpa(q, k, v, F32, -1.0, causal, mask)
-    assert kern == (f"mfma_f32_d{D}" if D in (32, 64, 128) else "generic")
+    assert kern == (f"mfma_f32_d{D}" if D <= 128 and D % 4 == 0 else "generic")
     if B * H * Sq * Skv <= 1 << 24:
         want = naive_attention64(q, k, v, 1 / math.sqrt(D), causal, mask)
     else:
@@ -177,6 +177,39 @@ def test_head_sizes_between_the_compiled_ones(dt):
     qf, kf, vf = (axo.to_f32(t, dt)[..., :D].transpose(0, 2, 1, 3) for t in packed)
     want = naive_attention64(qf, kf, vf, 1 / math.sqrt(D), True)
     assert np.max(np.abs(gf[..., :D].transpose(0, 2, 1, 3) - want)) < 2e-2
+
+
+def test_fp32_multiples_of_four_and_small_16_bit_head_sizes_run_on_the_matrix_cores():
+    """fp32 head sizes that are multiples of 4 (4 .. 124) run on the fp32 matrix-core kernel of the next of 32 / 64 / 128,
+    16-bit head sizes 8 / 16 / 24 on the head_dim-32 kernel: zeros in the missing dims, the output keeps its width
+    (guard values behind every row of a wider buffer), every key split of the fp32 kernel, causal and masked."""
+    for D, (B, H, Sq, Skv), causal, mk in ((4, (1, 2, 70, 70), False, None), (20, (2, 3, 130, 70), True, None), (36, (1, 4, 64, 200), False, "mod3"),
+                                           (100, (1, 2, 100, 100), True, None), (124, (2, 2, 257, 300), False, None), (52, (1, 40, 300, 300), True, None)):
+        q, k, v = inputs(B, H, Sq, Skv, D, F32, seed=500 + D)
+        mask = make_mask(mk, Sq, Skv)
+        got, kern = gh.sdpa(q, k, v, F32, -1.0, causal, mask)
+        assert kern == f"mfma_f32_d{D}", kern
+        want = naive_attention64(q, k, v, 1 / math.sqrt(D), causal, mask)
+        assert np.max(np.abs(got - want)) < 1e-4, D
+    for dt, tag in ((BF16, "bf16"), (F16, "f16")):
+        for D in (8, 16, 24):
+            q, k, v = inputs(2, 3, 90, 150, D, dt, seed=600 + D)
+            got, kern = gh.sdpa(q, k, v, dt, -1.0, D == 16, None)
+            assert kern == f"mfma_{tag}_d{D}", kern
+            want = naive_attention64(*(axo.to_f32(t, dt) for t in (q, k, v)), 1 / math.sqrt(D), D == 16, None)
+            assert np.max(np.abs(axo.to_f32(got, dt) - want)) < 2e-2, (tag, D)
+    # fp32 rows of 40 inside rows of 64: what lies behind a row's 40 values must survive
+    B, S, H, D, W = 1, 150, 3, 40, 64
+    g = axo.PCG64(18)
+    packed = [g.normal((B, S, H, W)).astype(np.float32) for _ in range(3)]
+    st = (S * H * W, W, H * W)
+    out_init = np.full((B, S, H, W), 7.0, np.float32)
+    got, kern = gh.sdpa(*packed, F32, -1.0, False, None, q_strides=st, k_strides=st, v_strides=st, o_strides=st, shape=(B, H, S, S, D), out_init=out_init)
+    assert kern == "mfma_f32_d40"
+    gf = got.reshape(B, S, H, W)
+    assert np.all(gf[..., D:] == 7.0)
+    qf, kf, vf = (t[..., :D].transpose(0, 2, 1, 3) for t in packed)
+    assert np.max(np.abs(gf[..., :D].transpose(0, 2, 1, 3) - naive_attention64(qf, kf, vf, 1 / math.sqrt(D), False))) < 1e-4
 
 
 def test_fully_masked_rows_give_zeros_everywhere_else_matches():
