@@ -372,6 +372,124 @@ __global__ __launch_bounds__(256) void argreduce_strided_vec_kernel(const void *
     }
 }
 
+// ------------------------------------------------ reductions along an inner axis
+// Sum / max / min along the middle extent of a contiguous (outer, axis, inner) view, inner > 1: the layout of
+// argreduce_strided_vec_kernel (a thread owns the V inner positions of one 16-byte vector, TX threads side by side,
+// the TY = 256 / TX thread rows of a work-group share the axis and merge through LDS); fp32 accumulation, the result
+// scaled (mean) and rounded to the output type.
+template <int RED> __device__ __forceinline__ float red_identity() { return RED == AXHIP_RED_MAX ? -INFINITY : RED == AXHIP_RED_MIN ? INFINITY : 0.0f; }
+template <int RED> __device__ __forceinline__ float red_combine(float a, float b) { return RED == AXHIP_RED_MAX ? fmaxf(a, b) : RED == AXHIP_RED_MIN ? fminf(a, b) : a + b; }
+
+template <int RED, int DT, int TX>
+__global__ __launch_bounds__(256) void reduce_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, float scale, void *dst, int dst_dt) {
+    constexpr int TY = 256 / TX, U = 4, V = DT == AXHIP_DTYPE_F32 ? 4 : 8;
+    __shared__ float sv[TY == 1 ? 1 : TY][TY == 1 ? 1 : TX][V + 1];
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t ivecs = inner / V, groups = (ivecs + TX - 1) / TX, total = outer * groups;
+    const int n = static_cast<int>(axis);
+    for (int64_t g = blockIdx.x; g < total; g += gridDim.x) {
+        const int64_t o = g / groups, iv = (g - o * groups) * TX + tx;
+        const bool there = iv < ivecs;
+        const uint4_t *first = reinterpret_cast<const uint4_t *>(src) + o * axis * ivecs + iv;
+        float acc[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] = red_identity<RED>();
+        if (there)
+            for (int k = ty; k < n; k += TY * U) {
+                uint4_t raw[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (k + u * TY < n) {
+                        float v[V];
+                        arg_unpack<DT>(raw[u], v);
+#pragma unroll
+                        for (int e = 0; e < V; ++e) acc[e] = red_combine<RED>(acc[e], v[e]);
+                    }
+            }
+        if constexpr (TY == 1) { // a thread walked the whole (short) axis: nothing to merge, one vector store
+            if (there) {
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc[e] *= scale;
+                store_vec<V>(dst, dst_dt, o * inner + iv * V, acc);
+            }
+        } else {
+            __syncthreads(); // the previous group's partials have been read
+#pragma unroll
+            for (int e = 0; e < V; ++e) sv[ty][tx][e] = acc[e];
+            __syncthreads();
+            if (there)
+                for (int e = ty; e < V; e += TY) {
+                    float r = sv[0][tx][e];
+                    for (int y = 1; y < TY; ++y) r = red_combine<RED>(r, sv[y][tx][e]);
+                    store_any(dst, dst_dt, o * inner + iv * V + e, r * scale);
+                }
+        }
+    }
+}
+
+// any inner extent and alignment: a thread per (outer, inner) position walks the axis
+template <int RED>
+__global__ __launch_bounds__(256) void reduce_strided_kernel(const void *src, int dt, int64_t outer, int64_t axis, int64_t inner, float scale, void *dst, int dst_dt) {
+    const int64_t total = outer * inner;
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; p < total; p += static_cast<int64_t>(gridDim.x) * 256) {
+        const int64_t o = p / inner, i = p - o * inner;
+        const int64_t first = o * axis * inner + i;
+        float acc = red_identity<RED>();
+        int64_t k = 0;
+        for (; k + 4 <= axis; k += 4) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load_any(src, dt, first + (k + u) * inner);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = red_combine<RED>(acc, v[u]);
+        }
+        for (; k < axis; ++k) acc = red_combine<RED>(acc, load_any(src, dt, first + k * inner));
+        store_any(dst, dst_dt, p, acc * scale);
+    }
+}
+
+} // namespace axhip
+
+namespace axhip {
+// one launch: RED is sum, max or min; the result is multiplied by `scale`
+int launch_reduce_axis(const void *src, int dtype, int64_t outer, int64_t axis, int64_t inner, int red, float scale, void *dst, int dst_dtype, hipStream_t s) {
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    if (inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
+        const int64_t ivecs = inner / (16 / es);
+        // a short axis with plenty of results: a thread per vector walks it alone (no merge through LDS)
+        const bool flat = axis <= 32 && outer * ((ivecs + 255) / 256) >= 1024 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0;
+        const bool wide = outer * ((ivecs + 31) / 32) >= 1024;
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (flat ? (ivecs + 255) / 256 : wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
+#define AXHIP_RED_VEC_TX(RED, DT, TX) hipLaunchKernelGGL((reduce_strided_vec_kernel<RED, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, scale, dst, dst_dtype)
+#define AXHIP_RED_VEC_DT(RED, DT)                                                                                                          \
+    do {                                                                                                                                   \
+        if (flat) AXHIP_RED_VEC_TX(RED, DT, 256);                                                                                          \
+        else if (wide) AXHIP_RED_VEC_TX(RED, DT, 32);                                                                                      \
+        else AXHIP_RED_VEC_TX(RED, DT, 8);                                                                                                 \
+    } while (0)
+#define AXHIP_RED_VEC(RED)                                                                                                                 \
+    do {                                                                                                                                   \
+        if (dtype == AXHIP_DTYPE_F32) AXHIP_RED_VEC_DT(RED, AXHIP_DTYPE_F32);                                                              \
+        else if (dtype == AXHIP_DTYPE_F16) AXHIP_RED_VEC_DT(RED, AXHIP_DTYPE_F16);                                                         \
+        else AXHIP_RED_VEC_DT(RED, AXHIP_DTYPE_BF16);                                                                                      \
+    } while (0)
+        if (red == AXHIP_RED_SUM) AXHIP_RED_VEC(AXHIP_RED_SUM);
+        else if (red == AXHIP_RED_MAX) AXHIP_RED_VEC(AXHIP_RED_MAX);
+        else AXHIP_RED_VEC(AXHIP_RED_MIN);
+#undef AXHIP_RED_VEC
+#undef AXHIP_RED_VEC_DT
+#undef AXHIP_RED_VEC_TX
+    } else {
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
+        if (red == AXHIP_RED_SUM) hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_SUM>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
+        else if (red == AXHIP_RED_MAX) hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_MAX>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
+        else hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_MIN>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
+    }
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
 } // namespace axhip
 
 using namespace axhip;
@@ -662,6 +780,50 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
     }
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;
+}
+
+int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t reduce, void *dst, int32_t dst_dtype,
+                      void *stream) {
+    AXHIP_REQUIRE(valid_dtype(dtype) && valid_dtype(dst_dtype), AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: bad dtype");
+    AXHIP_REQUIRE(reduce == AXHIP_RED_SUM || reduce == AXHIP_RED_MEAN || reduce == AXHIP_RED_MAX || reduce == AXHIP_RED_MIN, AXHIP_ERR_INVALID_ARG,
+                  "axhip_reduce_axis: bad reduction %d", reduce);
+    AXHIP_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: negative extent");
+    if (outer == 0 || inner == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(axis > 0, AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: empty axis");
+    AXHIP_REQUIRE(axis < (int64_t(1) << 31) - 64, AXHIP_ERR_UNSUPPORTED, "axhip_reduce_axis: axis of %lld elements", static_cast<long long>(axis));
+    AXHIP_REQUIRE(src && dst, AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: NULL buffer");
+    if (inner == 1) { // rows: the fused row kernels
+        AxhipRowsProgram P{};
+        P.rows = outer; P.cols = axis; P.input = src; P.input_dtype = dtype; P.output = dst; P.output_dtype = dst_dtype;
+        P.norm_weight = P.norm_bias = -1; P.reduce = reduce;
+        return axhip_fused_rows(&P, stream);
+    }
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = resolve_stream(stream);
+    const float scale = reduce == AXHIP_RED_MEAN ? 1.0f / static_cast<float>(axis) : 1.0f;
+    const int red = reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : reduce;
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    const bool vec = inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
+    // Few results over a long axis (column sums of a tall matrix): too few work-groups for the chip.  The axis is cut
+    // into `parts` equal segments, reduced to fp32 partials in stream-ordered temporary memory, and those reduced again.
+    if (vec) {
+        const int64_t groups8 = outer * ((inner / (16 / es) + 7) / 8);
+        int64_t parts = 1;
+        if (groups8 < 512 && axis >= 2048)
+            for (int64_t p = 2; p <= 64 && groups8 * parts < 1024; ++p)
+                if (axis % p == 0 && axis / p >= 256) parts = p;
+        if (parts > 1) {
+            void *tmp = nullptr;
+            AXHIP_CHECK_HIP(hipMallocAsync(&tmp, static_cast<size_t>(outer * parts * inner) * 4, s));
+            rc = launch_reduce_axis(src, dtype, outer * parts, axis / parts, inner, red, 1.0f, tmp, AXHIP_DTYPE_F32, s);
+            if (!rc) rc = launch_reduce_axis(tmp, AXHIP_DTYPE_F32, outer, parts, inner, red, scale, dst, dst_dtype, s);
+            const hipError_t freed = hipFreeAsync(tmp, s);
+            if (!rc) AXHIP_CHECK_HIP(freed);
+            return rc;
+        }
+    }
+    return launch_reduce_axis(src, dtype, outer, axis, inner, red, scale, dst, dst_dtype, s);
 }
 
 } // extern "C"

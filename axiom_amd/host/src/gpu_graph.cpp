@@ -80,14 +80,21 @@ struct GatherStep {
     int table = -1, indices = -1, dst = -1;
 };
 
+struct AxisReduceStep { // a reduction along the middle extent of a contiguous (outer, axis, inner) value
+    int src = -1, dst = -1;
+    int64_t outer = 1, axis = 1, inner = 1;
+    int reduce = 0;
+};
+
 struct Step {
-    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER } kind;
+    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER, AXIS_REDUCE } kind;
     RowsStep rows;
     GemmStep gemm;
     CopyStep copy;
     PadStep pad;
     MaskedFillStep mfill;
     GatherStep gather;
+    AxisReduceStep axred;
 };
 
 struct Plan {
@@ -240,6 +247,33 @@ class PlanBuilder {
         return out;
     }
 
+    // A reduction whose axes are one run of neighbours that stops short of the last axis: (outer, axis, inner) of the
+    // input, with more than one kept element behind the run.  False for everything the row kernels take (the last
+    // axis, all axes, a single kept element).
+    static bool inner_axis_run(const GraphNode *n, int64_t *outer, int64_t *axis, int64_t *inner) {
+        const auto &rp = get_params<ReductionParams>(n->params);
+        const Shape &F = n->inputs[0]->output_shape;
+        const int nd = static_cast<int>(F.size());
+        if (rp.axes.empty() || nd < 2) return false;
+        std::vector<bool> red(static_cast<size_t>(nd), false);
+        for (int a : rp.axes) red[static_cast<size_t>(ShapeUtils::normalize_axis(a, nd))] = true;
+        int first = -1, last = -1, count = 0;
+        for (int i = 0; i < nd; ++i)
+            if (red[static_cast<size_t>(i)]) {
+                if (first < 0) first = i;
+                last = i;
+                ++count;
+            }
+        if (count != last - first + 1 || last == nd - 1) return false;
+        int64_t o = 1, a = 1, in = 1;
+        for (int i = 0; i < nd; ++i) (i < first ? o : i <= last ? a : in) *= static_cast<int64_t>(F[static_cast<size_t>(i)]);
+        if (in <= 1 || a == 0 || o * in <= 1) return false;
+        if (outer) *outer = o;
+        if (axis) *axis = a;
+        if (inner) *inner = in;
+        return true;
+    }
+
     bool consumable(const GraphNode *c, const GraphNode *entry) const {
         return !is_leaf(c, root_) && (c == entry || !shared_.count(c)) && !memo_.count(c);
     }
@@ -338,6 +372,20 @@ class PlanBuilder {
             plan_.steps.push_back(st);
         } else if (op == OpType::MatMul) {
             v = emit_gemm(n, {}, -1, -1, 0);
+        } else if (is_reduction(op) && inner_axis_run(n, nullptr, nullptr, nullptr)) {
+            // one run of neighbouring axes that ends before the last one: reduced where the data lie, no transposing copy
+            int64_t outer, axis, inner;
+            inner_axis_run(n, &outer, &axis, &inner);
+            Step st{};
+            st.kind = Step::AXIS_REDUCE;
+            st.axred.src = make_contiguous(eval(n->inputs[0].get()));
+            st.axred.outer = outer;
+            st.axred.axis = axis;
+            st.axred.inner = inner;
+            st.axred.reduce = op == OpType::Sum ? AXHIP_RED_SUM : op == OpType::Mean ? AXHIP_RED_MEAN : op == OpType::Max ? AXHIP_RED_MAX : AXHIP_RED_MIN;
+            detail::to_axhip_dtype(val(st.axred.src).dtype);
+            st.axred.dst = v = new_temp(n->output_shape, n->output_dtype);
+            plan_.steps.push_back(st);
         } else if (is_elementwise(op) || is_row_op(op) || is_reduction(op)) {
             v = emit_rows(n);
         } else {
@@ -879,6 +927,11 @@ void materialize_gpu_graph(GraphNode *root) {
             if (record) tl_last_kernels.emplace_back("masked_fill");
             AXHIP_CALL(axhip_masked_fill(ptr_of(st.mfill.src), detail::to_axhip_dtype(src.dtype), static_cast<const uint8_t *>(ptr_of(st.mfill.mask)),
                                          ptr_of(st.mfill.dst), static_cast<int32_t>(shp.size()), shp.data(), est.data(), mst.data(), st.mfill.value, nullptr));
+        } else if (st.kind == Step::AXIS_REDUCE) {
+            const ValueSpec &src = plan->values[st.axred.src], &dst = plan->values[st.axred.dst];
+            if (record) tl_last_kernels.emplace_back("reduce_axis");
+            AXHIP_CALL(axhip_reduce_axis(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
+                                         ptr_of(st.axred.dst), detail::to_axhip_dtype(dst.dtype), nullptr));
         } else if (st.kind == Step::GATHER) {
             const ValueSpec &tab = plan->values[st.gather.table], &idx = plan->values[st.gather.indices];
             if (record) tl_last_kernels.emplace_back("gather_rows");

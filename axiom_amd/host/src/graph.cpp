@@ -196,7 +196,11 @@ Tensor GraphRegistry::create_lazy_reduction(ops::OpType op, const Tensor &input,
         }
         const bool all = kept_axes.empty() || kept == 1;
         const bool last_only = red_axes.size() == 1 && red_axes[0] == nd - 1;
-        if (!all && !last_only && !red_axes.empty() && kept * folded > 0) {
+        // (one run of neighbouring axes that ends before the last one is reduced where it lies: the planner has a
+        // kernel for the middle extent of an (outer, axis, inner) array)
+        const bool inner_run = !red_axes.empty() && red_axes.back() != nd - 1 && red_axes.back() - red_axes.front() + 1 == static_cast<int>(red_axes.size()) &&
+                               [&] { size_t in = 1; for (int i = red_axes.back() + 1; i < nd; ++i) in *= input.shape()[static_cast<size_t>(i)]; return in > 1; }();
+        if (!all && !last_only && !inner_run && !red_axes.empty() && kept * folded > 0) {
             std::vector<int> order = kept_axes;
             order.insert(order.end(), red_axes.begin(), red_axes.end());
             bool identity = true;

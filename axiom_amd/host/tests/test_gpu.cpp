@@ -350,7 +350,23 @@ GPU_TEST(CpuGpuParity, ReductionsAndSoftmaxOverAnyAxis) {
             EXPECT_NEAR(hx[i], mx[i], 0);
         }
     }
-    // a chain below the reduction still fuses behind the gather: sum(relu(x) * 2, axis 1)
+    // one run of neighbouring axes that ends before the last one is reduced in place: one kernel, no transposing copy
+    {
+        ops::sum(ga, {1, 2}, false).sync();
+        ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+        EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("reduce_axis"));
+        auto hb = a.astype(DType::BFloat16);
+        auto mean16 = ops::mean(hb.gpu(), {0}, false);
+        EXPECT_EQ(mean16.dtype(), DType::Float32); // graph_registry.cpp:278-287
+        auto hm = host_floats(mean16);
+        auto hb32 = hb.astype(DType::Float32);
+        for (size_t k = 0; k < 7 * 6 * 9; ++k) {
+            double t = 0;
+            for (size_t i = 0; i < 5; ++i) t += hb32.typed_data<float>()[i * strides[0] + k];
+            EXPECT_NEAR(hm[k], t / 5.0, 1e-5);
+        }
+    }
+    // a chain below such a reduction is materialised first: sum(relu(x) * 2, axis 1)
     {
         auto got = host_floats(ops::sum(ops::relu(ga) * 2.0f, {1}, false));
         for (size_t i = 0; i < 5; ++i)

@@ -284,6 +284,17 @@ int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int6
 int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
                     int32_t want_min, int64_t *dst, void *stream);
 
+/* Sum / mean / max / min (AXHIP_RED_*) along the middle extent of a contiguous
+ * (outer, axis, inner) view -> outer * inner values of dst_dtype: Reduction
+ * nodes over axes other than the last one
+ * (src/backends/metal/mpsgraph_graph_compiler.mm:576-604 reduces over any axes),
+ * without a transposing copy.  fp32 accumulation; the mean divides by the axis
+ * length.  inner == 1 is a row reduction and goes to the fused row kernels.
+ * Few results over a long axis are reduced in two passes through fp32
+ * partials in stream-ordered temporary memory (hipMallocAsync on `stream`). */
+int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
+                      int32_t reduce, void *dst, int32_t dst_dtype, void *stream);
+
 /* -------------------------------------------------------------------- GEMM
  * Stands behind the GPU MatMul registry entry and gpu_linear
  * (src/backends/metal/mpsgraph_operations.mm:2409-2532; lazy builder

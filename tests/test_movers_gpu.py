@@ -247,6 +247,48 @@ def test_argreduce_known_answers_and_errors():
     assert L.axhip_argreduce(d.data_ptr(), F32, 1, 1 << 31, 1, 0, d.data_ptr(), None) == capi.ERR_UNSUPPORTED
 
 
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+def test_reductions_along_inner_axes_match_the_oracle(dt):
+    """Sum / mean / max / min along the middle extent of (outer, axis, inner) views: vector-aligned and odd inner
+    extents, few and many outputs, an axis of one element; against the oracle's reduction of the same axis moved last
+    (sums: fp32 accumulation in another order, 1e-4 relative to the sum of magnitudes; max / min bit-exact)."""
+    rng = np.random.default_rng(5 + dt)
+    for outer, axis, inner in ((1, 37, 4096), (6, 130, 72), (3, 1, 64), (64, 300, 8), (5, 77, 9), (2, 1000, 33), (300, 5, 256), (1, 4100, 24),
+                               (1, 8192, 512), (2, 6000, 64),  # few results over a long axis: two passes
+                               (1200, 7, 1024), (5000, 2, 264)):  # a short axis with many results: a thread per vector
+        x = (rng.normal(size=(outer, axis, inner)) * 3).astype(np.float32)
+        bits = x if dt == F32 else axo.to_bits(x, dt)
+        xf = axo.to_f32(bits, dt)
+        d = gh.to_dev(bits)
+        for red in ("sum", "mean", "max", "min"):
+            odt = F32 if red == "mean" else dt
+            out = gh.empty_dev((outer, inner), odt)
+            gh.sync()
+            capi.check(capi.lib().axhip_reduce_axis(d.data_ptr(), dt, outer, axis, inner, capi.RED[red], out.data_ptr(), odt, None))
+            gh.sync()
+            got = axo.to_f32(gh.to_host(out, gh.np_store_dtype(odt)), odt)
+            if red in ("max", "min"):
+                want = axo.to_f32(axo.reduce_last(red, np.ascontiguousarray(np.moveaxis(bits, 1, -1)), dt), dt)
+                assert np.array_equal(got, want), (red, outer, axis, inner)
+            else:
+                want = xf.astype(np.float64).sum(1) / (axis if red == "mean" else 1)
+                mag = np.abs(xf).astype(np.float64).sum(1) / (axis if red == "mean" else 1)
+                tol = 1e-4 * mag + (0 if odt == F32 else 2.0 ** (-8 if odt == BF16 else -11) * np.abs(want)) + 1e-6
+                assert np.all(np.abs(got - want) <= tol), (red, outer, axis, inner, float(np.max(np.abs(got - want) - tol)))
+    # inner == 1 goes to the row kernels
+    x = rng.normal(size=(50, 333)).astype(np.float32)
+    bits = x if dt == F32 else axo.to_bits(x, dt)
+    d, out = gh.to_dev(bits), gh.empty_dev((50,), dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_reduce_axis(d.data_ptr(), dt, 50, 333, 1, capi.RED["max"], out.data_ptr(), dt, None))
+    gh.sync()
+    assert np.array_equal(gh.to_host(out, gh.np_store_dtype(dt)), axo.reduce_last("max", bits, dt))
+    L = capi.lib()
+    assert L.axhip_reduce_axis(d.data_ptr(), dt, 1, 0, 4, capi.RED["sum"], out.data_ptr(), dt, None) == capi.ERR_INVALID_ARG
+    assert L.axhip_reduce_axis(d.data_ptr(), dt, 1, 4, 4, 9, out.data_ptr(), dt, None) == capi.ERR_INVALID_ARG
+    assert L.axhip_reduce_axis(None, dt, 0, 4, 4, capi.RED["sum"], None, dt, None) == 0
+
+
 def test_mover_argument_errors():
     L = capi.lib()
     assert L.axhip_pad(None, None, 7, 1, i64([1]), i64([1]), i64([0]), i64([0]), 0.0, None) == capi.ERR_INVALID_ARG
