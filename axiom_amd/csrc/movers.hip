@@ -453,6 +453,107 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const void *src, in
 } // namespace axhip
 
 namespace axhip {
+// ----------------------------------------------- softmax along an inner axis
+// softmax / log-softmax along the middle extent of a contiguous (outer, axis, inner) view, inner > 1, in the layout of
+// reduce_strided_vec_kernel.  One sweep gathers a running maximum and the sum of 2^(x log2(e) - maximum) per inner
+// position (rescaled once per four elements), the thread rows merge their pairs through LDS, a second sweep over the
+// same elements writes the result: two reads of the input (the second mostly from the caches) and one write.
+template <bool LOG, int DT, int TX>
+__global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, void *dst) {
+    constexpr int TY = 256 / TX, U = 4, V = DT == AXHIP_DTYPE_F32 ? 4 : 8;
+    constexpr float LOG2E = 1.44269504088896340736f, LN2 = 0.69314718055994530942f;
+    __shared__ float sm[TY][TX][V + 1], sl[TY][TX][V + 1];
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t ivecs = inner / V, groups = (ivecs + TX - 1) / TX, total = outer * groups;
+    const int n = static_cast<int>(axis);
+    for (int64_t g = blockIdx.x; g < total; g += gridDim.x) {
+        const int64_t o = g / groups, iv = (g - o * groups) * TX + tx;
+        const bool there = iv < ivecs;
+        const uint4_t *first = reinterpret_cast<const uint4_t *>(src) + o * axis * ivecs + iv;
+        float m[V], l[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            m[e] = -INFINITY;
+            l[e] = 0.0f;
+        }
+        if (there)
+            for (int k = ty; k < n; k += TY * U) {
+                uint4_t raw[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+                float t[U][V];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    arg_unpack<DT>(raw[u], t[u]);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) t[u][e] = k + u * TY < n ? t[u][e] * LOG2E : -INFINITY;
+                }
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const float mx = fmaxf(fmaxf(fmaxf(t[0][e], t[1][e]), fmaxf(t[2][e], t[3][e])), m[e]);
+                    const float ref = mx == -INFINITY ? 0.0f : mx; // (nothing finite yet: every term below is 2^-inf = 0)
+                    float add = 0.0f;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) add += __builtin_amdgcn_exp2f(t[u][e] - ref);
+                    l[e] = l[e] * __builtin_amdgcn_exp2f(m[e] - ref) + add;
+                    m[e] = mx;
+                }
+            }
+        __syncthreads(); // the previous group's pairs have been read
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            sm[ty][tx][e] = m[e];
+            sl[ty][tx][e] = l[e];
+        }
+        __syncthreads();
+        float shift[V], inv[V]; // result = 2^(t - shift) * inv, or (t - shift) * ln 2 with the logarithm of the sum inside shift
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            float M = sm[0][tx][e];
+            for (int y = 1; y < TY; ++y) M = fmaxf(M, sm[y][tx][e]);
+            const float ref = M == -INFINITY ? 0.0f : M;
+            float L = 0.0f;
+            for (int y = 0; y < TY; ++y) L += sl[y][tx][e] * __builtin_amdgcn_exp2f(sm[y][tx][e] - ref);
+            shift[e] = LOG ? M + __builtin_amdgcn_logf(L) : M; // (v_log_f32 is the base-2 logarithm)
+            inv[e] = 1.0f / L;
+        }
+        if (there)
+            for (int k = ty; k < n; k += TY * U) {
+                uint4_t raw[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (k + u * TY < n) {
+                        float v[V];
+                        arg_unpack<DT>(raw[u], v);
+#pragma unroll
+                        for (int e = 0; e < V; ++e) v[e] = LOG ? (v[e] * LOG2E - shift[e]) * LN2 : __builtin_amdgcn_exp2f(v[e] * LOG2E - shift[e]) * inv[e];
+                        store_vec<V>(dst, DT, (o * axis + k + u * TY) * inner + iv * V, v);
+                    }
+            }
+    }
+}
+
+// any inner extent and alignment: a thread per (outer, inner) position, three sweeps
+template <bool LOG>
+__global__ __launch_bounds__(256) void softmax_strided_kernel(const void *src, int dt, int64_t outer, int64_t axis, int64_t inner, void *dst) {
+    const int64_t total = outer * inner;
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; p < total; p += static_cast<int64_t>(gridDim.x) * 256) {
+        const int64_t o = p / inner, i = p - o * inner;
+        const int64_t first = o * axis * inner + i;
+        float m = -INFINITY;
+        for (int64_t k = 0; k < axis; ++k) m = fmaxf(m, load_any(src, dt, first + k * inner));
+        float l = 0.0f;
+        for (int64_t k = 0; k < axis; ++k) l += __expf(load_any(src, dt, first + k * inner) - m);
+        const float logl = __logf(l), inv = 1.0f / l;
+        for (int64_t k = 0; k < axis; ++k) {
+            const float x = load_any(src, dt, first + k * inner);
+            store_any(dst, dt, first + k * inner, LOG ? x - m - logl : __expf(x - m) * inv);
+        }
+    }
+}
+
 // one launch: RED is sum, max or min; the result is multiplied by `scale`
 int launch_reduce_axis(const void *src, int dtype, int64_t outer, int64_t axis, int64_t inner, int red, float scale, void *dst, int dst_dtype, hipStream_t s) {
     const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
@@ -824,6 +925,52 @@ int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axi
         }
     }
     return launch_reduce_axis(src, dtype, outer, axis, inner, red, scale, dst, dst_dtype, s);
+}
+
+int axhip_softmax_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t is_log, void *dst, void *stream) {
+    AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_softmax_axis: bad dtype");
+    AXHIP_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, AXHIP_ERR_INVALID_ARG, "axhip_softmax_axis: negative extent");
+    if (outer == 0 || inner == 0 || axis == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(axis < (int64_t(1) << 31) - 64, AXHIP_ERR_UNSUPPORTED, "axhip_softmax_axis: axis of %lld elements", static_cast<long long>(axis));
+    AXHIP_REQUIRE(src && dst, AXHIP_ERR_INVALID_ARG, "axhip_softmax_axis: NULL buffer");
+    if (inner == 1) { // rows: the fused row kernels
+        AxhipRowsProgram P{};
+        P.rows = outer; P.cols = axis; P.input = src; P.input_dtype = dtype; P.output = dst; P.output_dtype = dtype;
+        P.norm_weight = P.norm_bias = -1; P.row_op = is_log ? AXHIP_ROWOP_LOGSOFTMAX : AXHIP_ROWOP_SOFTMAX;
+        return axhip_fused_rows(&P, stream);
+    }
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = resolve_stream(stream);
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    if (inner % (16 / es) == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0) {
+        const int64_t ivecs = inner / (16 / es);
+        const bool wide = outer * ((ivecs + 31) / 32) >= 1024;
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
+#define AXHIP_SM_TX(LOG, DT, TX) hipLaunchKernelGGL((softmax_strided_vec_kernel<LOG, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, dst)
+#define AXHIP_SM_DT(LOG, DT)                                                                                                               \
+    do {                                                                                                                                   \
+        if (wide) AXHIP_SM_TX(LOG, DT, 32);                                                                                                \
+        else AXHIP_SM_TX(LOG, DT, 8);                                                                                                      \
+    } while (0)
+#define AXHIP_SM(LOG)                                                                                                                      \
+    do {                                                                                                                                   \
+        if (dtype == AXHIP_DTYPE_F32) AXHIP_SM_DT(LOG, AXHIP_DTYPE_F32);                                                                   \
+        else if (dtype == AXHIP_DTYPE_F16) AXHIP_SM_DT(LOG, AXHIP_DTYPE_F16);                                                              \
+        else AXHIP_SM_DT(LOG, AXHIP_DTYPE_BF16);                                                                                           \
+    } while (0)
+        if (is_log) AXHIP_SM(true);
+        else AXHIP_SM(false);
+#undef AXHIP_SM
+#undef AXHIP_SM_DT
+#undef AXHIP_SM_TX
+    } else {
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
+        if (is_log) hipLaunchKernelGGL(softmax_strided_kernel<true>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, dst);
+        else hipLaunchKernelGGL(softmax_strided_kernel<false>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, dst);
+    }
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
 }
 
 } // extern "C"

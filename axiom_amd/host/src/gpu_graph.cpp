@@ -80,14 +80,14 @@ struct GatherStep {
     int table = -1, indices = -1, dst = -1;
 };
 
-struct AxisReduceStep { // a reduction along the middle extent of a contiguous (outer, axis, inner) value
+struct AxisReduceStep { // a reduction, or a softmax, along the middle extent of a contiguous (outer, axis, inner) value
     int src = -1, dst = -1;
     int64_t outer = 1, axis = 1, inner = 1;
-    int reduce = 0;
+    int reduce = 0;  // AXHIP_RED_*; for AXIS_SOFTMAX: 1 = log-softmax
 };
 
 struct Step {
-    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER, AXIS_REDUCE } kind;
+    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER, AXIS_REDUCE, AXIS_SOFTMAX } kind;
     RowsStep rows;
     GemmStep gemm;
     CopyStep copy;
@@ -274,6 +274,14 @@ class PlanBuilder {
         return true;
     }
 
+    // the row kernels take softmax and the norms over the last axis
+    static bool row_axis_is_last(const GraphNode *n) {
+        const int nd = static_cast<int>(n->output_shape.size());
+        const int axis = n->op_type == OpType::Softmax || n->op_type == OpType::LogSoftmax ? get_params<ActivationParams>(n->params).axis
+                                                                                           : get_params<NormParams>(n->params).axis;
+        return nd == 0 || ShapeUtils::normalize_axis(axis, nd) == nd - 1;
+    }
+
     bool consumable(const GraphNode *c, const GraphNode *entry) const {
         return !is_leaf(c, root_) && (c == entry || !shared_.count(c)) && !memo_.count(c);
     }
@@ -385,6 +393,19 @@ class PlanBuilder {
             st.axred.reduce = op == OpType::Sum ? AXHIP_RED_SUM : op == OpType::Mean ? AXHIP_RED_MEAN : op == OpType::Max ? AXHIP_RED_MAX : AXHIP_RED_MIN;
             detail::to_axhip_dtype(val(st.axred.src).dtype);
             st.axred.dst = v = new_temp(n->output_shape, n->output_dtype);
+            plan_.steps.push_back(st);
+        } else if ((op == OpType::Softmax || op == OpType::LogSoftmax) && !row_axis_is_last(n)) {
+            // softmax over an axis other than the last: where the data lie, no transposing copies
+            const Shape &F = n->output_shape;
+            const int ax = ShapeUtils::normalize_axis(get_params<ActivationParams>(n->params).axis, static_cast<int>(F.size()));
+            Step st{};
+            st.kind = Step::AXIS_SOFTMAX;
+            st.axred.src = make_contiguous(eval(n->inputs[0].get()));
+            for (int i = 0; i < static_cast<int>(F.size()); ++i)
+                (i < ax ? st.axred.outer : i == ax ? st.axred.axis : st.axred.inner) *= static_cast<int64_t>(F[static_cast<size_t>(i)]);
+            st.axred.reduce = op == OpType::LogSoftmax ? 1 : 0;
+            detail::to_axhip_dtype(val(st.axred.src).dtype);
+            st.axred.dst = v = new_temp(F, n->output_dtype);
             plan_.steps.push_back(st);
         } else if (is_elementwise(op) || is_row_op(op) || is_reduction(op)) {
             v = emit_rows(n);
@@ -501,7 +522,8 @@ class PlanBuilder {
         std::vector<ChainItem> upper, lower;
         collect(cur, entry, F, upper, AXHIP_MAX_CHAIN, operands);
         const GraphNode *rowop = nullptr;
-        if (!rs.full_reduce && consumable(cur, entry) && is_row_op(cur->op_type) && cur->output_shape == F) {
+        if (!rs.full_reduce && consumable(cur, entry) && is_row_op(cur->op_type) && cur->output_shape == F &&
+            (row_axis_is_last(cur) || (cur->op_type != OpType::Softmax && cur->op_type != OpType::LogSoftmax))) { // (a softmax over another axis is a step of its own)
             const int axis = cur->op_type == OpType::Softmax || cur->op_type == OpType::LogSoftmax ? get_params<ActivationParams>(cur->params).axis
                                                                                                   : get_params<NormParams>(cur->params).axis;
             if (ShapeUtils::normalize_axis(axis, static_cast<int>(F.size())) != static_cast<int>(F.size()) - 1)
@@ -932,6 +954,11 @@ void materialize_gpu_graph(GraphNode *root) {
             if (record) tl_last_kernels.emplace_back("reduce_axis");
             AXHIP_CALL(axhip_reduce_axis(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
                                          ptr_of(st.axred.dst), detail::to_axhip_dtype(dst.dtype), nullptr));
+        } else if (st.kind == Step::AXIS_SOFTMAX) {
+            const ValueSpec &src = plan->values[st.axred.src];
+            if (record) tl_last_kernels.emplace_back("softmax_axis");
+            AXHIP_CALL(axhip_softmax_axis(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
+                                          ptr_of(st.axred.dst), nullptr));
         } else if (st.kind == Step::GATHER) {
             const ValueSpec &tab = plan->values[st.gather.table], &idx = plan->values[st.gather.indices];
             if (record) tl_last_kernels.emplace_back("gather_rows");

@@ -236,13 +236,7 @@ Tensor GraphRegistry::create_lazy_matmul(const Tensor &a, const Tensor &b, bool 
 Tensor GraphRegistry::create_lazy_softmax(ops::OpType op, const Tensor &input, int axis) {
     require_gpu(pick_device({&input}), op);
     const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
-    // over another axis than the last: that axis and the last one change places, before and after
-    if (a != static_cast<int>(input.ndim()) - 1) {
-        std::vector<int> swap(input.ndim());
-        for (size_t i = 0; i < swap.size(); ++i) swap[i] = static_cast<int>(i);
-        std::swap(swap[static_cast<size_t>(a)], swap.back());
-        return create_lazy_transpose(create_lazy_softmax(op, create_lazy_transpose(input, swap), -1), swap);
-    }
+    // (over another axis than the last: the planner has a kernel for the middle extent of an (outer, axis, inner) array)
     auto n = std::make_shared<GraphNode>();
     n->op_type = op;
     n->inputs = {input_node(input)};

@@ -376,6 +376,23 @@ GPU_TEST(CpuGpuParity, ReductionsAndSoftmaxOverAnyAxis) {
                 EXPECT_NEAR(got[i * 54 + k], t, 1e-4);
             }
     }
+    // softmax over an inner axis is one kernel where the data lie, also below an elementwise chain
+    {
+        ops::softmax(ga, 1).sync();
+        ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+        EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("softmax_axis"));
+        auto b16 = axtest::randn({4, 10, 64}, 4242).astype(DType::BFloat16);
+        auto got = host_floats((ops::softmax(b16.gpu(), 1) * 2.0f).astype(DType::Float32));
+        auto b32 = b16.astype(DType::Float32);
+        for (size_t o = 0; o < 4; ++o)
+            for (size_t i = 0; i < 64; ++i) {
+                double m = -1e300, z = 0;
+                for (size_t k = 0; k < 10; ++k) m = std::max(m, static_cast<double>(b32.typed_data<float>()[(o * 10 + k) * 64 + i]));
+                for (size_t k = 0; k < 10; ++k) z += std::exp(b32.typed_data<float>()[(o * 10 + k) * 64 + i] - m);
+                for (size_t k = 0; k < 10; ++k)
+                    EXPECT_NEAR(got[(o * 10 + k) * 64 + i], 2.0 * std::exp(b32.typed_data<float>()[(o * 10 + k) * 64 + i] - m) / z, 2e-2);
+            }
+    }
     // softmax and log-softmax over each axis
     for (int axis = 0; axis < 4; ++axis) {
         auto sm = host_floats(ops::softmax(ga, axis)), lsm = host_floats(ops::log_softmax(ga, axis - 4));

@@ -295,6 +295,15 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
 int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
                       int32_t reduce, void *dst, int32_t dst_dtype, void *stream);
 
+/* softmax (is_log = 0) / log-softmax along the middle extent of a contiguous
+ * (outer, axis, inner) view, dst of the same shape and dtype: Softmax /
+ * LogSoftmax nodes over an axis other than the last one
+ * (src/backends/metal/mpsgraph_graph_compiler.mm:287-300 takes any axis),
+ * without the two transposing copies.  inner == 1 goes to the fused row
+ * kernels. */
+int axhip_softmax_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
+                       int32_t is_log, void *dst, void *stream);
+
 /* -------------------------------------------------------------------- GEMM
  * Stands behind the GPU MatMul registry entry and gpu_linear
  * (src/backends/metal/mpsgraph_operations.mm:2409-2532; lazy builder

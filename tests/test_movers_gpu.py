@@ -289,6 +289,36 @@ def test_reductions_along_inner_axes_match_the_oracle(dt):
     assert L.axhip_reduce_axis(None, dt, 0, 4, 4, capi.RED["sum"], None, dt, None) == 0
 
 
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+def test_softmax_along_inner_axes_matches_the_oracle(dt):
+    """softmax / log-softmax along the middle extent of (outer, axis, inner) views against the oracle's softmax over
+    that axis: vector-aligned and odd inner extents, an axis of one element, long axes, large logits; fp32 1e-5
+    (log: 1e-4), 16-bit one rounding step of the result."""
+    rng = np.random.default_rng(9 + dt)
+    for outer, axis, inner, scale in ((1, 37, 4096, 1.0), (6, 130, 72, 3.0), (3, 1, 64, 1.0), (64, 300, 8, 10.0), (5, 77, 9, 2.0), (2, 1000, 33, 1.0),
+                                      (1, 5000, 24, 4.0)):
+        x = (rng.normal(size=(outer, axis, inner)) * scale).astype(np.float32)
+        bits = x if dt == F32 else axo.to_bits(x, dt)
+        d = gh.to_dev(bits)
+        for log in (False, True):
+            out = gh.empty_dev((outer, axis, inner), dt)
+            gh.sync()
+            capi.check(capi.lib().axhip_softmax_axis(d.data_ptr(), dt, outer, axis, inner, int(log), out.data_ptr(), None))
+            gh.sync()
+            got = axo.to_f32(gh.to_host(out, gh.np_store_dtype(dt)), dt)
+            xf = axo.to_f32(bits, dt).astype(np.float64)
+            z = xf - xf.max(1, keepdims=True)
+            want = z - np.log(np.exp(z).sum(1, keepdims=True)) if log else np.exp(z) / np.exp(z).sum(1, keepdims=True)
+            step = 0.0 if dt == F32 else 2.0 ** (-8 if dt == BF16 else -11)
+            tol = (1e-4 if log else 1e-5) + step * np.abs(want) + (1e-5 * np.abs(want) if log else 0)
+            assert np.all(np.abs(got - want) <= tol), (log, outer, axis, inner, float(np.max(np.abs(got - want) - tol)))
+            if not log:
+                assert np.allclose(got.astype(np.float64).sum(1), 1.0, atol=1e-5 if dt == F32 else 2e-2)
+            # and the oracle's own evaluation of the same axis (cpu path restated), to its 16-bit rounding
+            lit = axo.to_f32(axo.softmax(bits, dt, 1, log), dt)
+            assert np.all(np.abs(got - lit) <= 2 * tol + 1e-6)
+
+
 def test_mover_argument_errors():
     L = capi.lib()
     assert L.axhip_pad(None, None, 7, 1, i64([1]), i64([1]), i64([0]), i64([0]), 0.0, None) == capi.ERR_INVALID_ARG
