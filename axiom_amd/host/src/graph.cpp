@@ -253,6 +253,14 @@ Tensor GraphRegistry::create_lazy_softmax(ops::OpType op, const Tensor &input, i
 Tensor GraphRegistry::create_lazy_layernorm(const Tensor &input, const Tensor &weight, const Tensor &bias, int axis, float eps) {
     require_gpu(pick_device({&input}), ops::OpType::LayerNorm);
     const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
+    // over another axis than the last (per-channel statistics of a channels-first array): that axis and the last one
+    // change places, before and after the row kernel
+    if (a != static_cast<int>(input.ndim()) - 1) {
+        std::vector<int> swap(input.ndim());
+        for (size_t i = 0; i < swap.size(); ++i) swap[i] = static_cast<int>(i);
+        std::swap(swap[static_cast<size_t>(a)], swap.back());
+        return create_lazy_transpose(create_lazy_layernorm(create_lazy_transpose(input, swap), weight, bias, -1, eps), swap);
+    }
     auto n = std::make_shared<GraphNode>();
     n->op_type = ops::OpType::LayerNorm;
     n->inputs = {input_node(input)};
@@ -271,6 +279,12 @@ Tensor GraphRegistry::create_lazy_layernorm(const Tensor &input, const Tensor &w
 Tensor GraphRegistry::create_lazy_rmsnorm(const Tensor &input, const Tensor &weight, int axis, float eps) {
     require_gpu(pick_device({&input}), ops::OpType::RMSNorm);
     const int a = ShapeUtils::normalize_axis(axis, static_cast<int>(input.ndim()));
+    if (a != static_cast<int>(input.ndim()) - 1) { // as for layer_norm
+        std::vector<int> swap(input.ndim());
+        for (size_t i = 0; i < swap.size(); ++i) swap[i] = static_cast<int>(i);
+        std::swap(swap[static_cast<size_t>(a)], swap.back());
+        return create_lazy_transpose(create_lazy_rmsnorm(create_lazy_transpose(input, swap), weight, -1, eps), swap);
+    }
     auto n = std::make_shared<GraphNode>();
     n->op_type = ops::OpType::RMSNorm;
     n->inputs = {input_node(input)};

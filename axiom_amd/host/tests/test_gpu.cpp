@@ -393,6 +393,31 @@ GPU_TEST(CpuGpuParity, ReductionsAndSoftmaxOverAnyAxis) {
                     EXPECT_NEAR(got[(o * 10 + k) * 64 + i], 2.0 * std::exp(b32.typed_data<float>()[(o * 10 + k) * 64 + i] - m) / z, 2e-2);
             }
     }
+    // layer norm and RMS norm over an inner axis (weights along that axis)
+    {
+        auto xn = axtest::randn({3, 12, 20}, 4343), w = axtest::randn({12}, 4344), bb = axtest::randn({12}, 4345);
+        auto ln = host_floats(ops::layer_norm(xn.gpu(), w.gpu(), bb.gpu(), 1, 1e-5f)), rn = host_floats(ops::rms_norm(xn.gpu(), w.gpu(), 1, 1e-5f));
+        const float *p = xn.typed_data<float>(), *pw = w.typed_data<float>(), *pb = bb.typed_data<float>();
+        for (size_t o = 0; o < 3; ++o)
+            for (size_t i = 0; i < 20; ++i) {
+                double mean = 0, sq = 0;
+                for (size_t k = 0; k < 12; ++k) mean += p[(o * 12 + k) * 20 + i];
+                mean /= 12;
+                double var = 0;
+                for (size_t k = 0; k < 12; ++k) {
+                    const double d = p[(o * 12 + k) * 20 + i] - mean;
+                    var += d * d;
+                    sq += static_cast<double>(p[(o * 12 + k) * 20 + i]) * p[(o * 12 + k) * 20 + i];
+                }
+                var /= 12;
+                sq /= 12;
+                for (size_t k = 0; k < 12; ++k) {
+                    const double v = p[(o * 12 + k) * 20 + i];
+                    EXPECT_NEAR(ln[(o * 12 + k) * 20 + i], (v - mean) / std::sqrt(var + 1e-5) * pw[k] + pb[k], 1e-4);
+                    EXPECT_NEAR(rn[(o * 12 + k) * 20 + i], v / std::sqrt(sq + 1e-5) * pw[k], 1e-4);
+                }
+            }
+    }
     // softmax and log-softmax over each axis
     for (int axis = 0; axis < 4; ++axis) {
         auto sm = host_floats(ops::softmax(ga, axis)), lsm = host_floats(ops::log_softmax(ga, axis - 4));
