@@ -945,12 +945,15 @@ int axhip_softmax_axis(const void *src, int32_t dtype, int64_t outer, int64_t ax
     const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
     if (inner % (16 / es) == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0) {
         const int64_t ivecs = inner / (16 / es);
+        // a short axis with plenty of results: a thread per vector walks it alone
+        const bool flat = axis <= 32 && outer * ((ivecs + 255) / 256) >= 1024;
         const bool wide = outer * ((ivecs + 31) / 32) >= 1024;
-        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (flat ? (ivecs + 255) / 256 : wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
 #define AXHIP_SM_TX(LOG, DT, TX) hipLaunchKernelGGL((softmax_strided_vec_kernel<LOG, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, dst)
 #define AXHIP_SM_DT(LOG, DT)                                                                                                               \
     do {                                                                                                                                   \
-        if (wide) AXHIP_SM_TX(LOG, DT, 32);                                                                                                \
+        if (flat) AXHIP_SM_TX(LOG, DT, 256);                                                                                               \
+        else if (wide) AXHIP_SM_TX(LOG, DT, 32);                                                                                           \
         else AXHIP_SM_TX(LOG, DT, 8);                                                                                                      \
     } while (0)
 #define AXHIP_SM(LOG)                                                                                                                      \

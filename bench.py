@@ -403,6 +403,23 @@ def bench_survey(torch, capi, stream, steps, warmup):
                                                                "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                                                "finite": bool(torch.equal(out.view(outer, inner), t.float().argmax(1)))}
         del t, out
+    # reductions and softmax along an inner axis of a contiguous array (no transposing copy)
+    for (outer, axis, inner), dt, name in (((1, 4096, 16384), f32, "f32"), ((64, 4096, 1024), bf, "bf16"), ((8192, 8, 1024), f32, "f32")):
+        t = rnd((outer, axis, inner), dt, 3.0)
+        code = capi.DTYPE_BF16 if dt == bf else capi.DTYPE_F32
+        out = torch.empty((outer, inner), device="cuda", dtype=dt)
+        torch.cuda.synchronize()
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_reduce_axis(t.data_ptr(), code, outer, axis, inner, capi.RED["sum"], out.data_ptr(), code, sp)), steps, warmup)
+        nbytes = (t.numel() + out.numel()) * t.element_size()
+        res[f"sum_axis1_{name}_{outer}x{axis}x{inner}"] = {"kernel": "reduce_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+                                                            "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(out.float()).all().item())}
+        full = torch.empty_like(t)
+        torch.cuda.synchronize()
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_softmax_axis(t.data_ptr(), code, outer, axis, inner, 0, full.data_ptr(), sp)), steps, warmup)
+        nbytes = 2 * t.numel() * t.element_size()
+        res[f"softmax_axis1_{name}_{outer}x{axis}x{inner}"] = {"kernel": "softmax_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+                                                                "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(full.float()).all().item())}
+        del t, out, full
     return res
 
 
