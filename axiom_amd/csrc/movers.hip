@@ -326,8 +326,11 @@ __global__ __launch_bounds__(256) void argreduce_strided_kernel(const void *src,
 // positions of one vector, TX such threads side by side read TX * 16 consecutive bytes, and the TY = 256 / TX thread
 // rows of a work-group share the axis (k = ty, ty + TY, ..), merging through LDS at the end.  TX = 32 when that
 // still gives the chip a thousand work-groups, else 8 (whole 128-byte lines still).
+// part_v / part_i (both or neither): instead of the answer, the candidate of every position -- its value and its index
+// within this axis segment, INT32_MAX for none -- for argreduce_merge_kernel.
 template <bool MIN, int DT, int TX>
-__global__ __launch_bounds__(256) void argreduce_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, float start, int64_t *dst) {
+__global__ __launch_bounds__(256) void argreduce_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, float start, int64_t *dst,
+                                                                    float *part_v, int32_t *part_i) {
     constexpr int TY = 256 / TX, U = 4, V = DT == AXHIP_DTYPE_F32 ? 4 : 8;
     __shared__ float sv[TY][TX][V + 1];
     __shared__ int32_t si[TY][TX][V + 1];
@@ -367,8 +370,31 @@ __global__ __launch_bounds__(256) void argreduce_strided_vec_kernel(const void *
             for (int e = ty; e < V; e += TY) {
                 ArgBest r{sv[0][tx][e], si[0][tx][e]};
                 for (int y = 1; y < TY; ++y) arg_merge<MIN>(r, sv[y][tx][e], si[y][tx][e]);
-                dst[o * inner + iv * V + e] = r.i == INT32_MAX ? 0 : r.i;
+                if (part_v) {
+                    part_v[o * inner + iv * V + e] = r.v;
+                    part_i[o * inner + iv * V + e] = r.i;
+                } else {
+                    dst[o * inner + iv * V + e] = r.i == INT32_MAX ? 0 : r.i;
+                }
             }
+    }
+}
+
+// Second pass of an argmax / argmin whose axis was cut into `parts` segments of `seg` elements: position p of result o
+// has one candidate per segment, at [(o * parts + part) * inner + p].
+template <bool MIN>
+__global__ __launch_bounds__(256) void argreduce_merge_kernel(const float *part_v, const int32_t *part_i, int64_t outer, int64_t parts, int64_t seg, int64_t inner, float start,
+                                                              int64_t *dst) {
+    const int64_t total = outer * inner;
+    for (int64_t q = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; q < total; q += static_cast<int64_t>(gridDim.x) * 256) {
+        const int64_t o = q / inner, p = q - o * inner;
+        ArgBest b{start, INT32_MAX};
+        for (int64_t part = 0; part < parts; ++part) {
+            const int64_t at = (o * parts + part) * inner + p;
+            const int32_t i = part_i[at];
+            if (i != INT32_MAX) arg_merge<MIN>(b, part_v[at], static_cast<int32_t>(part * seg) + i);
+        }
+        dst[q] = b.i == INT32_MAX ? 0 : b.i;
     }
 }
 
@@ -857,12 +883,27 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
 #undef AXHIP_ARG_ROWS_DT
     } else if (inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
         const int64_t ivecs = inner / (16 / es);
-        const bool wide = outer * ((ivecs + 31) / 32) >= 1024;
-        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
+        // Few results over a long axis: too few work-groups for the chip.  The axis is cut into `parts` equal segments
+        // whose candidates (value, index) go to stream-ordered temporary memory and are merged by a second kernel.
+        int64_t parts = 1;
+        if (outer * ((ivecs + 7) / 8) < 512 && axis >= 2048)
+            for (int64_t p = 2; p <= 64 && outer * ((ivecs + 7) / 8) * parts < 1024; ++p)
+                if (axis % p == 0 && axis / p >= 256) parts = p;
+        const int64_t v_outer = outer * parts, v_axis = axis / parts;
+        float *part_v = nullptr;
+        int32_t *part_i = nullptr;
+        if (parts > 1) {
+            void *tmp = nullptr;
+            AXHIP_CHECK_HIP(hipMallocAsync(&tmp, static_cast<size_t>(v_outer * inner) * 8, s));
+            part_v = static_cast<float *>(tmp);
+            part_i = reinterpret_cast<int32_t *>(part_v + v_outer * inner);
+        }
+        const bool wide = v_outer * ((ivecs + 31) / 32) >= 1024;
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(v_outer * (wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
 #define AXHIP_ARG_VEC_TX(DT, TX)                                                                                                           \
     do {                                                                                                                                   \
-        if (want_min) hipLaunchKernelGGL((argreduce_strided_vec_kernel<true, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, start, dst); \
-        else hipLaunchKernelGGL((argreduce_strided_vec_kernel<false, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, start, dst);         \
+        if (want_min) hipLaunchKernelGGL((argreduce_strided_vec_kernel<true, DT, TX>), dim3(blocks), dim3(256), 0, s, src, v_outer, v_axis, inner, start, dst, part_v, part_i); \
+        else hipLaunchKernelGGL((argreduce_strided_vec_kernel<false, DT, TX>), dim3(blocks), dim3(256), 0, s, src, v_outer, v_axis, inner, start, dst, part_v, part_i);         \
     } while (0)
 #define AXHIP_ARG_VEC(DT)                                                                                                                  \
     do {                                                                                                                                   \
@@ -874,6 +915,12 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
         else AXHIP_ARG_VEC(AXHIP_DTYPE_BF16);
 #undef AXHIP_ARG_VEC
 #undef AXHIP_ARG_VEC_TX
+        if (parts > 1) {
+            const unsigned mblocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
+            if (want_min) hipLaunchKernelGGL(argreduce_merge_kernel<true>, dim3(mblocks), dim3(256), 0, s, part_v, part_i, outer, parts, v_axis, inner, start, dst);
+            else hipLaunchKernelGGL(argreduce_merge_kernel<false>, dim3(mblocks), dim3(256), 0, s, part_v, part_i, outer, parts, v_axis, inner, start, dst);
+            AXHIP_CHECK_HIP(hipFreeAsync(part_v, s));
+        }
     } else {
         const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
         if (want_min) hipLaunchKernelGGL(argreduce_strided_kernel<true>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, start, dst);

@@ -280,7 +280,9 @@ int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int6
  * rule (src/backends/cpu/cpu_operations.cpp:2157-2229): the first occurrence of
  * the extreme wins, a NaN never does, and a slice with nothing above the type's
  * lowest() (argmin: below max()) -- all -inf, all NaN -- answers 0.  inner == 1
- * is the row form (greedy decoding over [batch, vocabulary] logits). */
+ * is the row form (greedy decoding over [batch, vocabulary] logits).  Few
+ * results over a long inner-axis run go through stream-ordered temporary
+ * memory (hipMallocAsync on `stream`). */
 int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
                     int32_t want_min, int64_t *dst, void *stream);
 

@@ -221,6 +221,14 @@ def test_argmax_argmin_along_inner_axes_and_on_unaligned_bases(dt):
         for want_min in (False, True):
             got = _argreduce(d, dt, outer, n, inner, want_min).reshape(axo.argreduce(bits, axis, want_min, dt).shape)
             assert np.array_equal(got, axo.argreduce(bits, axis, want_min, dt)), (axis, want_min)
+    # few results over a long axis: the axis is cut into segments and the candidates merged (ties across segments, NaN)
+    y = rng.integers(-3, 4, (1, 8192, 64)).astype(np.float32)
+    y[0, rng.integers(0, 8192, 40), rng.integers(0, 64, 40)] = np.nan
+    y[0, :, 5] = np.nan
+    yb = y if dt == F32 else axo.to_bits(y, dt)
+    dy = gh.to_dev(yb)
+    for want_min in (False, True):
+        assert np.array_equal(_argreduce(dy, dt, 1, 8192, 64, want_min), axo.argreduce(yb, 1, want_min, dt).reshape(-1)), want_min
     # a view that starts one element into the buffer: rows of 4099 elements at every alignment
     flat = rng.normal(size=1 + 12 * 4099).astype(np.float32)
     fb = flat if dt == F32 else axo.to_bits(flat, dt)
