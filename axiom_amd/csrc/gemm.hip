@@ -49,6 +49,84 @@ __device__ __forceinline__ float gemm_epilogue16(int op, float x) {
     }
 }
 
+// ------------------------------------------------------------ skinny products
+// x W^T with at most 8 rows of x (a decoding step: one token, or a handful, against a weight matrix), both operands
+// along k, 16-bit.  The product is bound by reading W once, and a tiling by output tiles would give the chip N / 128
+// work-groups.  Here a wavefront owns R rows of W (R = 1, 2 or 4: enough wavefronts for every SIMD) and walks k with
+// its 64 lanes side by side -- every load covers 1 KiB of one row -- keeping M x R fp32 sums per lane
+// (v_dot2_f32 on the packed pairs: products exact, fp32 accumulation), which the lanes add up at the end; lane 0
+// applies bias, residual and activation.
+struct SkinnyArgs {
+    const uint16_t *x, *w;
+    void *c;
+    const void *bias, *residual;
+    int dtype, epilogue;
+    int N, K, ldx, ldw, ldc;
+};
+
+template <bool BF16> __device__ __forceinline__ float dot8(const uint4_t &a, const uint4_t &b, float acc) {
+    const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (BF16) {
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, aw[i]), __builtin_bit_cast(bf16x2_t, bw[i]), acc, false);
+        } else {
+            typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, aw[i]), __builtin_bit_cast(half2_t, bw[i]), acc, false);
+        }
+    }
+    return acc;
+}
+
+template <bool BF16, int M, int R>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const SkinnyArgs a) {
+    const int lane = threadIdx.x % 64;
+    const int n0 = (blockIdx.x * 4 + threadIdx.x / 64) * R;
+    if (n0 >= a.N) return; // (whole wavefronts)
+    float acc[M][R];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    const uint16_t *wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wrow[r] = a.w + static_cast<int64_t>(min(n0 + r, a.N - 1)) * a.ldw; // (rows past N: the last row again, not stored)
+    constexpr int U = R == 1 ? 4 : R == 2 ? 2 : 1; // k steps requested together: U * R loads of W in flight per lane
+    for (int k0 = lane * 8; k0 < a.K; k0 += 512 * U) {
+        uint4_t wf[U][R], xf[U][M];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + 512 * u;
+            const bool inside = k < a.K; // (K is a multiple of 8)
+#pragma unroll
+            for (int r = 0; r < R; ++r) wf[u][r] = inside ? *reinterpret_cast<const uint4_t *>(wrow[r] + k) : uint4_t{0, 0, 0, 0};
+#pragma unroll
+            for (int m = 0; m < M; ++m) xf[u][m] = inside ? *reinterpret_cast<const uint4_t *>(a.x + static_cast<int64_t>(m) * a.ldx + k) : uint4_t{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[m][r] = dot8<BF16>(wf[u][r], xf[u][m], acc[m][r]);
+    }
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float v = acc[m][r];
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, WAVE);
+            const int n = n0 + r;
+            if (lane == 0 && n < a.N) {
+                if (a.bias) v += load_any(a.bias, a.dtype, n);
+                if (a.residual) v += load_any(a.residual, a.dtype, static_cast<int64_t>(m) * a.ldc + n);
+                store_any(a.c, a.dtype, static_cast<int64_t>(m) * a.ldc + n, gemm_epilogue(a.epilogue, v));
+            }
+        }
+}
+
 // ------------------------------------------------------------------- generic
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const GemmArgs g) {
     __shared__ float As[16][17], Bs[16][17];
@@ -684,6 +762,12 @@ static bool f32_mfma_enabled() {
     return on;
 }
 
+// AXHIP_GEMM_SKINNY=0: products with at most 8 rows on the tiled kernels (for A/B timing)
+static bool skinny_enabled() {
+    static const bool on = [] { const char *e = std::getenv("AXHIP_GEMM_SKINNY"); return !(e && e[0] == '0'); }();
+    return on;
+}
+
 // AXHIP_GEMM_RING_TILE=0..2 forces one ring tile shape (128x128, 64x128, 128x192) for A/B timing
 static int ring_tile_override() {
     static const int v = [] { const char *e = std::getenv("AXHIP_GEMM_RING_TILE"); return (e && e[0] >= '0' && e[0] <= '2') ? e[0] - '0' : -1; }();
@@ -767,7 +851,45 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool nt = !p.trans_a && p.trans_b && p.k % 8 == 0 && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.stride_a % 8 == 0 &&
                     p.stride_b % 8 == 0 && al16(a) && al16(b) && p.ldc < (1 << 21);
-    if (half && nt && p.k > 0 && p.k % TK == 0 && p.m >= BIG && p.n >= BIG && p.lda < (1 << 21) && p.ldb < (1 << 21) && p.batch < 65536 &&
+    // (measured against the tiled kernels, whose k loop costs about 5.5 us per 1024 elements of k whatever N is: one or
+    // two rows always win -- 1 x 4096 x 4096 23.2 -> 4.4 us --, up to four while W stays below 48 M elements, up to
+    // eight on long-k products of up to 24 M elements; beyond that the per-lane sums make the kernel VALU-bound)
+    const int64_t w_elems = p.n * p.k;
+    const bool skinny_pays = p.m <= 2 || (p.m <= 4 && w_elems <= (int64_t(48) << 20)) || (p.m <= 8 && p.k >= 2048 && w_elems <= (int64_t(24) << 20));
+    if (half && nt && p.batch == 1 && skinny_pays && p.k >= 256 && p.n < (1 << 30) && p.k < (1 << 30) && skinny_enabled()) {
+        // a decoding step: bound by one read of W
+        SkinnyArgs k{};
+        k.x = static_cast<const uint16_t *>(a); k.w = static_cast<const uint16_t *>(b); k.c = c; k.bias = p.bias; k.residual = p.residual;
+        k.dtype = p.dtype; k.epilogue = p.epilogue_op;
+        k.N = static_cast<int>(p.n); k.K = static_cast<int>(p.k);
+        k.ldx = static_cast<int>(p.lda); k.ldw = static_cast<int>(p.ldb); k.ldc = static_cast<int>(p.ldc);
+        const int rows_per_wave = p.n >= 16384 ? 4 : p.n >= 4096 ? 2 : 1; // at least two wavefronts per SIMD where N allows
+        const unsigned blocks = static_cast<unsigned>((p.n + 4 * rows_per_wave - 1) / (4 * rows_per_wave));
+        const bool bf = p.dtype == AXHIP_DTYPE_BF16;
+#define AXHIP_SKINNY_R(M, R)                                                                                              \
+    do {                                                                                                                  \
+        if (bf) hipLaunchKernelGGL((gemm_skinny_kernel<true, M, R>), dim3(blocks), dim3(256), 0, s, k);                   \
+        else hipLaunchKernelGGL((gemm_skinny_kernel<false, M, R>), dim3(blocks), dim3(256), 0, s, k);                     \
+    } while (0)
+#define AXHIP_SKINNY(M)                                                                                                   \
+    do {                                                                                                                  \
+        if (rows_per_wave == 4) AXHIP_SKINNY_R(M, 4);                                                                     \
+        else if (rows_per_wave == 2) AXHIP_SKINNY_R(M, 2);                                                                \
+        else AXHIP_SKINNY_R(M, 1);                                                                                        \
+    } while (0)
+        switch (p.m) { // (x's row count is a template constant: the sums live in registers)
+        case 1: AXHIP_SKINNY(1); break;
+        case 2: AXHIP_SKINNY(2); break;
+        case 3: AXHIP_SKINNY(3); break;
+        case 4: AXHIP_SKINNY(4); break;
+        case 5: AXHIP_SKINNY(5); break;
+        case 6: AXHIP_SKINNY(6); break;
+        case 7: AXHIP_SKINNY(7); break;
+        default: AXHIP_SKINNY(8); break;
+        }
+#undef AXHIP_SKINNY
+#undef AXHIP_SKINNY_R
+    } else if (half && nt && p.k > 0 && p.k % TK == 0 && p.m >= BIG && p.n >= BIG && p.lda < (1 << 21) && p.ldb < (1 << 21) && p.batch < 65536 &&
         ((p.m + BIG - 1) / BIG) * ((p.n + BIG - 1) / BIG) * p.batch >= 128) {
         // 256 x 256 tiles once they give at least half the CUs a work-group
         const int tiles_m = static_cast<int>((p.m + BIG - 1) / BIG), tiles_n = static_cast<int>((p.n + BIG - 1) / BIG);

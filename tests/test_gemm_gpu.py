@@ -1,5 +1,7 @@
 """GPU parity of axhip_gemm (the nn::Linear / ops::matmul path) against float64
 and against the CPU oracle's matmul."""
+import math
+
 import numpy as np
 import pytest
 
@@ -144,6 +146,25 @@ def test_large_products_with_operands_not_along_k(dt, ta, tb, K):
     want = (a64.transpose(0, 2, 1) if ta else a64) @ (bb64.transpose(0, 2, 1) if tb else bb64)
     tol = 1e-4 + 1e-4 * np.abs(want) if dt == F32 else 2e-2 + 2.0**-8 * np.abs(want)
     assert np.all(np.abs(got - want) <= tol)
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,extras", [(1, 1280, 1280, False), (1, 4096, 4096, True), (5, 100, 5120, True), (32, 1283, 264, False), (8, 51865, 384, False),
+                                          (3, 2048, 4104, True), (1, 32, 256, False), (2, 4099, 776, True), (7, 16390, 520, False), (4, 1, 264, True)])
+def test_skinny_products_of_a_decoding_step_match_fp64(dt, M, N, K, extras):
+    """A few rows against a weight matrix (x W^T): up to 8 rows take the kernel that walks W's rows with whole
+    wavefronts (1, 2 or 4 rows of W each, by N), ragged N and k tails, bias + residual + GELU; 32 rows stay on the
+    tiled kernels; same bar for both."""
+    g = axo.PCG64(M * 7 + N + K)
+    x, W = axo.to_bits(g.normal((M, K)), dt), axo.to_bits(g.normal((N, K)) * 0.05, dt)
+    bias = axo.to_bits(g.normal((N,)) * 0.1, dt) if extras else None
+    res = axo.to_bits(g.normal((M, N)), dt) if extras else None
+    got = axo.to_f32(gh.gemm(x, W, dt, trans_b=True, bias=bias, residual=res, epilogue="gelu" if extras else None)[0], dt)
+    want = axo.to_f32(x, dt).astype(np.float64) @ axo.to_f32(W, dt).astype(np.float64).T
+    if extras:
+        want = want + axo.to_f32(bias, dt) + axo.to_f32(res, dt)
+        want = 0.5 * want * (1.0 + np.vectorize(math.erf)(want / math.sqrt(2.0)))
+    assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
