@@ -425,12 +425,13 @@ def bench_survey(torch, capi, stream, steps, warmup):
 
 def bench_gemm(torch, capi, stream, steps, warmup):
     """x W^T through axhip_gemm (the nn::Linear product): a large square, the tall product of a
-    long batch, and the Whisper-block projection of BASELINE.json configs[4]."""
+    long batch, the Whisper-block projection of BASELINE.json configs[4], and two decoding steps."""
     lib = capi.lib()
     sp = C.c_void_p(stream.cuda_stream)
     res = {}
     g = torch.Generator(device="cuda").manual_seed(42)
-    for M, N, K in ((4096, 4096, 4096), (8192, 4096, 4096), (1500, 1280, 1280)):
+    # (the last two: decoding steps, one and four tokens against a weight matrix -- bound by reading the weights)
+    for M, N, K in ((4096, 4096, 4096), (8192, 4096, 4096), (1500, 1280, 1280), (1, 4096, 4096), (4, 4096, 4096)):
         a = torch.randn((M, K), generator=g, device="cuda").to(torch.bfloat16)
         w = (torch.randn((N, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
         c = torch.empty((M, N), device="cuda", dtype=torch.bfloat16)
@@ -450,6 +451,9 @@ def bench_gemm(torch, capi, stream, steps, warmup):
                                              "frac_of_mfma_peak": flops / (avg_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                                              "finite": bool(torch.isfinite(c.float()).all().item()),
                                              "hipblaslt_avg_ms": lib_ms}
+        if M <= 8:  # what bounds a decoding step is the one read of W
+            nbytes = 2.0 * (N * K + M * K + M * N)
+            res[f"gemm_nt_bf16_{M}x{N}x{K}"].update({"bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9})
         del a, w, c
     return res
 
