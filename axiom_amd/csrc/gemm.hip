@@ -51,24 +51,28 @@ __device__ __forceinline__ float gemm_epilogue16(int op, float x) {
 
 // ------------------------------------------------------------ skinny products
 // x W^T with at most 8 rows of x (a decoding step: one token, or a handful, against a weight matrix), both operands
-// along k, 16-bit.  The product is bound by reading W once, and a tiling by output tiles would give the chip N / 128
+// along k.  The product is bound by reading W once, and a tiling by output tiles would give the chip N / 128
 // work-groups.  Here a wavefront owns R rows of W (R = 1, 2 or 4: enough wavefronts for every SIMD) and walks k with
 // its 64 lanes side by side -- every load covers 1 KiB of one row -- keeping M x R fp32 sums per lane
-// (v_dot2_f32 on the packed pairs: products exact, fp32 accumulation), which the lanes add up at the end; lane 0
+// (16-bit: v_dot2_f32 on the packed pairs, products exact, fp32 accumulation; fp32: FMAs), which the lanes add up at
+// the end; lane 0
 // applies bias, residual and activation.
 struct SkinnyArgs {
-    const uint16_t *x, *w;
+    const void *x, *w;
     void *c;
     const void *bias, *residual;
     int dtype, epilogue;
     int N, K, ldx, ldw, ldc;
 };
 
-template <bool BF16> __device__ __forceinline__ float dot8(const uint4_t &a, const uint4_t &b, float acc) {
+// acc + the dot product of two 16-byte vectors of DT elements (fp32: four FMAs)
+template <int DT> __device__ __forceinline__ float dot16b(const uint4_t &a, const uint4_t &b, float acc) {
     const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        if constexpr (BF16) {
+        if constexpr (DT == AXHIP_DTYPE_F32) {
+            acc = __builtin_fmaf(__uint_as_float(aw[i]), __uint_as_float(bw[i]), acc);
+        } else if constexpr (DT == AXHIP_DTYPE_BF16) {
             typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
             acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, aw[i]), __builtin_bit_cast(bf16x2_t, bw[i]), acc, false);
         } else {
@@ -79,8 +83,9 @@ template <bool BF16> __device__ __forceinline__ float dot8(const uint4_t &a, con
     return acc;
 }
 
-template <bool BF16, int M, int R>
+template <int DT, int M, int R>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const SkinnyArgs a) {
+    constexpr int E = DT == AXHIP_DTYPE_F32 ? 4 : 8, ES = 16 / E; // elements per 16-byte vector, bytes per element
     const int lane = threadIdx.x % 64;
     const int n0 = (blockIdx.x * 4 + threadIdx.x / 64) * R;
     if (n0 >= a.N) return; // (whole wavefronts)
@@ -89,27 +94,28 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const SkinnyArgs a) {
     for (int m = 0; m < M; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
-    const uint16_t *wrow[R];
+    const char *wrow[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wrow[r] = a.w + static_cast<int64_t>(min(n0 + r, a.N - 1)) * a.ldw; // (rows past N: the last row again, not stored)
+    for (int r = 0; r < R; ++r) wrow[r] = static_cast<const char *>(a.w) + static_cast<int64_t>(min(n0 + r, a.N - 1)) * a.ldw * ES; // (rows past N: the last row again, not stored)
     constexpr int U = R == 1 ? 4 : R == 2 ? 2 : 1; // k steps requested together: U * R loads of W in flight per lane
-    for (int k0 = lane * 8; k0 < a.K; k0 += 512 * U) {
+    for (int k0 = lane * E; k0 < a.K; k0 += 64 * E * U) {
         uint4_t wf[U][R], xf[U][M];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int k = k0 + 512 * u;
-            const bool inside = k < a.K; // (K is a multiple of 8)
+            const int k = k0 + 64 * E * u;
+            const bool inside = k < a.K; // (K is a multiple of E)
 #pragma unroll
-            for (int r = 0; r < R; ++r) wf[u][r] = inside ? *reinterpret_cast<const uint4_t *>(wrow[r] + k) : uint4_t{0, 0, 0, 0};
+            for (int r = 0; r < R; ++r) wf[u][r] = inside ? *reinterpret_cast<const uint4_t *>(wrow[r] + static_cast<int64_t>(k) * ES) : uint4_t{0, 0, 0, 0};
 #pragma unroll
-            for (int m = 0; m < M; ++m) xf[u][m] = inside ? *reinterpret_cast<const uint4_t *>(a.x + static_cast<int64_t>(m) * a.ldx + k) : uint4_t{0, 0, 0, 0};
+            for (int m = 0; m < M; ++m)
+                xf[u][m] = inside ? *reinterpret_cast<const uint4_t *>(static_cast<const char *>(a.x) + (static_cast<int64_t>(m) * a.ldx + k) * ES) : uint4_t{0, 0, 0, 0};
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int m = 0; m < M; ++m)
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[m][r] = dot8<BF16>(wf[u][r], xf[u][m], acc[m][r]);
+                for (int r = 0; r < R; ++r) acc[m][r] = dot16b<DT>(wf[u][r], xf[u][m], acc[m][r]);
     }
 #pragma unroll
     for (int m = 0; m < M; ++m)
@@ -854,22 +860,26 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     // (measured against the tiled kernels, whose k loop costs about 5.5 us per 1024 elements of k whatever N is: one or
     // two rows always win -- 1 x 4096 x 4096 23.2 -> 4.4 us --, up to four while W stays below 48 M elements, up to
     // eight on long-k products of up to 24 M elements; beyond that the per-lane sums make the kernel VALU-bound)
+    // (fp32: the tiled fp32 kernels are an order of magnitude off on such shapes -- 1 x 4096 x 4096 138 -> 12 us --, so
+    // every product of up to eight rows goes here)
     const int64_t w_elems = p.n * p.k;
-    const bool skinny_pays = p.m <= 2 || (p.m <= 4 && w_elems <= (int64_t(48) << 20)) || (p.m <= 8 && p.k >= 2048 && w_elems <= (int64_t(24) << 20));
-    if (half && nt && p.batch == 1 && skinny_pays && p.k >= 256 && p.n < (1 << 30) && p.k < (1 << 30) && skinny_enabled()) {
+    const bool skinny_pays = p.m <= 2 || (p.m <= 8 && p.dtype == AXHIP_DTYPE_F32) || (p.m <= 4 && w_elems <= (int64_t(48) << 20)) ||
+                             (p.m <= 8 && p.k >= 2048 && w_elems <= (int64_t(24) << 20));
+    const bool f32_nt = p.dtype == AXHIP_DTYPE_F32 && !p.trans_a && p.trans_b && p.k % 4 == 0 && p.lda % 4 == 0 && p.ldb % 4 == 0 && al16(a) && al16(b);
+    if (((half && nt) || f32_nt) && p.batch == 1 && skinny_pays && p.k >= 256 && p.n < (1 << 30) && p.k < (1 << 30) && skinny_enabled()) {
         // a decoding step: bound by one read of W
         SkinnyArgs k{};
-        k.x = static_cast<const uint16_t *>(a); k.w = static_cast<const uint16_t *>(b); k.c = c; k.bias = p.bias; k.residual = p.residual;
+        k.x = a; k.w = b; k.c = c; k.bias = p.bias; k.residual = p.residual;
         k.dtype = p.dtype; k.epilogue = p.epilogue_op;
         k.N = static_cast<int>(p.n); k.K = static_cast<int>(p.k);
         k.ldx = static_cast<int>(p.lda); k.ldw = static_cast<int>(p.ldb); k.ldc = static_cast<int>(p.ldc);
         const int rows_per_wave = p.n >= 16384 ? 4 : p.n >= 4096 ? 2 : 1; // at least two wavefronts per SIMD where N allows
         const unsigned blocks = static_cast<unsigned>((p.n + 4 * rows_per_wave - 1) / (4 * rows_per_wave));
-        const bool bf = p.dtype == AXHIP_DTYPE_BF16;
 #define AXHIP_SKINNY_R(M, R)                                                                                              \
     do {                                                                                                                  \
-        if (bf) hipLaunchKernelGGL((gemm_skinny_kernel<true, M, R>), dim3(blocks), dim3(256), 0, s, k);                   \
-        else hipLaunchKernelGGL((gemm_skinny_kernel<false, M, R>), dim3(blocks), dim3(256), 0, s, k);                     \
+        if (p.dtype == AXHIP_DTYPE_BF16) hipLaunchKernelGGL((gemm_skinny_kernel<AXHIP_DTYPE_BF16, M, R>), dim3(blocks), dim3(256), 0, s, k); \
+        else if (p.dtype == AXHIP_DTYPE_F16) hipLaunchKernelGGL((gemm_skinny_kernel<AXHIP_DTYPE_F16, M, R>), dim3(blocks), dim3(256), 0, s, k); \
+        else hipLaunchKernelGGL((gemm_skinny_kernel<AXHIP_DTYPE_F32, M, R>), dim3(blocks), dim3(256), 0, s, k);           \
     } while (0)
 #define AXHIP_SKINNY(M)                                                                                                   \
     do {                                                                                                                  \
