@@ -42,6 +42,11 @@ struct SdpaArgs {
     int nqb; // query blocks per (batch, head)
     int dtype;
     int64_t qs[3], ks[3], vs[3], os[3], ms[2];
+    // key split of sdpa_mfma_kernel (decoding: few query rows, few heads, a long key sequence): `ksplit` work-groups
+    // per (batch, head) take `kchunk` keys each and leave normalised fp32 partial outputs and the base-2 logarithm of
+    // their softmax denominators (reference maximum included) for sdpa_splitk_merge_kernel
+    int ksplit, kchunk;
+    float *opart, *lse;
 };
 
 constexpr float NEG_INF_F = -__builtin_huge_valf();
@@ -102,8 +107,19 @@ __device__ __forceinline__ uint2_t lds_read_tr16(const uint16_t *p) {
 template <int D> constexpr size_t sdpa_mfma_lds_bytes() { return 2 * BN * ((D + 8) + (D + 32)) * 2; }
 extern __shared__ __attribute__((aligned(16))) unsigned char sdpa_dyn_lds[];
 
-template <bool BF16, int D, bool HAS_MASK>
-__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const SdpaArgs a) {
+template <bool BF16, int D, bool HAS_MASK, bool SPLITK = false>
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const SdpaArgs a_in) {
+    static_assert(!SPLITK || !HAS_MASK, "the key split is for unmasked decoding steps");
+    SdpaArgs a = a_in;
+    int L = blockIdx.x, split = 0;
+    if constexpr (SPLITK) { // this work-group's share of the keys: a shorter sequence from a later start
+        split = L % a.ksplit;
+        L /= a.ksplit;
+        const int begin = split * a.kchunk;
+        a.k = static_cast<const uint16_t *>(a.k) + begin * a.ks[2];
+        a.v = static_cast<const uint16_t *>(a.v) + begin * a.vs[2];
+        a.Skv = min(a.kchunk, a.Skv - begin);
+    }
     constexpr int KS_STRIDE = D + 8;   // K row stride (elements): +16 B shifts consecutive rows by 4 banks
     constexpr int VS_STRIDE = D + 32;  // V row stride: +64 B shifts rows by 16 banks, what the 4-row transpose reads need
     constexpr int KT = D / 16;         // k-steps of the first product
@@ -112,10 +128,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
     constexpr int NLD = BN * KCH / 256 > 0 ? BN * KCH / 256 : 1; // 16-byte chunks per thread per tile
     constexpr int ROWS_PER_PASS = 256 / KCH; // rows covered by one chunk pass of the whole workgroup
     constexpr int KBUF = BN * KS_STRIDE, VBUF = BN * VS_STRIDE; // elements per tile buffer
-    __shared__ __attribute__((aligned(16))) uint16_t Ks_static[D > 128 ? 8 : 2 * KBUF];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs_static[D > 128 ? 8 : 2 * VBUF];
-    uint16_t *const Ks = D > 128 ? reinterpret_cast<uint16_t *>(sdpa_dyn_lds) : Ks_static;
-    uint16_t *const Vs = D > 128 ? reinterpret_cast<uint16_t *>(sdpa_dyn_lds) + 2 * KBUF : Vs_static;
+    constexpr bool DYN = D >= 128; // (more than the 64 KiB of static LDS)
+    __shared__ __attribute__((aligned(16))) uint16_t Ks_static[DYN ? 8 : 2 * KBUF];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs_static[DYN ? 8 : 2 * VBUF];
+    uint16_t *const Ks = DYN ? reinterpret_cast<uint16_t *>(sdpa_dyn_lds) : Ks_static;
+    uint16_t *const Vs = DYN ? reinterpret_cast<uint16_t *>(sdpa_dyn_lds) + 2 * KBUF : Vs_static;
 
     const int tid = threadIdx.x;
     const int wave = tid / WAVE, lane = tid % WAVE;
@@ -124,7 +141,6 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
     // Work-group -> (batch*head, query block).  Work-groups are dealt to the 8
     // XCDs round-robin by id; keeping one (batch, head) on one XCD lets its K/V
     // live in that XCD's L2.  Causal blocks are issued heaviest first.
-    const int L = blockIdx.x;
     const int BH = a.B * a.H;
     int bh, qb;
     if (BH % 8 == 0) {
@@ -343,6 +359,21 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
     // ---- epilogue: O = O^T / l, written as 4 consecutive dims (8 bytes) per store
     const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if constexpr (SPLITK) {
+        if (q_ok) {
+            const int64_t slot = (static_cast<int64_t>(bh) * a.ksplit + split) * a.Sq + q;
+            float *orow = a.opart + slot * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const float4_t w = {oacc[dt][4 * i4] * inv, oacc[dt][4 * i4 + 1] * inv, oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv};
+                    *reinterpret_cast<float4_t *>(orow + dt * 32 + i4 * 8 + g * 4) = w;
+                }
+            if (g == 0) a.lse[slot] = l_tot > 0.0f ? m_run + __builtin_amdgcn_logf(l_tot) : NEG_INF_F; // (v_log_f32: base 2, as the exponentials)
+        }
+        return;
+    }
     if (q_ok) {
         uint16_t *orow = O + static_cast<int64_t>(q) * a.os[2];
 #pragma unroll
@@ -354,6 +385,36 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void sdpa_mfma_kernel(const S
                              pack2<BF16>(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv)};
                 if (d < dv) *reinterpret_cast<uint2_t *>(orow + d) = w;
             }
+    }
+}
+
+// out = sum_s 2^(lse_s - max lse) O_s / sum_s 2^(lse_s - max lse) over the `ksplit` partial results of a (batch, head,
+// query row); a thread per (row, four dims)
+template <bool BF16>
+__global__ __launch_bounds__(256) void sdpa_splitk_merge_kernel(const SdpaArgs a, int D) {
+    const int64_t quads = D / 4, total = static_cast<int64_t>(a.B) * a.H * a.Sq * quads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * 256) {
+        const int64_t row = i / quads; // (batch, head, query row)
+        const int d = static_cast<int>(i - row * quads) * 4;
+        const int64_t bh = row / a.Sq;
+        const int q = static_cast<int>(row - bh * a.Sq);
+        float top = NEG_INF_F;
+        for (int s = 0; s < a.ksplit; ++s) top = fmaxf(top, a.lse[(bh * a.ksplit + s) * a.Sq + q]);
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f}, den = 0.0f;
+        if (top != NEG_INF_F)
+            for (int s = 0; s < a.ksplit; ++s) {
+                const int64_t slot = (bh * a.ksplit + s) * a.Sq + q;
+                const float w = __builtin_amdgcn_exp2f(a.lse[slot] - top);
+                const float4_t o = *reinterpret_cast<const float4_t *>(a.opart + slot * D + d);
+                acc[0] += w * o[0]; acc[1] += w * o[1]; acc[2] += w * o[2]; acc[3] += w * o[3];
+                den += w;
+            }
+        const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+        if (d < a.D) {
+            uint16_t *orow = static_cast<uint16_t *>(a.o) + (bh / a.H) * a.os[0] + (bh % a.H) * a.os[1] + static_cast<int64_t>(q) * a.os[2];
+            const uint2_t w = {pack2<BF16>(acc[0] * inv, acc[1] * inv), pack2<BF16>(acc[2] * inv, acc[3] * inv)};
+            *reinterpret_cast<uint2_t *>(orow + d) = w;
+        }
     }
 }
 
@@ -1249,6 +1310,12 @@ int sdpa_d128_waves = [] {
     return e ? atoi(e) : 0;
 }();
 
+// AXHIP_SDPA_DECODE_SPLIT=0: decoding steps on the ordinary kernels (for A/B timing)
+bool sdpa_decode_split = [] {
+    const char *e = getenv("AXHIP_SDPA_DECODE_SPLIT");
+    return !(e && e[0] == '0');
+}();
+
 // AXHIP_SDPA_KEY_SPLIT=0 keeps small head_dim-64 problems on the unsplit kernel (for A/B timing)
 bool sdpa_key_split = [] {
     const char *e = getenv("AXHIP_SDPA_KEY_SPLIT");
@@ -1419,6 +1486,46 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         a.nqb = (p.seq_q + BM - 1) / BM;
         AXHIP_REQUIRE(static_cast<int64_t>(a.nqb) * p.batch * p.heads < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: grid too large");
         const bool bf = p.dtype == AXHIP_DTYPE_BF16;
+        // A decoding step -- one block of query rows, few (batch, head) slices, a long key sequence -- would give the
+        // chip a work-group per slice: the keys are split between work-groups instead (flash decoding), partial
+        // results in stream-ordered temporary memory, merged by a second kernel.
+        const int64_t slices = static_cast<int64_t>(p.batch) * p.heads;
+        // (from 8 M key elements on: below that the second kernel and the temporary memory cost more than they gain --
+        // 20 heads of 1500 keys of 64: 12.5 us unsplit, 21.6 split; 32 heads of 4096 keys of 128: 78.7 -> 27.2 us)
+        if (!mask && !a.causal && p.seq_q <= BM && slices <= 96 && p.seq_kv >= 1024 && p.head_dim > 32 && p.head_dim <= 128 &&
+            slices * p.seq_kv * p.head_dim >= (int64_t(8) << 20) && sdpa_decode_split) {
+            const int DD = p.head_dim <= 64 ? 64 : 128;
+            int parts = static_cast<int>(std::min<int64_t>(std::min<int64_t>(64, (512 + slices - 1) / slices), p.seq_kv / 256));
+            a.kchunk = ((p.seq_kv + parts - 1) / parts + BN - 1) / BN * BN;
+            a.ksplit = (p.seq_kv + a.kchunk - 1) / a.kchunk;
+            const size_t rows = static_cast<size_t>(slices) * a.ksplit * p.seq_q;
+            void *tmp = nullptr;
+            AXHIP_CHECK_HIP(hipMallocAsync(&tmp, rows * (DD + 1) * sizeof(float), s));
+            a.opart = static_cast<float *>(tmp);
+            a.lse = a.opart + rows * DD;
+            a.nqb = 1;
+            const unsigned grid = static_cast<unsigned>(slices * a.ksplit);
+            if (DD == 64) {
+                if (bf) hipLaunchKernelGGL((sdpa_mfma_kernel<true, 64, false, true>), dim3(grid), dim3(256), 0, s, a);
+                else hipLaunchKernelGGL((sdpa_mfma_kernel<false, 64, false, true>), dim3(grid), dim3(256), 0, s, a);
+            } else {
+                constexpr size_t lds = sdpa_mfma_lds_bytes<128>();
+                static const bool configured = [] {
+                    return hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_mfma_kernel<true, 128, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
+                           hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_mfma_kernel<false, 128, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
+                }();
+                AXHIP_REQUIRE(configured, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: cannot reserve %zu bytes of LDS", lds);
+                if (bf) hipLaunchKernelGGL((sdpa_mfma_kernel<true, 128, false, true>), dim3(grid), dim3(256), lds, s, a);
+                else hipLaunchKernelGGL((sdpa_mfma_kernel<false, 128, false, true>), dim3(grid), dim3(256), lds, s, a);
+            }
+            const int64_t items = slices * p.seq_q * (DD / 4);
+            const unsigned mgrid = static_cast<unsigned>(std::min<int64_t>((items + 255) / 256, 4096));
+            if (bf) hipLaunchKernelGGL(sdpa_splitk_merge_kernel<true>, dim3(mgrid), dim3(256), 0, s, a, DD);
+            else hipLaunchKernelGGL(sdpa_splitk_merge_kernel<false>, dim3(mgrid), dim3(256), 0, s, a, DD);
+            AXHIP_CHECK_HIP(hipFreeAsync(tmp, s));
+            AXHIP_CHECK_HIP(hipGetLastError());
+            return AXHIP_OK;
+        }
         switch (p.head_dim <= 32 ? 32 : p.head_dim > 128 ? 256 : 64) {
         case 32: rc = bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
         case 256: rc = bf ? launch_mfma<true, 256>(a, s) : launch_mfma<false, 256>(a, s); break;

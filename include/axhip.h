@@ -78,7 +78,11 @@ int axhip_stream_sync(void *stream);
  * pointers, strides that are multiples of 8 elements; fp32: 4); everything
  * else up to D = 256 runs on the generic fp32-FMA kernel, which takes the
  * place of the reference's decomposed_attention fallback
- * (flash_attention_dispatch.mm:125-162).  axhip_sdpa_kernel_name tells which. */
+ * (flash_attention_dispatch.mm:125-162).  axhip_sdpa_kernel_name tells which.
+ * A decoding step (up to 128 query rows, at most 96 (batch, head) slices, a
+ * long unmasked key sequence) splits its keys between work-groups and merges
+ * the partial results through stream-ordered temporary memory
+ * (hipMallocAsync on `stream`). */
 typedef struct {
     int32_t dtype;
     int32_t batch, heads, seq_q, seq_kv, head_dim;

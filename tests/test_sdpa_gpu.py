@@ -212,6 +212,24 @@ def test_fp32_multiples_of_four_and_small_16_bit_head_sizes_run_on_the_matrix_co
     assert np.max(np.abs(gf[..., :D].transpose(0, 2, 1, 3) - naive_attention64(qf, kf, vf, 1 / math.sqrt(D), False))) < 1e-4
 
 
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+def test_decoding_steps_split_their_keys_between_work_groups(dt):
+    """Few query rows, few (batch, head) slices, a long key sequence: the keys are split between work-groups and the
+    partial results merged (head sizes 64, 128 and in between, ragged last chunks, one to 128 query rows, a key
+    sequence with one dominant key in the last chunk); against float64."""
+    tag = "bf16" if dt == BF16 else "f16"
+    for B, H, Sq, Skv, D in ((1, 8, 1, 8192, 128), (2, 8, 5, 9001, 64), (1, 30, 128, 3030, 96), (1, 32, 1, 4096, 128), (1, 64, 33, 3072, 48), (3, 32, 2, 1500, 64)):
+        q, k, v = inputs(B, H, Sq, Skv, D, dt, seed=700 + Sq + D)
+        kf = axo.to_f32(k, dt)
+        kf[..., Skv - 3, :] = 4.0 * axo.to_f32(q, dt)[..., 0, :]  # a key far above the rest, in the last chunk
+        k = axo.to_bits(kf, dt)
+        got, kern = gh.sdpa(q, k, v, dt, -1.0, False, None)
+        assert kern == f"mfma_{tag}_d{D}"
+        want = naive_attention64(*(axo.to_f32(t, dt) for t in (q, k, v)), 1 / math.sqrt(D), False, None)
+        err = np.max(np.abs(axo.to_f32(got, dt) - want))
+        assert err < 2e-2, (B, H, Sq, Skv, D, float(err))
+
+
 def test_fully_masked_rows_give_zeros_everywhere_else_matches():
     q, k, v = inputs(1, 2, 70, 70, 64, BF16, seed=3)
     m = np.zeros((70, 70), np.uint8)
