@@ -151,7 +151,48 @@ def _rows_program(capi, x, out, dt, out_dt):
     return p
 
 
+COLD_MIN_BYTES = 1 << 30  # bytes of other buffers touched between two uses of one buffer set in the rotating ("cold") timing
+
+
+def time_rotating(torch, stream, launchers, steps, warmup):
+    """Average launch duration in ms over exactly `steps` launches that rotate through `launchers` (the same program
+    over independent buffer sets, sized by the caller so that at least COLD_MIN_BYTES of other data pass through the
+    caches between two uses of one set: the inputs then come from HBM, not from the 256 MiB memory-side cache)."""
+    state = {"i": 0}
+
+    def launch():
+        launchers[state["i"] % len(launchers)]()
+        state["i"] += 1
+
+    avg_ms, min_ms, ran = time_launches(torch, stream, launch, steps, warmup)
+    return avg_ms, min_ms, ran
+
+
+def _chain_record(lib, capi, p, avg_ms, min_ms, warm_n, cold_ms, cold_min_ms, n_sets, set_bytes, nbytes):
+    import ctypes as C
+
+    return {
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "bytes": nbytes,
+        # inputs from HBM: launches rotate over `buffer_sets` independent input/output sets
+        "avg_ms": cold_ms, "min_ms": cold_min_ms, "gbs": nbytes / (cold_ms * 1e-3) / 1e9,
+        "frac_of_hbm_peak": nbytes / (cold_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "frac_of_hbm_peak_cold": nbytes / (cold_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "buffer_sets": n_sets, "bytes_touched_between_reuse": (n_sets - 1) * set_bytes,
+        # back-to-back launches on ONE buffer set: part of the input is re-found in the memory-side cache
+        "avg_ms_same_buffers": avg_ms, "min_ms_same_buffers": min_ms, "warmup_launches": warm_n,
+        "frac_of_hbm_peak_same_buffers": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+    }
+
+
+def _sets_for(set_bytes: int) -> int:
+    return max(3, -(-COLD_MIN_BYTES // set_bytes) + 1)
+
+
 def bench_chains(torch, capi, stream, steps, warmup):
+    """The fused-chain kernels of BASELINE.json configs[1] and [2].  Two timings each: `frac_of_hbm_peak` (=
+    `frac_of_hbm_peak_cold`) rotates every launch over enough independent buffer sets that at least 1 GiB of other
+    data is touched between two uses of a buffer -- the inputs come from HBM; `frac_of_hbm_peak_same_buffers` is the
+    back-to-back figure on one set, part of whose input survives in the 256 MiB memory-side cache."""
     lib = capi.lib()
     sp = C.c_void_p(stream.cuda_stream)
     res = {}
@@ -159,30 +200,37 @@ def bench_chains(torch, capi, stream, steps, warmup):
 
     # configs[1]: softmax((relu(a)+1)*b, -1).sum(1), fp32 [8192, 8192]
     R = Cc = 8192
-    a = torch.randn((R, Cc), generator=g, device="cuda")
-    b = torch.randn((R, Cc), generator=g, device="cuda")
+    set_bytes = 2 * R * Cc * 4
+    n_sets = _sets_for(set_bytes)
     one = torch.ones(1, device="cuda")
-    out = torch.empty(R, device="cuda")
-    p = _rows_program(capi, a, out, capi.DTYPE_F32, capi.DTYPE_F32)
-    p.n_operands = 2
-    p.operands[0].ptr, p.operands[0].dtype, p.operands[0].kind = one.data_ptr(), capi.DTYPE_F32, capi.BK["scalar"]
-    p.operands[1].ptr, p.operands[1].dtype, p.operands[1].kind = b.data_ptr(), capi.DTYPE_F32, capi.BK["full"]
-    p.n_pre = 3
-    p.pre[0].op, p.pre[0].operand = capi.OP["relu"], -1
-    p.pre[1].op, p.pre[1].operand = capi.OP["add"], 0
-    p.pre[2].op, p.pre[2].operand = capi.OP["mul"], 1
-    p.row_op = capi.ROWOP["softmax"]
-    p.reduce = capi.RED["sum"]
+    sets, progs = [], []
+    for _ in range(n_sets):
+        a = torch.randn((R, Cc), generator=g, device="cuda")
+        b = torch.randn((R, Cc), generator=g, device="cuda")
+        out = torch.empty(R, device="cuda")
+        p = _rows_program(capi, a, out, capi.DTYPE_F32, capi.DTYPE_F32)
+        p.n_operands = 2
+        p.operands[0].ptr, p.operands[0].dtype, p.operands[0].kind = one.data_ptr(), capi.DTYPE_F32, capi.BK["scalar"]
+        p.operands[1].ptr, p.operands[1].dtype, p.operands[1].kind = b.data_ptr(), capi.DTYPE_F32, capi.BK["full"]
+        p.n_pre = 3
+        p.pre[0].op, p.pre[0].operand = capi.OP["relu"], -1
+        p.pre[1].op, p.pre[1].operand = capi.OP["add"], 0
+        p.pre[2].op, p.pre[2].operand = capi.OP["mul"], 1
+        p.row_op = capi.ROWOP["softmax"]
+        p.reduce = capi.RED["sum"]
+        sets.append((a, b, out))
+        progs.append(p)
+    launchers = [(lambda q=q: capi.check(lib.axhip_fused_rows(C.byref(q), sp))) for q in progs]
     torch.cuda.synchronize()
-    avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, launchers[0], steps, warmup)
+    cold_ms, cold_min, _ = time_rotating(torch, stream, launchers, steps, warmup)
     nbytes = 2 * R * Cc * 4 + R * 4
-    res["chain_relu_add_mul_softmax_sum_f32_8192x8192"] = {
-        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
-        "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-        "rows_sum_to_one": bool(torch.allclose(out, torch.ones_like(out), atol=1e-4)),
-    }
+    rec = _chain_record(lib, capi, progs[0], avg_ms, min_ms, warm_n, cold_ms, cold_min, n_sets, set_bytes, nbytes)
+    rec["rows_sum_to_one"] = bool(all(torch.allclose(s[2], torch.ones_like(s[2]), atol=1e-4) for s in sets))
+    res["chain_relu_add_mul_softmax_sum_f32_8192x8192"] = rec
     # plain copy of the same matrix through the elementwise kernel (empty chain): the kernel of
     # known traffic that the rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by
+    a = sets[0][0]
     cp = torch.empty_like(a)
     pc = _rows_program(capi, a, cp, capi.DTYPE_F32, capi.DTYPE_F32)
     torch.cuda.synchronize()
@@ -193,47 +241,57 @@ def bench_chains(torch, capi, stream, steps, warmup):
         "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
         "bit_exact": bool(torch.equal(cp, a)),
     }
-    del a, b, cp
+    del a, cp, sets, progs, launchers
 
     # configs[2]: gelu(layernorm(x)*gamma+beta) and the RMSNorm variant, bf16 [16384, 4096]
     R, Cc = 16384, 4096
-    x = torch.randn((R, Cc), generator=g, device="cuda").to(torch.bfloat16)
+    set_bytes = 2 * R * Cc * 2
+    n_sets = _sets_for(set_bytes)
+    xs = [torch.randn((R, Cc), generator=g, device="cuda").to(torch.bfloat16) for _ in range(n_sets)]
+    ys = [torch.empty_like(x) for x in xs]
     gamma = (torch.rand(Cc, generator=g, device="cuda") + 0.5).to(torch.bfloat16)
     beta = (torch.rand(Cc, generator=g, device="cuda") * 0.2 - 0.1).to(torch.bfloat16)
-    y = torch.empty_like(x)
     for name, rowop, has_bias in (("layernorm", "layernorm", True), ("rmsnorm", "rmsnorm", False)):
-        p = _rows_program(capi, x, y, capi.DTYPE_BF16, capi.DTYPE_BF16)
-        p.n_operands = 2
-        p.operands[0].ptr, p.operands[0].dtype, p.operands[0].kind = gamma.data_ptr(), capi.DTYPE_BF16, capi.BK["rowvec"]
-        p.operands[1].ptr, p.operands[1].dtype, p.operands[1].kind = beta.data_ptr(), capi.DTYPE_BF16, capi.BK["rowvec"]
-        p.row_op, p.eps = capi.ROWOP[rowop], 1e-5
-        p.norm_weight, p.norm_bias = 0, (1 if has_bias else -1)
-        p.n_post = 1
-        p.post[0].op, p.post[0].operand = capi.OP["gelu"], -1
-        p.reduce = capi.RED["none"]
+        progs = []
+        for x, y in zip(xs, ys):
+            p = _rows_program(capi, x, y, capi.DTYPE_BF16, capi.DTYPE_BF16)
+            p.n_operands = 2
+            p.operands[0].ptr, p.operands[0].dtype, p.operands[0].kind = gamma.data_ptr(), capi.DTYPE_BF16, capi.BK["rowvec"]
+            p.operands[1].ptr, p.operands[1].dtype, p.operands[1].kind = beta.data_ptr(), capi.DTYPE_BF16, capi.BK["rowvec"]
+            p.row_op, p.eps = capi.ROWOP[rowop], 1e-5
+            p.norm_weight, p.norm_bias = 0, (1 if has_bias else -1)
+            p.n_post = 1
+            p.post[0].op, p.post[0].operand = capi.OP["gelu"], -1
+            p.reduce = capi.RED["none"]
+            progs.append(p)
+        launchers = [(lambda q=q: capi.check(lib.axhip_fused_rows(C.byref(q), sp))) for q in progs]
         torch.cuda.synchronize()
-        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launchers[0], steps, warmup)
+        cold_ms, cold_min, _ = time_rotating(torch, stream, launchers, steps, warmup)
         nbytes = 2 * R * Cc * 2 + Cc * 2 * (2 if has_bias else 1)
-        res[f"chain_gelu_{name}_bf16_16384x4096"] = {
-            "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
-            "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-            "finite": bool(torch.isfinite(y.float()).all().item()),
-        }
+        rec = _chain_record(lib, capi, progs[0], avg_ms, min_ms, warm_n, cold_ms, cold_min, n_sets, set_bytes, nbytes)
+        rec["finite"] = bool(all(torch.isfinite(y.float()).all().item() for y in ys))
+        res[f"chain_gelu_{name}_bf16_16384x4096"] = rec
+    del xs, ys
     # a row length that the 16-byte vector does not divide (Whisper's 1500 frames): the kernels' ragged variant
     Rr, Cr = 30000, 1500
-    xr = torch.randn((Rr, Cr), generator=g, device="cuda").to(torch.bfloat16)
-    yr = torch.empty_like(xr)
-    p = _rows_program(capi, xr, yr, capi.DTYPE_BF16, capi.DTYPE_BF16)
-    p.row_op, p.reduce = capi.ROWOP["softmax"], capi.RED["none"]
+    set_bytes = 2 * Rr * Cr * 2
+    n_sets = _sets_for(set_bytes)
+    xs = [torch.randn((Rr, Cr), generator=g, device="cuda").to(torch.bfloat16) for _ in range(n_sets)]
+    ys = [torch.empty_like(x) for x in xs]
+    progs = []
+    for x, y in zip(xs, ys):
+        p = _rows_program(capi, x, y, capi.DTYPE_BF16, capi.DTYPE_BF16)
+        p.row_op, p.reduce = capi.ROWOP["softmax"], capi.RED["none"]
+        progs.append(p)
+    launchers = [(lambda q=q: capi.check(lib.axhip_fused_rows(C.byref(q), sp))) for q in progs]
     torch.cuda.synchronize()
-    avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(p), sp)), steps, warmup)
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, launchers[0], steps, warmup)
+    cold_ms, cold_min, _ = time_rotating(torch, stream, launchers, steps, warmup)
     nbytes = 2 * Rr * Cr * 2
-    sums = yr.float().sum(1)
-    res["softmax_bf16_30000x1500_odd_row_length"] = {
-        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
-        "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-        "rows_sum_to_one": bool(((sums - 1.0).abs() < 2e-2).all().item()),
-    }
+    rec = _chain_record(lib, capi, progs[0], avg_ms, min_ms, warm_n, cold_ms, cold_min, n_sets, set_bytes, nbytes)
+    rec["rows_sum_to_one"] = bool(all(((y.float().sum(1) - 1.0).abs() < 2e-2).all().item() for y in ys))
+    res["softmax_bf16_30000x1500_odd_row_length"] = rec
     return res
 
 
