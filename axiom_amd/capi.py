@@ -87,6 +87,7 @@ def lib() -> C.CDLL:
         l.axhip_default_stream.restype = C.c_void_p
         l.axhip_sdpa_kernel_name.restype = C.c_char_p
         l.axhip_sdpa_kernel_name.argtypes = [C.POINTER(SdpaParams)]
+        l.axhip_sdpa_last_schedule.restype = C.c_char_p
         l.axhip_fused_rows_kernel_name.restype = C.c_char_p
         l.axhip_fused_rows_kernel_name.argtypes = [C.POINTER(RowsProgram)]
         l.axhip_full_reduce_workspace_bytes.restype = C.c_size_t
@@ -100,7 +101,12 @@ def lib() -> C.CDLL:
             getattr(l, name).argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         l.axhip_stream_sync.argtypes = [C.c_void_p]
         l.axhip_sdpa_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(SdpaParams), C.c_void_p]
+        l.axhip_sdpa_workspace_bytes.restype = C.c_size_t
+        l.axhip_sdpa_workspace_bytes.argtypes = [C.POINTER(SdpaParams), C.c_int]
+        l.axhip_sdpa_fwd_ws.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(SdpaParams), C.c_void_p, C.c_size_t, C.c_void_p]
         l.axhip_fused_rows.argtypes = [C.POINTER(RowsProgram), C.c_void_p]
+        l.axhip_fused_rows_jit_counters.restype = None
+        l.axhip_fused_rows_jit_counters.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int)]
         l.axhip_fused_rows_prepare.argtypes = [C.POINTER(RowsProgram)]
         l.axhip_fused_full_reduce.argtypes = [C.POINTER(RowsProgram), C.c_void_p, C.c_size_t, C.c_void_p]
         l.axhip_fused_full_reduce_noalloc.argtypes = [C.POINTER(RowsProgram), C.c_void_p]
@@ -109,11 +115,20 @@ def lib() -> C.CDLL:
                                          C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p]
         l.axhip_fill.argtypes = [C.c_void_p, C.c_int32, C.c_double, C.c_int64, C.c_void_p]
         l.axhip_gemm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(GemmParams), C.c_void_p]
+        l.axhip_gemm_workspace_bytes.restype = C.c_size_t
+        l.axhip_gemm_workspace_bytes.argtypes = [C.POINTER(GemmParams)]
+        l.axhip_gemm_ws.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(GemmParams), C.c_void_p, C.c_size_t, C.c_void_p]
         i64p = C.POINTER(C.c_int64)
         l.axhip_pad.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, i64p, i64p, i64p, i64p, C.c_double, C.c_void_p]
         l.axhip_masked_fill.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, i64p, i64p, i64p, C.c_double, C.c_void_p]
         l.axhip_argreduce.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         l.axhip_reduce_axis.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]
+        l.axhip_argreduce_workspace_bytes.restype = C.c_size_t
+        l.axhip_argreduce_workspace_bytes.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64]
+        l.axhip_argreduce_ws.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        l.axhip_reduce_axis_workspace_bytes.restype = C.c_size_t
+        l.axhip_reduce_axis_workspace_bytes.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64]
+        l.axhip_reduce_axis_ws.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_size_t, C.c_void_p]
         l.axhip_softmax_axis.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         l.axhip_gather_rows.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]
         _lib = l

@@ -35,6 +35,63 @@ int rows_setup_device(); // per-device set-up of the fused-row kernels (rows.hip
         }                                             \
     } while (0)
 
+// Temporary device memory of ONE call.  With a caller's workspace (the *_ws entry points) it hands out 256-byte
+// aligned slices of that and allocates nothing; without one (workspace == NULL) every request is a stream-ordered
+// allocation that is returned in stream order when the call ends.
+class CallScratch {
+public:
+    CallScratch(void *workspace, size_t workspace_bytes, hipStream_t stream)
+        : base_(static_cast<char *>(workspace)), bytes_(workspace_bytes), stream_(stream) {}
+    CallScratch(const CallScratch &) = delete;
+    CallScratch &operator=(const CallScratch &) = delete;
+    ~CallScratch() { (void)release(); }
+    static size_t rounded(size_t n) { return (n + 255) & ~static_cast<size_t>(255); }
+    int take(void **out, size_t n, const char *who) {
+        *out = nullptr;
+        if (base_) {
+            const size_t at = rounded(used_);
+            if (at + n > bytes_) {
+                set_last_error("%s: the workspace holds %zu bytes, the call needs %zu (ask %s_workspace_bytes)", who, bytes_, at + n, who);
+                return AXHIP_ERR_WORKSPACE;
+            }
+            *out = base_ + at;
+            used_ = at + n;
+            return AXHIP_OK;
+        }
+        if (n_own_ >= MAX_OWN) {
+            set_last_error("%s: too many temporary allocations in one call", who);
+            return AXHIP_ERR_UNSUPPORTED;
+        }
+        const hipError_t e = hipMallocAsync(out, n, stream_);
+        if (e != hipSuccess) {
+            set_last_error("%s: hipMallocAsync of %zu bytes failed: %s", who, n, hipGetErrorString(e));
+            return static_cast<int>(e);
+        }
+        own_[n_own_++] = *out;
+        return AXHIP_OK;
+    }
+    // everything handed out so far may be handed out again (work on one stream runs in order)
+    void rewind() { if (base_) used_ = 0; }
+    int release() {
+        hipError_t first = hipSuccess;
+        for (int i = 0; i < n_own_; ++i) {
+            const hipError_t e = hipFreeAsync(own_[i], stream_);
+            if (first == hipSuccess) first = e;
+        }
+        n_own_ = 0;
+        if (first != hipSuccess) set_last_error("hipFreeAsync failed: %s", hipGetErrorString(first));
+        return static_cast<int>(first);
+    }
+
+private:
+    static constexpr int MAX_OWN = 8;
+    char *base_;
+    size_t bytes_, used_ = 0;
+    hipStream_t stream_;
+    void *own_[MAX_OWN] = {};
+    int n_own_ = 0;
+};
+
 inline bool valid_dtype(int dt) { return dt >= AXHIP_DTYPE_F32 && dt <= AXHIP_DTYPE_BF16; }
 inline size_t dtype_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
 // Outputs of at least this size are written with non-temporal stores: they cannot stay in the

@@ -780,7 +780,51 @@ static int ring_tile_override() {
     return v;
 }
 
+namespace {
+// whether (and into how many padded columns) a product is repacked before it runs on the k-contiguous kernels
+struct Repack { bool on, a, b; int64_t kp; };
+Repack repack_plan(const AxhipGemmParams &p) {
+    const int64_t kvec = p.dtype == AXHIP_DTYPE_F32 ? 4 : 8;
+    const bool pad_k = p.k % kvec != 0;
+    Repack r{false, false, false, p.k};
+    if ((p.trans_a || !p.trans_b || pad_k) && p.k >= 32 &&
+        2.0 * static_cast<double>(p.m) * static_cast<double>(p.n) * static_cast<double>(p.k) * static_cast<double>(p.batch) >= double(1 << 30)) { // (about 70 us on the FMA kernel)
+        r.on = true;
+        r.kp = pad_k ? (p.k + 63) / 64 * 64 : p.k;
+        r.a = p.trans_a || pad_k;
+        r.b = !p.trans_b || pad_k;
+    }
+    return r;
+}
+size_t repack_bytes(const AxhipGemmParams &p) {
+    const Repack r = repack_plan(p);
+    if (!r.on) return 0;
+    const size_t es = p.dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    size_t n = 0;
+    if (r.a) n += CallScratch::rounded(static_cast<size_t>(p.stride_a == 0 ? 1 : p.batch) * p.m * r.kp * es);
+    if (r.b) n += CallScratch::rounded(static_cast<size_t>(p.stride_b == 0 ? 1 : p.batch) * p.n * r.kp * es);
+    return n;
+}
+int gemm_impl(const void *a, const void *b, void *c, const AxhipGemmParams *params, CallScratch *scratch_in, void *workspace, size_t workspace_bytes, void *stream);
+} // namespace
+
+extern "C" size_t axhip_gemm_workspace_bytes(const AxhipGemmParams *params) {
+    if (!params || !valid_dtype(params->dtype) || params->m <= 0 || params->n <= 0 || params->k < 0 || params->batch <= 0) return 0;
+    AxhipGemmParams part = *params;
+    part.batch = std::min<int64_t>(part.batch, 65535); // larger batches run as consecutive launches that share the workspace
+    return repack_bytes(part);
+}
+
 extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemmParams *params, void *stream) {
+    return gemm_impl(a, b, c, params, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int axhip_gemm_ws(const void *a, const void *b, void *c, const AxhipGemmParams *params, void *workspace, size_t workspace_bytes, void *stream) {
+    return gemm_impl(a, b, c, params, nullptr, workspace, workspace_bytes, stream);
+}
+
+namespace {
+int gemm_impl(const void *a, const void *b, void *c, const AxhipGemmParams *params, CallScratch *scratch_in, void *workspace, size_t workspace_bytes, void *stream) {
     AXHIP_REQUIRE(params != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_gemm: params is NULL");
     const AxhipGemmParams &p = *params;
     AXHIP_REQUIRE(valid_dtype(p.dtype), AXHIP_ERR_INVALID_ARG, "axhip_gemm: bad dtype %d", p.dtype);
@@ -798,8 +842,8 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
             AxhipGemmParams part = p;
             part.batch = std::min<int64_t>(65535, p.batch - b0);
             if (p.residual) part.residual = static_cast<const char *>(p.residual) + b0 * p.stride_c * es;
-            const int rc_part = axhip_gemm(static_cast<const char *>(a) + b0 * p.stride_a * es, static_cast<const char *>(b) + b0 * p.stride_b * es,
-                                           static_cast<char *>(c) + b0 * p.stride_c * es, &part, stream);
+            const int rc_part = gemm_impl(static_cast<const char *>(a) + b0 * p.stride_a * es, static_cast<const char *>(b) + b0 * p.stride_b * es,
+                                          static_cast<char *>(c) + b0 * p.stride_c * es, &part, nullptr, workspace, workspace_bytes, stream);
             if (rc_part) return rc_part;
         }
         return AXHIP_OK;
@@ -813,36 +857,34 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     // number of vectors, leaves only the FMA kernel below, a hundred times slower on a large product.  Such a product
     // is repacked first, into stream-ordered temporary memory (freed in stream order behind the product): the operand
     // that lies the other way is transposed; an unaligned k is zero-padded to the next multiple of 64 in both operands.
-    const int64_t kvec = p.dtype == AXHIP_DTYPE_F32 ? 4 : 8;
-    const bool pad_k = p.k % kvec != 0;
-    if ((p.trans_a || !p.trans_b || pad_k) && p.k >= 32 &&
-        2.0 * static_cast<double>(p.m) * static_cast<double>(p.n) * static_cast<double>(p.k) * static_cast<double>(p.batch) >= double(1 << 30)) { // (about 70 us on the FMA kernel)
-        const int64_t es = p.dtype == AXHIP_DTYPE_F32 ? 4 : 2, kp = pad_k ? (p.k + 63) / 64 * 64 : p.k;
+    const Repack rp = repack_plan(p);
+    if (rp.on && !scratch_in) {
+        const bool pad_k = rp.kp != p.k;
+        const int64_t es = p.dtype == AXHIP_DTYPE_F32 ? 4 : 2, kp = rp.kp;
         AxhipGemmParams q = p;
         q.k = kp;
+        CallScratch scratch(workspace, workspace_bytes, s);
         void *ta = nullptr, *tb = nullptr;
         // a contiguous [copies, rows, kp] image of an operand whose element (row, kk) lies at row * rs + kk * cs
         auto repacked = [&](const void *src, int64_t rows, int64_t rs, int64_t cs, int64_t batch_stride, void **out) -> int {
             const int64_t copies = batch_stride == 0 ? 1 : p.batch;
-            AXHIP_CHECK_HIP(hipMallocAsync(out, static_cast<size_t>(copies * rows * kp * es), s));
+            const int rc_take = scratch.take(out, static_cast<size_t>(copies * rows * kp * es), "axhip_gemm");
+            if (rc_take) return rc_take;
             const int64_t shape[3] = {copies, rows, p.k}, strides[3] = {batch_stride, rs, cs}, before[3] = {0, 0, 0}, after[3] = {0, 0, kp - p.k};
             if (pad_k) return axhip_pad(src, *out, p.dtype, 3, shape, strides, before, after, 0.0, stream);
             return axhip_strided_copy(src, p.dtype, *out, p.dtype, 3, shape, strides, stream);
         };
-        if (p.trans_a || pad_k) {
+        if (rp.a) {
             rc = repacked(a, p.m, p.trans_a ? 1 : p.lda, p.trans_a ? p.lda : 1, p.stride_a, &ta);
             q.trans_a = 0; q.lda = kp; q.stride_a = p.stride_a == 0 ? 0 : p.m * kp;
         }
-        if (!rc && (!p.trans_b || pad_k)) {
+        if (!rc && rp.b) {
             rc = repacked(b, p.n, p.trans_b ? p.ldb : 1, p.trans_b ? 1 : p.ldb, p.stride_b, &tb);
             q.trans_b = 1; q.ldb = kp; q.stride_b = p.stride_b == 0 ? 0 : p.n * kp;
         }
-        if (!rc) rc = axhip_gemm(ta ? ta : a, tb ? tb : b, c, &q, stream);
-        hipError_t freed = ta ? hipFreeAsync(ta, s) : hipSuccess;
-        if (tb && freed == hipSuccess) freed = hipFreeAsync(tb, s);
-        else if (tb) (void)hipFreeAsync(tb, s);
-        if (!rc) AXHIP_CHECK_HIP(freed);
-        return rc;
+        if (!rc) rc = gemm_impl(ta ? ta : a, tb ? tb : b, c, &q, &scratch, nullptr, 0, stream); // (q is not repacked again)
+        const int freed = scratch.release();
+        return rc ? rc : freed;
     }
 
     GemmArgs g{};
@@ -866,7 +908,9 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     const bool skinny_pays = p.m <= 2 || (p.m <= 8 && p.dtype == AXHIP_DTYPE_F32) || (p.m <= 4 && w_elems <= (int64_t(48) << 20)) ||
                              (p.m <= 8 && p.k >= 2048 && w_elems <= (int64_t(24) << 20));
     const bool f32_nt = p.dtype == AXHIP_DTYPE_F32 && !p.trans_a && p.trans_b && p.k % 4 == 0 && p.lda % 4 == 0 && p.ldb % 4 == 0 && al16(a) && al16(b);
-    if (((half && nt) || f32_nt) && p.batch == 1 && skinny_pays && p.k >= 256 && p.n < (1 << 30) && p.k < (1 << 30) && skinny_enabled()) {
+    // (the kernel carries leading dimensions as 32-bit element counts)
+    const bool ld32 = p.lda < (int64_t(1) << 31) && p.ldb < (int64_t(1) << 31) && p.ldc < (int64_t(1) << 31);
+    if (((half && nt) || f32_nt) && p.batch == 1 && skinny_pays && p.k >= 256 && p.n < (1 << 30) && p.k < (1 << 30) && ld32 && skinny_enabled()) {
         // a decoding step: bound by one read of W
         SkinnyArgs k{};
         k.x = a; k.w = b; k.c = c; k.bias = p.bias; k.residual = p.residual;
@@ -1015,3 +1059,4 @@ extern "C" int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemm
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;
 }
+} // namespace

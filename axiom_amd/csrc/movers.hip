@@ -840,7 +840,30 @@ int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int6
     return AXHIP_OK;
 }
 
+// segments the axis is cut into when few results stand over a long axis (1: no cut, no temporary memory)
+static int64_t argreduce_parts(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner) {
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    if (inner <= 1 || inner % (16 / es) != 0 || (reinterpret_cast<uintptr_t>(src) & 15u) != 0) return 1;
+    const int64_t ivecs = inner / (16 / es);
+    int64_t parts = 1;
+    if (outer * ((ivecs + 7) / 8) < 512 && axis >= 2048)
+        for (int64_t p = 2; p <= 64 && outer * ((ivecs + 7) / 8) * parts < 1024; ++p)
+            if (axis % p == 0 && axis / p >= 256) parts = p;
+    return parts;
+}
+
+size_t axhip_argreduce_workspace_bytes(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner) {
+    if (!valid_dtype(dtype) || outer <= 0 || axis <= 0 || inner <= 0) return 0;
+    const int64_t parts = argreduce_parts(src, dtype, outer, axis, inner);
+    return parts > 1 ? CallScratch::rounded(static_cast<size_t>(outer * parts * inner) * 8) : 0;
+}
+
 int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t want_min, int64_t *dst, void *stream) {
+    return axhip_argreduce_ws(src, dtype, outer, axis, inner, want_min, dst, nullptr, 0, stream);
+}
+
+int axhip_argreduce_ws(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t want_min, int64_t *dst, void *workspace,
+                       size_t workspace_bytes, void *stream) {
     AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_argreduce: bad dtype");
     AXHIP_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, AXHIP_ERR_INVALID_ARG, "axhip_argreduce: negative extent");
     if (outer == 0 || inner == 0) return AXHIP_OK;
@@ -885,16 +908,15 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
         const int64_t ivecs = inner / (16 / es);
         // Few results over a long axis: too few work-groups for the chip.  The axis is cut into `parts` equal segments
         // whose candidates (value, index) go to stream-ordered temporary memory and are merged by a second kernel.
-        int64_t parts = 1;
-        if (outer * ((ivecs + 7) / 8) < 512 && axis >= 2048)
-            for (int64_t p = 2; p <= 64 && outer * ((ivecs + 7) / 8) * parts < 1024; ++p)
-                if (axis % p == 0 && axis / p >= 256) parts = p;
+        const int64_t parts = argreduce_parts(src, dtype, outer, axis, inner);
         const int64_t v_outer = outer * parts, v_axis = axis / parts;
         float *part_v = nullptr;
         int32_t *part_i = nullptr;
+        CallScratch scratch(workspace, workspace_bytes, s);
         if (parts > 1) {
             void *tmp = nullptr;
-            AXHIP_CHECK_HIP(hipMallocAsync(&tmp, static_cast<size_t>(v_outer * inner) * 8, s));
+            rc = scratch.take(&tmp, static_cast<size_t>(v_outer * inner) * 8, "axhip_argreduce");
+            if (rc) return rc;
             part_v = static_cast<float *>(tmp);
             part_i = reinterpret_cast<int32_t *>(part_v + v_outer * inner);
         }
@@ -919,7 +941,8 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
             const unsigned mblocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
             if (want_min) hipLaunchKernelGGL(argreduce_merge_kernel<true>, dim3(mblocks), dim3(256), 0, s, part_v, part_i, outer, parts, v_axis, inner, start, dst);
             else hipLaunchKernelGGL(argreduce_merge_kernel<false>, dim3(mblocks), dim3(256), 0, s, part_v, part_i, outer, parts, v_axis, inner, start, dst);
-            AXHIP_CHECK_HIP(hipFreeAsync(part_v, s));
+            rc = scratch.release();
+            if (rc) return rc;
         }
     } else {
         const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
@@ -930,8 +953,31 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
     return AXHIP_OK;
 }
 
+// segments the axis is cut into when few results stand over a long axis (1: one pass, no temporary memory)
+static int64_t reduce_axis_parts(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner) {
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+    if (inner <= 1 || inner % (16 / es) != 0 || (reinterpret_cast<uintptr_t>(src) & 15u) != 0) return 1;
+    const int64_t groups8 = outer * ((inner / (16 / es) + 7) / 8);
+    int64_t parts = 1;
+    if (groups8 < 512 && axis >= 2048)
+        for (int64_t p = 2; p <= 64 && groups8 * parts < 1024; ++p)
+            if (axis % p == 0 && axis / p >= 256) parts = p;
+    return parts;
+}
+
+size_t axhip_reduce_axis_workspace_bytes(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner) {
+    if (!valid_dtype(dtype) || outer <= 0 || axis <= 0 || inner <= 0) return 0;
+    const int64_t parts = reduce_axis_parts(src, dtype, outer, axis, inner);
+    return parts > 1 ? CallScratch::rounded(static_cast<size_t>(outer * parts * inner) * 4) : 0;
+}
+
 int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t reduce, void *dst, int32_t dst_dtype,
                       void *stream) {
+    return axhip_reduce_axis_ws(src, dtype, outer, axis, inner, reduce, dst, dst_dtype, nullptr, 0, stream);
+}
+
+int axhip_reduce_axis_ws(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t reduce, void *dst, int32_t dst_dtype,
+                         void *workspace, size_t workspace_bytes, void *stream) {
     AXHIP_REQUIRE(valid_dtype(dtype) && valid_dtype(dst_dtype), AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: bad dtype");
     AXHIP_REQUIRE(reduce == AXHIP_RED_SUM || reduce == AXHIP_RED_MEAN || reduce == AXHIP_RED_MAX || reduce == AXHIP_RED_MIN, AXHIP_ERR_INVALID_ARG,
                   "axhip_reduce_axis: bad reduction %d", reduce);
@@ -955,21 +1001,16 @@ int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axi
     const bool vec = inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
     // Few results over a long axis (column sums of a tall matrix): too few work-groups for the chip.  The axis is cut
     // into `parts` equal segments, reduced to fp32 partials in stream-ordered temporary memory, and those reduced again.
-    if (vec) {
-        const int64_t groups8 = outer * ((inner / (16 / es) + 7) / 8);
-        int64_t parts = 1;
-        if (groups8 < 512 && axis >= 2048)
-            for (int64_t p = 2; p <= 64 && groups8 * parts < 1024; ++p)
-                if (axis % p == 0 && axis / p >= 256) parts = p;
-        if (parts > 1) {
-            void *tmp = nullptr;
-            AXHIP_CHECK_HIP(hipMallocAsync(&tmp, static_cast<size_t>(outer * parts * inner) * 4, s));
-            rc = launch_reduce_axis(src, dtype, outer * parts, axis / parts, inner, red, 1.0f, tmp, AXHIP_DTYPE_F32, s);
-            if (!rc) rc = launch_reduce_axis(tmp, AXHIP_DTYPE_F32, outer, parts, inner, red, scale, dst, dst_dtype, s);
-            const hipError_t freed = hipFreeAsync(tmp, s);
-            if (!rc) AXHIP_CHECK_HIP(freed);
-            return rc;
-        }
+    const int64_t parts = vec ? reduce_axis_parts(src, dtype, outer, axis, inner) : 1;
+    if (parts > 1) {
+        CallScratch scratch(workspace, workspace_bytes, s);
+        void *tmp = nullptr;
+        rc = scratch.take(&tmp, static_cast<size_t>(outer * parts * inner) * 4, "axhip_reduce_axis");
+        if (rc) return rc;
+        rc = launch_reduce_axis(src, dtype, outer * parts, axis / parts, inner, red, 1.0f, tmp, AXHIP_DTYPE_F32, s);
+        if (!rc) rc = launch_reduce_axis(tmp, AXHIP_DTYPE_F32, outer, parts, inner, red, scale, dst, dst_dtype, s);
+        const int freed = scratch.release();
+        return rc ? rc : freed;
     }
     return launch_reduce_axis(src, dtype, outer, axis, inner, red, scale, dst, dst_dtype, s);
 }

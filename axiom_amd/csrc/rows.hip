@@ -456,6 +456,7 @@ __global__ __launch_bounds__(THREADS) void elementwise_flat_kernel(const AxhipRo
 constexpr int FULL_RED_BLOCKS = 2048;      // blocks of the generic stage 1
 constexpr int FULL_RED_ROWS = 16384;       // rows of a flat array handed to a row-reduction kernel
 constexpr int FULL_RED_PARTIALS = FULL_RED_ROWS + 256; // capacity of the workspace, in floats (the rows plus the blocks of a remainder)
+static_assert(sizeof(scratch) / sizeof(float) >= FULL_RED_PARTIALS, "the file-scope scratch array holds every partial of a full reduction");
 
 template <int THREADS, int E>
 __global__ __launch_bounds__(THREADS) void full_reduce_stage1(const AxhipRowsProgram P, float *partials) {
@@ -887,6 +888,8 @@ int axhip_fused_rows_prepare(const AxhipRowsProgram *program) {
     }
     return AXHIP_OK;
 }
+
+void axhip_fused_rows_jit_counters(int *from_disk, int *compiled) { rows_prog_jit_counters(from_disk, compiled); }
 
 size_t axhip_full_reduce_workspace_bytes(void) { return FULL_RED_PARTIALS * sizeof(float); }
 

@@ -4,6 +4,11 @@
 
 #include <hip/hiprtc.h>
 
+#include <sys/stat.h>
+#include <sys/types.h>
+#include <unistd.h>
+
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
@@ -102,6 +107,9 @@ Entry *find_or_make_entry(const AxhipRowsProgram &P) {
     auto range = g_entries.equal_range(h);
     for (auto it = range.first; it != range.second; ++it)
         if (memcmp(&it->second->key, &k, sizeof(k)) == 0) return it->second.get();
+    // (one entry per row length and program structure: a loop over ever-changing row lengths must not grow this
+    // without bound; compiled kernels live in g_kernels and are found again by their configuration text)
+    if (g_entries.size() >= 4096) g_entries.clear();
     auto e = std::make_unique<Entry>();
     e->key = k;
     // Two candidate plans: the tightest fit for this row length, and the nearest of the shapes the build compiles.
@@ -129,16 +137,103 @@ Entry *find_or_make_entry(const AxhipRowsProgram &P) {
     return raw;
 }
 
-// compiles the program's kernel through hipRTC; on failure the reason goes to the library's error text
-std::shared_ptr<Kernel> compile(const RowsProgSpec &spec) {
+// ---- on-disk cache of run-time compiled kernels.  A code object is stored under the hash of everything it depends
+// on (generated source, compiler options, hipRTC version), so a new process loads it instead of compiling again
+// (0.5 s for the first compile of a process, 10-35 ms for later ones).  AXHIP_CACHE_DIR names the folder (default
+// $XDG_CACHE_HOME/axhip, else $HOME/.cache/axhip); AXHIP_DISK_CACHE=0 turns it off.
+const char *const kCompileOptions[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+constexpr int kNumCompileOptions = static_cast<int>(sizeof(kCompileOptions) / sizeof(kCompileOptions[0]));
+
+std::string cache_dir() {
+    const char *off = getenv("AXHIP_DISK_CACHE");
+    if (off && off[0] == '0') return "";
+    if (const char *d = getenv("AXHIP_CACHE_DIR")) return d[0] ? std::string(d) : "";
+    if (const char *x = getenv("XDG_CACHE_HOME")) if (x[0]) return std::string(x) + "/axhip";
+    if (const char *h = getenv("HOME")) if (h[0]) return std::string(h) + "/.cache/axhip";
+    return "";
+}
+
+bool make_dirs(const std::string &path) {
+    for (size_t i = 1; i <= path.size(); ++i)
+        if (i == path.size() || path[i] == '/') {
+            const std::string part = path.substr(0, i);
+            if (mkdir(part.c_str(), 0777) != 0 && errno != EEXIST) return false;
+        }
+    return true;
+}
+
+std::string cache_path(const RowsProgSpec &spec, const std::string &src) {
+    const std::string dir = cache_dir();
+    if (dir.empty()) return "";
+    int major = 0, minor = 0;
+    (void)hiprtcVersion(&major, &minor);
+    std::string what = src;
+    for (const char *o : kCompileOptions) what += std::string("\n") + o;
+    what += "\nhiprtc " + std::to_string(major) + "." + std::to_string(minor);
+    char name[32];
+    snprintf(name, sizeof(name), "%016llx", static_cast<unsigned long long>(hash_bytes(what.data(), what.size())));
+    return dir + "/" + spec.symbol + "_" + name + ".hsaco";
+}
+
+bool read_file(const std::string &path, std::vector<char> *out) {
+    FILE *f = fopen(path.c_str(), "rb");
+    if (!f) return false;
+    bool ok = fseek(f, 0, SEEK_END) == 0;
+    const long n = ok ? ftell(f) : -1;
+    ok = ok && n > 0 && fseek(f, 0, SEEK_SET) == 0;
+    if (ok) {
+        out->resize(static_cast<size_t>(n));
+        ok = fread(out->data(), 1, out->size(), f) == out->size();
+    }
+    fclose(f);
+    return ok;
+}
+
+void write_file_atomically(const std::string &path, const std::vector<char> &data) {
+    const size_t slash = path.rfind('/');
+    if (slash == std::string::npos || !make_dirs(path.substr(0, slash))) return;
+    const std::string tmp = path + ".tmp." + std::to_string(static_cast<long long>(getpid()));
+    FILE *f = fopen(tmp.c_str(), "wb");
+    if (!f) return;
+    const bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
+    if (fclose(f) != 0 || !ok || rename(tmp.c_str(), path.c_str()) != 0) (void)remove(tmp.c_str());
+}
+
+std::shared_ptr<Kernel> load_code(const std::vector<char> &code, const RowsProgSpec &spec, bool report) {
+    auto k = std::make_shared<Kernel>();
+    hipError_t e = hipModuleLoadData(&k->module, code.data());
+    if (e == hipSuccess) e = hipModuleGetFunction(&k->function, k->module, spec.symbol.c_str());
+    if (e != hipSuccess) {
+        if (report) set_last_error("fused rows: loading the compiled %s failed: %s", spec.label.c_str(), hipGetErrorString(e));
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return k;
+}
+
+int g_disk_hits = 0, g_compiles = 0; // (under g_mutex)
+
+// the program's kernel from the on-disk cache, else compiled through hipRTC (and stored); on failure the reason goes
+// to the library's error text.  Called WITHOUT g_mutex: other threads keep dispatching while this one compiles.
+std::shared_ptr<Kernel> compile(const RowsProgSpec &spec, bool *from_disk) {
+    *from_disk = false;
     const std::string src = rows_prog_source(spec, kRowsProgBody);
+    const std::string path = cache_path(spec, src);
+    if (!path.empty()) {
+        std::vector<char> code;
+        if (read_file(path, &code)) {
+            if (auto k = load_code(code, spec, false)) {
+                *from_disk = true;
+                return k;
+            } // (an unreadable or stale file is compiled again and replaced)
+        }
+    }
     hiprtcProgram prog = nullptr;
     if (hiprtcCreateProgram(&prog, src.c_str(), (spec.symbol + ".hip").c_str(), 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
         set_last_error("fused rows: hiprtcCreateProgram failed for %s", spec.label.c_str());
         return nullptr;
     }
-    const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    const hiprtcResult r = hiprtcCompileProgram(prog, static_cast<int>(sizeof(opts) / sizeof(opts[0])), opts);
+    const hiprtcResult r = hiprtcCompileProgram(prog, kNumCompileOptions, const_cast<const char **>(kCompileOptions));
     if (r != HIPRTC_SUCCESS) {
         size_t n = 0;
         hiprtcGetProgramLogSize(prog, &n);
@@ -153,14 +248,8 @@ std::shared_ptr<Kernel> compile(const RowsProgSpec &spec) {
     std::vector<char> code(size);
     hiprtcGetCode(prog, code.data());
     hiprtcDestroyProgram(&prog);
-    auto k = std::make_shared<Kernel>();
-    hipError_t e = hipModuleLoadData(&k->module, code.data());
-    if (e == hipSuccess) e = hipModuleGetFunction(&k->function, k->module, spec.symbol.c_str());
-    if (e != hipSuccess) {
-        set_last_error("fused rows: loading the compiled %s failed: %s", spec.label.c_str(), hipGetErrorString(e));
-        (void)hipGetLastError();
-        return nullptr;
-    }
+    auto k = load_code(code, spec, true);
+    if (k && !path.empty()) write_file_atomically(path, code);
     return k;
 }
 
@@ -180,8 +269,7 @@ bool rows_prog_compile_only(const AxhipRowsProgram &P, std::string *label, std::
         if (error) *error = "hiprtcCreateProgram failed";
         return false;
     }
-    const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    const hiprtcResult r = hiprtcCompileProgram(prog, static_cast<int>(sizeof(opts) / sizeof(opts[0])), opts);
+    const hiprtcResult r = hiprtcCompileProgram(prog, kNumCompileOptions, const_cast<const char **>(kCompileOptions));
     if (r != HIPRTC_SUCCESS && error) {
         size_t n = 0;
         hiprtcGetProgramLogSize(prog, &n);
@@ -199,7 +287,14 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
     std::shared_ptr<Kernel> kernel;
     RowsProgArgs args;
     int threads = 0, rows_per_block = 1;
-    {
+    // A kernel that has to be compiled is compiled with g_mutex released (hundreds of milliseconds during which
+    // other threads' dispatches go on); the loop then takes the lock again and publishes it.
+    std::shared_ptr<Kernel> compiled;
+    bool compile_done = false, compiled_from_disk = false;
+    RowsProgSpec to_compile;
+    for (;;) {
+        bool need_compile = false;
+        {
         std::lock_guard<std::mutex> lock(g_mutex);
         Entry *e = find_or_make_entry(P);
         if (!e->eligible) return false;
@@ -221,20 +316,26 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
                 if (e->is_builtin) {
                     k = std::make_shared<Kernel>();
                     k->builtin = rows_prog_find_builtin(key);
+                } else if (!compile_done) {
+                    need_compile = true;
+                    to_compile = e->spec;
                 } else {
-                    k = compile(e->spec);
-                    if (!k) {
+                    k = compiled;
+                    if (k) {
+                        ++(compiled_from_disk ? g_disk_hits : g_compiles);
+                    } else {
                         e->jit_failed = true;
                         if (!e->has_builtin_alternative) return false;
                         use_alt = true;
                     }
                 }
                 if (k) {
-                    g_kernels.emplace(key, k);
-                    e->kernel = k;
+                    g_kernels.emplace(key, k); // (another thread may have published the same kernel meanwhile: its copy stays)
+                    e->kernel = g_kernels.find(key)->second;
                 }
             }
         }
+        if (!need_compile) {
         if (use_alt && !e->alt_kernel) {
             e->alt_kernel = std::make_shared<Kernel>();
             e->alt_kernel->builtin = rows_prog_find_builtin(e->builtin_spec.config + e->builtin_spec.chains);
@@ -261,6 +362,11 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
         rows_prog_bind(P, spec, &args);
         threads = spec.threads;
         rows_per_block = spec.rows_per_block;
+        }
+        }
+        if (!need_compile) break;
+        compiled = compile(to_compile, &compiled_from_disk);
+        compile_done = true;
     }
     const int64_t row_groups = (P.rows + rows_per_block - 1) / rows_per_block;
     // As many blocks as fit on the device at once, then fewer, so that every block walks the same number of rows
@@ -276,6 +382,13 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
         if (rc) *rc = static_cast<int>(err);
     }
     return true;
+}
+
+// how many run-time kernels this process loaded from the on-disk cache / compiled (diagnostic)
+void rows_prog_jit_counters(int *from_disk, int *compiled) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (from_disk) *from_disk = g_disk_hits;
+    if (compiled) *compiled = g_compiles;
 }
 
 } // namespace axhip

@@ -18,4 +18,7 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
 // generator's text is valid for a program shape.
 bool rows_prog_compile_only(const AxhipRowsProgram &P, std::string *label, std::string *error);
 
+// how many run-time kernels this process took from the on-disk cache / compiled with hipRTC so far
+void rows_prog_jit_counters(int *from_disk, int *compiled);
+
 } // namespace axhip

@@ -1,6 +1,11 @@
 // Scaled-dot-product attention, forward, for gfx950.
 //
-// Three kernels:
+// The kernels:
+//   sdpa_mfma_pingpong_kernel   bf16 / f16, head_dim 128, no explicit mask,
+//                       problems that fill the chip: the pipelined kernel's
+//                       tiling with the two waves of a SIMD half a step apart
+//                       (one in its matrix phase, one in its softmax phase) and
+//                       persistent work-groups.
 //   sdpa_mfma_pipelined_kernel  bf16 / f16, head_dim 64 / 128.  FlashAttention-2
 //                       schedule on v_mfma_f32_32x32x16_{bf16,f16}: one
 //                       workgroup = 4 or 8 wave64, each wave owns 32 query
@@ -28,6 +33,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 namespace axhip {
 
@@ -870,6 +876,348 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sdpa_mfma_pipelined_
     }
 }
 
+// ------------------------------------------ ping-pong MFMA kernel, head_dim 128
+// The pipelined kernel above lets both waves of a SIMD run the same mix of matrix and vector instructions at the same
+// time: the older wave wins every arbitration, finishes its step early and the younger one trails behind it.  Here
+// the eight waves of a work-group form two groups (waves 0-3 and 4-7: one wave of each group per SIMD) that run HALF A
+// STEP APART.  Between two work-group barriers (one per 64-key tile)
+//     group 0 issues the 2 * (KT + 2 DT) MFMAs of a step back to back -- O^T += V^T P^T of tile j and S^T = K Q^T of
+//             tile j+1, alternating, fragments from LDS -- and then runs the softmax of tile j+1 on the VALU,
+//     group 1 runs the softmax of tile j first and the same MFMAs after it,
+// so a SIMD always has one wave in its matrix phase and one in its vector phase.  Measured against the pipelined
+// kernel, back to back on one box (bf16 B4 H32 S4096 D128): causal 981 -> 1060 TFLOP/s, non-causal 1111 -> 1188.
+// What else differs:
+//  * row sums are fp32 adds of the exponentials.  v_dot2c_f32_bf16 (the pipelined kernel's choice) waits for the
+//    matrix pipe: next to MFMAs every one of them costs about 18 cycles.
+//  * the score accumulators of a tile exist once (the softmax of tile j ends before the MFMAs of tile j+1 start in
+//    the same wave), which leaves registers for everything else without spills.
+//  * a work-group is persistent: it walks the units blockIdx.x, blockIdx.x + gridDim.x, ... and requests the first K
+//    and V tiles of the next segment (the second query block of a causal pair, or the next unit) during the last two
+//    steps of the one at hand, so a segment does not start with an empty pipeline.
+//  * the output is written as 16 bytes per lane after one exchange between the half-waves.
+// No explicit mask and exact head sizes only (the pipelined kernel keeps those cases).
+template <bool BF16, int D>
+__global__ __launch_bounds__(512, 1) void sdpa_mfma_pingpong_kernel(const SdpaArgs a) {
+    static_assert(D == 128, "tuned and tested for head_dim 128 (the index arithmetic also holds for 64)");
+    constexpr int NW = 8, PF = 3; // PF: LDS fragment reads run this many MFMAs ahead
+    constexpr int KT = D / 16, DT = D / 32, BMW = 32 * NW, ROWB = 2 * D, CHUNKS = ROWB / 16, RPL = 64 / CHUNKS;
+    constexpr int NLOAD = BN / (RPL * NW), TILEB = BN * ROWB;
+    constexpr int NM = D / 4; // MFMAs of a step: D / 8 for the scores of the next tile, D / 8 for the output of this one
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * TILEB]; // K0 K1 V0 V1
+
+    const int tid = threadIdx.x;
+    const int lane = tid % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int grp = wave >> 2;
+    const int ql = lane % 32, g = lane / 32;
+
+    const int BH = a.B * a.H;
+    const int nqb = (a.Sq + BMW - 1) / BMW;
+    const int per_bh = a.causal ? (nqb + 1) / 2 : nqb;
+    const int n_wg = per_bh * BH; // units of work: a (batch, head) and a query block (a pair of them under a causal mask)
+    const int krow_bytes = static_cast<int>(a.ks[2]) * 2, vrow_bytes = static_cast<int>(a.vs[2]) * 2;
+    // A work-group walks the units blockIdx.x, blockIdx.x + gridDim.x, ... (units are dealt to the 8 XCDs round-robin by
+    // id, and gridDim.x is a multiple of 8: one (batch, head) stays on one XCD); a unit is one or two segments (passes).
+    struct Segment { int bh, qb, ntiles; };
+    auto segment_of = [&](int L, int pass) {
+        int bh, slot;
+        if (BH % 8 == 0) {
+            const int xcd = L % 8, j = L / 8;
+            bh = (j / per_bh) * 8 + xcd;
+            slot = j % per_bh;
+        } else {
+            bh = L / per_bh;
+            slot = L % per_bh;
+        }
+        const int qb = a.causal ? (pass == 0 ? nqb - 1 - slot : slot) : slot;
+        int kv_end = a.Skv;
+        if (a.causal) kv_end = min(a.Skv, qb * BMW + BMW);
+        return Segment{bh, qb, (kv_end + BN - 1) / BN};
+    };
+    auto passes_of = [&](int L) {
+        const int slot = BH % 8 == 0 ? (L / 8) % per_bh : L % per_bh;
+        return (a.causal && slot != nqb - 1 - slot) ? 2 : 1;
+    };
+    auto k_rsrc_of = [&](int bh) { return make_rsrc(static_cast<const uint16_t *>(a.k) + (bh / a.H) * a.ks[0] + (bh % a.H) * a.ks[1], (a.Skv - 1) * krow_bytes + D * 2); };
+    auto v_rsrc_of = [&](int bh) { return make_rsrc(static_cast<const uint16_t *>(a.v) + (bh / a.H) * a.vs[0] + (bh % a.H) * a.vs[1], (a.Skv - 1) * vrow_bytes + D * 2); };
+
+    const int ld_r = RPL * wave + lane / CHUNKS;
+    const int k_chunk = (lane % CHUNKS) ^ swizzle_k<D>(ld_r), v_chunk = (lane % CHUNKS) ^ swizzle_v<D>(ld_r);
+    const int k_voff = ld_r * krow_bytes + k_chunk * 16;
+    const int v_voff = ld_r * vrow_bytes + v_chunk * 16;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + RPL * wave * ROWB);
+    auto load_k = [&](const int4_t &krsrc, int tile, int buf) {
+#pragma unroll
+        for (int n = 0; n < NLOAD; ++n)
+            load_to_lds_16(krsrc, lds_wave + buf * TILEB + n * RPL * NW * ROWB, k_voff + (tile * BN + RPL * NW * n) * krow_bytes);
+    };
+    auto load_v = [&](const int4_t &vrsrc, int tile, int buf) {
+#pragma unroll
+        for (int n = 0; n < NLOAD; ++n)
+            load_to_lds_16(vrsrc, lds_wave + (2 + buf) * TILEB + n * RPL * NW * ROWB, v_voff + (tile * BN + RPL * NW * n) * vrow_bytes);
+    };
+
+    int k_off[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) k_off[t] = ql * ROWB + (((2 * t + g) ^ swizzle_k<D>(ql)) * 16);
+    int v_off[2][DT];
+    {
+        const int s2 = (lane & 15) >> 2, cl = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1), half = lane & 1;
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int row = g * 4 + s2 + 8 * hi;
+                v_off[hi][dt] = row * ROWB + (((dt * 4 + cl) ^ swizzle_v<D>(row)) * 16) + half * 8;
+            }
+    }
+    uint32_t touch = 0; // destination of the load that pulls the next segment's query rows into L2
+    // work-group barrier without a memory fence of its own: tile loads are waited for explicitly, LDS fragment reads
+    // have been consumed by the MFMAs in front of it
+    auto bar = [] { asm volatile("s_barrier" ::: "memory"); };
+    auto wait_tiles = [&] { __builtin_amdgcn_s_waitcnt(0x0F70); asm volatile("" :: "v"(touch)); }; // vmcnt(0) (and the touch register stays reserved until here)
+
+    bool prefetched = false; // the first tiles of the segment at hand were requested during the previous one
+    for (int L = blockIdx.x; L < n_wg; L += gridDim.x) {
+    const int npass = passes_of(L);
+    for (int pass = 0; pass < npass; ++pass) {
+        const Segment seg = segment_of(L, pass);
+        const int b = seg.bh / a.H, h = seg.bh % a.H;
+        const uint16_t *Q = static_cast<const uint16_t *>(a.q) + b * a.qs[0] + h * a.qs[1];
+        uint16_t *O = static_cast<uint16_t *>(a.o) + b * a.os[0] + h * a.os[1];
+        const int4_t krsrc = k_rsrc_of(seg.bh), vrsrc = v_rsrc_of(seg.bh);
+        // the segment after this one: its first K and V tiles are requested in this segment's last two steps
+        const bool has_next = pass + 1 < npass || L + static_cast<int>(gridDim.x) < n_wg;
+        const Segment nxt = has_next ? (pass + 1 < npass ? segment_of(L, pass + 1) : segment_of(L + gridDim.x, 0)) : seg;
+        const int4_t krsrc_n = k_rsrc_of(nxt.bh), vrsrc_n = v_rsrc_of(nxt.bh);
+        const int qb = seg.qb;
+        const int q0 = qb * BMW;
+        const int qw0 = q0 + wave * 32;
+        const int q = qw0 + ql;
+        const bool q_ok = q < a.Sq;
+        const int ntiles = seg.ntiles; // >= 1
+        const bool pf_next = has_next && ntiles % 2 == 0; // (an even count keeps tile t of the next segment in buffer t & 1)
+
+        uint4_t qf[KT];
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            qf[t] = uint4_t{0, 0, 0, 0};
+            if (q_ok) qf[t] = *reinterpret_cast<const uint4_t *>(Q + static_cast<int64_t>(q) * a.qs[2] + 16 * t + 8 * g);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t w = qf[t][c];
+                const float lo = BF16 ? bf16_bits_to_f32(w & 0xFFFFu) : f16_bits_to_f32(w & 0xFFFFu);
+                const float hi = BF16 ? bf16_bits_to_f32(w >> 16) : f16_bits_to_f32(w >> 16);
+                qf[t][c] = pack2<BF16>(lo * a.scale_log2e, hi * a.scale_log2e);
+            }
+        }
+
+        float16_t oacc[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.0f;
+        float m_run = NEG_INF_F, l_run = 0.0f, l_run1 = 0.0f;
+
+        auto max3 = [](float x, float y, float z) { return __builtin_elementwise_maximum(__builtin_elementwise_maximum(x, y), z); };
+        auto max_across_halves = [&](float x) {
+            const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+            return __builtin_elementwise_maximum(__uint_as_float(r[0]), __uint_as_float(r[1]));
+        };
+        auto row_max = [&](const float16_t (&s)[2]) {
+            float m0 = max3(s[0][0], s[0][1], s[0][2]), m1 = max3(s[0][8], s[0][9], s[0][10]);
+            float m2 = max3(s[1][0], s[1][1], s[1][2]), m3 = max3(s[1][8], s[1][9], s[1][10]);
+            m0 = max3(m0, s[0][3], s[0][4]); m1 = max3(m1, s[0][11], s[0][12]);
+            m2 = max3(m2, s[1][3], s[1][4]); m3 = max3(m3, s[1][11], s[1][12]);
+            m0 = max3(m0, s[0][5], s[0][6]); m1 = max3(m1, s[0][13], s[0][14]);
+            m2 = max3(m2, s[1][5], s[1][6]); m3 = max3(m3, s[1][13], s[1][14]);
+            m0 = max3(m0, s[0][7], m1); m2 = max3(m2, s[1][7], m3);
+            return max_across_halves(max3(m0, s[0][15], __builtin_elementwise_maximum(m2, s[1][15])));
+        };
+        auto mask_and_max = [&](int kv0, float16_t (&s)[2]) {
+            const int kv_limit = a.causal ? min(a.Skv - 1, q) : a.Skv - 1;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int kv = kv0 + kt * 32 + (i / 4) * 8 + g * 4 + (i % 4);
+                    if (kv > kv_limit) s[kt][i] = NEG_INF_F;
+                }
+            return row_max(s);
+        };
+        auto update_max = [&](float mloc, float16_t (&cur)[2]) {
+            const float ref = m_run == NEG_INF_F ? 0.0f : m_run;
+            const float m_new = __builtin_elementwise_maximum(m_run, mloc + ref);
+            if (__builtin_amdgcn_ballot_w64(m_new - m_run > RESCALE_THRESHOLD) != 0) {
+                const float alpha = m_new == NEG_INF_F ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                const float ref_new = m_new == NEG_INF_F ? 0.0f : m_new;
+                const float delta = ref_new - ref;
+                m_run = m_new;
+                l_run *= alpha;
+                l_run1 *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) cur[kt][i] -= delta;
+            }
+        };
+
+        float16_t s[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+        uint32_t w[16];
+
+        // softmax of the tile in s (scores relative to the reference): masks, row maximum, rescale, P = 2^s packed to w
+        auto softmax_phase = [&](int j) {
+            const int kv0 = j * BN;
+            const bool need_mask = (a.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > a.Skv);
+            const float mloc = need_mask ? mask_and_max(kv0, s) : row_max(s);
+            update_max(mloc, s);
+#pragma unroll
+            for (int pr = 0; pr < 16; ++pr) {
+                const int kt = pr / 8, i = (pr % 8) * 2;
+                const float p0 = __builtin_amdgcn_exp2f(s[kt][i]);
+                const float p1 = __builtin_amdgcn_exp2f(s[kt][i + 1]);
+                w[pr] = pack2<BF16>(p0, p1);
+                l_run += p0; // (v_dot2c waits for the matrix pipe: 18 cycles each next to MFMAs)
+                l_run1 += p1;
+            }
+            // the next tile's scores start from minus the reference: its logits come out relative to it
+            const float m_use = m_run == NEG_INF_F ? 0.0f : m_run;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[kt][i] = -m_use;
+        };
+        // the NM MFMAs of a step: O^T += V^T P^T of tile j (P in w, V fragments from Vb) and S^T = K Q^T of tile j+1
+        // (K fragments from Kn) alternate, so consecutive MFMAs never share an accumulator
+        auto mfma_phase = [&](const unsigned char *Kn, const unsigned char *Vb) {
+            constexpr int RING = PF + 1;
+            uint4_t fr[RING];
+            // slot m: even -> score MFMA (m / 2): sub-tile kt = (m/2) & 1, k-step t = (m/2) >> 1; odd -> PV MFMA (m / 2): ks = idx / DT, dt = idx % DT
+            auto read_frag = [&](int m) {
+                const int idx = m / 2;
+                if (m % 2 == 0) {
+                    fr[m % RING] = *reinterpret_cast<const uint4_t *>(Kn + (idx & 1) * 32 * ROWB + k_off[idx >> 1]);
+                } else {
+                    const int ks = idx / DT, dt = idx % DT;
+                    const uint2_t lo = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[0][dt]));
+                    const uint2_t hi = lds_read_tr16(reinterpret_cast<const uint16_t *>(Vb + ks * 16 * ROWB + v_off[1][dt]));
+                    fr[m % RING] = uint4_t{lo.x, lo.y, hi.x, hi.y};
+                }
+            };
+#pragma unroll
+            for (int m = 0; m < PF; ++m) read_frag(m);
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                if (m + PF < NM) read_frag(m + PF);
+                const int idx = m / 2;
+                if (m % 2 == 0) {
+                    const int kt = idx & 1, t = idx >> 1;
+                    s[kt] = mfma_32x32x16<BF16>(fr[m % RING], qf[t], s[kt]);
+                } else {
+                    const int ks = idx / DT, dt = idx % DT;
+                    const uint4_t pf = {w[4 * ks], w[4 * ks + 1], w[4 * ks + 2], w[4 * ks + 3]};
+                    oacc[dt] = mfma_32x32x16<BF16>(fr[m % RING], pf, oacc[dt]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        // ---- prologue: K(0), V(0), K(1); every wave computes the scores of tile 0
+        if (!prefetched) {
+            load_k(krsrc, 0, 0);
+            load_v(vrsrc, 0, 0);
+            if (ntiles > 1) load_k(krsrc, 1, 1);
+        }
+        wait_tiles();
+        bar();
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int t = 0; t < KT; ++t) {
+                const uint4_t kf = *reinterpret_cast<const uint4_t *>(lds + kt * 32 * ROWB + k_off[t]);
+                s[kt] = mfma_32x32x16<BF16>(kf, qf[t], s[kt]);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): K buffer 0 is read
+
+        auto request = [&](int j, auto par) { // K(j+2) into the buffer of K(j), V(j+1) into the buffer of V(j-1)
+            constexpr int PAR = decltype(par)::value;
+            if (j + 2 < ntiles) load_k(krsrc, j + 2, PAR);
+            else if (pf_next && j + 2 - ntiles < nxt.ntiles) load_k(krsrc_n, j + 2 - ntiles, PAR);
+            if (j + 1 < ntiles) load_v(vrsrc, j + 1, 1 - PAR);
+            else if (pf_next) load_v(vrsrc_n, 0, 1 - PAR);
+        };
+        auto active_at = [&](int j) { return !(a.causal && j * BN > qw0 + 31); };
+        // One interval per tile, one barrier each: group 0 runs MFMAs(j+1) then softmax(j+1), group 1 softmax(j) then
+        // MFMAs(j+1) -- the two waves of a SIMD are always in opposite phases.  PAR = j & 1 picks the tile buffers.
+        auto interval0 = [&](int j, auto par) {
+            constexpr int PAR = decltype(par)::value;
+            wait_tiles();
+            bar();
+            request(j, par);
+            if (active_at(j)) mfma_phase(lds + (1 - PAR) * TILEB, lds + (2 + PAR) * TILEB);
+            if (j + 1 < ntiles && active_at(j + 1)) softmax_phase(j + 1);
+        };
+        auto interval1 = [&](int j, auto par) {
+            constexpr int PAR = decltype(par)::value;
+            wait_tiles();
+            bar();
+            request(j, par);
+            if (active_at(j)) {
+                softmax_phase(j);
+                mfma_phase(lds + (1 - PAR) * TILEB, lds + (2 + PAR) * TILEB);
+            }
+        };
+        if (grp == 0) {
+            softmax_phase(0);
+            for (int j = 0; j < ntiles; j += 2) {
+                interval0(j, std::integral_constant<int, 0>{});
+                if (j + 1 < ntiles) interval0(j + 1, std::integral_constant<int, 1>{});
+            }
+        } else {
+            for (int j = 0; j < ntiles; j += 2) {
+                interval1(j, std::integral_constant<int, 0>{});
+                if (j + 1 < ntiles) interval1(j + 1, std::integral_constant<int, 1>{});
+            }
+        }
+        if (!pf_next) bar(); // every wave is done with the tile buffers (nothing is written to them before the next segment's first barrier otherwise)
+        prefetched = pf_next;
+
+        l_run += l_run1;
+        const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        // A lane holds 4 consecutive dims per (dt, i4); the half-waves trade every second group so that each lane
+        // stores 8 consecutive dims (16 bytes): lanes 0-31 the even groups, lanes 32-63 the odd ones
+        {
+            uint16_t *orow = O + static_cast<int64_t>(q) * a.os[2];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int ip = 0; ip < 2; ++ip) {
+                    const int ia = 8 * ip, ib = 8 * ip + 4; // accumulator elements of groups i4 = 2 ip and 2 ip + 1
+                    const uint32_t x0 = pack2<BF16>(oacc[dt][ia] * inv, oacc[dt][ia + 1] * inv), x1 = pack2<BF16>(oacc[dt][ia + 2] * inv, oacc[dt][ia + 3] * inv);
+                    const uint32_t y0 = pack2<BF16>(oacc[dt][ib] * inv, oacc[dt][ib + 1] * inv), y1 = pack2<BF16>(oacc[dt][ib + 2] * inv, oacc[dt][ib + 3] * inv);
+                    // after the exchange lanes 0-31 hold (own group 2 ip, partner's group 2 ip), lanes 32-63 (partner's group 2 ip + 1, own group 2 ip + 1)
+                    const auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+                    const auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+                    const uint4_t wv = {r0[0], r1[0], r0[1], r1[1]};
+                    const int d = dt * 32 + (2 * ip + g) * 8;
+                    if (q_ok) *reinterpret_cast<uint4_t *>(orow + d) = wv;
+                }
+        }
+    }
+    }
+}
+
 // ------------------------------------------------------------- fp32 MFMA kernel
 // fp32 inputs, head_dim 32 / 64 / 128, on v_mfma_f32_32x32x2_f32: fp32 products and fp32 accumulation, so nothing
 // is given up against the FMA kernel below, at about ten times its rate.  Same transposed formulation as the 16-bit
@@ -1299,10 +1647,24 @@ __global__ __launch_bounds__(256) void sdpa_generic_kernel(const SdpaArgs a) {
     }
 }
 
+// every element of an output given through its (batch, head, row) strides: no key at all means every row is "fully masked"
+__global__ __launch_bounds__(256) void sdpa_zero_output_kernel(void *o, int dtype, int B, int H, int Sq, int D, int64_t sb, int64_t sh, int64_t ss) {
+    const int64_t total = static_cast<int64_t>(B) * H * Sq * D;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int d = static_cast<int>(i % D);
+        const int64_t r = i / D;
+        const int sq = static_cast<int>(r % Sq), h = static_cast<int>((r / Sq) % H), b = static_cast<int>(r / Sq / H);
+        store_any(o, dtype, b * sb + h * sh + sq * ss + d, 0.0f);
+    }
+}
+
 // ------------------------------------------------------------------ host side
 namespace {
 
 enum class SdpaKind { EMPTY, MFMA, MFMA_F32, GENERIC, INVALID };
+
+// which schedule the calling thread's last axhip_sdpa_fwd launched (diagnostic, for tests and A/B timing)
+thread_local const char *last_schedule = "none";
 
 // 0 = automatic; 4 / 8 forces the work-group width of the head_dim-128 kernel (AXHIP_SDPA_D128_WAVES)
 int sdpa_d128_waves = [] {
@@ -1332,6 +1694,12 @@ bool sdpa_f32_mfma = [] {
 int sdpa_f32_split = [] {
     const char *e = getenv("AXHIP_SDPA_F32_SPLIT");
     return e ? atoi(e) : 0;
+}();
+
+// AXHIP_SDPA_PINGPONG=0: unmasked head_dim-128 problems that fill the chip on the in-phase pipelined kernel (for A/B timing)
+bool sdpa_pingpong = [] {
+    const char *e = getenv("AXHIP_SDPA_PINGPONG");
+    return !(e && e[0] == '0');
 }();
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1376,6 +1744,26 @@ int validate(const AxhipSdpaParams &p) {
                       "axhip_sdpa_fwd: negative stride");
     AXHIP_REQUIRE(p.mask_strides[0] >= 0 && p.mask_strides[1] >= 0, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: negative mask stride");
     return AXHIP_OK;
+}
+
+// A decoding step -- one block of query rows, few (batch, head) slices, a long unmasked key sequence -- splits its keys
+// between work-groups; the partial results need temporary memory.  Returns the number of key chunks (0: no split).
+// (from 8 M key elements on: below that the second kernel and the temporary memory cost more than they gain --
+// 20 heads of 1500 keys of 64: 12.5 us unsplit, 21.6 split; 32 heads of 4096 keys of 128: 78.7 -> 27.2 us)
+struct DecodeSplit { int ksplit, kchunk, DD; size_t bytes; };
+DecodeSplit decode_split_plan(const AxhipSdpaParams &p, bool has_mask) {
+    DecodeSplit d{0, 0, 0, 0};
+    const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
+    const int64_t slices = static_cast<int64_t>(p.batch) * p.heads;
+    if (!half || has_mask || p.is_causal || p.seq_q <= 0 || p.seq_q > BM || slices <= 0 || slices > 96 || p.seq_kv < 1024 || p.head_dim <= 32 ||
+        p.head_dim > 128 || p.head_dim % 8 != 0 || slices * p.seq_kv * p.head_dim < (int64_t(8) << 20) || !sdpa_decode_split)
+        return d;
+    d.DD = p.head_dim <= 64 ? 64 : 128;
+    const int parts = static_cast<int>(std::min<int64_t>(std::min<int64_t>(64, (512 + slices - 1) / slices), p.seq_kv / 256));
+    d.kchunk = ((p.seq_kv + parts - 1) / parts + BN - 1) / BN * BN;
+    d.ksplit = (p.seq_kv + d.kchunk - 1) / d.kchunk;
+    d.bytes = static_cast<size_t>(slices) * d.ksplit * p.seq_q * (d.DD + 1) * sizeof(float);
+    return d;
 }
 
 template <bool BF16, int D> int launch_mfma(const SdpaArgs &a, hipStream_t s) {
@@ -1429,6 +1817,8 @@ int axhip_sdpa_d128_occupancy(int waves) {
     return e == hipSuccess ? n : -static_cast<int>(e);
 }
 
+const char *axhip_sdpa_last_schedule(void) { return last_schedule; }
+
 const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *p) {
     static thread_local char name[48];
     if (!p) return "invalid";
@@ -1445,23 +1835,36 @@ const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *p) {
     }
 }
 
+size_t axhip_sdpa_workspace_bytes(const AxhipSdpaParams *params, int has_mask) {
+    if (!params || validate(*params) != AXHIP_OK) return 0;
+    if (pick_kernel(*params, nullptr, nullptr, nullptr, nullptr) != SdpaKind::MFMA) return 0;
+    return CallScratch::rounded(decode_split_plan(*params, has_mask != 0).bytes);
+}
+
 int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const uint8_t *mask,
                    const AxhipSdpaParams *params, void *stream) {
+    return axhip_sdpa_fwd_ws(q, k, v, o, mask, params, nullptr, 0, stream);
+}
+
+int axhip_sdpa_fwd_ws(const void *q, const void *k, const void *v, void *o, const uint8_t *mask,
+                      const AxhipSdpaParams *params, void *workspace, size_t workspace_bytes, void *stream) {
     AXHIP_REQUIRE(params != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: params is NULL");
     const AxhipSdpaParams &p = *params;
     int rc = validate(p);
     if (rc) return rc;
     const SdpaKind kind = pick_kernel(p, q, k, v, o);
+    last_schedule = "empty";
     if (kind == SdpaKind::EMPTY) return AXHIP_OK;
     if (p.seq_kv == 0) { // no key at all: every row is "fully masked" -> zeros
         AXHIP_REQUIRE(o != nullptr, AXHIP_ERR_INVALID_ARG, "axhip_sdpa_fwd: NULL tensor");
-        for (int b = 0; b < p.batch; ++b)
-            for (int h = 0; h < p.heads; ++h)
-                for (int sq = 0; sq < p.seq_q; ++sq) {
-                    char *row = static_cast<char *>(o) + (b * p.o_strides[0] + h * p.o_strides[1] + sq * p.o_strides[2]) * dtype_size(p.dtype);
-                    int rc0 = axhip_fill(row, p.dtype, 0.0, p.head_dim, stream);
-                    if (rc0) return rc0;
-                }
+        // one launch: the output viewed as (batch, head, row, dim) through its strides
+        rc = ensure_init();
+        if (rc) return rc;
+        const int64_t total = static_cast<int64_t>(p.batch) * p.heads * p.seq_q * p.head_dim;
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((total + 255) / 256, 256 * 32));
+        hipLaunchKernelGGL(sdpa_zero_output_kernel, dim3(blocks), dim3(256), 0, resolve_stream(stream), o, p.dtype, p.batch, p.heads, p.seq_q, p.head_dim,
+                           p.o_strides[0], p.o_strides[1], p.o_strides[2]);
+        AXHIP_CHECK_HIP(hipGetLastError());
         return AXHIP_OK;
     }
     AXHIP_REQUIRE(kind != SdpaKind::INVALID, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: head_dim %d > %d is not supported", p.head_dim, GMAXD);
@@ -1490,17 +1893,17 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         // chip a work-group per slice: the keys are split between work-groups instead (flash decoding), partial
         // results in stream-ordered temporary memory, merged by a second kernel.
         const int64_t slices = static_cast<int64_t>(p.batch) * p.heads;
-        // (from 8 M key elements on: below that the second kernel and the temporary memory cost more than they gain --
-        // 20 heads of 1500 keys of 64: 12.5 us unsplit, 21.6 split; 32 heads of 4096 keys of 128: 78.7 -> 27.2 us)
-        if (!mask && !a.causal && p.seq_q <= BM && slices <= 96 && p.seq_kv >= 1024 && p.head_dim > 32 && p.head_dim <= 128 &&
-            slices * p.seq_kv * p.head_dim >= (int64_t(8) << 20) && sdpa_decode_split) {
-            const int DD = p.head_dim <= 64 ? 64 : 128;
-            int parts = static_cast<int>(std::min<int64_t>(std::min<int64_t>(64, (512 + slices - 1) / slices), p.seq_kv / 256));
-            a.kchunk = ((p.seq_kv + parts - 1) / parts + BN - 1) / BN * BN;
-            a.ksplit = (p.seq_kv + a.kchunk - 1) / a.kchunk;
+        const DecodeSplit ds = decode_split_plan(p, mask != nullptr);
+        if (ds.ksplit > 0) {
+            last_schedule = "decode_split";
+            const int DD = ds.DD;
+            a.kchunk = ds.kchunk;
+            a.ksplit = ds.ksplit;
             const size_t rows = static_cast<size_t>(slices) * a.ksplit * p.seq_q;
+            CallScratch scratch(workspace, workspace_bytes, s);
             void *tmp = nullptr;
-            AXHIP_CHECK_HIP(hipMallocAsync(&tmp, rows * (DD + 1) * sizeof(float), s));
+            rc = scratch.take(&tmp, ds.bytes, "axhip_sdpa");
+            if (rc) return rc;
             a.opart = static_cast<float *>(tmp);
             a.lse = a.opart + rows * DD;
             a.nqb = 1;
@@ -1514,7 +1917,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
                     return hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_mfma_kernel<true, 128, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
                            hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_mfma_kernel<false, 128, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
                 }();
-                AXHIP_REQUIRE(configured, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: cannot reserve %zu bytes of LDS", lds);
+                AXHIP_REQUIRE(configured, AXHIP_ERR_UNSUPPORTED, "axhip_sdpa_fwd: cannot reserve %zu bytes of LDS", lds); // (scratch returns its memory on the way out)
                 if (bf) hipLaunchKernelGGL((sdpa_mfma_kernel<true, 128, false, true>), dim3(grid), dim3(256), lds, s, a);
                 else hipLaunchKernelGGL((sdpa_mfma_kernel<false, 128, false, true>), dim3(grid), dim3(256), lds, s, a);
             }
@@ -1522,10 +1925,12 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             const unsigned mgrid = static_cast<unsigned>(std::min<int64_t>((items + 255) / 256, 4096));
             if (bf) hipLaunchKernelGGL(sdpa_splitk_merge_kernel<true>, dim3(mgrid), dim3(256), 0, s, a, DD);
             else hipLaunchKernelGGL(sdpa_splitk_merge_kernel<false>, dim3(mgrid), dim3(256), 0, s, a, DD);
-            AXHIP_CHECK_HIP(hipFreeAsync(tmp, s));
+            rc = scratch.release();
+            if (rc) return rc;
             AXHIP_CHECK_HIP(hipGetLastError());
             return AXHIP_OK;
         }
+        last_schedule = "register_staged";
         switch (p.head_dim <= 32 ? 32 : p.head_dim > 128 ? 256 : 64) {
         case 32: rc = bf ? launch_mfma<true, 32>(a, s) : launch_mfma<false, 32>(a, s); break;
         case 256: rc = bf ? launch_mfma<true, 256>(a, s) : launch_mfma<false, 256>(a, s); break;
@@ -1541,6 +1946,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             // split changes nothing -- a SIMD issues the same instructions as one wave or as two.
             const int64_t g4 = static_cast<int64_t>((p.seq_q + 127) / 128) * a.B * a.H;
             if (p.head_dim > 32 && p.head_dim <= 64 && !mask && !a.causal && p.seq_kv > BN && g4 <= 128 && sdpa_key_split) {
+                last_schedule = "key_split";
                 const unsigned gs = static_cast<unsigned>((p.seq_q + 63) / 64) * static_cast<unsigned>(a.B * a.H);
                 if (p.head_dim == 64) {
                     if (bf) hipLaunchKernelGGL((sdpa_mfma_pipelined_kernel<true, false, 4, 64, 2>), dim3(gs), dim3(256), 0, s, a);
@@ -1571,7 +1977,16 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         else if (mask) AXHIP_LAUNCH_DX(false, true, DD);                                                                  \
         else AXHIP_LAUNCH_DX(false, false, DD);                                                                           \
     } while (0)
-            if (p.head_dim <= 64) AXHIP_LAUNCH_D(64);
+            last_schedule = wide ? "pipelined8" : "pipelined4";
+            if (p.head_dim == 128 && !mask && wide && sdpa_pingpong) {
+                last_schedule = "pingpong";
+                // persistent work-groups, one per CU (a multiple of 8: a (batch, head) keeps its XCD)
+                // (head_dim 64 stays on the pipelined kernel: with twice the softmax work per MFMA the two phases are
+                // too uneven -- measured 846 against 867 TFLOP/s on bf16 B4 H32 S4096 causal)
+                const unsigned gp = std::min<unsigned>(g, 256);
+                if (bf) hipLaunchKernelGGL((sdpa_mfma_pingpong_kernel<true, 128>), dim3(gp), dim3(512), 0, s, a);
+                else hipLaunchKernelGGL((sdpa_mfma_pingpong_kernel<false, 128>), dim3(gp), dim3(512), 0, s, a);
+            } else if (p.head_dim <= 64) AXHIP_LAUNCH_D(64);
             else AXHIP_LAUNCH_D(128);
 #undef AXHIP_LAUNCH_D
 #undef AXHIP_LAUNCH_DX
@@ -1579,6 +1994,7 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
             break;
         }
     } else if (kind == SdpaKind::MFMA_F32) {
+        last_schedule = "mfma_f32";
         // waves per 32-row query block, by how many such blocks there are for the 1024 SIMDs (thresholds from timings
         // of 128 .. 1024 blocks: below 0.75 blocks per SIMD the four-way split wins by up to 2.7x, above 1.5 none is needed)
         const int64_t blocks32 = static_cast<int64_t>((p.seq_q + 31) / 32) * p.batch * p.heads;
@@ -1590,13 +2006,13 @@ int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o, const u
         rc = p.head_dim <= 32 ? launch_mfma_f32_d<32>(a, split, s) : p.head_dim <= 64 ? launch_mfma_f32_d<64>(a, split, s) : launch_mfma_f32_d<128>(a, split, s);
         if (rc) return rc;
     } else {
+        last_schedule = "generic";
         a.nqb = (p.seq_q + GM - 1) / GM;
         const size_t lds = sizeof(float) * (static_cast<size_t>(GM) * a.D + static_cast<size_t>(GN) * (a.D + 1) + static_cast<size_t>(GN) * a.D + GM * GN);
-        static bool attr_set = false;
-        if (!attr_set) {
-            AXHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_generic_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-            attr_set = true;
-        }
+        static std::once_flag attr_once;
+        static hipError_t attr = hipSuccess;
+        std::call_once(attr_once, [] { attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_generic_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); });
+        AXHIP_CHECK_HIP(attr);
         hipLaunchKernelGGL(sdpa_generic_kernel, dim3(a.nqb, a.B * a.H), dim3(256), lds, s, a);
     }
     AXHIP_CHECK_HIP(hipGetLastError());

@@ -932,7 +932,10 @@ void materialize_gpu_graph(GraphNode *root) {
             p.bias = st.gemm.bias >= 0 ? ptr_of(st.gemm.bias) : nullptr;
             p.residual = st.gemm.residual >= 0 ? ptr_of(st.gemm.residual) : nullptr;
             if (record) tl_last_kernels.emplace_back("gemm");
-            AXHIP_CALL(axhip_gemm(ptr_of(st.gemm.a), ptr_of(st.gemm.b), ptr_of(st.gemm.c), &p, nullptr));
+            // (operands the library repacks go through a block of this layer's cache; steady-state graphs allocate nothing)
+            const size_t ws_bytes = axhip_gemm_workspace_bytes(&p);
+            const std::unique_ptr<Storage> ws = ws_bytes ? make_storage(ws_bytes, Device::GPU) : nullptr;
+            AXHIP_CALL(axhip_gemm_ws(ptr_of(st.gemm.a), ptr_of(st.gemm.b), ptr_of(st.gemm.c), &p, ws ? ws->raw() : nullptr, ws_bytes, nullptr));
         } else if (st.kind == Step::PAD) {
             const ValueSpec &src = plan->values[st.pad.src];
             const int64_t isz = static_cast<int64_t>(dtype_size(src.dtype));
@@ -952,8 +955,10 @@ void materialize_gpu_graph(GraphNode *root) {
         } else if (st.kind == Step::AXIS_REDUCE) {
             const ValueSpec &src = plan->values[st.axred.src], &dst = plan->values[st.axred.dst];
             if (record) tl_last_kernels.emplace_back("reduce_axis");
-            AXHIP_CALL(axhip_reduce_axis(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
-                                         ptr_of(st.axred.dst), detail::to_axhip_dtype(dst.dtype), nullptr));
+            const size_t ws_bytes = axhip_reduce_axis_workspace_bytes(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner);
+            const std::unique_ptr<Storage> ws = ws_bytes ? make_storage(ws_bytes, Device::GPU) : nullptr;
+            AXHIP_CALL(axhip_reduce_axis_ws(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
+                                            ptr_of(st.axred.dst), detail::to_axhip_dtype(dst.dtype), ws ? ws->raw() : nullptr, ws_bytes, nullptr));
         } else if (st.kind == Step::AXIS_SOFTMAX) {
             const ValueSpec &src = plan->values[st.axred.src];
             if (record) tl_last_kernels.emplace_back("softmax_axis");

@@ -136,9 +136,13 @@ Tensor arg_reduce(const Tensor &x, int axis, bool keep_dims, bool want_min) {
     }
     if (sh[axis] == 0) throw ShapeError("argmax / argmin along an empty axis");
     Tensor out(out_shape, DType::Int64, Device::GPU);
-    AXHIP_CALL(axhip_argreduce(static_cast<const char *>(src.storage()->raw()) + src.offset(), ::axiom::detail::to_axhip_dtype(src.dtype()),
-                               static_cast<int64_t>(outer), static_cast<int64_t>(sh[axis]), static_cast<int64_t>(inner), want_min ? 1 : 0,
-                               static_cast<int64_t *>(out.storage()->raw()), nullptr));
+    // temporary memory (few results over a long axis) comes from this layer's block cache, not from the library
+    const char *src_ptr = static_cast<const char *>(src.storage()->raw()) + src.offset();
+    const int32_t dt = ::axiom::detail::to_axhip_dtype(src.dtype());
+    const size_t ws_bytes = axhip_argreduce_workspace_bytes(src_ptr, dt, static_cast<int64_t>(outer), static_cast<int64_t>(sh[axis]), static_cast<int64_t>(inner));
+    const std::unique_ptr<Storage> ws = ws_bytes ? make_storage(ws_bytes, Device::GPU) : nullptr;
+    AXHIP_CALL(axhip_argreduce_ws(src_ptr, dt, static_cast<int64_t>(outer), static_cast<int64_t>(sh[axis]), static_cast<int64_t>(inner), want_min ? 1 : 0,
+                                  static_cast<int64_t *>(out.storage()->raw()), ws ? ws->raw() : nullptr, ws_bytes, nullptr));
     return out; // asynchronous; .cpu() / item() synchronise
 }
 } // namespace
@@ -346,7 +350,11 @@ Tensor detail::sdpa(const Tensor &query, const Tensor &key, const Tensor &value,
         if (!out_bshd) return o;
         return o.transpose({0, 2, 1, 3}).ascontiguousarray().transpose({0, 2, 1, 3});
     }
-    AXHIP_CALL(axhip_sdpa_fwd(ptr(q), ptr(k), ptr(v), out.storage()->raw(), mask_ptr, &p, nullptr));
+    // (a decoding step's partial results live in a block of this layer's cache: the block goes back when this
+    // function returns and is handed out again in stream order)
+    const size_t ws_bytes = axhip_sdpa_workspace_bytes(&p, mask_ptr != nullptr);
+    const std::unique_ptr<Storage> ws = ws_bytes ? make_storage(ws_bytes, Device::GPU) : nullptr;
+    AXHIP_CALL(axhip_sdpa_fwd_ws(ptr(q), ptr(k), ptr(v), out.storage()->raw(), mask_ptr, &p, ws ? ws->raw() : nullptr, ws_bytes, nullptr));
     return out; // asynchronous; .cpu() / item() synchronise
 }
 

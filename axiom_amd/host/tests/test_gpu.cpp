@@ -291,9 +291,9 @@ GPU_TEST(FusedRows, OddRowLengthsRunOnTheRaggedKernels) {
     const float *x = a.typed_data<float>();
     auto sm = host_floats(ops::softmax(a.gpu() * 0.5f, -1));
     ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
-    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_static_muls_softmax_f32_g64_it6_grid"));
+    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_jit_muls_softmax_f32_g64_it6_grid"));
     auto ln = host_floats(ops::layer_norm(a.gpu(), Tensor(), Tensor(), -1, 1e-5f));
-    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_static_layernorm_f32_g64_it6_grid"));
+    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("rows_jit_layernorm_f32_g64_it6_grid"));
     for (size_t i = 0; i < R; ++i) {
         double mx = -1e300, s = 0, mean = 0, var = 0;
         for (size_t j = 0; j < C; ++j) mx = std::max(mx, 0.5 * x[i * C + j]);

@@ -8,7 +8,16 @@
  *     hipError_t, a negative value is one of AXHIP_ERR_*.  A human-readable
  *     message for the calling thread's last failure is at axhip_last_error().
  *   - the caller owns every buffer; kernels never allocate.  Pointers are
- *     device pointers unless a parameter says "host".
+ *     device pointers unless a parameter says "host".  Four entry points need
+ *     temporary device memory for some argument values (axhip_sdpa_fwd,
+ *     axhip_gemm, axhip_argreduce, axhip_reduce_axis: each says when).  Their
+ *     *_ws forms take it from the caller -- `workspace` of at least
+ *     *_workspace_bytes(...) bytes, 256-byte aligned -- and allocate nothing;
+ *     the plain forms (and a *_ws call with workspace == NULL) take it from the
+ *     stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`), a
+ *     convenience that graph capture and no-allocation harnesses must avoid.
+ *     A workspace that is too small fails with AXHIP_ERR_WORKSPACE before
+ *     anything is launched.
  *   - `stream` is a hipStream_t passed as void* (NULL = the backend's own
  *     stream, created by axhip_init and shared process-wide).
  *   - no exception crosses this boundary.
@@ -97,10 +106,24 @@ typedef struct {
 
 int axhip_sdpa_fwd(const void *q, const void *k, const void *v, void *o,
                    const uint8_t *mask, const AxhipSdpaParams *params_host, void *stream);
+/* The same with the temporary memory of a decoding step handed in by the
+ * caller (the role of the reference's caller-owned command buffers,
+ * src/backends/metal/metal_common.hpp:53-123: the backend allocates nothing
+ * behind the caller's back).  axhip_sdpa_workspace_bytes answers 0 for every
+ * problem that needs none; has_mask: whether a mask will be passed. */
+size_t axhip_sdpa_workspace_bytes(const AxhipSdpaParams *params_host, int has_mask);
+int axhip_sdpa_fwd_ws(const void *q, const void *k, const void *v, void *o,
+                      const uint8_t *mask, const AxhipSdpaParams *params_host,
+                      void *workspace, size_t workspace_bytes, void *stream);
 /* name of the kernel axhip_sdpa_fwd would launch for these parameters
  * ("mfma_bf16_d128", "generic", ...); the pointer stays valid for the life of
  * the process. */
 const char *axhip_sdpa_kernel_name(const AxhipSdpaParams *params_host);
+/* diagnostic: the schedule the calling thread's last axhip_sdpa_fwd launched ("pingpong", "pipelined8",
+ * "pipelined4", "key_split", "decode_split", "register_staged", "mfma_f32", "generic", "empty"); several
+ * schedules share one kernel name.  AXHIP_SDPA_PINGPONG=0 in the environment (read when the library loads)
+ * sends "pingpong" problems to "pipelined8". */
+const char *axhip_sdpa_last_schedule(void);
 
 /* ------------------------------------------------------------ fused chains
  * Stands behind graph::materialize_gpu_graph (called from
@@ -211,6 +234,10 @@ const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *program_host);
  * a compile error instead of leaving it to the first launch, which would fall back to the
  * interpreter.  Pointers in the program are only looked at for their alignment. */
 int axhip_fused_rows_prepare(const AxhipRowsProgram *program_host);
+/* diagnostic: how many "rows_jit_" kernels this process has so far loaded from the on-disk cache of
+ * compiled code objects (AXHIP_CACHE_DIR, default $XDG_CACHE_HOME/axhip or $HOME/.cache/axhip; AXHIP_DISK_CACHE=0
+ * turns it off) and how many it compiled with hipRTC.  Either pointer may be NULL. */
+void axhip_fused_rows_jit_counters(int *from_disk, int *compiled);
 
 /* Elementwise chain followed by a reduction over ALL elements -> one value
  * (the FusedReductionStep of include/axiom/graph/compiled_graph.hpp:41-70,
@@ -289,6 +316,11 @@ int axhip_gather_rows(const void *table, int32_t dtype, int64_t table_rows, int6
  * memory (hipMallocAsync on `stream`). */
 int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
                     int32_t want_min, int64_t *dst, void *stream);
+/* The same with that temporary memory handed in by the caller (0 bytes for
+ * every shape that needs none; `src` only matters for its 16-byte alignment). */
+size_t axhip_argreduce_workspace_bytes(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner);
+int axhip_argreduce_ws(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
+                       int32_t want_min, int64_t *dst, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Sum / mean / max / min (AXHIP_RED_*) along the middle extent of a contiguous
  * (outer, axis, inner) view -> outer * inner values of dst_dtype: Reduction
@@ -300,6 +332,11 @@ int axhip_argreduce(const void *src, int32_t dtype, int64_t outer, int64_t axis,
  * partials in stream-ordered temporary memory (hipMallocAsync on `stream`). */
 int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
                       int32_t reduce, void *dst, int32_t dst_dtype, void *stream);
+/* The same with the fp32 partials in memory handed in by the caller (0 bytes
+ * for every shape that needs none; `src` only matters for its alignment). */
+size_t axhip_reduce_axis_workspace_bytes(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner);
+int axhip_reduce_axis_ws(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner,
+                         int32_t reduce, void *dst, int32_t dst_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
 /* softmax (is_log = 0) / log-softmax along the middle extent of a contiguous
  * (outer, axis, inner) view, dst of the same shape and dtype: Softmax /
@@ -336,6 +373,11 @@ typedef struct {
 } AxhipGemmParams;
 
 int axhip_gemm(const void *a, const void *b, void *c, const AxhipGemmParams *params_host, void *stream);
+/* The same with the repacked operands in memory handed in by the caller (0
+ * bytes for every product that is not repacked). */
+size_t axhip_gemm_workspace_bytes(const AxhipGemmParams *params_host);
+int axhip_gemm_ws(const void *a, const void *b, void *c, const AxhipGemmParams *params_host,
+                  void *workspace, size_t workspace_bytes, void *stream);
 
 /* sizeof() of the parameter structs as this library was compiled, so that a
  * foreign-language binding can verify its own struct layout at load time:

@@ -68,7 +68,8 @@ def test_known_patterns_map_to_built_in_kernels():
     assert Prog(8192, 8192, F32).op("relu").op("add", imm=1.0).op("mul", "full").row("softmax").reduce("sum").name() == \
         "rows_static_relu_adds_mulf_softmax_sum_f32_g256_it8"
     assert Prog(30000, 1500, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it3_grid"  # 1500 * 2 bytes: rows not 16-byte aligned
-    assert Prog(64, 1024, F16).op("add", "full").row("layernorm", 2).name() == "rows_static_addf_layernorm_wb_f16_g64_it2"
+    assert Prog(64, 1024, BF16).op("add", "full").row("layernorm", 2).name() == "rows_static_addf_layernorm_wb_bf16_g64_it2"
+    assert Prog(64, 1024, F16).op("add", "full").row("layernorm", 2).name() == "rows_jit_addf_layernorm_wb_f16_g64_it2"  # f16 shapes are compiled on first use
 
 
 def test_other_shapes_are_compiled_at_run_time_and_named_after_their_chain():
@@ -121,12 +122,12 @@ def test_ragged_rows_take_the_grid_form_when_every_stream_is_full_size_and_equal
     the row's start ("_ragged": every access unaligned)."""
     assert Prog(4096, 4099, BF16).row("softmax").name() == "rows_jit_softmax_bf16_g64_it9_grid"
     assert Prog(4096, 4099, BF16, misalign=6).row("softmax").name() == "rows_jit_softmax_bf16_g64_it9_grid"  # input and output shifted alike
-    assert Prog(4096, 1500, F16).op("add", "full").row("softmax").name() == "rows_static_addf_softmax_f16_g64_it3_grid"
+    assert Prog(4096, 1500, BF16).op("add", "full").row("softmax").name() == "rows_jit_addf_softmax_bf16_g64_it3_grid"  # (built in for the main plans only: 1, 2, 4, 8 chunks per lane)
     assert Prog(4096, 4099, BF16, out_dt=F32).op("square").reduce("sum").name() == "rows_jit_square_reduce_sum_bf16_g64_it9_grid"  # [rows] results: any alignment
     # a per-column operand: its position in the row does not follow the grid
     assert Prog(4096, 1500, BF16).row("layernorm", 2).name() == "rows_static_layernorm_wb_bf16_g64_it3_ragged"
     assert Prog(4096, 1500, BF16).op("mul", "rowvec").row("softmax").name().endswith("_it3_ragged")
-    assert Prog(4096, 1500, BF16).row("layernorm").name() == "rows_static_layernorm_bf16_g64_it3_grid"  # no weight, no bias
+    assert Prog(4096, 1500, BF16).row("layernorm").name() == "rows_jit_layernorm_bf16_g64_it3_grid"  # no weight, no bias
     assert Prog(4096, 4099, F32).row("layernorm", 2).name() == "rows_jit_layernorm_wb_f32_g256_it5_ragged"
     # ... but for 1024-thread rows, whose unaligned form would spill
     assert Prog(64, 50257, F32).row("layernorm", 2).name() == "rows_jit_layernorm_wb_f32_g1024_it13_grid"
@@ -148,16 +149,16 @@ def test_short_aligned_rows_share_a_wavefront():
     a wavefront; built in like the longer plans.  Odd lengths keep a wavefront per row."""
     assert Prog(1 << 20, 64, BF16).row("softmax").name() == "rows_static_softmax_bf16_g8_it1"
     assert Prog(1 << 20, 16, BF16).row("rmsnorm", 1).name() == "rows_static_rmsnorm_w_bf16_g4_it1"
-    assert Prog(1 << 20, 128, F16).row("layernorm", 2).op("gelu").name() == "rows_static_layernorm_gelu_wb_f16_g16_it1"
+    assert Prog(1 << 20, 128, BF16).row("layernorm", 2).op("gelu").name() == "rows_static_layernorm_gelu_wb_bf16_g16_it1"
     assert Prog(1 << 20, 128, F32).row("softmax").name() == "rows_static_softmax_f32_g32_it1"
     assert Prog(1 << 20, 100, F32).row("softmax").name() == "rows_static_softmax_f32_g32_it1"  # 25 chunks: seven idle lanes per row
     assert Prog(1 << 20, 256, BF16).op("square").reduce("mean").name() == "rows_static_square_reduce_sum_bf16_g32_it1"
     assert Prog(1 << 20, 264, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1"  # 33 chunks
     # odd lengths: the same on memory's 16-byte grid, a masked partial chunk at either end of every row
     assert Prog(1 << 20, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g16_it1_grid"
-    assert Prog(1 << 20, 10, F32).row("logsoftmax").name() == "rows_static_logsoftmax_f32_g4_it1_grid"
+    assert Prog(1 << 20, 10, F32).row("logsoftmax").name() == "rows_jit_logsoftmax_f32_g4_it1_grid"
     assert Prog(1 << 20, 5, BF16).row("softmax").name() == "rows_static_softmax_bf16_g4_it1_grid"  # shorter than a chunk
-    assert Prog(1 << 20, 197, F16).row("layernorm", 2).name() == "rows_static_layernorm_wb_f16_g32_it1_grid"
+    assert Prog(1 << 20, 197, BF16).row("layernorm", 2).name() == "rows_static_layernorm_wb_bf16_g32_it1_grid"
     assert Prog(1 << 20, 250, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1_ragged"  # 33 chunks on the grid
     p = Prog(1 << 20, 77, BF16).row("softmax")
     p.p.output += 2  # input and output at different addresses modulo 16: a wavefront per row, from the row's first element

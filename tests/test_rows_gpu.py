@@ -132,7 +132,7 @@ def test_short_rows_that_share_a_wavefront(dt):
             p = gh.Rows(x, dt).row_op("softmax")
             p.keep.append(dst)
             p.p.output, p.p.output_dtype = dst.data_ptr(), dt
-            assert p.kernel_name() == f"rows_static_softmax_{tag}_g{group}_it1", (cols, p.kernel_name())
+            assert p.kernel_name() == f"rows_{'jit' if dt == F16 else 'static'}_softmax_{tag}_g{group}_it1", (cols, p.kernel_name())
             gh.sync()
             gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
             gh.sync()
@@ -179,7 +179,7 @@ def test_short_rows_of_odd_length_share_a_wavefront_on_the_16_byte_grid(dt):
             p.keep += [src, dst]
             p.p.rows, p.p.input = rows, src.data_ptr() + off * es
             p.p.output, p.p.output_dtype = dst.data_ptr() + (pad + off) * es, dt
-            assert p.kernel_name() == f"rows_static_softmax_{tag}_g{group}_it1_grid", (cols, p.kernel_name())
+            assert p.kernel_name() == f"rows_{'jit' if dt == F16 else 'static'}_softmax_{tag}_g{group}_it1_grid", (cols, p.kernel_name())
             gh.sync()
             gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
             gh.sync()
@@ -452,7 +452,9 @@ def test_scaled_and_biased_softmax_on_the_specialised_kernels(dt):
             got = prog.run()
             # a built-in kernel, or for a row length between the built-in plans (8200 columns) one compiled for it
             assert prog.kernel_name().startswith(("rows_static_" + tag, "rows_jit_" + tag)), prog.kernel_name()
-            assert cols % 1024 != 0 or prog.kernel_name().startswith("rows_static_"), prog.kernel_name()
+            # (built in: softmax(x * s) and softmax(x + y) for fp32 and bf16 at the stock row lengths; the rest is compiled when first launched)
+            assert not (cols % 1024 == 0 and dt != F16 and tag != "muls_addf_softmax" and prog.p.n_operands == (0 if tag == "muls_softmax" else 1)) \
+                or prog.kernel_name().startswith("rows_static_"), prog.kernel_name()
             got = got.astype(np.float64) if dt == F32 else axo.to_f32(got, dt).astype(np.float64)
             e = np.exp(logits - logits.max(-1, keepdims=True))
             want = e / e.sum(-1, keepdims=True)
@@ -470,7 +472,7 @@ def test_fast_activations_after_a_norm_in_16_bit(post):
     w, b = axo.to_bits(g.uniform((1024,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((1024,), -0.5, 0.5), BF16)
     prog = gh.Rows(x, BF16).row_op("layernorm", 1e-5, w=w, b=b).unary(post)
     got = axo.to_f32(prog.run(), BF16).astype(np.float64)
-    assert prog.kernel_name() == ("rows_static_" if post == "silu" else "rows_jit_") + f"layernorm_{post}_wb_bf16_g64_it2", prog.kernel_name()
+    assert prog.kernel_name() == f"rows_jit_layernorm_{post}_wb_bf16_g64_it2", prog.kernel_name()  # (of the activations only gelu is built in)
     xf = axo.to_f32(x, BF16).astype(np.float64)
     n = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
     want = {"silu": n / (1 + np.exp(-n)), "sigmoid": 1 / (1 + np.exp(-n)), "tanh": np.tanh(n)}[post]
@@ -628,7 +630,7 @@ def test_unary_then_row_reduction_runs_on_the_specialised_reduce_kernels():
     xbf = axo.to_f32(xb, BF16).astype(np.float64)
     p = gh.Rows(x, F32).unary("relu")
     got = p.run(reduce="sum")
-    assert p.kernel_name().startswith("rows_static_relu_reduce_sum_f32"), p.kernel_name()
+    assert p.kernel_name().startswith("rows_jit_relu_reduce_sum_f32"), p.kernel_name()  # (square and abs are built in, relu is compiled on first use)
     assert np.allclose(got, np.maximum(x.astype(np.float64), 0).sum(-1), rtol=1e-4, atol=1e-3)
     p = gh.Rows(xb, BF16, F32).unary("square")
     got = p.run(reduce="mean")
@@ -745,7 +747,7 @@ def test_bases_that_are_only_element_aligned(dt):
     p.p.operands[1].ptr = shifted(p, w, 5)
     p.p.operands[2].ptr = shifted(p, b, 2)
     got = f(p.run())
-    assert p.kernel_name().startswith("rows_static_addf_layernorm") and p.kernel_name().endswith("_ragged"), p.kernel_name()
+    assert p.kernel_name().startswith(("rows_static_addf_layernorm", "rows_jit_addf_layernorm")) and p.kernel_name().endswith("_ragged"), p.kernel_name()
     t = f(x) + f(y)
     ref = (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * f(w) + f(b)
     assert np.max(np.abs(got - ref)) < (1e-4 if dt == F32 else 4e-2)
@@ -988,4 +990,38 @@ def test_seeded_random_row_programs_match_fp64(dt):
             tol = tol + 2e-4  # the polynomial activations behind a 16-bit result
         err = np.abs(got.reshape(ref.shape) - ref)
         assert np.all(err <= tol), (case, desc, name, float(np.max(err / tol)))
-    assert {"static", "jit"} <= kinds, kinds
+    assert ({"jit"} if dt == F16 else {"static", "jit"}) <= kinds, kinds  # (no f16 shape is built in)
+
+
+def test_run_time_compiled_kernels_come_back_from_the_on_disk_cache(tmp_path):
+    """A process that finds the code object of a "rows_jit_" kernel in AXHIP_CACHE_DIR loads it instead of compiling
+    it again; the result is the same bits.  Two fresh processes, the second after the first."""
+    import os
+    import subprocess
+    import sys
+
+    script = r'''
+import ctypes as C, sys, numpy as np
+from oracle import axo
+from tests import gpu_harness as gh
+g = axo.PCG64(77)
+x = axo.to_bits(g.normal((33, 1536)), axo.BF16)
+w, b = axo.to_bits(g.uniform((1536,), 0.5, 1.5), axo.BF16), axo.to_bits(g.uniform((1536,), -0.1, 0.1), axo.BF16)
+prog = gh.Rows(x, axo.BF16).row_op("layernorm", 1e-5, w=w, b=b).unary("sigmoid")
+y = prog.run()
+assert prog.kernel_name().startswith("rows_jit_"), prog.kernel_name()
+d, c = C.c_int(0), C.c_int(0)
+gh.capi.lib().axhip_fused_rows_jit_counters(C.byref(d), C.byref(c))
+print("COUNTERS", d.value, c.value, int(np.asarray(y, np.uint16).astype(np.uint64).sum()))
+'''
+    env = dict(os.environ, AXHIP_CACHE_DIR=str(tmp_path / "axhip-cache"), PYTHONPATH=os.pathsep.join([os.getcwd(), os.environ.get("PYTHONPATH", "")]))
+    outs = []
+    for _ in range(2):
+        r = subprocess.run([sys.executable, "-c", script], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert r.returncode == 0, r.stdout[-2000:]
+        outs.append([ln for ln in r.stdout.splitlines() if ln.startswith("COUNTERS")][-1].split()[1:])
+    (d1, c1, sum1), (d2, c2, sum2) = outs
+    assert (int(d1), int(c1)) == (0, 1), outs  # compiled, stored
+    assert (int(d2), int(c2)) == (1, 0), outs  # loaded
+    assert sum1 == sum2
+    assert any(f.suffix == ".hsaco" for f in (tmp_path / "axhip-cache").iterdir())

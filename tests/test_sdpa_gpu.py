@@ -295,6 +295,9 @@ def test_full_size_causal_bf16_properties():
     q, k, v = (axo.to_bits(g.normal((B, H, S, D)), BF16) for _ in range(3))
     got, kern = gh.sdpa(q, k, v, BF16, -1.0, True)
     assert kern == "mfma_bf16_d128"
+    from axiom_amd import capi
+
+    assert capi.lib().axhip_sdpa_last_schedule() == b"pingpong"
     gf = axo.to_f32(got, BF16)
     assert np.isfinite(gf).all()
     vf = axo.to_f32(v, BF16)
@@ -368,3 +371,59 @@ def test_seeded_random_problems_match_fp64(dt):
         want = naive_attention64(*(axo.to_f32(t, dt) for t in (q, k, v)), sc, causal, mask)
         err = np.max(np.abs(axo.to_f32(got, dt).astype(np.float64) - want))
         assert err < (1e-4 if dt == F32 else 2e-2), (case, B, H, Sq, Skv, D, causal, mkind, scale, float(err))
+
+
+# (B, H, Sq, Skv, causal): unmasked head_dim-128 problems with a 256-row work-group for every CU -- the ping-pong
+# schedule with persistent work-groups.  Ragged query blocks and key tails, one and two passes per causal pair, even
+# and odd tile counts (only an even count requests the next segment's first tiles ahead), more units than
+# work-groups, a (batch, head) count that 8 does not divide, cross attention.
+PINGPONG_CASES = [
+    (8, 32, 256, 256, False), (8, 32, 256, 256, True), (8, 32, 300, 333, False), (4, 32, 1000, 1000, True),
+    (8, 32, 700, 150, False), (8, 32, 260, 64, False), (8, 32, 257, 70, True), (4, 65, 256, 192, False),
+    (2, 64, 1030, 1030, True), (8, 32, 512, 1000, True), (16, 32, 129, 640, False),
+]
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", PINGPONG_CASES, ids=lambda c: "x".join(str(int(x)) for x in c))
+def test_chip_filling_head_dim_128_problems_on_the_ping_pong_schedule(case, dt):
+    from axiom_amd import capi
+
+    B, H, Sq, Skv, causal = case
+    D = 128
+    q, k, v = inputs(B, H, Sq, Skv, D, dt, seed=11)
+    got, kern = gh.sdpa(q, k, v, dt, -1.0, causal)
+    assert kern == f"mfma_{'bf16' if dt == BF16 else 'f16'}_d128"
+    assert capi.lib().axhip_sdpa_last_schedule() == b"pingpong"
+    gotf = axo.to_f32(got, dt)
+    assert np.isfinite(gotf).all()
+    # float64 textbook attention on slices spread over the units: first, last, and every 19th in between
+    slices = sorted(set([0, B * H - 1] + list(range(3, B * H, 19))))
+    for sl in slices:
+        b, h = divmod(sl, H)
+        qs, ks, vs = (axo.to_f32(t[b:b + 1, h:h + 1], dt) for t in (q, k, v))
+        want = naive_attention64(qs, ks, vs, 1 / math.sqrt(D), causal, None)
+        err = np.max(np.abs(gotf[b:b + 1, h:h + 1] - want))
+        assert err < 2e-2, (sl, err)
+
+
+def test_ping_pong_schedule_on_head_split_views_and_a_row_dominated_by_a_late_key():
+    """Strided (B,S,H,D) -> (B,H,S,D) views as nn::MultiHeadAttention hands them over, and a key far down the
+    sequence whose logit dwarfs the running maximum (the accumulators are rescaled late)."""
+    from axiom_amd import capi
+
+    B, H, S, D = 4, 64, 512, 128
+    g = axo.PCG64(5)
+    raw = [g.normal((B, S, H, D)) for _ in range(3)]
+    raw[1][:, 450, :, :] *= 6.0  # one key with large logits for many queries
+    raw[2] *= 0.5  # (outputs stay below 2: a bf16 step of 2^-7, well inside the 2e-2 bar)
+    q, k, v = (axo.to_bits(t, BF16) for t in raw)
+    st = (S * H * D, D, H * D)
+    got, _ = gh.sdpa(q, k, v, BF16, -1.0, False, None, q_strides=st, k_strides=st, v_strides=st, shape=(B, H, S, S, D))
+    assert capi.lib().axhip_sdpa_last_schedule() == b"pingpong"
+    gotf = axo.to_f32(got, BF16)
+    for b, h in ((0, 0), (1, 17), (3, 63)):
+        qs, ks, vs = (axo.to_f32(t[b:b + 1, :, h:h + 1], BF16).transpose(0, 2, 1, 3) for t in (q, k, v))
+        want = naive_attention64(qs, ks, vs, 1 / math.sqrt(D), False, None)
+        err = np.max(np.abs(gotf[b:b + 1, h:h + 1] - want))
+        assert err < 2e-2, ((b, h), err)
