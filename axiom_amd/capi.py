@@ -10,13 +10,17 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libaxhip.so"
 
-DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
+DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_U8 = 0, 1, 2, 3
 
 OP = dict(add=1, sub=2, mul=3, div=4, max=5, min=6, rsub=7, rdiv=8,
           relu=16, gelu=17, sqrt=18, exp=19, neg=20, abs=21, sigmoid=22, tanh=23,
-          silu=24, log=25, square=26, rsqrt=27, recip=28)
+          silu=24, log=25, square=26, rsqrt=27, recip=28,
+          pow=40, rpow=41, mod=42, rmod=43, atan2=44, ratan2=45, hypot=46, eq=47, ne=48, lt=49, le=50, gt=51, ge=52,
+          **{"and": 53, "or": 54, "xor": 55, "not": 77}, leaky_relu=56,
+          erf=64, sin=65, cos=66, tan=67, sign=68, floor=69, ceil=70, round=71, trunc=72, cbrt=73,
+          isnan=74, isinf=75, isfinite=76)
 ROWOP = dict(none=0, softmax=1, logsoftmax=2, layernorm=3, rmsnorm=4)
-RED = dict(none=0, sum=1, mean=2, max=3, min=4)
+RED = dict(none=0, sum=1, mean=2, max=3, min=4, prod=5)
 BK = dict(full=0, rowvec=1, colvec=2, scalar=3, imm=4)
 
 MAX_CHAIN, MAX_OPERANDS = 16, 8
@@ -121,6 +125,8 @@ def lib() -> C.CDLL:
         i64p = C.POINTER(C.c_int64)
         l.axhip_pad.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, i64p, i64p, i64p, i64p, C.c_double, C.c_void_p]
         l.axhip_masked_fill.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, i64p, i64p, i64p, C.c_double, C.c_void_p]
+        l.axhip_where.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32,
+                                  i64p, i64p, i64p, i64p, C.c_void_p]
         l.axhip_argreduce.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         l.axhip_reduce_axis.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]
         l.axhip_argreduce_workspace_bytes.restype = C.c_size_t

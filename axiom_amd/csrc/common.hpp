@@ -93,7 +93,8 @@ private:
 };
 
 inline bool valid_dtype(int dt) { return dt >= AXHIP_DTYPE_F32 && dt <= AXHIP_DTYPE_BF16; }
-inline size_t dtype_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
+inline bool valid_dtype_or_u8(int dt) { return valid_dtype(dt) || dt == AXHIP_DTYPE_U8; }
+inline size_t dtype_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : dt == AXHIP_DTYPE_U8 ? 1 : 2; }
 // Outputs of at least this size are written with non-temporal stores: they cannot stay in the
 // 256 MiB last-level cache next to the launch's inputs anyway, and a consumer that follows
 // immediately could not find them there either.
@@ -160,12 +161,15 @@ template <> struct Elem<AXHIP_DTYPE_BF16> {
 
 __device__ __forceinline__ float load_any(const void *p, int dt, int64_t i) {
     if (dt == AXHIP_DTYPE_F32) return static_cast<const float *>(p)[i];
+    if (dt == AXHIP_DTYPE_U8) return static_cast<const uint8_t *>(p)[i] ? 1.0f : 0.0f;
     uint32_t h = static_cast<const uint16_t *>(p)[i];
     return dt == AXHIP_DTYPE_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
 }
 __device__ __forceinline__ void store_any(void *p, int dt, int64_t i, float v) {
     if (dt == AXHIP_DTYPE_F32) {
         static_cast<float *>(p)[i] = v;
+    } else if (dt == AXHIP_DTYPE_U8) {
+        static_cast<uint8_t *>(p)[i] = v != 0.0f ? 1 : 0;
     } else {
         static_cast<uint16_t *>(p)[i] =
             static_cast<uint16_t>(dt == AXHIP_DTYPE_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v));
@@ -225,9 +229,22 @@ template <bool UNALIGNED> __device__ __forceinline__ void vec_store(uint2_t *p, 
 
 // Load / store N consecutive elements (N*sizeof(elem) is 16 or 32 bytes and, unless UNALIGNED, the
 // address is aligned to min(16, that)) as fp32 values.
+struct __attribute__((packed, aligned(1))) uint32_unaligned_t { uint32_t v; };
+
 template <int N, bool UNALIGNED = false>
 __device__ __forceinline__ void load_vec(const void *p, int dt, int64_t i, float (&v)[N]) {
-    if (dt == AXHIP_DTYPE_F32) {
+    if (dt == AXHIP_DTYPE_U8) { // N bytes, in 32-bit words (the address is N-aligned unless UNALIGNED)
+        static_assert(N % 4 == 0, "vector width");
+        const uint8_t *q = static_cast<const uint8_t *>(p) + i;
+#pragma unroll
+        for (int j = 0; j < N / 4; ++j) {
+            uint32_t w;
+            if constexpr (UNALIGNED) w = reinterpret_cast<const uint32_unaligned_t *>(q + 4 * j)->v;
+            else w = *reinterpret_cast<const uint32_t *>(q + 4 * j);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[4 * j + k] = ((w >> (8 * k)) & 0xFFu) ? 1.0f : 0.0f;
+        }
+    } else if (dt == AXHIP_DTYPE_F32) {
         const float4_t *q = reinterpret_cast<const float4_t *>(static_cast<const float *>(p) + i);
 #pragma unroll
         for (int j = 0; j < N / 4; ++j) {
@@ -281,7 +298,18 @@ __device__ __forceinline__ void store16_streaming(void *p, uint4_t v) {
 // push the inputs of the same launch out of the last-level cache)
 template <int N, bool UNALIGNED = false>
 __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const float (&v)[N], bool streaming = false) {
-    if (dt == AXHIP_DTYPE_F32) {
+    if (dt == AXHIP_DTYPE_U8) {
+        static_assert(N % 4 == 0, "vector width");
+        uint8_t *q = static_cast<uint8_t *>(p) + i;
+#pragma unroll
+        for (int j = 0; j < N / 4; ++j) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) w |= (v[4 * j + k] != 0.0f ? 1u : 0u) << (8 * k);
+            if constexpr (UNALIGNED) reinterpret_cast<uint32_unaligned_t *>(q + 4 * j)->v = w;
+            else *reinterpret_cast<uint32_t *>(q + 4 * j) = w;
+        }
+    } else if (dt == AXHIP_DTYPE_F32) {
         float4_t *q = reinterpret_cast<float4_t *>(static_cast<float *>(p) + i);
 #pragma unroll
         for (int j = 0; j < N / 4; ++j) {
@@ -319,6 +347,11 @@ __device__ __forceinline__ void store_vec(void *p, int dt, int64_t i, const floa
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_prod(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v *= __shfl_xor(v, o, WAVE);
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {

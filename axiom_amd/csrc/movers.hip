@@ -185,6 +185,49 @@ __global__ __launch_bounds__(256) void masked_fill_kernel(const MaskedFillArgs a
     }
 }
 
+// where(cond, a, b): dst[i] = cond[i] ? a[i] : b[i] over an iteration space of up to 8 dimensions; the three inputs
+// are strided views (stride 0 on broadcast dimensions), each of a type of its own; dst is contiguous.
+struct WhereArgs {
+    const void *cond, *a, *b;
+    void *dst;
+    int cond_dtype, a_dtype, b_dtype, dst_dtype, ndim;
+    int64_t total;
+    int64_t shape[AXHIP_MAX_DIMS], cond_strides[AXHIP_MAX_DIMS], a_strides[AXHIP_MAX_DIMS], b_strides[AXHIP_MAX_DIMS];
+};
+
+__global__ __launch_bounds__(256) void where_kernel(const WhereArgs w) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < w.total; i += stride) {
+        int64_t rem = i, coff = 0, aoff = 0, boff = 0;
+        for (int d = w.ndim - 1; d >= 0; --d) {
+            const int64_t c = rem % w.shape[d];
+            rem /= w.shape[d];
+            coff += c * w.cond_strides[d];
+            aoff += c * w.a_strides[d];
+            boff += c * w.b_strides[d];
+        }
+        const bool pick = load_any(w.cond, w.cond_dtype, coff) != 0.0f;
+        store_any(w.dst, w.dst_dtype, i, pick ? load_any(w.a, w.a_dtype, aoff) : load_any(w.b, w.b_dtype, boff));
+    }
+}
+
+// the three inputs contiguous and of the output's extent (a and b may each be one broadcast element): V elements
+// per thread, every access a whole vector
+template <int V>
+__global__ __launch_bounds__(256) void where_vec_kernel(const WhereArgs w, const bool a_scalar, const bool b_scalar) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256, chunks = w.total / V;
+    const float a0 = a_scalar ? load_any(w.a, w.a_dtype, 0) : 0.0f, b0 = b_scalar ? load_any(w.b, w.b_dtype, 0) : 0.0f;
+    for (int64_t c = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; c < chunks; c += stride) {
+        float m[V], x[V], y[V];
+        load_vec<V>(w.cond, w.cond_dtype, c * V, m);
+        if (!a_scalar) load_vec<V>(w.a, w.a_dtype, c * V, x);
+        if (!b_scalar) load_vec<V>(w.b, w.b_dtype, c * V, y);
+#pragma unroll
+        for (int e = 0; e < V; ++e) x[e] = m[e] != 0.0f ? (a_scalar ? a0 : x[e]) : (b_scalar ? b0 : y[e]);
+        store_vec<V>(w.dst, w.dst_dtype, c * V, x);
+    }
+}
+
 // One thread moves `chunk` bytes (16, or the element size when rows are not 16-byte
 // multiples) of one output row.
 template <typename V>
@@ -403,8 +446,8 @@ __global__ __launch_bounds__(256) void argreduce_merge_kernel(const float *part_
 // argreduce_strided_vec_kernel (a thread owns the V inner positions of one 16-byte vector, TX threads side by side,
 // the TY = 256 / TX thread rows of a work-group share the axis and merge through LDS); fp32 accumulation, the result
 // scaled (mean) and rounded to the output type.
-template <int RED> __device__ __forceinline__ float red_identity() { return RED == AXHIP_RED_MAX ? -INFINITY : RED == AXHIP_RED_MIN ? INFINITY : 0.0f; }
-template <int RED> __device__ __forceinline__ float red_combine(float a, float b) { return RED == AXHIP_RED_MAX ? fmaxf(a, b) : RED == AXHIP_RED_MIN ? fminf(a, b) : a + b; }
+template <int RED> __device__ __forceinline__ float red_identity() { return RED == AXHIP_RED_MAX ? -INFINITY : RED == AXHIP_RED_MIN ? INFINITY : RED == AXHIP_RED_PROD ? 1.0f : 0.0f; }
+template <int RED> __device__ __forceinline__ float red_combine(float a, float b) { return RED == AXHIP_RED_MAX ? fmaxf(a, b) : RED == AXHIP_RED_MIN ? fminf(a, b) : RED == AXHIP_RED_PROD ? a * b : a + b; }
 
 template <int RED, int DT, int TX>
 __global__ __launch_bounds__(256) void reduce_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, float scale, void *dst, int dst_dt) {
@@ -583,7 +626,8 @@ __global__ __launch_bounds__(256) void softmax_strided_kernel(const void *src, i
 // one launch: RED is sum, max or min; the result is multiplied by `scale`
 int launch_reduce_axis(const void *src, int dtype, int64_t outer, int64_t axis, int64_t inner, int red, float scale, void *dst, int dst_dtype, hipStream_t s) {
     const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
-    if (inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
+    const bool bytes = dtype == AXHIP_DTYPE_U8 || dst_dtype == AXHIP_DTYPE_U8;
+    if (red != AXHIP_RED_PROD && !bytes && inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) { // (products, truth values: the element-wise kernel)
         const int64_t ivecs = inner / (16 / es);
         // a short axis with plenty of results: a thread per vector walks it alone (no merge through LDS)
         const bool flat = axis <= 32 && outer * ((ivecs + 255) / 256) >= 1024 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0;
@@ -612,6 +656,7 @@ int launch_reduce_axis(const void *src, int dtype, int64_t outer, int64_t axis, 
         const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((outer * inner + 255) / 256, 256 * 32));
         if (red == AXHIP_RED_SUM) hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_SUM>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
         else if (red == AXHIP_RED_MAX) hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_MAX>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
+        else if (red == AXHIP_RED_PROD) hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_PROD>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
         else hipLaunchKernelGGL(reduce_strided_kernel<AXHIP_RED_MIN>, dim3(blocks), dim3(256), 0, s, src, dtype, outer, axis, inner, scale, dst, dst_dtype);
     }
     AXHIP_CHECK_HIP(hipGetLastError());
@@ -625,7 +670,8 @@ extern "C" {
 
 int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t dst_dtype, int32_t ndim,
                        const int64_t *shape, const int64_t *strides, void *stream) {
-    AXHIP_REQUIRE(valid_dtype(src_dtype) && valid_dtype(dst_dtype), AXHIP_ERR_INVALID_ARG, "axhip_strided_copy: bad dtype");
+    AXHIP_REQUIRE(valid_dtype_or_u8(src_dtype) && valid_dtype_or_u8(dst_dtype), AXHIP_ERR_INVALID_ARG, "axhip_strided_copy: bad dtype");
+    const bool bytes = src_dtype == AXHIP_DTYPE_U8 || dst_dtype == AXHIP_DTYPE_U8; // truth values: the element-wise kernel
     AXHIP_REQUIRE(ndim >= 0 && ndim <= AXHIP_MAX_DIMS, AXHIP_ERR_INVALID_ARG, "axhip_strided_copy: ndim %d out of range", ndim);
     AXHIP_REQUIRE(ndim == 0 || (shape && strides), AXHIP_ERR_INVALID_ARG, "axhip_strided_copy: NULL shape/strides");
     CopyArgs a{};
@@ -667,12 +713,12 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
     const int v = raw ? (src_dtype == AXHIP_DTYPE_F32 ? 4 : 8) : (dst_dtype == AXHIP_DTYPE_F32 ? 4 : 8);
     const int src_es = src_dtype == AXHIP_DTYPE_F32 ? 4 : 2, dst_es = dst_dtype == AXHIP_DTYPE_F32 ? 4 : 2;
     const int src_align = src_es == 4 ? 16 : v * 2; // bytes a vector load needs
-    bool vec = nd >= 1 && a.strides[nd - 1] == 1 && a.shape[nd - 1] % v == 0 && reinterpret_cast<uintptr_t>(src) % src_align == 0 &&
+    bool vec = !bytes && nd >= 1 && a.strides[nd - 1] == 1 && a.shape[nd - 1] % v == 0 && reinterpret_cast<uintptr_t>(src) % src_align == 0 &&
                reinterpret_cast<uintptr_t>(dst) % (v * dst_es >= 16 ? 16 : 8) == 0;
     for (int d = 0; vec && d + 1 < nd; ++d) vec = (a.strides[d] * src_es) % src_align == 0;
     // transposes: the innermost dimension is strided, some other dimension is contiguous in the source
     int transpose_j = -1;
-    if (!vec && nd >= 2 && a.strides[nd - 1] > 1 && a.shape[nd - 1] >= 16) {
+    if (!vec && !bytes && nd >= 2 && a.strides[nd - 1] > 1 && a.shape[nd - 1] >= 16) {
         for (int d = 0; d + 1 < nd; ++d)
             if (a.strides[d] == 1 && a.shape[d] >= 16) transpose_j = d;
     }
@@ -809,6 +855,55 @@ int axhip_masked_fill(const void *src, int32_t dtype, const uint8_t *mask, void 
     if (rc) return rc;
     const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
     hipLaunchKernelGGL(masked_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), a);
+    AXHIP_CHECK_HIP(hipGetLastError());
+    return AXHIP_OK;
+}
+
+int axhip_where(const void *cond, int32_t cond_dtype, const void *a, int32_t a_dtype, const void *b, int32_t b_dtype, void *dst, int32_t dst_dtype,
+                int32_t ndim, const int64_t *shape, const int64_t *cond_strides, const int64_t *a_strides, const int64_t *b_strides, void *stream) {
+    AXHIP_REQUIRE(valid_dtype_or_u8(cond_dtype) && valid_dtype_or_u8(a_dtype) && valid_dtype_or_u8(b_dtype) && valid_dtype_or_u8(dst_dtype),
+                  AXHIP_ERR_INVALID_ARG, "axhip_where: bad dtype");
+    AXHIP_REQUIRE(ndim >= 0 && ndim <= AXHIP_MAX_DIMS, AXHIP_ERR_INVALID_ARG, "axhip_where: ndim %d out of range", ndim);
+    AXHIP_REQUIRE(ndim == 0 || (shape && cond_strides && a_strides && b_strides), AXHIP_ERR_INVALID_ARG, "axhip_where: NULL shape/strides");
+    WhereArgs w{};
+    w.cond = cond; w.a = a; w.b = b; w.dst = dst;
+    w.cond_dtype = cond_dtype; w.a_dtype = a_dtype; w.b_dtype = b_dtype; w.dst_dtype = dst_dtype; w.ndim = ndim;
+    w.total = 1;
+    bool cond_flat = true, a_flat = true, b_flat = true, a_one = true, b_one = true; // contiguous over the whole extent / one element
+    int64_t run = 1;
+    for (int d = ndim - 1; d >= 0; --d) {
+        AXHIP_REQUIRE(shape[d] >= 0, AXHIP_ERR_INVALID_ARG, "axhip_where: negative extent");
+        AXHIP_REQUIRE(cond_strides[d] >= 0 && a_strides[d] >= 0 && b_strides[d] >= 0, AXHIP_ERR_UNSUPPORTED, "axhip_where: negative strides are not supported");
+        w.shape[d] = shape[d];
+        w.cond_strides[d] = cond_strides[d];
+        w.a_strides[d] = a_strides[d];
+        w.b_strides[d] = b_strides[d];
+        if (shape[d] != 1) {
+            cond_flat = cond_flat && cond_strides[d] == run;
+            a_flat = a_flat && a_strides[d] == run;
+            b_flat = b_flat && b_strides[d] == run;
+            a_one = a_one && a_strides[d] == 0;
+            b_one = b_one && b_strides[d] == 0;
+        }
+        run *= shape[d];
+        w.total *= shape[d];
+    }
+    if (w.total == 0) return AXHIP_OK;
+    AXHIP_REQUIRE(cond && a && b && dst, AXHIP_ERR_INVALID_ARG, "axhip_where: NULL buffer");
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = resolve_stream(stream);
+    auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    const bool wide = (!a_one && a_dtype == AXHIP_DTYPE_F32) || (!b_one && b_dtype == AXHIP_DTYPE_F32) || dst_dtype == AXHIP_DTYPE_F32;
+    const int v = wide ? 4 : 8;
+    if (cond_flat && (a_flat || a_one) && (b_flat || b_one) && w.total % v == 0 && aligned(cond) && aligned(dst) && (a_one || aligned(a)) && (b_one || aligned(b))) {
+        const int64_t blocks = std::min<int64_t>((w.total / v + 255) / 256, 256 * 64);
+        if (v == 4) hipLaunchKernelGGL(where_vec_kernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w, a_one, b_one);
+        else hipLaunchKernelGGL(where_vec_kernel<8>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w, a_one, b_one);
+    } else {
+        const int64_t blocks = std::min<int64_t>((w.total + 255) / 256, 256 * 64);
+        hipLaunchKernelGGL(where_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w);
+    }
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;
 }
@@ -978,9 +1073,8 @@ int axhip_reduce_axis(const void *src, int32_t dtype, int64_t outer, int64_t axi
 
 int axhip_reduce_axis_ws(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner, int32_t reduce, void *dst, int32_t dst_dtype,
                          void *workspace, size_t workspace_bytes, void *stream) {
-    AXHIP_REQUIRE(valid_dtype(dtype) && valid_dtype(dst_dtype), AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: bad dtype");
-    AXHIP_REQUIRE(reduce == AXHIP_RED_SUM || reduce == AXHIP_RED_MEAN || reduce == AXHIP_RED_MAX || reduce == AXHIP_RED_MIN, AXHIP_ERR_INVALID_ARG,
-                  "axhip_reduce_axis: bad reduction %d", reduce);
+    AXHIP_REQUIRE(valid_dtype_or_u8(dtype) && valid_dtype_or_u8(dst_dtype), AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: bad dtype");
+    AXHIP_REQUIRE(reduce >= AXHIP_RED_SUM && reduce <= AXHIP_RED_PROD, AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: bad reduction %d", reduce);
     AXHIP_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: negative extent");
     if (outer == 0 || inner == 0) return AXHIP_OK;
     AXHIP_REQUIRE(axis > 0, AXHIP_ERR_INVALID_ARG, "axhip_reduce_axis: empty axis");
@@ -998,10 +1092,10 @@ int axhip_reduce_axis_ws(const void *src, int32_t dtype, int64_t outer, int64_t 
     const float scale = reduce == AXHIP_RED_MEAN ? 1.0f / static_cast<float>(axis) : 1.0f;
     const int red = reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : reduce;
     const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
-    const bool vec = inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
+    const bool vec = dtype != AXHIP_DTYPE_U8 && dst_dtype != AXHIP_DTYPE_U8 && inner % (16 / es) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
     // Few results over a long axis (column sums of a tall matrix): too few work-groups for the chip.  The axis is cut
     // into `parts` equal segments, reduced to fp32 partials in stream-ordered temporary memory, and those reduced again.
-    const int64_t parts = vec ? reduce_axis_parts(src, dtype, outer, axis, inner) : 1;
+    const int64_t parts = vec && red != AXHIP_RED_PROD ? reduce_axis_parts(src, dtype, outer, axis, inner) : 1;
     if (parts > 1) {
         CallScratch scratch(workspace, workspace_bytes, s);
         void *tmp = nullptr;

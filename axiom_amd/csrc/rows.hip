@@ -99,9 +99,9 @@ __device__ __forceinline__ void apply_affine(int operand, const AxhipRowsProgram
 
 // Reduce across the GROUP threads that share a row.  GROUP == 64: shuffles
 // only.  GROUP == blockDim: shuffles, then one LDS exchange between waves.
-template <int GROUP, int THREADS, int KIND /*0 sum, 1 max, 2 min*/>
+template <int GROUP, int THREADS, int KIND /*0 sum, 1 max, 2 min, 3 product*/>
 __device__ __forceinline__ float group_reduce(float x, float *lds) {
-    x = KIND == 0 ? wave_sum(x) : KIND == 1 ? wave_max(x) : wave_min(x);
+    x = KIND == 0 ? wave_sum(x) : KIND == 1 ? wave_max(x) : KIND == 2 ? wave_min(x) : wave_prod(x);
     if constexpr (GROUP > WAVE) {
         constexpr int NW = THREADS / WAVE;
         const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
@@ -112,11 +112,26 @@ __device__ __forceinline__ float group_reduce(float x, float *lds) {
 #pragma unroll
         for (int o = NW / 2; o > 0; o >>= 1) {
             float z = __shfl_xor(y, o, WAVE);
-            y = KIND == 0 ? y + z : KIND == 1 ? fmaxf(y, z) : fminf(y, z);
+            y = KIND == 0 ? y + z : KIND == 1 ? fmaxf(y, z) : KIND == 2 ? fminf(y, z) : y * z;
         }
         x = y;
     }
     return x;
+}
+
+// the reduction kinds as run-time values (AXHIP_RED_*; MEAN folds like SUM and is scaled by the caller)
+__device__ __forceinline__ float red_start(int reduce) {
+    return reduce == AXHIP_RED_MAX ? NEG_INF : reduce == AXHIP_RED_MIN ? POS_INF : reduce == AXHIP_RED_PROD ? 1.0f : 0.0f;
+}
+__device__ __forceinline__ float red_fold(int reduce, float acc, float x) {
+    return reduce == AXHIP_RED_MAX ? fmaxf(acc, x) : reduce == AXHIP_RED_MIN ? fminf(acc, x) : reduce == AXHIP_RED_PROD ? acc * x : acc + x;
+}
+template <int GROUP, int THREADS>
+__device__ __forceinline__ float group_reduce_of(int reduce, float acc, float *lds) {
+    if (reduce == AXHIP_RED_MAX) return group_reduce<GROUP, THREADS, 1>(acc, lds);
+    if (reduce == AXHIP_RED_MIN) return group_reduce<GROUP, THREADS, 2>(acc, lds);
+    if (reduce == AXHIP_RED_PROD) return group_reduce<GROUP, THREADS, 3>(acc, lds);
+    return group_reduce<GROUP, THREADS, 0>(acc, lds);
 }
 
 // One row per GROUP threads, the whole row resident in registers.
@@ -281,6 +296,14 @@ __global__ __launch_bounds__(THREADS) void rows_resident_kernel(const AxhipRowsP
             for (int e = 0; e < E; ++e)
                 if (valid(it, e)) acc = fmaxf(acc, v[it][e]);
         acc = group_reduce<GROUP, THREADS, 1>(acc, lds);
+    } else if (P.reduce == AXHIP_RED_PROD) {
+        acc = 1.0f;
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                if (valid(it, e)) acc *= v[it][e];
+        acc = group_reduce<GROUP, THREADS, 3>(acc, lds);
     } else {
         acc = POS_INF;
 #pragma unroll
@@ -309,7 +332,7 @@ __global__ __launch_bounds__(THREADS) void rows_streamed_kernel(const AxhipRowsP
     const int first_pass = is_sm || P.row_op == AXHIP_ROWOP_LAYERNORM ? 0 : is_norm ? 1 : 2;
 
     float stat_a = 0.0f, stat_b = 1.0f; // softmax: (max, 1/sum or log-sum); norms: (mean, rstd)
-    float out_acc = P.reduce == AXHIP_RED_MAX ? NEG_INF : P.reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+    float out_acc = red_start(P.reduce);
 #pragma nounroll
     for (int pass = first_pass; pass < 3; ++pass) {
         float acc = (pass == 0 && is_sm) ? NEG_INF : 0.0f;
@@ -348,9 +371,7 @@ __global__ __launch_bounds__(THREADS) void rows_streamed_kernel(const AxhipRowsP
                     else store_vec<E>(P.output, P.output_dtype, row * cols + col0[0], v[0]);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < E; ++e)
-                        out_acc = P.reduce == AXHIP_RED_MAX ? fmaxf(out_acc, v[0][e])
-                                  : P.reduce == AXHIP_RED_MIN ? fminf(out_acc, v[0][e]) : out_acc + v[0][e];
+                    for (int e = 0; e < E; ++e) out_acc = red_fold(P.reduce, out_acc, v[0][e]);
                 }
             }
         }
@@ -368,9 +389,7 @@ __global__ __launch_bounds__(THREADS) void rows_streamed_kernel(const AxhipRowsP
         }
     }
     if (P.reduce != AXHIP_RED_NONE) {
-        if (P.reduce == AXHIP_RED_MAX) out_acc = group_reduce<THREADS, THREADS, 1>(out_acc, lds);
-        else if (P.reduce == AXHIP_RED_MIN) out_acc = group_reduce<THREADS, THREADS, 2>(out_acc, lds);
-        else out_acc = group_reduce<THREADS, THREADS, 0>(out_acc, lds);
+        out_acc = group_reduce_of<THREADS, THREADS>(P.reduce, out_acc, lds);
         if (P.reduce == AXHIP_RED_MEAN) out_acc *= inv_n;
         if (threadIdx.x == 0) store_any(P.output, P.output_dtype, row, out_acc);
     }
@@ -464,7 +483,7 @@ __global__ __launch_bounds__(THREADS) void full_reduce_stage1(const AxhipRowsPro
     const int64_t cols = P.cols;
     const int64_t nchunk = P.rows * cols / E;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * THREADS;
-    float acc = P.reduce == AXHIP_RED_MAX ? NEG_INF : P.reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+    float acc = red_start(P.reduce);
     for (int64_t c = static_cast<int64_t>(blockIdx.x) * THREADS + threadIdx.x; c < nchunk; c += stride) {
         const int64_t flat = c * E;
         const int64_t row = flat / cols;
@@ -475,12 +494,9 @@ __global__ __launch_bounds__(THREADS) void full_reduce_stage1(const AxhipRowsPro
         else load_vec<E>(P.input, P.input_dtype, flat, v[0]);
         for (int i = 0; i < P.n_pre; ++i) apply_op<1, E>(P.pre[i], P, v, row, col0, ok);
 #pragma unroll
-        for (int e = 0; e < E; ++e)
-            acc = P.reduce == AXHIP_RED_MAX ? fmaxf(acc, v[0][e]) : P.reduce == AXHIP_RED_MIN ? fminf(acc, v[0][e]) : acc + v[0][e];
+        for (int e = 0; e < E; ++e) acc = red_fold(P.reduce, acc, v[0][e]);
     }
-    if (P.reduce == AXHIP_RED_MAX) acc = group_reduce<THREADS, THREADS, 1>(acc, lds);
-    else if (P.reduce == AXHIP_RED_MIN) acc = group_reduce<THREADS, THREADS, 2>(acc, lds);
-    else acc = group_reduce<THREADS, THREADS, 0>(acc, lds);
+    acc = group_reduce_of<THREADS, THREADS>(P.reduce, acc, lds);
     if (threadIdx.x == 0) partials[blockIdx.x] = acc;
 }
 
@@ -488,15 +504,10 @@ template <int THREADS>
 __global__ __launch_bounds__(THREADS) void full_reduce_stage2(const float *partials, int n, int reduce, float inv_count,
                                                               void *out, int out_dtype) {
     __shared__ float lds[THREADS / WAVE];
-    float acc = reduce == AXHIP_RED_MAX ? NEG_INF : reduce == AXHIP_RED_MIN ? POS_INF : 0.0f;
+    float acc = red_start(reduce);
 #pragma unroll 4
-    for (int i = threadIdx.x; i < n; i += THREADS) {
-        float x = partials[i];
-        acc = reduce == AXHIP_RED_MAX ? fmaxf(acc, x) : reduce == AXHIP_RED_MIN ? fminf(acc, x) : acc + x;
-    }
-    if (reduce == AXHIP_RED_MAX) acc = group_reduce<THREADS, THREADS, 1>(acc, lds);
-    else if (reduce == AXHIP_RED_MIN) acc = group_reduce<THREADS, THREADS, 2>(acc, lds);
-    else acc = group_reduce<THREADS, THREADS, 0>(acc, lds);
+    for (int i = threadIdx.x; i < n; i += THREADS) acc = red_fold(reduce, acc, partials[i]);
+    acc = group_reduce_of<THREADS, THREADS>(reduce, acc, lds);
     if (reduce == AXHIP_RED_MEAN) acc *= inv_count;
     if (threadIdx.x == 0) store_any(out, out_dtype, 0, acc);
 }
@@ -512,7 +523,7 @@ int validate_chain(const AxhipChainOp *ops, int n, const AxhipRowsProgram &P, co
     for (int i = 0; i < n; ++i) {
         const int op = ops[i].op;
         const bool bin = is_binary_op(op);
-        const bool un = op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP;
+        const bool un = is_unary_op(op);
         AXHIP_REQUIRE(bin || un, AXHIP_ERR_INVALID_ARG, "fused rows: %s[%d] has unknown op code %d", which, i, op);
         if (bin && ops[i].imm_kind != AXHIP_BK_IMM)
             AXHIP_REQUIRE(ops[i].operand >= 0 && ops[i].operand < P.n_operands, AXHIP_ERR_INVALID_ARG,
@@ -562,11 +573,11 @@ int flat_vector_width(const AxhipRowsProgram &P) {
 
 int validate_program(const AxhipRowsProgram &P, const char *who) {
     AXHIP_REQUIRE(P.rows >= 0 && P.cols >= 0, AXHIP_ERR_INVALID_ARG, "%s: negative extent", who);
-    AXHIP_REQUIRE(valid_dtype(P.input_dtype) && valid_dtype(P.output_dtype), AXHIP_ERR_INVALID_ARG, "%s: bad dtype", who);
+    AXHIP_REQUIRE(valid_dtype_or_u8(P.input_dtype) && valid_dtype_or_u8(P.output_dtype), AXHIP_ERR_INVALID_ARG, "%s: bad dtype", who);
     AXHIP_REQUIRE(P.n_operands >= 0 && P.n_operands <= AXHIP_MAX_OPERANDS, AXHIP_ERR_INVALID_ARG, "%s: bad operand count %d", who, P.n_operands);
     for (int i = 0; i < P.n_operands; ++i) {
         AXHIP_REQUIRE(P.operands[i].ptr != nullptr, AXHIP_ERR_INVALID_ARG, "%s: operand %d is NULL", who, i);
-        AXHIP_REQUIRE(valid_dtype(P.operands[i].dtype), AXHIP_ERR_INVALID_ARG, "%s: operand %d has bad dtype", who, i);
+        AXHIP_REQUIRE(valid_dtype_or_u8(P.operands[i].dtype), AXHIP_ERR_INVALID_ARG, "%s: operand %d has bad dtype", who, i);
         AXHIP_REQUIRE(P.operands[i].kind >= AXHIP_BK_FULL && P.operands[i].kind <= AXHIP_BK_SCALAR, AXHIP_ERR_INVALID_ARG, "%s: operand %d has bad kind", who, i);
     }
     int rc = validate_chain(P.pre, P.n_pre, P, "pre");
@@ -574,7 +585,7 @@ int validate_program(const AxhipRowsProgram &P, const char *who) {
     rc = validate_chain(P.post, P.n_post, P, "post");
     if (rc) return rc;
     AXHIP_REQUIRE(P.row_op >= AXHIP_ROWOP_NONE && P.row_op <= AXHIP_ROWOP_RMSNORM, AXHIP_ERR_INVALID_ARG, "%s: bad row_op %d", who, P.row_op);
-    AXHIP_REQUIRE(P.reduce >= AXHIP_RED_NONE && P.reduce <= AXHIP_RED_MIN, AXHIP_ERR_INVALID_ARG, "%s: bad reduce %d", who, P.reduce);
+    AXHIP_REQUIRE(P.reduce >= AXHIP_RED_NONE && P.reduce <= AXHIP_RED_PROD, AXHIP_ERR_INVALID_ARG, "%s: bad reduce %d", who, P.reduce);
     for (int idx : {P.norm_weight, P.norm_bias})
         if (idx >= 0) {
             AXHIP_REQUIRE(idx < P.n_operands && P.operands[idx].kind == AXHIP_BK_ROWVEC, AXHIP_ERR_INVALID_ARG, "%s: norm weight/bias must be a ROWVEC operand", who);

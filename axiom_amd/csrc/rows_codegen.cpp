@@ -14,8 +14,8 @@ namespace {
 int elem_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 const char *dt_name(int dt) { return dt == AXHIP_DTYPE_F32 ? "f32" : dt == AXHIP_DTYPE_F16 ? "f16" : "bf16"; }
-bool is_unary(int op) { return op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP; }
-bool is_binary(int op) { return op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV; }
+bool is_unary(int op) { return (op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP) || (op >= AXHIP_OP_ERF && op <= AXHIP_OP_NOT); }
+bool is_binary(int op) { return (op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV) || (op >= AXHIP_OP_POW && op <= AXHIP_OP_LEAKY_RELU); }
 
 const char *op_token(int op) {
     switch (op) {
@@ -40,6 +40,37 @@ const char *op_token(int op) {
     case AXHIP_OP_SQUARE: return "square";
     case AXHIP_OP_RSQRT: return "rsqrt";
     case AXHIP_OP_RECIP: return "recip";
+    case AXHIP_OP_POW: return "pow";
+    case AXHIP_OP_RPOW: return "rpow";
+    case AXHIP_OP_MOD: return "mod";
+    case AXHIP_OP_RMOD: return "rmod";
+    case AXHIP_OP_ATAN2: return "atan2";
+    case AXHIP_OP_RATAN2: return "ratan2";
+    case AXHIP_OP_HYPOT: return "hypot";
+    case AXHIP_OP_EQ: return "eq";
+    case AXHIP_OP_NE: return "ne";
+    case AXHIP_OP_LT: return "lt";
+    case AXHIP_OP_LE: return "le";
+    case AXHIP_OP_GT: return "gt";
+    case AXHIP_OP_GE: return "ge";
+    case AXHIP_OP_AND: return "and";
+    case AXHIP_OP_OR: return "or";
+    case AXHIP_OP_XOR: return "xor";
+    case AXHIP_OP_LEAKY_RELU: return "leaky";
+    case AXHIP_OP_ERF: return "erf";
+    case AXHIP_OP_SIN: return "sin";
+    case AXHIP_OP_COS: return "cos";
+    case AXHIP_OP_TAN: return "tan";
+    case AXHIP_OP_SIGN: return "sign";
+    case AXHIP_OP_FLOOR: return "floor";
+    case AXHIP_OP_CEIL: return "ceil";
+    case AXHIP_OP_ROUND: return "round";
+    case AXHIP_OP_TRUNC: return "trunc";
+    case AXHIP_OP_CBRT: return "cbrt";
+    case AXHIP_OP_ISNAN: return "isnan";
+    case AXHIP_OP_ISINF: return "isinf";
+    case AXHIP_OP_ISFINITE: return "isfinite";
+    case AXHIP_OP_NOT: return "not";
     default: return nullptr;
     }
 }
@@ -172,7 +203,24 @@ struct Builder {
                 case AXHIP_OP_MAX: o << "    t = fmaxf(t, " << b << ");\n"; break;
                 case AXHIP_OP_MIN: o << "    t = fminf(t, " << b << ");\n"; break;
                 case AXHIP_OP_RSUB: o << "    t = " << b << " - t;\n"; break;
-                default: o << "    t = " << b << " / t;\n"; break;
+                case AXHIP_OP_RDIV: o << "    t = " << b << " / t;\n"; break;
+                case AXHIP_OP_POW: o << "    t = powf(t, " << b << ");\n"; break;
+                case AXHIP_OP_RPOW: o << "    t = powf(" << b << ", t);\n"; break;
+                case AXHIP_OP_MOD: o << "    t = fmodf(t, " << b << ");\n"; break;
+                case AXHIP_OP_RMOD: o << "    t = fmodf(" << b << ", t);\n"; break;
+                case AXHIP_OP_ATAN2: o << "    t = atan2f(t, " << b << ");\n"; break;
+                case AXHIP_OP_RATAN2: o << "    t = atan2f(" << b << ", t);\n"; break;
+                case AXHIP_OP_HYPOT: o << "    t = hypotf(t, " << b << ");\n"; break;
+                case AXHIP_OP_EQ: o << "    t = t == " << b << " ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_NE: o << "    t = t != " << b << " ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_LT: o << "    t = t < " << b << " ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_LE: o << "    t = t <= " << b << " ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_GT: o << "    t = t > " << b << " ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_GE: o << "    t = t >= " << b << " ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_AND: o << "    t = (t != 0.0f) && (" << b << " != 0.0f) ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_OR: o << "    t = (t != 0.0f) || (" << b << " != 0.0f) ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_XOR: o << "    t = (t != 0.0f) != (" << b << " != 0.0f) ? 1.0f : 0.0f;\n"; break;
+                default: o << "    t = t > 0.0f ? t : " << b << " * t;\n"; break; // leaky ReLU
                 }
             } else if (is_unary(op)) {
                 switch (op) {
@@ -188,7 +236,21 @@ struct Builder {
                 case AXHIP_OP_LOG: o << "    t = logf(t);\n"; break;
                 case AXHIP_OP_SQUARE: o << "    t = t * t;\n"; break;
                 case AXHIP_OP_RSQRT: o << "    t = 1.0f / sqrtf(t);\n"; break;
-                default: o << "    t = 1.0f / t;\n"; break;
+                case AXHIP_OP_RECIP: o << "    t = 1.0f / t;\n"; break;
+                case AXHIP_OP_ERF: o << "    t = erff(t);\n"; break;
+                case AXHIP_OP_SIN: o << "    t = sinf(t);\n"; break;
+                case AXHIP_OP_COS: o << "    t = cosf(t);\n"; break;
+                case AXHIP_OP_TAN: o << "    t = tanf(t);\n"; break;
+                case AXHIP_OP_SIGN: o << "    t = t > 0.0f ? 1.0f : t < 0.0f ? -1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_FLOOR: o << "    t = floorf(t);\n"; break;
+                case AXHIP_OP_CEIL: o << "    t = ceilf(t);\n"; break;
+                case AXHIP_OP_ROUND: o << "    t = roundf(t);\n"; break;
+                case AXHIP_OP_TRUNC: o << "    t = truncf(t);\n"; break;
+                case AXHIP_OP_CBRT: o << "    t = cbrtf(t);\n"; break;
+                case AXHIP_OP_ISNAN: o << "    t = t != t ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_ISINF: o << "    t = fabsf(t) == __builtin_huge_valf() ? 1.0f : 0.0f;\n"; break;
+                case AXHIP_OP_ISFINITE: o << "    t = fabsf(t) < __builtin_huge_valf() ? 1.0f : 0.0f;\n"; break;
+                default: o << "    t = t == 0.0f ? 1.0f : 0.0f;\n"; break; // logical not
                 }
             } else {
                 ok = false;
@@ -308,6 +370,11 @@ bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, Ro
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     if (P.cols <= 0) return false;
     if (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE) return false; // flat elementwise chains have a kernel of their own
+    // products and one-byte streams (a Bool input, operand or full-size result) stay with the interpreter; a reduced
+    // [rows] result may be a byte (any / all)
+    if (P.reduce > AXHIP_RED_MIN || P.input_dtype == AXHIP_DTYPE_U8 || (P.reduce == AXHIP_RED_NONE && P.output_dtype == AXHIP_DTYPE_U8)) return false;
+    for (int i = 0; i < P.n_operands; ++i)
+        if (P.operands[i].dtype == AXHIP_DTYPE_U8) return false;
     const int dt = P.input_dtype;
     const int e = rows_prog_chunk_elems(P);
     bool ragged = P.cols % e != 0 || !aligned16(P.input) || (P.reduce == AXHIP_RED_NONE && !aligned16(P.output));

@@ -10,6 +10,48 @@ namespace axhip {
 constexpr float NEG_INF = -__builtin_huge_valf();
 constexpr float POS_INF = __builtin_huge_valf();
 
+// The wider operator table (codes from AXHIP_OP_POW up) as ONE function that the chain interpreters call per value:
+// inlined into every arm of every interpreter kernel, its 32 operations (powf, fmodf, the trigonometric routines ...)
+// multiplied the build time and the code size of this file by five.  The call is made once per wavefront for 64
+// values and the switch inside is a scalar branch: far below the cost of the memory accesses around it.  The
+// compiled row programs have these operations inline.
+__device__ __attribute__((noinline)) inline float extended_op(int op, float a, float b) {
+    switch (op) {
+    case AXHIP_OP_POW: return powf(a, b);
+    case AXHIP_OP_RPOW: return powf(b, a);
+    case AXHIP_OP_MOD: return fmodf(a, b);
+    case AXHIP_OP_RMOD: return fmodf(b, a);
+    case AXHIP_OP_ATAN2: return atan2f(a, b);
+    case AXHIP_OP_RATAN2: return atan2f(b, a);
+    case AXHIP_OP_HYPOT: return hypotf(a, b);
+    case AXHIP_OP_EQ: return a == b ? 1.0f : 0.0f;
+    case AXHIP_OP_NE: return a != b ? 1.0f : 0.0f;
+    case AXHIP_OP_LT: return a < b ? 1.0f : 0.0f;
+    case AXHIP_OP_LE: return a <= b ? 1.0f : 0.0f;
+    case AXHIP_OP_GT: return a > b ? 1.0f : 0.0f;
+    case AXHIP_OP_GE: return a >= b ? 1.0f : 0.0f;
+    case AXHIP_OP_AND: return (a != 0.0f) && (b != 0.0f) ? 1.0f : 0.0f;
+    case AXHIP_OP_OR: return (a != 0.0f) || (b != 0.0f) ? 1.0f : 0.0f;
+    case AXHIP_OP_XOR: return (a != 0.0f) != (b != 0.0f) ? 1.0f : 0.0f;
+    case AXHIP_OP_LEAKY_RELU: return a > 0.0f ? a : b * a;
+    case AXHIP_OP_ERF: return erff(a);
+    case AXHIP_OP_SIN: return sinf(a);
+    case AXHIP_OP_COS: return cosf(a);
+    case AXHIP_OP_TAN: return tanf(a);
+    case AXHIP_OP_SIGN: return a > 0.0f ? 1.0f : a < 0.0f ? -1.0f : 0.0f;
+    case AXHIP_OP_FLOOR: return floorf(a);
+    case AXHIP_OP_CEIL: return ceilf(a);
+    case AXHIP_OP_ROUND: return roundf(a);
+    case AXHIP_OP_TRUNC: return truncf(a);
+    case AXHIP_OP_CBRT: return cbrtf(a);
+    case AXHIP_OP_ISNAN: return a != a ? 1.0f : 0.0f;
+    case AXHIP_OP_ISINF: return fabsf(a) == POS_INF ? 1.0f : 0.0f;
+    case AXHIP_OP_ISFINITE: return fabsf(a) < POS_INF ? 1.0f : 0.0f;
+    case AXHIP_OP_NOT: return a == 0.0f ? 1.0f : 0.0f;
+    default: return a;
+    }
+}
+
 __device__ __forceinline__ float apply_unary(int op, float a) {
     switch (op) {
     case AXHIP_OP_RELU: return a > 0.0f ? a : 0.0f;
@@ -28,7 +70,7 @@ __device__ __forceinline__ float apply_unary(int op, float a) {
     case AXHIP_OP_SQUARE: return a * a;
     case AXHIP_OP_RSQRT: return 1.0f / sqrtf(a);
     case AXHIP_OP_RECIP: return 1.0f / a;
-    default: return a;
+    default: return op >= AXHIP_OP_POW ? extended_op(op, a, 0.0f) : a;
     }
 }
 
@@ -42,11 +84,16 @@ __device__ __forceinline__ float apply_binary(int op, float a, float b) {
     case AXHIP_OP_MIN: return fminf(a, b);
     case AXHIP_OP_RSUB: return b - a;
     case AXHIP_OP_RDIV: return b / a;
-    default: return a;
+    default: return op >= AXHIP_OP_POW ? extended_op(op, a, b) : a;
     }
 }
 
-__host__ __device__ inline bool is_binary_op(int op) { return op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV; }
+__host__ __device__ inline bool is_binary_op(int op) {
+    return (op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV) || (op >= AXHIP_OP_POW && op <= AXHIP_OP_LEAKY_RELU);
+}
+__host__ __device__ inline bool is_unary_op(int op) {
+    return (op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP) || (op >= AXHIP_OP_ERF && op <= AXHIP_OP_NOT);
+}
 
 // Apply one chain op to a thread's register tile.  The op code is a kernel
 // argument, so the switch is a scalar (wave-uniform) branch taken once per op;
@@ -94,7 +141,9 @@ __device__ __forceinline__ void apply_unary_tile(int op, float (&v)[IT][E]) {
         AXHIP_UNARY_CASE(AXHIP_OP_SQUARE);
         AXHIP_UNARY_LONG(AXHIP_OP_RSQRT);
         AXHIP_UNARY_LONG(AXHIP_OP_RECIP);
-    default: break;
+    default:
+        if (op >= AXHIP_OP_ERF) for_each_value<IT, E>(v, [op](float a, int, int) { return extended_op(op, a, 0.0f); });
+        break;
     }
 #undef AXHIP_UNARY_CASE
 #undef AXHIP_UNARY_LONG
@@ -116,7 +165,9 @@ __device__ __forceinline__ void apply_binary_tile(int op, float (&v)[IT][E], W w
         AXHIP_BINARY_CASE(AXHIP_OP_MIN);
         AXHIP_BINARY_CASE(AXHIP_OP_RSUB);
         AXHIP_BINARY_LONG(AXHIP_OP_RDIV);
-    default: break;
+    default:
+        if (op >= AXHIP_OP_POW) for_each_value<IT, E>(v, [&](float a, int it, int e) { return extended_op(op, a, w(it, e)); });
+        break;
     }
 #undef AXHIP_BINARY_CASE
 #undef AXHIP_BINARY_LONG

@@ -30,6 +30,8 @@ class GraphRegistry {
   public:
     static Tensor create_lazy_unary(ops::OpType op, const Tensor &input, const OpParams &params = NoParams{});
     static Tensor create_lazy_binary(ops::OpType op, const Tensor &lhs, const Tensor &rhs, const OpParams &params = NoParams{});
+    static Tensor create_lazy_where(const Tensor &condition, const Tensor &a, const Tensor &b);
+    static Tensor create_lazy_cast(const Tensor &input, DType target);
     static Tensor create_lazy_reduction(ops::OpType op, const Tensor &input, const std::vector<int> &axes, bool keep_dims);
     static Tensor create_lazy_matmul(const Tensor &a, const Tensor &b, bool transpose_a, bool transpose_b);
     static Tensor create_lazy_softmax(ops::OpType op, const Tensor &input, int axis);

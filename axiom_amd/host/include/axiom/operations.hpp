@@ -91,6 +91,23 @@ Tensor multiply(const Tensor &a, const Tensor &b);
 Tensor divide(const Tensor &a, const Tensor &b);
 Tensor maximum(const Tensor &a, const Tensor &b);
 Tensor minimum(const Tensor &a, const Tensor &b);
+// include/axiom/operations.hpp:313-341.  power / modulo follow the CPU functors (std::pow; std::fmod, the sign of the
+// dividend: src/backends/cpu/cpu_operations.hpp:214-235); comparisons and logical operations give Bool tensors, a
+// logical operation reads any nonzero element as true
+Tensor power(const Tensor &a, const Tensor &b);
+Tensor modulo(const Tensor &a, const Tensor &b);
+Tensor atan2(const Tensor &a, const Tensor &b);
+Tensor hypot(const Tensor &a, const Tensor &b);
+Tensor equal(const Tensor &a, const Tensor &b);
+Tensor not_equal(const Tensor &a, const Tensor &b);
+Tensor less(const Tensor &a, const Tensor &b);
+Tensor less_equal(const Tensor &a, const Tensor &b);
+Tensor greater(const Tensor &a, const Tensor &b);
+Tensor greater_equal(const Tensor &a, const Tensor &b);
+Tensor logical_and(const Tensor &a, const Tensor &b);
+Tensor logical_or(const Tensor &a, const Tensor &b);
+Tensor logical_xor(const Tensor &a, const Tensor &b);
+Tensor logical_not(const Tensor &x);
 
 Tensor negate(const Tensor &x);
 Tensor abs(const Tensor &x);
@@ -104,6 +121,29 @@ Tensor silu(const Tensor &x);
 Tensor sigmoid(const Tensor &x);
 Tensor tanh(const Tensor &x);
 Tensor gelu(const Tensor &x);
+// include/axiom/operations.hpp:349-380.  sign(NaN) is 0, round moves halves away from zero (std::round), the is* tests
+// give Bool tensors (src/backends/cpu/cpu_operations.hpp:724-860); round with decimals != 0 is round(x 10^d) / 10^d
+// (src/tensor/operations.cpp:1330-1341); clip is maximum(minimum(x, hi), lo) (:1369-1371)
+Tensor sin(const Tensor &x);
+Tensor cos(const Tensor &x);
+Tensor tan(const Tensor &x);
+Tensor erf(const Tensor &x);
+Tensor sign(const Tensor &x);
+Tensor floor(const Tensor &x);
+Tensor ceil(const Tensor &x);
+Tensor trunc(const Tensor &x);
+Tensor round(const Tensor &x, int decimals = 0);
+Tensor cbrt(const Tensor &x);
+Tensor isnan(const Tensor &x);
+Tensor isinf(const Tensor &x);
+Tensor isfinite(const Tensor &x);
+Tensor clip(const Tensor &x, const Tensor &min_val, const Tensor &max_val);
+Tensor leaky_relu(const Tensor &x, float negative_slope = 0.01f);
+// numpy.where(condition, a, b): the three broadcast together, the result has promote_types(a, b)
+// (include/axiom/operations.hpp:425-429).  A lazy node here; the reference runs it when called.
+Tensor where(const Tensor &condition, const Tensor &a, const Tensor &b);
+// the GPU Cast (src/tensor/tensor.cpp:1665-1670) as a lazy node among Float32, Float16, BFloat16 and Bool
+Tensor cast(const Tensor &x, DType target);
 
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor log_softmax(const Tensor &x, int axis = -1);
@@ -112,6 +152,11 @@ Tensor sum(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = 
 Tensor mean(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
 Tensor max(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
 Tensor min(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+// include/axiom/operations.hpp:403-411: any / all give Bool tensors (an element counts when it is nonzero); they
+// are built as max / min over not_equal(x, 0), which fuses into one kernel
+Tensor any(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+Tensor all(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
+Tensor prod(const Tensor &x, const std::vector<int> &axes = {}, bool keep_dims = false);
 // Int64 index of the first occurrence of the extreme along one axis (include/axiom/operations.hpp:400-401); runs when
 // called, like scaled_dot_product_attention, on the materialised input
 Tensor argmax(const Tensor &x, int axis = -1, bool keep_dims = false);

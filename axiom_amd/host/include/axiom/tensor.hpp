@@ -118,6 +118,26 @@ class Tensor {
     Tensor silu() const;
     Tensor tanh() const;
     Tensor glu(int dim = -1) const;
+    // the NumPy-style members of include/axiom/tensor.hpp:330-437
+    Tensor leaky_relu(float negative_slope = 0.01f) const;
+    Tensor sign() const;
+    Tensor floor() const;
+    Tensor ceil() const;
+    Tensor trunc() const;
+    Tensor round(int decimals = 0) const;
+    Tensor cbrt() const;
+    Tensor isnan() const;
+    Tensor isinf() const;
+    Tensor isfinite() const;
+    Tensor clip(double min_val, double max_val) const;
+    Tensor where(const Tensor &condition, const Tensor &other) const; // condition ? *this : other
+    Tensor prod(int axis = -1, bool keep_dims = false) const;
+    Tensor prod(const std::vector<int> &axes, bool keep_dims = false) const;
+    Tensor any(int axis = -1, bool keep_dims = false) const;
+    Tensor any(const std::vector<int> &axes, bool keep_dims = false) const;
+    Tensor all(int axis = -1, bool keep_dims = false) const;
+    Tensor all(const std::vector<int> &axes, bool keep_dims = false) const;
+    Tensor to_bool() const { return astype(DType::Bool); }
     Tensor masked_fill(const Tensor &mask, float value) const;
     Tensor masked_fill(const Tensor &mask, double value) const;
     Tensor matmul(const Tensor &other, bool transpose_self = false, bool transpose_other = false) const;
@@ -170,6 +190,23 @@ Tensor operator-(const Tensor &a, const Tensor &b);
 Tensor operator*(const Tensor &a, const Tensor &b);
 Tensor operator/(const Tensor &a, const Tensor &b);
 Tensor make_scalar_like(const Tensor &t, double value);
+// comparisons give Bool tensors (include/axiom/tensor_operators.hpp)
+Tensor operator<(const Tensor &a, const Tensor &b);
+Tensor operator<=(const Tensor &a, const Tensor &b);
+Tensor operator>(const Tensor &a, const Tensor &b);
+Tensor operator>=(const Tensor &a, const Tensor &b);
+Tensor operator==(const Tensor &a, const Tensor &b);
+Tensor operator!=(const Tensor &a, const Tensor &b);
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator<(const Tensor &a, S s) { return a < make_scalar_like(a, static_cast<double>(s)); }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator<=(const Tensor &a, S s) { return a <= make_scalar_like(a, static_cast<double>(s)); }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator>(const Tensor &a, S s) { return a > make_scalar_like(a, static_cast<double>(s)); }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator>=(const Tensor &a, S s) { return a >= make_scalar_like(a, static_cast<double>(s)); }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator==(const Tensor &a, S s) { return a == make_scalar_like(a, static_cast<double>(s)); }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator!=(const Tensor &a, S s) { return a != make_scalar_like(a, static_cast<double>(s)); }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator<(S s, const Tensor &a) { return make_scalar_like(a, static_cast<double>(s)) < a; }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator<=(S s, const Tensor &a) { return make_scalar_like(a, static_cast<double>(s)) <= a; }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator>(S s, const Tensor &a) { return make_scalar_like(a, static_cast<double>(s)) > a; }
+template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator>=(S s, const Tensor &a) { return make_scalar_like(a, static_cast<double>(s)) >= a; }
 template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator+(const Tensor &a, S s) { return a + make_scalar_like(a, static_cast<double>(s)); }
 template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator-(const Tensor &a, S s) { return a - make_scalar_like(a, static_cast<double>(s)); }
 template <typename S, typename = std::enable_if_t<std::is_arithmetic_v<S>>> Tensor operator*(const Tensor &a, S s) { return a * make_scalar_like(a, static_cast<double>(s)); }

@@ -80,6 +80,11 @@ struct GatherStep {
     int table = -1, indices = -1, dst = -1;
 };
 
+struct WhereStep { // dst = cond ? a : b over dst's shape; strides in bytes, 0 on broadcast dims
+    int cond = -1, a = -1, b = -1, dst = -1;
+    Strides cond_strides, a_strides, b_strides;
+};
+
 struct AxisReduceStep { // a reduction, or a softmax, along the middle extent of a contiguous (outer, axis, inner) value
     int src = -1, dst = -1;
     int64_t outer = 1, axis = 1, inner = 1;
@@ -87,7 +92,7 @@ struct AxisReduceStep { // a reduction, or a softmax, along the middle extent of
 };
 
 struct Step {
-    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER, AXIS_REDUCE, AXIS_SOFTMAX } kind;
+    enum Kind { ROWS, GEMM, COPY, PAD, MASKED_FILL, GATHER, AXIS_REDUCE, AXIS_SOFTMAX, WHERE } kind;
     RowsStep rows;
     GemmStep gemm;
     CopyStep copy;
@@ -95,6 +100,7 @@ struct Step {
     MaskedFillStep mfill;
     GatherStep gather;
     AxisReduceStep axred;
+    WhereStep where;
 };
 
 struct Plan {
@@ -114,17 +120,38 @@ bool is_unary_ew(OpType op) {
     switch (op) {
     case OpType::Negate: case OpType::Abs: case OpType::Sqrt: case OpType::Exp: case OpType::Log: case OpType::Reciprocal:
     case OpType::Square: case OpType::ReLU: case OpType::SiLU: case OpType::Sigmoid: case OpType::Tanh: case OpType::GELU:
+    case OpType::Sin: case OpType::Cos: case OpType::Tan: case OpType::Erf: case OpType::Sign: case OpType::Floor: case OpType::Ceil:
+    case OpType::Trunc: case OpType::Round: case OpType::Cbrt: case OpType::IsNaN: case OpType::IsInf: case OpType::IsFinite:
+    case OpType::LogicalNot: case OpType::LeakyReLU: case OpType::Cast:
         return true;
     default: return false;
     }
 }
 bool is_binary_ew(OpType op) {
-    return op == OpType::Add || op == OpType::Subtract || op == OpType::Multiply || op == OpType::Divide || op == OpType::Maximum ||
-           op == OpType::Minimum;
+    switch (op) {
+    case OpType::Add: case OpType::Subtract: case OpType::Multiply: case OpType::Divide: case OpType::Maximum: case OpType::Minimum:
+    case OpType::Power: case OpType::Modulo: case OpType::Atan2: case OpType::Hypot: case OpType::Equal: case OpType::NotEqual:
+    case OpType::Less: case OpType::LessEqual: case OpType::Greater: case OpType::GreaterEqual: case OpType::LogicalAnd:
+    case OpType::LogicalOr: case OpType::LogicalXor:
+        return true;
+    default: return false;
+    }
 }
 bool is_elementwise(OpType op) { return is_unary_ew(op) || is_binary_ew(op); }
 bool is_row_op(OpType op) { return op == OpType::Softmax || op == OpType::LogSoftmax || op == OpType::LayerNorm || op == OpType::RMSNorm; }
-bool is_reduction(OpType op) { return op == OpType::Sum || op == OpType::Mean || op == OpType::Max || op == OpType::Min; }
+bool is_reduction(OpType op) { return op == OpType::Sum || op == OpType::Mean || op == OpType::Max || op == OpType::Min || op == OpType::Prod; }
+int reduce_code(OpType op) {
+    return op == OpType::Sum ? AXHIP_RED_SUM : op == OpType::Mean ? AXHIP_RED_MEAN : op == OpType::Max ? AXHIP_RED_MAX : op == OpType::Min ? AXHIP_RED_MIN : AXHIP_RED_PROD;
+}
+// a Cast that loses precision in the middle of a chain would need a rounding step of its own: such a node ends the
+// chain below it (on top of a chain it is the kernel's output type).  Widening casts and casts from Bool change no
+// value; a cast to Bool is "!= 0".
+bool narrowing_cast(const GraphNode *n) {
+    if (n->op_type != OpType::Cast) return false;
+    const DType from = n->inputs[0]->output_dtype, to = n->output_dtype;
+    if (to == DType::Bool || from == DType::Bool || from == to) return false;
+    return !(to == DType::Float32);
+}
 
 int unary_code(OpType op) {
     switch (op) {
@@ -140,6 +167,20 @@ int unary_code(OpType op) {
     case OpType::Sigmoid: return AXHIP_OP_SIGMOID;
     case OpType::Tanh: return AXHIP_OP_TANH;
     case OpType::GELU: return AXHIP_OP_GELU;
+    case OpType::Sin: return AXHIP_OP_SIN;
+    case OpType::Cos: return AXHIP_OP_COS;
+    case OpType::Tan: return AXHIP_OP_TAN;
+    case OpType::Erf: return AXHIP_OP_ERF;
+    case OpType::Sign: return AXHIP_OP_SIGN;
+    case OpType::Floor: return AXHIP_OP_FLOOR;
+    case OpType::Ceil: return AXHIP_OP_CEIL;
+    case OpType::Trunc: return AXHIP_OP_TRUNC;
+    case OpType::Round: return AXHIP_OP_ROUND;
+    case OpType::Cbrt: return AXHIP_OP_CBRT;
+    case OpType::IsNaN: return AXHIP_OP_ISNAN;
+    case OpType::IsInf: return AXHIP_OP_ISINF;
+    case OpType::IsFinite: return AXHIP_OP_ISFINITE;
+    case OpType::LogicalNot: return AXHIP_OP_NOT;
     default: return 0;
     }
 }
@@ -152,6 +193,19 @@ int binary_code(OpType op, bool chain_is_rhs) {
     case OpType::Minimum: return AXHIP_OP_MIN;
     case OpType::Subtract: return chain_is_rhs ? AXHIP_OP_RSUB : AXHIP_OP_SUB;
     case OpType::Divide: return chain_is_rhs ? AXHIP_OP_RDIV : AXHIP_OP_DIV;
+    case OpType::Power: return chain_is_rhs ? AXHIP_OP_RPOW : AXHIP_OP_POW;
+    case OpType::Modulo: return chain_is_rhs ? AXHIP_OP_RMOD : AXHIP_OP_MOD;
+    case OpType::Atan2: return chain_is_rhs ? AXHIP_OP_RATAN2 : AXHIP_OP_ATAN2;
+    case OpType::Hypot: return AXHIP_OP_HYPOT;
+    case OpType::Equal: return AXHIP_OP_EQ;
+    case OpType::NotEqual: return AXHIP_OP_NE;
+    case OpType::Less: return chain_is_rhs ? AXHIP_OP_GT : AXHIP_OP_LT; // a < v  <=>  v > a
+    case OpType::LessEqual: return chain_is_rhs ? AXHIP_OP_GE : AXHIP_OP_LE;
+    case OpType::Greater: return chain_is_rhs ? AXHIP_OP_LT : AXHIP_OP_GT;
+    case OpType::GreaterEqual: return chain_is_rhs ? AXHIP_OP_LE : AXHIP_OP_GE;
+    case OpType::LogicalAnd: return AXHIP_OP_AND;
+    case OpType::LogicalOr: return AXHIP_OP_OR;
+    case OpType::LogicalXor: return AXHIP_OP_XOR;
     default: return 0;
     }
 }
@@ -229,7 +283,7 @@ class PlanBuilder {
     int make_contiguous(int v, const Shape *to = nullptr) {
         const Shape target = to ? *to : val(v).shape;
         if (target == val(v).shape && contiguous(v)) return v;
-        detail::to_axhip_dtype(val(v).dtype); // only kernel dtypes can be gathered on the device
+        detail::to_axhip_dtype_or_bool(val(v).dtype); // only kernel dtypes can be gathered on the device
         const ValueSpec src = val(v);
         const int out = new_temp(target, src.dtype);
         Step s{};
@@ -280,6 +334,14 @@ class PlanBuilder {
         const int axis = n->op_type == OpType::Softmax || n->op_type == OpType::LogSoftmax ? get_params<ActivationParams>(n->params).axis
                                                                                            : get_params<NormParams>(n->params).axis;
         return nd == 0 || ShapeUtils::normalize_axis(axis, nd) == nd - 1;
+    }
+
+    // is the input of this Cast node a view (of a leaf or of a computed value) that is not contiguous
+    bool strided_view_below(const GraphNode *n) {
+        const GraphNode *in = n->inputs[0].get();
+        const bool view = is_leaf(in, root_) || in->op_type == OpType::Transpose || in->op_type == OpType::Slice || in->op_type == OpType::Reshape ||
+                          memo_.count(in) > 0;
+        return view && !contiguous(eval(in));
     }
 
     bool consumable(const GraphNode *c, const GraphNode *entry) const {
@@ -368,6 +430,34 @@ class PlanBuilder {
             const size_t lead = F.size() - M.size();
             for (size_t i = 0; i < M.size(); ++i) st.mfill.mask_strides[lead + i] = M[i] == 1 ? 0 : mask_strides[i];
             plan_.steps.push_back(st);
+        } else if (op == OpType::Where) {
+            if (n->inputs.size() < 3) throw RuntimeError("malformed graph node 'where': missing inputs");
+            const int c = eval(n->inputs[0].get()), a = eval(n->inputs[1].get()), b = eval(n->inputs[2].get());
+            const Shape F = n->output_shape;
+            if (F.size() > AXHIP_MAX_DIMS) throw RuntimeError::not_implemented("GPU where of more than 8 dimensions");
+            Step st{};
+            st.kind = Step::WHERE;
+            st.where.cond = c;
+            st.where.a = a;
+            st.where.b = b;
+            auto broadcast_strides = [&](int v) {
+                detail::to_axhip_dtype_or_bool(val(v).dtype);
+                const Shape S = val(v).shape;
+                const Strides in = val(v).strides;
+                Strides out(F.size(), 0);
+                const size_t lead = F.size() - S.size();
+                for (size_t i = 0; i < S.size(); ++i) {
+                    if (in[i] < 0) throw RuntimeError::not_implemented("negative strides (flipped views)");
+                    out[lead + i] = S[i] == 1 ? 0 : in[i];
+                }
+                return out;
+            };
+            st.where.cond_strides = broadcast_strides(c);
+            st.where.a_strides = broadcast_strides(a);
+            st.where.b_strides = broadcast_strides(b);
+            st.where.dst = v = new_temp(F, n->output_dtype);
+            detail::to_axhip_dtype_or_bool(n->output_dtype);
+            plan_.steps.push_back(st);
         } else if (op == OpType::Gather) { // embedding rows
             if (n->inputs.size() < 2) throw RuntimeError("malformed graph node 'embedding': missing inputs");
             const int table = make_contiguous(eval(n->inputs[0].get())), idx = eval(n->inputs[1].get());
@@ -390,8 +480,8 @@ class PlanBuilder {
             st.axred.outer = outer;
             st.axred.axis = axis;
             st.axred.inner = inner;
-            st.axred.reduce = op == OpType::Sum ? AXHIP_RED_SUM : op == OpType::Mean ? AXHIP_RED_MEAN : op == OpType::Max ? AXHIP_RED_MAX : AXHIP_RED_MIN;
-            detail::to_axhip_dtype(val(st.axred.src).dtype);
+            st.axred.reduce = reduce_code(op);
+            detail::to_axhip_dtype_or_bool(val(st.axred.src).dtype);
             st.axred.dst = v = new_temp(n->output_shape, n->output_dtype);
             plan_.steps.push_back(st);
         } else if ((op == OpType::Softmax || op == OpType::LogSoftmax) && !row_axis_is_last(n)) {
@@ -406,6 +496,24 @@ class PlanBuilder {
             st.axred.reduce = op == OpType::LogSoftmax ? 1 : 0;
             detail::to_axhip_dtype(val(st.axred.src).dtype);
             st.axred.dst = v = new_temp(F, n->output_dtype);
+            plan_.steps.push_back(st);
+        } else if (op == OpType::Cast && strided_view_below(n)) {
+            // a cast of a strided view: the gather converts on its way, one pass instead of a gather and a cast
+            const int in = eval(n->inputs[0].get());
+            const ValueSpec src = val(in);
+            detail::to_axhip_dtype_or_bool(src.dtype);
+            detail::to_axhip_dtype_or_bool(n->output_dtype);
+            if (src.shape.size() > AXHIP_MAX_DIMS) throw RuntimeError::not_implemented("GPU gather of more than 8 dimensions");
+            Step st{};
+            st.kind = Step::COPY;
+            st.copy.src = in;
+            st.copy.dst = v = new_temp(src.shape, n->output_dtype);
+            st.copy.shape = src.shape;
+            st.copy.src_strides = src.strides;
+            for (size_t i = 0; i < src.shape.size(); ++i)
+                if (src.shape[i] == 1) st.copy.src_strides[i] = 0;
+            for (int64_t sd : st.copy.src_strides)
+                if (sd < 0) throw RuntimeError::not_implemented("negative strides (flipped views)");
             plan_.steps.push_back(st);
         } else if (is_elementwise(op) || is_row_op(op) || is_reduction(op)) {
             v = emit_rows(n);
@@ -425,6 +533,7 @@ class PlanBuilder {
     // Collects elementwise nodes downwards from `c` while each is consumable and keeps the full shape F.
     void collect(const GraphNode *&c, const GraphNode *entry, const Shape &F, std::vector<ChainItem> &list, size_t limit, size_t &operands) {
         while (consumable(c, entry) && is_elementwise(c->op_type) && c->output_shape == F && list.size() < limit) {
+            if (!list.empty() && narrowing_cast(c)) break; // rounds in mid-chain: a kernel of its own below this one
             int primary = 0;
             if (is_binary_ew(c->op_type)) {
                 if (c->inputs.size() < 2) throw RuntimeError(std::string("malformed graph node '") + ops::op_name(c->op_type) + "': missing inputs");
@@ -465,7 +574,7 @@ class PlanBuilder {
         }
         v = make_contiguous(v);
         const int slot = rs.prog.n_operands++;
-        rs.prog.operands[slot].dtype = detail::to_axhip_dtype(val(v).dtype);
+        rs.prog.operands[slot].dtype = detail::to_axhip_dtype_or_bool(val(v).dtype);
         rs.prog.operands[slot].kind = kind;
         rs.operand_value[slot] = v;
         cop.op = binary_code(op, chain_is_rhs);
@@ -477,7 +586,21 @@ class PlanBuilder {
     void fill_chain(RowsStep &rs, const std::vector<ChainItem> &bottom_up, AxhipChainOp *dst, int32_t &count, const Shape &F) {
         for (const ChainItem &it : bottom_up) {
             AxhipChainOp &cop = dst[count++];
-            if (is_unary_ew(it.node->op_type)) {
+            if (it.node->op_type == OpType::LeakyReLU) { // the slope rides along as an immediate operand
+                cop.op = AXHIP_OP_LEAKY_RELU;
+                cop.operand = -1;
+                cop.imm = get_params<ActivationParams>(it.node->params).alpha;
+                cop.imm_kind = AXHIP_BK_IMM;
+            } else if (it.node->op_type == OpType::Cast) {
+                if (it.node->output_dtype == DType::Bool && it.node->inputs[0]->output_dtype != DType::Bool) {
+                    cop.op = AXHIP_OP_NE; // a truth value: != 0
+                    cop.operand = -1;
+                    cop.imm = 0.0f;
+                    cop.imm_kind = AXHIP_BK_IMM;
+                } else {
+                    --count; // no arithmetic: the kernel converts on load and on store
+                }
+            } else if (is_unary_ew(it.node->op_type)) {
                 cop.op = unary_code(it.node->op_type);
                 cop.operand = -1;
                 cop.imm = 0.0f;
@@ -511,8 +634,7 @@ class PlanBuilder {
             const bool last_only = !all && n_red == 1 && red[nd - 1];
             if (!all && !last_only) throw RuntimeError::not_implemented("GPU reduction over axes other than the last one (or all)");
             rs.full_reduce = all;
-            rs.prog.reduce = n->op_type == OpType::Sum ? AXHIP_RED_SUM : n->op_type == OpType::Mean ? AXHIP_RED_MEAN
-                             : n->op_type == OpType::Max ? AXHIP_RED_MAX : AXHIP_RED_MIN;
+            rs.prog.reduce = reduce_code(n->op_type);
             cur = in;
             entry = nullptr; // below the reduction only unshared nodes fuse
         }
@@ -560,7 +682,7 @@ class PlanBuilder {
         if (val(in_v).shape != F) in_v = make_contiguous(in_v, &F);
         in_v = make_contiguous(in_v);
         rs.input = in_v;
-        rs.prog.input_dtype = detail::to_axhip_dtype(val(in_v).dtype);
+        rs.prog.input_dtype = detail::to_axhip_dtype_or_bool(val(in_v).dtype);
         rs.prog.cols = F.empty() ? 1 : static_cast<int64_t>(F.back());
         rs.prog.rows = static_cast<int64_t>(ShapeUtils::size(F)) / std::max<int64_t>(rs.prog.cols, 1);
         if (ShapeUtils::size(F) == 0) rs.prog.rows = 0;
@@ -590,7 +712,7 @@ class PlanBuilder {
         }
 
         rs.output = new_temp(n->output_shape, n->output_dtype);
-        rs.prog.output_dtype = detail::to_axhip_dtype(n->output_dtype);
+        rs.prog.output_dtype = detail::to_axhip_dtype_or_bool(n->output_dtype);
         if (rs.full_reduce) {
             rs.workspace = static_cast<int>(plan_.temp_bytes.size());
             plan_.temp_bytes.push_back(axhip_full_reduce_workspace_bytes());
@@ -955,15 +1077,28 @@ void materialize_gpu_graph(GraphNode *root) {
         } else if (st.kind == Step::AXIS_REDUCE) {
             const ValueSpec &src = plan->values[st.axred.src], &dst = plan->values[st.axred.dst];
             if (record) tl_last_kernels.emplace_back("reduce_axis");
-            const size_t ws_bytes = axhip_reduce_axis_workspace_bytes(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner);
+            const int sdt = detail::to_axhip_dtype_or_bool(src.dtype);
+            const size_t ws_bytes = axhip_reduce_axis_workspace_bytes(ptr_of(st.axred.src), sdt, st.axred.outer, st.axred.axis, st.axred.inner);
             const std::unique_ptr<Storage> ws = ws_bytes ? make_storage(ws_bytes, Device::GPU) : nullptr;
-            AXHIP_CALL(axhip_reduce_axis_ws(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
-                                            ptr_of(st.axred.dst), detail::to_axhip_dtype(dst.dtype), ws ? ws->raw() : nullptr, ws_bytes, nullptr));
+            AXHIP_CALL(axhip_reduce_axis_ws(ptr_of(st.axred.src), sdt, st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce, ptr_of(st.axred.dst),
+                                            detail::to_axhip_dtype_or_bool(dst.dtype), ws ? ws->raw() : nullptr, ws_bytes, nullptr));
         } else if (st.kind == Step::AXIS_SOFTMAX) {
             const ValueSpec &src = plan->values[st.axred.src];
             if (record) tl_last_kernels.emplace_back("softmax_axis");
             AXHIP_CALL(axhip_softmax_axis(ptr_of(st.axred.src), detail::to_axhip_dtype(src.dtype), st.axred.outer, st.axred.axis, st.axred.inner, st.axred.reduce,
                                           ptr_of(st.axred.dst), nullptr));
+        } else if (st.kind == Step::WHERE) {
+            const ValueSpec &c = plan->values[st.where.cond], &a = plan->values[st.where.a], &b = plan->values[st.where.b], &d = plan->values[st.where.dst];
+            std::vector<int64_t> shp(d.shape.begin(), d.shape.end()), cst(shp.size()), ast(shp.size()), bst(shp.size());
+            for (size_t i = 0; i < shp.size(); ++i) {
+                cst[i] = st.where.cond_strides[i] / static_cast<int64_t>(dtype_size(c.dtype));
+                ast[i] = st.where.a_strides[i] / static_cast<int64_t>(dtype_size(a.dtype));
+                bst[i] = st.where.b_strides[i] / static_cast<int64_t>(dtype_size(b.dtype));
+            }
+            if (record) tl_last_kernels.emplace_back("where");
+            AXHIP_CALL(axhip_where(ptr_of(st.where.cond), detail::to_axhip_dtype_or_bool(c.dtype), ptr_of(st.where.a), detail::to_axhip_dtype_or_bool(a.dtype),
+                                   ptr_of(st.where.b), detail::to_axhip_dtype_or_bool(b.dtype), ptr_of(st.where.dst), detail::to_axhip_dtype_or_bool(d.dtype),
+                                   static_cast<int32_t>(shp.size()), shp.data(), cst.data(), ast.data(), bst.data(), nullptr));
         } else if (st.kind == Step::GATHER) {
             const ValueSpec &tab = plan->values[st.gather.table], &idx = plan->values[st.gather.indices];
             if (record) tl_last_kernels.emplace_back("gather_rows");
@@ -972,11 +1107,11 @@ void materialize_gpu_graph(GraphNode *root) {
                                          static_cast<int64_t>(ShapeUtils::size(idx.shape)), ptr_of(st.gather.dst), nullptr));
         } else {
             const ValueSpec &src = plan->values[st.copy.src];
-            const int dt = detail::to_axhip_dtype(src.dtype);
+            const int dt = detail::to_axhip_dtype_or_bool(src.dtype), ddt = detail::to_axhip_dtype_or_bool(plan->values[st.copy.dst].dtype);
             std::vector<int64_t> shp(st.copy.shape.begin(), st.copy.shape.end()), est(st.copy.src_strides.size());
             for (size_t i = 0; i < est.size(); ++i) est[i] = st.copy.src_strides[i] / static_cast<int64_t>(dtype_size(src.dtype));
             if (record) tl_last_kernels.emplace_back("strided_copy");
-            AXHIP_CALL(axhip_strided_copy(ptr_of(st.copy.src), dt, ptr_of(st.copy.dst), dt, static_cast<int32_t>(shp.size()), shp.data(),
+            AXHIP_CALL(axhip_strided_copy(ptr_of(st.copy.src), dt, ptr_of(st.copy.dst), ddt, static_cast<int32_t>(shp.size()), shp.data(),
                                           est.data(), nullptr));
         }
     }

@@ -65,7 +65,23 @@ Shape infer_matmul_shape(const Shape &a, const Shape &b, bool ta, bool tb) {
 }
 
 DType infer_binary_dtype(DType lhs, DType rhs) { return ops::promote_types(lhs, rhs); }
-DType infer_unary_dtype(ops::OpType, DType input) { return input; }
+// comparisons and logical operations give Bool (src/graph/graph_registry.cpp:231-263)
+DType infer_binary_output_dtype(ops::OpType op, DType lhs, DType rhs) {
+    using ops::OpType;
+    switch (op) {
+    case OpType::Equal: case OpType::NotEqual: case OpType::Less: case OpType::LessEqual: case OpType::Greater: case OpType::GreaterEqual:
+    case OpType::LogicalAnd: case OpType::LogicalOr: case OpType::LogicalXor:
+        return DType::Bool;
+    default: return ops::promote_types(lhs, rhs);
+    }
+}
+DType infer_unary_dtype(ops::OpType op, DType input) {
+    using ops::OpType;
+    switch (op) {
+    case OpType::IsNaN: case OpType::IsInf: case OpType::IsFinite: case OpType::LogicalNot: return DType::Bool;
+    default: return input;
+    }
+}
 DType infer_reduction_dtype(ops::OpType op, DType input) {
     if (op == ops::OpType::Mean) return input == DType::Float64 ? input : DType::Float32; // src/graph/graph_registry.cpp:278-287
     return input;
@@ -172,9 +188,34 @@ Tensor GraphRegistry::create_lazy_binary(ops::OpType op, const Tensor &lhs, cons
     n->op_type = op;
     n->inputs = {input_node(on_gpu(lhs)), input_node(on_gpu(rhs))};
     n->output_shape = out;
-    n->output_dtype = infer_binary_dtype(lhs.dtype(), rhs.dtype());
+    n->output_dtype = infer_binary_output_dtype(op, lhs.dtype(), rhs.dtype());
     n->target_device = Device::GPU;
     n->params = params;
+    return finalize_lazy_node(std::move(n));
+}
+
+// where(condition, a, b): the three broadcast together; promote_types(a, b) is the result type
+Tensor GraphRegistry::create_lazy_where(const Tensor &condition, const Tensor &a, const Tensor &b) {
+    require_gpu(pick_device({&condition, &a, &b}), ops::OpType::Where);
+    const Shape out = infer_binary_shape(infer_binary_shape(condition.shape(), a.shape()), b.shape());
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Where;
+    n->inputs = {input_node(on_gpu(condition)), input_node(on_gpu(a)), input_node(on_gpu(b))};
+    n->output_shape = out;
+    n->output_dtype = infer_binary_dtype(a.dtype(), b.dtype());
+    n->target_device = Device::GPU;
+    return finalize_lazy_node(std::move(n));
+}
+
+// the GPU Cast as a node: the planner folds it into the kernel that produces or consumes the value
+Tensor GraphRegistry::create_lazy_cast(const Tensor &input, DType target) {
+    require_gpu(pick_device({&input}), ops::OpType::Cast);
+    auto n = std::make_shared<GraphNode>();
+    n->op_type = ops::OpType::Cast;
+    n->inputs = {input_node(input)};
+    n->output_shape = input.shape();
+    n->output_dtype = target;
+    n->target_device = Device::GPU;
     return finalize_lazy_node(std::move(n));
 }
 

@@ -24,4 +24,10 @@ inline int to_axhip_dtype(DType d) {
     default: throw TypeError("the gfx950 kernels compute on float32, float16 and bfloat16; got " + dtype_name(d));
     }
 }
+// the element types of the fused chains, the strided copy, where and the axis reductions: the above plus one-byte
+// truth values (Bool; UInt8 is read the same way)
+inline int to_axhip_dtype_or_bool(DType d) {
+    if (d == DType::Bool || d == DType::UInt8) return AXHIP_DTYPE_U8;
+    return to_axhip_dtype(d);
+}
 } // namespace axiom::detail

@@ -20,6 +20,39 @@ const char *op_name(OpType op) {
     case OpType::Divide: return "divide";
     case OpType::Maximum: return "maximum";
     case OpType::Minimum: return "minimum";
+    case OpType::Power: return "power";
+    case OpType::Modulo: return "modulo";
+    case OpType::Atan2: return "atan2";
+    case OpType::Hypot: return "hypot";
+    case OpType::Equal: return "equal";
+    case OpType::NotEqual: return "not_equal";
+    case OpType::Less: return "less";
+    case OpType::LessEqual: return "less_equal";
+    case OpType::Greater: return "greater";
+    case OpType::GreaterEqual: return "greater_equal";
+    case OpType::LogicalAnd: return "logical_and";
+    case OpType::LogicalOr: return "logical_or";
+    case OpType::LogicalXor: return "logical_xor";
+    case OpType::LogicalNot: return "logical_not";
+    case OpType::Sin: return "sin";
+    case OpType::Cos: return "cos";
+    case OpType::Tan: return "tan";
+    case OpType::Erf: return "erf";
+    case OpType::Sign: return "sign";
+    case OpType::Floor: return "floor";
+    case OpType::Ceil: return "ceil";
+    case OpType::Trunc: return "trunc";
+    case OpType::Round: return "round";
+    case OpType::Cbrt: return "cbrt";
+    case OpType::IsNaN: return "isnan";
+    case OpType::IsInf: return "isinf";
+    case OpType::IsFinite: return "isfinite";
+    case OpType::LeakyReLU: return "leaky_relu";
+    case OpType::Where: return "where";
+    case OpType::Cast: return "cast";
+    case OpType::Prod: return "prod";
+    case OpType::Any: return "any";
+    case OpType::All: return "all";
     case OpType::Negate: return "negate";
     case OpType::Abs: return "abs";
     case OpType::Sqrt: return "sqrt";
@@ -90,6 +123,54 @@ Tensor divide(const Tensor &a, const Tensor &b) { return GraphRegistry::create_l
 Tensor maximum(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Maximum, a, b); }
 Tensor minimum(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Minimum, a, b); }
 
+Tensor power(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Power, a, b); }
+Tensor modulo(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Modulo, a, b); }
+Tensor atan2(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Atan2, a, b); }
+Tensor hypot(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Hypot, a, b); }
+Tensor equal(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Equal, a, b); }
+Tensor not_equal(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::NotEqual, a, b); }
+Tensor less(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Less, a, b); }
+Tensor less_equal(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::LessEqual, a, b); }
+Tensor greater(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::Greater, a, b); }
+Tensor greater_equal(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::GreaterEqual, a, b); }
+Tensor logical_and(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::LogicalAnd, a, b); }
+Tensor logical_or(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::LogicalOr, a, b); }
+Tensor logical_xor(const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_binary(OpType::LogicalXor, a, b); }
+Tensor logical_not(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::LogicalNot, x); }
+
+Tensor sin(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Sin, x); }
+Tensor cos(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Cos, x); }
+Tensor tan(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Tan, x); }
+Tensor erf(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Erf, x); }
+Tensor sign(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Sign, x); }
+Tensor floor(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Floor, x); }
+Tensor ceil(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Ceil, x); }
+Tensor trunc(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Trunc, x); }
+Tensor round(const Tensor &x, int decimals) {
+    if (decimals == 0) return GraphRegistry::create_lazy_unary(OpType::Round, x);
+    const double scale = std::pow(10.0, decimals); // src/tensor/operations.cpp:1334-1340
+    return GraphRegistry::create_lazy_unary(OpType::Round, x * static_cast<float>(scale)) * static_cast<float>(1.0 / scale);
+}
+Tensor cbrt(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Cbrt, x); }
+Tensor isnan(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::IsNaN, x); }
+Tensor isinf(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::IsInf, x); }
+Tensor isfinite(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::IsFinite, x); }
+Tensor clip(const Tensor &x, const Tensor &lo, const Tensor &hi) { return maximum(minimum(x, hi), lo); }
+// one node with the slope as its parameter (the reference builds other slopes than 0.01 from two ReLUs,
+// src/tensor/operations.cpp:1391-1403: the same function)
+Tensor leaky_relu(const Tensor &x, float negative_slope) {
+    graph::ActivationParams p;
+    p.alpha = negative_slope;
+    return GraphRegistry::create_lazy_unary(OpType::LeakyReLU, x, p);
+}
+Tensor where(const Tensor &condition, const Tensor &a, const Tensor &b) { return GraphRegistry::create_lazy_where(condition, a, b); }
+Tensor cast(const Tensor &x, DType target) {
+    if (x.dtype() == target) return x;
+    auto ok = [](DType d) { return d == DType::Float32 || d == DType::Float16 || d == DType::BFloat16 || d == DType::Bool; };
+    if (!ok(x.dtype()) || !ok(target)) throw TypeError("ops::cast on the GPU: Float32, Float16, BFloat16 and Bool; got " + dtype_name(x.dtype()) + " -> " + dtype_name(target));
+    return GraphRegistry::create_lazy_cast(x, target);
+}
+
 Tensor negate(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Negate, x); }
 Tensor abs(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Abs, x); }
 Tensor sqrt(const Tensor &x) { return GraphRegistry::create_lazy_unary(OpType::Sqrt, x); }
@@ -111,6 +192,16 @@ Tensor sum(const Tensor &x, const std::vector<int> &axes, bool keep) { return Gr
 Tensor mean(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Mean, x, axes, keep); }
 Tensor max(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Max, x, axes, keep); }
 Tensor min(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Min, x, axes, keep); }
+Tensor prod(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Prod, x, axes, keep); }
+// Bool results (src/graph/graph_registry.cpp:273-276): the largest / smallest truth value of x != 0
+Tensor any(const Tensor &x, const std::vector<int> &axes, bool keep) {
+    const Tensor truth = x.dtype() == DType::Bool ? x : cast(x, DType::Bool);
+    return GraphRegistry::create_lazy_reduction(OpType::Max, truth, axes, keep);
+}
+Tensor all(const Tensor &x, const std::vector<int> &axes, bool keep) {
+    const Tensor truth = x.dtype() == DType::Bool ? x : cast(x, DType::Bool);
+    return GraphRegistry::create_lazy_reduction(OpType::Min, truth, axes, keep);
+}
 
 namespace {
 // src/backends/cpu/cpu_operations.cpp:2157-2229 (shape rules) on the device kernel; the input is made contiguous

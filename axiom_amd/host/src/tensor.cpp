@@ -311,6 +311,9 @@ Tensor Tensor::to(Device target) const {
 
 Tensor Tensor::astype(DType nd) const {
     if (nd == dtype()) return *this;
+    // among the kernel types and Bool the GPU Cast is a graph node: it folds into the kernel next to it
+    if (device() == Device::GPU && !empty() && (gpu_kernel_dtype(dtype_) || dtype_ == DType::Bool) && (gpu_kernel_dtype(nd) || nd == DType::Bool))
+        return ops::cast(*this, nd);
     materialize_if_needed();
     if (device() == Device::GPU) {
         if (gpu_kernel_dtype(dtype_) && gpu_kernel_dtype(nd)) { // the GPU Cast op (src/tensor/tensor.cpp:1665-1670)
@@ -362,6 +365,24 @@ Tensor Tensor::softmax(int axis) const { return ops::softmax(*this, axis); }
 Tensor Tensor::log_softmax(int axis) const { return ops::log_softmax(*this, axis); }
 Tensor Tensor::relu() const { return ops::relu(*this); }
 Tensor Tensor::gelu() const { return ops::gelu(*this); }
+Tensor Tensor::leaky_relu(float negative_slope) const { return ops::leaky_relu(*this, negative_slope); }
+Tensor Tensor::sign() const { return ops::sign(*this); }
+Tensor Tensor::floor() const { return ops::floor(*this); }
+Tensor Tensor::ceil() const { return ops::ceil(*this); }
+Tensor Tensor::trunc() const { return ops::trunc(*this); }
+Tensor Tensor::round(int decimals) const { return ops::round(*this, decimals); }
+Tensor Tensor::cbrt() const { return ops::cbrt(*this); }
+Tensor Tensor::isnan() const { return ops::isnan(*this); }
+Tensor Tensor::isinf() const { return ops::isinf(*this); }
+Tensor Tensor::isfinite() const { return ops::isfinite(*this); }
+Tensor Tensor::clip(double lo, double hi) const { return ops::clip(*this, make_scalar_like(*this, lo), make_scalar_like(*this, hi)); }
+Tensor Tensor::where(const Tensor &condition, const Tensor &other) const { return ops::where(condition, *this, other); }
+Tensor Tensor::prod(int axis, bool keep_dims) const { return ops::prod(*this, {axis}, keep_dims); }
+Tensor Tensor::prod(const std::vector<int> &axes, bool keep_dims) const { return ops::prod(*this, axes, keep_dims); }
+Tensor Tensor::any(int axis, bool keep_dims) const { return ops::any(*this, {axis}, keep_dims); }
+Tensor Tensor::any(const std::vector<int> &axes, bool keep_dims) const { return ops::any(*this, axes, keep_dims); }
+Tensor Tensor::all(int axis, bool keep_dims) const { return ops::all(*this, {axis}, keep_dims); }
+Tensor Tensor::all(const std::vector<int> &axes, bool keep_dims) const { return ops::all(*this, axes, keep_dims); }
 Tensor Tensor::sigmoid() const { return ops::sigmoid(*this); }
 Tensor Tensor::silu() const { return ops::silu(*this); }
 Tensor Tensor::tanh() const { return ops::tanh(*this); }
@@ -453,6 +474,12 @@ Tensor make_scalar_like(const Tensor &t, double value) {
     return d;
 }
 Tensor operator+(const Tensor &a, const Tensor &b) { return ops::add(a, b); }
+Tensor operator<(const Tensor &a, const Tensor &b) { return ops::less(a, b); }
+Tensor operator<=(const Tensor &a, const Tensor &b) { return ops::less_equal(a, b); }
+Tensor operator>(const Tensor &a, const Tensor &b) { return ops::greater(a, b); }
+Tensor operator>=(const Tensor &a, const Tensor &b) { return ops::greater_equal(a, b); }
+Tensor operator==(const Tensor &a, const Tensor &b) { return ops::equal(a, b); }
+Tensor operator!=(const Tensor &a, const Tensor &b) { return ops::not_equal(a, b); }
 Tensor operator-(const Tensor &a, const Tensor &b) { return ops::subtract(a, b); }
 Tensor operator*(const Tensor &a, const Tensor &b) { return ops::multiply(a, b); }
 Tensor operator/(const Tensor &a, const Tensor &b) { return ops::divide(a, b); }

@@ -1131,7 +1131,7 @@ static void matmul_layout_case(DType dt, double tol) {
             for (size_t j = 0; j < N; ++j) want[i * N + j] += double(af[i * K + k]) * double(bf[k * N + j]);
     auto check = [&](const Tensor &r, const char *what) {
         EXPECT_TRUE(r.shape() == Shape({M, N}));
-        const auto h = host_floats(r.astype(DType::Float32));
+        const auto h = host_floats(r);
         double worst = 0.0;
         for (size_t i = 0; i < M * N; ++i) worst = std::max(worst, std::abs(double(h[i]) - want[i]) / (1.0 + std::abs(want[i])));
         if (!(worst < tol)) std::fprintf(stderr, "    matmul layout case: %s\n", what);
@@ -1246,6 +1246,176 @@ GPU_TEST(LazyNodes, PadAndMaskedFill) { // tests/test_shape_ops_extended.cpp:42-
     EXPECT_NEAR(sm[0], 1.0f, 1e-6); EXPECT_NEAR(sm[1], 0.0f, 1e-6);
     std::vector<float> fm(16, 0.0f);
     EXPECT_THROW(ops::masked_fill(x.gpu(), Tensor::from_data(fm.data(), {4, 4}, Device::GPU), 0.0f), TypeError);
+}
+
+// The wider operator table: the reference's expectations (tests/test_tensor_comparisons.cpp:24-113,
+// test_tensor_logical_bitwise.cpp:11-70 and :245-292, test_tensor_numpy_ops.cpp:13-104, test_tensor_where.cpp:26-205,
+// test_tensor_activations.cpp:356-478, test_tensor_operations.cpp:107-121), result types, and what fuses.
+static std::vector<int> host_truth(const Tensor &t) {
+    EXPECT_TRUE(t.dtype() == DType::Bool);
+    Tensor c = t.cpu().ascontiguousarray();
+    const uint8_t *p = static_cast<const uint8_t *>(c.data());
+    return std::vector<int>(p, p + c.size());
+}
+
+GPU_TEST(LazyNodes, ComparisonsLogicalOperationsAndWhere) {
+    auto a = gpu_f32({0, 1, 2, 3, 4}, {5});
+    auto two = Tensor::full({5}, 2.0f, Device::GPU);
+    EXPECT_TRUE(host_truth(ops::less(a, two)) == std::vector<int>({1, 1, 0, 0, 0}));
+    EXPECT_TRUE(host_truth(ops::less_equal(a, two)) == std::vector<int>({1, 1, 1, 0, 0}));
+    EXPECT_TRUE(host_truth(ops::greater(a, two)) == std::vector<int>({0, 0, 0, 1, 1}));
+    EXPECT_TRUE(host_truth(ops::greater_equal(a, two)) == std::vector<int>({0, 0, 1, 1, 1}));
+    EXPECT_TRUE(host_truth(ops::equal(a, two)) == std::vector<int>({0, 0, 1, 0, 0}));
+    EXPECT_TRUE(host_truth(a != two) == std::vector<int>({1, 1, 0, 1, 1}));
+    EXPECT_TRUE(host_truth(2.5f > a + 0.0f) == std::vector<int>({1, 1, 1, 0, 0})); // the chain on the right-hand side
+    EXPECT_TRUE((a < 2.0f).dtype() == DType::Bool);
+    // broadcasting (test_tensor_comparisons.cpp:222-236): (3, 1) against (4) -> (3, 4)
+    auto col = gpu_f32({0, 1, 2}, {3, 1}), row = gpu_f32({0, 1, 2, 3}, {4});
+    auto lt = ops::less(col, row);
+    EXPECT_TRUE(lt.shape() == Shape({3, 4}));
+    EXPECT_TRUE(host_truth(lt) == std::vector<int>({0, 1, 1, 1, 0, 0, 1, 1, 0, 0, 0, 1}));
+
+    bool la[] = {true, true, false, false}, lb[] = {true, false, true, false};
+    auto ta = Tensor::from_data(la, {4}, Device::GPU), tb = Tensor::from_data(lb, {4}, Device::GPU);
+    EXPECT_TRUE(host_truth(ops::logical_and(ta, tb)) == std::vector<int>({1, 0, 0, 0}));
+    EXPECT_TRUE(host_truth(ops::logical_or(ta, tb)) == std::vector<int>({1, 1, 1, 0}));
+    EXPECT_TRUE(host_truth(ops::logical_xor(ta, tb)) == std::vector<int>({0, 1, 1, 0}));
+    EXPECT_TRUE(host_truth(ops::logical_not(ta)) == std::vector<int>({0, 0, 1, 1}));
+    EXPECT_TRUE(host_truth(ops::logical_not(gpu_f32({1.0f, 0.0f, -3.5f, 0.0f}, {4}))) == std::vector<int>({0, 1, 0, 1}));
+
+    // where
+    auto cond = Tensor::from_data(lb, {4}, Device::GPU); // {1, 0, 1, 0}
+    auto w = host_floats(ops::where(cond, Tensor::full({4}, 1.0f, Device::GPU), Tensor::full({4}, 0.0f, Device::GPU)));
+    EXPECT_TRUE(w == std::vector<float>({1, 0, 1, 0}));
+    auto x = gpu_f32({1, -2, 3, -4, 0}, {5});
+    auto zero = Tensor::zeros({5}, DType::Float32, Device::GPU);
+    EXPECT_TRUE(host_floats(ops::where(ops::greater(x, zero), x, zero)) == std::vector<float>({1, 0, 3, 0, 0})); // ReLU pattern
+    EXPECT_TRUE(host_floats(x.where(x > 0.0f, zero - 1.0f)) == std::vector<float>({1, -1, 3, -1, -1}));
+    // scalars broadcast on either branch; a (2, 1) condition against (2, 3) branches; mixed branch types promote
+    auto m = gpu_f32({1, 2, 3, 4, 5, 6}, {2, 3});
+    bool rows_on[] = {true, false};
+    auto rc = Tensor::from_data(rows_on, {2, 1}, Device::GPU);
+    EXPECT_TRUE(host_floats(ops::where(rc, m, Tensor::full({1}, -1.0f, Device::GPU))) == std::vector<float>({1, 2, 3, -1, -1, -1}));
+    auto mixed = ops::where(rc, m.bfloat16(), m * 10.0f);
+    EXPECT_TRUE(mixed.dtype() == DType::Float32);
+    EXPECT_TRUE(host_floats(mixed) == std::vector<float>({1, 2, 3, 40, 50, 60}));
+    // the attention use: where(mask, -1e9, scores) then softmax
+    auto sc = gpu_f32({0.5f, 0.3f, 0.2f, 0.1f}, {2, 2});
+    bool mk[] = {false, true, false, false};
+    auto masked = ops::where(Tensor::from_data(mk, {2, 2}, Device::GPU), Tensor::full({2, 2}, -1e9f, Device::GPU), sc);
+    auto sm = host_floats(ops::softmax(masked, -1));
+    EXPECT_NEAR(sm[0], 1.0f, 1e-6); EXPECT_NEAR(sm[1], 0.0f, 1e-6);
+    EXPECT_THROW(ops::less(Tensor::zeros({3}), Tensor::zeros({3})), RuntimeError); // CPU tensors: no CPU compute path here
+}
+
+GPU_TEST(LazyNodes, MathOperatorsRoundingTestsAndActivations) {
+    EXPECT_TRUE(host_floats(gpu_f32({-3, -1, 0, 1, 3}, {5}).sign()) == std::vector<float>({-1, -1, 0, 1, 1}));
+    auto x = gpu_f32({-2.7f, -0.5f, 0.5f, 2.7f}, {4});
+    EXPECT_TRUE(host_floats(x.floor()) == std::vector<float>({-3, -1, 0, 2}));
+    EXPECT_TRUE(host_floats(x.ceil()) == std::vector<float>({-2, 0, 1, 3}));
+    EXPECT_TRUE(host_floats(x.trunc()) == std::vector<float>({-2, 0, 0, 2}));
+    EXPECT_TRUE(host_floats(gpu_f32({0.5f, 1.5f, -0.5f, 2.4f}, {4}).round()) == std::vector<float>({1, 2, -1, 2}));
+    auto r2 = host_floats(ops::round(gpu_f32({3.14159f, -2.71828f}, {2}), 2));
+    EXPECT_NEAR(r2[0], 3.14f, 1e-5); EXPECT_NEAR(r2[1], -2.72f, 1e-5);
+    auto cb = host_floats(gpu_f32({8, 27, 64}, {3}).cbrt());
+    EXPECT_NEAR(cb[0], 2.0f, 1e-5); EXPECT_NEAR(cb[1], 3.0f, 1e-5); EXPECT_NEAR(cb[2], 4.0f, 1e-5);
+    auto t = gpu_f32({1.0f, NAN, INFINITY, -INFINITY, 0.0f}, {5});
+    EXPECT_TRUE(host_truth(t.isnan()) == std::vector<int>({0, 1, 0, 0, 0}));
+    EXPECT_TRUE(host_truth(t.isinf()) == std::vector<int>({0, 0, 1, 1, 0}));
+    EXPECT_TRUE(host_truth(t.isfinite()) == std::vector<int>({1, 0, 0, 0, 1}));
+    EXPECT_TRUE(host_floats(gpu_f32({-5, -1, 0, 1, 5}, {5}).clip(-2.0, 2.0)) == std::vector<float>({-2, -1, 0, 1, 2}));
+    auto p = host_floats(ops::power(Tensor::full({2, 2}, 3.0f, Device::GPU), Tensor::full({2, 2}, 4.0f, Device::GPU)));
+    for (float v : p) EXPECT_NEAR(v, 81.0f, 1e-4);
+    EXPECT_TRUE(host_floats(ops::modulo(gpu_f32({5.5f, -5.5f, 7.0f}, {3}), gpu_f32({2, 2, -3}, {3}))) == std::vector<float>({1.5f, -1.5f, 1.0f}));
+    auto at = host_floats(ops::atan2(gpu_f32({1, 1, 0}, {3}), gpu_f32({1, 0, 1}, {3})));
+    EXPECT_NEAR(at[0], M_PI / 4, 1e-6); EXPECT_NEAR(at[1], M_PI / 2, 1e-6); EXPECT_NEAR(at[2], 0.0, 1e-6);
+    auto hy = host_floats(ops::hypot(gpu_f32({3, 0, 5}, {3}), gpu_f32({4, 5, 12}, {3})));
+    EXPECT_NEAR(hy[0], 5.0f, 1e-5); EXPECT_NEAR(hy[1], 5.0f, 1e-5); EXPECT_NEAR(hy[2], 13.0f, 1e-5);
+    auto e = host_floats(ops::erf(gpu_f32({0, 1, -1}, {3})));
+    EXPECT_NEAR(e[0], 0.0f, 1e-6); EXPECT_NEAR(e[1], 0.8427f, 1e-4); EXPECT_NEAR(e[1] + e[2], 0.0f, 1e-6);
+    auto lk = host_floats(gpu_f32({-2, 3, 0}, {3}).leaky_relu());
+    EXPECT_NEAR(lk[0], -0.02f, 1e-8); EXPECT_NEAR(lk[1], 3.0f, 0); EXPECT_NEAR(lk[2], 0.0f, 0);
+    EXPECT_NEAR(host_floats(gpu_f32({-2}, {1}).leaky_relu(0.2f))[0], -0.4f, 1e-7);
+
+    // a long mixed chain is still ONE launch, float64 check on random data
+    auto v = axtest::randn({33, 200}, 120);
+    auto g = v.gpu();
+    auto y = ops::sin(g) * ops::cos(g) + ops::floor(g * 2.0f) - ops::leaky_relu(g, 0.1f);
+    auto got = host_floats(y), vf = host_floats(v);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 4u); // sin, cos and leaky_relu of the shared input are chains of their own
+    for (size_t i = 0; i < vf.size(); ++i) {
+        const double d = vf[i];
+        EXPECT_NEAR(got[i], std::sin(d) * std::cos(d) + std::floor(double(vf[i] * 2.0f)) - (d > 0 ? d : double(0.1f) * d), 1e-5);
+    }
+    auto z = host_floats(ops::tan(ops::sign(g) * ops::sqrt(ops::abs(g) + 1.0f) * 0.25f));
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 2u);
+    for (size_t i = 0; i < vf.size(); i += 7) {
+        const double d = vf[i], sg = d > 0 ? 1 : d < 0 ? -1 : 0;
+        EXPECT_NEAR(z[i], std::tan(sg * std::sqrt(std::fabs(d) + 1.0) * 0.25), 1e-5);
+    }
+    // softmax(x) > 1/cols, in one kernel up to the Bool result; bf16 input
+    auto pr = ops::greater(ops::softmax(g, -1), Tensor::full({1}, 1.0f / 200.0f, Device::GPU));
+    auto truth = host_truth(pr);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    size_t ones = 0;
+    for (int b : truth) ones += b;
+    EXPECT_TRUE(ones > 33u * 20u && ones < 33u * 180u);
+    auto hb = host_truth(ops::less(g.bfloat16(), Tensor::zeros({1}, DType::BFloat16, Device::GPU)));
+    for (size_t i = 0; i < vf.size(); ++i) EXPECT_EQ(hb[i], float(bfloat16_t(vf[i])) < 0.0f ? 1 : 0);
+}
+
+GPU_TEST(LazyNodes, ProductsAnyAllAndCasts) {
+    auto t = gpu_f32({1, 2, 3, 4}, {2, 2});
+    EXPECT_NEAR(ops::prod(t).item<float>(), 24.0f, 1e-5);
+    EXPECT_TRUE(host_floats(t.prod(0)) == std::vector<float>({3, 8}));
+    EXPECT_TRUE(host_floats(t.prod(1)) == std::vector<float>({2, 12}));
+    EXPECT_NEAR(ops::prod(ops::sqrt(gpu_f32({4, 9, 16}, {3}))).item<float>(), 24.0f, 1e-4); // tests/test_fusion_extended.cpp:376-385
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    EXPECT_TRUE(host_truth(ops::any(gpu_f32({0, 0, 1, 0}, {4}))) == std::vector<int>({1}));
+    EXPECT_TRUE(host_truth(ops::all(gpu_f32({1, 1, 1, 1}, {4}))) == std::vector<int>({1}));
+    EXPECT_TRUE(host_truth(ops::all(gpu_f32({1, 0, 1, 1}, {4}))) == std::vector<int>({0}));
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u); // != 0 and the reduction in one launch
+    auto m = gpu_f32({0, 0, 0, 1, 0, 2, 3, 4, 5}, {3, 3});
+    EXPECT_TRUE(host_truth(m.any(1)) == std::vector<int>({0, 1, 1}));
+    EXPECT_TRUE(host_truth(m.all(1)) == std::vector<int>({0, 0, 1}));
+    EXPECT_TRUE(host_truth(m.any(0)) == std::vector<int>({1, 1, 1}));
+    EXPECT_TRUE(host_truth(m.all(0)) == std::vector<int>({0, 0, 0}));
+    EXPECT_TRUE(m.any(0, true).shape() == Shape({1, 3}));
+    // all(isfinite(x)) as the reference's audio tests use it (tests/test_audio.cpp:118-123)
+    auto v = axtest::randn({64, 100}, 121).gpu();
+    EXPECT_TRUE(host_truth(ops::all(ops::isfinite(v))) == std::vector<int>({1}));
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    EXPECT_TRUE(host_truth(ops::any(ops::isnan((v - v) / (v - v)))) == std::vector<int>({1}));
+    // products along a middle axis and over everything, against float64
+    auto s = axtest::uniform({4, 9, 16}, 122, 0.9f, 1.1f);
+    auto sf = host_floats(s), pm = host_floats(s.gpu().prod(1));
+    for (size_t o = 0; o < 4; ++o)
+        for (size_t i = 0; i < 16; ++i) {
+            double want = 1;
+            for (size_t a = 0; a < 9; ++a) want *= sf[(o * 9 + a) * 16 + i];
+            EXPECT_NEAR(pm[o * 16 + i], want, 1e-5);
+        }
+    // casts: lazy nodes that fold into the neighbouring kernel
+    auto c = (v * 2.0f).astype(DType::BFloat16);
+    EXPECT_TRUE(c.dtype() == DType::BFloat16);
+    auto cf = host_floats(c), vf = host_floats(v);
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u); // multiply and round in one launch
+    for (size_t i = 0; i < vf.size(); ++i) EXPECT_NEAR(cf[i], float(bfloat16_t(vf[i] * 2.0f)), 0);
+    auto widened = host_floats(ops::relu(c.to_float()) + 1.0f); // bf16 -> f32 in front of a chain: converted on load
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    for (size_t i = 0; i < vf.size(); ++i) EXPECT_NEAR(widened[i], std::max(0.0f, float(bfloat16_t(vf[i] * 2.0f))) + 1.0f, 0);
+    // a narrowing cast in mid-chain rounds there: relu(bf16(x * 3)) * 1.5 computed from the rounded value
+    auto mid = host_floats(ops::relu((v * 3.0f).astype(DType::BFloat16)).to_float() * 1.5f);
+    for (size_t i = 0; i < vf.size(); ++i) EXPECT_NEAR(mid[i], std::max(0.0f, float(bfloat16_t(vf[i] * 3.0f))) * 1.5f, 0);
+    EXPECT_TRUE(host_truth(gpu_f32({0, 2, -1, 0}, {4}).to_bool()) == std::vector<int>({0, 1, 1, 0}));
+    EXPECT_TRUE(host_floats(gpu_f32({0, 2, -1, 0}, {4}).to_bool().to_float() * 3.0f) == std::vector<float>({0, 3, 3, 0}));
+    auto tv = v.transpose({1, 0}).astype(DType::Float16); // a strided view: one converting gather
+    EXPECT_EQ(host_floats(tv).size(), vf.size());
+    EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    EXPECT_EQ(graph::last_gpu_plan_kernels()[0], std::string("strided_copy"));
+    auto tvf = host_floats(tv);
+    for (size_t i = 0; i < 64; ++i)
+        for (size_t j = 0; j < 100; j += 9) EXPECT_NEAR(tvf[j * 64 + i], float(float16_t(vf[i * 100 + j])), 0);
 }
 
 GPU_TEST(LazyNodes, BatchNorm1dInference) {

@@ -45,6 +45,10 @@ extern "C" {
 #define AXHIP_DTYPE_F32 0
 #define AXHIP_DTYPE_F16 1
 #define AXHIP_DTYPE_BF16 2
+/* Bool / UInt8 (one byte; any nonzero byte reads as 1.0, a nonzero result is stored as 1): the result type of
+ * comparisons, logical operations and any / all, and an input type of the fused chains and of axhip_strided_copy
+ * and axhip_where.  Attention, GEMM and the other entry points take the three floating-point types only. */
+#define AXHIP_DTYPE_U8 3
 
 /* ------------------------------------------------------------------ runtime
  * Stands behind system::is_metal_available (src/tensor/system.cpp:11-29),
@@ -168,6 +172,43 @@ const char *axhip_sdpa_last_schedule(void);
 #define AXHIP_OP_SQUARE 26
 #define AXHIP_OP_RSQRT 27
 #define AXHIP_OP_RECIP 28
+/* The wider operator table of the lazy graph (binary: 40-63, unary: 64-95), with the CPU functors' rules
+ * (src/backends/cpu/cpu_operations.hpp:214-235 power / fmod, :237-291 comparisons and logical operations, :360-381
+ * atan2 / hypot, :395-400 logical not, :497-505 erf, :655-660 leaky ReLU, :724-787 sign / floor / ceil / trunc /
+ * round, :808-860 cbrt / isnan / isinf / isfinite).  Comparisons, logical operations and the is* tests yield 1.0 or
+ * 0.0 inside a chain; stored to an AXHIP_DTYPE_U8 output that is the reference's Bool result.  A logical operation
+ * reads any nonzero value (NaN included) as true. */
+#define AXHIP_OP_POW 40    /* powf(v, operand) */
+#define AXHIP_OP_RPOW 41   /* powf(operand, v) */
+#define AXHIP_OP_MOD 42    /* fmodf(v, operand): the sign of the dividend, like the CPU functor */
+#define AXHIP_OP_RMOD 43   /* fmodf(operand, v) */
+#define AXHIP_OP_ATAN2 44  /* atan2f(v, operand) */
+#define AXHIP_OP_RATAN2 45 /* atan2f(operand, v) */
+#define AXHIP_OP_HYPOT 46
+#define AXHIP_OP_EQ 47
+#define AXHIP_OP_NE 48
+#define AXHIP_OP_LT 49 /* v < operand; with the chain value on the right-hand side the planner emits GT */
+#define AXHIP_OP_LE 50
+#define AXHIP_OP_GT 51
+#define AXHIP_OP_GE 52
+#define AXHIP_OP_AND 53
+#define AXHIP_OP_OR 54
+#define AXHIP_OP_XOR 55
+#define AXHIP_OP_LEAKY_RELU 56 /* v > 0 ? v : operand * v -- the slope is the operand (an immediate) */
+#define AXHIP_OP_ERF 64
+#define AXHIP_OP_SIN 65
+#define AXHIP_OP_COS 66
+#define AXHIP_OP_TAN 67
+#define AXHIP_OP_SIGN 68 /* 1, -1, or 0 (also for NaN) */
+#define AXHIP_OP_FLOOR 69
+#define AXHIP_OP_CEIL 70
+#define AXHIP_OP_ROUND 71 /* halves away from zero (std::round) */
+#define AXHIP_OP_TRUNC 72
+#define AXHIP_OP_CBRT 73
+#define AXHIP_OP_ISNAN 74
+#define AXHIP_OP_ISINF 75
+#define AXHIP_OP_ISFINITE 76
+#define AXHIP_OP_NOT 77 /* v == 0 */
 
 #define AXHIP_ROWOP_NONE 0
 #define AXHIP_ROWOP_SOFTMAX 1
@@ -180,6 +221,7 @@ const char *axhip_sdpa_last_schedule(void);
 #define AXHIP_RED_MEAN 2
 #define AXHIP_RED_MAX 3
 #define AXHIP_RED_MIN 4
+#define AXHIP_RED_PROD 5 /* (any / all are NE 0 under MAX / MIN with an AXHIP_DTYPE_U8 result) */
 
 /* how a binary op's second operand maps onto the [rows, cols] view */
 #define AXHIP_BK_FULL 0   /* [rows, cols] */
@@ -272,7 +314,8 @@ int axhip_fused_full_reduce_noalloc(const AxhipRowsProgram *program_host, void *
  * 60-63, kernel gather_strided src/backends/metal/kernels.metal:33-149) and
  * the GPU Cast op (src/tensor/tensor.cpp:1665-1670).  Copies a strided view
  * (<= 8 dims, non-negative element strides) into a contiguous row-major
- * buffer, converting dtype on the way. */
+ * buffer, converting dtype on the way (AXHIP_DTYPE_U8 on either side: the
+ * Bool casts, nonzero <-> 1). */
 #define AXHIP_MAX_DIMS 8
 int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t dst_dtype,
                        int32_t ndim, const int64_t *shape_host, const int64_t *src_strides_host,
@@ -295,6 +338,17 @@ int axhip_pad(const void *src, void *dst, int32_t dtype, int32_t ndim, const int
 int axhip_masked_fill(const void *src, int32_t dtype, const uint8_t *mask, void *dst, int32_t ndim,
                       const int64_t *shape_host, const int64_t *src_strides_host,
                       const int64_t *mask_strides_host, double value, void *stream);
+
+/* where (ops::where, include/axiom/operations.hpp:425-429 and
+ * src/tensor/operations.cpp:1543-1566; GPU MPSGraphTernaryOperation::execute_where,
+ * src/backends/metal/mpsgraph_operations.mm:637): dst[i] = cond[i] != 0 ?
+ * a[i] : b[i] over an iteration space of <= 8 dims.  cond (normally
+ * AXHIP_DTYPE_U8), a and b are strided views with element strides, 0 on
+ * broadcast dims, each of its own element type; dst is contiguous. */
+int axhip_where(const void *cond, int32_t cond_dtype, const void *a, int32_t a_dtype, const void *b,
+                int32_t b_dtype, void *dst, int32_t dst_dtype, int32_t ndim, const int64_t *shape_host,
+                const int64_t *cond_strides_host, const int64_t *a_strides_host,
+                const int64_t *b_strides_host, void *stream);
 
 /* Embedding lookup (ops::embedding, include/axiom/operations.hpp:483-486):
  * dst[i, :] = table[indices[i], :] for n_indices rows of row_elems elements.

@@ -375,7 +375,11 @@ int axo_softmax(int dtype, const void *in, void *out, size_t outer, size_t axis,
 /* ------------------------------------------------------------------------ */
 /* Elementwise functors: src/backends/cpu/cpu_operations.hpp:186-202        */
 /* (add/sub/mul/div), :635-653 (gelu erf form, relu), and the scalar forms  */
-/* beside them.  Half types evaluate in float and round once per op         */
+/* beside them; :214-235 power (std::pow) and modulo (std::fmod), :237-291   */
+/* comparisons and logical operations (any nonzero value is true), :360-381  */
+/* atan2 / hypot, :395-400 logical not, :497-505 erf, :655-660 leaky ReLU,   */
+/* :724-787 sign (0 for NaN) / floor / ceil / trunc / round (std::round),    */
+/* :808-860 cbrt / isnan / isinf / isfinite.  Half types evaluate in float and round once per op         */
 /* (include/axiom/bfloat16.hpp:55-73); gelu on a half type goes through     */
 /* double (cpu_operations.hpp:643-646).                                     */
 /* ------------------------------------------------------------------------ */
@@ -398,6 +402,20 @@ static inline float unary_f32(int op, float a) {
     case AXO_OP_SQUARE: return a * a;
     case AXO_OP_RSQRT: return 1.0f / sqrtf(a);
     case AXO_OP_RECIP: return 1.0f / a;
+    case AXO_OP_ERF: return erff(a);
+    case AXO_OP_SIN: return sinf(a);
+    case AXO_OP_COS: return cosf(a);
+    case AXO_OP_TAN: return tanf(a);
+    case AXO_OP_SIGN: return a > 0.0f ? 1.0f : a < 0.0f ? -1.0f : 0.0f;
+    case AXO_OP_FLOOR: return floorf(a);
+    case AXO_OP_CEIL: return ceilf(a);
+    case AXO_OP_ROUND: return roundf(a);
+    case AXO_OP_TRUNC: return truncf(a);
+    case AXO_OP_CBRT: return cbrtf(a);
+    case AXO_OP_ISNAN: return isnan(a) ? 1.0f : 0.0f;
+    case AXO_OP_ISINF: return isinf(a) ? 1.0f : 0.0f;
+    case AXO_OP_ISFINITE: return isfinite(a) ? 1.0f : 0.0f;
+    case AXO_OP_NOT: return a != 0.0f ? 0.0f : 1.0f;
     default: return NAN;
     }
 }
@@ -410,6 +428,23 @@ static inline float binary_f32(int op, float a, float b) {
     case AXO_OP_DIV: return a / b;
     case AXO_OP_MAX: return a > b ? a : b;
     case AXO_OP_MIN: return a < b ? a : b;
+    case AXO_OP_POW: return powf(a, b);
+    case AXO_OP_RPOW: return powf(b, a);
+    case AXO_OP_MOD: return fmodf(a, b);
+    case AXO_OP_RMOD: return fmodf(b, a);
+    case AXO_OP_ATAN2: return atan2f(a, b);
+    case AXO_OP_RATAN2: return atan2f(b, a);
+    case AXO_OP_HYPOT: return hypotf(a, b);
+    case AXO_OP_EQ: return a == b ? 1.0f : 0.0f;
+    case AXO_OP_NE: return a != b ? 1.0f : 0.0f;
+    case AXO_OP_LT: return a < b ? 1.0f : 0.0f;
+    case AXO_OP_LE: return a <= b ? 1.0f : 0.0f;
+    case AXO_OP_GT: return a > b ? 1.0f : 0.0f;
+    case AXO_OP_GE: return a >= b ? 1.0f : 0.0f;
+    case AXO_OP_AND: return (a != 0.0f) && (b != 0.0f) ? 1.0f : 0.0f;
+    case AXO_OP_OR: return (a != 0.0f) || (b != 0.0f) ? 1.0f : 0.0f;
+    case AXO_OP_XOR: return (a != 0.0f) != (b != 0.0f) ? 1.0f : 0.0f;
+    case AXO_OP_LEAKY_RELU: return a > 0.0f ? a : b * a; /* b: the slope */
     default: return NAN;
     }
 }
@@ -441,6 +476,12 @@ int axo_binary(int op, int dtype, const void *a, const void *b, void *out,
     return 0;
 }
 
+int axo_where(int dtype, const uint8_t *cond, const void *a, const void *b, void *out, size_t n) {
+    if (dtype < 0 || dtype > 2) return -1;
+    for (size_t i = 0; i < n; ++i) st(dtype, out, i, cond[i] ? ld(dtype, a, i) : ld(dtype, b, i));
+    return 0;
+}
+
 /* ------------------------------------------------------------------------ */
 /* Last-axis reduction: src/backends/cpu/cpu_operations.cpp:1555-1617.      */
 /* Float accumulation (also for half inputs, :1421-1424), mean divides the  */
@@ -460,6 +501,11 @@ static float row_reduce(int red, int dtype, const void *in, size_t base, size_t 
         for (; j < n; ++j) s += ld(dtype, in, base + j);
         return s;
     }
+    if (red == AXO_RED_PROD) { /* a running float product, in index order */
+        float p = 1.0f;
+        for (size_t j = 0; j < n; ++j) p *= ld(dtype, in, base + j);
+        return p;
+    }
     float r = ld(dtype, in, base);
     for (size_t j = 1; j < n; ++j) {
         float x = ld(dtype, in, base + j);
@@ -469,7 +515,7 @@ static float row_reduce(int red, int dtype, const void *in, size_t base, size_t 
 }
 
 int axo_reduce_last(int red, int dtype, const void *in, void *out, size_t rows, size_t cols) {
-    if (dtype < 0 || dtype > 2 || red < 1 || red > 4 || cols == 0) return -1;
+    if (dtype < 0 || dtype > 2 || red < 1 || red > 5 || cols == 0) return -1;
 #pragma omp parallel for schedule(static) if (rows >= 64)
     for (ptrdiff_t r = 0; r < (ptrdiff_t)rows; ++r) {
         float s = row_reduce(red, dtype, in, (size_t)r * cols, cols);

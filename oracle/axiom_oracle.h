@@ -66,9 +66,18 @@ enum {
     AXO_OP_RELU = 16, AXO_OP_GELU = 17, AXO_OP_SQRT = 18, AXO_OP_EXP = 19,
     AXO_OP_NEG = 20, AXO_OP_ABS = 21, AXO_OP_SIGMOID = 22, AXO_OP_TANH = 23,
     AXO_OP_SILU = 24, AXO_OP_LOG = 25, AXO_OP_SQUARE = 26, AXO_OP_RSQRT = 27,
-    AXO_OP_RECIP = 28
+    AXO_OP_RECIP = 28,
+    /* binary: the running value is the first argument; R* forms take it as the second */
+    AXO_OP_POW = 40, AXO_OP_RPOW = 41, AXO_OP_MOD = 42, AXO_OP_RMOD = 43, AXO_OP_ATAN2 = 44,
+    AXO_OP_RATAN2 = 45, AXO_OP_HYPOT = 46, AXO_OP_EQ = 47, AXO_OP_NE = 48, AXO_OP_LT = 49,
+    AXO_OP_LE = 50, AXO_OP_GT = 51, AXO_OP_GE = 52, AXO_OP_AND = 53, AXO_OP_OR = 54,
+    AXO_OP_XOR = 55, AXO_OP_LEAKY_RELU = 56,
+    /* unary */
+    AXO_OP_ERF = 64, AXO_OP_SIN = 65, AXO_OP_COS = 66, AXO_OP_TAN = 67, AXO_OP_SIGN = 68,
+    AXO_OP_FLOOR = 69, AXO_OP_CEIL = 70, AXO_OP_ROUND = 71, AXO_OP_TRUNC = 72, AXO_OP_CBRT = 73,
+    AXO_OP_ISNAN = 74, AXO_OP_ISINF = 75, AXO_OP_ISFINITE = 76, AXO_OP_NOT = 77
 };
-enum { AXO_RED_SUM = 1, AXO_RED_MEAN = 2, AXO_RED_MAX = 3, AXO_RED_MIN = 4 };
+enum { AXO_RED_SUM = 1, AXO_RED_MEAN = 2, AXO_RED_MAX = 3, AXO_RED_MIN = 4, AXO_RED_PROD = 5 };
 
 /* broadcast kind of the second operand of a binary op over a [rows, cols] view */
 enum { AXO_BK_FULL = 0, AXO_BK_ROWVEC = 1, AXO_BK_COLVEC = 2, AXO_BK_SCALAR = 3 };
@@ -105,7 +114,11 @@ int axo_sdpa(int dtype, const void *q, const void *k, const void *v, void *o,
 int axo_softmax(int dtype, const void *in, void *out, size_t outer, size_t axis,
                 size_t inner, int is_log);
 
+/* Comparisons, logical operations and the is* tests write 1 or 0 in `dtype`
+ * (the reference's Bool result: nonzero = true). */
 int axo_unary(int op, int dtype, const void *in, void *out, size_t n);
+/* out[i] = cond[i] ? a[i] : b[i]; cond is one byte per element, nonzero = true */
+int axo_where(int dtype, const uint8_t *cond, const void *a, const void *b, void *out, size_t n);
 int axo_binary(int op, int dtype, const void *a, const void *b, void *out,
                size_t rows, size_t cols, int b_kind);
 /* last-axis reduction; out has `rows` elements of `dtype` (float accumulate,

@@ -19,8 +19,12 @@ REF_PATH = HERE / "_ref" / "libaxiom_ref.so"
 F32, F16, BF16 = 0, 1, 2
 OP = dict(add=1, sub=2, mul=3, div=4, max=5, min=6,
           relu=16, gelu=17, sqrt=18, exp=19, neg=20, abs=21, sigmoid=22, tanh=23,
-          silu=24, log=25, square=26, rsqrt=27, recip=28)
-RED = dict(sum=1, mean=2, max=3, min=4)
+          silu=24, log=25, square=26, rsqrt=27, recip=28,
+          pow=40, rpow=41, mod=42, rmod=43, atan2=44, ratan2=45, hypot=46, eq=47, ne=48, lt=49, le=50, gt=51, ge=52,
+          **{"and": 53, "or": 54, "xor": 55, "not": 77}, leaky_relu=56,
+          erf=64, sin=65, cos=66, tan=67, sign=68, floor=69, ceil=70, round=71, trunc=72, cbrt=73,
+          isnan=74, isinf=75, isfinite=76)
+RED = dict(sum=1, mean=2, max=3, min=4, prod=5)
 BK = dict(full=0, rowvec=1, colvec=2, scalar=3)
 
 _lib = None
@@ -58,6 +62,7 @@ def lib() -> C.CDLL:
                                C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         l.axo_softmax.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int]
         l.axo_unary.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]
+        l.axo_where.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
         l.axo_binary.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int]
         l.axo_argreduce.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]
         l.axo_reduce_last.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t]
@@ -184,6 +189,16 @@ def binary(op, a, b, dt=F32, kind="full"):
     cols = a.shape[-1]
     out = np.empty_like(a)
     assert lib().axo_binary(OP[op], dt, _p(a), _p(b), _p(out), rows, cols, BK[kind]) == 0
+    return out
+
+
+def where(cond, a, b, dt=F32):
+    """cond: uint8 / bool array of a's shape."""
+    cond = np.ascontiguousarray(cond).astype(np.uint8)
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    out = np.empty_like(a)
+    assert lib().axo_where(dt, _p(cond), _p(a), _p(b), _p(out), a.size) == 0
     return out
 
 

@@ -9,7 +9,7 @@ import torch
 
 from axiom_amd import capi
 
-F32, F16, BF16 = capi.DTYPE_F32, capi.DTYPE_F16, capi.DTYPE_BF16
+F32, F16, BF16, U8 = capi.DTYPE_F32, capi.DTYPE_F16, capi.DTYPE_BF16, capi.DTYPE_U8
 
 
 def to_dev(a: np.ndarray) -> torch.Tensor:
@@ -26,11 +26,11 @@ def to_host(t: torch.Tensor, like_dtype) -> np.ndarray:
 
 
 def np_store_dtype(dt):
-    return np.float32 if dt == F32 else np.uint16
+    return np.float32 if dt == F32 else np.uint8 if dt == U8 else np.uint16
 
 
 def empty_dev(shape, dt) -> torch.Tensor:
-    return torch.empty(shape, dtype=torch.float32 if dt == F32 else torch.int16, device="cuda")
+    return torch.empty(shape, dtype=torch.float32 if dt == F32 else torch.uint8 if dt == U8 else torch.int16, device="cuda")
 
 
 def sync():
@@ -148,7 +148,7 @@ class Rows:
         self.p.reduce = capi.RED[reduce]
         shape = self.x.shape[:-1] if reduce != "none" else self.x.shape
         out = empty_dev(shape if len(shape) else (1,), self.out_dt)
-        out.fill_(float("nan") if self.out_dt == F32 else 0x7FC1)
+        out.fill_(float("nan") if self.out_dt == F32 else 0xCC if self.out_dt == U8 else 0x7FC1)
         self.p.output = out.data_ptr()
         self.p.output_dtype = self.out_dt
         sync()

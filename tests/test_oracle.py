@@ -346,6 +346,77 @@ def test_reduce_known_answers():
     assert np.array_equal(m, axo.to_bits(axo.to_f32(xb, BF16).astype(np.float64).mean(-1).astype(np.float32), BF16))
 
 
+def test_wider_operator_table_known_answers():
+    """The reference's own expectations for the operators beyond the hot-path subset."""
+    f = lambda *v: np.array(v, np.float32)
+    truth = lambda a: (a != 0).tolist()
+    two5, two4 = np.full(5, 2.0, np.float32), np.full(4, 2.0, np.float32)
+    a5, a4 = np.arange(5, dtype=np.float32), np.arange(4, dtype=np.float32)
+    # tests/test_tensor_comparisons.cpp:24-113
+    assert truth(axo.binary("ne", a4, two4)) == [True, True, False, True]
+    assert truth(axo.binary("lt", a5, two5)) == [True, True, False, False, False]
+    assert truth(axo.binary("le", a5, two5)) == [True, True, True, False, False]
+    assert truth(axo.binary("gt", a5, two5)) == [False, False, False, True, True]
+    assert truth(axo.binary("ge", a5, two5)) == [False, False, True, True, True]
+    assert truth(axo.binary("eq", a5, two5)) == [False, False, True, False, False]
+    # tests/test_tensor_logical_bitwise.cpp:11-70
+    la, lb = f(1, 1, 0, 0), f(1, 0, 1, 0)
+    assert truth(axo.binary("and", la, lb)) == [True, False, False, False]
+    assert truth(axo.binary("or", la, lb)) == [True, True, True, False]
+    assert truth(axo.binary("xor", la, lb)) == [False, True, True, False]
+    assert truth(axo.unary("not", f(1, 0, 1, 0))) == [False, True, False, True]
+    assert truth(axo.unary("not", f(1.0, 0.0, -3.5, 0.0))) == [False, True, False, True]
+    # :245-277
+    assert np.allclose(axo.binary("atan2", f(1, 1, 0), f(1, 0, 1)), [math.pi / 4, math.pi / 2, 0.0], atol=1e-6)
+    assert np.allclose(axo.binary("hypot", f(3, 0, 5), f(4, 5, 12)), [5, 5, 13], atol=1e-5)
+    # tests/test_tensor_numpy_ops.cpp:13-79
+    assert np.array_equal(axo.unary("sign", f(-3, -1, 0, 1, 3)), f(-1, -1, 0, 1, 1))
+    x = f(-2.7, -0.5, 0.5, 2.7)
+    assert np.array_equal(axo.unary("floor", x), f(-3, -1, 0, 2))
+    assert np.array_equal(axo.unary("ceil", x), f(-2, 0, 1, 3))  # (-0.0 == 0.0)
+    assert np.array_equal(axo.unary("trunc", x), f(-2, 0, 0, 2))
+    assert np.allclose(axo.unary("cbrt", f(8, 27, 64)), [2, 3, 4], atol=1e-5)
+    t = f(1.0, np.nan, np.inf, -np.inf, 0.0)
+    assert truth(axo.unary("isnan", t)) == [False, True, False, False, False]
+    assert truth(axo.unary("isinf", t)) == [False, False, True, True, False]
+    assert truth(axo.unary("isfinite", t)) == [True, False, False, False, True]
+    clip = axo.binary("max", axo.binary("min", f(-5, -1, 0, 1, 5), f(2.0), kind="scalar"), f(-2.0), kind="scalar")
+    assert np.array_equal(clip, f(-2, -1, 0, 1, 2))  # :81-88, clip = maximum(minimum(x, hi), lo)
+    # :91-104 prod; tests/test_fusion_extended.cpp:376-385 prod(sqrt([4, 9, 16])) = 24
+    assert axo.reduce_last("prod", f(1, 2, 3, 4).reshape(1, 4))[0] == 24.0
+    assert np.array_equal(axo.reduce_last("prod", f(1, 3, 2, 4).reshape(2, 2)), f(3, 8))  # prod over axis 0 of [[1,2],[3,4]]
+    assert abs(axo.reduce_last("prod", axo.unary("sqrt", f(4, 9, 16)).reshape(1, 3))[0] - 24.0) < 1e-4
+    # tests/test_tensor_activations.cpp:356-375 erf; :446-478 any / all as the extreme truth value
+    e = axo.unary("erf", f(0, 1, -1))
+    assert abs(e[0]) < 1e-6 and abs(e[1] - 0.8427) < 1e-4 and e[1] == -e[2]
+    nz = lambda v: axo.binary("ne", v, f(0.0), kind="scalar").reshape(1, -1)
+    assert axo.reduce_last("max", nz(f(0, 0, 1, 0)))[0] != 0  # any
+    assert axo.reduce_last("min", nz(f(1, 1, 1, 1)))[0] != 0  # all
+    assert axo.reduce_last("min", nz(f(1, 0, 1, 1)))[0] == 0
+    # tests/test_tensor_operations.cpp:107-121: 3 ** 4 = 81; tests/test_tensor_where.cpp:26-36, 176-205
+    assert np.all(axo.binary("pow", np.full(4, 3.0, np.float32), np.full(4, 4.0, np.float32)) == 81.0)
+    assert np.array_equal(axo.where(np.array([1, 0, 1, 0], np.uint8), np.ones(4, np.float32), np.zeros(4, np.float32)), f(1, 0, 1, 0))
+    xs = f(1, -2, 3, -4, 0)
+    cond = axo.binary("gt", xs, np.zeros(5, np.float32))
+    assert np.array_equal(axo.where(cond != 0, xs, np.zeros(5, np.float32)), f(1, 0, 3, 0, 0))
+    # what the mathematics fixes where the reference's tests hold no value: fmod keeps the dividend's sign
+    # (cpu_operations.hpp:225-235), round moves halves away from zero (:777-787), leaky ReLU (:655-660), the
+    # reversed forms, and the trigonometric functions against libm in float64
+    assert np.array_equal(axo.binary("mod", f(5.5, -5.5, 5.5, -5.5), f(2, 2, -2, -2)), f(1.5, -1.5, 1.5, -1.5))
+    assert np.array_equal(axo.unary("round", f(0.5, 1.5, 2.5, -0.5, -1.5, 2.4)), f(1, 2, 3, -1, -2, 2))
+    assert np.allclose(axo.binary("leaky_relu", f(-2, 3, 0), f(0.01), kind="scalar"), [-0.02, 3.0, 0.0], atol=1e-9)
+    assert np.array_equal(axo.binary("rpow", f(1, 2, 3), f(2.0), kind="scalar"), f(2, 4, 8))
+    assert np.array_equal(axo.binary("rmod", f(2, 3, 4), f(7.0), kind="scalar"), f(1, 1, 3))
+    assert np.allclose(axo.binary("ratan2", f(1, 0), f(1.0), kind="scalar"), [math.pi / 4, math.pi / 2], atol=1e-6)
+    v = rng(11).standard_normal(64).astype(np.float32) * 3
+    for name, fn in (("sin", np.sin), ("cos", np.cos), ("tan", np.tan)):
+        assert np.allclose(axo.unary(name, v), fn(v.astype(np.float64)), rtol=1e-5, atol=1e-6), name
+    assert np.isnan(axo.unary("sign", f(np.nan))[0]) == False and axo.unary("sign", f(np.nan))[0] == 0.0  # neither > 0 nor < 0
+    # half types: evaluated in float, rounded once
+    hb = axo.to_bits(v, BF16)
+    assert np.array_equal(axo.unary("sin", hb, BF16), axo.to_bits(np.sin(axo.to_f32(hb, BF16).astype(np.float64)).astype(np.float32), BF16))
+
+
 # ----------------------------------------------------------------------- norms
 
 def test_layer_norm_closed_form():
