@@ -22,6 +22,7 @@ OP = dict(add=1, sub=2, mul=3, div=4, max=5, min=6, rsub=7, rdiv=8,
 ROWOP = dict(none=0, softmax=1, logsoftmax=2, layernorm=3, rmsnorm=4)
 RED = dict(none=0, sum=1, mean=2, max=3, min=4, prod=5)
 BK = dict(full=0, rowvec=1, colvec=2, scalar=3, imm=4)
+PAD = dict(constant=0, reflect=1, replicate=2, circular=3)
 
 MAX_CHAIN, MAX_OPERANDS = 16, 8
 ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_WORKSPACE = -1, -2, -3, -4
@@ -124,6 +125,7 @@ def lib() -> C.CDLL:
         l.axhip_gemm_ws.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(GemmParams), C.c_void_p, C.c_size_t, C.c_void_p]
         i64p = C.POINTER(C.c_int64)
         l.axhip_pad.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, i64p, i64p, i64p, i64p, C.c_double, C.c_void_p]
+        l.axhip_pad_mode.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, i64p, i64p, i64p, i64p, C.c_int32, C.c_double, C.c_void_p]
         l.axhip_masked_fill.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, i64p, i64p, i64p, C.c_double, C.c_void_p]
         l.axhip_where.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32,
                                   i64p, i64p, i64p, i64p, C.c_void_p]

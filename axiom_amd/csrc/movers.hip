@@ -112,8 +112,26 @@ struct PadArgs {
     int dtype, ndim;
     int64_t total;
     float value;
+    int mode; // AXHIP_PAD_*
     int64_t out_shape[AXHIP_MAX_DIMS], src_shape[AXHIP_MAX_DIMS], src_strides[AXHIP_MAX_DIMS], before[AXHIP_MAX_DIMS];
 };
+
+// Source coordinate of output coordinate c (already shifted by the leading pad) along an extent of n elements, -1
+// where the constant goes.  Reflection leaves the border element out (… 2 1 | 0 1 2 … n-1 | n-2 n-3 …); the host
+// has checked that a reflected pad is shorter than the extent, so one fold is enough.
+template <typename IDX>
+__device__ __forceinline__ IDX pad_source(IDX c, IDX n, int mode) {
+    if (c >= 0 && c < n) return c;
+    switch (mode) {
+    case AXHIP_PAD_REFLECT: return c < 0 ? -c : 2 * n - c - 2;
+    case AXHIP_PAD_REPLICATE: return c < 0 ? 0 : n - 1;
+    case AXHIP_PAD_CIRCULAR: {
+        const IDX m = c % n;
+        return m < 0 ? m + n : m;
+    }
+    default: return -1;
+    }
+}
 
 __global__ __launch_bounds__(256) void pad_kernel(const PadArgs a) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
@@ -121,9 +139,9 @@ __global__ __launch_bounds__(256) void pad_kernel(const PadArgs a) {
         int64_t rem = i, off = 0;
         bool inside = true;
         for (int d = a.ndim - 1; d >= 0; --d) {
-            const int64_t c = rem % a.out_shape[d] - a.before[d];
+            const int64_t c = pad_source<int64_t>(rem % a.out_shape[d] - a.before[d], a.src_shape[d], a.mode);
             rem /= a.out_shape[d];
-            inside = inside && c >= 0 && c < a.src_shape[d];
+            inside = inside && c >= 0;
             off += c * a.src_strides[d];
         }
         store_any(a.dst, a.dtype, i, inside ? load_any(a.src, a.dtype, off) : a.value);
@@ -146,16 +164,16 @@ __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
         for (int d = L - 1; d >= 0; --d) {
             const IDX n = static_cast<IDX>(a.out_shape[d]);
             const IDX q = rem / n;
-            const IDX c = rem - q * n - static_cast<IDX>(a.before[d]);
+            const IDX c = pad_source<IDX>(rem - q * n - static_cast<IDX>(a.before[d]), static_cast<IDX>(a.src_shape[d]), a.mode);
             rem = q;
-            inside = inside && c >= 0 && c < static_cast<IDX>(a.src_shape[d]);
+            inside = inside && c >= 0;
             off += c * static_cast<IDX>(a.src_strides[d]);
         }
         float v[V];
 #pragma unroll
         for (int e = 0; e < V; ++e) {
-            const IDX c = c0 + e;
-            v[e] = inside && c >= 0 && c < n_src ? load_any(a.src, a.dtype, off + c * st) : a.value;
+            const IDX c = pad_source<IDX>(c0 + e, n_src, a.mode);
+            v[e] = inside && c >= 0 ? load_any(a.src, a.dtype, off + c * st) : a.value;
         }
         store_vec<V>(a.dst, a.dtype, static_cast<int64_t>(i) * V, v);
     }
@@ -789,15 +807,27 @@ int axhip_fill(void *dst, int32_t dtype, double value, int64_t count, void *stre
 
 int axhip_pad(const void *src, void *dst, int32_t dtype, int32_t ndim, const int64_t *src_shape, const int64_t *src_strides,
               const int64_t *pad_before, const int64_t *pad_after, double value, void *stream) {
+    return axhip_pad_mode(src, dst, dtype, ndim, src_shape, src_strides, pad_before, pad_after, AXHIP_PAD_CONSTANT, value, stream);
+}
+
+int axhip_pad_mode(const void *src, void *dst, int32_t dtype, int32_t ndim, const int64_t *src_shape, const int64_t *src_strides,
+                   const int64_t *pad_before, const int64_t *pad_after, int32_t mode, double value, void *stream) {
     AXHIP_REQUIRE(valid_dtype(dtype), AXHIP_ERR_INVALID_ARG, "axhip_pad: bad dtype");
+    AXHIP_REQUIRE(mode >= AXHIP_PAD_CONSTANT && mode <= AXHIP_PAD_CIRCULAR, AXHIP_ERR_INVALID_ARG, "axhip_pad: bad mode %d", mode);
     AXHIP_REQUIRE(ndim >= 1 && ndim <= AXHIP_MAX_DIMS, AXHIP_ERR_INVALID_ARG, "axhip_pad: ndim %d out of range", ndim);
     AXHIP_REQUIRE(src_shape && src_strides && pad_before && pad_after, AXHIP_ERR_INVALID_ARG, "axhip_pad: NULL shape/strides/pads");
     PadArgs a{};
-    a.src = src; a.dst = dst; a.dtype = dtype; a.ndim = ndim; a.value = static_cast<float>(value);
+    a.src = src; a.dst = dst; a.dtype = dtype; a.ndim = ndim; a.value = static_cast<float>(value); a.mode = mode;
     a.total = 1;
     int64_t src_total = 1;
     for (int d = 0; d < ndim; ++d) {
         AXHIP_REQUIRE(src_shape[d] >= 0 && pad_before[d] >= 0 && pad_after[d] >= 0, AXHIP_ERR_INVALID_ARG, "axhip_pad: negative extent or pad");
+        if (mode == AXHIP_PAD_REFLECT && (pad_before[d] > 0 || pad_after[d] > 0))
+            AXHIP_REQUIRE(pad_before[d] < src_shape[d] && pad_after[d] < src_shape[d], AXHIP_ERR_INVALID_ARG,
+                          "axhip_pad: a reflected pad (%lld, %lld) must be shorter than the extent %lld", static_cast<long long>(pad_before[d]),
+                          static_cast<long long>(pad_after[d]), static_cast<long long>(src_shape[d]));
+        if (mode != AXHIP_PAD_CONSTANT && (pad_before[d] > 0 || pad_after[d] > 0))
+            AXHIP_REQUIRE(src_shape[d] > 0, AXHIP_ERR_INVALID_ARG, "axhip_pad: nothing to repeat along an empty extent");
         AXHIP_REQUIRE(src_strides[d] >= 0, AXHIP_ERR_UNSUPPORTED, "axhip_pad: negative strides (flipped views) are not supported");
         a.src_shape[d] = src_shape[d];
         a.src_strides[d] = src_strides[d];

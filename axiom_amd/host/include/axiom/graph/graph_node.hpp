@@ -45,6 +45,7 @@ struct SliceParams { // per dimension; steps are positive
 struct PadParams {
     std::vector<std::pair<size_t, size_t>> pad_widths;
     double value = 0.0;
+    int mode = 0; // AXHIP_PAD_*: constant, reflect, replicate, circular
 };
 struct MaskedFillParams {
     float value = 0.0f;
@@ -52,6 +53,7 @@ struct MaskedFillParams {
 struct UnfoldParams { // windows of `kernel` taps along the last dimension (and `kernel_h` along the one before it, for 2-D)
     int kernel = 1, stride = 1, dilation = 1;
     int kernel_h = 1, stride_h = 1, dilation_h = 1;
+    int groups = 1; // > 1: the channels are cut into groups, which lead the window view: (G, N, ..., C_in / G, K...)
 };
 
 using OpParams = std::variant<NoParams, ReductionParams, MatMulParams, ActivationParams, ReshapeParams, NormParams, TransposeParams, SliceParams,

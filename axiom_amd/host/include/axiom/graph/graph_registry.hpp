@@ -43,14 +43,15 @@ class GraphRegistry {
     // the remaining node kinds of whole forward passes (include/axiom/graph/graph_registry.hpp:70-122)
     static Tensor create_lazy_slice(const Tensor &input, const std::vector<int64_t> &starts, const std::vector<int64_t> &ends,
                                     const std::vector<int64_t> &steps, const Shape &output_shape);
-    static Tensor create_lazy_pad(const Tensor &input, const std::vector<std::pair<size_t, size_t>> &pad_widths, double value, const Shape &output_shape);
+    static Tensor create_lazy_pad(const Tensor &input, const std::vector<std::pair<size_t, size_t>> &pad_widths, double value, const Shape &output_shape,
+                                  int mode = 0);
     static Tensor create_lazy_masked_fill(const Tensor &input, const Tensor &mask, float value);
     static Tensor create_lazy_glu(const Tensor &input, int dim, const Shape &output_shape);
     static Tensor create_lazy_batchnorm(const Tensor &input, const Tensor &weight, const Tensor &bias, const Tensor &running_mean,
                                         const Tensor &running_var, float eps);
-    static Tensor create_lazy_conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation);
+    static Tensor create_lazy_conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation, int groups = 1);
     static Tensor create_lazy_conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride,
-                                     std::array<int, 2> padding, std::array<int, 2> dilation);
+                                     std::array<int, 2> padding, std::array<int, 2> dilation, int groups = 1);
     static Tensor create_lazy_embedding(const Tensor &weight, const Tensor &indices);
 
     // signature -> plan cache -> compile -> execute; GPU graphs go to materialize_gpu_graph

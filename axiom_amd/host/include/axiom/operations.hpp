@@ -174,18 +174,19 @@ Tensor glu(const Tensor &x, int dim = -1);
 // (include/axiom/operations.hpp:437-440)
 Tensor masked_fill(const Tensor &x, const Tensor &mask, float value);
 Tensor masked_fill(const Tensor &x, const Tensor &mask, double value);
-// constant padding; pad_width holds (before, after) per dimension (include/axiom/operations.hpp:519-526)
+// pad_width holds (before, after) per dimension; mode "constant", "reflect" (the border element is not repeated; each
+// pad shorter than its dimension), "replicate" or "circular" (include/axiom/operations.hpp:519-526)
 Tensor pad(const Tensor &x, const std::vector<std::pair<size_t, size_t>> &pad_width, const std::string &mode = "constant", double value = 0.0);
 // rows of weight (vocab, dim) selected by integer indices of any shape -> (*indices.shape, dim)
 // (include/axiom/operations.hpp:483-486).  On the GPU an index out of range gives a row of zeros.
 Tensor embedding(const Tensor &weight, const Tensor &indices);
 // PyTorch-compatible 1-D convolution: input (N, C_in, L) or (C_in, L), weight (C_out, C_in, K),
 // output (N, C_out, L_out), L_out = (L + 2 padding - dilation (K-1) - 1) / stride + 1
-// (include/axiom/operations.hpp:594-601).  groups must be 1.
+// (include/axiom/operations.hpp:594-601).  groups > 1: weight (C_out, C_in / groups, K), one batched product over the groups.
 Tensor conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride = 1, int padding = 0, int dilation = 1, int groups = 1);
 Tensor conv1d(const Tensor &input, const Tensor &weight); // no bias, stride 1, no padding
 // 2-D convolution: input (N, C_in, H, W) or (C_in, H, W), weight (C_out, C_in, KH, KW), output (N, C_out, H_out, W_out)
-// (include/axiom/operations.hpp:603-611).  groups must be 1.
+// (include/axiom/operations.hpp:603-611).  groups as for conv1d.
 Tensor conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride = {1, 1}, std::array<int, 2> padding = {0, 0},
               std::array<int, 2> dilation = {1, 1}, int groups = 1);
 Tensor conv2d(const Tensor &input, const Tensor &weight);

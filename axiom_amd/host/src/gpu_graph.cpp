@@ -68,6 +68,7 @@ struct PadStep {
     int src = -1, dst = -1;
     std::vector<int64_t> before, after;
     double value = 0.0;
+    int mode = 0;
 };
 
 struct MaskedFillStep {
@@ -388,6 +389,7 @@ class PlanBuilder {
             const Strides is = val(in).strides;
             s.shape = n->output_shape;
             s.strides = {is[0], is[2] * up.stride, is[1], is[2] * up.dilation};
+            if (up.groups > 1) s.strides.insert(s.strides.begin(), is[1] * static_cast<int64_t>(n->output_shape[3])); // (G, N, L_out, C / G, K)
             v = add_value(s);
         } else if (op == OpType::Unfold2D) {
             // (N, C, H, W) -> windows (N, H_out, W_out, C, KH, KW): element (n, i, j, c, a, b) is input (n, c, i sh + a dh, j sw + b dw)
@@ -397,6 +399,7 @@ class PlanBuilder {
             const Strides is = val(in).strides;
             s.shape = n->output_shape;
             s.strides = {is[0], is[2] * up.stride_h, is[3] * up.stride, is[1], is[2] * up.dilation_h, is[3] * up.dilation};
+            if (up.groups > 1) s.strides.insert(s.strides.begin(), is[1] * static_cast<int64_t>(n->output_shape[4])); // (G, N, H_out, W_out, C / G, KH, KW)
             v = add_value(s);
         } else if (op == OpType::Pad) {
             const int in = eval(n->inputs[0].get());
@@ -412,6 +415,7 @@ class PlanBuilder {
                 st.pad.after.push_back(static_cast<int64_t>(w.second));
             }
             st.pad.value = pp.value;
+            st.pad.mode = pp.mode;
             plan_.steps.push_back(st);
         } else if (op == OpType::MaskedFill) {
             if (n->inputs.size() < 2) throw RuntimeError("malformed graph node 'masked_fill': missing inputs");
@@ -1064,8 +1068,8 @@ void materialize_gpu_graph(GraphNode *root) {
             std::vector<int64_t> shp(src.shape.begin(), src.shape.end()), est(src.strides.size());
             for (size_t i = 0; i < est.size(); ++i) est[i] = src.strides[i] / isz;
             if (record) tl_last_kernels.emplace_back("pad");
-            AXHIP_CALL(axhip_pad(ptr_of(st.pad.src), ptr_of(st.pad.dst), detail::to_axhip_dtype(src.dtype), static_cast<int32_t>(shp.size()), shp.data(),
-                                 est.data(), st.pad.before.data(), st.pad.after.data(), st.pad.value, nullptr));
+            AXHIP_CALL(axhip_pad_mode(ptr_of(st.pad.src), ptr_of(st.pad.dst), detail::to_axhip_dtype(src.dtype), static_cast<int32_t>(shp.size()), shp.data(),
+                                      est.data(), st.pad.before.data(), st.pad.after.data(), st.pad.mode, st.pad.value, nullptr));
         } else if (st.kind == Step::MASKED_FILL) {
             const ValueSpec &src = plan->values[st.mfill.src];
             const int64_t isz = static_cast<int64_t>(dtype_size(src.dtype));

@@ -389,7 +389,7 @@ Tensor GraphRegistry::create_lazy_slice(const Tensor &input, const std::vector<i
 }
 
 Tensor GraphRegistry::create_lazy_pad(const Tensor &input, const std::vector<std::pair<size_t, size_t>> &pad_widths, double value,
-                                      const Shape &output_shape) {
+                                      const Shape &output_shape, int mode) {
     require_gpu(pick_device({&input}), ops::OpType::Pad);
     auto n = std::make_shared<GraphNode>();
     n->op_type = ops::OpType::Pad;
@@ -397,7 +397,7 @@ Tensor GraphRegistry::create_lazy_pad(const Tensor &input, const std::vector<std
     n->output_shape = output_shape;
     n->output_dtype = input.dtype();
     n->target_device = Device::GPU;
-    n->params = PadParams{pad_widths, value};
+    n->params = PadParams{pad_widths, value, mode};
     return finalize_lazy_node(std::move(n));
 }
 
@@ -453,7 +453,7 @@ Tensor GraphRegistry::create_lazy_batchnorm(const Tensor &input, const Tensor &w
 // Convolution as a GEMM: constant padding, the (N, L_out, C_in, K) window view of the padded signal, its
 // gather to (N, L_out, C_in K), a product with the (C_out, C_in K) filter matrix (bias and a following
 // activation ride in the GEMM epilogue), and the (N, C_out, L_out) view of the result.
-Tensor GraphRegistry::create_lazy_conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation) {
+Tensor GraphRegistry::create_lazy_conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation, int groups) {
     require_gpu(pick_device({&input}), ops::OpType::Conv1D);
     const size_t N = input.shape()[0], Cin = input.shape()[1], L = input.shape()[2];
     const size_t Cout = weight.shape()[0], K = weight.shape()[2];
@@ -468,7 +468,21 @@ Tensor GraphRegistry::create_lazy_conv1d(const Tensor &input, const Tensor &weig
     un->output_shape = Shape{N, Lout, Cin, K};
     un->output_dtype = x.dtype();
     un->target_device = Device::GPU;
-    un->params = UnfoldParams{static_cast<int>(K), stride, dilation};
+    UnfoldParams up{static_cast<int>(K), stride, dilation};
+    up.groups = groups;
+    un->params = up;
+    if (groups > 1) {
+        // Grouped: the windows lead with the group, (G, N, L_out, C_in / G, K), one batched product against the
+        // (G, C_out / G, C_in / G * K) filters gives (G, N L_out, C_out / G), which is brought to (N, C_out, L_out).
+        const size_t G = static_cast<size_t>(groups), Cg = Cin / G, Og = Cout / G;
+        un->output_shape = Shape{G, N, Lout, Cg, K};
+        const Tensor cols = create_lazy_reshape(finalize_lazy_node(std::move(un)), Shape{G, N * Lout, Cg * K});
+        const Tensor w3 = on_gpu(weight).reshape({G, Og, Cg * K});
+        Tensor y = create_lazy_matmul(cols, w3, false, true); // (G, N L_out, O_g)
+        if (!bias.empty()) y = create_lazy_binary(ops::OpType::Add, y, on_gpu(bias).reshape({G, 1, Og}));
+        const Tensor moved = create_lazy_transpose(create_lazy_reshape(y, Shape{G, N, Lout, Og}), {1, 0, 3, 2}); // (N, G, O_g, L_out)
+        return create_lazy_reshape(moved, Shape{N, Cout, Lout});
+    }
     const Tensor cols = create_lazy_reshape(finalize_lazy_node(std::move(un)), Shape{N, Lout, Cin * K});
     const Tensor w2 = on_gpu(weight).reshape({Cout, Cin * K});
     Tensor y = create_lazy_matmul(cols, w2, false, true);
@@ -479,7 +493,7 @@ Tensor GraphRegistry::create_lazy_conv1d(const Tensor &input, const Tensor &weig
 // The same lowering in two dimensions: windows (N, H_out, W_out, C_in, KH, KW), product with the (C_out, C_in KH KW)
 // filter matrix, result laid out (N, H_out, W_out, C_out) and returned as its (N, C_out, H_out, W_out) view.
 Tensor GraphRegistry::create_lazy_conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride,
-                                         std::array<int, 2> padding, std::array<int, 2> dilation) {
+                                         std::array<int, 2> padding, std::array<int, 2> dilation, int groups) {
     require_gpu(pick_device({&input}), ops::OpType::Conv2D);
     const size_t N = input.shape()[0], Cin = input.shape()[1], Hin = input.shape()[2], Win = input.shape()[3];
     const size_t Cout = weight.shape()[0], KH = weight.shape()[2], KW = weight.shape()[3];
@@ -504,7 +518,18 @@ Tensor GraphRegistry::create_lazy_conv2d(const Tensor &input, const Tensor &weig
     up.kernel_h = static_cast<int>(KH);
     up.stride_h = stride[0];
     up.dilation_h = dilation[0];
+    up.groups = groups;
     un->params = up;
+    if (groups > 1) { // as for conv1d: (G, N, H_out, W_out, C_in / G, KH, KW) windows, one batched product
+        const size_t G = static_cast<size_t>(groups), Cg = Cin / G, Og = Cout / G;
+        un->output_shape = Shape{G, N, Hout, Wout, Cg, KH, KW};
+        const Tensor cols = create_lazy_reshape(finalize_lazy_node(std::move(un)), Shape{G, N * Hout * Wout, Cg * KH * KW});
+        const Tensor w3 = on_gpu(weight).reshape({G, Og, Cg * KH * KW});
+        Tensor y = create_lazy_matmul(cols, w3, false, true); // (G, N H_out W_out, O_g)
+        if (!bias.empty()) y = create_lazy_binary(ops::OpType::Add, y, on_gpu(bias).reshape({G, 1, Og}));
+        const Tensor moved = create_lazy_transpose(create_lazy_reshape(y, Shape{G, N, Hout * Wout, Og}), {1, 0, 3, 2}); // (N, G, O_g, H_out W_out)
+        return create_lazy_reshape(moved, Shape{N, Cout, Hout, Wout});
+    }
     const Tensor cols = create_lazy_reshape(finalize_lazy_node(std::move(un)), Shape{N, Hout * Wout, Cin * KH * KW});
     const Tensor w2 = on_gpu(weight).reshape({Cout, Cin * KH * KW});
     Tensor y = create_lazy_matmul(cols, w2, false, true);
@@ -640,10 +665,11 @@ void feed(Fnv1a &h, const PadParams &p) {
         h.u64(w.second);
     });
     h.bytes(&p.value, sizeof(p.value));
+    h.i32(p.mode);
 }
 void feed(Fnv1a &h, const MaskedFillParams &p) { h.f32(p.value); }
 void feed(Fnv1a &h, const UnfoldParams &p) {
-    for (int v : {p.kernel, p.stride, p.dilation, p.kernel_h, p.stride_h, p.dilation_h}) h.i32(v);
+    for (int v : {p.kernel, p.stride, p.dilation, p.kernel_h, p.stride_h, p.dilation_h, p.groups}) h.i32(v);
 }
 
 // one node: operation, result, where it sits in the order, what it reads

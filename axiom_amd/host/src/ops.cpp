@@ -274,11 +274,20 @@ Tensor masked_fill(const Tensor &x, const Tensor &mask, float value) { return Gr
 Tensor masked_fill(const Tensor &x, const Tensor &mask, double value) { return masked_fill(x, mask, static_cast<float>(value)); }
 
 Tensor pad(const Tensor &x, const std::vector<std::pair<size_t, size_t>> &pad_width, const std::string &mode, double value) {
-    if (mode != "constant") throw RuntimeError::not_implemented("pad mode '" + mode + "' on the GPU (constant only)");
+    // src/tensor/operations.cpp:2178-2184 (the reference's GPU path leaves "circular" to the CPU; here it has a kernel)
+    const int m = mode == "constant" ? AXHIP_PAD_CONSTANT : mode == "reflect" ? AXHIP_PAD_REFLECT : mode == "replicate" ? AXHIP_PAD_REPLICATE
+                  : mode == "circular" ? AXHIP_PAD_CIRCULAR : -1;
+    if (m < 0) throw ValueError("pad: mode must be 'constant', 'reflect', 'replicate', or 'circular', got '" + mode + "'");
     if (pad_width.size() != x.ndim()) throw ShapeError("pad: pad_width must have one (before, after) pair per dimension");
     Shape out = x.shape();
-    for (size_t d = 0; d < out.size(); ++d) out[d] += pad_width[d].first + pad_width[d].second;
-    return GraphRegistry::create_lazy_pad(x, pad_width, value, out);
+    for (size_t d = 0; d < out.size(); ++d) {
+        const size_t widest = std::max(pad_width[d].first, pad_width[d].second);
+        if (m == AXHIP_PAD_REFLECT && widest > 0 && widest >= x.shape()[d])
+            throw ValueError("pad: a reflected pad must be shorter than the dimension it reflects");
+        if (m != AXHIP_PAD_CONSTANT && widest > 0 && x.shape()[d] == 0) throw ValueError("pad: nothing to repeat along an empty dimension");
+        out[d] += pad_width[d].first + pad_width[d].second;
+    }
+    return GraphRegistry::create_lazy_pad(x, pad_width, value, out, m);
 }
 
 Tensor embedding(const Tensor &weight, const Tensor &indices) {
@@ -288,32 +297,36 @@ Tensor embedding(const Tensor &weight, const Tensor &indices) {
 }
 
 Tensor conv1d(const Tensor &input, const Tensor &weight, const Tensor &bias, int stride, int padding, int dilation, int groups) {
-    if (groups != 1) throw RuntimeError::not_implemented("grouped conv1d on the GPU");
+    if (groups <= 0) throw ValueError("conv1d: groups must be > 0, got " + std::to_string(groups)); // src/tensor/operations.cpp:2982-3016
     if (stride < 1 || dilation < 1 || padding < 0) throw ValueError("conv1d: stride and dilation must be positive, padding non-negative");
     if (input.ndim() == 2) { // unbatched (C_in, L)
         const Tensor y = conv1d(input.unsqueeze(0), weight, bias, stride, padding, dilation, groups);
         return y.squeeze(0);
     }
-    if (input.ndim() != 3 || weight.ndim() != 3) throw ShapeError("conv1d expects input (N, C_in, L) and weight (C_out, C_in, K)");
-    if (input.shape()[1] != weight.shape()[1])
-        throw ShapeError("conv1d: input has " + std::to_string(input.shape()[1]) + " channels, weight expects " + std::to_string(weight.shape()[1]));
+    if (input.ndim() != 3 || weight.ndim() != 3) throw ShapeError("conv1d expects input (N, C_in, L) and weight (C_out, C_in / groups, K)");
+    if (input.shape()[1] != weight.shape()[1] * static_cast<size_t>(groups))
+        throw ShapeError("conv1d: input has " + std::to_string(input.shape()[1]) + " channels, weight expects " + std::to_string(weight.shape()[1]) +
+                         " per group times " + std::to_string(groups) + " groups");
+    if (weight.shape()[0] % static_cast<size_t>(groups) != 0) throw ShapeError("conv1d: C_out must be divisible by groups");
     if (!bias.empty() && (bias.ndim() != 1 || bias.shape()[0] != weight.shape()[0])) throw ShapeError("conv1d: bias must have shape (C_out)");
-    return GraphRegistry::create_lazy_conv1d(input, weight, bias, stride, padding, dilation);
+    return GraphRegistry::create_lazy_conv1d(input, weight, bias, stride, padding, dilation, groups);
 }
 
 Tensor conv1d(const Tensor &input, const Tensor &weight) { return conv1d(input, weight, Tensor(), 1, 0, 1, 1); }
 
 Tensor conv2d(const Tensor &input, const Tensor &weight, const Tensor &bias, std::array<int, 2> stride, std::array<int, 2> padding,
               std::array<int, 2> dilation, int groups) {
-    if (groups != 1) throw RuntimeError::not_implemented("grouped conv2d on the GPU");
+    if (groups <= 0) throw ValueError("conv2d: groups must be > 0, got " + std::to_string(groups)); // src/tensor/operations.cpp:3153-3189
     for (int i = 0; i < 2; ++i)
         if (stride[i] < 1 || dilation[i] < 1 || padding[i] < 0) throw ValueError("conv2d: stride and dilation must be positive, padding non-negative");
     if (input.ndim() == 3) return conv2d(input.unsqueeze(0), weight, bias, stride, padding, dilation, groups).squeeze(0); // unbatched (C_in, H, W)
-    if (input.ndim() != 4 || weight.ndim() != 4) throw ShapeError("conv2d expects input (N, C_in, H, W) and weight (C_out, C_in, KH, KW)");
-    if (input.shape()[1] != weight.shape()[1])
-        throw ShapeError("conv2d: input has " + std::to_string(input.shape()[1]) + " channels, weight expects " + std::to_string(weight.shape()[1]));
+    if (input.ndim() != 4 || weight.ndim() != 4) throw ShapeError("conv2d expects input (N, C_in, H, W) and weight (C_out, C_in / groups, KH, KW)");
+    if (input.shape()[1] != weight.shape()[1] * static_cast<size_t>(groups))
+        throw ShapeError("conv2d: input has " + std::to_string(input.shape()[1]) + " channels, weight expects " + std::to_string(weight.shape()[1]) +
+                         " per group times " + std::to_string(groups) + " groups");
+    if (weight.shape()[0] % static_cast<size_t>(groups) != 0) throw ShapeError("conv2d: C_out must be divisible by groups");
     if (!bias.empty() && (bias.ndim() != 1 || bias.shape()[0] != weight.shape()[0])) throw ShapeError("conv2d: bias must have shape (C_out)");
-    return GraphRegistry::create_lazy_conv2d(input, weight, bias, stride, padding, dilation);
+    return GraphRegistry::create_lazy_conv2d(input, weight, bias, stride, padding, dilation, groups);
 }
 Tensor conv2d(const Tensor &input, const Tensor &weight) { return conv2d(input, weight, Tensor(), {1, 1}, {0, 0}, {1, 1}, 1); }
 

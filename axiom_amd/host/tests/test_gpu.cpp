@@ -1075,7 +1075,7 @@ GPU_TEST(LazyNodes, Conv1dKnownAnswers) {
     r = ops::conv1d(gpu_f32({1, 2, 3, 4, 5}, {1, 5}), w3); // :92-102, unbatched
     EXPECT_TRUE(r.shape() == Shape({1, 3}));
     EXPECT_NEAR(host_floats(r)[0], 6.0f, 0);
-    EXPECT_THROW(ops::conv1d(x5, w3, Tensor(), 1, 0, 1, 2), RuntimeError);               // groups
+    EXPECT_THROW(ops::conv1d(x5, w3, Tensor(), 1, 0, 1, 2), ShapeError);                 // 1 channel cannot be cut into 2 groups
     EXPECT_THROW(ops::conv1d(x5, gpu_f32({1, 1, 1, 1, 1, 1}, {1, 2, 3})), ShapeError); // channel mismatch
 }
 
@@ -1228,7 +1228,6 @@ GPU_TEST(LazyNodes, PadAndMaskedFill) { // tests/test_shape_ops_extended.cpp:42-
     EXPECT_TRUE(p.shape() == Shape({5, 5}));
     h = host_floats(p);
     EXPECT_NEAR(h[0], 5.0f, 0); EXPECT_NEAR(h[24], 5.0f, 0); EXPECT_NEAR(h[5], 1.0f, 0);
-    EXPECT_THROW(ops::pad(p, {{1, 1}, {1, 1}}, "reflect"), RuntimeError);
     EXPECT_THROW(ops::pad(p, {{1, 1}}), ShapeError);
     // ReLU through masked_fill, and the attention use: a (Sq, Skv) causal mask over (B, H, Sq, Skv) scores
     auto x = axtest::randn({2, 3, 4, 4}, 81);
@@ -1418,6 +1417,108 @@ GPU_TEST(LazyNodes, ProductsAnyAllAndCasts) {
         for (size_t j = 0; j < 100; j += 9) EXPECT_NEAR(tvf[j * 64 + i], float(float16_t(vf[i * 100 + j])), 0);
 }
 
+// Grouped convolutions (tests/test_conv1d.cpp:104-119, tests/test_conv2d.cpp:113-127 give the shapes; the values are
+// checked against float64 loops) and the pad modes other than "constant" (src/tensor/operations.cpp:2216-2246).
+GPU_TEST(LazyNodes, GroupedConvolutions) {
+    {
+        auto input = gpu_f32({1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12}, {1, 4, 3});
+        std::vector<float> ones(8, 1.0f);
+        auto r = ops::conv1d(input, Tensor::from_data(ones.data(), {4, 2, 1}, Device::GPU), Tensor(), 1, 0, 1, 2);
+        EXPECT_TRUE(r.shape() == Shape({1, 4, 3}));
+        EXPECT_TRUE(host_floats(r) == std::vector<float>({5, 7, 9, 5, 7, 9, 17, 19, 21, 17, 19, 21})); // channel pairs summed
+        std::vector<float> in2(36);
+        for (int i = 0; i < 36; ++i) in2[i] = float(i + 1);
+        auto r2 = ops::conv2d(Tensor::from_data(in2.data(), {1, 4, 3, 3}, Device::GPU), Tensor::from_data(ones.data(), {4, 2, 1, 1}, Device::GPU), Tensor(), {1, 1},
+                              {0, 0}, {1, 1}, 2);
+        EXPECT_TRUE(r2.shape() == Shape({1, 4, 3, 3}));
+        auto h2 = host_floats(r2);
+        for (int i = 0; i < 9; ++i) {
+            EXPECT_NEAR(h2[i], in2[i] + in2[9 + i], 0); EXPECT_NEAR(h2[9 + i], in2[i] + in2[9 + i], 0);
+            EXPECT_NEAR(h2[18 + i], in2[18 + i] + in2[27 + i], 0); EXPECT_NEAR(h2[27 + i], in2[18 + i] + in2[27 + i], 0);
+        }
+    }
+    for (DType dt : {DType::Float32, DType::BFloat16}) {
+        const size_t N = 2, Cin = 12, L = 37, Cout = 18, K = 3;
+        for (int groups : {2, 3, 6}) {
+            const size_t Cg = Cin / groups, Og = Cout / groups;
+            const int stride = 2, padding = 1, dilation = 2;
+            auto x = axtest::randn({N, Cin, L}, 130 + groups).astype(dt), w = axtest::randn({Cout, Cg, K}, 140 + groups).astype(dt), b = axtest::randn({Cout}, 150).astype(dt);
+            auto xf = host_floats(x), wf = host_floats(w), bf = host_floats(b);
+            auto y = ops::conv1d(x.gpu(), w.gpu(), b.gpu(), stride, padding, dilation, groups);
+            const size_t Lout = (L + 2 * padding - dilation * (K - 1) - 1) / stride + 1;
+            EXPECT_TRUE(y.shape() == Shape({N, Cout, Lout}));
+            auto got = host_floats(y);
+            const double tol = dt == DType::Float32 ? 1e-4 : 6e-2;
+            for (size_t n = 0; n < N; ++n)
+                for (size_t o = 0; o < Cout; ++o)
+                    for (size_t l = 0; l < Lout; ++l) {
+                        double acc = bf[o];
+                        const size_t g = o / Og;
+                        for (size_t c = 0; c < Cg; ++c)
+                            for (size_t k = 0; k < K; ++k) {
+                                const long pos = long(l * stride + k * dilation) - padding;
+                                if (pos >= 0 && pos < long(L)) acc += double(xf[(n * Cin + g * Cg + c) * L + pos]) * wf[(o * Cg + c) * K + k];
+                            }
+                        EXPECT_NEAR(got[(n * Cout + o) * Lout + l], acc, tol * (1 + std::fabs(acc)));
+                    }
+        }
+    }
+    { // depthwise 2-D (groups == C_in == C_out), no bias
+        const size_t N = 2, C = 5, H = 9, W = 11, KH = 3, KW = 2;
+        auto x = axtest::randn({N, C, H, W}, 160), w = axtest::randn({C, 1, KH, KW}, 161);
+        auto xf = host_floats(x), wf = host_floats(w);
+        auto y = ops::conv2d(x.gpu(), w.gpu(), Tensor(), {1, 2}, {1, 0}, {1, 1}, static_cast<int>(C));
+        const size_t Ho = H + 2 - KH + 1, Wo = (W - KW) / 2 + 1;
+        EXPECT_TRUE(y.shape() == Shape({N, C, Ho, Wo}));
+        auto got = host_floats(y);
+        for (size_t n = 0; n < N; ++n)
+            for (size_t c = 0; c < C; ++c)
+                for (size_t i = 0; i < Ho; ++i)
+                    for (size_t j = 0; j < Wo; ++j) {
+                        double acc = 0;
+                        for (size_t a = 0; a < KH; ++a)
+                            for (size_t bb = 0; bb < KW; ++bb) {
+                                const long r = long(i + a) - 1, q = long(j * 2 + bb);
+                                if (r >= 0 && r < long(H)) acc += double(xf[((n * C + c) * H + r) * W + q]) * wf[(c * KH + a) * KW + bb];
+                            }
+                        EXPECT_NEAR(got[((n * C + c) * Ho + i) * Wo + j], acc, 1e-4);
+                    }
+    }
+    EXPECT_THROW(ops::conv1d(Tensor::zeros({1, 4, 3}, DType::Float32, Device::GPU), Tensor::zeros({4, 2, 1}, DType::Float32, Device::GPU), Tensor(), 1, 0, 1, 0), ValueError);
+    EXPECT_THROW(ops::conv1d(Tensor::zeros({1, 4, 3}, DType::Float32, Device::GPU), Tensor::zeros({4, 2, 1}, DType::Float32, Device::GPU), Tensor(), 1, 0, 1, 4), ShapeError);
+    EXPECT_THROW(ops::conv1d(Tensor::zeros({1, 4, 3}, DType::Float32, Device::GPU), Tensor::zeros({3, 2, 1}, DType::Float32, Device::GPU), Tensor(), 1, 0, 1, 2), ShapeError);
+}
+
+GPU_TEST(LazyNodes, PadModes) {
+    auto x = gpu_f32({1, 2, 3, 4}, {4});
+    EXPECT_TRUE(host_floats(ops::pad(x, {{2, 3}}, "reflect")) == std::vector<float>({3, 2, 1, 2, 3, 4, 3, 2, 1}));
+    EXPECT_TRUE(host_floats(ops::pad(x, {{2, 3}}, "replicate")) == std::vector<float>({1, 1, 1, 2, 3, 4, 4, 4, 4}));
+    EXPECT_TRUE(host_floats(ops::pad(x, {{2, 5}}, "circular")) == std::vector<float>({3, 4, 1, 2, 3, 4, 1, 2, 3, 4, 1}));
+    EXPECT_THROW(ops::pad(x, {{4, 0}}, "reflect"), ValueError);
+    EXPECT_THROW(ops::pad(x, {{1, 1}}, "mirror"), ValueError);
+    auto idx = [](long c, long n, int mode) { // the reference's get_source_idx
+        if (c >= 0 && c < n) return c;
+        if (mode == 1) return c < 0 ? -c : 2 * n - c - 2;
+        if (mode == 2) return c < 0 ? 0L : n - 1;
+        return ((c % n) + n) % n;
+    };
+    const char *names[4] = {"constant", "reflect", "replicate", "circular"};
+    for (DType dt : {DType::Float32, DType::Float16}) {
+        auto v = axtest::randn({3, 6, 40}, 170).astype(dt);
+        auto vf = host_floats(v);
+        for (int mode = 1; mode <= 3; ++mode) {
+            auto got = host_floats(ops::pad(v.gpu().transpose({1, 0, 2}), {{1, 2}, {2, 0}, {3, 5}}, names[mode])); // a (6, 3, 40) view -> (9, 5, 48)
+            ASSERT_EQ(got.size(), size_t(9 * 5 * 48));
+            for (long a = 0; a < 9; ++a)
+                for (long b = 0; b < 5; ++b)
+                    for (long c = 0; c < 48; ++c) {
+                        const long sa = idx(a - 1, 6, mode), sb = idx(b - 2, 3, mode), sc = idx(c - 3, 40, mode);
+                        EXPECT_NEAR(got[(a * 5 + b) * 48 + c], vf[(sb * 6 + sa) * 40 + sc], 0);
+                    }
+        }
+    }
+}
+
 GPU_TEST(LazyNodes, BatchNorm1dInference) {
     const size_t N = 3, C = 5, L = 7;
     auto w = axtest::uniform({C}, 90, 0.5f, 1.5f), b = axtest::randn({C}, 91), rm = axtest::randn({C}, 92), rv = axtest::uniform({C}, 93, 0.2f, 2.0f);
@@ -1542,7 +1643,7 @@ GPU_TEST(LazyNodes, Conv2dKnownAnswers) { // tests/test_conv2d.cpp:3-111 of the 
     r = ops::conv2d(gpu_f32({1, 2, 3, 4, 5, 6, 7, 8, 9}, {1, 3, 3}), w4); // unbatched
     EXPECT_TRUE(r.shape() == Shape({1, 2, 2}));
     EXPECT_NEAR(host_floats(r)[0], 12.0f, 0);
-    EXPECT_THROW(ops::conv2d(x9, w4, Tensor(), {1, 1}, {0, 0}, {1, 1}, 2), RuntimeError); // groups
+    EXPECT_THROW(ops::conv2d(x9, w4, Tensor(), {1, 1}, {0, 0}, {1, 1}, 2), ShapeError); // 1 channel cannot be cut into 2 groups
 }
 
 GPU_TEST(LazyNodes, Conv2dMatchesFloat64Loops) {

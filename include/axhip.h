@@ -330,6 +330,17 @@ int axhip_fill(void *dst, int32_t dtype, double value, int64_t count, void *stre
 int axhip_pad(const void *src, void *dst, int32_t dtype, int32_t ndim, const int64_t *src_shape_host,
               const int64_t *src_strides_host, const int64_t *pad_before_host,
               const int64_t *pad_after_host, double value, void *stream);
+/* The other modes of ops::pad (src/tensor/operations.cpp:2216-2246): reflect
+ * (the border element is not repeated; each pad must be shorter than the
+ * extent it reflects), replicate (the border element repeated) and circular
+ * (wrap around); `value` only matters for AXHIP_PAD_CONSTANT. */
+#define AXHIP_PAD_CONSTANT 0
+#define AXHIP_PAD_REFLECT 1
+#define AXHIP_PAD_REPLICATE 2
+#define AXHIP_PAD_CIRCULAR 3
+int axhip_pad_mode(const void *src, void *dst, int32_t dtype, int32_t ndim, const int64_t *src_shape_host,
+                   const int64_t *src_strides_host, const int64_t *pad_before_host,
+                   const int64_t *pad_after_host, int32_t mode, double value, void *stream);
 
 /* masked_fill (include/axiom/operations.hpp:437-440): dst[i] = mask[i] ? value :
  * src[i] over an iteration space of <= 8 dims; src and the byte mask (Bool:

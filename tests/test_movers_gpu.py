@@ -120,6 +120,35 @@ def test_pad_matches_numpy(dt, shape, before, after):
     assert np.array_equal(gh.to_host(out, x.dtype), want)
 
 
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("mode,np_mode", [("reflect", "reflect"), ("replicate", "edge"), ("circular", "wrap")])
+@pytest.mark.parametrize("shape,before,after", [((5,), (2,), (3,)), ((3, 4), (0, 1), (2, 0)), ((3, 5, 27), (1, 0, 2), (0, 2, 3)),
+                                                ((2, 2, 30, 48), (0, 1, 0, 7), (1, 0, 0, 9)), ((7, 1001), (3, 0), (0, 23))])
+def test_pad_modes_match_numpy(dt, mode, np_mode, shape, before, after):
+    """reflect / replicate / circular as the reference indexes them (src/tensor/operations.cpp:2216-2246), which is
+    what numpy's 'reflect' / 'edge' / 'wrap' do."""
+    x = sample(shape, dt, 13)
+    want = np.pad(x, list(zip(before, after)), mode=np_mode)
+    d = gh.to_dev(x)
+    out = gh.empty_dev(want.shape, dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_pad_mode(d.data_ptr(), out.data_ptr(), dt, x.ndim, i64(shape), i64(elem_strides(x)), i64(before), i64(after),
+                                         capi.PAD[mode], 0.0, None))
+    gh.sync()
+    assert np.array_equal(gh.to_host(out, x.dtype), want)
+
+
+def test_pad_mode_errors():
+    x = gh.to_dev(np.zeros((4,), np.float32))
+    out = gh.empty_dev((12,), F32)
+    l = capi.lib()
+    assert l.axhip_pad_mode(x.data_ptr(), out.data_ptr(), F32, 1, i64([4]), i64([1]), i64([4]), i64([4]), capi.PAD["reflect"], 0.0, None) == capi.ERR_INVALID_ARG
+    assert l.axhip_pad_mode(x.data_ptr(), out.data_ptr(), F32, 1, i64([4]), i64([1]), i64([4]), i64([4]), 4, 0.0, None) == capi.ERR_INVALID_ARG
+    assert l.axhip_pad_mode(x.data_ptr(), out.data_ptr(), F32, 1, i64([0]), i64([1]), i64([1]), i64([1]), capi.PAD["replicate"], 0.0, None) == capi.ERR_INVALID_ARG
+    assert l.axhip_pad_mode(x.data_ptr(), out.data_ptr(), F32, 1, i64([4]), i64([1]), i64([4]), i64([4]), capi.PAD["circular"], 0.0, None) == 0
+    gh.sync()
+
+
 def test_pad_of_a_transposed_view():
     base = sample((4, 6), F32, 12)
     view = base.T
