@@ -2,6 +2,7 @@
 #include "rows_codegen.hpp"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -446,8 +447,19 @@ bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, Ro
         // the tightest fit among 64, 256, 512 and 1024 threads per row with up to 8 chunks each: fewest chunk slots (idle lanes
         // still issue their loads and arithmetic), then the smaller group
         static const int groups[4] = {64, 256, 512, 1024};
+        // AXHIP_ROWS_GROUP (64, 256, 512, 1024; read once): take that many threads per row wherever the row fits them with up
+        // to 8 chunks each -- a tuning switch for measurements, the default choice below is what the benchmarks ran
+        static const int forced = [] {
+            const char *e = std::getenv("AXHIP_ROWS_GROUP");
+            return e ? std::atoi(e) : 0;
+        }();
         int64_t best = 0;
         for (int i = 0; i < 4; ++i) {
+            if (forced == groups[i] && (chunks + groups[i] - 1) / groups[i] <= 8 && chunks >= groups[i]) {
+                group = groups[i];
+                it = static_cast<int>((chunks + groups[i] - 1) / groups[i]);
+                break;
+            }
             const int64_t n = (chunks + groups[i] - 1) / groups[i];
             // up to 8 chunks per thread; a wavefront row may take 9 or 10 (a row just past 512 chunks would otherwise
             // leave a third of a 256-thread block idle) while its registers still allow 4 waves per SIMD

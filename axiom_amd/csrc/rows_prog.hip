@@ -122,7 +122,8 @@ Entry *find_or_make_entry(const AxhipRowsProgram &P) {
                            rows_prog_find_builtin(stock_spec.config + stock_spec.chains) != nullptr;
     e->eligible = has_tight || has_stock;
     e->has_builtin_alternative = false;
-    if (has_stock && (!has_tight || stock.slots() * 100 <= tight.slots() * 115)) {
+    static const bool forced_group = getenv("AXHIP_ROWS_GROUP") != nullptr; // (the tuning switch of the tight plan wins over the built-in shapes)
+    if (has_stock && (!has_tight || (!forced_group && stock.slots() * 100 <= tight.slots() * 115))) {
         e->spec = stock_spec;
         e->is_builtin = true;
     } else if (has_tight) {

@@ -26,7 +26,7 @@ WORKLOADS = {
     "chain_gelu_layernorm_bf16_16384x4096": ("layernorm_gelu_wb_bf16", 2 * 16384 * 4096 * 2 + 2 * 4096 * 2),
     "chain_gelu_rmsnorm_bf16_16384x4096": ("rmsnorm_gelu_w_bf16", 2 * 16384 * 4096 * 2 + 4096 * 2),
     "softmax_bf16_30000x1500_odd_row_length": ("axp_softmax_bf16_g64_it3_grid", 2 * 30000 * 1500 * 2),
-    "sdpa_bf16_causal_b4h32s4096d128": ("sdpa_mfma_pipelined_kernel<true, false, 8, 128, 1, false>", 4 * 4 * 32 * 4096 * 128 * 2),
+    "sdpa_bf16_causal_b4h32s4096d128": ("sdpa_mfma_pingpong_kernel<true, 128>", 4 * 4 * 32 * 4096 * 128 * 2),
 }
 CALIBRATION = "copy_f32_8192x8192"
 

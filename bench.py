@@ -272,7 +272,32 @@ def bench_chains(torch, capi, stream, steps, warmup):
         rec = _chain_record(lib, capi, progs[0], avg_ms, min_ms, warm_n, cold_ms, cold_min, n_sets, set_bytes, nbytes)
         rec["finite"] = bool(all(torch.isfinite(y.float()).all().item() for y in ys))
         res[f"chain_gelu_{name}_bf16_16384x4096"] = rec
-    del xs, ys
+    # What the memory system gives a one-read-one-write stream of this size when nothing is found in the caches: the
+    # runtime's own device-to-device copy (hipMemcpyAsync behind axhip_memcpy_d2d_async) and the library's elementwise
+    # copy kernel (an empty chain), on the same rotation of 128 MiB buffers as the norm chains above
+    copy_launchers = [(lambda x=x, y=y: capi.check(lib.axhip_memcpy_d2d_async(y.data_ptr(), x.data_ptr(), R * Cc * 2, sp))) for x, y in zip(xs, ys)]
+    cold_ms, cold_min, _ = time_rotating(torch, stream, copy_launchers, steps, warmup)
+    same_ms, _, _ = time_launches(torch, stream, copy_launchers[0], steps, warmup)
+    nbytes = 2 * R * Cc * 2
+    res["hbm_copy_reference_128MiB"] = {
+        "what": "hipMemcpyAsync device-to-device, 128 MiB in + 128 MiB out per launch, same buffer rotation as the norm chains",
+        "avg_ms": cold_ms, "min_ms": cold_min, "bytes": nbytes, "buffer_sets": n_sets,
+        "frac_of_hbm_peak_cold": nbytes / (cold_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "frac_of_hbm_peak_same_buffers": nbytes / (same_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+    }
+    progs = [_rows_program(capi, x, y, capi.DTYPE_BF16, capi.DTYPE_BF16) for x, y in zip(xs, ys)]
+    ew_launchers = [(lambda q=q: capi.check(lib.axhip_fused_rows(C.byref(q), sp))) for q in progs]
+    cold_ms, cold_min, _ = time_rotating(torch, stream, ew_launchers, steps, warmup)
+    same_ms, _, _ = time_launches(torch, stream, ew_launchers[0], steps, warmup)
+    res["elementwise_copy_bf16_16384x4096"] = {
+        "kernel": lib.axhip_fused_rows_kernel_name(C.byref(progs[0])).decode(), "avg_ms": cold_ms, "min_ms": cold_min, "bytes": nbytes, "buffer_sets": n_sets,
+        "frac_of_hbm_peak_cold": nbytes / (cold_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "frac_of_hbm_peak_same_buffers": nbytes / (same_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "bit_exact": bool(torch.equal(ys[0], xs[0])),
+    }
+    for name in ("chain_gelu_layernorm_bf16_16384x4096", "chain_gelu_rmsnorm_bf16_16384x4096"):
+        res[name]["frac_of_cold_copy_reference"] = res[name]["frac_of_hbm_peak_cold"] / res["hbm_copy_reference_128MiB"]["frac_of_hbm_peak_cold"]
+    del xs, ys, progs
     # a row length that the 16-byte vector does not divide (Whisper's 1500 frames): the kernels' ragged variant
     Rr, Cr = 30000, 1500
     set_bytes = 2 * Rr * Cr * 2
