@@ -10,11 +10,12 @@ namespace axhip {
 constexpr float NEG_INF = -__builtin_huge_valf();
 constexpr float POS_INF = __builtin_huge_valf();
 
-// The wider operator table (codes from AXHIP_OP_POW up) as ONE function that the chain interpreters call per value:
-// inlined into every arm of every interpreter kernel, its 32 operations (powf, fmodf, the trigonometric routines ...)
-// multiplied the build time and the code size of this file by five.  The call is made once per wavefront for 64
-// values and the switch inside is a scalar branch: far below the cost of the memory accesses around it.  The
-// compiled row programs have these operations inline.
+// The long library routines of the wider operator table (powf, fmodf, atan2f, hypotf, erff, the trigonometric
+// functions, cbrtf) as ONE function that the chain interpreters call per value: inlined into every arm of every
+// interpreter kernel they multiplied the build time and the code size of this file by five.  A chain through this
+// call runs at about 40 % of the HBM peak; comparisons, logical operations, rounding and the is* tests are inline
+// arms like the first table's.  (The switch also lists those, for callers that come here with any extended code.)
+// The compiled row programs have all of them inline.
 __device__ __attribute__((noinline)) inline float extended_op(int op, float a, float b) {
     switch (op) {
     case AXHIP_OP_POW: return powf(a, b);
@@ -70,6 +71,15 @@ __device__ __forceinline__ float apply_unary(int op, float a) {
     case AXHIP_OP_SQUARE: return a * a;
     case AXHIP_OP_RSQRT: return 1.0f / sqrtf(a);
     case AXHIP_OP_RECIP: return 1.0f / a;
+    case AXHIP_OP_SIGN: return a > 0.0f ? 1.0f : a < 0.0f ? -1.0f : 0.0f;
+    case AXHIP_OP_FLOOR: return floorf(a);
+    case AXHIP_OP_CEIL: return ceilf(a);
+    case AXHIP_OP_ROUND: return roundf(a);
+    case AXHIP_OP_TRUNC: return truncf(a);
+    case AXHIP_OP_ISNAN: return a != a ? 1.0f : 0.0f;
+    case AXHIP_OP_ISINF: return fabsf(a) == POS_INF ? 1.0f : 0.0f;
+    case AXHIP_OP_ISFINITE: return fabsf(a) < POS_INF ? 1.0f : 0.0f;
+    case AXHIP_OP_NOT: return a == 0.0f ? 1.0f : 0.0f;
     default: return op >= AXHIP_OP_POW ? extended_op(op, a, 0.0f) : a;
     }
 }
@@ -84,6 +94,16 @@ __device__ __forceinline__ float apply_binary(int op, float a, float b) {
     case AXHIP_OP_MIN: return fminf(a, b);
     case AXHIP_OP_RSUB: return b - a;
     case AXHIP_OP_RDIV: return b / a;
+    case AXHIP_OP_EQ: return a == b ? 1.0f : 0.0f;
+    case AXHIP_OP_NE: return a != b ? 1.0f : 0.0f;
+    case AXHIP_OP_LT: return a < b ? 1.0f : 0.0f;
+    case AXHIP_OP_LE: return a <= b ? 1.0f : 0.0f;
+    case AXHIP_OP_GT: return a > b ? 1.0f : 0.0f;
+    case AXHIP_OP_GE: return a >= b ? 1.0f : 0.0f;
+    case AXHIP_OP_AND: return (a != 0.0f) && (b != 0.0f) ? 1.0f : 0.0f;
+    case AXHIP_OP_OR: return (a != 0.0f) || (b != 0.0f) ? 1.0f : 0.0f;
+    case AXHIP_OP_XOR: return (a != 0.0f) != (b != 0.0f) ? 1.0f : 0.0f;
+    case AXHIP_OP_LEAKY_RELU: return a > 0.0f ? a : b * a;
     default: return op >= AXHIP_OP_POW ? extended_op(op, a, b) : a;
     }
 }
@@ -141,7 +161,16 @@ __device__ __forceinline__ void apply_unary_tile(int op, float (&v)[IT][E]) {
         AXHIP_UNARY_CASE(AXHIP_OP_SQUARE);
         AXHIP_UNARY_LONG(AXHIP_OP_RSQRT);
         AXHIP_UNARY_LONG(AXHIP_OP_RECIP);
-    default:
+        AXHIP_UNARY_CASE(AXHIP_OP_SIGN);
+        AXHIP_UNARY_CASE(AXHIP_OP_FLOOR);
+        AXHIP_UNARY_CASE(AXHIP_OP_CEIL);
+        AXHIP_UNARY_CASE(AXHIP_OP_ROUND);
+        AXHIP_UNARY_CASE(AXHIP_OP_TRUNC);
+        AXHIP_UNARY_CASE(AXHIP_OP_ISNAN);
+        AXHIP_UNARY_CASE(AXHIP_OP_ISINF);
+        AXHIP_UNARY_CASE(AXHIP_OP_ISFINITE);
+        AXHIP_UNARY_CASE(AXHIP_OP_NOT);
+    default: // the long library routines, through one call per value
         if (op >= AXHIP_OP_ERF) for_each_value<IT, E>(v, [op](float a, int, int) { return extended_op(op, a, 0.0f); });
         break;
     }
@@ -165,7 +194,17 @@ __device__ __forceinline__ void apply_binary_tile(int op, float (&v)[IT][E], W w
         AXHIP_BINARY_CASE(AXHIP_OP_MIN);
         AXHIP_BINARY_CASE(AXHIP_OP_RSUB);
         AXHIP_BINARY_LONG(AXHIP_OP_RDIV);
-    default:
+        AXHIP_BINARY_CASE(AXHIP_OP_EQ);
+        AXHIP_BINARY_CASE(AXHIP_OP_NE);
+        AXHIP_BINARY_CASE(AXHIP_OP_LT);
+        AXHIP_BINARY_CASE(AXHIP_OP_LE);
+        AXHIP_BINARY_CASE(AXHIP_OP_GT);
+        AXHIP_BINARY_CASE(AXHIP_OP_GE);
+        AXHIP_BINARY_CASE(AXHIP_OP_AND);
+        AXHIP_BINARY_CASE(AXHIP_OP_OR);
+        AXHIP_BINARY_CASE(AXHIP_OP_XOR);
+        AXHIP_BINARY_CASE(AXHIP_OP_LEAKY_RELU);
+    default: // the long library routines, through one call per value
         if (op >= AXHIP_OP_POW) for_each_value<IT, E>(v, [&](float a, int it, int e) { return extended_op(op, a, w(it, e)); });
         break;
     }

@@ -154,6 +154,39 @@ def _rows_program(capi, x, out, dt, out_dt):
 COLD_MIN_BYTES = 1 << 30  # bytes of other buffers touched between two uses of one buffer set in the rotating ("cold") timing
 
 
+class ColdTimer:
+    """Duration of single launches whose inputs come from HBM: between two timed launches a reduction reads 1 GiB of
+    other data through the caches (read only: a flush that writes leaves hundreds of MiB of modified lines behind,
+    whose write-back then competes with the launch that is being timed).  Every launch is bracketed by two HIP events
+    of its own; what that bracketing adds to a launch is measured once per use (the same bracketing without the
+    flush, against the back-to-back average) and taken off."""
+
+    def __init__(self, torch, stream):
+        self.torch, self.stream = torch, stream
+        self.src = torch.zeros((1 << 30) // 4, device="cuda", dtype=torch.float32)
+        self.acc = torch.zeros((), device="cuda", dtype=torch.float32)
+
+    def _bracketed(self, launch, steps, flush):
+        torch, stream = self.torch, self.stream
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        with torch.cuda.stream(stream):
+            for e0, e1 in pairs:
+                if flush:
+                    torch.amax(self.src, dim=0, out=self.acc)
+                e0.record(stream)
+                launch()
+                e1.record(stream)
+            stream.synchronize()
+        t = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+        return t[len(t) // 2]
+
+    def cold_ms(self, launch, steps, hot_avg_ms):
+        """median cold launch in ms, and the event overhead that was taken off"""
+        steps = max(steps, 20)
+        overhead = max(0.0, self._bracketed(launch, steps, False) - hot_avg_ms)
+        return max(self._bracketed(launch, steps, True) - overhead, 1e-6), overhead
+
+
 def time_rotating(torch, stream, launchers, steps, warmup):
     """Average launch duration in ms over exactly `steps` launches that rotate through `launchers` (the same program
     over independent buffer sets, sized by the caller so that at least COLD_MIN_BYTES of other data pass through the
@@ -390,13 +423,24 @@ def bench_survey(torch, capi, stream, steps, warmup):
     def rnd(shape, dtype, scale=1.0, shift=0.0):
         return (torch.randn(shape, generator=g, device="cuda") * scale + shift).to(dtype)
 
+    cold = ColdTimer(torch, stream)
+
+    def with_cold(rec, launch, avg_ms, nbytes):
+        # the same launch with its inputs flushed out of the caches first (frac_of_hbm_peak is the back-to-back figure)
+        cold_ms, overhead_ms = cold.cold_ms(launch, steps, avg_ms)
+        rec["cold_us"] = cold_ms * 1e3
+        rec["event_overhead_us"] = overhead_ms * 1e3
+        rec["frac_of_hbm_peak_cold"] = nbytes / (cold_ms * 1e-3) / 1e9 / PEAK_HBM_GBS
+        return rec
+
     def run(name, prog):
         lib.axhip_fused_rows_prepare(C.byref(prog.p))
         torch.cuda.synchronize()
-        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_fused_rows(C.byref(prog.p), sp)), steps, warmup)
-        res[name] = {"kernel": lib.axhip_fused_rows_kernel_name(C.byref(prog.p)).decode(), "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3,
-                     "bytes": prog.bytes, "frac_of_hbm_peak": prog.bytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                     "finite": bool(torch.isfinite(prog.out.float()).all().item())}
+        launch = lambda: capi.check(lib.axhip_fused_rows(C.byref(prog.p), sp))
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
+        res[name] = with_cold({"kernel": lib.axhip_fused_rows_kernel_name(C.byref(prog.p)).decode(), "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3,
+                               "bytes": prog.bytes, "frac_of_hbm_peak": prog.bytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                               "finite": bool(torch.isfinite(prog.out.float()).all().item())}, launch, avg_ms, prog.bytes)
 
     bf, f32 = torch.bfloat16, torch.float32
     R, Cc = 16384, 4096
@@ -439,6 +483,32 @@ def bench_survey(torch, capi, stream, steps, warmup):
     run(f"gelu(layernorm(a+b))_{tag}", P(a).op("add", c).row("layernorm", w32, b32).op("gelu").finish(torch))
     run(f"sum(a)_{tag}", P(a).finish(torch, "sum"))
     del a, c
+    # the wider operator table: a comparison to a Bool array, where() on it, a leaky ReLU chain, any() per row
+    xb, yb = rnd((16384, 4096), bf), rnd((16384, 4096), bf)
+    mask = torch.empty((16384, 4096), device="cuda", dtype=torch.uint8)
+    pg = _Prog(capi, xb)
+    pg.op("gt", yb)
+    pg.p.output, pg.p.output_dtype, pg.p.reduce = mask.data_ptr(), capi.DTYPE_U8, capi.RED["none"]
+    pg.out, pg.bytes = mask, 2 * xb.numel() * 2 + mask.numel()
+    run("x>y_to_bool_bf16_16384x4096", pg)
+    run("leaky_relu(x)*y_bf16_16384x4096", _Prog(capi, xb).op("leaky_relu", imm=0.01).op("mul", yb).finish(torch))
+    anyout = torch.empty((16384,), device="cuda", dtype=torch.uint8)
+    pa = _Prog(capi, xb)
+    pa.op("gt", imm=3.5)
+    pa.p.output, pa.p.output_dtype, pa.p.reduce = anyout.data_ptr(), capi.DTYPE_U8, capi.RED["max"]
+    pa.out, pa.bytes = anyout, xb.numel() * 2 + anyout.numel()
+    run("any(x>3.5)_bf16_16384x4096", pa)
+    wout = torch.empty_like(xb)
+    shp, st = (C.c_int64 * 2)(16384, 4096), (C.c_int64 * 2)(4096, 1)
+    launch = lambda: capi.check(lib.axhip_where(mask.data_ptr(), capi.DTYPE_U8, xb.data_ptr(), capi.DTYPE_BF16, yb.data_ptr(), capi.DTYPE_BF16, wout.data_ptr(),
+                                               capi.DTYPE_BF16, 2, shp, st, st, st, sp))
+    torch.cuda.synchronize()
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
+    nbytes = 3 * xb.numel() * 2 + mask.numel()
+    res["where(mask,x,y)_bf16_16384x4096"] = with_cold(
+        {"kernel": "where_vec", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+         "finite": bool(torch.equal(wout, torch.where(mask.bool(), xb, yb)))}, launch, avg_ms, nbytes)
+    del xb, yb, mask, wout
     # rows of odd length
     for rows, cols, dt, name in ((30000, 1500, bf, "bf16"), (16384, 4100, bf, "bf16"), (16384, 4097, bf, "bf16"), (16384, 1501, f32, "f32")):
         t = rnd((rows, cols), dt)
@@ -480,11 +550,13 @@ def bench_survey(torch, capi, stream, steps, warmup):
         out = torch.empty((outer * inner,), device="cuda", dtype=torch.int64)
         code = capi.DTYPE_BF16 if dt == bf else capi.DTYPE_F32
         torch.cuda.synchronize()
-        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_argreduce(t.data_ptr(), code, outer, axis, inner, 0, out.data_ptr(), sp)), steps, warmup)
+        launch = lambda: capi.check(lib.axhip_argreduce(t.data_ptr(), code, outer, axis, inner, 0, out.data_ptr(), sp))
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
         nbytes = t.numel() * t.element_size() + out.numel() * 8
-        res[f"argmax_axis1_{name}_{outer}x{axis}x{inner}"] = {"kernel": "argreduce_rows" if inner == 1 else "argreduce_strided", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3,
-                                                               "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                                                               "finite": bool(torch.equal(out.view(outer, inner), t.float().argmax(1)))}
+        res[f"argmax_axis1_{name}_{outer}x{axis}x{inner}"] = with_cold(
+            {"kernel": "argreduce_rows" if inner == 1 else "argreduce_strided", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+             "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.equal(out.view(outer, inner), t.float().argmax(1)))},
+            launch, avg_ms, nbytes)
         del t, out
     # reductions and softmax along an inner axis of a contiguous array (no transposing copy)
     for (outer, axis, inner), dt, name in (((1, 4096, 16384), f32, "f32"), ((64, 4096, 1024), bf, "bf16"), ((8192, 8, 1024), f32, "f32")):
@@ -492,16 +564,20 @@ def bench_survey(torch, capi, stream, steps, warmup):
         code = capi.DTYPE_BF16 if dt == bf else capi.DTYPE_F32
         out = torch.empty((outer, inner), device="cuda", dtype=dt)
         torch.cuda.synchronize()
-        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_reduce_axis(t.data_ptr(), code, outer, axis, inner, capi.RED["sum"], out.data_ptr(), code, sp)), steps, warmup)
+        launch = lambda: capi.check(lib.axhip_reduce_axis(t.data_ptr(), code, outer, axis, inner, capi.RED["sum"], out.data_ptr(), code, sp))
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
         nbytes = (t.numel() + out.numel()) * t.element_size()
-        res[f"sum_axis1_{name}_{outer}x{axis}x{inner}"] = {"kernel": "reduce_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
-                                                            "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(out.float()).all().item())}
+        res[f"sum_axis1_{name}_{outer}x{axis}x{inner}"] = with_cold(
+            {"kernel": "reduce_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+             "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(out.float()).all().item())}, launch, avg_ms, nbytes)
         full = torch.empty_like(t)
         torch.cuda.synchronize()
-        avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_softmax_axis(t.data_ptr(), code, outer, axis, inner, 0, full.data_ptr(), sp)), steps, warmup)
+        launch = lambda: capi.check(lib.axhip_softmax_axis(t.data_ptr(), code, outer, axis, inner, 0, full.data_ptr(), sp))
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
         nbytes = 2 * t.numel() * t.element_size()
-        res[f"softmax_axis1_{name}_{outer}x{axis}x{inner}"] = {"kernel": "softmax_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
-                                                                "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(full.float()).all().item())}
+        res[f"softmax_axis1_{name}_{outer}x{axis}x{inner}"] = with_cold(
+            {"kernel": "softmax_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+             "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(full.float()).all().item())}, launch, avg_ms, nbytes)
         del t, out, full
     return res
 
