@@ -545,9 +545,12 @@ namespace axhip {
 // reduce_strided_vec_kernel.  One sweep gathers a running maximum and the sum of 2^(x log2(e) - maximum) per inner
 // position (rescaled once per four elements), the thread rows merge their pairs through LDS, a second sweep over the
 // same elements writes the result: two reads of the input (the second mostly from the caches) and one write.
-template <bool LOG, int DT, int TX>
+// HOLD > 0 (with TX = 256, a thread per vector walking the axis alone): the axis has at most HOLD elements and the thread
+// keeps them in registers between the two sweeps -- one read of the input.
+template <bool LOG, int DT, int TX, int HOLD = 0>
 __global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, void *dst) {
     constexpr int TY = 256 / TX, U = 4, V = DT == AXHIP_DTYPE_F32 ? 4 : 8;
+    static_assert(HOLD == 0 || (TX == 256 && HOLD % U == 0), "rows held in registers: one thread per vector");
     constexpr float LOG2E = 1.44269504088896340736f, LN2 = 0.69314718055994530942f;
     __shared__ float sm[TY][TX][V + 1], sl[TY][TX][V + 1];
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -563,11 +566,14 @@ __global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *sr
             m[e] = -INFINITY;
             l[e] = 0.0f;
         }
-        if (there)
-            for (int k = ty; k < n; k += TY * U) {
-                uint4_t raw[U];
+        uint4_t keep[HOLD > 0 ? HOLD : 1];
+        if constexpr (HOLD > 0) {
+            if (there) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+                for (int k = 0; k < HOLD; ++k) keep[k] = first[static_cast<int64_t>(min(k, n - 1)) * ivecs];
+            }
+        }
+        auto gather = [&](int k, const uint4_t (&raw)[U]) { // running maximum and rescaled sum over U axis elements
                 float t[U][V];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -585,7 +591,24 @@ __global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *sr
                     l[e] = l[e] * __builtin_amdgcn_exp2f(m[e] - ref) + add;
                     m[e] = mx;
                 }
+        };
+        if (there) {
+            if constexpr (HOLD > 0) {
+#pragma unroll
+                for (int k = 0; k < HOLD; k += U)
+                    if (k < n) {
+                        const uint4_t raw[U] = {keep[k], keep[k + 1], keep[k + 2], keep[k + 3]};
+                        gather(k, raw);
+                    }
+            } else {
+                for (int k = ty; k < n; k += TY * U) {
+                    uint4_t raw[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+                    gather(k, raw);
+                }
             }
+        }
         __syncthreads(); // the previous group's pairs have been read
 #pragma unroll
         for (int e = 0; e < V; ++e) {
@@ -604,11 +627,7 @@ __global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *sr
             shift[e] = LOG ? M + __builtin_amdgcn_logf(L) : M; // (v_log_f32 is the base-2 logarithm)
             inv[e] = 1.0f / L;
         }
-        if (there)
-            for (int k = ty; k < n; k += TY * U) {
-                uint4_t raw[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+        auto emit = [&](int k, const uint4_t (&raw)[U]) {
 #pragma unroll
                 for (int u = 0; u < U; ++u)
                     if (k + u * TY < n) {
@@ -618,7 +637,24 @@ __global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *sr
                         for (int e = 0; e < V; ++e) v[e] = LOG ? (v[e] * LOG2E - shift[e]) * LN2 : __builtin_amdgcn_exp2f(v[e] * LOG2E - shift[e]) * inv[e];
                         store_vec<V>(dst, DT, (o * axis + k + u * TY) * inner + iv * V, v);
                     }
+        };
+        if (there) {
+            if constexpr (HOLD > 0) {
+#pragma unroll
+                for (int k = 0; k < HOLD; k += U)
+                    if (k < n) {
+                        const uint4_t raw[U] = {keep[k], keep[k + 1], keep[k + 2], keep[k + 3]};
+                        emit(k, raw);
+                    }
+            } else {
+                for (int k = ty; k < n; k += TY * U) {
+                    uint4_t raw[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) raw[u] = first[static_cast<int64_t>(min(k + u * TY, n - 1)) * ivecs];
+                    emit(k, raw);
+                }
             }
+        }
     }
 }
 
@@ -1164,7 +1200,8 @@ int axhip_softmax_axis(const void *src, int32_t dtype, int64_t outer, int64_t ax
 #define AXHIP_SM_TX(LOG, DT, TX) hipLaunchKernelGGL((softmax_strided_vec_kernel<LOG, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, dst)
 #define AXHIP_SM_DT(LOG, DT)                                                                                                               \
     do {                                                                                                                                   \
-        if (flat) AXHIP_SM_TX(LOG, DT, 256);                                                                                               \
+        if (flat && axis <= 16) hipLaunchKernelGGL((softmax_strided_vec_kernel<LOG, DT, 256, 16>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, dst); \
+        else if (flat) AXHIP_SM_TX(LOG, DT, 256);                                                                                          \
         else if (wide) AXHIP_SM_TX(LOG, DT, 32);                                                                                           \
         else AXHIP_SM_TX(LOG, DT, 8);                                                                                                      \
     } while (0)

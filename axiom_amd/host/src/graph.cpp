@@ -2,6 +2,7 @@
 // the pending list, the structural signature and GraphRegistry::materialize
 // (behaviour of src/graph/graph_registry.cpp and graph_signature.cpp for the hot-path ops).
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <string>
@@ -221,6 +222,16 @@ Tensor GraphRegistry::create_lazy_cast(const Tensor &input, DType target) {
 
 Tensor GraphRegistry::create_lazy_reduction(ops::OpType op, const Tensor &input, const std::vector<int> &axes, bool keep_dims) {
     require_gpu(pick_device({&input}), op);
+    // Nothing to read: an empty result stays empty; a reduction over an empty extent gives the operation's identity
+    // (sum 0, product 1, mean 0/0), and there is no largest or smallest element of nothing.
+    if (ShapeUtils::size(input.shape()) == 0) {
+        const Shape wanted = infer_reduction_shape(input.shape(), axes, keep_dims);
+        const DType rd = infer_reduction_dtype(op, input.dtype());
+        if (ShapeUtils::size(wanted) == 0) return Tensor(wanted, rd, Device::GPU);
+        if (op == ops::OpType::Max || op == ops::OpType::Min) throw ValueError(std::string("ops::") + ops::op_name(op) + " over an empty axis");
+        const double identity = op == ops::OpType::Prod ? 1.0 : op == ops::OpType::Mean ? std::nan("") : 0.0;
+        return Tensor::full(wanted, static_cast<float>(identity), Device::CPU).astype(rd).to(Device::GPU);
+    }
     // The device reduces over the last axis or over everything.  Any other set of axes is brought there first: the
     // kept axes in front, the reduced ones behind them and folded into one (a transposed view that the planner
     // gathers into a contiguous array), then the result takes the shape the caller asked for.

@@ -194,11 +194,22 @@ Tensor max(const Tensor &x, const std::vector<int> &axes, bool keep) { return Gr
 Tensor min(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Min, x, axes, keep); }
 Tensor prod(const Tensor &x, const std::vector<int> &axes, bool keep) { return GraphRegistry::create_lazy_reduction(OpType::Prod, x, axes, keep); }
 // Bool results (src/graph/graph_registry.cpp:273-276): the largest / smallest truth value of x != 0
+namespace {
+// any / all over nothing: false / true wherever the result has elements
+Tensor empty_truth(const Tensor &x, const std::vector<int> &axes, bool keep, bool value) {
+    const Tensor shape_only = GraphRegistry::create_lazy_reduction(OpType::Sum, x, axes, keep); // (validates the axes, gives the shape)
+    Tensor out(shape_only.shape(), DType::Bool, Device::CPU);
+    for (size_t i = 0; i < out.size(); ++i) static_cast<uint8_t *>(out.data())[i] = value ? 1 : 0;
+    return out.to(Device::GPU);
+}
+} // namespace
 Tensor any(const Tensor &x, const std::vector<int> &axes, bool keep) {
+    if (x.size() == 0) return empty_truth(x, axes, keep, false);
     const Tensor truth = x.dtype() == DType::Bool ? x : cast(x, DType::Bool);
     return GraphRegistry::create_lazy_reduction(OpType::Max, truth, axes, keep);
 }
 Tensor all(const Tensor &x, const std::vector<int> &axes, bool keep) {
+    if (x.size() == 0) return empty_truth(x, axes, keep, true);
     const Tensor truth = x.dtype() == DType::Bool ? x : cast(x, DType::Bool);
     return GraphRegistry::create_lazy_reduction(OpType::Min, truth, axes, keep);
 }

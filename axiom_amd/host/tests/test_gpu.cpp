@@ -1385,6 +1385,19 @@ GPU_TEST(LazyNodes, ProductsAnyAllAndCasts) {
     EXPECT_TRUE(host_truth(ops::all(ops::isfinite(v))) == std::vector<int>({1}));
     EXPECT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
     EXPECT_TRUE(host_truth(ops::any(ops::isnan((v - v) / (v - v)))) == std::vector<int>({1}));
+    // reductions over nothing: an empty result stays empty, an empty extent gives the identity
+    auto z = Tensor::zeros({2, 0, 4}, DType::Float32, Device::GPU), z0 = Tensor::zeros({0, 3, 4}, DType::Float32, Device::GPU);
+    EXPECT_TRUE(host_floats(ops::sum(z, {1})) == std::vector<float>(8, 0.0f));
+    EXPECT_TRUE(host_floats(ops::prod(z, {1})) == std::vector<float>(8, 1.0f));
+    EXPECT_TRUE(ops::sum(z, {1}).shape() == Shape({2, 4}));
+    EXPECT_TRUE(ops::sum(z, {2}).shape() == Shape({2, 0}));
+    EXPECT_EQ(ops::sum(z, {2}).size(), 0u);
+    EXPECT_TRUE(ops::sum(z0, {1}).shape() == Shape({0, 4}));
+    EXPECT_NEAR(ops::sum(z).item<float>(), 0.0f, 0);
+    EXPECT_TRUE(std::isnan(host_floats(ops::mean(z, {1}))[0]));
+    EXPECT_TRUE(host_truth(ops::any(z, {1})) == std::vector<int>(8, 0));
+    EXPECT_TRUE(host_truth(ops::all(z, {1})) == std::vector<int>(8, 1));
+    EXPECT_THROW(ops::max(z, {1}), ValueError);
     // products along a middle axis and over everything, against float64
     auto s = axtest::uniform({4, 9, 16}, 122, 0.9f, 1.1f);
     auto sf = host_floats(s), pm = host_floats(s.gpu().prod(1));

@@ -333,7 +333,9 @@ def test_softmax_along_inner_axes_matches_the_oracle(dt):
     (log: 1e-4), 16-bit one rounding step of the result."""
     rng = np.random.default_rng(9 + dt)
     for outer, axis, inner, scale in ((1, 37, 4096, 1.0), (6, 130, 72, 3.0), (3, 1, 64, 1.0), (64, 300, 8, 10.0), (5, 77, 9, 2.0), (2, 1000, 33, 1.0),
-                                      (1, 5000, 24, 4.0), (1200, 7, 1024, 2.0)):
+                                      (1, 5000, 24, 4.0), (1200, 7, 1024, 2.0),
+                                      # short axes with many results: the axis stays in a thread's registers (up to 16 elements)
+                                      (1100, 16, 512, 3.0), (1030, 13, 2048, 1.0), (1100, 17, 512, 2.0), (1500, 1, 512, 1.0), (1040, 4, 520, 5.0)):
         x = (rng.normal(size=(outer, axis, inner)) * scale).astype(np.float32)
         bits = x if dt == F32 else axo.to_bits(x, dt)
         d = gh.to_dev(bits)
