@@ -32,8 +32,23 @@
  *   axo_unary/axo_binary   exact IEEE single-rounding identities; gelu(0)=0,
  *       erf(1)=0.8427 (tests/test_tensor_activations.cpp:310-375); the 12
  *       fused-pattern known answers of tests/test_fusion_extended.cpp:114-220.
+ *       The wider operator table (op codes 40-77): the comparison vectors of
+ *       tests/test_tensor_comparisons.cpp:24-113, the logical truth tables and
+ *       atan2 / hypot values of tests/test_tensor_logical_bitwise.cpp:11-70,
+ *       245-277, sign / floor / ceil / trunc / cbrt / isnan / isinf / isfinite /
+ *       clip of tests/test_tensor_numpy_ops.cpp:13-88, erf of
+ *       tests/test_tensor_activations.cpp:356-375, 3^4 = 81 of
+ *       tests/test_tensor_operations.cpp:107-121; where the reference's tests
+ *       hold no value, what the functor's definition fixes: fmod keeps the
+ *       dividend's sign, round moves halves away from zero, sign(NaN) = 0,
+ *       leaky ReLU's slope, the reversed forms against the forward ones, sin /
+ *       cos / tan against libm in float64.
+ *   axo_where      the vectors of tests/test_tensor_where.cpp:26-36, 176-205.
  *   axo_reduce_last  sum(a+b)=80 and 1 Mi ones*2 = 2097152
- *       (tests/test_fusion_extended.cpp:346-352,436-443); float64 reference.
+ *       (tests/test_fusion_extended.cpp:346-352,436-443); float64 reference;
+ *       prod: 24 and {3, 8} of tests/test_tensor_numpy_ops.cpp:91-104,
+ *       prod(sqrt([4,9,16])) = 24 of tests/test_fusion_extended.cpp:376-385;
+ *       any / all as the extreme truth value, tests/test_tensor_activations.cpp:446-478.
  *   axo_layer_norm   mean~0 / var~1 (tests/test_tensor_normalization.cpp:9-74);
  *       float64 closed form.
  *   axo_rms_norm     [3,4] -> [3,4]/sqrt(12.5)
