@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
+#include <cstring>
 #include <map>
 #include <string>
 #include <vector>
@@ -16,7 +17,10 @@
 using namespace axiom;
 using Clock = std::chrono::steady_clock;
 
+static const char *g_only = nullptr; // argv[3]: run only the configurations whose name contains this
+
 template <typename F> static void measure(const char *name, F f, int warmup, int iters, double work, const char *unit, bool last) {
+    if (g_only && !std::strstr(name, g_only)) return;
     for (int i = 0; i < warmup; ++i) f();
     backends::hip::synchronize();
     std::vector<double> us;
@@ -46,12 +50,14 @@ template <typename F> static void measure(const char *name, F f, int warmup, int
     graph::record_gpu_plan_kernels(false);
     std::string kernels;
     for (const auto &k : graph::last_gpu_plan_kernels()) kernels += (kernels.empty() ? "" : " ") + k;
-    std::printf("  \"%s\": {\"median_us\": %.1f, \"min_us\": %.1f, \"%s\": %.1f, \"queued_16_per_wait_us\": %.1f, \"queued_%s\": %.1f, \"last_graph_kernels\": \"%s\"}%s\n",
-                name, med, us.front(), unit, work / (med * 1e-6) / 1e9, pmed, unit, work / (pmed * 1e-6) / 1e9, kernels.c_str(), last ? "" : ",");
+    (void)last; // every entry leads with its comma, so a filtered run still prints valid JSON
+    std::printf(",\n  \"%s\": {\"median_us\": %.1f, \"min_us\": %.1f, \"%s\": %.1f, \"queued_16_per_wait_us\": %.1f, \"queued_%s\": %.1f, \"last_graph_kernels\": \"%s\"}",
+                name, med, us.front(), unit, work / (med * 1e-6) / 1e9, pmed, unit, work / (pmed * 1e-6) / 1e9, kernels.c_str());
 }
 
 int main(int argc, char **argv) {
     const int iters = argc > 1 ? std::atoi(argv[1]) : 50, warmup = argc > 2 ? std::atoi(argv[2]) : 10;
+    g_only = argc > 3 ? argv[3] : nullptr;
     if (!system::is_gpu_available()) {
         std::fprintf(stderr, "host_bench: no GPU visible; the gfx950 backend has no CPU fallback\n");
         return 3;
@@ -69,7 +75,7 @@ int main(int argc, char **argv) {
             if (i >= warmup) us.push_back(std::chrono::duration<double, std::micro>(Clock::now() - t0).count());
         }
         std::sort(us.begin(), us.end());
-        std::printf("  \"launch_and_wait_floor\": {\"median_us\": %.1f, \"min_us\": %.1f},\n", us[us.size() / 2], us.front());
+        std::printf("  \"launch_and_wait_floor\": {\"median_us\": %.1f, \"min_us\": %.1f}", us[us.size() / 2], us.front());
     }
     { // configs[0]: the reference's CPU-runnable case, fp32, on the fp32 matrix instruction here
         auto q = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU), k = Tensor::randn({1, 8, 512, 64}, DType::Float32, Device::GPU),
@@ -132,6 +138,6 @@ int main(int argc, char **argv) {
         };
         measure("whisper_encoder_layer_bf16_s1500_d1280_h20", layer, warmup, iters, 24.0 * S * Dm * Dm + 4.0 * S * S * Dm, "GFLOP_per_s", true);
     }
-    std::printf("}\n");
+    std::printf("\n}\n");
     return 0;
 }

@@ -11,16 +11,29 @@ namespace axiom::nn {
 
 Tensor Module::forward(const Tensor &) const { throw RuntimeError::not_implemented("forward(const Tensor&) for this module"); }
 
+// A parameter is memory, never a deferred computation: a lazy tensor handed in as a weight (say
+// (randn * 0.02).astype(bf16)) is run once here.  Left lazy, every forward would recompute it as a fused input
+// of the product it feeds, and the stacked q/k/v projection could not take its address.
+static void settle(Tensor &p) {
+    if (!p.empty() && p.is_lazy()) p.sync();
+}
+
 Module &Module::to(Device device) {
     for (auto &[name, p] : params_)
-        if (!p->empty()) *p = p->to(device);
+        if (!p->empty()) {
+            *p = p->to(device);
+            settle(*p);
+        }
     for (auto &[name, m] : submodules_) m->to(device);
     return *this;
 }
 
 Module &Module::to(DType dtype) {
     for (auto &[name, p] : params_)
-        if (!p->empty()) *p = p->astype(dtype);
+        if (!p->empty()) {
+            *p = p->astype(dtype);
+            settle(*p);
+        }
     for (auto &[name, m] : submodules_) m->to(dtype);
     return *this;
 }
@@ -28,8 +41,10 @@ Module &Module::to(DType dtype) {
 void Module::load_state_dict(const std::map<std::string, Tensor> &sd, const std::string &prefix, bool strict) {
     for (auto &[name, p] : params_) {
         auto it = sd.find(prefix + name);
-        if (it != sd.end()) *p = it->second;
-        else if (strict) throw ValueError("missing key '" + prefix + name + "' in state_dict");
+        if (it != sd.end()) {
+            *p = it->second;
+            settle(*p);
+        } else if (strict) throw ValueError("missing key '" + prefix + name + "' in state_dict");
     }
     for (auto &[name, m] : submodules_) m->load_state_dict(sd, prefix + name + ".", strict);
 }
@@ -67,6 +82,8 @@ Linear::Linear(bool bias) : has_bias_(bias) {
 
 Tensor Linear::forward(const Tensor &input) const {
     if (weight_.empty()) throw RuntimeError("Linear: weight not initialized (load_state_dict first)");
+    if (weight_.is_lazy()) weight_.sync(); // a lazy tensor assigned through parameters(): run it once, not per forward
+    if (has_bias_ && bias_.is_lazy()) bias_.sync();
     Tensor y = ops::matmul(input, weight_, false, true);
     if (has_bias_ && !bias_.empty()) y = ops::add(y, bias_);
     return y;
@@ -187,10 +204,12 @@ bool MultiHeadAttention::fused_qkv(const Tensor &x, Tensor &q, Tensor &k, Tensor
     size_t offsets[6] = {};
     for (int i = 0; i < 3; ++i) {
         const Tensor &w = proj[i]->weight(), &b = proj[i]->bias();
-        if (w.empty() || w.is_lazy() || w.device() != Device::GPU || w.dtype() != dt || !w.is_contiguous() || w.ndim() != 2 || w.shape()[0] != Dm || w.shape()[1] != Dm)
+        if (w.is_lazy()) w.sync();
+        if (b.is_lazy()) b.sync();
+        if (w.empty() || w.device() != Device::GPU || w.dtype() != dt || !w.is_contiguous() || w.ndim() != 2 || w.shape()[0] != Dm || w.shape()[1] != Dm)
             return false;
         const bool has_b = proj[i]->has_bias() && !b.empty();
-        if (has_b && (b.is_lazy() || b.device() != Device::GPU || b.dtype() != dt || !b.is_contiguous() || b.size() != Dm)) return false;
+        if (has_b && (b.device() != Device::GPU || b.dtype() != dt || !b.is_contiguous() || b.size() != Dm)) return false;
         any_bias = any_bias || has_b;
         sources[2 * i] = static_cast<const char *>(w.storage()->raw()) + w.offset();
         sources[2 * i + 1] = has_b ? static_cast<const char *>(b.storage()->raw()) + b.offset() : nullptr;

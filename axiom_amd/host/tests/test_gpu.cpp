@@ -1630,6 +1630,34 @@ GPU_TEST(FlashAttentionMHA, StackedProjectionFollowsAParameterSwappedInPlace) {
     EXPECT_LT(apart, 1e-4); // ... to what the three separate projections give
 }
 
+// Lazy tensors handed in as parameters (a scaled, narrowed random matrix is the usual way to write one) are run once
+// when the module takes them: forwards see memory, the stacked projection applies, and no forward repeats the
+// parameter's own arithmetic.
+GPU_TEST(FlashAttentionMHA, LazyParametersAreMaterialisedOnce) {
+    const size_t S = 48, Dm = 64;
+    auto x = axtest::randn({1, S, Dm}, 500, DType::Float32).gpu().astype(DType::BFloat16);
+    x.sync();
+    std::map<std::string, Tensor> sd;
+    uint64_t seed = 510;
+    for (const char *name : {"q_proj", "k_proj", "v_proj", "out_proj"}) {
+        sd[std::string(name) + ".weight"] = (axtest::randn({Dm, Dm}, seed++, DType::Float32).gpu() * 0.125f).astype(DType::BFloat16);
+        sd[std::string(name) + ".bias"] = (axtest::randn({Dm}, seed++, DType::Float32).gpu() * 0.1f).astype(DType::BFloat16);
+        EXPECT_TRUE(sd[std::string(name) + ".weight"].is_lazy());
+    }
+    nn::MultiHeadAttention mha(4);
+    mha.load_state_dict(sd);
+    for (auto &np : mha.named_parameters()) EXPECT_FALSE(np.second->is_lazy());
+    Tensor y = x + mha.forward(x, x, x);
+    y.sync();
+    ASSERT_EQ(graph::last_gpu_plan_kernels().size(), 1u);
+    for (const auto &k : graph::last_gpu_plan_kernels()) EXPECT_EQ(k, std::string("gemm")); // the output projection with bias and residual, nothing else
+    // a lazy weight assigned through the mutable parameter list is settled by the first forward
+    for (auto &np : mha.named_parameters())
+        if (np.first == "out_proj.weight") *np.second = (axtest::randn({Dm, Dm}, 599, DType::Float32).gpu() * 0.125f).astype(DType::BFloat16);
+    (x + mha.forward(x, x, x)).sync();
+    for (auto &np : mha.named_parameters()) EXPECT_FALSE(np.second->is_lazy());
+}
+
 GPU_TEST(LazyNodes, Conv2dKnownAnswers) { // tests/test_conv2d.cpp:3-111 of the reference
     auto x9 = gpu_f32({1, 2, 3, 4, 5, 6, 7, 8, 9}, {1, 1, 3, 3});
     auto w4 = gpu_f32({1, 1, 1, 1}, {1, 1, 2, 2});
