@@ -106,7 +106,7 @@ std::vector<AxhipRowsProgram> shapes_of(int dt, int *n_primary) {
     norm(AXHIP_ROWOP_LAYERNORM, PRE_NONE, true, AXHIP_OP_GELU);
     norm(AXHIP_ROWOP_RMSNORM, PRE_NONE, true, AXHIP_OP_GELU);
     *n_primary = static_cast<int>(out.size());
-    // secondary shapes (the main plans only)
+    // secondary shapes (the main plans only, and only for rows of whole, aligned vectors)
     softmax_like(AXHIP_ROWOP_LOGSOFTMAX, PRE_NONE, true);
     softmax_like(AXHIP_ROWOP_SOFTMAX, PRE_MULS, true);
     softmax_like(AXHIP_ROWOP_SOFTMAX, PRE_ADDF, true);
@@ -155,6 +155,7 @@ int main(int argc, char **argv) {
             for (int pi = 0; pi < (static_cast<int>(si) < n_primary ? n_plans : n_main_plans); ++pi) {
                 const int *pl = plans[pi];
                 for (bool ragged : {false, true}) {
+                    if (ragged && static_cast<int>(si) >= n_primary) continue; // secondary shapes: whole-vector rows only
                     RowsProgPlan plan;
                     rows_prog_plan_for(p, pl[0], pl[1], ragged, &plan, /*the built-in ragged kernels are those for equally aligned streams*/ ragged && rows_prog_grid_pays(p, pl[0], pl[1]));
                     RowsProgSpec s;

@@ -1,0 +1,6 @@
+// The interpreter's row kernels at 4 elements per vector (see rows_kernels.hpp); launched from rows.hip.
+#include "rows_kernels.hpp"
+
+namespace axhip {
+template int launch_plan_e<4>(const AxhipRowsProgram &, const RowsPlan &, hipStream_t);
+} // namespace axhip
