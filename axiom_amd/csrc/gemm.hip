@@ -71,6 +71,7 @@ __device__ __forceinline__ void store16(void *p, int64_t i, float x) {
 // columns past the end are masked per lane.  When all MI*32 rows are valid (FULL_ROWS)
 // the row offset travels in the scalar offset of the instruction, otherwise it is added
 // to the lane's offset, which is what the bounds check looks at.
+// (Column tiles outside, rows inside: on the ring kernels' products the other nesting measured 3 - 5 % slower.)
 // Requires MI*32 * ldc * 2 < 2^31.
 template <bool BF16, int RESIDUAL_T, bool FULL_ROWS, int OP, int MI, int NJ> // RESIDUAL_T: 0 no, 1 yes, 2 decided at run time
 __device__ __forceinline__ void gemm_store_tiles_as(const GemmArgs &g, const float16_t (&acc)[MI][NJ], int64_t m_base, int64_t n_base, int64_t coff, int l32, int g2) {
@@ -238,14 +239,23 @@ __global__ __launch_bounds__(256, BM == 128 ? 2 : 1) void gemm_mfma_nt_kernel(co
 }
 
 // ----------------------------------------------------------- MFMA NT, 256x256
-// Large products: work-group tile 256 x 256 x 64, 8 waves in a 2 x 4 layout, each
-// owning 128 x 64 of C (4 x 2 MFMA tiles, 128 accumulator registers).  A and B
-// k-tiles go L2 -> LDS directly (buffer_load ... lds: no staging registers, no
-// ds_write) into two 64 KiB buffers; tile j+1 streams in while tile j is multiplied,
-// one barrier per k-tile.  LDS rows are the 128 bytes of one k-tile row with the
-// 16-byte chunk index XOR-ed by (row >> 1) & 7, which spreads the 16 rows of a
-// fragment read over all banks.  Work-groups are dealt to the 8 XCDs so that each
-// XCD owns a compact block of C tiles and its L2 sees every A / B panel few times.
+// Large products: work-group tile 256 x 256 x 64, 8 waves in a 2 x 4 layout, each owning 128 x 64 of C as 8 x 4
+// tiles of v_mfma_f32_16x16x32 (128 accumulator registers).  The kernel runs on the chip's power limit, where time
+// follows the energy a launch spends rather than its cycle count, and on operands that change every k-step the
+// 16x16x32 form does the same flops for about 15 % less than 32x32x16 (a bare loop of either: 1.9 - 2.0 against
+// 1.67 - 1.75 PFLOP/s).  A and B k-tiles go L2 -> LDS directly (buffer_load ... lds: no staging registers, no
+// ds_write; staging through registers spends as many cycles and more power) into two 64 KiB buffers, one barrier per
+// k-tile.  LDS rows are the 128 bytes of one k-tile row with the 16-byte chunk index XOR-ed by (row >> 1) & 7, which
+// spreads the 16 rows of a fragment read over all banks.
+// A k-tile is two k-steps of 32 MFMAs.  The A fragments are single-buffered: the registers of fragment row i are
+// refilled for the next k-step right behind the row's fourth MFMA, 28 MFMAs before they are needed; the B fragments
+// are double-buffered.  Every LDS read and every global load sits between two MFMAs (scheduling fences pin the
+// order): a wave that meets a batch of reads, or several loads in a row -- a direct-to-LDS load holds the wave's
+// issue for about 60 cycles --, starves the matrix pipe of its SIMD.  The barrier comes after the first fragment row
+// of the second k-step: by then every wave has read the whole tile, so the buffer takes the tile after next (the
+// loads are dealt out one per three MFMAs from there) and the reads turn to the next tile.
+// Work-groups are dealt to the 8 XCDs so that each XCD owns a compact block of C tiles and its L2 sees every A / B
+// panel few times.
 typedef int int4_t __attribute__((ext_vector_type(4)));
 constexpr int BIG = 256;              // tile rows (M) and columns (N)
 constexpr int BIG_ROWB = TK * 2;      // bytes per LDS row
@@ -263,12 +273,109 @@ __device__ __forceinline__ int4_t gemm_rsrc(const void *base, int bytes) {
     return int4_t{static_cast<int>(static_cast<uint32_t>(pa)), static_cast<int>(static_cast<uint32_t>(pa >> 32) & 0xFFFFu), bytes, 0x00020000};
 }
 
+// The epilogue for 16x16 accumulator tiles computed as B-fragment x A-fragment^T: lane (l16, g4) holds, of tile
+// (i, j), row 16 i + l16 and the four consecutive columns 16 j + 4 g4 .. + 3 -- one 8-byte store where C allows it
+// (even ldc, 4-byte aligned origin), 2-byte stores otherwise.  C and the residual go through buffer descriptors that
+// cover exactly the block's valid rows (a row past the end is dropped by the bounds check); columns are masked.
+// Requires 128 * ldc * 2 < 2^31.
+typedef float float4_t __attribute__((ext_vector_type(4)));
+template <bool BF16, int RESIDUAL_T, int OP> // RESIDUAL_T: 0 no, 1 yes, 2 decided at run time
+__device__ __forceinline__ void gemm_store_tiles16_as(const GemmArgs &g, const float4_t (&acc)[8][4], int64_t m_base, int64_t n_base, int64_t coff, int l16, int g4) {
+    const bool RESIDUAL = RESIDUAL_T == 1 || (RESIDUAL_T == 2 && g.residual != nullptr);
+    const int ldc2 = static_cast<int>(g.ldc) * 2;
+    const int cols_valid = static_cast<int>(min<int64_t>(64, g.N - n_base));
+    const int rows_valid = static_cast<int>(min<int64_t>(128, g.M - m_base));
+    const int extent = (rows_valid - 1) * ldc2 + cols_valid * 2;
+    const int64_t origin = coff + m_base * g.ldc + n_base;
+    uint16_t *cbase = static_cast<uint16_t *>(g.c) + origin;
+    const uint16_t *rbase = static_cast<const uint16_t *>(RESIDUAL ? g.residual : g.c) + origin;
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(cbase, 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(rbase), 0, extent, 0x00020000);
+    const bool wide = (g.ldc & 1) == 0 && (reinterpret_cast<uintptr_t>(cbase) & 3u) == 0 && (reinterpret_cast<uintptr_t>(rbase) & 3u) == 0;
+    float bias[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int col = 16 * j + 4 * g4 + e;
+            bias[j][e] = g.bias && col < cols_valid ? load16<BF16>(g.bias, n_base + col) : 0.0f;
+        }
+    // rows outside, columns inside: the four stores that complete a row's 128-byte line follow one another (with the
+    // column tiles outside, 16 rows apart in between, the same kernel takes 7 % longer on 4096^3)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = 16 * j + 4 * g4;
+            if (col >= cols_valid) continue;
+            const bool whole = wide && col + 4 <= cols_valid;
+            const int voff = (16 * i + l16) * ldc2 + col * 2;
+            float x[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = acc[i][j][e] + bias[j][e];
+            if (RESIDUAL) {
+                if (whole) {
+                    const uint2_t r = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(rrsrc, voff, 0, 0));
+                    const uint32_t rw[2] = {r.x, r.y};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint16_t h = static_cast<uint16_t>(rw[e / 2] >> (16 * (e % 2)));
+                        x[e] += BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < cols_valid) {
+                            const uint16_t h = __builtin_amdgcn_raw_buffer_load_b16(rrsrc, voff + 2 * e, 0, 0);
+                            x[e] += BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+                        }
+                }
+            }
+            uint32_t w[2];
+#pragma unroll
+            for (int e = 0; e < 4; e += 2) {
+                const float y0 = gemm_epilogue16(OP, x[e]), y1 = gemm_epilogue16(OP, x[e + 1]);
+                w[e / 2] = BF16 ? pack_bf16x2(y0, y1) : pack_f16x2(y0, y1);
+            }
+            if (whole) {
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(decltype(__builtin_amdgcn_raw_buffer_load_b64(rrsrc, 0, 0, 0)), uint2_t{w[0], w[1]}), crsrc, voff, 0, 0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (col + e < cols_valid)
+                        __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(w[e / 2] >> (16 * (e % 2))), crsrc, voff + 2 * e, 0, 0);
+            }
+        }
+    }
+}
+
+template <bool BF16>
+__device__ __forceinline__ void gemm_store_tiles16(const GemmArgs &g, const float4_t (&acc)[8][4], int64_t m_base, int64_t n_base, int64_t coff, int l16, int g4) {
+    if (m_base >= g.M || n_base >= g.N) return;
+    // the cheap epilogues get a specialisation with and without residual; the transcendental ones are large when
+    // unrolled 128 times, and one general instance each is enough
+    switch (g.epilogue) {
+    case AXHIP_OP_RELU:
+        if (g.residual) gemm_store_tiles16_as<BF16, 1, AXHIP_OP_RELU>(g, acc, m_base, n_base, coff, l16, g4);
+        else gemm_store_tiles16_as<BF16, 0, AXHIP_OP_RELU>(g, acc, m_base, n_base, coff, l16, g4);
+        break;
+    case AXHIP_OP_GELU: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_GELU>(g, acc, m_base, n_base, coff, l16, g4); break;
+    case AXHIP_OP_SILU: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_SILU>(g, acc, m_base, n_base, coff, l16, g4); break;
+    case AXHIP_OP_SIGMOID: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_SIGMOID>(g, acc, m_base, n_base, coff, l16, g4); break;
+    case AXHIP_OP_TANH: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_TANH>(g, acc, m_base, n_base, coff, l16, g4); break;
+    default:
+        if (g.residual) gemm_store_tiles16_as<BF16, 1, 0>(g, acc, m_base, n_base, coff, l16, g4);
+        else gemm_store_tiles16_as<BF16, 0, 0>(g, acc, m_base, n_base, coff, l16, g4);
+        break;
+    }
+}
+
 // Requires K % 64 == 0 and 256 * max(lda, ldb) * 2 < 2^31 (checked by the launcher).
 template <bool BF16>
 __global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs g, const int tiles_m, const int tiles_n) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char big_lds[]; // A0 B0 A1 B1
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
-    const int l32 = lane % 32, g2 = lane / 32;
+    const int l16 = lane % 16, g4 = lane / 16;
 
     // work-group -> C tile: XCD x (work-groups x, x+8, ...) owns a contiguous range of the
     // tile order; within it tiles run down groups of 4 tile rows
@@ -302,83 +409,114 @@ __global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs
     }
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(big_lds));
     const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + 8 * wave * BIG_ROWB);
-    auto load_tile = [&](int kt, int buf) {
+    auto load_one = [&](const int4_t &ar, const int4_t &br, int kt, int buf, int n) { // n: 0..3 of A, 4..7 of B
         const int soff = kt * BIG_ROWB;
-#pragma unroll
-        for (int n = 0; n < 4; ++n) gemm_load_to_lds(arsrc, lds_wave + buf * 2 * BIG_TILEB + n * 64 * BIG_ROWB, a_voff[n], soff);
-#pragma unroll
-        for (int n = 0; n < 4; ++n) gemm_load_to_lds(brsrc, lds_wave + buf * 2 * BIG_TILEB + BIG_TILEB + n * 64 * BIG_ROWB, b_voff[n], soff);
+        if (n < 4) gemm_load_to_lds(ar, lds_wave + buf * 2 * BIG_TILEB + n * 64 * BIG_ROWB, a_voff[n % 4], soff);
+        else gemm_load_to_lds(br, lds_wave + buf * 2 * BIG_TILEB + BIG_TILEB + (n - 4) * 64 * BIG_ROWB, b_voff[n % 4], soff);
     };
 
-    // ---- fragment reads: row l32 (+ tile origin, a multiple of 32), k chunk 2 ks + g2
+    // ---- fragment reads: row l16 of a 16-row block, 16-byte chunk 4 s + g4 of the row's eight (s: k-step of the tile)
     const int wm = (wave / 4) * 128, wn = (wave % 4) * 64;
-    int f_off[TK / 16];
+    int f_off[2];
 #pragma unroll
-    for (int ks = 0; ks < TK / 16; ++ks) f_off[ks] = l32 * BIG_ROWB + (((2 * ks + g2) ^ ((l32 >> 1) & 7)) * 16);
+    for (int s = 0; s < 2; ++s) f_off[s] = l16 * BIG_ROWB + (((4 * s + g4) ^ ((l16 >> 1) & 7)) * 16);
 
-    float16_t acc[4][2];
+    float4_t acc[8][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+        for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // Fragments are double-buffered in registers and the loop is rotated: the reads of
-    // k-step 0 of the next tile are issued right after the barrier, under the MFMAs of
-    // k-step 3 of the current one, so no LDS latency is exposed at the tile boundary.
-    uint4_t fa[2][4], fb[2][2];
-    auto read_frags = [&](int slot, int buf, int ks) {
-        const unsigned char *As = big_lds + buf * 2 * BIG_TILEB + wm * BIG_ROWB;
-        const unsigned char *Bs = big_lds + buf * 2 * BIG_TILEB + BIG_TILEB + wn * BIG_ROWB;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) fb[slot][j] = *reinterpret_cast<const uint4_t *>(Bs + 32 * j * BIG_ROWB + f_off[ks]);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) fa[slot][i] = *reinterpret_cast<const uint4_t *>(As + 32 * i * BIG_ROWB + f_off[ks]);
+    uint4_t fa[8], fb[2][4];
+    auto read_a = [&](int buf, int s, int i) {
+        fa[i] = *reinterpret_cast<const uint4_t *>(big_lds + buf * 2 * BIG_TILEB + (wm + 16 * i) * BIG_ROWB + f_off[s]);
     };
-    auto multiply = [&](int slot) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                if constexpr (BF16)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[slot][i]), __builtin_bit_cast(bf16x8_t, fb[slot][j]), acc[i][j], 0, 0, 0);
-                else
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fa[slot][i]), __builtin_bit_cast(half8_t, fb[slot][j]), acc[i][j], 0, 0, 0);
-            }
+    auto read_b = [&](int slot, int buf, int s, int j) {
+        fb[slot][j] = *reinterpret_cast<const uint4_t *>(big_lds + buf * 2 * BIG_TILEB + BIG_TILEB + (wn + 16 * j) * BIG_ROWB + f_off[s]);
     };
+    // D = (B fragment) x (A fragment)^T: the lane holds four consecutive columns of one row of C
+    auto mfma = [&](int slot, int i, int j) {
+        if constexpr (BF16)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fb[slot][j]), __builtin_bit_cast(bf16x8_t, fa[i]), acc[i][j], 0, 0, 0);
+        else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, fb[slot][j]), __builtin_bit_cast(half8_t, fa[i]), acc[i][j], 0, 0, 0);
+    };
+#define AXHIP_FENCE() __builtin_amdgcn_sched_barrier(0)
 
     const int nk = static_cast<int>(g.K / TK);
-    load_tile(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+#pragma unroll
+    for (int n = 0; n < 8; ++n) load_one(arsrc, brsrc, 0, 0, n);
+    if (nk > 1) {
+#pragma unroll
+        for (int n = 0; n < 8; ++n) load_one(arsrc, brsrc, 1, 1, n);
+        __builtin_amdgcn_s_waitcnt(0x0F78); // vmcnt(8): tile 0 has landed
+    } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    }
     __syncthreads();
-    read_frags(0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) read_a(0, 0, i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) read_b(0, 0, 0, j);
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) load_tile(kt + 1, buf ^ 1);
-        // the scheduling fences keep each batch of reads ahead of the MFMAs it overlaps with
-        // (left alone, the scheduler sinks every read to just before its first use)
-        read_frags(1, buf, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(0);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(0, buf, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(1);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(1, buf, 3);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(0);
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's share of tile kt+1 has landed
-        __syncthreads();                    // ... everyone's has, and tile kt is no longer read
-        read_frags(0, buf ^ 1, 0);          // (after the last tile: a harmless read of stale LDS)
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(1);
-        __builtin_amdgcn_sched_barrier(0);
+        // past the last tile the loads run on empty descriptors (every lane out of range: zeros into a buffer nobody
+        // reads, no memory traffic) rather than behind eight branches
+        const bool more = kt + 2 < nk;
+        const int4_t ar = int4_t{arsrc.x, arsrc.y, more ? arsrc.z : 0, arsrc.w}, br = int4_t{brsrc.x, brsrc.y, more ? brsrc.z : 0, brsrc.w};
+        AXHIP_FENCE();
+        // k-step 0: B slot 0; the refills fetch k-step 1 of this tile
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                mfma(0, i, j);
+                AXHIP_FENCE();
+                if (j == 2 && i < 4) {
+                    read_b(1, buf, 1, i);
+                    AXHIP_FENCE();
+                }
+                if (j == 3) {
+                    read_a(buf, 1, i);
+                    AXHIP_FENCE();
+                }
+            }
+        // k-step 1: B slot 1; behind the barrier the refills fetch k-step 0 of the next tile (after the last tile: a
+        // harmless read of stale LDS) and this tile's buffer takes the tile after next
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i == 1) {
+                __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's share of tile kt+1 has landed
+                __syncthreads();                    // ... everyone's has, and tile kt is no longer read
+                AXHIP_FENCE();
+                read_a(buf ^ 1, 0, 0);
+                AXHIP_FENCE();
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                mfma(1, i, j);
+                AXHIP_FENCE();
+                if (i >= 1) {
+                    const int q = (i - 1) * 4 + j; // MFMAs since the barrier
+                    if (q % 3 == 1 && q / 3 < 8) {
+                        load_one(ar, br, kt + 2, buf, q / 3);
+                        AXHIP_FENCE();
+                    }
+                    if (q % 2 == 0 && q >= 2 && q <= 8) {
+                        read_b(0, buf ^ 1, 0, q / 2 - 1);
+                        AXHIP_FENCE();
+                    }
+                    if (j == 3) {
+                        read_a(buf ^ 1, 0, i);
+                        AXHIP_FENCE();
+                    }
+                }
+            }
+        }
     }
+#undef AXHIP_FENCE
 
-    gemm_store_tiles<BF16, 4, 2>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l32, g2);
+    gemm_store_tiles16<BF16>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l16, g4);
 }
 
 // --------------------------------------------------- MFMA NT, multi-stage ring

@@ -101,6 +101,40 @@ def test_half_large_tile_path_matches_fp64(dt, M, N, K, extras):
 
 
 @pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,epilogue,with_bias,with_res", [
+    (2050, 3803, 128, "gelu", True, True),    # odd row pitch of C: two-byte stores everywhere
+    (2049, 3802, 256, None, False, True),     # a last column group of two: masked tail beside 8-byte stores
+    (2304, 3801, 64, "silu", True, False),    # one k-tile
+    (2100, 2310, 448, "tanh", False, False),
+    (4096, 2048, 512, "sigmoid", True, True)])
+def test_half_large_tile_epilogues_and_column_tails(dt, M, N, K, epilogue, with_bias, with_res):
+    """The 256 x 256 kernel's epilogue: a lane owns four consecutive columns of a row, stored as 8 bytes where the
+    row pitch and the origin allow it and as masked 2-byte stores otherwise; every activation, with and without bias
+    and residual, against float64."""
+    g = axo.PCG64(3 * M + N + K)
+    x, W = axo.to_bits(g.normal((M, K)), dt), axo.to_bits(g.normal((N, K)) * 0.05, dt)
+    bias = axo.to_bits(g.normal((N,)) * 0.1, dt) if with_bias else None
+    res = axo.to_bits(g.normal((M, N)), dt) if with_res else None
+    got = axo.to_f32(gh.gemm(x, W, dt, trans_b=True, bias=bias, residual=res, epilogue=epilogue)[0], dt)
+    want = axo.to_f32(x, dt).astype(np.float64) @ axo.to_f32(W, dt).astype(np.float64).T
+    if with_bias:
+        want = want + axo.to_f32(bias, dt)
+    if with_res:
+        want = want + axo.to_f32(res, dt)
+    if epilogue == "gelu":
+        from scipy.special import erf
+        want = 0.5 * want * (1.0 + erf(want / np.sqrt(2.0)))
+    elif epilogue == "silu":
+        want = want / (1.0 + np.exp(-want))
+    elif epilogue == "tanh":
+        want = np.tanh(want)
+    elif epilogue == "sigmoid":
+        want = 1.0 / (1.0 + np.exp(-want))
+    assert got.shape == want.shape
+    assert np.max(np.abs(got - want)) < 2e-2 + 2.0**-8 * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("M,N,K,extras", [(1500, 5120, 1280, False), (1500, 1280, 5120, True), (200, 330, 256, True), (129, 257, 320, False),
                                           (1000, 2000, 448, True), (64, 128, 4096, False),
                                           (1500, 3840, 1280, False), (1500, 3700, 320, True)])
