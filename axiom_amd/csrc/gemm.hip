@@ -280,7 +280,7 @@ __device__ __forceinline__ int4_t gemm_rsrc(const void *base, int bytes) {
 // Requires 128 * ldc * 2 < 2^31.
 typedef float float4_t __attribute__((ext_vector_type(4)));
 template <bool BF16, int RESIDUAL_T, int OP> // RESIDUAL_T: 0 no, 1 yes, 2 decided at run time
-__device__ __forceinline__ void gemm_store_tiles16_as(const GemmArgs &g, const float4_t (&acc)[8][4], int64_t m_base, int64_t n_base, int64_t coff, int l16, int g4) {
+__device__ __forceinline__ void gemm_store_tiles16_as(const GemmArgs &g, const float4_t (&acc)[8][4], int64_t m_base, int64_t n_base, int64_t coff, int l16, int g4, unsigned char *stage) {
     const bool RESIDUAL = RESIDUAL_T == 1 || (RESIDUAL_T == 2 && g.residual != nullptr);
     const int ldc2 = static_cast<int>(g.ldc) * 2;
     const int cols_valid = static_cast<int>(min<int64_t>(64, g.N - n_base));
@@ -300,6 +300,12 @@ __device__ __forceinline__ void gemm_store_tiles16_as(const GemmArgs &g, const f
             const int col = 16 * j + 4 * g4 + e;
             bias[j][e] = g.bias && col < cols_valid ? load16<BF16>(g.bias, n_base + col) : 0.0f;
         }
+    // A block with all 64 columns inside and 16-byte aligned rows goes through the wave's 16 KiB of LDS (free once the
+    // k loop has ended): the finished 16-bit values are written in accumulator layout and read back row by row, so that
+    // every global store carries 16 bytes per lane and a store instruction fills eight whole 128-byte lines.  While C is
+    // written no MFMA runs anywhere on the chip (all work-groups end their k loops together), so the write phase is
+    // pure HBM time: 8-byte stores, 32 bytes of a row per instruction, take 9.3 us for the 32 MiB of 4096^2 values.
+    const bool staged = stage != nullptr && cols_valid == 64 && (g.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(cbase) & 15u) == 0;
     // rows outside, columns inside: the four stores that complete a row's 128-byte line follow one another (with the
     // column tiles outside, 16 rows apart in between, the same kernel takes 7 % longer on 4096^3)
 #pragma unroll
@@ -337,7 +343,10 @@ __device__ __forceinline__ void gemm_store_tiles16_as(const GemmArgs &g, const f
                 const float y0 = gemm_epilogue16(OP, x[e]), y1 = gemm_epilogue16(OP, x[e + 1]);
                 w[e / 2] = BF16 ? pack_bf16x2(y0, y1) : pack_f16x2(y0, y1);
             }
-            if (whole) {
+            if (staged) {
+                const int r = 16 * i + l16; // 128-byte rows; the 16-byte chunk index is XOR-ed with the row so that neither pass meets bank conflicts
+                *reinterpret_cast<uint2_t *>(stage + r * 128 + (((2 * j + (g4 >> 1)) ^ (r & 7)) * 16) + (g4 & 1) * 8) = uint2_t{w[0], w[1]};
+            } else if (whole) {
                 __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(decltype(__builtin_amdgcn_raw_buffer_load_b64(rrsrc, 0, 0, 0)), uint2_t{w[0], w[1]}), crsrc, voff, 0, 0);
             } else {
 #pragma unroll
@@ -347,25 +356,34 @@ __device__ __forceinline__ void gemm_store_tiles16_as(const GemmArgs &g, const f
             }
         }
     }
+    if (staged) {
+        const int lane = 16 * g4 + l16;
+#pragma unroll
+        for (int n = 0; n < 16; ++n) {
+            const int r = 8 * n + (lane >> 3), q = lane & 7;
+            const uint4_t v = *reinterpret_cast<const uint4_t *>(stage + r * 128 + ((q ^ (r & 7)) * 16));
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(decltype(__builtin_amdgcn_raw_buffer_load_b128(rrsrc, 0, 0, 0)), v), crsrc, r * ldc2 + q * 16, 0, 0);
+        }
+    }
 }
 
 template <bool BF16>
-__device__ __forceinline__ void gemm_store_tiles16(const GemmArgs &g, const float4_t (&acc)[8][4], int64_t m_base, int64_t n_base, int64_t coff, int l16, int g4) {
+__device__ __forceinline__ void gemm_store_tiles16(const GemmArgs &g, const float4_t (&acc)[8][4], int64_t m_base, int64_t n_base, int64_t coff, int l16, int g4, unsigned char *stage) {
     if (m_base >= g.M || n_base >= g.N) return;
     // the cheap epilogues get a specialisation with and without residual; the transcendental ones are large when
     // unrolled 128 times, and one general instance each is enough
     switch (g.epilogue) {
     case AXHIP_OP_RELU:
-        if (g.residual) gemm_store_tiles16_as<BF16, 1, AXHIP_OP_RELU>(g, acc, m_base, n_base, coff, l16, g4);
-        else gemm_store_tiles16_as<BF16, 0, AXHIP_OP_RELU>(g, acc, m_base, n_base, coff, l16, g4);
+        if (g.residual) gemm_store_tiles16_as<BF16, 1, AXHIP_OP_RELU>(g, acc, m_base, n_base, coff, l16, g4, stage);
+        else gemm_store_tiles16_as<BF16, 0, AXHIP_OP_RELU>(g, acc, m_base, n_base, coff, l16, g4, stage);
         break;
-    case AXHIP_OP_GELU: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_GELU>(g, acc, m_base, n_base, coff, l16, g4); break;
-    case AXHIP_OP_SILU: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_SILU>(g, acc, m_base, n_base, coff, l16, g4); break;
-    case AXHIP_OP_SIGMOID: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_SIGMOID>(g, acc, m_base, n_base, coff, l16, g4); break;
-    case AXHIP_OP_TANH: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_TANH>(g, acc, m_base, n_base, coff, l16, g4); break;
+    case AXHIP_OP_GELU: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_GELU>(g, acc, m_base, n_base, coff, l16, g4, stage); break;
+    case AXHIP_OP_SILU: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_SILU>(g, acc, m_base, n_base, coff, l16, g4, stage); break;
+    case AXHIP_OP_SIGMOID: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_SIGMOID>(g, acc, m_base, n_base, coff, l16, g4, stage); break;
+    case AXHIP_OP_TANH: gemm_store_tiles16_as<BF16, 2, AXHIP_OP_TANH>(g, acc, m_base, n_base, coff, l16, g4, stage); break;
     default:
-        if (g.residual) gemm_store_tiles16_as<BF16, 1, 0>(g, acc, m_base, n_base, coff, l16, g4);
-        else gemm_store_tiles16_as<BF16, 0, 0>(g, acc, m_base, n_base, coff, l16, g4);
+        if (g.residual) gemm_store_tiles16_as<BF16, 1, 0>(g, acc, m_base, n_base, coff, l16, g4, stage);
+        else gemm_store_tiles16_as<BF16, 0, 0>(g, acc, m_base, n_base, coff, l16, g4, stage);
         break;
     }
 }
@@ -516,7 +534,11 @@ __global__ __launch_bounds__(512, 1) void gemm_mfma_nt_256_kernel(const GemmArgs
     }
 #undef AXHIP_FENCE
 
-    gemm_store_tiles16<BF16>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l16, g4);
+    // the tile buffers become the staging area of the epilogue: no load of this work-group is still on its way into them
+    // (past the last tile they write zeros), and every wave has its last fragments
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    gemm_store_tiles16<BF16>(g, acc, m0 + wm, n0 + wn, bz * g.sc, l16, g4, big_lds + wave * 16384);
 }
 
 // --------------------------------------------------- MFMA NT, multi-stage ring
