@@ -6,6 +6,8 @@
     python -m axiom_amd.profile_summary traffic <FETCH_SIZE dir> <WRITE_SIZE dir>
                                                                        HBM bytes per launch of bench.py's workloads
     python -m axiom_amd.profile_summary survey  <bench.py output>      the `row_program_survey` of a bench line as a table
+    python -m axiom_amd.profile_summary by-grid <dir> [<dir> ...]      durations and counter averages of the product kernels
+                                                                       per (kernel, grid size): one kernel, several sizes
 
 `<dir>` is what `rocprofv3 ... -f csv -d <dir> -o <name>` wrote: `<name>_kernel_trace.csv` and, for a counter run,
 `<name>_counter_collection.csv` (searched recursively).  `traffic` scales FETCH_SIZE / WRITE_SIZE (KiB per dispatch) by
@@ -123,6 +125,45 @@ def survey(path: str) -> None:
               f"{100 * max(fc):.1f} %); the event bracketing that was taken off: median {ov[len(ov) // 2]:.1f} us per launch.")
 
 
+def by_grid(dirs: list[str], needles: tuple[str, ...] = ("gemm", "Cijk")) -> None:
+    """Durations and counter averages per (kernel, grid size): one kernel serves several problem sizes in a run.  A
+    kernel whose grid is the same for every size (the vendor's stream-K kernels) is split at 130 us instead."""
+    import collections
+    import csv
+
+    def short(n: str) -> str:
+        n = n.replace("(axhip::GemmArgs, int, int)", "")
+        return n if len(n) < 70 else "..." + n[-60:]
+
+    for d in dirs:
+        dur = {}
+        for f in _find(d, "kernel_trace.csv"):
+            acc = collections.defaultdict(list)
+            for r in csv.DictReader(open(f)):
+                us = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
+                dur[r["Dispatch_Id"]] = us
+                if not any(n in r["Kernel_Name"] for n in needles):
+                    continue
+                grid = r.get("Grid_Size") or r.get("Grid_Size_X")
+                if "MT256x256x64" in r["Kernel_Name"]:
+                    grid += " short" if us < 130 else " long"
+                acc[(short(r["Kernel_Name"]), grid)].append(us)
+            for k, v in sorted(acc.items()):
+                v.sort()
+                print(f"{d}: `{k[0]}` grid {k[1]}: {len(v)} launches, average {sum(v) / len(v):.1f} us, median {v[len(v) // 2]:.1f}, shortest {v[0]:.1f}")
+        for f in _find(d, "counter_collection.csv"):
+            acc = collections.defaultdict(lambda: collections.defaultdict(list))
+            for r in csv.DictReader(open(f)):
+                if not any(n in r["Kernel_Name"] for n in needles):
+                    continue
+                grid = r.get("Grid_Size") or r.get("Grid_Size_X")
+                if "MT256x256x64" in r["Kernel_Name"]:
+                    grid += " short" if dur.get(r["Dispatch_Id"], 0) < 130 else " long"
+                acc[(short(r["Kernel_Name"]), grid)][r["Counter_Name"]].append(float(r["Counter_Value"]))
+            for k, cs in sorted(acc.items()):
+                print(f"{d}: `{k[0]}` grid {k[1]}: " + " ".join(f"{c}={sum(v) / len(v):.4g}" for c, v in sorted(cs.items())))
+
+
 def main() -> int:
     if len(sys.argv) >= 3 and sys.argv[1] == "trace":
         trace(sys.argv[2])
@@ -130,6 +171,8 @@ def main() -> int:
         counters(sys.argv[2:])
     elif len(sys.argv) == 4 and sys.argv[1] == "traffic":
         traffic(sys.argv[2], sys.argv[3])
+    elif len(sys.argv) >= 3 and sys.argv[1] == "by-grid":
+        by_grid(sys.argv[2:])
     elif len(sys.argv) == 3 and sys.argv[1] == "survey":
         survey(sys.argv[2])
     else:
