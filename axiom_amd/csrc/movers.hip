@@ -148,18 +148,32 @@ __global__ __launch_bounds__(256) void pad_kernel(const PadArgs a) {
     }
 }
 
-// The same with V consecutive elements of the innermost output dimension per thread (its extent is a multiple of V,
-// the output 16-byte aligned): one decomposition of the index and one 16-byte store per V elements.
+// The same with V consecutive elements of the innermost output dimension per thread (V elements are 16 bytes): one
+// decomposition of the index per V elements.  A group whose sources are a run of the innermost source dimension --
+// the interior, a wrapped-around run of a circular pad, or, backwards, the mirror image of a reflected pad -- is one
+// 16-byte load and one 16-byte store (2- or 4-byte aligned: rows start wherever the extents put them); the groups on
+// a border, a row's last, shorter group and strided sources go element by element.
 // IDX: int32_t when every index and offset fits.
 template <typename IDX, int V>
 __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
-    const IDX stride = static_cast<IDX>(gridDim.x) * 256, groups = static_cast<IDX>(a.total / V);
     const int L = a.ndim - 1;
-    const IDX inner = static_cast<IDX>(a.out_shape[L]) / V, before = static_cast<IDX>(a.before[L]), n_src = static_cast<IDX>(a.src_shape[L]),
-              st = static_cast<IDX>(a.src_strides[L]);
+    const IDX out_last = static_cast<IDX>(a.out_shape[L]), inner = (out_last + V - 1) / V;
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, groups = static_cast<IDX>(a.total / out_last) * inner;
+    const IDX before = static_cast<IDX>(a.before[L]), n_src = static_cast<IDX>(a.src_shape[L]), st = static_cast<IDX>(a.src_strides[L]);
+    constexpr int ES = 16 / V;
+    uint4_t fill; // V copies of the constant in the element type
+    if constexpr (V == 4) {
+        fill = uint4_t{__float_as_uint(a.value), __float_as_uint(a.value), __float_as_uint(a.value), __float_as_uint(a.value)};
+    } else {
+        const uint32_t h = a.dtype == AXHIP_DTYPE_BF16 ? pack_bf16x2(a.value, a.value) : pack_f16x2(a.value, a.value);
+        fill = uint4_t{h, h, h, h};
+    }
+    const bool rows_aligned = out_last % V == 0 && (reinterpret_cast<uintptr_t>(a.dst) & 15u) == 0; // every group's 16 bytes of output are aligned
     for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < groups; i += stride) {
-        IDX rem = i / inner, off = 0;
-        const IDX c0 = (i - rem * inner) * V - before;
+        const IDX row = i / inner, g = i - row * inner;
+        IDX rem = row, off = 0;
+        const IDX c0 = g * V - before;
+        const int nvalid = static_cast<int>(out_last - g * V < V ? out_last - g * V : V);
         bool inside = true;
         for (int d = L - 1; d >= 0; --d) {
             const IDX n = static_cast<IDX>(a.out_shape[d]);
@@ -169,13 +183,42 @@ __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
             inside = inside && c >= 0;
             off += c * static_cast<IDX>(a.src_strides[d]);
         }
-        float v[V];
-#pragma unroll
-        for (int e = 0; e < V; ++e) {
-            const IDX c = pad_source<IDX>(c0 + e, n_src, a.mode);
-            v[e] = inside && c >= 0 ? load_any(a.src, a.dtype, off + c * st) : a.value;
+        const int64_t out_index = static_cast<int64_t>(row) * out_last + static_cast<int64_t>(g) * V;
+        if (nvalid == V && a.mode == AXHIP_PAD_CONSTANT && (!inside || c0 + V <= 0 || c0 >= n_src)) { // nothing but the constant
+            char *out = static_cast<char *>(a.dst) + out_index * ES;
+            if (rows_aligned) *reinterpret_cast<uint4_t *>(out) = fill;
+            else reinterpret_cast<uint4_unaligned_t *>(out)->v = fill;
+            continue;
         }
-        store_vec<V>(a.dst, a.dtype, static_cast<int64_t>(i) * V, v);
+        if (inside && st == 1 && nvalid == V) {
+            const IDX first = pad_source<IDX>(c0, n_src, a.mode), last = pad_source<IDX>(c0 + V - 1, n_src, a.mode);
+            const bool forward = first >= 0 && last - first == V - 1, backward = last >= 0 && first - last == V - 1;
+            if (forward || backward) {
+                uint4_t w = reinterpret_cast<const uint4_unaligned_t *>(static_cast<const char *>(a.src) + (static_cast<int64_t>(off) + (forward ? first : last)) * ES)->v;
+                if (backward) {
+                    if constexpr (V == 4) w = uint4_t{w.w, w.z, w.y, w.x};
+                    else w = uint4_t{(w.w >> 16) | (w.w << 16), (w.z >> 16) | (w.z << 16), (w.y >> 16) | (w.y << 16), (w.x >> 16) | (w.x << 16)};
+                }
+                char *out = static_cast<char *>(a.dst) + out_index * ES;
+                if (rows_aligned) *reinterpret_cast<uint4_t *>(out) = w;
+                else reinterpret_cast<uint4_unaligned_t *>(out)->v = w;
+                continue;
+            }
+        }
+        if (rows_aligned) { // (then every group is whole)
+            float v[V];
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const IDX c = pad_source<IDX>(c0 + e, n_src, a.mode);
+                v[e] = inside && c >= 0 ? load_any(a.src, a.dtype, off + c * st) : a.value;
+            }
+            store_vec<V>(a.dst, a.dtype, out_index, v);
+            continue;
+        }
+        for (int e = 0; e < nvalid; ++e) {
+            const IDX c = pad_source<IDX>(c0 + e, n_src, a.mode);
+            store_any(a.dst, a.dtype, out_index + e, inside && c >= 0 ? load_any(a.src, a.dtype, off + c * st) : a.value);
+        }
     }
 }
 
@@ -877,11 +920,13 @@ int axhip_pad_mode(const void *src, void *dst, int32_t dtype, int32_t ndim, cons
     int rc = ensure_init();
     if (rc) return rc;
     const int V = dtype == AXHIP_DTYPE_F32 ? 4 : 8;
-    if (ndim >= 1 && a.out_shape[ndim - 1] % V == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+    if (ndim >= 1 && a.out_shape[ndim - 1] >= V && a.total > 0 && (reinterpret_cast<uintptr_t>(dst) & (dtype == AXHIP_DTYPE_F32 ? 3u : 1u)) == 0 &&
+        (reinterpret_cast<uintptr_t>(src) & (dtype == AXHIP_DTYPE_F32 ? 3u : 1u)) == 0) {
         int64_t reach = a.total; // the largest index or source offset the kernel forms
         for (int d = 0; d < ndim; ++d) reach = std::max(reach, (a.src_shape[d] + a.out_shape[d]) * std::max<int64_t>(a.src_strides[d], 1));
         const bool small = reach < (int64_t(1) << 31) - (1 << 20);
-        const int64_t blocks = std::min<int64_t>((a.total / V + 255) / 256, 256 * 64);
+        const int64_t n_groups = a.total / a.out_shape[ndim - 1] * ((a.out_shape[ndim - 1] + V - 1) / V);
+        const int64_t blocks = std::min<int64_t>((n_groups + 255) / 256, 256 * 64);
         hipStream_t s = resolve_stream(stream);
         if (V == 4) {
             if (small) hipLaunchKernelGGL((pad_vec_kernel<int32_t, 4>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);

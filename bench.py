@@ -508,7 +508,20 @@ def bench_survey(torch, capi, stream, steps, warmup):
     res["where(mask,x,y)_bf16_16384x4096"] = with_cold(
         {"kernel": "where_vec", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
          "finite": bool(torch.equal(wout, torch.where(mask.bool(), xb, yb)))}, launch, avg_ms, nbytes)
-    del xb, yb, mask, wout
+    del yb, mask, wout
+    # the convolution front end's mover: reflect padding of a (N, C, L) signal along L (Whisper pads its mel frames this way)
+    pin = xb.view(16, 1024, 4096)
+    pout = torch.empty((16, 1024, 4096 + 512), dtype=bf, device="cuda")
+    pshape, pstr = (C.c_int64 * 3)(16, 1024, 4096), (C.c_int64 * 3)(1024 * 4096, 4096, 1)
+    pb, pa_ = (C.c_int64 * 3)(0, 0, 256), (C.c_int64 * 3)(0, 0, 256)
+    launch = lambda: capi.check(lib.axhip_pad_mode(pin.data_ptr(), pout.data_ptr(), capi.DTYPE_BF16, 3, pshape, pstr, pb, pa_, capi.PAD["reflect"], 0.0, sp))
+    torch.cuda.synchronize()
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
+    nbytes = (pin.numel() + pout.numel()) * 2
+    res["pad_reflect_bf16_16x1024x4096_by_256"] = with_cold(
+        {"kernel": "pad", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+         "finite": bool(torch.equal(pout, torch.nn.functional.pad(pin.float(), (256, 256), mode="reflect").to(bf)))}, launch, avg_ms, nbytes)
+    del xb, pin, pout
     # rows of odd length
     for rows, cols, dt, name in ((30000, 1500, bf, "bf16"), (16384, 4100, bf, "bf16"), (16384, 4097, bf, "bf16"), (16384, 1501, f32, "f32")):
         t = rnd((rows, cols), dt)
