@@ -329,6 +329,14 @@ bool rows_prog_grid_pays(const AxhipRowsProgram &P, int group, int it) {
     // threads (wavefront rows stage it in LDS once per block when the chunks start at the row's first element) --
     // 1024-thread rows gain even so: their unaligned form spills (layer norm over 50 257 fp32 columns: 404 -> 172 us).
     if (group < 64) return true; // short rows: on the grid they share a wavefront, from their first element each takes one
+    // AXHIP_ROWS_GRID=1 / 0 (read once): the grid wherever a plan exists for it / never beyond the short rows -- a
+    // tuning switch for measurements
+    static const int forced = [] {
+        const char *e = getenv("AXHIP_ROWS_GRID");
+        return e && *e ? atoi(e) : -1;
+    }();
+    if (forced == 1) return true;
+    if (forced == 0) return false;
     if (group * it <= 128) return false;
     if (group > 512) return true;
     auto rowvec = [&](int idx) { return idx >= 0 && idx < P.n_operands && P.operands[idx].kind == AXHIP_BK_ROWVEC; };
@@ -455,18 +463,19 @@ bool plan_rows(const AxhipRowsProgram &P, bool tight, bool ragged, bool grid, Ro
         }();
         int64_t best = 0;
         for (int i = 0; i < 4; ++i) {
-            if (forced == groups[i] && (chunks + groups[i] - 1) / groups[i] <= 8 && chunks >= groups[i]) {
+            if (forced == groups[i] && (chunks + groups[i] - 1) / groups[i] <= (groups[i] == 64 ? 10 : 8) && chunks >= groups[i]) {
                 group = groups[i];
                 it = static_cast<int>((chunks + groups[i] - 1) / groups[i]);
                 break;
             }
             const int64_t n = (chunks + groups[i] - 1) / groups[i];
             // up to 8 chunks per thread; a wavefront row may take 9 or 10 (a row just past 512 chunks would otherwise
-            // leave a third of a 256-thread block idle) while its registers still allow 4 waves per SIMD
+            // leave a third of a 256-thread block idle) while the row fits the registers of 2 waves per SIMD (two 16-bit
+            // streams of 4099 columns, held as fp32 as well: 144 registers, 72 against 95 us for the 256-thread plan)
             if (n > 8) {
                 const bool resident_f32 = P.row_op != AXHIP_ROWOP_NONE && (dt == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX);
                 const int64_t held = (raw_words_per_chunk(P) + (resident_f32 ? rows_prog_chunk_elems(P) : 0)) * n;
-                if (!(groups[i] == 64 && n <= 10 && held <= 112)) continue;
+                if (!(groups[i] == 64 && n <= 10 && held <= 160)) continue;
             }
             if (group == 0 || n * groups[i] < best) {
                 group = groups[i];

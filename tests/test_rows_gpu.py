@@ -465,6 +465,28 @@ def test_scaled_and_biased_softmax_on_the_specialised_kernels(dt):
     assert close32(got, axo.softmax(axo.binary("add", axo.binary("mul", x, np.array([0.3], np.float32), kind="scalar"), y)))
 
 
+def test_two_stream_rows_just_past_512_chunks_take_nine_or_ten_chunks_per_lane():
+    """Rows of 513 to 640 chunks with a second full-size stream: a wavefront with 9 or 10 chunks per lane (the registers
+    of 2 waves per SIMD) instead of a 256-thread block with a third of it idle; values against float64."""
+    g = axo.PCG64(123)
+    for cols, ragged in ((4099, True), (4104, False), (5000, False)):
+        x, y = axo.to_bits(g.normal((37, cols)) * 2, BF16), axo.to_bits(g.normal((37, cols)), BF16)
+        w, b = axo.to_bits(g.uniform((cols,), 0.5, 1.5), BF16), axo.to_bits(g.uniform((cols,), -0.5, 0.5), BF16)
+        t = axo.to_f32(x, BF16).astype(np.float64) + axo.to_f32(y, BF16)
+        it = 9 if cols < 4609 else 10
+        prog = gh.Rows(x, BF16).binary("add", y).row_op("layernorm", 1e-5, w=w, b=b)
+        got = axo.to_f32(prog.run(), BF16).astype(np.float64)
+        assert prog.kernel_name() == f"rows_jit_addf_layernorm_wb_bf16_g64_it{it}" + ("_ragged" if ragged else ""), prog.kernel_name()
+        mu, var = t.mean(-1, keepdims=True), t.var(-1, keepdims=True)
+        want = (t - mu) / np.sqrt(var + 1e-5) * axo.to_f32(w, BF16) + axo.to_f32(b, BF16)
+        assert np.max(np.abs(got - want)) < 3e-2, cols
+        prog = gh.Rows(x, BF16).binary("add", y).row_op("softmax")
+        got = axo.to_f32(prog.run(), BF16).astype(np.float64)
+        assert f"_g64_it{it}" in prog.kernel_name(), prog.kernel_name()
+        e = np.exp(t - t.max(-1, keepdims=True))
+        assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < 2e-2, cols
+
+
 @pytest.mark.parametrize("post", ["silu", "sigmoid", "tanh"])
 def test_fast_activations_after_a_norm_in_16_bit(post):
     g = axo.PCG64(17)
