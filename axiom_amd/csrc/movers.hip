@@ -701,6 +701,100 @@ __global__ __launch_bounds__(256) void softmax_strided_vec_kernel(const void *sr
     }
 }
 
+// A long axis read ONCE: a 1024-thread block holds an [axis, TX vectors] tile of the input in registers, as the raw
+// 16-byte vectors it was loaded as -- thread (ty, tx) the rows ty, ty + TY, ... (RPT of them, TY = 1024 / TX) of
+// vector column tx, so TX neighbouring lanes read TX * 16 consecutive bytes of a row --, works out the columns'
+// maxima and sums across its threads (shuffles between the lanes of a wave that share a column, LDS between the
+// waves) and writes the results from the same registers.  TX = 16, 8 or 4 for axes of up to 1024, 2048 or 4096
+// elements (16 rows per thread at most: 64 registers of raw words).  With TX = 4 a row's 64 bytes are half a cache
+// line: the two blocks that share the lines run on the same XCD (block b lands on XCD b % 8), so the second one finds
+// them in that L2.
+template <bool LOG, int DT, int RPT>
+__global__ __launch_bounds__(1024) void softmax_axis_tile_kernel(const void *src, int64_t outer, int64_t axis, int64_t inner, int tx_log2, void *dst) {
+    constexpr int V = DT == AXHIP_DTYPE_F32 ? 4 : 8;
+    constexpr float LOG2E = 1.44269504088896340736f, LN2 = 0.69314718055994530942f;
+    __shared__ float red[16][16][V + 1];
+    const int TX = 1 << tx_log2, TY = 1024 >> tx_log2;
+    const int tid = threadIdx.x, tx = tid & (TX - 1), ty = tid >> tx_log2, wave = tid / WAVE;
+    const int64_t ivecs = inner / V, ctiles = (ivecs + TX - 1) / TX, tiles = outer * ctiles;
+    const int share = TX >= 8 ? 1 : 8 / TX; // blocks per cache line of a row
+    const int n = static_cast<int>(axis);
+    const int64_t slot = blockIdx.x / 8, xcd = blockIdx.x % 8;
+    const int64_t tile = ((slot / share) * 8 + xcd) * share + slot % share;
+    if (tile >= tiles) return; // (whole block)
+    const int64_t o = tile / ctiles, iv = (tile - o * ctiles) * TX + tx;
+    const bool there = iv < ivecs;
+    const uint4_t *first = reinterpret_cast<const uint4_t *>(src) + o * axis * ivecs + (there ? iv : 0);
+    uint4_t raw[RPT];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) raw[r] = first[static_cast<int64_t>(min(ty + r * TY, n - 1)) * ivecs];
+    // column statistic over the block: lanes of a wave that share tx, then the 16 waves
+    auto across = [&](float (&x)[V], bool is_max) {
+        for (int d = TX; d < WAVE; d <<= 1) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float y = __shfl_xor(x[e], d, WAVE);
+                x[e] = is_max ? fmaxf(x[e], y) : x[e] + y;
+            }
+        }
+        __syncthreads(); // the previous statistic has been read
+        if ((tid % WAVE) < TX) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) red[wave][tx][e] = x[e];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            float a = red[0][tx][e];
+            for (int w = 1; w < 16; ++w) a = is_max ? fmaxf(a, red[w][tx][e]) : a + red[w][tx][e];
+            x[e] = a;
+        }
+    };
+    float m[V], l[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        m[e] = -INFINITY;
+        l[e] = 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+        if (ty + r * TY < n) {
+            float t[V];
+            arg_unpack<DT>(raw[r], t);
+#pragma unroll
+            for (int e = 0; e < V; ++e) m[e] = fmaxf(m[e], t[e] * LOG2E);
+        }
+    across(m, true);
+    float ref[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) ref[e] = m[e] == -INFINITY ? 0.0f : m[e]; // (nothing finite: every term is 2^-inf = 0)
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+        if (ty + r * TY < n) {
+            float t[V];
+            arg_unpack<DT>(raw[r], t);
+#pragma unroll
+            for (int e = 0; e < V; ++e) l[e] += __builtin_amdgcn_exp2f(t[e] * LOG2E - ref[e]);
+        }
+    across(l, false);
+    float shift[V], inv[V]; // result = 2^(t - shift) * inv, or (t - shift) * ln 2 with the logarithm of the sum inside shift
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        shift[e] = LOG ? m[e] + __builtin_amdgcn_logf(l[e]) : ref[e]; // (v_log_f32 is the base-2 logarithm)
+        inv[e] = 1.0f / l[e];
+    }
+    if (!there) return;
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+        if (ty + r * TY < n) {
+            float v[V];
+            arg_unpack<DT>(raw[r], v);
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[e] = LOG ? (v[e] * LOG2E - shift[e]) * LN2 : __builtin_amdgcn_exp2f(v[e] * LOG2E - shift[e]) * inv[e];
+            store_vec<V>(dst, DT, (o * axis + ty + r * TY) * inner + iv * V, v);
+        }
+}
+
 // any inner extent and alignment: a thread per (outer, inner) position, three sweeps
 template <bool LOG>
 __global__ __launch_bounds__(256) void softmax_strided_kernel(const void *src, int dt, int64_t outer, int64_t axis, int64_t inner, void *dst) {
@@ -762,6 +856,14 @@ int launch_reduce_axis(const void *src, int dtype, int64_t outer, int64_t axis, 
 } // namespace axhip
 
 using namespace axhip;
+
+namespace {
+// AXHIP_SOFTMAX_AXIS_TILE=0 (read at every call): long axes on the two-sweep kernel instead of the one-read tile kernel
+bool softmax_axis_tile_enabled() {
+    const char *e = getenv("AXHIP_SOFTMAX_AXIS_TILE");
+    return !(e && e[0] == '0');
+}
+} // namespace
 
 extern "C" {
 
@@ -1238,6 +1340,40 @@ int axhip_softmax_axis(const void *src, int32_t dtype, int64_t outer, int64_t ax
     const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
     if (inner % (16 / es) == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0) {
         const int64_t ivecs = inner / (16 / es);
+        // a long axis that a block can hold: one read.  Where it pays against the two-sweep kernel (one 1024-thread block per
+        // CU, whose load, arithmetic and store phases do not overlap): fp32 axes of 512 to 2048 elements (126 against 179 us
+        // on [16, 2048, 2048]), 16-bit axes of 1024 to 4096 (274 against 348 us on [64, 2048, 2048]); shorter axes and
+        // fp32 axes of 4096 (64-byte row pieces) stay on the two-sweep kernel
+        const bool tile_pays = dtype == AXHIP_DTYPE_F32 ? axis >= 512 && axis <= 2048 : axis >= 1024 && axis <= 4096;
+        if (tile_pays && softmax_axis_tile_enabled()) {
+            const int tx_log2 = axis <= 1024 ? 4 : axis <= 2048 ? 3 : 2;
+            const int TXv = 1 << tx_log2, TYv = 1024 >> tx_log2;
+            const int64_t tiles = outer * ((ivecs + TXv - 1) / TXv);
+            const int share = TXv >= 8 ? 1 : 8 / TXv;
+            const int64_t nblocks = (tiles + 8 * share - 1) / (8 * share) * (8 * share);
+            if (nblocks < (int64_t(1) << 31)) {
+                const bool few = (axis + TYv - 1) / TYv <= 4; // rows per thread
+#define AXHIP_SMT_R(LOG, DT, R) hipLaunchKernelGGL((softmax_axis_tile_kernel<LOG, DT, R>), dim3(static_cast<unsigned>(nblocks)), dim3(1024), 0, s, src, outer, axis, inner, tx_log2, dst)
+#define AXHIP_SMT_DT(LOG, DT)                                                                                                              \
+    do {                                                                                                                                   \
+        if (few) AXHIP_SMT_R(LOG, DT, 4);                                                                                                  \
+        else AXHIP_SMT_R(LOG, DT, 16);                                                                                                     \
+    } while (0)
+#define AXHIP_SMT(LOG)                                                                                                                     \
+    do {                                                                                                                                   \
+        if (dtype == AXHIP_DTYPE_F32) AXHIP_SMT_DT(LOG, AXHIP_DTYPE_F32);                                                                  \
+        else if (dtype == AXHIP_DTYPE_F16) AXHIP_SMT_DT(LOG, AXHIP_DTYPE_F16);                                                             \
+        else AXHIP_SMT_DT(LOG, AXHIP_DTYPE_BF16);                                                                                          \
+    } while (0)
+                if (is_log) AXHIP_SMT(true);
+                else AXHIP_SMT(false);
+#undef AXHIP_SMT
+#undef AXHIP_SMT_DT
+#undef AXHIP_SMT_R
+                AXHIP_CHECK_HIP(hipGetLastError());
+                return AXHIP_OK;
+            }
+        }
         // a short axis with plenty of results: a thread per vector walks it alone
         const bool flat = axis <= 32 && outer * ((ivecs + 255) / 256) >= 1024;
         const bool wide = outer * ((ivecs + 31) / 32) >= 1024;

@@ -338,7 +338,11 @@ def test_softmax_along_inner_axes_matches_the_oracle(dt):
     for outer, axis, inner, scale in ((1, 37, 4096, 1.0), (6, 130, 72, 3.0), (3, 1, 64, 1.0), (64, 300, 8, 10.0), (5, 77, 9, 2.0), (2, 1000, 33, 1.0),
                                       (1, 5000, 24, 4.0), (1200, 7, 1024, 2.0),
                                       # short axes with many results: the axis stays in a thread's registers (up to 16 elements)
-                                      (1100, 16, 512, 3.0), (1030, 13, 2048, 1.0), (1100, 17, 512, 2.0), (1500, 1, 512, 1.0), (1040, 4, 520, 5.0)):
+                                      (1100, 16, 512, 3.0), (1030, 13, 2048, 1.0), (1100, 17, 512, 2.0), (1500, 1, 512, 1.0), (1040, 4, 520, 5.0),
+                                      # long axes that a block holds in registers (fp32: 512 to 2048 elements, 16-bit: 1024 to 4096; tiles of 16, 8 or 4 vectors,
+                                      # column tiles that are not whole, one element past a tile size)
+                                      (2, 1024, 136, 3.0), (3, 1025, 72, 1.0), (2, 2048, 40, 8.0), (1, 2049, 24, 2.0), (2, 4096, 24, 1.0), (5, 600, 264, 2.0),
+                                      (3, 256, 4096, 1.0), (1, 4097, 16, 1.0)):
         x = (rng.normal(size=(outer, axis, inner)) * scale).astype(np.float32)
         bits = x if dt == F32 else axo.to_bits(x, dt)
         d = gh.to_dev(bits)
