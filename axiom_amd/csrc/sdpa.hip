@@ -1755,11 +1755,13 @@ DecodeSplit decode_split_plan(const AxhipSdpaParams &p, bool has_mask) {
     DecodeSplit d{0, 0, 0, 0};
     const bool half = p.dtype == AXHIP_DTYPE_BF16 || p.dtype == AXHIP_DTYPE_F16;
     const int64_t slices = static_cast<int64_t>(p.batch) * p.heads;
-    if (!half || has_mask || p.is_causal || p.seq_q <= 0 || p.seq_q > BM || slices <= 0 || slices > 96 || p.seq_kv < 1024 || p.head_dim <= 32 ||
+    if (!half || has_mask || p.is_causal || p.seq_q <= 0 || p.seq_q > BM || slices <= 0 || slices > 384 || p.seq_kv < 1024 || p.head_dim <= 32 ||
         p.head_dim > 128 || p.head_dim % 8 != 0 || slices * p.seq_kv * p.head_dim < (int64_t(8) << 20) || !sdpa_decode_split)
         return d;
     d.DD = p.head_dim <= 64 ? 64 : 128;
-    const int parts = static_cast<int>(std::min<int64_t>(std::min<int64_t>(64, (512 + slices - 1) / slices), p.seq_kv / 256));
+    // (enough work-groups for four per CU: 128 (batch, head) slices of 16384 keys ran at 32 % of the HBM peak unsplit -- half
+    // the CUs idle --, 256 slices of 8192 keys at 52 %)
+    const int parts = static_cast<int>(std::min<int64_t>(std::min<int64_t>(64, ((slices <= 96 ? 512 : 1024) + slices - 1) / slices), p.seq_kv / 256));
     d.kchunk = ((p.seq_kv + parts - 1) / parts + BN - 1) / BN * BN;
     d.ksplit = (p.seq_kv + d.kchunk - 1) / d.kchunk;
     d.bytes = static_cast<size_t>(slices) * d.ksplit * p.seq_q * (d.DD + 1) * sizeof(float);

@@ -6,7 +6,7 @@
     python -m axiom_amd.profile_summary traffic <FETCH_SIZE dir> <WRITE_SIZE dir>
                                                                        HBM bytes per launch of bench.py's workloads
     python -m axiom_amd.profile_summary survey  <bench.py output>      the `row_program_survey` of a bench line as a table
-    python -m axiom_amd.profile_summary by-grid <dir> [<dir> ...]      durations and counter averages of the product kernels
+    python -m axiom_amd.profile_summary by-grid [--match=a,b] <dir> [<dir> ...]   durations and counter averages of the product kernels (or of those whose names contain a, b, ...)
                                                                        per (kernel, grid size): one kernel, several sizes
 
 `<dir>` is what `rocprofv3 ... -f csv -d <dir> -o <name>` wrote: `<name>_kernel_trace.csv` and, for a counter run,
@@ -132,7 +132,7 @@ def by_grid(dirs: list[str], needles: tuple[str, ...] = ("gemm", "Cijk")) -> Non
     import csv
 
     def short(n: str) -> str:
-        n = n.replace("(axhip::GemmArgs, int, int)", "")
+        n = n.replace("(axhip::GemmArgs, int, int)", "").split("(")[0]
         return n if len(n) < 70 else "..." + n[-60:]
 
     for d in dirs:
@@ -172,7 +172,11 @@ def main() -> int:
     elif len(sys.argv) == 4 and sys.argv[1] == "traffic":
         traffic(sys.argv[2], sys.argv[3])
     elif len(sys.argv) >= 3 and sys.argv[1] == "by-grid":
-        by_grid(sys.argv[2:])
+        args = sys.argv[2:]
+        if args[0].startswith("--match="):  # substrings of the kernel names to keep (default: the product kernels)
+            by_grid(args[1:], tuple(args[0][len("--match="):].split(",")))
+        else:
+            by_grid(args)
     elif len(sys.argv) == 3 and sys.argv[1] == "survey":
         survey(sys.argv[2])
     else:

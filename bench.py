@@ -602,8 +602,9 @@ def bench_gemm(torch, capi, stream, steps, warmup):
     sp = C.c_void_p(stream.cuda_stream)
     res = {}
     g = torch.Generator(device="cuda").manual_seed(42)
-    # (the last two: decoding steps, one and four tokens against a weight matrix -- bound by reading the weights)
-    for M, N, K in ((4096, 4096, 4096), (8192, 4096, 4096), (1500, 1280, 1280), (1, 4096, 4096), (4, 4096, 4096)):
+    # (the last three: decoding steps, one and four tokens against a weight matrix -- bound by reading the weights; the 512 MiB
+    # matrix is larger than the 256 MiB memory-side cache, so its rate is an HBM rate)
+    for M, N, K in ((4096, 4096, 4096), (8192, 4096, 4096), (1500, 1280, 1280), (1, 4096, 4096), (4, 4096, 4096), (1, 16384, 16384)):
         a = torch.randn((M, K), generator=g, device="cuda").to(torch.bfloat16)
         w = (torch.randn((N, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
         c = torch.empty((M, N), device="cuda", dtype=torch.bfloat16)
@@ -627,6 +628,28 @@ def bench_gemm(torch, capi, stream, steps, warmup):
             nbytes = 2.0 * (N * K + M * K + M * N)
             res[f"gemm_nt_bf16_{M}x{N}x{K}"].update({"bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9})
         del a, w, c
+    # a decoding step of attention: one query per (batch, head) against 16384 keys -- the keys are split between
+    # work-groups and the partial states merged by a second kernel; K and V (1 GiB) are larger than the memory-side cache
+    B, H, S, D = 4, 32, 16384, 128
+    q = torch.randn((B, H, 1, D), generator=g, device="cuda").to(torch.bfloat16)
+    k, v = (torch.randn((B, H, S, D), generator=g, device="cuda").to(torch.bfloat16) for _ in range(2))
+    o = torch.empty_like(q)
+    p = capi.SdpaParams()
+    p.dtype, p.batch, p.heads, p.seq_q, p.seq_kv, p.head_dim = capi.DTYPE_BF16, B, H, 1, S, D
+    p.scale, p.is_causal = -1.0, 0
+    p.q_strides[:] = (H * D, D, D)
+    p.o_strides[:] = (H * D, D, D)
+    for arr in (p.k_strides, p.v_strides):
+        arr[:] = (H * S * D, S * D, D)
+    args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, C.byref(p), sp)
+    torch.cuda.synchronize()
+    avg_ms, min_ms, warm_n = time_launches(torch, stream, lambda: capi.check(lib.axhip_sdpa_fwd(*args)), steps, warmup)
+    nbytes = 2.0 * (2 * B * H * S * D + 2 * B * H * D)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    res[f"sdpa_decode_bf16_b{B}h{H}s{S}d{D}"] = {"kernel": lib.axhip_sdpa_kernel_name(C.byref(p)).decode(), "avg_ms": avg_ms, "min_ms": min_ms, "warmup_launches": warm_n,
+                                                  "bytes": nbytes, "gbs": nbytes / (avg_ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                                  "max_abs_err_vs_fp32": float((o.float() - ref).abs().max().item())}
+    del q, k, v, o, ref
     return res
 
 

@@ -218,7 +218,9 @@ def test_decoding_steps_split_their_keys_between_work_groups(dt):
     partial results merged (head sizes 64, 128 and in between, ragged last chunks, one to 128 query rows, a key
     sequence with one dominant key in the last chunk); against float64."""
     tag = "bf16" if dt == BF16 else "f16"
-    for B, H, Sq, Skv, D in ((1, 8, 1, 8192, 128), (2, 8, 5, 9001, 64), (1, 30, 128, 3030, 96), (1, 32, 1, 4096, 128), (1, 64, 33, 3072, 48), (3, 32, 2, 1500, 64)):
+    for B, H, Sq, Skv, D in ((1, 8, 1, 8192, 128), (2, 8, 5, 9001, 64), (1, 30, 128, 3030, 96), (1, 32, 1, 4096, 128), (1, 64, 33, 3072, 48), (3, 32, 2, 1500, 64),
+                               # up to 384 (batch, head) slices are split (enough work-groups for four per CU)
+                               (4, 32, 1, 2100, 128), (2, 160, 3, 1100, 64)):
         q, k, v = inputs(B, H, Sq, Skv, D, dt, seed=700 + Sq + D)
         kf = axo.to_f32(k, dt)
         kf[..., Skv - 3, :] = 4.0 * axo.to_f32(q, dt)[..., 0, :]  # a key far above the rest, in the last chunk
