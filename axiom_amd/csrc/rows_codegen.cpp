@@ -366,8 +366,11 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     const bool resident_f32 = P.input_dtype == AXHIP_DTYPE_F32 || P.n_pre > 0 || P.row_op == AXHIP_ROWOP_SOFTMAX || P.row_op == AXHIP_ROWOP_LOGSOFTMAX;
     const int held = all * it + (resident_f32 && P.row_op != AXHIP_ROWOP_NONE ? rows_prog_chunk_elems(P) * it : 0);
     plan->min_waves = (held + (heavy ? 3 * it + 16 : 0) > 72 || it > 8) ? 2 : 4;
-    // short rows on the grid: every row has a shift of its own, so the next row's chunk offsets are not this row's
-    if (group < 64 && plan->grid) plan->pipe = false;
+    // short rows on the grid: every row has a shift of its own, so a pipelined plan works out the next row's chunk
+    // offsets on top of this row's (AXHIP_ROWS_PIPE_SHORT_GRID=0, read once: not pipelined; layer norm with weight
+    // and bias over 170000 rows of 197 16-bit columns 63 against 79 us, softmax the same either way)
+    static const bool pipe_short_grid = [] { const char *e = getenv("AXHIP_ROWS_PIPE_SHORT_GRID"); return !(e && e[0] == '0'); }();
+    if (group < 64 && plan->grid && !pipe_short_grid) plan->pipe = false;
     // a 1024-thread block has 128 registers per thread whatever is asked for: no second set of raw words beyond that
     if (group == 1024 && held + (plan->pipe ? raw * it : 0) > 115) plan->pipe = false;
 }
@@ -403,6 +406,49 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
         if (o.kind == AXHIP_BK_FULL || o.kind == AXHIP_BK_ROWVEC) {
             if (!aligned16(o.ptr)) ragged = true;
             if (elem_size(o.dtype) != elem_size(dt)) same_size = false;
+        }
+    }
+    // Short rows of odd length, many of them: a row per lane (or per 2, 4 or 8 lanes) out of a span staged in LDS
+    // (every stream has its own geometry there, so the element sizes may differ).  All full-size streams must start
+    // on a 16-byte boundary.  Tuning switches, read once: AXHIP_ROWS_LANE=0 switches the plan off,
+    // AXHIP_ROWS_LANE_L=<1|2|4|8> sets the lanes per row, AXHIP_ROWS_LANE_VALS=<n> the values per lane from which a
+    // row is spread over more lanes, AXHIP_ROWS_LANE_MAX=<n> the values per lane beyond which the plan is not taken.
+    // Measured (16-bit softmax, % of the HBM peak with 1 / 2 / 4 / 8 lanes per row): 77 columns 71 / 73 / 61 / 54,
+    // 197 columns 54 / 66 / 68 / 71, 250 columns 50 / 67 / 75 / 74, 513 columns - / - / 61 / 68 (a wavefront per row:
+    // 50), 1001 columns - / - / 49 / 63 (a wavefront per row: 69).
+    if (tight && P.cols % e != 0 && P.rows >= kRowsProgLaneMinRows) {
+        static const bool lane_on = [] { const char *v = getenv("AXHIP_ROWS_LANE"); return !(v && v[0] == '0'); }();
+        static const int lane_l = [] { const char *v = getenv("AXHIP_ROWS_LANE_L"); return v ? std::atoi(v) : 0; }();
+        static const int lane_vals = [] { const char *v = getenv("AXHIP_ROWS_LANE_VALS"); return v ? std::atoi(v) : 64; }();
+        static const int lane_most = [] { const char *v = getenv("AXHIP_ROWS_LANE_MAX"); return v ? std::atoi(v) : 96; }();
+        bool ok = lane_on && aligned16(P.input) && (P.reduce != AXHIP_RED_NONE || aligned16(P.output));
+        int widest = elem_size(dt), nreg = 1;
+        if (P.reduce == AXHIP_RED_NONE) {
+            widest = std::max(widest, static_cast<int>(elem_size(P.output_dtype)));
+            if (elem_size(P.output_dtype) != elem_size(dt)) ++nreg;
+        }
+        for (int i = 0; i < P.n_operands; ++i)
+            if (used[i] && P.operands[i].kind == AXHIP_BK_FULL) {
+                ok = ok && aligned16(P.operands[i].ptr);
+                widest = std::max(widest, static_cast<int>(elem_size(P.operands[i].dtype)));
+                ++nreg;
+            }
+        const int64_t chunks = (P.cols + e - 1) / e;
+        int lanes = (lane_l == 1 || lane_l == 2 || lane_l == 4 || lane_l == 8) ? lane_l : 1;
+        // LDS bytes per wavefront and stream: the span, and room for a chunk that a lane reads past its end
+        auto bytes_for = [&](int l) { return (64 / l * P.cols * widest + 32 + 16 * l + 1023) / 1024 * 1024; };
+        if (lanes != lane_l)
+            while (lanes < 8 && ((chunks + lanes - 1) / lanes * e > lane_vals || nreg * bytes_for(lanes) > 36864)) lanes *= 2;
+        const int64_t it = (chunks + lanes - 1) / lanes;
+        const int64_t lane_bytes = bytes_for(lanes);
+        if (ok && it * e <= std::min(lane_most, 256) && nreg * lane_bytes <= 36864) {
+            rows_prog_plan_for(P, 64, static_cast<int>(it), false, plan, false);
+            plan->pipe = false;
+            plan->min_waves = it * e > 160 ? 1 : it * e > 64 ? 2 : 4;
+            plan->lane = true;
+            plan->lane_l = lanes;
+            plan->lane_bytes = static_cast<int>(lane_bytes);
+            return true;
         }
     }
     // a ragged row is addressed in 16-byte chunks of every vector it touches: all of them must share the element size
@@ -549,7 +595,7 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     const int red = P.reduce == AXHIP_RED_MEAN ? AXHIP_RED_SUM : P.reduce;
     std::ostringstream c;
     c << "constexpr int DT_IN = " << dt << ", DT_OUT = " << (P.reduce == AXHIP_RED_NONE ? P.output_dtype : dt) << ";\n";
-    c << "constexpr int GROUP = " << plan.group << ", IT = " << plan.it << ", E = " << rows_prog_chunk_elems(P) << ";\n";
+    c << "constexpr int GROUP = " << plan.group << ", IT = " << (plan.lane ? 1 : plan.it) << ", E = " << rows_prog_chunk_elems(P) << ";\n";
     const bool rerun = plan.rerun && resident; // (a 16-bit norm without a pre chain never holds its row as fp32 anyway)
     if (rerun) pipe = false;
     c << "constexpr bool RAGGED = " << (plan.ragged ? "true" : "false") << ", PIPE = " << (pipe ? "true" : "false") << ", RERUN = " << (rerun ? "true" : "false")
@@ -559,6 +605,7 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     c << "constexpr int HOLD = " << (plan.loop && P.row_op != AXHIP_ROWOP_NONE ? 48 / (raw_words_per_chunk(P) * plan.it) : 0) << ";\n";
     c << "constexpr int TAIL_FROM = " << (plan.ragged && plan.grid ? plan.tail_from : 0) << ";\n";
     c << "constexpr int MIN_WAVES = " << plan.min_waves << ";\n";
+    if (plan.lane) c << "constexpr int LANE_BYTES = " << plan.lane_bytes << ", LANE_IT = " << plan.it << ", LANE_L = " << plan.lane_l << ";\n";
     c << "constexpr int ROWOP = " << P.row_op << ", RED = " << red << ";\n";
     c << "constexpr int W_DT = " << w_dt << ", B_DT = " << b_dt << ", W_SLOT = " << w_slot << ", B_SLOT = " << b_slot << ";\n";
     static const char *kind_name[4] = {"FULL", "ROWV", "COLV", "SCAL"};
@@ -577,8 +624,9 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
 
     char hash[24];
     snprintf(hash, sizeof(hash), "%016llx", static_cast<unsigned long long>(fnv1a(S.chains, fnv1a(S.config))));
-    S.threads = plan.group > 256 ? plan.group : 256;
-    S.rows_per_block = S.threads / plan.group;
+    S.threads = plan.lane ? 64 : plan.group > 256 ? plan.group : 256;
+    S.rows_per_block = plan.lane ? 64 / plan.lane_l : S.threads / plan.group;
+    S.lane = plan.lane;
 
     std::string label = pre_label + rowop_token(P.row_op) + "_" + post_label;
     if (w_dt >= 0) label += b_dt >= 0 ? "wb_" : "w_";
@@ -586,6 +634,10 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     if (red != AXHIP_RED_NONE) label += red == AXHIP_RED_SUM ? "sum_" : red == AXHIP_RED_MAX ? "max_" : "min_";
     char tail[64];
     const bool other_out = P.reduce == AXHIP_RED_NONE && P.output_dtype != dt;
+    if (plan.lane) // (a row per lane; the LDS bytes per wavefront and stream in KiB)
+        snprintf(tail, sizeof(tail), "%s%s%s_lane%d_%dk_it%d", dt_name(dt), other_out ? "_to_" : "", other_out ? dt_name(P.output_dtype) : "", plan.lane_l,
+                 plan.lane_bytes / 1024, plan.it);
+    else
     snprintf(tail, sizeof(tail), "%s%s%s_g%d_it%d%s", dt_name(dt), other_out ? "_to_" : "", other_out ? dt_name(P.output_dtype) : "", plan.group, plan.it,
              plan.loop ? "_loop" : !plan.ragged ? "" : plan.grid ? "_grid" : "_ragged"); // (grid: ragged rows addressed on memory's 16-byte grid)
     S.label = label + tail;
@@ -616,6 +668,7 @@ std::string rows_prog_source(const RowsProgSpec &S, const std::string &body) {
     std::string src;
     src.reserve(body.size() + S.config.size() + S.chains.size() + 256);
     src += "#define AXP_NS " + ns + "\n#define AXP_KERNEL_NAME " + S.symbol + "\n";
+    if (S.lane) src += "#define AXP_LANE 1\n";
     src += "namespace " + ns + " { namespace cfg {\n" + S.config + "} }\n";
     src += body;
     src += "\nnamespace " + ns + " {\n" + S.chains + "}\n";

@@ -40,6 +40,9 @@ struct RowsProgPlan {
     bool pipe = false;     // the next row is requested before the current one is computed
     bool rerun = false;    // the row stays in registers as raw words; every pass unpacks it and applies the pre chain again
     int min_waves = 4;     // waves per SIMD the kernel's register allocation aims for
+    bool lane = false;     // short rows of odd length: a wavefront stages 64 / lane_l consecutive rows in LDS and lane_l lanes walk each
+    int lane_l = 1;        // (lane) lanes per row; `it` chunks per lane, held as fp32 after the first pass
+    int lane_bytes = 0;    // (lane) LDS bytes per wavefront and full-size stream
     int slots() const { return group * it; }
 };
 
@@ -51,6 +54,7 @@ struct RowsProgSpec {
     std::string symbol;     // extern "C" name of the kernel: axp_<hash of config and chains>
     int threads = 256;
     int rows_per_block = 4;
+    bool lane = false;      // the row-per-lane body (its text is compiled only for these kernels)
     int n_slots = 0;
     int slot_operand[8] = {}; // pointer slot -> index into AxhipRowsProgram::operands
     int n_imm = 0;
@@ -61,6 +65,8 @@ struct RowsProgSpec {
 // too short, a vector operand whose element size keeps a ragged row from its 16-byte chunks): the interpreter takes it.
 // tight = false: among the plan shapes the build compiles (64 or 256 threads per row, a few chunk counts per thread);
 // tight = true: the plan with the fewest idle chunk slots for this row length (64, 256 or 512 threads per row, any chunk count up to 8).
+// the row-per-lane plan is for arrays of at least this many rows (fewer rows want more than a wavefront per 64 of them)
+constexpr int64_t kRowsProgLaneMinRows = 32768;
 int rows_prog_chunk_elems(const AxhipRowsProgram &P); // elements per chunk: 4 when a full-size stream is fp32, else 8
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan);
 // The plan with its shape given (the build's generator enumerates the shapes itself).

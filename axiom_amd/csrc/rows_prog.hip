@@ -33,6 +33,7 @@ void make_struct_key(const AxhipRowsProgram &P, StructKey *k) {
     // (the address modulo 16 decides between the aligned, the grid and the unaligned form of a kernel)
     auto align_tag = [](const void *p) { return reinterpret_cast<const void *>(static_cast<uintptr_t>(reinterpret_cast<uintptr_t>(p) & 15u) + 16u); };
     q.cols = P.cols;
+    q.rows = P.rows >= kRowsProgLaneMinRows ? 1 : 0; // (arrays of many short rows have a plan of their own)
     q.input = align_tag(P.input);
     q.input_dtype = P.input_dtype;
     q.n_operands = P.n_operands;
@@ -123,7 +124,7 @@ Entry *find_or_make_entry(const AxhipRowsProgram &P) {
     e->eligible = has_tight || has_stock;
     e->has_builtin_alternative = false;
     static const bool forced_group = getenv("AXHIP_ROWS_GROUP") != nullptr; // (the tuning switch of the tight plan wins over the built-in shapes)
-    if (has_stock && (!has_tight || (!forced_group && stock.slots() * 100 <= tight.slots() * 115))) {
+    if (has_stock && (!has_tight || (!forced_group && !tight.lane && stock.slots() * 100 <= tight.slots() * 115))) {
         e->spec = stock_spec;
         e->is_builtin = true;
     } else if (has_tight) {

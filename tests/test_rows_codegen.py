@@ -159,15 +159,31 @@ def test_short_aligned_rows_share_a_wavefront():
     assert Prog(1 << 20, 256, BF16).op("square").reduce("mean").name() == "rows_static_square_reduce_sum_bf16_g32_it1"
     assert Prog(1 << 20, 264, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1"  # 33 chunks
     # odd lengths: the same on memory's 16-byte grid, a masked partial chunk at either end of every row
-    assert Prog(1 << 20, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g16_it1_grid"
-    assert Prog(1 << 20, 10, F32).row("logsoftmax").name() == "rows_jit_logsoftmax_f32_g4_it1_grid"
-    assert Prog(1 << 20, 5, BF16).row("softmax").name() == "rows_static_softmax_bf16_g4_it1_grid"  # shorter than a chunk
-    assert Prog(1 << 20, 197, BF16).row("layernorm", 2).name() == "rows_static_layernorm_wb_bf16_g32_it1_grid"
-    assert Prog(1 << 20, 250, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1_ragged"  # 33 chunks on the grid
+    assert Prog(1 << 14, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g16_it1_grid"
+    assert Prog(1 << 14, 10, F32).row("logsoftmax").name() == "rows_jit_logsoftmax_f32_g4_it1_grid"
+    assert Prog(1 << 14, 5, BF16).row("softmax").name() == "rows_static_softmax_bf16_g4_it1_grid"  # shorter than a chunk
+    assert Prog(1 << 14, 197, BF16).row("layernorm", 2).name() == "rows_static_layernorm_wb_bf16_g32_it1_grid"
+    assert Prog(1 << 14, 250, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it1_ragged"  # 33 chunks on the grid
     p = Prog(1 << 20, 77, BF16).row("softmax")
     p.p.output += 2  # input and output at different addresses modulo 16: a wavefront per row, from the row's first element
     assert p.name() == "rows_static_softmax_bf16_g64_it1_ragged"
     assert Prog(1 << 20, 96, BF16).op("mul", "colvec").op("tanh").row("softmax").name() == "rows_jit_mulc_tanh_softmax_bf16_g16_it1"
+
+
+def test_many_short_rows_of_odd_length_go_through_lds():
+    """From 32768 rows on: 64 / L consecutive rows per wavefront staged in LDS, L lanes per row (as few as keep a
+    lane's share of the row at 64 values or fewer), up to 96 values per lane; the label gives L, the LDS KiB per
+    wavefront and stream, and the chunks per lane.  The streams may differ in element size."""
+    assert Prog(1 << 20, 77, BF16).row("softmax").name() == "rows_jit_softmax_bf16_lane2_5k_it5"
+    assert Prog(1 << 20, 10, F32).row("logsoftmax").name() == "rows_jit_logsoftmax_f32_lane1_3k_it3"
+    assert Prog(1 << 20, 5, BF16).row("softmax").name() == "rows_jit_softmax_bf16_lane1_1k_it1"
+    assert Prog(1 << 20, 197, BF16).row("layernorm", 2).name() == "rows_jit_layernorm_wb_bf16_lane4_7k_it7"
+    assert Prog(1 << 20, 250, BF16).row("softmax").name() == "rows_jit_softmax_bf16_lane4_8k_it8"
+    assert Prog(1 << 20, 513, BF16).row("softmax").name() == "rows_jit_softmax_bf16_lane8_9k_it9"
+    assert Prog(1 << 20, 1001, BF16).row("softmax").name() == "rows_static_softmax_bf16_g64_it2_ragged"  # 128 values per lane: a wavefront per row
+    assert Prog(1 << 20, 77, BF16, out_dt=F32).op("mul", "full").row("rmsnorm", 1).name() == "rows_jit_mulf_rmsnorm_w_bf16_to_f32_lane2_10k_it10"
+    assert Prog(1 << 20, 77, BF16, misalign=2).row("softmax").name().endswith("_g16_it1_grid")  # the arrays must start on a 16-byte boundary
+    assert Prog((1 << 15) - 1, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g16_it1_grid"
 
 
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
@@ -186,8 +202,10 @@ def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     lambda: Prog(64, 128256, F16).op("mul", imm=0.5).row("logsoftmax"),
     lambda: Prog(64, 128256, F32).op("mul", "rowvec").op("add", "full").row("logsoftmax").op("exp").reduce("sum"),
     lambda: Prog(1 << 16, 96, BF16).op("mul", "colvec").op("add", "rowvec").row("layernorm", 2).op("silu"),
+    lambda: Prog(1 << 16, 197, F16, out_dt=F32).op("mul", "colvec").op("add", "rowvec").op("sub", "full").row("layernorm", 2).op("silu"),
+    lambda: Prog(1 << 16, 45, F32).op("abs").reduce("mean"),
 ], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10", "raw_resident_it16",
-        "looped_row", "short_rows_16_lanes"])
+        "looped_row", "short_rows_16_lanes", "lds_rows_three_spans", "lds_rows_reduction"])
 def test_generated_kernels_compile(build):
     prog = build()
     assert prog.name().startswith("rows_jit_"), prog.name()

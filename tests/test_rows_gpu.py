@@ -204,6 +204,87 @@ def test_short_rows_of_odd_length_share_a_wavefront_on_the_16_byte_grid(dt):
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_many_short_rows_of_odd_length_are_staged_in_lds_a_row_per_lane(dt):
+    """From 32768 rows on, rows whose length no vector divides go through LDS: a wavefront copies the contiguous span of
+    its 64 / L rows with whole 16-byte accesses, L = 1, 2, 4 or 8 lanes walk each row there, and the results leave the
+    same way (the last bytes of the array, where they do not fill a vector, element by element).  Lengths from one
+    element to more than 64 chunks, row counts that leave the last wavefront partial and the array's end inside a
+    vector, guard words on both sides of the output; softmax and log-softmax against float64, a norm with weight, bias
+    and per-row operand, a norm behind a two-operand pre chain with a post chain, a row reduction."""
+    g = axo.PCG64(4300 + dt)
+    e, es = (4, 4) if dt == F32 else (8, 2)
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
+    step = 1e-5 if dt == F32 else (2.0 ** -8 if dt == BF16 else 2.0 ** -10)
+    sentinel = np.float32(-77.0) if dt == F32 else np.uint16(0x7FC1)
+    pad = 64
+    for cols, rows in ((1, 32768 + 37), (3, 33023), (e + 1, 32768), (10, 32805), (77, 32768 + 37), (101, 33023), (197 if dt != F32 else 125, 32805),
+                       (513 if dt != F32 else 259, 32768 + 5)):
+        x = store(g.normal((rows, cols)) * 2)
+        xf = wide(x)
+        dst = gh.to_dev(np.full(pad + rows * cols + pad, sentinel, x.dtype))
+        p = gh.Rows(x, dt).row_op("softmax")
+        p.keep += [dst]
+        p.p.output, p.p.output_dtype = dst.data_ptr() + pad * es, dt
+        assert "_lane" in p.kernel_name(), (cols, p.kernel_name())
+        gh.sync()
+        gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
+        gh.sync()
+        out = gh.to_host(dst, x.dtype)
+        assert np.all(out[:pad] == sentinel) and np.all(out[pad + rows * cols:] == sentinel), (rows, cols)
+        got = wide(out[pad:pad + rows * cols].reshape(rows, cols))
+        ex = np.exp(xf - xf.max(-1, keepdims=True))
+        want = ex / ex.sum(-1, keepdims=True)
+        assert np.all(np.abs(got - want) <= step * want + (2.0 ** -24 if dt == F16 else 1e-9)), (rows, cols)
+        got = wide(gh.Rows(x, dt).row_op("logsoftmax").run())
+        want = (xf - xf.max(-1, keepdims=True)) - np.log(ex.sum(-1, keepdims=True))
+        assert np.all(np.abs(got - want) <= step * np.abs(want) + 1e-4), (rows, cols)
+        if cols < 2:
+            continue
+        w, b, cv = store(g.uniform((cols,), 0.5, 1.5)), store(g.uniform((cols,), -0.5, 0.5)), store(g.uniform((rows,), 0.5, 1.5))
+        p = gh.Rows(x, dt).binary("mul", cv, "colvec").row_op("layernorm", 1e-5, w=w, b=b)
+        got = wide(p.run())
+        assert "_lane" in p.kernel_name(), p.kernel_name()
+        t = xf * wide(cv)[:, None]
+        n = (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * wide(w) + wide(b)
+        assert np.max(np.abs(got - n)) < (2e-4 if dt == F32 else 4e-2), (rows, cols, np.max(np.abs(got - n)))
+        y = store(g.normal((rows, cols)))
+        p = gh.Rows(x, dt).binary("add", y).binary("mul", w, "rowvec").row_op("rmsnorm", 1e-5, w=b).post().unary("relu")
+        got = wide(p.run())
+        assert "_lane" in p.kernel_name(), p.kernel_name()
+        t = (xf + wide(y)) * wide(w)
+        n = np.maximum(t / np.sqrt((t * t).mean(-1, keepdims=True) + 1e-5) * wide(b), 0)
+        assert np.max(np.abs(got - n)) < (2e-4 if dt == F32 else 4e-2), (rows, cols, np.max(np.abs(got - n)))
+        p = gh.Rows(x, dt, F32).unary("abs")
+        got = p.run(reduce="max").astype(np.float64).reshape(-1)
+        assert "_lane" in p.kernel_name(), p.kernel_name()
+        assert np.array_equal(got, np.abs(xf).max(-1)), (rows, cols)
+
+
+def test_short_odd_rows_in_lds_take_streams_of_different_element_sizes():
+    """The row-per-lane plan gives every stream its own geometry in LDS: a 16-bit input with an fp32 full-size operand
+    and an fp32 result (three spans of two sizes), and an fp32 input with a 16-bit result."""
+    g = axo.PCG64(4400)
+    rows, cols = 32768 + 21, 45
+    x = axo.to_bits(g.normal((rows, cols)), BF16)
+    y = g.normal((rows, cols)).astype(np.float32)
+    w = g.uniform((cols,), 0.5, 1.5).astype(np.float32)
+    p = gh.Rows(x, BF16, F32).binary("add", y, dt=F32).row_op("rmsnorm", 1e-5, w=w, wdt=F32)
+    got = p.run().astype(np.float64)
+    assert "_to_f32_lane" in p.kernel_name(), p.kernel_name()
+    t = axo.to_f32(x, BF16).astype(np.float64) + y
+    want = t / np.sqrt((t * t).mean(-1, keepdims=True) + 1e-5) * w
+    assert np.max(np.abs(got - want)) < 2e-4, np.max(np.abs(got - want))
+    xf = g.normal((rows, cols)).astype(np.float32) * 2
+    p = gh.Rows(xf, F32, F16).row_op("softmax")
+    got = axo.to_f32(p.run(), F16).astype(np.float64)
+    assert "_to_f16_lane" in p.kernel_name(), p.kernel_name()
+    ex = np.exp(xf.astype(np.float64) - xf.max(-1, keepdims=True))
+    want = ex / ex.sum(-1, keepdims=True)
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * want + 2.0 ** -24)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_elementwise_chains_over_rows_no_vector_divides(dt):
     """Flat chains (no row operation, no reduction) over row lengths that no 16-byte vector divides walk the arrays as
     one run of chunks: a chunk may straddle two rows, so per-column and per-row operands are picked by position.
