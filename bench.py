@@ -543,9 +543,15 @@ def bench_survey(torch, capi, stream, steps, warmup):
         run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
         run(f"rmsnorm_{name}_{rows}x{cols}", P(t).row("rmsnorm", wr).finish(torch))
         del t
-    for rows, cols, dt, name in ((3000000, 10, f32, "f32"), (400000, 77, bf, "bf16"), (170000, 197, bf, "bf16")):
+    # (from 32768 rows on: 64 / L consecutive rows per wavefront staged in LDS, L lanes per row)
+    for rows, cols, dt, name in ((3000000, 10, f32, "f32"), (400000, 77, bf, "bf16"), (170000, 197, bf, "bf16"), (200000, 250, bf, "bf16"),
+                                 (100000, 513, bf, "bf16")):
         t = rnd((rows, cols), dt, 2.0)
         run(f"softmax_{name}_{rows}x{cols}", P(t).row("softmax").finish(torch))
+        if cols in (77, 197):
+            wr, br = rnd((cols,), dt, 0.3, 1.0), rnd((cols,), dt, 0.1)
+            run(f"rmsnorm_{name}_{rows}x{cols}", P(t).row("rmsnorm", wr).finish(torch))
+            run(f"layernorm_{name}_{rows}x{cols}", P(t).row("layernorm", wr, br).finish(torch))
         del t
     # vocabulary-sized rows (language-model logits): 1024-thread blocks; beyond 8 chunks per thread the row stays in
     # registers as raw words, beyond 16 (fp32 logits over 128 256 entries) the block walks the row once per pass
