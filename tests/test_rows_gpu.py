@@ -1000,12 +1000,16 @@ def test_layer_norm_of_16_bit_rows_far_from_zero(dt, offset, spread, cols):
     assert np.all(np.abs(got - want) <= tol(want)), float(np.max(np.abs(got - want)))
 
 
-def _random_row_program(r, g, dt):
+def _random_row_program(r, g, dt, many_short_rows=False):
     """A seeded random program and its float64 evaluation on the values the device reads (16-bit inputs widened)."""
     store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
     wide = (lambda t: t.astype(np.float64)) if dt == F32 else (lambda t: axo.to_f32(t, dt).astype(np.float64))
-    rows = int(r.integers(1, 24))
-    cols = int(r.choice([5, 64, 100, 777, 1001, 1024, 1500, 2048, 3000, 4097, 5000, 9000, 12288, 20000, 40001, 140000]))
+    if many_short_rows:
+        rows = int(r.integers(32768, 33100))
+        cols = int(r.choice([3, 10, 45, 77, 101, 197, 250, 333]))
+    else:
+        rows = int(r.integers(1, 24))
+        cols = int(r.choice([5, 64, 100, 777, 1001, 1024, 1500, 2048, 3000, 4097, 5000, 9000, 12288, 20000, 40001, 140000]))
     x = store(g.normal((rows, cols)) * 1.5)
     row_op = str(r.choice(["none", "softmax", "logsoftmax", "layernorm", "rmsnorm", "softmax", "layernorm"]))
     reduce = str(r.choice(["sum", "max", "mean"])) if row_op == "none" else str(r.choice(["none", "none", "none", "sum", "max"]))
@@ -1029,7 +1033,7 @@ def _random_row_program(r, g, dt):
                 p.unary(op)
                 ref = {"relu": lambda t: np.maximum(t, 0), "abs": np.abs, "neg": lambda t: -t, "tanh": np.tanh,
                        "sigmoid": lambda t: 1 / (1 + np.exp(-t)), "silu": lambda t: t / (1 + np.exp(-t)),
-                       "gelu": lambda t: 0.5 * t * (1 + np.vectorize(__import__("math").erf)(t / np.sqrt(2.0))), "square": lambda t: t * t}[op](ref)
+                       "gelu": lambda t: 0.5 * t * (1 + __import__("scipy.special").special.erf(t / np.sqrt(2.0))), "square": lambda t: t * t}[op](ref)
             elif op in ("mul_imm", "add_imm"):
                 c = float(np.float32(r.uniform(0.25, 2.0)))
                 p.imm(op[:3], c)
@@ -1094,6 +1098,29 @@ def test_seeded_random_row_programs_match_fp64(dt):
         err = np.abs(got.reshape(ref.shape) - ref)
         assert np.all(err <= tol), (case, desc, name, float(np.max(err / tol)))
     assert ({"jit"} if dt == F16 else {"static", "jit"}) <= kinds, kinds  # (no f16 shape is built in)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_seeded_random_row_programs_over_many_short_odd_rows_match_fp64(dt):
+    """Twelve of the same random programs per element type over 32768 to 33100 rows of 3 to 333 columns: the rows of
+    a wavefront staged in LDS, one to eight lanes per row, full-size operands as further spans, per-column operands as
+    tables, results of the input's type or fp32, row reductions -- against float64."""
+    r = np.random.default_rng(777 + dt)
+    g = axo.PCG64(55 + dt)
+    staged = 0
+    for case in range(12):
+        p, reduce, ref, mag, out_dt, desc = _random_row_program(r, g, dt, many_short_rows=True)
+        got = p.run(reduce=reduce)
+        name = p.kernel_name()
+        staged += "_lane" in name
+        got = got.astype(np.float64) if out_dt == F32 else axo.to_f32(got, out_dt).astype(np.float64)
+        ulp = {F32: 0.0, BF16: 2.0 ** -8, F16: 2.0 ** -11}[out_dt]
+        tol = 4e-5 * np.maximum(1.0, mag) + ulp * np.abs(ref) + (0.0 if out_dt == F32 else 1e-7)
+        if dt != F32 and out_dt != F32:
+            tol = tol + 2e-4
+        err = np.abs(got.reshape(ref.shape) - ref)
+        assert np.all(err <= tol), (case, desc, name, float(np.max(err / tol)))
+    assert staged >= 8, staged
 
 
 def test_run_time_compiled_kernels_come_back_from_the_on_disk_cache(tmp_path):
