@@ -371,6 +371,9 @@ void rows_prog_plan_for(const AxhipRowsProgram &P, int group, int it, bool ragge
     // and bias over 170000 rows of 197 16-bit columns 63 against 79 us, softmax the same either way)
     static const bool pipe_short_grid = [] { const char *e = getenv("AXHIP_ROWS_PIPE_SHORT_GRID"); return !(e && e[0] == '0'); }();
     if (group < 64 && plan->grid && !pipe_short_grid) plan->pipe = false;
+    // (AXHIP_ROWS_PIPE=0, read once: no plan is pipelined -- for measurements)
+    static const bool pipe_off = [] { const char *v = getenv("AXHIP_ROWS_PIPE"); return v && v[0] == '0'; }();
+    if (pipe_off) plan->pipe = false;
     // a 1024-thread block has 128 registers per thread whatever is asked for: no second set of raw words beyond that
     if (group == 1024 && held + (plan->pipe ? raw * it : 0) > 115) plan->pipe = false;
 }
@@ -625,6 +628,11 @@ bool rows_prog_spec(const AxhipRowsProgram &P, const RowsProgPlan &plan, RowsPro
     char hash[24];
     snprintf(hash, sizeof(hash), "%016llx", static_cast<unsigned long long>(fnv1a(S.chains, fnv1a(S.config))));
     S.threads = plan.lane ? 64 : plan.group > 256 ? plan.group : 256;
+    // bytes a block has requested and not yet used: its threads' chunks of every full-size input, twice when pipelined
+    S.pipelined = pipe;
+    S.post_ops = P.n_post;
+    // (rows of odd length spend their time on instructions: they keep every wave slot)
+    S.inflight_bytes = plan.lane || plan.ragged ? 0 : static_cast<int64_t>(S.threads) * plan.it * 4 * raw_words_per_chunk(P) * (pipe ? 2 : 1);
     S.rows_per_block = plan.lane ? 64 / plan.lane_l : S.threads / plan.group;
     S.lane = plan.lane;
 

@@ -55,6 +55,9 @@ struct RowsProgSpec {
     int threads = 256;
     int rows_per_block = 4;
     bool lane = false;      // the row-per-lane body (its text is compiled only for these kernels)
+    int64_t inflight_bytes = 0; // bytes of input a block keeps requested at a time (0: not counted)
+    bool pipelined = false;     // the kernel requests a row while it computes the one before
+    int post_ops = 0;           // operations behind the row operation (the output pass carries them)
     int n_slots = 0;
     int slot_operand[8] = {}; // pointer slot -> index into AxhipRowsProgram::operands
     int n_imm = 0;

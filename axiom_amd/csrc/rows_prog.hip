@@ -352,6 +352,20 @@ bool rows_prog_dispatch(const AxhipRowsProgram &P, hipStream_t s, bool launch, c
                                              : hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel->function, spec.threads, 0);
             if (err != hipSuccess) (void)hipGetLastError();
             kernel->blocks_per_cu = err == hipSuccess && n > 0 ? n : 2;
+            // Fewer resident blocks than fit, where a block keeps much of its input requested at a time: with inputs
+            // that come from HBM aligned rows run faster with about 128 KiB of requests per CU (two blocks of four
+            // wavefront rows of 4096 16-bit columns, pipelined) than with every wave slot filled -- softmax bf16
+            // [16384,4096] 67.9 -> 69.7 % of the HBM peak, fp32 [8192,8192] 65.9 -> 69.1 %, RMS norm [32768,2048]
+            // 67.7 -> 72.2 %, row sums 68.2 -> 71.4 %; unchanged back to back on one buffer pair.  Never fewer than two
+            // blocks (with one, 64 KiB, chains that are heavy on arithmetic lose: softmax(exp(x)) 70 -> 64 %), four
+            // where the output pass carries a chain of its own (gelu(layer norm) back to back: 77.8 % with four or
+            // more, 75.9 % with two).
+            // AXHIP_ROWS_INFLIGHT_KB=<n> (read once) sets the figure, 0 fills the CU.
+            static const int inflight_kb = [] { const char *v = getenv("AXHIP_ROWS_INFLIGHT_KB"); return v ? atoi(v) : 128; }();
+            if (inflight_kb > 0 && spec.inflight_bytes > 0) {
+                const int64_t want = std::max<int64_t>(spec.post_ops > 0 ? 4 : 2, (static_cast<int64_t>(inflight_kb) * 1024 + spec.inflight_bytes / 2) / spec.inflight_bytes);
+                if (kernel->blocks_per_cu > want) kernel->blocks_per_cu = static_cast<int>(want);
+            }
         }
         if (g_num_cus == 0) {
             int dev = 0, n = 0;
