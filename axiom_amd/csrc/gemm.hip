@@ -972,7 +972,14 @@ int gemm_impl(const void *a, const void *b, void *c, const AxhipGemmParams *para
         k.dtype = p.dtype; k.epilogue = p.epilogue_op;
         k.N = static_cast<int>(p.n); k.K = static_cast<int>(p.k);
         k.ldx = static_cast<int>(p.lda); k.ldw = static_cast<int>(p.ldb); k.ldc = static_cast<int>(p.ldc);
-        const int rows_per_wave = p.n >= 16384 ? 4 : p.n >= 4096 ? 2 : 1; // at least two wavefronts per SIMD where N allows
+        // A wavefront per row of W, each lane with four 16-byte pieces of it requested at a time: the fewest rows are
+        // streamed at once, each in the longest runs (1 x 16384 x 16384: 88.8 us = 76 % of the HBM peak against
+        // 95.2 / 101.2 us with two / four rows per wavefront; 1 x 50304 x 4096: 64.2 against 68.4 / 71.8 us; 1 x 4096 x
+        // 4096 from the caches: 4.3 against 6.6 / 7.1 us).  Two rows per wavefront share the reads of x where two or
+        // more rows of x meet a large W (2 x 16384 x 16384: 97.4 against 102.7 us).
+        // AXHIP_GEMM_SKINNY_ROWS=1|2|4 (read once) forces the count.
+        static const int forced_rows = [] { const char *e = std::getenv("AXHIP_GEMM_SKINNY_ROWS"); return e ? std::atoi(e) : 0; }();
+        const int rows_per_wave = forced_rows == 1 || forced_rows == 2 || forced_rows == 4 ? forced_rows : (p.m >= 2 && w_elems >= (int64_t(64) << 20)) ? 2 : 1;
         const unsigned blocks = static_cast<unsigned>((p.n + 4 * rows_per_wave - 1) / (4 * rows_per_wave));
         launch_skinny(k, static_cast<int>(p.m), rows_per_wave, blocks, s);
     } else if (half && nt && p.k > 0 && p.k % TK == 0 && p.m >= BIG && p.n >= BIG && p.lda < (1 << 21) && p.ldb < (1 << 21) && p.batch < 65536 &&
