@@ -325,6 +325,34 @@ int rows_setup_device() {
     return scratch_of_current_device(&unused);
 }
 
+// A large elementwise chain (no row operation, no reduction) whose operands are full-size arrays, one-element arrays
+// or immediates does not care where its rows end: seen as rows of 512 chunks (a wavefront per row, eight chunks per
+// lane) any such array takes the same compiled kernel, whatever its own shape -- a vector of 2^26 elements included.
+// False when the chain reads an operand by column or by row, when the size is no multiple of such a row, or when an
+// array does not start on a 16-byte boundary: the program then runs with the shape it came with.
+bool flat_chain_as_rows(const AxhipRowsProgram &P, AxhipRowsProgram *out) {
+    if (P.row_op != AXHIP_ROWOP_NONE || P.reduce != AXHIP_RED_NONE) return false;
+    auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (!al16(P.input) || !al16(P.output)) return false;
+    for (int stage = 0; stage < 2; ++stage) {
+        const AxhipChainOp *ops = stage ? P.post : P.pre;
+        const int n = stage ? P.n_post : P.n_pre;
+        for (int i = 0; i < n; ++i) {
+            if (!is_binary_op(ops[i].op) || ops[i].imm_kind == AXHIP_BK_IMM) continue;
+            if (ops[i].operand < 0 || ops[i].operand >= P.n_operands) return false;
+            const AxhipOperand &o = P.operands[ops[i].operand];
+            if (o.kind == AXHIP_BK_ROWVEC || o.kind == AXHIP_BK_COLVEC) return false;
+            if (o.kind == AXHIP_BK_FULL && !al16(o.ptr)) return false;
+        }
+    }
+    const int64_t row = 512 * rows_prog_chunk_elems(P), total = P.rows * P.cols;
+    if (total % row != 0 || P.cols == row) return false;
+    *out = P;
+    out->rows = total / row;
+    out->cols = row;
+    return true;
+}
+
 } // namespace axhip
 
 using namespace axhip;
@@ -334,7 +362,9 @@ extern "C" {
 const char *axhip_fused_rows_kernel_name(const AxhipRowsProgram *P) {
     static thread_local char name[192];
     if (!P) return "invalid";
-    if (validate_program(*P, "axhip_fused_rows_kernel_name") == AXHIP_OK && rows_prog_dispatch(*P, nullptr, false, name, sizeof(name), nullptr))
+    AxhipRowsProgram flat;
+    if (validate_program(*P, "axhip_fused_rows_kernel_name") == AXHIP_OK &&
+        rows_prog_dispatch(flat_chain_as_rows(*P, &flat) ? flat : *P, nullptr, false, name, sizeof(name), nullptr))
         return name;
     RowsPlan pl = plan_rows(*P);
     snprintf(name, sizeof(name), "%s", pl.name);
@@ -354,7 +384,8 @@ int axhip_fused_rows(const AxhipRowsProgram *program, void *stream) {
     hipStream_t s = resolve_stream(stream);
     // a kernel compiled for this program's shape (built in, or compiled now if this is its first launch) ...
     int launch_rc = AXHIP_OK;
-    if (rows_prog_dispatch(P, s, true, nullptr, 0, &launch_rc)) {
+    AxhipRowsProgram flat;
+    if (rows_prog_dispatch(flat_chain_as_rows(P, &flat) ? flat : P, s, true, nullptr, 0, &launch_rc)) {
         if (launch_rc) return launch_rc;
         AXHIP_CHECK_HIP(hipGetLastError());
         return AXHIP_OK;
@@ -371,10 +402,12 @@ int axhip_fused_rows_prepare(const AxhipRowsProgram *program) {
     int rc = validate_program(*program, "axhip_fused_rows_prepare");
     if (rc) return rc;
     char name[192];
-    if (!rows_prog_dispatch(*program, nullptr, false, name, sizeof(name), nullptr)) return AXHIP_OK; // the interpreter's: nothing to prepare
-    if (strncmp(name, "rows_static_", 12) == 0) return AXHIP_OK;                                    // built into the library
+    AxhipRowsProgram flat;
+    const AxhipRowsProgram &as_run = flat_chain_as_rows(*program, &flat) ? flat : *program;
+    if (!rows_prog_dispatch(as_run, nullptr, false, name, sizeof(name), nullptr)) return AXHIP_OK; // the interpreter's: nothing to prepare
+    if (strncmp(name, "rows_static_", 12) == 0) return AXHIP_OK;                                // built into the library
     std::string label, error;
-    if (!rows_prog_compile_only(*program, &label, &error)) {
+    if (!rows_prog_compile_only(as_run, &label, &error)) {
         set_last_error("axhip_fused_rows_prepare: %s: %.400s", label.c_str(), error.c_str());
         return AXHIP_ERR_UNSUPPORTED;
     }

@@ -70,6 +70,8 @@ struct RowsProgSpec {
 // tight = true: the plan with the fewest idle chunk slots for this row length (64, 256 or 512 threads per row, any chunk count up to 8).
 // the row-per-lane plan is for arrays of at least this many rows (fewer rows want more than a wavefront per 64 of them)
 constexpr int64_t kRowsProgLaneMinRows = 32768;
+// an elementwise chain (no row operation, no reduction) takes a compiled kernel from this size on: 1024 rows, 8 MiB of input
+bool rows_prog_flat_large(const AxhipRowsProgram &P);
 int rows_prog_chunk_elems(const AxhipRowsProgram &P); // elements per chunk: 4 when a full-size stream is fp32, else 8
 bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan);
 // The plan with its shape given (the build's generator enumerates the shapes itself).

@@ -33,7 +33,8 @@ void make_struct_key(const AxhipRowsProgram &P, StructKey *k) {
     // (the address modulo 16 decides between the aligned, the grid and the unaligned form of a kernel)
     auto align_tag = [](const void *p) { return reinterpret_cast<const void *>(static_cast<uintptr_t>(reinterpret_cast<uintptr_t>(p) & 15u) + 16u); };
     q.cols = P.cols;
-    q.rows = P.rows >= kRowsProgLaneMinRows ? 1 : 0; // (arrays of many short rows have a plan of their own)
+    // (arrays of many short rows have a plan of their own; elementwise chains are compiled from a size on)
+    q.rows = (P.rows >= kRowsProgLaneMinRows ? 1 : 0) | (P.row_op == AXHIP_ROWOP_NONE && P.reduce == AXHIP_RED_NONE && rows_prog_flat_large(P) ? 2 : 0);
     q.input = align_tag(P.input);
     q.input_dtype = P.input_dtype;
     q.n_operands = P.n_operands;

@@ -186,8 +186,23 @@ def test_many_short_rows_of_odd_length_go_through_lds():
     assert Prog((1 << 15) - 1, 77, BF16).row("softmax").name() == "rows_static_softmax_bf16_g16_it1_grid"
 
 
+def test_large_elementwise_chains_run_as_row_programs_without_a_row_operation():
+    """From 8 MiB on, a chain with no row operation and no reduction takes a compiled kernel too.  Where its operands are
+    full-size arrays, one-element arrays or immediates the array is seen as rows of 512 chunks whatever its shape; a
+    per-column or per-row operand keeps the shape (aligned rows of up to 2048 chunks)."""
+    assert Prog(1024, 4096, F32).op("relu").op("mul", "full").name() == "rows_jit_relu_mulf_map_f32_g64_it8"
+    assert Prog(1, 1 << 26, BF16).op("gelu").name() == "rows_jit_gelu_map_bf16_g64_it8"  # a vector: 16384 rows of 4096
+    assert Prog(1 << 20, 64, BF16).op("mul", imm=0.5).op("add", "scalar").name() == "rows_jit_muls_adds_map_bf16_g64_it8"
+    assert Prog(16384, 1024, BF16).op("add", "rowvec").op("relu").name() == "rows_jit_addr_relu_map_bf16_g64_it2"  # a bias: by column
+    assert Prog(1 << 20, 64, BF16).op("mul", "colvec").name() == "rows_jit_mulc_map_bf16_g8_it1"
+    assert Prog(16384, 4100, BF16).op("add", "rowvec").name().startswith("elementwise_")  # rows that are not whole 16-byte vectors
+    assert Prog(4099, 4099, BF16).op("relu").name().startswith("elementwise_")  # no whole number of 4096-element rows
+    assert Prog(16384, 4096, BF16, misalign=2).op("relu").name().startswith("elementwise")
+    assert Prog(16384, 4096, BF16, out_dt=F32).op("relu").name() == "rows_jit_relu_map_bf16_to_f32_g64_it8"  # fp32 out: rows of 2048
+
+
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
-    assert Prog(1024, 4096, F32).op("relu").op("mul", "full").name() == "elementwise_e4"  # no row op, no reduction
+    assert Prog(256, 4096, F32).op("relu").op("mul", "full").name() == "elementwise_e4"  # no row op, no reduction, under 8 MiB
     assert Prog(4, 1000001, BF16).row("softmax").name() == "rows_streamed_e1"  # beyond 16384 chunks and not whole vectors
     # ragged rows whose streams differ in element size
     assert Prog(64, 1001, BF16, out_dt=F32).row("softmax").name().startswith("rows_resident_")
@@ -204,8 +219,9 @@ def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():
     lambda: Prog(1 << 16, 96, BF16).op("mul", "colvec").op("add", "rowvec").row("layernorm", 2).op("silu"),
     lambda: Prog(1 << 16, 197, F16, out_dt=F32).op("mul", "colvec").op("add", "rowvec").op("sub", "full").row("layernorm", 2).op("silu"),
     lambda: Prog(1 << 16, 45, F32).op("abs").reduce("mean"),
+    lambda: Prog(16384, 4096, BF16).op("mul", "full").op("add", "rowvec").op("silu"),
 ], ids=["post_activation", "gated_norm_fp32_out", "ragged_two_streams", "block_512_with_row_and_scalar_operands", "reduction_it10", "raw_resident_it16",
-        "looped_row", "short_rows_16_lanes", "lds_rows_three_spans", "lds_rows_reduction"])
+        "looped_row", "short_rows_16_lanes", "lds_rows_three_spans", "lds_rows_reduction", "elementwise_chain"])
 def test_generated_kernels_compile(build):
     prog = build()
     assert prog.name().startswith("rows_jit_"), prog.name()

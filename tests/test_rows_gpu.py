@@ -285,6 +285,61 @@ def test_short_odd_rows_in_lds_take_streams_of_different_element_sizes():
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+def test_large_elementwise_chains_take_compiled_row_kernels(dt):
+    """From 8 MiB on an elementwise chain runs as a compiled row program without a row operation: an array whose
+    operands are full-size, one-element or immediate is seen as rows of 512 chunks whatever its shape (a vector, short
+    rows, a shape that is no multiple of 4096 columns), one with a per-column or per-row operand keeps its rows.
+    relu / add / mul chains are exact against the oracle's fp32 evaluation of the same inputs; activations to a
+    16-bit step; an fp32 result from 16-bit inputs; guard words around the output."""
+    g = axo.PCG64(5100 + dt)
+    store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
+    wide = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_f32(t, dt))
+    es = 4 if dt == F32 else 2
+    sentinel = np.float32(-77.0) if dt == F32 else np.uint16(0x7FC1)
+    for shape in ((1, 1 << 22), (3 << 16, 24), (2048, 2304)):
+        rows, cols = shape
+        a, b = store(g.normal(shape)), store(g.normal(shape))
+        one = store(np.array([1.25]))
+        pad = 64
+        dst = gh.to_dev(np.full(pad + rows * cols + pad, sentinel, a.dtype))
+        p = gh.Rows(a, dt).unary("relu").binary("add", one, "scalar").binary("mul", b).imm("mul", 0.5)
+        p.keep.append(dst)
+        p.p.output, p.p.output_dtype = dst.data_ptr() + pad * es, dt
+        assert "_map_" in p.kernel_name() and "_g64_it8" in p.kernel_name(), p.kernel_name()
+        gh.sync()
+        gh.capi.check(gh.capi.lib().axhip_fused_rows(gh.C.byref(p.p), None))
+        gh.sync()
+        out = gh.to_host(dst, a.dtype)
+        assert np.all(out[:pad] == sentinel) and np.all(out[pad + rows * cols:] == sentinel), shape
+        want = store((np.maximum(wide(a), 0) + wide(one)) * wide(b) * np.float32(0.5))
+        assert np.array_equal(out[pad:pad + rows * cols].reshape(shape), want), shape
+    # per-column and per-row operands: the array keeps its rows
+    rows, cols = 8192, 1024
+    a = store(g.normal((rows, cols)))
+    bias, gate = store(g.normal((cols,))), store(g.uniform((rows,), 0.5, 1.5))
+    p = gh.Rows(a, dt).binary("add", bias, "rowvec").binary("mul", gate, "colvec").unary("relu")
+    got = p.run()
+    assert "_map_" in p.kernel_name(), p.kernel_name()
+    assert np.array_equal(got, store(np.maximum((wide(a) + wide(bias)) * wide(gate)[:, None], 0)))
+    # activations, and an fp32 result
+    x = store(g.normal((4096, 4096)) * 2)
+    xf = wide(x).astype(np.float64)
+    tol = 2e-6 if dt == F32 else (2.0 ** -8 if dt == BF16 else 2.0 ** -10)
+    for op, ref in (("gelu", lambda t: 0.5 * t * (1 + __import__("scipy.special").special.erf(t / np.sqrt(2.0)))), ("silu", lambda t: t / (1 + np.exp(-t))),
+                    ("tanh", np.tanh)):
+        p = gh.Rows(x, dt).unary(op)
+        got = wide(p.run()).astype(np.float64)
+        assert "_map_" in p.kernel_name(), p.kernel_name()
+        want = ref(xf)
+        assert np.all(np.abs(got - want) <= tol * np.abs(want) + (1e-6 if dt == F32 else 3e-4)), (op, float(np.max(np.abs(got - want))))
+    if dt != F32:
+        p = gh.Rows(x, dt, F32).unary("square").imm("add", 1.0)
+        got = p.run()
+        assert "_to_f32_" in p.kernel_name() and "_map_" in p.kernel_name(), p.kernel_name()
+        assert np.array_equal(got, wide(x) * wide(x) + np.float32(1.0))
+
+
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 def test_elementwise_chains_over_rows_no_vector_divides(dt):
     """Flat chains (no row operation, no reduction) over row lengths that no 16-byte vector divides walk the arrays as
     one run of chunks: a chunk may straddle two rows, so per-column and per-row operands are picked by position.
