@@ -12,9 +12,9 @@ namespace axhip {
 
 namespace {
 
-int elem_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : 2; }
+int elem_size(int dt) { return dt == AXHIP_DTYPE_F32 ? 4 : dt == AXHIP_DTYPE_U8 ? 1 : 2; }
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-const char *dt_name(int dt) { return dt == AXHIP_DTYPE_F32 ? "f32" : dt == AXHIP_DTYPE_F16 ? "f16" : "bf16"; }
+const char *dt_name(int dt) { return dt == AXHIP_DTYPE_F32 ? "f32" : dt == AXHIP_DTYPE_F16 ? "f16" : dt == AXHIP_DTYPE_U8 ? "u8" : "bf16"; }
 bool is_unary(int op) { return (op >= AXHIP_OP_RELU && op <= AXHIP_OP_RECIP) || (op >= AXHIP_OP_ERF && op <= AXHIP_OP_NOT); }
 bool is_binary(int op) { return (op >= AXHIP_OP_ADD && op <= AXHIP_OP_RDIV) || (op >= AXHIP_OP_POW && op <= AXHIP_OP_LEAKY_RELU); }
 
@@ -401,7 +401,8 @@ bool rows_prog_plan(const AxhipRowsProgram &P, bool tight, RowsProgPlan *plan) {
     }
     // products and one-byte streams (a Bool input, operand or full-size result) stay with the interpreter; a reduced
     // [rows] result may be a byte (any / all)
-    if (P.reduce > AXHIP_RED_MIN || P.input_dtype == AXHIP_DTYPE_U8 || (P.reduce == AXHIP_RED_NONE && P.output_dtype == AXHIP_DTYPE_U8)) return false;
+    // (an elementwise chain may leave truth values: a comparison's result, one byte per element)
+    if (P.reduce > AXHIP_RED_MIN || P.input_dtype == AXHIP_DTYPE_U8 || (P.reduce == AXHIP_RED_NONE && P.output_dtype == AXHIP_DTYPE_U8 && P.row_op != AXHIP_ROWOP_NONE)) return false;
     for (int i = 0; i < P.n_operands; ++i)
         if (P.operands[i].dtype == AXHIP_DTYPE_U8) return false;
     const int dt = P.input_dtype;

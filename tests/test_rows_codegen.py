@@ -199,6 +199,7 @@ def test_large_elementwise_chains_run_as_row_programs_without_a_row_operation():
     assert Prog(4099, 4099, BF16).op("relu").name().startswith("elementwise_")  # no whole number of 4096-element rows
     assert Prog(16384, 4096, BF16, misalign=2).op("relu").name().startswith("elementwise")
     assert Prog(16384, 4096, BF16, out_dt=F32).op("relu").name() == "rows_jit_relu_map_bf16_to_f32_g64_it8"  # fp32 out: rows of 2048
+    assert Prog(16384, 4096, BF16, out_dt=capi.DTYPE_U8).op("gt", "full").name() == "rows_jit_gtf_map_bf16_to_u8_g64_it8"  # a comparison's truth values
 
 
 def test_what_the_compiled_form_does_not_take_goes_to_the_interpreter():

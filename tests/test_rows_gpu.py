@@ -290,7 +290,8 @@ def test_large_elementwise_chains_take_compiled_row_kernels(dt):
     operands are full-size, one-element or immediate is seen as rows of 512 chunks whatever its shape (a vector, short
     rows, a shape that is no multiple of 4096 columns), one with a per-column or per-row operand keeps its rows.
     relu / add / mul chains are exact against the oracle's fp32 evaluation of the same inputs; activations to a
-    16-bit step; an fp32 result from 16-bit inputs; guard words around the output."""
+    16-bit step; an fp32 result from 16-bit inputs; comparisons that leave one-byte truth values; guard words around
+    the output."""
     g = axo.PCG64(5100 + dt)
     store = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_bits(t, dt))
     wide = (lambda t: t.astype(np.float32)) if dt == F32 else (lambda t: axo.to_f32(t, dt))
@@ -337,6 +338,16 @@ def test_large_elementwise_chains_take_compiled_row_kernels(dt):
         got = p.run()
         assert "_to_f32_" in p.kernel_name() and "_map_" in p.kernel_name(), p.kernel_name()
         assert np.array_equal(got, wide(x) * wide(x) + np.float32(1.0))
+    # truth values: one byte per element, four or eight of them per store
+    y = store(g.normal((4096, 4096)) * 2)
+    p = gh.Rows(x, dt, gh.U8).binary("gt", y)
+    got = p.run()
+    assert "_to_u8_" in p.kernel_name() and "_map_" in p.kernel_name(), p.kernel_name()
+    assert np.array_equal(got, (wide(x) > wide(y)).astype(np.uint8))
+    p = gh.Rows(x, dt, gh.U8).unary("abs").imm("lt", 0.5)
+    got = p.run()
+    assert "_to_u8_" in p.kernel_name(), p.kernel_name()
+    assert np.array_equal(got, (np.abs(wide(x)) < np.float32(0.5)).astype(np.uint8))
 
 
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
