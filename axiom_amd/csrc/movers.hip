@@ -822,7 +822,10 @@ int launch_reduce_axis(const void *src, int dtype, int64_t outer, int64_t axis, 
         const int64_t ivecs = inner / (16 / es);
         // a short axis with plenty of results: a thread per vector walks it alone (no merge through LDS)
         const bool flat = axis <= 32 && outer * ((ivecs + 255) / 256) >= 1024 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0;
-        const bool wide = outer * ((ivecs + 31) / 32) >= 1024;
+        // (32-vector column groups from 512 of them on: sum over axis 1 of bf16 [256, 1024, 512] 44.5 -> 38.2 us, 75 -> 88 %
+        // of the HBM peak; AXHIP_REDUCE_AXIS_WIDE_FROM=<n>, read once, moves the threshold)
+        static const int wide_from = [] { const char *e = getenv("AXHIP_REDUCE_AXIS_WIDE_FROM"); return e ? atoi(e) : 512; }();
+        const bool wide = outer * ((ivecs + 31) / 32) >= wide_from;
         const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(outer * (flat ? (ivecs + 255) / 256 : wide ? (ivecs + 31) / 32 : (ivecs + 7) / 8), 256 * 64));
 #define AXHIP_RED_VEC_TX(RED, DT, TX) hipLaunchKernelGGL((reduce_strided_vec_kernel<RED, DT, TX>), dim3(blocks), dim3(256), 0, s, src, outer, axis, inner, scale, dst, dst_dtype)
 #define AXHIP_RED_VEC_DT(RED, DT)                                                                                                          \
@@ -1265,8 +1268,20 @@ int axhip_argreduce_ws(const void *src, int32_t dtype, int64_t outer, int64_t ax
 static int64_t reduce_axis_parts(const void *src, int32_t dtype, int64_t outer, int64_t axis, int64_t inner) {
     const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2;
     if (inner <= 1 || inner % (16 / es) != 0 || (reinterpret_cast<uintptr_t>(src) & 15u) != 0) return 1;
-    const int64_t groups8 = outer * ((inner / (16 / es) + 7) / 8);
+    // Large arrays of short inner rows (up to 8 KiB) do better in 32-vector column groups -- 512-byte runs per row
+    // instead of 128 -- once the axis is cut so that there are about 1024 of them: sum over axis 1 of bf16
+    // [64, 4096, 1024] 99.5 -> 91.8 us (67 -> 73 % of the HBM peak), [8, 8192, 4096] 97.2 -> 92.8 us.  Smaller arrays lose
+    // to the second launch ([16, 2048, 2048]: 22.5 -> 25.9 us), long inner rows to the split itself (fp32
+    // [1, 4096, 16384]: 40.0 -> 43.3 us): they keep the rule below.  AXHIP_REDUCE_AXIS_SPLIT32=0 (read once): never.
+    static const bool split32 = [] { const char *e = getenv("AXHIP_REDUCE_AXIS_SPLIT32"); return !(e && e[0] == '0'); }();
+    const int64_t groups8 = outer * ((inner / (16 / es) + 7) / 8), groups32 = outer * ((inner / (16 / es) + 31) / 32);
     int64_t parts = 1;
+    if (split32 && outer * axis * inner * es >= (int64_t(256) << 20) && inner * es <= 8192) {
+        if (groups32 < 512 && axis >= 1024)
+            for (int64_t p = 2; p <= 64 && groups32 * parts < 1024; ++p)
+                if (axis % p == 0 && axis / p >= 256) parts = p;
+        return parts;
+    }
     if (groups8 < 512 && axis >= 2048)
         for (int64_t p = 2; p <= 64 && groups8 * parts < 1024; ++p)
             if (axis % p == 0 && axis / p >= 256) parts = p;
