@@ -492,6 +492,9 @@ def bench_survey(torch, capi, stream, steps, warmup):
     pg.out, pg.bytes = mask, 2 * xb.numel() * 2 + mask.numel()
     run("x>y_to_bool_bf16_16384x4096", pg)
     run("leaky_relu(x)*y_bf16_16384x4096", _Prog(capi, xb).op("leaky_relu", imm=0.01).op("mul", yb).finish(torch))
+    # (elementwise chains of 8 MiB or more: compiled, the array seen as rows of 512 chunks)
+    run("gelu(x)_bf16_16384x4096", _Prog(capi, xb).op("gelu").finish(torch))
+    run("relu(x)_as_vector_bf16_1x67108864", _Prog(capi, xb.view(1, -1)).op("relu").finish(torch))
     anyout = torch.empty((16384,), device="cuda", dtype=torch.uint8)
     pa = _Prog(capi, xb)
     pa.op("gt", imm=3.5)
