@@ -72,6 +72,99 @@ struct TransposeArgs {
     int64_t oshape[AXHIP_MAX_DIMS], osrc[AXHIP_MAX_DIMS], odst[AXHIP_MAX_DIMS];
 };
 
+// The same for views that move whole 16-byte vectors on both sides (equal 2- or 4-byte element types; extents, strides
+// and bases multiples of a vector -- or of half a vector on a side, LG / SG = 8: that side moves 8-byte pieces, e.g. the
+// 3000-byte rows of a [.., 1500] 16-bit array): tiles of 16 x 16 vectors -- 128 x 128 16-bit or 64 x 64 32-bit
+// elements, 256-byte runs on the read and on the write side.  A thread reads vectors along J, scatters their elements as 32-bit words into
+// a tile that is stored transposed (16-bit: two neighbouring rows of L packed into one word first), and the tile
+// leaves as 16-byte LDS reads along L.  Tile rows are 256 bytes = 16 chunks; chunk c of row j sits at c ^ (j / V mod 16),
+// which spreads the words of one scatter over all 64 banks and keeps the 16 reads of a row apart.
+template <int ES, int LG, int SG>
+__global__ __launch_bounds__(256) void transpose_vec_kernel(const TransposeArgs a) {
+    constexpr int V = 16 / ES, T = 16 * V; // elements per vector, tile edge
+    // 16 bytes at `at`, of which the elements below `n` exist (whole pieces of LG bytes)
+    auto load16 = [](const char *at, int64_t n) {
+        if constexpr (LG == 16) {
+            return n > 0 ? *reinterpret_cast<const uint4_t *>(at) : uint4_t{0, 0, 0, 0};
+        } else {
+            const uint2_t lo = n > 0 ? *reinterpret_cast<const uint2_t *>(at) : uint2_t{0, 0};
+            const uint2_t hi = n > V / 2 ? *reinterpret_cast<const uint2_t *>(at + 8) : uint2_t{0, 0};
+            return uint4_t{lo.x, lo.y, hi.x, hi.y};
+        }
+    };
+    __shared__ __attribute__((aligned(16))) uint32_t tile[T * 64];
+    int64_t b = blockIdx.x;
+    const int64_t tl = b % a.tiles_l;
+    b /= a.tiles_l;
+    // (work-groups that run side by side take tiles along a diagonal: with a power of two as row length, tiles of one
+    // tile row or column start a multiple of 2 MiB apart on one of the two sides and would queue on the same channels)
+    const int64_t tj = (b % a.tiles_j + tl) % a.tiles_j;
+    int64_t o = b / a.tiles_j;
+    int64_t src_base = 0, dst_base = 0;
+    for (int d = a.n_other - 1; d >= 0; --d) {
+        const int64_t c = o % a.oshape[d];
+        o /= a.oshape[d];
+        src_base += c * a.osrc[d];
+        dst_base += c * a.odst[d];
+    }
+    const int tid = threadIdx.x, jv = tid % 16, hi = tid / 16;
+    const int64_t j0 = tj * T, l0 = tl * T;
+    const char *src = static_cast<const char *>(a.src);
+    char *dst = static_cast<char *>(a.dst);
+    const int64_t j_left = a.nJ - (j0 + jv * V); // elements of this thread's vectors that exist (whole pieces)
+    if constexpr (ES == 2) {
+        // pairs of rows: pair p = rows 2p, 2p + 1 of the tile; four per thread
+        uint4_t r0[4], r1[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int64_t l = l0 + 2 * (hi + 16 * it);
+            const int64_t at = (src_base + l * a.src_stride_l + j0 + jv * V) * ES;
+            r0[it] = load16(src + at, l < a.nL ? j_left : 0);
+            r1[it] = load16(src + at + a.src_stride_l * ES, l + 1 < a.nL ? j_left : 0);
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int p = hi + 16 * it; // the pair's word: chunk p / 4, word p % 4 of row j
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const uint32_t w0 = r0[it][e / 2], w1 = r1[it][e / 2];
+                const uint32_t word = e % 2 ? __builtin_amdgcn_perm(w1, w0, 0x07060302u) : __builtin_amdgcn_perm(w1, w0, 0x05040100u);
+                tile[(jv * V + e) * 64 + (((p / 4) ^ jv) * 4) + p % 4] = word;
+            }
+        }
+    } else {
+        uint4_t r[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int64_t l = l0 + hi + 16 * it;
+            r[it] = load16(src + (src_base + l * a.src_stride_l + j0 + jv * V) * ES, l < a.nL ? j_left : 0);
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int l = hi + 16 * it;
+#pragma unroll
+            for (int e = 0; e < V; ++e) tile[(jv * V + e) * 64 + (((l / 4) ^ jv) * 4) + l % 4] = r[it][e];
+        }
+    }
+    __syncthreads();
+    // rows j of the transposed tile, 16 vectors along L each
+    const int lv = tid % 16;
+    const int64_t l_left = a.nL - (l0 + lv * V);
+#pragma unroll
+    for (int it = 0; it < T / 16; ++it) {
+        const int j = hi + 16 * it;
+        const uint4_t t = *reinterpret_cast<const uint4_t *>(&tile[j * 64 + ((lv ^ ((j / V) & 15)) * 4)]);
+        char *to = dst + (dst_base + (j0 + j) * a.dst_stride_j + l0 + lv * V) * ES;
+        if (j0 + j >= a.nJ) continue;
+        if constexpr (SG == 16) {
+            if (l_left > 0) *reinterpret_cast<uint4_t *>(to) = t;
+        } else {
+            if (l_left > 0) *reinterpret_cast<uint2_t *>(to) = uint2_t{t.x, t.y};
+            if (l_left > V / 2) *reinterpret_cast<uint2_t *>(to + 8) = uint2_t{t.z, t.w};
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void transpose_copy_kernel(const TransposeArgs a) {
     __shared__ float tile[64][65];
     int64_t b = blockIdx.x;
@@ -963,6 +1056,39 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
             ++no;
         }
         t.n_other = no;
+        // whole 16-byte vectors (or 8-byte pieces) on both sides: the vector tiles
+        const int es = src_dtype == AXHIP_DTYPE_F32 ? 4 : 2;
+        auto side = [&](int64_t extent, int64_t stride, const int64_t *others, const void *base) { // bytes per access: 16, 8 or 0
+            for (int g = 16; g >= 8; g /= 2) {
+                const int64_t n = g / es;
+                bool ok = extent % n == 0 && stride % n == 0 && (reinterpret_cast<uintptr_t>(base) & static_cast<uintptr_t>(g - 1)) == 0;
+                for (int d = 0; d < no; ++d) ok = ok && others[d] % n == 0;
+                if (ok) return g;
+            }
+            return 0;
+        };
+        const int lg = side(t.nJ, t.src_stride_l, t.osrc, src), sg = side(t.nL, t.dst_stride_j, t.odst, dst);
+        const bool whole = src_dtype == dst_dtype && src_dtype != AXHIP_DTYPE_U8 && lg > 0 && sg > 0;
+        static const bool vec_tiles = [] { const char *e = getenv("AXHIP_TRANSPOSE_VEC"); return !(e && e[0] == '0'); }();
+        if (whole && vec_tiles) {
+            const int64_t edge = 16 * (16 / es);
+            t.tiles_j = (t.nJ + edge - 1) / edge; t.tiles_l = (t.nL + edge - 1) / edge;
+            blocks = blocks / (((t.nJ + 63) / 64) * ((t.nL + 63) / 64)) * t.tiles_j * t.tiles_l;
+            AXHIP_REQUIRE(blocks < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_strided_copy: view too large");
+            const dim3 grid(static_cast<unsigned>(blocks));
+#define AXHIP_TRANSPOSE(ES)                                                                                              \
+    do {                                                                                                                 \
+        if (lg == 16 && sg == 16) hipLaunchKernelGGL((transpose_vec_kernel<ES, 16, 16>), grid, dim3(256), 0, s, t);      \
+        else if (lg == 16) hipLaunchKernelGGL((transpose_vec_kernel<ES, 16, 8>), grid, dim3(256), 0, s, t);              \
+        else if (sg == 16) hipLaunchKernelGGL((transpose_vec_kernel<ES, 8, 16>), grid, dim3(256), 0, s, t);              \
+        else hipLaunchKernelGGL((transpose_vec_kernel<ES, 8, 8>), grid, dim3(256), 0, s, t);                             \
+    } while (0)
+            if (es == 2) AXHIP_TRANSPOSE(2);
+            else AXHIP_TRANSPOSE(4);
+#undef AXHIP_TRANSPOSE
+            AXHIP_CHECK_HIP(hipGetLastError());
+            return AXHIP_OK;
+        }
         AXHIP_REQUIRE(blocks < (int64_t(1) << 31), AXHIP_ERR_UNSUPPORTED, "axhip_strided_copy: view too large");
         hipLaunchKernelGGL(transpose_copy_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, t);
     } else {

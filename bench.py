@@ -525,6 +525,22 @@ def bench_survey(torch, capi, stream, steps, warmup):
         {"kernel": "pad", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes, "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
          "finite": bool(torch.equal(pout, torch.nn.functional.pad(pin.float(), (256, 256), mode="reflect").to(bf)))}, launch, avg_ms, nbytes)
     del xb, pin, pout
+    # transposed copies (axhip_strided_copy: 16 x 16 vector tiles through LDS)
+    for tname, shape, perm, dt in (("transpose_bf16_8192x8192", (8192, 8192), (1, 0), bf), ("transpose_f32_8192x8192", (8192, 8192), (1, 0), f32),
+                                   ("nchw_to_nhwc_bf16_64x64x128x128", (64, 64, 128, 128), (0, 2, 3, 1), bf),
+                                   ("transpose_bf16_32x1500x1280_to_32x1280x1500", (32, 1500, 1280), (0, 2, 1), bf)):
+        tin = rnd(shape, dt)
+        tv = tin.permute(*perm)
+        tout = torch.empty(tv.shape, dtype=dt, device="cuda")
+        tshape, tstr = (C.c_int64 * tv.dim())(*tv.shape), (C.c_int64 * tv.dim())(*tv.stride())
+        code = capi.DTYPE_BF16 if dt == bf else capi.DTYPE_F32
+        launch = lambda: capi.check(lib.axhip_strided_copy(tin.data_ptr(), code, tout.data_ptr(), code, tv.dim(), tshape, tstr, sp))
+        torch.cuda.synchronize()
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
+        nbytes = 2 * tin.numel() * tin.element_size()
+        res[tname] = with_cold({"kernel": "strided_copy (transpose tiles)", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+                                "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.equal(tout, tv))}, launch, avg_ms, nbytes)
+        del tin, tv, tout
     # rows of odd length
     for rows, cols, dt, name in ((30000, 1500, bf, "bf16"), (16384, 4100, bf, "bf16"), (16384, 4097, bf, "bf16"), (16384, 1501, f32, "f32")):
         t = rnd((rows, cols), dt)

@@ -59,6 +59,38 @@ def test_strided_copy_fast_paths_are_bit_exact(dt):
         assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view)), view.shape
 
 
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+def test_transposes_in_vector_tiles_are_bit_exact(dt):
+    """Transposed views whose two sides move whole 16-byte vectors, or 8-byte pieces (rows of 1500 16-bit elements): tiles
+    of 16 x 16 vectors through LDS.  Several tiles each way with ragged last tiles, extents that are multiples of a
+    vector on one side and of half a vector on the other, further dimensions before, between and behind the
+    transposed pair, a view at an offset inside its array, and extents that fall back to the element-wise tiles."""
+    vec = 4 if dt == F32 else 8
+    cases = [((300, 264), (1, 0)), ((3, 136, 200), (0, 2, 1)), ((2, 3, 72, 40 * vec), (0, 1, 3, 2)), ((2, 24 * vec, 5, 136), (0, 3, 2, 1)),
+             ((130, vec * 33 + vec // 2), (1, 0)), ((vec * 17 + vec // 2, 520), (1, 0)), ((2, 100, vec * 9 + vec // 2), (0, 2, 1)),
+             ((5, 129, 257), (0, 2, 1))]  # (the last: odd extents, the element-wise tiles)
+    g = axo.PCG64(600 + dt)
+    for shape, perm in cases:
+        base = sample(shape, dt, int(g.uniform((1,), 1, 100)[0]))
+        d = gh.to_dev(base)
+        view = base.transpose(perm)
+        out = gh.empty_dev(view.shape, dt)
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr(), dt, out.data_ptr(), dt, view.ndim, i64(view.shape), i64(elem_strides(view)), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view)), (shape, perm)
+    # a window of a larger array, transposed (its rows start every 264 elements, its first element at a vector boundary)
+    base = sample((4, 200, 264), dt, 7)
+    d = gh.to_dev(base)
+    view = base[1:3, 8:168, 2 * vec:2 * vec + 128].transpose(0, 2, 1)
+    off = view.__array_interface__["data"][0] - base.__array_interface__["data"][0]
+    out = gh.empty_dev(view.shape, dt)
+    gh.sync()
+    capi.check(capi.lib().axhip_strided_copy(d.data_ptr() + off, dt, out.data_ptr(), dt, view.ndim, i64(view.shape), i64(elem_strides(view)), None))
+    gh.sync()
+    assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view))
+
+
 def test_strided_copy_casts_on_the_fast_paths():
     x = axo.PCG64(10).normal((96, 200))
     d = gh.to_dev(x)
