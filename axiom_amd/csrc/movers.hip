@@ -999,6 +999,16 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
         }
     }
     a.ndim = nd;
+    // A cast of a contiguous array (nothing to gather) of 8 MiB or more is an elementwise chain with no operation: the
+    // compiled row kernel of that chain moves it (bf16 -> fp32 [16384,4096]: 72.6 -> 57.4 us, 69 -> 88 % of the HBM peak).
+    if (!bytes && src_dtype != dst_dtype && nd == 1 && a.strides[0] == 1 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0 &&
+        a.total * (src_dtype == AXHIP_DTYPE_F32 ? 4 : 2) >= (int64_t(8) << 20) && a.total % 4096 == 0) {
+        AxhipRowsProgram P{};
+        P.rows = a.total / 4096; P.cols = 4096;
+        P.input = src; P.input_dtype = src_dtype; P.output = dst; P.output_dtype = dst_dtype;
+        P.norm_weight = P.norm_bias = -1;
+        return axhip_fused_rows(&P, stream);
+    }
     int64_t max_off = 0;
     for (int d = 0; d < nd; ++d) max_off += (a.shape[d] - 1) * a.strides[d];
     const bool idx32 = a.total < (int64_t(1) << 31) - (1 << 23) && max_off < (int64_t(1) << 31) - (1 << 23); // room for the grid stride

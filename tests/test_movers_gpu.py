@@ -111,6 +111,26 @@ def test_strided_copy_casts_on_the_fast_paths():
         assert np.array_equal(gh.to_host(out, np.float32), axo.to_f32(bits, dt))
 
 
+def test_large_contiguous_casts_are_bit_exact():
+    """A cast of a contiguous array of 8 MiB or more runs as a compiled elementwise chain with no operation; the bits
+    are those of the oracle's conversions (round to nearest even into the 16-bit types, exact widening)."""
+    x = axo.PCG64(12).normal((1 << 22,)) * 3
+    d = gh.to_dev(x)
+    for dt in (F16, BF16):
+        out = gh.empty_dev(x.shape, dt)
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr(), F32, out.data_ptr(), dt, 1, i64(x.shape), i64([1]), None))
+        gh.sync()
+        bits = gh.to_host(out, np.uint16)
+        assert np.array_equal(bits, axo.to_bits(x, dt))
+        db = gh.to_dev(bits)
+        back = gh.empty_dev((1 << 11, 1 << 11), F32)  # (the same array as a matrix: contiguous all the same)
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(db.data_ptr(), dt, back.data_ptr(), F32, 2, i64((1 << 11, 1 << 11)), i64([1 << 11, 1]), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(back, np.float32).ravel(), axo.to_f32(bits, dt))
+
+
 def test_strided_copy_casts_like_the_oracle():
     x = axo.PCG64(9).normal((33, 17))
     d = gh.to_dev(x)
