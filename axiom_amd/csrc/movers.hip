@@ -36,8 +36,9 @@ __global__ __launch_bounds__(256) void strided_copy_kernel(const CopyArgs a) {
 
 // Views whose innermost dimension is contiguous (head splits, slices, broadcasts of rows, plain casts): one thread
 // moves V consecutive elements with 16-byte accesses; a.shape[ndim-1] counts such groups and a.strides[ndim-1] is V.
-// RAW: same dtype on both sides, the bytes are moved as they are.
-template <typename IDX, int V, bool RAW>
+// RAW: same dtype on both sides, the bytes are moved as they are.  UNALIGNED: the groups start anywhere in the source
+// (a column slice from an odd column, the windows of a convolution): unaligned 16-byte loads, aligned stores.
+template <typename IDX, int V, bool RAW, bool UNALIGNED = false>
 __global__ __launch_bounds__(256) void strided_copy_vec_kernel(const CopyArgs a) {
     const IDX stride = static_cast<IDX>(gridDim.x) * 256, total = static_cast<IDX>(a.total);
     for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
@@ -50,13 +51,51 @@ __global__ __launch_bounds__(256) void strided_copy_vec_kernel(const CopyArgs a)
         }
         if constexpr (RAW) { // V elements = 16 bytes
             const int es = a.src_dtype == AXHIP_DTYPE_F32 ? 4 : 2;
-            const uint4_t t = *reinterpret_cast<const uint4_t *>(static_cast<const char *>(a.src) + static_cast<int64_t>(off) * es);
+            const uint4_t t = vec_load<UNALIGNED>(reinterpret_cast<const uint4_t *>(static_cast<const char *>(a.src) + static_cast<int64_t>(off) * es));
             reinterpret_cast<uint4_t *>(a.dst)[i] = t;
         } else {
             float v[V];
-            load_vec<V>(a.src, a.src_dtype, off, v);
+            load_vec<V, UNALIGNED>(a.src, a.src_dtype, off, v);
             store_vec<V>(a.dst, a.dst_dtype, static_cast<int64_t>(i) * V, v);
         }
+    }
+}
+
+// Every other element of the source's innermost dimension (x[:, ::2], the windows of a stride-2 convolution), same type
+// on both sides: a group of V results comes out of two unaligned 16-byte loads -- the second one starts an element
+// early, so that it ends with the group's last picked element and nothing behind the view is touched -- with the
+// wanted elements picked in registers, and leaves as one aligned 16-byte store.  a.shape[ndim-1] counts groups,
+// a.strides[ndim-1] is 2 V.  HALF: groups of half a vector (rows of 1500 16-bit results: 8-byte loads and stores).
+template <typename IDX, int ES, bool HALF>
+__global__ __launch_bounds__(256) void strided_copy_every_other_kernel(const CopyArgs a) {
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, total = static_cast<IDX>(a.total);
+    for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        IDX rem = i, off = 0;
+        for (int d = a.ndim - 1; d >= 0; --d) {
+            const IDX n = static_cast<IDX>(a.shape[d]);
+            const IDX q = rem / n;
+            off += (rem - q * n) * static_cast<IDX>(a.strides[d]);
+            rem = q;
+        }
+        const char *p = static_cast<const char *>(a.src) + static_cast<int64_t>(off) * ES;
+        if constexpr (HALF) {
+            const uint2_t lo = vec_load<true>(reinterpret_cast<const uint2_t *>(p)), hi = vec_load<true>(reinterpret_cast<const uint2_t *>(p + 8 - ES));
+            uint2_t t;
+            if constexpr (ES == 4) t = uint2_t{lo.x, hi.y};
+            else t = uint2_t{__builtin_amdgcn_perm(lo.y, lo.x, 0x05040100u), __builtin_amdgcn_perm(hi.y, hi.x, 0x07060302u)};
+            reinterpret_cast<uint2_t *>(a.dst)[i] = t;
+            continue;
+        }
+        const uint4_t lo = vec_load<true>(reinterpret_cast<const uint4_t *>(p));            // elements 0 .. V - 1
+        const uint4_t hi = vec_load<true>(reinterpret_cast<const uint4_t *>(p + 16 - ES)); // elements V - 1 .. 2 V - 2
+        uint4_t t;
+        if constexpr (ES == 4) {
+            t = uint4_t{lo.x, lo.z, hi.y, hi.w};
+        } else { // lo: the low halves of consecutive words; hi (an element late): the high halves
+            t = uint4_t{__builtin_amdgcn_perm(lo.y, lo.x, 0x05040100u), __builtin_amdgcn_perm(lo.w, lo.z, 0x05040100u),
+                        __builtin_amdgcn_perm(hi.y, hi.x, 0x07060302u), __builtin_amdgcn_perm(hi.w, hi.z, 0x07060302u)};
+        }
+        reinterpret_cast<uint4_t *>(a.dst)[i] = t;
     }
 }
 
@@ -1021,13 +1060,37 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
     bool vec = !bytes && nd >= 1 && a.strides[nd - 1] == 1 && a.shape[nd - 1] % v == 0 && reinterpret_cast<uintptr_t>(src) % src_align == 0 &&
                reinterpret_cast<uintptr_t>(dst) % (v * dst_es >= 16 ? 16 : 8) == 0;
     for (int d = 0; vec && d + 1 < nd; ++d) vec = (a.strides[d] * src_es) % src_align == 0;
+    // the same with groups that start anywhere in the source (x[:, 1:], convolution windows): unaligned loads
+    static const bool unaligned_on = [] { const char *e = getenv("AXHIP_COPY_UNALIGNED"); return !(e && e[0] == '0'); }();
+    const bool vec_unaligned = !vec && unaligned_on && !bytes && nd >= 1 && a.strides[nd - 1] == 1 && a.shape[nd - 1] % v == 0 &&
+                               reinterpret_cast<uintptr_t>(dst) % (v * dst_es >= 16 ? 16 : 8) == 0;
+    vec = vec || vec_unaligned;
+    // every other element, same type, whole groups of a vector or of half a vector
+    const int gv = nd >= 1 && a.shape[nd - 1] % v == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 ? v : v / 2;
+    const bool every_other = !vec && unaligned_on && !bytes && raw && nd >= 1 && a.strides[nd - 1] == 2 && a.shape[nd - 1] % gv == 0 &&
+                             reinterpret_cast<uintptr_t>(dst) % (gv == v ? 16 : 8) == 0;
     // transposes: the innermost dimension is strided, some other dimension is contiguous in the source
     int transpose_j = -1;
     if (!vec && !bytes && nd >= 2 && a.strides[nd - 1] > 1 && a.shape[nd - 1] >= 16) {
         for (int d = 0; d + 1 < nd; ++d)
             if (a.strides[d] == 1 && a.shape[d] >= 16) transpose_j = d;
     }
-    if (vec) {
+    if (every_other) {
+        a.shape[nd - 1] /= gv;
+        a.strides[nd - 1] = 2 * gv;
+        a.total /= gv;
+        const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        auto launch = [&](auto idx_tag) {
+            using IDX = decltype(idx_tag);
+            if (src_es == 4 && gv == v) hipLaunchKernelGGL((strided_copy_every_other_kernel<IDX, 4, false>), grid, dim3(256), 0, s, a);
+            else if (src_es == 4) hipLaunchKernelGGL((strided_copy_every_other_kernel<IDX, 4, true>), grid, dim3(256), 0, s, a);
+            else if (gv == v) hipLaunchKernelGGL((strided_copy_every_other_kernel<IDX, 2, false>), grid, dim3(256), 0, s, a);
+            else hipLaunchKernelGGL((strided_copy_every_other_kernel<IDX, 2, true>), grid, dim3(256), 0, s, a);
+        };
+        if (idx32) launch(int32_t{});
+        else launch(int64_t{});
+    } else if (vec) {
         a.shape[nd - 1] /= v;
         a.strides[nd - 1] = v;
         a.total /= v;
@@ -1035,6 +1098,13 @@ int axhip_strided_copy(const void *src, int32_t src_dtype, void *dst, int32_t ds
         const dim3 grid(static_cast<unsigned>(blocks));
         auto launch = [&](auto idx_tag) {
             using IDX = decltype(idx_tag);
+            if (vec_unaligned) {
+                if (raw && v == 4) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 4, true, true>), grid, dim3(256), 0, s, a);
+                else if (raw) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 8, true, true>), grid, dim3(256), 0, s, a);
+                else if (v == 4) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 4, false, true>), grid, dim3(256), 0, s, a);
+                else hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 8, false, true>), grid, dim3(256), 0, s, a);
+                return;
+            }
             if (raw && v == 4) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 4, true>), grid, dim3(256), 0, s, a);
             else if (raw) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 8, true>), grid, dim3(256), 0, s, a);
             else if (v == 4) hipLaunchKernelGGL((strided_copy_vec_kernel<IDX, 4, false>), grid, dim3(256), 0, s, a);

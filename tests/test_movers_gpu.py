@@ -111,6 +111,42 @@ def test_strided_copy_casts_on_the_fast_paths():
         assert np.array_equal(gh.to_host(out, np.float32), axo.to_f32(bits, dt))
 
 
+@pytest.mark.parametrize("dt", [F32, F16, BF16], ids=["f32", "f16", "bf16"])
+def test_gathers_from_unaligned_and_every_other_positions_are_bit_exact(dt):
+    """Views whose innermost dimension is contiguous in the source but starts anywhere (a column slice from an odd
+    column, the windows of a convolution) move as unaligned 16-byte loads and aligned stores; views that take every
+    other element (x[:, ::2], the windows of a stride-2 convolution) pick a group out of two such loads, the second of
+    which ends with the group's last element -- the array's very last element included.  With a cast on the way for
+    the contiguous kind."""
+    vec = 4 if dt == F32 else 8
+    base = sample((3, 5, 40, 12 * vec + 3), dt, 21)
+    d = gh.to_dev(base)
+    w = 8 * vec
+    views = [base[:, :, :, 1:1 + w], base[:, :, 3:, 3:3 + w], base[1, :, ::3, 2:2 + w],
+             np.lib.stride_tricks.as_strided(base, (3, 5, 3, 38, w), base.strides[:2] + (base.strides[2], base.strides[2], base.strides[3])),  # windows of 3 rows
+             base[:, :, :, ::2][..., :5 * vec], base[:, :, :, 1::2][..., :6 * vec], base[2, 4, 39:, 3::2][..., :6 * vec],
+             np.lib.stride_tricks.as_strided(base[0, 0, 0], (3, 4 * vec), (base.strides[3], 2 * base.strides[3]))]  # windows of a stride-2 convolution
+    flat = base.reshape(-1)
+    views.append(flat[flat.size - 2 * (2 * vec) + 1::2])  # ends with the array's last element
+    views.append(flat[flat.size - 2 * (vec + vec // 2) + 1::2])  # the same with a half group at its end
+    views.append(base[:, :, :, ::2][..., :5 * vec + vec // 2])  # rows of whole half groups (8-byte loads and stores)
+    for view in views:
+        out = gh.empty_dev(view.shape, dt)
+        off = view.__array_interface__["data"][0] - base.__array_interface__["data"][0]
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr() + off, dt, out.data_ptr(), dt, view.ndim, i64(view.shape), i64(elem_strides(view)), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, base.dtype), np.ascontiguousarray(view)), view.shape
+    if dt != F32:
+        view = base[:, :, :, 1:1 + w]
+        out = gh.empty_dev(view.shape, F32)
+        off = view.__array_interface__["data"][0] - base.__array_interface__["data"][0]
+        gh.sync()
+        capi.check(capi.lib().axhip_strided_copy(d.data_ptr() + off, dt, out.data_ptr(), F32, view.ndim, i64(view.shape), i64(elem_strides(view)), None))
+        gh.sync()
+        assert np.array_equal(gh.to_host(out, np.float32), axo.to_f32(np.ascontiguousarray(view), dt))
+
+
 def test_large_contiguous_casts_are_bit_exact():
     """A cast of a contiguous array of 8 MiB or more runs as a compiled elementwise chain with no operation; the bits
     are those of the oracle's conversions (round to nearest even into the 16-bit types, exact widening)."""
