@@ -378,6 +378,56 @@ __global__ __launch_bounds__(256) void masked_fill_kernel(const MaskedFillArgs a
     }
 }
 
+// The same over views whose innermost dimension is contiguous in the source and contiguous or broadcast in the mask
+// (an attention mask over [batch, heads, queries, keys], a key-padding mask that repeats over the queries): one
+// thread takes 16 bytes of the source and the 16 / ES mask bytes that go with them (one byte when the mask repeats
+// along the row), picks per element in registers and stores 16 bytes.  a.shape[ndim-1] counts such groups;
+// a.src_strides[ndim-1] is 16 / ES and a.mask_strides[ndim-1] is 16 / ES or 0.
+template <typename IDX, int ES>
+__global__ __launch_bounds__(256) void masked_fill_vec_kernel(const MaskedFillArgs a) {
+    constexpr int V = 16 / ES;
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, total = static_cast<IDX>(a.total);
+    uint32_t fill;
+    if constexpr (ES == 4) fill = __float_as_uint(a.value);
+    else fill = a.dtype == AXHIP_DTYPE_F16 ? f32_to_f16_bits(a.value) & 0xffffu : f32_to_bf16_bits(a.value) & 0xffffu;
+    const bool mask_row = a.mask_strides[a.ndim - 1] != 0;
+    for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        IDX rem = i, soff = 0, moff = 0;
+        for (int d = a.ndim - 1; d >= 0; --d) {
+            const IDX n = static_cast<IDX>(a.shape[d]);
+            const IDX q = rem / n, c = rem - q * n;
+            soff += c * static_cast<IDX>(a.src_strides[d]);
+            moff += c * static_cast<IDX>(a.mask_strides[d]);
+            rem = q;
+        }
+        uint4_t t = *reinterpret_cast<const uint4_t *>(static_cast<const char *>(a.src) + static_cast<int64_t>(soff) * ES);
+        uint32_t m[2]; // the group's mask bytes, one per element
+        if (mask_row) {
+            if constexpr (V == 8) {
+                const uint2_t mm = *reinterpret_cast<const uint2_t *>(a.mask + moff);
+                m[0] = mm.x; m[1] = mm.y;
+            } else {
+                m[0] = *reinterpret_cast<const uint32_t *>(a.mask + moff); m[1] = 0;
+            }
+        } else {
+            m[0] = m[1] = a.mask[moff] ? 0x01010101u : 0u;
+        }
+        uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if constexpr (ES == 4) {
+                if ((m[0] >> (8 * k)) & 0xffu) w[k] = fill;
+            } else {
+                const uint32_t mk = m[k >> 1] >> (16 * (k & 1));
+                if (mk & 0xffu) w[k] = (w[k] & 0xffff0000u) | fill;
+                if (mk & 0xff00u) w[k] = (w[k] & 0x0000ffffu) | (fill << 16);
+            }
+        }
+        t.x = w[0]; t.y = w[1]; t.z = w[2]; t.w = w[3];
+        reinterpret_cast<uint4_t *>(a.dst)[i] = t;
+    }
+}
+
 // where(cond, a, b): dst[i] = cond[i] ? a[i] : b[i] over an iteration space of up to 8 dimensions; the three inputs
 // are strided views (stride 0 on broadcast dimensions), each of a type of its own; dst is contiguous.
 struct WhereArgs {
@@ -1275,6 +1325,33 @@ int axhip_masked_fill(const void *src, int32_t dtype, const uint8_t *mask, void 
     AXHIP_REQUIRE(src && mask && dst, AXHIP_ERR_INVALID_ARG, "axhip_masked_fill: NULL buffer");
     int rc = ensure_init();
     if (rc) return rc;
+    // Rows that are contiguous in the source and contiguous or repeated in the mask go 16 bytes a thread.
+    const int es = dtype == AXHIP_DTYPE_F32 ? 4 : 2, v = 16 / es, last = ndim - 1;
+    static const bool vec_on = [] { const char *e = getenv("AXHIP_MASKED_FILL_VEC"); return !(e && e[0] == '0'); }();
+    bool vec = vec_on && ndim >= 1 && src_strides[last] == 1 && (mask_strides[last] == 0 || mask_strides[last] == 1) && shape[last] % v == 0 &&
+               (reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % 16 == 0;
+    const bool mask_row = vec && mask_strides[last] == 1;
+    if (mask_row && reinterpret_cast<uintptr_t>(mask) % v != 0) vec = false;
+    int64_t src_span = 0, mask_span = 0; // the largest element offsets
+    for (int d = 0; d < ndim && vec; ++d) {
+        src_span += (shape[d] - 1) * src_strides[d];
+        mask_span += (shape[d] - 1) * mask_strides[d];
+        if (d == last) continue;
+        if (src_strides[d] % v != 0 || (mask_row && mask_strides[d] % v != 0)) vec = false;
+    }
+    if (vec) {
+        a.shape[last] = shape[last] / v;
+        a.src_strides[last] = v;
+        a.mask_strides[last] = mask_row ? v : 0;
+        a.total /= v;
+        const bool idx32 = a.total < (1ll << 31) && src_span < (1ll << 31) && mask_span < (1ll << 31);
+        const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 32);
+        auto kernel = idx32 ? (es == 4 ? masked_fill_vec_kernel<uint32_t, 4> : masked_fill_vec_kernel<uint32_t, 2>)
+                            : (es == 4 ? masked_fill_vec_kernel<int64_t, 4> : masked_fill_vec_kernel<int64_t, 2>);
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), a);
+        AXHIP_CHECK_HIP(hipGetLastError());
+        return AXHIP_OK;
+    }
     const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 64);
     hipLaunchKernelGGL(masked_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, resolve_stream(stream), a);
     AXHIP_CHECK_HIP(hipGetLastError());

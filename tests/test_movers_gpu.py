@@ -285,6 +285,30 @@ def test_masked_fill_with_broadcast_masks(dt):
         assert np.array_equal(gh.to_host(out, x.dtype), np.where(bm != 0, fill, x))
 
 
+@pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("cols,pitch", [(64, 64), (48, 72), (12, 12), (40, 44)], ids=["64", "48of72", "12", "40of44"])
+def test_masked_fill_of_row_views_sixteen_bytes_at_a_time(dt, cols, pitch):
+    """Rows that are contiguous in the source take the vector kernel when their length, pitch and the mask's pitches
+    are whole 16-byte groups (64, 48 of 72) and the element kernel otherwise (12; 40 of 44 for the 16-bit types); the
+    mask's bytes are any non-zero value; a mask over [queries, keys], one over everything, and one that repeats along
+    the keys."""
+    base = sample((3, 5, 33, pitch), dt, 31)
+    x = base[..., :cols]
+    d = gh.to_dev(base)
+    rng = axo.PCG64(32)
+    any_byte = lambda shape: ((rng.normal(shape) > 0.3) * (1 + (np.abs(rng.normal(shape)) * 100).astype(np.int64) % 255)).astype(np.uint8)
+    fill = np.float32(-3.5)
+    for mshape, mstr in (((33, cols), [0, 0, cols, 1]), (x.shape, [5 * 33 * cols, 33 * cols, cols, 1]), ((3, 1, 33, 1), [33, 0, 1, 0]), ((3, 1, 1, cols), [cols, 0, 0, 1])):
+        mask = any_byte(mshape)
+        m = torch.from_numpy(mask).cuda()
+        out = gh.empty_dev(x.shape, dt)
+        gh.sync()
+        capi.check(capi.lib().axhip_masked_fill(d.data_ptr(), dt, m.data_ptr(), out.data_ptr(), 4, i64(x.shape), i64(elem_strides(x)), i64(mstr), float(fill), None))
+        gh.sync()
+        want = np.where(np.broadcast_to(mask, x.shape) != 0, fill if dt == F32 else axo.to_bits(np.array([fill], np.float32), dt)[0], x)
+        assert np.array_equal(gh.to_host(out, x.dtype), want), (mshape, mstr)
+
+
 @pytest.mark.parametrize("dt,cols", [(F32, 8), (BF16, 64), (F16, 7), (F32, 3)], ids=["f32x8", "bf16x64", "f16x7", "f32x3"])
 @pytest.mark.parametrize("itype", [np.int64, np.int32], ids=["i64", "i32"])
 def test_gather_rows_is_an_embedding_lookup(dt, cols, itype):
