@@ -280,17 +280,40 @@ __global__ __launch_bounds__(256) void pad_kernel(const PadArgs a) {
     }
 }
 
+// V elements of a constant pad's output row from source coordinate c0 on, for rows of V contiguous elements or more:
+// the elements inside [0, n) come out of one unaligned 16-byte load placed inside the row and shifted into place in
+// registers (the result is 16 of the 48 bytes constant | load | constant); the rest are the constant f.
+template <typename IDX, int V>
+__device__ __forceinline__ uint4_t pad_const_group(const char *row, IDX c0, IDX n, uint32_t f) {
+    constexpr int ES = 16 / V;
+    if (c0 + V <= 0 || c0 >= n) return uint4_t{f, f, f, f};
+    const IDX at = c0 < 0 ? 0 : c0 > n - V ? n - V : c0;
+    const uint4_t w = reinterpret_cast<const uint4_unaligned_t *>(row + static_cast<int64_t>(at) * ES)->v;
+    if (at == c0) return w;
+    const int b = 16 - static_cast<int>(at - c0) * ES, k = b >> 2, r = b & 3; // 0 < b < 32
+    auto word = [&](int i) { return i == 4 ? w.x : i == 5 ? w.y : i == 6 ? w.z : i == 7 ? w.w : f; };
+    uint32_t d[5];
+#pragma unroll
+    for (int j = 0; j < 5; ++j) d[j] = word(k + j);
+    return uint4_t{__builtin_amdgcn_alignbyte(d[1], d[0], r), __builtin_amdgcn_alignbyte(d[2], d[1], r),
+                   __builtin_amdgcn_alignbyte(d[3], d[2], r), __builtin_amdgcn_alignbyte(d[4], d[3], r)};
+}
+
 // The same with V consecutive elements of the innermost output dimension per thread (V elements are 16 bytes): one
 // decomposition of the index per V elements.  A group whose sources are a run of the innermost source dimension --
 // the interior, a wrapped-around run of a circular pad, or, backwards, the mirror image of a reflected pad -- is one
 // 16-byte load and one 16-byte store (2- or 4-byte aligned: rows start wherever the extents put them); the groups on
 // a border, a row's last, shorter group and strided sources go element by element.
+// FLAT (output rows that are not whole groups, in an aligned output): the groups are the aligned 16-byte pieces of the
+// whole output instead of pieces counted from each row's start, so that every store is aligned; a group that runs
+// over a row's end goes element by element, the rest of it in the next row.
 // IDX: int32_t when every index and offset fits.
-template <typename IDX, int V>
+template <typename IDX, int V, bool FLAT = false>
 __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
     const int L = a.ndim - 1;
     const IDX out_last = static_cast<IDX>(a.out_shape[L]), inner = (out_last + V - 1) / V;
-    const IDX stride = static_cast<IDX>(gridDim.x) * 256, groups = static_cast<IDX>(a.total / out_last) * inner;
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, n_rows = static_cast<IDX>(a.total / out_last);
+    const IDX groups = FLAT ? static_cast<IDX>((a.total + V - 1) / V) : n_rows * inner;
     const IDX before = static_cast<IDX>(a.before[L]), n_src = static_cast<IDX>(a.src_shape[L]), st = static_cast<IDX>(a.src_strides[L]);
     constexpr int ES = 16 / V;
     uint4_t fill; // V copies of the constant in the element type
@@ -300,22 +323,56 @@ __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
         const uint32_t h = a.dtype == AXHIP_DTYPE_BF16 ? pack_bf16x2(a.value, a.value) : pack_f16x2(a.value, a.value);
         fill = uint4_t{h, h, h, h};
     }
-    const bool rows_aligned = out_last % V == 0 && (reinterpret_cast<uintptr_t>(a.dst) & 15u) == 0; // every group's 16 bytes of output are aligned
+    const bool rows_aligned = FLAT || (out_last % V == 0 && (reinterpret_cast<uintptr_t>(a.dst) & 15u) == 0); // every group's 16 bytes of output are aligned
     for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < groups; i += stride) {
-        const IDX row = i / inner, g = i - row * inner;
-        IDX rem = row, off = 0;
-        const IDX c0 = g * V - before;
-        const int nvalid = static_cast<int>(out_last - g * V < V ? out_last - g * V : V);
-        bool inside = true;
-        for (int d = L - 1; d >= 0; --d) {
-            const IDX n = static_cast<IDX>(a.out_shape[d]);
-            const IDX q = rem / n;
-            const IDX c = pad_source<IDX>(rem - q * n - static_cast<IDX>(a.before[d]), static_cast<IDX>(a.src_shape[d]), a.mode);
-            rem = q;
-            inside = inside && c >= 0;
-            off += c * static_cast<IDX>(a.src_strides[d]);
+        IDX row, col; // where the group starts
+        if constexpr (FLAT) {
+            row = i * V / out_last;
+            col = i * V - row * out_last;
+        } else {
+            row = i / inner;
+            col = (i - row * inner) * V;
         }
-        const int64_t out_index = static_cast<int64_t>(row) * out_last + static_cast<int64_t>(g) * V;
+        IDX off = 0;
+        const IDX c0 = col - before;
+        const int nvalid = static_cast<int>(out_last - col < V ? out_last - col : V); // elements of the group in this row
+        bool inside = true;
+        auto outer = [&](IDX rem) { // the source offset of an output row, or that all of it is padding
+            off = 0;
+            inside = true;
+            for (int d = L - 1; d >= 0; --d) {
+                const IDX n = static_cast<IDX>(a.out_shape[d]);
+                const IDX q = rem / n;
+                const IDX c = pad_source<IDX>(rem - q * n - static_cast<IDX>(a.before[d]), static_cast<IDX>(a.src_shape[d]), a.mode);
+                rem = q;
+                inside = inside && c >= 0;
+                off += c * static_cast<IDX>(a.src_strides[d]);
+            }
+        };
+        outer(row);
+        const int64_t out_index = static_cast<int64_t>(row) * out_last + static_cast<int64_t>(col);
+        if (a.mode == AXHIP_PAD_CONSTANT && st == 1 && n_src >= V && (nvalid == V || (FLAT && row + 1 < n_rows))) {
+            // constant pads of contiguous rows: every group, borders included, is one load (two where the group runs
+            // over a row's end in a flat output) and one store
+            const char *src = static_cast<const char *>(a.src);
+            uint4_t w = inside ? pad_const_group<IDX, V>(src + static_cast<int64_t>(off) * ES, c0, n_src, fill.x) : fill;
+            if (nvalid < V) {
+                outer(row + 1);
+                const uint4_t u = inside ? pad_const_group<IDX, V>(src + static_cast<int64_t>(off) * ES, -static_cast<IDX>(nvalid) - before, n_src, fill.x) : fill;
+                const uint32_t wa[4] = {w.x, w.y, w.z, w.w}, ua[4] = {u.x, u.y, u.z, u.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if constexpr (V == 4) o[j] = j < nvalid ? wa[j] : ua[j];
+                    else o[j] = ((2 * j < nvalid ? wa[j] : ua[j]) & 0xffffu) | ((2 * j + 1 < nvalid ? wa[j] : ua[j]) & 0xffff0000u);
+                }
+                w = uint4_t{o[0], o[1], o[2], o[3]};
+            }
+            char *out = static_cast<char *>(a.dst) + out_index * ES;
+            if (rows_aligned) *reinterpret_cast<uint4_t *>(out) = w;
+            else reinterpret_cast<uint4_unaligned_t *>(out)->v = w;
+            continue;
+        }
         if (nvalid == V && a.mode == AXHIP_PAD_CONSTANT && (!inside || c0 + V <= 0 || c0 >= n_src)) { // nothing but the constant
             char *out = static_cast<char *>(a.dst) + out_index * ES;
             if (rows_aligned) *reinterpret_cast<uint4_t *>(out) = fill;
@@ -337,7 +394,7 @@ __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
                 continue;
             }
         }
-        if (rows_aligned) { // (then every group is whole)
+        if (rows_aligned && nvalid == V) {
             float v[V];
 #pragma unroll
             for (int e = 0; e < V; ++e) {
@@ -346,6 +403,24 @@ __global__ __launch_bounds__(256) void pad_vec_kernel(const PadArgs a) {
             }
             store_vec<V>(a.dst, a.dtype, out_index, v);
             continue;
+        }
+        if constexpr (FLAT) { // the rest of the group is the start of the next row (rows hold V elements or more)
+            if (row + 1 < n_rows) {
+                float v[V]; // all loads first, one store
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const IDX c = pad_source<IDX>(c0 + e, n_src, a.mode);
+                    if (e < nvalid) v[e] = inside && c >= 0 ? load_any(a.src, a.dtype, off + c * st) : a.value;
+                }
+                outer(row + 1);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const IDX c = pad_source<IDX>(e - nvalid - before, n_src, a.mode);
+                    if (e >= nvalid) v[e] = inside && c >= 0 ? load_any(a.src, a.dtype, off + c * st) : a.value;
+                }
+                store_vec<V>(a.dst, a.dtype, out_index, v);
+                continue;
+            }
         }
         for (int e = 0; e < nvalid; ++e) {
             const IDX c = pad_source<IDX>(c0 + e, n_src, a.mode);
@@ -1286,10 +1361,21 @@ int axhip_pad_mode(const void *src, void *dst, int32_t dtype, int32_t ndim, cons
         int64_t reach = a.total; // the largest index or source offset the kernel forms
         for (int d = 0; d < ndim; ++d) reach = std::max(reach, (a.src_shape[d] + a.out_shape[d]) * std::max<int64_t>(a.src_strides[d], 1));
         const bool small = reach < (int64_t(1) << 31) - (1 << 20);
-        const int64_t n_groups = a.total / a.out_shape[ndim - 1] * ((a.out_shape[ndim - 1] + V - 1) / V);
+        // Rows that are not whole 16-byte groups in an aligned output: the groups are cut from the whole output.
+        static const bool flat_on = [] { const char *e = getenv("AXHIP_PAD_FLAT"); return !(e && e[0] == '0'); }();
+        const bool flat = flat_on && a.out_shape[ndim - 1] % V != 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0;
+        const int64_t n_groups = flat ? (a.total + V - 1) / V : a.total / a.out_shape[ndim - 1] * ((a.out_shape[ndim - 1] + V - 1) / V);
         const int64_t blocks = std::min<int64_t>((n_groups + 255) / 256, 256 * 64);
         hipStream_t s = resolve_stream(stream);
-        if (V == 4) {
+        if (flat) {
+            if (V == 4) {
+                if (small) hipLaunchKernelGGL((pad_vec_kernel<int32_t, 4, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+                else hipLaunchKernelGGL((pad_vec_kernel<int64_t, 4, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+            } else {
+                if (small) hipLaunchKernelGGL((pad_vec_kernel<int32_t, 8, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+                else hipLaunchKernelGGL((pad_vec_kernel<int64_t, 8, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+            }
+        } else if (V == 4) {
             if (small) hipLaunchKernelGGL((pad_vec_kernel<int32_t, 4>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
             else hipLaunchKernelGGL((pad_vec_kernel<int64_t, 4>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
         } else {

@@ -194,7 +194,9 @@ def test_fill(dt):
                                                 ((2, 1, 3, 4), (1, 0, 2, 0), (0, 3, 0, 5)),
                                                 # innermost output extents of whole 16-byte vectors: one store per vector
                                                 ((3, 5, 27), (1, 0, 2), (0, 2, 3)), ((2, 2, 30, 48), (0, 0, 0, 0), (0, 0, 0, 16)), ((7, 1001), (0, 0), (0, 23)),
-                                                ((64,), (0,), (0,)), ((4, 300), (0, 40), (1, 37)), ((2, 3, 256), (0, 0, 64), (0, 1, 64))])
+                                                ((64,), (0,), (0,)), ((4, 300), (0, 40), (1, 37)), ((2, 3, 256), (0, 0, 64), (0, 1, 64)),
+                                                # odd rows in an aligned output: groups cut from the whole output, some across two rows
+                                                ((3, 7, 301), (0, 1, 1), (1, 0, 1)), ((5, 9), (1, 0), (0, 0))])
 def test_pad_matches_numpy(dt, shape, before, after):
     x = sample(shape, dt, 11)
     value = -2.5
@@ -214,7 +216,8 @@ def test_pad_matches_numpy(dt, shape, before, after):
                                                 ((2, 2, 30, 48), (0, 1, 0, 7), (1, 0, 0, 9)), ((7, 1001), (3, 0), (0, 23)),
                                                 # pads longer than a 16-byte group along the innermost extent: whole groups are mirror images
                                                 # (read backwards) or wrapped-around runs; odd and whole-vector output rows
-                                                ((4, 300), (0, 40), (0, 37)), ((2, 3, 256), (0, 0, 64), (0, 1, 64)), ((3, 100), (1, 99), (0, 99))])
+                                                ((4, 300), (0, 40), (0, 37)), ((2, 3, 256), (0, 0, 64), (0, 1, 64)), ((3, 100), (1, 99), (0, 99)),
+                                                ((3, 7, 301), (0, 1, 1), (1, 0, 1)), ((5, 9), (1, 0), (0, 0))])
 def test_pad_modes_match_numpy(dt, mode, np_mode, shape, before, after):
     """reflect / replicate / circular as the reference indexes them (src/tensor/operations.cpp:2216-2246), which is
     what numpy's 'reflect' / 'edge' / 'wrap' do."""
