@@ -546,6 +546,39 @@ __global__ __launch_bounds__(256) void where_vec_kernel(const WhereArgs w, const
     }
 }
 
+// Views whose innermost dimension each input either runs along or repeats over (a mask over [queries, keys] against
+// [batch, heads, queries, keys] scores, a row vector, a column of per-row values): one thread takes V consecutive
+// elements of a row -- a vector load from the inputs that run along it, one element from those that repeat -- and
+// stores them as whole vectors.  w.shape[ndim-1] counts such groups; the inputs' strides there are V or 0.
+template <typename IDX, int V>
+__global__ __launch_bounds__(256) void where_rows_kernel(const WhereArgs w) {
+    const int L = w.ndim - 1;
+    const bool c_row = w.cond_strides[L] != 0, a_row = w.a_strides[L] != 0, b_row = w.b_strides[L] != 0;
+    const IDX stride = static_cast<IDX>(gridDim.x) * 256, total = static_cast<IDX>(w.total);
+    for (IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        IDX rem = i, coff = 0, aoff = 0, boff = 0;
+        for (int d = L; d >= 0; --d) {
+            const IDX n = static_cast<IDX>(w.shape[d]);
+            const IDX q = rem / n, c = rem - q * n;
+            rem = q;
+            coff += c * static_cast<IDX>(w.cond_strides[d]);
+            aoff += c * static_cast<IDX>(w.a_strides[d]);
+            boff += c * static_cast<IDX>(w.b_strides[d]);
+        }
+        float m[V], x[V], y[V];
+        if (c_row) load_vec<V>(w.cond, w.cond_dtype, coff, m);
+        else m[0] = load_any(w.cond, w.cond_dtype, coff);
+        if (a_row) load_vec<V>(w.a, w.a_dtype, aoff, x);
+        else x[0] = load_any(w.a, w.a_dtype, aoff);
+        if (b_row) load_vec<V>(w.b, w.b_dtype, boff, y);
+        else y[0] = load_any(w.b, w.b_dtype, boff);
+        const float m0 = m[0], x0 = x[0], y0 = y[0];
+#pragma unroll
+        for (int e = 0; e < V; ++e) x[e] = (c_row ? m[e] : m0) != 0.0f ? (a_row ? x[e] : x0) : (b_row ? y[e] : y0);
+        store_vec<V>(w.dst, w.dst_dtype, static_cast<int64_t>(i) * V, x);
+    }
+}
+
 // One thread moves `chunk` bytes (16, or the element size when rows are not 16-byte
 // multiples) of one output row.
 template <typename V>
@@ -1486,8 +1519,36 @@ int axhip_where(const void *cond, int32_t cond_dtype, const void *a, int32_t a_d
         if (v == 4) hipLaunchKernelGGL(where_vec_kernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w, a_one, b_one);
         else hipLaunchKernelGGL(where_vec_kernel<8>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w, a_one, b_one);
     } else {
-        const int64_t blocks = std::min<int64_t>((w.total + 255) / 256, 256 * 64);
-        hipLaunchKernelGGL(where_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w);
+        // Inputs that run along the innermost dimension or repeat over it, in whole aligned vectors: V elements a thread.
+        static const bool rows_on = [] { const char *e = getenv("AXHIP_WHERE_ROWS"); return !(e && e[0] == '0'); }();
+        const int L = ndim - 1;
+        bool rows = rows_on && ndim >= 1 && shape[L] % v == 0 && aligned(dst);
+        int64_t reach = w.total;
+        auto fits = [&](const void *p, int dt, const int64_t *st) {
+            const int es = dt == AXHIP_DTYPE_F32 ? 4 : dt == AXHIP_DTYPE_U8 ? 1 : 2;
+            int64_t span = 0;
+            for (int d = 0; d < ndim; ++d) span += (shape[d] - 1) * st[d];
+            reach = std::max(reach, span + v);
+            if (st[L] == 0) return true;
+            if (st[L] != 1 || reinterpret_cast<uintptr_t>(p) % (static_cast<uintptr_t>(v) * es) != 0) return false;
+            for (int d = 0; d < L; ++d)
+                if (st[d] % v != 0) return false;
+            return true;
+        };
+        rows = rows && fits(cond, cond_dtype, cond_strides) && fits(a, a_dtype, a_strides) && fits(b, b_dtype, b_strides);
+        if (rows) {
+            w.shape[L] /= v;
+            w.total /= v;
+            w.cond_strides[L] *= v; w.a_strides[L] *= v; w.b_strides[L] *= v;
+            const bool small = reach < (int64_t(1) << 31) - (1 << 20);
+            const int64_t blocks = std::min<int64_t>((w.total + 255) / 256, 256 * 32);
+            auto kernel = v == 4 ? (small ? where_rows_kernel<uint32_t, 4> : where_rows_kernel<int64_t, 4>)
+                                 : (small ? where_rows_kernel<uint32_t, 8> : where_rows_kernel<int64_t, 8>);
+            hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w);
+        } else {
+            const int64_t blocks = std::min<int64_t>((w.total + 255) / 256, 256 * 64);
+            hipLaunchKernelGGL(where_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, w);
+        }
     }
     AXHIP_CHECK_HIP(hipGetLastError());
     return AXHIP_OK;

@@ -243,7 +243,7 @@ def test_products_and_truth_reductions_along_inner_axes():
 def _where(cond, a, b, a_dt, b_dt, out_dt, shape, cond_strides, a_strides, b_strides):
     dc, da, db = gh.to_dev(cond), gh.to_dev(a), gh.to_dev(b)
     out = gh.empty_dev(tuple(shape), out_dt)
-    out.fill_(float("nan") if out_dt == F32 else 0x7FC1)
+    out.fill_(float("nan") if out_dt == F32 else 0xC1 if out_dt == U8 else 0x7FC1)
     gh.sync()
     capi.check(capi.lib().axhip_where(dc.data_ptr(), U8, da.data_ptr(), a_dt, db.data_ptr(), b_dt, out.data_ptr(), out_dt, len(shape), i64(list(shape)),
                                       i64(list(cond_strides)), i64(list(a_strides)), i64(list(b_strides)), None))
@@ -282,6 +282,24 @@ def test_where_contiguous_broadcast_and_scalar_branches(dt):
     row = a.reshape(-1)[:64].copy()
     got = _where(c2, row, b, dt, dt, dt, shape, elem_strides((10, 1), shape), elem_strides((64,), shape), full)
     assert same(got, axo.where(np.broadcast_to(c2, shape).copy(), np.broadcast_to(row, shape).copy(), b, dt))
+    # a (10, 64) mask over the batch (attention scores under a [queries, keys] mask), one branch a scalar; the same with
+    # the other branch a (6, 1, 1) column of per-batch values and an fp32 result
+    c4 = (g.uniform((10, 64)) > 0.5).astype(np.uint8) * 3
+    got = _where(c4, zero, b, dt, dt, dt, shape, elem_strides((10, 64), shape), [0, 0, 0], full)
+    assert same(got, axo.where(np.broadcast_to(c4, shape).copy(), np.broadcast_to(zero, shape).copy(), b, dt))
+    col = g.normal((6, 1, 1))
+    got = _where(c4, a, col, dt, F32, F32, shape, elem_strides((10, 64), shape), full, elem_strides((6, 1, 1), shape))
+    assert same(got, np.where(np.broadcast_to(c4, shape) != 0, a if dt == F32 else axo.to_f32(a, dt), np.broadcast_to(col, shape)))
+    # rows of a wider array (pitch 64, 48 taken) and a truth-valued result
+    s3 = (6, 10, 48)
+    pitched = [640, 64, 1]
+    c5 = (g.uniform(s3) > 0.5).astype(np.uint8)
+    got = _where(c5, a, b, dt, dt, dt, s3, elem_strides(s3, s3), pitched, pitched)
+    assert same(got, axo.where(c5, np.ascontiguousarray(a[..., :48]), np.ascontiguousarray(b[..., :48]), dt))
+    bf32 = b if dt == F32 else axo.to_f32(b, dt)
+    got = _where(c5, a, b, dt, dt, U8, s3, elem_strides(s3, s3), [0, 0, 0], pitched)
+    a0 = (a if dt == F32 else axo.to_f32(a, dt)).reshape(-1)[0]
+    assert same(got, np.where(c5 != 0, a0 != 0, bf32[..., :48] != 0).astype(np.uint8))
     # odd sizes (the element-wise kernel) and mixed branch types with an fp32 result
     s2 = (5, 37)
     c3 = (g.uniform(s2) > 0.3).astype(np.uint8)
