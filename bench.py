@@ -617,6 +617,39 @@ def bench_survey(torch, capi, stream, steps, warmup):
             {"kernel": "softmax_axis", "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
              "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(torch.isfinite(full.float()).all().item())}, launch, avg_ms, nbytes)
         del t, out, full
+    # the movers around attention scores and convolutions: a [queries, keys] mask and a key-padding mask filled into
+    # [batch, heads, queries, keys] scores, where() under the same mask, a convolution input padded by one on each side
+    i64 = lambda *v: (C.c_int64 * len(v))(*v)
+    S = (4, 32, 1024, 1024)
+    full_st = i64(32 << 20, 1 << 20, 1024, 1)
+    scores, other, out = rnd(S, bf, 2.0), rnd(S, bf, 2.0), torch.empty(S, device="cuda", dtype=bf)
+    mask = (torch.rand((1024, 1024), device="cuda") > 0.5).to(torch.uint8)
+    keys = (torch.rand((4, 1024), device="cuda") > 0.5).to(torch.uint8)
+    BF, U8 = capi.DTYPE_BF16, capi.DTYPE_U8
+
+    def mover(name, kernel, launch, nbytes, check):
+        torch.cuda.synchronize()
+        avg_ms, min_ms, warm_n = time_launches(torch, stream, launch, steps, warmup)
+        res[name] = with_cold({"kernel": kernel, "avg_us": avg_ms * 1e3, "min_us": min_ms * 1e3, "bytes": nbytes,
+                               "frac_of_hbm_peak": nbytes / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "finite": bool(check())}, launch, avg_ms, nbytes)
+
+    nb = 2 * scores.numel() * 2
+    mover("masked_fill_bf16_4x32x1024x1024_mask_1024x1024", "masked_fill_vec",
+          lambda: capi.check(lib.axhip_masked_fill(scores.data_ptr(), BF, mask.data_ptr(), out.data_ptr(), 4, i64(*S), full_st, i64(0, 0, 1024, 1), -1e9, sp)),
+          nb, lambda: torch.equal(out, scores.masked_fill(mask.bool(), -1e9)))
+    mover("masked_fill_bf16_4x32x1024x1024_key_padding_4x1x1x1024", "masked_fill_vec",
+          lambda: capi.check(lib.axhip_masked_fill(scores.data_ptr(), BF, keys.data_ptr(), out.data_ptr(), 4, i64(*S), full_st, i64(1024, 0, 0, 1), -1e9, sp)),
+          nb, lambda: torch.equal(out, scores.masked_fill(keys.bool()[:, None, None, :], -1e9)))
+    mover("where_bf16_4x32x1024x1024_cond_1024x1024", "where_rows",
+          lambda: capi.check(lib.axhip_where(mask.data_ptr(), U8, scores.data_ptr(), BF, other.data_ptr(), BF, out.data_ptr(), BF, 4, i64(*S), i64(0, 0, 1024, 1), full_st, full_st, sp)),
+          3 * scores.numel() * 2, lambda: torch.equal(out, torch.where(mask.bool(), scores, other)))
+    del scores, other, out
+    x = rnd((32, 1280, 3000), bf, 1.0)
+    padded = torch.empty((32, 1280, 3002), device="cuda", dtype=bf)
+    mover("pad_bf16_32x1280x3000_by_1_1_last", "pad_vec",
+          lambda: capi.check(lib.axhip_pad(x.data_ptr(), padded.data_ptr(), BF, 3, i64(32, 1280, 3000), i64(1280 * 3000, 3000, 1), i64(0, 0, 1), i64(0, 0, 1), 0.0, sp)),
+          (x.numel() + padded.numel()) * 2, lambda: torch.equal(padded, torch.nn.functional.pad(x, (1, 1))))
+    del x, padded
     return res
 
 
